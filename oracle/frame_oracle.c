@@ -1,0 +1,124 @@
+/* TEST INFRASTRUCTURE - NOT PART OF THE PRODUCT.
+ *
+ * CPU restatement ("oracle") of the N2D2 Frame (CPU) cells on the quantized
+ * inference path: conv / fc / pool / scaling / activations and the SAT / LSQ
+ * fake-quant kernels.  Only tests, the smoke check and the CPU-baseline leg of
+ * the benchmark may load this library; the shipped HIP path never does.
+ *
+ * Every function cites the reference file:line it follows (paths relative to
+ * the N2D2 source tree).  Element type T is instantiated for float (the type
+ * N2D2 registers its cells with) and double (exact for all integer sums).
+ *
+ * Build: make -C oracle   (gcc, -ffp-contract=off so that no a*b+c is fused:
+ * the reference is built for baseline x86-64, which has no FMA).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+static inline int imax_(int a, int b) { return a > b ? a : b; }
+/* Utils::clamp<int>, include/utils/Utils.hpp:1038-1042 */
+static inline int iclamp_(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+#define CAT_(a, b) a##b
+#define CAT(a, b) CAT_(a, b)
+
+#define T float
+#define FN(name) CAT(oracle_, CAT(name, _f32))
+#define ROUND roundf
+#define TRUNC truncf
+#define TANH tanhf
+#define COSH coshf
+#define FABS fabsf
+#define SQRT sqrtf
+#include "frame_oracle_impl.inc"
+#undef T
+#undef FN
+#undef ROUND
+#undef TRUNC
+#undef TANH
+#undef COSH
+#undef FABS
+#undef SQRT
+
+#define T double
+#define FN(name) CAT(oracle_, CAT(name, _f64))
+#define ROUND round
+#define TRUNC trunc
+#define TANH tanh
+#define COSH cosh
+#define FABS fabs
+#define SQRT sqrt
+#include "frame_oracle_impl.inc"
+#undef T
+#undef FN
+
+/* src/Cell/ElemWiseCell_Frame.cpp:116-136 (Sum). ElemWiseCell_Frame is
+ * Float_T only. coeffMode: 0 PerLayer, 1 PerInput, 2 PerChannel.
+ * inputs: nbInputs pointers to NCHW tensors of identical shape. */
+void oracle_elemwise_sum_f32(const float* const* inputs, int nbInputs, int B, int C, int H, int W,
+                             const float* weights, const float* shifts, int coeffMode, float* out)
+{
+    for (int b = 0; b < B; ++b)
+        for (int ch = 0; ch < C; ++ch)
+            for (int y = 0; y < H; ++y)
+                for (int x = 0; x < W; ++x) {
+                    const size_t i = (size_t)x + (size_t)W * ((size_t)y + (size_t)H * ((size_t)ch + (size_t)C * b));
+                    const size_t c0 = (coeffMode == 2) ? (size_t)ch : 0;
+                    out[i] = weights[c0] * inputs[0][i] + shifts[c0];
+                    for (int k = 1; k < nbInputs; ++k) {
+                        const size_t c1 = (coeffMode == 2) ? c0 : (size_t)k;
+                        out[i] += weights[c1] * inputs[k][i] + shifts[c1];
+                    }
+                }
+}
+
+/* src/Cell/Cell.cpp:251-300 (getNbGroups), regular case only: returns -1 where
+ * the reference falls back to getNbGroupsHandMade (irregular mappings).
+ * map[o + O*c], Tensor<bool> {O,C}. */
+long oracle_get_nb_groups(const unsigned char* map, size_t nbOutputs, size_t nbChannels)
+{
+    size_t nbChannelsPerGroup = 0;
+    for (; nbChannelsPerGroup < nbChannels && map[0 + nbOutputs * nbChannelsPerGroup];
+         ++nbChannelsPerGroup) {}
+    if (nbChannelsPerGroup == 0)
+        return 0;
+    if (nbChannels % nbChannelsPerGroup != 0)
+        return -1;
+    const size_t nbGroups = nbChannels / nbChannelsPerGroup;
+    if (nbOutputs % nbGroups != 0)
+        return -1;
+    const size_t nbOutputsPerGroup = nbOutputs / nbGroups;
+    size_t outputGroupOffset = 0, channelGroupOffset = 0;
+    for (size_t group = 0; group < nbGroups; ++group) {
+        for (size_t output = outputGroupOffset; output < outputGroupOffset + nbOutputsPerGroup; ++output) {
+            size_t channel = 0;
+            for (; channel < channelGroupOffset; ++channel)
+                if (map[output + nbOutputs * channel]) return -1;
+            for (; channel < channelGroupOffset + nbChannelsPerGroup; ++channel)
+                if (!map[output + nbOutputs * channel]) return -1;
+            for (; channel < nbChannels; ++channel)
+                if (map[output + nbOutputs * channel]) return -1;
+        }
+        outputGroupOffset += nbOutputsPerGroup;
+        channelGroupOffset += nbChannelsPerGroup;
+    }
+    return (long)nbGroups;
+}
+
+/* src/Cell/ConvCell.cpp:1169-1195 (setOutputsDims, no ext padding) */
+unsigned int oracle_conv_out_dim(unsigned int in, unsigned int k, unsigned int stride,
+                                 unsigned int pad, unsigned int dil, unsigned int subSample)
+{
+    const int kernelExtent = (int)(dil * (k - 1) + 1);
+    return (unsigned int)ceil(floor(((int)in + 2 * (int)pad - kernelExtent + (int)stride)
+                                    / (double)stride) / (double)subSample);
+}
+
+/* src/Cell/PoolCell.cpp:219-240 (setOutputsDims, no ext padding) */
+unsigned int oracle_pool_out_dim(unsigned int in, unsigned int pool, unsigned int stride, unsigned int pad)
+{
+    return (unsigned int)(((int)in + 2 * (int)pad - (int)pool + (int)stride) / (double)stride);
+}
