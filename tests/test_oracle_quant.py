@@ -163,10 +163,10 @@ def test_sat_activation_forward_reference_formula(nb_bits, alpha):
 
 
 def test_sat_activation_round_is_half_away():
-    rng, alpha = 15.0, 6.0
-    x = (np.array([0.5, 1.5, 2.5, 13.5]) * alpha / rng)          # float64 oracle keeps the ties exact
+    rng, alpha = 16.0, 8.0                                       # powers of two: the ties are exact
+    x = (np.array([0.5, 1.5, 2.5, 13.5]) * alpha / rng).astype(np.float32)
     y, _ = orc.sat_act_forward(x, rng, alpha)
-    assert np.allclose(y / alpha * rng, [1, 2, 3, 14], atol=1e-9)
+    assert (y / alpha * rng).tolist() == [1, 2, 3, 14]
 
 
 def test_sat_activation_backward_ste_edges_and_alpha_gradient():
