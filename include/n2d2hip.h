@@ -1,0 +1,234 @@
+/*
+ * n2d2hip.h - C ABI of the MI355X (gfx950) implementation of N2D2's quantized
+ * inference hot path ("Frame_HIP" model).
+ *
+ * Plain C: opaque handles, plain pointers and sizes, int status codes
+ * (0 = success).  No exceptions cross this boundary; the C++ cell glue turns a
+ * non-zero status into std::runtime_error(n2d2hip_last_error()), which is how
+ * the reference reports errors.  All tensors are caller-owned DEVICE buffers
+ * unless a parameter is documented as HOST.  Every call takes an explicit HIP
+ * stream (hipStream_t passed as void*) and is asynchronous on it.
+ *
+ * Citations "ref: file:line" name the N2D2 (v1.3.0) interface an entry point
+ * replaces; paths are relative to the N2D2 source tree.
+ */
+#ifndef N2D2HIP_H
+#define N2D2HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* n2d2hip_stream_t; /* hipStream_t */
+
+/* ---------------------------------------------------------------- status */
+enum {
+    N2D2HIP_OK = 0,
+    N2D2HIP_ERR_INVALID = 1,       /* null pointer, shape mismatch, bad enum */
+    N2D2HIP_ERR_UNSUPPORTED = 2,   /* valid in N2D2 but outside this path */
+    N2D2HIP_ERR_HIP = 3,           /* a HIP runtime call failed */
+    N2D2HIP_ERR_NOT_QUANTIZED = 4, /* integer rescale on nb_bits == 0 (the reference throws) */
+    N2D2HIP_ERR_WORKSPACE = 5      /* workspace too small */
+};
+const char* n2d2hip_strerror(int status);
+/* Message of the last failing call on the calling thread ("" if none). */
+const char* n2d2hip_last_error(void);
+/* Library version string and the gfx target the kernels were built for. */
+const char* n2d2hip_version(void);
+
+/* --------------------------------------------------------------- tensors */
+/* Element types.  N2D2 holds integer values in float storage
+ * (ref: src/Cell/ConvCell_Frame.cpp:28-44); here they are stored narrow. */
+enum {
+    N2D2HIP_U8 = 0,  /* unsigned 8-bit value */
+    N2D2HIP_I8 = 1,  /* signed 8-bit value */
+    N2D2HIP_I32 = 2, /* signed 32-bit value (accumulators, logits) */
+    N2D2HIP_F32 = 3, /* float holding an integer value (graph edges) */
+    N2D2HIP_U8B = 4  /* unsigned 8-bit value v stored as the signed byte v-128:
+                        the form the signed int8 matrix cores consume */
+};
+/* Layouts.  NCHW is N2D2's Tensor order {X,Y,Z,B}, X fastest
+ * (ref: include/containers/Tensor.hpp:162-193).  NHWC is the private
+ * channel-inner order used between Frame_HIP cells; its channel stride `cs`
+ * is a multiple of 16 (4 is accepted for network inputs with <= 4 channels). */
+enum { N2D2HIP_NCHW = 0, N2D2HIP_NHWC = 1 };
+
+typedef struct n2d2hip_tensor {
+    void* data;
+    int dtype;  /* N2D2HIP_U8 ... */
+    int layout; /* N2D2HIP_NCHW / N2D2HIP_NHWC */
+    int B, C, H, W;
+    int cs;     /* NHWC: bytes-per-pixel channel stride in elements (>= C); NCHW: ignored */
+} n2d2hip_tensor;
+
+/* Channel stride the library uses for an NHWC tensor with C channels. */
+int n2d2hip_nhwc_cs(int C);
+/* Bytes needed for a tensor (uses cs for NHWC). */
+size_t n2d2hip_tensor_bytes(const n2d2hip_tensor* t);
+
+/* Graph-edge conversion between any two dtype/layout combinations of the same
+ * logical shape (e.g. F32 NCHW <-> U8B NHWC).  Values that do not fit the
+ * destination type are saturated.  Channels C..cs-1 of an NHWC destination
+ * are written as logical zero. */
+int n2d2hip_convert(const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream);
+
+/* ------------------------------------------------- scaling + activation */
+/* ref: include/ScalingMode.hpp:27-62 (same order as N2D2::ScalingMode) */
+enum {
+    N2D2HIP_SCALING_NONE = 0,
+    N2D2HIP_SCALING_FLOAT_MULT = 1,
+    N2D2HIP_SCALING_FIXED_MULT16 = 2,
+    N2D2HIP_SCALING_FIXED_MULT32 = 3,
+    N2D2HIP_SCALING_SINGLE_SHIFT = 4,
+    N2D2HIP_SCALING_DOUBLE_SHIFT = 5
+};
+enum { N2D2HIP_ACT_LINEAR = 0, N2D2HIP_ACT_RECTIFIER = 1 };
+
+/* What an N2D2 Activation carries on the quantized path
+ * (ref: include/Activation/Activation.hpp:36-110, include/Scaling.hpp:336-432).
+ * All pointers are HOST pointers to per-output-channel vectors. */
+typedef struct n2d2hip_activation {
+    int kind;               /* N2D2HIP_ACT_LINEAR / N2D2HIP_ACT_RECTIFIER */
+    float leak_slope;       /* Rectifier LeakSlope; must be 0 on the integer path */
+    int scaling_mode;       /* N2D2HIP_SCALING_* */
+    const void* scaling;    /* FLOAT_MULT: float[C]; FIXED_*: int32_t[C];
+                               SINGLE_SHIFT: uint8_t[C]; DOUBLE_SHIFT: uint8_t[C][2] = {first, second} */
+    int frac_bits;          /* FIXED_*: nbFractionalBits (one value per cell) */
+    int is_clipped;         /* FLOAT_MULT / FIXED_*: apply Clip before the rescale */
+    const float* clipping;  /* float[C] when is_clipped */
+    int nb_bits;            /* quantizedNbBits handed to Scaling::propagate: the activation's
+                               bits if set, else the cell's (ref: RectifierActivation_Frame.hpp:65-66) */
+    int unsigned_out;       /* DeepNetExport::isCellOutputUnsigned(cell) (ref: src/Export/DeepNetExport.cpp:370-388) */
+} n2d2hip_activation;
+
+typedef struct n2d2hip_act_s* n2d2hip_act_t;
+
+/* Builds the per-channel device tables for `Scaling::propagate` followed by
+ * the Rectifier / Linear pass (ref: include/Scaling.hpp:434-459,
+ * src/Scaling_Kernels.cpp:29-199, include/Activation/RectifierActivation_Frame.hpp:55-87,
+ * include/Activation/LinearActivation_Frame.hpp:56-81). */
+int n2d2hip_act_create(const n2d2hip_activation* desc, int nb_channels, n2d2hip_act_t* act);
+int n2d2hip_act_destroy(n2d2hip_act_t act);
+
+/* Stand-alone Scaling (+ activation) over a tensor: ScalingCell_Frame::propagate
+ * (ref: src/Cell/ScalingCell_Frame.cpp:67-75) and the tail of Cell_Frame::propagate
+ * (ref: src/Cell/Cell_Frame.cpp:473-478).  `in` is U8/I8/U8B/I32/F32 of either layout,
+ * `out` has the same layout and shape. */
+int n2d2hip_scaling_forward(n2d2hip_act_t act, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                            n2d2hip_stream_t stream);
+
+/* ------------------------------------------------------------------ conv */
+/* ref: include/Cell/ConvCell_Frame_Kernels.hpp:40-54 (Descriptor), include/Cell/ConvCell.hpp:45-55 */
+typedef struct n2d2hip_conv_desc {
+    int C, O;               /* input channels, output channels */
+    int kW, kH;
+    int strideX, strideY;
+    int padL, padT, padR, padB;
+    int dilX, dilY;
+    int groups;             /* Cell::getNbGroups of the mapping (ref: src/Cell/Cell.cpp:251-300): 1, or C == O (depthwise) */
+    int weight_bits;        /* 8: int8_t weights; 4: two weights per byte, element 2i in the low nibble */
+} n2d2hip_conv_desc;
+
+typedef struct n2d2hip_conv_s* n2d2hip_conv_t;
+
+/* Prepares a quantized ConvCell: weights HOST int8 OCHW ({kW,kH,C/groups,O}, kW fastest;
+ * nibble-packed in the same order when weight_bits == 4), bias HOST int32[O] or NULL
+ * (NoBias).  `act` is borrowed and must outlive the conv.  `in_dtype` is the element
+ * type the cell will be fed (U8B, I8 or U8), fixed at creation.
+ * Replaces ConvCell_Frame<T>::initialize + propagate
+ * (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/ConvCell_Frame_Kernels.cpp:26-174). */
+int n2d2hip_conv_create(const n2d2hip_conv_desc* desc, const void* weights, const int32_t* bias,
+                        n2d2hip_act_t act, int in_dtype, n2d2hip_conv_t* conv);
+int n2d2hip_conv_destroy(n2d2hip_conv_t conv);
+/* Output spatial size (ref: src/Cell/ConvCell.cpp:1169-1195). */
+int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH, int* outW);
+/* in / out: NHWC.  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE). */
+int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                         n2d2hip_stream_t stream);
+
+/* -------------------------------------------------------------------- fc */
+typedef struct n2d2hip_conv_s* n2d2hip_fc_t;
+/* Quantized FcCell over a C x H x W input: weights HOST int8 [O][C*H*W] in N2D2's CHW
+ * flattening, bias HOST int32[O] or NULL.  Executed as a convolution whose kernel spans
+ * the input (ref: src/Cell/FcCell_Frame.cpp:234-340). */
+int n2d2hip_fc_create(int C, int H, int W, int O, int weight_bits, const void* weights, const int32_t* bias,
+                      n2d2hip_act_t act, int in_dtype, n2d2hip_fc_t* fc);
+int n2d2hip_fc_destroy(n2d2hip_fc_t fc);
+int n2d2hip_fc_forward(n2d2hip_fc_t fc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                       n2d2hip_stream_t stream);
+
+/* ------------------------------------------------------------------ pool */
+enum { N2D2HIP_POOL_MAX = 0, N2D2HIP_POOL_AVERAGE = 1 };
+/* ref: include/Cell/PoolCell_Frame_Kernels.hpp (Descriptor), include/Cell/PoolCell.hpp:47-55 */
+typedef struct n2d2hip_pool_desc {
+    int pooling;            /* N2D2HIP_POOL_MAX / N2D2HIP_POOL_AVERAGE */
+    int poolW, poolH;
+    int strideX, strideY;
+    int padX, padY;
+} n2d2hip_pool_desc;
+int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* desc, int H, int W, int* outH, int* outW);
+/* Per-channel (unit map) quantized pooling on NHWC U8/I8/U8B; average is the truncated
+ * quotient sum / (poolW*poolH) (ref: src/Cell/PoolCell_Frame_Kernels.cpp:26-197,
+ * src/Cell/PoolCell_Frame.cpp:123-174).  out has the dtype of in. */
+int n2d2hip_pool_forward(const n2d2hip_pool_desc* desc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                         n2d2hip_stream_t stream);
+
+/* -------------------------------------------------------------- elemwise */
+enum { N2D2HIP_COEFF_PER_LAYER = 0, N2D2HIP_COEFF_PER_INPUT = 1, N2D2HIP_COEFF_PER_CHANNEL = 2 };
+typedef struct n2d2hip_elemwise_s* n2d2hip_elemwise_t;
+/* ElemWiseCell Sum: out = act( w[c0]*in0 + s[c0] + sum_k (w[c1]*in_k + s[c1]) ), float
+ * coefficient arithmetic exactly as the reference (ref: src/Cell/ElemWiseCell_Frame.cpp:116-136).
+ * weights / shifts: HOST float vectors already sized as ElemWiseCell_Frame::initialize leaves
+ * them (nb_inputs entries, or C entries for PER_CHANNEL); NULL means all 1 / all 0. */
+int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, const float* weights,
+                            const float* shifts, n2d2hip_act_t act, n2d2hip_elemwise_t* ew);
+int n2d2hip_elemwise_destroy(n2d2hip_elemwise_t ew);
+int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
+                             n2d2hip_stream_t stream);
+
+/* --------------------------------------------------- SAT / LSQ fake-quant */
+/* Weight quantizer modes, numbered as SATQuantizerCell_Frame::propagate selects them
+ * (ref: src/Quantizer/QAT/Cell/SAT/SATQuantizerCell_Frame.cpp:188-200). */
+enum {
+    N2D2HIP_SAT_NONE = 0, N2D2HIP_SAT_DEFAULT = 1, N2D2HIP_SAT_FULLRANGE = 2,
+    N2D2HIP_SAT_SYMRANGE = 3, N2D2HIP_SAT_ASYMRANGE = 4, N2D2HIP_SAT_NONE_ASYM = 5
+};
+/* Bytes of device scratch the SAT/LSQ entry points need for their reductions. */
+size_t n2d2hip_quantizer_workspace_bytes(size_t n);
+/* tanh-normalised DoReFa weight fake-quant, optional SAT scaling
+ * (ref: src/Quantizer/QAT/Kernel/SATQuantizer_Frame_Kernels.cpp:66-262).
+ * stats (device float[2]) receives {tanh_max, sat_scaling}. */
+int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range, int mode,
+                               int apply_scaling, unsigned outputs_size, float* stats,
+                               void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
+/* ref: SATQuantizer_Frame_Kernels.cpp:349-404; factor = tanh_max * scaling read from stats */
+int n2d2hip_sat_weight_backward(const float* diff_wq, const float* w, float* diff_w, size_t n, float range,
+                                int mode, int apply_scaling, const float* stats, n2d2hip_stream_t stream);
+/* ref: SATQuantizer_Frame_Kernels.cpp:268-322; alpha: device float[1]; fp_copy NULL when inference */
+int n2d2hip_sat_act_forward(float* x, float* fp_copy, size_t n, float range, const float* alpha,
+                            n2d2hip_stream_t stream);
+/* ref: SATQuantizer_Frame_Kernels.cpp:410-448 + SATQuantizerActivation_Frame.cpp:133-135:
+ * diff_alpha[0] = sum_i dalpha_i + beta * diff_alpha[0] */
+int n2d2hip_sat_act_backward(const float* diff_in, const float* fp_x, float* diff_out, size_t n, float range,
+                             const float* alpha, float beta, float* diff_alpha,
+                             void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
+/* LSQ forward for weights (lo,hi) = (-(R+1)/2,(R-1)/2) and activations (0,R); step: device float[1]
+ * (ref: src/Quantizer/QAT/Cell/LSQ/LSQQuantizerCell_Frame.cpp:194-208,
+ *       src/Quantizer/QAT/Activation/LSQ/LSQQuantizerActivation_Frame.cpp:131-141). */
+int n2d2hip_lsq_forward(const float* x, float* xq, size_t n, const float* step, int lo, int hi,
+                        n2d2hip_stream_t stream);
+/* STE mask + step-size gradient.  diff_step[0] = (sum_i term_i + beta * diff_step[0]) * grad_scale:
+ * the update of LSQQuantizerCell_Frame::back_propagate (ref: ...LSQQuantizerCell_Frame.cpp:234-303)
+ * and LSQQuantizerActivation_Frame::back_propagate (ref: ...LSQQuantizerActivation_Frame.cpp:193-271);
+ * beta = 0 on a new solver iteration, 1 otherwise; grad_scale = 1/sqrt(N*hi). */
+int n2d2hip_lsq_backward(const float* diff_q, const float* fp_x, float* diff_fp, size_t n, const float* step,
+                         int lo, int hi, float grad_scale, float beta, float* diff_step,
+                         void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* N2D2HIP_H */

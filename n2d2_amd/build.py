@@ -1,0 +1,56 @@
+"""Builds libn2d2hip.so (the C-ABI library of hand-written gfx950 kernels) with hipcc.
+
+hipcc cross-compiles for gfx950 without a GPU.  The library is built in-tree
+(n2d2_amd/lib/) so that it travels with the source tree.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIBDIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIBDIR, "libn2d2hip.so")
+SOURCES = ["act.hip", "conv_igemm.hip", "bandwidth.hip", "quantizer.hip"]
+
+# -ffp-contract=off: float rescales must round the product and the sum
+# separately, as the reference (built for baseline x86-64) does.
+# The packed-fp32 target feature is switched off for all device code.
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build(verbose=False):
+    os.makedirs(LIBDIR, exist_ok=True)
+    objdir = os.path.join(LIBDIR, "obj")
+    os.makedirs(objdir, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        return _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        outs = list(ex.map(compile_one, zip(SOURCES, objs)))
+    outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs))
+    if verbose:
+        for o in outs:
+            if o.strip():
+                print(o)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

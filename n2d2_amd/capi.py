@@ -1,0 +1,110 @@
+"""ctypes binding of include/n2d2hip.h, one Python function per C entry point.
+
+This is the binding the test-suite and the benchmark go through; it adds no
+arithmetic of its own.  Loading fails loudly when the HIP library has not been
+built (python -m n2d2_amd.build): there is no CPU fallback.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libn2d2hip.so")
+
+# enums of n2d2hip.h
+U8, I8, I32, F32, U8B = 0, 1, 2, 3, 4
+NCHW, NHWC = 0, 1
+SCALING_NONE, SCALING_FLOAT_MULT, SCALING_FIXED_MULT16, SCALING_FIXED_MULT32, SCALING_SINGLE_SHIFT, SCALING_DOUBLE_SHIFT = range(6)
+ACT_LINEAR, ACT_RECTIFIER = 0, 1
+POOL_MAX, POOL_AVERAGE = 0, 1
+COEFF_PER_LAYER, COEFF_PER_INPUT, COEFF_PER_CHANNEL = 0, 1, 2
+SAT_NONE, SAT_DEFAULT, SAT_FULLRANGE, SAT_SYMRANGE, SAT_ASYMRANGE, SAT_NONE_ASYM = range(6)
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOT_QUANTIZED, ERR_WORKSPACE = range(6)
+
+# every symbol include/n2d2hip.h declares
+SYMBOLS = [
+    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes",
+    "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
+    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward",
+    "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
+    "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
+    "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward",
+    "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_backward",
+    "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
+]
+
+
+class Tensor(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dtype", C.c_int), ("layout", C.c_int),
+                ("B", C.c_int), ("C", C.c_int), ("H", C.c_int), ("W", C.c_int), ("cs", C.c_int)]
+
+
+class Activation(C.Structure):
+    _fields_ = [("kind", C.c_int), ("leak_slope", C.c_float), ("scaling_mode", C.c_int), ("scaling", C.c_void_p),
+                ("frac_bits", C.c_int), ("is_clipped", C.c_int), ("clipping", C.c_void_p),
+                ("nb_bits", C.c_int), ("unsigned_out", C.c_int)]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [("C", C.c_int), ("O", C.c_int), ("kW", C.c_int), ("kH", C.c_int), ("strideX", C.c_int), ("strideY", C.c_int),
+                ("padL", C.c_int), ("padT", C.c_int), ("padR", C.c_int), ("padB", C.c_int), ("dilX", C.c_int), ("dilY", C.c_int),
+                ("groups", C.c_int), ("weight_bits", C.c_int)]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [("pooling", C.c_int), ("poolW", C.c_int), ("poolH", C.c_int), ("strideX", C.c_int), ("strideY", C.c_int),
+                ("padX", C.c_int), ("padY", C.c_int)]
+
+
+class N2D2HipError(RuntimeError):
+    def __init__(self, status, message):
+        RuntimeError.__init__(self, message)
+        self.status = status
+
+
+def load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("libn2d2hip.so is not built (%s): run `python -m n2d2_amd.build`; "
+                          "there is no CPU fallback for the Frame_HIP path" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name in ("n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version"):
+        getattr(lib, name).restype = C.c_char_p
+    lib.n2d2hip_tensor_bytes.restype = C.c_size_t
+    lib.n2d2hip_quantizer_workspace_bytes.restype = C.c_size_t
+    lib.n2d2hip_quantizer_workspace_bytes.argtypes = [C.c_size_t]
+    P, I, F, SZ, U = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
+    lib.n2d2hip_convert.argtypes = [P, P, P]
+    lib.n2d2hip_act_create.argtypes = [P, I, P]
+    lib.n2d2hip_act_destroy.argtypes = [P]
+    lib.n2d2hip_scaling_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_conv_create.argtypes = [P, P, P, P, I, P]
+    lib.n2d2hip_conv_destroy.argtypes = [P]
+    lib.n2d2hip_conv_out_dims.argtypes = [P, I, I, P, P]
+    lib.n2d2hip_conv_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_fc_create.argtypes = [I, I, I, I, I, P, P, P, I, P]
+    lib.n2d2hip_fc_destroy.argtypes = [P]
+    lib.n2d2hip_fc_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_pool_out_dims.argtypes = [P, I, I, P, P]
+    lib.n2d2hip_pool_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_elemwise_create.argtypes = [I, I, I, P, P, P, P]
+    lib.n2d2hip_elemwise_destroy.argtypes = [P]
+    lib.n2d2hip_elemwise_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_sat_weight_forward.argtypes = [P, P, SZ, F, I, I, U, P, P, SZ, P]
+    lib.n2d2hip_sat_weight_backward.argtypes = [P, P, P, SZ, F, I, I, P, P]
+    lib.n2d2hip_sat_act_forward.argtypes = [P, P, SZ, F, P, P]
+    lib.n2d2hip_sat_act_backward.argtypes = [P, P, P, SZ, F, P, F, P, P, SZ, P]
+    lib.n2d2hip_lsq_forward.argtypes = [P, P, SZ, P, I, I, P]
+    lib.n2d2hip_lsq_backward.argtypes = [P, P, P, SZ, P, I, I, F, F, P, P, SZ, P]
+    return lib
+
+
+lib = load()
+
+
+def check(status):
+    if status != OK:
+        msg = lib.n2d2hip_last_error().decode() or lib.n2d2hip_strerror(status).decode()
+        raise N2D2HipError(status, msg)
+
+
+def nhwc_cs(c):
+    return int(lib.n2d2hip_nhwc_cs(int(c)))

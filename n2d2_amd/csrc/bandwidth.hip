@@ -1,0 +1,262 @@
+// Bandwidth-bound cells on NHWC byte tensors: PoolCell (max / truncated
+// average) and ElemWiseCell Sum with its activation.  One thread moves 4
+// consecutive channels (one dword) per tensor, so that a wavefront touches 256
+// contiguous bytes of every operand.
+#include <algorithm>
+
+#include "common.h"
+#include "epilogue.cuh"
+
+namespace n2d2hip {
+
+__device__ __forceinline__ void unpack4(int x, int zp, int v[4])
+{
+    v[0] = (int)(signed char)(x) + zp;
+    v[1] = (int)(signed char)(x >> 8) + zp;
+    v[2] = (int)(signed char)(x >> 16) + zp;
+    v[3] = (x >> 24) + zp;
+}
+__device__ __forceinline__ unsigned pack4(const int v[4])
+{
+    return ((unsigned)v[0] & 255u) | (((unsigned)v[1] & 255u) << 8) | (((unsigned)v[2] & 255u) << 16) | ((unsigned)v[3] << 24);
+}
+
+// ref: src/Cell/PoolCell_Frame_Kernels.cpp:26-197 with the unit mapping PoolCell builds
+// (one output per channel).  `flip` = 0x80808080 makes plain U8 bytes comparable as signed.
+template <bool IS_MAX>
+__global__ __launch_bounds__(256) void pool_kernel(const signed char* __restrict__ in, int cs, int B, int H, int W,
+                                                   signed char* __restrict__ out, int OH, int OW, int poolW, int poolH,
+                                                   int strideX, int strideY, int padX, int padY, int zp, unsigned flip)
+{
+    const int cq = cs >> 2;
+    const long long total = (long long)B * OH * OW * cq;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        const int c4 = (int)(idx % cq) * 4;
+        long long r = idx / cq;
+        const int ox = (int)(r % OW); r /= OW;
+        const int oy = (int)(r % OH);
+        const int b = (int)(r / OH);
+        const int bx = ox * strideX - padX, by = oy * strideY - padY;
+        // window limits as the reference clamps them
+        const int sxMin = max(-bx, 0), syMin = max(-by, 0);
+        const int sxMax = min(max(W - bx, 0), poolW), syMax = min(max(H - by, 0), poolH);
+        int acc[4];
+        bool valid = false;
+        acc[0] = acc[1] = acc[2] = acc[3] = 0;
+        for (int sy = syMin; sy < syMax; ++sy) {
+            for (int sx = sxMin; sx < sxMax; ++sx) {
+                const int xv = *(const int*)(in + (((long long)b * H + by + sy) * W + bx + sx) * cs + c4) ^ (int)flip;
+                int v[4];
+                unpack4(xv, zp, v);
+                if (IS_MAX) {
+                    if (!valid) { acc[0] = v[0]; acc[1] = v[1]; acc[2] = v[2]; acc[3] = v[3]; valid = true; }
+                    else { acc[0] = max(acc[0], v[0]); acc[1] = max(acc[1], v[1]); acc[2] = max(acc[2], v[2]); acc[3] = max(acc[3], v[3]); }
+                } else {
+                    acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
+                }
+            }
+        }
+        if (!IS_MAX) {
+            const int count = poolW * poolH;      // countIncludePadding = true
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                acc[t] = acc[t] / count;           // C division truncates toward zero, as std::trunc(sum / count)
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] -= zp;
+        *(unsigned*)(out + idx * 4) = pack4(acc) ^ flip;
+    }
+}
+
+constexpr int EW_MAX_INPUTS = 4;
+struct ElemWiseArgs {
+    const signed char* in[EW_MAX_INPUTS];
+    int zp[EW_MAX_INPUTS];
+    unsigned flip[EW_MAX_INPUTS];
+    int nb_inputs;
+    const float* w;     // [nb_inputs][cpad] coefficient per input and channel
+    const float* s;
+    int cpad;
+    void* out;
+    int out_dtype;
+    unsigned out_xor;
+    int cs;
+    long long npix;
+    EpiArgs epi;
+};
+
+// ref: src/Cell/ElemWiseCell_Frame.cpp:116-136 (Sum): float32 arithmetic in the same order,
+// products and sums rounded individually (no fused multiply-add), then the cell's activation.
+__global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
+{
+    const int cq = p.cs >> 2;
+    const long long total = p.npix * cq;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        const int c4 = (int)(idx % cq) * 4;
+        float o[4];
+        {
+            int v[4];
+            unpack4(*(const int*)(p.in[0] + idx * 4) ^ (int)p.flip[0], p.zp[0], v);
+            const float4 w = *(const float4*)(p.w + c4), s = *(const float4*)(p.s + c4);
+            o[0] = __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x);
+            o[1] = __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y);
+            o[2] = __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z);
+            o[3] = __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w);
+        }
+        for (int k = 1; k < p.nb_inputs; ++k) {
+            int v[4];
+            unpack4(*(const int*)(p.in[k] + idx * 4) ^ (int)p.flip[k], p.zp[k], v);
+            const float4 w = *(const float4*)(p.w + (long long)k * p.cpad + c4), s = *(const float4*)(p.s + (long long)k * p.cpad + c4);
+            o[0] = __fadd_rn(o[0], __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x));
+            o[1] = __fadd_rn(o[1], __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y));
+            o[2] = __fadd_rn(o[2], __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z));
+            o[3] = __fadd_rn(o[3], __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w));
+        }
+        int r[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            r[t] = epi_apply_dyn_f(p.epi, o[t], c4 + t);
+        if (p.out_dtype == N2D2HIP_I32)
+            *(int4*)((int*)p.out + idx * 4) = int4{r[0], r[1], r[2], r[3]};
+        else
+            *(unsigned*)((signed char*)p.out + idx * 4) = pack4(r) ^ p.out_xor;
+    }
+}
+
+} // namespace n2d2hip
+
+using namespace n2d2hip;
+
+struct n2d2hip_elemwise_s {
+    int nb_inputs, nb_channels, cpad;
+    n2d2hip_act_t act;
+    float* d_coeff;     // w then s, each [nb_inputs][cpad]
+};
+
+extern "C" {
+
+int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* d, int H, int W, int* outH, int* outW)
+{
+    N2D2HIP_REQUIRE(d && outH && outW, N2D2HIP_ERR_INVALID, "pool_out_dims: null argument");
+    N2D2HIP_REQUIRE(d->poolW > 0 && d->poolH > 0 && d->strideX > 0 && d->strideY > 0 && d->padX >= 0 && d->padY >= 0,
+                    N2D2HIP_ERR_INVALID, "pool_out_dims: bad descriptor");
+    // ref: src/Cell/PoolCell.cpp:219-240
+    *outW = (int)((W + 2 * d->padX - d->poolW + d->strideX) / (double)d->strideX);
+    *outH = (int)((H + 2 * d->padY - d->poolH + d->strideY) / (double)d->strideY);
+    N2D2HIP_REQUIRE(*outW > 0 && *outH > 0, N2D2HIP_ERR_INVALID, "pool_out_dims: empty output");
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    int rc, OH, OW;
+    N2D2HIP_REQUIRE(d != nullptr, N2D2HIP_ERR_INVALID, "pool_forward: null descriptor");
+    N2D2HIP_REQUIRE(d->pooling == N2D2HIP_POOL_MAX || d->pooling == N2D2HIP_POOL_AVERAGE, N2D2HIP_ERR_INVALID, "pool_forward: bad pooling %d", d->pooling);
+    if ((rc = check_tensor(in, "pool input")) || (rc = check_tensor(out, "pool output")) || (rc = n2d2hip_pool_out_dims(d, in->H, in->W, &OH, &OW)))
+        return rc;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED, "pool_forward: tensors must be NHWC");
+    N2D2HIP_REQUIRE(is_byte_type(in->dtype) && out->dtype == in->dtype, N2D2HIP_ERR_INVALID, "pool_forward: byte tensors of one dtype expected");
+    N2D2HIP_REQUIRE(out->B == in->B && out->C == in->C && out->H == OH && out->W == OW && out->cs == in->cs, N2D2HIP_ERR_INVALID,
+                    "pool_forward: output is %dx%dx%dx%d (cs %d), expected %dx%dx%dx%d (cs %d)", out->B, out->C, out->H, out->W, out->cs,
+                    in->B, in->C, OH, OW, in->cs);
+    const long long total = (long long)in->B * OH * OW * (in->cs / 4);
+    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
+    const unsigned flip = in->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
+    const int zp = in->dtype == N2D2HIP_I8 ? 0 : 128;      // after the flip, U8 bytes read as value-128 too
+    if (d->pooling == N2D2HIP_POOL_MAX)
+        hipLaunchKernelGGL(pool_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
+                           in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
+    else
+        hipLaunchKernelGGL(pool_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
+                           in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, const float* weights, const float* shifts,
+                            n2d2hip_act_t act, n2d2hip_elemwise_t* ew)
+{
+    N2D2HIP_REQUIRE(act && ew, N2D2HIP_ERR_INVALID, "elemwise_create: null argument");
+    N2D2HIP_REQUIRE(nb_inputs >= 1 && nb_inputs <= EW_MAX_INPUTS, N2D2HIP_ERR_UNSUPPORTED, "elemwise_create: %d inputs (1..%d)", nb_inputs, EW_MAX_INPUTS);
+    N2D2HIP_REQUIRE(coeff_mode >= N2D2HIP_COEFF_PER_LAYER && coeff_mode <= N2D2HIP_COEFF_PER_CHANNEL, N2D2HIP_ERR_INVALID, "elemwise_create: bad coeff mode");
+    N2D2HIP_REQUIRE(act->nb_channels == nb_channels, N2D2HIP_ERR_INVALID, "elemwise_create: activation built for %d channels, cell has %d", act->nb_channels, nb_channels);
+    const int cpad = act->cpad;
+    std::vector<float> h(2 * (size_t)nb_inputs * cpad);
+    float* hw = h.data();
+    float* hs = hw + (size_t)nb_inputs * cpad;
+    for (int k = 0; k < nb_inputs; ++k)
+        for (int c = 0; c < cpad; ++c) {
+            const int cc = c < nb_channels ? c : nb_channels - 1;
+            // ref: src/Cell/ElemWiseCell_Frame.cpp:121-130: input 0 uses index c0 (= channel when
+            // PerChannel, else 0); input k >= 1 uses c0 when PerChannel, else k.
+            const int c0 = coeff_mode == N2D2HIP_COEFF_PER_CHANNEL ? cc : 0;
+            const int idx = (k == 0) ? c0 : (coeff_mode == N2D2HIP_COEFF_PER_CHANNEL ? c0 : k);
+            hw[(size_t)k * cpad + c] = weights ? weights[idx] : 1.0f;
+            hs[(size_t)k * cpad + c] = shifts ? shifts[idx] : 0.0f;
+        }
+    n2d2hip_elemwise_s* e = new n2d2hip_elemwise_s();
+    e->nb_inputs = nb_inputs; e->nb_channels = nb_channels; e->cpad = cpad; e->act = act; e->d_coeff = nullptr;
+    hipError_t herr = hipMalloc((void**)&e->d_coeff, h.size() * sizeof(float));
+    if (herr == hipSuccess) herr = hipMemcpy(e->d_coeff, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (herr != hipSuccess) {
+        n2d2hip_elemwise_destroy(e);
+        return fail(N2D2HIP_ERR_HIP, "elemwise_create: device upload failed: %s", hipGetErrorString(herr));
+    }
+    *ew = e;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_elemwise_destroy(n2d2hip_elemwise_t ew)
+{
+    if (!ew) return N2D2HIP_OK;
+    if (ew->d_coeff) (void)hipFree(ew->d_coeff);
+    delete ew;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    int rc;
+    N2D2HIP_REQUIRE(ew && inputs, N2D2HIP_ERR_INVALID, "elemwise_forward: null argument");
+    if ((rc = check_tensor(out, "elemwise output")))
+        return rc;
+    N2D2HIP_REQUIRE(out->layout == N2D2HIP_NHWC && out->C == ew->nb_channels, N2D2HIP_ERR_INVALID, "elemwise_forward: NHWC output with %d channels expected", ew->nb_channels);
+    ElemWiseArgs a = {};
+    for (int k = 0; k < ew->nb_inputs; ++k) {
+        const n2d2hip_tensor* t = inputs[k];
+        if ((rc = check_tensor(t, "elemwise input")))
+            return rc;
+        N2D2HIP_REQUIRE(t->layout == N2D2HIP_NHWC && is_byte_type(t->dtype), N2D2HIP_ERR_UNSUPPORTED, "elemwise_forward: inputs must be NHWC byte tensors");
+        N2D2HIP_REQUIRE(t->B == out->B && t->C == out->C && t->H == out->H && t->W == out->W && t->cs == out->cs, N2D2HIP_ERR_INVALID,
+                        "elemwise_forward: input %d shape differs from the output", k);
+        a.in[k] = (const signed char*)t->data;
+        a.flip[k] = t->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
+        a.zp[k] = t->dtype == N2D2HIP_I8 ? 0 : 128;
+    }
+    const n2d2hip_act_s* act = ew->act;
+    if (is_byte_type(out->dtype)) {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(act->min_out >= lo && act->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "elemwise_forward: activation range [%d,%d] does not fit output dtype %d", act->min_out, act->max_out, out->dtype);
+    } else {
+        N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_UNSUPPORTED, "elemwise_forward: output must be a byte type or I32");
+    }
+    a.nb_inputs = ew->nb_inputs;
+    a.w = ew->d_coeff;
+    a.s = ew->d_coeff + (size_t)ew->nb_inputs * ew->cpad;
+    a.cpad = ew->cpad;
+    a.out = out->data;
+    a.out_dtype = out->dtype;
+    a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    a.cs = out->cs;
+    a.npix = (long long)out->B * out->H * out->W;
+    a.epi = act->args;
+    const long long total = a.npix * (a.cs / 4);
+    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
+    hipLaunchKernelGGL(elemwise_sum_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, a);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+} // extern "C"

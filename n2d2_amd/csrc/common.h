@@ -1,0 +1,84 @@
+// Internal definitions shared by the HIP translation units of libn2d2hip.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "n2d2hip.h"
+
+namespace n2d2hip {
+
+// Records the message returned by n2d2hip_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define N2D2HIP_HIP_CHECK(expr)                                                            \
+    do {                                                                                   \
+        hipError_t e__ = (expr);                                                           \
+        if (e__ != hipSuccess)                                                             \
+            return ::n2d2hip::fail(N2D2HIP_ERR_HIP, "%s failed: %s (%s:%d)", #expr,      \
+                                   hipGetErrorString(e__), __FILE__, __LINE__);            \
+    } while (0)
+
+#define N2D2HIP_REQUIRE(cond, code, ...)                                                   \
+    do {                                                                                   \
+        if (!(cond))                                                                       \
+            return ::n2d2hip::fail(code, __VA_ARGS__);                                    \
+    } while (0)
+
+inline int elem_size(int dtype)
+{
+    return (dtype == N2D2HIP_I32 || dtype == N2D2HIP_F32) ? 4 : 1;
+}
+inline bool is_byte_type(int dtype)
+{
+    return dtype == N2D2HIP_U8 || dtype == N2D2HIP_I8 || dtype == N2D2HIP_U8B;
+}
+// Value added to a stored byte to obtain the logical value.
+inline int zero_point(int dtype)
+{
+    return dtype == N2D2HIP_U8B ? 128 : 0;
+}
+inline int round_up(int x, int m)
+{
+    return (x + m - 1) / m * m;
+}
+int check_tensor(const n2d2hip_tensor* t, const char* what);
+
+// ---------------------------------------------------------------- epilogue
+// Device-side form of "Scaling::propagate, saturate, Rectifier/Linear" for one
+// cell.  Per-channel tables live in one device allocation of 5 int arrays of
+// `cpad` entries each (channels >= C replicate neutral values).
+enum EpiKind {
+    EPI_RAW = 0, // ScalingMode NONE: value passes through (ReLU if rectifier)
+    EPI_I24 = 1, // integer rescale, every intermediate fits 32 bits (24-bit multiply)
+    EPI_I64 = 2, // integer rescale with a 64-bit product
+    EPI_F32 = 3  // FloatingPointScaling: float32 multiply, round half away
+};
+
+struct EpiArgs {
+    int kind;
+    int lo, hi;        // saturation range with the ReLU folded in
+    int relu;          // EPI_RAW only
+    const int* a;      // I24/I64: pre-clamp low  | F32: clip low  (float bits)
+    const int* b;      // I24/I64: pre-clamp high | F32: clip high (float bits)
+    const int* c;      // I24/I64: multiplier     | F32: scale     (float bits)
+    const int* d;      // I24: rounding half (int32)
+    const int* e;      // I24/I64: right shift
+};
+
+} // namespace n2d2hip
+
+struct n2d2hip_act_s {
+    n2d2hip_activation desc;   // pointers inside are NOT kept valid; do not dereference
+    int nb_channels;
+    int cpad;
+    int* tables;               // device, 5 * cpad ints
+    n2d2hip::EpiArgs args;
+    int min_out, max_out;      // range of produced values (for dtype checks); RAW: INT range
+};

@@ -1,0 +1,644 @@
+// Quantized ConvCell / FcCell forward as an implicit GEMM on the gfx950 int8
+// matrix cores (v_mfma_i32_32x32x32_i8), with the cell's bias, rescale,
+// saturation and ReLU fused into the accumulator epilogue.
+//
+// Data layout in HBM
+//   activations  NHWC signed bytes, channel stride `cs` (multiple of 16, or 4 for
+//                <=4-channel network inputs).  Unsigned values are stored minus
+//                128 (N2D2HIP_U8B) so that the signed MFMA consumes them directly;
+//                the constant 128*sum(w) is folded into the bias at creation.
+//   weights      [Opad][ktot] signed bytes, K ordered as 16-byte "sub-chunks":
+//                (ky, kx, 16 channels) for cs%16==0, (ky, 4 taps kx..kx+3, 4
+//                channels) for cs==4.  int4 weights stay nibble-packed in HBM
+//                ([Opad][ktot/2]) and are widened to int8 on their way into LDS.
+//   sub-chunk table  one int4 {ky, kx, channel offset, valid} per sub-chunk.
+//
+// GEMM view: D[channel][pixel] += W[channel][k] * X[pixel][k].  The weights are
+// the MFMA "A" operand and the pixels the "B" operand, so that every lane ends
+// up with 4 consecutive output channels of one pixel: one packed dword.
+#include <algorithm>
+#include <limits>
+
+#include "common.h"
+#include "epilogue.cuh"
+
+namespace n2d2hip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct ConvArgs {
+    const signed char* in;
+    int in_cs, B, H, W;
+    int OH, OW, M;          // M = B*OH*OW output pixels
+    const signed char* w;   // prepared weights
+    int ktot;               // K bytes per weight row (multiple of 64)
+    int niter;              // ktot / 64
+    const int4* sub;        // sub-chunk table, ktot/16 entries
+    const int* bias;        // [Opad], zero-point fold included
+    void* out;
+    int out_cs, out_dtype;
+    int strideX, strideY, padL, padT, dilX, dilY;
+    int ntiles_n, nblocks;
+    unsigned fill;          // padding byte replicated 4x (logical zero of the input)
+    unsigned out_xor;       // 0x80808080 when the output is stored as value-128
+    EpiArgs epi;
+};
+
+__device__ __forceinline__ int swz(int row, int q)
+{
+    // 16-byte slot of (row, sub-chunk q) in a [rows][64 B] tile; the XOR spreads
+    // 16 consecutive rows of one sub-chunk over all 64 banks.
+    return ((row << 2) + (q ^ ((row >> 2) & 3))) << 4;
+}
+
+// Widens 8 nibble-packed weights (one dword: byte b = {low: w[b], high: w[b+4]})
+// to two dwords of int8.
+__device__ __forceinline__ void unpack_w4(unsigned p, int& lo, int& hi)
+{
+    const unsigned l = p & 0x0F0F0F0Fu, h = (p >> 4) & 0x0F0F0F0Fu;
+    // sign-extend each nibble inside its byte: ((n ^ 8) | 0x80) - 8, then clear the guard bit
+    lo = (int)(((((l ^ 0x08080808u) | 0x80808080u) - 0x08080808u)) ^ 0x80808080u);
+    hi = (int)(((((h ^ 0x08080808u) | 0x80808080u) - 0x08080808u)) ^ 0x80808080u);
+}
+
+template <int BM, int BN, int WGM, int EPI, bool PIX4, bool W4>
+__global__ __launch_bounds__(256) void conv_igemm_kernel(ConvArgs p)
+{
+    constexpr int WGN = 4 / WGM;
+    constexpr int TM = BM / WGM;      // pixels per wave
+    constexpr int TN = BN / WGN;      // channels per wave
+    constexpr int NI = TN / 32;       // channel tiles per wave
+    constexpr int NJ = TM / 32;       // pixel tiles per wave
+    constexpr int P_LOADS = BM / 64;  // 16 B loads per thread and K step, pixels
+    constexpr int W_LOADS = BN / 64;  // same, weights
+    constexpr int TILE_BYTES = (BM + BN) * 64;
+    constexpr int STAGE_STRIDE = BN + 16;
+    static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of 32x32");
+    static_assert(2 * TILE_BYTES >= BM * STAGE_STRIDE, "output staging must fit the operand buffers");
+
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * TILE_BYTES];
+
+    // XCD-aware block order: consecutive logical tiles run on the same XCD (they
+    // share the pixel tile in that XCD's L2); the grid is padded to a multiple of 8.
+    const int nbp = gridDim.x;
+    const int logical = (blockIdx.x & 7) * (nbp >> 3) + (blockIdx.x >> 3);
+    if (logical >= p.nblocks)
+        return;
+    const int tile_n = logical % p.ntiles_n;
+    const int tile_m = logical / p.ntiles_n;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave % WGM;
+    const int wn = wave / WGM;
+    const int lq = tid & 3;       // sub-chunk this thread loads
+    const int lr = tid >> 2;      // first tile row this thread loads
+
+    // ---- per-thread pixel rows
+    const signed char* rowptr[P_LOADS];
+    int base_y[P_LOADS], base_x[P_LOADS];
+    const int ohw = p.OH * p.OW;
+#pragma unroll
+    for (int i = 0; i < P_LOADS; ++i) {
+        const int m = m0 + lr + 64 * i;
+        if (m < p.M) {
+            const int b = m / ohw;
+            const int rem = m - b * ohw;
+            const int oy = rem / p.OW;
+            const int ox = rem - oy * p.OW;
+            base_y[i] = oy * p.strideY - p.padT;
+            base_x[i] = ox * p.strideX - p.padL;
+            rowptr[i] = p.in + (((long long)b * p.H + base_y[i]) * p.W + base_x[i]) * (long long)p.in_cs;
+        } else {
+            base_y[i] = -(1 << 28);     // every tap test fails: the row is all padding
+            base_x[i] = -(1 << 28);
+            rowptr[i] = p.in;
+        }
+    }
+    const signed char* wptr[W_LOADS];
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i)
+        wptr[i] = p.w + (long long)(n0 + lr + 64 * i) * (W4 ? (p.ktot >> 1) : p.ktot) + (W4 ? lq * 8 : lq * 16);
+
+    v4i preg[P_LOADS];
+    v4i wreg[W_LOADS];
+
+    auto load_global = [&](int it) {
+        const int4 s = p.sub[it * 4 + lq];     // {ky, kx, channel offset, valid}
+        const int dy = s.x * p.dilY;
+#pragma unroll
+        for (int i = 0; i < P_LOADS; ++i) {
+            // Tap validity exactly as the reference computes its window
+            // (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83): tap index >= max(pad - o*stride, 0)
+            // and dilated offset inside the input.
+            const bool yok = s.w && s.x >= -base_y[i] && base_y[i] + dy < p.H;
+            if (PIX4) {
+                const int* src = (const int*)(rowptr[i] + ((long long)dy * p.W + s.y) * 4);
+                v4i v;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int kx = s.y + t;
+                    const bool ok = yok && kx >= -base_x[i] && base_x[i] + kx < p.W;
+                    v[t] = ok ? src[t] : (int)p.fill;
+                }
+                preg[i] = v;
+            } else {
+                const int dx = s.y * p.dilX;
+                const bool ok = yok && s.y >= -base_x[i] && base_x[i] + dx < p.W;
+                if (ok) {
+                    preg[i] = *(const v4i*)(rowptr[i] + ((long long)dy * p.W + dx) * p.in_cs + s.z);
+                } else {
+                    const int f = (int)p.fill;
+                    preg[i] = v4i{f, f, f, f};
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            if (W4) {
+                // nibble-packed: 8 bytes carry this thread's 16 weights; widened in store_lds
+                const uint2 pk = *(const uint2*)(wptr[i] + (long long)it * 32);
+                wreg[i] = v4i{(int)pk.x, (int)pk.y, 0, 0};
+            } else {
+                wreg[i] = *(const v4i*)(wptr[i] + (long long)it * 64);
+            }
+        }
+    };
+    auto store_lds = [&](int buf) {
+        unsigned char* tp = smem + buf * TILE_BYTES;
+        unsigned char* tw = tp + BM * 64;
+#pragma unroll
+        for (int i = 0; i < P_LOADS; ++i)
+            *(v4i*)(tp + swz(lr + 64 * i, lq)) = preg[i];
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            if (W4) {
+                v4i v;
+                int a, b;
+                unpack_w4((unsigned)wreg[i][0], a, b); v[0] = a; v[1] = b;
+                unpack_w4((unsigned)wreg[i][1], a, b); v[2] = a; v[3] = b;
+                *(v4i*)(tw + swz(lr + 64 * i, lq)) = v;
+            } else {
+                *(v4i*)(tw + swz(lr + 64 * i, lq)) = wreg[i];
+            }
+        }
+    };
+
+    v16i acc[NI][NJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = 0;
+
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    const int l32 = lane & 31;
+    const int lh = lane >> 5;
+    for (int it = 0; it < p.niter; ++it) {
+        const int buf = it & 1;
+        if (it + 1 < p.niter)
+            load_global(it + 1);          // in flight while the matrix cores work
+        const unsigned char* tp = smem + buf * TILE_BYTES;
+        const unsigned char* tw = tp + BM * 64;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            v4i wf[NI], pf[NJ];
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+                wf[i] = *(const v4i*)(tw + swz(wn * TN + i * 32 + l32, 2 * ks + lh));
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                pf[j] = *(const v4i*)(tp + swz(wm * TM + j * 32 + l32, 2 * ks + lh));
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i], pf[j], acc[i][j], 0, 0, 0);
+        }
+        if (it + 1 < p.niter)
+            store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: bias, rescale, saturate, ReLU, pack, coalesced store.
+    // Accumulator layout of the 32x32 tile: lane holds column (pixel) lane%32 and rows
+    // (channels) 8*(r/4) + 4*(lane/32) + r%4 for r = 0..15.
+    const bool out_bytes = p.out_dtype != N2D2HIP_I32;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int ch_local = wn * TN + i * 32 + 8 * g + 4 * lh;
+            const int ch = n0 + ch_local;
+            const int4 bias4 = *(const int4*)(p.bias + ch);
+            int4 ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
+            if (EPI != EPI_RAW) {
+                ta = *(const int4*)(p.epi.a + ch);
+                tb = *(const int4*)(p.epi.b + ch);
+                tc = *(const int4*)(p.epi.c + ch);
+                if (EPI == EPI_I24)
+                    td = *(const int4*)(p.epi.d + ch);
+                if (EPI != EPI_F32)
+                    te = *(const int4*)(p.epi.e + ch);
+            }
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int pix_local = wm * TM + j * 32 + l32;
+                const int r0 = epi_apply<EPI>(acc[i][j][4 * g + 0] + bias4.x, ta.x, tb.x, tc.x, td.x, te.x, p.epi.lo, p.epi.hi, p.epi.relu);
+                const int r1 = epi_apply<EPI>(acc[i][j][4 * g + 1] + bias4.y, ta.y, tb.y, tc.y, td.y, te.y, p.epi.lo, p.epi.hi, p.epi.relu);
+                const int r2 = epi_apply<EPI>(acc[i][j][4 * g + 2] + bias4.z, ta.z, tb.z, tc.z, td.z, te.z, p.epi.lo, p.epi.hi, p.epi.relu);
+                const int r3 = epi_apply<EPI>(acc[i][j][4 * g + 3] + bias4.w, ta.w, tb.w, tc.w, td.w, te.w, p.epi.lo, p.epi.hi, p.epi.relu);
+                if (out_bytes) {
+                    const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8)
+                                          | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+                    *(unsigned*)(smem + pix_local * STAGE_STRIDE + ch_local) = packed ^ p.out_xor;
+                } else {
+                    const int m = m0 + pix_local;
+                    if (m < p.M && ch < p.out_cs)
+                        *(int4*)((int*)p.out + (long long)m * p.out_cs + ch) = int4{r0, r1, r2, r3};
+                }
+            }
+        }
+    }
+    if (out_bytes) {
+        __syncthreads();
+        constexpr int CHUNKS = BN / 16;
+        for (int id = tid; id < BM * CHUNKS; id += 256) {
+            const int row = id / CHUNKS;
+            const int cq = id - row * CHUNKS;
+            const int m = m0 + row;
+            const int ch = n0 + cq * 16;
+            if (m < p.M && ch < p.out_cs)
+                *(v4i*)((signed char*)p.out + (long long)m * p.out_cs + ch) = *(const v4i*)(smem + row * STAGE_STRIDE + cq * 16);
+        }
+    }
+}
+
+// ------------------------------------------------------------ depthwise
+// groups == C == O: one output channel per input channel, no reduction over
+// channels, hence no matrix core: a bandwidth kernel.  Each thread produces 4
+// consecutive channels of one output pixel; weights are prepared as [tap][cs]
+// so that consecutive lanes read consecutive bytes of both operands.
+__global__ __launch_bounds__(256) void depthwise_kernel(const signed char* __restrict__ in, int cs, int B, int H, int W,
+                                                        int OH, int OW, const signed char* __restrict__ w, int kH, int kW,
+                                                        const int* __restrict__ bias, void* __restrict__ out, int out_dtype,
+                                                        int strideX, int strideY, int padL, int padT, int dilX, int dilY,
+                                                        int in_zp, unsigned out_xor, EpiArgs epi)
+{
+    const int cq = cs >> 2;
+    const long long total = (long long)B * OH * OW * cq;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        const int c4 = (int)(idx % cq) * 4;
+        long long r = idx / cq;
+        const int ox = (int)(r % OW); r /= OW;
+        const int oy = (int)(r % OH);
+        const int b = (int)(r / OH);
+        const int by = oy * strideY - padT, bx = ox * strideX - padL;
+        int a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+        for (int ky = 0; ky < kH; ++ky) {
+            const int iy = by + ky * dilY;
+            if (ky < -by || iy >= H) continue;
+            for (int kx = 0; kx < kW; ++kx) {
+                const int ix = bx + kx * dilX;
+                if (kx < -bx || ix >= W) continue;
+                const int xv = *(const int*)(in + (((long long)b * H + iy) * W + ix) * cs + c4);
+                const int wv = *(const int*)(w + (long long)(ky * kW + kx) * cs + c4);
+                a0 += ((int)(signed char)(xv) + in_zp) * (int)(signed char)(wv);
+                a1 += ((int)(signed char)(xv >> 8) + in_zp) * (int)(signed char)(wv >> 8);
+                a2 += ((int)(signed char)(xv >> 16) + in_zp) * (int)(signed char)(wv >> 16);
+                a3 += ((xv >> 24) + in_zp) * (wv >> 24);
+            }
+        }
+        const int4 b4 = *(const int4*)(bias + c4);
+        const int r0 = epi_apply_dyn(epi, a0 + b4.x, c4 + 0);
+        const int r1 = epi_apply_dyn(epi, a1 + b4.y, c4 + 1);
+        const int r2 = epi_apply_dyn(epi, a2 + b4.z, c4 + 2);
+        const int r3 = epi_apply_dyn(epi, a3 + b4.w, c4 + 3);
+        if (out_dtype == N2D2HIP_I32) {
+            *(int4*)((int*)out + idx * 4) = int4{r0, r1, r2, r3};
+        } else {
+            const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+            *(unsigned*)((signed char*)out + idx * 4) = packed ^ out_xor;
+        }
+    }
+}
+
+} // namespace n2d2hip
+
+using namespace n2d2hip;
+
+struct n2d2hip_conv_s {
+    n2d2hip_conv_desc desc;
+    n2d2hip_act_t act;
+    int in_dtype;
+    int in_cs;            // channel stride the weights were prepared for
+    bool depthwise;
+    bool pix4;
+    int opad;             // weight rows (multiple of 128)
+    int ktot;
+    signed char* d_w;
+    int4* d_sub;
+    int* d_bias;
+    bool is_fc;
+    int fcH, fcW;
+};
+
+namespace {
+
+int conv_out_dim(int in, int k, int stride, int pad0, int pad1, int dil)
+{
+    // ref: src/Cell/ConvCell_Frame_Kernels.cpp:37-45
+    return (int)((in + pad0 + pad1 - dil * (k - 1) - 1 + stride) / (double)stride);
+}
+
+template <int BM, int BN, int WGM, bool PIX4, bool W4>
+void launch_cfg(const ConvArgs& a, hipStream_t stream)
+{
+    const int grid = round_up(a.nblocks, 8);
+    switch (a.epi.kind) {
+    case EPI_RAW: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_RAW, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_I24, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_I64, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_F32, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
+    }
+}
+
+int sext4(int n) { return (n & 8) ? (n | ~15) : (n & 15); }
+
+// Reads weight element `idx` of the caller's OCHW array (int8 or nibble-packed).
+int read_weight(const void* w, long long idx, int bits)
+{
+    if (bits == 8)
+        return ((const signed char*)w)[idx];
+    const unsigned char byte = ((const unsigned char*)w)[idx >> 1];
+    return sext4((idx & 1) ? (byte >> 4) : (byte & 15));
+}
+
+} // namespace
+
+extern "C" {
+
+int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* d, int H, int W, int* outH, int* outW)
+{
+    N2D2HIP_REQUIRE(d && outH && outW, N2D2HIP_ERR_INVALID, "conv_out_dims: null argument");
+    N2D2HIP_REQUIRE(d->strideX > 0 && d->strideY > 0 && d->kW > 0 && d->kH > 0 && d->dilX > 0 && d->dilY > 0,
+                    N2D2HIP_ERR_INVALID, "conv_out_dims: non-positive kernel / stride / dilation");
+    *outW = conv_out_dim(W, d->kW, d->strideX, d->padL, d->padR, d->dilX);
+    *outH = conv_out_dim(H, d->kH, d->strideY, d->padT, d->padB, d->dilY);
+    N2D2HIP_REQUIRE(*outW > 0 && *outH > 0, N2D2HIP_ERR_INVALID, "conv_out_dims: empty output %dx%d", *outW, *outH);
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const int32_t* bias, n2d2hip_act_t act,
+                        int in_dtype, n2d2hip_conv_t* conv)
+{
+    N2D2HIP_REQUIRE(d && weights && act && conv, N2D2HIP_ERR_INVALID, "conv_create: null argument");
+    N2D2HIP_REQUIRE(d->C > 0 && d->O > 0 && d->kW > 0 && d->kH > 0 && d->strideX > 0 && d->strideY > 0
+                    && d->dilX > 0 && d->dilY > 0 && d->padL >= 0 && d->padT >= 0 && d->padR >= 0 && d->padB >= 0,
+                    N2D2HIP_ERR_INVALID, "conv_create: bad descriptor");
+    N2D2HIP_REQUIRE(d->weight_bits == 8 || d->weight_bits == 4, N2D2HIP_ERR_INVALID, "conv_create: weight_bits %d (8 or 4)", d->weight_bits);
+    N2D2HIP_REQUIRE(is_byte_type(in_dtype), N2D2HIP_ERR_INVALID, "conv_create: input dtype must be U8, I8 or U8B");
+    N2D2HIP_REQUIRE(in_dtype != N2D2HIP_U8, N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_create: plain U8 inputs cannot feed the signed matrix cores; convert to U8B first");
+    N2D2HIP_REQUIRE(act->nb_channels == d->O, N2D2HIP_ERR_INVALID, "conv_create: activation built for %d channels, conv has %d outputs",
+                    act->nb_channels, d->O);
+    const bool depthwise = d->groups > 1;
+    if (depthwise)
+        N2D2HIP_REQUIRE(d->groups == d->C && d->C == d->O, N2D2HIP_ERR_UNSUPPORTED,
+                        "conv_create: groups = %d is supported only as depthwise (groups == C == O)", d->groups);
+    N2D2HIP_REQUIRE(d->groups >= 1, N2D2HIP_ERR_UNSUPPORTED, "conv_create: irregular mapping (nbGroups = %d)", d->groups);
+
+    n2d2hip_conv_s* c = new n2d2hip_conv_s();
+    c->desc = *d;
+    c->act = act;
+    c->in_dtype = in_dtype;
+    c->in_cs = n2d2hip_nhwc_cs(d->C);
+    c->depthwise = depthwise;
+    c->pix4 = (!depthwise && c->in_cs == 4);
+    c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr;
+    c->is_fc = false; c->fcH = c->fcW = 0;
+    if (c->pix4 && d->dilX != 1) {
+        delete c;
+        return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_create: <=4 input channels with dilationX = %d", d->dilX);
+    }
+    if (depthwise && d->weight_bits != 8) {
+        delete c;
+        return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_create: depthwise with 4-bit weights");
+    }
+    const int zp = zero_point(in_dtype);
+    const int Cg = d->C / d->groups;
+    const int cs = c->in_cs;
+    std::vector<signed char> hw;
+    std::vector<int4> hsub;
+    c->opad = round_up(d->O, 128);
+    std::vector<int> hbias((size_t)std::max(c->opad, act->cpad), 0);
+    const long long wstrideO = (long long)Cg * d->kH * d->kW;
+    for (int o = 0; o < d->O; ++o) {
+        long long s = 0;
+        for (long long i = 0; i < wstrideO; ++i)
+            s += read_weight(weights, o * wstrideO + i, d->weight_bits);
+        const long long b = (bias ? (long long)bias[o] : 0) + (long long)zp * s;
+        if (b < std::numeric_limits<int>::min() || b > std::numeric_limits<int>::max()) {
+            delete c;
+            return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_create: folded bias of output %d overflows int32", o);
+        }
+        hbias[o] = (int)b;
+    }
+
+    if (depthwise) {
+        // [tap][cs]
+        hw.assign((size_t)d->kH * d->kW * cs, 0);
+        for (int ch = 0; ch < d->C; ++ch)
+            for (int ky = 0; ky < d->kH; ++ky)
+                for (int kx = 0; kx < d->kW; ++kx)
+                    hw[(size_t)(ky * d->kW + kx) * cs + ch] = (signed char)read_weight(weights, ((long long)ch * d->kH + ky) * d->kW + kx, 8);
+        // the kernel adds the zero point to every loaded input, so the fold is not wanted here
+        for (int o = 0; o < d->O; ++o)
+            hbias[o] = bias ? bias[o] : 0;
+        c->ktot = 0;
+    } else {
+        // sub-chunk table
+        if (c->pix4) {
+            for (int ky = 0; ky < d->kH; ++ky)
+                for (int kx0 = 0; kx0 < d->kW; kx0 += 4)
+                    hsub.push_back(int4{ky, kx0, 0, 1});
+        } else {
+            for (int ky = 0; ky < d->kH; ++ky)
+                for (int kx = 0; kx < d->kW; ++kx)
+                    for (int c0 = 0; c0 < cs; c0 += 16)
+                        hsub.push_back(int4{ky, kx, c0, 1});
+        }
+        while (hsub.size() % 4 != 0)
+            hsub.push_back(int4{0, 0, 0, 0});
+        c->ktot = (int)hsub.size() * 16;
+        std::vector<signed char> full((size_t)c->opad * c->ktot, 0);
+        for (int o = 0; o < d->O; ++o) {
+            signed char* row = full.data() + (size_t)o * c->ktot;
+            for (size_t j = 0; j < hsub.size(); ++j) {
+                if (!hsub[j].w) continue;
+                for (int e = 0; e < 16; ++e) {
+                    int ky = hsub[j].x, kx, ch;
+                    if (c->pix4) { kx = hsub[j].y + e / 4; ch = e % 4; }
+                    else { kx = hsub[j].y; ch = hsub[j].z + e; }
+                    if (kx >= d->kW || ch >= d->C) continue;
+                    row[j * 16 + e] = (signed char)read_weight(weights, (((long long)o * d->C + ch) * d->kH + ky) * d->kW + kx, d->weight_bits);
+                }
+            }
+        }
+        if (d->weight_bits == 4) {
+            // nibble-pack per 16-weight sub-chunk: byte b of dword q holds weight 8q+b (low) and 8q+4+b (high)
+            hw.assign(full.size() / 2, 0);
+            for (size_t s16 = 0; s16 < full.size() / 16; ++s16)
+                for (int q = 0; q < 2; ++q)
+                    for (int b = 0; b < 4; ++b) {
+                        const int lo = full[s16 * 16 + 8 * q + b] & 15, hi = full[s16 * 16 + 8 * q + 4 + b] & 15;
+                        hw[s16 * 8 + 4 * q + b] = (signed char)(lo | (hi << 4));
+                    }
+        } else {
+            hw.swap(full);
+        }
+    }
+
+    hipError_t e = hipMalloc((void**)&c->d_w, hw.size());
+    if (e == hipSuccess) e = hipMemcpy(c->d_w, hw.data(), hw.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void**)&c->d_bias, hbias.size() * sizeof(int));
+    if (e == hipSuccess) e = hipMemcpy(c->d_bias, hbias.data(), hbias.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e == hipSuccess && !hsub.empty()) {
+        e = hipMalloc((void**)&c->d_sub, hsub.size() * sizeof(int4));
+        if (e == hipSuccess) e = hipMemcpy(c->d_sub, hsub.data(), hsub.size() * sizeof(int4), hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) {
+        n2d2hip_conv_destroy(c);
+        return fail(N2D2HIP_ERR_HIP, "conv_create: device upload failed: %s", hipGetErrorString(e));
+    }
+    *conv = c;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv_destroy(n2d2hip_conv_t c)
+{
+    if (!c) return N2D2HIP_OK;
+    if (c->d_w) (void)hipFree(c->d_w);
+    if (c->d_sub) (void)hipFree(c->d_sub);
+    if (c->d_bias) (void)hipFree(c->d_bias);
+    delete c;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    int rc;
+    N2D2HIP_REQUIRE(c != nullptr, N2D2HIP_ERR_INVALID, "conv_forward: null conv");
+    if ((rc = check_tensor(in, "conv input")) || (rc = check_tensor(out, "conv output")))
+        return rc;
+    const n2d2hip_conv_desc& d = c->desc;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward: tensors must be NHWC (use n2d2hip_convert at graph edges)");
+    N2D2HIP_REQUIRE(in->dtype == c->in_dtype, N2D2HIP_ERR_INVALID, "conv_forward: input dtype %d, conv created for %d", in->dtype, c->in_dtype);
+    N2D2HIP_REQUIRE(in->C == d.C && in->cs == c->in_cs, N2D2HIP_ERR_INVALID,
+                    "conv_forward: input has %d channels (stride %d), conv expects %d (stride %d)", in->C, in->cs, d.C, c->in_cs);
+    int OH, OW;
+    if ((rc = n2d2hip_conv_out_dims(&d, in->H, in->W, &OH, &OW)))
+        return rc;
+    N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
+                    "conv_forward: output is %dx%dx%dx%d, expected %dx%dx%dx%d", out->B, out->C, out->H, out->W, in->B, d.O, OH, OW);
+    N2D2HIP_REQUIRE(out->cs % 16 == 0, N2D2HIP_ERR_INVALID, "conv_forward: output channel stride %d must be a multiple of 16", out->cs);
+    const n2d2hip_act_s* act = c->act;
+    if (act->args.kind == EPI_RAW) {
+        N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_INVALID,
+                        "conv_forward: without a rescale the cell outputs raw sums; the output dtype must be I32");
+    } else if (is_byte_type(out->dtype)) {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(act->min_out >= lo && act->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "conv_forward: activation range [%d,%d] does not fit output dtype %d", act->min_out, act->max_out, out->dtype);
+    } else {
+        N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: F32 outputs are produced with n2d2hip_convert");
+    }
+    const long long Mll = (long long)in->B * OH * OW;
+    N2D2HIP_REQUIRE(Mll < (1ll << 31) && (long long)in->B * in->H * in->W * in->cs < (1ll << 40), N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward: tensor too large");
+    const unsigned out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+
+    if (c->depthwise) {
+        N2D2HIP_REQUIRE(out->cs == in->cs, N2D2HIP_ERR_INVALID, "conv_forward: depthwise needs equal channel strides");
+        const long long total = Mll * (in->cs / 4);
+        const unsigned grid = (unsigned)std::min<long long>((total + 255) / 256, 256 * 64);
+        hipLaunchKernelGGL(depthwise_kernel, dim3(grid), dim3(256), 0, stream, (const signed char*)in->data, in->cs, in->B, in->H,
+                           in->W, OH, OW, c->d_w, d.kH, d.kW, c->d_bias, out->data, out->dtype, d.strideX, d.strideY, d.padL,
+                           d.padT, d.dilX, d.dilY, zero_point(in->dtype), out_xor, act->args);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
+
+    ConvArgs a;
+    a.in = (const signed char*)in->data;
+    a.in_cs = in->cs; a.B = in->B; a.H = in->H; a.W = in->W;
+    a.OH = OH; a.OW = OW; a.M = (int)Mll;
+    a.w = c->d_w; a.ktot = c->ktot; a.niter = c->ktot / 64; a.sub = c->d_sub; a.bias = c->d_bias;
+    a.out = out->data; a.out_cs = out->cs; a.out_dtype = out->dtype;
+    a.strideX = d.strideX; a.strideY = d.strideY; a.padL = d.padL; a.padT = d.padT; a.dilX = d.dilX; a.dilY = d.dilY;
+    a.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
+    a.out_xor = out_xor;
+    a.epi = act->args;
+
+    // Tile choice: 128 channels per block when the layer has them, and 64-pixel
+    // tiles when 128-pixel tiles would leave most of the 256 CUs idle.
+    const bool w4 = d.weight_bits == 4;
+    const int opad_n = round_up(d.O, 64);
+    const bool bn128 = opad_n % 128 == 0 || opad_n > 256;
+    const int BN = bn128 ? 128 : 64;
+    a.ntiles_n = (round_up(d.O, 16) + BN - 1) / BN;
+    const long long blocks128 = ((Mll + 127) / 128) * a.ntiles_n;
+    const bool bm64 = bn128 && !c->pix4 && blocks128 < 512;
+    const int BM = bm64 ? 64 : 128;
+    a.nblocks = (int)(((Mll + BM - 1) / BM) * a.ntiles_n);
+    if (c->pix4) {
+        if (bn128) { if (w4) launch_cfg<128, 128, 2, true, true>(a, stream); else launch_cfg<128, 128, 2, true, false>(a, stream); }
+        else { if (w4) launch_cfg<128, 64, 2, true, true>(a, stream); else launch_cfg<128, 64, 2, true, false>(a, stream); }
+    } else if (!bn128) {
+        if (w4) launch_cfg<128, 64, 2, false, true>(a, stream); else launch_cfg<128, 64, 2, false, false>(a, stream);
+    } else if (bm64) {
+        if (w4) launch_cfg<64, 128, 1, false, true>(a, stream); else launch_cfg<64, 128, 1, false, false>(a, stream);
+    } else {
+        if (w4) launch_cfg<128, 128, 2, false, true>(a, stream); else launch_cfg<128, 128, 2, false, false>(a, stream);
+    }
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+// ------------------------------------------------------------------- fc
+int n2d2hip_fc_create(int C, int H, int W, int O, int weight_bits, const void* weights, const int32_t* bias,
+                      n2d2hip_act_t act, int in_dtype, n2d2hip_fc_t* fc)
+{
+    N2D2HIP_REQUIRE(C > 0 && H > 0 && W > 0 && O > 0, N2D2HIP_ERR_INVALID, "fc_create: bad shape");
+    // [O][C*H*W] in CHW order is exactly an OCHW kernel of size H x W.
+    n2d2hip_conv_desc d = {};
+    d.C = C; d.O = O; d.kW = W; d.kH = H;
+    d.strideX = d.strideY = 1; d.dilX = d.dilY = 1; d.groups = 1; d.weight_bits = weight_bits;
+    int rc = n2d2hip_conv_create(&d, weights, bias, act, in_dtype, fc);
+    if (rc == N2D2HIP_OK) { (*fc)->is_fc = true; (*fc)->fcH = H; (*fc)->fcW = W; }
+    return rc;
+}
+
+int n2d2hip_fc_destroy(n2d2hip_fc_t fc) { return n2d2hip_conv_destroy(fc); }
+
+int n2d2hip_fc_forward(n2d2hip_fc_t fc, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(fc != nullptr && in != nullptr, N2D2HIP_ERR_INVALID, "fc_forward: null argument");
+    N2D2HIP_REQUIRE(fc->is_fc, N2D2HIP_ERR_INVALID, "fc_forward: handle was not created by n2d2hip_fc_create");
+    N2D2HIP_REQUIRE(in->H == fc->fcH && in->W == fc->fcW, N2D2HIP_ERR_INVALID, "fc_forward: input is %dx%d, cell built for %dx%d",
+                    in->H, in->W, fc->fcH, fc->fcW);
+    return n2d2hip_conv_forward(fc, in, out, stream);
+}
+
+} // extern "C"

@@ -1,0 +1,226 @@
+"""Thin object layer over the C ABI for the tests and the benchmark.
+
+torch is used for device memory and streams only; every computation goes
+through libn2d2hip.so.  Handles own their C objects and keep alive the host
+arrays they were built from.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import lib, check
+
+_TORCH_DT = {capi.U8: torch.uint8, capi.I8: torch.int8, capi.U8B: torch.int8, capi.I32: torch.int32, capi.F32: torch.float32}
+_NP_DT = {capi.U8: np.uint8, capi.I8: np.int8, capi.U8B: np.int8, capi.I32: np.int32, capi.F32: np.float32}
+
+
+def stream_ptr():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class DTensor:
+    """A device tensor plus its n2d2hip_tensor descriptor."""
+
+    def __init__(self, B, Cc, H, W, dtype, layout=capi.NHWC, buf=None):
+        self.B, self.C, self.H, self.W, self.dtype, self.layout = B, Cc, H, W, dtype, layout
+        self.cs = capi.nhwc_cs(Cc) if layout == capi.NHWC else Cc
+        n = B * H * W * self.cs
+        self.buf = buf if buf is not None else torch.empty(n, dtype=_TORCH_DT[dtype], device="cuda")
+        assert self.buf.numel() == n
+        self.desc = capi.Tensor(self.buf.data_ptr(), dtype, layout, B, Cc, H, W, self.cs)
+
+    @property
+    def ref(self):
+        return C.byref(self.desc)
+
+    @property
+    def nbytes(self):
+        return self.buf.numel() * self.buf.element_size()
+
+    @staticmethod
+    def from_numpy(x, dtype, layout=capi.NHWC):
+        """x: integer-valued NCHW numpy array. Uploads it as I32/F32 NCHW and converts on the device."""
+        x = np.ascontiguousarray(x)
+        B, Cc, H, W = x.shape
+        if x.dtype == np.float32:
+            src = DTensor(B, Cc, H, W, capi.F32, capi.NCHW, torch.from_numpy(x.reshape(-1)).cuda())
+        else:
+            src = DTensor(B, Cc, H, W, capi.I32, capi.NCHW, torch.from_numpy(x.astype(np.int32).reshape(-1)).cuda())
+        if dtype == src.dtype and layout == capi.NCHW:
+            return src
+        dst = DTensor(B, Cc, H, W, dtype, layout)
+        check(lib.n2d2hip_convert(src.ref, dst.ref, stream_ptr()))
+        return dst
+
+    def to_numpy(self):
+        """Logical integer values as an int64 NCHW numpy array."""
+        dst = DTensor(self.B, self.C, self.H, self.W, capi.I32, capi.NCHW)
+        check(lib.n2d2hip_convert(self.ref, dst.ref, stream_ptr()))
+        torch.cuda.synchronize()
+        return dst.buf.cpu().numpy().reshape(self.B, self.C, self.H, self.W).astype(np.int64)
+
+    def raw(self):
+        torch.cuda.synchronize()
+        return self.buf.cpu().numpy()
+
+
+class Act:
+    """n2d2hip_act_t: Scaling + Rectifier/Linear of one cell."""
+
+    def __init__(self, nb_channels, kind="Linear", mode="None", scaling=None, frac_bits=0, clipping=None,
+                 nb_bits=8, unsigned_out=False, leak_slope=0.0):
+        modes = {"None": capi.SCALING_NONE, "FloatMult": capi.SCALING_FLOAT_MULT, "FixedMult16": capi.SCALING_FIXED_MULT16,
+                 "FixedMult32": capi.SCALING_FIXED_MULT32, "SingleShift": capi.SCALING_SINGLE_SHIFT,
+                 "DoubleShift": capi.SCALING_DOUBLE_SHIFT}
+        m = modes[mode]
+        self._keep = []
+        sp = None
+        if scaling is not None:
+            np_t = {capi.SCALING_FLOAT_MULT: np.float32, capi.SCALING_FIXED_MULT16: np.int32, capi.SCALING_FIXED_MULT32: np.int32,
+                    capi.SCALING_SINGLE_SHIFT: np.uint8, capi.SCALING_DOUBLE_SHIFT: np.uint8}[m]
+            s = np.ascontiguousarray(scaling, dtype=np_t)
+            self._keep.append(s)
+            sp = s.ctypes.data
+        cp = None
+        if clipping is not None:
+            cl = np.ascontiguousarray(clipping, dtype=np.float32)
+            self._keep.append(cl)
+            cp = cl.ctypes.data
+        d = capi.Activation(capi.ACT_RECTIFIER if kind == "Rectifier" else capi.ACT_LINEAR, float(leak_slope), m, sp,
+                            int(frac_bits), int(clipping is not None), cp, int(nb_bits), int(bool(unsigned_out)))
+        self.nb_channels = nb_channels
+        self.mode = mode
+        self.unsigned_out = bool(unsigned_out)
+        self.handle = C.c_void_p()
+        check(lib.n2d2hip_act_create(C.byref(d), nb_channels, C.byref(self.handle)))
+
+    def out_dtype(self):
+        """Storage type of this cell's output between Frame_HIP cells."""
+        if self.mode == "None":
+            return capi.I32
+        return capi.U8B if self.unsigned_out else capi.I8
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib.n2d2hip_act_destroy(self.handle)
+            self.handle = None
+
+
+def scaling_forward(act, x, out_dtype=None):
+    out = DTensor(x.B, x.C, x.H, x.W, out_dtype if out_dtype is not None else act.out_dtype(), x.layout)
+    check(lib.n2d2hip_scaling_forward(act.handle, x.ref, out.ref, stream_ptr()))
+    return out
+
+
+def pack_int4(w):
+    """int array in [-8,7] -> bytes, element 2i in the low nibble."""
+    f = np.ascontiguousarray(w).reshape(-1).astype(np.int64)
+    if f.size % 2:
+        f = np.concatenate([f, [0]])
+    return ((f[0::2] & 15) | ((f[1::2] & 15) << 4)).astype(np.uint8)
+
+
+class Conv:
+    def __init__(self, w, bias, act, in_dtype, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, weight_bits=8):
+        """w: integer-valued [O, C/groups, kH, kW]; stride/dil (x,y); pad (L,T,R,B)."""
+        O, Cg, kH, kW = w.shape
+        self.desc = capi.ConvDesc(Cg * groups, O, kW, kH, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
+                                  dil[0], dil[1], groups, weight_bits)
+        self.act = act
+        hw = pack_int4(w) if weight_bits == 4 else np.ascontiguousarray(w, dtype=np.int8)
+        hb = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        self.handle = C.c_void_p()
+        check(lib.n2d2hip_conv_create(C.byref(self.desc), hw.ctypes.data, None if hb is None else hb.ctypes.data,
+                                      act.handle, in_dtype, C.byref(self.handle)))
+
+    def out_shape(self, H, W):
+        oh, ow = C.c_int(), C.c_int()
+        check(lib.n2d2hip_conv_out_dims(C.byref(self.desc), H, W, C.byref(oh), C.byref(ow)))
+        return oh.value, ow.value
+
+    def make_output(self, x, out_dtype=None):
+        oh, ow = self.out_shape(x.H, x.W)
+        return DTensor(x.B, self.desc.O, oh, ow, out_dtype if out_dtype is not None else self.act.out_dtype())
+
+    def forward(self, x, out=None, out_dtype=None):
+        if out is None:
+            out = self.make_output(x, out_dtype)
+        check(lib.n2d2hip_conv_forward(self.handle, x.ref, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib.n2d2hip_conv_destroy(self.handle)
+            self.handle = None
+
+
+class Fc:
+    def __init__(self, w, bias, act, in_dtype, in_shape, weight_bits=8):
+        """w: integer-valued [O, C*H*W] (CHW flattening); in_shape = (C, H, W)."""
+        Cc, H, W = in_shape
+        O = w.shape[0]
+        self.O = O
+        self.act = act
+        hw = pack_int4(w) if weight_bits == 4 else np.ascontiguousarray(w, dtype=np.int8)
+        hb = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)
+        self.handle = C.c_void_p()
+        check(lib.n2d2hip_fc_create(Cc, H, W, O, weight_bits, hw.ctypes.data, None if hb is None else hb.ctypes.data,
+                                    act.handle, in_dtype, C.byref(self.handle)))
+
+    def make_output(self, x, out_dtype=None):
+        return DTensor(x.B, self.O, 1, 1, out_dtype if out_dtype is not None else self.act.out_dtype())
+
+    def forward(self, x, out=None, out_dtype=None):
+        if out is None:
+            out = self.make_output(x, out_dtype)
+        check(lib.n2d2hip_fc_forward(self.handle, x.ref, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib.n2d2hip_fc_destroy(self.handle)
+            self.handle = None
+
+
+class Pool:
+    def __init__(self, kind, pool, stride, pad=(0, 0)):
+        self.desc = capi.PoolDesc(capi.POOL_MAX if kind == "max" else capi.POOL_AVERAGE, pool[0], pool[1],
+                                  stride[0], stride[1], pad[0], pad[1])
+
+    def make_output(self, x):
+        oh, ow = C.c_int(), C.c_int()
+        check(lib.n2d2hip_pool_out_dims(C.byref(self.desc), x.H, x.W, C.byref(oh), C.byref(ow)))
+        return DTensor(x.B, x.C, oh.value, ow.value, x.dtype)
+
+    def forward(self, x, out=None):
+        if out is None:
+            out = self.make_output(x)
+        check(lib.n2d2hip_pool_forward(C.byref(self.desc), x.ref, out.ref, stream_ptr()))
+        return out
+
+
+class ElemWiseSum:
+    def __init__(self, nb_inputs, nb_channels, act, weights=None, shifts=None, coeff_mode="PerLayer"):
+        mode = {"PerLayer": capi.COEFF_PER_LAYER, "PerInput": capi.COEFF_PER_INPUT, "PerChannel": capi.COEFF_PER_CHANNEL}[coeff_mode]
+        self.act = act
+        self.nb_inputs = nb_inputs
+        w = None if weights is None else np.ascontiguousarray(weights, dtype=np.float32)
+        s = None if shifts is None else np.ascontiguousarray(shifts, dtype=np.float32)
+        self.handle = C.c_void_p()
+        check(lib.n2d2hip_elemwise_create(nb_inputs, nb_channels, mode, None if w is None else w.ctypes.data,
+                                          None if s is None else s.ctypes.data, act.handle, C.byref(self.handle)))
+
+    def forward(self, xs, out=None, out_dtype=None):
+        x0 = xs[0]
+        if out is None:
+            out = DTensor(x0.B, x0.C, x0.H, x0.W, out_dtype if out_dtype is not None else self.act.out_dtype())
+        arr = (C.c_void_p * len(xs))(*[C.addressof(x.desc) for x in xs])
+        check(lib.n2d2hip_elemwise_forward(self.handle, arr, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            lib.n2d2hip_elemwise_destroy(self.handle)
+            self.handle = None

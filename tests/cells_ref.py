@@ -1,0 +1,71 @@
+"""Reference cells assembled from the CPU oracle, in the order the N2D2 Frame
+cells call their kernels (ConvCell_Frame::propagate, FcCell_Frame::propagate,
+Cell_Frame::propagate -> Activation::propagate -> Scaling::propagate)."""
+import numpy as np
+
+from oracle import oracle as orc
+
+
+class ActSpec:
+    """Host description of a cell's activation (kind, Scaling, bits, signedness)."""
+
+    def __init__(self, kind="Linear", mode="None", scaling=None, frac_bits=0, clipping=None, nb_bits=8, unsigned_out=False):
+        self.kind, self.mode, self.scaling, self.frac_bits = kind, mode, scaling, frac_bits
+        self.clipping, self.nb_bits, self.unsigned_out = clipping, nb_bits, unsigned_out
+
+    def kwargs(self):
+        return dict(kind=self.kind, mode=self.mode, scaling=self.scaling, frac_bits=self.frac_bits,
+                    clipping=self.clipping, nb_bits=self.nb_bits, unsigned_out=self.unsigned_out)
+
+    def apply(self, x):
+        """Scaling::propagate dispatch (include/Scaling.hpp:434-459) then the activation pass."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        if self.mode == "None":
+            y = x.copy()
+        elif self.mode == "FloatMult":
+            y = orc.scaling_float(x, self.scaling, self.nb_bits, self.unsigned_out, self.clipping)
+        elif self.mode in ("FixedMult16", "FixedMult32"):
+            y = orc.scaling_fixed(x, self.scaling, self.frac_bits, self.nb_bits, self.unsigned_out, self.clipping)
+        elif self.mode == "SingleShift":
+            y = orc.scaling_single_shift(x, self.scaling, self.nb_bits, self.unsigned_out)
+        elif self.mode == "DoubleShift":
+            y = orc.scaling_double_shift(x, self.scaling, self.nb_bits, self.unsigned_out)
+        else:
+            raise ValueError(self.mode)
+        if self.kind == "Rectifier":
+            y = orc.rectifier(y)
+        else:
+            y = orc.linear(y)
+        return y
+
+
+def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    maps = None
+    if groups > 1:
+        maps = orc.group_maps(x.shape[1], w.shape[0], groups)
+    y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps)
+    if bias is not None:
+        orc.conv_forward_bias(y, np.asarray(bias, dtype=np.float32))
+    return act.apply(y)
+
+
+def fc_cell(x, w, bias, act):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = orc.fc_forward(x, np.asarray(w, dtype=np.float32), None if bias is None else np.asarray(bias, dtype=np.float32))
+    return act.apply(y.reshape(y.shape[0], y.shape[1], 1, 1))
+
+
+def pool_cell(x, kind, pool, stride, pad=(0, 0)):
+    return orc.pool_forward(np.ascontiguousarray(x, dtype=np.float32), pool, stride, pad, kind=kind, quantized=True)
+
+
+def elemwise_cell(xs, act, weights=None, shifts=None, coeff_mode="PerLayer"):
+    n = len(xs)
+    Cc = xs[0].shape[1]
+    size = Cc if coeff_mode == "PerChannel" else n
+    w = np.ones(size, dtype=np.float32) if weights is None else np.asarray(weights, dtype=np.float32)
+    s = np.zeros(size, dtype=np.float32) if shifts is None else np.asarray(shifts, dtype=np.float32)
+    y = orc.elemwise_sum([np.asarray(x, dtype=np.float32) for x in xs], w, s, coeff_mode)
+    return act.apply(y)

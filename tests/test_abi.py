@@ -1,0 +1,59 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads without a
+GPU and exports every symbol include/n2d2hip.h declares; argument validation
+that needs no device works."""
+import ctypes as C
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "n2d2hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(n2d2hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from n2d2_amd import capi
+    names = _declared()
+    assert len(names) >= 25
+    assert sorted(capi.SYMBOLS) == names          # the binding lists exactly the header's entry points
+    for n in names:
+        assert hasattr(capi.lib, n), n
+
+
+def test_status_strings_and_host_only_helpers():
+    from n2d2_amd import capi
+    lib = capi.lib
+    assert lib.n2d2hip_strerror(0) == b"success"
+    assert b"quantized network" in lib.n2d2hip_strerror(capi.ERR_NOT_QUANTIZED)
+    assert b"gfx950" in lib.n2d2hip_version()
+    assert [capi.nhwc_cs(c) for c in (1, 3, 4, 6, 16, 17, 64, 1000)] == [4, 4, 4, 16, 16, 32, 64, 1008]
+    # output-size formulas (ConvCell::setOutputsDims / PoolCell::setOutputsDims)
+    oh, ow = C.c_int(), C.c_int()
+    d = capi.ConvDesc(3, 64, 7, 7, 2, 2, 3, 3, 3, 3, 1, 1, 1, 8)
+    assert lib.n2d2hip_conv_out_dims(C.byref(d), 224, 224, C.byref(oh), C.byref(ow)) == 0 and (oh.value, ow.value) == (112, 112)
+    p = capi.PoolDesc(capi.POOL_MAX, 3, 3, 2, 2, 0, 0)
+    assert lib.n2d2hip_pool_out_dims(C.byref(p), 112, 112, C.byref(oh), C.byref(ow)) == 0 and (oh.value, ow.value) == (55, 55)
+    p = capi.PoolDesc(capi.POOL_MAX, 3, 3, 2, 2, 1, 1)
+    assert lib.n2d2hip_pool_out_dims(C.byref(p), 112, 112, C.byref(oh), C.byref(ow)) == 0 and (oh.value, ow.value) == (56, 56)
+
+
+def test_invalid_arguments_are_rejected_before_any_device_work():
+    from n2d2_amd import capi
+    lib = capi.lib
+    h = C.c_void_p()
+    assert lib.n2d2hip_act_create(None, 4, C.byref(h)) == capi.ERR_INVALID
+    a = capi.Activation(capi.ACT_LINEAR, 0.0, capi.SCALING_SINGLE_SHIFT, None, 0, 0, None, 8, 0)
+    assert lib.n2d2hip_act_create(C.byref(a), 4, C.byref(h)) == capi.ERR_INVALID          # null scaling vector
+    assert b"null scaling" in lib.n2d2hip_last_error()
+    shifts = (C.c_ubyte * 4)(1, 2, 3, 4)
+    a = capi.Activation(capi.ACT_LINEAR, 0.0, capi.SCALING_SINGLE_SHIFT, C.cast(shifts, C.c_void_p), 0, 0, None, 0, 0)
+    assert lib.n2d2hip_act_create(C.byref(a), 4, C.byref(h)) == capi.ERR_NOT_QUANTIZED   # the reference throws here
+    assert b"SingleShiftScaling::propagate can only be used on quantized network." in lib.n2d2hip_last_error()
+    a = capi.Activation(capi.ACT_LINEAR, 0.0, 9, None, 0, 0, None, 8, 0)
+    assert lib.n2d2hip_act_create(C.byref(a), 4, C.byref(h)) == capi.ERR_INVALID
+    assert b"Unsupported scaling propagation" in lib.n2d2hip_last_error()
+    assert lib.n2d2hip_conv_forward(None, None, None, None) == capi.ERR_INVALID
+    assert lib.n2d2hip_convert(None, None, None) == capi.ERR_INVALID

@@ -1,0 +1,322 @@
+"""GPU parity of the integer cells: every result is compared bit-for-bit with
+the CPU oracle on the same seeded inputs, calling through the C ABI."""
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(2024)
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from n2d2_amd import runtime
+    return runtime
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def _u8(shape):
+    return RNG.integers(0, 256, size=shape).astype(np.int32)
+
+
+def _i8(shape, lo=-127, hi=127):
+    return RNG.integers(lo, hi + 1, size=shape).astype(np.int32)
+
+
+def _acts(O, bits=8):
+    """One activation spec per rescale mode / signedness, with per-channel parameters."""
+    from cells_ref import ActSpec
+    hi = 2 ** bits
+    return {
+        "none_linear": ActSpec("Linear", "None"),
+        "none_relu": ActSpec("Rectifier", "None"),
+        "sshift_relu_u": ActSpec("Rectifier", "SingleShift", RNG.integers(8, 13, size=O), nb_bits=bits, unsigned_out=True),
+        "sshift_lin_s": ActSpec("Linear", "SingleShift", RNG.integers(7, 12, size=O), nb_bits=bits, unsigned_out=False),
+        "dshift_relu_u": ActSpec("Rectifier", "DoubleShift", np.stack([RNG.integers(0, 6, size=O), RNG.integers(9, 15, size=O)], 1),
+                                 nb_bits=bits, unsigned_out=True),
+        "dshift_lin_s": ActSpec("Linear", "DoubleShift", np.stack([RNG.integers(1, 4, size=O), RNG.integers(10, 14, size=O)], 1),
+                                nb_bits=bits, unsigned_out=False),
+        "fixed_relu_u": ActSpec("Rectifier", "FixedMult32", RNG.integers(2 ** 14, 2 ** 15, size=O), frac_bits=24,
+                                nb_bits=bits, unsigned_out=True),
+        "fixed_clip_s": ActSpec("Linear", "FixedMult16", RNG.integers(2 ** 10, 2 ** 12, size=O), frac_bits=20,
+                                clipping=RNG.uniform(2000.0, 60000.0, size=O).astype(np.float32), nb_bits=bits, unsigned_out=False),
+        "fixed_wide": ActSpec("Linear", "FixedMult32", RNG.integers(2 ** 28, 2 ** 30, size=O), frac_bits=40,
+                              nb_bits=bits, unsigned_out=False),                    # needs the 64-bit product
+        "fixed_neg": ActSpec("Linear", "FixedMult32", -RNG.integers(2 ** 10, 2 ** 12, size=O), frac_bits=20,
+                             nb_bits=bits, unsigned_out=False),                     # negative multiplier
+        "float_relu_u": ActSpec("Rectifier", "FloatMult", RNG.uniform(2e-4, 4e-3, size=O).astype(np.float32),
+                                nb_bits=bits, unsigned_out=True),
+        "float_clip_s": ActSpec("Linear", "FloatMult", RNG.uniform(2e-4, 4e-3, size=O).astype(np.float32),
+                                clipping=np.where(RNG.random(O) < 0.5, 30000.5, -20000.0).astype(np.float32),
+                                nb_bits=bits, unsigned_out=False),
+    }
+
+
+# ------------------------------------------------------------ conversion
+
+def test_convert_round_trips(rt):
+    from n2d2_amd import capi
+    for Cc in (3, 16, 20, 64):
+        x = _u8((2, Cc, 5, 7))
+        for dt, vals in ((capi.U8B, x), (capi.U8, x), (capi.I8, x - 128), (capi.I32, x * 1000 - 7)):
+            for layout in (capi.NHWC, capi.NCHW):
+                t = rt.DTensor.from_numpy(vals, dt, layout)
+                assert np.array_equal(t.to_numpy(), vals), (Cc, dt, layout)
+        # F32 graph edge
+        t = rt.DTensor.from_numpy(x.astype(np.float32), capi.U8B)
+        assert np.array_equal(t.to_numpy(), x)
+    # raw NHWC U8B bytes: value - 128, channel fastest, padded channels hold logical zero
+    x = _u8((1, 3, 2, 2))
+    raw = rt.DTensor.from_numpy(x, capi.U8B).raw().reshape(1, 2, 2, 4)
+    assert np.array_equal(raw[..., :3].astype(np.int64) + 128, x.transpose(0, 2, 3, 1))
+    assert (raw[..., 3] == -128).all()
+
+
+# --------------------------------------------------------------- scaling
+
+@pytest.mark.parametrize("layout", ["NHWC", "NCHW"])
+def test_scaling_cell_all_modes(rt, layout):
+    from n2d2_amd import capi
+    lay = capi.NHWC if layout == "NHWC" else capi.NCHW
+    Cc = 24
+    acc = RNG.integers(-200000, 200001, size=(3, Cc, 6, 5)).astype(np.int32)
+    acc[0, :, 0, 0] = 2 ** 24 - 1
+    acc[0, :, 0, 1] = -(2 ** 24 - 1)
+    acc[0, :, 0, 2] = 0
+    for name, spec in _acts(Cc).items():
+        _say("scaling %s %s" % (layout, name))
+        act = rt.Act(Cc, **spec.kwargs())
+        x = rt.DTensor.from_numpy(acc, capi.I32, lay)
+        got = rt.scaling_forward(act, x).to_numpy()
+        want = spec.apply(acc.astype(np.float32))
+        assert np.array_equal(got, want.astype(np.int64)), name
+    for bits, uns in ((4, True), (4, False)):
+        spec = _acts(Cc, bits)["sshift_relu_u" if uns else "dshift_lin_s"]
+        act = rt.Act(Cc, **spec.kwargs())
+        got = rt.scaling_forward(act, rt.DTensor.from_numpy(acc, capi.I32, lay)).to_numpy()
+        assert np.array_equal(got, spec.apply(acc.astype(np.float32)).astype(np.int64))
+        assert got.max() <= (15 if uns else 7)
+
+
+def test_scaling_on_byte_inputs_is_the_residual_branch_rescale(rt):
+    from n2d2_amd import capi
+    from cells_ref import ActSpec
+    Cc = 32
+    x = _i8((2, Cc, 7, 7), -128, 127)
+    spec = ActSpec("Linear", "FixedMult16", RNG.integers(2 ** 13, 2 ** 15, size=Cc), frac_bits=14, nb_bits=8, unsigned_out=False)
+    act = rt.Act(Cc, **spec.kwargs())
+    got = rt.scaling_forward(act, rt.DTensor.from_numpy(x, capi.I8)).to_numpy()
+    assert np.array_equal(got, spec.apply(x.astype(np.float32)).astype(np.int64))
+
+
+def test_error_behaviour_matches_reference(rt):
+    from n2d2_amd import capi
+    with pytest.raises(capi.N2D2HipError) as e:
+        rt.Act(4, "Linear", "SingleShift", [1, 1, 1, 1], nb_bits=0)
+    assert e.value.status == capi.ERR_NOT_QUANTIZED and "can only be used on quantized network" in str(e.value)
+    with pytest.raises(capi.N2D2HipError):
+        rt.Act(4, "Rectifier", "SingleShift", [1, 1, 1, 1], leak_slope=0.1)
+    act = rt.Act(4, "Linear", "SingleShift", [1, 1, 1, 1], nb_bits=8, unsigned_out=False)
+    x = rt.DTensor.from_numpy(_u8((1, 5, 2, 2)), capi.I32)
+    with pytest.raises(capi.N2D2HipError):            # channel mismatch: nothing is written
+        rt.scaling_forward(act, x)
+    with pytest.raises(capi.N2D2HipError):            # signed range into an unsigned store
+        rt.scaling_forward(act, rt.DTensor.from_numpy(_u8((1, 4, 2, 2)), capi.I32), out_dtype=capi.U8B)
+
+
+# ------------------------------------------------------------------ conv
+
+CONV_CASES = [
+    # name, B, C, H, W, O, (kW,kH), (sx,sy), (L,T,R,B), (dx,dy), input kind
+    ("3x3_c64", 2, 64, 14, 14, 64, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
+    ("1x1_c64_o256", 3, 64, 9, 11, 256, (1, 1), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
+    ("1x1_s2", 2, 128, 14, 14, 96, (1, 1), (2, 2), (0, 0, 0, 0), (1, 1), "i8"),
+    ("3x3_s2_c32", 2, 32, 15, 17, 48, (3, 3), (2, 2), (1, 1, 1, 1), (1, 1), "u8"),
+    ("stem7x7_c3", 2, 3, 37, 41, 64, (7, 7), (2, 2), (3, 3, 3, 3), (1, 1), "u8"),
+    ("stem3x3_c3", 2, 3, 20, 20, 32, (3, 3), (2, 2), (1, 1, 1, 1), (1, 1), "u8"),
+    ("lenet5x5_c1", 4, 1, 32, 32, 6, (5, 5), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
+    ("lenet5x5_c6", 4, 6, 14, 14, 16, (5, 5), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
+    ("c20_o10_asym", 2, 20, 9, 8, 10, (2, 5), (1, 3), (1, 2, 0, 1), (1, 1), "i8"),
+    ("dilated_nopad", 2, 16, 17, 17, 16, (3, 3), (1, 1), (0, 0, 0, 0), (2, 3), "u8"),
+    ("dilated_pad_quirk", 2, 16, 12, 12, 16, (3, 3), (1, 3), (2, 2, 2, 2), (3, 3), "u8"),
+    ("big_k", 1, 512, 7, 7, 130, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
+    ("tall_m", 5, 16, 33, 31, 16, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=[c[0] for c in CONV_CASES])
+def test_conv_cell_bit_exact(rt, case):
+    from n2d2_amd import capi
+    import cells_ref
+    name, B, Cc, H, W, O, k, s, p, d, kind = case
+    x = _u8((B, Cc, H, W)) if kind == "u8" else _i8((B, Cc, H, W), -128, 127)
+    w = np.clip(np.rint(RNG.normal(0, 40, size=(O, Cc, k[1], k[0]))), -127, 127).astype(np.int32)
+    bias = RNG.integers(-4096, 4097, size=O).astype(np.int32)
+    in_dt = capi.U8B if kind == "u8" else capi.I8
+    xd = rt.DTensor.from_numpy(x, in_dt)
+    acts = _acts(O)
+    names = list(acts) if name in ("3x3_c64", "c20_o10_asym") else ["none_linear", "sshift_relu_u", "dshift_lin_s", "fixed_relu_u", "float_relu_u"]
+    for an in names:
+        spec = acts[an]
+        _say("conv %s %s" % (name, an))
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=s, pad=p, dil=d)
+        assert np.abs(want).max() < 2 ** 24
+        conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), in_dt, stride=s, pad=p, dil=d)
+        got = conv.forward(xd).to_numpy()
+        assert got.shape == want.shape
+        assert np.array_equal(got, want.astype(np.int64)), (name, an)
+    # NoBias
+    spec = acts["sshift_relu_u"]
+    conv = rt.Conv(w, None, rt.Act(O, **spec.kwargs()), in_dt, stride=s, pad=p, dil=d)
+    want = cells_ref.conv_cell(x, w, None, spec, stride=s, pad=p, dil=d)
+    assert np.array_equal(conv.forward(xd).to_numpy(), want.astype(np.int64))
+
+
+def test_conv_config2_resnet18_stage_single_shift(rt):
+    """3x3 s1 p1 64->64 on 56x56, uint8 input, N(0,40) weights, per-channel single shift in [8,12], ReLU clip [0,255];
+    the oracle runs a 4-image slice, the GPU the same slice."""
+    from n2d2_amd import capi
+    import cells_ref
+    from cells_ref import ActSpec
+    B = 4
+    x = _u8((B, 64, 56, 56))
+    w = np.clip(np.rint(RNG.normal(0, 40, size=(64, 64, 3, 3))), -127, 127).astype(np.int32)
+    spec = ActSpec("Rectifier", "SingleShift", RNG.integers(8, 13, size=64), nb_bits=8, unsigned_out=True)
+    want = cells_ref.conv_cell(x, w, None, spec, pad=(1, 1, 1, 1))
+    conv = rt.Conv(w, None, rt.Act(64, **spec.kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+    assert np.array_equal(got, want.astype(np.int64))
+    assert got.min() == 0 and got.max() == 255
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_depthwise_conv_bit_exact(rt, stride):
+    from n2d2_amd import capi
+    import cells_ref
+    Cc = 48
+    x = _u8((3, Cc, 13, 12))
+    w = _i8((Cc, 1, 3, 3))
+    bias = RNG.integers(-2000, 2001, size=Cc).astype(np.int32)
+    acts = _acts(Cc)
+    for an in ("fixed_relu_u", "sshift_lin_s", "none_linear", "float_relu_u"):
+        spec = acts[an]
+        if an == "fixed_relu_u":
+            spec.scaling = RNG.integers(2 ** 13, 2 ** 14, size=Cc)
+            spec.frac_bits = 18
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(1, 1, 1, 1), groups=Cc)
+        conv = rt.Conv(w, bias, rt.Act(Cc, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(1, 1, 1, 1), groups=Cc)
+        got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+        assert np.array_equal(got, want.astype(np.int64)), an
+
+
+def test_conv_int4_weights_uint4_activations(rt):
+    """Weights in [-7,7] nibble-packed, activations in [0,15], fixed-point rescale with clip, 4-bit unsigned output."""
+    from n2d2_amd import capi
+    import cells_ref
+    from cells_ref import ActSpec
+    for (Cc, O, k, s, p) in ((64, 64, 3, 1, 1), (64, 128, 3, 2, 1), (64, 128, 1, 2, 0), (32, 40, 5, 1, 2)):
+        x = RNG.integers(0, 16, size=(2, Cc, 14, 14)).astype(np.int32)
+        w = RNG.integers(-7, 8, size=(O, Cc, k, k)).astype(np.int32)
+        bias = RNG.integers(-300, 301, size=O).astype(np.int32)
+        spec = ActSpec("Rectifier", "FixedMult32", RNG.integers(300, 900, size=O), frac_bits=16,
+                       clipping=RNG.uniform(500.0, 3000.0, size=O).astype(np.float32), nb_bits=4, unsigned_out=True)
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(s, s), pad=(p, p, p, p))
+        conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(s, s), pad=(p, p, p, p), weight_bits=4)
+        got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+        assert np.array_equal(got, want.astype(np.int64)), (Cc, O, k, s)
+        assert got.max() <= 15 and len(np.unique(got)) > 4
+        # same weights through the 8-bit path give the same cell
+        conv8 = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(s, s), pad=(p, p, p, p))
+        assert np.array_equal(conv8.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), got)
+
+
+def test_conv_linearity_and_batch_independence_at_full_width(rt):
+    """Size-independent properties at a ResNet-50 layer shape (1x1, 256->64 on 56x56, batch 16): raw sums are additive in
+    the weights, and an image's result does not depend on its position in the batch."""
+    from n2d2_amd import capi
+    B, Cc, O, H = 16, 256, 64, 56
+    x = _u8((B, Cc, H, H))
+    x[5] = x[0]
+    w1 = _i8((O, Cc, 1, 1), -60, 60)
+    w2 = _i8((O, Cc, 1, 1), -60, 60)
+    xd = rt.DTensor.from_numpy(x, capi.U8B)
+    raw = lambda w: rt.Conv(w, None, rt.Act(O, "Linear", "None"), capi.U8B).forward(xd).to_numpy()
+    a, b, ab = raw(w1), raw(w2), raw(w1 + w2)
+    assert np.array_equal(a + b, ab)
+    assert np.array_equal(a[0], a[5])
+    ref = np.einsum("chw,oc->ohw", x[3].astype(np.int64), w1[:, :, 0, 0].astype(np.int64))
+    assert np.array_equal(a[3], ref)
+
+
+# -------------------------------------------------------------------- fc
+
+@pytest.mark.parametrize("shape", [(16, 5, 5, 120), (120, 1, 1, 84), (84, 1, 1, 10), (2048, 1, 1, 1000), (1, 6, 6, 20)])
+def test_fc_cell_bit_exact(rt, shape):
+    from n2d2_amd import capi
+    import cells_ref
+    Cc, H, W, O = shape
+    B = 9
+    x = _u8((B, Cc, H, W))
+    w = np.clip(np.rint(RNG.normal(0, 30, size=(O, Cc * H * W))), -127, 127).astype(np.int32)
+    bias = RNG.integers(-4096, 4097, size=O).astype(np.int32)
+    acts = _acts(O)
+    for an in ("none_linear", "fixed_relu_u", "dshift_lin_s"):
+        spec = acts[an]
+        want = cells_ref.fc_cell(x, w, bias, spec)
+        assert np.abs(want).max() < 2 ** 24
+        fc = rt.Fc(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, (Cc, H, W))
+        got = fc.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+        assert np.array_equal(got, want.astype(np.int64)), an
+
+
+# ------------------------------------------------------------------ pool
+
+@pytest.mark.parametrize("kind,pool,stride,pad", [("max", (2, 2), (2, 2), (0, 0)), ("max", (3, 3), (2, 2), (0, 0)),
+                                                  ("max", (3, 3), (2, 2), (1, 1)), ("avg", (7, 7), (7, 7), (0, 0)),
+                                                  ("avg", (3, 3), (2, 2), (1, 1)), ("avg", (2, 2), (2, 2), (0, 0))])
+def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
+    from n2d2_amd import capi
+    import cells_ref
+    for dt, x in ((capi.U8B, _u8((3, 24, 14, 15))), (capi.I8, _i8((3, 24, 14, 15), -128, 127)), (capi.U8, _u8((2, 3, 14, 14)))):
+        want = cells_ref.pool_cell(x, kind, pool, stride, pad)
+        got = rt.Pool(kind, pool, stride, pad).forward(rt.DTensor.from_numpy(x, dt)).to_numpy()
+        assert np.array_equal(got, want.astype(np.int64)), (kind, dt)
+
+
+# -------------------------------------------------------------- elemwise
+
+def test_elemwise_sum_cell_bit_exact(rt):
+    from n2d2_amd import capi
+    import cells_ref
+    from cells_ref import ActSpec
+    Cc = 40
+    a, b, c = _u8((2, Cc, 7, 9)), _i8((2, Cc, 7, 9), -128, 127), _u8((2, Cc, 7, 9))
+    da, db, dc = rt.DTensor.from_numpy(a, capi.U8B), rt.DTensor.from_numpy(b, capi.I8), rt.DTensor.from_numpy(c, capi.U8B)
+    acts = _acts(Cc)
+    # residual add as PTQ leaves it: unit weights, zero shifts, rescale in the activation
+    for an, spec in (("dshift", ActSpec("Rectifier", "DoubleShift", np.stack([RNG.integers(0, 3, size=Cc), RNG.integers(1, 4, size=Cc)], 1),
+                                        nb_bits=8, unsigned_out=True)),
+                     ("fixed", ActSpec("Rectifier", "FixedMult16", RNG.integers(2 ** 12, 2 ** 14, size=Cc), frac_bits=14, nb_bits=8, unsigned_out=True)),
+                     ("float", ActSpec("Linear", "FloatMult", RNG.uniform(0.2, 0.9, size=Cc).astype(np.float32), nb_bits=8, unsigned_out=False)),
+                     ("none", acts["none_relu"])):
+        want = cells_ref.elemwise_cell([a, b], spec)
+        ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **spec.kwargs()))
+        assert np.array_equal(ew.forward([da, db]).to_numpy(), want.astype(np.int64)), an
+    # general coefficients, three inputs, float arithmetic as the reference
+    spec = ActSpec("Linear", "FixedMult16", RNG.integers(2 ** 10, 2 ** 12, size=Cc), frac_bits=13, nb_bits=8, unsigned_out=False)
+    w = np.array([1.5, -0.75, 2.0], dtype=np.float32)
+    s = np.array([3.0, -10.5, 0.25], dtype=np.float32)
+    want = cells_ref.elemwise_cell([a, b, c], spec, w, s, "PerInput")
+    ew = rt.ElemWiseSum(3, Cc, rt.Act(Cc, **spec.kwargs()), w, s, "PerInput")
+    assert np.array_equal(ew.forward([da, db, dc]).to_numpy(), want.astype(np.int64))
+    wc = RNG.uniform(-2, 2, size=Cc).astype(np.float32)
+    sc = RNG.uniform(-20, 20, size=Cc).astype(np.float32)
+    want = cells_ref.elemwise_cell([a, b], spec, wc, sc, "PerChannel")
+    ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **spec.kwargs()), wc, sc, "PerChannel")
+    assert np.array_equal(ew.forward([da, db]).to_numpy(), want.astype(np.int64))
