@@ -1,0 +1,413 @@
+"""Synthetic quantized networks (the benchmark configurations) and their
+execution through the C ABI.
+
+A network is a layer-ordered list of cells as N2D2's post-training quantization
+leaves them: integer weights and biases, a Scaling in each activation, stand-alone
+ScalingCells on residual shortcuts, ElemWise sums with unit weights.  Parameters
+are seeded random draws; the per-layer rescale magnitudes are calibrated on one
+image with numpy so that activations keep a healthy dynamic range through the
+depth of the net (a stand-in for N2D2's calibration pass, not part of inference).
+"""
+import math
+
+import numpy as np
+
+
+class ActDesc:
+    """Activation of a cell: kind, Scaling parameters, bits and signedness."""
+
+    def __init__(self, kind="Linear", mode="None", scaling=None, frac_bits=0, clipping=None, nb_bits=8, unsigned_out=False):
+        self.kind, self.mode, self.scaling, self.frac_bits = kind, mode, scaling, frac_bits
+        self.clipping, self.nb_bits, self.unsigned_out = clipping, nb_bits, unsigned_out
+
+    def kwargs(self):
+        return dict(kind=self.kind, mode=self.mode, scaling=self.scaling, frac_bits=self.frac_bits,
+                    clipping=self.clipping, nb_bits=self.nb_bits, unsigned_out=self.unsigned_out)
+
+    def bounds(self):
+        if self.unsigned_out:
+            lo, hi = 0, (1 << self.nb_bits) - 1
+        else:
+            lo, hi = -(1 << (self.nb_bits - 1)), (1 << (self.nb_bits - 1)) - 1
+        if self.kind == "Rectifier":
+            lo = max(lo, 0)
+        return lo, hi
+
+    def apply_np(self, acc, channel_axis=1):
+        """Exact integer form of the rescale on an int64 array (calibration only)."""
+        if self.mode == "None":
+            return np.maximum(acc, 0) if self.kind == "Rectifier" else acc
+        shape = [1] * acc.ndim
+        shape[channel_axis] = -1
+        v = acc.astype(np.int64)
+        if self.clipping is not None and self.mode in ("FixedMult16", "FixedMult32", "FloatMult"):
+            cl = np.rint(np.asarray(self.clipping, dtype=np.float64)).astype(np.int64).reshape(shape)
+            v = np.where(cl > 0, np.clip(v, 0, np.maximum(cl, 0)), np.clip(v, np.minimum(cl, 0), 0))
+        if self.mode == "FloatMult":
+            r = v.astype(np.float32) * np.asarray(self.scaling, dtype=np.float32).reshape(shape)
+            r = (np.sign(r) * np.floor(np.abs(r.astype(np.float64)) + 0.5)).astype(np.int64)
+        else:
+            if self.mode == "SingleShift":
+                m = np.ones(len(self.scaling), dtype=np.int64)
+                p = np.asarray(self.scaling, dtype=np.int64)
+            elif self.mode == "DoubleShift":
+                s = np.asarray(self.scaling, dtype=np.int64).reshape(-1, 2)
+                m = 1 + (1 << s[:, 0])
+                p = s[:, 1]
+            else:
+                m = np.asarray(self.scaling, dtype=np.int64)
+                p = np.full(len(m), self.frac_bits, dtype=np.int64)
+            half = np.where(p > 0, 1 << np.maximum(p - 1, 0), 0)
+            r = (v * m.reshape(shape) + half.reshape(shape)) >> p.reshape(shape)
+        lo, hi = self.bounds()
+        return np.clip(r, lo, hi)
+
+
+class Layer:
+    def __init__(self, name, type_, inputs, **kw):
+        self.name, self.type, self.inputs = name, type_, inputs
+        self.__dict__.update(kw)
+
+
+class NetSpec:
+    def __init__(self, name, in_shape, input_unsigned=True):
+        self.name, self.in_shape, self.input_unsigned = name, in_shape, input_unsigned
+        self.layers = []
+        self.shapes = {"input": in_shape}
+        self.unsigned = {"input": input_unsigned}
+
+    def add(self, layer, out_shape, unsigned_out):
+        layer.out_shape = out_shape
+        layer.unsigned_out = unsigned_out
+        self.layers.append(layer)
+        self.shapes[layer.name] = out_shape
+        self.unsigned[layer.name] = unsigned_out
+        return layer.name
+
+    @property
+    def output(self):
+        return self.layers[-1].name
+
+    def macs_per_image(self):
+        total = 0
+        for l in self.layers:
+            if l.type == "conv":
+                O, Cg, kH, kW = l.w.shape
+                total += l.out_shape[1] * l.out_shape[2] * O * Cg * kH * kW
+            elif l.type == "fc":
+                total += l.w.size
+        return total
+
+    def conv_macs_per_image(self):
+        return sum(l.out_shape[1] * l.out_shape[2] * l.w.size for l in self.layers if l.type == "conv" and l.groups == 1)
+
+
+# ------------------------------------------------------------ numpy helpers (calibration only)
+
+def _out_dim(n, k, s, p0, p1, d=1):
+    return int((n + p0 + p1 - d * (k - 1) - 1 + s) / float(s))
+
+
+def _conv_acc_np(x, w, stride, pad, groups):
+    """x [C,H,W] ints, w [O,C/g,kH,kW]; zero-padded correlation through im2col + BLAS (exact in float64)."""
+    C, H, W = x.shape
+    O, Cg, kH, kW = w.shape
+    sx, sy = stride
+    oH, oW = _out_dim(H, kH, sy, pad[1], pad[3]), _out_dim(W, kW, sx, pad[0], pad[2])
+    xp = np.zeros((C, H + pad[1] + pad[3] + kH, W + pad[0] + pad[2] + kW), dtype=np.float64)
+    xp[:, pad[1]:pad[1] + H, pad[0]:pad[0] + W] = x
+    out = np.empty((O, oH, oW), dtype=np.float64)
+    og = O // groups
+    for g in range(groups):
+        cols = np.empty((Cg, kH, kW, oH, oW), dtype=np.float64)
+        for ky in range(kH):
+            for kx in range(kW):
+                cols[:, ky, kx] = xp[g * Cg:(g + 1) * Cg, ky:ky + sy * (oH - 1) + 1:sy, kx:kx + sx * (oW - 1) + 1:sx]
+        out[g * og:(g + 1) * og] = (w[g * og:(g + 1) * og].reshape(og, -1).astype(np.float64)
+                                    @ cols.reshape(Cg * kH * kW, oH * oW)).reshape(og, oH, oW)
+    return np.rint(out).astype(np.int64)
+
+
+def _pool_np(x, kind, pool, stride, pad):
+    C, H, W = x.shape
+    oH = int((H + 2 * pad[1] - pool[1] + stride[1]) / float(stride[1]))
+    oW = int((W + 2 * pad[0] - pool[0] + stride[0]) / float(stride[0]))
+    out = np.zeros((C, oH, oW), dtype=np.int64)
+    for oy in range(oH):
+        for ox in range(oW):
+            y0, x0 = oy * stride[1] - pad[1], ox * stride[0] - pad[0]
+            win = x[:, max(y0, 0):min(y0 + pool[1], H), max(x0, 0):min(x0 + pool[0], W)]
+            if kind == "max":
+                out[:, oy, ox] = win.max(axis=(1, 2))
+            else:
+                s = win.sum(axis=(1, 2))
+                out[:, oy, ox] = np.sign(s) * (np.abs(s) // (pool[0] * pool[1]))
+    return out
+
+
+class _Builder:
+    """Adds cells to a NetSpec while pushing one calibration image through them."""
+
+    def __init__(self, name, in_shape, seed, scaling_mode, nb_bits=8, unsigned_data=True, frac_bits=16):
+        self.rng = np.random.default_rng(seed)
+        self.spec = NetSpec(name, in_shape, input_unsigned=True)
+        self.mode, self.nb_bits, self.unsigned_data, self.frac_bits = scaling_mode, nb_bits, unsigned_data, frac_bits
+        self.values = {"input": self.rng.integers(0, 256, size=in_shape).astype(np.int64)}
+
+    # per-channel Scaling parameters approximating the float factors s (one per channel)
+    def _scaling_params(self, s, mode=None):
+        mode = mode or self.mode
+        if mode == "SingleShift":
+            return np.clip(np.rint(-np.log2(s)), 0, 31).astype(np.uint8), 0
+        if mode == "DoubleShift":
+            best = None
+            for a in range(0, 5):
+                b = np.clip(np.rint(np.log2((1 + 2.0 ** a) / s)), 0, 31)
+                err = np.abs((1 + 2.0 ** a) / 2.0 ** b - s) / s
+                if best is None:
+                    best = (np.full(len(s), a), b, err)
+                else:
+                    take = err < best[2]
+                    best = (np.where(take, a, best[0]), np.where(take, b, best[1]), np.where(take, err, best[2]))
+            return np.stack([best[0], best[1]], 1).astype(np.uint8), 0
+        if mode in ("FixedMult16", "FixedMult32"):
+            p = self.frac_bits
+            return np.maximum(np.rint(s * 2.0 ** p), 1).astype(np.int32), p
+        return s.astype(np.float32), 0
+
+    def _make_act(self, acc, kind, O, nb_bits=None, mode=None, clip=False, target=None):
+        nb_bits = nb_bits or self.nb_bits
+        mode = mode or self.mode
+        unsigned = self.unsigned_data and kind == "Rectifier"
+        if mode == "None":
+            return ActDesc(kind, "None", nb_bits=nb_bits, unsigned_out=unsigned)
+        full = (1 << nb_bits) - 1 if unsigned else (1 << (nb_bits - 1)) - 1
+        target = target or 0.8 * full
+        ref = max(float(np.percentile(np.abs(acc), 99.5)), 1.0)
+        s = (target / ref) * self.rng.uniform(0.75, 1.3, size=O)
+        scaling, frac = self._scaling_params(s, mode)
+        clipping = None
+        if clip:
+            clipping = (ref * self.rng.uniform(0.9, 1.6, size=O)).astype(np.float32)
+        return ActDesc(kind, mode, scaling, frac, clipping, nb_bits, unsigned)
+
+    def _weights(self, shape, wstd, wmax, uniform):
+        if uniform:
+            return self.rng.integers(-wmax, wmax + 1, size=shape).astype(np.int8)
+        return np.clip(np.rint(self.rng.normal(0, wstd, size=shape)), -wmax, wmax).astype(np.int8)
+
+    def conv(self, name, inp, O, k, stride=1, pad=0, kind="Rectifier", groups=1, wstd=30.0, wmax=127, weight_bits=8,
+             bias=True, nb_bits=None, mode=None, clip=False, uniform=False):
+        C, H, W = self.spec.shapes[inp]
+        w = self._weights((O, C // groups, k, k), wstd, wmax, uniform)
+        p4 = (pad, pad, pad, pad)
+        acc = _conv_acc_np(self.values[inp], w.astype(np.int64), (stride, stride), p4, groups)
+        b = None
+        if bias:
+            mag = max(int(np.percentile(np.abs(acc), 90) / 4), 16)
+            b = self.rng.integers(-mag, mag + 1, size=O).astype(np.int32)
+            acc = acc + b[:, None, None]
+        act = self._make_act(acc, kind, O, nb_bits, mode, clip)
+        self.values[name] = act.apply_np(acc, 0)
+        l = Layer(name, "conv", [inp], w=w, bias=b, stride=(stride, stride), pad=p4, dil=(1, 1), groups=groups,
+                  weight_bits=weight_bits, act=act)
+        return self.spec.add(l, (O,) + acc.shape[1:], act.unsigned_out)
+
+    def fc(self, name, inp, O, kind="Linear", wstd=30.0, wmax=127, weight_bits=8, mode=None, nb_bits=None, uniform=False):
+        C, H, W = self.spec.shapes[inp]
+        w = self._weights((O, C * H * W), wstd, wmax, uniform)
+        acc = w.astype(np.int64) @ self.values[inp].reshape(-1)
+        mag = max(int(np.percentile(np.abs(acc), 90) / 4), 16)
+        b = self.rng.integers(-mag, mag + 1, size=O).astype(np.int32)
+        acc = (acc + b).reshape(O, 1, 1)
+        act = self._make_act(acc, kind, O, nb_bits, mode)
+        self.values[name] = act.apply_np(acc, 0)
+        l = Layer(name, "fc", [inp], w=w, bias=b, weight_bits=weight_bits, act=act)
+        return self.spec.add(l, (O, 1, 1), act.unsigned_out)
+
+    def pool(self, name, inp, kind, pool, stride, pad=0):
+        v = _pool_np(self.values[inp], kind, (pool, pool), (stride, stride), (pad, pad))
+        self.values[name] = v
+        l = Layer(name, "pool", [inp], kind=kind, pool=(pool, pool), stride=(stride, stride), pad=(pad, pad))
+        # no activation: range of the parents (PoolCell::getOutputsRange)
+        return self.spec.add(l, v.shape, self.spec.unsigned[inp])
+
+    def scaling(self, name, inp, frac_bits=14):
+        """Stand-alone ScalingCell as `_rescale_branch` leaves it: FIXED_MULT16, factor <= 1, no activation."""
+        C = self.spec.shapes[inp][0]
+        s = self.rng.uniform(0.55, 1.0, size=C)
+        mult = np.maximum(np.rint(s * 2.0 ** frac_bits), 1).astype(np.int32)
+        # ScalingCell::getOutputsRange: unsigned iff the parent is and every factor is >= 0
+        unsigned = self.spec.unsigned[inp]
+        act = ActDesc("Linear", "FixedMult16", mult, frac_bits, None, self.nb_bits, unsigned)
+        self.values[name] = act.apply_np(self.values[inp], 0)
+        return self.spec.add(Layer(name, "scaling", [inp], act=act), self.spec.shapes[inp], unsigned)
+
+    def sum(self, name, inps, kind="Rectifier", nb_bits=None):
+        acc = sum(self.values[i] for i in inps)
+        C = acc.shape[0]
+        act = self._make_act(acc, kind, C, nb_bits, target=None)
+        self.values[name] = act.apply_np(acc, 0)
+        l = Layer(name, "elemwise", list(inps), act=act, weights=None, shifts=None, coeff_mode="PerLayer")
+        return self.spec.add(l, acc.shape, act.unsigned_out)
+
+
+# --------------------------------------------------------------- the configurations
+
+def lenet(seed=1):
+    """LeNet-style 8-bit PTQ net: 1x32x32 u8, conv 6@5x5, maxpool 2, conv 16@5x5, maxpool 2, FC 120-84-10;
+    weights U[-127,127], per-layer fixed-point rescale with shift 20, integer logits."""
+    b = _Builder("lenet", (1, 32, 32), seed, "FixedMult32", frac_bits=20)
+    x = b.conv("conv1", "input", 6, 5, uniform=True)
+    x = b.pool("pool1", x, "max", 2, 2)
+    x = b.conv("conv2", x, 16, 5, uniform=True)
+    x = b.pool("pool2", x, "max", 2, 2)
+    x = b.fc("fc1", x, 120, kind="Rectifier", uniform=True)
+    x = b.fc("fc2", x, 84, kind="Rectifier", uniform=True)
+    b.fc("fc3", x, 10, kind="Linear", uniform=True, mode="None")
+    return b.spec
+
+
+def resnet50(seed=4, pool_pad=1, unsigned_data=True, image=224):
+    """ResNet-50, 8-bit PTQ: 7x7 s2 stem, 3x3 s2 max-pool (pad 1 -> 56x56; pad 0 is N2D2's own model file),
+    bottlenecks [3,4,6,3] with the stride in the 3x3, per-channel double-shift rescales, FIXED_MULT16 ScalingCells
+    on identity shortcuts, ElemWise sums, global average pool, FC 1000 with raw int32 logits."""
+    b = _Builder("resnet50", (3, image, image), seed, "DoubleShift", unsigned_data=unsigned_data)
+    x = b.conv("conv1", "input", 64, 7, 2, 3)
+    x = b.pool("pool1", x, "max", 3, 2, pool_pad)
+    stage = 2
+    for nf, blocks, stride in ((64, 3, 1), (128, 4, 2), (256, 6, 2), (512, 3, 2)):
+        for i in range(blocks):
+            n = "conv%d.%d" % (stage, i + 1)
+            s = stride if i == 0 else 1
+            y = b.conv(n + "_1x1", x, nf, 1)
+            y = b.conv(n + "_3x3", y, nf, 3, s, 1)
+            y = b.conv(n + "_1x1_x4", y, 4 * nf, 1, kind="Linear")
+            if i == 0:
+                sc = b.conv(n + "_1x1_proj", x, 4 * nf, 1, s, 0, kind="Linear")
+            else:
+                sc = b.scaling(n + "_shortcut_rescale", x)
+            x = b.sum(n + "_sum", [y, sc])
+        stage += 1
+    C, H, W = b.spec.shapes[x]
+    x = b.pool("pool", x, "avg", H, H)
+    b.fc("fc", x, 1000, mode="None")
+    return b.spec
+
+
+def mobilenet_v1(seed=3, image=224):
+    """MobileNet-v1 1.0, 8-bit PTQ: 3x3 s2 stem, 13 depthwise 3x3 + pointwise 1x1 blocks, per-channel fixed-point
+    rescale (one shift per cell), ReLU6 == saturation at 255, global average pool, FC 1000."""
+    b = _Builder("mobilenet_v1", (3, image, image), seed, "FixedMult32", frac_bits=16)
+    x = b.conv("conv1", "input", 32, 3, 2, 1)
+    cfg = [(64, 1), (128, 2), (128, 1), (256, 2), (256, 1), (512, 2), (512, 1), (512, 1), (512, 1), (512, 1), (512, 1),
+           (1024, 2), (1024, 1)]
+    for i, (O, s) in enumerate(cfg):
+        C = b.spec.shapes[x][0]
+        b.frac_bits = 16 + (i % 9)
+        x = b.conv("conv%d_dw" % (i + 2), x, C, 3, s, 1, groups=C, wstd=50.0)
+        x = b.conv("conv%d_pw" % (i + 2), x, O, 1)
+    C, H, W = b.spec.shapes[x]
+    x = b.pool("pool", x, "avg", H, H)
+    b.fc("fc", x, 1000, mode="None")
+    return b.spec
+
+
+def resnet18_w4a4(seed=5, image=224):
+    """ResNet-18 with 4-bit weights in [-7,7] (nibble-packed) and 4-bit activations in [0,15] as the SAT export
+    leaves it: per-channel fixed-point rescale (16 fractional bits) with clipping; first and last layer 8-bit."""
+    b = _Builder("resnet18_w4a4", (3, image, image), seed, "FixedMult32", frac_bits=16)
+    x = b.conv("conv1", "input", 64, 7, 2, 3, nb_bits=4, clip=True)          # 8-bit weights, 4-bit activations out
+    x = b.pool("pool1", x, "max", 3, 2, 1)
+    stage = 2
+    for nf, stride in ((64, 1), (128, 2), (256, 2), (512, 2)):
+        for i in range(2):
+            n = "conv%d.%d" % (stage, i + 1)
+            s = stride if i == 0 else 1
+            y = b.conv(n + "_a", x, nf, 3, s, 1, wstd=3.0, wmax=7, weight_bits=4, nb_bits=4, clip=True)
+            y = b.conv(n + "_b", y, nf, 3, 1, 1, kind="Linear", wstd=3.0, wmax=7, weight_bits=4, nb_bits=4, clip=True)
+            if s != 1 or b.spec.shapes[x][0] != nf:
+                sc = b.conv(n + "_proj", x, nf, 1, s, 0, kind="Linear", wstd=3.0, wmax=7, weight_bits=4, nb_bits=4, clip=True)
+            else:
+                sc = x
+            x = b.sum(n + "_sum", [y, sc], nb_bits=4)
+        stage += 1
+    C, H, W = b.spec.shapes[x]
+    x = b.pool("pool", x, "avg", H, H)
+    b.fc("fc", x, 1000, mode="None")
+    return b.spec
+
+
+def single_conv_stage(seed=2):
+    """One ResNet-18 stage conv: 3x3 s1 p1 64->64 on 56x56, u8 input, N(0,40) weights, per-channel single shift in
+    [8,12], ReLU clip [0,255]."""
+    spec = NetSpec("conv3x3_64", (64, 56, 56))
+    rng = np.random.default_rng(seed)
+    w = np.clip(np.rint(rng.normal(0, 40, size=(64, 64, 3, 3))), -127, 127).astype(np.int8)
+    act = ActDesc("Rectifier", "SingleShift", rng.integers(8, 13, size=64).astype(np.uint8), nb_bits=8, unsigned_out=True)
+    spec.add(Layer("conv", "conv", ["input"], w=w, bias=None, stride=(1, 1), pad=(1, 1, 1, 1), dil=(1, 1), groups=1,
+                   weight_bits=8, act=act), (64, 56, 56), True)
+    return spec
+
+
+# ------------------------------------------------------------------ execution on the GPU
+
+class GpuNet:
+    """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
+    Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
+
+    def __init__(self, spec, batch):
+        from . import capi, runtime as rt
+        self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
+        C, H, W = spec.in_shape
+        self.input = rt.DTensor(batch, C, H, W, capi.U8B if spec.input_unsigned else capi.I8)
+        self.tensors = {"input": self.input}
+        self.steps = []
+        for l in spec.layers:
+            ins = [self.tensors[i] for i in l.inputs]
+            Co, Ho, Wo = l.out_shape
+            if l.type in ("conv", "fc"):
+                act = rt.Act(Co, **l.act.kwargs())
+                if l.type == "conv":
+                    cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits)
+                else:
+                    cell = rt.Fc(l.w, l.bias, act, ins[0].dtype, (ins[0].C, ins[0].H, ins[0].W), l.weight_bits)
+                out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype())
+                self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
+            elif l.type == "pool":
+                cell = rt.Pool(l.kind, l.pool, l.stride, l.pad)
+                out = rt.DTensor(batch, Co, Ho, Wo, ins[0].dtype)
+                self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
+            elif l.type == "scaling":
+                cell = rt.Act(Co, **l.act.kwargs())
+                out = rt.DTensor(batch, Co, Ho, Wo, cell.out_dtype())
+                self.steps.append((l, cell, (lambda c, i, o: rt.check(rt.lib.n2d2hip_scaling_forward(c.handle, i[0].ref, o.ref, rt.stream_ptr())))))
+            elif l.type == "elemwise":
+                act = rt.Act(Co, **l.act.kwargs())
+                cell = rt.ElemWiseSum(len(ins), Co, act, l.weights, l.shifts, l.coeff_mode)
+                out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype())
+                self.steps.append((l, cell, (lambda c, i, o: c.forward(i, o))))
+            else:
+                raise ValueError(l.type)
+            self.tensors[l.name] = out
+        self._io = [([self.tensors[i] for i in l.inputs], self.tensors[l.name]) for l in spec.layers]
+
+    def set_input(self, x):
+        """x: integer NCHW numpy array [B,C,H,W]."""
+        t = self.rt.DTensor.from_numpy(x, self.input.dtype)
+        self.input.buf.copy_(t.buf)
+
+    def forward(self):
+        for (l, cell, fn), (ins, out) in zip(self.steps, self._io):
+            fn(cell, ins, out)
+        return self.tensors[self.spec.output]
+
+    def activation_bytes(self):
+        """Algorithmic HBM bytes of one forward: every cell reads its inputs and writes its output once, plus weights."""
+        total = 0
+        for l, (ins, out) in zip(self.spec.layers, self._io):
+            total += sum(t.B * t.C * t.H * t.W * (4 if t.dtype == self.capi.I32 else 1) for t in ins)
+            total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
+            if l.type in ("conv", "fc"):
+                total += l.w.size // (2 if l.weight_bits == 4 else 1)
+        return total

@@ -3,7 +3,7 @@ cells call their kernels (ConvCell_Frame::propagate, FcCell_Frame::propagate,
 Cell_Frame::propagate -> Activation::propagate -> Scaling::propagate)."""
 import numpy as np
 
-from oracle import oracle as orc
+from . import oracle as orc
 
 
 class ActSpec:
@@ -69,3 +69,38 @@ def elemwise_cell(xs, act, weights=None, shifts=None, coeff_mode="PerLayer"):
     s = np.zeros(size, dtype=np.float32) if shifts is None else np.asarray(shifts, dtype=np.float32)
     y = orc.elemwise_sum([np.asarray(x, dtype=np.float32) for x in xs], w, s, coeff_mode)
     return act.apply(y)
+
+
+def run_net(spec, x, keep=None):
+    """Layer-ordered forward of a network description (n2d2_amd.nets.NetSpec) on the CPU oracle, as
+    DeepNet::propagate calls each cell (src/DeepNet.cpp:2692-2706).  x: integer-valued [B,C,H,W].
+    Returns {name: float32 NCHW output} for the names in `keep` (default: the last cell)."""
+    vals = {"input": np.ascontiguousarray(x, dtype=np.float32)}
+    keep = set(keep) if keep is not None else {spec.output}
+    out = {}
+    for i, l in enumerate(spec.layers):
+        ins = [vals[n] for n in l.inputs]
+        if l.type in ("conv", "fc", "elemwise", "scaling"):
+            a = l.act
+            act = ActSpec(a.kind, a.mode, a.scaling, a.frac_bits, a.clipping, a.nb_bits, a.unsigned_out)
+        if l.type == "conv":
+            y = conv_cell(ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups)
+        elif l.type == "fc":
+            y = fc_cell(ins[0], l.w, l.bias, act)
+        elif l.type == "pool":
+            y = pool_cell(ins[0], l.kind, l.pool, l.stride, l.pad)
+        elif l.type == "scaling":
+            y = act.apply(ins[0])           # ScalingCell_Frame::propagate: the Scaling alone
+        elif l.type == "elemwise":
+            y = elemwise_cell(ins, act, l.weights, l.shifts, l.coeff_mode)
+        else:
+            raise ValueError(l.type)
+        vals[l.name] = y
+        if l.name in keep:
+            out[l.name] = y
+        # free tensors nobody reads any more
+        later = set(n for m in spec.layers[i + 1:] for n in m.inputs)
+        for n in list(vals):
+            if n not in later and n != l.name:
+                del vals[n]
+    return out

@@ -31,7 +31,7 @@ def _i8(shape, lo=-127, hi=127):
 
 def _acts(O, bits=8):
     """One activation spec per rescale mode / signedness, with per-channel parameters."""
-    from cells_ref import ActSpec
+    from oracle.cells import ActSpec
     hi = 2 ** bits
     return {
         "none_linear": ActSpec("Linear", "None"),
@@ -106,7 +106,7 @@ def test_scaling_cell_all_modes(rt, layout):
 
 def test_scaling_on_byte_inputs_is_the_residual_branch_rescale(rt):
     from n2d2_amd import capi
-    from cells_ref import ActSpec
+    from oracle.cells import ActSpec
     Cc = 32
     x = _i8((2, Cc, 7, 7), -128, 127)
     spec = ActSpec("Linear", "FixedMult16", RNG.integers(2 ** 13, 2 ** 15, size=Cc), frac_bits=14, nb_bits=8, unsigned_out=False)
@@ -153,7 +153,7 @@ CONV_CASES = [
 @pytest.mark.parametrize("case", CONV_CASES, ids=[c[0] for c in CONV_CASES])
 def test_conv_cell_bit_exact(rt, case):
     from n2d2_amd import capi
-    import cells_ref
+    from oracle import cells as cells_ref
     name, B, Cc, H, W, O, k, s, p, d, kind = case
     x = _u8((B, Cc, H, W)) if kind == "u8" else _i8((B, Cc, H, W), -128, 127)
     w = np.clip(np.rint(RNG.normal(0, 40, size=(O, Cc, k[1], k[0]))), -127, 127).astype(np.int32)
@@ -182,8 +182,8 @@ def test_conv_config2_resnet18_stage_single_shift(rt):
     """3x3 s1 p1 64->64 on 56x56, uint8 input, N(0,40) weights, per-channel single shift in [8,12], ReLU clip [0,255];
     the oracle runs a 4-image slice, the GPU the same slice."""
     from n2d2_amd import capi
-    import cells_ref
-    from cells_ref import ActSpec
+    from oracle import cells as cells_ref
+    from oracle.cells import ActSpec
     B = 4
     x = _u8((B, 64, 56, 56))
     w = np.clip(np.rint(RNG.normal(0, 40, size=(64, 64, 3, 3))), -127, 127).astype(np.int32)
@@ -198,7 +198,7 @@ def test_conv_config2_resnet18_stage_single_shift(rt):
 @pytest.mark.parametrize("stride", [1, 2])
 def test_depthwise_conv_bit_exact(rt, stride):
     from n2d2_amd import capi
-    import cells_ref
+    from oracle import cells as cells_ref
     Cc = 48
     x = _u8((3, Cc, 13, 12))
     w = _i8((Cc, 1, 3, 3))
@@ -218,8 +218,8 @@ def test_depthwise_conv_bit_exact(rt, stride):
 def test_conv_int4_weights_uint4_activations(rt):
     """Weights in [-7,7] nibble-packed, activations in [0,15], fixed-point rescale with clip, 4-bit unsigned output."""
     from n2d2_amd import capi
-    import cells_ref
-    from cells_ref import ActSpec
+    from oracle import cells as cells_ref
+    from oracle.cells import ActSpec
     for (Cc, O, k, s, p) in ((64, 64, 3, 1, 1), (64, 128, 3, 2, 1), (64, 128, 1, 2, 0), (32, 40, 5, 1, 2)):
         x = RNG.integers(0, 16, size=(2, Cc, 14, 14)).astype(np.int32)
         w = RNG.integers(-7, 8, size=(O, Cc, k, k)).astype(np.int32)
@@ -259,7 +259,7 @@ def test_conv_linearity_and_batch_independence_at_full_width(rt):
 @pytest.mark.parametrize("shape", [(16, 5, 5, 120), (120, 1, 1, 84), (84, 1, 1, 10), (2048, 1, 1, 1000), (1, 6, 6, 20)])
 def test_fc_cell_bit_exact(rt, shape):
     from n2d2_amd import capi
-    import cells_ref
+    from oracle import cells as cells_ref
     Cc, H, W, O = shape
     B = 9
     x = _u8((B, Cc, H, W))
@@ -282,7 +282,7 @@ def test_fc_cell_bit_exact(rt, shape):
                                                   ("avg", (3, 3), (2, 2), (1, 1)), ("avg", (2, 2), (2, 2), (0, 0))])
 def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
     from n2d2_amd import capi
-    import cells_ref
+    from oracle import cells as cells_ref
     for dt, x in ((capi.U8B, _u8((3, 24, 14, 15))), (capi.I8, _i8((3, 24, 14, 15), -128, 127)), (capi.U8, _u8((2, 3, 14, 14)))):
         want = cells_ref.pool_cell(x, kind, pool, stride, pad)
         got = rt.Pool(kind, pool, stride, pad).forward(rt.DTensor.from_numpy(x, dt)).to_numpy()
@@ -293,8 +293,8 @@ def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
 
 def test_elemwise_sum_cell_bit_exact(rt):
     from n2d2_amd import capi
-    import cells_ref
-    from cells_ref import ActSpec
+    from oracle import cells as cells_ref
+    from oracle.cells import ActSpec
     Cc = 40
     a, b, c = _u8((2, Cc, 7, 9)), _i8((2, Cc, 7, 9), -128, 127), _u8((2, Cc, 7, 9))
     da, db, dc = rt.DTensor.from_numpy(a, capi.U8B), rt.DTensor.from_numpy(b, capi.I8), rt.DTensor.from_numpy(c, capi.U8B)
