@@ -309,6 +309,8 @@ int n2d2hip_scaling_forward(n2d2hip_act_t act, const n2d2hip_tensor* in, const n
         N2D2HIP_REQUIRE(act->min_out >= lo && act->max_out <= hi, N2D2HIP_ERR_INVALID,
                         "scaling_forward: output range [%d,%d] does not fit the output dtype", act->min_out, act->max_out);
     }
+    if (in->layout == N2D2HIP_NHWC && is_byte_type(in->dtype) && in->cs == out->cs && out->dtype != N2D2HIP_F32)
+        return run_scaling_nhwc(act, in, out, (hipStream_t)stream);
     const size_t total = (size_t)out->B * out->H * out->W * (out->layout == N2D2HIP_NHWC ? out->cs : out->C);
     hipLaunchKernelGGL(elementwise_kernel<true>, dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
                        in->data, in->dtype, in->layout, in->cs, out->data, out->dtype, out->layout, out->cs,

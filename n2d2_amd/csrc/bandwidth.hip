@@ -70,6 +70,8 @@ __global__ __launch_bounds__(256) void pool_kernel(const signed char* __restrict
 }
 
 constexpr int EW_MAX_INPUTS = 4;
+struct ElemWiseArgs;
+int run_elemwise(const ElemWiseArgs& a, bool fcoef, hipStream_t stream);
 struct ElemWiseArgs {
     const signed char* in[EW_MAX_INPUTS];
     int zp[EW_MAX_INPUTS];
@@ -86,42 +88,137 @@ struct ElemWiseArgs {
     EpiArgs epi;
 };
 
-// ref: src/Cell/ElemWiseCell_Frame.cpp:116-136 (Sum): float32 arithmetic in the same order,
-// products and sums rounded individually (no fused multiply-add), then the cell's activation.
+// ref: src/Cell/ElemWiseCell_Frame.cpp:116-136 (Sum) followed by the cell's activation; with one input and unit
+// coefficients it is ScalingCell_Frame::propagate (ref: src/Cell/ScalingCell_Frame.cpp:67-75).
+// FCOEF: float32 arithmetic in the reference's order, products and sums rounded individually (no fused
+// multiply-add).  !FCOEF: all weights are 1 and all shifts 0, the sum is formed in int32 (the same value: every
+// float operation of the reference is exact on these operands).
+// HOIST: the launch makes the grid stride a multiple of the dwords per pixel, so a thread keeps its 4 channels
+// and loads their table rows once.
+template <int KIND, bool FCOEF, bool HOIST>
 __global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
 {
     const int cq = p.cs >> 2;
     const long long total = p.npix * cq;
-    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
-        const int c4 = (int)(idx % cq) * 4;
-        float o[4];
-        {
-            int v[4];
-            unpack4(*(const int*)(p.in[0] + idx * 4) ^ (int)p.flip[0], p.zp[0], v);
-            const float4 w = *(const float4*)(p.w + c4), s = *(const float4*)(p.s + c4);
-            o[0] = __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x);
-            o[1] = __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y);
-            o[2] = __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z);
-            o[3] = __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w);
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    int c4 = (int)(idx % cq) * 4;
+    int4 ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
+    auto load_tables = [&](int c) {
+        if (KIND != EPI_RAW) {
+            ta = *(const int4*)(p.epi.a + c);
+            tb = *(const int4*)(p.epi.b + c);
+            tc = *(const int4*)(p.epi.c + c);
+            if (KIND == EPI_I24) td = *(const int4*)(p.epi.d + c);
+            if (KIND != EPI_F32) te = *(const int4*)(p.epi.e + c);
         }
-        for (int k = 1; k < p.nb_inputs; ++k) {
-            int v[4];
-            unpack4(*(const int*)(p.in[k] + idx * 4) ^ (int)p.flip[k], p.zp[k], v);
-            const float4 w = *(const float4*)(p.w + (long long)k * p.cpad + c4), s = *(const float4*)(p.s + (long long)k * p.cpad + c4);
-            o[0] = __fadd_rn(o[0], __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x));
-            o[1] = __fadd_rn(o[1], __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y));
-            o[2] = __fadd_rn(o[2], __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z));
-            o[3] = __fadd_rn(o[3], __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w));
+    };
+    if (HOIST) load_tables(c4);
+#pragma unroll 4
+    for (; idx < total; idx += stride) {
+        if (!HOIST) {
+            c4 = (int)(idx % cq) * 4;
+            load_tables(c4);
         }
         int r[4];
+        if (FCOEF) {
+            float o[4];
+            {
+                int v[4];
+                unpack4(*(const int*)(p.in[0] + idx * 4) ^ (int)p.flip[0], p.zp[0], v);
+                const float4 w = *(const float4*)(p.w + c4), s = *(const float4*)(p.s + c4);
+                o[0] = __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x);
+                o[1] = __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y);
+                o[2] = __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z);
+                o[3] = __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w);
+            }
+            for (int k = 1; k < p.nb_inputs; ++k) {
+                int v[4];
+                unpack4(*(const int*)(p.in[k] + idx * 4) ^ (int)p.flip[k], p.zp[k], v);
+                const float4 w = *(const float4*)(p.w + (long long)k * p.cpad + c4), s = *(const float4*)(p.s + (long long)k * p.cpad + c4);
+                o[0] = __fadd_rn(o[0], __fadd_rn(__fmul_rn(w.x, (float)v[0]), s.x));
+                o[1] = __fadd_rn(o[1], __fadd_rn(__fmul_rn(w.y, (float)v[1]), s.y));
+                o[2] = __fadd_rn(o[2], __fadd_rn(__fmul_rn(w.z, (float)v[2]), s.z));
+                o[3] = __fadd_rn(o[3], __fadd_rn(__fmul_rn(w.w, (float)v[3]), s.w));
+            }
+            if (KIND == EPI_F32) {
+                const int a4[4] = {ta.x, ta.y, ta.z, ta.w}, b4[4] = {tb.x, tb.y, tb.z, tb.w}, c4v[4] = {tc.x, tc.y, tc.z, tc.w};
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-            r[t] = epi_apply_dyn_f(p.epi, o[t], c4 + t);
+                for (int t = 0; t < 4; ++t) {
+                    float f = fminf(fmaxf(o[t], as_f32(a4[t])), as_f32(b4[t]));
+                    f = round_half_away(__fmul_rn(f, as_f32(c4v[t])));
+                    r[t] = (int)fminf(fmaxf(f, (float)p.epi.lo), (float)p.epi.hi);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    r[t] = (int)fminf(fmaxf(round_half_away(o[t]), -2147483520.0f), 2147483520.0f);   // round(realInput)
+            }
+        } else {
+            unpack4(*(const int*)(p.in[0] + idx * 4) ^ (int)p.flip[0], p.zp[0], r);
+            for (int k = 1; k < p.nb_inputs; ++k) {
+                int v[4];
+                unpack4(*(const int*)(p.in[k] + idx * 4) ^ (int)p.flip[k], p.zp[k], v);
+                r[0] += v[0]; r[1] += v[1]; r[2] += v[2]; r[3] += v[3];
+            }
+        }
+        if (!(FCOEF && KIND == EPI_F32)) {
+            r[0] = epi_apply<KIND>(r[0], ta.x, tb.x, tc.x, td.x, te.x, p.epi.lo, p.epi.hi, p.epi.relu);
+            r[1] = epi_apply<KIND>(r[1], ta.y, tb.y, tc.y, td.y, te.y, p.epi.lo, p.epi.hi, p.epi.relu);
+            r[2] = epi_apply<KIND>(r[2], ta.z, tb.z, tc.z, td.z, te.z, p.epi.lo, p.epi.hi, p.epi.relu);
+            r[3] = epi_apply<KIND>(r[3], ta.w, tb.w, tc.w, td.w, te.w, p.epi.lo, p.epi.hi, p.epi.relu);
+        }
         if (p.out_dtype == N2D2HIP_I32)
             *(int4*)((int*)p.out + idx * 4) = int4{r[0], r[1], r[2], r[3]};
         else
             *(unsigned*)((signed char*)p.out + idx * 4) = pack4(r) ^ p.out_xor;
     }
+}
+
+template <bool FCOEF, bool HOIST>
+static void launch_elemwise(const ElemWiseArgs& a, unsigned grid, hipStream_t stream)
+{
+    switch (a.epi.kind) {
+    case EPI_RAW: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_RAW, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I24, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I64, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_F32, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
+    }
+}
+
+// Launches the sum / rescale kernel over NHWC byte tensors described by `a`.
+int run_elemwise(const ElemWiseArgs& a, bool fcoef, hipStream_t stream)
+{
+    const int cq = a.cs >> 2;
+    const long long total = a.npix * cq;
+    long long want = std::max<long long>(1, std::min<long long>((total + 1023) / 1024, 256 * 16));   // ~4 dwords per thread and pass
+    // grid stride (grid*256) must be a multiple of cq for the hoisted form
+    int g = cq, b = 256;
+    while (b) { const int t = g % b; g = b; b = t; }
+    const long long unit = cq / g;                // grid must be a multiple of this
+    bool hoist = unit <= want;
+    unsigned grid = (unsigned)(hoist ? (want / unit) * unit : want);
+    if (fcoef) { if (hoist) launch_elemwise<true, true>(a, grid, stream); else launch_elemwise<true, false>(a, grid, stream); }
+    else { if (hoist) launch_elemwise<false, true>(a, grid, stream); else launch_elemwise<false, false>(a, grid, stream); }
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+// ScalingCell on an NHWC byte tensor: the one-input, unit-coefficient case of the kernel above.
+int run_scaling_nhwc(const n2d2hip_act_s* act, const n2d2hip_tensor* in, const n2d2hip_tensor* out, hipStream_t stream)
+{
+    ElemWiseArgs a = {};
+    a.in[0] = (const signed char*)in->data;
+    a.flip[0] = in->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
+    a.zp[0] = in->dtype == N2D2HIP_I8 ? 0 : 128;
+    a.nb_inputs = 1;
+    a.out = out->data;
+    a.out_dtype = out->dtype;
+    a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    a.cs = out->cs;
+    a.npix = (long long)out->B * out->H * out->W;
+    a.epi = act->args;
+    return run_elemwise(a, false, stream);
 }
 
 } // namespace n2d2hip
@@ -132,6 +229,7 @@ struct n2d2hip_elemwise_s {
     int nb_inputs, nb_channels, cpad;
     n2d2hip_act_t act;
     float* d_coeff;     // w then s, each [nb_inputs][cpad]
+    bool unit_coeff;    // every weight 1 and every shift 0
 };
 
 extern "C" {
@@ -196,6 +294,9 @@ int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, cons
             hs[(size_t)k * cpad + c] = shifts ? shifts[idx] : 0.0f;
         }
     n2d2hip_elemwise_s* e = new n2d2hip_elemwise_s();
+    e->unit_coeff = true;
+    for (size_t i = 0; i < (size_t)nb_inputs * cpad; ++i)
+        if (hw[i] != 1.0f || hs[i] != 0.0f) e->unit_coeff = false;
     e->nb_inputs = nb_inputs; e->nb_channels = nb_channels; e->cpad = cpad; e->act = act; e->d_coeff = nullptr;
     hipError_t herr = hipMalloc((void**)&e->d_coeff, h.size() * sizeof(float));
     if (herr == hipSuccess) herr = hipMemcpy(e->d_coeff, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
@@ -252,11 +353,10 @@ int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const*
     a.cs = out->cs;
     a.npix = (long long)out->B * out->H * out->W;
     a.epi = act->args;
-    const long long total = a.npix * (a.cs / 4);
-    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
-    hipLaunchKernelGGL(elemwise_sum_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, a);
-    N2D2HIP_HIP_CHECK(hipGetLastError());
-    return N2D2HIP_OK;
+    // EPI_RAW on float coefficients would emit non-integers: only the integer form is defined there
+    if (act->args.kind == EPI_RAW)
+        N2D2HIP_REQUIRE(ew->unit_coeff, N2D2HIP_ERR_UNSUPPORTED, "elemwise_forward: non-unit coefficients need a rescaling activation");
+    return run_elemwise(a, !ew->unit_coeff, (hipStream_t)stream);
 }
 
 } // extern "C"

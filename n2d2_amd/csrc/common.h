@@ -74,6 +74,12 @@ struct EpiArgs {
 
 } // namespace n2d2hip
 
+struct n2d2hip_act_s;
+namespace n2d2hip {
+// Fast path of the stand-alone Scaling for NHWC byte inputs (bandwidth.hip).
+int run_scaling_nhwc(const n2d2hip_act_s* act, const n2d2hip_tensor* in, const n2d2hip_tensor* out, hipStream_t stream);
+}
+
 struct n2d2hip_act_s {
     n2d2hip_activation desc;   // pointers inside are NOT kept valid; do not dereference
     int nb_channels;

@@ -402,6 +402,36 @@ class GpuNet:
             fn(cell, ins, out)
         return self.tensors[self.spec.output]
 
+    def forward_timed(self):
+        """One forward with a pair of events around every cell launch, recorded on the stream the kernels run on.
+        Returns [(layer, milliseconds)]."""
+        import torch
+        evs = []
+        for (l, cell, fn), (ins, out) in zip(self.steps, self._io):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn(cell, ins, out)
+            e1.record()
+            evs.append((l, e0, e1))
+        torch.cuda.synchronize()
+        return [(l, e0.elapsed_time(e1)) for l, e0, e1 in evs]
+
+    def layer_bytes(self, l):
+        """Algorithmic HBM bytes of one cell: inputs and output once at storage width, weights once."""
+        ins, out = self._io[self.spec.layers.index(l)]
+        total = sum(t.B * t.C * t.H * t.W * (4 if t.dtype == self.capi.I32 else 1) for t in ins)
+        total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
+        if l.type in ("conv", "fc"):
+            total += l.w.size // (2 if l.weight_bits == 4 else 1)
+        return total
+
+    def layer_macs(self, l):
+        if l.type == "conv":
+            return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
+        if l.type == "fc":
+            return self.B * l.w.size
+        return 0
+
     def activation_bytes(self):
         """Algorithmic HBM bytes of one forward: every cell reads its inputs and writes its output once, plus weights."""
         total = 0

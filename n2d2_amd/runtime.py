@@ -103,7 +103,7 @@ class Act:
         return capi.U8B if self.unsigned_out else capi.I8
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_act_destroy(self.handle)
             self.handle = None
 
@@ -151,7 +151,7 @@ class Conv:
         return out
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_conv_destroy(self.handle)
             self.handle = None
 
@@ -179,7 +179,7 @@ class Fc:
         return out
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_fc_destroy(self.handle)
             self.handle = None
 
@@ -221,6 +221,6 @@ class ElemWiseSum:
         return out
 
     def __del__(self):
-        if getattr(self, "handle", None):
+        if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_elemwise_destroy(self.handle)
             self.handle = None
