@@ -13,6 +13,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libn2d2hip.so")
+GLUE_LIB = os.path.join(LIBDIR, "libn2d2_frame_hip.so")
 SOURCES = ["act.hip", "conv_igemm.hip", "bandwidth.hip", "quantizer.hip"]
 
 # -ffp-contract=off: float rescales must round the product and the sum
@@ -45,6 +46,12 @@ def build(verbose=False):
     with ThreadPoolExecutor(max_workers=4) as ex:
         outs = list(ex.map(compile_one, zip(SOURCES, objs)))
     outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs))
+    # host cells ("Frame_HIP" model): plain C++ over the C ABI
+    glue = os.path.join(CSRC, "frame_hip")
+    outs.append(_run([os.environ.get("CXX", "g++"), "-std=c++14", "-O2", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
+                      "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"), "-shared",
+                      os.path.join(glue, "frame_hip.cpp"), os.path.join(glue, "frame_hip_capi.cpp"), "-o", GLUE_LIB,
+                      "-L" + LIBDIR, "-ln2d2hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]))
     if verbose:
         for o in outs:
             if o.strip():

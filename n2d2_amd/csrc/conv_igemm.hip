@@ -63,7 +63,7 @@ __device__ __forceinline__ void unpack_w4(unsigned p, int& lo, int& hi)
 }
 
 template <int BM, int BN, int WGM, int EPI, bool PIX4, bool W4>
-__global__ __launch_bounds__(256) void conv_igemm_kernel(ConvArgs p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_igemm_kernel(ConvArgs p)
 {
     constexpr int WGN = 4 / WGM;
     constexpr int TM = BM / WGM;      // pixels per wave

@@ -1,0 +1,1301 @@
+// Implementation of the Frame_HIP host cells and of their registrations.
+#include "frame_hip.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstring>
+
+namespace N2D2 {
+
+void checkStatus(int status)
+{
+    if (status != N2D2HIP_OK) {
+        const char* msg = n2d2hip_last_error();
+        throw std::runtime_error((msg && *msg) ? std::string(msg) : std::string(n2d2hip_strerror(status)));
+    }
+}
+
+static void checkHip(hipError_t e, const char* what)
+{
+    if (e != hipSuccess)
+        throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// ------------------------------------------------------------------ HipTensor
+HipTensor::~HipTensor()
+{
+    if (mDesc.data)
+        (void)hipFree(mDesc.data);
+}
+
+void HipTensor::resize(int B, int C, int H, int W, int dtype)
+{
+    n2d2hip_tensor d;
+    d.data = nullptr;
+    d.dtype = dtype;
+    d.layout = N2D2HIP_NHWC;
+    d.B = B; d.C = C; d.H = H; d.W = W;
+    d.cs = n2d2hip_nhwc_cs(C);
+    const size_t bytes = n2d2hip_tensor_bytes(&d);
+    if (mDesc.data && bytes == mBytes) {
+        d.data = mDesc.data;
+    } else {
+        if (mDesc.data)
+            (void)hipFree(mDesc.data);
+        mDesc.data = nullptr;
+        checkHip(hipMalloc(&d.data, bytes), "HipTensor::resize(): hipMalloc");
+        mBytes = bytes;
+    }
+    mDesc = d;
+    mHostValid = false;
+}
+
+const Tensor<Float_T>& HipTensor::synchronizeDToH(void* stream)
+{
+    if (mHostValid)
+        return mHost;
+    if (!mDesc.data)
+        throw std::runtime_error("HipTensor::synchronizeDToH(): empty tensor");
+    n2d2hip_tensor f = mDesc;
+    f.dtype = N2D2HIP_F32;
+    f.layout = N2D2HIP_NCHW;
+    const size_t n = (size_t)f.B * f.C * f.H * f.W;
+    checkHip(hipMalloc(&f.data, n * sizeof(float)), "HipTensor::synchronizeDToH(): hipMalloc");
+    int rc = n2d2hip_convert(&mDesc, &f, stream);
+    mHost.resize({(size_t)f.W, (size_t)f.H, (size_t)f.C, (size_t)f.B});
+    hipError_t e = hipSuccess;
+    if (rc == N2D2HIP_OK) {
+        e = hipStreamSynchronize((hipStream_t)stream);
+        if (e == hipSuccess)
+            e = hipMemcpy(mHost.data(), f.data, n * sizeof(float), hipMemcpyDeviceToHost);
+    }
+    (void)hipFree(f.data);
+    checkStatus(rc);
+    checkHip(e, "HipTensor::synchronizeDToH()");
+    mHostValid = true;
+    return mHost;
+}
+
+void HipTensor::synchronizeHToD(const Tensor<Float_T>& host, void* stream)
+{
+    if (!mDesc.data)
+        throw std::runtime_error("HipTensor::synchronizeHToD(): empty tensor");
+    if (host.dimX() != (size_t)mDesc.W || host.dimY() != (size_t)mDesc.H || host.dimZ() != (size_t)mDesc.C || host.dimB() != (size_t)mDesc.B)
+        throw std::runtime_error("HipTensor::synchronizeHToD(): host tensor dimensions do not match");
+    n2d2hip_tensor f = mDesc;
+    f.dtype = N2D2HIP_F32;
+    f.layout = N2D2HIP_NCHW;
+    checkHip(hipMalloc(&f.data, host.size() * sizeof(float)), "HipTensor::synchronizeHToD(): hipMalloc");
+    hipError_t e = hipMemcpy(f.data, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice);
+    int rc = N2D2HIP_OK;
+    if (e == hipSuccess) {
+        rc = n2d2hip_convert(&f, &mDesc, stream);
+        e = hipStreamSynchronize((hipStream_t)stream);
+    }
+    (void)hipFree(f.data);
+    checkHip(e, "HipTensor::synchronizeHToD()");
+    checkStatus(rc);
+    mHostValid = false;
+}
+
+// -------------------------------------------------------------------- Scaling
+ScalingMode parseScalingMode(const std::string& str)
+{
+    // the spellings of include/ScalingMode.hpp
+    if (str == "None") return ScalingMode::NONE;
+    if (str == "Floating-point") return ScalingMode::FLOAT_MULT;
+    if (str == "Fixed-point16") return ScalingMode::FIXED_MULT16;
+    if (str == "Fixed-point32") return ScalingMode::FIXED_MULT32;
+    if (str == "Single-shift") return ScalingMode::SINGLE_SHIFT;
+    if (str == "Double-shift") return ScalingMode::DOUBLE_SHIFT;
+    throw std::runtime_error("Unknown scaling mode \"" + str + "\"");
+}
+
+bool Scaling::allScalingsPositive() const
+{
+    switch (mMode) {
+    case ScalingMode::FLOAT_MULT: return std::all_of(mFloat.begin(), mFloat.end(), [](Float_T v) { return v >= 0.0; });
+    case ScalingMode::FIXED_MULT16:
+    case ScalingMode::FIXED_MULT32: return std::all_of(mFixed.begin(), mFixed.end(), [](std::int32_t v) { return v >= 0; });
+    case ScalingMode::SINGLE_SHIFT:
+    case ScalingMode::DOUBLE_SHIFT: return true;
+    default: throw std::runtime_error("Unsupported scaling mode");
+    }
+}
+
+std::size_t Scaling::nbOutputs() const
+{
+    switch (mMode) {
+    case ScalingMode::FLOAT_MULT: return mFloat.size();
+    case ScalingMode::FIXED_MULT16:
+    case ScalingMode::FIXED_MULT32: return mFixed.size();
+    case ScalingMode::SINGLE_SHIFT: return mShift.size();
+    case ScalingMode::DOUBLE_SHIFT: return mShift.size() / 2;
+    default: return 0;
+    }
+}
+
+// Builds the C-ABI object for "Scaling::propagate + activation" of one cell.
+static n2d2hip_act_t makeAct(const Scaling& s, int kind, float leak, std::size_t nbBits, bool unsignedOut, unsigned int nbChannels,
+                             const std::string& cellName)
+{
+    n2d2hip_activation d;
+    std::memset(&d, 0, sizeof(d));
+    d.kind = kind;
+    d.leak_slope = leak;
+    d.nb_bits = (int)nbBits;
+    d.unsigned_out = unsignedOut ? 1 : 0;
+    d.frac_bits = (int)s.getFractionalBits();
+    d.is_clipped = s.getIsClipped() ? 1 : 0;
+    d.clipping = s.getClippingPerOutput().empty() ? nullptr : s.getClippingPerOutput().data();
+    switch (s.getMode()) {
+    case ScalingMode::NONE: d.scaling_mode = N2D2HIP_SCALING_NONE; break;
+    case ScalingMode::FLOAT_MULT: d.scaling_mode = N2D2HIP_SCALING_FLOAT_MULT; d.scaling = s.getFloatScalingPerOutput().data(); break;
+    case ScalingMode::FIXED_MULT16: d.scaling_mode = N2D2HIP_SCALING_FIXED_MULT16; d.scaling = s.getFixedScalingPerOutput().data(); break;
+    case ScalingMode::FIXED_MULT32: d.scaling_mode = N2D2HIP_SCALING_FIXED_MULT32; d.scaling = s.getFixedScalingPerOutput().data(); break;
+    case ScalingMode::SINGLE_SHIFT: d.scaling_mode = N2D2HIP_SCALING_SINGLE_SHIFT; d.scaling = s.getShiftScalingPerOutput().data(); break;
+    case ScalingMode::DOUBLE_SHIFT: d.scaling_mode = N2D2HIP_SCALING_DOUBLE_SHIFT; d.scaling = s.getShiftScalingPerOutput().data(); break;
+    }
+    if (s.getMode() != ScalingMode::NONE && s.nbOutputs() != nbChannels)
+        throw std::runtime_error("Cell " + cellName + ": the scaling has " + std::to_string(s.nbOutputs()) + " entries for "
+                                 + std::to_string(nbChannels) + " outputs");
+    if (d.is_clipped && s.getClippingPerOutput().size() != nbChannels && s.getMode() != ScalingMode::SINGLE_SHIFT
+        && s.getMode() != ScalingMode::DOUBLE_SHIFT)
+        throw std::runtime_error("Cell " + cellName + ": clipping vector size does not match the number of outputs");
+    n2d2hip_act_t h = nullptr;
+    checkStatus(n2d2hip_act_create(&d, (int)nbChannels, &h));
+    return h;
+}
+
+// ----------------------------------------------------------- static state
+int CellExport::mPrecision = 0;
+bool DeepNetExport::mUnsignedData = true;
+bool DeepNetExport::mEnvDataUnsigned = false;
+
+bool DeepNetExport::isCellOutputUnsigned(const Cell& cell)
+{
+    if (CellExport::mPrecision <= 0 || !DeepNetExport::mUnsignedData)
+        return false;            // unsigned cells are not allowed
+    return cell.getOutputsRange().first >= 0.0;
+}
+
+// ---------------------------------------------------------------- activations
+const char* RectifierActivation::Type = "Rectifier";
+const char* LinearActivation::Type = "Linear";
+
+void RectifierActivation::setParameter(const std::string& name, double value)
+{
+    if (name == "LeakSlope") mLeakSlope = value;
+    else if (name == "Clipping") mClipping = value;
+    else throw std::runtime_error("Parameter does not exist: " + name);
+    ++mRevision;
+}
+void LinearActivation::setParameter(const std::string& name, double value)
+{
+    if (name == "Clipping") mClipping = value;
+    else throw std::runtime_error("Parameter does not exist: " + name);
+    ++mRevision;
+}
+
+template <> Registrar<RectifierActivation> RectifierActivation_Frame_HIP<float>::mRegistrar(
+    "Frame_HIP", RectifierActivation_Frame_HIP<float>::create, Registrar<RectifierActivation>::Type<float>());
+template <> Registrar<LinearActivation> LinearActivation_Frame_HIP<float>::mRegistrar(
+    "Frame_HIP", LinearActivation_Frame_HIP<float>::create, Registrar<LinearActivation>::Type<float>());
+
+// ----------------------------------------------------------------------- Cell
+std::pair<double, double> Cell::getOutputsRangeParents() const
+{
+    if (mParents.empty())
+        throw std::runtime_error("Cell " + mName + " must have a parent.");
+    std::pair<double, double> range;
+    for (size_t i = 0; i < mParents.size(); ++i) {
+        if (!mParents[i])
+            throw std::runtime_error("Environment shouldn't be connected to cell " + mName + ".");
+        const std::pair<double, double> r = mParents[i]->getOutputsRange();
+        if (i == 0) range = r;
+        else { range.first = std::min(range.first, r.first); range.second = std::max(range.second, r.second); }
+    }
+    return range;
+}
+
+Cell_Frame_HIP::~Cell_Frame_HIP()
+{
+    if (mActHandle)
+        n2d2hip_act_destroy(mActHandle);
+}
+
+void Cell_Frame_HIP::addInput(Cell_Frame_HIP* parent)
+{
+    if (!parent)
+        throw std::runtime_error("Cell " + mName + ": null parent");
+    if (!mInputs.empty() && (parent->getOutputsWidth() != mInW || parent->getOutputsHeight() != mInH || parent->batchSize() != mBatch))
+        throw std::runtime_error("Cell " + mName + ": inputs of different sizes");
+    mParents.push_back(parent);
+    mInputs.push_back(&parent->mOutputs);
+    if (mInputs.size() == 1)
+        mNbChannels = parent->getNbOutputs();
+    else if (parent->getNbOutputs() != mNbChannels)
+        throw std::runtime_error("Cell " + mName + ": inputs with different numbers of channels are not supported by Frame_HIP");
+    mInW = parent->getOutputsWidth();
+    mInH = parent->getOutputsHeight();
+    mBatch = parent->batchSize();
+    setOutputsDims();
+}
+
+void Cell_Frame_HIP::addInput(HipTensor& stimuli, unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize)
+{
+    if (!mInputs.empty())
+        throw std::runtime_error("Cell " + mName + ": the environment must be the only input");
+    mParents.push_back(nullptr);
+    mInputs.push_back(&stimuli);
+    mNbChannels = nbChannels;
+    mInW = width;
+    mInH = height;
+    mBatch = batchSize;
+    setOutputsDims();
+}
+
+const Tensor<Float_T>& Cell_Frame_HIP::getOutputs()
+{
+    return mOutputs.synchronizeDToH(mStream);
+}
+
+int Cell_Frame_HIP::outputDType(const Scaling* standalone) const
+{
+    const Scaling* s = standalone ? standalone : (mActivation ? &mActivation->getActivationScaling() : nullptr);
+    if (!s || s->getMode() == ScalingMode::NONE)
+        return N2D2HIP_I32;
+    return DeepNetExport::isCellOutputUnsigned(*this) ? N2D2HIP_U8B : N2D2HIP_I8;
+}
+
+void Cell_Frame_HIP::allocateOutputs(const Scaling* standalone)
+{
+    if (mInputs.empty())
+        throw std::runtime_error("Cell " + mName + " has no input");
+    mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, outputDType(standalone));
+}
+
+n2d2hip_act_t Cell_Frame_HIP::activationHandle(const Scaling* standalone)
+{
+    const bool uns = DeepNetExport::isCellOutputUnsigned(*this);
+    const unsigned rev = mActivation ? mActivation->revision() : 0u;
+    if (mActHandle && mActRevision == rev && mActUnsigned == (int)uns && !standalone)
+        return mActHandle;
+    if (mActHandle) {
+        n2d2hip_act_destroy(mActHandle);
+        mActHandle = nullptr;
+    }
+    Scaling none;
+    const Scaling& s = standalone ? *standalone : (mActivation ? mActivation->getActivationScaling() : none);
+    // RectifierActivation_Frame.hpp:65-66: the activation's bit width when set, else the cell's
+    const std::size_t nbBits = (mActivation && mActivation->getQuantizedNbBits() > 0) ? mActivation->getQuantizedNbBits() : mQuantizedNbBits;
+    const int kind = (mActivation && !standalone) ? mActivation->abiKind() : N2D2HIP_ACT_LINEAR;
+    const float leak = (mActivation && !standalone) ? mActivation->leakSlope() : 0.0f;
+    mActHandle = makeAct(s, kind, leak, nbBits, uns, mNbOutputs, mName);
+    mActRevision = rev;
+    mActUnsigned = (int)uns;
+    // the storage type follows the signedness decision
+    if (mOutputs.empty() || mOutputs.desc().dtype != outputDType(standalone))
+        allocateOutputs(standalone);
+    return mActHandle;
+}
+
+// Integer check of a float parameter on its way to the device.
+static long long toInteger(Float_T v, long long lo, long long hi, const std::string& what)
+{
+    const double r = std::nearbyint((double)v);
+    if (r != (double)v || r < (double)lo || r > (double)hi) {
+        std::ostringstream msg;
+        msg << what << ": value " << v << " is not an integer in [" << lo << "," << hi << "]; quantize the network before running it on Frame_HIP";
+        throw std::runtime_error(msg.str());
+    }
+    return (long long)r;
+}
+
+static std::vector<unsigned char> packWeights(const Tensor<Float_T>& w, int bits, const std::string& name)
+{
+    const long long lo = bits == 4 ? -8 : -128, hi = bits == 4 ? 7 : 127;
+    std::vector<unsigned char> out(bits == 4 ? (w.size() + 1) / 2 : w.size(), 0);
+    for (size_t i = 0; i < w.size(); ++i) {
+        const long long v = toInteger(w(i), lo, hi, "Cell " + name + " weights");
+        if (bits == 4)
+            out[i >> 1] |= (unsigned char)((v & 15) << ((i & 1) ? 4 : 0));
+        else
+            out[i] = (unsigned char)(signed char)v;
+    }
+    return out;
+}
+
+// ------------------------------------------------------------------- ConvCell
+const char* ConvCell::Type = "Conv";
+
+ConvCell::ConvCell(const std::vector<unsigned int>& kernelDims, const std::vector<unsigned int>& subSampleDims,
+                   const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+                   const std::vector<unsigned int>& dilationDims)
+    : mKernelDims(kernelDims), mSubSampleDims(subSampleDims), mStrideDims(strideDims), mDilationDims(dilationDims),
+      mPaddingDims(paddingDims), mNoBias(false), mNbGroups(1), mWeightBits(8), mDirty(true)
+{
+    if (mKernelDims.size() != 2)
+        throw std::runtime_error("ConvCell: only 2D convolutions are supported by Frame_HIP");
+    if (mSubSampleDims.empty()) mSubSampleDims.assign(2, 1U);
+    if (mStrideDims.empty()) mStrideDims.assign(2, 1U);
+    if (mPaddingDims.empty()) mPaddingDims.assign(2, 0);
+    if (mDilationDims.empty()) mDilationDims.assign(2, 1U);
+    if (mSubSampleDims[0] != 1 || mSubSampleDims[1] != 1)
+        throw std::runtime_error("ConvCell: sub-sampling is not supported by Frame_HIP");
+}
+
+void ConvCell::setParameter(const std::string& name, bool value)
+{
+    if (name == "NoBias") { mNoBias = value; mDirty = true; }
+    else throw std::runtime_error("Parameter does not exist: " + name);
+}
+
+template <class T>
+ConvCell_Frame_HIP<T>::ConvCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& kernelDims,
+                                          unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
+                                          const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+                                          const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr)
+{
+    mActivation = activation;
+}
+
+template <class T>
+ConvCell_Frame_HIP<T>::~ConvCell_Frame_HIP()
+{
+    if (mConv) n2d2hip_conv_destroy(mConv);
+}
+
+template <class T>
+void ConvCell_Frame_HIP<T>::setOutputsDims()
+{
+    // src/Cell/ConvCell.cpp:1169-1195
+    const unsigned int in[2] = {mInW, mInH};
+    unsigned int out[2];
+    for (int dim = 0; dim < 2; ++dim) {
+        const int kernelExtent = (int)(mDilationDims[dim] * (mKernelDims[dim] - 1) + 1);
+        out[dim] = (unsigned int)std::ceil(std::floor(((int)in[dim] + 2 * mPaddingDims[dim] - kernelExtent + (int)mStrideDims[dim])
+                                                      / (double)mStrideDims[dim]) / (double)mSubSampleDims[dim]);
+    }
+    mOutW = out[0];
+    mOutH = out[1];
+}
+
+template <class T>
+void ConvCell_Frame_HIP<T>::initialize()
+{
+    if (mInputs.size() != 1)
+        throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": exactly one input tensor is supported");
+    allocateOutputs();
+}
+
+template <class T>
+void ConvCell_Frame_HIP<T>::propagate(bool /*inference*/)
+{
+    n2d2hip_act_t act = activationHandle();
+    const int inDType = mInputs[0]->desc().dtype;
+    if (mDirty || act != mConvAct || !mConv) {
+        if (mConv) { n2d2hip_conv_destroy(mConv); mConv = nullptr; }
+        const unsigned int cg = mNbChannels / mNbGroups;
+        if (mWeights.dimX() != mKernelDims[0] || mWeights.dimY() != mKernelDims[1] || mWeights.dimZ() != cg || mWeights.dimB() != mNbOutputs)
+            throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": weights must be {kW, kH, nbChannels/groups, nbOutputs}");
+        n2d2hip_conv_desc d;
+        d.C = (int)mNbChannels; d.O = (int)mNbOutputs; d.kW = (int)mKernelDims[0]; d.kH = (int)mKernelDims[1];
+        d.strideX = (int)mStrideDims[0]; d.strideY = (int)mStrideDims[1];
+        d.padL = d.padR = mPaddingDims[0]; d.padT = d.padB = mPaddingDims[1];
+        d.dilX = (int)mDilationDims[0]; d.dilY = (int)mDilationDims[1];
+        d.groups = (int)mNbGroups; d.weight_bits = mWeightBits;
+        const std::vector<unsigned char> w = packWeights(mWeights, mWeightBits, mName);
+        std::vector<std::int32_t> b;
+        if (!mNoBias) {
+            if (mBias.size() != mNbOutputs)
+                throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": one bias per output expected");
+            for (size_t i = 0; i < mBias.size(); ++i)
+                b.push_back((std::int32_t)toInteger(mBias(i), std::numeric_limits<std::int32_t>::min(), std::numeric_limits<std::int32_t>::max(),
+                                                    "Cell " + mName + " biases"));
+        }
+        checkStatus(n2d2hip_conv_create(&d, w.data(), mNoBias ? nullptr : b.data(), act, inDType, &mConv));
+        mConvAct = act;
+        mDirty = false;
+    }
+    checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <> Registrar<ConvCell> ConvCell_Frame_HIP<float>::mRegistrar("Frame_HIP", ConvCell_Frame_HIP<float>::create,
+                                                                      Registrar<ConvCell>::Type<float>());
+
+// --------------------------------------------------------------------- FcCell
+const char* FcCell::Type = "Fc";
+
+void FcCell::setParameter(const std::string& name, bool value)
+{
+    if (name == "NoBias") { mNoBias = value; mDirty = true; }
+    else throw std::runtime_error("Parameter does not exist: " + name);
+}
+
+template <class T>
+FcCell_Frame_HIP<T>::FcCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
+                                      const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), mFc(nullptr), mFcAct(nullptr)
+{
+    mActivation = activation;
+}
+
+template <class T>
+FcCell_Frame_HIP<T>::~FcCell_Frame_HIP()
+{
+    if (mFc) n2d2hip_fc_destroy(mFc);
+}
+
+template <class T>
+void FcCell_Frame_HIP<T>::setOutputsDims()
+{
+    mOutW = 1;
+    mOutH = 1;
+}
+
+template <class T>
+void FcCell_Frame_HIP<T>::initialize()
+{
+    if (mInputs.size() != 1)
+        throw std::runtime_error("FcCell_Frame_HIP " + mName + ": exactly one input tensor is supported");
+    allocateOutputs();
+}
+
+template <class T>
+void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
+{
+    n2d2hip_act_t act = activationHandle();
+    const int inDType = mInputs[0]->desc().dtype;
+    if (mDirty || act != mFcAct || !mFc) {
+        if (mFc) { n2d2hip_fc_destroy(mFc); mFc = nullptr; }
+        const size_t K = (size_t)mNbChannels * mInH * mInW;
+        if (mWeights.size() != K * mNbOutputs)
+            throw std::runtime_error("FcCell_Frame_HIP " + mName + ": weights must hold nbOutputs x (channels*height*width) values");
+        const std::vector<unsigned char> w = packWeights(mWeights, 8, mName);
+        std::vector<std::int32_t> b;
+        if (!mNoBias) {
+            if (mBias.size() != mNbOutputs)
+                throw std::runtime_error("FcCell_Frame_HIP " + mName + ": one bias per output expected");
+            for (size_t i = 0; i < mBias.size(); ++i)
+                b.push_back((std::int32_t)toInteger(mBias(i), std::numeric_limits<std::int32_t>::min(), std::numeric_limits<std::int32_t>::max(),
+                                                    "Cell " + mName + " biases"));
+        }
+        checkStatus(n2d2hip_fc_create((int)mNbChannels, (int)mInH, (int)mInW, (int)mNbOutputs, 8, w.data(), mNoBias ? nullptr : b.data(), act,
+                                      inDType, &mFc));
+        mFcAct = act;
+        mDirty = false;
+    }
+    checkStatus(n2d2hip_fc_forward(mFc, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <> Registrar<FcCell> FcCell_Frame_HIP<float>::mRegistrar("Frame_HIP", FcCell_Frame_HIP<float>::create, Registrar<FcCell>::Type<float>());
+
+// ------------------------------------------------------------------- PoolCell
+const char* PoolCell::Type = "Pool";
+
+template <class T>
+PoolCell_Frame_HIP<T>::PoolCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& poolDims,
+                                          unsigned int nbOutputs, const std::vector<unsigned int>& strideDims,
+                                          const std::vector<unsigned int>& paddingDims, Pooling pooling,
+                                          const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), PoolCell(poolDims, strideDims, paddingDims, pooling)
+{
+    if (mPoolDims.size() != 2)
+        throw std::runtime_error("PoolCell: only 2D pooling is supported by Frame_HIP");
+    if (mStrideDims.empty()) mStrideDims.assign(2, 1U);
+    if (mPaddingDims.empty()) mPaddingDims.assign(2, 0U);
+    mActivation = activation;
+    if (activation)
+        throw std::runtime_error("PoolCell_Frame_HIP " + name + ": an activation on a pooling cell is not supported");
+}
+
+template <class T>
+void PoolCell_Frame_HIP<T>::setOutputsDims()
+{
+    // src/Cell/PoolCell.cpp:219-240
+    mOutW = (unsigned int)((mInW + 2 * mPaddingDims[0] - mPoolDims[0] + mStrideDims[0]) / (double)mStrideDims[0]);
+    mOutH = (unsigned int)((mInH + 2 * mPaddingDims[1] - mPoolDims[1] + mStrideDims[1]) / (double)mStrideDims[1]);
+}
+
+template <class T>
+void PoolCell_Frame_HIP<T>::initialize()
+{
+    if (mInputs.size() != 1 || mNbOutputs != mNbChannels)
+        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": one input and a unit mapping (NbOutputs == channels) are supported");
+    mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
+}
+
+template <class T>
+void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
+{
+    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype)
+        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
+    n2d2hip_pool_desc d;
+    d.pooling = mPooling == Max ? N2D2HIP_POOL_MAX : N2D2HIP_POOL_AVERAGE;
+    d.poolW = (int)mPoolDims[0]; d.poolH = (int)mPoolDims[1];
+    d.strideX = (int)mStrideDims[0]; d.strideY = (int)mStrideDims[1];
+    d.padX = (int)mPaddingDims[0]; d.padY = (int)mPaddingDims[1];
+    checkStatus(n2d2hip_pool_forward(&d, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <> Registrar<PoolCell> PoolCell_Frame_HIP<float>::mRegistrar("Frame_HIP", PoolCell_Frame_HIP<float>::create,
+                                                                      Registrar<PoolCell>::Type<float>());
+
+// --------------------------------------------------------------- ElemWiseCell
+const char* ElemWiseCell::Type = "ElemWise";
+
+std::pair<double, double> ElemWiseCell::elemWiseOutputsRange() const
+{
+    const std::pair<double, double> parents = getOutputsRangeParents();
+    const double inf = std::numeric_limits<double>::infinity();
+    if (mOperation == EuclideanSum)
+        return std::make_pair(0.0, inf);
+    if (parents.first >= 0.0) {
+        const bool shiftsPos = std::all_of(mShifts.begin(), mShifts.end(), [](Float_T v) { return v >= 0.0; });
+        const bool weightsPos = std::all_of(mWeights.begin(), mWeights.end(), [](Float_T v) { return v >= 0.0; });
+        if (mOperation == Sum && shiftsPos && weightsPos) return std::make_pair(0.0, inf);
+        if (mOperation == AbsSum && weightsPos) return std::make_pair(0.0, inf);
+        if (mOperation == Prod || mOperation == Max) return std::make_pair(0.0, inf);
+    }
+    return std::make_pair(-inf, inf);
+}
+
+ElemWiseCell_Frame_HIP::ElemWiseCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs, Operation operation,
+                                               CoeffMode mode, const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts,
+                                               const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts), mEw(nullptr), mEwAct(nullptr)
+{
+    mActivation = activation;
+    if (operation != Sum)
+        throw std::runtime_error("ElemWiseCell_Frame_HIP " + name + ": only the Sum operation is on the quantized path");
+}
+
+ElemWiseCell_Frame_HIP::~ElemWiseCell_Frame_HIP()
+{
+    if (mEw) n2d2hip_elemwise_destroy(mEw);
+}
+
+void ElemWiseCell_Frame_HIP::setOutputsDims()
+{
+    mOutW = mInW;
+    mOutH = mInH;
+}
+
+void ElemWiseCell_Frame_HIP::initialize()
+{
+    if (mNbOutputs != mNbChannels)
+        throw std::runtime_error("ElemWiseCell_Frame_HIP " + mName + ": the number of output channels must be equal to the sum of inputs channels.");
+    // src/Cell/ElemWiseCell_Frame.cpp:75-87: default 1.0 / 0.0, one entry per input (per channel when PerChannel)
+    const size_t n = mCoeffMode == PerChannel ? (size_t)mNbChannels : mInputs.size();
+    mWeights.resize(n, 1.0f);
+    mShifts.resize(n, 0.0f);
+    allocateOutputs();
+}
+
+void ElemWiseCell_Frame_HIP::propagate(bool /*inference*/)
+{
+    n2d2hip_act_t act = activationHandle();
+    if (!mEw || act != mEwAct) {
+        if (mEw) { n2d2hip_elemwise_destroy(mEw); mEw = nullptr; }
+        const int mode = mCoeffMode == PerChannel ? N2D2HIP_COEFF_PER_CHANNEL : (mCoeffMode == PerInput ? N2D2HIP_COEFF_PER_INPUT : N2D2HIP_COEFF_PER_LAYER);
+        checkStatus(n2d2hip_elemwise_create((int)mInputs.size(), (int)mNbOutputs, mode, mWeights.data(), mShifts.data(), act, &mEw));
+        mEwAct = act;
+    }
+    std::vector<const n2d2hip_tensor*> ins;
+    for (HipTensor* t : mInputs) ins.push_back(&t->desc());
+    checkStatus(n2d2hip_elemwise_forward(mEw, ins.data(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+Registrar<ElemWiseCell> ElemWiseCell_Frame_HIP::mRegistrar("Frame_HIP", ElemWiseCell_Frame_HIP::create, Registrar<ElemWiseCell>::Type<float>());
+
+// ---------------------------------------------------------------- ScalingCell
+const char* ScalingCell::Type = "Scaling";
+
+std::pair<double, double> ScalingCell::scalingOutputsRange() const
+{
+    if (mScaling.getMode() == ScalingMode::NONE)
+        throw std::runtime_error("Unsupported scaling mode for cell " + getName() + ".");
+    const bool allScalingsPositive = mScaling.allScalingsPositive();
+    const double inf = std::numeric_limits<double>::infinity();
+    const std::pair<double, double> parents = getOutputsRangeParents();
+    if (parents.first >= 0.0 && allScalingsPositive)
+        return std::make_pair(0.0, inf);
+    return std::make_pair(-inf, inf);
+}
+
+template <class T>
+ScalingCell_Frame_HIP<T>::ScalingCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs, Scaling scaling)
+    : Cell(name, nbOutputs), ScalingCell(std::move(scaling)), mScalingAct(nullptr), mBuiltRevision(~0u), mBuiltUnsigned(-1)
+{
+}
+
+template <class T>
+ScalingCell_Frame_HIP<T>::~ScalingCell_Frame_HIP()
+{
+    if (mScalingAct) n2d2hip_act_destroy(mScalingAct);
+}
+
+template <class T>
+void ScalingCell_Frame_HIP<T>::setOutputsDims()
+{
+    mOutW = mInW;
+    mOutH = mInH;
+}
+
+template <class T>
+void ScalingCell_Frame_HIP<T>::initialize()
+{
+    if (mInputs.size() != 1)
+        throw std::runtime_error("ScalingCell_Frame_HIP " + mName + ": exactly one input is supported");
+    if (mScaling.getMode() != ScalingMode::NONE)
+        allocateOutputs(&mScaling);
+}
+
+template <class T>
+void ScalingCell_Frame_HIP<T>::propagate(bool /*inference*/)
+{
+    // src/Cell/ScalingCell_Frame.cpp:67-75: mScaling.propagate(*this, in, out, mQuantizedNbBits), no activation
+    const bool uns = DeepNetExport::isCellOutputUnsigned(*this);
+    if (!mScalingAct || mBuiltRevision != mScalingRevision || mBuiltUnsigned != (int)uns) {
+        if (mScalingAct) { n2d2hip_act_destroy(mScalingAct); mScalingAct = nullptr; }
+        mScalingAct = makeAct(mScaling, N2D2HIP_ACT_LINEAR, 0.0f, mQuantizedNbBits, uns, mNbOutputs, mName);
+        mBuiltRevision = mScalingRevision;
+        mBuiltUnsigned = (int)uns;
+        if (mOutputs.empty() || mOutputs.desc().dtype != outputDType(&mScaling))
+            allocateOutputs(&mScaling);
+    }
+    checkStatus(n2d2hip_scaling_forward(mScalingAct, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <> Registrar<ScalingCell> ScalingCell_Frame_HIP<float>::mRegistrar("Frame_HIP", ScalingCell_Frame_HIP<float>::create,
+                                                                            Registrar<ScalingCell>::Type<float>());
+
+// ------------------------------------------------------------------- SGDSolver
+void SGDSolver::setParameter(const std::string& name, double value)
+{
+    if (name == "LearningRate") mLearningRate = value;
+    else if (name == "IterationSize") mIterationSize = (unsigned int)value;
+    else throw std::runtime_error("Parameter does not exist: " + name);
+}
+
+void SGDSolver::update(float& data, float diff, unsigned int batchSize)
+{
+    // include/Solver/SGDSolver_Frame.hpp:84-109 without momentum / decay: data += rate/(batch*iterSize) * diff,
+    // applied on the last pass of an iteration
+    ++mIterationPass;
+    if (mIterationPass < mIterationSize)
+        return;
+    mIterationPass = 0;
+    const float rate = (float)(mLearningRate / (double)(batchSize * mIterationSize));
+    data += rate * diff;
+}
+
+template <> Registrar<SGDSolver> SGDSolver_Frame_HIP<float>::mRegistrar("Frame_HIP", SGDSolver_Frame_HIP<float>::create,
+                                                                        Registrar<SGDSolver>::Type<float>());
+
+// ---------------------------------------------------------------- SAT weights
+const char* SATQuantizerCell::Type = "SAT";
+const char* SATQuantizerActivation::Type = "SAT";
+const char* LSQQuantizerCell::Type = "LSQ";
+const char* LSQQuantizerActivation::Type = "LSQ";
+
+static float* deviceFloats(size_t n, const char* what)
+{
+    float* p = nullptr;
+    checkHip(hipMalloc((void**)&p, n * sizeof(float)), what);
+    return p;
+}
+
+static void ensureWorkspace(void*& ws, size_t& bytes, size_t n)
+{
+    const size_t need = n2d2hip_quantizer_workspace_bytes(n);
+    if (bytes >= need) return;
+    if (ws) (void)hipFree(ws);
+    ws = nullptr;
+    checkHip(hipMalloc(&ws, need), "quantizer workspace");
+    bytes = need;
+}
+
+template <class T>
+SATQuantizerCell_Frame_HIP<T>::~SATQuantizerCell_Frame_HIP()
+{
+    for (auto& b : mW) { (void)hipFree(b.q); (void)hipFree(b.diffFp); }
+    if (mStats) (void)hipFree(mStats);
+    if (mWorkspace) (void)hipFree(mWorkspace);
+}
+
+template <class T>
+void SATQuantizerCell_Frame_HIP<T>::addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize)
+{
+    QuantizerBuffers b;
+    b.fp = weights; b.diffQ = diffQuantizedWeights; b.size = size; b.outputsSize = outputsSize;
+    b.q = deviceFloats(size, "SATQuantizerCell_Frame_HIP::addWeights()");
+    b.diffFp = deviceFloats(size, "SATQuantizerCell_Frame_HIP::addWeights()");
+    mW.push_back(b);
+    mOutputsSize += outputsSize;       // SATQuantizerCell_Frame.cpp:79: sum of dimB*dimY*dimX over the weight tensors
+}
+
+template <class T>
+int SATQuantizerCell_Frame_HIP<T>::satMode() const
+{
+    // SATQuantizerCell_Frame.cpp:188-200
+    if (mQuantMode == QuantizerCell::FullRange) return mApplyQuantization ? N2D2HIP_SAT_FULLRANGE : N2D2HIP_SAT_NONE;
+    if (mQuantMode == QuantizerCell::Symmetric) return mApplyQuantization ? N2D2HIP_SAT_SYMRANGE : N2D2HIP_SAT_NONE;
+    if (mQuantMode == QuantizerCell::Asymmetric) return mApplyQuantization ? N2D2HIP_SAT_ASYMRANGE : N2D2HIP_SAT_NONE_ASYM;
+    return mApplyQuantization ? N2D2HIP_SAT_DEFAULT : N2D2HIP_SAT_NONE;
+}
+
+template <class T>
+void SATQuantizerCell_Frame_HIP<T>::initialize()
+{
+    if (!mStats && !mW.empty())
+        mStats = deviceFloats(2 * mW.size(), "SATQuantizerCell_Frame_HIP::initialize()");
+    propagate();         // initializeQWeights
+}
+
+template <class T>
+void SATQuantizerCell_Frame_HIP<T>::propagate()
+{
+    if (!mStats && !mW.empty())
+        mStats = deviceFloats(2 * mW.size(), "SATQuantizerCell_Frame_HIP::propagate()");
+    for (size_t k = 0; k < mW.size(); ++k) {
+        ensureWorkspace(mWorkspace, mWorkspaceBytes, mW[k].size);
+        checkStatus(n2d2hip_sat_weight_forward(mW[k].fp, mW[k].q, mW[k].size, (float)mRange, satMode(), mApplyScaling ? 1 : 0,
+                                               (unsigned)mOutputsSize, mStats + 2 * k, mWorkspace, mWorkspaceBytes, mStream));
+    }
+}
+
+template <class T>
+void SATQuantizerCell_Frame_HIP<T>::back_propagate()
+{
+    for (size_t k = 0; k < mW.size(); ++k) {
+        // SATQuantizerCell_Frame.cpp:249-283: Asymmetric and FullRange select their kernel by QuantMode alone
+        int mode = N2D2HIP_SAT_DEFAULT;
+        if (mQuantMode == QuantizerCell::Asymmetric) mode = N2D2HIP_SAT_ASYMRANGE;
+        else if (mQuantMode == QuantizerCell::FullRange) mode = N2D2HIP_SAT_FULLRANGE;
+        checkStatus(n2d2hip_sat_weight_backward(mW[k].diffQ, mW[k].fp, mW[k].diffFp, mW[k].size, (float)mRange, mode, mApplyScaling ? 1 : 0,
+                                                mStats + 2 * k, mStream));
+    }
+}
+
+template <class T>
+std::pair<float, float> SATQuantizerCell_Frame_HIP<T>::getStats(unsigned int k) const
+{
+    float h[2] = {0, 0};
+    checkHip(hipMemcpy(h, mStats + 2 * k, sizeof(h), hipMemcpyDeviceToHost), "SATQuantizerCell_Frame_HIP::getStats()");
+    return std::make_pair(h[0], h[1]);
+}
+
+template <> Registrar<SATQuantizerCell> SATQuantizerCell_Frame_HIP<float>::mRegistrar("Frame_HIP", SATQuantizerCell_Frame_HIP<float>::create,
+                                                                                      Registrar<SATQuantizerCell>::Type<float>());
+
+// ------------------------------------------------------------ SAT activations
+template <class T>
+SATQuantizerActivation_Frame_HIP<T>::~SATQuantizerActivation_Frame_HIP()
+{
+    if (mDev) (void)hipFree(mDev);
+    if (mFp) (void)hipFree(mFp);
+    if (mWorkspace) (void)hipFree(mWorkspace);
+}
+
+template <class T>
+void SATQuantizerActivation_Frame_HIP<T>::lazyInit(std::size_t size, bool needCopy)
+{
+    if (!mDev) {
+        // alpha tensor {1,1,1,1} initialised from the Alpha parameter at the first propagate
+        mDev = deviceFloats(2, "SATQuantizerActivation_Frame_HIP");
+        const float h[2] = {(float)mAlphaParameter, 0.0f};
+        checkHip(hipMemcpy(mDev, h, sizeof(h), hipMemcpyHostToDevice), "SATQuantizerActivation_Frame_HIP");
+    }
+    if (needCopy && mFpSize != size) {
+        if (mFp) (void)hipFree(mFp);
+        mFp = deviceFloats(size, "SATQuantizerActivation_Frame_HIP");
+        mFpSize = size;
+    }
+}
+
+template <class T>
+void SATQuantizerActivation_Frame_HIP<T>::propagate(float* inOut, std::size_t size, bool inference)
+{
+    lazyInit(size, !inference);
+    checkStatus(n2d2hip_sat_act_forward(inOut, inference ? nullptr : mFp, size, (float)mRange, mDev, mStream));
+}
+
+template <class T>
+void SATQuantizerActivation_Frame_HIP<T>::back_propagate(const float* diffInput, float* diffOutput, std::size_t size)
+{
+    if (!mFp || mFpSize != size)
+        throw std::runtime_error("SATQuantizerActivation_Frame_HIP::back_propagate(): no full-precision activations saved (propagate with inference = false first)");
+    lazyInit(size, true);
+    ensureWorkspace(mWorkspace, mWorkspaceBytes, size);
+    const float beta = (mSolver && !mSolver->isNewIteration()) ? 1.0f : 0.0f;
+    checkStatus(n2d2hip_sat_act_backward(diffInput, mFp, diffOutput, size, (float)mRange, mDev, beta, mDev + 1, mWorkspace, mWorkspaceBytes, mStream));
+}
+
+template <class T>
+float SATQuantizerActivation_Frame_HIP<T>::getAlpha()
+{
+    lazyInit(0, false);
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev, sizeof(float), hipMemcpyDeviceToHost), "getAlpha");
+    return h;
+}
+template <class T>
+float SATQuantizerActivation_Frame_HIP<T>::getDiffAlpha()
+{
+    lazyInit(0, false);
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev + 1, sizeof(float), hipMemcpyDeviceToHost), "getDiffAlpha");
+    return h;
+}
+template <class T>
+void SATQuantizerActivation_Frame_HIP<T>::update(unsigned int batchSize)
+{
+    if (!mSolver) return;
+    float h[2];
+    lazyInit(0, false);
+    checkHip(hipMemcpy(h, mDev, sizeof(h), hipMemcpyDeviceToHost), "SATQuantizerActivation_Frame_HIP::update()");
+    mSolver->update(h[0], h[1], batchSize);
+    checkHip(hipMemcpy(mDev, h, sizeof(float), hipMemcpyHostToDevice), "SATQuantizerActivation_Frame_HIP::update()");
+}
+
+template <> Registrar<SATQuantizerActivation> SATQuantizerActivation_Frame_HIP<float>::mRegistrar(
+    "Frame_HIP", SATQuantizerActivation_Frame_HIP<float>::create, Registrar<SATQuantizerActivation>::Type<float>());
+
+// ---------------------------------------------------------------- LSQ weights
+template <class T>
+LSQQuantizerCell_Frame_HIP<T>::~LSQQuantizerCell_Frame_HIP()
+{
+    for (auto& b : mW) { (void)hipFree(b.q); (void)hipFree(b.diffFp); }
+    if (mDev) (void)hipFree(mDev);
+    if (mWorkspace) (void)hipFree(mWorkspace);
+}
+
+template <class T>
+void LSQQuantizerCell_Frame_HIP<T>::addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize)
+{
+    QuantizerBuffers b;
+    b.fp = weights; b.diffQ = diffQuantizedWeights; b.size = size; b.outputsSize = outputsSize;
+    b.q = deviceFloats(size, "LSQQuantizerCell_Frame_HIP::addWeights()");
+    b.diffFp = deviceFloats(size, "LSQQuantizerCell_Frame_HIP::addWeights()");
+    mW.push_back(b);
+}
+
+// mean(|w|) of a device tensor, for the step-size initialisation of the LSQ paper
+static double meanAbsOnHost(const float* dev, size_t n)
+{
+    std::vector<float> h(n);
+    checkHip(hipMemcpy(h.data(), dev, n * sizeof(float), hipMemcpyDeviceToHost), "LSQ step-size initialisation");
+    double s = 0.0;
+    for (float v : h) s += std::fabs((double)v);
+    return s / (double)n;
+}
+
+template <class T>
+void LSQQuantizerCell_Frame_HIP<T>::initialize()
+{
+    // LSQQuantizerCell_Frame.cpp:106-145: range [-(R+1)/2, (R-1)/2]; optimal initial step 2*mean|w|/sqrt(hi)
+    mLo = -(int)((mRange + 1) >> 1);
+    mHi = (int)((mRange - 1) >> 1);
+    size_t total = 0;
+    for (auto& b : mW) total += b.size;
+    if (!mDev) {
+        if (mSetOptInitStepSize && !mW.empty())
+            mStepSizeVal = 2.0f * (float)(meanAbsOnHost(mW[0].fp, mW[0].size) / std::sqrt((double)mHi));
+        mDev = deviceFloats(2, "LSQQuantizerCell_Frame_HIP::initialize()");
+        const float h[2] = {mStepSizeVal, 0.0f};
+        checkHip(hipMemcpy(mDev, h, sizeof(h), hipMemcpyHostToDevice), "LSQQuantizerCell_Frame_HIP::initialize()");
+    }
+    mGradScale = (float)(1.0 / std::sqrt((double)total * (double)mHi));
+    mInitialized = true;
+    propagate();
+}
+
+template <class T>
+void LSQQuantizerCell_Frame_HIP<T>::propagate()
+{
+    if (!mInitialized) { initialize(); return; }
+    for (auto& b : mW)
+        checkStatus(n2d2hip_lsq_forward(b.fp, b.q, b.size, mDev, mLo, mHi, nullptr));
+}
+
+template <class T>
+void LSQQuantizerCell_Frame_HIP<T>::back_propagate()
+{
+    if (!mInitialized)
+        throw std::runtime_error("LSQQuantizerCell_Frame_HIP::back_propagate(): not initialized");
+    // the step-size gradient accumulates over the weight tensors of the cell and, inside one solver
+    // iteration, over passes; the scale factor is applied once per call as the reference does
+    float beta = (mSolver && !mSolver->isNewIteration()) ? 1.0f : 0.0f;
+    for (size_t k = 0; k < mW.size(); ++k) {
+        ensureWorkspace(mWorkspace, mWorkspaceBytes, mW[k].size);
+        const bool last = k + 1 == mW.size();
+        checkStatus(n2d2hip_lsq_backward(mW[k].diffQ, mW[k].fp, mW[k].diffFp, mW[k].size, mDev, mLo, mHi, last ? mGradScale : 1.0f, beta,
+                                         mDev + 1, mWorkspace, mWorkspaceBytes, nullptr));
+        beta = 1.0f;
+    }
+}
+
+template <class T>
+float LSQQuantizerCell_Frame_HIP<T>::getStepSize()
+{
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev, sizeof(float), hipMemcpyDeviceToHost), "getStepSize");
+    return h;
+}
+template <class T>
+float LSQQuantizerCell_Frame_HIP<T>::getDiffStepSize()
+{
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev + 1, sizeof(float), hipMemcpyDeviceToHost), "getDiffStepSize");
+    return h;
+}
+template <class T>
+void LSQQuantizerCell_Frame_HIP<T>::update(unsigned int batchSize)
+{
+    if (!mSolver) return;
+    float h[2];
+    checkHip(hipMemcpy(h, mDev, sizeof(h), hipMemcpyDeviceToHost), "LSQQuantizerCell_Frame_HIP::update()");
+    mSolver->update(h[0], h[1], batchSize);
+    checkHip(hipMemcpy(mDev, h, sizeof(float), hipMemcpyHostToDevice), "LSQQuantizerCell_Frame_HIP::update()");
+}
+
+template <> Registrar<LSQQuantizerCell> LSQQuantizerCell_Frame_HIP<float>::mRegistrar("Frame_HIP", LSQQuantizerCell_Frame_HIP<float>::create,
+                                                                                      Registrar<LSQQuantizerCell>::Type<float>());
+
+// ------------------------------------------------------------ LSQ activations
+template <class T>
+LSQQuantizerActivation_Frame_HIP<T>::~LSQQuantizerActivation_Frame_HIP()
+{
+    if (mDev) (void)hipFree(mDev);
+    if (mFp) (void)hipFree(mFp);
+    if (mWorkspace) (void)hipFree(mWorkspace);
+}
+
+template <class T>
+void LSQQuantizerActivation_Frame_HIP<T>::propagate(float* inOut, std::size_t size, bool /*inference*/)
+{
+    // LSQQuantizerActivation_Frame.cpp:92-141: range [0, R]; the full-precision input is always saved
+    mGradScale = (float)(1.0 / std::sqrt((double)size * (double)mRange));
+    if (!mDev) {
+        if (mSetOptInitStepSize) {
+            std::vector<float> h(size);
+            checkHip(hipMemcpy(h.data(), inOut, size * sizeof(float), hipMemcpyDeviceToHost), "LSQ activation step-size initialisation");
+            double s = 0.0;
+            for (float v : h) s += std::fabs((double)v);
+            mStepSizeParameter = 2.0f * (float)((s / (double)size) / std::sqrt((double)mRange));
+            mSetOptInitStepSize = false;
+        }
+        mDev = deviceFloats(2, "LSQQuantizerActivation_Frame_HIP");
+        const float h2[2] = {mStepSizeParameter, 0.0f};
+        checkHip(hipMemcpy(mDev, h2, sizeof(h2), hipMemcpyHostToDevice), "LSQQuantizerActivation_Frame_HIP");
+    }
+    if (mFpSize != size) {
+        if (mFp) (void)hipFree(mFp);
+        mFp = deviceFloats(size, "LSQQuantizerActivation_Frame_HIP");
+        mFpSize = size;
+    }
+    checkHip(hipMemcpyAsync(mFp, inOut, size * sizeof(float), hipMemcpyDeviceToDevice, nullptr), "LSQQuantizerActivation_Frame_HIP::propagate()");
+    checkStatus(n2d2hip_lsq_forward(mFp, inOut, size, mDev, 0, (int)mRange, nullptr));
+}
+
+template <class T>
+void LSQQuantizerActivation_Frame_HIP<T>::back_propagate(const float* diffInput, float* diffOutput, std::size_t size)
+{
+    if (!mDev || !mFp || mFpSize != size)
+        throw std::runtime_error("LSQQuantizerActivation_Frame_HIP::back_propagate(): propagate first");
+    ensureWorkspace(mWorkspace, mWorkspaceBytes, size);
+    const float beta = (mSolver && !mSolver->isNewIteration()) ? 1.0f : 0.0f;
+    checkStatus(n2d2hip_lsq_backward(diffInput, mFp, diffOutput, size, mDev, 0, (int)mRange, mGradScale, beta, mDev + 1, mWorkspace,
+                                     mWorkspaceBytes, nullptr));
+}
+
+template <class T>
+float LSQQuantizerActivation_Frame_HIP<T>::getStepSize()
+{
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev, sizeof(float), hipMemcpyDeviceToHost), "getStepSize");
+    return h;
+}
+template <class T>
+float LSQQuantizerActivation_Frame_HIP<T>::getDiffStepSize()
+{
+    float h = 0;
+    checkHip(hipMemcpy(&h, mDev + 1, sizeof(float), hipMemcpyDeviceToHost), "getDiffStepSize");
+    return h;
+}
+template <class T>
+void LSQQuantizerActivation_Frame_HIP<T>::update(unsigned int batchSize)
+{
+    if (!mSolver || !mDev) return;
+    float h[2];
+    checkHip(hipMemcpy(h, mDev, sizeof(h), hipMemcpyDeviceToHost), "LSQQuantizerActivation_Frame_HIP::update()");
+    mSolver->update(h[0], h[1], batchSize);
+    checkHip(hipMemcpy(mDev, h, sizeof(float), hipMemcpyHostToDevice), "LSQQuantizerActivation_Frame_HIP::update()");
+}
+
+template <> Registrar<LSQQuantizerActivation> LSQQuantizerActivation_Frame_HIP<float>::mRegistrar(
+    "Frame_HIP", LSQQuantizerActivation_Frame_HIP<float>::create, Registrar<LSQQuantizerActivation>::Type<float>());
+
+template class SATQuantizerCell_Frame_HIP<float>;
+template class SATQuantizerActivation_Frame_HIP<float>;
+template class LSQQuantizerCell_Frame_HIP<float>;
+template class LSQQuantizerActivation_Frame_HIP<float>;
+template class ConvCell_Frame_HIP<float>;
+template class FcCell_Frame_HIP<float>;
+template class PoolCell_Frame_HIP<float>;
+template class ScalingCell_Frame_HIP<float>;
+
+// -------------------------------------------------------------------- DeepNet
+void DeepNet::addCell(const std::shared_ptr<Cell>& cell, const std::vector<std::shared_ptr<Cell> >& parents)
+{
+    if (mCells.count(cell->getName()))
+        throw std::runtime_error("DeepNet::addCell(): cell " + cell->getName() + " already exists");
+    auto frame = std::dynamic_pointer_cast<Cell_Frame_HIP>(cell);
+    if (!frame)
+        throw std::runtime_error("DeepNet::addCell(): cell " + cell->getName() + " is not a Frame_HIP cell");
+    if (parents.empty()) {
+        if (mEnvB == 0)
+            throw std::runtime_error("DeepNet::addCell(): set the stimuli size before connecting cell " + cell->getName() + " to the environment");
+        frame->addInput(mStimuli, mEnvC, mEnvH, mEnvW, mEnvB);
+    }
+    for (const auto& p : parents) {
+        auto pf = std::dynamic_pointer_cast<Cell_Frame_HIP>(p);
+        if (!pf)
+            throw std::runtime_error("DeepNet::addCell(): parent of " + cell->getName() + " is not a Frame_HIP cell");
+        frame->addInput(pf.get());
+    }
+    mOrder.push_back(cell);
+    mCells[cell->getName()] = cell;
+}
+
+std::shared_ptr<Cell> DeepNet::getCell(const std::string& name) const
+{
+    auto it = mCells.find(name);
+    if (it == mCells.end())
+        throw std::runtime_error("DeepNet::getCell(): layer " + name + " does not exist");
+    return it->second;
+}
+
+void DeepNet::setStimuli(unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize)
+{
+    mEnvC = nbChannels; mEnvH = height; mEnvW = width; mEnvB = batchSize;
+}
+
+void DeepNet::setStimuliData(const Tensor<Float_T>& data)
+{
+    // network input unsigned <=> DeepNetExport::mEnvDataUnsigned (StimuliProviderExport::unsignedStimuli)
+    const int dtype = (CellExport::mPrecision > 0 && DeepNetExport::mUnsignedData && DeepNetExport::mEnvDataUnsigned) ? N2D2HIP_U8B : N2D2HIP_I8;
+    if (mStimuli.empty() || mStimuli.desc().dtype != dtype)
+        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype);
+    for (size_t i = 0; i < data.size(); ++i)
+        toInteger(data(i), dtype == N2D2HIP_U8B ? 0 : -128, dtype == N2D2HIP_U8B ? 255 : 127, "stimuli");
+    mStimuli.synchronizeHToD(data);
+}
+
+void DeepNet::initialize()
+{
+    const int dtype = (CellExport::mPrecision > 0 && DeepNetExport::mUnsignedData && DeepNetExport::mEnvDataUnsigned) ? N2D2HIP_U8B : N2D2HIP_I8;
+    if (mEnvB > 0 && mStimuli.empty())
+        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype);
+    for (auto& c : mOrder)
+        std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->initialize();
+}
+
+void DeepNet::propagate(bool inference)
+{
+    for (auto& c : mOrder)
+        std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->propagate(inference);
+}
+
+void DeepNet::synchronize()
+{
+    checkHip(hipDeviceSynchronize(), "DeepNet::synchronize()");
+}
+
+// ------------------------------------------------------------------ INI subset
+namespace {
+std::string trim(const std::string& s)
+{
+    const size_t a = s.find_first_not_of(" \t\r\n");
+    if (a == std::string::npos) return "";
+    const size_t b = s.find_last_not_of(" \t\r\n");
+    return s.substr(a, b - a + 1);
+}
+std::vector<std::string> split(const std::string& s, const std::string& seps)
+{
+    std::vector<std::string> out;
+    size_t pos = 0;
+    while (pos <= s.size()) {
+        const size_t next = s.find_first_of(seps, pos);
+        const std::string tok = trim(s.substr(pos, next == std::string::npos ? std::string::npos : next - pos));
+        if (!tok.empty()) out.push_back(tok);
+        if (next == std::string::npos) break;
+        pos = next + 1;
+    }
+    return out;
+}
+typedef std::map<std::string, std::string> Section;
+unsigned int getUInt(const Section& s, const std::string& key, unsigned int def, bool required = false, const std::string& sec = "")
+{
+    auto it = s.find(key);
+    if (it == s.end()) {
+        if (required) throw std::runtime_error("Missing parameter " + key + " in section [" + sec + "]");
+        return def;
+    }
+    return (unsigned int)std::stoul(it->second);
+}
+std::vector<unsigned int> getDims(const Section& s, const std::string& vec, const std::string& scalar, const std::string& x, const std::string& y,
+                                  unsigned int def)
+{
+    auto it = s.find(vec);
+    if (it != s.end()) {
+        std::vector<unsigned int> v;
+        for (const auto& t : split(it->second, " \t")) v.push_back((unsigned int)std::stoul(t));
+        if (v.size() == 1) v.push_back(v[0]);
+        return v;
+    }
+    const unsigned int both = getUInt(s, scalar, def);
+    return {getUInt(s, x, both), getUInt(s, y, both)};
+}
+} // namespace
+
+std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string* modelOut)
+{
+    std::vector<std::string> order;
+    std::map<std::string, Section> sections;
+    std::map<std::string, std::string> inherits;
+    Section global;
+    std::string current;
+    std::istringstream in(iniText);
+    std::string line;
+    while (std::getline(in, line)) {
+        const size_t c = line.find(';');
+        if (c != std::string::npos) line = line.substr(0, c);
+        line = trim(line);
+        if (line.empty()) continue;
+        if (line[0] == '[') {
+            const size_t end = line.find(']');
+            if (end == std::string::npos) throw std::runtime_error("Malformed section header: " + line);
+            current = trim(line.substr(1, end - 1));
+            const std::string parent = trim(line.substr(end + 1));
+            if (!parent.empty()) inherits[current] = parent;
+            if (!sections.count(current)) order.push_back(current);
+            sections[current];
+            continue;
+        }
+        const size_t eq = line.find('=');
+        if (eq == std::string::npos) throw std::runtime_error("Malformed line: " + line);
+        const std::string key = trim(line.substr(0, eq)), value = trim(line.substr(eq + 1));
+        if (current.empty()) global[key] = value; else sections[current][key] = value;
+    }
+    auto resolved = [&](const std::string& name) {
+        Section s;
+        auto ih = inherits.find(name);
+        if (ih != inherits.end()) {
+            auto base = sections.find(ih->second);
+            if (base == sections.end()) throw std::runtime_error("Section [" + name + "] inherits from unknown section " + ih->second);
+            s = base->second;
+        }
+        for (const auto& kv : sections[name]) s[kv.first] = kv.second;
+        return s;
+    };
+
+    // src/Generator/DeepNetGenerator.cpp:124-125
+    const std::string model = global.count("DefaultModel") ? global["DefaultModel"] : "Frame";
+    if (modelOut) *modelOut = model;
+    auto deepNet = std::make_shared<DeepNet>();
+    Network net;
+    std::string envName;
+    for (const std::string& n : {std::string("sp"), std::string("env")})
+        if (sections.count(n)) envName = n;
+    if (envName.empty()) throw std::runtime_error("Missing [sp] or [env] section");
+    {
+        const Section env = resolved(envName);
+        deepNet->setStimuli(getUInt(env, "NbChannels", 1), getUInt(env, "SizeY", 0, true, envName), getUInt(env, "SizeX", 0, true, envName),
+                            getUInt(env, "BatchSize", 1));
+    }
+    auto makeActivation = [&](const Section& s, const std::string& name) -> std::shared_ptr<Activation> {
+        auto it = s.find("ActivationFunction");
+        if (it == s.end() || it->second == "None") return std::shared_ptr<Activation>();
+        if (it->second == "Rectifier") {
+            // src/Generator/RectifierActivationGenerator.cpp:31-43: same model key as the cells
+            auto f = Registrar<RectifierActivation>::create<float>(model);
+            if (!f) throw std::runtime_error("Activation model \"" + model + "\" is not valid in section [" + name + "]");
+            return f();
+        }
+        if (it->second == "Linear") {
+            auto f = Registrar<LinearActivation>::create<float>(model);
+            if (!f) throw std::runtime_error("Activation model \"" + model + "\" is not valid in section [" + name + "]");
+            return f();
+        }
+        throw std::runtime_error("Activation " + it->second + " is not on the quantized path (section [" + name + "])");
+    };
+
+    for (const std::string& name : order) {
+        const Section s = resolved(name);
+        if (!s.count("Type") || !s.count("Input")) continue;       // template / config sections
+        const std::string type = s.at("Type");
+        std::vector<std::shared_ptr<Cell> > parents;
+        for (const std::string& p : split(s.at("Input"), ","))
+            if (p != envName) parents.push_back(deepNet->getCell(p));
+        std::shared_ptr<Cell> cell;
+        if (type == "Conv") {
+            auto f = Registrar<ConvCell>::create<float>(model);
+            if (!f) // src/Generator/ConvCellGenerator.cpp:191-195
+                throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
+            const std::vector<unsigned int> stride = getDims(s, "StrideDims", "Stride", "StrideX", "StrideY", 1);
+            const std::vector<unsigned int> padU = getDims(s, "PaddingDims", "Padding", "PaddingX", "PaddingY", 0);
+            auto conv = f(net, *deepNet, name, getDims(s, "KernelDims", "KernelSize", "KernelWidth", "KernelHeight", 1),
+                          getUInt(s, "NbOutputs", 0, true, name), getDims(s, "SubSampleDims", "SubSample", "SubSampleX", "SubSampleY", 1), stride,
+                          std::vector<int>{(int)padU[0], (int)padU[1]}, getDims(s, "DilationDims", "Dilation", "DilationX", "DilationY", 1),
+                          makeActivation(s, name));
+            if (s.count("NoBias")) conv->setParameter("NoBias", s.at("NoBias") != "0");
+            cell = conv;
+        } else if (type == "Fc") {
+            auto f = Registrar<FcCell>::create<float>(model);
+            if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
+            auto fc = f(net, *deepNet, name, getUInt(s, "NbOutputs", 0, true, name), makeActivation(s, name));
+            if (s.count("NoBias")) fc->setParameter("NoBias", s.at("NoBias") != "0");
+            cell = fc;
+        } else if (type == "Pool") {
+            auto f = Registrar<PoolCell>::create<float>(model);
+            if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
+            const std::string pooling = s.count("Pooling") ? s.at("Pooling") : "Max";
+            if (pooling != "Max" && pooling != "Average") throw std::runtime_error("Unknown pooling " + pooling + " in section [" + name + "]");
+            cell = f(net, *deepNet, name, getDims(s, "PoolDims", "PoolSize", "PoolWidth", "PoolHeight", 1), getUInt(s, "NbOutputs", 0, true, name),
+                     getDims(s, "StrideDims", "Stride", "StrideX", "StrideY", 1), getDims(s, "PaddingDims", "Padding", "PaddingX", "PaddingY", 0),
+                     pooling == "Max" ? PoolCell::Max : PoolCell::Average, makeActivation(s, name));
+        } else if (type == "ElemWise") {
+            auto f = Registrar<ElemWiseCell>::create<float>(model);
+            if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
+            const std::string op = s.count("Operation") ? s.at("Operation") : "Sum";
+            if (op != "Sum") throw std::runtime_error("ElemWise operation " + op + " is not on the quantized path (section [" + name + "])");
+            cell = f(net, *deepNet, name, getUInt(s, "NbOutputs", 0, true, name), ElemWiseCell::Sum, ElemWiseCell::PerLayer, std::vector<Float_T>(),
+                     std::vector<Float_T>(), makeActivation(s, name));
+        } else if (type == "Scaling") {
+            auto f = Registrar<ScalingCell>::create<float>(model);
+            if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
+            cell = f(*deepNet, name, getUInt(s, "NbOutputs", 0, true, name), Scaling());
+        } else {
+            throw std::runtime_error("Cell type " + type + " is not on the quantized path (section [" + name + "])");
+        }
+        deepNet->addCell(cell, parents);
+        if (type == "Conv") {
+            const unsigned int perGroup = getUInt(s, "Mapping.ChannelsPerGroup", 0);
+            const unsigned int groups = perGroup ? cell->getNbChannels() / perGroup : getUInt(s, "Mapping.NbGroups", 1);
+            if (groups > 1) std::dynamic_pointer_cast<ConvCell>(cell)->setNbGroups(groups);
+        }
+    }
+    return deepNet;
+}
+
+} // namespace N2D2

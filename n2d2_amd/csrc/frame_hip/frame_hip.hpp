@@ -1,0 +1,900 @@
+// Host side of the "Frame_HIP" model: C++ cells that plug into N2D2's Registrar
+// under the key "Frame_HIP" and drive the HIP kernels through the C ABI of
+// n2d2hip.h.  The classes mirror the N2D2 interfaces they stand in for (same
+// names, constructor / factory signatures, parameter names and error behaviour);
+// each cites the reference header it follows (paths relative to the N2D2 tree).
+//
+// This file also carries the small amount of N2D2 infrastructure the cells need
+// to run without an N2D2 checkout (Registrar, Tensor, Scaling, a layer-ordered
+// DeepNet): in an N2D2 build those come from N2D2's own headers and only the
+// *_Frame_HIP classes and their registrations are compiled in (N2D2_EXTRAMODULE).
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <functional>
+#include <iostream>
+#include <limits>
+#include <map>
+#include <memory>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <typeindex>
+#include <utility>
+#include <vector>
+
+#include "n2d2hip.h"
+
+namespace N2D2 {
+
+typedef float Float_T;
+
+// ------------------------------------------------------------------ Registrar
+// Semantics of include/utils/Registrar.hpp:46-149: a static object whose constructor files a
+// factory under (key, type); a duplicate (key, type) throws; an unknown key or type prints a
+// message and yields an empty function.
+struct BaseCommand {
+    virtual ~BaseCommand() {}
+};
+typedef std::map<std::string, std::map<std::type_index, std::unique_ptr<BaseCommand> > > RegistryMap_T;
+
+template <typename C, typename F = typename C::RegistryCreate_T>
+struct Registrar {
+    struct Command : public BaseCommand {
+        F mFunc;
+        explicit Command(F func) : mFunc(func) {}
+    };
+    template <class T>
+    struct Type {};
+
+    template <class T = void>
+    Registrar(const std::string& key, F func, const Type<T>& = Type<T>())
+    {
+        auto& perType = C::registry()[key];
+        const std::type_index idx(typeid(T));
+        if (perType.count(idx))
+            throw std::runtime_error("Registrar \"" + key + "\" already exists");
+        perType[idx].reset(new Command(func));
+    }
+    static bool exists(const std::string& key) { return C::registry().count(key) != 0; }
+    template <class T>
+    static bool exists(const std::string& key)
+    {
+        auto it = C::registry().find(key);
+        return it != C::registry().end() && it->second.count(std::type_index(typeid(T))) != 0;
+    }
+    template <class T = void>
+    static F create(const std::string& key)
+    {
+        auto it = C::registry().find(key);
+        if (it == C::registry().end()) {
+            std::cout << "Invalid registrar key \"" << key << "\"" << std::endl;
+            return F();
+        }
+        auto itType = it->second.find(std::type_index(typeid(T)));
+        if (itType == it->second.end()) {
+            std::cout << "Invalid registrar key type (" << typeid(T).name() << ") for key \"" << key << "\"" << std::endl;
+            return F();
+        }
+        return static_cast<Command*>(itType->second.get())->mFunc;
+    }
+};
+
+// --------------------------------------------------------------------- Tensor
+// Host tensor with N2D2's dimension order {X, Y, Z, B}, X fastest
+// (include/containers/Tensor.hpp:162-193).
+template <class T>
+class Tensor {
+public:
+    Tensor() : mDims{0, 0, 0, 0} {}
+    explicit Tensor(const std::vector<size_t>& dims, T value = T()) { resize(dims, value); }
+    void resize(const std::vector<size_t>& dims, T value = T())
+    {
+        mDims = dims;
+        while (mDims.size() < 4) mDims.push_back(1);
+        mData.assign(size(), value);
+    }
+    size_t dimX() const { return mDims[0]; }
+    size_t dimY() const { return mDims[1]; }
+    size_t dimZ() const { return mDims[2]; }
+    size_t dimB() const { return mDims[3]; }
+    const std::vector<size_t>& dims() const { return mDims; }
+    size_t size() const { return mDims[0] * mDims[1] * mDims[2] * mDims[3]; }
+    bool empty() const { return mData.empty(); }
+    T& operator()(size_t i) { return mData[i]; }
+    const T& operator()(size_t i) const { return mData[i]; }
+    T& operator()(size_t x, size_t y, size_t z, size_t b) { return mData[x + mDims[0] * (y + mDims[1] * (z + mDims[2] * b))]; }
+    const T& operator()(size_t x, size_t y, size_t z, size_t b) const { return mData[x + mDims[0] * (y + mDims[1] * (z + mDims[2] * b))]; }
+    T* data() { return mData.data(); }
+    const T* data() const { return mData.data(); }
+    void fill(T v) { std::fill(mData.begin(), mData.end(), v); }
+
+private:
+    std::vector<size_t> mDims;
+    std::vector<T> mData;
+};
+
+// Throws std::runtime_error carrying the library's message when a C-ABI call fails:
+// the reference reports every error as a C++ exception.
+void checkStatus(int status);
+
+// Device tensor of a Frame_HIP cell: narrow integer storage in the private NHWC form,
+// with a host float mirror refreshed on demand so that Frame cells, Targets or tests can
+// still read N2D2-style float tensors (the role CudaTensor plays, include/containers/CudaTensor.hpp:256-359).
+class HipTensor {
+public:
+    HipTensor() : mDesc(), mBytes(0), mHostValid(false) {}
+    ~HipTensor();
+    HipTensor(const HipTensor&) = delete;
+    HipTensor& operator=(const HipTensor&) = delete;
+    void resize(int B, int C, int H, int W, int dtype);
+    const n2d2hip_tensor& desc() const { return mDesc; }
+    bool empty() const { return mDesc.data == nullptr; }
+    void invalidateHost() { mHostValid = false; }
+    // Integer-valued floats, NCHW / {W,H,C,B}
+    const Tensor<Float_T>& synchronizeDToH(void* stream = nullptr);
+    void synchronizeHToD(const Tensor<Float_T>& host, void* stream = nullptr);
+
+private:
+    n2d2hip_tensor mDesc;
+    size_t mBytes;
+    Tensor<Float_T> mHost;
+    bool mHostValid;
+};
+
+// ---------------------------------------------------------------- ScalingMode
+// include/ScalingMode.hpp:27-62
+enum class ScalingMode { NONE, FLOAT_MULT, FIXED_MULT16, FIXED_MULT32, SINGLE_SHIFT, DOUBLE_SHIFT };
+ScalingMode parseScalingMode(const std::string& str);
+
+// -------------------------------------------------------------------- Scaling
+// Value type with the factories and getters of include/Scaling.hpp:336-432.
+class Scaling {
+public:
+    Scaling() : mMode(ScalingMode::NONE), mNbFractionalBits(0), mIsClipped(false) {}
+    static Scaling floatingPointScaling(std::vector<Float_T> scalingPerOutput, bool isClipped, std::vector<Float_T> clippingPerOutput)
+    {
+        Scaling s;
+        s.mMode = ScalingMode::FLOAT_MULT;
+        s.mFloat = std::move(scalingPerOutput);
+        s.mIsClipped = isClipped;
+        s.mClipping = std::move(clippingPerOutput);
+        return s;
+    }
+    static Scaling fixedPointScaling(ScalingMode mode, std::size_t nbFractionalBits, std::vector<std::int32_t> scalingPerOutput,
+                                     bool isClipped, std::vector<Float_T> clippingPerOutput)
+    {
+        if (mode != ScalingMode::FIXED_MULT16 && mode != ScalingMode::FIXED_MULT32)
+            throw std::runtime_error("Scaling::fixedPointScaling(): mode must be FIXED_MULT16 or FIXED_MULT32");
+        Scaling s;
+        s.mMode = mode;
+        s.mNbFractionalBits = nbFractionalBits;
+        s.mFixed = std::move(scalingPerOutput);
+        s.mIsClipped = isClipped;
+        s.mClipping = std::move(clippingPerOutput);
+        return s;
+    }
+    static Scaling singleShiftScaling(std::vector<unsigned char> scalingPerOutput, bool isClipped, std::vector<Float_T> clippingPerOutput)
+    {
+        Scaling s;
+        s.mMode = ScalingMode::SINGLE_SHIFT;
+        s.mShift = std::move(scalingPerOutput);
+        s.mIsClipped = isClipped;
+        s.mClipping = std::move(clippingPerOutput);
+        return s;
+    }
+    static Scaling doubleShiftScaling(std::vector<std::pair<unsigned char, unsigned char> > scalingPerOutput, bool isClipped,
+                                      std::vector<std::pair<unsigned char, unsigned char> > /*clippingPerOutput*/)
+    {
+        Scaling s;
+        s.mMode = ScalingMode::DOUBLE_SHIFT;
+        for (const auto& p : scalingPerOutput) {
+            s.mShift.push_back(p.first);
+            s.mShift.push_back(p.second);
+        }
+        s.mIsClipped = isClipped;
+        return s;
+    }
+    ScalingMode getMode() const { return mMode; }
+    const std::vector<Float_T>& getFloatScalingPerOutput() const { return mFloat; }
+    const std::vector<std::int32_t>& getFixedScalingPerOutput() const { return mFixed; }
+    const std::vector<unsigned char>& getShiftScalingPerOutput() const { return mShift; }
+    std::size_t getFractionalBits() const { return mNbFractionalBits; }
+    bool getIsClipped() const { return mIsClipped; }
+    const std::vector<Float_T>& getClippingPerOutput() const { return mClipping; }
+    // true when every factor is >= 0 (ScalingCell::getOutputsRange, src/Cell/ScalingCell.cpp:68-104)
+    bool allScalingsPositive() const;
+    std::size_t nbOutputs() const;
+
+private:
+    ScalingMode mMode;
+    std::size_t mNbFractionalBits;
+    std::vector<Float_T> mFloat;
+    std::vector<std::int32_t> mFixed;
+    std::vector<unsigned char> mShift;     // SINGLE_SHIFT: one per output; DOUBLE_SHIFT: {first, second} per output
+    bool mIsClipped;
+    std::vector<Float_T> mClipping;
+};
+
+class Cell;
+class Cell_Frame_HIP;
+class DeepNet;
+class Network {};
+
+// Static state that decides the saturation range (src/Export/DeepNetExport.cpp:370-388,
+// set by calibNetwork, src/utils/Helper.cpp:670-673).
+struct CellExport {
+    static int mPrecision;
+};
+struct DeepNetExport {
+    static bool mUnsignedData;
+    static bool mEnvDataUnsigned;
+    static bool isCellOutputUnsigned(const Cell& cell);
+};
+
+// ----------------------------------------------------------------- Activation
+// include/Activation/Activation.hpp:36-110
+class Activation {
+public:
+    virtual ~Activation() {}
+    virtual const char* getType() const = 0;
+    virtual std::pair<double, double> getOutputRange() const = 0;
+    const Scaling& getActivationScaling() const { return mScaling; }
+    void setActivationScaling(Scaling scaling) { mScaling = std::move(scaling); ++mRevision; }
+    void setQuantized(std::size_t nbBits) { mQuantizedNbBits = nbBits; ++mRevision; }
+    std::size_t getQuantizedNbBits() const { return mQuantizedNbBits; }
+    virtual void setParameter(const std::string& name, double value) = 0;
+    unsigned revision() const { return mRevision; }
+    // kind / leak for the C ABI
+    virtual int abiKind() const = 0;
+    virtual float leakSlope() const { return 0.0f; }
+
+protected:
+    Activation() : mQuantizedNbBits(0), mRevision(0) {}
+    Scaling mScaling;
+    std::size_t mQuantizedNbBits;
+    unsigned mRevision;
+};
+
+// src/Activation/RectifierActivation.cpp:26-40 (LeakSlope 0.0, Clipping 0.0)
+class RectifierActivation : public Activation {
+public:
+    typedef std::function<std::shared_ptr<RectifierActivation>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    RectifierActivation() : mLeakSlope(0.0), mClipping(0.0) {}
+    const char* getType() const { return Type; }
+    std::pair<double, double> getOutputRange() const
+    {
+        const double max = mClipping > 0.0 ? mClipping : std::numeric_limits<double>::infinity();
+        return mLeakSlope > 0.0 ? std::make_pair(-max, max) : std::make_pair(0.0, max);
+    }
+    void setParameter(const std::string& name, double value);
+    int abiKind() const { return N2D2HIP_ACT_RECTIFIER; }
+    float leakSlope() const { return (float)mLeakSlope; }
+
+protected:
+    double mLeakSlope, mClipping;
+};
+
+// src/Activation/LinearActivation.cpp:24-25 (Clipping 0.0)
+class LinearActivation : public Activation {
+public:
+    typedef std::function<std::shared_ptr<LinearActivation>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    LinearActivation() : mClipping(0.0) {}
+    const char* getType() const { return Type; }
+    std::pair<double, double> getOutputRange() const
+    {
+        const double inf = std::numeric_limits<double>::infinity();
+        return mClipping > 0.0 ? std::make_pair(-mClipping, mClipping) : std::make_pair(-inf, inf);
+    }
+    void setParameter(const std::string& name, double value);
+    int abiKind() const { return N2D2HIP_ACT_LINEAR; }
+
+protected:
+    double mClipping;
+};
+
+template <class T>
+class RectifierActivation_Frame_HIP : public RectifierActivation {
+public:
+    static std::shared_ptr<RectifierActivation> create() { return std::make_shared<RectifierActivation_Frame_HIP<T> >(); }
+private:
+    static Registrar<RectifierActivation> mRegistrar;
+};
+template <class T>
+class LinearActivation_Frame_HIP : public LinearActivation {
+public:
+    static std::shared_ptr<LinearActivation> create() { return std::make_shared<LinearActivation_Frame_HIP<T> >(); }
+private:
+    static Registrar<LinearActivation> mRegistrar;
+};
+
+// ----------------------------------------------------------------------- Cell
+// The part of include/Cell/Cell.hpp + include/Cell/Cell_Frame_Top.hpp the quantized path uses.
+class Cell {
+public:
+    virtual ~Cell() {}
+    virtual const char* getType() const = 0;
+    const std::string& getName() const { return mName; }
+    unsigned int getNbOutputs() const { return mNbOutputs; }
+    unsigned int getNbChannels() const { return mNbChannels; }
+    unsigned int getChannelsWidth() const { return mInW; }
+    unsigned int getChannelsHeight() const { return mInH; }
+    unsigned int getOutputsWidth() const { return mOutW; }
+    unsigned int getOutputsHeight() const { return mOutH; }
+    void setQuantized(std::size_t nbBits) { mQuantizedNbBits = nbBits; }
+    bool isQuantized() const { return mQuantizedNbBits > 0; }
+    std::size_t getQuantizedNbBits() const { return mQuantizedNbBits; }
+    const std::vector<Cell*>& getParentsCells() const { return mParents; }   // nullptr entry = the environment
+    // Cell_Frame_Top::getOutputsRange, include/Cell/Cell_Frame_Top.hpp:118-121
+    virtual std::pair<double, double> getOutputsRange() const
+    {
+        const double inf = std::numeric_limits<double>::infinity();
+        return mActivation ? mActivation->getOutputRange() : std::make_pair(-inf, inf);
+    }
+    // Cell::getOutputsRangeParents, src/Cell/Cell.cpp:310-337
+    std::pair<double, double> getOutputsRangeParents() const;
+    const std::shared_ptr<Activation>& getActivation() const { return mActivation; }
+    void setActivation(const std::shared_ptr<Activation>& activation) { mActivation = activation; }
+
+protected:
+    Cell(const std::string& name, unsigned int nbOutputs)
+        : mName(name), mNbOutputs(nbOutputs), mNbChannels(0), mInW(0), mInH(0), mOutW(0), mOutH(0), mQuantizedNbBits(0) {}
+    // virtual base: only the most derived class runs the constructor above
+    Cell() : mNbOutputs(0), mNbChannels(0), mInW(0), mInH(0), mOutW(0), mOutH(0), mQuantizedNbBits(0) {}
+    std::string mName;
+    unsigned int mNbOutputs, mNbChannels, mInW, mInH, mOutW, mOutH;
+    std::size_t mQuantizedNbBits;
+    std::vector<Cell*> mParents;
+    std::shared_ptr<Activation> mActivation;
+};
+
+// Common part of the Frame_HIP cells (the role of Cell_Frame_CUDA<T>, include/Cell/Cell_Frame_CUDA.hpp:44-178).
+class Cell_Frame_HIP : public virtual Cell {
+public:
+    // Connects a parent cell (Cell::addInput(Cell*), include/Cell/Cell.hpp:265) ...
+    virtual void addInput(Cell_Frame_HIP* parent);
+    // ... or the environment: an integer-valued tensor of nbChannels x height x width per batch item
+    // (Cell::addInput(StimuliProvider&), include/Cell/Cell.hpp:208).
+    virtual void addInput(HipTensor& stimuli, unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize);
+    virtual void initialize() {}
+    virtual void propagate(bool inference = false) = 0;
+    // Outputs as N2D2 sees them: float tensor {W,H,C,B} holding integer values.
+    const Tensor<Float_T>& getOutputs();
+    HipTensor& getDeviceOutputs() { return mOutputs; }
+    bool isCuda() const { return false; }
+    std::string getPyModel() const { return "Frame_HIP"; }
+    std::string getPyDataType() const { return "float"; }
+    unsigned int batchSize() const { return mBatch; }
+    void setStream(void* stream) { mStream = stream; }
+
+protected:
+    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
+    ~Cell_Frame_HIP();
+    virtual void setOutputsDims() = 0;
+    // (Re)builds the device tables of the activation when its Scaling, its bit width or the
+    // signedness decision changed; cells without activation get a pass-through / Scaling-only table.
+    n2d2hip_act_t activationHandle(const Scaling* standalone = nullptr);
+    int outputDType(const Scaling* standalone = nullptr) const;
+    void allocateOutputs(const Scaling* standalone = nullptr);
+    std::vector<HipTensor*> mInputs;
+    HipTensor mOutputs;
+    unsigned int mBatch;
+    void* mStream;
+
+private:
+    n2d2hip_act_t mActHandle;
+    unsigned mActRevision;
+    int mActUnsigned;
+};
+
+// ------------------------------------------------------------------- ConvCell
+// include/Cell/ConvCell.hpp:41-252
+class ConvCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<ConvCell>(Network&, const DeepNet&, const std::string&, const std::vector<unsigned int>&,
+                                                    unsigned int, const std::vector<unsigned int>&, const std::vector<unsigned int>&,
+                                                    const std::vector<int>&, const std::vector<unsigned int>&,
+                                                    const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    void setParameter(const std::string& name, bool value);
+    // Depthwise / grouped connection: the regular mapping Cell::getNbGroups recognises (src/Cell/Cell.cpp:251-300).
+    void setNbGroups(unsigned int groups) { mNbGroups = groups; mDirty = true; }
+    // Weights as N2D2 holds them: float tensor {kW, kH, C/groups, O} with integer values; bias {O}.
+    void setWeights(const Tensor<Float_T>& weights) { mWeights = weights; mDirty = true; }
+    void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }
+    // 4: weights are handed to the device nibble-packed (values must fit [-8,7])
+    void setWeightsPrecision(int bits) { mWeightBits = bits; mDirty = true; }
+
+protected:
+    ConvCell(const std::vector<unsigned int>& kernelDims, const std::vector<unsigned int>& subSampleDims,
+             const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+             const std::vector<unsigned int>& dilationDims);
+    std::vector<unsigned int> mKernelDims, mSubSampleDims, mStrideDims, mDilationDims;
+    std::vector<int> mPaddingDims;
+    bool mNoBias;
+    unsigned int mNbGroups;
+    int mWeightBits;
+    Tensor<Float_T> mWeights, mBias;
+    bool mDirty;
+};
+
+template <class T>
+class ConvCell_Frame_HIP : public ConvCell, public Cell_Frame_HIP {
+public:
+    ConvCell_Frame_HIP(const DeepNet& deepNet, const std::string& name, const std::vector<unsigned int>& kernelDims,
+                       unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
+                       const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+                       const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation);
+    ~ConvCell_Frame_HIP();
+    static std::shared_ptr<ConvCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name,
+                                            const std::vector<unsigned int>& kernelDims, unsigned int nbOutputs,
+                                            const std::vector<unsigned int>& subSampleDims, const std::vector<unsigned int>& strideDims,
+                                            const std::vector<int>& paddingDims, const std::vector<unsigned int>& dilationDims,
+                                            const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<ConvCell_Frame_HIP<T> >(deepNet, name, kernelDims, nbOutputs, subSampleDims, strideDims,
+                                                        paddingDims, dilationDims, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+
+protected:
+    void setOutputsDims();
+
+private:
+    n2d2hip_conv_t mConv;
+    n2d2hip_act_t mConvAct;
+    static Registrar<ConvCell> mRegistrar;
+};
+
+// --------------------------------------------------------------------- FcCell
+// include/Cell/FcCell.hpp:43-49
+class FcCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<FcCell>(Network&, const DeepNet&, const std::string&, unsigned int,
+                                                  const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    void setParameter(const std::string& name, bool value);
+    // {K, O} float tensor (K = C*H*W in CHW order), bias {O}
+    void setWeights(const Tensor<Float_T>& weights) { mWeights = weights; mDirty = true; }
+    void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }
+
+protected:
+    FcCell() : mNoBias(false), mDirty(true) {}
+    bool mNoBias;
+    Tensor<Float_T> mWeights, mBias;
+    bool mDirty;
+};
+
+template <class T>
+class FcCell_Frame_HIP : public FcCell, public Cell_Frame_HIP {
+public:
+    FcCell_Frame_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, const std::shared_ptr<Activation>& activation);
+    ~FcCell_Frame_HIP();
+    static std::shared_ptr<FcCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                          const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<FcCell_Frame_HIP<T> >(deepNet, name, nbOutputs, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+
+protected:
+    void setOutputsDims();
+
+private:
+    n2d2hip_fc_t mFc;
+    n2d2hip_act_t mFcAct;
+    static Registrar<FcCell> mRegistrar;
+};
+
+// ------------------------------------------------------------------- PoolCell
+// include/Cell/PoolCell.hpp:47-55
+class PoolCell : public virtual Cell {
+public:
+    enum Pooling { Max, Average };
+    typedef std::function<std::shared_ptr<PoolCell>(Network&, const DeepNet&, const std::string&, const std::vector<unsigned int>&,
+                                                    unsigned int, const std::vector<unsigned int>&, const std::vector<unsigned int>&,
+                                                    Pooling, const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    Pooling getPooling() const { return mPooling; }
+
+protected:
+    PoolCell(const std::vector<unsigned int>& poolDims, const std::vector<unsigned int>& strideDims,
+             const std::vector<unsigned int>& paddingDims, Pooling pooling)
+        : mPoolDims(poolDims), mStrideDims(strideDims), mPaddingDims(paddingDims), mPooling(pooling) {}
+    std::vector<unsigned int> mPoolDims, mStrideDims, mPaddingDims;
+    Pooling mPooling;
+};
+
+template <class T>
+class PoolCell_Frame_HIP : public PoolCell, public Cell_Frame_HIP {
+public:
+    PoolCell_Frame_HIP(const DeepNet& deepNet, const std::string& name, const std::vector<unsigned int>& poolDims, unsigned int nbOutputs,
+                       const std::vector<unsigned int>& strideDims, const std::vector<unsigned int>& paddingDims, Pooling pooling,
+                       const std::shared_ptr<Activation>& activation);
+    static std::shared_ptr<PoolCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name,
+                                            const std::vector<unsigned int>& poolDims, unsigned int nbOutputs,
+                                            const std::vector<unsigned int>& strideDims, const std::vector<unsigned int>& paddingDims,
+                                            Pooling pooling, const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<PoolCell_Frame_HIP<T> >(deepNet, name, poolDims, nbOutputs, strideDims, paddingDims, pooling, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    // src/Cell/PoolCell_Frame.cpp:263-266
+    std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : getOutputsRangeParents(); }
+
+protected:
+    void setOutputsDims();
+
+private:
+    static Registrar<PoolCell> mRegistrar;
+};
+
+// --------------------------------------------------------------- ElemWiseCell
+// include/Cell/ElemWiseCell.hpp:54-63
+class ElemWiseCell : public virtual Cell {
+public:
+    enum Operation { Sum, AbsSum, EuclideanSum, Prod, Max };
+    enum CoeffMode { PerLayer, PerInput, PerChannel };
+    typedef std::function<std::shared_ptr<ElemWiseCell>(Network&, const DeepNet&, const std::string&, unsigned int, Operation, CoeffMode,
+                                                        const std::vector<Float_T>&, const std::vector<Float_T>&,
+                                                        const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    Operation getOperation() const { return mOperation; }
+    const std::vector<Float_T>& getWeights() const { return mWeights; }
+    const std::vector<Float_T>& getShifts() const { return mShifts; }
+
+protected:
+    ElemWiseCell(Operation operation, CoeffMode mode, const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts)
+        : mOperation(operation), mCoeffMode(mode), mWeights(weights), mShifts(shifts) {}
+    // src/Cell/ElemWiseCell.cpp:59-88
+    std::pair<double, double> elemWiseOutputsRange() const;
+    Operation mOperation;
+    CoeffMode mCoeffMode;
+    std::vector<Float_T> mWeights, mShifts;
+};
+
+class ElemWiseCell_Frame_HIP : public ElemWiseCell, public Cell_Frame_HIP {
+public:
+    ElemWiseCell_Frame_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, Operation operation, CoeffMode mode,
+                           const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts,
+                           const std::shared_ptr<Activation>& activation);
+    ~ElemWiseCell_Frame_HIP();
+    static std::shared_ptr<ElemWiseCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                                Operation operation, CoeffMode mode, const std::vector<Float_T>& weights,
+                                                const std::vector<Float_T>& shifts, const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<ElemWiseCell_Frame_HIP>(deepNet, name, nbOutputs, operation, mode, weights, shifts, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    // src/Cell/ElemWiseCell_Frame.cpp:313-316
+    std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : elemWiseOutputsRange(); }
+
+protected:
+    void setOutputsDims();
+
+private:
+    n2d2hip_elemwise_t mEw;
+    n2d2hip_act_t mEwAct;
+    static Registrar<ElemWiseCell> mRegistrar;
+};
+
+// ---------------------------------------------------------------- ScalingCell
+// include/Cell/ScalingCell.hpp:39-43
+class ScalingCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<ScalingCell>(const DeepNet&, const std::string&, unsigned int, Scaling)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    const Scaling& getScaling() const { return mScaling; }
+    void setScaling(Scaling scaling) { mScaling = std::move(scaling); ++mScalingRevision; }
+
+protected:
+    explicit ScalingCell(Scaling scaling) : mScaling(std::move(scaling)), mScalingRevision(0) {}
+    // src/Cell/ScalingCell.cpp:68-104
+    std::pair<double, double> scalingOutputsRange() const;
+    Scaling mScaling;
+    unsigned mScalingRevision;
+};
+
+template <class T>
+class ScalingCell_Frame_HIP : public ScalingCell, public Cell_Frame_HIP {
+public:
+    ScalingCell_Frame_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, Scaling scaling);
+    ~ScalingCell_Frame_HIP();
+    static std::shared_ptr<ScalingCell> create(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, Scaling scaling)
+    {
+        return std::make_shared<ScalingCell_Frame_HIP<T> >(deepNet, name, nbOutputs, std::move(scaling));
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    // src/Cell/ScalingCell_Frame.cpp:93-96
+    std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : scalingOutputsRange(); }
+
+protected:
+    void setOutputsDims();
+
+private:
+    n2d2hip_act_t mScalingAct;
+    unsigned mBuiltRevision;
+    int mBuiltUnsigned;
+    static Registrar<ScalingCell> mRegistrar;
+};
+
+// ------------------------------------------------------------------ quantizers
+// Solver used by the quantizers' update() (include/Solver/SGDSolver_Frame.hpp:84-109: N2D2 ADDS
+// rate/(batch*iterationSize)*diff, because its diffInputs carry target - output).
+class SGDSolver {
+public:
+    typedef std::function<std::shared_ptr<SGDSolver>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    SGDSolver() : mLearningRate(0.01), mIterationSize(1), mIterationPass(0) {}
+    virtual ~SGDSolver() {}
+    void setParameter(const std::string& name, double value);
+    bool isNewIteration() const { return mIterationPass == 0; }
+    // scalar parameter update on the host
+    void update(float& data, float diff, unsigned int batchSize);
+
+protected:
+    double mLearningRate;
+    unsigned int mIterationSize, mIterationPass;
+};
+template <class T>
+class SGDSolver_Frame_HIP : public SGDSolver {
+public:
+    static std::shared_ptr<SGDSolver> create() { return std::make_shared<SGDSolver_Frame_HIP<T> >(); }
+private:
+    static Registrar<SGDSolver> mRegistrar;
+};
+
+// include/Quantizer/QAT/Cell/QuantizerCell.hpp:25-66: Range (255), QuantMode
+class QuantizerCell {
+public:
+    enum QuantMode { Default, Symmetric, Asymmetric, FullRange };
+    virtual ~QuantizerCell() {}
+    void setRange(std::size_t range) { mRange = range; }
+    void setQuantMode(QuantMode mode) { mQuantMode = mode; }
+    void setSolver(const std::shared_ptr<SGDSolver>& solver) { mSolver = solver; }
+    // device float buffers of n weights: full precision, and the gradient w.r.t. the quantized weights
+    virtual void addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize) = 0;
+    virtual void initialize() = 0;
+    virtual void propagate() = 0;
+    virtual void back_propagate() = 0;
+    virtual void update(unsigned int batchSize) = 0;
+    virtual float* getQuantizedWeights(unsigned int k) = 0;
+    virtual float* getDiffFullPrecisionWeights(unsigned int k) = 0;
+
+protected:
+    QuantizerCell() : mRange(255), mQuantMode(Default) {}
+    std::size_t mRange;
+    QuantMode mQuantMode;
+    std::shared_ptr<SGDSolver> mSolver;
+};
+
+struct QuantizerBuffers {
+    float *fp, *diffQ, *q, *diffFp;
+    std::size_t size, outputsSize;
+};
+
+// src/Quantizer/QAT/Cell/SAT/SATQuantizerCell.cpp:28-33: ApplyQuantization (true), ApplyScaling (false)
+class SATQuantizerCell : public QuantizerCell {
+public:
+    typedef std::function<std::shared_ptr<SATQuantizerCell>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    void setQuantization(bool v) { mApplyQuantization = v; }
+    void setScaling(bool v) { mApplyScaling = v; }
+protected:
+    SATQuantizerCell() : mApplyQuantization(true), mApplyScaling(false) {}
+    bool mApplyQuantization, mApplyScaling;
+};
+
+// src/Quantizer/QAT/Cell/SAT/SATQuantizerCell_Frame.cpp:65-294
+template <class T>
+class SATQuantizerCell_Frame_HIP : public SATQuantizerCell {
+public:
+    SATQuantizerCell_Frame_HIP() : mOutputsSize(0), mStats(nullptr), mWorkspace(nullptr), mWorkspaceBytes(0), mStream(nullptr) {}
+    ~SATQuantizerCell_Frame_HIP();
+    static std::shared_ptr<SATQuantizerCell> create() { return std::make_shared<SATQuantizerCell_Frame_HIP<T> >(); }
+    void addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize);
+    void initialize();
+    void propagate();
+    void back_propagate();
+    void update(unsigned int /*batchSize*/) {}           // nothing to do for SAT in cell mode
+    float* getQuantizedWeights(unsigned int k) { return mW.at(k).q; }
+    float* getDiffFullPrecisionWeights(unsigned int k) { return mW.at(k).diffFp; }
+    // {tanh_max, scaling} of tensor k, read back from the device
+    std::pair<float, float> getStats(unsigned int k) const;
+    int satMode() const;
+
+private:
+    std::vector<QuantizerBuffers> mW;
+    std::size_t mOutputsSize;
+    float* mStats;          // 2 floats per tensor
+    void* mWorkspace;
+    std::size_t mWorkspaceBytes;
+    void* mStream;
+    static Registrar<SATQuantizerCell> mRegistrar;
+};
+
+// include/Quantizer/QAT/Activation/QuantizerActivation.hpp:23-25: Range (255)
+class QuantizerActivation {
+public:
+    virtual ~QuantizerActivation() {}
+    void setRange(std::size_t range) { mRange = range; }
+    void setSolver(const std::shared_ptr<SGDSolver>& solver) { mSolver = solver; }
+    // in-place on a device float buffer
+    virtual void propagate(float* inOut, std::size_t size, bool inference) = 0;
+    virtual void back_propagate(const float* diffInput, float* diffOutput, std::size_t size) = 0;
+    virtual void update(unsigned int batchSize) = 0;
+
+protected:
+    QuantizerActivation() : mRange(255) {}
+    std::size_t mRange;
+    std::shared_ptr<SGDSolver> mSolver;
+};
+
+// src/Quantizer/QAT/Activation/SAT/SATQuantizerActivation_Frame.cpp:73-143: Alpha (1.0)
+class SATQuantizerActivation : public QuantizerActivation {
+public:
+    typedef std::function<std::shared_ptr<SATQuantizerActivation>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    void setAlpha(double alpha) { mAlphaParameter = alpha; }
+protected:
+    SATQuantizerActivation() : mAlphaParameter(1.0) {}
+    double mAlphaParameter;
+};
+
+template <class T>
+class SATQuantizerActivation_Frame_HIP : public SATQuantizerActivation {
+public:
+    SATQuantizerActivation_Frame_HIP() : mDev(nullptr), mFp(nullptr), mFpSize(0), mWorkspace(nullptr), mWorkspaceBytes(0), mStream(nullptr) {}
+    ~SATQuantizerActivation_Frame_HIP();
+    static std::shared_ptr<SATQuantizerActivation> create() { return std::make_shared<SATQuantizerActivation_Frame_HIP<T> >(); }
+    void propagate(float* inOut, std::size_t size, bool inference);
+    void back_propagate(const float* diffInput, float* diffOutput, std::size_t size);
+    void update(unsigned int batchSize);
+    float getAlpha();
+    float getDiffAlpha();
+
+private:
+    void lazyInit(std::size_t size, bool needCopy);
+    float* mDev;            // {alpha, diffAlpha}
+    float* mFp;             // full-precision copy saved by the training forward
+    std::size_t mFpSize;
+    void* mWorkspace;
+    std::size_t mWorkspaceBytes;
+    void* mStream;
+    static Registrar<SATQuantizerActivation> mRegistrar;
+};
+
+// src/Quantizer/QAT/Cell/LSQ/LSQQuantizerCell.cpp:28-33: StepSize (100), SetOptInitStepSize (true)
+class LSQQuantizerCell : public QuantizerCell {
+public:
+    typedef std::function<std::shared_ptr<LSQQuantizerCell>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    void setStepSizeValue(float v) { mStepSizeVal = v; }
+    void setOptInitStepSize(bool v) { mSetOptInitStepSize = v; }
+protected:
+    LSQQuantizerCell() : mStepSizeVal(100.0f), mSetOptInitStepSize(true) {}
+    float mStepSizeVal;
+    bool mSetOptInitStepSize;
+};
+
+// src/Quantizer/QAT/Cell/LSQ/LSQQuantizerCell_Frame.cpp:106-310
+template <class T>
+class LSQQuantizerCell_Frame_HIP : public LSQQuantizerCell {
+public:
+    LSQQuantizerCell_Frame_HIP() : mLo(0), mHi(0), mGradScale(0.0f), mDev(nullptr), mWorkspace(nullptr), mWorkspaceBytes(0), mInitialized(false) {}
+    ~LSQQuantizerCell_Frame_HIP();
+    static std::shared_ptr<LSQQuantizerCell> create() { return std::make_shared<LSQQuantizerCell_Frame_HIP<T> >(); }
+    void addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize);
+    void initialize();
+    void propagate();
+    void back_propagate();
+    void update(unsigned int batchSize);
+    float* getQuantizedWeights(unsigned int k) { return mW.at(k).q; }
+    float* getDiffFullPrecisionWeights(unsigned int k) { return mW.at(k).diffFp; }
+    float getStepSize();
+    float getDiffStepSize();
+    std::pair<int, int> getBitRanges() const { return std::make_pair(mLo, mHi); }
+
+private:
+    std::vector<QuantizerBuffers> mW;
+    int mLo, mHi;
+    float mGradScale;
+    float* mDev;            // {stepSize, diffStepSize}
+    void* mWorkspace;
+    std::size_t mWorkspaceBytes;
+    bool mInitialized;
+    static Registrar<LSQQuantizerCell> mRegistrar;
+};
+
+// src/Quantizer/QAT/Activation/LSQ/LSQQuantizerActivation.cpp:28-33 and ..._Frame.cpp:92-278
+class LSQQuantizerActivation : public QuantizerActivation {
+public:
+    typedef std::function<std::shared_ptr<LSQQuantizerActivation>()> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    void setStepSizeValue(float v) { mStepSizeParameter = v; }
+    void setOptInitStepSize(bool v) { mSetOptInitStepSize = v; }
+protected:
+    LSQQuantizerActivation() : mStepSizeParameter(100.0f), mSetOptInitStepSize(true) {}
+    float mStepSizeParameter;
+    bool mSetOptInitStepSize;
+};
+
+template <class T>
+class LSQQuantizerActivation_Frame_HIP : public LSQQuantizerActivation {
+public:
+    LSQQuantizerActivation_Frame_HIP() : mGradScale(0.0f), mDev(nullptr), mFp(nullptr), mFpSize(0), mWorkspace(nullptr), mWorkspaceBytes(0) {}
+    ~LSQQuantizerActivation_Frame_HIP();
+    static std::shared_ptr<LSQQuantizerActivation> create() { return std::make_shared<LSQQuantizerActivation_Frame_HIP<T> >(); }
+    void propagate(float* inOut, std::size_t size, bool inference);
+    void back_propagate(const float* diffInput, float* diffOutput, std::size_t size);
+    void update(unsigned int batchSize);
+    float getStepSize();
+    float getDiffStepSize();
+
+private:
+    float mGradScale;
+    float* mDev;            // {stepSize, diffStepSize}
+    float* mFp;
+    std::size_t mFpSize;
+    void* mWorkspace;
+    std::size_t mWorkspaceBytes;
+    static Registrar<LSQQuantizerActivation> mRegistrar;
+};
+
+// -------------------------------------------------------------------- DeepNet
+// Layer-ordered container: what DeepNet::addCell / getParentCells / propagate provide to the path
+// (src/DeepNet.cpp:2692-2719).
+class DeepNet {
+public:
+    DeepNet() {}
+    // parents empty = connected to the environment
+    void addCell(const std::shared_ptr<Cell>& cell, const std::vector<std::shared_ptr<Cell> >& parents);
+    std::shared_ptr<Cell> getCell(const std::string& name) const;
+    const std::vector<std::shared_ptr<Cell> >& getCells() const { return mOrder; }
+    // environment: integer-valued stimuli {W,H,C,B}
+    void setStimuli(unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize);
+    void setStimuliData(const Tensor<Float_T>& data);
+    HipTensor& getStimuli() { return mStimuli; }
+    void initialize();
+    void propagate(bool inference = true);
+    void synchronize();
+
+private:
+    std::vector<std::shared_ptr<Cell> > mOrder;
+    std::map<std::string, std::shared_ptr<Cell> > mCells;
+    HipTensor mStimuli;
+    unsigned int mEnvC = 0, mEnvH = 0, mEnvW = 0, mEnvB = 0;
+};
+
+// Builds a DeepNet from the subset of N2D2's INI format the quantized path needs
+// (DefaultModel, [env]/[sp] sizes, Conv / Fc / Pool / ElemWise / Scaling sections with Input=,
+// KernelDims / KernelWidth / KernelHeight, NbOutputs, Stride, Padding, Dilation, PoolDims, Pooling, Operation,
+// ActivationFunction, Mapping.ChannelsPerGroup=1 for depthwise).  Cells are created through the Registrar
+// with the model key found in DefaultModel, as src/Generator/*CellGenerator.cpp do.
+std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string* modelOut = nullptr);
+
+} // namespace N2D2

@@ -1,0 +1,319 @@
+// C entry points over the Frame_HIP host cells, for the Python test-suite and demos: build a net from INI text
+// through the Registrar, set parameters the way N2D2's quantization pass leaves them, propagate, read outputs.
+// Every function returns 0 on success; the message of the last C++ exception is kept per thread.
+#include <cstring>
+
+#include <hip/hip_runtime_api.h>
+
+#include "frame_hip.hpp"
+
+using namespace N2D2;
+
+namespace {
+thread_local std::string g_error;
+struct Net {
+    std::shared_ptr<DeepNet> deepNet;
+    std::string model;
+};
+template <class F>
+int guarded(F f)
+{
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+Scaling makeScaling(int mode, const void* scaling, size_t n, int fracBits, int isClipped, const float* clip)
+{
+    std::vector<Float_T> cl;
+    if (isClipped && clip) cl.assign(clip, clip + n);
+    switch (mode) {
+    case N2D2HIP_SCALING_NONE: return Scaling();
+    case N2D2HIP_SCALING_FLOAT_MULT:
+        return Scaling::floatingPointScaling(std::vector<Float_T>((const float*)scaling, (const float*)scaling + n), isClipped != 0, cl);
+    case N2D2HIP_SCALING_FIXED_MULT16:
+    case N2D2HIP_SCALING_FIXED_MULT32:
+        return Scaling::fixedPointScaling(mode == N2D2HIP_SCALING_FIXED_MULT16 ? ScalingMode::FIXED_MULT16 : ScalingMode::FIXED_MULT32,
+                                          (size_t)fracBits, std::vector<std::int32_t>((const std::int32_t*)scaling, (const std::int32_t*)scaling + n),
+                                          isClipped != 0, cl);
+    case N2D2HIP_SCALING_SINGLE_SHIFT:
+        return Scaling::singleShiftScaling(std::vector<unsigned char>((const unsigned char*)scaling, (const unsigned char*)scaling + n), isClipped != 0, cl);
+    case N2D2HIP_SCALING_DOUBLE_SHIFT: {
+        std::vector<std::pair<unsigned char, unsigned char> > v;
+        for (size_t i = 0; i < n; ++i) v.push_back(std::make_pair(((const unsigned char*)scaling)[2 * i], ((const unsigned char*)scaling)[2 * i + 1]));
+        return Scaling::doubleShiftScaling(v, isClipped != 0, std::vector<std::pair<unsigned char, unsigned char> >());
+    }
+    default: throw std::runtime_error("Unsupported scaling propagation.");
+    }
+}
+} // namespace
+
+extern "C" {
+
+const char* fh_last_error(void) { return g_error.c_str(); }
+
+// 1 if a factory is registered for (cell type, model key, float)
+int fh_registrar_exists(const char* type, const char* key)
+{
+    const std::string t(type), k(key);
+    if (t == "Conv") return Registrar<ConvCell>::exists<float>(k);
+    if (t == "Fc") return Registrar<FcCell>::exists<float>(k);
+    if (t == "Pool") return Registrar<PoolCell>::exists<float>(k);
+    if (t == "ElemWise") return Registrar<ElemWiseCell>::exists<float>(k);
+    if (t == "Scaling") return Registrar<ScalingCell>::exists<float>(k);
+    if (t == "Rectifier") return Registrar<RectifierActivation>::exists<float>(k);
+    if (t == "Linear") return Registrar<LinearActivation>::exists<float>(k);
+    if (t == "SATCell") return Registrar<SATQuantizerCell>::exists<float>(k);
+    if (t == "SATAct") return Registrar<SATQuantizerActivation>::exists<float>(k);
+    if (t == "LSQCell") return Registrar<LSQQuantizerCell>::exists<float>(k);
+    if (t == "LSQAct") return Registrar<LSQQuantizerActivation>::exists<float>(k);
+    if (t == "SGDSolver") return Registrar<SGDSolver>::exists<float>(k);
+    return -1;
+}
+
+// Registers (Conv, "Frame_HIP", float) a second time: returns 1 and leaves the message in fh_last_error()
+// when the Registrar throws as the reference's does.
+int fh_registrar_duplicate_throws(void)
+{
+    try {
+        Registrar<ConvCell> again("Frame_HIP", ConvCell_Frame_HIP<float>::create, Registrar<ConvCell>::Type<float>());
+        return 0;
+    } catch (const std::runtime_error& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+// 1 when create() on an unknown key yields an empty function (after printing, as the reference does)
+int fh_registrar_unknown_key_is_null(const char* key)
+{
+    return !Registrar<ConvCell>::create<float>(key) ? 1 : 0;
+}
+
+void fh_set_globals(int precision, int unsignedData, int envDataUnsigned)
+{
+    CellExport::mPrecision = precision;
+    DeepNetExport::mUnsignedData = unsignedData != 0;
+    DeepNetExport::mEnvDataUnsigned = envDataUnsigned != 0;
+}
+
+void* fh_net_from_ini(const char* text)
+{
+    Net* n = new Net();
+    const int rc = guarded([&] { n->deepNet = generateFromINI(text, &n->model); });
+    if (rc) { delete n; return nullptr; }
+    return n;
+}
+void fh_net_free(void* net) { delete (Net*)net; }
+const char* fh_net_model(void* net) { return ((Net*)net)->model.c_str(); }
+int fh_net_nb_cells(void* net) { return (int)((Net*)net)->deepNet->getCells().size(); }
+int fh_net_initialize(void* net) { return guarded([&] { ((Net*)net)->deepNet->initialize(); }); }
+int fh_net_propagate(void* net) { return guarded([&] { ((Net*)net)->deepNet->propagate(true); ((Net*)net)->deepNet->synchronize(); }); }
+
+// data: integer-valued floats in N2D2 order {W,H,C,B} (= NCHW flat)
+int fh_net_set_stimuli(void* net, const float* data, int C, int H, int W, int B)
+{
+    return guarded([&] {
+        Tensor<Float_T> t({(size_t)W, (size_t)H, (size_t)C, (size_t)B});
+        std::memcpy(t.data(), data, t.size() * sizeof(float));
+        ((Net*)net)->deepNet->setStimuliData(t);
+    });
+}
+
+// dims = {W, H, C, B} of the cell's outputs; unsignedOut = DeepNetExport::isCellOutputUnsigned(cell)
+int fh_cell_info(void* net, const char* name, int* dims, int* unsignedOut, char* typeOut, int typeLen)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        auto f = std::dynamic_pointer_cast<Cell_Frame_HIP>(c);
+        dims[0] = (int)c->getOutputsWidth(); dims[1] = (int)c->getOutputsHeight(); dims[2] = (int)c->getNbOutputs(); dims[3] = (int)f->batchSize();
+        *unsignedOut = DeepNetExport::isCellOutputUnsigned(*c) ? 1 : 0;
+        if (typeOut && typeLen > 0) { std::strncpy(typeOut, c->getType(), (size_t)typeLen - 1); typeOut[typeLen - 1] = 0; }
+    });
+}
+
+int fh_cell_set_quantized(void* net, const char* name, int nbBits, int activationNbBits)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        c->setQuantized((size_t)nbBits);
+        if (c->getActivation() && activationNbBits > 0) c->getActivation()->setQuantized((size_t)activationNbBits);
+    });
+}
+
+// Conv: weights {kW,kH,C/groups,O} (= OCHW flat); Fc: [O][K]
+int fh_cell_set_weights(void* net, const char* name, const float* w, size_t n, int kW, int kH, int Cg, int O, int weightBits)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        Tensor<Float_T> t({(size_t)kW, (size_t)kH, (size_t)Cg, (size_t)O});
+        if (t.size() != n) throw std::runtime_error("fh_cell_set_weights(): size mismatch");
+        std::memcpy(t.data(), w, n * sizeof(float));
+        if (auto conv = std::dynamic_pointer_cast<ConvCell>(c)) { conv->setWeights(t); conv->setWeightsPrecision(weightBits); }
+        else if (auto fc = std::dynamic_pointer_cast<FcCell>(c)) fc->setWeights(t);
+        else throw std::runtime_error("fh_cell_set_weights(): cell has no weights");
+    });
+}
+
+int fh_cell_set_biases(void* net, const char* name, const float* b, size_t n)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        Tensor<Float_T> t({n});
+        std::memcpy(t.data(), b, n * sizeof(float));
+        if (auto conv = std::dynamic_pointer_cast<ConvCell>(c)) conv->setBiases(t);
+        else if (auto fc = std::dynamic_pointer_cast<FcCell>(c)) fc->setBiases(t);
+        else throw std::runtime_error("fh_cell_set_biases(): cell has no biases");
+    });
+}
+
+// Installs a Scaling in the cell's activation (what fuseScalingCells does), or in a ScalingCell.
+int fh_cell_set_scaling(void* net, const char* name, int mode, const void* scaling, size_t n, int fracBits, int isClipped, const float* clip)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        Scaling s = makeScaling(mode, scaling, n, fracBits, isClipped, clip);
+        if (auto sc = std::dynamic_pointer_cast<ScalingCell>(c)) sc->setScaling(s);
+        else if (c->getActivation()) c->getActivation()->setActivationScaling(s);
+        else throw std::runtime_error("fh_cell_set_scaling(): cell " + std::string(name) + " has no activation");
+    });
+}
+
+int fh_cell_get_outputs(void* net, const char* name, float* out, size_t n)
+{
+    return guarded([&] {
+        auto f = std::dynamic_pointer_cast<Cell_Frame_HIP>(((Net*)net)->deepNet->getCell(name));
+        const Tensor<Float_T>& t = f->getOutputs();
+        if (t.size() != n) throw std::runtime_error("fh_cell_get_outputs(): size mismatch");
+        std::memcpy(out, t.data(), n * sizeof(float));
+    });
+}
+
+// ---- quantizers, each created through the Registrar under the given model key.  Host buffers in and out.
+int fh_sat_cell_run(const char* model, const float* w, const float* diffQ, size_t n, size_t outputsSize, int range, int quantMode,
+                    int applyQuantization, int applyScaling, float* wq, float* diffW, float* stats)
+{
+    return guarded([&] {
+        auto f = Registrar<SATQuantizerCell>::create<float>(model);
+        if (!f) throw std::runtime_error("Quantizer model \"" + std::string(model) + "\" is not valid");
+        auto q = std::dynamic_pointer_cast<SATQuantizerCell_Frame_HIP<float> >(f());
+        float *dW = nullptr, *dD = nullptr;
+        if (hipMalloc((void**)&dW, n * 4) != hipSuccess || hipMalloc((void**)&dD, n * 4) != hipSuccess) throw std::runtime_error("hipMalloc");
+        hipMemcpy(dW, w, n * 4, hipMemcpyHostToDevice);
+        hipMemcpy(dD, diffQ, n * 4, hipMemcpyHostToDevice);
+        q->setRange((size_t)range);
+        q->setQuantMode((QuantizerCell::QuantMode)quantMode);
+        q->setQuantization(applyQuantization != 0);
+        q->setScaling(applyScaling != 0);
+        q->addWeights(dW, dD, n, outputsSize);
+        q->initialize();
+        q->propagate();
+        q->back_propagate();
+        hipDeviceSynchronize();
+        hipMemcpy(wq, q->getQuantizedWeights(0), n * 4, hipMemcpyDeviceToHost);
+        hipMemcpy(diffW, q->getDiffFullPrecisionWeights(0), n * 4, hipMemcpyDeviceToHost);
+        const auto st = q->getStats(0);
+        stats[0] = st.first; stats[1] = st.second;
+        q.reset();
+        hipFree(dW); hipFree(dD);
+    });
+}
+
+// Two training passes inside one solver iteration (IterationSize = 2) then an update: alphas[0..2] = alpha before,
+// accumulated diffAlpha, alpha after the solver step.
+int fh_sat_act_run(const char* model, const float* x, const float* diffIn, size_t n, int range, float alpha, float learningRate, float* y,
+                   float* diffOut, float* alphas)
+{
+    return guarded([&] {
+        auto f = Registrar<SATQuantizerActivation>::create<float>(model);
+        auto fs = Registrar<SGDSolver>::create<float>(model);
+        if (!f || !fs) throw std::runtime_error("Quantizer model \"" + std::string(model) + "\" is not valid");
+        auto q = std::dynamic_pointer_cast<SATQuantizerActivation_Frame_HIP<float> >(f());
+        auto solver = fs();
+        solver->setParameter("LearningRate", learningRate);
+        solver->setParameter("IterationSize", 2);
+        q->setSolver(solver);
+        q->setRange((size_t)range);
+        q->setAlpha(alpha);
+        float *dX = nullptr, *dG = nullptr, *dO = nullptr;
+        if (hipMalloc((void**)&dX, n * 4) != hipSuccess || hipMalloc((void**)&dG, n * 4) != hipSuccess || hipMalloc((void**)&dO, n * 4) != hipSuccess)
+            throw std::runtime_error("hipMalloc");
+        hipMemcpy(dG, diffIn, n * 4, hipMemcpyHostToDevice);
+        for (int pass = 0; pass < 2; ++pass) {
+            hipMemcpy(dX, x, n * 4, hipMemcpyHostToDevice);
+            q->propagate(dX, n, false);
+            q->back_propagate(dG, dO, n);          // pass 0: new iteration (beta 0); pass 1: accumulates (beta 1)
+            if (pass == 0) { alphas[0] = q->getAlpha(); q->update(1); }     // first pass of the iteration: no parameter step yet
+        }
+        hipDeviceSynchronize();
+        alphas[1] = q->getDiffAlpha();
+        q->update(1);
+        alphas[2] = q->getAlpha();
+        hipMemcpy(y, dX, n * 4, hipMemcpyDeviceToHost);
+        hipMemcpy(diffOut, dO, n * 4, hipMemcpyDeviceToHost);
+        q.reset();
+        hipFree(dX); hipFree(dG); hipFree(dO);
+    });
+}
+
+int fh_lsq_cell_run(const char* model, const float* w, const float* diffQ, size_t n, int range, float stepSize, int optInit, float* wq,
+                    float* diffW, float* steps)
+{
+    return guarded([&] {
+        auto f = Registrar<LSQQuantizerCell>::create<float>(model);
+        if (!f) throw std::runtime_error("Quantizer model \"" + std::string(model) + "\" is not valid");
+        auto q = std::dynamic_pointer_cast<LSQQuantizerCell_Frame_HIP<float> >(f());
+        float *dW = nullptr, *dD = nullptr;
+        if (hipMalloc((void**)&dW, n * 4) != hipSuccess || hipMalloc((void**)&dD, n * 4) != hipSuccess) throw std::runtime_error("hipMalloc");
+        hipMemcpy(dW, w, n * 4, hipMemcpyHostToDevice);
+        hipMemcpy(dD, diffQ, n * 4, hipMemcpyHostToDevice);
+        q->setRange((size_t)range);
+        q->setStepSizeValue(stepSize);
+        q->setOptInitStepSize(optInit != 0);
+        q->addWeights(dW, dD, n, 1);
+        q->initialize();
+        q->propagate();
+        q->back_propagate();
+        hipDeviceSynchronize();
+        hipMemcpy(wq, q->getQuantizedWeights(0), n * 4, hipMemcpyDeviceToHost);
+        hipMemcpy(diffW, q->getDiffFullPrecisionWeights(0), n * 4, hipMemcpyDeviceToHost);
+        steps[0] = q->getStepSize();
+        steps[1] = q->getDiffStepSize();
+        steps[2] = (float)q->getBitRanges().first;
+        steps[3] = (float)q->getBitRanges().second;
+        q.reset();
+        hipFree(dW); hipFree(dD);
+    });
+}
+
+int fh_lsq_act_run(const char* model, const float* x, const float* diffIn, size_t n, int range, float stepSize, int optInit, float* y,
+                   float* diffOut, float* steps)
+{
+    return guarded([&] {
+        auto f = Registrar<LSQQuantizerActivation>::create<float>(model);
+        if (!f) throw std::runtime_error("Quantizer model \"" + std::string(model) + "\" is not valid");
+        auto q = std::dynamic_pointer_cast<LSQQuantizerActivation_Frame_HIP<float> >(f());
+        q->setRange((size_t)range);
+        q->setStepSizeValue(stepSize);
+        q->setOptInitStepSize(optInit != 0);
+        float *dX = nullptr, *dG = nullptr, *dO = nullptr;
+        if (hipMalloc((void**)&dX, n * 4) != hipSuccess || hipMalloc((void**)&dG, n * 4) != hipSuccess || hipMalloc((void**)&dO, n * 4) != hipSuccess)
+            throw std::runtime_error("hipMalloc");
+        hipMemcpy(dX, x, n * 4, hipMemcpyHostToDevice);
+        hipMemcpy(dG, diffIn, n * 4, hipMemcpyHostToDevice);
+        q->propagate(dX, n, false);
+        q->back_propagate(dG, dO, n);
+        hipDeviceSynchronize();
+        hipMemcpy(y, dX, n * 4, hipMemcpyDeviceToHost);
+        hipMemcpy(diffOut, dO, n * 4, hipMemcpyDeviceToHost);
+        steps[0] = q->getStepSize();
+        steps[1] = q->getDiffStepSize();
+        q.reset();
+        hipFree(dX); hipFree(dG); hipFree(dO);
+    });
+}
+
+} // extern "C"

@@ -1,0 +1,173 @@
+"""ctypes access to the C++ Frame_HIP host cells (libn2d2_frame_hip.so): nets are built from N2D2-style INI text
+through the Registrar under the model key named by DefaultModel, parameters are installed the way N2D2's
+quantization pass leaves them, and outputs come back as N2D2 float tensors."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import capi
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libn2d2_frame_hip.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError("libn2d2_frame_hip.so is not built (%s): run `python -m n2d2_amd.build`" % LIB_PATH)
+lib = C.CDLL(LIB_PATH)
+lib.fh_last_error.restype = C.c_char_p
+lib.fh_net_from_ini.restype = C.c_void_p
+lib.fh_net_from_ini.argtypes = [C.c_char_p]
+lib.fh_net_model.restype = C.c_char_p
+for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize", "fh_net_propagate"):
+    getattr(lib, _n).argtypes = [C.c_void_p]
+lib.fh_net_set_stimuli.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
+lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
+lib.fh_cell_set_quantized.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int]
+lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+lib.fh_cell_set_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
+lib.fh_cell_get_outputs.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+lib.fh_registrar_exists.argtypes = [C.c_char_p, C.c_char_p]
+lib.fh_registrar_unknown_key_is_null.argtypes = [C.c_char_p]
+lib.fh_set_globals.argtypes = [C.c_int, C.c_int, C.c_int]
+_F, _P, _SZ, _I = C.c_float, C.c_void_p, C.c_size_t, C.c_int
+lib.fh_sat_cell_run.argtypes = [C.c_char_p, _P, _P, _SZ, _SZ, _I, _I, _I, _I, _P, _P, _P]
+lib.fh_sat_act_run.argtypes = [C.c_char_p, _P, _P, _SZ, _I, _F, _F, _P, _P, _P]
+lib.fh_lsq_cell_run.argtypes = [C.c_char_p, _P, _P, _SZ, _I, _F, _I, _P, _P, _P]
+lib.fh_lsq_act_run.argtypes = [C.c_char_p, _P, _P, _SZ, _I, _F, _I, _P, _P, _P]
+
+
+class FrameHipError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise FrameHipError(lib.fh_last_error().decode())
+
+
+def set_globals(precision, unsigned_data, env_data_unsigned):
+    """CellExport::mPrecision, DeepNetExport::mUnsignedData, DeepNetExport::mEnvDataUnsigned."""
+    lib.fh_set_globals(int(precision), int(bool(unsigned_data)), int(bool(env_data_unsigned)))
+
+
+_MODE = {"None": capi.SCALING_NONE, "FloatMult": capi.SCALING_FLOAT_MULT, "FixedMult16": capi.SCALING_FIXED_MULT16,
+         "FixedMult32": capi.SCALING_FIXED_MULT32, "SingleShift": capi.SCALING_SINGLE_SHIFT, "DoubleShift": capi.SCALING_DOUBLE_SHIFT}
+_MODE_DT = {"FloatMult": np.float32, "FixedMult16": np.int32, "FixedMult32": np.int32, "SingleShift": np.uint8, "DoubleShift": np.uint8}
+
+
+class Net:
+    def __init__(self, ini_text):
+        self.h = lib.fh_net_from_ini(ini_text.encode())
+        if not self.h:
+            raise FrameHipError(lib.fh_last_error().decode())
+
+    def __del__(self):
+        if getattr(self, "h", None) and lib is not None:
+            lib.fh_net_free(self.h)
+            self.h = None
+
+    @property
+    def model(self):
+        return lib.fh_net_model(self.h).decode()
+
+    @property
+    def nb_cells(self):
+        return lib.fh_net_nb_cells(self.h)
+
+    def cell_info(self, name):
+        dims = (C.c_int * 4)()
+        uns = C.c_int()
+        typ = C.create_string_buffer(32)
+        _check(lib.fh_cell_info(self.h, name.encode(), dims, C.byref(uns), typ, 32))
+        return {"W": dims[0], "H": dims[1], "C": dims[2], "B": dims[3], "unsigned": bool(uns.value), "type": typ.value.decode()}
+
+    def set_quantized(self, name, nb_bits, act_nb_bits=0):
+        _check(lib.fh_cell_set_quantized(self.h, name.encode(), int(nb_bits), int(act_nb_bits)))
+
+    def set_weights(self, name, w, weight_bits=8):
+        """w: [O, C/groups, kH, kW] (conv) or [O, K] (fc), integer-valued."""
+        a = np.ascontiguousarray(w, dtype=np.float32)
+        if a.ndim == 4:
+            O, Cg, kH, kW = a.shape
+        else:
+            O, Cg, kH, kW = a.shape[0], a.shape[1], 1, 1
+        _check(lib.fh_cell_set_weights(self.h, name.encode(), a.ctypes.data, a.size, kW, kH, Cg, O, int(weight_bits)))
+
+    def set_biases(self, name, b):
+        a = np.ascontiguousarray(b, dtype=np.float32)
+        _check(lib.fh_cell_set_biases(self.h, name.encode(), a.ctypes.data, a.size))
+
+    def set_scaling(self, name, mode, scaling=None, frac_bits=0, clipping=None):
+        if mode == "None":
+            _check(lib.fh_cell_set_scaling(self.h, name.encode(), capi.SCALING_NONE, None, 0, 0, 0, None))
+            return
+        s = np.ascontiguousarray(scaling, dtype=_MODE_DT[mode])
+        n = s.size // 2 if mode == "DoubleShift" else s.size
+        cl = None if clipping is None else np.ascontiguousarray(clipping, dtype=np.float32)
+        _check(lib.fh_cell_set_scaling(self.h, name.encode(), _MODE[mode], s.ctypes.data, n, int(frac_bits), int(cl is not None),
+                                       None if cl is None else cl.ctypes.data))
+
+    def initialize(self):
+        _check(lib.fh_net_initialize(self.h))
+
+    def set_stimuli(self, x):
+        a = np.ascontiguousarray(x, dtype=np.float32)
+        B, Cc, H, W = a.shape
+        _check(lib.fh_net_set_stimuli(self.h, a.ctypes.data, Cc, H, W, B))
+
+    def propagate(self):
+        _check(lib.fh_net_propagate(self.h))
+
+    def outputs(self, name):
+        """Outputs of a cell as N2D2 exposes them: float32 [B, C, H, W] holding integer values."""
+        i = self.cell_info(name)
+        out = np.empty((i["B"], i["C"], i["H"], i["W"]), dtype=np.float32)
+        _check(lib.fh_cell_get_outputs(self.h, name.encode(), out.ctypes.data, out.size))
+        return out
+
+
+def spec_to_ini(spec, batch, model="Frame_HIP"):
+    """N2D2 INI text of a nets.NetSpec (the structural part; parameters are installed afterwards)."""
+    C_, H, W = spec.in_shape
+    lines = ["DefaultModel=%s" % model, "", "[sp]", "SizeX=%d" % W, "SizeY=%d" % H, "NbChannels=%d" % C_, "BatchSize=%d" % batch, ""]
+    for l in spec.layers:
+        ins = ",".join("sp" if i == "input" else i for i in l.inputs)
+        lines += ["[%s]" % l.name, "Input=%s" % ins]
+        if l.type == "conv":
+            O, Cg, kH, kW = l.w.shape
+            lines += ["Type=Conv", "KernelDims=%d %d" % (kW, kH), "NbOutputs=%d" % O, "StrideDims=%d %d" % l.stride,
+                      "PaddingDims=%d %d" % (l.pad[0], l.pad[1]), "DilationDims=%d %d" % l.dil, "ActivationFunction=%s" % l.act.kind,
+                      "NoBias=%d" % (l.bias is None)]
+            if l.groups > 1:
+                lines.append("Mapping.NbGroups=%d" % l.groups)
+        elif l.type == "fc":
+            lines += ["Type=Fc", "NbOutputs=%d" % l.w.shape[0], "ActivationFunction=%s" % l.act.kind]
+        elif l.type == "pool":
+            lines += ["Type=Pool", "PoolDims=%d %d" % l.pool, "NbOutputs=%d" % l.out_shape[0], "StrideDims=%d %d" % l.stride,
+                      "PaddingDims=%d %d" % l.pad, "Pooling=%s" % ("Max" if l.kind == "max" else "Average")]
+        elif l.type == "elemwise":
+            lines += ["Type=ElemWise", "NbOutputs=%d" % l.out_shape[0], "Operation=Sum", "ActivationFunction=%s" % l.act.kind]
+        elif l.type == "scaling":
+            lines += ["Type=Scaling", "NbOutputs=%d" % l.out_shape[0]]
+        lines.append("")
+    return "\n".join(lines)
+
+
+def build_net(spec, batch, model="Frame_HIP"):
+    """Instantiates a nets.NetSpec on the C++ Frame_HIP cells: INI -> Registrar -> cells, then parameters."""
+    net = Net(spec_to_ini(spec, batch, model))
+    for l in spec.layers:
+        if l.type in ("conv", "fc"):
+            net.set_weights(l.name, l.w, getattr(l, "weight_bits", 8))
+            if l.bias is not None:
+                net.set_biases(l.name, l.bias)
+        if l.type in ("conv", "fc", "elemwise", "scaling"):
+            a = l.act
+            net.set_quantized(l.name, 8, a.nb_bits)
+            if l.type == "scaling":
+                net.set_quantized(l.name, a.nb_bits)
+            net.set_scaling(l.name, a.mode, a.scaling, a.frac_bits, a.clipping)
+        elif l.type == "pool":
+            net.set_quantized(l.name, 8)
+    return net

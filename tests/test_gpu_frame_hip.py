@@ -1,0 +1,167 @@
+"""The C++ Frame_HIP cells end to end on the GPU: nets built from INI text through the Registrar, parameters installed
+as N2D2's quantization pass leaves them, outputs read back as N2D2 float tensors and compared bit-for-bit with the CPU
+oracle; the SAT / LSQ quantizer classes created through the Registrar against the oracle's formulas."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def fh():
+    from n2d2_amd import frame_hip
+    frame_hip.set_globals(8, True, True)          # what calibNetwork sets: 8-bit export, unsigned data allowed, u8 stimuli
+    yield frame_hip
+    frame_hip.set_globals(0, True, False)
+
+
+def _compare(fh, spec, x, keep):
+    from oracle import cells
+    net = fh.build_net(spec, x.shape[0])
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        got = net.outputs(name)
+        assert got.dtype == np.float32 and got.shape == want[name].shape, name
+        assert np.array_equal(got, want[name]), name
+        assert net.cell_info(name)["unsigned"] == spec.unsigned[name], name
+    return net
+
+
+def test_lenet_through_the_registrar(fh):
+    from n2d2_amd import nets
+    spec = nets.lenet()
+    x = np.random.default_rng(31).integers(0, 256, size=(64, 1, 32, 32))
+    _compare(fh, spec, x, [l.name for l in spec.layers])
+
+
+def test_resnet50_through_the_registrar(fh):
+    from n2d2_amd import nets
+    spec = nets.resnet50()
+    x = np.random.default_rng(32).integers(0, 256, size=(2, 3, 224, 224))
+    net = _compare(fh, spec, x, ["conv1", "pool1", "conv2.1_sum", "conv2.2_shortcut_rescale", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
+    # a second propagate on new stimuli reuses the prepared cells
+    from oracle import cells
+    x2 = np.random.default_rng(33).integers(0, 256, size=(2, 3, 224, 224))
+    net.set_stimuli(x2)
+    net.propagate()
+    assert np.array_equal(net.outputs("fc"), cells.run_net(spec, x2)["fc"])
+
+
+def test_mobilenet_and_w4a4_through_the_registrar(fh):
+    from n2d2_amd import nets
+    x = np.random.default_rng(34).integers(0, 256, size=(1, 3, 224, 224))
+    _compare(fh, nets.mobilenet_v1(), x, ["conv2_dw", "conv2_pw", "conv14_pw", "fc"])
+    _compare(fh, nets.resnet18_w4a4(), x, ["conv2.1_a", "conv2.1_sum", "conv5.2_sum", "fc"])
+
+
+def test_signedness_change_rebuilds_the_cells(fh):
+    """-no-unsigned (DeepNetExport::mUnsignedData = false): every cell saturates to the signed range."""
+    from n2d2_amd import nets
+    from oracle import cells
+    spec_u = nets.resnet50(image=64)
+    spec_s = nets.resnet50(image=64, unsigned_data=False)
+    x = np.random.default_rng(35).integers(0, 128, size=(1, 3, 64, 64))
+    try:
+        fh.set_globals(8, False, False)
+        net = fh.build_net(spec_s, 1)
+        net.initialize()
+        net.set_stimuli(x)
+        net.propagate()
+        assert np.array_equal(net.outputs("fc"), cells.run_net(spec_s, x)["fc"])
+        assert net.outputs("conv2.1_sum").max() <= 127
+    finally:
+        fh.set_globals(8, True, True)
+    assert spec_u.unsigned["conv1"] and not spec_s.unsigned["conv1"]
+
+
+def test_non_integer_weights_are_refused(fh):
+    from n2d2_amd import nets
+    spec = nets.lenet()
+    net = fh.build_net(spec, 4)
+    net.set_weights("conv1", spec.layers[0].w.astype(np.float32) + 0.25)
+    net.initialize()
+    net.set_stimuli(np.zeros((4, 1, 32, 32)))
+    with pytest.raises(fh.FrameHipError) as e:
+        net.propagate()
+    assert "is not an integer" in str(e.value)
+
+
+# ------------------------------------------------------------ quantizer classes
+
+def test_sat_quantizer_cell_class(fh):
+    from oracle import oracle as orc
+    rng = np.random.default_rng(41)
+    w = rng.normal(0, 0.05, size=64 * 64 * 9).astype(np.float32)
+    g = rng.normal(size=w.size).astype(np.float32)
+    for quant_mode, name in ((1, "symrange"), (0, "default"), (3, "fullrange"), (2, "asymrange")):       # QuantizerCell::QuantMode order
+        wq, dw, stats = np.empty_like(w), np.empty_like(w), np.zeros(2, dtype=np.float32)
+        rc = fh.lib.fh_sat_cell_run(b"Frame_HIP", w.ctypes.data, g.ctypes.data, w.size, 64 * 9, 15, quant_mode, 1, 0,
+                                    wq.ctypes.data, dw.ctypes.data, stats.ctypes.data)
+        assert rc == 0, fh.lib.fh_last_error()
+        want, tmax, _ = orc.sat_weight_forward(w, 15.0, name)
+        assert abs(stats[0] - tmax) <= 1e-5 * tmax and stats[1] == 1.0
+        bad = np.abs(wq - want) > 1e-5
+        assert bad.sum() <= max(2, int(2e-4 * w.size))
+        want_b = orc.sat_weight_backward(g, w, 15.0, np.float32(tmax), name if name in ("fullrange", "asymrange") else "default")
+        assert np.all(np.abs(dw - want_b) <= 1e-5 * np.maximum(np.abs(want_b), 1e-2))
+    # ApplyScaling with outputsSize = dimB*dimY*dimX
+    wq, dw, stats = np.empty_like(w), np.empty_like(w), np.zeros(2, dtype=np.float32)
+    assert fh.lib.fh_sat_cell_run(b"Frame_HIP", w.ctypes.data, g.ctypes.data, w.size, 64 * 9, 15, 1, 1, 1, wq.ctypes.data, dw.ctypes.data,
+                                  stats.ctypes.data) == 0
+    want, tmax, scal = orc.sat_weight_forward(w.astype(np.float64), 15.0, "symrange", apply_scaling=True, outputs_size=64 * 9)
+    assert abs(stats[1] - scal) <= 1e-5 * scal
+    assert (np.abs(wq - want) > 1e-5 * np.abs(want).max()).sum() <= 8
+    assert fh.lib.fh_sat_cell_run(b"Frame", w.ctypes.data, g.ctypes.data, w.size, 1, 15, 1, 1, 0, wq.ctypes.data, dw.ctypes.data,
+                                  stats.ctypes.data) == 1                      # unknown model key
+
+
+def test_sat_quantizer_activation_class_with_solver(fh):
+    from oracle import oracle as orc
+    rng = np.random.default_rng(42)
+    n = 32 * 28 * 28
+    x = rng.normal(2.0, 3.0, size=n).astype(np.float32)
+    g = rng.normal(size=n).astype(np.float32)
+    y, dx, alphas = np.empty_like(x), np.empty_like(x), np.zeros(3, dtype=np.float32)
+    lr = 1e-4
+    assert fh.lib.fh_sat_act_run(b"Frame_HIP", x.ctypes.data, g.ctypes.data, n, 15, 6.0, lr, y.ctypes.data, dx.ctypes.data, alphas.ctypes.data) == 0
+    want_y, fp = orc.sat_act_forward(x, 15.0, 6.0, inference=False)
+    assert (np.abs(y - want_y) > 6e-5).sum() <= 2
+    want_dx, want_da, terms = orc.sat_act_backward(g.astype(np.float64), x.astype(np.float64), 15.0, 6.0)
+    assert np.array_equal(dx, want_dx.astype(np.float32))
+    assert alphas[0] == 6.0
+    # two passes of one iteration accumulate: diffAlpha = 2 * sum; the solver ADDS rate/(batch*iterSize)*diff
+    assert abs(alphas[1] - 2 * want_da) <= 1e-5 * 2 * np.abs(terms).sum()
+    assert abs(alphas[2] - (6.0 + lr / 2 * alphas[1])) <= 1e-6
+
+
+def test_lsq_quantizer_classes(fh):
+    from oracle import oracle as orc
+    rng = np.random.default_rng(43)
+    w = rng.normal(0, 0.05, size=128 * 64 * 9 + 3).astype(np.float32)
+    g = rng.normal(size=w.size).astype(np.float32)
+    wq, dw, steps = np.empty_like(w), np.empty_like(w), np.zeros(4, dtype=np.float32)
+    assert fh.lib.fh_lsq_cell_run(b"Frame_HIP", w.ctypes.data, g.ctypes.data, w.size, 15, 100.0, 1, wq.ctypes.data, dw.ctypes.data, steps.ctypes.data) == 0
+    lo, hi = int(steps[2]), int(steps[3])
+    assert (lo, hi) == (-8, 7)
+    step0 = 2.0 * np.abs(w.astype(np.float64)).mean() / np.sqrt(hi)          # optimal initial step of the LSQ paper
+    assert abs(steps[0] - step0) <= 1e-5 * step0
+    want = orc.lsq_forward(w, steps[0], lo, hi)
+    assert (np.abs(wq - want) > 1e-5 * np.maximum(np.abs(want), steps[0])).sum() <= 2
+    want_dfp, want_sum = orc.lsq_backward(g.astype(np.float64), w.astype(np.float64), float(steps[0]), lo, hi)
+    assert np.array_equal(dw, want_dfp.astype(np.float32))
+    gs = 1.0 / np.sqrt(w.size * hi)
+    assert abs(steps[1] - want_sum * gs) <= 1e-4 * abs(want_sum * gs) + 1e-7
+    # activations: range [0, R], fixed step
+    x = np.abs(rng.normal(0, 1.0, size=4096)).astype(np.float32)
+    gx = rng.normal(size=x.size).astype(np.float32)
+    y, dx, st = np.empty_like(x), np.empty_like(x), np.zeros(2, dtype=np.float32)
+    assert fh.lib.fh_lsq_act_run(b"Frame_HIP", x.ctypes.data, gx.ctypes.data, x.size, 15, 0.2, 0, y.ctypes.data, dx.ctypes.data, st.ctypes.data) == 0
+    assert st[0] == np.float32(0.2)
+    want = orc.lsq_forward(x, np.float32(0.2), 0, 15)
+    assert (np.abs(y - want) > 1e-5 * np.maximum(np.abs(want), 0.2)).sum() <= 2
+    want_dx, want_sum = orc.lsq_backward(gx.astype(np.float64), x.astype(np.float64), float(np.float32(0.2)), 0, 15)
+    assert np.array_equal(dx, want_dx.astype(np.float32))
+    assert abs(st[1] - want_sum / np.sqrt(x.size * 15)) <= 1e-4 * abs(want_sum / np.sqrt(x.size * 15)) + 1e-7
