@@ -97,14 +97,14 @@ def main():
     conv_ms = sum(per[l.name] for l in convs)
     conv_ops = 2.0 * sum(net.layer_macs(l) for l in convs)
     all_ms = sum(per.values())
-    all_bytes = sum(net.layer_bytes(l) for l in spec.layers)
+    all_bytes = sum(net.layer_bytes(l) for l in net.launched)
     achieved = conv_ops / (conv_ms * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "conv_igemm_kernel (all %d conv/fc launches of one forward)" % len(convs),
                 "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
                 "traffic": None, "launches_per_step": len(convs), "avg_launch_us": round(conv_ms * 1000.0 / len(convs), 2),
                 "ops_per_step": conv_ops}
     hbm = all_bytes / (all_ms * 1e-3) / 1e9
-    roofline_hbm = {"bound": "hbm", "kernel": "whole forward (%d launches)" % len(spec.layers), "achieved": round(hbm, 1),
+    roofline_hbm = {"bound": "hbm", "kernel": "whole forward (%d launches)" % len(net.launched), "achieved": round(hbm, 1),
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(hbm / PEAK_HBM_GBS, 4), "bytes_per_step": all_bytes,
                     "sum_kernel_ms": round(all_ms, 4)}
 

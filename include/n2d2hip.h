@@ -185,6 +185,13 @@ typedef struct n2d2hip_elemwise_s* n2d2hip_elemwise_t;
  * them (nb_inputs entries, or C entries for PER_CHANNEL); NULL means all 1 / all 0. */
 int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, const float* weights,
                             const float* shifts, n2d2hip_act_t act, n2d2hip_elemwise_t* ew);
+/* Graph-level fusion: folds the ScalingCell that feeds input `input_index` into this cell.  That input is then
+ * the ScalingCell's own input and the Scaling is applied on the fly, i.e. ScalingCell_Frame::propagate
+ * (ref: src/Cell/ScalingCell_Frame.cpp:67-75) followed by ElemWiseCell_Frame::propagate in one pass, without
+ * materialising the rescaled tensor.  `scaling` (built with n2d2hip_act_create, kind LINEAR) is borrowed; NULL undoes
+ * the fold.  Returns N2D2HIP_ERR_UNSUPPORTED (and folds nothing) unless the sum has unit coefficients and the Scaling is
+ * an integer mode whose products fit 32 bits: the caller then keeps the ScalingCell as a separate launch. */
+int n2d2hip_elemwise_fold_input_scaling(n2d2hip_elemwise_t ew, int input_index, n2d2hip_act_t scaling);
 int n2d2hip_elemwise_destroy(n2d2hip_elemwise_t ew);
 int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
                              n2d2hip_stream_t stream);

@@ -86,6 +86,8 @@ struct ElemWiseArgs {
     int cs;
     long long npix;
     EpiArgs epi;
+    int pre_input;      // input that carries a folded ScalingCell (-1: none)
+    EpiArgs pre;        // its Scaling (EPI_I24 tables), applied to the input before the sum
 };
 
 // ref: src/Cell/ElemWiseCell_Frame.cpp:116-136 (Sum) followed by the cell's activation; with one input and unit
@@ -95,7 +97,8 @@ struct ElemWiseArgs {
 // float operation of the reference is exact on these operands).
 // HOIST: the launch makes the grid stride a multiple of the dwords per pixel, so a thread keeps its 4 channels
 // and loads their table rows once.
-template <int KIND, bool FCOEF, bool HOIST>
+// PRE: one input is rescaled on the fly by the ScalingCell folded into this cell.
+template <int KIND, bool FCOEF, bool HOIST, bool PRE>
 __global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
 {
     const int cq = p.cs >> 2;
@@ -104,7 +107,15 @@ __global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
     long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     int c4 = (int)(idx % cq) * 4;
     int4 ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
+    int4 pa = ta, pb = ta, pc = ta, pd = ta, pe = ta;
     auto load_tables = [&](int c) {
+        if (PRE) {
+            pa = *(const int4*)(p.pre.a + c);
+            pb = *(const int4*)(p.pre.b + c);
+            pc = *(const int4*)(p.pre.c + c);
+            pd = *(const int4*)(p.pre.d + c);
+            pe = *(const int4*)(p.pre.e + c);
+        }
         if (KIND != EPI_RAW) {
             ta = *(const int4*)(p.epi.a + c);
             tb = *(const int4*)(p.epi.b + c);
@@ -155,10 +166,18 @@ __global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
                     r[t] = (int)fminf(fmaxf(round_half_away(o[t]), -2147483520.0f), 2147483520.0f);   // round(realInput)
             }
         } else {
+            auto prescale = [&](int v[4]) {
+                v[0] = epi_apply<EPI_I24>(v[0], pa.x, pb.x, pc.x, pd.x, pe.x, p.pre.lo, p.pre.hi, 0);
+                v[1] = epi_apply<EPI_I24>(v[1], pa.y, pb.y, pc.y, pd.y, pe.y, p.pre.lo, p.pre.hi, 0);
+                v[2] = epi_apply<EPI_I24>(v[2], pa.z, pb.z, pc.z, pd.z, pe.z, p.pre.lo, p.pre.hi, 0);
+                v[3] = epi_apply<EPI_I24>(v[3], pa.w, pb.w, pc.w, pd.w, pe.w, p.pre.lo, p.pre.hi, 0);
+            };
             unpack4(*(const int*)(p.in[0] + idx * 4) ^ (int)p.flip[0], p.zp[0], r);
+            if (PRE && p.pre_input == 0) prescale(r);
             for (int k = 1; k < p.nb_inputs; ++k) {
                 int v[4];
                 unpack4(*(const int*)(p.in[k] + idx * 4) ^ (int)p.flip[k], p.zp[k], v);
+                if (PRE && p.pre_input == k) prescale(v);
                 r[0] += v[0]; r[1] += v[1]; r[2] += v[2]; r[3] += v[3];
             }
         }
@@ -175,14 +194,14 @@ __global__ __launch_bounds__(256) void elemwise_sum_kernel(ElemWiseArgs p)
     }
 }
 
-template <bool FCOEF, bool HOIST>
+template <bool FCOEF, bool HOIST, bool PRE>
 static void launch_elemwise(const ElemWiseArgs& a, unsigned grid, hipStream_t stream)
 {
     switch (a.epi.kind) {
-    case EPI_RAW: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_RAW, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I24: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I24, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I64: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I64, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
-    default: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_F32, FCOEF, HOIST>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_RAW: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_RAW, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I24, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I64, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_F32, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
     }
 }
 
@@ -198,8 +217,10 @@ int run_elemwise(const ElemWiseArgs& a, bool fcoef, hipStream_t stream)
     const long long unit = cq / g;                // grid must be a multiple of this
     bool hoist = unit <= want;
     unsigned grid = (unsigned)(hoist ? (want / unit) * unit : want);
-    if (fcoef) { if (hoist) launch_elemwise<true, true>(a, grid, stream); else launch_elemwise<true, false>(a, grid, stream); }
-    else { if (hoist) launch_elemwise<false, true>(a, grid, stream); else launch_elemwise<false, false>(a, grid, stream); }
+    const bool pre = a.pre_input >= 0;
+    if (fcoef) { if (hoist) launch_elemwise<true, true, false>(a, grid, stream); else launch_elemwise<true, false, false>(a, grid, stream); }
+    else if (pre) { if (hoist) launch_elemwise<false, true, true>(a, grid, stream); else launch_elemwise<false, false, true>(a, grid, stream); }
+    else { if (hoist) launch_elemwise<false, true, false>(a, grid, stream); else launch_elemwise<false, false, false>(a, grid, stream); }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
@@ -212,6 +233,7 @@ int run_scaling_nhwc(const n2d2hip_act_s* act, const n2d2hip_tensor* in, const n
     a.flip[0] = in->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
     a.zp[0] = in->dtype == N2D2HIP_I8 ? 0 : 128;
     a.nb_inputs = 1;
+    a.pre_input = -1;
     a.out = out->data;
     a.out_dtype = out->dtype;
     a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
@@ -230,6 +252,8 @@ struct n2d2hip_elemwise_s {
     n2d2hip_act_t act;
     float* d_coeff;     // w then s, each [nb_inputs][cpad]
     bool unit_coeff;    // every weight 1 and every shift 0
+    int pre_input;      // input carrying a folded ScalingCell (-1: none)
+    n2d2hip_act_t pre_act;
 };
 
 extern "C" {
@@ -297,6 +321,7 @@ int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, cons
     e->unit_coeff = true;
     for (size_t i = 0; i < (size_t)nb_inputs * cpad; ++i)
         if (hw[i] != 1.0f || hs[i] != 0.0f) e->unit_coeff = false;
+    e->pre_input = -1; e->pre_act = nullptr;
     e->nb_inputs = nb_inputs; e->nb_channels = nb_channels; e->cpad = cpad; e->act = act; e->d_coeff = nullptr;
     hipError_t herr = hipMalloc((void**)&e->d_coeff, h.size() * sizeof(float));
     if (herr == hipSuccess) herr = hipMemcpy(e->d_coeff, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
@@ -305,6 +330,19 @@ int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, cons
         return fail(N2D2HIP_ERR_HIP, "elemwise_create: device upload failed: %s", hipGetErrorString(herr));
     }
     *ew = e;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_elemwise_fold_input_scaling(n2d2hip_elemwise_t ew, int input_index, n2d2hip_act_t scaling)
+{
+    N2D2HIP_REQUIRE(ew != nullptr, N2D2HIP_ERR_INVALID, "elemwise_fold_input_scaling: null cell");
+    if (!scaling) { ew->pre_input = -1; ew->pre_act = nullptr; return N2D2HIP_OK; }
+    N2D2HIP_REQUIRE(input_index >= 0 && input_index < ew->nb_inputs, N2D2HIP_ERR_INVALID, "elemwise_fold_input_scaling: input %d of %d", input_index, ew->nb_inputs);
+    N2D2HIP_REQUIRE(scaling->nb_channels == ew->nb_channels, N2D2HIP_ERR_INVALID, "elemwise_fold_input_scaling: channel count mismatch");
+    N2D2HIP_REQUIRE(ew->unit_coeff && scaling->args.kind == EPI_I24 && scaling->min_out >= -128 && scaling->max_out <= 255, N2D2HIP_ERR_UNSUPPORTED,
+                    "elemwise_fold_input_scaling: only an integer Scaling in front of a unit-coefficient sum can be folded");
+    ew->pre_input = input_index;
+    ew->pre_act = scaling;
     return N2D2HIP_OK;
 }
 
@@ -344,6 +382,8 @@ int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const*
         N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_UNSUPPORTED, "elemwise_forward: output must be a byte type or I32");
     }
     a.nb_inputs = ew->nb_inputs;
+    a.pre_input = ew->pre_input;
+    if (ew->pre_input >= 0) a.pre = ew->pre_act->args;
     a.w = ew->d_coeff;
     a.s = ew->d_coeff + (size_t)ew->nb_inputs * ew->cpad;
     a.cpad = ew->cpad;

@@ -17,7 +17,9 @@
 // the MFMA "A" operand and the pixels the "B" operand, so that every lane ends
 // up with 4 consecutive output channels of one pixel: one packed dword.
 #include <algorithm>
+#include <cstdlib>
 #include <limits>
+#include <type_traits>
 
 #include "common.h"
 #include "epilogue.cuh"
@@ -283,6 +285,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     }
 }
 
+} // namespace n2d2hip
+#include "conv_dma.cuh"
+namespace n2d2hip {
+
 // ------------------------------------------------------------ depthwise
 // groups == C == O: one output channel per input channel, no reduction over
 // channels, hence no matrix core: a bandwidth kernel.  Each thread produces 4
@@ -348,6 +354,7 @@ struct n2d2hip_conv_s {
     signed char* d_w;
     int4* d_sub;
     int* d_bias;
+    signed char* d_fill;  // 16 bytes of the input's logical zero, source of padded taps in the direct-to-LDS kernel
     bool is_fc;
     int fcH, fcW;
 };
@@ -370,6 +377,31 @@ void launch_cfg(const ConvArgs& a, hipStream_t stream)
     case EPI_I64: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_I64, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
     default: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_F32, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
     }
+}
+
+template <int BM, int BN, int WGM>
+void launch_dma(const ConvDmaArgs& a, int grid, hipStream_t stream)
+{
+    constexpr int S = 4;
+    switch (a.c.epi.kind) {
+    case EPI_RAW: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_RAW, S>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_I24, S>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_I64, S>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_F32, S>), dim3(grid), dim3(256), 0, stream, a); break;
+    }
+}
+
+int num_cus()
+{
+    static int n = 0;
+    if (n == 0) {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+            n = prop.multiProcessorCount;
+        if (n <= 0) n = 256;
+    }
+    return n;
 }
 
 int sext4(int n) { return (n & 8) ? (n | ~15) : (n & 15); }
@@ -424,7 +456,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->in_cs = n2d2hip_nhwc_cs(d->C);
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
-    c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr;
+    c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
         delete c;
@@ -516,6 +548,12 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_sub, hsub.size() * sizeof(int4));
         if (e == hipSuccess) e = hipMemcpy(c->d_sub, hsub.data(), hsub.size() * sizeof(int4), hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess) {
+        signed char fill[16];
+        memset(fill, zp ? 0x80 : 0x00, sizeof(fill));
+        e = hipMalloc((void**)&c->d_fill, sizeof(fill));
+        if (e == hipSuccess) e = hipMemcpy(c->d_fill, fill, sizeof(fill), hipMemcpyHostToDevice);
+    }
     if (e != hipSuccess) {
         n2d2hip_conv_destroy(c);
         return fail(N2D2HIP_ERR_HIP, "conv_create: device upload failed: %s", hipGetErrorString(e));
@@ -530,6 +568,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_w) (void)hipFree(c->d_w);
     if (c->d_sub) (void)hipFree(c->d_sub);
     if (c->d_bias) (void)hipFree(c->d_bias);
+    if (c->d_fill) (void)hipFree(c->d_fill);
     delete c;
     return N2D2HIP_OK;
 }
@@ -602,6 +641,23 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     const bool bm64 = bn128 && !c->pix4 && blocks128 < 512;
     const int BM = bm64 ? 64 : 128;
     a.nblocks = (int)(((Mll + BM - 1) / BM) * a.ntiles_n);
+    const bool fits32 = (long long)in->B * in->H * in->W * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
+    if (!c->pix4 && !w4 && c->ktot <= 8192 && fits32 && getenv("N2D2HIP_NO_DMA") == nullptr) {
+        // persistent direct-to-LDS pipeline: 2 blocks per CU, each walking pixel tiles of one channel tile
+        ConvDmaArgs q;
+        q.c = a;
+        q.fill16 = c->d_fill;
+        q.all_valid = (d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0) ? 1 : 0;
+        q.mtiles = (int)((Mll + BM - 1) / BM);
+        const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, (2 * num_cus()) / (8 * a.ntiles_n)));
+        q.mlanes = 8 * per_xcd;
+        const int grid = 8 * a.ntiles_n * per_xcd;
+        if (!bn128) launch_dma<128, 64, 2>(q, grid, stream);
+        else if (bm64) launch_dma<64, 128, 1>(q, grid, stream);
+        else launch_dma<128, 128, 2>(q, grid, stream);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
     if (c->pix4) {
         if (bn128) { if (w4) launch_cfg<128, 128, 2, true, true>(a, stream); else launch_cfg<128, 128, 2, true, false>(a, stream); }
         else { if (w4) launch_cfg<128, 64, 2, true, true>(a, stream); else launch_cfg<128, 64, 2, true, false>(a, stream); }

@@ -356,13 +356,21 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch):
+    def __init__(self, spec, batch, fuse=True):
+        """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
+        the rescaled tensor is never written)."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
+        consumers = {}
+        for l in spec.layers:
+            for i in l.inputs:
+                consumers.setdefault(i, []).append(l)
+        self.folded = set()
         C, H, W = spec.in_shape
         self.input = rt.DTensor(batch, C, H, W, capi.U8B if spec.input_unsigned else capi.I8)
         self.tensors = {"input": self.input}
         self.steps = []
+        ins_of = {}
         for l in spec.layers:
             ins = [self.tensors[i] for i in l.inputs]
             Co, Ho, Wo = l.out_shape
@@ -386,11 +394,27 @@ class GpuNet:
                 act = rt.Act(Co, **l.act.kwargs())
                 cell = rt.ElemWiseSum(len(ins), Co, act, l.weights, l.shifts, l.coeff_mode)
                 out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype())
+                if fuse:
+                    for k, name in enumerate(l.inputs):
+                        prod = next((m for m in spec.layers if m.name == name), None)
+                        if prod is not None and prod.type == "scaling" and len(consumers[name]) == 1 and not self.folded & set(l.inputs):
+                            sc_cell = next(c for (m, c, f) in self.steps if m is prod)
+                            if cell.fold_input_scaling(k, sc_cell):
+                                self.folded.add(name)
+                                ins[k] = self.tensors[prod.inputs[0]]
                 self.steps.append((l, cell, (lambda c, i, o: c.forward(i, o))))
             else:
                 raise ValueError(l.type)
             self.tensors[l.name] = out
-        self._io = [([self.tensors[i] for i in l.inputs], self.tensors[l.name]) for l in spec.layers]
+            ins_of[l.name] = ins
+        self._io = [(ins_of[l.name], self.tensors[l.name]) for l in spec.layers]
+        # folded ScalingCells are not launched and their output is never materialised
+        for name in self.folded:
+            del self.tensors[name]
+        keep = [k for k, l in enumerate(spec.layers) if l.name not in self.folded]
+        self.steps = [self.steps[k] for k in keep]
+        self._io = [self._io[k] for k in keep]
+        self.launched = [spec.layers[k] for k in keep]
 
     def set_input(self, x):
         """x: integer NCHW numpy array [B,C,H,W]."""
@@ -418,7 +442,7 @@ class GpuNet:
 
     def layer_bytes(self, l):
         """Algorithmic HBM bytes of one cell: inputs and output once at storage width, weights once."""
-        ins, out = self._io[self.spec.layers.index(l)]
+        ins, out = self._io[self.launched.index(l)]
         total = sum(t.B * t.C * t.H * t.W * (4 if t.dtype == self.capi.I32 else 1) for t in ins)
         total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
         if l.type in ("conv", "fc"):
@@ -435,7 +459,7 @@ class GpuNet:
     def activation_bytes(self):
         """Algorithmic HBM bytes of one forward: every cell reads its inputs and writes its output once, plus weights."""
         total = 0
-        for l, (ins, out) in zip(self.spec.layers, self._io):
+        for l, (ins, out) in zip(self.launched, self._io):
             total += sum(t.B * t.C * t.H * t.W * (4 if t.dtype == self.capi.I32 else 1) for t in ins)
             total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
             if l.type in ("conv", "fc"):

@@ -212,6 +212,15 @@ class ElemWiseSum:
         check(lib.n2d2hip_elemwise_create(nb_inputs, nb_channels, mode, None if w is None else w.ctypes.data,
                                           None if s is None else s.ctypes.data, act.handle, C.byref(self.handle)))
 
+    def fold_input_scaling(self, input_index, act):
+        """Folds the ScalingCell feeding input `input_index`; returns False when the library keeps them separate."""
+        rc = lib.n2d2hip_elemwise_fold_input_scaling(self.handle, input_index, act.handle if act is not None else None)
+        if rc == capi.ERR_UNSUPPORTED:
+            return False
+        check(rc)
+        self._folded = act
+        return True
+
     def forward(self, xs, out=None, out_dtype=None):
         x0 = xs[0]
         if out is None:

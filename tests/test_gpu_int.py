@@ -320,3 +320,35 @@ def test_elemwise_sum_cell_bit_exact(rt):
     want = cells_ref.elemwise_cell([a, b], spec, wc, sc, "PerChannel")
     ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **spec.kwargs()), wc, sc, "PerChannel")
     assert np.array_equal(ew.forward([da, db]).to_numpy(), want.astype(np.int64))
+
+
+def test_elemwise_with_folded_scaling_cell(rt):
+    """ScalingCell -> ElemWise sum in one launch equals the two reference cells run one after the other."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    for Cc, shape in ((40, (2, 40, 7, 9)), (256, (3, 256, 14, 14))):
+        a, b = _u8(shape), _u8(shape)
+        da, db = rt.DTensor.from_numpy(a, capi.U8B), rt.DTensor.from_numpy(b, capi.U8B)
+        sum_spec = ActSpec("Rectifier", "DoubleShift", np.stack([RNG.integers(0, 3, size=Cc), RNG.integers(1, 4, size=Cc)], 1),
+                           nb_bits=8, unsigned_out=True)
+        for mode, sc_spec in (("fixed16", ActSpec("Linear", "FixedMult16", RNG.integers(2 ** 12, 2 ** 15, size=Cc), frac_bits=14, nb_bits=8, unsigned_out=True)),
+                              ("sshift", ActSpec("Linear", "SingleShift", RNG.integers(0, 3, size=Cc), nb_bits=8, unsigned_out=False)),
+                              ("dshift", ActSpec("Linear", "DoubleShift", np.stack([RNG.integers(0, 3, size=Cc), RNG.integers(1, 4, size=Cc)], 1),
+                                                 nb_bits=8, unsigned_out=True))):
+            for k in (0, 1):
+                xs = [a, b]
+                xs[k] = sc_spec.apply(xs[k].astype(np.float32))
+                want = cells_ref.elemwise_cell(xs, sum_spec)
+                sc = rt.Act(Cc, **sc_spec.kwargs())
+                ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **sum_spec.kwargs()))
+                assert ew.fold_input_scaling(k, sc), mode
+                assert np.array_equal(ew.forward([da, db]).to_numpy(), want.astype(np.int64)), (mode, k, Cc)
+                assert ew.fold_input_scaling(k, None)      # undo: plain sum again
+                assert np.array_equal(ew.forward([da, db]).to_numpy(), cells_ref.elemwise_cell([a, b], sum_spec).astype(np.int64))
+    # a float Scaling or a weighted sum is left to the caller as a separate launch
+    fl = rt.Act(Cc, **ActSpec("Linear", "FloatMult", np.full(Cc, 0.5, np.float32), nb_bits=8, unsigned_out=True).kwargs())
+    ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **sum_spec.kwargs()))
+    assert ew.fold_input_scaling(0, fl) is False
+    ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **sum_spec.kwargs()), np.array([2.0, 1.0], np.float32), np.zeros(2, np.float32), "PerInput")
+    assert ew.fold_input_scaling(0, sc) is False
