@@ -8,7 +8,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libn2d2hip.so")
+LIB_PATH = os.environ.get("N2D2HIP_LIB") or os.path.join(_HERE, "lib", "libn2d2hip.so")
 
 # enums of n2d2hip.h
 U8, I8, I32, F32, U8B = 0, 1, 2, 3, 4

@@ -175,6 +175,7 @@ int n2d2hip_act_create(const n2d2hip_activation* desc, int nb_channels, n2d2hip_
     a->nb_channels = nb_channels;
     a->cpad = round_up(nb_channels, 256);
     a->tables = nullptr;
+    a->clipped = clipped;
     EpiArgs& e = a->args;
     e = EpiArgs();
 
@@ -271,6 +272,7 @@ int n2d2hip_act_create(const n2d2hip_activation* desc, int nb_channels, n2d2hip_
         e.kind = fast ? EPI_I24 : EPI_I64;
     }
 
+    a->htab = t;
     hipError_t herr = hipMalloc((void**)&a->tables, t.size() * sizeof(int));
     if (herr == hipSuccess)
         herr = hipMemcpy(a->tables, t.data(), t.size() * sizeof(int), hipMemcpyHostToDevice);

@@ -87,4 +87,6 @@ struct n2d2hip_act_s {
     int* tables;               // device, 5 * cpad ints
     n2d2hip::EpiArgs args;
     int min_out, max_out;      // range of produced values (for dtype checks); RAW: INT range
+    std::vector<int> htab;     // host copy of the tables (empty for RAW)
+    bool clipped;              // the Scaling applies a Clip
 };

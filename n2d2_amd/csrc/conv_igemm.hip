@@ -286,7 +286,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 }
 
 } // namespace n2d2hip
-#include "conv_dma.cuh"
+#include "conv_pipe.cuh"
 namespace n2d2hip {
 
 // ------------------------------------------------------------ depthwise
@@ -355,6 +355,7 @@ struct n2d2hip_conv_s {
     int4* d_sub;
     int* d_bias;
     signed char* d_fill;  // 16 bytes of the input's logical zero, source of padded taps in the direct-to-LDS kernel
+    bool preclamp;        // some accumulator could overflow the rescale's 24x24 -> 32 bit product, or the cell has a Clip
     bool is_fc;
     int fcH, fcW;
 };
@@ -379,16 +380,30 @@ void launch_cfg(const ConvArgs& a, hipStream_t stream)
     }
 }
 
-template <int BM, int BN, int WGM>
-void launch_dma(const ConvDmaArgs& a, int grid, hipStream_t stream)
+template <int NW, int BK, int NI, int NJ, int WGM, int S>
+void launch_pipe(ConvPipeArgs a, bool all_valid, int grid, hipStream_t stream)
 {
-    constexpr int S = 4;
+    a.c.niter = a.c.ktot / BK;
+    a.cper = a.c.in_cs / BK;
+#define N2D2HIP_PIPE(EPI) \
+    do { if (all_valid) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, true>), dim3(grid), dim3(NW * 64), 0, stream, a); \
+         else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, false>), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
     switch (a.c.epi.kind) {
-    case EPI_RAW: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_RAW, S>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I24: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_I24, S>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I64: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_I64, S>), dim3(grid), dim3(256), 0, stream, a); break;
-    default: hipLaunchKernelGGL((conv_dma_kernel<BM, BN, WGM, EPI_F32, S>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_RAW: N2D2HIP_PIPE(EPI_RAW); break;
+    case EPI_I24: N2D2HIP_PIPE(EPI_I24); break;
+    default: N2D2HIP_PIPE(EPI_F32); break;
     }
+#undef N2D2HIP_PIPE
+}
+
+// (multiplier, shift) with n / d == umulhi(n, multiplier) >> shift for 0 <= n < 2^31; multiplier 0 stands for d == 1
+void magic_div(unsigned d, unsigned* mul, unsigned* sh)
+{
+    if (d <= 1) { *mul = 0; *sh = 0; return; }
+    unsigned s = 0;
+    while ((1ull << s) < d) ++s;
+    *mul = (unsigned)((1ull << (31 + s)) / d + 1);
+    *sh = s - 1;
 }
 
 int num_cus()
@@ -484,6 +499,22 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_create: folded bias of output %d overflows int32", o);
         }
         hbias[o] = (int)b;
+    }
+    // Can the rescale multiply raw accumulators?  |sum| <= 128 * sum|w| + |folded bias| for byte inputs.
+    c->preclamp = act->clipped;
+    if (act->args.kind == EPI_I24 && !c->preclamp) {
+        const int cp = act->cpad;
+        for (int o = 0; o < d->O && !c->preclamp; ++o) {
+            long long s = 0;
+            for (long long i = 0; i < wstrideO; ++i)
+                s += std::abs(read_weight(weights, o * wstrideO + i, d->weight_bits));
+            const long long bound = 128 * s + std::llabs((long long)hbias[o]);
+            const long long mult = act->htab[2 * (size_t)cp + o], half = act->htab[3 * (size_t)cp + o];
+            if (bound >= (1ll << 23) || bound * mult + half > std::numeric_limits<int>::max())
+                c->preclamp = true;
+        }
+    } else if (act->args.kind != EPI_F32) {
+        c->preclamp = true;
     }
 
     if (depthwise) {
@@ -642,19 +673,36 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     const int BM = bm64 ? 64 : 128;
     a.nblocks = (int)(((Mll + BM - 1) / BM) * a.ntiles_n);
     const bool fits32 = (long long)in->B * in->H * in->W * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
-    if (!c->pix4 && !w4 && c->ktot <= 8192 && fits32 && getenv("N2D2HIP_NO_DMA") == nullptr) {
-        // persistent direct-to-LDS pipeline: 2 blocks per CU, each walking pixel tiles of one channel tile
-        ConvDmaArgs q;
+    const bool pipe_kind = act->args.kind == EPI_RAW || act->args.kind == EPI_I24 || act->args.kind == EPI_F32;
+    if (!c->pix4 && !w4 && in->cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 32 && pipe_kind && fits32
+        && getenv("N2D2HIP_NO_PIPE") == nullptr) {
+        // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
+        ConvPipeArgs q;
         q.c = a;
         q.fill16 = c->d_fill;
-        q.all_valid = (d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0) ? 1 : 0;
-        q.mtiles = (int)((Mll + BM - 1) / BM);
-        const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, (2 * num_cus()) / (8 * a.ntiles_n)));
+        q.cper = d.C / 64;
+        q.kW = d.kW; q.kH = d.kH;
+        q.preclamp = c->preclamp ? 1 : 0;
+#ifdef N2D2HIP_PROFILE
+        q.prof = (long long*)strtoull(getenv("N2D2HIP_PROF_PTR"), nullptr, 16);
+#endif
+        magic_div((unsigned)(OH * OW), &q.ohw_mul, &q.ohw_sh);
+        magic_div((unsigned)OW, &q.ow_mul, &q.ow_sh);
+        const bool all_valid = d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0;
+        // Two independent 4-wave blocks per CU, 128 pixels x 128 (or 64) channels each: one block's epilogue and
+        // barrier waits overlap the other's MFMAs.  K advances by whole 128-byte lines when the channel count allows.
+        const int BMp = 128;
+        q.mtiles = (int)((Mll + BMp - 1) / BMp);
+        const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
         q.mlanes = 8 * per_xcd;
         const int grid = 8 * a.ntiles_n * per_xcd;
-        if (!bn128) launch_dma<128, 64, 2>(q, grid, stream);
-        else if (bm64) launch_dma<64, 128, 1>(q, grid, stream);
-        else launch_dma<128, 128, 2>(q, grid, stream);
+        if (d.C % 128 == 0) {
+            if (bn128) launch_pipe<4, 128, 2, 2, 2, 2>(q, all_valid, grid, stream);
+            else launch_pipe<4, 128, 2, 1, 4, 3>(q, all_valid, grid, stream);
+        } else {
+            if (bn128) launch_pipe<4, 64, 2, 2, 2, 4>(q, all_valid, grid, stream);
+            else launch_pipe<4, 64, 2, 1, 4, 4>(q, all_valid, grid, stream);
+        }
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }

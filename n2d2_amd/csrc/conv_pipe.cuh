@@ -1,0 +1,473 @@
+// Persistent, software-pipelined implicit-GEMM convolution for int8 weights
+// and activations whose channel count is a multiple of 64.
+//
+// What bounds such a layer on this chip is not memory but instruction issue:
+// a 32x32x32 int8 MFMA keeps a SIMD's matrix core busy for 32 cycles, every
+// other vector instruction costs 4 cycles of the same SIMD, and rescaling one
+// accumulator to a byte takes 4-5 of them.  The kernel is organised so that the
+// matrix core never waits for anything that can be had earlier:
+//  * operands go global -> LDS by direct loads (global_load_lds_dwordx4) into an
+//    S-stage ring that runs across tile boundaries; the loads of a step are
+//    issued S-1 steps before they are consumed, so S-1 stages are in flight;
+//  * fragments go LDS -> registers one MFMA K step (32 of K) ahead: while the
+//    MFMAs of one K step run, the ds_reads of the next are in flight, into the
+//    other of two register sets;
+//  * one barrier per stage, at its last K step, hands a stage over in both
+//    directions (the next stage has landed for everybody; this stage has been
+//    read by everybody and is refilled at once);
+//  * a block keeps one channel tile for its whole life and walks pixel tiles:
+//    bias lives in registers and is the C operand of a tile's first MFMAs, the
+//    rescale tables live in LDS;
+//  * the epilogue has no LDS staging and no barrier: rescaled values are packed
+//    to bytes, exchanged between the two lane halves (v_permlane32_swap) until
+//    a lane owns 16 or 32 consecutive channels of its pixel, and stored;
+//  * the steady state carries no address arithmetic for 1x1 kernels (uniform
+//    base + constant per-lane offset), and for KxK kernels one validity bit
+//    per tap and row, computed once per tile.
+//
+// Because the loads complete asynchronously, LDS accesses are explicit inline
+// ds_* instructions and the waits are written by hand.  s_waitcnt vmcnt(n)
+// counts the youngest operations that may still be outstanding; loads return
+// in order, so "at most n outstanding" implies every load older than the
+// youngest n has landed, whatever the epilogue's stores (which also count) do.
+// A thread issues the same number of loads at every step: steps past the end
+// of its work fetch rows that are marked invalid.
+#pragma once
+
+namespace n2d2hip {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+template <int OFF>
+__device__ __forceinline__ void lds_read128_nowait(v4i& v, unsigned addr)
+{
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_lgkm()
+{
+    asm volatile("s_waitcnt lgkmcnt(%0)" : : "n"(N) : "memory");
+}
+// Makes a register filled by an earlier asynchronous LDS read depend on the wait that precedes this call.
+__device__ __forceinline__ void tie(v4i& x) { asm volatile("" : "+v"(x)); }
+template <int N>
+__device__ __forceinline__ void wait_loads_and_barrier()
+{
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ int med3_i32(int x, int lo, int hi)
+{
+    int r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(lo), "v"(hi));
+    return r;
+}
+__device__ __forceinline__ float med3_f32(float x, float lo, float hi)
+{
+    float r;
+    asm("v_med3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(lo), "v"(hi));
+    return r;
+}
+// 4 saturated values -> one dword of bytes
+__device__ __forceinline__ unsigned pack_bytes(int r0, int r1, int r2, int r3)
+{
+    const unsigned t01 = __builtin_amdgcn_perm((unsigned)r1, (unsigned)r0, 0x0c0c0400u);
+    const unsigned t23 = __builtin_amdgcn_perm((unsigned)r3, (unsigned)r2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+}
+// n / d for 0 <= n < 2^31 with a host-made (multiplier, shift); multiplier 0 stands for d == 1
+__device__ __forceinline__ int div_magic(int n, unsigned mul, unsigned sh)
+{
+    return mul ? (int)(__umulhi((unsigned)n, mul) >> sh) : n;
+}
+
+struct ConvPipeArgs {
+    ConvArgs c;
+    const signed char* fill16;   // 16 bytes of the input's logical zero (device)
+    int mtiles, mlanes;          // pixel tiles, and how many block "lanes" walk them
+    int cper;                    // 64-byte K steps per kernel tap (C / 64)
+    int kW, kH;
+    unsigned ohw_mul, ohw_sh, ow_mul, ow_sh;     // division by OH*OW and by OW
+    int preclamp;                // I24: clamp before the multiply; F32: the cell has a Clip
+#ifdef N2D2HIP_PROFILE
+    long long* prof;             // 8 timestamps per block
+#endif
+};
+
+// 16-byte slot of (row, logical slot s) in a [rows][BK bytes] tile.  The XOR spreads the rows that one
+// ds_read_b128 touches for a fixed s over all banks.
+template <int BK>
+__device__ __forceinline__ int swz_k(int row, int s)
+{
+    return BK == 64 ? ((row << 2) + (s ^ ((row >> 2) & 3))) << 4 : ((row << 3) + (s ^ ((row >> 1) & 7))) << 4;
+}
+
+// NW waves as WGM (pixels) x NW/WGM (channels); a wave owns NJ x NI MFMA tiles of 32 pixels x 32 channels.
+// BK: bytes of K per ring stage and row (64 or 128); 128 makes every row segment a whole 128-byte line, which is
+// what the L2 -> LDS path moves fastest.
+template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pipe_kernel(ConvPipeArgs q)
+{
+    const ConvArgs& p = q.c;
+    constexpr int NT = NW * 64;                        // threads
+    constexpr int WGN = NW / WGM;
+    constexpr int TM = 32 * NJ, TN = 32 * NI;          // pixels x channels of a wave
+    constexpr int BM = TM * WGM, BN = TN * WGN;        // of the block
+    constexpr int LPR = BK / 16;                       // lanes (16-byte slots) per row
+    constexpr int RPC = 64 / LPR;                      // rows per 1 KB chunk = per wave-wide load
+    constexpr int KH = BK / 32;                        // MFMA K steps per stage
+    constexpr int TOFF = 32 * BK;                      // LDS bytes between MFMA tiles of one operand
+    // chunks each wave loads per step; when there are fewer chunks than waves some are loaded twice
+    constexpr int A_CH = BM / RPC, B_CH = BN / RPC;
+    constexpr int A_J = (A_CH + NW - 1) / NW, B_J = (B_CH + NW - 1) / NW;
+    constexpr int LPI = A_J + B_J;                     // loads per thread and step
+    constexpr int STAGE = (BM + BN) * BK;
+    constexpr int TAB_OFF = S * STAGE;                 // 6 int arrays of BN entries: bias, a, b, c, d, e
+    constexpr int NF = NI + NJ;                        // fragment reads per MFMA K step
+    static_assert(BK == 64 || BK == 128, "K bytes per stage");
+    static_assert(WGM * WGN == NW && BM % RPC == 0 && BN % RPC == 0, "wave grid");
+    static_assert(BK == 64 || (NW % 2 == 0 && A_CH % 2 == 0 && B_CH % 2 == 0), "a wave's chunks keep their parity");
+    static_assert(S >= 2, "ring depth");
+    static_assert(LPI * (S - 1) < 60, "vmcnt is a 6-bit counter");
+    static_assert((NJ - 1) * TOFF < 65536 && 6 * BN * 4 + 256 < 65536, "ds_read immediate offsets are 16 bits");
+
+    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + 6 * BN * 4];
+    const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WGM, wn = wave / WGM;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    // ---- which tiles this block walks: one channel tile, every mlanes-th pixel tile.
+    // Blocks 8 apart run on the same XCD; they take the same pixel tiles for neighbouring channel tiles.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int tile_n = slot % p.ntiles_n;
+    const int mlane = (slot / p.ntiles_n) * 8 + xcd;
+    const int n0 = tile_n * BN;
+    const int ntile = (mlane < q.mtiles) ? (q.mtiles - mlane + q.mlanes - 1) / q.mlanes : 0;
+    const int niter = p.niter;
+#ifdef N2D2HIP_PROFILE
+    long long pr_t0 = clock64(), pr_t1 = 0, pr_t2 = 0, pr_t3 = 0, pr_epi = 0, pr_w0 = wall_clock64();
+#endif
+
+    // ---- loader state.  Lane l of a wave fills 16-byte slot l of a 1 KB chunk: row l/LPR of the chunk,
+    // physical slot l%LPR, which holds the logical slot swz_k() maps there (chunk parity is the wave's parity).
+    const int lrow = lane / LPR;
+    const int lq = BK == 64 ? (lane & 3) ^ ((lane >> 4) & 3) : (lane & 7) ^ (((wave & 1) << 2) | (lane >> 4));
+    unsigned woff[B_J];            // byte offset of this thread's weight rows (without the K offset)
+#pragma unroll
+    for (int j = 0; j < B_J; ++j)
+        woff[j] = (unsigned)((n0 + ((wave + NW * j) % B_CH) * RPC + lrow) * p.ktot + lq * 16);
+    int rowoff[A_J];               // byte offset of the window origin of this thread's pixel rows (+ sub-chunk)
+    unsigned rowmask[A_J];         // bit t: kernel tap t of the row reads inside the input
+    int l_tile = 0, l_it = 0, l_koff = 0, l_stage = 0;
+    int l_c = 0, l_kx = 0, l_ky = 0, l_tap = 0, l_tapoff = 0;
+    auto loader_new_tile = [&]() {
+        const int m0 = (mlane + l_tile * q.mlanes) * BM;
+#pragma unroll
+        for (int j = 0; j < A_J; ++j) {
+            const int m = m0 + ((wave + NW * j) % A_CH) * RPC + lrow;
+            // branch-free (the block-uniform loader state must stay in scalar registers): rows past the end of
+            // the work are computed like pixel 0 and then masked
+            const bool live = (l_tile < ntile) & (m < p.M);
+            const int mm = live ? m : 0;
+            const int b = div_magic(mm, q.ohw_mul, q.ohw_sh);
+            const int rem = mm - b * (p.OH * p.OW);
+            const int oy = div_magic(rem, q.ow_mul, q.ow_sh);
+            const int ox = rem - oy * p.OW;
+            const int by = oy * p.strideY - p.padT, bx = ox * p.strideX - p.padL;
+            rowoff[j] = ((b * p.H + by) * p.W + bx) * p.in_cs + lq * 16;
+            rowmask[j] = 0u;
+            if (!ALLVALID) {
+                // tap index >= max(pad - o*stride, 0) and dilated offset inside the input
+                // (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83)
+                unsigned xmask = 0u;
+                for (int kx = 0; kx < q.kW; ++kx)
+                    xmask |= (unsigned)((kx >= -bx) & (kx * p.dilX < p.W - bx)) << kx;
+                unsigned mk = 0u;
+                for (int ky = 0; ky < q.kH; ++ky)
+                    mk |= ((ky >= -by) & (ky * p.dilY < p.H - by)) ? (xmask << (ky * q.kW)) : 0u;
+                rowmask[j] = live ? mk : 0u;
+            }
+        }
+    };
+    loader_new_tile();
+
+    // Issues the LPI loads of the loader's current step into its current ring stage, then advances the loader.
+    auto issue = [&]() {
+        unsigned char* sbase = smem + l_stage * STAGE;
+        if (ALLVALID) {
+            const signed char* ibase = p.in + l_koff;        // uniform; rows past the end read pixel 0
+#pragma unroll
+            for (int j = 0; j < A_J; ++j)
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)(ibase + (unsigned)rowoff[j]), (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
+        } else {
+            const unsigned tapbit = 1u << l_tap;
+#pragma unroll
+            for (int j = 0; j < A_J; ++j) {
+                const signed char* src = (rowmask[j] & tapbit) ? p.in + (rowoff[j] + l_tapoff) : q.fill16;
+                __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
+            }
+        }
+        const signed char* wbase = p.w + l_koff;
+#pragma unroll
+        for (int j = 0; j < B_J; ++j)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(wbase + woff[j]), (lds_ptr_t)(sbase + BM * BK + ((wave + NW * j) % B_CH) * 1024), 16, 0, 0);
+        l_stage = (l_stage + 1 == S) ? 0 : l_stage + 1;
+        l_koff += BK;
+        if (++l_it == niter) {
+            l_it = 0; l_koff = 0;
+            l_c = 0; l_kx = 0; l_ky = 0; l_tap = 0; l_tapoff = 0;
+            ++l_tile;
+            loader_new_tile();
+        } else if (!ALLVALID) {
+            l_tapoff += BK;
+            if (++l_c == q.cper) {
+                l_c = 0;
+                ++l_tap;
+                if (++l_kx == q.kW) { l_kx = 0; ++l_ky; }
+                l_tapoff = (l_ky * p.dilY * p.W + l_kx * p.dilX) * p.in_cs;
+            }
+        }
+    };
+
+    // ---- fragment addresses of the stage to read next: (operand, MFMA K step); tiles are immediates
+    unsigned pa[KH], wa[KH];
+#pragma unroll
+    for (int kk = 0; kk < KH; ++kk) {
+        pa[kk] = lds0 + swz_k<BK>(wm * TM + l32, 2 * kk + lh);
+        wa[kk] = lds0 + BM * BK + swz_k<BK>(wn * TN + l32, 2 * kk + lh);
+    }
+    int r_stage = 0;
+    const unsigned tab = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 4u;      // this lane's first channel in the tables
+
+    // two fragment sets: while the MFMAs of K step g run from set g%2, the reads of step g+1 fly into the other
+    v4i fw[2][NI], fp[2][NJ];
+    auto read_k = [&](auto kkc) {
+        constexpr int kk = decltype(kkc)::value;
+        constexpr int set = kk & 1;
+        lds_read128_nowait<0>(fw[set][0], wa[kk]);
+        if (NI > 1) lds_read128_nowait<TOFF>(fw[set][NI > 1 ? 1 : 0], wa[kk]);
+        lds_read128_nowait<0>(fp[set][0], pa[kk]);
+        if (NJ > 1) lds_read128_nowait<TOFF>(fp[set][NJ > 1 ? 1 : 0], pa[kk]);
+        if (NJ > 2) lds_read128_nowait<2 * TOFF>(fp[set][NJ > 2 ? 2 : 0], pa[kk]);
+        if (NJ > 3) lds_read128_nowait<3 * TOFF>(fp[set][NJ > 3 ? 3 : 0], pa[kk]);
+        if (kk == KH - 1) {
+            // every K step of this stage is requested: move on to the next stage of the ring
+            const bool wrap = r_stage + 1 == S;
+            const unsigned inc = wrap ? (unsigned)(-(S - 1) * STAGE) : (unsigned)STAGE;
+            r_stage = wrap ? 0 : r_stage + 1;
+#pragma unroll
+            for (int k2 = 0; k2 < KH; ++k2) { pa[k2] += inc; wa[k2] += inc; }
+        }
+    };
+
+    v16i acc[NI][NJ];
+    const bool out_bytes = p.out_dtype != N2D2HIP_I32;
+    const int vlo = p.epi.lo, vhi = p.epi.hi;
+    const float flo = (float)p.epi.lo, fhi = (float)p.epi.hi;
+
+    // ---- rescale, pack and store the finished tile
+    auto epilogue = [&](int c_tile) {
+        const int m0 = (mlane + c_tile * q.mlanes) * BM;
+        unsigned pk[NI][NJ][4];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
+                v4i ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
+                if (EPI != EPI_RAW) {
+                    lds_read128_nowait<BN * 4>(ta, trow);
+                    lds_read128_nowait<2 * BN * 4>(tb, trow);
+                    lds_read128_nowait<3 * BN * 4>(tc, trow);
+                    if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(td, trow);
+                    if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(te, trow);
+                    wait_lgkm<0>();
+                    tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                }
+                if (EPI == EPI_I24 && q.preclamp) {
+                    // the pre-clamp keeps the product inside 32 bits; it is skipped when the host has shown that no
+                    // accumulator of this layer can overflow it
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            acc[i][j][4 * g + t] = med3_i32(acc[i][j][4 * g + t], ta[t], tb[t]);
+                }
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    int r[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int v = acc[i][j][4 * g + t];
+                        if (EPI == EPI_I24) {
+                            // (v * c + half) >> e, saturated
+                            r[t] = med3_i32((__mul24(v, tc[t]) + td[t]) >> te[t], vlo, vhi);
+                        } else if (EPI == EPI_F32) {
+                            float f = (float)v;
+                            if (q.preclamp) f = fminf(fmaxf(f, as_f32(ta[t])), as_f32(tb[t]));
+                            f = round_half_away(f * as_f32(tc[t]));
+                            r[t] = (int)med3_f32(f, flo, fhi);
+                        } else {
+                            r[t] = epi_apply<EPI>(v, ta[t], tb[t], tc[t], td[t], te[t], p.epi.lo, p.epi.hi, p.epi.relu);
+                        }
+                    }
+                    if (out_bytes) {
+                        pk[i][j][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ p.out_xor;
+                    } else {
+                        const int m = m0 + wm * TM + j * 32 + l32;
+                        const int ch = n0 + wn * TN + i * 32 + 8 * g + 4 * lh;
+                        if (m < p.M && ch < p.out_cs)
+                            *(int4*)((int*)p.out + (long long)m * p.out_cs + ch) = int4{r[0], r[1], r[2], r[3]};
+                    }
+                }
+            }
+        }
+        if (!out_bytes)
+            return;
+        // pk[i][j][g] holds channels 8g + 4*lh .. +3 of tile i.  Swapping g = 2,3 of the lower lane half with g = 0,1 of
+        // the upper one leaves every lane with 16 consecutive channels (16*lh ..) of its pixel; a second exchange
+        // between the two channel tiles makes that 32 (32*lh ..).
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int m = m0 + wm * TM + j * 32 + l32;
+            signed char* orow = (signed char*)p.out + (long long)m * p.out_cs + (n0 + wn * TN);
+            unsigned qd[NI][4];
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const auto s02 = __builtin_amdgcn_permlane32_swap(pk[i][j][0], pk[i][j][2], false, false);
+                const auto s13 = __builtin_amdgcn_permlane32_swap(pk[i][j][1], pk[i][j][3], false, false);
+                qd[i][0] = s02[0]; qd[i][1] = s02[1]; qd[i][2] = s13[0]; qd[i][3] = s13[1];
+            }
+            if (NI == 2) {
+                v4i first, second;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const auto x = __builtin_amdgcn_permlane32_swap(qd[0][e], qd[NI - 1][e], false, false);
+                    first[e] = (int)x[0];
+                    second[e] = (int)x[1];
+                }
+                const int ch = n0 + wn * TN + 32 * lh;
+                if (m < p.M) {
+                    if (ch < p.out_cs) *(v4i*)(orow + 32 * lh) = first;
+                    if (ch + 16 < p.out_cs) *(v4i*)(orow + 32 * lh + 16) = second;
+                }
+            } else {
+                static_assert(NI <= 2, "one or two channel tiles per wave");
+                const v4i only = {(int)qd[0][0], (int)qd[0][1], (int)qd[0][2], (int)qd[0][3]};
+                const int ch = n0 + wn * TN + 16 * lh;
+                if (m < p.M && ch < p.out_cs) *(v4i*)(orow + 16 * lh) = only;
+            }
+        }
+    };
+
+    // ---- fill the ring: the first S steps occupy all S stages
+#ifdef N2D2HIP_PROFILE
+    pr_t1 = clock64();
+#endif
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+        issue();
+
+    // ---- per-block constants into LDS while the first loads fly: bias and rescale tables of the channel tile
+    {
+        int* tabw = (int*)(smem + TAB_OFF);
+        for (int i = tid; i < BN; i += NT) {
+            tabw[i] = p.bias[n0 + i];
+            if (EPI != EPI_RAW) {
+                tabw[BN + i] = p.epi.a[n0 + i];
+                tabw[2 * BN + i] = p.epi.b[n0 + i];
+                tabw[3 * BN + i] = p.epi.c[n0 + i];
+                tabw[4 * BN + i] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
+                tabw[5 * BN + i] = (EPI != EPI_F32) ? p.epi.e[n0 + i] : 0;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- the bias of this lane's channels (rows 8g + 4*lh + t of each 32-channel tile): C operand of a tile's first MFMAs
+    v16i biasv[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        v4i b0, b1, b2, b3;
+        const unsigned t = tab + (unsigned)i * 128u;
+        lds_read128_nowait<0>(b0, t); lds_read128_nowait<32>(b1, t); lds_read128_nowait<64>(b2, t); lds_read128_nowait<96>(b3, t);
+        wait_lgkm<0>();
+        tie(b0); tie(b1); tie(b2); tie(b3);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            biasv[i][e] = b0[e]; biasv[i][4 + e] = b1[e]; biasv[i][8 + e] = b2[e]; biasv[i][12 + e] = b3[e];
+        }
+    }
+
+
+    if (ntile > 0) {
+        wait_loads_and_barrier<LPI*(S - 1)>();         // step 0 has landed
+#ifdef N2D2HIP_PROFILE
+        pr_t2 = clock64();
+#endif
+        read_k(std::integral_constant<int, 0>());
+        for (int c_tile = 0; c_tile < ntile; ++c_tile) {
+            for (int it = 0; it < niter; ++it) {
+                // MFMA K step kk of this stage.  Its fragments were requested one K step ago; the next ones are
+                // requested before its MFMAs are issued, so that they return while those run.
+                auto kstep = [&](auto kkc) {
+                    constexpr int kk = decltype(kkc)::value;
+                    constexpr int set = kk & 1;
+                    wait_lgkm<0>();
+#pragma unroll
+                    for (int i = 0; i < NI; ++i) tie(fw[set][i]);
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) tie(fp[set][j]);
+                    if (kk == KH - 1) {
+                        // Every wave has its last fragments of this stage, so the stage can be refilled; and the next
+                        // stage has landed for every wave.
+                        wait_loads_and_barrier<LPI*(S - 2)>();
+                        issue();
+                    }
+                    read_k(std::integral_constant<int, (kk + 1) % KH>());      // of this stage, or of the next one
+                    if (kk == 0 && it == 0) {
+#pragma unroll
+                        for (int i = 0; i < NI; ++i)
+#pragma unroll
+                            for (int j = 0; j < NJ; ++j)
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[set][i], fp[set][j], biasv[i], 0, 0, 0);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < NI; ++i)
+#pragma unroll
+                            for (int j = 0; j < NJ; ++j)
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[set][i], fp[set][j], acc[i][j], 0, 0, 0);
+                    }
+                };
+                kstep(std::integral_constant<int, 0>());
+                kstep(std::integral_constant<int, 1>());
+                if constexpr (KH > 2) {
+                    kstep(std::integral_constant<int, 2 % KH>());
+                    kstep(std::integral_constant<int, 3 % KH>());
+                }
+            }
+#ifdef N2D2HIP_PROFILE
+            const long long e0 = clock64();
+            epilogue(c_tile);
+            pr_epi += clock64() - e0;
+#else
+            epilogue(c_tile);
+#endif
+        }
+    }
+#ifdef N2D2HIP_PROFILE
+    pr_t3 = clock64();
+    if (tid == 0) {
+        long long* o = q.prof + (long long)blockIdx.x * 8;
+        o[0] = pr_t0; o[1] = pr_t1; o[2] = pr_t2; o[3] = pr_t3; o[4] = pr_epi; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = ntile * niter;
+    }
+#endif
+    // no load may still be writing into LDS when the block's LDS is handed to another block
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
+}
+
+} // namespace n2d2hip
