@@ -149,6 +149,7 @@ int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH
 int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
 
+
 /* -------------------------------------------------------------------- fc */
 typedef struct n2d2hip_conv_s* n2d2hip_fc_t;
 /* Quantized FcCell over a C x H x W input: weights HOST int8 [O][C*H*W] in N2D2's CHW
@@ -193,6 +194,20 @@ int n2d2hip_elemwise_create(int nb_inputs, int nb_channels, int coeff_mode, cons
  * an integer mode whose products fit 32 bits: the caller then keeps the ScalingCell as a separate launch. */
 int n2d2hip_elemwise_fold_input_scaling(n2d2hip_elemwise_t ew, int input_index, n2d2hip_act_t scaling);
 int n2d2hip_elemwise_destroy(n2d2hip_elemwise_t ew);
+
+/* Graph-level fusion: the two-input ElemWise sum that consumes this convolution's output is computed in the
+ * convolution's epilogue, i.e. ConvCell_Frame::propagate followed by ElemWiseCell_Frame::propagate (Sum)
+ * (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/ElemWiseCell_Frame.cpp:104-136) in one launch; the convolution's
+ * own output tensor is never written.  `conv_input_index` (0 or 1) is the sum's input the convolution feeds; the other
+ * input is passed to n2d2hip_conv_forward_sum and has storage type `other_dtype`.  A ScalingCell folded into the sum
+ * with n2d2hip_elemwise_fold_input_scaling must sit on that other input and is applied too.  `sum` is borrowed and must
+ * outlive the convolution; NULL undoes the fusion.  Returns N2D2HIP_ERR_UNSUPPORTED (and changes nothing) unless the
+ * convolution is 1x1, unpadded, 8-bit, with input and output channel counts that are multiples of 64, and both cells
+ * rescale with an integer Scaling mode: the caller then keeps the two launches. */
+int n2d2hip_conv_fuse_sum(n2d2hip_conv_t conv, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype);
+/* out = sum(conv(in), other) for a convolution prepared with n2d2hip_conv_fuse_sum; `out` has the sum cell's range. */
+int n2d2hip_conv_forward_sum(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
+                             const n2d2hip_tensor* out, n2d2hip_stream_t stream);
 int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
                              n2d2hip_stream_t stream);
 

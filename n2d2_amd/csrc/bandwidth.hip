@@ -247,15 +247,6 @@ int run_scaling_nhwc(const n2d2hip_act_s* act, const n2d2hip_tensor* in, const n
 
 using namespace n2d2hip;
 
-struct n2d2hip_elemwise_s {
-    int nb_inputs, nb_channels, cpad;
-    n2d2hip_act_t act;
-    float* d_coeff;     // w then s, each [nb_inputs][cpad]
-    bool unit_coeff;    // every weight 1 and every shift 0
-    int pre_input;      // input carrying a folded ScalingCell (-1: none)
-    n2d2hip_act_t pre_act;
-};
-
 extern "C" {
 
 int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* d, int H, int W, int* outH, int* outW)

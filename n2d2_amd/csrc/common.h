@@ -90,3 +90,12 @@ struct n2d2hip_act_s {
     std::vector<int> htab;     // host copy of the tables (empty for RAW)
     bool clipped;              // the Scaling applies a Clip
 };
+
+struct n2d2hip_elemwise_s {
+    int nb_inputs, nb_channels, cpad;
+    n2d2hip_act_t act;
+    float* d_coeff;     // w then s, each [nb_inputs][cpad]
+    bool unit_coeff;    // every weight 1 and every shift 0
+    int pre_input;      // input carrying a folded ScalingCell (-1: none)
+    n2d2hip_act_t pre_act;
+};

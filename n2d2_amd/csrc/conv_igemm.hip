@@ -356,6 +356,14 @@ struct n2d2hip_conv_s {
     int* d_bias;
     signed char* d_fill;  // 16 bytes of the input's logical zero, source of padded taps in the direct-to-LDS kernel
     bool preclamp;        // some accumulator could overflow the rescale's 24x24 -> 32 bit product, or the cell has a Clip
+    // residual sum folded into the epilogue (n2d2hip_conv_fuse_sum)
+    n2d2hip_elemwise_t sum;
+    int sum_other_dtype;  // storage type the tables below were made for
+    int* d_res_tab;       // sum a,b,c,d,e then pre a,b,c,d,e, each [cpad], zero point of the other input folded in
+    bool has_pre, pre_clamp, sum_clamp;
+    // integer rescale with the bias folded in, for the pipelined kernel: a - bias, b - bias, c, d + bias * c, e, each [cpad]
+    int* d_epi_tab;
+    bool bias_folded;
     bool is_fc;
     int fcH, fcW;
 };
@@ -394,6 +402,14 @@ void launch_pipe(ConvPipeArgs a, bool all_valid, int grid, hipStream_t stream)
     default: N2D2HIP_PIPE(EPI_F32); break;
     }
 #undef N2D2HIP_PIPE
+}
+
+template <int NW, int BK, int NI, int NJ, int WGM, int S>
+void launch_pipe_res(ConvPipeArgs a, int grid, hipStream_t stream)
+{
+    a.c.niter = a.c.ktot / BK;
+    a.cper = a.c.in_cs / BK;
+    hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
 }
 
 // (multiplier, shift) with n / d == umulhi(n, multiplier) >> shift for 0 <= n < 2^31; multiplier 0 stands for d == 1
@@ -472,6 +488,8 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false;
+    c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
         delete c;
@@ -515,6 +533,27 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         }
     } else if (act->args.kind != EPI_F32) {
         c->preclamp = true;
+    }
+    // The pipelined kernel starts its accumulators from zero and finds the bias inside the integer rescale:
+    // ((v + bias) * c + d) >> e == (v * c + (d + bias * c)) >> e in wrapping 32-bit arithmetic, the pre-clamp bounds move
+    // by the bias and must stay 24-bit for the multiplier.
+    std::vector<int> hepi;
+    if (act->args.kind == EPI_I24 && !depthwise) {
+        const int cp = act->cpad;
+        hepi.assign(5 * (size_t)cp, 0);
+        c->bias_folded = true;
+        for (int ch = 0; ch < cp; ++ch) {
+            const long long b = hbias[ch];
+            const long long lo = (long long)act->htab[ch] - b, hi = (long long)act->htab[cp + ch] - b;
+            const long long m = act->htab[2 * (size_t)cp + ch];
+            if (c->preclamp && (lo <= -(1ll << 23) || hi >= (1ll << 23)))
+                c->bias_folded = false;
+            hepi[ch] = (int)std::max<long long>(std::min<long long>(lo, std::numeric_limits<int>::max()), std::numeric_limits<int>::min());
+            hepi[cp + ch] = (int)std::max<long long>(std::min<long long>(hi, std::numeric_limits<int>::max()), std::numeric_limits<int>::min());
+            hepi[2 * (size_t)cp + ch] = (int)m;
+            hepi[3 * (size_t)cp + ch] = (int)(unsigned)(unsigned long long)((long long)act->htab[3 * (size_t)cp + ch] + b * m);
+            hepi[4 * (size_t)cp + ch] = act->htab[4 * (size_t)cp + ch];
+        }
     }
 
     if (depthwise) {
@@ -575,6 +614,10 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     if (e == hipSuccess) e = hipMemcpy(c->d_w, hw.data(), hw.size(), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMalloc((void**)&c->d_bias, hbias.size() * sizeof(int));
     if (e == hipSuccess) e = hipMemcpy(c->d_bias, hbias.data(), hbias.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e == hipSuccess && !hepi.empty()) {
+        e = hipMalloc((void**)&c->d_epi_tab, hepi.size() * sizeof(int));
+        if (e == hipSuccess) e = hipMemcpy(c->d_epi_tab, hepi.data(), hepi.size() * sizeof(int), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hsub.empty()) {
         e = hipMalloc((void**)&c->d_sub, hsub.size() * sizeof(int4));
         if (e == hipSuccess) e = hipMemcpy(c->d_sub, hsub.data(), hsub.size() * sizeof(int4), hipMemcpyHostToDevice);
@@ -600,11 +643,25 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_sub) (void)hipFree(c->d_sub);
     if (c->d_bias) (void)hipFree(c->d_bias);
     if (c->d_fill) (void)hipFree(c->d_fill);
+    if (c->d_res_tab) (void)hipFree(c->d_res_tab);
+    if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
     delete c;
     return N2D2HIP_OK;
 }
 
-int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream_)
+// Can this convolution run on the pipelined kernel, and with which channel tile?
+static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
+{
+    const n2d2hip_conv_desc& d = c->desc;
+    const int opad_n = round_up(d.O, 64);
+    *bn128 = opad_n % 128 == 0 || opad_n > 256;
+    const int k = c->act->args.kind;
+    return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 32
+        && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
+}
+
+static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* other, const n2d2hip_tensor* out,
+                             n2d2hip_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     int rc;
@@ -623,7 +680,16 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
                     "conv_forward: output is %dx%dx%dx%d, expected %dx%dx%dx%d", out->B, out->C, out->H, out->W, in->B, d.O, OH, OW);
     N2D2HIP_REQUIRE(out->cs % 16 == 0, N2D2HIP_ERR_INVALID, "conv_forward: output channel stride %d must be a multiple of 16", out->cs);
-    const n2d2hip_act_s* act = c->act;
+    // with a folded sum the stored values are the sum cell's
+    const n2d2hip_act_s* act = other ? c->sum->act : c->act;
+    if (other) {
+        if ((rc = check_tensor(other, "sum input")))
+            return rc;
+        N2D2HIP_REQUIRE(other->layout == N2D2HIP_NHWC && other->dtype == c->sum_other_dtype && other->B == out->B && other->C == out->C
+                        && other->H == out->H && other->W == out->W && other->cs % 16 == 0 && other->cs >= round_up(d.O, 16),
+                        N2D2HIP_ERR_INVALID, "conv_forward_sum: the other input must be an NHWC tensor of the output's shape and of the "
+                        "storage type given to n2d2hip_conv_fuse_sum");
+    }
     if (act->args.kind == EPI_RAW) {
         N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_INVALID,
                         "conv_forward: without a rescale the cell outputs raw sums; the output dtype must be I32");
@@ -645,7 +711,7 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
         const unsigned grid = (unsigned)std::min<long long>((total + 255) / 256, 256 * 64);
         hipLaunchKernelGGL(depthwise_kernel, dim3(grid), dim3(256), 0, stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, OH, OW, c->d_w, d.kH, d.kW, c->d_bias, out->data, out->dtype, d.strideX, d.strideY, d.padL,
-                           d.padT, d.dilX, d.dilY, zero_point(in->dtype), out_xor, act->args);
+                           d.padT, d.dilX, d.dilY, zero_point(in->dtype), out_xor, c->act->args);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }
@@ -659,7 +725,7 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     a.strideX = d.strideX; a.strideY = d.strideY; a.padL = d.padL; a.padT = d.padT; a.dilX = d.dilX; a.dilY = d.dilY;
     a.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
     a.out_xor = out_xor;
-    a.epi = act->args;
+    a.epi = c->act->args;
 
     // Tile choice: 128 channels per block when the layer has them, and 64-pixel
     // tiles when 128-pixel tiles would leave most of the 256 CUs idle.
@@ -673,9 +739,10 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     const int BM = bm64 ? 64 : 128;
     a.nblocks = (int)(((Mll + BM - 1) / BM) * a.ntiles_n);
     const bool fits32 = (long long)in->B * in->H * in->W * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
-    const bool pipe_kind = act->args.kind == EPI_RAW || act->args.kind == EPI_I24 || act->args.kind == EPI_F32;
-    if (!c->pix4 && !w4 && in->cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 32 && pipe_kind && fits32
-        && getenv("N2D2HIP_NO_PIPE") == nullptr) {
+    bool bn128_unused;
+    const bool pipe = pipe_eligible(c, &bn128_unused) && fits32;
+    N2D2HIP_REQUIRE(!other || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward_sum: tensor too large for the fused kernel");
+    if (pipe && (other || getenv("N2D2HIP_NO_PIPE") == nullptr)) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
         ConvPipeArgs q;
         q.c = a;
@@ -683,6 +750,11 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
         q.cper = d.C / 64;
         q.kW = d.kW; q.kH = d.kH;
         q.preclamp = c->preclamp ? 1 : 0;
+        if (c->act->args.kind == EPI_I24) {
+            const int cp = c->act->cpad;
+            q.c.epi.a = c->d_epi_tab; q.c.epi.b = c->d_epi_tab + cp; q.c.epi.c = c->d_epi_tab + 2 * cp;
+            q.c.epi.d = c->d_epi_tab + 3 * cp; q.c.epi.e = c->d_epi_tab + 4 * cp;
+        }
 #ifdef N2D2HIP_PROFILE
         q.prof = (long long*)strtoull(getenv("N2D2HIP_PROF_PTR"), nullptr, 16);
 #endif
@@ -696,7 +768,30 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
         q.mlanes = 8 * per_xcd;
         const int grid = 8 * a.ntiles_n * per_xcd;
-        if (d.C % 128 == 0) {
+        q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
+        q.sum = EpiArgs(); q.pre = EpiArgs();
+        if (other) {
+            const int cp = c->sum->act->cpad;
+            q.res = (const signed char*)other->data;
+            q.res_cs = other->cs;
+            q.res_flip = other->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
+            q.sum = c->sum->act->args;
+            q.sum.a = c->d_res_tab; q.sum.b = c->d_res_tab + cp; q.sum.c = c->d_res_tab + 2 * cp;
+            q.sum.d = c->d_res_tab + 3 * cp; q.sum.e = c->d_res_tab + 4 * cp;
+            q.has_pre = c->has_pre; q.pre_clamp = c->pre_clamp; q.sum_clamp = c->sum_clamp;
+            if (c->has_pre) {
+                q.pre = c->sum->pre_act->args;
+                q.pre.a = c->d_res_tab + 5 * cp; q.pre.b = c->d_res_tab + 6 * cp; q.pre.c = c->d_res_tab + 7 * cp;
+                q.pre.d = c->d_res_tab + 8 * cp; q.pre.e = c->d_res_tab + 9 * cp;
+            }
+            if (d.C % 128 == 0) {
+                if (bn128) launch_pipe_res<4, 128, 2, 2, 2, 2>(q, grid, stream);
+                else launch_pipe_res<4, 128, 2, 1, 4, 3>(q, grid, stream);
+            } else {
+                if (bn128) launch_pipe_res<4, 64, 2, 2, 2, 4>(q, grid, stream);
+                else launch_pipe_res<4, 64, 2, 1, 4, 4>(q, grid, stream);
+            }
+        } else if (d.C % 128 == 0) {
             if (bn128) launch_pipe<4, 128, 2, 2, 2, 2>(q, all_valid, grid, stream);
             else launch_pipe<4, 128, 2, 1, 4, 3>(q, all_valid, grid, stream);
         } else {
@@ -718,6 +813,94 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
+}
+
+int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    return conv_forward_impl(c, in, nullptr, out, stream);
+}
+
+int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype)
+{
+    N2D2HIP_REQUIRE(c != nullptr, N2D2HIP_ERR_INVALID, "conv_fuse_sum: null conv");
+    if (c->d_res_tab) { (void)hipFree(c->d_res_tab); c->d_res_tab = nullptr; }
+    c->sum = nullptr;
+    if (!sum)
+        return N2D2HIP_OK;
+    N2D2HIP_REQUIRE(conv_input_index == 0 || conv_input_index == 1, N2D2HIP_ERR_INVALID, "conv_fuse_sum: input index %d", conv_input_index);
+    N2D2HIP_REQUIRE(is_byte_type(other_dtype), N2D2HIP_ERR_INVALID, "conv_fuse_sum: the other input must be U8, I8 or U8B");
+    const n2d2hip_conv_desc& d = c->desc;
+    N2D2HIP_REQUIRE(sum->nb_channels == d.O, N2D2HIP_ERR_INVALID, "conv_fuse_sum: the sum has %d channels, the conv %d outputs", sum->nb_channels, d.O);
+    bool bn128;
+    const bool one_by_one = d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0;
+    const n2d2hip_act_s* ca = c->act;
+    const n2d2hip_act_s* sa = sum->act;
+    const n2d2hip_act_s* pa = sum->pre_input >= 0 ? sum->pre_act : nullptr;
+    const bool ok = pipe_eligible(c, &bn128) && one_by_one && round_up(d.O, 16) % (bn128 ? 128 : 64) == 0
+        && ca->args.kind == EPI_I24 && ca->min_out >= -128 && ca->max_out <= 255
+        && sum->nb_inputs == 2 && sum->unit_coeff && sa->args.kind == EPI_I24 && sa->min_out >= -128 && sa->max_out <= 255
+        && (sum->pre_input < 0 || sum->pre_input == 1 - conv_input_index);
+    N2D2HIP_REQUIRE(ok, N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_fuse_sum: needs a 1x1 unpadded 8-bit convolution with a multiple of 64 input and output channels and integer "
+                    "rescales on the convolution and on a two-input unit-coefficient sum");
+    // Tables of the sum (and of the ScalingCell folded onto the other input) with the other input's zero point
+    // folded in: the kernel adds the stored byte as a signed value.
+    const int cp = sa->cpad;
+    const long long zp = zero_point(other_dtype == N2D2HIP_U8 ? N2D2HIP_U8B : other_dtype);
+    const long long IMIN = std::numeric_limits<int>::min(), IMAX = std::numeric_limits<int>::max();
+    std::vector<int> t(10 * (size_t)cp, 0);
+    bool pre_clamp = pa ? pa->clipped : false, sum_clamp = sa->clipped;
+    const long long other_lo = pa ? pa->min_out : (other_dtype == N2D2HIP_I8 ? -128 : 0);
+    const long long other_hi = pa ? pa->max_out : (other_dtype == N2D2HIP_I8 ? 127 : 255);
+    for (int ch = 0; ch < cp; ++ch) {
+        // sum: s = conv + other (+ zp when there is no ScalingCell in between)
+        const long long szp = pa ? 0 : zp;
+        const long long a = sa->htab[ch], b = sa->htab[cp + ch], m = sa->htab[2 * (size_t)cp + ch], dd = sa->htab[3 * (size_t)cp + ch];
+        t[ch] = (int)std::min(IMAX, std::max(IMIN, a - szp));
+        t[cp + ch] = (int)std::min(IMAX, std::max(IMIN, b - szp));
+        t[2 * (size_t)cp + ch] = (int)m;
+        const long long d2 = dd + szp * m;
+        t[4 * (size_t)cp + ch] = sa->htab[4 * (size_t)cp + ch];
+        const long long smax = std::max(std::llabs(ca->min_out + other_lo - szp), std::llabs(ca->max_out + other_hi - szp)) + 1;
+        if (d2 < IMIN || d2 > IMAX)
+            return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_fuse_sum: the sum's rescale of channel %d leaves 32 bits once folded", ch);
+        if (smax * m + std::llabs(d2) > IMAX)
+            sum_clamp = true;
+        t[3 * (size_t)cp + ch] = (int)d2;
+        if (pa) {
+            const long long xa = pa->htab[ch], xb = pa->htab[cp + ch], xm = pa->htab[2 * (size_t)cp + ch], xd = pa->htab[3 * (size_t)cp + ch];
+            const long long xd2 = xd + zp * xm;
+            if (xd2 < IMIN || xd2 > IMAX || 256 * xm + std::llabs(xd2) > IMAX)
+                pre_clamp = true;
+            if (xd2 < IMIN || xd2 > IMAX)
+                return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_fuse_sum: the folded ScalingCell of channel %d leaves 32 bits", ch);
+            t[5 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xa - zp));
+            t[6 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xb - zp));
+            t[7 * (size_t)cp + ch] = (int)xm;
+            t[8 * (size_t)cp + ch] = (int)xd2;
+            t[9 * (size_t)cp + ch] = pa->htab[4 * (size_t)cp + ch];
+        }
+    }
+    hipError_t e = hipMalloc((void**)&c->d_res_tab, t.size() * sizeof(int));
+    if (e == hipSuccess) e = hipMemcpy(c->d_res_tab, t.data(), t.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (c->d_res_tab) { (void)hipFree(c->d_res_tab); c->d_res_tab = nullptr; }
+        return fail(N2D2HIP_ERR_HIP, "conv_fuse_sum: device upload failed: %s", hipGetErrorString(e));
+    }
+    c->sum = sum;
+    c->sum_other_dtype = other_dtype;
+    c->has_pre = pa != nullptr;
+    c->pre_clamp = pre_clamp;
+    c->sum_clamp = sum_clamp;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv_forward_sum(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* other, const n2d2hip_tensor* out,
+                             n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(c != nullptr && other != nullptr, N2D2HIP_ERR_INVALID, "conv_forward_sum: null argument");
+    N2D2HIP_REQUIRE(c->sum != nullptr, N2D2HIP_ERR_INVALID, "conv_forward_sum: no sum has been folded into this convolution");
+    return conv_forward_impl(c, in, other, out, stream);
 }
 
 // ------------------------------------------------------------------- fc

@@ -89,6 +89,13 @@ struct ConvPipeArgs {
     int kW, kH;
     unsigned ohw_mul, ohw_sh, ow_mul, ow_sh;     // division by OH*OW and by OW
     int preclamp;                // I24: clamp before the multiply; F32: the cell has a Clip
+    // Folded residual sum (RES kernels): out = sum_act(conv_act(conv) + pre(other)), all EPI_I24
+    const signed char* res;      // the sum's other input, NHWC bytes
+    int res_cs;
+    unsigned res_flip;           // 0x80808080 for plain U8 storage (turns it into value-128)
+    EpiArgs sum;                 // the sum cell's rescale; its d table has the other input's zero point folded in
+    EpiArgs pre;                 // ScalingCell folded onto the other input (d table with the zero point folded in)
+    int has_pre, pre_clamp, sum_clamp;
 #ifdef N2D2HIP_PROFILE
     long long* prof;             // 8 timestamps per block
 #endif
@@ -105,7 +112,8 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // NW waves as WGM (pixels) x NW/WGM (channels); a wave owns NJ x NI MFMA tiles of 32 pixels x 32 channels.
 // BK: bytes of K per ring stage and row (64 or 128); 128 makes every row segment a whole 128-byte line, which is
 // what the L2 -> LDS path moves fastest.
-template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID>
+// RES: the residual sum that follows the convolution is computed in the epilogue (1x1 convolutions, EPI_I24).
+template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID, bool RES = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pipe_kernel(ConvPipeArgs q)
 {
     const ConvArgs& p = q.c;
@@ -123,15 +131,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int LPI = A_J + B_J;                     // loads per thread and step
     constexpr int STAGE = (BM + BN) * BK;
     constexpr int TAB_OFF = S * STAGE;                 // 6 int arrays of BN entries: bias, a, b, c, d, e
+    constexpr int NTAB = RES ? 16 : 6;                 // RES: + a..e of the sum cell, + a..e of the folded ScalingCell
+    static_assert(!RES || EPI == EPI_I24, "the folded sum is integer arithmetic");
     constexpr int NF = NI + NJ;                        // fragment reads per MFMA K step
+    constexpr bool BIAS_REG = EPI != EPI_I24;          // the integer rescale carries the bias in its tables
     static_assert(BK == 64 || BK == 128, "K bytes per stage");
     static_assert(WGM * WGN == NW && BM % RPC == 0 && BN % RPC == 0, "wave grid");
     static_assert(BK == 64 || (NW % 2 == 0 && A_CH % 2 == 0 && B_CH % 2 == 0), "a wave's chunks keep their parity");
     static_assert(S >= 2, "ring depth");
     static_assert(LPI * (S - 1) < 60, "vmcnt is a 6-bit counter");
-    static_assert((NJ - 1) * TOFF < 65536 && 6 * BN * 4 + 256 < 65536, "ds_read immediate offsets are 16 bits");
+    static_assert((NJ - 1) * TOFF < 65536 && NTAB * BN * 4 + 256 < 65536, "ds_read immediate offsets are 16 bits");
 
-    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + 6 * BN * 4];
+    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + NTAB * BN * 4];
     const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
 
     const int tid = threadIdx.x;
@@ -268,60 +279,164 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const bool out_bytes = p.out_dtype != N2D2HIP_I32;
     const int vlo = p.epi.lo, vhi = p.epi.hi;
     const float flo = (float)p.epi.lo, fhi = (float)p.epi.hi;
+    const int plo = q.pre.lo, phi = q.pre.hi, slo = q.sum.lo, shi = q.sum.hi;
 
     // ---- rescale, pack and store the finished tile
     auto epilogue = [&](int c_tile) {
         const int m0 = (mlane + c_tile * q.mlanes) * BM;
         unsigned pk[NI][NJ][4];
+        // RES: the other input's bytes for this lane's accumulators, 4 channels per dword.  They are read the way the
+        // output is written, 32 consecutive channels of a pixel per lane (whole 32-byte sectors, every line touched
+        // once), and brought into the accumulators' layout by running the output's lane-half exchanges backwards
+        // (the exchange is its own inverse).  These loads are younger than every load of the ring, so waiting for
+        // them also waits for the stage in flight.
+        unsigned resw[RES ? NI * 4 : 1][RES ? NJ : 1];
+        if (RES) {
+            static_assert(!RES || NI == 2, "the folded sum is written for two channel tiles per wave");
+            v4i first[NJ], second[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int m = m0 + wm * TM + j * 32 + l32;
+                const signed char* rp = q.res + (long long)(m < p.M ? m : 0) * q.res_cs + (n0 + wn * TN + 32 * lh);
+                asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
+                             : "=&v"(first[j]), "=&v"(second[j]) : "v"(rp) : "memory");
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                tie(first[j]); tie(second[j]);
+                unsigned qd[2][4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const auto y = __builtin_amdgcn_permlane32_swap((unsigned)first[j][e], (unsigned)second[j][e], false, false);
+                    qd[0][e] = y[0]; qd[1][e] = y[1];
+                }
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(qd[i][0], qd[i][1], false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(qd[i][2], qd[i][3], false, false);
+                    resw[RES ? i * 4 + 0 : 0][RES ? j : 0] = s02[0];
+                    resw[RES ? i * 4 + 2 : 0][RES ? j : 0] = s02[1];
+                    resw[RES ? i * 4 + 1 : 0][RES ? j : 0] = s13[0];
+                    resw[RES ? i * 4 + 3 : 0][RES ? j : 0] = s13[1];
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                const int idx = i * 4 + g;
                 const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
-                v4i ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
-                if (EPI != EPI_RAW) {
-                    lds_read128_nowait<BN * 4>(ta, trow);
-                    lds_read128_nowait<2 * BN * 4>(tb, trow);
-                    lds_read128_nowait<3 * BN * 4>(tc, trow);
-                    if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(td, trow);
-                    if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(te, trow);
-                    wait_lgkm<0>();
-                    tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                int r[NJ][4];
+                {
+                    // ---- the convolution's own rescale
+                    v4i ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
+                    if (EPI != EPI_RAW) {
+                        lds_read128_nowait<BN * 4>(ta, trow);
+                        lds_read128_nowait<2 * BN * 4>(tb, trow);
+                        lds_read128_nowait<3 * BN * 4>(tc, trow);
+                        if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(td, trow);
+                        if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(te, trow);
+                        wait_lgkm<0>();
+                        tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                    }
+                    if (EPI == EPI_I24 && q.preclamp) {
+                        // the pre-clamp keeps the product inside 32 bits; it is skipped when the host has shown that no
+                        // accumulator of this layer can overflow it
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                acc[i][j][4 * g + t] = med3_i32(acc[i][j][4 * g + t], ta[t], tb[t]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) {
+                            const int v = acc[i][j][4 * g + t];
+                            if (EPI == EPI_I24) {
+                                // (v * c + half) >> e, saturated; the bias is inside `half`
+                                r[j][t] = med3_i32((__mul24(v, tc[t]) + td[t]) >> te[t], vlo, vhi);
+                            } else if (EPI == EPI_F32) {
+                                float f = (float)v;
+                                if (q.preclamp) f = fminf(fmaxf(f, as_f32(ta[t])), as_f32(tb[t]));
+                                f = round_half_away(f * as_f32(tc[t]));
+                                r[j][t] = (int)med3_f32(f, flo, fhi);
+                            } else {
+                                r[j][t] = epi_apply<EPI>(v, ta[t], tb[t], tc[t], td[t], te[t], p.epi.lo, p.epi.hi, p.epi.relu);
+                            }
+                        }
                 }
-                if (EPI == EPI_I24 && q.preclamp) {
-                    // the pre-clamp keeps the product inside 32 bits; it is skipped when the host has shown that no
-                    // accumulator of this layer can overflow it
+                if (RES) {
+                    // ---- + the other input of the sum, through its folded ScalingCell if there is one, then the sum's
+                    // own rescale (ref: src/Cell/ElemWiseCell_Frame.cpp:116-136 with unit coefficients)
+                    int o[NJ][4];
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const unsigned w = resw[RES ? idx : 0][RES ? j : 0] ^ q.res_flip;
+                        o[j][0] = (int)(signed char)(w & 0xffu);
+                        o[j][1] = (int)(signed char)((w >> 8) & 0xffu);
+                        o[j][2] = (int)(signed char)((w >> 16) & 0xffu);
+                        o[j][3] = (int)w >> 24;
+                    }
+                    if (q.has_pre) {
+                        v4i xa, xb, xc, xd, xe;
+                        lds_read128_nowait<11 * BN * 4>(xa, trow);
+                        lds_read128_nowait<12 * BN * 4>(xb, trow);
+                        lds_read128_nowait<13 * BN * 4>(xc, trow);
+                        lds_read128_nowait<14 * BN * 4>(xd, trow);
+                        lds_read128_nowait<15 * BN * 4>(xe, trow);
+                        wait_lgkm<0>();
+                        tie(xa); tie(xb); tie(xc); tie(xd); tie(xe);
+                        if (q.pre_clamp) {
+#pragma unroll
+                            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                                for (int t = 0; t < 4; ++t)
+                                    o[j][t] = med3_i32(o[j][t], xa[t], xb[t]);
+                        }
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                o[j][t] = med3_i32((__mul24(o[j][t], xc[t]) + xd[t]) >> xe[t], plo, phi);
+                    }
+                    v4i sa, sb, sc, sd, se;
+                    lds_read128_nowait<6 * BN * 4>(sa, trow);
+                    lds_read128_nowait<7 * BN * 4>(sb, trow);
+                    lds_read128_nowait<8 * BN * 4>(sc, trow);
+                    lds_read128_nowait<9 * BN * 4>(sd, trow);
+                    lds_read128_nowait<10 * BN * 4>(se, trow);
+                    wait_lgkm<0>();
+                    tie(sa); tie(sb); tie(sc); tie(sd); tie(se);
 #pragma unroll
                     for (int j = 0; j < NJ; ++j)
 #pragma unroll
                         for (int t = 0; t < 4; ++t)
-                            acc[i][j][4 * g + t] = med3_i32(acc[i][j][4 * g + t], ta[t], tb[t]);
+                            r[j][t] += o[j][t];
+                    if (q.sum_clamp) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                r[j][t] = med3_i32(r[j][t], sa[t], sb[t]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)
+                            r[j][t] = med3_i32((__mul24(r[j][t], sc[t]) + sd[t]) >> se[t], slo, shi);
                 }
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
-                    int r[4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const int v = acc[i][j][4 * g + t];
-                        if (EPI == EPI_I24) {
-                            // (v * c + half) >> e, saturated
-                            r[t] = med3_i32((__mul24(v, tc[t]) + td[t]) >> te[t], vlo, vhi);
-                        } else if (EPI == EPI_F32) {
-                            float f = (float)v;
-                            if (q.preclamp) f = fminf(fmaxf(f, as_f32(ta[t])), as_f32(tb[t]));
-                            f = round_half_away(f * as_f32(tc[t]));
-                            r[t] = (int)med3_f32(f, flo, fhi);
-                        } else {
-                            r[t] = epi_apply<EPI>(v, ta[t], tb[t], tc[t], td[t], te[t], p.epi.lo, p.epi.hi, p.epi.relu);
-                        }
-                    }
                     if (out_bytes) {
-                        pk[i][j][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ p.out_xor;
+                        pk[i][j][g] = pack_bytes(r[j][0], r[j][1], r[j][2], r[j][3]) ^ p.out_xor;
                     } else {
                         const int m = m0 + wm * TM + j * 32 + l32;
                         const int ch = n0 + wn * TN + i * 32 + 8 * g + 4 * lh;
                         if (m < p.M && ch < p.out_cs)
-                            *(int4*)((int*)p.out + (long long)m * p.out_cs + ch) = int4{r[0], r[1], r[2], r[3]};
+                            *(int4*)((int*)p.out + (long long)m * p.out_cs + ch) = int4{r[j][0], r[j][1], r[j][2], r[j][3]};
                     }
                 }
             }
@@ -376,7 +491,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     {
         int* tabw = (int*)(smem + TAB_OFF);
         for (int i = tid; i < BN; i += NT) {
-            tabw[i] = p.bias[n0 + i];
+            tabw[i] = BIAS_REG ? p.bias[n0 + i] : 0;
             if (EPI != EPI_RAW) {
                 tabw[BN + i] = p.epi.a[n0 + i];
                 tabw[2 * BN + i] = p.epi.b[n0 + i];
@@ -384,14 +499,29 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 tabw[4 * BN + i] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
                 tabw[5 * BN + i] = (EPI != EPI_F32) ? p.epi.e[n0 + i] : 0;
             }
+            if (RES) {
+                tabw[6 * BN + i] = q.sum.a[n0 + i];
+                tabw[7 * BN + i] = q.sum.b[n0 + i];
+                tabw[8 * BN + i] = q.sum.c[n0 + i];
+                tabw[9 * BN + i] = q.sum.d[n0 + i];
+                tabw[10 * BN + i] = q.sum.e[n0 + i];
+                if (q.has_pre) {
+                    tabw[11 * BN + i] = q.pre.a[n0 + i];
+                    tabw[12 * BN + i] = q.pre.b[n0 + i];
+                    tabw[13 * BN + i] = q.pre.c[n0 + i];
+                    tabw[14 * BN + i] = q.pre.d[n0 + i];
+                    tabw[15 * BN + i] = q.pre.e[n0 + i];
+                }
+            }
         }
     }
     __syncthreads();
 
-    // ---- the bias of this lane's channels (rows 8g + 4*lh + t of each 32-channel tile): C operand of a tile's first MFMAs
-    v16i biasv[NI];
+    // ---- the bias of this lane's channels (rows 8g + 4*lh + t of each 32-channel tile): C operand of a tile's first
+    // MFMAs.  The integer rescale has it folded into its tables instead and starts from zero.
+    v16i biasv[BIAS_REG ? NI : 1];
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
+    for (int i = 0; i < (BIAS_REG ? NI : 0); ++i) {
         v4i b0, b1, b2, b3;
         const unsigned t = tab + (unsigned)i * 128u;
         lds_read128_nowait<0>(b0, t); lds_read128_nowait<32>(b1, t); lds_read128_nowait<64>(b2, t); lds_read128_nowait<96>(b3, t);
@@ -434,7 +564,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                         for (int i = 0; i < NI; ++i)
 #pragma unroll
                             for (int j = 0; j < NJ; ++j)
-                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[set][i], fp[set][j], biasv[i], 0, 0, 0);
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[set][i], fp[set][j], BIAS_REG ? biasv[BIAS_REG ? i : 0] : v16i{}, 0, 0, 0);
                     } else {
 #pragma unroll
                         for (int i = 0; i < NI; ++i)

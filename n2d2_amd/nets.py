@@ -366,6 +366,10 @@ class GpuNet:
             for i in l.inputs:
                 consumers.setdefault(i, []).append(l)
         self.folded = set()
+        self.fused_sums = {}
+        by_name = {l.name: l for l in spec.layers}
+        order = {l.name: k for k, l in enumerate(spec.layers)}
+        order["input"] = -1
         C, H, W = spec.in_shape
         self.input = rt.DTensor(batch, C, H, W, capi.U8B if spec.input_unsigned else capi.I8)
         self.tensors = {"input": self.input}
@@ -402,7 +406,26 @@ class GpuNet:
                             if cell.fold_input_scaling(k, sc_cell):
                                 self.folded.add(name)
                                 ins[k] = self.tensors[prod.inputs[0]]
-                self.steps.append((l, cell, (lambda c, i, o: c.forward(i, o))))
+                step = (l, cell, (lambda c, i, o: c.forward(i, o)))
+                if fuse and len(ins) == 2:
+                    # the convolution that runs last among the inputs takes the sum into its epilogue
+                    for k in (1, 0):
+                        prod = by_name.get(l.inputs[k])
+                        other = l.inputs[1 - k]
+                        if (prod is None or prod.type != "conv" or prod.groups != 1 or len(consumers[prod.name]) != 1
+                                or prod.name in self.folded or other in self.folded and by_name[other].type != "scaling"):
+                            continue
+                        other_src = by_name[other].inputs[0] if other in self.folded else other
+                        if order[other_src] > order[prod.name]:
+                            continue
+                        conv_cell = next(c for (m, c, f) in self.steps if m is prod)
+                        if conv_cell.fuse_sum(cell, k, ins[1 - k].dtype):
+                            self.folded.add(prod.name)
+                            self.fused_sums[l.name] = (cell, prod)  # keeps the sum cell alive
+                            ins = [ins_of[prod.name][0], ins[1 - k]]
+                            step = (l, conv_cell, (lambda c, i, o: c.forward_sum(i[0], i[1], o)))
+                            break
+                self.steps.append(step)
             else:
                 raise ValueError(l.type)
             self.tensors[l.name] = out
@@ -447,9 +470,13 @@ class GpuNet:
         total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
         if l.type in ("conv", "fc"):
             total += l.w.size // (2 if l.weight_bits == 4 else 1)
+        if l.name in self.fused_sums:
+            total += self.fused_sums[l.name][1].w.size
         return total
 
     def layer_macs(self, l):
+        if l.name in self.fused_sums:
+            return self.layer_macs(self.fused_sums[l.name][1])
         if l.type == "conv":
             return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
         if l.type == "fc":
@@ -464,4 +491,6 @@ class GpuNet:
             total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
             if l.type in ("conv", "fc"):
                 total += l.w.size // (2 if l.weight_bits == 4 else 1)
+            if l.name in self.fused_sums:
+                total += self.fused_sums[l.name][1].w.size
         return total

@@ -150,6 +150,19 @@ class Conv:
         check(lib.n2d2hip_conv_forward(self.handle, x.ref, out.ref, stream_ptr()))
         return out
 
+    def fuse_sum(self, ew, conv_input_index, other_dtype):
+        """Folds the ElemWise sum fed by this convolution into its epilogue; False when the library keeps them apart."""
+        rc = lib.n2d2hip_conv_fuse_sum(self.handle, ew.handle if ew is not None else None, conv_input_index, other_dtype)
+        if rc == capi.ERR_UNSUPPORTED:
+            return False
+        check(rc)
+        self._sum = ew
+        return True
+
+    def forward_sum(self, x, other, out):
+        check(lib.n2d2hip_conv_forward_sum(self.handle, x.ref, other.ref, out.ref, stream_ptr()))
+        return out
+
     def __del__(self):
         if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_conv_destroy(self.handle)

@@ -352,3 +352,75 @@ def test_elemwise_with_folded_scaling_cell(rt):
     assert ew.fold_input_scaling(0, fl) is False
     ew = rt.ElemWiseSum(2, Cc, rt.Act(Cc, **sum_spec.kwargs()), np.array([2.0, 1.0], np.float32), np.zeros(2, np.float32), "PerInput")
     assert ew.fold_input_scaling(0, sc) is False
+
+
+def test_conv_with_folded_residual_sum(rt):
+    """1x1 convolution + ElemWise sum (+ ScalingCell on the shortcut) in one launch equals the reference cells run in turn."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(77)
+    cases = [  # C, O, H, stride, B
+        (64, 256, 9, 1, 3), (256, 128, 7, 1, 2), (128, 512, 8, 2, 2), (64, 64, 5, 1, 2), (256, 64, 6, 1, 3), (512, 1024, 7, 2, 5)]
+    for C, O, H, stride, B in cases:
+        x = rng.integers(0, 256, size=(B, C, H, H))
+        w = np.clip(np.rint(rng.normal(0, 20, size=(O, C, 1, 1))), -127, 127).astype(np.int64)
+        bias = rng.integers(-2000, 2000, size=O)
+        conv_spec = ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1),
+                            nb_bits=8, unsigned_out=False)
+        sum_spec = ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(0, 3, size=O)], 1),
+                           nb_bits=8, unsigned_out=True)
+        y = cells_ref.conv_cell(x, w, bias, conv_spec, stride=(stride, stride))
+        OH = y.shape[2]
+        dx = rt.DTensor.from_numpy(x, capi.U8B)
+        for other_dtype, other in ((capi.U8B, rng.integers(0, 256, size=(B, O, OH, OH))), (capi.I8, rng.integers(-128, 128, size=(B, O, OH, OH)))):
+            dother = rt.DTensor.from_numpy(other, other_dtype)
+            for pre_mode in (None, "FixedMult16", "SingleShift"):
+                if pre_mode == "FixedMult16":
+                    pre_spec = ActSpec("Linear", "FixedMult16", rng.integers(2 ** 12, 2 ** 15, size=O), frac_bits=14, nb_bits=8,
+                                       unsigned_out=other_dtype == capi.U8B)
+                elif pre_mode == "SingleShift":
+                    pre_spec = ActSpec("Linear", "SingleShift", rng.integers(0, 3, size=O), nb_bits=8, unsigned_out=other_dtype == capi.U8B)
+                else:
+                    pre_spec = None
+                o2 = other.astype(np.float32) if pre_spec is None else pre_spec.apply(other.astype(np.float32))
+                for k in (0, 1):
+                    ins = [y, o2] if k == 0 else [o2, y]
+                    want = cells_ref.elemwise_cell(ins, sum_spec).astype(np.int64)
+                    conv = rt.Conv(w, bias, rt.Act(O, **conv_spec.kwargs()), capi.U8B, stride=(stride, stride))
+                    ew = rt.ElemWiseSum(2, O, rt.Act(O, **sum_spec.kwargs()))
+                    pre = None
+                    if pre_spec is not None:
+                        pre = rt.Act(O, **pre_spec.kwargs())
+                        assert ew.fold_input_scaling(1 - k, pre)
+                    assert conv.fuse_sum(ew, k, other_dtype), (C, O)
+                    out = rt.DTensor(B, O, OH, OH, capi.U8B)
+                    conv.forward_sum(dx, dother, out)
+                    got = out.to_numpy()
+                    assert np.array_equal(got, want), (C, O, H, stride, other_dtype, pre_mode, k, np.count_nonzero(got != want))
+                    # the plain convolution is still available on the same handle
+                    assert np.array_equal(conv.forward(dx).to_numpy(), y.astype(np.int64))
+    # what cannot be folded is reported, and the cells then run separately
+    w3 = np.clip(np.rint(rng.normal(0, 20, size=(64, 64, 3, 3))), -127, 127).astype(np.int64)
+    conv3 = rt.Conv(w3, None, rt.Act(64, **conv_spec_for(64, rng).kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    ew = rt.ElemWiseSum(2, 64, rt.Act(64, **sum_spec_for(64, rng).kwargs()))
+    assert conv3.fuse_sum(ew, 0, capi.U8B) is False
+    wc = np.clip(np.rint(rng.normal(0, 20, size=(64, 48, 1, 1))), -127, 127).astype(np.int64)
+    conv48 = rt.Conv(wc, None, rt.Act(64, **conv_spec_for(64, rng).kwargs()), capi.U8B)
+    assert conv48.fuse_sum(ew, 0, capi.U8B) is False
+    w1 = np.clip(np.rint(rng.normal(0, 20, size=(64, 64, 1, 1))), -127, 127).astype(np.int64)
+    conv1 = rt.Conv(w1, None, rt.Act(64, **conv_spec_for(64, rng).kwargs()), capi.U8B)
+    ewf = rt.ElemWiseSum(2, 64, rt.Act(64, "Linear", "FloatMult", np.full(64, 0.5, np.float32), nb_bits=8, unsigned_out=True))
+    assert conv1.fuse_sum(ewf, 0, capi.U8B) is False
+    with pytest.raises(capi.N2D2HipError):
+        conv1.forward_sum(rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B))
+
+
+def conv_spec_for(O, rng):
+    from oracle.cells import ActSpec
+    return ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=False)
+
+
+def sum_spec_for(O, rng):
+    from oracle.cells import ActSpec
+    return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(0, 3, size=O)], 1), nb_bits=8, unsigned_out=True)

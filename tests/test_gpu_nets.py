@@ -46,7 +46,9 @@ def test_resnet50_config(variant):
             "conv5.3_sum", "pool", "fc"]
     print("resnet50", variant, flush=True)
     net = _run_both(spec, x, keep)
-    assert "conv2.2_shortcut_rescale" in net.folded and len(net.folded) == 12
+    # 12 shortcut ScalingCells folded into their sums, 16 sums folded into the convolution that feeds them
+    assert "conv2.2_shortcut_rescale" in net.folded and "conv2.1_1x1_proj" in net.folded and "conv2.2_1x1_x4" in net.folded
+    assert len(net.folded) == 28 and len(net.launched) == len(spec.layers) - 28
     if variant == "pad1":
         unfused = _run_both(spec, x, keep, fuse=False)
         assert not unfused.folded
