@@ -41,6 +41,7 @@ struct ConvArgs {
     void* out;
     int out_cs, out_dtype;
     int strideX, strideY, padL, padT, dilX, dilY;
+    int kW, kH;
     int ntiles_n, nblocks;
     unsigned fill;          // padding byte replicated 4x (logical zero of the input)
     unsigned out_xor;       // 0x80808080 when the output is stored as value-128
@@ -103,6 +104,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     // ---- per-thread pixel rows
     const signed char* rowptr[P_LOADS];
     int base_y[P_LOADS], base_x[P_LOADS];
+    bool compact[P_LOADS];        // the reference's hand-unrolled 3x3 window: first 3x3 taps at undilated offsets
+    const bool dilated = p.dilX != 1 || p.dilY != 1;
+    const int dil_kw = p.kW + (p.dilX - 1) * (p.kW - 1), dil_kh = p.kH + (p.dilY - 1) * (p.kH - 1);
     const int ohw = p.OH * p.OW;
 #pragma unroll
     for (int i = 0; i < P_LOADS; ++i) {
@@ -115,7 +119,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             base_y[i] = oy * p.strideY - p.padT;
             base_x[i] = ox * p.strideX - p.padL;
             rowptr[i] = p.in + (((long long)b * p.H + base_y[i]) * p.W + base_x[i]) * (long long)p.in_cs;
+            // The reference recognises "a 3x3 window fully inside" by its tap bounds alone and unrolls it without the
+            // dilation (ref: src/Cell/ConvCell_Frame_Kernels.cpp:95-117); a dilated kernel can meet those bounds.
+            compact[i] = dilated && base_x[i] >= 0 && base_y[i] >= 0 && min(max(p.W - base_x[i], 0), dil_kw) == 3
+                && min(max(p.H - base_y[i], 0), dil_kh) == 3;
         } else {
+            compact[i] = false;
             base_y[i] = -(1 << 28);     // every tap test fails: the row is all padding
             base_x[i] = -(1 << 28);
             rowptr[i] = p.in;
@@ -137,22 +146,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             // Tap validity exactly as the reference computes its window
             // (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83): tap index >= max(pad - o*stride, 0)
             // and dilated offset inside the input.
-            const bool yok = s.w && s.x >= -base_y[i] && base_y[i] + dy < p.H;
+            const bool cmp = compact[i];
+            const int dyy = cmp ? s.x : dy;
+            const bool yok = s.w && (cmp ? s.x < 3 : (s.x >= -base_y[i] && base_y[i] + dy < p.H));
             if (PIX4) {
-                const int* src = (const int*)(rowptr[i] + ((long long)dy * p.W + s.y) * 4);
+                const int* src = (const int*)(rowptr[i] + ((long long)dyy * p.W + s.y) * 4);
                 v4i v;
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
                     const int kx = s.y + t;
-                    const bool ok = yok && kx >= -base_x[i] && base_x[i] + kx < p.W;
+                    const bool ok = yok && (cmp ? kx < 3 : (kx >= -base_x[i] && base_x[i] + kx < p.W));
                     v[t] = ok ? src[t] : (int)p.fill;
                 }
                 preg[i] = v;
             } else {
-                const int dx = s.y * p.dilX;
-                const bool ok = yok && s.y >= -base_x[i] && base_x[i] + dx < p.W;
+                const int dx = cmp ? s.y : s.y * p.dilX;
+                const bool ok = yok && (cmp ? s.y < 3 : (s.y >= -base_x[i] && base_x[i] + dx < p.W));
                 if (ok) {
-                    preg[i] = *(const v4i*)(rowptr[i] + ((long long)dy * p.W + dx) * p.in_cs + s.z);
+                    preg[i] = *(const v4i*)(rowptr[i] + ((long long)dyy * p.W + dx) * p.in_cs + s.z);
                 } else {
                     const int f = (int)p.fill;
                     preg[i] = v4i{f, f, f, f};
@@ -310,12 +321,15 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const signed char* __res
         const int b = (int)(r / OH);
         const int by = oy * strideY - padT, bx = ox * strideX - padL;
         int a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+        // the reference's hand-unrolled 3x3 window ignores the dilation (ref: src/Cell/ConvCell_Frame_Kernels.cpp:95-117)
+        const bool cmp = (dilX != 1 || dilY != 1) && bx >= 0 && by >= 0
+            && min(max(W - bx, 0), kW + (dilX - 1) * (kW - 1)) == 3 && min(max(H - by, 0), kH + (dilY - 1) * (kH - 1)) == 3;
         for (int ky = 0; ky < kH; ++ky) {
-            const int iy = by + ky * dilY;
-            if (ky < -by || iy >= H) continue;
+            const int iy = by + (cmp ? ky : ky * dilY);
+            if (cmp ? ky >= 3 : (ky < -by || iy >= H)) continue;
             for (int kx = 0; kx < kW; ++kx) {
-                const int ix = bx + kx * dilX;
-                if (kx < -bx || ix >= W) continue;
+                const int ix = bx + (cmp ? kx : kx * dilX);
+                if (cmp ? kx >= 3 : (kx < -bx || ix >= W)) continue;
                 const int xv = *(const int*)(in + (((long long)b * H + iy) * W + ix) * cs + c4);
                 const int wv = *(const int*)(w + (long long)(ky * kW + kx) * cs + c4);
                 a0 += ((int)(signed char)(xv) + in_zp) * (int)(signed char)(wv);
@@ -656,7 +670,7 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
     const int opad_n = round_up(d.O, 64);
     *bn128 = opad_n % 128 == 0 || opad_n > 256;
     const int k = c->act->args.kind;
-    return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 32
+    return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 31
         && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
 }
 
@@ -723,6 +737,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     a.w = c->d_w; a.ktot = c->ktot; a.niter = c->ktot / 64; a.sub = c->d_sub; a.bias = c->d_bias;
     a.out = out->data; a.out_cs = out->cs; a.out_dtype = out->dtype;
     a.strideX = d.strideX; a.strideY = d.strideY; a.padL = d.padL; a.padT = d.padT; a.dilX = d.dilX; a.dilY = d.dilY;
+    a.kW = d.kW; a.kH = d.kH;
     a.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
     a.out_xor = out_xor;
     a.epi = c->act->args;
@@ -763,7 +778,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         const bool all_valid = d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0;
         // Two independent 4-wave blocks per CU, 128 pixels x 128 (or 64) channels each: one block's epilogue and
         // barrier waits overlap the other's MFMAs.  K advances by whole 128-byte lines when the channel count allows.
-        const int BMp = 128;
+        // Layers with few pixels (deep stages) take 64-pixel tiles so that every CU still gets its two blocks.
+        const long long tiles128 = ((Mll + 127) / 128) * a.ntiles_n;
+        const char* bm_env = getenv("N2D2HIP_BM64");
+        const bool small_m = bn128 && d.C % 128 == 0 && (bm_env ? atoi(bm_env) != 0 : tiles128 < (3 * num_cus()) / 2);
+        const int BMp = small_m ? 64 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
         q.mlanes = 8 * per_xcd;
@@ -784,13 +803,17 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
                 q.pre.a = c->d_res_tab + 5 * cp; q.pre.b = c->d_res_tab + 6 * cp; q.pre.c = c->d_res_tab + 7 * cp;
                 q.pre.d = c->d_res_tab + 8 * cp; q.pre.e = c->d_res_tab + 9 * cp;
             }
-            if (d.C % 128 == 0) {
+            if (small_m) {
+                launch_pipe_res<4, 128, 2, 1, 2, 3>(q, grid, stream);
+            } else if (d.C % 128 == 0) {
                 if (bn128) launch_pipe_res<4, 128, 2, 2, 2, 2>(q, grid, stream);
                 else launch_pipe_res<4, 128, 2, 1, 4, 3>(q, grid, stream);
             } else {
                 if (bn128) launch_pipe_res<4, 64, 2, 2, 2, 4>(q, grid, stream);
                 else launch_pipe_res<4, 64, 2, 1, 4, 4>(q, grid, stream);
             }
+        } else if (small_m) {
+            launch_pipe<4, 128, 2, 1, 2, 3>(q, all_valid, grid, stream);
         } else if (d.C % 128 == 0) {
             if (bn128) launch_pipe<4, 128, 2, 2, 2, 2>(q, all_valid, grid, stream);
             else launch_pipe<4, 128, 2, 1, 4, 3>(q, all_valid, grid, stream);

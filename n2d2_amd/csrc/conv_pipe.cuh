@@ -172,9 +172,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     for (int j = 0; j < B_J; ++j)
         woff[j] = (unsigned)((n0 + ((wave + NW * j) % B_CH) * RPC + lrow) * p.ktot + lq * 16);
     int rowoff[A_J];               // byte offset of the window origin of this thread's pixel rows (+ sub-chunk)
-    unsigned rowmask[A_J];         // bit t: kernel tap t of the row reads inside the input
+    unsigned rowmask[A_J];         // bit t < 31: kernel tap t of the row reads inside the input; bit 31: undilated window
     int l_tile = 0, l_it = 0, l_koff = 0, l_stage = 0;
-    int l_c = 0, l_kx = 0, l_ky = 0, l_tap = 0, l_tapoff = 0;
+    int l_c = 0, l_kx = 0, l_ky = 0, l_tap = 0, l_tapoff = 0, l_ctapoff = 0;
+    const bool dilated = p.dilX != 1 || p.dilY != 1;
+    const int dil_kw = q.kW + (p.dilX - 1) * (q.kW - 1), dil_kh = q.kH + (p.dilY - 1) * (q.kH - 1);
     auto loader_new_tile = [&]() {
         const int m0 = (mlane + l_tile * q.mlanes) * BM;
 #pragma unroll
@@ -200,6 +202,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 unsigned mk = 0u;
                 for (int ky = 0; ky < q.kH; ++ky)
                     mk |= ((ky >= -by) & (ky * p.dilY < p.H - by)) ? (xmask << (ky * q.kW)) : 0u;
+                // The reference unrolls "a 3x3 window fully inside" by hand, recognising it by its tap bounds alone
+                // (ref: src/Cell/ConvCell_Frame_Kernels.cpp:95-117): a dilated kernel whose bounds happen to be
+                // [0,3) x [0,3) is evaluated there with its first 3x3 taps at undilated offsets.
+                const int sx_max = min(max(p.W - bx, 0), dil_kw), sy_max = min(max(p.H - by, 0), dil_kh);
+                if (dilated && bx >= 0 && by >= 0 && sx_max == 3 && sy_max == 3)
+                    mk = 0x80000000u | 7u | (7u << q.kW) | (7u << (2 * q.kW));
                 rowmask[j] = live ? mk : 0u;
             }
         }
@@ -218,7 +226,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
             const unsigned tapbit = 1u << l_tap;
 #pragma unroll
             for (int j = 0; j < A_J; ++j) {
-                const signed char* src = (rowmask[j] & tapbit) ? p.in + (rowoff[j] + l_tapoff) : q.fill16;
+                const int toff = (int)rowmask[j] < 0 ? l_ctapoff : l_tapoff;
+                const signed char* src = (rowmask[j] & tapbit) ? p.in + (rowoff[j] + toff) : q.fill16;
                 __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
             }
         }
@@ -230,16 +239,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         l_koff += BK;
         if (++l_it == niter) {
             l_it = 0; l_koff = 0;
-            l_c = 0; l_kx = 0; l_ky = 0; l_tap = 0; l_tapoff = 0;
+            l_c = 0; l_kx = 0; l_ky = 0; l_tap = 0; l_tapoff = 0; l_ctapoff = 0;
             ++l_tile;
             loader_new_tile();
         } else if (!ALLVALID) {
             l_tapoff += BK;
+            l_ctapoff += BK;
             if (++l_c == q.cper) {
                 l_c = 0;
                 ++l_tap;
                 if (++l_kx == q.kW) { l_kx = 0; ++l_ky; }
                 l_tapoff = (l_ky * p.dilY * p.W + l_kx * p.dilX) * p.in_cs;
+                l_ctapoff = (l_ky * p.W + l_kx) * p.in_cs;
             }
         }
     };

@@ -449,6 +449,33 @@ class GpuNet:
             fn(cell, ins, out)
         return self.tensors[self.spec.output]
 
+    def capture(self):
+        """Records one forward into a HIP graph (every launch of the C ABI goes to the capturing stream and none of
+        them allocates or clears memory) and returns a callable that replays it."""
+        import torch
+        self.forward()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                self.forward()
+        torch.cuda.synchronize()
+        self._graph = graph
+
+        def replay():
+            graph.replay()
+            return self.tensors[self.spec.output]
+        return replay
+
+    def forward_subset(self, indices):
+        """Replays only the launches with these indices into self.launched (their inputs keep the values of the last
+        full forward)."""
+        for k in indices:
+            l, cell, fn = self.steps[k]
+            ins, out = self._io[k]
+            fn(cell, ins, out)
+
     def forward_timed(self):
         """One forward with a pair of events around every cell launch, recorded on the stream the kernels run on.
         Returns [(layer, milliseconds)]."""

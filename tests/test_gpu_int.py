@@ -147,6 +147,17 @@ CONV_CASES = [
     ("dilated_pad_quirk", 2, 16, 12, 12, 16, (3, 3), (1, 3), (2, 2, 2, 2), (3, 3), "u8"),
     ("big_k", 1, 512, 7, 7, 130, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
     ("tall_m", 5, 16, 33, 31, 16, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
+    # channel counts that are multiples of 64 (the pipelined kernel): every window quirk again, both K step widths
+    ("c64_dilated_pad_quirk", 2, 64, 12, 12, 70, (3, 3), (1, 3), (2, 2, 2, 2), (3, 3), "u8"),
+    ("c128_asym", 3, 128, 9, 8, 40, (2, 5), (2, 3), (1, 2, 0, 1), (1, 1), "i8"),
+    ("c64_5x5", 2, 64, 11, 13, 64, (5, 5), (1, 1), (2, 2, 2, 2), (1, 1), "u8"),
+    ("c192_1x7", 2, 192, 9, 15, 130, (7, 1), (1, 1), (3, 0, 3, 0), (1, 1), "u8"),
+    ("c320_dil2", 1, 320, 13, 13, 300, (3, 3), (2, 2), (2, 2, 2, 2), (2, 2), "i8"),
+    ("c256_ragged_m", 7, 256, 5, 7, 128, (3, 3), (1, 1), (1, 1, 1, 1), (1, 1), "u8"),
+    # the reference's hand-unrolled 3x3 window met by a dilated kernel (bounds [0,3) x [0,3) at the last pixel)
+    ("c16_dil2_unrolled_window", 2, 16, 13, 13, 16, (3, 3), (2, 2), (2, 2, 2, 2), (2, 2), "u8"),
+    ("c3_dily2_unrolled_window", 2, 3, 13, 13, 16, (3, 3), (2, 2), (1, 2, 1, 2), (1, 2), "u8"),
+    ("c128_1x1_many_tiles", 6, 128, 23, 21, 256, (1, 1), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
 ]
 
 
@@ -213,6 +224,12 @@ def test_depthwise_conv_bit_exact(rt, stride):
         conv = rt.Conv(w, bias, rt.Act(Cc, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(1, 1, 1, 1), groups=Cc)
         got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
         assert np.array_equal(got, want.astype(np.int64)), an
+    # dilated depthwise whose last pixel meets the reference's hand-unrolled 3x3 window
+    x = _u8((2, Cc, 13, 13))
+    spec = acts["sshift_lin_s"]
+    want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(2, 2, 2, 2), dil=(2, 2), groups=Cc)
+    conv = rt.Conv(w, bias, rt.Act(Cc, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(2, 2, 2, 2), dil=(2, 2), groups=Cc)
+    assert np.array_equal(conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), want.astype(np.int64))
 
 
 def test_conv_int4_weights_uint4_activations(rt):

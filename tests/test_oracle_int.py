@@ -46,6 +46,32 @@ def test_conv_dilation_without_padding(d):
     assert np.array_equal(got.astype(np.int64), rm.conv_int(x, w, dil=d))
 
 
+def test_conv_unrolled_3x3_window_ignores_dilation():
+    """ConvCell_Frame_Kernels.cpp:95-117 unrolls "sxMin == syMin == 0 and sxMax == syMax == 3" by hand, without the
+    dilation.  A dilated kernel meets those bounds where W + pad - ox*stride == 3: there the reference sums the first
+    3x3 taps over the undilated window, everywhere else the dilated taps that fall inside the input."""
+    x = _u8((1, 4, 13, 13))
+    w = _i8((3, 4, 3, 3))
+    got = orc.conv_forward(x, w, stride=(2, 2), pad=(2, 2, 2, 2), dil=(2, 2)).astype(np.int64)
+    xi, wi = x.astype(np.int64), w.astype(np.int64)
+    assert got.shape == (1, 3, 7, 7)
+    for oy in range(7):
+        for ox in range(7):
+            iy0, ix0 = 2 * oy - 2, 2 * ox - 2
+            want = np.zeros(3, dtype=np.int64)
+            if (oy, ox) == (6, 6):          # 13 + 2 - 12 == 3 in both directions
+                for ky in range(3):
+                    for kx in range(3):
+                        want += wi[:, :, ky, kx] @ xi[0, :, iy0 + ky, ix0 + kx]
+            else:
+                for ky in range(3):
+                    for kx in range(3):
+                        iy, ix = iy0 + 2 * ky, ix0 + 2 * kx
+                        if 0 <= iy < 13 and 0 <= ix < 13:
+                            want += wi[:, :, ky, kx] @ xi[0, :, iy, ix]
+            assert np.array_equal(got[0, :, oy, ox], want), (oy, ox)
+
+
 # (kW, kH, subX, subY, strideX, strideY, padX, padY, dilX, dilY): the tuples of
 # tests/Cell/class_ConvCell_Frame.cpp:402-438 (channel sizes reduced).
 REF_GRID = [
