@@ -49,7 +49,8 @@ def test_conv_dilation_without_padding(d):
 def test_conv_unrolled_3x3_window_ignores_dilation():
     """ConvCell_Frame_Kernels.cpp:95-117 unrolls "sxMin == syMin == 0 and sxMax == syMax == 3" by hand, without the
     dilation.  A dilated kernel meets those bounds where W + pad - ox*stride == 3: there the reference sums the first
-    3x3 taps over the undilated window, everywhere else the dilated taps that fall inside the input."""
+    3x3 taps over the undilated window; everywhere else the taps whose INDEX is at least pad - o*stride (lines 72-75,
+    also undilated) and whose dilated position is below the input's far edge."""
     x = _u8((1, 4, 13, 13))
     w = _i8((3, 4, 3, 3))
     got = orc.conv_forward(x, w, stride=(2, 2), pad=(2, 2, 2, 2), dil=(2, 2)).astype(np.int64)
@@ -67,7 +68,7 @@ def test_conv_unrolled_3x3_window_ignores_dilation():
                 for ky in range(3):
                     for kx in range(3):
                         iy, ix = iy0 + 2 * ky, ix0 + 2 * kx
-                        if 0 <= iy < 13 and 0 <= ix < 13:
+                        if ky >= max(2 - 2 * oy, 0) and kx >= max(2 - 2 * ox, 0) and iy < 13 and ix < 13:
                             want += wi[:, :, ky, kx] @ xi[0, :, iy, ix]
             assert np.array_equal(got[0, :, oy, ox], want), (oy, ox)
 
