@@ -298,6 +298,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
 } // namespace n2d2hip
 #include "conv_pipe.cuh"
+#include "conv_stem.cuh"
 namespace n2d2hip {
 
 // ------------------------------------------------------------ depthwise
@@ -378,6 +379,8 @@ struct n2d2hip_conv_s {
     // integer rescale with the bias folded in, for the pipelined kernel: a - bias, b - bias, c, d + bias * c, e, each [cpad]
     int* d_epi_tab;
     bool bias_folded;
+    // first-layer kernel (<= 4 input channels, horizontal stride 2): weights as [channel][kH * 32]
+    signed char* d_wstem;
     bool is_fc;
     int fcH, fcW;
 };
@@ -416,6 +419,16 @@ void launch_pipe(ConvPipeArgs a, bool all_valid, int grid, hipStream_t stream)
     default: N2D2HIP_PIPE(EPI_F32); break;
     }
 #undef N2D2HIP_PIPE
+}
+
+template <int KH>
+void launch_stem(const ConvStemArgs& a, int grid, hipStream_t stream)
+{
+    switch (a.c.epi.kind) {
+    case EPI_RAW: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_RAW>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_F32>), dim3(grid), dim3(256), 0, stream, a); break;
+    }
 }
 
 template <int NW, int BK, int NI, int NJ, int WGM, int S>
@@ -502,7 +515,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->d_wstem = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -628,6 +641,20 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     if (e == hipSuccess) e = hipMemcpy(c->d_w, hw.data(), hw.size(), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMalloc((void**)&c->d_bias, hbias.size() * sizeof(int));
     if (e == hipSuccess) e = hipMemcpy(c->d_bias, hbias.data(), hbias.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e == hipSuccess && c->pix4 && d->weight_bits == 8 && d->strideX == 2 && d->dilX == 1 && d->dilY == 1 && d->kW <= 8
+        && (d->kH == 3 || d->kH == 5 || d->kH == 7)) {
+        // [channel][kernel row][8 tap slots][4 channel slots], zero where the kernel has nothing
+        const int orows = round_up(d->O, 64);
+        std::vector<signed char> ws((size_t)orows * d->kH * 32, 0);
+        for (int o = 0; o < d->O; ++o)
+            for (int ky = 0; ky < d->kH; ++ky)
+                for (int kx = 0; kx < d->kW; ++kx)
+                    for (int ch = 0; ch < d->C; ++ch)
+                        ws[((size_t)o * d->kH + ky) * 32 + kx * 4 + ch] =
+                            (signed char)read_weight(weights, (((long long)o * d->C + ch) * d->kH + ky) * d->kW + kx, 8);
+        e = hipMalloc((void**)&c->d_wstem, ws.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_wstem, ws.data(), ws.size(), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hepi.empty()) {
         e = hipMalloc((void**)&c->d_epi_tab, hepi.size() * sizeof(int));
         if (e == hipSuccess) e = hipMemcpy(c->d_epi_tab, hepi.data(), hepi.size() * sizeof(int), hipMemcpyHostToDevice);
@@ -659,6 +686,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_fill) (void)hipFree(c->d_fill);
     if (c->d_res_tab) (void)hipFree(c->d_res_tab);
     if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
+    if (c->d_wstem) (void)hipFree(c->d_wstem);
     delete c;
     return N2D2HIP_OK;
 }
@@ -782,7 +810,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         const long long tiles128 = ((Mll + 127) / 128) * a.ntiles_n;
         const char* bm_env = getenv("N2D2HIP_BM64");
         const bool small_m = bn128 && d.C % 128 == 0 && (bm_env ? atoi(bm_env) != 0 : tiles128 < (3 * num_cus()) / 2);
-        const int BMp = small_m ? 64 : 128;
+        const char* wide_env = getenv("N2D2HIP_WIDE64");
+        const bool wide64 = !bn128 && !other && wide_env && atoi(wide_env) != 0;      // 256 pixels x 64 channels
+        const int BMp = small_m ? 64 : wide64 ? 256 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
         q.mlanes = 8 * per_xcd;
@@ -812,6 +842,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
                 if (bn128) launch_pipe_res<4, 64, 2, 2, 2, 4>(q, grid, stream);
                 else launch_pipe_res<4, 64, 2, 1, 4, 4>(q, grid, stream);
             }
+        } else if (wide64) {
+            launch_pipe<4, 64, 2, 2, 4, 3>(q, all_valid, grid, stream);
         } else if (small_m) {
             launch_pipe<4, 128, 2, 1, 2, 3>(q, all_valid, grid, stream);
         } else if (d.C % 128 == 0) {
@@ -823,6 +855,34 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         }
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
+    }
+    {
+        const int k = c->act->args.kind;
+        if (c->d_wstem && !other && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32) && fits32
+            && getenv("N2D2HIP_NO_STEM") == nullptr) {
+            ConvStemArgs q;
+            q.c = a;
+            if (k == EPI_I24) {
+                const int cp = c->act->cpad;
+                q.c.epi.a = c->d_epi_tab; q.c.epi.b = c->d_epi_tab + cp; q.c.epi.c = c->d_epi_tab + 2 * cp;
+                q.c.epi.d = c->d_epi_tab + 3 * cp; q.c.epi.e = c->d_epi_tab + 4 * cp;
+            }
+            q.wk = c->d_wstem;
+            q.fill16 = c->d_fill;
+            q.preclamp = c->preclamp ? 1 : 0;
+            q.tiles_per_row = (OW + 127) / 128;
+            q.ntiles = in->B * OH * q.tiles_per_row;
+            q.c.ntiles_n = (round_up(d.O, 16) + 63) / 64;
+            q.nlanes = std::max(1, std::min(q.ntiles, (3 * num_cus()) / q.c.ntiles_n));
+            magic_div((unsigned)OH, &q.oh_mul, &q.oh_sh);
+            magic_div((unsigned)q.tiles_per_row, &q.tpr_mul, &q.tpr_sh);
+            const int grid = q.nlanes * q.c.ntiles_n;
+            if (d.kH == 3) launch_stem<3>(q, grid, stream);
+            else if (d.kH == 5) launch_stem<5>(q, grid, stream);
+            else launch_stem<7>(q, grid, stream);
+            N2D2HIP_HIP_CHECK(hipGetLastError());
+            return N2D2HIP_OK;
+        }
     }
     if (c->pix4) {
         if (bn128) { if (w4) launch_cfg<128, 128, 2, true, true>(a, stream); else launch_cfg<128, 128, 2, true, false>(a, stream); }

@@ -1,0 +1,231 @@
+// First-layer convolution: at most 4 input channels stored as one dword per
+// pixel, horizontal stride 2, no dilation (the 7x7 / 3x3 stride-2 stems).
+//
+// Such a layer has almost no arithmetic per byte it writes (K = 7*7*3 against
+// 64 output channels), so the kernel is built around moving data once:
+//  * a tile is 128 consecutive output pixels of one output row; the KH input
+//    rows it needs (2*128 + 6 pixels each) are copied global -> LDS by 4-byte
+//    direct loads, one pixel per lane, so that padding is decided per pixel
+//    (a lane outside the image fetches the input's zero instead) and every
+//    window of the tile is then read from LDS;
+//  * one MFMA K step is one kernel row: 8 taps x 4 channel slots = 32; the tap
+//    past the kernel's width and the channel slots past C meet zero weights.
+//    A lane's 16-byte pixel operand is 4 consecutive pixels of the row, at
+//    8 bytes * pixel + 16 bytes * lane half: two ds_read_b64;
+//  * the weights (64 channels x KH x 32 bytes) stay in registers for the
+//    block's whole life;
+//  * three LDS stages: the rows of the next two tiles are in flight while this
+//    one is multiplied and rescaled; one barrier per tile.  Two tiles ahead,
+//    not one, because the wait is a count of outstanding operations and the
+//    epilogue's stores count too: with NLOAD younger loads allowed, the wait
+//    is over when this tile's rows have landed (loads return in order) without
+//    having to see the previous tile's stores acknowledged;
+//  * the epilogue is the pipelined kernel's: rescale, pack to bytes, exchange
+//    between lane halves until a lane owns 32 consecutive channels, store.
+#pragma once
+
+namespace n2d2hip {
+
+struct ConvStemArgs {
+    ConvArgs c;
+    const signed char* wk;       // [channel][KH * 32]: kernel row, tap (8 slots), channel (4 slots)
+    const signed char* fill16;   // the input's logical zero
+    int ntiles;                  // pixel tiles: B * OH * tiles_per_row
+    int tiles_per_row;
+    int nlanes;                  // blocks that share the pixel tiles of one channel tile
+    unsigned oh_mul, oh_sh;      // division by OH
+    unsigned tpr_mul, tpr_sh;    // division by tiles_per_row
+    int preclamp;
+};
+
+template <int KH, int EPI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) void conv_stem_kernel(ConvStemArgs q)
+{
+    const ConvArgs& p = q.c;
+    constexpr int TW = 128;                    // output pixels per tile
+    constexpr int PITCH = 1280;                // bytes per patch row in LDS: 5 loads of 64 pixels
+    constexpr int NCHUNK = KH * 5;             // 256-byte chunks per stage
+    constexpr int NLOAD = (NCHUNK + 3) / 4;    // per wave (chunks past the end land in the spare row)
+    constexpr int STAGE = (KH + 1) * PITCH;
+    constexpr int BN = 64;
+    constexpr int TAB_OFF = 3 * STAGE;
+    constexpr bool BIAS_ADD = EPI != EPI_I24;  // the integer rescale carries the bias in its tables
+    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + 6 * BN * 4];
+    const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int tile_n = blockIdx.x % p.ntiles_n;
+    const int blane = blockIdx.x / p.ntiles_n;
+    const int n0 = tile_n * BN;
+    const int ntile = (blane < q.ntiles) ? (q.ntiles - blane + q.nlanes - 1) / q.nlanes : 0;
+
+    // ---- loader: chunk c = wave + 4*j is 64 pixels (part c%5) of patch row c/5
+    auto issue = [&](int t, int stage) {
+        const int id = blane + t * q.nlanes;
+        const bool live = t < ntile;
+        const int rowid = div_magic(live ? id : 0, q.tpr_mul, q.tpr_sh);          // b * OH + oy
+        const int txi = (live ? id : 0) - rowid * q.tiles_per_row;
+        const int b = div_magic(rowid, q.oh_mul, q.oh_sh);
+        const int oy = rowid - b * p.OH;
+        const int x0 = txi * TW * p.strideX - p.padL, y0 = oy * p.strideY - p.padT;
+        unsigned char* sbase = smem + stage * STAGE;
+        const signed char* img = p.in + (long long)b * p.H * p.W * 4;
+#pragma unroll
+        for (int j = 0; j < NLOAD; ++j) {
+            const int c = wave + 4 * j;
+            const int r = c / 5, part = c - r * 5;
+            const int iy = y0 + r;
+            // everything about the row is block-uniform; a row outside the image sends every lane to the zero
+            const bool row_ok = live & (c < NCHUNK) & ((unsigned)iy < (unsigned)p.H);
+            const signed char* rowp = img + (long long)(row_ok ? iy : 0) * p.W * 4;
+            const int ix = (row_ok ? x0 + part * 64 : -(1 << 20)) + lane;
+            const signed char* src = (unsigned)ix < (unsigned)p.W ? rowp + (unsigned)ix * 4u : q.fill16;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + r * PITCH + part * 256), 4, 0, 0);
+        }
+    };
+    issue(0, 0);
+    issue(1, 1);
+
+    // ---- weights of this lane's channels: A operand of kernel row ky is 16 bytes at ky*32 + 16*lh
+    v4i wf[2][KH];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky)
+            wf[i][ky] = *(const v4i*)(q.wk + (long long)(n0 + i * 32 + l32) * (KH * 32) + ky * 32 + 16 * lh);
+
+    // ---- rescale tables of the channel tile
+    {
+        int* tabw = (int*)(smem + TAB_OFF);
+        for (int i = tid; i < BN; i += 256) {
+            tabw[i] = BIAS_ADD ? p.bias[n0 + i] : 0;
+            if (EPI != EPI_RAW) {
+                tabw[BN + i] = p.epi.a[n0 + i];
+                tabw[2 * BN + i] = p.epi.b[n0 + i];
+                tabw[3 * BN + i] = p.epi.c[n0 + i];
+                tabw[4 * BN + i] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
+                tabw[5 * BN + i] = (EPI != EPI_F32) ? p.epi.e[n0 + i] : 0;
+            }
+        }
+    }
+    __syncthreads();
+    const unsigned tab = lds0 + TAB_OFF + (unsigned)(4 * lh) * 4u;
+    const bool out_bytes = p.out_dtype != N2D2HIP_I32;
+    const int vlo = p.epi.lo, vhi = p.epi.hi;
+    const float flo = (float)p.epi.lo, fhi = (float)p.epi.hi;
+    // this lane's window origin inside a patch row: pixel 2 * (32*wave + l32), tap slot 4*lh
+    const unsigned frag = lds0 + (unsigned)((p.strideX * (32 * wave + l32) + 4 * lh) * 4);
+
+    for (int t = 0; t < ntile; ++t) {
+        const int stage = t % 3;
+        // this tile's rows have landed for every wave, and every wave is done with the stage of the previous tile
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(NLOAD) : "memory");
+        issue(t + 2, (t + 2) % 3);
+
+        v16i acc[2];
+        {
+            typedef int v2i __attribute__((ext_vector_type(2)));
+            v2i lo[KH], hi[KH];
+            const unsigned fa = frag + (unsigned)(stage * STAGE);
+#pragma unroll
+            for (int ky = 0; ky < KH; ++ky)
+                asm volatile("ds_read_b64 %0, %2 offset:%3\n\tds_read_b64 %1, %2 offset:%4"
+                             : "=&v"(lo[ky]), "=&v"(hi[ky]) : "v"(fa), "n"(ky * PITCH), "n"(ky * PITCH + 8) : "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int ky = 0; ky < KH; ++ky) {
+                asm volatile("" : "+v"(lo[ky]), "+v"(hi[ky]));
+                const v4i pf = {lo[ky][0], lo[ky][1], hi[ky][0], hi[ky][1]};
+                if (ky == 0) {
+                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][ky], pf, v16i{}, 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][ky], pf, v16i{}, 0, 0, 0);
+                } else {
+                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][ky], pf, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][ky], pf, acc[1], 0, 0, 0);
+                }
+            }
+        }
+
+        // ---- epilogue: this lane holds channels 8g + 4*lh .. +3 of both 32-channel tiles for output pixel ox
+        const int id = blane + t * q.nlanes;
+        const int rowid = div_magic(id, q.tpr_mul, q.tpr_sh);
+        const int ox = (id - rowid * q.tiles_per_row) * TW + 32 * wave + l32;
+        const long long m = (long long)rowid * p.OW + ox;
+        const bool pix_ok = ox < p.OW;
+        unsigned pk[2][4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
+                v4i tbias = {0, 0, 0, 0}, ta = tbias, tb = tbias, tc = tbias, td = tbias, te = tbias;
+                if (BIAS_ADD) lds_read128_nowait<0>(tbias, trow);
+                if (EPI != EPI_RAW) {
+                    lds_read128_nowait<BN * 4>(ta, trow);
+                    lds_read128_nowait<2 * BN * 4>(tb, trow);
+                    lds_read128_nowait<3 * BN * 4>(tc, trow);
+                    if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(td, trow);
+                    if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(te, trow);
+                }
+                wait_lgkm<0>();
+                tie(tbias); tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                int r[4];
+                if (EPI == EPI_I24 && q.preclamp) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        acc[i][4 * g + e] = med3_i32(acc[i][4 * g + e], ta[e], tb[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    int v = acc[i][4 * g + e];
+                    if (BIAS_ADD) v += tbias[e];
+                    if (EPI == EPI_I24) {
+                        r[e] = med3_i32((__mul24(v, tc[e]) + td[e]) >> te[e], vlo, vhi);
+                    } else if (EPI == EPI_F32) {
+                        float f = (float)v;
+                        if (q.preclamp) f = fminf(fmaxf(f, as_f32(ta[e])), as_f32(tb[e]));
+                        f = round_half_away(f * as_f32(tc[e]));
+                        r[e] = (int)med3_f32(f, flo, fhi);
+                    } else {
+                        r[e] = epi_apply<EPI>(v, ta[e], tb[e], tc[e], td[e], te[e], p.epi.lo, p.epi.hi, p.epi.relu);
+                    }
+                }
+                if (out_bytes) {
+                    pk[i][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ p.out_xor;
+                } else {
+                    const int ch = n0 + i * 32 + 8 * g + 4 * lh;
+                    if (pix_ok && ch < p.out_cs)
+                        *(int4*)((int*)p.out + m * p.out_cs + ch) = int4{r[0], r[1], r[2], r[3]};
+                }
+            }
+        }
+        if (out_bytes) {
+            unsigned qd[2][4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const auto s02 = __builtin_amdgcn_permlane32_swap(pk[i][0], pk[i][2], false, false);
+                const auto s13 = __builtin_amdgcn_permlane32_swap(pk[i][1], pk[i][3], false, false);
+                qd[i][0] = s02[0]; qd[i][1] = s02[1]; qd[i][2] = s13[0]; qd[i][3] = s13[1];
+            }
+            v4i first, second;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const auto x = __builtin_amdgcn_permlane32_swap(qd[0][e], qd[1][e], false, false);
+                first[e] = (int)x[0];
+                second[e] = (int)x[1];
+            }
+            signed char* orow = (signed char*)p.out + m * p.out_cs + n0 + 32 * lh;
+            const int ch = n0 + 32 * lh;
+            if (pix_ok) {
+                if (ch < p.out_cs) *(v4i*)orow = first;
+                if (ch + 16 < p.out_cs) *(v4i*)(orow + 16) = second;
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+} // namespace n2d2hip
