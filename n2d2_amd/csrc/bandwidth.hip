@@ -69,6 +69,63 @@ __global__ __launch_bounds__(256) void pool_kernel(const signed char* __restrict
     }
 }
 
+// Max pooling with a small compile-time window, 16 channels per thread.  The maximum of signed bytes is taken on the
+// packed words themselves: even and odd bytes are moved to the high halves of two 16-bit pairs, where the packed
+// 16-bit maximum orders them as bytes.  A tap outside the input is replaced by the nearest tap inside, which cannot
+// change a maximum; the host guarantees that every window has one.  Every load of a window is issued before any use.
+typedef short v2s __attribute__((ext_vector_type(2)));
+template <int PW, int PH>
+__global__ __launch_bounds__(256) void pool_max_fast_kernel(const signed char* __restrict__ in, int cs, int B, int H, int W,
+                                                            signed char* __restrict__ out, int OH, int OW,
+                                                            int strideX, int strideY, int padX, int padY, unsigned flip)
+{
+    const int cq = cs >> 4;
+    const long long total = (long long)B * OH * OW * cq;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        const int c16 = (int)(idx % cq) * 16;
+        long long r = idx / cq;
+        const int ox = (int)(r % OW); r /= OW;
+        const int oy = (int)(r % OH);
+        const int b = (int)(r / OH);
+        const int bx = ox * strideX - padX, by = oy * strideY - padY;
+        const int xlo = max(bx, 0), xhi = min(bx + PW, W) - 1, ylo = max(by, 0), yhi = min(by + PH, H) - 1;
+        const signed char* img = in + (long long)b * H * W * cs + c16;
+        int4 v[PH][PW];
+#pragma unroll
+        for (int sy = 0; sy < PH; ++sy) {
+            const int iy = min(max(by + sy, ylo), yhi);
+#pragma unroll
+            for (int sx = 0; sx < PW; ++sx) {
+                const int ix = min(max(bx + sx, xlo), xhi);
+                v[sy][sx] = *(const int4*)(img + ((long long)iy * W + ix) * cs);
+            }
+        }
+        unsigned res[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            v2s me, mo;
+#pragma unroll
+            for (int sy = 0; sy < PH; ++sy)
+#pragma unroll
+                for (int sx = 0; sx < PW; ++sx) {
+                    const int4 t = v[sy][sx];
+                    const unsigned w = (unsigned)(q == 0 ? t.x : q == 1 ? t.y : q == 2 ? t.z : t.w) ^ flip;
+                    const unsigned ev = (w << 8) & 0xFF00FF00u, od = w & 0xFF00FF00u;
+                    v2s e, o;
+                    __builtin_memcpy(&e, &ev, 4);
+                    __builtin_memcpy(&o, &od, 4);
+                    if (sy == 0 && sx == 0) { me = e; mo = o; }
+                    else { me = __builtin_elementwise_max(me, e); mo = __builtin_elementwise_max(mo, o); }
+                }
+            unsigned ue, uo;
+            __builtin_memcpy(&ue, &me, 4);
+            __builtin_memcpy(&uo, &mo, 4);
+            res[q] = (((ue >> 8) & 0x00FF00FFu) | (uo & 0xFF00FF00u)) ^ flip;
+        }
+        *(uint4*)(out + idx * 16) = uint4{res[0], res[1], res[2], res[3]};
+    }
+}
+
 constexpr int EW_MAX_INPUTS = 4;
 struct ElemWiseArgs;
 int run_elemwise(const ElemWiseArgs& a, bool fcoef, hipStream_t stream);
@@ -277,7 +334,19 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
     const unsigned flip = in->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
     const int zp = in->dtype == N2D2HIP_I8 ? 0 : 128;      // after the flip, U8 bytes read as value-128 too
-    if (d->pooling == N2D2HIP_POOL_MAX)
+    // windows that all hold at least one input element, square 2x2 or 3x3, 16-byte channel groups
+    const bool fast = d->pooling == N2D2HIP_POOL_MAX && in->cs % 16 == 0 && d->poolW == d->poolH && (d->poolW == 2 || d->poolW == 3)
+        && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < in->W && (OH - 1) * d->strideY - d->padY < in->H;
+    if (fast) {
+        const long long total16 = (long long)in->B * OH * OW * (in->cs / 16);
+        const unsigned g16 = (unsigned)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64));
+        if (d->poolW == 3)
+            hipLaunchKernelGGL((pool_max_fast_kernel<3, 3>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
+                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip);
+        else
+            hipLaunchKernelGGL((pool_max_fast_kernel<2, 2>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
+                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip);
+    } else if (d->pooling == N2D2HIP_POOL_MAX)
         hipLaunchKernelGGL(pool_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
     else

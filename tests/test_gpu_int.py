@@ -296,11 +296,14 @@ def test_fc_cell_bit_exact(rt, shape):
 
 @pytest.mark.parametrize("kind,pool,stride,pad", [("max", (2, 2), (2, 2), (0, 0)), ("max", (3, 3), (2, 2), (0, 0)),
                                                   ("max", (3, 3), (2, 2), (1, 1)), ("avg", (7, 7), (7, 7), (0, 0)),
-                                                  ("avg", (3, 3), (2, 2), (1, 1)), ("avg", (2, 2), (2, 2), (0, 0))])
+                                                  ("avg", (3, 3), (2, 2), (1, 1)), ("avg", (2, 2), (2, 2), (0, 0)),
+                                                  ("max", (3, 3), (1, 1), (1, 1)), ("max", (2, 2), (1, 1), (1, 1)),
+                                                  ("max", (3, 3), (3, 2), (2, 0)), ("max", (3, 2), (2, 2), (1, 1))])
 def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
     from n2d2_amd import capi
     from oracle import cells as cells_ref
-    for dt, x in ((capi.U8B, _u8((3, 24, 14, 15))), (capi.I8, _i8((3, 24, 14, 15), -128, 127)), (capi.U8, _u8((2, 3, 14, 14)))):
+    for dt, x in ((capi.U8B, _u8((3, 24, 14, 15))), (capi.I8, _i8((3, 24, 14, 15), -128, 127)), (capi.U8, _u8((2, 3, 14, 14))),
+                  (capi.U8, _u8((2, 16, 9, 14))), (capi.U8B, _u8((2, 64, 13, 13)))):
         want = cells_ref.pool_cell(x, kind, pool, stride, pad)
         got = rt.Pool(kind, pool, stride, pad).forward(rt.DTensor.from_numpy(x, dt)).to_numpy()
         assert np.array_equal(got, want.astype(np.int64)), (kind, dt)
