@@ -333,6 +333,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 }
             }
         }
+        // Without a folded sum, the convolution's tables of the next channel group are requested before this group is
+        // rescaled (two register sets), so that their LDS latency is hidden behind the arithmetic.
+        v4i tq[2][5];
+        auto request_tables = [&](v4i* t, unsigned trow) {
+            lds_read128_nowait<BN * 4>(t[0], trow);
+            lds_read128_nowait<2 * BN * 4>(t[1], trow);
+            lds_read128_nowait<3 * BN * 4>(t[2], trow);
+            if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(t[3], trow);
+            if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(t[4], trow);
+        };
+        constexpr int NTR = 3 + (EPI == EPI_I24 ? 1 : 0) + (EPI != EPI_F32 ? 1 : 0);      // reads per request
+        if (!RES && EPI != EPI_RAW)
+            request_tables(tq[0], tab);
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
 #pragma unroll
@@ -340,16 +353,48 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 const int idx = i * 4 + g;
                 const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
                 int r[NJ][4];
+                // RES: every table of the group is requested at once (LDS answers in order); each phase then waits only
+                // for its own, so one LDS latency is paid per group instead of three
+                v4i xa, xb, xc, xd, xe, sa, sb, sc, sd, se;
                 {
                     // ---- the convolution's own rescale
                     v4i ta = {0, 0, 0, 0}, tb = ta, tc = ta, td = ta, te = ta;
-                    if (EPI != EPI_RAW) {
+                    if (EPI != EPI_RAW && !RES) {
+                        if (idx + 1 < NI * 4) {
+                            const int nx = idx + 1;
+                            request_tables(tq[nx & 1], tab + (unsigned)((nx / 4) * 32 + 8 * (nx % 4)) * 4u);
+                            wait_lgkm<NTR>();
+                        } else {
+                            wait_lgkm<0>();
+                        }
+                        ta = tq[idx & 1][0]; tb = tq[idx & 1][1]; tc = tq[idx & 1][2];
+                        if (EPI == EPI_I24) td = tq[idx & 1][3];
+                        if (EPI != EPI_F32) te = tq[idx & 1][4];
+                        tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                    }
+                    if (EPI != EPI_RAW && RES) {
                         lds_read128_nowait<BN * 4>(ta, trow);
                         lds_read128_nowait<2 * BN * 4>(tb, trow);
                         lds_read128_nowait<3 * BN * 4>(tc, trow);
                         if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(td, trow);
                         if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(te, trow);
-                        wait_lgkm<0>();
+                        if (RES) {
+                            if (q.has_pre) {
+                                lds_read128_nowait<11 * BN * 4>(xa, trow);
+                                lds_read128_nowait<12 * BN * 4>(xb, trow);
+                                lds_read128_nowait<13 * BN * 4>(xc, trow);
+                                lds_read128_nowait<14 * BN * 4>(xd, trow);
+                                lds_read128_nowait<15 * BN * 4>(xe, trow);
+                            }
+                            lds_read128_nowait<6 * BN * 4>(sa, trow);
+                            lds_read128_nowait<7 * BN * 4>(sb, trow);
+                            lds_read128_nowait<8 * BN * 4>(sc, trow);
+                            lds_read128_nowait<9 * BN * 4>(sd, trow);
+                            lds_read128_nowait<10 * BN * 4>(se, trow);
+                            if (q.has_pre) wait_lgkm<10>(); else wait_lgkm<5>();
+                        } else {
+                            wait_lgkm<0>();
+                        }
                         tie(ta); tie(tb); tie(tc); tie(td); tie(te);
                     }
                     if (EPI == EPI_I24 && q.preclamp) {
@@ -392,13 +437,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                         o[j][3] = (int)w >> 24;
                     }
                     if (q.has_pre) {
-                        v4i xa, xb, xc, xd, xe;
-                        lds_read128_nowait<11 * BN * 4>(xa, trow);
-                        lds_read128_nowait<12 * BN * 4>(xb, trow);
-                        lds_read128_nowait<13 * BN * 4>(xc, trow);
-                        lds_read128_nowait<14 * BN * 4>(xd, trow);
-                        lds_read128_nowait<15 * BN * 4>(xe, trow);
-                        wait_lgkm<0>();
+                        wait_lgkm<5>();
                         tie(xa); tie(xb); tie(xc); tie(xd); tie(xe);
                         if (q.pre_clamp) {
 #pragma unroll
@@ -413,12 +452,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                             for (int t = 0; t < 4; ++t)
                                 o[j][t] = med3_i32((__mul24(o[j][t], xc[t]) + xd[t]) >> xe[t], plo, phi);
                     }
-                    v4i sa, sb, sc, sd, se;
-                    lds_read128_nowait<6 * BN * 4>(sa, trow);
-                    lds_read128_nowait<7 * BN * 4>(sb, trow);
-                    lds_read128_nowait<8 * BN * 4>(sc, trow);
-                    lds_read128_nowait<9 * BN * 4>(sd, trow);
-                    lds_read128_nowait<10 * BN * 4>(se, trow);
                     wait_lgkm<0>();
                     tie(sa); tie(sb); tie(sc); tie(sd); tie(se);
 #pragma unroll
