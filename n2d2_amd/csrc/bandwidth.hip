@@ -81,7 +81,10 @@ __global__ __launch_bounds__(256) void pool_max_fast_kernel(const signed char* _
 {
     const int cq = cs >> 4;
     const long long total = (long long)B * OH * OW * cq;
-    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+    // blocks 8 apart run on the same XCD: give an XCD consecutive logical blocks, so that the rows two neighbouring
+    // windows share come out of that XCD's L2 (the grid is a multiple of 8)
+    const long long lblock = (long long)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    for (long long idx = lblock * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
         const int c16 = (int)(idx % cq) * 16;
         long long r = idx / cq;
         const int ox = (int)(r % OW); r /= OW;
@@ -339,7 +342,7 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
         && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < in->W && (OH - 1) * d->strideY - d->padY < in->H;
     if (fast) {
         const long long total16 = (long long)in->B * OH * OW * (in->cs / 16);
-        const unsigned g16 = (unsigned)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64));
+        const unsigned g16 = (unsigned)round_up((int)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64)), 8);
         if (d->poolW == 3)
             hipLaunchKernelGGL((pool_max_fast_kernel<3, 3>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
                                in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip);

@@ -815,7 +815,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         const int BMp = small_m ? 64 : wide64 ? 256 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
-        q.mlanes = 8 * per_xcd;
+        q.mlanes = per_xcd;
+        q.xcd_tiles = (q.mtiles + 7) / 8;
         const int grid = 8 * a.ntiles_n * per_xcd;
         q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
         q.sum = EpiArgs(); q.pre = EpiArgs();
@@ -873,10 +874,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.tiles_per_row = (OW + 127) / 128;
             q.ntiles = in->B * OH * q.tiles_per_row;
             q.c.ntiles_n = (round_up(d.O, 16) + 63) / 64;
-            q.nlanes = std::max(1, std::min(q.ntiles, (3 * num_cus()) / q.c.ntiles_n));
+            q.nlanes = std::max(1, std::min((q.ntiles + 7) / 8, (3 * num_cus()) / (8 * q.c.ntiles_n)));
+            q.xcd_tiles = (q.ntiles + 7) / 8;
             magic_div((unsigned)OH, &q.oh_mul, &q.oh_sh);
             magic_div((unsigned)q.tiles_per_row, &q.tpr_mul, &q.tpr_sh);
-            const int grid = q.nlanes * q.c.ntiles_n;
+            const int grid = 8 * q.nlanes * q.c.ntiles_n;
             if (d.kH == 3) launch_stem<3>(q, grid, stream);
             else if (d.kH == 5) launch_stem<5>(q, grid, stream);
             else launch_stem<7>(q, grid, stream);

@@ -84,7 +84,9 @@ __device__ __forceinline__ int div_magic(int n, unsigned mul, unsigned sh)
 struct ConvPipeArgs {
     ConvArgs c;
     const signed char* fill16;   // 16 bytes of the input's logical zero (device)
-    int mtiles, mlanes;          // pixel tiles, and how many block "lanes" walk them
+    int mtiles;                  // pixel tiles
+    int xcd_tiles;               // consecutive pixel tiles given to one XCD
+    int mlanes;                  // blocks of one XCD (and channel tile) that share its pixel tiles
     int cper;                    // 64-byte K steps per kernel tap (C / 64)
     int kW, kH;
     unsigned ohw_mul, ohw_sh, ow_mul, ow_sh;     // division by OH*OW and by OW
@@ -151,13 +153,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const int wm = wave % WGM, wn = wave / WGM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    // ---- which tiles this block walks: one channel tile, every mlanes-th pixel tile.
+    // ---- which tiles this block walks: one channel tile, every mlanes-th pixel tile of its XCD's run.
     // Blocks 8 apart run on the same XCD; they take the same pixel tiles for neighbouring channel tiles.
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int tile_n = slot % p.ntiles_n;
-    const int mlane = (slot / p.ntiles_n) * 8 + xcd;
+    // An XCD gets a run of consecutive pixel tiles (neighbouring tiles share their window halo through that XCD's L2)
+    // and its blocks take them in turn.
+    const int mlane = xcd * q.xcd_tiles + slot / p.ntiles_n;
+    const int mend = min((xcd + 1) * q.xcd_tiles, q.mtiles);
     const int n0 = tile_n * BN;
-    const int ntile = (mlane < q.mtiles) ? (q.mtiles - mlane + q.mlanes - 1) / q.mlanes : 0;
+    const int ntile = (mlane < mend) ? (mend - mlane + q.mlanes - 1) / q.mlanes : 0;
     const int niter = p.niter;
 #ifdef N2D2HIP_PROFILE
     long long pr_t0 = clock64(), pr_t1 = 0, pr_t2 = 0, pr_t3 = 0, pr_epi = 0, pr_w0 = wall_clock64();

@@ -32,7 +32,8 @@ struct ConvStemArgs {
     const signed char* fill16;   // the input's logical zero
     int ntiles;                  // pixel tiles: B * OH * tiles_per_row
     int tiles_per_row;
-    int nlanes;                  // blocks that share the pixel tiles of one channel tile
+    int nlanes;                  // blocks of one XCD that share its run of pixel tiles
+    int xcd_tiles;               // consecutive pixel tiles given to one XCD
     unsigned oh_mul, oh_sh;      // division by OH
     unsigned tpr_mul, tpr_sh;    // division by tiles_per_row
     int preclamp;
@@ -57,14 +58,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
-    const int tile_n = blockIdx.x % p.ntiles_n;
-    const int blane = blockIdx.x / p.ntiles_n;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;      // blocks 8 apart run on the same XCD
+    const int tile_n = slot % p.ntiles_n;
     const int n0 = tile_n * BN;
-    const int ntile = (blane < q.ntiles) ? (q.ntiles - blane + q.nlanes - 1) / q.nlanes : 0;
+    // An XCD gets a run of consecutive tiles (consecutive output rows share most of their input rows through that XCD's
+    // L2) and its blocks take them in turn.
+    const int first = xcd * q.xcd_tiles + slot / p.ntiles_n;
+    const int last = min((xcd + 1) * q.xcd_tiles, q.ntiles);
+    const int ntile = (first < last) ? (last - first + q.nlanes - 1) / q.nlanes : 0;
 
     // ---- loader: chunk c = wave + 4*j is 64 pixels (part c%5) of patch row c/5
     auto issue = [&](int t, int stage) {
-        const int id = blane + t * q.nlanes;
+        const int id = first + t * q.nlanes;
         const bool live = t < ntile;
         const int rowid = div_magic(live ? id : 0, q.tpr_mul, q.tpr_sh);          // b * OH + oy
         const int txi = (live ? id : 0) - rowid * q.tiles_per_row;
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         }
 
         // ---- epilogue: this lane holds channels 8g + 4*lh .. +3 of both 32-channel tiles for output pixel ox
-        const int id = blane + t * q.nlanes;
+        const int id = first + t * q.nlanes;
         const int rowid = div_magic(id, q.tpr_mul, q.tpr_sh);
         const int ox = (id - rowid * q.tiles_per_row) * TW + 32 * wave + l32;
         const long long m = (long long)rowid * p.OW + ox;
