@@ -17,6 +17,9 @@ if ROOT not in sys.path:
 
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
+# HBM bytes one conv_pipe_kernel launch of this workload moves on average: rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy), summary under profiles/
+PIPE_TRAFFIC_BYTES_PER_LAUNCH = (38.53 + 23.76) * 1048576.0
 
 
 def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
@@ -128,7 +131,9 @@ def main():
     roofline = {"bound": "mfma", "kernel": "conv_pipe_kernel (%d launches of one forward: every conv/fc cell with a multiple of 64 input "
                 "channels, residual sums folded in)" % len(pipe),
                 "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                "traffic": None, "launches_per_step": len(pipe), "avg_launch_us": round(conv_ms * 1000.0 / len(pipe), 2),
+                "traffic": round(PIPE_TRAFFIC_BYTES_PER_LAUNCH) if B == 128 else None,
+                "algorithmic_bytes_per_launch": round(sum(net.layer_bytes(net.launched[k]) for k in pipe) / len(pipe)),
+                "launches_per_step": len(pipe), "avg_launch_us": round(conv_ms * 1000.0 / len(pipe), 2),
                 "ops_per_launch": conv_ops / len(pipe)}
     all_bytes = sum(net.layer_bytes(l) for l in net.launched)
     hbm = all_bytes / (ms * 1e-3) / 1e9
