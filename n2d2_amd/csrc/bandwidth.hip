@@ -129,6 +129,37 @@ __global__ __launch_bounds__(256) void pool_max_fast_kernel(const signed char* _
     }
 }
 
+// Global average pooling (the window is the whole input, no padding): a block takes 256 channels of one image, its four
+// waves share the pixels and meet in LDS.  Same arithmetic as pool_kernel<false>: integer sum, division truncated
+// toward zero (ref: src/Cell/PoolCell_Frame_Kernels.cpp:120-197 followed by the export's std::trunc).
+__global__ __launch_bounds__(256) void global_avg_pool_kernel(const signed char* __restrict__ in, int cs, int npix,
+                                                              signed char* __restrict__ out, int zp, unsigned flip)
+{
+    __shared__ int part[4][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int slabs = (cs + 255) / 256;
+    const int b = blockIdx.x / slabs, c4 = (blockIdx.x % slabs) * 256 + lane * 4;
+    int acc[4] = {0, 0, 0, 0};
+    if (c4 < cs) {
+        const signed char* src = in + (long long)b * npix * cs + c4;
+        for (int p = wave; p < npix; p += 4) {
+            int v[4];
+            unpack4(*(const int*)(src + (long long)p * cs) ^ (int)flip, zp, v);
+            acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        part[wave][lane][t] = acc[t];
+    __syncthreads();
+    if (wave == 0 && c4 < cs) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] = (part[0][lane][t] + part[1][lane][t] + part[2][lane][t] + part[3][lane][t]) / npix - zp;
+        *(unsigned*)(out + (long long)b * cs + c4) = pack4(acc) ^ flip;
+    }
+}
+
 constexpr int EW_MAX_INPUTS = 4;
 struct ElemWiseArgs;
 int run_elemwise(const ElemWiseArgs& a, bool fcoef, hipStream_t stream);
@@ -340,7 +371,11 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     // windows that all hold at least one input element, square 2x2 or 3x3, 16-byte channel groups
     const bool fast = d->pooling == N2D2HIP_POOL_MAX && in->cs % 16 == 0 && d->poolW == d->poolH && (d->poolW == 2 || d->poolW == 3)
         && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < in->W && (OH - 1) * d->strideY - d->padY < in->H;
-    if (fast) {
+    if (d->pooling == N2D2HIP_POOL_AVERAGE && OH == 1 && OW == 1 && d->poolW == in->W && d->poolH == in->H && d->padX == 0 && d->padY == 0) {
+        const int slabs = (in->cs + 255) / 256;
+        hipLaunchKernelGGL(global_avg_pool_kernel, dim3((unsigned)(in->B * slabs)), dim3(256), 0, (hipStream_t)stream,
+                           (const signed char*)in->data, in->cs, in->H * in->W, (signed char*)out->data, zp, flip);
+    } else if (fast) {
         const long long total16 = (long long)in->B * OH * OW * (in->cs / 16);
         const unsigned g16 = (unsigned)round_up((int)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64)), 8);
         if (d->poolW == 3)

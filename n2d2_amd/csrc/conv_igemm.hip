@@ -810,8 +810,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         const long long tiles128 = ((Mll + 127) / 128) * a.ntiles_n;
         const char* bm_env = getenv("N2D2HIP_BM64");
         const bool small_m = bn128 && d.C % 128 == 0 && (bm_env ? atoi(bm_env) != 0 : tiles128 < (3 * num_cus()) / 2);
-        const char* wide_env = getenv("N2D2HIP_WIDE64");
-        const bool wide64 = !bn128 && !other && wide_env && atoi(wide_env) != 0;      // 256 pixels x 64 channels
+        // 64-channel layers whose K advances in 64-byte steps take 256-pixel tiles: twice the MFMAs per ring stage
+        const bool wide64 = !bn128 && !other && d.C % 128 != 0 && Mll >= 256ll * 4 * num_cus();
         const int BMp = small_m ? 64 : wide64 ? 256 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));

@@ -232,6 +232,7 @@ void Cell_Frame_HIP::addInput(Cell_Frame_HIP* parent)
     if (!mInputs.empty() && (parent->getOutputsWidth() != mInW || parent->getOutputsHeight() != mInH || parent->batchSize() != mBatch))
         throw std::runtime_error("Cell " + mName + ": inputs of different sizes");
     mParents.push_back(parent);
+    mParentCells.push_back(parent);
     mInputs.push_back(&parent->mOutputs);
     if (mInputs.size() == 1)
         mNbChannels = parent->getNbOutputs();
@@ -248,6 +249,7 @@ void Cell_Frame_HIP::addInput(HipTensor& stimuli, unsigned int nbChannels, unsig
     if (!mInputs.empty())
         throw std::runtime_error("Cell " + mName + ": the environment must be the only input");
     mParents.push_back(nullptr);
+    mParentCells.push_back(nullptr);
     mInputs.push_back(&stimuli);
     mNbChannels = nbChannels;
     mInW = width;
@@ -258,6 +260,9 @@ void Cell_Frame_HIP::addInput(HipTensor& stimuli, unsigned int nbChannels, unsig
 
 const Tensor<Float_T>& Cell_Frame_HIP::getOutputs()
 {
+    if (mFoldedInto)
+        throw std::runtime_error("Cell " + mName + ": its output is not materialised, cell " + mFoldedInto->getName()
+                                 + " computes it on the fly (DeepNet::setFusion(false) keeps every output)");
     return mOutputs.synchronizeDToH(mStream);
 }
 
@@ -357,7 +362,7 @@ ConvCell_Frame_HIP<T>::ConvCell_Frame_HIP(const DeepNet& /*deepNet*/, const std:
                                           unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
                                           const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
                                           const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr)
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr), mConvInDType(-1)
 {
     mActivation = activation;
 }
@@ -394,9 +399,24 @@ void ConvCell_Frame_HIP<T>::initialize()
 template <class T>
 void ConvCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
+    prepare();
+    launch();
+}
+
+template <class T>
+void ConvCell_Frame_HIP<T>::launch()
+{
+    checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <class T>
+bool ConvCell_Frame_HIP<T>::prepare()
+{
     n2d2hip_act_t act = activationHandle();
     const int inDType = mInputs[0]->desc().dtype;
-    if (mDirty || act != mConvAct || !mConv) {
+    bool rebuilt = false;
+    if (mDirty || act != mConvAct || !mConv || inDType != mConvInDType) {
         if (mConv) { n2d2hip_conv_destroy(mConv); mConv = nullptr; }
         const unsigned int cg = mNbChannels / mNbGroups;
         if (mWeights.dimX() != mKernelDims[0] || mWeights.dimY() != mKernelDims[1] || mWeights.dimZ() != cg || mWeights.dimB() != mNbOutputs)
@@ -418,10 +438,11 @@ void ConvCell_Frame_HIP<T>::propagate(bool /*inference*/)
         }
         checkStatus(n2d2hip_conv_create(&d, w.data(), mNoBias ? nullptr : b.data(), act, inDType, &mConv));
         mConvAct = act;
+        mConvInDType = inDType;
         mDirty = false;
+        rebuilt = true;
     }
-    checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
-    mOutputs.invalidateHost();
+    return rebuilt;
 }
 
 template <> Registrar<ConvCell> ConvCell_Frame_HIP<float>::mRegistrar("Frame_HIP", ConvCell_Frame_HIP<float>::create,
@@ -569,7 +590,7 @@ std::pair<double, double> ElemWiseCell::elemWiseOutputsRange() const
 ElemWiseCell_Frame_HIP::ElemWiseCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs, Operation operation,
                                                CoeffMode mode, const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts,
                                                const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts), mEw(nullptr), mEwAct(nullptr)
+    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts), mEw(nullptr), mEwAct(nullptr), mFusedConv(nullptr), mFusedIndex(0)
 {
     mActivation = activation;
     if (operation != Sum)
@@ -600,17 +621,87 @@ void ElemWiseCell_Frame_HIP::initialize()
 
 void ElemWiseCell_Frame_HIP::propagate(bool /*inference*/)
 {
+    prepare();
+    launch();
+}
+
+bool ElemWiseCell_Frame_HIP::prepare()
+{
     n2d2hip_act_t act = activationHandle();
-    if (!mEw || act != mEwAct) {
-        if (mEw) { n2d2hip_elemwise_destroy(mEw); mEw = nullptr; }
-        const int mode = mCoeffMode == PerChannel ? N2D2HIP_COEFF_PER_CHANNEL : (mCoeffMode == PerInput ? N2D2HIP_COEFF_PER_INPUT : N2D2HIP_COEFF_PER_LAYER);
-        checkStatus(n2d2hip_elemwise_create((int)mInputs.size(), (int)mNbOutputs, mode, mWeights.data(), mShifts.data(), act, &mEw));
-        mEwAct = act;
+    if (mEw && act == mEwAct)
+        return false;
+    // the convolution that took this sum over borrows mEw: release it first
+    clearFusion();
+    if (mEw) { n2d2hip_elemwise_destroy(mEw); mEw = nullptr; }
+    const int mode = mCoeffMode == PerChannel ? N2D2HIP_COEFF_PER_CHANNEL : (mCoeffMode == PerInput ? N2D2HIP_COEFF_PER_INPUT : N2D2HIP_COEFF_PER_LAYER);
+    checkStatus(n2d2hip_elemwise_create((int)mInputs.size(), (int)mNbOutputs, mode, mWeights.data(), mShifts.data(), act, &mEw));
+    mEwAct = act;
+    return true;
+}
+
+// The tensor input k is read from: the ScalingCell's own input once that cell is folded
+static HipTensor* sourceOf(const std::vector<Cell_Frame_HIP*>& folded, const std::vector<HipTensor*>& inputs, size_t k)
+{
+    return (k < folded.size() && folded[k]) ? folded[k]->inputTensor(0) : inputs[k];
+}
+
+void ElemWiseCell_Frame_HIP::launch()
+{
+    if (mFusedConv) {
+        checkStatus(n2d2hip_conv_forward_sum(mFusedConv->convHandle(), &mFusedConv->inputTensor(0)->desc(),
+                                             &sourceOf(mFoldedScaling, mInputs, 1 - mFusedIndex)->desc(), &mOutputs.desc(), mStream));
+    } else {
+        std::vector<const n2d2hip_tensor*> ins;
+        for (size_t k = 0; k < mInputs.size(); ++k)
+            ins.push_back(&sourceOf(mFoldedScaling, mInputs, k)->desc());
+        checkStatus(n2d2hip_elemwise_forward(mEw, ins.data(), &mOutputs.desc(), mStream));
     }
-    std::vector<const n2d2hip_tensor*> ins;
-    for (HipTensor* t : mInputs) ins.push_back(&t->desc());
-    checkStatus(n2d2hip_elemwise_forward(mEw, ins.data(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
+}
+
+bool ElemWiseCell_Frame_HIP::foldInputScaling(size_t k, Cell_Frame_HIP* scaling)
+{
+    if (!mEw || k >= mInputs.size() || !scaling || !scaling->scalingHandle() || mFusedConv)
+        return false;
+    const int rc = n2d2hip_elemwise_fold_input_scaling(mEw, (int)k, scaling->scalingHandle());
+    if (rc == N2D2HIP_ERR_UNSUPPORTED)
+        return false;
+    checkStatus(rc);
+    mFoldedScaling.resize(mInputs.size(), nullptr);
+    mFoldedScaling[k] = scaling;
+    scaling->setFoldedInto(this);
+    return true;
+}
+
+bool ElemWiseCell_Frame_HIP::fuseIntoConv(size_t k, Cell_Frame_HIP* conv)
+{
+    if (!mEw || mInputs.size() != 2 || k > 1 || !conv || !conv->convHandle() || mFusedConv)
+        return false;
+    const int rc = n2d2hip_conv_fuse_sum(conv->convHandle(), mEw, (int)k, sourceOf(mFoldedScaling, mInputs, 1 - k)->desc().dtype);
+    if (rc == N2D2HIP_ERR_UNSUPPORTED)
+        return false;
+    checkStatus(rc);
+    mFusedConv = conv;
+    mFusedIndex = k;
+    conv->setFoldedInto(this);
+    return true;
+}
+
+void ElemWiseCell_Frame_HIP::clearFusion()
+{
+    if (mFusedConv) {
+        if (mFusedConv->convHandle())
+            checkStatus(n2d2hip_conv_fuse_sum(mFusedConv->convHandle(), nullptr, 0, 0));
+        mFusedConv->setFoldedInto(nullptr);
+        mFusedConv = nullptr;
+    }
+    for (size_t k = 0; k < mFoldedScaling.size(); ++k) {
+        if (!mFoldedScaling[k]) continue;
+        if (mEw)
+            checkStatus(n2d2hip_elemwise_fold_input_scaling(mEw, (int)k, nullptr));
+        mFoldedScaling[k]->setFoldedInto(nullptr);
+        mFoldedScaling[k] = nullptr;
+    }
 }
 
 Registrar<ElemWiseCell> ElemWiseCell_Frame_HIP::mRegistrar("Frame_HIP", ElemWiseCell_Frame_HIP::create, Registrar<ElemWiseCell>::Type<float>());
@@ -661,8 +752,23 @@ void ScalingCell_Frame_HIP<T>::initialize()
 template <class T>
 void ScalingCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
+    prepare();
+    launch();
+}
+
+template <class T>
+void ScalingCell_Frame_HIP<T>::launch()
+{
+    checkStatus(n2d2hip_scaling_forward(mScalingAct, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <class T>
+bool ScalingCell_Frame_HIP<T>::prepare()
+{
     // src/Cell/ScalingCell_Frame.cpp:67-75: mScaling.propagate(*this, in, out, mQuantizedNbBits), no activation
     const bool uns = DeepNetExport::isCellOutputUnsigned(*this);
+    bool rebuilt = false;
     if (!mScalingAct || mBuiltRevision != mScalingRevision || mBuiltUnsigned != (int)uns) {
         if (mScalingAct) { n2d2hip_act_destroy(mScalingAct); mScalingAct = nullptr; }
         mScalingAct = makeAct(mScaling, N2D2HIP_ACT_LINEAR, 0.0f, mQuantizedNbBits, uns, mNbOutputs, mName);
@@ -670,9 +776,9 @@ void ScalingCell_Frame_HIP<T>::propagate(bool /*inference*/)
         mBuiltUnsigned = (int)uns;
         if (mOutputs.empty() || mOutputs.desc().dtype != outputDType(&mScaling))
             allocateOutputs(&mScaling);
+        rebuilt = true;
     }
-    checkStatus(n2d2hip_scaling_forward(mScalingAct, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
-    mOutputs.invalidateHost();
+    return rebuilt;
 }
 
 template <> Registrar<ScalingCell> ScalingCell_Frame_HIP<float>::mRegistrar("Frame_HIP", ScalingCell_Frame_HIP<float>::create,
@@ -1074,7 +1180,9 @@ void DeepNet::addCell(const std::shared_ptr<Cell>& cell, const std::vector<std::
         frame->addInput(pf.get());
     }
     mOrder.push_back(cell);
+    mFrames.push_back(frame.get());
     mCells[cell->getName()] = cell;
+    mPlanned = false;
 }
 
 std::shared_ptr<Cell> DeepNet::getCell(const std::string& name) const
@@ -1110,10 +1218,73 @@ void DeepNet::initialize()
         std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->initialize();
 }
 
-void DeepNet::propagate(bool inference)
+void DeepNet::propagate(bool /*inference*/)
 {
-    for (auto& c : mOrder)
-        std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->propagate(inference);
+    bool rebuilt = false;
+    for (Cell_Frame_HIP* f : mFrames)
+        rebuilt = f->prepare() || rebuilt;
+    if (mFusion && (rebuilt || !mPlanned))
+        planFusion();
+    for (Cell_Frame_HIP* f : mFrames) {
+        if (!f->foldedInto())
+            f->launch();
+    }
+}
+
+void DeepNet::setFusion(bool enabled)
+{
+    if (!enabled) {
+        for (Cell_Frame_HIP* f : mFrames) {
+            if (auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f))
+                ew->clearFusion();
+        }
+    }
+    mFusion = enabled;
+    mPlanned = false;
+}
+
+size_t DeepNet::nbFoldedCells() const
+{
+    return (size_t)std::count_if(mFrames.begin(), mFrames.end(), [](const Cell_Frame_HIP* f) { return f->foldedInto() != nullptr; });
+}
+
+// Every handle is current when this runs (all cells prepared).  Decisions follow the graph only; the device library has
+// the last word on each candidate and the cells stay separate launches where it declines.
+void DeepNet::planFusion()
+{
+    std::map<const Cell_Frame_HIP*, int> consumers, order;
+    order[nullptr] = -1;
+    for (size_t i = 0; i < mFrames.size(); ++i) {
+        order[mFrames[i]] = (int)i;
+        for (Cell_Frame_HIP* p : mFrames[i]->parentCells())
+            ++consumers[p];
+    }
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
+        if (!ew) continue;
+        ew->clearFusion();
+        const std::vector<Cell_Frame_HIP*>& parents = ew->parentCells();
+        // one ScalingCell read by this sum alone is applied inside the sum
+        size_t scaled = parents.size();
+        for (size_t k = 0; k < parents.size() && scaled == parents.size(); ++k) {
+            if (parents[k] && parents[k]->scalingHandle() && consumers[parents[k]] == 1 && !parents[k]->foldedInto()
+                && ew->foldInputScaling(k, parents[k]))
+                scaled = k;
+        }
+        if (parents.size() != 2) continue;
+        // the convolution that runs last among the two producers takes the sum into its epilogue
+        for (size_t k : {(size_t)1, (size_t)0}) {
+            Cell_Frame_HIP* conv = parents[k];
+            if (!conv || !conv->convHandle() || consumers[conv] != 1 || conv->foldedInto() || scaled == k)
+                continue;
+            const Cell_Frame_HIP* other = scaled == 1 - k ? parents[1 - k]->parentCells().at(0) : parents[1 - k];
+            if (other == conv || order[other] > order[conv])
+                continue;
+            if (ew->fuseIntoConv(k, conv))
+                break;
+        }
+    }
+    mPlanned = true;
 }
 
 void DeepNet::synchronize()

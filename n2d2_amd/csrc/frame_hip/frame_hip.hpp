@@ -363,8 +363,21 @@ public:
     virtual void addInput(HipTensor& stimuli, unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize);
     virtual void initialize() {}
     virtual void propagate(bool inference = false) = 0;
-    // Outputs as N2D2 sees them: float tensor {W,H,C,B} holding integer values.
+    // propagate() in two halves, for a runner that fuses cells: prepare() (re)builds the device handles a parameter
+    // change invalidated and tells whether it rebuilt any; launch() enqueues the kernels.
+    virtual bool prepare() { return false; }
+    virtual void launch() { propagate(true); }
+    // Outputs as N2D2 sees them: float tensor {W,H,C,B} holding integer values.  Throws for a cell whose work a
+    // consumer has taken over (DeepNet::setFusion): its tensor is never written.
     const Tensor<Float_T>& getOutputs();
+    // The cell that computes this one's result on the fly instead of reading its output, if any
+    Cell_Frame_HIP* foldedInto() const { return mFoldedInto; }
+    void setFoldedInto(Cell_Frame_HIP* consumer) { mFoldedInto = consumer; }
+    const std::vector<Cell_Frame_HIP*>& parentCells() const { return mParentCells; }
+    HipTensor* inputTensor(size_t k) const { return mInputs.at(k); }
+    // Device handles a consumer borrows when it folds this cell (null for cells that cannot be folded)
+    virtual n2d2hip_act_t scalingHandle() const { return nullptr; }
+    virtual n2d2hip_conv_t convHandle() const { return nullptr; }
     HipTensor& getDeviceOutputs() { return mOutputs; }
     bool isCuda() const { return false; }
     std::string getPyModel() const { return "Frame_HIP"; }
@@ -373,7 +386,7 @@ public:
     void setStream(void* stream) { mStream = stream; }
 
 protected:
-    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
+    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mFoldedInto(nullptr), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
     ~Cell_Frame_HIP();
     virtual void setOutputsDims() = 0;
     // (Re)builds the device tables of the activation when its Scaling, its bit width or the
@@ -382,9 +395,11 @@ protected:
     int outputDType(const Scaling* standalone = nullptr) const;
     void allocateOutputs(const Scaling* standalone = nullptr);
     std::vector<HipTensor*> mInputs;
+    std::vector<Cell_Frame_HIP*> mParentCells;  // null = the environment
     HipTensor mOutputs;
     unsigned int mBatch;
     void* mStream;
+    Cell_Frame_HIP* mFoldedInto;
 
 private:
     n2d2hip_act_t mActHandle;
@@ -444,6 +459,9 @@ public:
     }
     void initialize();
     void propagate(bool inference = false);
+    bool prepare();
+    void launch();
+    n2d2hip_conv_t convHandle() const { return mConv; }
 
 protected:
     void setOutputsDims();
@@ -451,6 +469,7 @@ protected:
 private:
     n2d2hip_conv_t mConv;
     n2d2hip_act_t mConvAct;
+    int mConvInDType;
     static Registrar<ConvCell> mRegistrar;
 };
 
@@ -583,6 +602,14 @@ public:
     }
     void initialize();
     void propagate(bool inference = false);
+    bool prepare();
+    void launch();
+    // Graph-level fusion (both return false, and change nothing, when the device library declines):
+    // the ScalingCell behind input k is applied on the fly and never launched ...
+    bool foldInputScaling(size_t k, Cell_Frame_HIP* scaling);
+    // ... and the convolution behind input k computes this sum in its epilogue: launch() then runs that one kernel.
+    bool fuseIntoConv(size_t k, Cell_Frame_HIP* conv);
+    void clearFusion();
     // src/Cell/ElemWiseCell_Frame.cpp:313-316
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : elemWiseOutputsRange(); }
 
@@ -592,6 +619,9 @@ protected:
 private:
     n2d2hip_elemwise_t mEw;
     n2d2hip_act_t mEwAct;
+    std::vector<Cell_Frame_HIP*> mFoldedScaling;  // per input, null = not folded
+    Cell_Frame_HIP* mFusedConv;
+    size_t mFusedIndex;
     static Registrar<ElemWiseCell> mRegistrar;
 };
 
@@ -625,6 +655,9 @@ public:
     }
     void initialize();
     void propagate(bool inference = false);
+    bool prepare();
+    void launch();
+    n2d2hip_act_t scalingHandle() const { return mScalingAct; }
     // src/Cell/ScalingCell_Frame.cpp:93-96
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : scalingOutputsRange(); }
 
@@ -882,9 +915,20 @@ public:
     void initialize();
     void propagate(bool inference = true);
     void synchronize();
+    // Fusion across cells (on by default): a ScalingCell read only by an ElemWise sum is applied inside that sum, and a
+    // two-input sum is computed in the epilogue of the 1x1 convolution that produces its later input.  Results are
+    // those of the separate cells, bit for bit; the folded cells' own outputs are not written (getOutputs() on them
+    // throws).  Turn it off to read every cell's output.
+    void setFusion(bool enabled);
+    bool getFusion() const { return mFusion; }
+    // Number of cells propagate() does not launch because a consumer computes them
+    size_t nbFoldedCells() const;
 
 private:
+    void planFusion();
+    bool mFusion = true, mPlanned = false;
     std::vector<std::shared_ptr<Cell> > mOrder;
+    std::vector<Cell_Frame_HIP*> mFrames;  // mOrder, as the cells' device side
     std::map<std::string, std::shared_ptr<Cell> > mCells;
     HipTensor mStimuli;
     unsigned int mEnvC = 0, mEnvH = 0, mEnvW = 0, mEnvB = 0;

@@ -110,6 +110,8 @@ void* fh_net_from_ini(const char* text)
 void fh_net_free(void* net) { delete (Net*)net; }
 const char* fh_net_model(void* net) { return ((Net*)net)->model.c_str(); }
 int fh_net_nb_cells(void* net) { return (int)((Net*)net)->deepNet->getCells().size(); }
+int fh_net_set_fusion(void* net, int enabled) { return guarded([&] { ((Net*)net)->deepNet->setFusion(enabled != 0); }); }
+int fh_net_nb_folded(void* net) { return (int)((Net*)net)->deepNet->nbFoldedCells(); }
 int fh_net_initialize(void* net) { return guarded([&] { ((Net*)net)->deepNet->initialize(); }); }
 int fh_net_propagate(void* net) { return guarded([&] { ((Net*)net)->deepNet->propagate(true); ((Net*)net)->deepNet->synchronize(); }); }
 

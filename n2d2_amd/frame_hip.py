@@ -18,7 +18,8 @@ lib.fh_last_error.restype = C.c_char_p
 lib.fh_net_from_ini.restype = C.c_void_p
 lib.fh_net_from_ini.argtypes = [C.c_char_p]
 lib.fh_net_model.restype = C.c_char_p
-for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize", "fh_net_propagate"):
+lib.fh_net_set_fusion.argtypes = [C.c_void_p, C.c_int]
+for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize", "fh_net_propagate", "fh_net_nb_folded"):
     getattr(lib, _n).argtypes = [C.c_void_p]
 lib.fh_net_set_stimuli.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
@@ -110,6 +111,14 @@ class Net:
 
     def initialize(self):
         _check(lib.fh_net_initialize(self.h))
+
+    def set_fusion(self, enabled):
+        """DeepNet::setFusion: cells folded into their consumer are not launched and their outputs not written."""
+        _check(lib.fh_net_set_fusion(self.h, int(bool(enabled))))
+
+    @property
+    def nb_folded(self):
+        return lib.fh_net_nb_folded(self.h)
 
     def set_stimuli(self, x):
         a = np.ascontiguousarray(x, dtype=np.float32)

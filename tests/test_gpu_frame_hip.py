@@ -15,9 +15,10 @@ def fh():
     frame_hip.set_globals(0, True, False)
 
 
-def _compare(fh, spec, x, keep):
+def _compare(fh, spec, x, keep, fusion=True):
     from oracle import cells
     net = fh.build_net(spec, x.shape[0])
+    net.set_fusion(fusion)
     net.initialize()
     net.set_stimuli(x)
     net.propagate()
@@ -41,13 +42,54 @@ def test_resnet50_through_the_registrar(fh):
     from n2d2_amd import nets
     spec = nets.resnet50()
     x = np.random.default_rng(32).integers(0, 256, size=(2, 3, 224, 224))
-    net = _compare(fh, spec, x, ["conv1", "pool1", "conv2.1_sum", "conv2.2_shortcut_rescale", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
+    net = _compare(fh, spec, x, ["conv1", "pool1", "conv2.1_sum", "conv2.2_1x1", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
+    # 12 shortcut ScalingCells applied inside their sums, 16 sums computed by the 1x1 convolution before them
+    assert net.nb_folded == 28
+    with pytest.raises(fh.FrameHipError) as e:
+        net.outputs("conv2.2_shortcut_rescale")
+    assert "not materialised" in str(e.value)
     # a second propagate on new stimuli reuses the prepared cells
     from oracle import cells
     x2 = np.random.default_rng(33).integers(0, 256, size=(2, 3, 224, 224))
     net.set_stimuli(x2)
     net.propagate()
     assert np.array_equal(net.outputs("fc"), cells.run_net(spec, x2)["fc"])
+    # without fusion every cell is launched and readable
+    net.set_fusion(False)
+    net.propagate()
+    assert net.nb_folded == 0
+    keep = ["conv2.2_shortcut_rescale", "conv2.2_1x1_x4", "conv2.2_sum", "fc"]
+    want = cells.run_net(spec, x2, keep=keep)
+    for name in keep:
+        assert np.array_equal(net.outputs(name), want[name]), name
+    # and back on: the plan is made again
+    net.set_fusion(True)
+    net.propagate()
+    assert net.nb_folded == 28 and np.array_equal(net.outputs("fc"), want["fc"])
+
+
+def test_fusion_follows_a_scaling_change(fh):
+    """Changing a folded ScalingCell's Scaling, or the sum's, rebuilds the handles and the fusion plan with them."""
+    from n2d2_amd import nets
+    from oracle import cells
+    spec = nets.resnet50(image=64)
+    x = np.random.default_rng(36).integers(0, 256, size=(2, 3, 64, 64))
+    net = fh.build_net(spec, 2)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    folded = net.nb_folded
+    assert folded > 0 and np.array_equal(net.outputs("fc"), cells.run_net(spec, x)["fc"])
+    by_name = {l.name: l for l in spec.layers}
+    sc = by_name["conv2.2_shortcut_rescale"]
+    sc.act.scaling = (np.asarray(sc.act.scaling) // 2).astype(sc.act.scaling.dtype)
+    sm = by_name["conv3.1_sum"]
+    sm.act.scaling = np.asarray(sm.act.scaling) + np.array([0, 1], dtype=np.asarray(sm.act.scaling).dtype)
+    for l in (sc, sm):
+        net.set_scaling(l.name, l.act.mode, l.act.scaling, l.act.frac_bits, l.act.clipping)
+    net.propagate()
+    assert net.nb_folded == folded
+    assert np.array_equal(net.outputs("fc"), cells.run_net(spec, x)["fc"])
 
 
 def test_mobilenet_and_w4a4_through_the_registrar(fh):

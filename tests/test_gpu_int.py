@@ -309,6 +309,18 @@ def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
         assert np.array_equal(got, want.astype(np.int64)), (kind, dt)
 
 
+def test_global_average_pool_bit_exact(rt):
+    """Whole-input average window (the classifier head's pooling): negative sums must truncate toward zero."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    for dt, x in ((capi.U8B, _u8((5, 2048, 7, 7))), (capi.I8, _i8((3, 300, 7, 5), -128, 127)), (capi.I8, _i8((2, 24, 3, 3), -128, 0)),
+                  (capi.U8, _u8((2, 3, 6, 6)))):
+        H, W = x.shape[2:]
+        want = cells_ref.pool_cell(x, "avg", (W, H), (W, H), (0, 0))
+        got = rt.Pool("avg", (W, H), (W, H), (0, 0)).forward(rt.DTensor.from_numpy(x, dt)).to_numpy()
+        assert got.shape == want.shape and np.array_equal(got, want.astype(np.int64)), (dt, x.shape)
+
+
 # -------------------------------------------------------------- elemwise
 
 def test_elemwise_sum_cell_bit_exact(rt):
