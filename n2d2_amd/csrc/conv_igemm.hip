@@ -27,6 +27,7 @@
 namespace n2d2hip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct ConvArgs {
@@ -374,8 +375,11 @@ struct n2d2hip_conv_s {
     // residual sum folded into the epilogue (n2d2hip_conv_fuse_sum)
     n2d2hip_elemwise_t sum;
     int sum_other_dtype;  // storage type the tables below were made for
-    int* d_res_tab;       // sum a,b,c,d,e then pre a,b,c,d,e, each [cpad], zero point of the other input folded in
+    // sum a,b,c,d,e then pre a,b,c,d,e, each [cpad], zero point of the other input folded in; then the sum's c, d, e as
+    // 16-bit pairs, each [cpad / 2]
+    int* d_res_tab;
     bool has_pre, pre_clamp, sum_clamp;
+    bool sum16;           // the 16-bit pairs may be used: every intermediate behind the convolution's shift fits 16 bits
     // integer rescale with the bias folded in, for the pipelined kernel: a - bias, b - bias, c, d + bias * c, e, each [cpad]
     int* d_epi_tab;
     bool bias_folded;
@@ -436,7 +440,10 @@ void launch_pipe_res(ConvPipeArgs a, int grid, hipStream_t stream)
 {
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
-    hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+    if (a.sum16)
+        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+    else
+        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true, false>), dim3(grid), dim3(NW * 64), 0, stream, a);
 }
 
 // (multiplier, shift) with n / d == umulhi(n, multiplier) >> shift for 0 <= n < 2^31; multiplier 0 stands for d == 1
@@ -516,7 +523,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
     c->d_epi_tab = nullptr; c->bias_folded = false; c->d_wstem = nullptr;
-    c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = false;
+    c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
         delete c;
@@ -784,7 +791,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     const bool fits32 = (long long)in->B * in->H * in->W * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
     bool bn128_unused;
     const bool pipe = pipe_eligible(c, &bn128_unused) && fits32;
-    N2D2HIP_REQUIRE(!other || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward_sum: tensor too large for the fused kernel");
+    N2D2HIP_REQUIRE(!other || (pipe && Mll * out->cs < (1ll << 31)), N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward_sum: tensor too large for the fused kernel");
     if (pipe && (other || getenv("N2D2HIP_NO_PIPE") == nullptr)) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
         ConvPipeArgs q;
@@ -819,12 +827,15 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.xcd_tiles = (q.mtiles + 7) / 8;
         const int grid = 8 * a.ntiles_n * per_xcd;
         q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
+        q.sum16 = nullptr; q.sum16_stride = 0;
         q.sum = EpiArgs(); q.pre = EpiArgs();
         if (other) {
             const int cp = c->sum->act->cpad;
             q.res = (const signed char*)other->data;
             q.res_cs = other->cs;
-            q.res_flip = other->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
+            q.res_flip = other->dtype == N2D2HIP_U8 ? 0u : 0x80808080u;
+            q.sum16 = c->sum16 ? c->d_res_tab + 10 * cp : nullptr;
+            q.sum16_stride = cp / 2;
             q.sum = c->sum->act->args;
             q.sum.a = c->d_res_tab; q.sum.b = c->d_res_tab + cp; q.sum.c = c->d_res_tab + 2 * cp;
             q.sum.d = c->d_res_tab + 3 * cp; q.sum.e = c->d_res_tab + 4 * cp;
@@ -929,11 +940,15 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
                     "conv_fuse_sum: needs a 1x1 unpadded 8-bit convolution with a multiple of 64 input and output channels and integer "
                     "rescales on the convolution and on a two-input unit-coefficient sum");
     // Tables of the sum (and of the ScalingCell folded onto the other input) with the other input's zero point
-    // folded in: the kernel adds the stored byte as a signed value.
+    // folded in: the kernel turns the stored byte into an unsigned one (U8B and I8 bytes with their top bit flipped,
+    // which is the value itself for U8B and the value + 128 for I8) and adds that.
     const int cp = sa->cpad;
-    const long long zp = zero_point(other_dtype == N2D2HIP_U8 ? N2D2HIP_U8B : other_dtype);
+    const long long zp = other_dtype == N2D2HIP_I8 ? -128 : 0;
     const long long IMIN = std::numeric_limits<int>::min(), IMAX = std::numeric_limits<int>::max();
-    std::vector<int> t(10 * (size_t)cp, 0);
+    std::vector<int> t(12 * (size_t)cp, 0);
+    // The sum stage in 16-bit pairs needs: no clamp before a multiply anywhere, and (conv + other) * c + d inside 16 bits
+    bool sum16 = !c->preclamp && cp % 2 == 0 && getenv("N2D2HIP_NO_SUM16") == nullptr;
+    short* t16 = (short*)(t.data() + 10 * (size_t)cp);
     bool pre_clamp = pa ? pa->clipped : false, sum_clamp = sa->clipped;
     const long long other_lo = pa ? pa->min_out : (other_dtype == N2D2HIP_I8 ? -128 : 0);
     const long long other_hi = pa ? pa->max_out : (other_dtype == N2D2HIP_I8 ? 127 : 255);
@@ -952,6 +967,12 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
         if (smax * m + std::llabs(d2) > IMAX)
             sum_clamp = true;
         t[3 * (size_t)cp + ch] = (int)d2;
+        const long long e2 = sa->htab[4 * (size_t)cp + ch];
+        if (m < 0 || e2 < 0 || e2 > 15 || smax * m + std::llabs(d2) > 32767)
+            sum16 = false;
+        t16[ch] = (short)m;
+        t16[cp + ch] = (short)d2;
+        t16[2 * (size_t)cp + ch] = (short)e2;
         if (pa) {
             const long long xa = pa->htab[ch], xb = pa->htab[cp + ch], xm = pa->htab[2 * (size_t)cp + ch], xd = pa->htab[3 * (size_t)cp + ch];
             const long long xd2 = xd + zp * xm;
@@ -959,6 +980,9 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
                 pre_clamp = true;
             if (xd2 < IMIN || xd2 > IMAX)
                 return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_fuse_sum: the folded ScalingCell of channel %d leaves 32 bits", ch);
+            // 16-bit pairs: the stored byte (0..255) times a 24-bit unsigned multiplier, inside 32 bits with the addend
+            if (xm < 0 || xm >= (1 << 24) || 255 * xm + std::llabs(xd2) > IMAX)
+                sum16 = false;
             t[5 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xa - zp));
             t[6 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xb - zp));
             t[7 * (size_t)cp + ch] = (int)xm;
@@ -977,6 +1001,7 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
     c->has_pre = pa != nullptr;
     c->pre_clamp = pre_clamp;
     c->sum_clamp = sum_clamp;
+    c->sum16 = sum16 && !pre_clamp && !sum_clamp;
     return N2D2HIP_OK;
 }
 

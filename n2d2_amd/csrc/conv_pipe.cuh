@@ -44,6 +44,11 @@ __device__ __forceinline__ void lds_read128_nowait(v4i& v, unsigned addr)
 {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
 }
+template <int OFF>
+__device__ __forceinline__ void lds_read64_nowait(v2i& v, unsigned addr)
+{
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void wait_lgkm()
 {
@@ -51,6 +56,14 @@ __device__ __forceinline__ void wait_lgkm()
 }
 // Makes a register filled by an earlier asynchronous LDS read depend on the wait that precedes this call.
 __device__ __forceinline__ void tie(v4i& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void tie(v2i& x) { asm volatile("" : "+v"(x)); }
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ v2s as_v2s(int x) { return __builtin_bit_cast(v2s, x); }
+__device__ __forceinline__ v2s splat_v2s(int x) { return v2s{(short)x, (short)x}; }
+__device__ __forceinline__ v2s clamp_v2s(v2s x, v2s lo, v2s hi)
+{
+    return __builtin_elementwise_min(__builtin_elementwise_max(x, lo), hi);
+}
 template <int N>
 __device__ __forceinline__ void wait_loads_and_barrier()
 {
@@ -94,10 +107,14 @@ struct ConvPipeArgs {
     // Folded residual sum (RES kernels): out = sum_act(conv_act(conv) + pre(other)), all EPI_I24
     const signed char* res;      // the sum's other input, NHWC bytes
     int res_cs;
-    unsigned res_flip;           // 0x80808080 for plain U8 storage (turns it into value-128)
+    unsigned res_flip;           // turns a stored byte into an unsigned one (0x80808080 unless plain U8 storage)
     EpiArgs sum;                 // the sum cell's rescale; its d table has the other input's zero point folded in
     EpiArgs pre;                 // ScalingCell folded onto the other input (d table with the zero point folded in)
     int has_pre, pre_clamp, sum_clamp;
+    // The sum's multiplier, addend and shift as pairs of 16-bit values (channels 2k, 2k+1 in one dword), three arrays of
+    // sum16_stride dwords, when the host has shown that the sum's arithmetic stays inside 16 bits; else null.
+    const int* sum16;
+    int sum16_stride;
 #ifdef N2D2HIP_PROFILE
     long long* prof;             // 8 timestamps per block
 #endif
@@ -115,7 +132,8 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // BK: bytes of K per ring stage and row (64 or 128); 128 makes every row segment a whole 128-byte line, which is
 // what the L2 -> LDS path moves fastest.
 // RES: the residual sum that follows the convolution is computed in the epilogue (1x1 convolutions, EPI_I24).
-template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID, bool RES = false>
+// P16 (with RES): the sum's arithmetic runs on pairs of 16-bit values (the host has shown that it fits).
+template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID, bool RES = false, bool P16 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pipe_kernel(ConvPipeArgs q)
 {
     const ConvArgs& p = q.c;
@@ -133,7 +151,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int LPI = A_J + B_J;                     // loads per thread and step
     constexpr int STAGE = (BM + BN) * BK;
     constexpr int TAB_OFF = S * STAGE;                 // 6 int arrays of BN entries: bias, a, b, c, d, e
-    constexpr int NTAB = RES ? 16 : 6;                 // RES: + a..e of the sum cell, + a..e of the folded ScalingCell
+    // RES: + a..e of the sum cell, + a..e of the folded ScalingCell.  When the sum runs on 16-bit pairs, its c, d, e in
+    // that form take the place of the bias and the convolution's a, which that path does not use.
+    constexpr int NTAB = RES ? 16 : 6;
     static_assert(!RES || EPI == EPI_I24, "the folded sum is integer arithmetic");
     constexpr int NF = NI + NJ;                        // fragment reads per MFMA K step
     constexpr bool BIAS_REG = EPI != EPI_I24;          // the integer rescale carries the bias in its tables
@@ -269,6 +289,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     int r_stage = 0;
     const unsigned tab = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 4u;      // this lane's first channel in the tables
+    const unsigned tab16 = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 2u;    // and in the 16-bit pairs
+    constexpr bool p16 = RES && P16;
+    static_assert(RES || !P16, "16-bit pairs are for the folded sum");
 
     // two fragment sets: while the MFMAs of K step g run from set g%2, the reads of step g+1 fly into the other
     v4i fw[2][NI], fp[2][NJ];
@@ -291,6 +314,27 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     };
 
+    // RES: the other input's bytes for this lane's accumulators.  They are read the way the output is written, 32
+    // consecutive channels of a pixel per lane (whole 32-byte sectors, every line touched once), one tile ahead: the
+    // loads of tile t+1 are issued at the start of tile t's epilogue and have a whole epilogue and K loop to arrive.
+    // Rows past the end read pixel 0, so the number of loads issued never depends on the data.
+    constexpr int NST = 2 * NJ;                        // RES: stores per thread and tile
+    static_assert(!RES || (S * LPI >= NST && NST + LPI < 60), "enough younger operations behind the first tile's residual loads");
+    v4i rfirst[RES ? NJ : 1], rsecond[RES ? NJ : 1];
+    auto issue_res = [&](int c_tile) {
+        const int m0 = (mlane + c_tile * q.mlanes) * BM;
+#pragma unroll
+        for (int j = 0; j < (RES ? NJ : 0); ++j) {
+            const int m = m0 + wm * TM + j * 32 + l32;
+            const signed char* rp = q.res + (long long)(m < p.M ? m : 0) * q.res_cs + (n0 + wn * TN + 32 * lh);
+            asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
+                         : "=&v"(rfirst[j]), "=&v"(rsecond[j]) : "v"(rp) : "memory");
+        }
+    };
+    // RES: the output goes through a buffer descriptor whose bounds check drops the rows past the end, so that every
+    // thread issues the same number of stores
+    __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, RES ? p.M * p.out_cs : 0, 0x00020000);
+
     v16i acc[NI][NJ];
     const bool out_bytes = p.out_dtype != N2D2HIP_I32;
     const int vlo = p.epi.lo, vhi = p.epi.hi;
@@ -301,30 +345,21 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     auto epilogue = [&](int c_tile) {
         const int m0 = (mlane + c_tile * q.mlanes) * BM;
         unsigned pk[NI][NJ][4];
-        // RES: the other input's bytes for this lane's accumulators, 4 channels per dword.  They are read the way the
-        // output is written, 32 consecutive channels of a pixel per lane (whole 32-byte sectors, every line touched
-        // once), and brought into the accumulators' layout by running the output's lane-half exchanges backwards
-        // (the exchange is its own inverse).  These loads are younger than every load of the ring, so waiting for
-        // them also waits for the stage in flight.
+        // RES: the other input's bytes, 4 channels per dword, are brought into the accumulators' layout by running the
+        // output's lane-half exchanges backwards (the exchange is its own inverse).  Memory operations complete in
+        // issue order: behind this tile's residual loads came the previous tile's NST stores and at least one step of
+        // ring loads (for the first tile, the ring's fill), so they have landed once no more than that is in flight.
         unsigned resw[RES ? NI * 4 : 1][RES ? NJ : 1];
         if (RES) {
             static_assert(!RES || NI == 2, "the folded sum is written for two channel tiles per wave");
-            v4i first[NJ], second[NJ];
+            asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NST + LPI) : "memory");
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                const int m = m0 + wm * TM + j * 32 + l32;
-                const signed char* rp = q.res + (long long)(m < p.M ? m : 0) * q.res_cs + (n0 + wn * TN + 32 * lh);
-                asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
-                             : "=&v"(first[j]), "=&v"(second[j]) : "v"(rp) : "memory");
-            }
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                tie(first[j]); tie(second[j]);
+                tie(rfirst[RES ? j : 0]); tie(rsecond[RES ? j : 0]);
                 unsigned qd[2][4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const auto y = __builtin_amdgcn_permlane32_swap((unsigned)first[j][e], (unsigned)second[j][e], false, false);
+                    const auto y = __builtin_amdgcn_permlane32_swap((unsigned)rfirst[RES ? j : 0][e], (unsigned)rsecond[RES ? j : 0][e], false, false);
                     qd[0][e] = y[0]; qd[1][e] = y[1];
                 }
 #pragma unroll
@@ -337,6 +372,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     resw[RES ? i * 4 + 3 : 0][RES ? j : 0] = s13[1];
                 }
             }
+            issue_res(c_tile + 1);
         }
         // Without a folded sum, the convolution's tables of the next channel group are requested before this group is
         // rescaled (two register sets), so that their LDS latency is hidden behind the arithmetic.
@@ -357,6 +393,80 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
             for (int g = 0; g < 4; ++g) {
                 const int idx = i * 4 + g;
                 const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
+                if constexpr (RES && P16) {
+                    // ---- the same three rescales with everything behind the convolution's shift held as pairs of
+                    // 16-bit values (channels 2h, 2h+1 of the lane's four): half the instructions per value.  The host
+                    // has shown that no intermediate leaves 16 bits and that none of the optional clamps is needed.
+                    const unsigned trow16 = tab16 + (unsigned)(i * 32 + 8 * g) * 2u;
+                    v4i tc, td, te, xc, xd, xe;
+                    v2i c16, d16, e16;
+                    lds_read128_nowait<3 * BN * 4>(tc, trow);
+                    lds_read128_nowait<4 * BN * 4>(td, trow);
+                    lds_read128_nowait<5 * BN * 4>(te, trow);
+                    // (the ScalingCell's tables are read whether there is one or not: three reads of whatever the LDS
+                    // holds cost less than a branch here)
+                    lds_read128_nowait<13 * BN * 4>(xc, trow);
+                    lds_read128_nowait<14 * BN * 4>(xd, trow);
+                    lds_read128_nowait<15 * BN * 4>(xe, trow);
+                    lds_read64_nowait<0>(c16, trow16);
+                    lds_read64_nowait<BN * 2>(d16, trow16);
+                    lds_read64_nowait<BN * 4>(e16, trow16);
+                    wait_lgkm<6>();
+                    tie(tc); tie(td); tie(te);
+                    const v2s lo1 = splat_v2s(vlo), hi1 = splat_v2s(vhi);
+                    v2s pq[NJ][2];
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int t0 = (__mul24(acc[i][j][4 * g + 2 * h], tc[2 * h]) + td[2 * h]) >> te[2 * h];
+                            const int t1 = (__mul24(acc[i][j][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1]) >> te[2 * h + 1];
+                            pq[j][h] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(t0, t1), lo1, hi1);
+                        }
+                    v2s oq[NJ][2];
+                    wait_lgkm<3>();
+                    tie(xc); tie(xd); tie(xe);
+                    if (q.has_pre) {
+                        const v2s lo3 = splat_v2s(plo), hi3 = splat_v2s(phi);
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) {
+                            const unsigned w = resw[RES ? idx : 0][RES ? j : 0] ^ q.res_flip;
+                            int u[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)
+                                u[t] = (int)(__umul24((w >> (8 * t)) & 0xffu, (unsigned)xc[t]) + (unsigned)xd[t]) >> xe[t];
+                            oq[j][0] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(u[0], u[1]), lo3, hi3);
+                            oq[j][1] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(u[2], u[3]), lo3, hi3);
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j) {
+                            const unsigned w = resw[RES ? idx : 0][RES ? j : 0] ^ q.res_flip;
+                            oq[j][0] = as_v2s((int)__builtin_amdgcn_perm(w, w, 0x0c010c00u));
+                            oq[j][1] = as_v2s((int)__builtin_amdgcn_perm(w, w, 0x0c030c02u));
+                        }
+                    }
+                    wait_lgkm<0>();
+                    tie(c16); tie(d16); tie(e16);
+                    const v2s lo2 = splat_v2s(slo), hi2 = splat_v2s(shi);
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            v2s v = pq[j][h] + oq[j][h];
+                            v = v * as_v2s(c16[h]) + as_v2s(d16[h]);
+                            v = v >> as_v2s(e16[h]);
+                            pq[j][h] = clamp_v2s(v, lo2, hi2);
+                        }
+                        pk[i][j][g] = __builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, pq[j][1]), (unsigned)__builtin_bit_cast(int, pq[j][0]),
+                                                            0x06040200u) ^ p.out_xor;
+                    }
+                    // Keeps the groups apart (their results are needed only after the last one, and the compiler would
+                    // otherwise compute them all there, with every group's tables live at once).
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+                        asm volatile("" : "+v"(pk[i][j][g]));
+                } else {
                 int r[NJ][4];
                 // RES: every table of the group is requested at once (LDS answers in order); each phase then waits only
                 // for its own, so one LDS latency is paid per group instead of three
@@ -436,10 +546,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) {
                         const unsigned w = resw[RES ? idx : 0][RES ? j : 0] ^ q.res_flip;
-                        o[j][0] = (int)(signed char)(w & 0xffu);
-                        o[j][1] = (int)(signed char)((w >> 8) & 0xffu);
-                        o[j][2] = (int)(signed char)((w >> 16) & 0xffu);
-                        o[j][3] = (int)w >> 24;
+                        o[j][0] = (int)(w & 0xffu);
+                        o[j][1] = (int)((w >> 8) & 0xffu);
+                        o[j][2] = (int)((w >> 16) & 0xffu);
+                        o[j][3] = (int)(w >> 24);
                     }
                     if (q.has_pre) {
                         wait_lgkm<5>();
@@ -488,6 +598,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                             *(int4*)((int*)p.out + (long long)m * p.out_cs + ch) = int4{r[j][0], r[j][1], r[j][2], r[j][3]};
                     }
                 }
+                }
             }
         }
         if (!out_bytes)
@@ -515,7 +626,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     second[e] = (int)x[1];
                 }
                 const int ch = n0 + wn * TN + 32 * lh;
-                if (m < p.M) {
+                if (RES) {
+                    const unsigned off = m < p.M ? (unsigned)(m * p.out_cs + ch) : 0x80000000u;
+                    __builtin_amdgcn_raw_buffer_store_b128(first, out_rsrc, off, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(second, out_rsrc, off + 16u, 0, 0);
+                } else if (m < p.M) {
                     if (ch < p.out_cs) *(v4i*)(orow + 32 * lh) = first;
                     if (ch + 16 < p.out_cs) *(v4i*)(orow + 32 * lh + 16) = second;
                 }
@@ -532,6 +647,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #ifdef N2D2HIP_PROFILE
     pr_t1 = clock64();
 #endif
+    if (RES)
+        issue_res(0);
 #pragma unroll
     for (int s = 0; s < S; ++s)
         issue();
@@ -540,9 +657,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     {
         int* tabw = (int*)(smem + TAB_OFF);
         for (int i = tid; i < BN; i += NT) {
-            tabw[i] = BIAS_REG ? p.bias[n0 + i] : 0;
+            if (!p16)
+                tabw[i] = BIAS_REG ? p.bias[n0 + i] : 0;
             if (EPI != EPI_RAW) {
-                tabw[BN + i] = p.epi.a[n0 + i];
+                if (!p16)
+                    tabw[BN + i] = p.epi.a[n0 + i];
                 tabw[2 * BN + i] = p.epi.b[n0 + i];
                 tabw[3 * BN + i] = p.epi.c[n0 + i];
                 tabw[4 * BN + i] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
@@ -554,6 +673,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 tabw[8 * BN + i] = q.sum.c[n0 + i];
                 tabw[9 * BN + i] = q.sum.d[n0 + i];
                 tabw[10 * BN + i] = q.sum.e[n0 + i];
+                if (p16 && i < BN / 2) {
+                    tabw[i] = q.sum16[n0 / 2 + i];
+                    tabw[BN / 2 + i] = q.sum16[q.sum16_stride + n0 / 2 + i];
+                    tabw[BN + i] = q.sum16[2 * q.sum16_stride + n0 / 2 + i];
+                }
                 if (q.has_pre) {
                     tabw[11 * BN + i] = q.pre.a[n0 + i];
                     tabw[12 * BN + i] = q.pre.b[n0 + i];

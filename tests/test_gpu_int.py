@@ -1,5 +1,6 @@
 """GPU parity of the integer cells: every result is compared bit-for-bit with
 the CPU oracle on the same seeded inputs, calling through the C ABI."""
+import os
 import sys
 
 import numpy as np
@@ -405,7 +406,8 @@ def test_conv_with_folded_residual_sum(rt):
         y = cells_ref.conv_cell(x, w, bias, conv_spec, stride=(stride, stride))
         OH = y.shape[2]
         dx = rt.DTensor.from_numpy(x, capi.U8B)
-        for other_dtype, other in ((capi.U8B, rng.integers(0, 256, size=(B, O, OH, OH))), (capi.I8, rng.integers(-128, 128, size=(B, O, OH, OH)))):
+        for other_dtype, other in ((capi.U8B, rng.integers(0, 256, size=(B, O, OH, OH))), (capi.I8, rng.integers(-128, 128, size=(B, O, OH, OH))),
+                                   (capi.U8B, rng.choice([0, 1, 254, 255], size=(B, O, OH, OH))), (capi.I8, rng.choice([-128, -1, 0, 127], size=(B, O, OH, OH)))):
             dother = rt.DTensor.from_numpy(other, other_dtype)
             for pre_mode in (None, "FixedMult16", "SingleShift"):
                 if pre_mode == "FixedMult16":
@@ -425,11 +427,16 @@ def test_conv_with_folded_residual_sum(rt):
                     if pre_spec is not None:
                         pre = rt.Act(O, **pre_spec.kwargs())
                         assert ew.fold_input_scaling(1 - k, pre)
-                    assert conv.fuse_sum(ew, k, other_dtype), (C, O)
-                    out = rt.DTensor(B, O, OH, OH, capi.U8B)
-                    conv.forward_sum(dx, dother, out)
-                    got = out.to_numpy()
-                    assert np.array_equal(got, want), (C, O, H, stride, other_dtype, pre_mode, k, np.count_nonzero(got != want))
+                    # twice: with the sum's arithmetic on 16-bit pairs where the tables allow it, and on 32 bits
+                    for no16 in ("", "1"):
+                        if no16:
+                            os.environ["N2D2HIP_NO_SUM16"] = no16
+                        assert conv.fuse_sum(ew, k, other_dtype), (C, O)
+                        os.environ.pop("N2D2HIP_NO_SUM16", None)
+                        out = rt.DTensor(B, O, OH, OH, capi.U8B)
+                        conv.forward_sum(dx, dother, out)
+                        got = out.to_numpy()
+                        assert np.array_equal(got, want), (C, O, H, stride, other_dtype, pre_mode, k, no16, np.count_nonzero(got != want))
                     # the plain convolution is still available on the same handle
                     assert np.array_equal(conv.forward(dx).to_numpy(), y.astype(np.int64))
     # what cannot be folded is reported, and the cells then run separately
