@@ -380,9 +380,13 @@ struct n2d2hip_conv_s {
     int* d_res_tab;
     bool has_pre, pre_clamp, sum_clamp;
     bool sum16;           // the 16-bit pairs may be used: every intermediate behind the convolution's shift fits 16 bits
+    bool pre_in_range;    // the folded ScalingCell maps every byte into its output range
     // integer rescale with the bias folded in, for the pipelined kernel: a - bias, b - bias, c, d + bias * c, e, each [cpad]
+    // ... then, when hi16: c << (16 - e) and (d + bias * c) << (16 - e), which leave the rescaled value in the upper half
+    // of the 32-bit result
     int* d_epi_tab;
     bool bias_folded;
+    bool hi16;
     // first-layer kernel (<= 4 input channels, horizontal stride 2): weights as [channel][kH * 32]
     signed char* d_wstem;
     bool is_fc;
@@ -522,7 +526,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->d_wstem = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -554,6 +558,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     }
     // Can the rescale multiply raw accumulators?  |sum| <= 128 * sum|w| + |folded bias| for byte inputs.
     c->preclamp = act->clipped;
+    std::vector<long long> acc_bound((size_t)act->cpad, 0);
     if (act->args.kind == EPI_I24 && !c->preclamp) {
         const int cp = act->cpad;
         for (int o = 0; o < d->O && !c->preclamp; ++o) {
@@ -561,6 +566,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             for (long long i = 0; i < wstrideO; ++i)
                 s += std::abs(read_weight(weights, o * wstrideO + i, d->weight_bits));
             const long long bound = 128 * s + std::llabs((long long)hbias[o]);
+            acc_bound[o] = bound;
             const long long mult = act->htab[2 * (size_t)cp + o], half = act->htab[3 * (size_t)cp + o];
             if (bound >= (1ll << 23) || bound * mult + half > std::numeric_limits<int>::max())
                 c->preclamp = true;
@@ -574,8 +580,9 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     std::vector<int> hepi;
     if (act->args.kind == EPI_I24 && !depthwise) {
         const int cp = act->cpad;
-        hepi.assign(5 * (size_t)cp, 0);
+        hepi.assign(7 * (size_t)cp, 0);
         c->bias_folded = true;
+        c->hi16 = !c->preclamp;
         for (int ch = 0; ch < cp; ++ch) {
             const long long b = hbias[ch];
             const long long lo = (long long)act->htab[ch] - b, hi = (long long)act->htab[cp + ch] - b;
@@ -587,6 +594,16 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             hepi[2 * (size_t)cp + ch] = (int)m;
             hepi[3 * (size_t)cp + ch] = (int)(unsigned)(unsigned long long)((long long)act->htab[3 * (size_t)cp + ch] + b * m);
             hepi[4 * (size_t)cp + ch] = act->htab[4 * (size_t)cp + ch];
+            // the same rescale scaled up by 2^(16 - e), if that still fits: |v| * m + half bounds the unscaled value
+            const long long e16 = act->htab[4 * (size_t)cp + ch], half = act->htab[3 * (size_t)cp + ch];
+            const long long up = (e16 >= 0 && e16 <= 16) ? (1ll << (16 - e16)) : 0;
+            if (up == 0 || std::llabs(m) * up >= (1ll << 23)
+                || (acc_bound[ch] * std::llabs(m) + std::llabs(half)) * up > std::numeric_limits<int>::max()) {
+                c->hi16 = false;
+            } else {
+                hepi[5 * (size_t)cp + ch] = (int)(m * up);
+                hepi[6 * (size_t)cp + ch] = (int)(unsigned)(unsigned long long)((half + b * m) * up);
+            }
         }
     }
 
@@ -827,7 +844,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.xcd_tiles = (q.mtiles + 7) / 8;
         const int grid = 8 * a.ntiles_n * per_xcd;
         q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
-        q.sum16 = nullptr; q.sum16_stride = 0;
+        q.sum16 = nullptr; q.sum16_stride = 0; q.pre_in_range = 0;
         q.sum = EpiArgs(); q.pre = EpiArgs();
         if (other) {
             const int cp = c->sum->act->cpad;
@@ -836,6 +853,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.res_flip = other->dtype == N2D2HIP_U8 ? 0u : 0x80808080u;
             q.sum16 = c->sum16 ? c->d_res_tab + 10 * cp : nullptr;
             q.sum16_stride = cp / 2;
+            q.pre_in_range = c->pre_in_range ? 1 : 0;
             q.sum = c->sum->act->args;
             q.sum.a = c->d_res_tab; q.sum.b = c->d_res_tab + cp; q.sum.c = c->d_res_tab + 2 * cp;
             q.sum.d = c->d_res_tab + 3 * cp; q.sum.e = c->d_res_tab + 4 * cp;
@@ -844,7 +862,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
                 q.pre = c->sum->pre_act->args;
                 q.pre.a = c->d_res_tab + 5 * cp; q.pre.b = c->d_res_tab + 6 * cp; q.pre.c = c->d_res_tab + 7 * cp;
                 q.pre.d = c->d_res_tab + 8 * cp; q.pre.e = c->d_res_tab + 9 * cp;
+                if (c->sum16) { q.pre.c = c->d_res_tab + 12 * cp; q.pre.d = c->d_res_tab + 13 * cp; }
             }
+            if (c->sum16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
             if (small_m) {
                 launch_pipe_res<4, 128, 2, 1, 2, 3>(q, grid, stream);
             } else if (d.C % 128 == 0) {
@@ -945,11 +965,13 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
     const int cp = sa->cpad;
     const long long zp = other_dtype == N2D2HIP_I8 ? -128 : 0;
     const long long IMIN = std::numeric_limits<int>::min(), IMAX = std::numeric_limits<int>::max();
-    std::vector<int> t(12 * (size_t)cp, 0);
-    // The sum stage in 16-bit pairs needs: no clamp before a multiply anywhere, and (conv + other) * c + d inside 16 bits
-    bool sum16 = !c->preclamp && cp % 2 == 0 && getenv("N2D2HIP_NO_SUM16") == nullptr;
+    std::vector<int> t(14 * (size_t)cp, 0);
+    // The sum stage in 16-bit pairs needs: no clamp before a multiply anywhere, (conv + other) * c + d inside 16 bits, and
+    // the two rescales in front of it in the form that leaves their result in the upper half of a 32-bit register
+    bool sum16 = !c->preclamp && c->hi16 && cp % 2 == 0 && getenv("N2D2HIP_NO_SUM16") == nullptr;
     short* t16 = (short*)(t.data() + 10 * (size_t)cp);
     bool pre_clamp = pa ? pa->clipped : false, sum_clamp = sa->clipped;
+    bool pre_in_range = pa != nullptr;
     const long long other_lo = pa ? pa->min_out : (other_dtype == N2D2HIP_I8 ? -128 : 0);
     const long long other_hi = pa ? pa->max_out : (other_dtype == N2D2HIP_I8 ? 127 : 255);
     for (int ch = 0; ch < cp; ++ch) {
@@ -980,9 +1002,19 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
                 pre_clamp = true;
             if (xd2 < IMIN || xd2 > IMAX)
                 return fail(N2D2HIP_ERR_UNSUPPORTED, "conv_fuse_sum: the folded ScalingCell of channel %d leaves 32 bits", ch);
-            // 16-bit pairs: the stored byte (0..255) times a 24-bit unsigned multiplier, inside 32 bits with the addend
-            if (xm < 0 || xm >= (1 << 24) || 255 * xm + std::llabs(xd2) > IMAX)
+            // 16-bit pairs: the stored byte (0..255) times a 24-bit unsigned multiplier scaled up by 2^(16 - e), inside 32
+            // bits with the addend
+            const long long xe = pa->htab[4 * (size_t)cp + ch];
+            // a non-negative multiplier makes the rescale monotonic: its extremes are at the bytes 0 and 255
+            if (xm < 0 || xe < 0 || xe > 31 || (xd2 >> xe) < pa->min_out || ((255 * xm + xd2) >> xe) > pa->max_out)
+                pre_in_range = false;
+            const long long up = (xe >= 0 && xe <= 16) ? (1ll << (16 - xe)) : 0;
+            if (up == 0 || xm < 0 || xm * up >= (1 << 24) || (255 * xm + std::llabs(xd2)) * up > IMAX) {
                 sum16 = false;
+            } else {
+                t[12 * (size_t)cp + ch] = (int)(xm * up);
+                t[13 * (size_t)cp + ch] = (int)(xd2 * up);
+            }
             t[5 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xa - zp));
             t[6 * (size_t)cp + ch] = (int)std::min(IMAX, std::max(IMIN, xb - zp));
             t[7 * (size_t)cp + ch] = (int)xm;
@@ -1002,6 +1034,7 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
     c->pre_clamp = pre_clamp;
     c->sum_clamp = sum_clamp;
     c->sum16 = sum16 && !pre_clamp && !sum_clamp;
+    c->pre_in_range = pre_in_range;
     return N2D2HIP_OK;
 }
 

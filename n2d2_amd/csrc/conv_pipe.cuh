@@ -64,6 +64,13 @@ __device__ __forceinline__ v2s clamp_v2s(v2s x, v2s lo, v2s hi)
 {
     return __builtin_elementwise_min(__builtin_elementwise_max(x, lo), hi);
 }
+// two 16-bit values saturated to [0, 255], as the two low bytes of the result
+__device__ __forceinline__ unsigned sat_pk_u8(v2s x)
+{
+    unsigned r;
+    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(r) : "v"(x));
+    return r;
+}
 template <int N>
 __device__ __forceinline__ void wait_loads_and_barrier()
 {
@@ -115,6 +122,7 @@ struct ConvPipeArgs {
     // sum16_stride dwords, when the host has shown that the sum's arithmetic stays inside 16 bits; else null.
     const int* sum16;
     int sum16_stride;
+    int pre_in_range;            // with sum16: the ScalingCell's result cannot leave its range, no saturation needed
 #ifdef N2D2HIP_PROFILE
     long long* prof;             // 8 timestamps per block
 #endif
@@ -398,45 +406,52 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     // 16-bit values (channels 2h, 2h+1 of the lane's four): half the instructions per value.  The host
                     // has shown that no intermediate leaves 16 bits and that none of the optional clamps is needed.
                     const unsigned trow16 = tab16 + (unsigned)(i * 32 + 8 * g) * 2u;
-                    v4i tc, td, te, xc, xd, xe;
+                    // The convolution's and the ScalingCell's multipliers and addends come scaled up by 2^(16 - shift):
+                    // the rescaled value is the upper half of the 32-bit result and needs no shift of its own.
+                    v4i tc, td, xc, xd;
                     v2i c16, d16, e16;
                     lds_read128_nowait<3 * BN * 4>(tc, trow);
                     lds_read128_nowait<4 * BN * 4>(td, trow);
-                    lds_read128_nowait<5 * BN * 4>(te, trow);
-                    // (the ScalingCell's tables are read whether there is one or not: three reads of whatever the LDS
+                    // (the ScalingCell's tables are read whether there is one or not: two reads of whatever the LDS
                     // holds cost less than a branch here)
                     lds_read128_nowait<13 * BN * 4>(xc, trow);
                     lds_read128_nowait<14 * BN * 4>(xd, trow);
-                    lds_read128_nowait<15 * BN * 4>(xe, trow);
                     lds_read64_nowait<0>(c16, trow16);
                     lds_read64_nowait<BN * 2>(d16, trow16);
                     lds_read64_nowait<BN * 4>(e16, trow16);
-                    wait_lgkm<6>();
-                    tie(tc); tie(td); tie(te);
+                    wait_lgkm<5>();
+                    tie(tc); tie(td);
                     const v2s lo1 = splat_v2s(vlo), hi1 = splat_v2s(vhi);
                     v2s pq[NJ][2];
 #pragma unroll
                     for (int j = 0; j < NJ; ++j)
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
-                            const int t0 = (__mul24(acc[i][j][4 * g + 2 * h], tc[2 * h]) + td[2 * h]) >> te[2 * h];
-                            const int t1 = (__mul24(acc[i][j][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1]) >> te[2 * h + 1];
-                            pq[j][h] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(t0, t1), lo1, hi1);
+                            const int t0 = __mul24(acc[i][j][4 * g + 2 * h], tc[2 * h]) + td[2 * h];
+                            const int t1 = __mul24(acc[i][j][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
+                            pq[j][h] = clamp_v2s(as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u)), lo1, hi1);
                         }
                     v2s oq[NJ][2];
                     wait_lgkm<3>();
-                    tie(xc); tie(xd); tie(xe);
+                    tie(xc); tie(xd);
                     if (q.has_pre) {
                         const v2s lo3 = splat_v2s(plo), hi3 = splat_v2s(phi);
 #pragma unroll
                         for (int j = 0; j < NJ; ++j) {
                             const unsigned w = resw[RES ? idx : 0][RES ? j : 0] ^ q.res_flip;
-                            int u[4];
+                            unsigned u[4];
 #pragma unroll
                             for (int t = 0; t < 4; ++t)
-                                u[t] = (int)(__umul24((w >> (8 * t)) & 0xffu, (unsigned)xc[t]) + (unsigned)xd[t]) >> xe[t];
-                            oq[j][0] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(u[0], u[1]), lo3, hi3);
-                            oq[j][1] = clamp_v2s(__builtin_amdgcn_cvt_pk_i16(u[2], u[3]), lo3, hi3);
+                                u[t] = __umul24((w >> (8 * t)) & 0xffu, (unsigned)xc[t]) + (unsigned)xd[t];
+                            oq[j][0] = as_v2s((int)__builtin_amdgcn_perm(u[1], u[0], 0x07060302u));
+                            oq[j][1] = as_v2s((int)__builtin_amdgcn_perm(u[3], u[2], 0x07060302u));
+                        }
+                        if (!q.pre_in_range) {
+#pragma unroll
+                            for (int j = 0; j < NJ; ++j) {
+                                oq[j][0] = clamp_v2s(oq[j][0], lo3, hi3);
+                                oq[j][1] = clamp_v2s(oq[j][1], lo3, hi3);
+                            }
                         }
                     } else {
 #pragma unroll
@@ -450,16 +465,23 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     tie(c16); tie(d16); tie(e16);
                     const v2s lo2 = splat_v2s(slo), hi2 = splat_v2s(shi);
 #pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
+                    for (int j = 0; j < NJ; ++j)
 #pragma unroll
                         for (int h = 0; h < 2; ++h) {
                             v2s v = pq[j][h] + oq[j][h];
                             v = v * as_v2s(c16[h]) + as_v2s(d16[h]);
-                            v = v >> as_v2s(e16[h]);
-                            pq[j][h] = clamp_v2s(v, lo2, hi2);
+                            pq[j][h] = v >> as_v2s(e16[h]);
                         }
-                        pk[i][j][g] = __builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, pq[j][1]), (unsigned)__builtin_bit_cast(int, pq[j][0]),
-                                                            0x06040200u) ^ p.out_xor;
+                    if (slo == 0 && shi == 255) {
+                        // the usual range of a rectified sum has an instruction of its own
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+                            pk[i][j][g] = (sat_pk_u8(pq[j][0]) | (sat_pk_u8(pq[j][1]) << 16)) ^ p.out_xor;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+                            pk[i][j][g] = __builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, clamp_v2s(pq[j][1], lo2, hi2)),
+                                                                (unsigned)__builtin_bit_cast(int, clamp_v2s(pq[j][0], lo2, hi2)), 0x06040200u) ^ p.out_xor;
                     }
                     // Keeps the groups apart (their results are needed only after the last one, and the compiler would
                     // otherwise compute them all there, with every group's tables live at once).
