@@ -19,7 +19,7 @@ PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # HBM bytes one conv_pipe_kernel launch of this workload moves on average: rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy), summary under profiles/
-PIPE_TRAFFIC_BYTES_PER_LAUNCH = (38.53 + 23.76) * 1048576.0
+PIPE_TRAFFIC_BYTES_PER_LAUNCH = (41.20 + 23.76) * 1048576
 
 
 def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
@@ -140,6 +140,30 @@ def main():
     roofline_hbm = {"bound": "hbm", "kernel": "whole forward (%d launches)" % len(net.launched), "achieved": round(hbm, 1),
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(hbm / PEAK_HBM_GBS, 4), "bytes_per_step": all_bytes}
 
+    # Per-class view: every launch timed with its own pair of events (median of 7 forwards), put against the larger of
+    # its two bounds (2*MAC at the int8 MFMA peak, algorithmic bytes at the HBM peak).  The per-launch events add about
+    # 10 % to the sum, so the class times are an upper estimate of their share of `ms_per_step`.
+    runs = [net.forward_timed() for _ in range(7)]
+    per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
+    classes = {}
+    floor_ms = 0.0
+    for l, t in zip(net.launched, per_launch):
+        ops, nbytes = 2.0 * net.layer_macs(l), float(net.layer_bytes(l))
+        t_mfma, t_hbm = ops / (PEAK_INT8_TOPS * 1e12) * 1e3, nbytes / (PEAK_HBM_GBS * 1e9) * 1e3
+        floor_ms += max(t_mfma, t_hbm)
+        c = classes.setdefault("mfma_bound" if t_mfma > t_hbm else "hbm_bound", {"launches": 0, "ms": 0.0, "ops": 0.0, "bytes": 0.0})
+        c["launches"] += 1; c["ms"] += t; c["ops"] += ops; c["bytes"] += nbytes
+    by_class = {}
+    for name, c in classes.items():
+        if name == "mfma_bound":
+            ach, peak, unit = c["ops"] / (c["ms"] * 1e-3) / 1e12, PEAK_INT8_TOPS, "TOP/s"
+        else:
+            ach, peak, unit = c["bytes"] / (c["ms"] * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        by_class[name] = {"launches": c["launches"], "ms": round(c["ms"], 4), "achieved": round(ach, 1), "peak": peak, "unit": unit,
+                          "frac": round(ach / peak, 4)}
+    by_class["floor_ms"] = round(floor_ms, 4)          # sum over launches of the larger bound
+    by_class["floor_frac"] = round(floor_ms / ms, 4)   # of the measured step
+
     result = {
         "metric": "int8 ResNet-50 images/sec @bs128 on 1 MI355X", "value": round(B / (ms * 1e-3), 1), "unit": "images/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
@@ -147,7 +171,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "resnet50_int8_ptq_forward_224", "global_batch": B, "input": "uint8 %dx3x224x224" % B,
                    "layers": len(spec.layers), "gmac_per_image": round(spec.macs_per_image() / 1e9, 3)},
-        "roofline": roofline, "roofline_hbm": roofline_hbm,
+        "roofline": roofline, "roofline_hbm": roofline_hbm, "roofline_by_class": by_class,
     }
     if not args.no_cpu_baseline:
         base, exact = cpu_baseline(spec, logits, images)

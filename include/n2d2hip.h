@@ -62,12 +62,22 @@ typedef struct n2d2hip_tensor {
     int layout; /* N2D2HIP_NCHW / N2D2HIP_NHWC */
     int B, C, H, W;
     int cs;     /* NHWC: bytes-per-pixel channel stride in elements (>= C); NCHW: ignored */
+    /* NHWC byte tensors between two convolutions may carry their padding physically: every image is stored as
+     * (H + 2*halo) x (W + 2*halo) pixels, `data` points at the first border pixel, and the border holds the storage form
+     * of the value 0 (n2d2hip_tensor_clear writes it; nothing writes there afterwards).  A convolution whose padding is
+     * not larger than the halo then reads every tap of every window from memory, which is what the reference's tap-skipping
+     * loop computes (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83: a skipped tap adds nothing, as a tap on a zero does).
+     * 0 everywhere else; only the entry points that say so accept a halo. */
+    int halo;
 } n2d2hip_tensor;
 
 /* Channel stride the library uses for an NHWC tensor with C channels. */
 int n2d2hip_nhwc_cs(int C);
-/* Bytes needed for a tensor (uses cs for NHWC). */
+/* Bytes needed for a tensor (uses cs for NHWC, and the halo). */
 size_t n2d2hip_tensor_bytes(const n2d2hip_tensor* t);
+/* Fills the whole buffer of a byte tensor, halo included, with the storage form of the value 0 (a kernel launch, no memset:
+ * it can be captured).  To be called once on a tensor with a halo before its producer first runs. */
+int n2d2hip_tensor_clear(const n2d2hip_tensor* t, n2d2hip_stream_t stream);
 
 /* Graph-edge conversion between any two dtype/layout combinations of the same
  * logical shape (e.g. F32 NCHW <-> U8B NHWC).  Values that do not fit the
@@ -145,9 +155,13 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* desc, const void* weights, cons
 int n2d2hip_conv_destroy(n2d2hip_conv_t conv);
 /* Output spatial size (ref: src/Cell/ConvCell.cpp:1169-1195). */
 int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH, int* outW);
-/* in / out: NHWC.  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE). */
+/* in / out: NHWC.  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE).  `in` and a byte `out` may have a halo if
+ * n2d2hip_conv_accepts_halo says so. */
 int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
+/* 1 if this convolution runs on the kernel that reads and writes tensors with a halo (8-bit weights, ungrouped, input
+ * channels a multiple of 64), else 0.  No counterpart in the reference, whose padding is implicit in its tap loop. */
+int n2d2hip_conv_accepts_halo(n2d2hip_conv_t conv);
 
 
 /* -------------------------------------------------------------------- fc */

@@ -22,9 +22,9 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOT_QUANTIZED, ERR_WORKSPACE = ra
 
 # every symbol include/n2d2hip.h declares
 SYMBOLS = [
-    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes",
+    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
-    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward",
+    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_accepts_halo",
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
@@ -36,7 +36,7 @@ SYMBOLS = [
 
 class Tensor(C.Structure):
     _fields_ = [("data", C.c_void_p), ("dtype", C.c_int), ("layout", C.c_int),
-                ("B", C.c_int), ("C", C.c_int), ("H", C.c_int), ("W", C.c_int), ("cs", C.c_int)]
+                ("B", C.c_int), ("C", C.c_int), ("H", C.c_int), ("W", C.c_int), ("cs", C.c_int), ("halo", C.c_int)]
 
 
 class Activation(C.Structure):
@@ -81,6 +81,8 @@ def load():
     lib.n2d2hip_conv_destroy.argtypes = [P]
     lib.n2d2hip_conv_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_conv_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_conv_accepts_halo.argtypes = [P]
+    lib.n2d2hip_tensor_clear.argtypes = [P, P]
     lib.n2d2hip_conv_fuse_sum.argtypes = [P, P, I, I]
     lib.n2d2hip_conv_forward_sum.argtypes = [P, P, P, P, P]
     lib.n2d2hip_fc_create.argtypes = [I, I, I, I, I, P, P, P, I, P]

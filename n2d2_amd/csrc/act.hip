@@ -21,7 +21,7 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
-int check_tensor(const n2d2hip_tensor* t, const char* what)
+int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok)
 {
     N2D2HIP_REQUIRE(t != nullptr, N2D2HIP_ERR_INVALID, "%s: null tensor descriptor", what);
     N2D2HIP_REQUIRE(t->data != nullptr, N2D2HIP_ERR_INVALID, "%s: null data pointer", what);
@@ -32,6 +32,12 @@ int check_tensor(const n2d2hip_tensor* t, const char* what)
     if (t->layout == N2D2HIP_NHWC)
         N2D2HIP_REQUIRE(t->cs >= t->C && (t->cs % 16 == 0 || t->cs == 4), N2D2HIP_ERR_INVALID,
                         "%s: NHWC channel stride %d invalid for %d channels (multiple of 16, or 4)", what, t->cs, t->C);
+    N2D2HIP_REQUIRE(t->halo >= 0 && t->halo <= 16, N2D2HIP_ERR_INVALID, "%s: halo %d", what, t->halo);
+    if (t->halo > 0) {
+        N2D2HIP_REQUIRE(halo_ok, N2D2HIP_ERR_UNSUPPORTED, "%s: tensors with a halo are not accepted here", what);
+        N2D2HIP_REQUIRE(t->layout == N2D2HIP_NHWC && elem_size(t->dtype) == 1, N2D2HIP_ERR_INVALID,
+                        "%s: only NHWC byte tensors have a halo", what);
+    }
     return N2D2HIP_OK;
 }
 
@@ -45,7 +51,7 @@ static long long clamp_ll(__int128 v, long long lo, long long hi) { return v < l
 // One thread per element of the OUTPUT tensor.  Handles every dtype / layout
 // pair; used at graph edges and by the stand-alone ScalingCell.
 template <bool WITH_EPI>
-__global__ void elementwise_kernel(const void* __restrict__ in, int in_dtype, int in_layout, int in_cs,
+__global__ void elementwise_kernel(const void* __restrict__ in, int in_dtype, int in_layout, int in_cs, int in_halo,
                                    void* __restrict__ out, int out_dtype, int out_layout, int out_cs,
                                    int B, int C, int H, int W, EpiArgs epi)
 {
@@ -69,7 +75,7 @@ __global__ void elementwise_kernel(const void* __restrict__ in, int in_dtype, in
         int v = 0;
         if (c < C) {
             const size_t j = (in_layout == N2D2HIP_NHWC)
-                ? (((size_t)b * H + y) * W + x) * (size_t)in_cs + c
+                ? (((size_t)b * (H + 2 * in_halo) + y + in_halo) * (W + 2 * in_halo) + x + in_halo) * (size_t)in_cs + c
                 : (((size_t)b * C + c) * H + y) * (size_t)W + x;
             v = load_value(in, j, in_dtype);
             if (WITH_EPI)
@@ -108,7 +114,30 @@ size_t n2d2hip_tensor_bytes(const n2d2hip_tensor* t)
 {
     if (!t) return 0;
     const size_t c = (t->layout == N2D2HIP_NHWC) ? (size_t)t->cs : (size_t)t->C;
-    return (size_t)t->B * t->H * t->W * c * (size_t)elem_size(t->dtype);
+    return (size_t)t->B * (t->H + 2 * t->halo) * (t->W + 2 * t->halo) * c * (size_t)elem_size(t->dtype);
+}
+
+namespace n2d2hip {
+__global__ void fill_bytes_kernel(uint4* __restrict__ p, size_t n16, unsigned v)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        p[i] = uint4{v, v, v, v};
+}
+} // namespace n2d2hip
+
+int n2d2hip_tensor_clear(const n2d2hip_tensor* t, n2d2hip_stream_t stream)
+{
+    int rc;
+    if ((rc = check_tensor(t, "tensor_clear", true)))
+        return rc;
+    N2D2HIP_REQUIRE(t->layout == N2D2HIP_NHWC && elem_size(t->dtype) == 1 && t->cs % 16 == 0, N2D2HIP_ERR_UNSUPPORTED,
+                    "tensor_clear: NHWC byte tensors with a channel stride that is a multiple of 16");
+    const size_t n16 = n2d2hip_tensor_bytes(t) / 16;
+    const size_t blocks = std::min<size_t>((n16 + 255) / 256, 256 * 32);
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)std::max<size_t>(blocks, 1)), dim3(256), 0, (hipStream_t)stream, (uint4*)t->data, n16,
+                       t->dtype == N2D2HIP_U8B ? 0x80808080u : 0u);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
 }
 
 static int same_shape(const n2d2hip_tensor* a, const n2d2hip_tensor* b, const char* what)
@@ -128,12 +157,12 @@ static unsigned grid_for(size_t total, int block)
 int n2d2hip_convert(const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
     int rc;
-    if ((rc = check_tensor(in, "convert input")) || (rc = check_tensor(out, "convert output")) || (rc = same_shape(in, out, "convert")))
+    if ((rc = check_tensor(in, "convert input", true)) || (rc = check_tensor(out, "convert output")) || (rc = same_shape(in, out, "convert")))
         return rc;
     const size_t total = (size_t)out->B * out->H * out->W * (out->layout == N2D2HIP_NHWC ? out->cs : out->C);
     EpiArgs none = {};
     hipLaunchKernelGGL(elementwise_kernel<false>, dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
-                       in->data, in->dtype, in->layout, in->cs, out->data, out->dtype, out->layout, out->cs,
+                       in->data, in->dtype, in->layout, in->cs, in->halo, out->data, out->dtype, out->layout, out->cs,
                        out->B, out->C, out->H, out->W, none);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
@@ -315,7 +344,7 @@ int n2d2hip_scaling_forward(n2d2hip_act_t act, const n2d2hip_tensor* in, const n
         return run_scaling_nhwc(act, in, out, (hipStream_t)stream);
     const size_t total = (size_t)out->B * out->H * out->W * (out->layout == N2D2HIP_NHWC ? out->cs : out->C);
     hipLaunchKernelGGL(elementwise_kernel<true>, dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
-                       in->data, in->dtype, in->layout, in->cs, out->data, out->dtype, out->layout, out->cs,
+                       in->data, in->dtype, in->layout, in->cs, 0, out->data, out->dtype, out->layout, out->cs,
                        out->B, out->C, out->H, out->W, act->args);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;

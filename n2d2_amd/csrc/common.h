@@ -48,7 +48,7 @@ inline int round_up(int x, int m)
 {
     return (x + m - 1) / m * m;
 }
-int check_tensor(const n2d2hip_tensor* t, const char* what);
+int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok = false);
 
 // ---------------------------------------------------------------- epilogue
 // Device-side form of "Scaling::propagate, saturate, Rectifier/Linear" for one

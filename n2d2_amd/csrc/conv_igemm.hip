@@ -414,13 +414,14 @@ void launch_cfg(const ConvArgs& a, hipStream_t stream)
 }
 
 template <int NW, int BK, int NI, int NJ, int WGM, int S>
-void launch_pipe(ConvPipeArgs a, bool all_valid, int grid, hipStream_t stream)
+void launch_pipe(ConvPipeArgs a, int valid, int grid, hipStream_t stream)
 {
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
 #define N2D2HIP_PIPE(EPI) \
-    do { if (all_valid) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, true>), dim3(grid), dim3(NW * 64), 0, stream, a); \
-         else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, false>), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
+    do { if (valid == 1) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 1>), dim3(grid), dim3(NW * 64), 0, stream, a); \
+         else if (valid == 2) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 2>), dim3(grid), dim3(NW * 64), 0, stream, a); \
+         else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 0>), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
     switch (a.c.epi.kind) {
     case EPI_RAW: N2D2HIP_PIPE(EPI_RAW); break;
     case EPI_I24: N2D2HIP_PIPE(EPI_I24); break;
@@ -445,9 +446,9 @@ void launch_pipe_res(ConvPipeArgs a, int grid, hipStream_t stream)
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
     if (a.sum16)
-        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
     else
-        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, true, true, false>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, false>), dim3(grid), dim3(NW * 64), 0, stream, a);
 }
 
 // (multiplier, shift) with n / d == umulhi(n, multiplier) >> shift for 0 <= n < 2^31; multiplier 0 stands for d == 1
@@ -732,9 +733,13 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     hipStream_t stream = (hipStream_t)stream_;
     int rc;
     N2D2HIP_REQUIRE(c != nullptr, N2D2HIP_ERR_INVALID, "conv_forward: null conv");
-    if ((rc = check_tensor(in, "conv input")) || (rc = check_tensor(out, "conv output")))
+    if ((rc = check_tensor(in, "conv input", true)) || (rc = check_tensor(out, "conv output", true)))
         return rc;
     const n2d2hip_conv_desc& d = c->desc;
+    bool bn128_unused;
+    N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0)
+                        || (pipe_eligible(c, &bn128_unused) && getenv("N2D2HIP_NO_PIPE") == nullptr && d.dilX == 1 && d.dilY == 1),
+                    N2D2HIP_ERR_UNSUPPORTED, "conv_forward: this convolution does not take tensors with a halo (n2d2hip_conv_accepts_halo)");
     N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED,
                     "conv_forward: tensors must be NHWC (use n2d2hip_convert at graph edges)");
     N2D2HIP_REQUIRE(in->dtype == c->in_dtype, N2D2HIP_ERR_INVALID, "conv_forward: input dtype %d, conv created for %d", in->dtype, c->in_dtype);
@@ -767,8 +772,12 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: F32 outputs are produced with n2d2hip_convert");
     }
     const long long Mll = (long long)in->B * OH * OW;
-    N2D2HIP_REQUIRE(Mll < (1ll << 31) && (long long)in->B * in->H * in->W * in->cs < (1ll << 40), N2D2HIP_ERR_UNSUPPORTED,
-                    "conv_forward: tensor too large");
+    // An input with a halo is a larger input with less padding: the kernels see its physical size
+    const int Hp = in->H + 2 * in->halo, Wp = in->W + 2 * in->halo;
+    const int padL = d.padL - in->halo, padT = d.padT - in->halo, padR = d.padR - in->halo, padB = d.padB - in->halo;
+    const long long out_pixels = (long long)in->B * (OH + 2 * out->halo) * (OW + 2 * out->halo);
+    N2D2HIP_REQUIRE(Mll < (1ll << 31) && out_pixels < (1ll << 31) && (long long)in->B * Hp * Wp * in->cs < (1ll << 40),
+                    N2D2HIP_ERR_UNSUPPORTED, "conv_forward: tensor too large");
     const unsigned out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
 
     if (c->depthwise) {
@@ -784,11 +793,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
 
     ConvArgs a;
     a.in = (const signed char*)in->data;
-    a.in_cs = in->cs; a.B = in->B; a.H = in->H; a.W = in->W;
+    a.in_cs = in->cs; a.B = in->B; a.H = Hp; a.W = Wp;
     a.OH = OH; a.OW = OW; a.M = (int)Mll;
     a.w = c->d_w; a.ktot = c->ktot; a.niter = c->ktot / 64; a.sub = c->d_sub; a.bias = c->d_bias;
     a.out = out->data; a.out_cs = out->cs; a.out_dtype = out->dtype;
-    a.strideX = d.strideX; a.strideY = d.strideY; a.padL = d.padL; a.padT = d.padT; a.dilX = d.dilX; a.dilY = d.dilY;
+    a.strideX = d.strideX; a.strideY = d.strideY; a.padL = padL; a.padT = padT; a.dilX = d.dilX; a.dilY = d.dilY;
     a.kW = d.kW; a.kH = d.kH;
     a.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
     a.out_xor = out_xor;
@@ -805,11 +814,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     const bool bm64 = bn128 && !c->pix4 && blocks128 < 512;
     const int BM = bm64 ? 64 : 128;
     a.nblocks = (int)(((Mll + BM - 1) / BM) * a.ntiles_n);
-    const bool fits32 = (long long)in->B * in->H * in->W * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
-    bool bn128_unused;
+    const bool fits32 = (long long)in->B * Hp * Wp * in->cs < (1ll << 31) && (long long)c->opad * c->ktot < (1ll << 31);
     const bool pipe = pipe_eligible(c, &bn128_unused) && fits32;
-    N2D2HIP_REQUIRE(!other || (pipe && Mll * out->cs < (1ll << 31)), N2D2HIP_ERR_UNSUPPORTED,
+    N2D2HIP_REQUIRE(!other || (pipe && out_pixels * out->cs < (1ll << 31)), N2D2HIP_ERR_UNSUPPORTED,
                     "conv_forward_sum: tensor too large for the fused kernel");
+    N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0) || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: tensor with a halo too large");
     if (pipe && (other || getenv("N2D2HIP_NO_PIPE") == nullptr)) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
         ConvPipeArgs q;
@@ -828,7 +837,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
 #endif
         magic_div((unsigned)(OH * OW), &q.ohw_mul, &q.ohw_sh);
         magic_div((unsigned)OW, &q.ow_mul, &q.ow_sh);
-        const bool all_valid = d.kW == 1 && d.kH == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0;
+        // no padding: every tap of every window reads inside the input (also a dilated kernel's, whose hand-unrolled
+        // special case in the reference needs a window cut to 3 taps by the input's edge, which cannot happen then)
+        const int all_valid = (padL <= 0 && padT <= 0 && padR <= 0 && padB <= 0) ? (d.kW * d.kH > 1 ? 2 : 1) : 0;
+        q.out_halo = out->halo;
+        q.out_pixels = (int)out_pixels;
         // Two independent 4-wave blocks per CU, 128 pixels x 128 (or 64) channels each: one block's epilogue and
         // barrier waits overlap the other's MFMAs.  K advances by whole 128-byte lines when the channel count allows.
         // Layers with few pixels (deep stages) take 64-pixel tiles so that every CU still gets its two blocks.
@@ -934,6 +947,12 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
 int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
     return conv_forward_impl(c, in, nullptr, out, stream);
+}
+
+int n2d2hip_conv_accepts_halo(n2d2hip_conv_t c)
+{
+    bool bn128;
+    return c && pipe_eligible(c, &bn128) && c->desc.dilX == 1 && c->desc.dilY == 1 && getenv("N2D2HIP_NO_PIPE") == nullptr ? 1 : 0;
 }
 
 int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype)

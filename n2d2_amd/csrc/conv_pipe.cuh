@@ -111,6 +111,8 @@ struct ConvPipeArgs {
     int kW, kH;
     unsigned ohw_mul, ohw_sh, ow_mul, ow_sh;     // division by OH*OW and by OW
     int preclamp;                // I24: clamp before the multiply; F32: the cell has a Clip
+    int out_halo;                // border pixels around every output image (byte outputs only)
+    int out_pixels;              // pixels of the output buffer, borders included
     // Folded residual sum (RES kernels): out = sum_act(conv_act(conv) + pre(other)), all EPI_I24
     const signed char* res;      // the sum's other input, NHWC bytes
     int res_cs;
@@ -141,7 +143,9 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // what the L2 -> LDS path moves fastest.
 // RES: the residual sum that follows the convolution is computed in the epilogue (1x1 convolutions, EPI_I24).
 // P16 (with RES): the sum's arithmetic runs on pairs of 16-bit values (the host has shown that it fits).
-template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, bool ALLVALID, bool RES = false, bool P16 = false>
+// VALID: 0 = windows may reach outside the input (per-tap validity bits), 1 = 1x1 kernel without padding, 2 = any kernel
+// without padding (every tap of every window inside the input: a tap only moves the uniform base address).
+template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, int VALID, bool RES = false, bool P16 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pipe_kernel(ConvPipeArgs q)
 {
     const ConvArgs& p = q.c;
@@ -210,6 +214,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     int l_c = 0, l_kx = 0, l_ky = 0, l_tap = 0, l_tapoff = 0, l_ctapoff = 0;
     const bool dilated = p.dilX != 1 || p.dilY != 1;
     const int dil_kw = q.kW + (p.dilX - 1) * (q.kW - 1), dil_kh = q.kH + (p.dilY - 1) * (q.kH - 1);
+    constexpr bool ALLVALID = VALID != 0;
+    constexpr bool kxk = VALID == 2;
     auto loader_new_tile = [&]() {
         const int m0 = (mlane + l_tile * q.mlanes) * BM;
 #pragma unroll
@@ -251,7 +257,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     auto issue = [&]() {
         unsigned char* sbase = smem + l_stage * STAGE;
         if (ALLVALID) {
-            const signed char* ibase = p.in + l_koff;        // uniform; rows past the end read pixel 0
+            // uniform; rows past the end read pixel 0.  Without padding every tap of every window lies inside the
+            // input, whatever the kernel size: a tap only moves the uniform base.
+            const signed char* ibase = p.in + (kxk ? l_tapoff : l_koff);
 #pragma unroll
             for (int j = 0; j < A_J; ++j)
                 __builtin_amdgcn_global_load_lds((gbl_ptr_t)(ibase + (unsigned)rowoff[j]), (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
@@ -275,7 +283,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
             l_c = 0; l_kx = 0; l_ky = 0; l_tap = 0; l_tapoff = 0; l_ctapoff = 0;
             ++l_tile;
             loader_new_tile();
-        } else if (!ALLVALID) {
+        } else if (!ALLVALID || kxk) {
             l_tapoff += BK;
             l_ctapoff += BK;
             if (++l_c == q.cper) {
@@ -341,7 +349,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     };
     // RES: the output goes through a buffer descriptor whose bounds check drops the rows past the end, so that every
     // thread issues the same number of stores
-    __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, RES ? p.M * p.out_cs : 0, 0x00020000);
+    __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(p.out, 0, RES ? q.out_pixels * p.out_cs : 0, 0x00020000);
+    // Position of output pixel m in the output buffer: m itself, or past the borders of a tensor with a halo
+    auto out_pix = [&](int m) -> int {
+        if (q.out_halo == 0)
+            return m;
+        const int mm = m < p.M ? m : 0;
+        const int b = div_magic(mm, q.ohw_mul, q.ohw_sh);
+        const int rem = mm - b * (p.OH * p.OW);
+        const int oy = div_magic(rem, q.ow_mul, q.ow_sh);
+        const int ox = rem - oy * p.OW;
+        return (b * (p.OH + 2 * q.out_halo) + oy + q.out_halo) * (p.OW + 2 * q.out_halo) + ox + q.out_halo;
+    };
 
     v16i acc[NI][NJ];
     const bool out_bytes = p.out_dtype != N2D2HIP_I32;
@@ -631,7 +650,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int m = m0 + wm * TM + j * 32 + l32;
-            signed char* orow = (signed char*)p.out + (long long)m * p.out_cs + (n0 + wn * TN);
+            const int mp = out_pix(m);
+            signed char* orow = (signed char*)p.out + (long long)mp * p.out_cs + (n0 + wn * TN);
             unsigned qd[NI][4];
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
@@ -649,7 +669,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 }
                 const int ch = n0 + wn * TN + 32 * lh;
                 if (RES) {
-                    const unsigned off = m < p.M ? (unsigned)(m * p.out_cs + ch) : 0x80000000u;
+                    const unsigned off = m < p.M ? (unsigned)(mp * p.out_cs + ch) : 0x80000000u;
                     __builtin_amdgcn_raw_buffer_store_b128(first, out_rsrc, off, 0, 0);
                     __builtin_amdgcn_raw_buffer_store_b128(second, out_rsrc, off + 16u, 0, 0);
                 } else if (m < p.M) {

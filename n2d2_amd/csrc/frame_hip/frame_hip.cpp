@@ -29,10 +29,11 @@ HipTensor::~HipTensor()
         (void)hipFree(mDesc.data);
 }
 
-void HipTensor::resize(int B, int C, int H, int W, int dtype)
+void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo)
 {
-    n2d2hip_tensor d;
+    n2d2hip_tensor d = {};
     d.data = nullptr;
+    d.halo = halo;
     d.dtype = dtype;
     d.layout = N2D2HIP_NHWC;
     d.B = B; d.C = C; d.H = H; d.W = W;
@@ -49,6 +50,10 @@ void HipTensor::resize(int B, int C, int H, int W, int dtype)
     }
     mDesc = d;
     mHostValid = false;
+    if (halo > 0) {
+        checkStatus(n2d2hip_tensor_clear(&mDesc, nullptr));
+        checkHip(hipStreamSynchronize(nullptr), "HipTensor::resize(): clearing the halo");
+    }
 }
 
 const Tensor<Float_T>& HipTensor::synchronizeDToH(void* stream)
@@ -60,6 +65,7 @@ const Tensor<Float_T>& HipTensor::synchronizeDToH(void* stream)
     n2d2hip_tensor f = mDesc;
     f.dtype = N2D2HIP_F32;
     f.layout = N2D2HIP_NCHW;
+    f.halo = 0;
     const size_t n = (size_t)f.B * f.C * f.H * f.W;
     checkHip(hipMalloc(&f.data, n * sizeof(float)), "HipTensor::synchronizeDToH(): hipMalloc");
     int rc = n2d2hip_convert(&mDesc, &f, stream);
@@ -83,6 +89,8 @@ void HipTensor::synchronizeHToD(const Tensor<Float_T>& host, void* stream)
         throw std::runtime_error("HipTensor::synchronizeHToD(): empty tensor");
     if (host.dimX() != (size_t)mDesc.W || host.dimY() != (size_t)mDesc.H || host.dimZ() != (size_t)mDesc.C || host.dimB() != (size_t)mDesc.B)
         throw std::runtime_error("HipTensor::synchronizeHToD(): host tensor dimensions do not match");
+    if (mDesc.halo != 0)
+        throw std::runtime_error("HipTensor::synchronizeHToD(): tensors with a halo are written by convolutions only");
     n2d2hip_tensor f = mDesc;
     f.dtype = N2D2HIP_F32;
     f.layout = N2D2HIP_NCHW;
@@ -278,7 +286,16 @@ void Cell_Frame_HIP::allocateOutputs(const Scaling* standalone)
 {
     if (mInputs.empty())
         throw std::runtime_error("Cell " + mName + " has no input");
-    mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, outputDType(standalone));
+    mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, outputDType(standalone), mOutputsHalo);
+}
+
+void Cell_Frame_HIP::setOutputsHalo(int halo)
+{
+    if (halo == mOutputsHalo)
+        return;
+    mOutputsHalo = halo;
+    if (!mOutputs.empty())
+        mOutputs.resize(mOutputs.desc().B, mOutputs.desc().C, mOutputs.desc().H, mOutputs.desc().W, mOutputs.desc().dtype, halo);
 }
 
 n2d2hip_act_t Cell_Frame_HIP::activationHandle(const Scaling* standalone)
@@ -1237,6 +1254,7 @@ void DeepNet::setFusion(bool enabled)
         for (Cell_Frame_HIP* f : mFrames) {
             if (auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f))
                 ew->clearFusion();
+            f->setOutputsHalo(0);
         }
     }
     mFusion = enabled;
@@ -1283,6 +1301,23 @@ void DeepNet::planFusion()
             if (ew->fuseIntoConv(k, conv))
                 break;
         }
+    }
+    // A convolution's output that only convolutions read carries the largest padding among them as a border of zeros,
+    // when all of them run on the kernel that takes such tensors.
+    std::map<const Cell_Frame_HIP*, int> halo;
+    std::map<const Cell_Frame_HIP*, bool> refused;
+    for (Cell_Frame_HIP* f : mFrames) {
+        for (Cell_Frame_HIP* p : f->parentCells()) {
+            if (!p) continue;
+            if (f->convHandle() && n2d2hip_conv_accepts_halo(f->convHandle()))
+                halo[p] = std::max(halo[p], f->maxPadding());
+            else
+                refused[p] = true;
+        }
+    }
+    for (Cell_Frame_HIP* f : mFrames) {
+        const bool writes = f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle());
+        f->setOutputsHalo(writes && !refused[f] ? halo[f] : 0);
     }
     mPlanned = true;
 }

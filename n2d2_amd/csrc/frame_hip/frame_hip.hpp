@@ -128,7 +128,8 @@ public:
     ~HipTensor();
     HipTensor(const HipTensor&) = delete;
     HipTensor& operator=(const HipTensor&) = delete;
-    void resize(int B, int C, int H, int W, int dtype);
+    // halo: border pixels stored around every image, holding the value 0 (tensors between two convolutions)
+    void resize(int B, int C, int H, int W, int dtype, int halo = 0);
     const n2d2hip_tensor& desc() const { return mDesc; }
     bool empty() const { return mDesc.data == nullptr; }
     void invalidateHost() { mHostValid = false; }
@@ -378,6 +379,11 @@ public:
     // Device handles a consumer borrows when it folds this cell (null for cells that cannot be folded)
     virtual n2d2hip_act_t scalingHandle() const { return nullptr; }
     virtual n2d2hip_conv_t convHandle() const { return nullptr; }
+    // Largest padding this cell applies to its input (0 for cells without one)
+    virtual int maxPadding() const { return 0; }
+    // Stores the outputs with a border of `halo` zero pixels around every image (see n2d2hip_tensor::halo)
+    void setOutputsHalo(int halo);
+    int outputsHalo() const { return mOutputsHalo; }
     HipTensor& getDeviceOutputs() { return mOutputs; }
     bool isCuda() const { return false; }
     std::string getPyModel() const { return "Frame_HIP"; }
@@ -386,7 +392,7 @@ public:
     void setStream(void* stream) { mStream = stream; }
 
 protected:
-    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mFoldedInto(nullptr), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
+    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mFoldedInto(nullptr), mOutputsHalo(0), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
     ~Cell_Frame_HIP();
     virtual void setOutputsDims() = 0;
     // (Re)builds the device tables of the activation when its Scaling, its bit width or the
@@ -400,6 +406,7 @@ protected:
     unsigned int mBatch;
     void* mStream;
     Cell_Frame_HIP* mFoldedInto;
+    int mOutputsHalo;
 
 private:
     n2d2hip_act_t mActHandle;
@@ -462,6 +469,7 @@ public:
     bool prepare();
     void launch();
     n2d2hip_conv_t convHandle() const { return mConv; }
+    int maxPadding() const { return std::max(mPaddingDims[0], mPaddingDims[1]); }
 
 protected:
     void setOutputsDims();
@@ -918,7 +926,8 @@ public:
     // Fusion across cells (on by default): a ScalingCell read only by an ElemWise sum is applied inside that sum, and a
     // two-input sum is computed in the epilogue of the 1x1 convolution that produces its later input.  Results are
     // those of the separate cells, bit for bit; the folded cells' own outputs are not written (getOutputs() on them
-    // throws).  Turn it off to read every cell's output.
+    // throws).  With it, a tensor written by a convolution and read only by convolutions is stored with the readers'
+    // padding as a border of zeros (n2d2hip_tensor::halo).  Turn it off to read every cell's output.
     void setFusion(bool enabled);
     bool getFusion() const { return mFusion; }
     // Number of cells propagate() does not launch because a consumer computes them

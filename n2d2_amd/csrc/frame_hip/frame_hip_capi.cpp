@@ -112,6 +112,13 @@ const char* fh_net_model(void* net) { return ((Net*)net)->model.c_str(); }
 int fh_net_nb_cells(void* net) { return (int)((Net*)net)->deepNet->getCells().size(); }
 int fh_net_set_fusion(void* net, int enabled) { return guarded([&] { ((Net*)net)->deepNet->setFusion(enabled != 0); }); }
 int fh_net_nb_folded(void* net) { return (int)((Net*)net)->deepNet->nbFoldedCells(); }
+int fh_net_nb_halo(void* net)
+{
+    int n = 0;
+    for (const auto& c : ((Net*)net)->deepNet->getCells())
+        n += std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->outputsHalo() > 0 ? 1 : 0;
+    return n;
+}
 int fh_net_initialize(void* net) { return guarded([&] { ((Net*)net)->deepNet->initialize(); }); }
 int fh_net_propagate(void* net) { return guarded([&] { ((Net*)net)->deepNet->propagate(true); ((Net*)net)->deepNet->synchronize(); }); }
 

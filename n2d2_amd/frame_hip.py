@@ -19,7 +19,7 @@ lib.fh_net_from_ini.restype = C.c_void_p
 lib.fh_net_from_ini.argtypes = [C.c_char_p]
 lib.fh_net_model.restype = C.c_char_p
 lib.fh_net_set_fusion.argtypes = [C.c_void_p, C.c_int]
-for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize", "fh_net_propagate", "fh_net_nb_folded"):
+for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize", "fh_net_propagate", "fh_net_nb_folded", "fh_net_nb_halo"):
     getattr(lib, _n).argtypes = [C.c_void_p]
 lib.fh_net_set_stimuli.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
@@ -119,6 +119,11 @@ class Net:
     @property
     def nb_folded(self):
         return lib.fh_net_nb_folded(self.h)
+
+    @property
+    def nb_halo(self):
+        """Cells whose output is stored with a border of zeros for the convolutions that read it."""
+        return lib.fh_net_nb_halo(self.h)
 
     def set_stimuli(self, x):
         a = np.ascontiguousarray(x, dtype=np.float32)

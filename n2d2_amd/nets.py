@@ -356,9 +356,11 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True):
+    def __init__(self, spec, batch, fuse=True, halo=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
-        the rescaled tensor is never written)."""
+        the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
+        halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
+        a border of zeros around every image, which lets a padded KxK reader fetch every tap without a validity test."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
         consumers = {}
@@ -371,6 +373,17 @@ class GpuNet:
         order = {l.name: k for k, l in enumerate(spec.layers)}
         order["input"] = -1
         C, H, W = spec.in_shape
+
+        def reads_halo(m):
+            return (m.type == "conv" and m.groups == 1 and m.weight_bits == 8 and m.w.shape[1] % 64 == 0
+                    and m.w.shape[2] * m.w.shape[3] <= 31 and tuple(m.dil) == (1, 1))
+
+        def halo_of(l, cell):
+            """Border to store around l's output: the largest padding among its readers, if all of them can use it."""
+            readers = consumers.get(l.name, [])
+            if not halo or not readers or not all(reads_halo(m) for m in readers) or not cell.accepts_halo():
+                return 0
+            return max(max(m.pad) for m in readers)
         self.input = rt.DTensor(batch, C, H, W, capi.U8B if spec.input_unsigned else capi.I8)
         self.tensors = {"input": self.input}
         self.steps = []
@@ -384,7 +397,9 @@ class GpuNet:
                     cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits)
                 else:
                     cell = rt.Fc(l.w, l.bias, act, ins[0].dtype, (ins[0].C, ins[0].H, ins[0].W), l.weight_bits)
-                out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype())
+                if ins[0].halo and not (l.type == "conv" and cell.accepts_halo()):
+                    raise RuntimeError("layer %s cannot read the halo its input was given (GpuNet(halo=False) avoids it)" % l.name)
+                out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype(), halo=halo_of(l, cell) if l.type == "conv" else 0)
                 self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
             elif l.type == "pool":
                 cell = rt.Pool(l.kind, l.pool, l.stride, l.pad)

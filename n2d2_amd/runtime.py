@@ -23,13 +23,16 @@ def stream_ptr():
 class DTensor:
     """A device tensor plus its n2d2hip_tensor descriptor."""
 
-    def __init__(self, B, Cc, H, W, dtype, layout=capi.NHWC, buf=None):
-        self.B, self.C, self.H, self.W, self.dtype, self.layout = B, Cc, H, W, dtype, layout
+    def __init__(self, B, Cc, H, W, dtype, layout=capi.NHWC, buf=None, halo=0):
+        """halo: border pixels stored around every image (NHWC byte tensors between two convolutions), holding the value 0."""
+        self.B, self.C, self.H, self.W, self.dtype, self.layout, self.halo = B, Cc, H, W, dtype, layout, halo
         self.cs = capi.nhwc_cs(Cc) if layout == capi.NHWC else Cc
-        n = B * H * W * self.cs
+        n = B * (H + 2 * halo) * (W + 2 * halo) * self.cs
         self.buf = buf if buf is not None else torch.empty(n, dtype=_TORCH_DT[dtype], device="cuda")
         assert self.buf.numel() == n
-        self.desc = capi.Tensor(self.buf.data_ptr(), dtype, layout, B, Cc, H, W, self.cs)
+        self.desc = capi.Tensor(self.buf.data_ptr(), dtype, layout, B, Cc, H, W, self.cs, halo)
+        if halo:
+            check(lib.n2d2hip_tensor_clear(self.ref, stream_ptr()))
 
     @property
     def ref(self):
@@ -140,9 +143,13 @@ class Conv:
         check(lib.n2d2hip_conv_out_dims(C.byref(self.desc), H, W, C.byref(oh), C.byref(ow)))
         return oh.value, ow.value
 
-    def make_output(self, x, out_dtype=None):
+    def make_output(self, x, out_dtype=None, halo=0):
         oh, ow = self.out_shape(x.H, x.W)
-        return DTensor(x.B, self.desc.O, oh, ow, out_dtype if out_dtype is not None else self.act.out_dtype())
+        return DTensor(x.B, self.desc.O, oh, ow, out_dtype if out_dtype is not None else self.act.out_dtype(), halo=halo)
+
+    def accepts_halo(self):
+        """True when this convolution reads and writes tensors that carry their padding as a border of zeros."""
+        return bool(lib.n2d2hip_conv_accepts_halo(self.handle))
 
     def forward(self, x, out=None, out_dtype=None):
         if out is None:

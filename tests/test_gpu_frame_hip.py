@@ -45,6 +45,8 @@ def test_resnet50_through_the_registrar(fh):
     net = _compare(fh, spec, x, ["conv1", "pool1", "conv2.1_sum", "conv2.2_1x1", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
     # 12 shortcut ScalingCells applied inside their sums, 16 sums computed by the 1x1 convolution before them
     assert net.nb_folded == 28
+    # the 16 tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border
+    assert net.nb_halo == 16
     with pytest.raises(fh.FrameHipError) as e:
         net.outputs("conv2.2_shortcut_rescale")
     assert "not materialised" in str(e.value)
@@ -57,7 +59,7 @@ def test_resnet50_through_the_registrar(fh):
     # without fusion every cell is launched and readable
     net.set_fusion(False)
     net.propagate()
-    assert net.nb_folded == 0
+    assert net.nb_folded == 0 and net.nb_halo == 0
     keep = ["conv2.2_shortcut_rescale", "conv2.2_1x1_x4", "conv2.2_sum", "fc"]
     want = cells.run_net(spec, x2, keep=keep)
     for name in keep:
@@ -65,7 +67,8 @@ def test_resnet50_through_the_registrar(fh):
     # and back on: the plan is made again
     net.set_fusion(True)
     net.propagate()
-    assert net.nb_folded == 28 and np.array_equal(net.outputs("fc"), want["fc"])
+    assert net.nb_folded == 28 and net.nb_halo == 16 and np.array_equal(net.outputs("fc"), want["fc"])
+    assert np.array_equal(net.outputs("conv2.2_1x1"), cells.run_net(spec, x2, keep=["conv2.2_1x1"])["conv2.2_1x1"])
 
 
 def test_fusion_follows_a_scaling_change(fh):

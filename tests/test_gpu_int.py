@@ -455,6 +455,62 @@ def test_conv_with_folded_residual_sum(rt):
         conv1.forward_sum(rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B))
 
 
+def test_conv_reads_and_writes_halo_tensors(rt):
+    """A tensor stored with its reader's padding as a border of zeros: a convolution writes it (plain and with a folded sum),
+    a padded KxK convolution reads it, the graph-edge conversion reads it, and every result equals the plain tensors'."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(91)
+    for C, O, O2, H, W, k, stride, pad, halo, B in ((64, 64, 64, 9, 7, 3, 1, 1, 1, 3), (128, 128, 192, 8, 8, 3, 2, 1, 1, 2),
+                                                     (64, 128, 64, 6, 10, 5, 1, 2, 2, 2), (256, 64, 64, 7, 7, 3, 1, 1, 2, 2),
+                                                     (64, 64, 128, 12, 12, 1, 2, 0, 1, 2)):
+        x = rng.integers(0, 256, size=(B, C, H, W))
+        w1 = np.clip(np.rint(rng.normal(0, 20, size=(O, C, 1, 1))), -127, 127).astype(np.int64)
+        w2 = np.clip(np.rint(rng.normal(0, 20, size=(O2, O, k, k))), -127, 127).astype(np.int64)
+        s1, s2 = conv_spec_for(O, rng), conv_spec_for(O2, rng)
+        s1.kind, s1.unsigned_out = "Rectifier", True
+        b1, b2 = rng.integers(-500, 500, size=O), rng.integers(-500, 500, size=O2)
+        y1 = cells_ref.conv_cell(x, w1, b1, s1)
+        y2 = cells_ref.conv_cell(y1, w2, b2, s2, stride=(stride, stride), pad=(pad, pad, pad, pad))
+        c1 = rt.Conv(w1, b1, rt.Act(O, **s1.kwargs()), capi.U8B)
+        c2 = rt.Conv(w2, b2, rt.Act(O2, **s2.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad, pad, pad, pad))
+        assert c1.accepts_halo() and c2.accepts_halo()
+        dx = rt.DTensor.from_numpy(x, capi.U8B)
+        mid = c1.make_output(dx, halo=halo)
+        assert mid.buf.numel() == B * (H + 2 * halo) * (W + 2 * halo) * mid.cs
+        c1.forward(dx, mid)
+        assert np.array_equal(mid.to_numpy(), y1.astype(np.int64)), (C, O, "written with a halo")
+        border = mid.buf.view(B, H + 2 * halo, W + 2 * halo, mid.cs).clone()
+        border[:, halo:H + halo, halo:W + halo, :] = -128
+        assert bool((border == -128).all()), "the border keeps the stored form of 0"
+        got = c2.forward(mid).to_numpy()
+        assert np.array_equal(got, y2.astype(np.int64)), (C, O, O2, k, stride, pad, halo)
+        # a reader with no padding of its own skips the border
+        w3 = np.clip(np.rint(rng.normal(0, 20, size=(64, O, 1, 1))), -127, 127).astype(np.int64)
+        s3 = conv_spec_for(64, rng)
+        c3 = rt.Conv(w3, None, rt.Act(64, **s3.kwargs()), capi.U8B)
+        assert np.array_equal(c3.forward(mid).to_numpy(), cells_ref.conv_cell(y1, w3, None, s3).astype(np.int64))
+        # the folded residual sum writes a halo too
+        ssum = sum_spec_for(O, rng)
+        other = rng.integers(0, 256, size=(B, O, H, W))
+        ew = rt.ElemWiseSum(2, O, rt.Act(O, **ssum.kwargs()))
+        c1b = rt.Conv(w1, b1, rt.Act(O, **conv_spec_for(O, rng).kwargs()), capi.U8B)
+        ylin = cells_ref.conv_cell(x, w1, b1, conv_spec_for(O, np.random.default_rng(5)))
+        c1b = rt.Conv(w1, b1, rt.Act(O, **conv_spec_for(O, np.random.default_rng(5)).kwargs()), capi.U8B)
+        assert c1b.fuse_sum(ew, 0, capi.U8B)
+        want = cells_ref.elemwise_cell([ylin, other.astype(np.float32)], ssum).astype(np.int64)
+        out = rt.DTensor(B, O, H, W, capi.U8B, halo=halo)
+        c1b.forward_sum(dx, rt.DTensor.from_numpy(other, capi.U8B), out)
+        assert np.array_equal(out.to_numpy(), want)
+    # cells that do not take a halo say so
+    xh = rt.DTensor(1, 64, 4, 4, capi.U8B, halo=1)
+    with pytest.raises(capi.N2D2HipError):
+        rt.Pool("max", (2, 2), (2, 2), (0, 0)).forward(xh)
+    wd = np.clip(np.rint(rng.normal(0, 20, size=(64, 48, 3, 3))), -127, 127).astype(np.int64)
+    c48 = rt.Conv(wd, None, rt.Act(64, **conv_spec_for(64, rng).kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    assert not c48.accepts_halo()
+
+
 def conv_spec_for(O, rng):
     from oracle.cells import ActSpec
     return ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=False)

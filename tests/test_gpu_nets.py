@@ -49,9 +49,15 @@ def test_resnet50_config(variant):
     # 12 shortcut ScalingCells folded into their sums, 16 sums folded into the convolution that feeds them
     assert "conv2.2_shortcut_rescale" in net.folded and "conv2.1_1x1_proj" in net.folded and "conv2.2_1x1_x4" in net.folded
     assert len(net.folded) == 28 and len(net.launched) == len(spec.layers) - 28
+    # the 16 tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border of zeros
+    assert sorted(n for n, t in net.tensors.items() if t.halo) == sorted(l.name[:-3] + "1x1" for l in spec.layers if l.name.endswith("_3x3"))
     if variant == "pad1":
         unfused = _run_both(spec, x, keep, fuse=False)
         assert not unfused.folded
+        plain = nets.GpuNet(spec, x.shape[0], halo=False)
+        plain.set_input(x)
+        assert not any(t.halo for t in plain.tensors.values())
+        assert np.array_equal(plain.forward().to_numpy(), net.tensors[spec.output].to_numpy())
     assert net.tensors["pool1"].H == (55 if variant == "pad0_n2d2_model" else 56)
     if variant == "all_signed":
         assert net.tensors["conv5.3_sum"].to_numpy().max() <= 127
