@@ -414,7 +414,7 @@ void launch_cfg(const ConvArgs& a, hipStream_t stream)
 }
 
 template <int NW, int BK, int NI, int NJ, int WGM, int S>
-void launch_pipe(ConvPipeArgs a, int valid, int grid, hipStream_t stream)
+void launch_pipe(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t stream)
 {
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
@@ -424,7 +424,17 @@ void launch_pipe(ConvPipeArgs a, int valid, int grid, hipStream_t stream)
          else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 0>), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
     switch (a.c.epi.kind) {
     case EPI_RAW: N2D2HIP_PIPE(EPI_RAW); break;
-    case EPI_I24: N2D2HIP_PIPE(EPI_I24); break;
+    case EPI_I24:
+        if (!hi16) {
+            N2D2HIP_PIPE(EPI_I24);
+        } else if (valid == 1) {
+            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        } else if (valid == 2) {
+            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 2, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        }
+        break;
     default: N2D2HIP_PIPE(EPI_F32); break;
     }
 #undef N2D2HIP_PIPE
@@ -859,6 +869,10 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
         q.sum16 = nullptr; q.sum16_stride = 0; q.pre_in_range = 0;
         q.sum = EpiArgs(); q.pre = EpiArgs();
+        // Byte outputs of an integer rescale whose scaled-up tables fit: the rescaled value is read from the upper half of
+        // the multiply-add's result
+        const bool hi16 = !other && c->hi16 && c->act->args.kind == EPI_I24 && is_byte_type(out->dtype) && getenv("N2D2HIP_NO_HI16") == nullptr;
+        if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
         if (other) {
             const int cp = c->sum->act->cpad;
             q.res = (const signed char*)other->data;
@@ -888,15 +902,15 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
                 else launch_pipe_res<4, 64, 2, 1, 4, 4>(q, grid, stream);
             }
         } else if (wide64) {
-            launch_pipe<4, 64, 2, 2, 4, 3>(q, all_valid, grid, stream);
+            launch_pipe<4, 64, 2, 2, 4, 3>(q, all_valid, hi16, grid, stream);
         } else if (small_m) {
-            launch_pipe<4, 128, 2, 1, 2, 3>(q, all_valid, grid, stream);
+            launch_pipe<4, 128, 2, 1, 2, 3>(q, all_valid, hi16, grid, stream);
         } else if (d.C % 128 == 0) {
-            if (bn128) launch_pipe<4, 128, 2, 2, 2, 2>(q, all_valid, grid, stream);
-            else launch_pipe<4, 128, 2, 1, 4, 3>(q, all_valid, grid, stream);
+            if (bn128) launch_pipe<4, 128, 2, 2, 2, 2>(q, all_valid, hi16, grid, stream);
+            else launch_pipe<4, 128, 2, 1, 4, 3>(q, all_valid, hi16, grid, stream);
         } else {
-            if (bn128) launch_pipe<4, 64, 2, 2, 2, 4>(q, all_valid, grid, stream);
-            else launch_pipe<4, 64, 2, 1, 4, 4>(q, all_valid, grid, stream);
+            if (bn128) launch_pipe<4, 64, 2, 2, 2, 4>(q, all_valid, hi16, grid, stream);
+            else launch_pipe<4, 64, 2, 1, 4, 4>(q, all_valid, hi16, grid, stream);
         }
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;

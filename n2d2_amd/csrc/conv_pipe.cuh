@@ -142,7 +142,9 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // BK: bytes of K per ring stage and row (64 or 128); 128 makes every row segment a whole 128-byte line, which is
 // what the L2 -> LDS path moves fastest.
 // RES: the residual sum that follows the convolution is computed in the epilogue (1x1 convolutions, EPI_I24).
-// P16 (with RES): the sum's arithmetic runs on pairs of 16-bit values (the host has shown that it fits).
+// P16: the integer rescale's tables come scaled up so that the result is the upper half of a 32-bit register (no
+// shift), and what follows runs on pairs of 16-bit values: with RES the whole sum, without it the saturation and the
+// pack.  The host chooses it when it has shown that nothing overflows.
 // VALID: 0 = windows may reach outside the input (per-tap validity bits), 1 = 1x1 kernel without padding, 2 = any kernel
 // without padding (every tap of every window inside the input: a tap only moves the uniform base address).
 template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, int VALID, bool RES = false, bool P16 = false>
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     const unsigned tab = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 4u;      // this lane's first channel in the tables
     const unsigned tab16 = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 2u;    // and in the 16-bit pairs
     constexpr bool p16 = RES && P16;
-    static_assert(RES || !P16, "16-bit pairs are for the folded sum");
+    static_assert(!P16 || EPI == EPI_I24, "16-bit pairs follow the integer rescale");
 
     // two fragment sets: while the MFMAs of K step g run from set g%2, the reads of step g+1 fly into the other
     v4i fw[2][NI], fp[2][NJ];
@@ -404,14 +406,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         // Without a folded sum, the convolution's tables of the next channel group are requested before this group is
         // rescaled (two register sets), so that their LDS latency is hidden behind the arithmetic.
         v4i tq[2][5];
+        // Every register such a read fills must be tied after the wait, used or not: a register the compiler takes for
+        // dead is handed to other values while the read is still on its way.  So only what is used is requested.
         auto request_tables = [&](v4i* t, unsigned trow) {
-            lds_read128_nowait<BN * 4>(t[0], trow);
-            lds_read128_nowait<2 * BN * 4>(t[1], trow);
+            if (!P16) lds_read128_nowait<BN * 4>(t[0], trow);
+            if (!P16) lds_read128_nowait<2 * BN * 4>(t[1], trow);
             lds_read128_nowait<3 * BN * 4>(t[2], trow);
             if (EPI == EPI_I24) lds_read128_nowait<4 * BN * 4>(t[3], trow);
-            if (EPI != EPI_F32) lds_read128_nowait<5 * BN * 4>(t[4], trow);
+            if (EPI != EPI_F32 && !P16) lds_read128_nowait<5 * BN * 4>(t[4], trow);
         };
-        constexpr int NTR = 3 + (EPI == EPI_I24 ? 1 : 0) + (EPI != EPI_F32 ? 1 : 0);      // reads per request
+        constexpr int NTR = P16 ? 2 : 3 + (EPI == EPI_I24 ? 1 : 0) + (EPI != EPI_F32 ? 1 : 0);      // reads per request
         if (!RES && EPI != EPI_RAW)
             request_tables(tq[0], tab);
 #pragma unroll
@@ -507,6 +511,42 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
                     for (int j = 0; j < NJ; ++j)
                         asm volatile("" : "+v"(pk[i][j][g]));
+                } else if constexpr (P16) {
+                    // ---- plain convolution, byte output: multiply-add, take the upper halves, saturate and pack.  The
+                    // tables of the next channel group are requested before this one is rescaled.
+                    if (idx + 1 < NI * 4) {
+                        const int nx = idx + 1;
+                        request_tables(tq[nx & 1], tab + (unsigned)((nx / 4) * 32 + 8 * (nx % 4)) * 4u);
+                        wait_lgkm<NTR>();
+                    } else {
+                        wait_lgkm<0>();
+                    }
+                    // (the wait is tied to the registers the reads write, not to copies the compiler could make early)
+                    tie(tq[idx & 1][2]); tie(tq[idx & 1][3]);
+                    const v4i tc = tq[idx & 1][2], td = tq[idx & 1][3];
+                    v2s pq[NJ][2];
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int t0 = __mul24(acc[i][j][4 * g + 2 * h], tc[2 * h]) + td[2 * h];
+                            const int t1 = __mul24(acc[i][j][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
+                            pq[j][h] = as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u));
+                        }
+                    if (vlo == 0 && vhi == 255) {
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+                            pk[i][j][g] = (sat_pk_u8(pq[j][0]) | (sat_pk_u8(pq[j][1]) << 16)) ^ p.out_xor;
+                    } else {
+                        const v2s lo1 = splat_v2s(vlo), hi1 = splat_v2s(vhi);
+#pragma unroll
+                        for (int j = 0; j < NJ; ++j)
+                            pk[i][j][g] = __builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, clamp_v2s(pq[j][1], lo1, hi1)),
+                                                                (unsigned)__builtin_bit_cast(int, clamp_v2s(pq[j][0], lo1, hi1)), 0x06040200u) ^ p.out_xor;
+                    }
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j)
+                        asm volatile("" : "+v"(pk[i][j][g]));
                 } else {
                 int r[NJ][4];
                 // RES: every table of the group is requested at once (LDS answers in order); each phase then waits only
@@ -523,10 +563,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                         } else {
                             wait_lgkm<0>();
                         }
+                        tie(tq[idx & 1][0]); tie(tq[idx & 1][1]); tie(tq[idx & 1][2]);
+                        if (EPI == EPI_I24) tie(tq[idx & 1][3]);
+                        if (EPI != EPI_F32) tie(tq[idx & 1][4]);
                         ta = tq[idx & 1][0]; tb = tq[idx & 1][1]; tc = tq[idx & 1][2];
                         if (EPI == EPI_I24) td = tq[idx & 1][3];
                         if (EPI != EPI_F32) te = tq[idx & 1][4];
-                        tie(ta); tie(tb); tie(tc); tie(td); tie(te);
                     }
                     if (EPI != EPI_RAW && RES) {
                         lds_read128_nowait<BN * 4>(ta, trow);

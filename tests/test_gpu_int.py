@@ -455,6 +455,34 @@ def test_conv_with_folded_residual_sum(rt):
         conv1.forward_sum(rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B), rt.DTensor(1, 64, 4, 4, capi.U8B))
 
 
+def test_conv_rescale_variants_agree(rt):
+    """The pipelined kernel has two integer epilogues (32-bit multiply-shift-saturate, and scaled-up tables whose result is
+    the upper register half, saturated as 16-bit pairs); both must give the oracle's bytes, for either output signedness."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(123)
+    for C, O, H, k, pad in ((64, 256, 9, 1, 0), (128, 64, 7, 3, 1), (64, 192, 6, 3, 0)):
+        x = rng.integers(0, 256, size=(3, C, H, H))
+        w = np.clip(np.rint(rng.normal(0, 25, size=(O, C, k, k))), -127, 127).astype(np.int64)
+        bias = rng.integers(-3000, 3000, size=O)
+        for spec in (ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(6, 13, size=O)], 1), nb_bits=8, unsigned_out=True),
+                     ActSpec("Linear", "SingleShift", rng.integers(5, 16, size=O), nb_bits=8, unsigned_out=False),
+                     ActSpec("Linear", "FixedMult16", rng.integers(2 ** 8, 2 ** 12, size=O), frac_bits=16, nb_bits=8, unsigned_out=False),
+                     ActSpec("Rectifier", "FixedMult32", rng.integers(2 ** 18, 2 ** 22, size=O), frac_bits=28, nb_bits=8, unsigned_out=True)):
+            want = cells_ref.conv_cell(x, w, bias, spec, pad=(pad, pad, pad, pad)).astype(np.int64)
+            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, pad=(pad, pad, pad, pad))
+            dx = rt.DTensor.from_numpy(x, capi.U8B)
+            for no16 in ("", "1"):
+                if no16:
+                    os.environ["N2D2HIP_NO_HI16"] = no16
+                try:
+                    got = conv.forward(dx).to_numpy()
+                finally:
+                    os.environ.pop("N2D2HIP_NO_HI16", None)
+                assert np.array_equal(got, want), (C, O, k, spec.mode, no16, np.count_nonzero(got != want))
+
+
 def test_conv_reads_and_writes_halo_tensors(rt):
     """A tensor stored with its reader's padding as a border of zeros: a convolution writes it (plain and with a folded sum),
     a padded KxK convolution reads it, the graph-edge conversion reads it, and every result equals the plain tensors'."""
