@@ -441,11 +441,14 @@ void launch_pipe(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t str
 }
 
 template <int KH>
-void launch_stem(const ConvStemArgs& a, int grid, hipStream_t stream)
+void launch_stem(const ConvStemArgs& a, bool hi16, int grid, hipStream_t stream)
 {
     switch (a.c.epi.kind) {
     case EPI_RAW: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_RAW>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I24: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24:
+        if (hi16) hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a);
+        break;
     default: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_F32>), dim3(grid), dim3(256), 0, stream, a); break;
     }
 }
@@ -937,9 +940,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             magic_div((unsigned)OH, &q.oh_mul, &q.oh_sh);
             magic_div((unsigned)q.tiles_per_row, &q.tpr_mul, &q.tpr_sh);
             const int grid = 8 * q.nlanes * q.c.ntiles_n;
-            if (d.kH == 3) launch_stem<3>(q, grid, stream);
-            else if (d.kH == 5) launch_stem<5>(q, grid, stream);
-            else launch_stem<7>(q, grid, stream);
+            const bool hi16 = k == EPI_I24 && c->hi16 && is_byte_type(out->dtype) && getenv("N2D2HIP_NO_HI16") == nullptr;
+            if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
+            if (d.kH == 3) launch_stem<3>(q, hi16, grid, stream);
+            else if (d.kH == 5) launch_stem<5>(q, hi16, grid, stream);
+            else launch_stem<7>(q, hi16, grid, stream);
             N2D2HIP_HIP_CHECK(hipGetLastError());
             return N2D2HIP_OK;
         }

@@ -22,6 +22,10 @@
 //    having to see the previous tile's stores acknowledged;
 //  * the epilogue is the pipelined kernel's: rescale, pack to bytes, exchange
 //    between lane halves until a lane owns 32 consecutive channels, store.
+//    H16 (integer rescale, byte output, tables scaled up by the host so that
+//    the result is the upper half of the multiply-add): a lane's 32 channels
+//    never change, so their multipliers and addends live in registers and the
+//    epilogue reads no table at all.
 #pragma once
 
 namespace n2d2hip {
@@ -39,9 +43,10 @@ struct ConvStemArgs {
     int preclamp;
 };
 
-template <int KH, int EPI>
+template <int KH, int EPI, bool H16 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) void conv_stem_kernel(ConvStemArgs q)
 {
+    static_assert(!H16 || EPI == EPI_I24, "scaled-up tables belong to the integer rescale");
     const ConvArgs& p = q.c;
     constexpr int TW = 128;                    // output pixels per tile
     constexpr int PITCH = 1280;                // bytes per patch row in LDS: 5 loads of 64 pixels
@@ -67,7 +72,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     const int last = min((xcd + 1) * q.xcd_tiles, q.ntiles);
     const int ntile = (first < last) ? (last - first + q.nlanes - 1) / q.nlanes : 0;
 
-    // ---- loader: chunk c = wave + 4*j is 64 pixels (part c%5) of patch row c/5
+    // ---- loader: chunk c = wave + 4*j is 64 pixels (part c%5) of patch row c/5.  Which row and part a wave's j-th
+    // load fetches never changes, so that is worked out once; the scalar unit is shared by every wave of the CU and
+    // the per-tile part of this arithmetic is what the kernel spends most of its issue slots on.
+    int ld_row[NLOAD], ld_x[NLOAD], ld_lds[NLOAD];
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+        const int c = wave + 4 * j;
+        const int r = c / 5, part = c - r * 5;
+        ld_row[j] = c < NCHUNK ? r : -(1 << 20);        // a chunk past the end reads a row that is never inside
+        ld_x[j] = part * 64;
+        ld_lds[j] = r * PITCH + part * 256;
+    }
+    const unsigned row_bytes = (unsigned)p.W * 4u;
     auto issue = [&](int t, int stage) {
         const int id = first + t * q.nlanes;
         const bool live = t < ntile;
@@ -75,20 +92,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         const int txi = (live ? id : 0) - rowid * q.tiles_per_row;
         const int b = div_magic(rowid, q.oh_mul, q.oh_sh);
         const int oy = rowid - b * p.OH;
-        const int x0 = txi * TW * p.strideX - p.padL, y0 = oy * p.strideY - p.padT;
+        const int x0 = txi * TW * p.strideX - p.padL + lane;
+        const int y0 = live ? oy * p.strideY - p.padT : -(1 << 21);
         unsigned char* sbase = smem + stage * STAGE;
-        const signed char* img = p.in + (long long)b * p.H * p.W * 4;
+        const signed char* img = p.in + (long long)b * p.H * row_bytes;
 #pragma unroll
         for (int j = 0; j < NLOAD; ++j) {
-            const int c = wave + 4 * j;
-            const int r = c / 5, part = c - r * 5;
-            const int iy = y0 + r;
+            const int iy = y0 + ld_row[j];
             // everything about the row is block-uniform; a row outside the image sends every lane to the zero
-            const bool row_ok = live & (c < NCHUNK) & ((unsigned)iy < (unsigned)p.H);
-            const signed char* rowp = img + (long long)(row_ok ? iy : 0) * p.W * 4;
-            const int ix = (row_ok ? x0 + part * 64 : -(1 << 20)) + lane;
-            const signed char* src = (unsigned)ix < (unsigned)p.W ? rowp + (unsigned)ix * 4u : q.fill16;
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + r * PITCH + part * 256), 4, 0, 0);
+            const bool row_ok = (unsigned)iy < (unsigned)p.H;
+            const signed char* rowp = img + (row_ok ? (unsigned)iy : 0u) * row_bytes;
+            const int ix = x0 + ld_x[j];
+            const signed char* src = (row_ok & ((unsigned)ix < (unsigned)p.W)) ? rowp + (unsigned)ix * 4u : q.fill16;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + ld_lds[j]), 4, 0, 0);
         }
     };
     issue(0, 0);
@@ -117,6 +133,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         }
     }
     __syncthreads();
+    v4i rc[H16 ? 2 : 1][H16 ? 4 : 1], rd[H16 ? 2 : 1][H16 ? 4 : 1];
+    if (H16) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                rc[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(p.epi.c + n0 + i * 32 + 8 * g + 4 * lh);
+                rd[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(p.epi.d + n0 + i * 32 + 8 * g + 4 * lh);
+            }
+    }
     const unsigned tab = lds0 + TAB_OFF + (unsigned)(4 * lh) * 4u;
     const bool out_bytes = p.out_dtype != N2D2HIP_I32;
     const int vlo = p.epi.lo, vhi = p.epi.hi;
@@ -165,6 +191,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                if constexpr (H16) {
+                    const v4i tc = rc[H16 ? i : 0][H16 ? g : 0], td = rd[H16 ? i : 0][H16 ? g : 0];
+                    v2s pq[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int t0 = __mul24(acc[i][4 * g + 2 * h], tc[2 * h]) + td[2 * h];
+                        const int t1 = __mul24(acc[i][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
+                        pq[h] = as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u));
+                    }
+                    if (vlo == 0 && vhi == 255) {
+                        pk[i][g] = (sat_pk_u8(pq[0]) | (sat_pk_u8(pq[1]) << 16)) ^ p.out_xor;
+                    } else {
+                        const v2s lo1 = splat_v2s(vlo), hi1 = splat_v2s(vhi);
+                        pk[i][g] = __builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, clamp_v2s(pq[1], lo1, hi1)),
+                                                         (unsigned)__builtin_bit_cast(int, clamp_v2s(pq[0], lo1, hi1)), 0x06040200u) ^ p.out_xor;
+                    }
+                    continue;
+                }
                 const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
                 v4i tbias = {0, 0, 0, 0}, ta = tbias, tb = tbias, tc = tbias, td = tbias, te = tbias;
                 if (BIAS_ADD) lds_read128_nowait<0>(tbias, trow);

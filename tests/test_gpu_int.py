@@ -462,7 +462,7 @@ def test_conv_rescale_variants_agree(rt):
     from oracle.cells import ActSpec
     from oracle import cells as cells_ref
     rng = np.random.default_rng(123)
-    for C, O, H, k, pad in ((64, 256, 9, 1, 0), (128, 64, 7, 3, 1), (64, 192, 6, 3, 0)):
+    for C, O, H, k, pad, stride in ((64, 256, 9, 1, 0, 1), (128, 64, 7, 3, 1, 1), (64, 192, 6, 3, 0, 1), (3, 64, 45, 7, 3, 2)):
         x = rng.integers(0, 256, size=(3, C, H, H))
         w = np.clip(np.rint(rng.normal(0, 25, size=(O, C, k, k))), -127, 127).astype(np.int64)
         bias = rng.integers(-3000, 3000, size=O)
@@ -470,8 +470,8 @@ def test_conv_rescale_variants_agree(rt):
                      ActSpec("Linear", "SingleShift", rng.integers(5, 16, size=O), nb_bits=8, unsigned_out=False),
                      ActSpec("Linear", "FixedMult16", rng.integers(2 ** 8, 2 ** 12, size=O), frac_bits=16, nb_bits=8, unsigned_out=False),
                      ActSpec("Rectifier", "FixedMult32", rng.integers(2 ** 18, 2 ** 22, size=O), frac_bits=28, nb_bits=8, unsigned_out=True)):
-            want = cells_ref.conv_cell(x, w, bias, spec, pad=(pad, pad, pad, pad)).astype(np.int64)
-            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, pad=(pad, pad, pad, pad))
+            want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(pad, pad, pad, pad)).astype(np.int64)
+            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad, pad, pad, pad))
             dx = rt.DTensor.from_numpy(x, capi.U8B)
             for no16 in ("", "1"):
                 if no16:
