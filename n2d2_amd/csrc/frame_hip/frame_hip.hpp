@@ -341,6 +341,13 @@ public:
     std::pair<double, double> getOutputsRangeParents() const;
     const std::shared_ptr<Activation>& getActivation() const { return mActivation; }
     void setActivation(const std::shared_ptr<Activation>& activation) { mActivation = activation; }
+    // Free parameters as text files, "<base>_weights<.ext>" and "<base>_biases<.ext>" (or one file holding both), the
+    // format N2D2 exports after training or quantization (include/Cell/Cell.hpp:355-372)
+    virtual void importFreeParameters(const std::string& fileName, bool ignoreNotExists = false) { (void)fileName; (void)ignoreNotExists; }
+    virtual void exportFreeParameters(const std::string& fileName) const { (void)fileName; }
+    // Applies func to every weight and the bias of one output (Cell::processFreeParametersPerOutput,
+    // include/Cell/Cell.hpp:402-407)
+    virtual void processFreeParametersPerOutput(const std::function<Float_T(Float_T)>& func, std::size_t output) { (void)func; (void)output; }
 
 protected:
     Cell(const std::string& name, unsigned int nbOutputs)
@@ -433,6 +440,13 @@ public:
     void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }
     // 4: weights are handed to the device nibble-packed (values must fit [-8,7])
     void setWeightsPrecision(int bits) { mWeightBits = bits; mDirty = true; }
+    const Tensor<Float_T>& getWeights() const { return mWeights; }
+    const Tensor<Float_T>& getBiases() const { return mBias; }
+    // OCHW text: one line per output, the kernels of its connected channels one after the other, kernel x fastest
+    // (src/Cell/ConvCell.cpp:299-353, 511-679)
+    void importFreeParameters(const std::string& fileName, bool ignoreNotExists = false);
+    void exportFreeParameters(const std::string& fileName) const;
+    void processFreeParametersPerOutput(const std::function<Float_T(Float_T)>& func, std::size_t output);
 
 protected:
     ConvCell(const std::vector<unsigned int>& kernelDims, const std::vector<unsigned int>& subSampleDims,
@@ -494,6 +508,12 @@ public:
     // {K, O} float tensor (K = C*H*W in CHW order), bias {O}
     void setWeights(const Tensor<Float_T>& weights) { mWeights = weights; mDirty = true; }
     void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }
+    const Tensor<Float_T>& getWeights() const { return mWeights; }
+    const Tensor<Float_T>& getBiases() const { return mBias; }
+    // OC text: one line per output, one weight per input in CHW order (src/Cell/FcCell.cpp:110-298)
+    void importFreeParameters(const std::string& fileName, bool ignoreNotExists = false);
+    void exportFreeParameters(const std::string& fileName) const;
+    void processFreeParametersPerOutput(const std::function<Float_T(Float_T)>& func, std::size_t output);
 
 protected:
     FcCell() : mNoBias(false), mDirty(true) {}
@@ -941,6 +961,25 @@ private:
     std::map<std::string, std::shared_ptr<Cell> > mCells;
     HipTensor mStimuli;
     unsigned int mEnvC = 0, mEnvH = 0, mEnvW = 0, mEnvB = 0;
+};
+
+// The step of N2D2's post-training quantization that turns the floating-point rescale of a cell into one of the integer
+// Scaling modes the quantized cells execute (src/DeepNetQuantization.cpp:1043-1287).  A graph whose activations carry
+// FLOAT_MULT scalings (from a calibration done elsewhere) becomes runnable on the integer path this way.
+class DeepNetQuantization {
+public:
+    // Largest number of fractional bits for which every rounded factor fits int16 (FIXED_MULT16, falling back to
+    // FIXED_MULT32, which `mode` then says) or int32; at most 50 (src/DeepNetQuantization.cpp:1043-1093)
+    static std::pair<std::size_t, std::vector<std::int32_t> > approximateScalingWithFixedPoint(ScalingMode& mode,
+                                                                                               const std::vector<Float_T>& scalingPerOutput);
+    // scaling <= 1 as a sum of nbDivisions powers of two 2^-e, greedily from the largest; .second is sum / scaling, the
+    // factor by which the result overshoots (>= 1; exactly 1 when the greedy sum reaches 98 % of the scaling)
+    // (src/DeepNetQuantization.cpp:1095-1134)
+    static std::pair<std::vector<unsigned char>, double> approximateScalingWithPowerOf2Divs(Float_T scaling, std::size_t nbDivisions);
+    // Replaces the FLOAT_MULT scaling of `activation` by its approximation in `actScalingMode`; for the shift modes the
+    // cell's weights and biases are divided by the overshoot, per output (src/DeepNetQuantization.cpp:1147-1178,
+    // 1201-1287).  Scalings above 1 cannot be shifts: FIXED_MULT16 is used for that cell instead.
+    static void approximateActivationScaling(Cell& cell, Activation& activation, ScalingMode actScalingMode);
 };
 
 // Builds a DeepNet from the subset of N2D2's INI format the quantized path needs

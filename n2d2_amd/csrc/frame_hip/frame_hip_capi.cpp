@@ -191,6 +191,89 @@ int fh_cell_set_scaling(void* net, const char* name, int mode, const void* scali
     });
 }
 
+// ---- ingestion of a trained / calibrated network (quantization.cpp)
+int fh_cell_import_free_parameters(void* net, const char* name, const char* fileName, int ignoreNotExists)
+{
+    return guarded([&] { ((Net*)net)->deepNet->getCell(name)->importFreeParameters(fileName, ignoreNotExists != 0); });
+}
+
+int fh_cell_export_free_parameters(void* net, const char* name, const char* fileName)
+{
+    return guarded([&] { ((Net*)net)->deepNet->getCell(name)->exportFreeParameters(fileName); });
+}
+
+// what = 0: weights, 1: biases.  Returns the element count through *n; copies when out has room for it.
+int fh_cell_get_free_parameters(void* net, const char* name, int what, float* out, size_t capacity, size_t* n)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        const Tensor<Float_T>* t = nullptr;
+        if (auto conv = std::dynamic_pointer_cast<ConvCell>(c)) t = what == 0 ? &conv->getWeights() : &conv->getBiases();
+        else if (auto fc = std::dynamic_pointer_cast<FcCell>(c)) t = what == 0 ? &fc->getWeights() : &fc->getBiases();
+        else throw std::runtime_error("fh_cell_get_free_parameters(): cell has no free parameters");
+        *n = t->empty() ? 0 : t->size();
+        if (out && capacity >= *n && *n > 0) std::memcpy(out, t->data(), *n * sizeof(float));
+    });
+}
+
+// mode: N2D2HIP_SCALING_FIXED_MULT16 / _FIXED_MULT32; *modeOut is the mode finally used
+int fh_approximate_scaling_with_fixed_point(int mode, const float* scaling, size_t n, int* modeOut, int* nbFractionalBits, std::int32_t* out)
+{
+    return guarded([&] {
+        ScalingMode m = mode == N2D2HIP_SCALING_FIXED_MULT16 ? ScalingMode::FIXED_MULT16 : ScalingMode::FIXED_MULT32;
+        const auto r = DeepNetQuantization::approximateScalingWithFixedPoint(m, std::vector<Float_T>(scaling, scaling + n));
+        *modeOut = m == ScalingMode::FIXED_MULT16 ? N2D2HIP_SCALING_FIXED_MULT16 : N2D2HIP_SCALING_FIXED_MULT32;
+        *nbFractionalBits = (int)r.first;
+        std::copy(r.second.begin(), r.second.end(), out);
+    });
+}
+
+int fh_approximate_scaling_with_power_of_2_divs(float scaling, int nbDivisions, unsigned char* exponents, double* precision)
+{
+    return guarded([&] {
+        const auto r = DeepNetQuantization::approximateScalingWithPowerOf2Divs(scaling, (size_t)nbDivisions);
+        std::copy(r.first.begin(), r.first.end(), exponents);
+        *precision = r.second;
+    });
+}
+
+// Turns the FLOAT_MULT scaling of the cell's activation into `mode` (N2D2HIP_SCALING_*), rescaling the cell's parameters
+// where the approximation overshoots
+int fh_cell_approximate_activation_scaling(void* net, const char* name, int mode)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        if (!c->getActivation()) throw std::runtime_error("fh_cell_approximate_activation_scaling(): cell has no activation");
+        static const ScalingMode modes[] = {ScalingMode::NONE, ScalingMode::FLOAT_MULT, ScalingMode::FIXED_MULT16, ScalingMode::FIXED_MULT32,
+                                            ScalingMode::SINGLE_SHIFT, ScalingMode::DOUBLE_SHIFT};
+        if (mode < 0 || mode > 5) throw std::runtime_error("Unsupported scaling mode.");
+        DeepNetQuantization::approximateActivationScaling(*c, *c->getActivation(), modes[mode]);
+    });
+}
+
+// The activation's Scaling: *mode (N2D2HIP_SCALING_*), *fracBits, and its per-output values as doubles (float factors,
+// fixed-point integers, shifts; two per output for DOUBLE_SHIFT); *n = number of values
+int fh_cell_get_scaling(void* net, const char* name, int* mode, int* fracBits, double* out, size_t capacity, size_t* n)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        if (!c->getActivation()) throw std::runtime_error("fh_cell_get_scaling(): cell has no activation");
+        const Scaling& s = c->getActivation()->getActivationScaling();
+        std::vector<double> v;
+        switch (s.getMode()) {
+        case ScalingMode::NONE: *mode = N2D2HIP_SCALING_NONE; break;
+        case ScalingMode::FLOAT_MULT: *mode = N2D2HIP_SCALING_FLOAT_MULT; v.assign(s.getFloatScalingPerOutput().begin(), s.getFloatScalingPerOutput().end()); break;
+        case ScalingMode::FIXED_MULT16: *mode = N2D2HIP_SCALING_FIXED_MULT16; v.assign(s.getFixedScalingPerOutput().begin(), s.getFixedScalingPerOutput().end()); break;
+        case ScalingMode::FIXED_MULT32: *mode = N2D2HIP_SCALING_FIXED_MULT32; v.assign(s.getFixedScalingPerOutput().begin(), s.getFixedScalingPerOutput().end()); break;
+        case ScalingMode::SINGLE_SHIFT: *mode = N2D2HIP_SCALING_SINGLE_SHIFT; v.assign(s.getShiftScalingPerOutput().begin(), s.getShiftScalingPerOutput().end()); break;
+        case ScalingMode::DOUBLE_SHIFT: *mode = N2D2HIP_SCALING_DOUBLE_SHIFT; v.assign(s.getShiftScalingPerOutput().begin(), s.getShiftScalingPerOutput().end()); break;
+        }
+        *fracBits = (int)s.getFractionalBits();
+        *n = v.size();
+        if (out && capacity >= v.size()) std::copy(v.begin(), v.end(), out);
+    });
+}
+
 int fh_cell_get_outputs(void* net, const char* name, float* out, size_t n)
 {
     return guarded([&] {

@@ -1,0 +1,315 @@
+// Host-side ingestion of a network N2D2 has trained or calibrated: free parameters from its text exports, and the
+// approximation of floating-point rescales by the integer Scaling modes.  Plain C++, no device code.
+#include "frame_hip.hpp"
+
+#include <algorithm>
+#include <cassert>
+#include <cctype>
+#include <fstream>
+#include <iomanip>
+
+namespace N2D2 {
+
+namespace {
+
+// Utils::fileBaseName / Utils::fileExtension (src/utils/Utils.cpp): the part before / after the last dot of the last
+// path component
+std::string fileBaseName(const std::string& fileName)
+{
+    const size_t slash = fileName.find_last_of("/\\");
+    const size_t dot = fileName.find_last_of('.');
+    return (dot == std::string::npos || (slash != std::string::npos && dot < slash)) ? fileName : fileName.substr(0, dot);
+}
+std::string fileExtension(const std::string& fileName)
+{
+    const size_t slash = fileName.find_last_of("/\\");
+    const size_t dot = fileName.find_last_of('.');
+    return (dot == std::string::npos || (slash != std::string::npos && dot < slash)) ? "" : fileName.substr(dot + 1);
+}
+
+struct SynapticFiles {
+    std::string weightsFile, biasesFile;
+    bool singleFile;
+    std::ifstream weights, biasesOwn;
+    bool opened;
+    std::istream& biases(bool noBias) { return (!singleFile && !noBias) ? biasesOwn : weights; }
+};
+
+// The file naming and opening rules shared by ConvCell and FcCell (src/Cell/ConvCell.cpp:511-549)
+void openSynapticFiles(SynapticFiles& f, const std::string& fileName, bool ignoreNotExists, bool noBias)
+{
+    const std::string fileBase = fileBaseName(fileName);
+    std::string fileExt = fileExtension(fileName);
+    if (!fileExt.empty())
+        fileExt = "." + fileExt;
+    f.singleFile = std::ifstream(fileName.c_str()).good();
+    f.weightsFile = f.singleFile ? fileName : fileBase + "_weights" + fileExt;
+    f.biasesFile = f.singleFile ? fileName : fileBase + "_biases" + fileExt;
+    f.opened = false;
+    f.weights.open(f.weightsFile.c_str());
+    if (!f.weights.good()) {
+        if (ignoreNotExists) {
+            std::cout << "Notice: Could not open synaptic file: " << f.weightsFile << std::endl;
+            return;
+        }
+        throw std::runtime_error("Could not open synaptic file: " + f.weightsFile);
+    }
+    if (!f.singleFile && !noBias) {
+        f.biasesOwn.open(f.biasesFile.c_str());
+        if (!f.biasesOwn.good())
+            throw std::runtime_error("Could not open synaptic file: " + f.biasesFile);
+    }
+    f.opened = true;
+}
+
+void expectEnd(std::istream& in, const std::string& name)
+{
+    while (std::isspace(in.peek()))
+        in.ignore();
+    if (in.get() != std::istream::traits_type::eof())
+        throw std::runtime_error("Synaptic file size larger than expected: " + name);
+}
+
+} // namespace
+
+// ------------------------------------------------------------------- ConvCell
+void ConvCell::importFreeParameters(const std::string& fileName, bool ignoreNotExists)
+{
+    if (mNbChannels == 0)
+        throw std::runtime_error("ConvCell::importFreeParameters(): connect cell " + mName + " before importing its parameters");
+    SynapticFiles f;
+    openSynapticFiles(f, fileName, ignoreNotExists, mNoBias);
+    if (!f.opened)
+        return;
+    std::istream& biases = f.biases(mNoBias);
+    const size_t cg = mNbChannels / mNbGroups;
+    const size_t kernelSize = (size_t)mKernelDims[0] * mKernelDims[1];
+    Tensor<Float_T> w({mKernelDims[0], mKernelDims[1], cg, mNbOutputs});
+    Tensor<Float_T> b({mNbOutputs});
+    double value;
+    for (size_t output = 0; output < mNbOutputs; ++output) {
+        // the channels of the output's group are its connections, in channel order
+        for (size_t channel = 0; channel < cg; ++channel) {
+            for (size_t index = 0; index < kernelSize; ++index) {
+                if (!(f.weights >> value))
+                    throw std::runtime_error("Error while reading synaptic file: " + f.weightsFile);
+                w(index + kernelSize * (channel + cg * output)) = (Float_T)value;
+            }
+        }
+        if (!mNoBias) {
+            if (!(biases >> value))
+                throw std::runtime_error("Error while reading synaptic file: " + f.biasesFile);
+            b(output) = (Float_T)value;
+        }
+    }
+    expectEnd(f.weights, f.weightsFile);
+    if (!f.singleFile && !mNoBias)
+        expectEnd(biases, f.biasesFile);
+    mWeights = w;
+    if (!mNoBias)
+        mBias = b;
+    mDirty = true;
+}
+
+void ConvCell::exportFreeParameters(const std::string& fileName) const
+{
+    const std::string fileBase = fileBaseName(fileName);
+    std::string fileExt = fileExtension(fileName);
+    if (!fileExt.empty())
+        fileExt = "." + fileExt;
+    const std::string weightsFile = fileBase + "_weights" + fileExt, biasesFile = fileBase + "_biases" + fileExt;
+    std::ofstream weights(weightsFile.c_str());
+    if (!weights.good())
+        throw std::runtime_error("Could not create synaptic file: " + weightsFile);
+    const size_t perOutput = mWeights.size() / std::max<size_t>(mNbOutputs, 1);
+    for (size_t output = 0; output < mNbOutputs; ++output) {
+        for (size_t i = 0; i < perOutput; ++i)
+            weights << std::setprecision(10) << mWeights(i + perOutput * output) << " ";
+        weights << "\n";
+    }
+    if (!mNoBias) {
+        std::ofstream biases(biasesFile.c_str());
+        if (!biases.good())
+            throw std::runtime_error("Could not create synaptic file: " + biasesFile);
+        for (size_t output = 0; output < mNbOutputs; ++output)
+            biases << std::setprecision(10) << mBias(output) << "\n";
+    }
+}
+
+void ConvCell::processFreeParametersPerOutput(const std::function<Float_T(Float_T)>& func, std::size_t output)
+{
+    const size_t perOutput = mWeights.size() / std::max<size_t>(mNbOutputs, 1);
+    for (size_t i = 0; i < perOutput; ++i)
+        mWeights(i + perOutput * output) = func(mWeights(i + perOutput * output));
+    if (!mNoBias && output < mBias.size())
+        mBias(output) = func(mBias(output));
+    mDirty = true;
+}
+
+// --------------------------------------------------------------------- FcCell
+void FcCell::importFreeParameters(const std::string& fileName, bool ignoreNotExists)
+{
+    const size_t channelsSize = (size_t)mNbChannels * mInW * mInH;
+    if (channelsSize == 0)
+        throw std::runtime_error("FcCell::importFreeParameters(): connect cell " + mName + " before importing its parameters");
+    SynapticFiles f;
+    openSynapticFiles(f, fileName, ignoreNotExists, mNoBias);
+    if (!f.opened)
+        return;
+    std::istream& biases = f.biases(mNoBias);
+    Tensor<Float_T> w({channelsSize, mNbOutputs});
+    Tensor<Float_T> b({mNbOutputs});
+    double value;
+    for (size_t output = 0; output < mNbOutputs; ++output) {
+        for (size_t channel = 0; channel < channelsSize; ++channel) {
+            if (!(f.weights >> value))
+                throw std::runtime_error("Error while reading synaptic file: " + fileName);
+            w(channel + channelsSize * output) = (Float_T)value;
+        }
+        if (!mNoBias) {
+            if (!(biases >> value))
+                throw std::runtime_error("Error while reading synaptic file: " + fileName);
+            b(output) = (Float_T)value;
+        }
+    }
+    expectEnd(f.weights, f.weightsFile);
+    if (!f.singleFile && !mNoBias)
+        expectEnd(biases, f.biasesFile);
+    mWeights = w;
+    if (!mNoBias)
+        mBias = b;
+    mDirty = true;
+}
+
+void FcCell::exportFreeParameters(const std::string& fileName) const
+{
+    const std::string fileBase = fileBaseName(fileName);
+    std::string fileExt = fileExtension(fileName);
+    if (!fileExt.empty())
+        fileExt = "." + fileExt;
+    const std::string weightsFile = fileBase + "_weights" + fileExt, biasesFile = fileBase + "_biases" + fileExt;
+    std::ofstream weights(weightsFile.c_str());
+    if (!weights.good())
+        throw std::runtime_error("Could not create synaptic file: " + weightsFile);
+    const size_t perOutput = mWeights.size() / std::max<size_t>(mNbOutputs, 1);
+    for (size_t output = 0; output < mNbOutputs; ++output) {
+        for (size_t i = 0; i < perOutput; ++i)
+            weights << std::setprecision(10) << mWeights(i + perOutput * output) << " ";
+        weights << "\n";
+    }
+    if (!mNoBias) {
+        std::ofstream biases(biasesFile.c_str());
+        if (!biases.good())
+            throw std::runtime_error("Could not create synaptic file: " + biasesFile);
+        for (size_t output = 0; output < mNbOutputs; ++output)
+            biases << std::setprecision(10) << mBias(output) << "\n";
+    }
+}
+
+void FcCell::processFreeParametersPerOutput(const std::function<Float_T(Float_T)>& func, std::size_t output)
+{
+    const size_t perOutput = mWeights.size() / std::max<size_t>(mNbOutputs, 1);
+    for (size_t i = 0; i < perOutput; ++i)
+        mWeights(i + perOutput * output) = func(mWeights(i + perOutput * output));
+    if (!mNoBias && output < mBias.size())
+        mBias(output) = func(mBias(output));
+    mDirty = true;
+}
+
+// -------------------------------------------------------- DeepNetQuantization
+std::pair<std::size_t, std::vector<std::int32_t> > DeepNetQuantization::approximateScalingWithFixedPoint(
+    ScalingMode& mode, const std::vector<Float_T>& scalingPerOutput)
+{
+    if (scalingPerOutput.empty())
+        throw std::runtime_error("approximateScalingWithFixedPoint(): no scaling");
+    const std::uint64_t limit = (mode == ScalingMode::FIXED_MULT16) ? (std::uint64_t)std::numeric_limits<std::int16_t>::max()
+                                                                    : (std::uint64_t)std::numeric_limits<std::int32_t>::max();
+    const double maxScaling = *std::max_element(scalingPerOutput.begin(), scalingPerOutput.end());
+    if (maxScaling >= limit) {
+        if (mode == ScalingMode::FIXED_MULT16) {
+            std::cout << "Warning: Max scaling (" << maxScaling << ") doesn't fit in FIXED_MULT16. Falling back to FIXED_MULT32." << std::endl;
+            mode = ScalingMode::FIXED_MULT32;
+            return approximateScalingWithFixedPoint(mode, scalingPerOutput);
+        }
+        std::stringstream errorStr;
+        errorStr << "Max scaling (" << maxScaling << ") doesn't fit in FIXED_MULT32." << std::endl;
+        throw std::runtime_error(errorStr.str());
+    }
+    const std::size_t maxNbFractionalBits = 50;
+    const std::size_t nbFractionalBits
+        = std::min((std::size_t)std::floor(std::log(limit / maxScaling) / std::log(2.0)), maxNbFractionalBits);
+    std::vector<std::int32_t> scalingFixedPoint;
+    for (Float_T sc : scalingPerOutput)
+        scalingFixedPoint.push_back((std::int32_t)std::round(sc * (1ull << nbFractionalBits)));
+    return std::make_pair(nbFractionalBits, scalingFixedPoint);
+}
+
+std::pair<std::vector<unsigned char>, double> DeepNetQuantization::approximateScalingWithPowerOf2Divs(Float_T scaling, std::size_t nbDivisions)
+{
+    static const double ROUNDING_THRESHOLD = 0.98;
+    if (nbDivisions == 0 || !(scaling > 0.0) || scaling > 1.0)
+        throw std::runtime_error("approximateScalingWithPowerOf2Divs(): needs 0 < scaling <= 1 and at least one division");
+    double precision = 0.0;
+    std::vector<unsigned char> powerOf2Divs(nbDivisions);
+    for (std::size_t iDiv = 0; iDiv < nbDivisions; ++iDiv) {
+        if (precision == 1.0) {
+            // the sum is exact already: split its last term into two equal halves
+            powerOf2Divs[iDiv - 1]++;
+            powerOf2Divs[iDiv] = powerOf2Divs[iDiv - 1];
+        } else {
+            const std::size_t exponent = (std::size_t)std::ceil(std::log2(1.0 / (scaling * (1.0 - precision))));
+            precision += 1.0 / (scaling * std::pow(2, exponent));
+            powerOf2Divs[iDiv] = static_cast<unsigned char>(exponent);
+        }
+    }
+    if (precision >= ROUNDING_THRESHOLD) {
+        precision = 1.0;
+    } else if (precision < 1.0) {
+        // too far below: double the last term, which takes the sum above the scaling
+        precision += 1.0 / (scaling * std::pow(2, powerOf2Divs.back()));
+        powerOf2Divs.back() = powerOf2Divs.back() - 1;
+    }
+    return std::make_pair(powerOf2Divs, precision);
+}
+
+void DeepNetQuantization::approximateActivationScaling(Cell& cell, Activation& activation, ScalingMode actScalingMode)
+{
+    if (activation.getActivationScaling().getMode() != ScalingMode::FLOAT_MULT)
+        throw std::runtime_error("approximateActivationScaling(): the activation of cell " + cell.getName() + " has no floating-point scaling");
+    const std::vector<Float_T> scalingPerOutput = activation.getActivationScaling().getFloatScalingPerOutput();
+    if ((actScalingMode == ScalingMode::SINGLE_SHIFT || actScalingMode == ScalingMode::DOUBLE_SHIFT)
+        && std::any_of(scalingPerOutput.begin(), scalingPerOutput.end(), [](Float_T s) { return s > 1.0; })) {
+        std::cout << "Warning: Scaling (" << scalingPerOutput[0] << ") > 1 for layer \"" << cell.getName()
+                  << "\" is not supported with Single/Double-shift scaling. Falling back to Fixed-point scaling for this layer." << std::endl;
+        actScalingMode = ScalingMode::FIXED_MULT16;
+    }
+    if (actScalingMode == ScalingMode::FLOAT_MULT) {
+        // nothing to do
+    } else if (actScalingMode == ScalingMode::FIXED_MULT32 || actScalingMode == ScalingMode::FIXED_MULT16) {
+        auto scalingFixedPoint = approximateScalingWithFixedPoint(actScalingMode, scalingPerOutput);
+        activation.setActivationScaling(Scaling::fixedPointScaling(actScalingMode, scalingFixedPoint.first, scalingFixedPoint.second, false,
+                                                                   std::vector<Float_T>(0)));
+    } else if (actScalingMode == ScalingMode::SINGLE_SHIFT || actScalingMode == ScalingMode::DOUBLE_SHIFT) {
+        const std::size_t nbDivisions = actScalingMode == ScalingMode::SINGLE_SHIFT ? 1 : 2;
+        std::vector<unsigned char> single;
+        std::vector<std::pair<unsigned char, unsigned char> > pairs;
+        for (std::size_t output = 0; output < scalingPerOutput.size(); ++output) {
+            const auto approx = approximateScalingWithPowerOf2Divs(scalingPerOutput[output], nbDivisions);
+            // the shifts scale by approx.second times too much: the cell's parameters take the difference
+            const Float_T rescaleOutputsBy = (Float_T)(1 / approx.second);
+            cell.processFreeParametersPerOutput([&](Float_T d) { return rescaleOutputsBy * d; }, output);
+            if (nbDivisions == 1)
+                single.push_back(approx.first[0]);
+            else
+                pairs.push_back({(unsigned char)(approx.first[1] - approx.first[0]), approx.first[1]});
+        }
+        if (nbDivisions == 1)
+            activation.setActivationScaling(Scaling::singleShiftScaling(single, false, std::vector<Float_T>(0)));
+        else
+            activation.setActivationScaling(Scaling::doubleShiftScaling(pairs, false, {std::make_pair((unsigned char)0, (unsigned char)0)}));
+    } else {
+        throw std::runtime_error("Unsupported scaling mode.");
+    }
+}
+
+} // namespace N2D2

@@ -38,6 +38,15 @@ lib.fh_lsq_cell_run.argtypes = [C.c_char_p, _P, _P, _SZ, _I, _F, _I, _P, _P, _P]
 lib.fh_lsq_act_run.argtypes = [C.c_char_p, _P, _P, _SZ, _I, _F, _I, _P, _P, _P]
 
 
+lib.fh_cell_import_free_parameters.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_int]
+lib.fh_cell_export_free_parameters.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
+lib.fh_cell_get_free_parameters.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]
+lib.fh_approximate_scaling_with_fixed_point.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p]
+lib.fh_approximate_scaling_with_power_of_2_divs.argtypes = [C.c_float, C.c_int, C.c_void_p, C.c_void_p]
+lib.fh_cell_approximate_activation_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+lib.fh_cell_get_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+
+
 class FrameHipError(RuntimeError):
     pass
 
@@ -55,6 +64,26 @@ def set_globals(precision, unsigned_data, env_data_unsigned):
 _MODE = {"None": capi.SCALING_NONE, "FloatMult": capi.SCALING_FLOAT_MULT, "FixedMult16": capi.SCALING_FIXED_MULT16,
          "FixedMult32": capi.SCALING_FIXED_MULT32, "SingleShift": capi.SCALING_SINGLE_SHIFT, "DoubleShift": capi.SCALING_DOUBLE_SHIFT}
 _MODE_DT = {"FloatMult": np.float32, "FixedMult16": np.int32, "FixedMult32": np.int32, "SingleShift": np.uint8, "DoubleShift": np.uint8}
+
+
+_MODE_NAME = {v: k for k, v in _MODE.items()}
+
+
+def approximate_scaling_with_fixed_point(mode, scaling_per_output):
+    """DeepNetQuantization::approximateScalingWithFixedPoint -> (mode finally used, nbFractionalBits, int32 factors)."""
+    sc = np.ascontiguousarray(scaling_per_output, dtype=np.float32)
+    out = np.zeros(sc.size, dtype=np.int32)
+    mode_out, bits = C.c_int(), C.c_int()
+    _check(lib.fh_approximate_scaling_with_fixed_point(_MODE[mode], sc.ctypes.data, sc.size, C.byref(mode_out), C.byref(bits), out.ctypes.data))
+    return _MODE_NAME[mode_out.value], bits.value, out
+
+
+def approximate_scaling_with_power_of_2_divs(scaling, nb_divisions):
+    """DeepNetQuantization::approximateScalingWithPowerOf2Divs -> (exponents, precision)."""
+    exps = np.zeros(max(int(nb_divisions), 1), dtype=np.uint8)
+    precision = C.c_double()
+    _check(lib.fh_approximate_scaling_with_power_of_2_divs(float(scaling), int(nb_divisions), exps.ctypes.data, C.byref(precision)))
+    return [int(e) for e in exps], precision.value
 
 
 class Net:
@@ -108,6 +137,39 @@ class Net:
         cl = None if clipping is None else np.ascontiguousarray(clipping, dtype=np.float32)
         _check(lib.fh_cell_set_scaling(self.h, name.encode(), _MODE[mode], s.ctypes.data, n, int(frac_bits), int(cl is not None),
                                        None if cl is None else cl.ctypes.data))
+
+    def import_free_parameters(self, name, file_name, ignore_not_exists=False):
+        """Cell::importFreeParameters: "<base>_weights<.ext>" (+ "<base>_biases<.ext>"), or one file with both."""
+        _check(lib.fh_cell_import_free_parameters(self.h, name.encode(), str(file_name).encode(), int(bool(ignore_not_exists))))
+
+    def export_free_parameters(self, name, file_name):
+        _check(lib.fh_cell_export_free_parameters(self.h, name.encode(), str(file_name).encode()))
+
+    def _free_parameters(self, name, what):
+        n = C.c_size_t()
+        _check(lib.fh_cell_get_free_parameters(self.h, name.encode(), what, None, 0, C.byref(n)))
+        out = np.zeros(n.value, dtype=np.float32)
+        _check(lib.fh_cell_get_free_parameters(self.h, name.encode(), what, out.ctypes.data, out.size, C.byref(n)))
+        return out
+
+    def weights(self, name):
+        """Flat float32 copy of the cell's weights, N2D2 order (conv: kernel x fastest, then y, channel, output)."""
+        return self._free_parameters(name, 0)
+
+    def biases(self, name):
+        return self._free_parameters(name, 1)
+
+    def approximate_activation_scaling(self, name, mode):
+        """DeepNetQuantization::approximateActivationScaling on the cell's FLOAT_MULT activation scaling."""
+        _check(lib.fh_cell_approximate_activation_scaling(self.h, name.encode(), _MODE[mode]))
+
+    def scaling(self, name):
+        """(mode, fractional bits, per-output values) of the cell's activation scaling."""
+        mode, frac, n = C.c_int(), C.c_int(), C.c_size_t()
+        _check(lib.fh_cell_get_scaling(self.h, name.encode(), C.byref(mode), C.byref(frac), None, 0, C.byref(n)))
+        out = np.zeros(n.value, dtype=np.float64)
+        _check(lib.fh_cell_get_scaling(self.h, name.encode(), C.byref(mode), C.byref(frac), out.ctypes.data, out.size, C.byref(n)))
+        return _MODE_NAME[mode.value], frac.value, out
 
     def initialize(self):
         _check(lib.fh_net_initialize(self.h))

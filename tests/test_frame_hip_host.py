@@ -122,3 +122,136 @@ def test_output_signedness_follows_the_export_globals(fh):
         assert not any(net.cell_info(n)["unsigned"] for n in uns)
     finally:
         fh.set_globals(0, True, False)
+
+
+# ------------------------------------------------------------------ ingestion of a trained / calibrated network
+
+LENET_INI = """
+DefaultModel=Frame_HIP
+
+[sp]
+SizeX=32
+SizeY=32
+NbChannels=1
+BatchSize=2
+
+[conv1]
+Input=sp
+Type=Conv
+KernelDims=5 5
+NbOutputs=6
+NoBias=1
+ActivationFunction=Rectifier
+
+[pool1]
+Input=conv1
+Type=Pool
+PoolDims=2 2
+NbOutputs=6
+Stride=2
+Pooling=Max
+
+[conv2]
+Input=pool1
+Type=Conv
+KernelDims=5 5
+NbOutputs=16
+ActivationFunction=Rectifier
+
+[fc2]
+Input=conv2
+Type=Fc
+NbOutputs=10
+NoBias=1
+ActivationFunction=Linear
+"""
+
+
+def test_free_parameters_are_read_from_the_reference_s_text_exports(fh, tmp_path):
+    """Files exported by N2D2 itself (held by its tests, tests/golden/sat_lenet4b): one line per output, OCHW."""
+    import os
+    import shutil
+    import numpy as np
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sat_lenet4b")
+    net = fh.Net(LENET_INI)
+    # conv1: 6 outputs x 1 channel x 5x5, no bias.  "<dir>/conv1.syntxt" names "<dir>/conv1_weights.syntxt".
+    net.import_free_parameters("conv1", os.path.join(golden, "conv1.syntxt"))
+    want = np.loadtxt(os.path.join(golden, "conv1_weights.syntxt"), dtype=np.float64).astype(np.float32)
+    assert want.shape == (6, 25)
+    assert np.array_equal(net.weights("conv1"), want.reshape(-1)) and net.biases("conv1").size == 0
+    # conv2 (16 x 6 x 5 x 5) has a bias here and the export holds none: the reference's error for the missing file
+    shutil.copy(os.path.join(golden, "conv2_weights.syntxt"), tmp_path / "conv2_weights.syntxt")
+    with pytest.raises(fh.FrameHipError) as e:
+        net.import_free_parameters("conv2", tmp_path / "conv2.syntxt")
+    assert str(e.value) == "Could not open synaptic file: %s" % (tmp_path / "conv2_biases.syntxt")
+    np.savetxt(tmp_path / "conv2_biases.syntxt", np.arange(16) * 0.5 - 3)
+    net.import_free_parameters("conv2", tmp_path / "conv2.syntxt")
+    want2 = np.loadtxt(os.path.join(golden, "conv2_weights.syntxt")).astype(np.float32)
+    assert want2.shape == (16, 150)
+    assert np.array_equal(net.weights("conv2"), want2.reshape(-1))
+    assert np.array_equal(net.biases("conv2"), (np.arange(16) * 0.5 - 3).astype(np.float32))
+    # one file holding weights then the bias of each output is read too (singleFile)
+    rows = [" ".join("%r" % float(v) for v in want2[o]) + " %r" % (o + 0.25) for o in range(16)]
+    (tmp_path / "both.syntxt").write_text("\n".join(rows) + "\n")
+    net.import_free_parameters("conv2", tmp_path / "both.syntxt")
+    assert np.array_equal(net.weights("conv2"), want2.reshape(-1)) and np.array_equal(net.biases("conv2"), np.arange(16, dtype=np.float32) + 0.25)
+    # the reference's other errors
+    with pytest.raises(fh.FrameHipError) as e:
+        net.import_free_parameters("conv1", tmp_path / "nothing.syntxt")
+    assert str(e.value) == "Could not open synaptic file: %s" % (tmp_path / "nothing_weights.syntxt")
+    net.import_free_parameters("conv1", tmp_path / "nothing.syntxt", ignore_not_exists=True)      # a notice, no error
+    (tmp_path / "short_weights.syntxt").write_text("1 2 3\n")
+    with pytest.raises(fh.FrameHipError) as e:
+        net.import_free_parameters("conv1", tmp_path / "short.syntxt")
+    assert "Error while reading synaptic file" in str(e.value)
+    (tmp_path / "long_weights.syntxt").write_text(" ".join(["1"] * 151) + "\n")
+    with pytest.raises(fh.FrameHipError) as e:
+        net.import_free_parameters("conv1", tmp_path / "long.syntxt")
+    assert "Synaptic file size larger than expected" in str(e.value)
+    assert np.array_equal(net.weights("conv1"), want.reshape(-1))                                  # a failed import changes nothing
+    # fc2: 10 outputs x 84 inputs would need an 84-input cell; here the cell has 16*10*10 inputs, so the file is short
+    with pytest.raises(fh.FrameHipError):
+        net.import_free_parameters("fc2", os.path.join(golden, "fc2.syntxt"))
+    # export -> import round trip, 10 significant digits as the reference writes quantized cells
+    net.export_free_parameters("conv2", tmp_path / "rt.syntxt")
+    before_w, before_b = net.weights("conv2"), net.biases("conv2")
+    net.import_free_parameters("conv2", tmp_path / "conv2.syntxt")
+    net.import_free_parameters("conv2", tmp_path / "rt.syntxt")
+    assert np.allclose(net.weights("conv2"), before_w, rtol=1e-9, atol=0) and np.array_equal(net.biases("conv2"), before_b)
+
+
+def test_float_rescales_become_integer_scalings_as_in_the_reference(fh):
+    """DeepNetQuantization::approximateActivationScaling: the Scaling that replaces a FLOAT_MULT one, and the per-output
+    correction of the cell's parameters for the shift modes, against the oracle's restatement."""
+    import numpy as np
+    from oracle import ptq_scaling as ref
+    rng = np.random.default_rng(17)
+    for mode in ("FixedMult16", "FixedMult32", "SingleShift", "DoubleShift", "FloatMult"):
+        net = fh.Net(LENET_INI)
+        w = rng.normal(0, 20, size=(16, 6, 5, 5)).astype(np.float32)
+        b = rng.normal(0, 100, size=16).astype(np.float32)
+        net.set_weights("conv2", w)
+        net.set_biases("conv2", b)
+        sc = np.exp(rng.uniform(-7, 0, size=16)).astype(np.float32)
+        net.set_scaling("conv2", "FloatMult", sc)
+        net.approximate_activation_scaling("conv2", mode)
+        want_mode, want_vals, want_bits, rescale = ref.approximate_activation_scaling(sc, mode)
+        got_mode, got_bits, got_vals = net.scaling("conv2")
+        assert got_mode == want_mode and got_bits == want_bits
+        assert np.array_equal(got_vals.reshape(np.asarray(want_vals).shape), np.asarray(want_vals, dtype=np.float64)), mode
+        assert np.array_equal(net.weights("conv2").reshape(16, -1), w.reshape(16, -1) * rescale[:, None]), mode
+        assert np.array_equal(net.biases("conv2"), b * rescale), mode
+        if mode == "DoubleShift":
+            # the pair is (difference, larger exponent): x * (2^-e0 + 2^-e1) = (x + (x << (e1 - e0))) >> e1
+            assert (got_vals.reshape(16, 2)[:, 0] <= got_vals.reshape(16, 2)[:, 1]).all()
+    # a factor above 1 cannot be a shift: the cell falls back to 16-bit fixed point, parameters untouched
+    net = fh.Net(LENET_INI)
+    w = rng.normal(0, 20, size=(16, 6, 5, 5)).astype(np.float32)
+    net.set_weights("conv2", w)
+    net.set_scaling("conv2", "FloatMult", np.linspace(0.5, 1.5, 16).astype(np.float32))
+    net.approximate_activation_scaling("conv2", "SingleShift")
+    mode, bits, vals = net.scaling("conv2")
+    assert mode == "FixedMult16" and bits == 14 and vals[-1] == 1.5 * 2 ** 14 and np.array_equal(net.weights("conv2"), w.reshape(-1))
+    # an activation without a floating-point scaling is refused
+    with pytest.raises(fh.FrameHipError):
+        net.approximate_activation_scaling("conv2", "SingleShift")

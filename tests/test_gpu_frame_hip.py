@@ -210,3 +210,42 @@ def test_lsq_quantizer_classes(fh):
     want_dx, want_sum = orc.lsq_backward(gx.astype(np.float64), x.astype(np.float64), float(np.float32(0.2)), 0, 15)
     assert np.array_equal(dx, want_dx.astype(np.float32))
     assert abs(st[1] - want_sum / np.sqrt(x.size * 15)) <= 1e-4 * abs(want_sum / np.sqrt(x.size * 15)) + 1e-7
+
+
+def test_float_rescaled_net_runs_after_approximation(fh, tmp_path):
+    """The ingestion path end to end: integer weights read from N2D2-format text files, FLOAT_MULT rescales (what a
+    calibration leaves) turned into 16-bit fixed point by DeepNetQuantization::approximateActivationScaling, the net
+    executed on the GPU, and the outputs compared with the CPU oracle running the approximated scalings."""
+    from n2d2_amd import nets
+    from oracle import cells
+    import copy
+    spec = copy.deepcopy(nets.lenet())
+    net = fh.Net(fh.spec_to_ini(spec, 8))
+    rng = np.random.default_rng(51)
+    for l in spec.layers:
+        if l.type not in ("conv", "fc"):
+            if l.type == "pool":
+                net.set_quantized(l.name, 8)
+            continue
+        # parameters through text files, as N2D2 exports them
+        np.savetxt(tmp_path / ("%s_weights.syntxt" % l.name), l.w.reshape(l.w.shape[0], -1), fmt="%d")
+        np.savetxt(tmp_path / ("%s_biases.syntxt" % l.name), l.bias, fmt="%d")
+        net.import_free_parameters(l.name, tmp_path / ("%s.syntxt" % l.name))
+        net.set_quantized(l.name, 8, l.act.nb_bits)
+        if l.act.mode == "None":
+            net.set_scaling(l.name, "None")
+            continue
+        scale = (np.asarray(l.act.scaling, dtype=np.float64) / 2.0 ** l.act.frac_bits * rng.uniform(0.8, 1.2, size=l.w.shape[0])).astype(np.float32)
+        net.set_scaling(l.name, "FloatMult", scale)
+        net.approximate_activation_scaling(l.name, "FixedMult16")
+        mode, bits, vals = net.scaling(l.name)
+        assert mode == "FixedMult16" and abs(vals).max() <= 32767 and abs(vals).max() > 16383
+        l.act.mode, l.act.frac_bits, l.act.scaling = mode, bits, vals.astype(np.int64)
+    x = rng.integers(0, 256, size=(8, 1, 32, 32))
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    keep = [l.name for l in spec.layers]
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        assert np.array_equal(net.outputs(name), want[name]), name
