@@ -547,3 +547,64 @@ def conv_spec_for(O, rng):
 def sum_spec_for(O, rng):
     from oracle.cells import ActSpec
     return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(0, 3, size=O)], 1), nb_bits=8, unsigned_out=True)
+
+
+def test_conv_randomized_sweep(rt):
+    """Seeded sweep over the pipelined kernel's shape space (channel counts that are multiples of 64, kernel sizes, strides,
+    paddings, dilations, ragged pixel counts, both input types, every integer rescale and both output signednesses, inputs
+    and outputs with and without a border of zeros), each case against the oracle bit for bit."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(20240607)
+    ncase = 0
+    for it in range(48):
+        C = int(rng.choice([64, 128, 192, 256, 320]))
+        O = int(rng.choice([16, 64, 96, 128, 192, 256]))
+        k = int(rng.choice([1, 1, 3, 3, 5]))
+        kh = k if rng.random() < 0.8 else int(rng.choice([1, 3]))
+        stride = int(rng.choice([1, 1, 2]))
+        pad = int(rng.integers(0, k // 2 + 2)) if k > 1 else int(rng.integers(0, 2))
+        dil = 2 if (k == 3 and rng.random() < 0.15) else 1
+        H, W = int(rng.integers(dil * (kh - 1) + 1, 15)), int(rng.integers(dil * (k - 1) + 1, 15))
+        B = int(rng.integers(1, 5))
+        signed_in = rng.random() < 0.3
+        x = rng.integers(-128, 128, size=(B, C, H, W)) if signed_in else rng.integers(0, 256, size=(B, C, H, W))
+        in_dt = capi.I8 if signed_in else capi.U8B
+        w = np.clip(np.rint(rng.normal(0, rng.choice([4, 20, 60]), size=(O, C, kh, k))), -127, 127).astype(np.int64)
+        bias = rng.integers(-5000, 5000, size=O) if rng.random() < 0.8 else None
+        unsigned_out = bool(rng.random() < 0.5)
+        kind = "Rectifier" if unsigned_out else "Linear"
+        mode = str(rng.choice(["SingleShift", "DoubleShift", "FixedMult16", "FixedMult32", "None"]))
+        if mode == "SingleShift":
+            spec = ActSpec(kind, mode, rng.integers(4, 18, size=O), nb_bits=8, unsigned_out=unsigned_out)
+        elif mode == "DoubleShift":
+            spec = ActSpec(kind, mode, np.stack([rng.integers(0, 5, size=O), rng.integers(6, 17, size=O)], 1), nb_bits=8, unsigned_out=unsigned_out)
+        elif mode == "FixedMult16":
+            spec = ActSpec(kind, mode, rng.integers(2 ** 6, 2 ** 15, size=O), frac_bits=int(rng.integers(14, 24)), nb_bits=8, unsigned_out=unsigned_out)
+        elif mode == "FixedMult32":
+            spec = ActSpec(kind, mode, rng.integers(2 ** 16, 2 ** 26, size=O), frac_bits=int(rng.integers(26, 36)), nb_bits=8, unsigned_out=unsigned_out)
+        else:
+            spec = ActSpec(kind, "None")
+        p4 = (pad, pad, pad, pad)
+        want = cells_ref.conv_cell(x.astype(np.float32), w, bias, spec, stride=(stride, stride), pad=p4, dil=(dil, dil))
+        if np.abs(want).max() >= 2 ** 24:
+            continue                                                    # the float-typed reference is exact below 2^24 only
+        want = want.astype(np.int64)
+        conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), in_dt, stride=(stride, stride), pad=p4, dil=(dil, dil))
+        tag = (it, C, O, k, kh, stride, pad, dil, H, W, B, mode, unsigned_out, signed_in)
+        _say("sweep %s" % (tag,))
+        dx = rt.DTensor.from_numpy(x, in_dt)
+        got = conv.forward(dx).to_numpy()
+        assert got.shape == want.shape and np.array_equal(got, want), tag
+        ncase += 1
+        if conv.accepts_halo() and dil == 1 and mode != "None":
+            # the same input stored with a border of zeros at least as wide as the padding, and a bordered output
+            halo_in, halo_out = max(pad, 1) + int(rng.integers(0, 2)), int(rng.integers(1, 3))
+            xin = rt.DTensor(B, C, H, W, in_dt, halo=halo_in)
+            view = xin.buf.view(B, H + 2 * halo_in, W + 2 * halo_in, xin.cs)
+            view[:, halo_in:H + halo_in, halo_in:W + halo_in, :] = dx.buf.view(B, H, W, dx.cs)
+            out = conv.make_output(dx, halo=halo_out)
+            conv.forward(xin, out)
+            assert np.array_equal(out.to_numpy(), want), ("halo", halo_in, halo_out) + tag
+    assert ncase >= 40
