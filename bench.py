@@ -53,8 +53,8 @@ def main():
                     help="run one 1 GiB device-to-device copy first (known traffic, to scale FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by batch, "
-              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by batch: one process "
+              "per GPU on its slice of the images, no exchange step)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
