@@ -101,3 +101,29 @@ def test_resnet50_full_batch_properties():
     assert np.array_equal(logits[:2], want)
     # a second forward over the same buffers reproduces the first
     assert np.array_equal(net.forward().to_numpy()[:, :, 0, 0], logits)
+
+
+def test_two_forwards_on_two_streams_agree_with_sequential_runs():
+    """Handles are independent: two networks launched on two streams at once (the benchmark's two-batches-in-flight mode)
+    give the bytes each gives alone."""
+    import torch
+    from n2d2_amd import nets
+    spec = nets.resnet50(image=96)
+    rng = np.random.default_rng(77)
+    xs = [rng.integers(0, 256, size=(6, 3, 96, 96)) for _ in range(2)]
+    gn = [nets.GpuNet(spec, 6) for _ in range(2)]
+    alone = []
+    for g, x in zip(gn, xs):
+        g.set_input(x)
+        alone.append(g.forward().to_numpy().copy())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    for _ in range(3):
+        for g, s in zip(gn, streams):
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                g.forward()
+        torch.cuda.synchronize()
+        for g, want in zip(gn, alone):
+            assert np.array_equal(g.tensors[spec.output].to_numpy(), want)
+    assert not np.array_equal(alone[0], alone[1])
