@@ -57,3 +57,25 @@ def test_invalid_arguments_are_rejected_before_any_device_work():
     assert b"Unsupported scaling propagation" in lib.n2d2hip_last_error()
     assert lib.n2d2hip_conv_forward(None, None, None, None) == capi.ERR_INVALID
     assert lib.n2d2hip_convert(None, None, None) == capi.ERR_INVALID
+
+
+def test_tensors_with_a_border_are_sized_and_policed_on_the_host():
+    """n2d2hip_tensor::halo: the byte count includes the border; entry points that do not take such tensors refuse them
+    before any device work; malformed borders are invalid everywhere."""
+    from n2d2_amd import capi
+    lib = capi.lib
+    fake = 0x1000                                                      # never dereferenced: validation comes first
+    t = capi.Tensor(fake, capi.U8B, capi.NHWC, 2, 64, 5, 7, 64, 0)
+    assert lib.n2d2hip_tensor_bytes(C.byref(t)) == 2 * 5 * 7 * 64
+    th = capi.Tensor(fake, capi.U8B, capi.NHWC, 2, 64, 5, 7, 64, 2)
+    assert lib.n2d2hip_tensor_bytes(C.byref(th)) == 2 * 9 * 11 * 64
+    p = capi.PoolDesc(capi.POOL_MAX, 2, 2, 2, 2, 0, 0)
+    out = capi.Tensor(fake, capi.U8B, capi.NHWC, 2, 64, 2, 3, 64, 0)
+    assert lib.n2d2hip_pool_forward(C.byref(p), C.byref(th), C.byref(out), None) == capi.ERR_UNSUPPORTED
+    assert b"halo" in lib.n2d2hip_last_error()
+    assert lib.n2d2hip_convert(C.byref(t), C.byref(th), None) == capi.ERR_UNSUPPORTED          # conversion reads a border, never writes one
+    bad = capi.Tensor(fake, capi.U8B, capi.NHWC, 2, 64, 5, 7, 64, -1)
+    assert lib.n2d2hip_tensor_clear(C.byref(bad), None) == capi.ERR_INVALID
+    nchw = capi.Tensor(fake, capi.I32, capi.NCHW, 2, 64, 5, 7, 64, 1)
+    assert lib.n2d2hip_tensor_clear(C.byref(nchw), None) == capi.ERR_INVALID                   # only NHWC byte tensors have one
+    assert lib.n2d2hip_conv_accepts_halo(None) == 0
