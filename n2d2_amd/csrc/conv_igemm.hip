@@ -863,6 +863,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         const bool small_m = bn128 && d.C % 128 == 0 && (bm_env ? atoi(bm_env) != 0 : tiles128 < (3 * num_cus()) / 2);
         // 64-channel layers whose K advances in 64-byte steps take 256-pixel tiles: twice the MFMAs per ring stage
         const bool wide64 = !bn128 && !other && d.C % 128 != 0 && Mll >= 256ll * 4 * num_cus();
+        // A handful of tiles (the classifier's FC): 64 x 64 tiles, four times as many blocks share the long K
+        const bool tiny = small_m && !other && ((Mll + 63) / 64) * a.ntiles_n * 8 < num_cus();
+        if (tiny) a.ntiles_n = (round_up(d.O, 16) + 63) / 64;
         const int BMp = small_m ? 64 : wide64 ? 256 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
         const int per_xcd = std::max(1, std::min((q.mtiles + 7) / 8, 2 * num_cus() / (8 * a.ntiles_n)));
@@ -906,6 +909,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             }
         } else if (wide64) {
             launch_pipe<4, 64, 2, 2, 4, 3>(q, all_valid, hi16, grid, stream);
+        } else if (tiny) {
+            q.c.ntiles_n = a.ntiles_n;
+            launch_pipe<4, 128, 1, 1, 2, 3>(q, all_valid, hi16, grid, stream);
         } else if (small_m) {
             launch_pipe<4, 128, 2, 1, 2, 3>(q, all_valid, hi16, grid, stream);
         } else if (d.C % 128 == 0) {
