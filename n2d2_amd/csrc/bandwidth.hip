@@ -142,7 +142,21 @@ __global__ __launch_bounds__(256) void global_avg_pool_kernel(const signed char*
     int acc[4] = {0, 0, 0, 0};
     if (c4 < cs) {
         const signed char* src = in + (long long)b * npix * cs + c4;
-        for (int p = wave; p < npix; p += 4) {
+        // the loads of several pixels are issued before the first one is consumed
+        int p = wave;
+        for (; p + 12 < npix; p += 16) {
+            int w[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                w[u] = *(const int*)(src + (long long)(p + 4 * u) * cs);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                int v[4];
+                unpack4(w[u] ^ (int)flip, zp, v);
+                acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
+            }
+        }
+        for (; p < npix; p += 4) {
             int v[4];
             unpack4(*(const int*)(src + (long long)p * cs) ^ (int)flip, zp, v);
             acc[0] += v[0]; acc[1] += v[1]; acc[2] += v[2]; acc[3] += v[3];
