@@ -33,6 +33,7 @@ static inline int iclamp_(int x, int lo, int hi) { return x < lo ? lo : (x > hi 
 #define COSH coshf
 #define FABS fabsf
 #define SQRT sqrtf
+#define EXP expf
 #include "frame_oracle_impl.inc"
 #undef T
 #undef FN
@@ -42,6 +43,7 @@ static inline int iclamp_(int x, int lo, int hi) { return x < lo ? lo : (x > hi 
 #undef COSH
 #undef FABS
 #undef SQRT
+#undef EXP
 
 #define T double
 #define FN(name) CAT(oracle_, CAT(name, _f64))
@@ -51,6 +53,7 @@ static inline int iclamp_(int x, int lo, int hi) { return x < lo ? lo : (x > hi 
 #define COSH cosh
 #define FABS fabs
 #define SQRT sqrt
+#define EXP exp
 #include "frame_oracle_impl.inc"
 #undef T
 #undef FN

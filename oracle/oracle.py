@@ -112,6 +112,76 @@ def conv_forward_bias(out, bias, alpha=1.0, beta=1.0):
     return out
 
 
+def _maps_groups(maps):
+    if maps is None:
+        return None, 1
+    m = np.ascontiguousarray(maps, dtype=np.uint8)
+    groups = get_nb_groups(m)
+    if groups < 0:
+        raise ValueError("irregular mapping")
+    return m, groups
+
+
+def conv_backward_data(w, dy, x_shape, stride=(1, 1), pad=(0, 0, 0, 0), maps=None, dx=None, alpha=1.0, beta=0.0,
+                       sub=(1, 1)):
+    """ConvCell_Frame_Kernels::backwardData. w [O,Cw,kH,kW], dy [B,O,oH,oW]; returns dx of x_shape [B,C,H,W]."""
+    dt = dy.dtype
+    w = np.ascontiguousarray(w, dtype=dt)
+    dy = np.ascontiguousarray(dy)
+    B, Cin, H, W = x_shape
+    O, Cw, kH, kW = w.shape
+    assert dy.shape[:2] == (B, O)
+    if dx is None:
+        dx = np.zeros(x_shape, dtype=dt)
+    m, groups = _maps_groups(maps)
+    ct = _CT[np.dtype(dt)]
+    a, b = ct(alpha), ct(beta)
+    _fn("conv_backward_data", dt)(C.byref(a), _p(w), kW, kH, Cw, O, _p(dy), dy.shape[3], dy.shape[2], B,
+                                  _ia(stride), _ia(pad), _ia(sub), C.byref(b), _p(dx), Cin, H, W, _p(m), groups)
+    return dx
+
+
+def conv_backward_filter(x, dy, w_shape, stride=(1, 1), pad=(0, 0, 0, 0), maps=None, dw=None, alpha=1.0, beta=0.0,
+                         sub=(1, 1)):
+    """ConvCell_Frame_Kernels::backwardFilter. x [B,C,H,W], dy [B,O,oH,oW]; returns dw of w_shape [O,Cw,kH,kW]."""
+    dt = x.dtype
+    x = np.ascontiguousarray(x)
+    dy = np.ascontiguousarray(dy, dtype=dt)
+    B, Cin, H, W = x.shape
+    O, Cw, kH, kW = w_shape
+    assert dy.shape[:2] == (B, O)
+    if dw is None:
+        dw = np.zeros(w_shape, dtype=dt)
+    m, groups = _maps_groups(maps)
+    ct = _CT[np.dtype(dt)]
+    a, b = ct(alpha), ct(beta)
+    _fn("conv_backward_filter", dt)(C.byref(a), _p(x), B, Cin, H, W, _p(dy), dy.shape[3], dy.shape[2], O,
+                                    _ia(stride), _ia(pad), _ia(sub), C.byref(b), _p(dw), kW, kH, Cw, _p(m), groups)
+    return dw
+
+
+def conv_backward_bias(dy, db=None, alpha=1.0, beta=0.0):
+    """ConvCell_Frame_Kernels::backwardBias. dy [B,O,oH,oW]; returns db [O]."""
+    dt = dy.dtype
+    dy = np.ascontiguousarray(dy)
+    B, O, oH, oW = dy.shape
+    if db is None:
+        db = np.zeros(O, dtype=dt)
+    ct = _CT[np.dtype(dt)]
+    a, b = ct(alpha), ct(beta)
+    _fn("conv_backward_bias", dt)(C.byref(a), _p(dy), oW, oH, O, B, C.byref(b), _p(db))
+    return db
+
+
+def softmax_forward(x):
+    """SoftmaxCell_Frame::propagate over the channels of x [B,C,H,W]."""
+    x = np.ascontiguousarray(x)
+    out = np.empty_like(x)
+    B, Cn, H, W = x.shape
+    _fn("softmax_forward", x.dtype)(_p(x), _p(out), B, Cn, H, W)
+    return out
+
+
 def fc_forward(x, w, bias=None, out=None, beta=0.0):
     """FcCell_Frame::propagate inner loop. x [B, ...] (CHW flattened), w [O,K]."""
     dt = x.dtype

@@ -1,0 +1,221 @@
+"""CPU oracle (TEST INFRASTRUCTURE, not the product) of the float cells a
+quantization-aware training step runs through: restatement of the reference's
+Frame classes around the kernels of oracle.py, for a sequential net of
+ActivationCell / ConvCell / SoftmaxCell with SAT quantizers and SGD solvers.
+
+Data is float32 as in the `<float>` instantiations; "diff" tensors carry the
+descent direction (target - output at the loss), so a solver *adds*
+rate * diff.  Cited paths are relative to the N2D2 source tree.
+"""
+import numpy as np
+
+from . import oracle as o
+
+F = np.float32
+
+
+class SGDSolver:
+    """src/Solver/SGDSolver.cpp:26-41 (defaults), :99-189 (getLearningRate, policy None) and
+    include/Solver/SGDSolver_Frame.hpp:77-146 (update)."""
+
+    def __init__(self, learning_rate=0.01, momentum=0.0, decay=0.0, iteration_size=1):
+        self.learning_rate, self.momentum, self.decay, self.iteration_size = learning_rate, momentum, decay, iteration_size
+        self.iteration_pass = 0
+        self.nb_iterations = 0
+        self.momentum_data = None
+
+    def is_new_iteration(self):
+        return self.iteration_pass == 0
+
+    def get_learning_rate(self):
+        if self.learning_rate == 0.0:
+            return 0.0
+        if self.iteration_pass < self.iteration_size - 1:
+            self.iteration_pass += 1
+            return 0.0
+        self.iteration_pass = 0
+        self.nb_iterations += 1
+        return self.learning_rate
+
+    def update(self, data, diff, batch_size):
+        """data (float32 array, updated in place) += rate / (batch * iterationSize) * diff."""
+        rate = F(self.get_learning_rate())
+        if rate == 0.0:
+            return
+        rate_diff = F(rate / F(F(batch_size) * F(self.iteration_size)))
+        if self.momentum == 0.0 and self.decay == 0.0:
+            data += rate_diff * diff.astype(F)
+            return
+        if self.momentum_data is None:
+            self.momentum_data = np.zeros_like(data)
+        m = self.momentum_data
+        m *= F(self.momentum)
+        m += rate_diff * diff.astype(F)
+        if self.decay != 0.0:
+            m += F(-F(self.decay) * rate) * data
+        data += m
+
+
+class SATQuantizerActivation:
+    """src/Quantizer/QAT/Activation/SAT/SATQuantizerActivation_Frame.cpp:73-143: one alpha for the whole
+    tensor, created at the first propagate; its gradient is the element-order sum of the per-element terms
+    (+ the previous value while the solver is inside an iteration); update() hands it to the solver."""
+
+    def __init__(self, rng, alpha, solver=None):
+        self.range, self.alpha_parameter = rng, alpha
+        self.alphas = None
+        self.diff_alphas = F(0.0)
+        self.full_precision = None
+        self.solver = solver or SGDSolver()
+
+    def propagate(self, x, inference):
+        if self.alphas is None:
+            self.alphas = np.full(1, self.alpha_parameter, dtype=F)
+        y, fp = o.sat_act_forward(x, self.range, float(self.alphas[0]), inference=inference)
+        if not inference:
+            self.full_precision = fp
+        return y
+
+    def back_propagate(self, diff_input):
+        beta = 0.0 if self.solver.is_new_iteration() else 1.0
+        dx, da, _ = o.sat_act_backward(diff_input, self.full_precision, self.range, float(self.alphas[0]),
+                                       beta=beta, prev_diff_alpha=float(self.diff_alphas))
+        self.diff_alphas = F(da)
+        return dx
+
+    def update(self, batch_size):
+        self.solver.update(self.alphas, np.full(1, self.diff_alphas, dtype=F), batch_size)
+
+
+class LinearActivation:
+    """include/Activation/LinearActivation_Frame.hpp:56-134 without Scaling and Clipping: the quantizer, if any, is all
+    that acts, forward and backward."""
+
+    def __init__(self, quantizer=None):
+        self.quantizer = quantizer
+
+    def propagate(self, x, inference):
+        return self.quantizer.propagate(x, inference) if self.quantizer else x
+
+    def back_propagate(self, diff_input):
+        return self.quantizer.back_propagate(diff_input) if self.quantizer else diff_input
+
+    def update(self, batch_size):
+        if self.quantizer:
+            self.quantizer.update(batch_size)
+
+
+class SATQuantizerCell:
+    """src/Quantizer/QAT/Cell/SAT/SATQuantizerCell_Frame.cpp:178-294: the weights are quantized again at every
+    propagate; backward scales by factor = max|tanh(w)| * scaling of that propagate; nothing to update."""
+
+    def __init__(self, rng, quantization=True, scaling=False, mode="default"):
+        self.range, self.quantization, self.scaling, self.mode = rng, quantization, scaling, mode
+        self.tanh_max, self.sat_scaling = 0.0, 1.0
+
+    def propagate(self, w, outputs_size):
+        mode = self.mode if self.quantization else {"asymrange": "none_asym"}.get(self.mode, "none")
+        wq, self.tanh_max, self.sat_scaling = o.sat_weight_forward(w, self.range, mode, self.scaling, outputs_size)
+        return wq
+
+    def back_propagate(self, dwq, w):
+        scale = self.sat_scaling if self.scaling else 1.0
+        return o.sat_weight_backward(dwq, w, self.range, float(F(F(self.tanh_max) * F(scale))),
+                                     self.mode if self.mode in ("fullrange", "asymrange") else "default")
+
+
+class ActivationCell:
+    """src/Cell/ActivationCell_Frame.cpp:95-205, one input: copy, then the activation in place."""
+
+    def __init__(self, activation):
+        self.activation = activation
+        self.outputs = None
+        self.diff_inputs = None      # written by the next cell's backPropagate
+        self.diff_outputs = None
+
+    def propagate(self, x, inference=False):
+        self.outputs = self.activation.propagate(np.array(x, dtype=F), inference)
+        return self.outputs
+
+    def back_propagate(self):
+        self.diff_outputs = self.activation.back_propagate(self.diff_inputs)
+        return self.diff_outputs
+
+    def update(self, batch_size):
+        self.activation.update(batch_size)
+
+
+class ConvCell:
+    """src/Cell/ConvCell_Frame.cpp:418-597 with one input and NoBias: propagate = quantize the weights, convolve, then
+    the activation in place; backPropagate = activation, backwardFilter on the quantized weights' gradient, backwardData
+    with the quantized weights, then the weight quantizer's backward; update = solver on the full-precision weights with
+    the quantizer's gradient, then the activation's quantizer."""
+
+    def __init__(self, weights, stride=(1, 1), pad=(0, 0, 0, 0), maps=None, activation=None, quantizer=None, solver=None):
+        self.w = np.array(weights, dtype=F)
+        self.stride, self.pad, self.maps = stride, pad, maps
+        self.activation, self.quantizer = activation, quantizer
+        self.solver = solver or SGDSolver()
+        self.diff_inputs = None
+
+    def propagate(self, x, inference=False):
+        self.x = x
+        O, Cw, kH, kW = self.w.shape
+        # mOutputsSize: dimB * dimY * dimX of the weight tensor {kW,kH,Cw,O} (SATQuantizerCell_Frame.cpp:80)
+        self.wq = self.quantizer.propagate(self.w, O * kH * kW) if self.quantizer else self.w
+        y = o.conv_forward(x, self.wq, stride=self.stride, pad=self.pad, maps=self.maps)
+        self.outputs = self.activation.propagate(y, inference) if self.activation else y
+        return self.outputs
+
+    def back_propagate(self):
+        d = self.diff_inputs
+        if self.activation:
+            d = self.activation.back_propagate(d)
+        self.diff_wq = o.conv_backward_filter(self.x, d, self.w.shape, stride=self.stride, pad=self.pad, maps=self.maps)
+        dx = o.conv_backward_data(self.wq, d, self.x.shape, stride=self.stride, pad=self.pad, maps=self.maps)
+        self.diff_w = self.quantizer.back_propagate(self.diff_wq, self.w) if self.quantizer else self.diff_wq
+        return dx
+
+    def update(self, batch_size):
+        self.solver.update(self.w, self.diff_w, batch_size)
+        if self.activation:
+            self.activation.update(batch_size)
+
+
+class SoftmaxCell:
+    """src/Cell/SoftmaxCell_Frame.cpp:93-137 and :140-207 with WithLoss: the gradient passes through unchanged;
+    applyLoss is Cell_Frame_Top::applyLoss (src/Cell/Cell_Frame_Top.cpp:27-40): diff = target - output, formed in
+    double and stored in T, loss = sum of squares / batch."""
+
+    def propagate(self, x):
+        self.outputs = o.softmax_forward(x)
+        return self.outputs
+
+    def apply_loss(self, targets):
+        err = targets.astype(np.float64) - self.outputs.astype(np.float64)
+        self.diff_inputs = err.astype(F)
+        return float((err * err).sum() / self.outputs.shape[0])
+
+    def back_propagate(self):
+        return self.diff_inputs
+
+
+def train_sequential(x, cells, softmax, targets, iterations):
+    """The loop of tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp:436-513: propagate front to back, loss, backPropagate
+    back to front (each cell's result is the previous cell's diffInputs), then update back to front with the
+    ActivationCell last."""
+    batch = x.shape[0]
+    loss = 0.0
+    for _ in range(iterations):
+        h = x
+        for c in cells:
+            h = c.propagate(h, inference=False)
+        softmax.propagate(h)
+        loss = softmax.apply_loss(targets)
+        d = softmax.back_propagate()
+        for c in reversed(cells):
+            c.diff_inputs = d
+            d = c.back_propagate()
+        for c in reversed(cells):
+            c.update(batch)
+    return loss

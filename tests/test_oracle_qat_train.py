@@ -1,0 +1,145 @@
+"""Pins the training part of the CPU oracle (float conv backward, softmax, loss, SGD, the SAT quantizers' backward
+and update) two ways: what the mathematics fixes (the backward kernels are the adjoints of the forward one, checked
+with dot products and against a Jacobian built from unit impulses), and the reference's own known-answer test: the
+three SAT alphas after 10 000 iterations on a hand-written three-convolution net, constants derived from PyTorch by
+the reference's authors (tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp:68-516, delta 0.01)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as o
+from oracle import qat_train as q
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sat_three_conv", "case.json")
+
+CASES = [  # B, C, H, W, O, k, stride, pad, groups
+    (2, 3, 7, 6, 4, 3, 1, 1, 1), (2, 4, 9, 9, 4, 3, 2, 1, 4), (1, 2, 5, 5, 3, 1, 1, 0, 1), (2, 3, 10, 9, 2, 5, 2, 2, 1),
+    (2, 2, 6, 6, 2, 3, 1, 0, 1), (3, 5, 8, 8, 5, 3, 1, 1, 5), (1, 3, 9, 7, 2, 3, 3, 0, 1), (2, 2, 4, 4, 3, 2, 2, 0, 1)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_backward_kernels_are_the_adjoints_of_forward(case):
+    B, C, H, W, O, k, s, p, groups = case
+    rng = np.random.default_rng(sum(case))
+    maps = None if groups == 1 else o.group_maps(C, O, groups)
+    kw = dict(stride=(s, s), pad=(p, p, p, p), maps=maps)
+    x = rng.normal(size=(B, C, H, W))
+    w = rng.normal(size=(O, C // groups, k, k))
+    y = o.conv_forward(x, w, **kw)
+    dy = rng.normal(size=y.shape)
+    dx = o.conv_backward_data(w, dy, x.shape, **kw)
+    dw = o.conv_backward_filter(x, dy, w.shape, **kw)
+    ref = (y * dy).sum()
+    assert abs(ref - (x * dx).sum()) < 1e-10 * max(1.0, abs(ref))
+    assert abs(ref - (w * dw).sum()) < 1e-10 * max(1.0, abs(ref))
+    # alpha / beta accumulate as in the forward kernel
+    old = rng.normal(size=w.shape)
+    acc = o.conv_backward_filter(x, dy, w.shape, dw=old.copy(), alpha=0.5, beta=2.0, **kw)
+    np.testing.assert_allclose(acc, 0.5 * dw + 2.0 * old, rtol=1e-12, atol=1e-12)
+    oldx = rng.normal(size=x.shape)
+    accx = o.conv_backward_data(w, dy, x.shape, dx=oldx.copy(), alpha=0.5, beta=2.0, **kw)
+    np.testing.assert_allclose(accx, 0.5 * dx + 2.0 * oldx, rtol=1e-12, atol=1e-12)
+    db = o.conv_backward_bias(dy)
+    np.testing.assert_allclose(db, dy.sum(axis=(0, 2, 3)), rtol=1e-12, atol=1e-12)
+
+
+def test_backward_data_against_the_jacobian_of_forward():
+    """Column j of the (linear) forward map is forward(unit impulse j); backward data must be its transpose times dy.
+    Covers the unrolled 3x3 stride-1 branch (interior pixels) and the generic one (borders) in one tensor."""
+    rng = np.random.default_rng(5)
+    B, C, H, W, O = 1, 2, 5, 5, 2
+    w = rng.normal(size=(O, C, 3, 3))
+    for pad, stride in ((1, 1), (0, 1), (1, 2)):
+        kw = dict(stride=(stride, stride), pad=(pad,) * 4)
+        cols = []
+        for j in range(C * H * W):
+            e = np.zeros(C * H * W)
+            e[j] = 1.0
+            cols.append(o.conv_forward(e.reshape(1, C, H, W), w, **kw).ravel())
+        J = np.stack(cols, axis=1)                      # [outputs, inputs]
+        dy = rng.normal(size=(J.shape[0],))
+        oh = int(np.sqrt(J.shape[0] // O))
+        dx = o.conv_backward_data(w, dy.reshape(1, O, oh, oh), (B, C, H, W), **kw)
+        np.testing.assert_allclose(dx.ravel(), J.T @ dy, rtol=1e-12, atol=1e-12)
+
+
+def test_grouped_backward_data_follows_the_reference_only_where_it_is_right():
+    """backwardData indexes the weight's channel by a count of connected *outputs* (ConvCell_Frame_Kernels.cpp:233,
+    :330): the adjoint for one output per group (depthwise) and without groups, not for wider groups. The restatement
+    keeps that; the product accepts depthwise and ungrouped convolutions only."""
+    rng = np.random.default_rng(9)
+    x = rng.normal(size=(2, 6, 8, 8))
+    w = rng.normal(size=(4, 3, 3, 3))
+    maps = o.group_maps(6, 4, 2)
+    y = o.conv_forward(x, w, maps=maps)
+    dy = rng.normal(size=y.shape)
+    dx = o.conv_backward_data(w, dy, x.shape, maps=maps)
+    assert abs((y * dy).sum() - (x * dx).sum()) > 1e-3
+
+
+def test_softmax_and_loss():
+    rng = np.random.default_rng(2)
+    x = rng.normal(size=(3, 5, 2, 2)).astype(np.float32) * 4
+    y = o.softmax_forward(x)
+    e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(y, e / e.sum(axis=1, keepdims=True), rtol=2e-6)
+    np.testing.assert_allclose(y.sum(axis=1), 1.0, rtol=1e-6)
+    sm = q.SoftmaxCell()
+    sm.propagate(x)
+    t = np.zeros_like(x)
+    t[:, 1] = 1
+    loss = sm.apply_loss(t)
+    assert abs(loss - ((t - y.astype(np.float64)) ** 2).sum() / 3) < 1e-12
+    assert np.array_equal(sm.back_propagate(), (t.astype(np.float64) - y).astype(np.float32))
+
+
+def test_sgd_solver_update():
+    s = q.SGDSolver()
+    d = np.array([1.0, -2.0], dtype=np.float32)
+    s.update(d, np.array([4.0, 4.0], dtype=np.float32), 2)
+    np.testing.assert_allclose(d, [1.02, -1.98], rtol=1e-7)          # + 0.01 / 2 * diff
+    assert s.nb_iterations == 1 and s.is_new_iteration()
+    m = q.SGDSolver(learning_rate=0.1, momentum=0.9, decay=0.01)
+    d = np.array([1.0], dtype=np.float32)
+    g = np.array([2.0], dtype=np.float32)
+    m.update(d, g, 1)      # v = 0.1*2 - 0.01*0.1*1 = 0.199
+    m.update(d, g, 1)      # v = 0.9*0.199 + 0.2 - 0.001*1.199
+    v1 = 0.199
+    v2 = 0.9 * v1 + 0.2 - 0.001 * (1 + v1)
+    np.testing.assert_allclose(d, [1 + v1 + v2], rtol=1e-6)
+    acc = q.SGDSolver(iteration_size=2)                               # every second call applies
+    d = np.array([0.0], dtype=np.float32)
+    acc.update(d, g, 1)
+    assert d[0] == 0.0 and not acc.is_new_iteration()
+    acc.update(d, g, 1)
+    np.testing.assert_allclose(d, [0.01 / 2 * 2.0], rtol=1e-6)
+
+
+def sat_three_conv_net(case):
+    x = (np.array(case["input_times_255"], dtype=np.float32) / np.float32(255.0)).reshape(2, 1, 5, 5)
+    qa = [q.SATQuantizerActivation(case["range_activation1"], case["alpha_init"]),
+          q.SATQuantizerActivation(case["range_conv"], case["alpha_init"]),
+          q.SATQuantizerActivation(case["range_conv"], case["alpha_init"])]
+    cells = [q.ActivationCell(q.LinearActivation(qa[0])),
+             q.ConvCell(np.array(case["conv1_weights"]).reshape(1, 1, 3, 3), activation=q.LinearActivation(qa[1]),
+                        quantizer=q.SATQuantizerCell(case["range_activation1"])),
+             q.ConvCell(np.array(case["conv2_weights"]).reshape(4, 1, 1, 1), activation=q.LinearActivation(qa[2]),
+                        quantizer=q.SATQuantizerCell(case["range_conv"])),
+             q.ConvCell(np.array(case["conv3_weights"]).reshape(4, 1, 3, 3), maps=np.eye(4, dtype=np.uint8),
+                        quantizer=q.SATQuantizerCell(case["range_conv"]))]
+    t = np.zeros((2, 4, 1, 1), dtype=np.float32)
+    for b, k in enumerate(case["target_class"]):
+        t[b, k] = 1
+    return x, cells, qa, t
+
+
+def test_known_answer_sat_alphas_after_training():
+    case = json.load(open(GOLD))
+    x, cells, qa, t = sat_three_conv_net(case)
+    loss = q.train_sequential(x, cells, q.SoftmaxCell(), t, case["iterations"])
+    got = {"activation1": float(qa[0].alphas[0]), "conv1": float(qa[1].alphas[0]), "conv2": float(qa[2].alphas[0])}
+    print("alphas", got, "loss", loss)
+    for name, want in case["expected_alpha"].items():
+        assert abs(got[name] - want) < case["delta"], (name, got[name], want)
