@@ -264,6 +264,49 @@ int n2d2hip_lsq_backward(const float* diff_q, const float* fp_x, float* diff_fp,
                          int lo, int hi, float grad_scale, float beta, float* diff_step,
                          void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
 
+/* ------------------------------------------- float cells of a training step */
+/* The float32 cells a quantization-aware training graph runs between the fake-quant kernels above.  Tensors are
+ * N2D2's own: activations NCHW ({X,Y,Z,B}, X fastest), weights OCHW ({kW,kH,C/groups,O}); `desc->weight_bits` is not
+ * read; groups is 1 or C == O (depthwise).  "diff" tensors carry the descent direction, as in the reference
+ * (target - output at the loss), so the solver adds rate * diff.
+ *
+ * y = conv(x, w) (+ bias[o] if bias != NULL) + beta * y; the window is clipped at the borders and a full 3x3 window
+ * is summed row by row (ref: src/Cell/ConvCell_Frame_Kernels.cpp:26-174, called from
+ * ConvCell_Frame<T>::propagate, src/Cell/ConvCell_Frame.cpp:418-473). */
+int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* w,
+                               const float* bias, float beta, float* y, n2d2hip_stream_t stream);
+/* diff_x = backwardData(w, diff_y) + beta * diff_x (ref: src/Cell/ConvCell_Frame_Kernels.cpp:176-333).  Dilation
+ * must be 1: the reference's backward kernels do not read it. */
+int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* w,
+                                     const float* diff_y, float beta, float* diff_x, n2d2hip_stream_t stream);
+/* diff_w = backwardFilter(x, diff_y) + beta * diff_w (ref: src/Cell/ConvCell_Frame_Kernels.cpp:335-427). */
+int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x,
+                                       const float* diff_y, float beta, float* diff_w, n2d2hip_stream_t stream);
+/* diff_bias[o] = sum over batch and pixels of diff_y + beta * diff_bias (ref: ...ConvCell_Frame_Kernels.cpp:429-452). */
+int n2d2hip_conv2d_f32_backward_bias(int B, int O, int oH, int oW, const float* diff_y, float beta, float* diff_bias,
+                                     n2d2hip_stream_t stream);
+/* Rectifier of an unquantized cell, in place: x > 0 ? (clipping > 0 ? min(x, clipping) : x) : leak_slope * x, and its
+ * backward diff_out = diff_in * (output == clipping ? 0 : output > 0 ? 1 : leak_slope), where `output` is what the cell
+ * holds after its activation and the activation's quantizer (ref: include/Activation/RectifierActivation_Frame.hpp:55-139;
+ * diff_in and diff_out may be the same buffer). */
+int n2d2hip_rectifier_f32_forward(float* x, size_t n, float leak_slope, float clipping, n2d2hip_stream_t stream);
+int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, float* diff_out, size_t n, float leak_slope,
+                                   float clipping, n2d2hip_stream_t stream);
+/* Softmax over the channels of each pixel, one group (ref: src/Cell/SoftmaxCell_Frame.cpp:93-137). */
+int n2d2hip_softmax_f32_forward(const float* x, float* y, int B, int C, int H, int W, n2d2hip_stream_t stream);
+/* diff = target - output, formed in double; loss[0] (device double) = sum of squares / batch
+ * (ref: Cell_Frame_Top::applyLoss, src/Cell/Cell_Frame_Top.cpp:27-40). */
+size_t n2d2hip_loss_workspace_bytes(size_t n);
+int n2d2hip_loss_f32(const float* target, const float* output, float* diff, size_t n, int batch, double* loss,
+                     void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
+/* One SGDSolver_Frame<float>::update on a device tensor (ref: include/Solver/SGDSolver_Frame.hpp:77-146):
+ * momentum_data == NULL: data += rate_diff * diff; otherwise m = m * momentum + rate_diff * diff
+ * - decay_times_rate * data, data += m.  rate_diff = rate / (batchSize * IterationSize), computed by the caller from
+ * SGDSolver::getLearningRate.  clamp != 0 clamps the result to [clamp_min, clamp_max]. */
+int n2d2hip_sgd_update_f32(float* data, const float* diff, size_t n, float rate_diff, float momentum,
+                           float decay_times_rate, float* momentum_data, int clamp, float clamp_min, float clamp_max,
+                           n2d2hip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

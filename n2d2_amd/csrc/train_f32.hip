@@ -1,0 +1,361 @@
+// Float32 cells of a quantization-aware training step: convolution forward, its three backward kernels, softmax,
+// the loss at the output and the SGD update.  Tensors are N2D2's own NCHW / OCHW float tensors (X fastest), so a
+// training graph exchanges them without conversion.
+//
+// These are direct kernels: one thread per produced element, walking channels and taps in the reference's order
+// (so forward and backward-data give the reference's float sums term for term), and one block per weight for
+// backward-filter, whose long sum over batch and pixels is wavefront-reduced in double.
+#include "common.h"
+
+namespace n2d2hip {
+
+constexpr int TBLOCK = 256;
+
+struct ConvF32 {
+    int B, C, H, W, O, oH, oW, kW, kH, Cw;      // Cw = C / groups
+    int sx, sy, pl, pt, pr, pb, dx, dy;
+    int depthwise;                                // groups == C == O
+};
+
+__device__ __forceinline__ double wave_sum_d(double v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ double block_sum_d(double v)
+{
+    __shared__ double red[TBLOCK / 64];
+    v = wave_sum_d(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    double t = 0.0;
+#pragma unroll
+    for (int i = 0; i < TBLOCK / 64; ++i) t += red[i];
+    return t;
+}
+
+// out[b,o,oy,ox] = alpha-less weighted sum (+ bias) + beta * out.  The window is clipped at the borders (no padded
+// zeros are read); a full 3x3 window is summed row by row, then the rows, as the reference's unrolled branch does.
+__global__ __launch_bounds__(TBLOCK) void conv_f32_forward_kernel(ConvF32 q, const float* __restrict__ x, const float* __restrict__ w,
+                                                                  const float* __restrict__ bias, float beta, float* __restrict__ y)
+{
+    const size_t total = (size_t)q.B * q.O * q.oH * q.oW;
+    for (size_t idx = (size_t)blockIdx.x * TBLOCK + threadIdx.x; idx < total; idx += (size_t)gridDim.x * TBLOCK) {
+        const int ox = idx % q.oW, oy = (idx / q.oW) % q.oH;
+        const int o = (idx / ((size_t)q.oW * q.oH)) % q.O, b = idx / ((size_t)q.oW * q.oH * q.O);
+        const int dilKx = q.kW + (q.dx - 1) * (q.kW - 1), dilKy = q.kH + (q.dy - 1) * (q.kH - 1);
+        const int sxMin = max(q.pl - ox * q.sx, 0), syMin = max(q.pt - oy * q.sy, 0);
+        const int sxMax = min(max(q.W + q.pl - ox * q.sx, 0), dilKx), syMax = min(max(q.H + q.pt - oy * q.sy, 0), dilKy);
+        const int ix = ox * q.sx - q.pl, iy = oy * q.sy - q.pt;
+        const int c0 = q.depthwise ? o : 0, c1 = q.depthwise ? o + 1 : q.C;
+        const bool full3 = sxMin == 0 && syMin == 0 && sxMax == 3 && syMax == 3 && q.kW == 3 && q.kH == 3;
+        float sum = 0.0f;
+        for (int c = c0; c < c1; ++c) {
+            const float* xc = x + ((size_t)b * q.C + c) * q.H * q.W;
+            const float* wc = w + ((size_t)o * q.Cw + (q.depthwise ? 0 : c)) * q.kH * q.kW;
+            if (full3) {
+                const float* r0 = xc + (size_t)iy * q.W + ix;
+                const float* r1 = r0 + q.W;
+                const float* r2 = r1 + q.W;
+                sum = sum + (wc[0] * r0[0] + wc[1] * r0[1] + wc[2] * r0[2])
+                          + (wc[3] * r1[0] + wc[4] * r1[1] + wc[5] * r1[2])
+                          + (wc[6] * r2[0] + wc[7] * r2[1] + wc[8] * r2[2]);
+            } else {
+                for (int ty = syMin; ty * q.dy < syMax; ++ty)
+                    for (int tx = sxMin; tx * q.dx < sxMax; ++tx)
+                        sum += wc[ty * q.kW + tx] * xc[(size_t)(iy + ty * q.dy) * q.W + ix + tx * q.dx];
+            }
+        }
+        float r = sum + (beta != 0.0f ? beta * y[idx] : 0.0f);
+        if (bias) r = bias[o] + r;
+        y[idx] = r;
+    }
+}
+
+// dx[b,c,iy,ix] = sum over connected outputs (ascending) and over the taps reaching this element + beta * dx.
+__global__ __launch_bounds__(TBLOCK) void conv_f32_backward_data_kernel(ConvF32 q, const float* __restrict__ w, const float* __restrict__ dy,
+                                                                        float beta, float* __restrict__ dx)
+{
+    const size_t total = (size_t)q.B * q.C * q.H * q.W;
+    const int oxStride = q.sx * q.oW, oyStride = q.sy * q.oH;
+    for (size_t idx = (size_t)blockIdx.x * TBLOCK + threadIdx.x; idx < total; idx += (size_t)gridDim.x * TBLOCK) {
+        const int ix = idx % q.W, iy = (idx / q.W) % q.H;
+        const int c = (idx / ((size_t)q.W * q.H)) % q.C, b = idx / ((size_t)q.W * q.H * q.C);
+        const int ixPad = ix + q.pl, iyPad = iy + q.pt;
+        const int sxMin = ixPad % q.sx + max(ixPad - ixPad % q.sx - oxStride + q.sx, 0);
+        const int syMin = iyPad % q.sy + max(iyPad - iyPad % q.sy - oyStride + q.sy, 0);
+        const int sxMax = min(q.kW, ixPad + 1), syMax = min(q.kH, iyPad + 1);
+        const bool full3 = syMax - syMin == 3 && q.sy == 1 && sxMax - sxMin == 3 && q.sx == 1;
+        const int o0 = q.depthwise ? c : 0, o1 = q.depthwise ? c + 1 : q.O;
+        float g = 0.0f;
+        for (int o = o0; o < o1; ++o) {
+            const float* wo = w + ((size_t)o * q.Cw + (q.depthwise ? 0 : c)) * q.kH * q.kW;
+            const float* dyo = dy + ((size_t)b * q.O + o) * q.oH * q.oW;
+            if (full3) {
+                const int ox = ixPad - sxMin, oy = iyPad - syMin;
+#pragma unroll
+                for (int t = 0; t < 9; ++t)
+                    g = g + wo[(syMin + t / 3) * q.kW + sxMin + t % 3] * dyo[(size_t)(oy - t / 3) * q.oW + ox - t % 3];
+            } else {
+                for (int ty = syMin; ty < syMax; ty += q.sy)
+                    for (int tx = sxMin; tx < sxMax; tx += q.sx)
+                        g += wo[ty * q.kW + tx] * dyo[(size_t)((iyPad - ty) / q.sy) * q.oW + (ixPad - tx) / q.sx];
+            }
+        }
+        dx[idx] = g + (beta != 0.0f ? beta * dx[idx] : 0.0f);
+    }
+}
+
+// dw[o,c',ty,tx] = sum over batch and the output pixels whose tap (ty,tx) falls inside the input + beta * dw.
+// One block per weight.
+__global__ __launch_bounds__(TBLOCK) void conv_f32_backward_filter_kernel(ConvF32 q, const float* __restrict__ x, const float* __restrict__ dy,
+                                                                          float beta, float* __restrict__ dw)
+{
+    const int widx = blockIdx.x;
+    const int tx = widx % q.kW, ty = (widx / q.kW) % q.kH;
+    const int cw = (widx / (q.kW * q.kH)) % q.Cw, o = widx / (q.kW * q.kH * q.Cw);
+    const int c = q.depthwise ? o : cw;
+    // ox range with 0 <= ox*sx + tx - pl < W
+    const int oxMin = max((q.pl - tx + q.sx - 1) / q.sx, 0), oyMin = max((q.pt - ty + q.sy - 1) / q.sy, 0);
+    const int oxMax = min((q.W + q.pl - tx + q.sx - 1) / q.sx, q.oW), oyMax = min((q.H + q.pt - ty + q.sy - 1) / q.sy, q.oH);
+    const int nx = max(oxMax - oxMin, 0), ny = max(oyMax - oyMin, 0);
+    const size_t total = (size_t)q.B * ny * nx;
+    double acc = 0.0;
+    for (size_t i = threadIdx.x; i < total; i += TBLOCK) {
+        const int ox = oxMin + i % nx, oy = oyMin + (i / nx) % ny, b = i / ((size_t)nx * ny);
+        const float xv = x[(((size_t)b * q.C + c) * q.H + (oy * q.sy + ty - q.pt)) * q.W + ox * q.sx + tx - q.pl];
+        const float dv = dy[(((size_t)b * q.O + o) * q.oH + oy) * q.oW + ox];
+        acc += (double)(xv * dv);
+    }
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0)
+        dw[widx] = (float)acc + (beta != 0.0f ? beta * dw[widx] : 0.0f);
+}
+
+// db[o] = sum over batch and pixels + beta * db.  One block per output channel.
+__global__ __launch_bounds__(TBLOCK) void conv_f32_backward_bias_kernel(int B, int O, int plane, const float* __restrict__ dy, float beta,
+                                                                        float* __restrict__ db)
+{
+    const int o = blockIdx.x;
+    double acc = 0.0;
+    for (size_t i = threadIdx.x; i < (size_t)B * plane; i += TBLOCK)
+        acc += (double)dy[((size_t)(i / plane) * O + o) * plane + i % plane];
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0)
+        db[o] = (float)acc + (beta != 0.0f ? beta * db[o] : 0.0f);
+}
+
+// Softmax over the channels of each pixel: exp(x - max) / sum, zeros if the sum is not positive.
+__global__ __launch_bounds__(TBLOCK) void softmax_f32_kernel(const float* __restrict__ x, float* __restrict__ y, int B, int C, int plane)
+{
+    const size_t total = (size_t)B * plane;
+    for (size_t idx = (size_t)blockIdx.x * TBLOCK + threadIdx.x; idx < total; idx += (size_t)gridDim.x * TBLOCK) {
+        const size_t base = (idx / plane) * (size_t)C * plane + idx % plane;
+        float m = x[base];
+        for (int c = 1; c < C; ++c) m = fmaxf(m, x[base + (size_t)c * plane]);
+        float s = 0.0f;
+        for (int c = 0; c < C; ++c) s += expf(x[base + (size_t)c * plane] - m);
+        for (int c = 0; c < C; ++c) y[base + (size_t)c * plane] = s > 0.0f ? expf(x[base + (size_t)c * plane] - m) / s : 0.0f;
+    }
+}
+
+// diff = target - output, formed in double; partial[block] = sum of squares (double).
+__global__ __launch_bounds__(TBLOCK) void loss_f32_kernel(const float* __restrict__ target, const float* __restrict__ out, float* __restrict__ diff,
+                                                          size_t n, double* __restrict__ partial)
+{
+    double acc = 0.0;
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * TBLOCK) {
+        const double e = (double)target[i] - (double)out[i];
+        diff[i] = (float)e;
+        acc += e * e;
+    }
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+}
+__global__ __launch_bounds__(TBLOCK) void loss_finish_kernel(const double* __restrict__ partial, int nb, double inv_batch, double* __restrict__ loss)
+{
+    double acc = 0.0;
+    for (int i = threadIdx.x; i < nb; i += TBLOCK) acc += partial[i];
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0) loss[0] = acc * inv_batch;
+}
+
+// SGDSolver_Frame::update for one tensor.
+__global__ __launch_bounds__(TBLOCK) void sgd_f32_kernel(float* __restrict__ data, const float* __restrict__ diff, size_t n, float rate_diff,
+                                                         float momentum, float decay_rate, float* __restrict__ mom, float lo, float hi, int clamp)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * TBLOCK) {
+        float v;
+        if (mom) {
+            float m = mom[i] * momentum;
+            m += rate_diff * diff[i];
+            if (decay_rate != 0.0f) m += -decay_rate * data[i];
+            mom[i] = m;
+            v = data[i] + m;
+        } else {
+            v = data[i] + rate_diff * diff[i];
+        }
+        data[i] = clamp ? fminf(fmaxf(v, lo), hi) : v;
+    }
+}
+
+// Rectifier on a float tensor, in place: x > 0 ? min(x, clipping) : leak * x (clipping == 0: none).
+__global__ __launch_bounds__(TBLOCK) void rectifier_f32_forward_kernel(float* __restrict__ x, size_t n, float leak, float clipping)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * TBLOCK) {
+        const float v = x[i];
+        x[i] = v > 0.0f ? (clipping > 0.0f ? fminf(v, clipping) : v) : leak * v;
+    }
+}
+// diff_out = diff_in * (out == clipping ? 0 : out > 0 ? 1 : leak); `out` is what the cell holds after its activation.
+__global__ __launch_bounds__(TBLOCK) void rectifier_f32_backward_kernel(const float* __restrict__ out, const float* __restrict__ diff_in,
+                                                                        float* __restrict__ diff_out, size_t n, float leak, float clipping)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * TBLOCK) {
+        const float o = out[i];
+        const float f = (clipping > 0.0f && o == clipping) ? 0.0f : (o > 0.0f ? 1.0f : leak);
+        diff_out[i] = diff_in[i] * f;
+    }
+}
+
+static int grid_for(size_t total)
+{
+    const size_t blocks = (total + TBLOCK - 1) / TBLOCK;
+    return (int)std::min<size_t>(std::max<size_t>(blocks, 1), 256 * 32);
+}
+
+static int make_conv(const n2d2hip_conv_desc* d, int B, int H, int W, bool backward, ConvF32* q, const char* who)
+{
+    N2D2HIP_REQUIRE(d != nullptr, N2D2HIP_ERR_INVALID, "%s: null descriptor", who);
+    N2D2HIP_REQUIRE(B > 0 && H > 0 && W > 0 && d->C > 0 && d->O > 0 && d->kW > 0 && d->kH > 0 && d->strideX > 0 && d->strideY > 0
+                        && d->dilX > 0 && d->dilY > 0 && d->padL >= 0 && d->padT >= 0 && d->padR >= 0 && d->padB >= 0,
+                    N2D2HIP_ERR_INVALID, "%s: bad shape", who);
+    N2D2HIP_REQUIRE(d->groups == 1 || (d->groups == d->C && d->C == d->O), N2D2HIP_ERR_UNSUPPORTED,
+                    "%s: groups=%d (C=%d, O=%d): only ungrouped and depthwise convolutions", who, d->groups, d->C, d->O);
+    N2D2HIP_REQUIRE(!backward || (d->dilX == 1 && d->dilY == 1), N2D2HIP_ERR_UNSUPPORTED,
+                    "%s: the reference's backward kernels do not read the dilation", who);
+    int oH = 0, oW = 0;
+    const int st = n2d2hip_conv_out_dims(d, H, W, &oH, &oW);
+    if (st != N2D2HIP_OK) return st;
+    N2D2HIP_REQUIRE(oH > 0 && oW > 0, N2D2HIP_ERR_INVALID, "%s: empty output", who);
+    N2D2HIP_REQUIRE((size_t)B * std::max(d->C, d->O) * std::max((size_t)H * W, (size_t)oH * oW) < ((size_t)1 << 40), N2D2HIP_ERR_INVALID,
+                    "%s: tensor too large", who);
+    *q = ConvF32{B, d->C, H, W, d->O, oH, oW, d->kW, d->kH, d->C / d->groups, d->strideX, d->strideY,
+                 d->padL, d->padT, d->padR, d->padB, d->dilX, d->dilY, d->groups > 1 ? 1 : 0};
+    return N2D2HIP_OK;
+}
+
+} // namespace n2d2hip
+
+using namespace n2d2hip;
+
+extern "C" {
+
+int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* w, const float* bias,
+                               float beta, float* y, n2d2hip_stream_t stream)
+{
+    ConvF32 q;
+    const int st = make_conv(desc, B, H, W, false, &q, "n2d2hip_conv2d_f32_forward");
+    if (st != N2D2HIP_OK) return st;
+    N2D2HIP_REQUIRE(x && w && y, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_forward: null pointer");
+    hipLaunchKernelGGL(conv_f32_forward_kernel, dim3(grid_for((size_t)q.B * q.O * q.oH * q.oW)), dim3(TBLOCK), 0, (hipStream_t)stream,
+                       q, x, w, bias, beta, y);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* w, const float* diff_y, float beta,
+                                     float* diff_x, n2d2hip_stream_t stream)
+{
+    ConvF32 q;
+    const int st = make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_backward_data");
+    if (st != N2D2HIP_OK) return st;
+    N2D2HIP_REQUIRE(w && diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_data: null pointer");
+    hipLaunchKernelGGL(conv_f32_backward_data_kernel, dim3(grid_for((size_t)q.B * q.C * q.H * q.W)), dim3(TBLOCK), 0, (hipStream_t)stream,
+                       q, w, diff_y, beta, diff_x);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* diff_y, float beta,
+                                       float* diff_w, n2d2hip_stream_t stream)
+{
+    ConvF32 q;
+    const int st = make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_backward_filter");
+    if (st != N2D2HIP_OK) return st;
+    N2D2HIP_REQUIRE(x && diff_y && diff_w, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_filter: null pointer");
+    const size_t nw = (size_t)q.O * q.Cw * q.kH * q.kW;
+    N2D2HIP_REQUIRE(nw < ((size_t)1 << 31), N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_filter: too many weights");
+    hipLaunchKernelGGL(conv_f32_backward_filter_kernel, dim3((unsigned)nw), dim3(TBLOCK), 0, (hipStream_t)stream, q, x, diff_y, beta, diff_w);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_conv2d_f32_backward_bias(int B, int O, int oH, int oW, const float* diff_y, float beta, float* diff_bias, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(B > 0 && O > 0 && oH > 0 && oW > 0 && diff_y && diff_bias, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_bias: bad argument");
+    hipLaunchKernelGGL(conv_f32_backward_bias_kernel, dim3(O), dim3(TBLOCK), 0, (hipStream_t)stream, B, O, oH * oW, diff_y, beta, diff_bias);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_softmax_f32_forward(const float* x, float* y, int B, int C, int H, int W, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && y, N2D2HIP_ERR_INVALID, "n2d2hip_softmax_f32_forward: bad argument");
+    hipLaunchKernelGGL(softmax_f32_kernel, dim3(grid_for((size_t)B * H * W)), dim3(TBLOCK), 0, (hipStream_t)stream, x, y, B, C, H * W);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_rectifier_f32_forward(float* x, size_t n, float leak_slope, float clipping, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(x && n > 0 && clipping >= 0.0f, N2D2HIP_ERR_INVALID, "n2d2hip_rectifier_f32_forward: bad argument");
+    hipLaunchKernelGGL(rectifier_f32_forward_kernel, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, x, n, leak_slope, clipping);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, float* diff_out, size_t n, float leak_slope, float clipping,
+                                   n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(output && diff_in && diff_out && n > 0 && clipping >= 0.0f, N2D2HIP_ERR_INVALID, "n2d2hip_rectifier_f32_backward: bad argument");
+    hipLaunchKernelGGL(rectifier_f32_backward_kernel, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, output, diff_in, diff_out, n,
+                       leak_slope, clipping);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+size_t n2d2hip_loss_workspace_bytes(size_t n)
+{
+    return (size_t)grid_for(n) * sizeof(double);
+}
+
+int n2d2hip_loss_f32(const float* target, const float* output, float* diff, size_t n, int batch, double* loss,
+                     void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(target && output && diff && loss && n > 0 && batch > 0, N2D2HIP_ERR_INVALID, "n2d2hip_loss_f32: bad argument");
+    const int nb = grid_for(n);
+    N2D2HIP_REQUIRE(workspace && workspace_bytes >= (size_t)nb * sizeof(double), N2D2HIP_ERR_WORKSPACE,
+                    "n2d2hip_loss_f32: workspace of %zu bytes, %zu needed", workspace_bytes, (size_t)nb * sizeof(double));
+    hipLaunchKernelGGL(loss_f32_kernel, dim3(nb), dim3(TBLOCK), 0, (hipStream_t)stream, target, output, diff, n, (double*)workspace);
+    hipLaunchKernelGGL(loss_finish_kernel, dim3(1), dim3(TBLOCK), 0, (hipStream_t)stream, (const double*)workspace, nb, 1.0 / batch, loss);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_sgd_update_f32(float* data, const float* diff, size_t n, float rate_diff, float momentum, float decay_times_rate,
+                           float* momentum_data, int clamp, float clamp_min, float clamp_max, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(data && diff && n > 0, N2D2HIP_ERR_INVALID, "n2d2hip_sgd_update_f32: bad argument");
+    N2D2HIP_REQUIRE(momentum_data || (momentum == 0.0f && decay_times_rate == 0.0f), N2D2HIP_ERR_INVALID,
+                    "n2d2hip_sgd_update_f32: momentum or decay without a momentum buffer");
+    hipLaunchKernelGGL(sgd_f32_kernel, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, data, diff, n, rate_diff, momentum,
+                       decay_times_rate, momentum_data, clamp_min, clamp_max, clamp);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,177 @@
+"""GPU parity of the float32 training kernels (convolution forward / backward, rectifier, softmax, loss, SGD) against
+the CPU oracle, through the C ABI.  Forward and backward-data walk their sums in the reference's order: compared to
+1e-5 relative (in practice identical).  Backward-filter and backward-bias reduce in double on the device while the
+reference adds float32 terms one after the other; they are held to 1e-5 of the sum of the terms' magnitudes against
+the float64 oracle, which is the bound the reference's own float32 sum obeys with room to spare."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+CASES = [  # B, C, H, W, O, k, stride, pad, groups
+    (2, 3, 7, 6, 4, 3, 1, 1, 1), (2, 4, 9, 9, 4, 3, 2, 1, 4), (1, 2, 5, 5, 3, 1, 1, 0, 1), (2, 3, 10, 9, 2, 5, 2, 2, 1),
+    (2, 1, 5, 5, 1, 3, 1, 0, 1), (3, 5, 8, 8, 5, 3, 1, 1, 5), (1, 3, 9, 7, 2, 3, 3, 0, 1), (2, 2, 4, 4, 3, 2, 2, 0, 1),
+    (4, 16, 14, 14, 32, 3, 1, 1, 1), (2, 32, 12, 12, 32, 3, 2, 1, 32), (3, 24, 10, 10, 8, 1, 1, 0, 1), (2, 8, 17, 13, 16, 7, 2, 3, 1)]
+
+
+@pytest.fixture(scope="module")
+def g():
+    import torch
+    from n2d2_amd import capi as capi_, runtime
+
+    class G:
+        lib, check, sp, capi = capi_.lib, staticmethod(capi_.check), staticmethod(runtime.stream_ptr), capi_
+
+        @staticmethod
+        def dev(a):
+            return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+        @staticmethod
+        def host(t):
+            torch.cuda.synchronize()
+            return t.cpu().numpy()
+
+        @staticmethod
+        def desc(C_, O, k, s, p, groups, dil=1):
+            return capi_.ConvDesc(C_, O, k, k, s, s, p, p, p, p, dil, dil, groups, 0)
+        torch_ = torch
+    return G
+
+
+def _rel(got, want, scale=None):
+    scale = np.maximum(np.abs(want), 1e-3) if scale is None else scale
+    return float((np.abs(got.astype(np.float64) - want.astype(np.float64)) / scale).max())
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_forward_and_backward(g, case):
+    from oracle import oracle as orc
+    B, Cn, H, W, O, k, s, p, groups = case
+    print("conv f32", case, flush=True)
+    rng = np.random.default_rng(sum(case))
+    maps = None if groups == 1 else orc.group_maps(Cn, O, groups)
+    kw = dict(stride=(s, s), pad=(p, p, p, p), maps=maps)
+    x = rng.normal(size=(B, Cn, H, W)).astype(np.float32)
+    w = rng.normal(size=(O, Cn // groups, k, k)).astype(np.float32)
+    bias = rng.normal(size=O).astype(np.float32)
+    want = orc.conv_forward_bias(orc.conv_forward(x, w, **kw), bias)
+    d = g.desc(Cn, O, k, s, p, groups)
+    dx_, dw_, db_ = g.dev(x), g.dev(w), g.dev(bias)
+    y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), db_.data_ptr(), 0.0, y.data_ptr(), g.sp()))
+    got = g.host(y)
+    assert got.shape == want.shape and _rel(got, want) <= TOL
+    # beta accumulates onto what the output held (second input tensor of a cell)
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), None, 1.0, y.data_ptr(), g.sp()))
+    want2 = orc.conv_forward(x, w, out=want.copy(), beta=1.0, **kw)
+    assert _rel(g.host(y), want2) <= TOL
+
+    dy = rng.normal(size=want.shape).astype(np.float32)
+    ddy = g.dev(dy)
+    wantdx = orc.conv_backward_data(w, dy, x.shape, **kw)
+    gdx = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 0.0, gdx.data_ptr(), g.sp()))
+    assert _rel(g.host(gdx), wantdx) <= TOL
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 1.0, gdx.data_ptr(), g.sp()))
+    assert _rel(g.host(gdx), orc.conv_backward_data(w, dy, x.shape, dx=wantdx.copy(), beta=1.0, **kw)) <= TOL
+
+    x64, dy64 = x.astype(np.float64), dy.astype(np.float64)
+    wantdw = orc.conv_backward_filter(x64, dy64, w.shape, **kw)
+    mag = orc.conv_backward_filter(np.abs(x64), np.abs(dy64), w.shape, **kw)
+    gdw = g.torch_.empty(w.shape, dtype=g.torch_.float32, device="cuda")
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 0.0, gdw.data_ptr(), g.sp()))
+    got = g.host(gdw)
+    assert _rel(got, wantdw, np.maximum(mag, 1e-3)) <= TOL
+    # and the reference's own float32 running sum stays within the same bound of it
+    assert _rel(orc.conv_backward_filter(x, dy, w.shape, **kw), wantdw, np.maximum(mag, 1e-3)) <= 5 * TOL
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 1.0, gdw.data_ptr(), g.sp()))
+    assert _rel(g.host(gdw), 2 * wantdw, np.maximum(2 * mag, 1e-3)) <= TOL
+
+    gdb = g.torch_.empty(O, dtype=g.torch_.float32, device="cuda")
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_bias(B, O, want.shape[2], want.shape[3], ddy.data_ptr(), 0.0, gdb.data_ptr(), g.sp()))
+    assert _rel(g.host(gdb), orc.conv_backward_bias(dy64), np.maximum(np.abs(dy64).sum(axis=(0, 2, 3)), 1e-3)) <= TOL
+
+
+def test_conv_f32_rejects_what_the_reference_cannot_do(g):
+    x = g.dev(np.zeros((1, 6, 8, 8)))
+    w = g.dev(np.zeros((4, 3, 3, 3)))
+    y = g.dev(np.zeros((1, 4, 6, 6)))
+    d = g.desc(6, 4, 3, 1, 0, 2)          # two groups of three channels: the reference's backward is not its adjoint
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), g.sp()) == g.capi.ERR_UNSUPPORTED
+    d = g.desc(6, 4, 3, 1, 0, 1, dil=2)    # backward with dilation: the reference does not read it
+    assert g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), 1, 8, 8, w.data_ptr(), y.data_ptr(), 0.0, x.data_ptr(), g.sp()) == g.capi.ERR_UNSUPPORTED
+    assert b"dilation" in g.lib.n2d2hip_last_error()
+    d = g.desc(6, 4, 3, 1, 0, 1)
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, None, w.data_ptr(), None, 0.0, y.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+
+
+def test_dilated_forward(g):
+    from oracle import oracle as orc
+    rng = np.random.default_rng(3)
+    x = rng.normal(size=(2, 3, 11, 11)).astype(np.float32)
+    w = rng.normal(size=(4, 3, 3, 3)).astype(np.float32)
+    want = orc.conv_forward(x, w, pad=(2, 2, 2, 2), dil=(2, 2))
+    d = g.desc(3, 4, 3, 1, 2, 1, dil=2)
+    y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
+    dx_, dw_ = g.dev(x), g.dev(w)
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 2, 11, 11, dx_.data_ptr(), dw_.data_ptr(), None, 0.0, y.data_ptr(), g.sp()))
+    assert _rel(g.host(y), want) <= TOL
+
+
+def test_rectifier_softmax_loss_sgd(g):
+    from oracle import oracle as orc
+    from oracle import qat_train as qt
+    rng = np.random.default_rng(8)
+    x = (rng.normal(size=(4, 10, 3, 3)) * 3).astype(np.float32)
+    for leak, clip in ((0.0, 0.0), (0.1, 0.0), (0.0, 2.0), (0.25, 1.5)):
+        t = g.dev(x)
+        g.check(g.lib.n2d2hip_rectifier_f32_forward(t.data_ptr(), x.size, leak, clip, g.sp()))
+        want = orc.rectifier(x.copy(), leak=leak, clipping=clip, cell_quantized=False)
+        out = g.host(t)
+        assert _rel(out, want) <= TOL
+        dy = rng.normal(size=x.shape).astype(np.float32)
+        dd = g.dev(dy)
+        g.check(g.lib.n2d2hip_rectifier_f32_backward(t.data_ptr(), dd.data_ptr(), dd.data_ptr(), x.size, leak, clip, g.sp()))
+        f = np.where((clip > 0) & (want == np.float32(clip)), 0.0, np.where(want > 0, 1.0, leak)).astype(np.float32)
+        assert _rel(g.host(dd), dy * f) <= TOL
+    y = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
+    dx_ = g.dev(x)
+    g.check(g.lib.n2d2hip_softmax_f32_forward(dx_.data_ptr(), y.data_ptr(), 4, 10, 3, 3, g.sp()))
+    sm = orc.softmax_forward(x)
+    assert _rel(g.host(y), sm) <= TOL
+    target = np.zeros_like(x)
+    target[:, 2] = 1
+    diff = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
+    loss = g.torch_.zeros(1, dtype=g.torch_.float64, device="cuda")
+    ws = g.torch_.empty(int(g.lib.n2d2hip_loss_workspace_bytes(x.size)), dtype=g.torch_.uint8, device="cuda")
+    dt_ = g.dev(target)
+    g.check(g.lib.n2d2hip_loss_f32(dt_.data_ptr(), y.data_ptr(), diff.data_ptr(), x.size, 4, loss.data_ptr(), ws.data_ptr(), ws.numel(), g.sp()))
+    cell = qt.SoftmaxCell()
+    cell.outputs = g.host(y)
+    want_loss = cell.apply_loss(target)
+    assert np.array_equal(g.host(diff), cell.diff_inputs)
+    assert abs(float(g.host(loss)[0]) - want_loss) <= 1e-12 * max(1.0, want_loss)
+    # SGD: plain, and with momentum and decay over three updates
+    for kwargs in (dict(), dict(learning_rate=0.1, momentum=0.9, decay=0.01)):
+        s = qt.SGDSolver(**kwargs)
+        data = rng.normal(size=1000).astype(np.float32)
+        dev = g.dev(data)
+        mom = g.torch_.zeros(1000, dtype=g.torch_.float32, device="cuda") if kwargs else None
+        for it in range(3):
+            grad = rng.normal(size=1000).astype(np.float32)
+            s.update(data, grad, 4)
+            rate = np.float32(s.learning_rate)
+            rate_diff = np.float32(rate / np.float32(4.0))
+            dgrad = g.dev(grad)
+            g.check(g.lib.n2d2hip_sgd_update_f32(dev.data_ptr(), dgrad.data_ptr(), 1000, float(rate_diff), float(s.momentum),
+                                                 float(np.float32(np.float32(s.decay) * rate)), mom.data_ptr() if kwargs else None,
+                                                 0, 0.0, 0.0, g.sp()))
+            assert _rel(g.host(dev), data) <= TOL
+    dev = g.dev(np.array([0.5, -0.5, 0.0]))
+    dgrad = g.dev(np.array([10.0, -10.0, 1.0]))
+    g.check(g.lib.n2d2hip_sgd_update_f32(dev.data_ptr(), dgrad.data_ptr(), 3, 1.0, 0.0, 0.0, None, 1, -1.0, 1.0, g.sp()))
+    assert np.array_equal(g.host(dev), np.array([1.0, -1.0, 1.0], dtype=np.float32))
+    assert g.lib.n2d2hip_sgd_update_f32(dev.data_ptr(), dev.data_ptr(), 3, 1.0, 0.9, 0.0, None, 0, 0.0, 0.0, g.sp()) == g.capi.ERR_INVALID
