@@ -802,23 +802,60 @@ template <> Registrar<ScalingCell> ScalingCell_Frame_HIP<float>::mRegistrar("Fra
                                                                             Registrar<ScalingCell>::Type<float>());
 
 // ------------------------------------------------------------------- SGDSolver
+SGDSolver::~SGDSolver()
+{
+    if (mMomentumData) (void)hipFree(mMomentumData);
+}
+
 void SGDSolver::setParameter(const std::string& name, double value)
 {
     if (name == "LearningRate") mLearningRate = value;
+    else if (name == "Momentum") mMomentum = value;
+    else if (name == "Decay") mDecay = value;
     else if (name == "IterationSize") mIterationSize = (unsigned int)value;
     else throw std::runtime_error("Parameter does not exist: " + name);
+}
+
+double SGDSolver::getLearningRate()
+{
+    if (mLearningRate == 0.0)
+        return 0.0;
+    if (mIterationPass < mIterationSize - 1) {
+        ++mIterationPass;
+        return 0.0;
+    }
+    mIterationPass = 0;
+    ++mNbIterations;
+    return mLearningRate;
 }
 
 void SGDSolver::update(float& data, float diff, unsigned int batchSize)
 {
     // include/Solver/SGDSolver_Frame.hpp:84-109 without momentum / decay: data += rate/(batch*iterSize) * diff,
     // applied on the last pass of an iteration
-    ++mIterationPass;
-    if (mIterationPass < mIterationSize)
+    const float rate = (float)getLearningRate();
+    if (rate == 0.0f)
         return;
-    mIterationPass = 0;
-    const float rate = (float)(mLearningRate / (double)(batchSize * mIterationSize));
-    data += rate * diff;
+    const float rateDiff = rate / ((float)batchSize * (float)mIterationSize);
+    data += rateDiff * diff;
+}
+
+void SGDSolver::update(float* data, const float* diff, std::size_t n, unsigned int batchSize, void* stream)
+{
+    const float rate = (float)getLearningRate();
+    if (rate == 0.0f)
+        return;
+    const float rateDiff = rate / ((float)batchSize * (float)mIterationSize);
+    const bool plain = (mMomentum == 0.0 && mDecay == 0.0);
+    if (!plain && mMomentumSize != n) {
+        if (mMomentumData) (void)hipFree(mMomentumData);
+        mMomentumData = nullptr;
+        checkHip(hipMalloc((void**)&mMomentumData, n * sizeof(float)), "SGDSolver::update()");
+        checkHip(hipMemsetAsync(mMomentumData, 0, n * sizeof(float), (hipStream_t)stream), "SGDSolver::update()");
+        mMomentumSize = n;
+    }
+    checkStatus(n2d2hip_sgd_update_f32(data, diff, n, rateDiff, (float)mMomentum, (float)mDecay * rate, plain ? nullptr : mMomentumData,
+                                       0, 0.0f, 0.0f, stream));
 }
 
 template <> Registrar<SGDSolver> SGDSolver_Frame_HIP<float>::mRegistrar("Frame_HIP", SGDSolver_Frame_HIP<float>::create,
@@ -983,11 +1020,8 @@ template <class T>
 void SATQuantizerActivation_Frame_HIP<T>::update(unsigned int batchSize)
 {
     if (!mSolver) return;
-    float h[2];
     lazyInit(0, false);
-    checkHip(hipMemcpy(h, mDev, sizeof(h), hipMemcpyDeviceToHost), "SATQuantizerActivation_Frame_HIP::update()");
-    mSolver->update(h[0], h[1], batchSize);
-    checkHip(hipMemcpy(mDev, h, sizeof(float), hipMemcpyHostToDevice), "SATQuantizerActivation_Frame_HIP::update()");
+    mSolver->update(mDev, mDev + 1, 1, batchSize, mStream);       // alpha and its gradient stay on the device
 }
 
 template <> Registrar<SATQuantizerActivation> SATQuantizerActivation_Frame_HIP<float>::mRegistrar(

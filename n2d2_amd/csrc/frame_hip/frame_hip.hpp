@@ -235,9 +235,15 @@ struct DeepNetExport {
 };
 
 // ----------------------------------------------------------------- Activation
+class QuantizerActivation;
 // include/Activation/Activation.hpp:36-110
 class Activation {
 public:
+    // Quantizer applied to the activation's output during quantization-aware training (Activation::setQuantizer,
+    // include/Activation/Activation.hpp:84-92); read by the float cells only
+    void setQuantizer(const std::shared_ptr<QuantizerActivation>& quantizer) { mQuantizer = quantizer; }
+    const std::shared_ptr<QuantizerActivation>& getQuantizer() const { return mQuantizer; }
+    virtual double clipping() const { return 0.0; }
     virtual ~Activation() {}
     virtual const char* getType() const = 0;
     virtual std::pair<double, double> getOutputRange() const = 0;
@@ -256,6 +262,7 @@ protected:
     Scaling mScaling;
     std::size_t mQuantizedNbBits;
     unsigned mRevision;
+    std::shared_ptr<QuantizerActivation> mQuantizer;
 };
 
 // src/Activation/RectifierActivation.cpp:26-40 (LeakSlope 0.0, Clipping 0.0)
@@ -274,6 +281,7 @@ public:
     void setParameter(const std::string& name, double value);
     int abiKind() const { return N2D2HIP_ACT_RECTIFIER; }
     float leakSlope() const { return (float)mLeakSlope; }
+    double clipping() const { return mClipping; }
 
 protected:
     double mLeakSlope, mClipping;
@@ -294,6 +302,7 @@ public:
     }
     void setParameter(const std::string& name, double value);
     int abiKind() const { return N2D2HIP_ACT_LINEAR; }
+    double clipping() const { return mClipping; }
 
 protected:
     double mClipping;
@@ -706,16 +715,29 @@ class SGDSolver {
 public:
     typedef std::function<std::shared_ptr<SGDSolver>()> RegistryCreate_T;
     static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
-    SGDSolver() : mLearningRate(0.01), mIterationSize(1), mIterationPass(0) {}
-    virtual ~SGDSolver() {}
+    SGDSolver() : mLearningRate(0.01), mMomentum(0.0), mDecay(0.0), mIterationSize(1), mIterationPass(0), mNbIterations(0),
+                  mMomentumData(nullptr), mMomentumSize(0) {}
+    virtual ~SGDSolver();
+    SGDSolver(const SGDSolver&) = delete;
+    SGDSolver& operator=(const SGDSolver&) = delete;
+    // LearningRate (0.01), Momentum (0.0), Decay (0.0), IterationSize (1): src/Solver/SGDSolver.cpp:26-41
     void setParameter(const std::string& name, double value);
     bool isNewIteration() const { return mIterationPass == 0; }
+    // SGDSolver::getLearningRate with LearningRatePolicy None (src/Solver/SGDSolver.cpp:99-189): 0 on every pass of an
+    // iteration but the last
+    double getLearningRate();
+    unsigned int nbIterations() const { return mNbIterations; }
     // scalar parameter update on the host
     void update(float& data, float diff, unsigned int batchSize);
+    // update of n device floats (include/Solver/SGDSolver_Frame.hpp:77-146); one solver serves one tensor, as in the
+    // reference, because it owns that tensor's momentum
+    void update(float* data, const float* diff, std::size_t n, unsigned int batchSize, void* stream = nullptr);
 
 protected:
-    double mLearningRate;
-    unsigned int mIterationSize, mIterationPass;
+    double mLearningRate, mMomentum, mDecay;
+    unsigned int mIterationSize, mIterationPass, mNbIterations;
+    float* mMomentumData;
+    std::size_t mMomentumSize;
 };
 template <class T>
 class SGDSolver_Frame_HIP : public SGDSolver {
@@ -827,7 +849,11 @@ protected:
 template <class T>
 class SATQuantizerActivation_Frame_HIP : public SATQuantizerActivation {
 public:
-    SATQuantizerActivation_Frame_HIP() : mDev(nullptr), mFp(nullptr), mFpSize(0), mWorkspace(nullptr), mWorkspaceBytes(0), mStream(nullptr) {}
+    // default solver as in the reference's constructor (SATQuantizerActivation_Frame.cpp:56-64)
+    SATQuantizerActivation_Frame_HIP() : mDev(nullptr), mFp(nullptr), mFpSize(0), mWorkspace(nullptr), mWorkspaceBytes(0), mStream(nullptr)
+    {
+        mSolver = std::make_shared<SGDSolver_Frame_HIP<T> >();
+    }
     ~SATQuantizerActivation_Frame_HIP();
     static std::shared_ptr<SATQuantizerActivation> create() { return std::make_shared<SATQuantizerActivation_Frame_HIP<T> >(); }
     void propagate(float* inOut, std::size_t size, bool inference);

@@ -1,0 +1,407 @@
+// Float cells of the Frame_HIP model for quantization-aware training (see frame_hip_train.hpp).
+#include <hip/hip_runtime_api.h>
+
+#include "frame_hip_train.hpp"
+
+namespace N2D2 {
+
+static void checkHipT(hipError_t e, const char* what)
+{
+    if (e != hipSuccess)
+        throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// --------------------------------------------------------------- DeviceFloats
+DeviceFloats::~DeviceFloats()
+{
+    if (mData) (void)hipFree(mData);
+}
+
+void DeviceFloats::resize(const std::vector<size_t>& dims)
+{
+    std::vector<size_t> d = dims;
+    while (d.size() < 4) d.push_back(1);
+    if (mData) (void)hipFree(mData);
+    mData = nullptr;
+    mDims = d;
+    mValid = false;
+    if (size() == 0)
+        return;
+    checkHipT(hipMalloc((void**)&mData, size() * sizeof(float)), "DeviceFloats::resize()");
+    checkHipT(hipMemset(mData, 0, size() * sizeof(float)), "DeviceFloats::resize()");
+}
+
+void DeviceFloats::fromHost(const float* host, size_t n)
+{
+    if (n != size())
+        throw std::runtime_error("DeviceFloats::fromHost(): size mismatch");
+    checkHipT(hipMemcpy(mData, host, n * sizeof(float), hipMemcpyHostToDevice), "DeviceFloats::fromHost()");
+}
+
+void DeviceFloats::fromHost(const Tensor<Float_T>& host)
+{
+    if (host.dims() != mDims)
+        resize(host.dims());
+    fromHost(host.data(), host.size());
+}
+
+Tensor<Float_T> DeviceFloats::toHost() const
+{
+    Tensor<Float_T> host(mDims);
+    if (size() > 0)
+        checkHipT(hipMemcpy(host.data(), mData, size() * sizeof(float), hipMemcpyDeviceToHost), "DeviceFloats::toHost()");
+    return host;
+}
+
+// -------------------------------------------------------- Cell_FrameTrain_HIP
+Cell_FrameTrain_HIP::~Cell_FrameTrain_HIP()
+{
+    if (mLoss) (void)hipFree(mLoss);
+    if (mLossWorkspace) (void)hipFree(mLossWorkspace);
+}
+
+void Cell_FrameTrain_HIP::addInput(Cell_FrameTrain_HIP* parent)
+{
+    if (!parent)
+        throw std::runtime_error("Cell " + mName + ": null parent");
+    if (mIn)
+        throw std::runtime_error("Cell " + mName + ": the float Frame_HIP cells take one input tensor");
+    if (parent->mOutputs.empty())
+        throw std::runtime_error("Cell " + mName + ": initialize() the parent cell " + parent->getName() + " first");
+    mParents.push_back(parent);
+    mIn = &parent->mOutputs;
+    mDiffOut = &parent->mDiffInputs;
+    mNbChannels = parent->getNbOutputs();
+    mInW = parent->getOutputsWidth();
+    mInH = parent->getOutputsHeight();
+    setOutputsDims();
+}
+
+void Cell_FrameTrain_HIP::addInput(DeviceFloats& inputs, DeviceFloats& diffOutputs)
+{
+    if (mIn)
+        throw std::runtime_error("Cell " + mName + ": the float Frame_HIP cells take one input tensor");
+    if (inputs.empty())
+        throw std::runtime_error("Cell " + mName + ": empty input tensor");
+    if (!diffOutputs.empty() && diffOutputs.dims() != inputs.dims())
+        throw std::runtime_error("Cell " + mName + ": inputs and diffOutputs of different sizes");
+    mParents.push_back(nullptr);
+    mIn = &inputs;
+    mDiffOut = &diffOutputs;
+    mNbChannels = (unsigned int)inputs.dimZ();
+    mInW = (unsigned int)inputs.dimX();
+    mInH = (unsigned int)inputs.dimY();
+    setOutputsDims();
+}
+
+void Cell_FrameTrain_HIP::allocateOutputs()
+{
+    if (!mIn)
+        throw std::runtime_error("Cell " + mName + ": no input");
+    const std::vector<size_t> dims = {mOutW, mOutH, mNbOutputs, mIn->dimB()};
+    mOutputs.resize(dims);
+    mDiffInputs.resize(dims);
+}
+
+void Cell_FrameTrain_HIP::activationPropagate(bool inference)
+{
+    if (!mActivation)
+        return;
+    // RectifierActivation_Frame<T>::propagate / LinearActivation_Frame<T>::propagate of an unquantized cell
+    // (include/Activation/RectifierActivation_Frame.hpp:55-87, LinearActivation_Frame.hpp:56-81), Scaling NONE
+    if (mActivation->getActivationScaling().getMode() != ScalingMode::NONE)
+        throw std::runtime_error("Cell " + mName + ": an activation Scaling belongs to the integer cells (model Frame_HIP)");
+    if (mActivation->abiKind() == N2D2HIP_ACT_RECTIFIER)
+        checkStatus(n2d2hip_rectifier_f32_forward(mOutputs.data(), mOutputs.size(), mActivation->leakSlope(), (float)mActivation->clipping(), mStream));
+    else if (mActivation->clipping() != 0.0)
+        throw std::runtime_error("Cell " + mName + ": LinearActivation Clipping is not supported by the float Frame_HIP cells");
+    if (mActivation->getQuantizer())
+        mActivation->getQuantizer()->propagate(mOutputs.data(), mOutputs.size(), inference);
+}
+
+void Cell_FrameTrain_HIP::activationBackPropagate()
+{
+    if (!mActivation)
+        return;
+    // in place on mDiffInputs: the quantizer first, then the activation's own derivative taken on the cell's outputs
+    // as they are after the quantizer (RectifierActivation_Frame.hpp:89-130, LinearActivation_Frame.hpp:83-123)
+    if (mActivation->getQuantizer())
+        mActivation->getQuantizer()->back_propagate(mDiffInputs.data(), mDiffInputs.data(), mDiffInputs.size());
+    if (mActivation->abiKind() == N2D2HIP_ACT_RECTIFIER)
+        checkStatus(n2d2hip_rectifier_f32_backward(mOutputs.data(), mDiffInputs.data(), mDiffInputs.data(), mDiffInputs.size(),
+                                                   mActivation->leakSlope(), (float)mActivation->clipping(), mStream));
+}
+
+void Cell_FrameTrain_HIP::activationUpdate()
+{
+    if (mActivation && mActivation->getQuantizer())
+        mActivation->getQuantizer()->update((unsigned int)mIn->dimB());
+}
+
+double Cell_FrameTrain_HIP::applyLoss()
+{
+    const size_t n = mOutputs.size();
+    if (!mLoss)
+        checkHipT(hipMalloc((void**)&mLoss, sizeof(double)), "Cell_FrameTrain_HIP::applyLoss()");
+    const size_t need = n2d2hip_loss_workspace_bytes(n);
+    if (mLossWorkspaceBytes < need) {
+        if (mLossWorkspace) (void)hipFree(mLossWorkspace);
+        mLossWorkspace = nullptr;
+        checkHipT(hipMalloc(&mLossWorkspace, need), "Cell_FrameTrain_HIP::applyLoss()");
+        mLossWorkspaceBytes = need;
+    }
+    // target and diff are the same buffer: each element is read, then written, by one thread
+    checkStatus(n2d2hip_loss_f32(mDiffInputs.data(), mOutputs.data(), mDiffInputs.data(), n, (int)mOutputs.dimB(), mLoss,
+                                 mLossWorkspace, mLossWorkspaceBytes, mStream));
+    mDiffInputs.setValid();
+    double loss = 0.0;
+    checkHipT(hipMemcpy(&loss, mLoss, sizeof(double), hipMemcpyDeviceToHost), "Cell_FrameTrain_HIP::applyLoss()");
+    return loss;
+}
+
+// ------------------------------------------------------ ConvCell_FrameTrain_HIP
+template <class T>
+ConvCell_FrameTrain_HIP<T>::ConvCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& kernelDims,
+                                                    unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
+                                                    const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+                                                    const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims),
+      mWeightsSolver(std::make_shared<SGDSolver_Frame_HIP<T> >()), mBiasSolver(std::make_shared<SGDSolver_Frame_HIP<T> >())
+{
+    mActivation = activation;
+}
+
+template <class T>
+ConvCell_FrameTrain_HIP<T>::~ConvCell_FrameTrain_HIP() {}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::setOutputsDims()
+{
+    // src/Cell/ConvCell.cpp:1169-1195
+    const unsigned int in[2] = {mInW, mInH};
+    unsigned int out[2];
+    for (int dim = 0; dim < 2; ++dim) {
+        const int kernelExtent = (int)(mDilationDims[dim] * (mKernelDims[dim] - 1) + 1);
+        out[dim] = (unsigned int)std::floor(((int)in[dim] + 2 * mPaddingDims[dim] - kernelExtent + (int)mStrideDims[dim]) / (double)mStrideDims[dim]);
+    }
+    mOutW = out[0];
+    mOutH = out[1];
+}
+
+template <class T>
+n2d2hip_conv_desc ConvCell_FrameTrain_HIP<T>::desc() const
+{
+    n2d2hip_conv_desc d = {};
+    d.C = (int)mNbChannels;
+    d.O = (int)mNbOutputs;
+    d.kW = (int)mKernelDims[0];
+    d.kH = (int)mKernelDims[1];
+    d.strideX = (int)mStrideDims[0];
+    d.strideY = (int)mStrideDims[1];
+    d.padL = d.padR = mPaddingDims[0];
+    d.padT = d.padB = mPaddingDims[1];
+    d.dilX = (int)mDilationDims[0];
+    d.dilY = (int)mDilationDims[1];
+    d.groups = (int)mNbGroups;
+    return d;
+}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::initialize()
+{
+    allocateOutputs();
+    const std::vector<size_t> wdims = {mKernelDims[0], mKernelDims[1], mNbChannels / mNbGroups, mNbOutputs};
+    if (mWeights.dims() != wdims)
+        throw std::runtime_error("ConvCell_FrameTrain_HIP " + mName + ": setWeights() with a {kW, kH, C/groups, O} tensor before initialize()");
+    mDevW.fromHost(mWeights);
+    mDevDiffW.resize(wdims);
+    if (!mNoBias) {
+        if (mBias.size() != mNbOutputs)
+            mBias.resize({mNbOutputs}, 0.0f);
+        mDevBias.resize({mNbOutputs});
+        mDevBias.fromHost(mBias.data(), mNbOutputs);
+        mDevDiffBias.resize({mNbOutputs});
+    }
+    if (mQuantizer) {
+        // Cell_Frame / ConvCell_Frame::initialize hand each weight tensor and its gradient to the quantizer
+        // (src/Cell/ConvCell_Frame.cpp:288-300); outputsSize = dimB * dimY * dimX of the weight tensor
+        mQuantizer->addWeights(mDevW.data(), mDevDiffW.data(), mDevW.size(), (size_t)mNbOutputs * mKernelDims[1] * mKernelDims[0]);
+        mQuantizer->initialize();
+    }
+}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::propagate(bool inference)
+{
+    if (mQuantizer)
+        mQuantizer->propagate();
+    const n2d2hip_conv_desc d = desc();
+    const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+    // a quantizer passes the biases through (quantize_bias_propagate copies them)
+    checkStatus(n2d2hip_conv2d_f32_forward(&d, (int)mIn->dimB(), (int)mInH, (int)mInW, mIn->data(), w, mNoBias ? nullptr : mDevBias.data(), 0.0f,
+                                           mOutputs.data(), mStream));
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+    mDevDiffW.clearValid();
+    mDevDiffBias.clearValid();
+}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::backPropagate()
+{
+    if (!mDiffInputs.isValid())
+        return;
+    activationBackPropagate();
+    const n2d2hip_conv_desc d = desc();
+    const int B = (int)mIn->dimB();
+    {
+        const float beta = mWeightsSolver->isNewIteration() ? 0.0f : 1.0f;
+        checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(), mStream));
+        mDevDiffW.setValid();
+    }
+    if (!mNoBias) {
+        const float beta = mBiasSolver->isNewIteration() ? 0.0f : 1.0f;
+        checkStatus(n2d2hip_conv2d_f32_backward_bias(B, (int)mNbOutputs, (int)mOutH, (int)mOutW, mDiffInputs.data(), beta, mDevDiffBias.data(), mStream));
+        mDevDiffBias.setValid();
+    }
+    if (mDiffOut && !mDiffOut->empty()) {
+        const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
+        const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+        checkStatus(n2d2hip_conv2d_f32_backward_data(&d, B, (int)mInH, (int)mInW, w, mDiffInputs.data(), beta, mDiffOut->data(), mStream));
+        mDiffOut->setValid();
+    }
+    if (mQuantizer)
+        mQuantizer->back_propagate();
+}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::update()
+{
+    const unsigned int batch = (unsigned int)mIn->dimB();
+    if (mDevDiffW.isValid())
+        mWeightsSolver->update(mDevW.data(), mQuantizer ? mQuantizer->getDiffFullPrecisionWeights(0) : mDevDiffW.data(), mDevW.size(), batch, mStream);
+    if (!mNoBias && mDevDiffBias.isValid())
+        mBiasSolver->update(mDevBias.data(), mDevDiffBias.data(), mDevBias.size(), batch, mStream);
+    if (mQuantizer)
+        mQuantizer->update(batch);
+    activationUpdate();
+}
+
+template <class T>
+void ConvCell_FrameTrain_HIP<T>::synchronizeWeightsToHost()
+{
+    mWeights = mDevW.toHost();
+    if (!mNoBias) {
+        const Tensor<Float_T> b = mDevBias.toHost();
+        mBias.resize({mNbOutputs});
+        for (size_t i = 0; i < mNbOutputs; ++i) mBias(i) = b(i);
+    }
+}
+
+template <class T>
+Tensor<Float_T> ConvCell_FrameTrain_HIP<T>::getQuantizedWeights() const
+{
+    Tensor<Float_T> host(mDevW.dims());
+    const float* src = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+    checkHipT(hipMemcpy(host.data(), src, host.size() * sizeof(float), hipMemcpyDeviceToHost), "ConvCell_FrameTrain_HIP::getQuantizedWeights()");
+    return host;
+}
+
+template class ConvCell_FrameTrain_HIP<float>;
+template <> Registrar<ConvCell> ConvCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", ConvCell_FrameTrain_HIP<float>::create,
+                                                                           Registrar<ConvCell>::Type<float>());
+
+// ------------------------------------------------ ActivationCell_FrameTrain_HIP
+const char* ActivationCell::Type = "Activation";
+
+template <class T>
+ActivationCell_FrameTrain_HIP<T>::ActivationCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
+                                                                const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs)
+{
+    mActivation = activation;
+}
+
+template <class T>
+void ActivationCell_FrameTrain_HIP<T>::initialize()
+{
+    if (!mActivation)
+        throw std::runtime_error("ActivationCell_FrameTrain_HIP " + mName + ": no activation");
+    if (mNbChannels != mNbOutputs)
+        throw std::runtime_error("ActivationCell_FrameTrain_HIP " + mName + ": the number of outputs must be the number of input channels");
+    allocateOutputs();
+}
+
+template <class T>
+void ActivationCell_FrameTrain_HIP<T>::propagate(bool inference)
+{
+    checkHipT(hipMemcpyAsync(mOutputs.data(), mIn->data(), mOutputs.size() * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)mStream),
+              "ActivationCell_FrameTrain_HIP::propagate()");
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+}
+
+template <class T>
+void ActivationCell_FrameTrain_HIP<T>::backPropagate()
+{
+    if (!mDiffInputs.isValid())
+        return;
+    if (!mDiffOut || mDiffOut->empty())
+        return;
+    // out of place in the reference (mDiffInputs -> diffOutput); the quantizers' gradients come out the same
+    activationBackPropagate();
+    checkHipT(hipMemcpyAsync(mDiffOut->data(), mDiffInputs.data(), mDiffInputs.size() * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)mStream),
+              "ActivationCell_FrameTrain_HIP::backPropagate()");
+    mDiffOut->setValid();
+}
+
+template class ActivationCell_FrameTrain_HIP<float>;
+template <> Registrar<ActivationCell> ActivationCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", ActivationCell_FrameTrain_HIP<float>::create,
+                                                                                       Registrar<ActivationCell>::Type<float>());
+
+// --------------------------------------------------- SoftmaxCell_FrameTrain_HIP
+const char* SoftmaxCell::Type = "Softmax";
+
+template <class T>
+SoftmaxCell_FrameTrain_HIP<T>::SoftmaxCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs, bool withLoss,
+                                                          unsigned int groupSize)
+    : Cell(name, nbOutputs), SoftmaxCell(withLoss, groupSize)
+{
+    if (groupSize != 0 && groupSize != nbOutputs)
+        throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + name + ": GroupSize is not supported by the float Frame_HIP cells");
+}
+
+template <class T>
+void SoftmaxCell_FrameTrain_HIP<T>::initialize()
+{
+    if (mNbChannels != mNbOutputs)
+        throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + mName + ": the number of outputs must be the number of input channels");
+    allocateOutputs();
+}
+
+template <class T>
+void SoftmaxCell_FrameTrain_HIP<T>::propagate(bool /*inference*/)
+{
+    checkStatus(n2d2hip_softmax_f32_forward(mIn->data(), mOutputs.data(), (int)mIn->dimB(), (int)mNbOutputs, (int)mOutH, (int)mOutW, mStream));
+    mDiffInputs.clearValid();
+}
+
+template <class T>
+void SoftmaxCell_FrameTrain_HIP<T>::backPropagate()
+{
+    if (!mDiffOut || mDiffOut->empty() || !mDiffInputs.isValid())
+        return;
+    if (!mWithLoss)
+        throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + mName + ": backPropagate() without WithLoss is not supported by the float Frame_HIP cells");
+    if (mDiffOut->isValid())
+        throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + mName + ": accumulation onto a valid diffOutputs is not supported");
+    checkHipT(hipMemcpyAsync(mDiffOut->data(), mDiffInputs.data(), mDiffInputs.size() * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)mStream),
+              "SoftmaxCell_FrameTrain_HIP::backPropagate()");
+    mDiffOut->setValid();
+}
+
+template class SoftmaxCell_FrameTrain_HIP<float>;
+template <> Registrar<SoftmaxCell> SoftmaxCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", SoftmaxCell_FrameTrain_HIP<float>::create,
+                                                                                 Registrar<SoftmaxCell>::Type<float>());
+
+} // namespace N2D2

@@ -1,0 +1,205 @@
+// Float cells of the Frame_HIP model for quantization-aware training: the cells a SAT / LSQ graph learns with
+// (convolution with a weight quantizer, activation with an activation quantizer, softmax with loss), device resident,
+// with propagate / backPropagate / update as the reference's Frame cells have them.  Tensors are N2D2's own float
+// tensors ({X,Y,Z,B}, X fastest) held in device memory; every computation goes through the C ABI (n2d2hip.h).
+//
+// These cells are registered under the model key "Frame_HIP_QAT": the key "Frame_HIP" holds the integer inference
+// cells, which have the same cell types and the same element type (float) in the Registrar.
+#ifndef N2D2_FRAME_HIP_TRAIN_HPP
+#define N2D2_FRAME_HIP_TRAIN_HPP
+
+#include "frame_hip.hpp"
+
+namespace N2D2 {
+
+// Device float tensor with N2D2's dimension order and the "valid" flag the reference keeps on gradient tensors
+// (BaseTensor::isValid / setValid / clearValid, include/containers/Tensor.hpp:137-139).
+class DeviceFloats {
+public:
+    DeviceFloats() : mData(nullptr), mDims{0, 0, 0, 0}, mValid(false) {}
+    ~DeviceFloats();
+    DeviceFloats(const DeviceFloats&) = delete;
+    DeviceFloats& operator=(const DeviceFloats&) = delete;
+    void resize(const std::vector<size_t>& dims);        // zero-filled
+    bool empty() const { return mData == nullptr; }
+    size_t dimX() const { return mDims[0]; }
+    size_t dimY() const { return mDims[1]; }
+    size_t dimZ() const { return mDims[2]; }
+    size_t dimB() const { return mDims[3]; }
+    const std::vector<size_t>& dims() const { return mDims; }
+    size_t size() const { return mDims[0] * mDims[1] * mDims[2] * mDims[3]; }
+    float* data() { return mData; }
+    const float* data() const { return mData; }
+    bool isValid() const { return mValid; }
+    void setValid() { mValid = true; }
+    void clearValid() { mValid = false; }
+    void fromHost(const Tensor<Float_T>& host);
+    void fromHost(const float* host, size_t n);
+    Tensor<Float_T> toHost() const;
+
+private:
+    float* mData;
+    std::vector<size_t> mDims;
+    bool mValid;
+};
+
+// Common part of the float cells (the role of Cell_Frame<T>, src/Cell/Cell_Frame.cpp:100-160 and :474-492): one input
+// tensor and the tensor its gradient goes to, own outputs and the gradient with respect to them, the activation
+// applied in place.
+class Cell_FrameTrain_HIP : public virtual Cell {
+public:
+    // Cell::addInput(Cell*): input = the parent's outputs, diffOutputs = the parent's diffInputs
+    virtual void addInput(Cell_FrameTrain_HIP* parent);
+    // Cell_Frame<T>::addInput(BaseTensor& inputs, BaseTensor& diffOutputs): an empty diffOutputs stops the gradient here
+    virtual void addInput(DeviceFloats& inputs, DeviceFloats& diffOutputs);
+    virtual void initialize() = 0;
+    virtual void propagate(bool inference = false) = 0;
+    virtual void backPropagate() = 0;
+    virtual void update() = 0;
+    DeviceFloats& getOutputs() { return mOutputs; }
+    DeviceFloats& getDiffInputs() { return mDiffInputs; }
+    // Cell_Frame<T>::applyLoss() (src/Cell/Cell_Frame.cpp:646-650 over Cell_Frame_Top::applyLoss,
+    // src/Cell/Cell_Frame_Top.cpp:27-40): diffInputs, holding the targets, becomes targets - outputs; returns the sum of
+    // squares over the batch size
+    double applyLoss();
+    bool isCuda() const { return false; }
+    std::string getPyModel() const { return "Frame_HIP_QAT"; }
+    void setStream(void* stream) { mStream = stream; }
+
+protected:
+    Cell_FrameTrain_HIP() : mIn(nullptr), mDiffOut(nullptr), mStream(nullptr), mLoss(nullptr), mLossWorkspace(nullptr), mLossWorkspaceBytes(0) {}
+    ~Cell_FrameTrain_HIP();
+    virtual void setOutputsDims() = 0;
+    void allocateOutputs();
+    // Cell_Frame<T>::propagate / backPropagate / update: the activation in place on mOutputs / mDiffInputs
+    void activationPropagate(bool inference);
+    void activationBackPropagate();
+    void activationUpdate();
+    DeviceFloats* mIn;
+    DeviceFloats* mDiffOut;
+    DeviceFloats mOutputs, mDiffInputs;
+    void* mStream;
+
+private:
+    double* mLoss;
+    void* mLossWorkspace;
+    size_t mLossWorkspaceBytes;
+};
+
+// src/Cell/ConvCell_Frame.cpp:418-597 for one input tensor.
+template <class T>
+class ConvCell_FrameTrain_HIP : public ConvCell, public Cell_FrameTrain_HIP {
+public:
+    ConvCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, const std::vector<unsigned int>& kernelDims,
+                            unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
+                            const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
+                            const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation);
+    ~ConvCell_FrameTrain_HIP();
+    static std::shared_ptr<ConvCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name,
+                                            const std::vector<unsigned int>& kernelDims, unsigned int nbOutputs,
+                                            const std::vector<unsigned int>& subSampleDims, const std::vector<unsigned int>& strideDims,
+                                            const std::vector<int>& paddingDims, const std::vector<unsigned int>& dilationDims,
+                                            const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<ConvCell_FrameTrain_HIP<T> >(deepNet, name, kernelDims, nbOutputs, subSampleDims, strideDims,
+                                                             paddingDims, dilationDims, activation);
+    }
+    // Cell::setQuantizer (include/Cell/Cell.hpp:455-463), before initialize()
+    void setQuantizer(const std::shared_ptr<QuantizerCell>& quantizer) { mQuantizer = quantizer; }
+    const std::shared_ptr<QuantizerCell>& getQuantizer() const { return mQuantizer; }
+    void setWeightsSolver(const std::shared_ptr<SGDSolver>& solver) { mWeightsSolver = solver; }
+    void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
+    // uploads the host weights / biases (ConvCell::setWeights), allocates gradients, hands the weights to the quantizer
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update();
+    // refreshes the host tensors ConvCell::getWeights() / getBiases() return from the device
+    void synchronizeWeightsToHost();
+    Tensor<Float_T> getDiffWeights() const { return mDevDiffW.toHost(); }
+    Tensor<Float_T> getQuantizedWeights() const;
+
+protected:
+    void setOutputsDims();
+
+private:
+    n2d2hip_conv_desc desc() const;
+    std::shared_ptr<QuantizerCell> mQuantizer;
+    std::shared_ptr<SGDSolver> mWeightsSolver, mBiasSolver;
+    DeviceFloats mDevW, mDevDiffW, mDevBias, mDevDiffBias;
+    static Registrar<ConvCell> mRegistrar;
+};
+
+// include/Cell/ActivationCell.hpp:36-60
+class ActivationCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<ActivationCell>(const DeepNet&, const std::string&, unsigned int,
+                                                          const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+};
+
+// src/Cell/ActivationCell_Frame.cpp:95-205 for one input: copy, then the activation in place.
+template <class T>
+class ActivationCell_FrameTrain_HIP : public ActivationCell, public Cell_FrameTrain_HIP {
+public:
+    ActivationCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                  const std::shared_ptr<Activation>& activation);
+    static std::shared_ptr<ActivationCell> create(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                                  const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<ActivationCell_FrameTrain_HIP<T> >(deepNet, name, nbOutputs, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update() { activationUpdate(); }
+
+protected:
+    void setOutputsDims() { mOutW = mInW; mOutH = mInH; }
+
+private:
+    static Registrar<ActivationCell> mRegistrar;
+};
+
+// include/Cell/SoftmaxCell.hpp:37-70: WithLoss (false), GroupSize (0)
+class SoftmaxCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<SoftmaxCell>(const DeepNet&, const std::string&, unsigned int, bool, unsigned int)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+
+protected:
+    SoftmaxCell(bool withLoss, unsigned int groupSize) : mWithLoss(withLoss), mGroupSize(groupSize) {}
+    bool mWithLoss;
+    unsigned int mGroupSize;
+};
+
+// src/Cell/SoftmaxCell_Frame.cpp:93-207, one group, WithLoss (the gradient of the loss passes through unchanged).
+template <class T>
+class SoftmaxCell_FrameTrain_HIP : public SoftmaxCell, public Cell_FrameTrain_HIP {
+public:
+    SoftmaxCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, bool withLoss = false,
+                               unsigned int groupSize = 0);
+    static std::shared_ptr<SoftmaxCell> create(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, bool withLoss,
+                                               unsigned int groupSize)
+    {
+        return std::make_shared<SoftmaxCell_FrameTrain_HIP<T> >(deepNet, name, nbOutputs, withLoss, groupSize);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update() {}
+
+protected:
+    void setOutputsDims() { mOutW = mInW; mOutH = mInH; }
+
+private:
+    static Registrar<SoftmaxCell> mRegistrar;
+};
+
+} // namespace N2D2
+
+#endif

@@ -1,0 +1,268 @@
+// C entry points over the float training cells, for the Python test-suite: build a sequential net of ActivationCell /
+// ConvCell / SoftmaxCell through the Registrar, attach SAT or LSQ quantizers, run learning iterations, read parameters.
+// Every function returns 0 on success; fh_train_last_error() holds the message of the last C++ exception.
+#include <cstring>
+
+#include <hip/hip_runtime_api.h>
+
+#include "frame_hip_train.hpp"
+
+using namespace N2D2;
+
+namespace {
+thread_local std::string g_train_error;
+template <class F>
+int guardedT(F f)
+{
+    try {
+        f();
+        return 0;
+    } catch (const std::exception& e) {
+        g_train_error = e.what();
+        return 1;
+    }
+}
+
+struct TrainNet {
+    std::string model;
+    Network net;
+    DeepNet deepNet;
+    DeviceFloats input, inputDiff, targets;
+    std::vector<std::shared_ptr<Cell_FrameTrain_HIP> > cells;
+    std::map<std::string, std::shared_ptr<SATQuantizerActivation_Frame_HIP<float> > > satAct;
+    std::map<std::string, std::shared_ptr<LSQQuantizerActivation_Frame_HIP<float> > > lsqAct;
+    Cell_FrameTrain_HIP* last() { return cells.empty() ? nullptr : cells.back().get(); }
+};
+
+// act: -1 none, 0 Linear, 1 Rectifier; actQuant: 0 none, 1 SAT (param = alpha), 2 LSQ (param = step size, <= 0: optimal init)
+std::shared_ptr<Activation> makeActivation(TrainNet& n, const std::string& name, int act, int actQuant, int range, float param)
+{
+    if (act < 0)
+        return std::shared_ptr<Activation>();
+    std::shared_ptr<Activation> a;
+    if (act == 0) {
+        auto f = Registrar<LinearActivation>::create<float>("Frame_HIP");
+        a = f();
+    } else {
+        auto f = Registrar<RectifierActivation>::create<float>("Frame_HIP");
+        a = f();
+    }
+    if (actQuant == 1) {
+        auto q = std::dynamic_pointer_cast<SATQuantizerActivation_Frame_HIP<float> >(Registrar<SATQuantizerActivation>::create<float>("Frame_HIP")());
+        q->setRange((size_t)range);
+        q->setAlpha(param);
+        a->setQuantizer(q);
+        n.satAct[name] = q;
+    } else if (actQuant == 2) {
+        auto q = std::dynamic_pointer_cast<LSQQuantizerActivation_Frame_HIP<float> >(Registrar<LSQQuantizerActivation>::create<float>("Frame_HIP")());
+        q->setRange((size_t)range);
+        if (param > 0.0f) { q->setStepSizeValue(param); q->setOptInitStepSize(false); }
+        q->setSolver(Registrar<SGDSolver>::create<float>("Frame_HIP")());
+        a->setQuantizer(q);
+        n.lsqAct[name] = q;
+    }
+    return a;
+}
+
+void connect(TrainNet& n, const std::shared_ptr<Cell_FrameTrain_HIP>& cell)
+{
+    if (n.cells.empty())
+        cell->addInput(n.input, n.inputDiff);
+    else
+        cell->addInput(n.cells.back().get());
+    cell->initialize();
+    n.cells.push_back(cell);
+}
+
+Cell_FrameTrain_HIP* find(TrainNet& n, const char* name)
+{
+    for (auto& c : n.cells)
+        if (c->getName() == name) return c.get();
+    throw std::runtime_error("No cell named \"" + std::string(name) + "\"");
+}
+} // namespace
+
+extern "C" {
+
+const char* fh_train_last_error(void) { return g_train_error.c_str(); }
+
+int fh_train_registrar_exists(const char* type, const char* key)
+{
+    const std::string t(type), k(key);
+    if (t == "Conv") return Registrar<ConvCell>::exists<float>(k);
+    if (t == "Activation") return Registrar<ActivationCell>::exists<float>(k);
+    if (t == "Softmax") return Registrar<SoftmaxCell>::exists<float>(k);
+    return -1;
+}
+
+// The environment: a float tensor [B,C,H,W]; propagateGradient != 0 gives the first cell a tensor to write its
+// input gradient to (an ActivationCell computes its quantizer's gradient only then, as in the reference).
+int fh_train_net_create(const char* model, const float* input, int B, int C, int H, int W, int propagateGradient, void** out)
+{
+    return guardedT([&] {
+        std::unique_ptr<TrainNet> n(new TrainNet);
+        n->model = model;
+        const std::vector<size_t> dims = {(size_t)W, (size_t)H, (size_t)C, (size_t)B};
+        n->input.resize(dims);
+        n->input.fromHost(input, n->input.size());
+        if (propagateGradient)
+            n->inputDiff.resize(dims);
+        *out = n.release();
+    });
+}
+
+void fh_train_net_destroy(void* net) { delete (TrainNet*)net; }
+
+int fh_train_add_activation_cell(void* net, const char* name, int act, int actQuant, int range, float param)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<ActivationCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        const unsigned int nbOutputs = n.cells.empty() ? (unsigned int)n.input.dimZ() : n.last()->getNbOutputs();
+        auto cell = std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(f(n.deepNet, name, nbOutputs, makeActivation(n, name, act, actQuant, range, param)));
+        connect(n, cell);
+    });
+}
+
+// weights: HOST float [O, C/groups, kH, kW]; bias HOST float [O] or NULL (NoBias).  weightQuant: 0 none, 1 SAT, 2 LSQ.
+int fh_train_add_conv(void* net, const char* name, int nbOutputs, int kW, int kH, int strideX, int strideY, int padX, int padY, int depthwise,
+                      const float* weights, const float* bias, int act, int actQuant, int actRange, float actParam,
+                      int weightQuant, int weightRange, int applyQuantization, int applyScaling, int quantMode)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<ConvCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        auto conv = f(n.net, n.deepNet, name, {(unsigned)kW, (unsigned)kH}, (unsigned)nbOutputs, {1U, 1U}, {(unsigned)strideX, (unsigned)strideY},
+                      {padX, padY}, {1U, 1U}, makeActivation(n, name, act, actQuant, actRange, actParam));
+        auto cell = std::dynamic_pointer_cast<ConvCell_FrameTrain_HIP<float> >(conv);
+        const unsigned int nbChannels = n.cells.empty() ? (unsigned int)n.input.dimZ() : n.last()->getNbOutputs();
+        const unsigned int groups = depthwise ? nbChannels : 1;
+        conv->setNbGroups(groups);
+        conv->setParameter("NoBias", bias == nullptr);
+        Tensor<Float_T> w({(size_t)kW, (size_t)kH, (size_t)(nbChannels / groups), (size_t)nbOutputs});
+        std::memcpy(w.data(), weights, w.size() * sizeof(float));
+        conv->setWeights(w);
+        if (bias) {
+            Tensor<Float_T> b({(size_t)nbOutputs});
+            std::memcpy(b.data(), bias, nbOutputs * sizeof(float));
+            conv->setBiases(b);
+        }
+        if (weightQuant == 1) {
+            auto q = Registrar<SATQuantizerCell>::create<float>("Frame_HIP")();
+            q->setRange((size_t)weightRange);
+            q->setQuantization(applyQuantization != 0);
+            q->setScaling(applyScaling != 0);
+            q->setQuantMode((QuantizerCell::QuantMode)quantMode);
+            cell->setQuantizer(q);
+        } else if (weightQuant == 2) {
+            auto q = Registrar<LSQQuantizerCell>::create<float>("Frame_HIP")();
+            q->setRange((size_t)weightRange);
+            q->setSolver(Registrar<SGDSolver>::create<float>("Frame_HIP")());
+            cell->setQuantizer(q);
+        }
+        connect(n, cell);
+    });
+}
+
+int fh_train_add_softmax(void* net, const char* name, int withLoss)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<SoftmaxCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        if (n.cells.empty()) throw std::runtime_error("A SoftmaxCell needs a parent cell");
+        auto cell = std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(f(n.deepNet, name, n.last()->getNbOutputs(), withLoss != 0, 0U));
+        connect(n, cell);
+    });
+}
+
+// Solver parameters of a convolution's weights ("LearningRate", "Momentum", "Decay", "IterationSize")
+int fh_train_set_solver_parameter(void* net, const char* cell, const char* name, double value)
+{
+    return guardedT([&] {
+        auto conv = dynamic_cast<ConvCell_FrameTrain_HIP<float>*>(find(*(TrainNet*)net, cell));
+        if (!conv) throw std::runtime_error("Not a ConvCell: " + std::string(cell));
+        auto s = Registrar<SGDSolver>::create<float>("Frame_HIP")();
+        s->setParameter(name, value);
+        conv->setWeightsSolver(s);
+    });
+}
+
+// targets: HOST float, the shape of the last cell's outputs.  Runs `iterations` times what the reference's learning
+// loop runs: propagate front to back, targets into the last cell's diffInputs, applyLoss, backPropagate back to front,
+// update back to front.  loss receives the last iteration's.
+int fh_train_learn(void* net, const float* targets, size_t nTargets, int iterations, double* loss)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        if (n.cells.empty()) throw std::runtime_error("Empty net");
+        Cell_FrameTrain_HIP* last = n.last();
+        if (nTargets != last->getOutputs().size()) throw std::runtime_error("fh_train_learn(): wrong number of targets");
+        n.targets.resize(last->getOutputs().dims());
+        n.targets.fromHost(targets, nTargets);
+        double l = 0.0;
+        for (int it = 0; it < iterations; ++it) {
+            for (auto& c : n.cells) c->propagate(false);
+            if (hipMemcpyAsync(last->getDiffInputs().data(), n.targets.data(), nTargets * sizeof(float), hipMemcpyDeviceToDevice, nullptr) != hipSuccess)
+                throw std::runtime_error("fh_train_learn(): copy of the targets failed");
+            l = last->applyLoss();
+            for (auto c = n.cells.rbegin(); c != n.cells.rend(); ++c) (*c)->backPropagate();
+            for (auto c = n.cells.rbegin(); c != n.cells.rend(); ++c) (*c)->update();
+        }
+        if (hipDeviceSynchronize() != hipSuccess) throw std::runtime_error("fh_train_learn(): device error");
+        if (loss) *loss = l;
+    });
+}
+
+// One forward pass; inference != 0 runs the quantizers without saving what backPropagate needs
+int fh_train_propagate(void* net, int inference)
+{
+    return guardedT([&] {
+        for (auto& c : ((TrainNet*)net)->cells) c->propagate(inference != 0);
+        if (hipDeviceSynchronize() != hipSuccess) throw std::runtime_error("fh_train_propagate(): device error");
+    });
+}
+
+// what: 0 outputs, 1 diffInputs, 2 weights, 3 gradient of the (quantized) weights, 4 quantized weights
+int fh_train_get(void* net, const char* cell, int what, float* out, size_t n)
+{
+    return guardedT([&] {
+        Cell_FrameTrain_HIP* c = find(*(TrainNet*)net, cell);
+        Tensor<Float_T> t;
+        auto conv = dynamic_cast<ConvCell_FrameTrain_HIP<float>*>(c);
+        if (what == 0) t = c->getOutputs().toHost();
+        else if (what == 1) t = c->getDiffInputs().toHost();
+        else if (!conv) throw std::runtime_error("Not a ConvCell: " + std::string(cell));
+        else if (what == 2) { conv->synchronizeWeightsToHost(); t = conv->getWeights(); }
+        else if (what == 3) t = conv->getDiffWeights();
+        else t = conv->getQuantizedWeights();
+        if (t.size() != n) throw std::runtime_error("fh_train_get(): size mismatch");
+        std::memcpy(out, t.data(), n * sizeof(float));
+    });
+}
+
+int fh_train_input_gradient(void* net, float* out, size_t n)
+{
+    return guardedT([&] {
+        const Tensor<Float_T> t = ((TrainNet*)net)->inputDiff.toHost();
+        if (t.size() != n) throw std::runtime_error("fh_train_input_gradient(): size mismatch");
+        std::memcpy(out, t.data(), n * sizeof(float));
+    });
+}
+
+// The learned parameter of a cell's activation quantizer: SAT alpha or LSQ step size; grad receives its last gradient
+int fh_train_get_activation_quantizer(void* net, const char* cell, float* value, float* grad)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto s = n.satAct.find(cell);
+        auto l = n.lsqAct.find(cell);
+        if (s != n.satAct.end()) { *value = s->second->getAlpha(); if (grad) *grad = s->second->getDiffAlpha(); }
+        else if (l != n.lsqAct.end()) { *value = l->second->getStepSize(); if (grad) *grad = l->second->getDiffStepSize(); }
+        else throw std::runtime_error("No activation quantizer on cell \"" + std::string(cell) + "\"");
+    });
+}
+
+} // extern "C"

@@ -247,3 +247,118 @@ def build_net(spec, batch, model="Frame_HIP"):
         elif l.type == "pool":
             net.set_quantized(l.name, 8)
     return net
+
+
+# ------------------------------------------------------------------ float cells for quantization-aware training
+lib.fh_train_last_error.restype = C.c_char_p
+lib.fh_train_registrar_exists.argtypes = [C.c_char_p, C.c_char_p]
+lib.fh_train_net_create.argtypes = [C.c_char_p, _P, _I, _I, _I, _I, _I, _P]
+lib.fh_train_net_destroy.argtypes = [_P]
+lib.fh_train_net_destroy.restype = None
+lib.fh_train_add_activation_cell.argtypes = [_P, C.c_char_p, _I, _I, _I, _F]
+lib.fh_train_add_conv.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _F, _I, _I, _I, _I, _I]
+lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
+lib.fh_train_set_solver_parameter.argtypes = [_P, C.c_char_p, C.c_char_p, C.c_double]
+lib.fh_train_learn.argtypes = [_P, _P, _SZ, _I, _P]
+lib.fh_train_propagate.argtypes = [_P, _I]
+lib.fh_train_get.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
+lib.fh_train_input_gradient.argtypes = [_P, _P, _SZ]
+lib.fh_train_get_activation_quantizer.argtypes = [_P, C.c_char_p, _P, _P]
+
+TRAIN_MODEL = "Frame_HIP_QAT"
+_ACT = {None: -1, "Linear": 0, "Rectifier": 1}
+_QUANT = {None: 0, "SAT": 1, "LSQ": 2}
+_QUANT_MODE = {"Default": 0, "Symmetric": 1, "Asymmetric": 2, "FullRange": 3}
+
+
+def _check_train(rc):
+    if rc != 0:
+        raise FrameHipError(lib.fh_train_last_error().decode())
+
+
+class TrainNet:
+    """A sequential net of the float Frame_HIP cells (ActivationCell, ConvCell, SoftmaxCell) with SAT / LSQ quantizers,
+    created through the Registrar under `model`. x: float32 [B,C,H,W]."""
+
+    def __init__(self, x, model=TRAIN_MODEL, propagate_gradient=True):
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        self._h = C.c_void_p()
+        self._shapes = {}
+        self._last = x.shape
+        _check_train(lib.fh_train_net_create(model.encode(), x.ctypes.data, x.shape[0], x.shape[1], x.shape[2], x.shape[3],
+                                             int(propagate_gradient), C.byref(self._h)))
+        self.input_shape = x.shape
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib.fh_train_net_destroy(self._h)
+            self._h = None
+
+    def add_activation_cell(self, name, act="Linear", act_quant=None, act_range=255, act_param=1.0):
+        _check_train(lib.fh_train_add_activation_cell(self._h, name.encode(), _ACT[act], _QUANT[act_quant], act_range, act_param))
+        self._shapes[name] = self._last
+
+    def add_conv(self, name, weights, bias=None, stride=(1, 1), pad=(0, 0), depthwise=False, act=None, act_quant=None, act_range=255,
+                 act_param=1.0, weight_quant=None, weight_range=255, apply_quantization=True, apply_scaling=False, quant_mode="Default"):
+        """weights: [O, C/groups, kH, kW]; stride / pad are (x, y)."""
+        w = np.ascontiguousarray(weights, dtype=np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+        O, _, kH, kW = w.shape
+        _check_train(lib.fh_train_add_conv(self._h, name.encode(), O, kW, kH, stride[0], stride[1], pad[0], pad[1], int(depthwise),
+                                           w.ctypes.data, None if b is None else b.ctypes.data, _ACT[act], _QUANT[act_quant], act_range,
+                                           act_param, _QUANT[weight_quant], weight_range, int(apply_quantization), int(apply_scaling),
+                                           _QUANT_MODE[quant_mode]))
+        B, _, H, W = self._last
+        oH = (H + 2 * pad[1] - kH + stride[1]) // stride[1]
+        oW = (W + 2 * pad[0] - kW + stride[0]) // stride[0]
+        self._last = (B, O, oH, oW)
+        self._shapes[name] = self._last
+        self._shapes[name + "/weights"] = w.shape
+
+    def add_softmax(self, name, with_loss=True):
+        _check_train(lib.fh_train_add_softmax(self._h, name.encode(), int(with_loss)))
+        self._shapes[name] = self._last
+
+    def set_solver_parameter(self, cell, name, value):
+        _check_train(lib.fh_train_set_solver_parameter(self._h, cell.encode(), name.encode(), float(value)))
+
+    def learn(self, targets, iterations=1):
+        """Runs learning iterations (propagate, loss against `targets`, backPropagate, update); returns the last loss."""
+        t = np.ascontiguousarray(targets, dtype=np.float32)
+        loss = C.c_double(0.0)
+        _check_train(lib.fh_train_learn(self._h, t.ctypes.data, t.size, iterations, C.byref(loss)))
+        return loss.value
+
+    def propagate(self, inference=True):
+        _check_train(lib.fh_train_propagate(self._h, int(inference)))
+
+    def _get(self, cell, what, shape):
+        out = np.empty(shape, dtype=np.float32)
+        _check_train(lib.fh_train_get(self._h, cell.encode(), what, out.ctypes.data, out.size))
+        return out
+
+    def outputs(self, cell):
+        return self._get(cell, 0, self._shapes[cell])
+
+    def diff_inputs(self, cell):
+        return self._get(cell, 1, self._shapes[cell])
+
+    def weights(self, cell):
+        return self._get(cell, 2, self._shapes[cell + "/weights"])
+
+    def diff_weights(self, cell):
+        return self._get(cell, 3, self._shapes[cell + "/weights"])
+
+    def quantized_weights(self, cell):
+        return self._get(cell, 4, self._shapes[cell + "/weights"])
+
+    def input_gradient(self):
+        out = np.empty(self.input_shape, dtype=np.float32)
+        _check_train(lib.fh_train_input_gradient(self._h, out.ctypes.data, out.size))
+        return out
+
+    def activation_quantizer(self, cell):
+        """(learned parameter, its last gradient): SAT alpha or LSQ step size."""
+        v, g = C.c_float(0), C.c_float(0)
+        _check_train(lib.fh_train_get_activation_quantizer(self._h, cell.encode(), C.byref(v), C.byref(g)))
+        return v.value, g.value

@@ -146,13 +146,16 @@ class ActivationCell:
 
 
 class ConvCell:
-    """src/Cell/ConvCell_Frame.cpp:418-597 with one input and NoBias: propagate = quantize the weights, convolve, then
+    """src/Cell/ConvCell_Frame.cpp:418-597 with one input: propagate = quantize the weights, convolve, then
     the activation in place; backPropagate = activation, backwardFilter on the quantized weights' gradient, backwardData
     with the quantized weights, then the weight quantizer's backward; update = solver on the full-precision weights with
     the quantizer's gradient, then the activation's quantizer."""
 
-    def __init__(self, weights, stride=(1, 1), pad=(0, 0, 0, 0), maps=None, activation=None, quantizer=None, solver=None):
+    def __init__(self, weights, stride=(1, 1), pad=(0, 0, 0, 0), maps=None, activation=None, quantizer=None, solver=None,
+                 bias=None, bias_solver=None):
         self.w = np.array(weights, dtype=F)
+        self.bias = None if bias is None else np.array(bias, dtype=F)      # None: NoBias
+        self.bias_solver = bias_solver or SGDSolver()
         self.stride, self.pad, self.maps = stride, pad, maps
         self.activation, self.quantizer = activation, quantizer
         self.solver = solver or SGDSolver()
@@ -164,6 +167,8 @@ class ConvCell:
         # mOutputsSize: dimB * dimY * dimX of the weight tensor {kW,kH,Cw,O} (SATQuantizerCell_Frame.cpp:80)
         self.wq = self.quantizer.propagate(self.w, O * kH * kW) if self.quantizer else self.w
         y = o.conv_forward(x, self.wq, stride=self.stride, pad=self.pad, maps=self.maps)
+        if self.bias is not None:       # the SAT / LSQ cell quantizers pass the biases through
+            y = o.conv_forward_bias(y, self.bias)
         self.outputs = self.activation.propagate(y, inference) if self.activation else y
         return self.outputs
 
@@ -172,12 +177,16 @@ class ConvCell:
         if self.activation:
             d = self.activation.back_propagate(d)
         self.diff_wq = o.conv_backward_filter(self.x, d, self.w.shape, stride=self.stride, pad=self.pad, maps=self.maps)
+        if self.bias is not None:
+            self.diff_bias = o.conv_backward_bias(d)
         dx = o.conv_backward_data(self.wq, d, self.x.shape, stride=self.stride, pad=self.pad, maps=self.maps)
         self.diff_w = self.quantizer.back_propagate(self.diff_wq, self.w) if self.quantizer else self.diff_wq
         return dx
 
     def update(self, batch_size):
         self.solver.update(self.w, self.diff_w, batch_size)
+        if self.bias is not None:
+            self.bias_solver.update(self.bias, self.diff_bias, batch_size)
         if self.activation:
             self.activation.update(batch_size)
 

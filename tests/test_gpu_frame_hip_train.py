@@ -1,0 +1,146 @@
+"""The float Frame_HIP cells for quantization-aware training (C++ host classes created through the Registrar under
+"Frame_HIP_QAT"), against the CPU oracle: one learning iteration compared tensor by tensor, a few more on the learned
+parameters, and the reference's own known-answer test, the three SAT alphas after 10 000 iterations
+(tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp:68-516, delta 0.01)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sat_three_conv", "case.json")
+
+
+def _gpu_net(case):
+    from n2d2_amd import frame_hip as fh
+    x = (np.array(case["input_times_255"], dtype=np.float32) / np.float32(255.0)).reshape(2, 1, 5, 5)
+    net = fh.TrainNet(x)
+    r1, r2, a = case["range_activation1"], case["range_conv"], case["alpha_init"]
+    net.add_activation_cell("activation1", "Linear", "SAT", r1, a)
+    net.add_conv("conv1", np.array(case["conv1_weights"]).reshape(1, 1, 3, 3), act="Linear", act_quant="SAT", act_range=r2, act_param=a,
+                 weight_quant="SAT", weight_range=r1)
+    net.add_conv("conv2", np.array(case["conv2_weights"]).reshape(4, 1, 1, 1), act="Linear", act_quant="SAT", act_range=r2, act_param=a,
+                 weight_quant="SAT", weight_range=r2)
+    net.add_conv("conv3", np.array(case["conv3_weights"]).reshape(4, 1, 3, 3), depthwise=True, weight_quant="SAT", weight_range=r2)
+    net.add_softmax("softmax1", with_loss=True)
+    t = np.zeros((2, 4, 1, 1), dtype=np.float32)
+    for b, k in enumerate(case["target_class"]):
+        t[b, k] = 1
+    return net, t
+
+
+def _oracle_net(case):
+    from test_oracle_qat_train import sat_three_conv_net
+    return sat_three_conv_net(case)
+
+
+def _close(got, want, tol=1e-5):
+    scale = np.maximum(np.abs(want), 1e-3)
+    return float((np.abs(got.astype(np.float64) - want.astype(np.float64)) / scale).max()) <= tol
+
+
+def test_registrar_holds_the_float_cells():
+    from n2d2_amd import frame_hip as fh
+    for t in ("Conv", "Activation", "Softmax"):
+        assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_HIP_QAT") == 1
+        assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_XYZ") == 0
+    assert fh.lib.fh_train_registrar_exists(b"Conv", b"Frame_HIP") == 1          # the integer inference cell
+    with pytest.raises(fh.FrameHipError, match="is not valid"):
+        net = fh.TrainNet(np.zeros((1, 1, 4, 4)), model="Frame_XYZ")
+        net.add_softmax("s")
+
+
+def test_one_learning_iteration_matches_the_oracle_tensor_by_tensor():
+    from oracle import qat_train as q
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    case = json.load(open(GOLD))
+    net, t = _gpu_net(case)
+    x, cells, qa, t2 = _oracle_net(case)
+    assert np.array_equal(t, t2)
+    print("one iteration", flush=True)
+    loss = net.learn(t, 1)
+    sm = q.SoftmaxCell()
+    want_loss = q.train_sequential(x, cells, sm, t, 1)
+    assert abs(loss - want_loss) <= 1e-6 * want_loss
+    names = ["activation1", "conv1", "conv2", "conv3"]
+    for name, c in zip(names, cells):
+        assert _close(net.outputs(name), c.outputs), name
+    assert _close(net.outputs("softmax1"), sm.outputs)
+    assert _close(net.diff_inputs("softmax1"), sm.diff_inputs)
+    for name, c in zip(names[1:], cells[1:]):
+        assert _close(net.quantized_weights(name), c.wq), name
+        assert _close(net.diff_weights(name), c.diff_wq, 1e-4), name       # gradient of the quantized weights
+        assert _close(net.weights(name), c.w), name                        # after the update
+    for name, a in zip(names[:3], qa):
+        got, grad = net.activation_quantizer(name)
+        assert abs(got - float(a.alphas[0])) <= 1e-6 * abs(got), name
+        assert abs(grad - float(a.diff_alphas)) <= 1e-5 * max(abs(float(a.diff_alphas)), 1e-3), name
+    # 50 more iterations: the learned parameters stay together
+    net.learn(t, 50)
+    q.train_sequential(x, cells, sm, t, 50)
+    for name, a in zip(names[:3], qa):
+        assert abs(net.activation_quantizer(name)[0] - float(a.alphas[0])) <= 1e-4, name
+    for name, c in zip(names[1:], cells[1:]):
+        assert _close(net.weights(name), c.w, 1e-3), name
+
+
+def test_known_answer_sat_alphas_after_training():
+    case = json.load(open(GOLD))
+    net, t = _gpu_net(case)
+    print("10000 iterations", flush=True)
+    loss = net.learn(t, case["iterations"])
+    got = {n: net.activation_quantizer(n)[0] for n in ("activation1", "conv1", "conv2")}
+    print("alphas", got, "loss", loss, flush=True)
+    for name, want in case["expected_alpha"].items():
+        assert abs(got[name] - want) < case["delta"], (name, got[name], want)
+
+
+def test_rectifier_bias_and_momentum_against_the_oracle():
+    """A two-convolution net with a bias, a Rectifier activation with a SAT quantizer, stride and padding, a Symmetric
+    weight quantizer and a momentum solver: five iterations against the oracle."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    rng = np.random.default_rng(21)
+    x = rng.uniform(0, 1, size=(4, 3, 9, 9)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, size=(6, 3, 3, 3)).astype(np.float32)
+    w2 = rng.normal(0, 0.3, size=(5, 6, 3, 3)).astype(np.float32)
+    net = fh.TrainNet(x, propagate_gradient=False)
+    net.add_conv("c1", w1, stride=(2, 2), pad=(1, 1), act="Rectifier", act_quant="SAT", act_range=15, act_param=2.0, weight_quant="SAT", weight_range=15)
+    b2 = rng.normal(0, 0.1, size=5).astype(np.float32)
+    net.add_conv("c2", w2, bias=b2, stride=(1, 1), pad=(0, 0), act=None, weight_quant="SAT", weight_range=15, quant_mode="Symmetric")
+    net.set_solver_parameter("c1", "Momentum", 0.9)
+    assert net._last == (4, 5, 3, 3)
+    t = rng.uniform(0, 1, size=net._last).astype(np.float32)
+
+    class Rect(q.LinearActivation):
+        def propagate(self, v, inference):
+            self.out = q.LinearActivation.propagate(self, np.maximum(v, 0).astype(np.float32), inference)
+            return self.out
+
+        def back_propagate(self, d):
+            d = q.LinearActivation.back_propagate(self, d)
+            return (d * (self.out > 0)).astype(np.float32)
+    qa = q.SATQuantizerActivation(15, 2.0)
+    c1 = q.ConvCell(w1, stride=(2, 2), pad=(1, 1, 1, 1), activation=Rect(qa), quantizer=q.SATQuantizerCell(15), solver=q.SGDSolver(momentum=0.9))
+    c2 = q.ConvCell(w2, bias=b2, quantizer=q.SATQuantizerCell(15, mode="symrange"))
+
+    class Last:                                  # loss straight on the last convolution's outputs
+        def propagate(self, v):
+            self.outputs = v
+
+        def apply_loss(self, targets):
+            err = targets.astype(np.float64) - self.outputs.astype(np.float64)
+            self.diff_inputs = err.astype(np.float32)
+            return float((err * err).sum() / self.outputs.shape[0])
+
+        def back_propagate(self):
+            return self.diff_inputs
+    print("rectifier / momentum net", flush=True)
+    for it in range(5):
+        loss = net.learn(t, 1)
+        want = q.train_sequential(x, [c1, c2], Last(), t, 1)
+        assert abs(loss - want) <= 1e-4 * want, it
+    assert _close(net.weights("c1"), c1.w, 1e-3) and _close(net.weights("c2"), c2.w, 1e-3)
+    assert abs(net.activation_quantizer("c1")[0] - float(qa.alphas[0])) <= 1e-4
