@@ -31,6 +31,7 @@ struct TrainNet {
     std::vector<std::shared_ptr<Cell_FrameTrain_HIP> > cells;
     std::map<std::string, std::shared_ptr<SATQuantizerActivation_Frame_HIP<float> > > satAct;
     std::map<std::string, std::shared_ptr<LSQQuantizerActivation_Frame_HIP<float> > > lsqAct;
+    std::map<std::string, std::shared_ptr<LSQQuantizerCell_Frame_HIP<float> > > lsqCell;
     Cell_FrameTrain_HIP* last() { return cells.empty() ? nullptr : cells.back().get(); }
 };
 
@@ -161,6 +162,7 @@ int fh_train_add_conv(void* net, const char* name, int nbOutputs, int kW, int kH
             q->setRange((size_t)weightRange);
             q->setSolver(Registrar<SGDSolver>::create<float>("Frame_HIP")());
             cell->setQuantizer(q);
+            n.lsqCell[name] = std::dynamic_pointer_cast<LSQQuantizerCell_Frame_HIP<float> >(q);
         }
         connect(n, cell);
     });
@@ -262,6 +264,18 @@ int fh_train_get_activation_quantizer(void* net, const char* cell, float* value,
         if (s != n.satAct.end()) { *value = s->second->getAlpha(); if (grad) *grad = s->second->getDiffAlpha(); }
         else if (l != n.lsqAct.end()) { *value = l->second->getStepSize(); if (grad) *grad = l->second->getDiffStepSize(); }
         else throw std::runtime_error("No activation quantizer on cell \"" + std::string(cell) + "\"");
+    });
+}
+
+// The learned step size of a cell's LSQ weight quantizer; grad receives its last gradient
+int fh_train_get_weight_quantizer(void* net, const char* cell, float* value, float* grad)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto l = n.lsqCell.find(cell);
+        if (l == n.lsqCell.end()) throw std::runtime_error("No LSQ weight quantizer on cell \"" + std::string(cell) + "\"");
+        *value = l->second->getStepSize();
+        if (grad) *grad = l->second->getDiffStepSize();
     });
 }
 

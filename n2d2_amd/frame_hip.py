@@ -264,6 +264,7 @@ lib.fh_train_propagate.argtypes = [_P, _I]
 lib.fh_train_get.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
 lib.fh_train_input_gradient.argtypes = [_P, _P, _SZ]
 lib.fh_train_get_activation_quantizer.argtypes = [_P, C.c_char_p, _P, _P]
+lib.fh_train_get_weight_quantizer.argtypes = [_P, C.c_char_p, _P, _P]
 
 TRAIN_MODEL = "Frame_HIP_QAT"
 _ACT = {None: -1, "Linear": 0, "Rectifier": 1}
@@ -361,4 +362,10 @@ class TrainNet:
         """(learned parameter, its last gradient): SAT alpha or LSQ step size."""
         v, g = C.c_float(0), C.c_float(0)
         _check_train(lib.fh_train_get_activation_quantizer(self._h, cell.encode(), C.byref(v), C.byref(g)))
+        return v.value, g.value
+
+    def weight_quantizer(self, cell):
+        """(LSQ step size of the cell's weight quantizer, its last gradient)."""
+        v, g = C.c_float(0), C.c_float(0)
+        _check_train(lib.fh_train_get_weight_quantizer(self._h, cell.encode(), C.byref(v), C.byref(g)))
         return v.value, g.value

@@ -124,6 +124,35 @@ class SATQuantizerCell:
                                      self.mode if self.mode in ("fullrange", "asymrange") else "default")
 
 
+class LSQQuantizerCell:
+    """src/Quantizer/QAT/Cell/LSQ/LSQQuantizerCell_Frame.cpp:106-310: range [-(R+1)/2, (R-1)/2]; at the first propagate
+    the step size becomes 2 * mean|w| / sqrt(hi) (SetOptInitStepSize, :166-184); the step-size gradient is the kernel's
+    sum (+ the previous value inside a solver iteration) times 1/sqrt(N * hi); update() hands it to the solver."""
+
+    def __init__(self, rng, step_size=None, solver=None):
+        self.lo, self.hi = -((rng + 1) >> 1), (rng - 1) >> 1
+        self.step = None if step_size is None else np.full(1, step_size, dtype=F)
+        self.diff_step = F(0.0)
+        self.solver = solver or SGDSolver()
+
+    def propagate(self, w, outputs_size):
+        if self.step is None:
+            self.step = np.full(1, F(2.0) * F(np.abs(w.astype(np.float64)).mean() / np.sqrt(self.hi)), dtype=F)
+        self.grad_scale = F(1.0 / np.sqrt(w.size * self.hi))
+        return o.lsq_forward(w, float(self.step[0]), self.lo, self.hi)
+
+    def back_propagate(self, dwq, w):
+        dw, total = o.lsq_backward(dwq, w, float(self.step[0]), self.lo, self.hi)
+        total = F(total)
+        if not self.solver.is_new_iteration():
+            total = F(total + self.diff_step)
+        self.diff_step = F(total * self.grad_scale)
+        return dw
+
+    def update(self, batch_size):
+        self.solver.update(self.step, np.full(1, self.diff_step, dtype=F), batch_size)
+
+
 class ActivationCell:
     """src/Cell/ActivationCell_Frame.cpp:95-205, one input: copy, then the activation in place."""
 
@@ -185,6 +214,8 @@ class ConvCell:
 
     def update(self, batch_size):
         self.solver.update(self.w, self.diff_w, batch_size)
+        if self.quantizer and hasattr(self.quantizer, "update"):
+            self.quantizer.update(batch_size)
         if self.bias is not None:
             self.bias_solver.update(self.bias, self.diff_bias, batch_size)
         if self.activation:

@@ -144,3 +144,62 @@ def test_rectifier_bias_and_momentum_against_the_oracle():
         assert abs(loss - want) <= 1e-4 * want, it
     assert _close(net.weights("c1"), c1.w, 1e-3) and _close(net.weights("c2"), c2.w, 1e-3)
     assert abs(net.activation_quantizer("c1")[0] - float(qa.alphas[0])) <= 1e-4
+
+
+LSQ_GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lsq_known_answers", "cases.json")
+
+
+def test_known_answer_lsq_step_sizes_three_conv():
+    """tests/Cell/class_ConvCell_QuantizerLSQ_Frame_CUDA.cpp: the step sizes of the three LSQ weight quantizers after
+    10 000 and after 100 000 iterations, delta 0.001; one iteration first, against the oracle."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from test_oracle_qat_train import lsq_three_conv_net
+    case = json.load(open(GOLD))
+    lsq = json.load(open(LSQ_GOLD))["three_conv"]
+    x, cells, qs, t = lsq_three_conv_net(case, lsq)
+    net = fh.TrainNet(x)
+    net.add_activation_cell("activation1", "Linear")
+    net.add_conv("conv1", cells[1].w, act="Linear", weight_quant="LSQ", weight_range=lsq["range_conv1"])
+    net.add_conv("conv2", cells[2].w, act="Linear", weight_quant="LSQ", weight_range=lsq["range_conv2"])
+    net.add_conv("conv3", cells[3].w, depthwise=True, weight_quant="LSQ", weight_range=lsq["range_conv3"])
+    net.add_softmax("softmax1", with_loss=True)
+    names = ("conv1", "conv2", "conv3")
+    print("lsq three conv", flush=True)
+    net.learn(t, 1)
+    q.train_sequential(x, cells, q.SoftmaxCell(), t, 1)
+    for name, s, c in zip(names, qs, cells[1:]):
+        step, grad = net.weight_quantizer(name)
+        assert abs(step - float(s.step[0])) <= 1e-6 * abs(step), name
+        assert abs(grad - float(s.diff_step)) <= 1e-5 * max(abs(float(s.diff_step)), 1e-3), name
+        assert _close(net.quantized_weights(name), c.wq), name
+        assert _close(net.weights(name), c.w), name
+    done = 1
+    for iters, key in ((10000, "expected_step_after_10000"), (100000, "expected_step_after_100000")):
+        net.learn(t, iters - done)
+        done = iters
+        got = {n: net.weight_quantizer(n)[0] for n in names}
+        print(iters, got, flush=True)
+        for name, want in lsq[key].items():
+            assert abs(got[name] - want) < lsq["delta"], (iters, name, got[name], want)
+
+
+def test_known_answer_lsq_step_size_fc():
+    """tests/Cell/class_FcCell_QuantizerLSQ_Frame_CUDA.cpp, run as the 3x3 convolution over the 3x3 input."""
+    from n2d2_amd import frame_hip as fh
+    fc = json.load(open(LSQ_GOLD))["fc"]
+    x = (np.float32(0.125) * np.arange(9, dtype=np.float32)).reshape(1, 1, 3, 3)
+    w = np.zeros((2, 1, 3, 3), dtype=np.float32)
+    for k, v in enumerate(fc["weights_per_output"]):
+        w[k] = v
+    net = fh.TrainNet(x)
+    net.add_activation_cell("activation1", "Linear")
+    net.add_conv("fc1", w, weight_quant="LSQ", weight_range=fc["range"])
+    net.add_softmax("softmax1", with_loss=True)
+    print("lsq fc", flush=True)
+    net.learn(np.array(fc["target"], dtype=np.float32).reshape(1, 2, 1, 1), fc["iterations"])
+    step = net.weight_quantizer("fc1")[0]
+    print("step", step, flush=True)
+    assert abs(step - fc["expected_step"]) < fc["delta"]

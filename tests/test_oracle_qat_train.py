@@ -143,3 +143,52 @@ def test_known_answer_sat_alphas_after_training():
     print("alphas", got, "loss", loss)
     for name, want in case["expected_alpha"].items():
         assert abs(got[name] - want) < case["delta"], (name, got[name], want)
+
+
+LSQ_GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "lsq_known_answers", "cases.json")
+
+
+def lsq_three_conv_net(case, lsq):
+    x = (np.array(case["input_times_255"], dtype=np.float32) / np.float32(255.0)).reshape(2, 1, 5, 5)
+    qs = [q.LSQQuantizerCell(lsq["range_conv1"]), q.LSQQuantizerCell(lsq["range_conv2"]), q.LSQQuantizerCell(lsq["range_conv3"])]
+    cells = [q.ActivationCell(q.LinearActivation(None)),
+             q.ConvCell(np.array(case["conv1_weights"]).reshape(1, 1, 3, 3), activation=q.LinearActivation(None), quantizer=qs[0]),
+             q.ConvCell(np.array(case["conv2_weights"]).reshape(4, 1, 1, 1), activation=q.LinearActivation(None), quantizer=qs[1]),
+             q.ConvCell(np.array(case["conv3_weights"]).reshape(4, 1, 3, 3), maps=np.eye(4, dtype=np.uint8), quantizer=qs[2])]
+    t = np.zeros((2, 4, 1, 1), dtype=np.float32)
+    for b, k in enumerate(case["target_class"]):
+        t[b, k] = 1
+    return x, cells, qs, t
+
+
+def test_known_answer_lsq_step_sizes_three_conv():
+    """tests/Cell/class_ConvCell_QuantizerLSQ_Frame_CUDA.cpp: PyTorch-derived step sizes of the three weight quantizers
+    after 10 000 (constants kept in a comment there) and 100 000 iterations (asserted there), delta 0.001."""
+    case = json.load(open(GOLD))
+    lsq = json.load(open(LSQ_GOLD))["three_conv"]
+    x, cells, qs, t = lsq_three_conv_net(case, lsq)
+    sm = q.SoftmaxCell()
+    done = 0
+    for iters, key in ((10000, "expected_step_after_10000"), (100000, "expected_step_after_100000")):
+        q.train_sequential(x, cells, sm, t, iters - done)
+        done = iters
+        got = dict(zip(("conv1", "conv2", "conv3"), (float(s.step[0]) for s in qs)))
+        print(iters, got)
+        for name, want in lsq[key].items():
+            assert abs(got[name] - want) < lsq["delta"], (iters, name, got[name], want)
+
+
+def test_known_answer_lsq_step_size_fc():
+    """tests/Cell/class_FcCell_QuantizerLSQ_Frame_CUDA.cpp: a 9 -> 2 FcCell with an LSQ weight quantizer, run here as the
+    3x3 convolution over the 3x3 input that computes the same products in the same order."""
+    fc = json.load(open(LSQ_GOLD))["fc"]
+    x = (np.float32(0.125) * np.arange(9, dtype=np.float32)).reshape(1, 1, 3, 3)
+    w = np.zeros((2, 1, 3, 3), dtype=np.float32)
+    for k, v in enumerate(fc["weights_per_output"]):
+        w[k] = v
+    quant = q.LSQQuantizerCell(fc["range"])
+    cells = [q.ActivationCell(q.LinearActivation(None)), q.ConvCell(w, quantizer=quant)]
+    t = np.array(fc["target"], dtype=np.float32).reshape(1, 2, 1, 1)
+    q.train_sequential(x, cells, q.SoftmaxCell(), t, fc["iterations"])
+    print("step", float(quant.step[0]))
+    assert abs(float(quant.step[0]) - fc["expected_step"]) < fc["delta"]
