@@ -268,10 +268,11 @@ int n2d2hip_lsq_backward(const float* diff_q, const float* fp_x, float* diff_fp,
 /* The float32 cells a quantization-aware training graph runs between the fake-quant kernels above.  Tensors are
  * N2D2's own: activations NCHW ({X,Y,Z,B}, X fastest), weights OCHW ({kW,kH,C/groups,O}); `desc->weight_bits` is not
  * read; groups is 1 or C == O (depthwise).  "diff" tensors carry the descent direction, as in the reference
- * (target - output at the loss), so the solver adds rate * diff.
+ * (target - output at the loss), so the solver adds rate * diff.  Ungrouped convolutions without dilation of at
+ * least 2e7 flops run as an implicit GEMM on the fp32 matrix cores, the others on direct kernels that add their terms
+ * in the reference's order.
  *
- * y = conv(x, w) (+ bias[o] if bias != NULL) + beta * y; the window is clipped at the borders and a full 3x3 window
- * is summed row by row (ref: src/Cell/ConvCell_Frame_Kernels.cpp:26-174, called from
+ * y = conv(x, w) (+ bias[o] if bias != NULL) + beta * y; the window is clipped at the borders (ref: src/Cell/ConvCell_Frame_Kernels.cpp:26-174, called from
  * ConvCell_Frame<T>::propagate, src/Cell/ConvCell_Frame.cpp:418-473). */
 int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* w,
                                const float* bias, float beta, float* y, n2d2hip_stream_t stream);
@@ -279,9 +280,13 @@ int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int 
  * must be 1: the reference's backward kernels do not read it. */
 int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* w,
                                      const float* diff_y, float beta, float* diff_x, n2d2hip_stream_t stream);
-/* diff_w = backwardFilter(x, diff_y) + beta * diff_w (ref: src/Cell/ConvCell_Frame_Kernels.cpp:335-427). */
+/* diff_w = backwardFilter(x, diff_y) + beta * diff_w (ref: src/Cell/ConvCell_Frame_Kernels.cpp:335-427).  The sum over
+ * batch and pixels is split into ranges whose partial results go through `workspace` (device memory, at least
+ * n2d2hip_conv2d_f32_workspace_bytes, which may be 0) and are added in a fixed order. */
+size_t n2d2hip_conv2d_f32_workspace_bytes(const n2d2hip_conv_desc* desc, int B, int H, int W);
 int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x,
-                                       const float* diff_y, float beta, float* diff_w, n2d2hip_stream_t stream);
+                                       const float* diff_y, float beta, float* diff_w, void* workspace,
+                                       size_t workspace_bytes, n2d2hip_stream_t stream);
 /* diff_bias[o] = sum over batch and pixels of diff_y + beta * diff_bias (ref: ...ConvCell_Frame_Kernels.cpp:429-452). */
 int n2d2hip_conv2d_f32_backward_bias(int B, int O, int oH, int oW, const float* diff_y, float beta, float* diff_bias,
                                      n2d2hip_stream_t stream);

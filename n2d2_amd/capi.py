@@ -31,7 +31,7 @@ SYMBOLS = [
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling",
     "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_backward",
     "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
-    "n2d2hip_conv2d_f32_forward", "n2d2hip_conv2d_f32_backward_data", "n2d2hip_conv2d_f32_backward_filter",
+    "n2d2hip_conv2d_f32_forward", "n2d2hip_conv2d_f32_backward_data", "n2d2hip_conv2d_f32_backward_filter", "n2d2hip_conv2d_f32_workspace_bytes",
     "n2d2hip_conv2d_f32_backward_bias", "n2d2hip_softmax_f32_forward", "n2d2hip_loss_workspace_bytes", "n2d2hip_loss_f32",
     "n2d2hip_sgd_update_f32", "n2d2hip_rectifier_f32_forward", "n2d2hip_rectifier_f32_backward",
 ]
@@ -105,7 +105,9 @@ def load():
     lib.n2d2hip_lsq_backward.argtypes = [P, P, P, SZ, P, I, I, F, F, P, P, SZ, P]
     lib.n2d2hip_conv2d_f32_forward.argtypes = [P, I, I, I, P, P, P, F, P, P]
     lib.n2d2hip_conv2d_f32_backward_data.argtypes = [P, I, I, I, P, P, F, P, P]
-    lib.n2d2hip_conv2d_f32_backward_filter.argtypes = [P, I, I, I, P, P, F, P, P]
+    lib.n2d2hip_conv2d_f32_backward_filter.argtypes = [P, I, I, I, P, P, F, P, P, SZ, P]
+    lib.n2d2hip_conv2d_f32_workspace_bytes.restype = C.c_size_t
+    lib.n2d2hip_conv2d_f32_workspace_bytes.argtypes = [P, I, I, I]
     lib.n2d2hip_conv2d_f32_backward_bias.argtypes = [I, I, I, I, P, F, P, P]
     lib.n2d2hip_softmax_f32_forward.argtypes = [P, P, I, I, I, I, P]
     lib.n2d2hip_loss_workspace_bytes.restype = C.c_size_t

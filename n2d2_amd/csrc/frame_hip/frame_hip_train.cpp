@@ -256,7 +256,11 @@ void ConvCell_FrameTrain_HIP<T>::backPropagate()
     const int B = (int)mIn->dimB();
     {
         const float beta = mWeightsSolver->isNewIteration() ? 0.0f : 1.0f;
-        checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(), mStream));
+        const size_t need = n2d2hip_conv2d_f32_workspace_bytes(&d, B, (int)mInH, (int)mInW);
+        if (need > mWorkspace.size() * sizeof(float))
+            mWorkspace.resize({(need + sizeof(float) - 1) / sizeof(float)});
+        checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(),
+                                                       mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
         mDevDiffW.setValid();
     }
     if (!mNoBias) {

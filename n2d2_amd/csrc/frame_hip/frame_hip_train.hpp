@@ -127,6 +127,7 @@ private:
     std::shared_ptr<QuantizerCell> mQuantizer;
     std::shared_ptr<SGDSolver> mWeightsSolver, mBiasSolver;
     DeviceFloats mDevW, mDevDiffW, mDevBias, mDevDiffBias;
+    DeviceFloats mWorkspace;        // partial sums of backward-filter
     static Registrar<ConvCell> mRegistrar;
 };
 

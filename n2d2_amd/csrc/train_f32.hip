@@ -5,7 +5,10 @@
 // These are direct kernels: one thread per produced element, walking channels and taps in the reference's order
 // (so forward and backward-data give the reference's float sums term for term), and one block per weight for
 // backward-filter, whose long sum over batch and pixels is wavefront-reduced in double.
+#include <cstdlib>
+
 #include "common.h"
+#include "conv_f32_gemm.cuh"
 
 namespace n2d2hip {
 
@@ -248,6 +251,45 @@ static int make_conv(const n2d2hip_conv_desc* d, int B, int H, int W, bool backw
     return N2D2HIP_OK;
 }
 
+// The matrix-core kernel serves ungrouped convolutions without dilation that are worth a 128 x 128 tile; the direct
+// kernels keep the rest (depthwise, dilated, tiny).  N2D2HIP_F32_PATH=direct|gemm overrides the size rule.
+static bool use_gemm(const ConvF32& q)
+{
+    if (q.depthwise || q.dx != 1 || q.dy != 1)
+        return false;
+    const char* e = getenv("N2D2HIP_F32_PATH");
+    if (e && !strcmp(e, "direct")) return false;
+    if (e && !strcmp(e, "gemm")) return true;
+    return 2.0 * q.B * q.O * q.oH * q.oW * q.C * q.kH * q.kW >= 2.0e7;
+}
+
+static GemmF32 make_gemm(const ConvF32& q, int mode)
+{
+    GemmF32 g = {q.B, q.C, q.H, q.W, q.O, q.oH, q.oW, q.kW, q.kH, q.sx, q.sy, q.pl, q.pt, 0, 0, 0, 0};
+    if (mode == GEMM_FWD) { g.P = q.B * q.oH * q.oW; g.Q = q.O; g.K = q.C * q.kH * q.kW; }
+    else if (mode == GEMM_BWD_DATA) { g.P = q.B * q.H * q.W; g.Q = q.C; g.K = q.O * q.kH * q.kW; }
+    else { g.P = q.C * q.kH * q.kW; g.Q = q.O; g.K = q.B * q.oH * q.oW; }
+    g.kchunk = round_up(g.K, GK);
+    return g;
+}
+
+// K ranges of backward-filter: enough blocks to fill the chip, each range at least 8 steps long
+static int filter_splits(GemmF32* g)
+{
+    const long tiles = (long)((g->P + GT - 1) / GT) * ((g->Q + GT - 1) / GT);
+    long splits = std::max(1L, 1024 / tiles);
+    splits = std::min<long>(splits, std::max(1, g->K / (8 * GK)));
+    g->kchunk = round_up((int)((g->K + splits - 1) / splits), GK);
+    return (g->K + g->kchunk - 1) / g->kchunk;
+}
+
+static bool fits_int(const ConvF32& q)
+{
+    // the GEMM extents are ints
+    return (size_t)q.B * std::max((size_t)q.H * q.W, (size_t)q.oH * q.oW) < ((size_t)1 << 31) && (size_t)q.C * q.kH * q.kW < ((size_t)1 << 31)
+           && (size_t)q.O * q.kH * q.kW < ((size_t)1 << 31);
+}
+
 } // namespace n2d2hip
 
 using namespace n2d2hip;
@@ -261,6 +303,13 @@ int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int 
     const int st = make_conv(desc, B, H, W, false, &q, "n2d2hip_conv2d_f32_forward");
     if (st != N2D2HIP_OK) return st;
     N2D2HIP_REQUIRE(x && w && y, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_forward: null pointer");
+    if (use_gemm(q) && fits_int(q)) {
+        const GemmF32 g = make_gemm(q, GEMM_FWD);
+        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_FWD>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0, (hipStream_t)stream,
+                           g, x, w, bias, beta, y);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
     hipLaunchKernelGGL(conv_f32_forward_kernel, dim3(grid_for((size_t)q.B * q.O * q.oH * q.oW)), dim3(TBLOCK), 0, (hipStream_t)stream,
                        q, x, w, bias, beta, y);
     N2D2HIP_HIP_CHECK(hipGetLastError());
@@ -274,14 +323,30 @@ int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H
     const int st = make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_backward_data");
     if (st != N2D2HIP_OK) return st;
     N2D2HIP_REQUIRE(w && diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_data: null pointer");
+    if (use_gemm(q) && fits_int(q)) {
+        const GemmF32 g = make_gemm(q, GEMM_BWD_DATA);
+        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_BWD_DATA>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0, (hipStream_t)stream,
+                           g, diff_y, w, (const float*)nullptr, beta, diff_x);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
     hipLaunchKernelGGL(conv_f32_backward_data_kernel, dim3(grid_for((size_t)q.B * q.C * q.H * q.W)), dim3(TBLOCK), 0, (hipStream_t)stream,
                        q, w, diff_y, beta, diff_x);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
 
+size_t n2d2hip_conv2d_f32_workspace_bytes(const n2d2hip_conv_desc* desc, int B, int H, int W)
+{
+    ConvF32 q;
+    if (make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_workspace_bytes") != N2D2HIP_OK || !use_gemm(q) || !fits_int(q))
+        return 0;
+    GemmF32 g = make_gemm(q, GEMM_BWD_FILTER);
+    return (size_t)filter_splits(&g) * g.Q * g.P * sizeof(float);
+}
+
 int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* diff_y, float beta,
-                                       float* diff_w, n2d2hip_stream_t stream)
+                                       float* diff_w, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
 {
     ConvF32 q;
     const int st = make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_backward_filter");
@@ -289,6 +354,20 @@ int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int
     N2D2HIP_REQUIRE(x && diff_y && diff_w, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_filter: null pointer");
     const size_t nw = (size_t)q.O * q.Cw * q.kH * q.kW;
     N2D2HIP_REQUIRE(nw < ((size_t)1 << 31), N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_filter: too many weights");
+    if (use_gemm(q) && fits_int(q)) {
+        GemmF32 g = make_gemm(q, GEMM_BWD_FILTER);
+        const int splits = filter_splits(&g);
+        const size_t need = (size_t)splits * nw * sizeof(float);
+        N2D2HIP_REQUIRE(workspace && workspace_bytes >= need, N2D2HIP_ERR_WORKSPACE,
+                        "n2d2hip_conv2d_f32_backward_filter: workspace of %zu bytes, %zu needed (n2d2hip_conv2d_f32_workspace_bytes)",
+                        workspace_bytes, need);
+        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_BWD_FILTER>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
+                           (hipStream_t)stream, g, x, diff_y, (const float*)nullptr, 0.0f, (float*)workspace);
+        hipLaunchKernelGGL(conv_f32_reduce_partials_kernel, dim3(grid_for(nw)), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, splits, nw,
+                           beta, diff_w);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
     hipLaunchKernelGGL(conv_f32_backward_filter_kernel, dim3((unsigned)nw), dim3(TBLOCK), 0, (hipStream_t)stream, q, x, diff_y, beta, diff_w);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
