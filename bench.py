@@ -41,6 +41,63 @@ def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
             "sample": "%d images of the same ResNet-50 forward (batch %d, 224x224), oracle/frame_oracle.c with OpenMP" % (n, n)}, exact
 
 
+PEAK_FP32_TFLOPS = 157.3
+
+
+def qat_conv_step(torch, steps=10):
+    """The float side of the path, reported beside the headline: one quantization-aware training iteration of a
+    ResNet-18 stage convolution (64 -> 64 channels, 3x3, 56x56, batch 64) through the C ABI: SAT weight quantization,
+    convolution, SAT activation quantization (range 15), then their backward passes, backward-filter, backward-data and
+    the SGD update.  Timed with events on the stream the kernels are launched on; flops are those of the three
+    convolution passes."""
+    import ctypes as C
+    from n2d2_amd import capi, runtime
+    lib, sp, chk = capi.lib, runtime.stream_ptr, capi.check
+    B, Cn, H, O, k = 64, 64, 56, 64, 3
+    d = capi.ConvDesc(Cn, O, k, k, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    f32 = dict(dtype=torch.float32, device="cuda")
+    x = torch.rand(B, Cn, H, H, generator=gen, **f32) * 6
+    w = torch.randn(O, Cn, k, k, generator=gen, **f32) * 0.05
+    wq, dwq, dw = torch.empty_like(w), torch.empty_like(w), torch.empty_like(w)
+    y = torch.empty(B, O, H, H, **f32)
+    fp, dy, dx = torch.empty_like(y), torch.randn(B, O, H, H, generator=gen, **f32), torch.empty_like(x)
+    stats, alpha, dalpha = torch.zeros(2, **f32), torch.full((1,), 6.0, **f32), torch.zeros(1, **f32)
+    n, nw = y.numel(), w.numel()
+    wsq = torch.empty(int(lib.n2d2hip_quantizer_workspace_bytes(max(n, nw))), dtype=torch.uint8, device="cuda")
+    need = int(lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, H))
+    wsf = torch.empty(max(need, 4), dtype=torch.uint8, device="cuda")
+    g = torch.empty_like(y)
+
+    def step():
+        s = sp()
+        chk(lib.n2d2hip_sat_weight_forward(w.data_ptr(), wq.data_ptr(), nw, 15.0, capi.SAT_DEFAULT, 0, 1, stats.data_ptr(), wsq.data_ptr(), wsq.numel(), s))
+        chk(lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, H, x.data_ptr(), wq.data_ptr(), None, 0.0, y.data_ptr(), s))
+        chk(lib.n2d2hip_sat_act_forward(y.data_ptr(), fp.data_ptr(), n, 15.0, alpha.data_ptr(), s))
+        chk(lib.n2d2hip_sat_act_backward(dy.data_ptr(), fp.data_ptr(), g.data_ptr(), n, 15.0, alpha.data_ptr(), 0.0, dalpha.data_ptr(),
+                                         wsq.data_ptr(), wsq.numel(), s))
+        chk(lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, H, x.data_ptr(), g.data_ptr(), 0.0, dwq.data_ptr(), wsf.data_ptr(), need, s))
+        chk(lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, H, wq.data_ptr(), g.data_ptr(), 0.0, dx.data_ptr(), s))
+        chk(lib.n2d2hip_sat_weight_backward(dwq.data_ptr(), w.data_ptr(), dw.data_ptr(), nw, 15.0, capi.SAT_DEFAULT, 0, stats.data_ptr(), s))
+        chk(lib.n2d2hip_sgd_update_f32(w.data_ptr(), dw.data_ptr(), nw, 0.01 / B, 0.0, 0.0, None, 0, 0.0, 0.0, s))
+        chk(lib.n2d2hip_sgd_update_f32(alpha.data_ptr(), dalpha.data_ptr(), 1, 0.01 / B, 0.0, 0.0, None, 0, 0.0, 0.0, s))
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = 3 * 2.0 * B * O * H * H * Cn * k * k
+    ach = flops / (ms * 1e-3) / 1e12
+    return {"workload": "SAT QAT iteration of one 64->64 3x3 convolution on 56x56, batch 64, float32", "ms_per_iteration": round(ms, 4),
+            "bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_FP32_TFLOPS, 4),
+            "finite": bool(torch.isfinite(w).all().item() and torch.isfinite(alpha).all().item())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -212,6 +269,7 @@ def main():
     }
     if overlapped is not None:
         result["two_batches_in_flight"] = overlapped
+    result["qat_conv_iteration"] = qat_conv_step(torch)
     if not args.no_cpu_baseline:
         base, exact = cpu_baseline(spec, logits, images)
         result["cpu_baseline"] = base
