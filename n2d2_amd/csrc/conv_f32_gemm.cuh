@@ -11,7 +11,8 @@
 //
 // A block of 256 threads (4 waves as 2 x 2) owns a 128 (q) x 128 (p) tile; each wave 64 x 64 as 2 x 2 MFMA tiles.
 // K advances in steps of 16 through two LDS tiles [k][p] and [k][q] (row stride 129 floats); the next step's
-// elements are fetched into registers while the matrix cores work on the current one.  Backward-filter, whose K is
+// elements are fetched into registers while the matrix cores work on the current one and are written to the other pair
+// of tiles, so one barrier per step suffices.  Backward-filter, whose K is
 // the whole batch of pixels and whose output is small, splits K over blockIdx.z into partial results that a second
 // kernel adds up in a fixed order.
 #pragma once
@@ -39,8 +40,8 @@ template <int MODE>
 __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const float* __restrict__ srcP, const float* __restrict__ srcQ,
                                                             const float* __restrict__ bias, float beta, float* __restrict__ out)
 {
-    __shared__ float Ps[GK * GLD];
-    __shared__ float Qs[GK * GLD];
+    __shared__ float Pbuf[2][GK * GLD];
+    __shared__ float Qbuf[2][GK * GLD];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wq = wave >> 1, wp = wave & 1;
     const int ptile = blockIdx.x * GT, qtile = blockIdx.y * GT;
@@ -54,17 +55,20 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
     // FWD Q operand (weights, contiguous along k): q = t / 2, k = (t % 2) * 8 + i
     const int lq_w = t >> 1, lk_w = (t & 1) * 8;
 
+    // All tensor offsets fit 32 bits (checked by the host).
     int pb = 0, py = 0, px = 0;             // decoded p (FWD: b,oy,ox; BWD_DATA: b,iy,ix)
     bool pvalid = false;
-    int pc[8], pty[8], ptx[8];              // BWD_FILTER: decoded p_i = (c,ty,tx)
+    int pbase = 0;                          // FWD: offset of tap (0,0) of channel 0 for this pixel; BWD_DATA: of (b, o = 0)
+    unsigned long long tapmask = 0;         // FWD: bit ty*kW+tx set if that tap lies inside the input (kH*kW <= 64)
+    int poff[8], pty[8], ptx[8];            // BWD_FILTER: p_i = (c,ty,tx): offset c*H*W + ty*W + tx (-1: no such p), ty, tx
     if (MODE == GEMM_BWD_FILTER) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int p = ptile + lp + 16 * i;
             const int pp = min(p, g.P - 1);
-            pc[i] = (p < g.P) ? pp / kHW : -1;
             pty[i] = (pp % kHW) / g.kW;
             ptx[i] = pp % g.kW;
+            poff[i] = (p < g.P) ? (pp / kHW) * g.H * g.W + pty[i] * g.W + ptx[i] : -1;
         }
     } else {
         const int p = ptile + lp;
@@ -75,6 +79,17 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
         pb = pp / plane;
         py = (pp % plane) / row;
         px = pp % row;
+        if (MODE == GEMM_FWD) {
+            const int iy0 = py * g.sy - g.pt, ix0 = px * g.sx - g.pl;
+            pbase = (pb * g.C * g.H + iy0) * g.W + ix0;
+            if (pvalid)
+                for (int ty = 0; ty < g.kH; ++ty)
+                    for (int tx = 0; tx < g.kW; ++tx)
+                        if (iy0 + ty >= 0 && iy0 + ty < g.H && ix0 + tx >= 0 && ix0 + tx < g.W)
+                            tapmask |= 1ull << (ty * g.kW + tx);
+        } else {
+            pbase = pb * g.O * g.oH * g.oW;
+        }
     }
 
     float rp[8], rq[8];
@@ -84,58 +99,74 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
             const bool kv = k < kend;
             const int kk = kv ? k : 0;
             const int plane = g.oH * g.oW;
-            const int b = kk / plane, oy = (kk % plane) / g.oW, ox = kk % g.oW;
+            const int b = kk / plane, rem = kk % plane, oy = rem / g.oW, ox = rem % g.oW;
             const int iy0 = oy * g.sy - g.pt, ix0 = ox * g.sx - g.pl;
+            const int xbase = (b * g.C * g.H + iy0) * g.W + ix0;
+            const int ybase = b * g.O * plane + rem;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int iy = iy0 + pty[i], ix = ix0 + ptx[i];
-                const bool v = kv && pc[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                rp[i] = v ? srcP[(((size_t)b * g.C + pc[i]) * g.H + iy) * g.W + ix] : 0.0f;
+                const bool v = kv && poff[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                rp[i] = v ? srcP[xbase + poff[i]] : 0.0f;
                 const int q = qtile + lp + 16 * i;
-                rq[i] = (kv && q < g.Q) ? srcQ[((size_t)b * g.O + q) * plane + kk % plane] : 0.0f;
+                rq[i] = (kv && q < g.Q) ? srcQ[ybase + q * plane] : 0.0f;
             }
         } else {
             // P operand: k = k0 + lk + i -> (channel-like, ty, tx), advanced with carries
-            int k = k0 + lk;
-            int ch = k / kHW, ty = (k % kHW) / g.kW, tx = k % g.kW;
+            const int k = k0 + lk;
+            int ch = k / kHW, tap = k % kHW, ty = tap / g.kW, tx = tap % g.kW;
+            if (MODE == GEMM_FWD) {
+                int off = pbase + ch * g.H * g.W + ty * g.W + tx;       // walks (c,ty,tx) with carries
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                float v = 0.0f;
-                if (pvalid && k + i < kend) {
-                    if (MODE == GEMM_FWD) {
-                        const int iy = py * g.sy - g.pt + ty, ix = px * g.sx - g.pl + tx;
-                        if (iy >= 0 && iy < g.H && ix >= 0 && ix < g.W)
-                            v = srcP[(((size_t)pb * g.C + ch) * g.H + iy) * g.W + ix];
-                    } else {
-                        const int ny = py + g.pt - ty, nx = px + g.pl - tx;
-                        if (ny >= 0 && nx >= 0 && ny % g.sy == 0 && nx % g.sx == 0) {
-                            const int oy = ny / g.sy, ox = nx / g.sx;
-                            if (oy < g.oH && ox < g.oW)
-                                v = srcP[(((size_t)pb * g.O + ch) * g.oH + oy) * g.oW + ox];
-                        }
+                for (int i = 0; i < 8; ++i) {
+                    const bool v = ((tapmask >> tap) & 1) && k + i < kend;
+                    rp[i] = v ? srcP[off] : 0.0f;
+                    ++off; ++tap;
+                    if (++tx == g.kW) {
+                        tx = 0; off += g.W - g.kW;
+                        if (tap == kHW) { tap = 0; off += (g.H - g.kH) * g.W; }
                     }
                 }
-                rp[i] = v;
-                if (++tx == g.kW) { tx = 0; if (++ty == g.kH) { ty = 0; ++ch; } }
+            } else {
+                const bool unit = g.sx == 1 && g.sy == 1;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float v = 0.0f;
+                    if (pvalid && k + i < kend) {
+                        const int ny = py + g.pt - ty, nx = px + g.pl - tx;
+                        if (unit) {
+                            if (ny >= 0 && nx >= 0 && ny < g.oH && nx < g.oW)
+                                v = srcP[pbase + (ch * g.oH + ny) * g.oW + nx];
+                        } else if (ny >= 0 && nx >= 0 && ny % g.sy == 0 && nx % g.sx == 0) {
+                            const int oy = ny / g.sy, ox = nx / g.sx;
+                            if (oy < g.oH && ox < g.oW)
+                                v = srcP[pbase + (ch * g.oH + oy) * g.oW + ox];
+                        }
+                    }
+                    rp[i] = v;
+                    if (++tx == g.kW) { tx = 0; if (++ty == g.kH) { ty = 0; ++ch; } }
+                }
             }
             if (MODE == GEMM_FWD) {
                 const int q = qtile + lq_w;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int kq = k0 + lk_w + i;
-                    rq[i] = (q < g.Q && kq < kend) ? srcQ[(size_t)q * g.K + kq] : 0.0f;
+                    rq[i] = (q < g.Q && kq < kend) ? srcQ[q * g.K + kq] : 0.0f;
                 }
             } else {
                 const int q = qtile + lp;           // input channel c; w[(o*C + c)*kHW + tap], k = o*kHW + tap
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int kq = k + i;
-                    rq[i] = (q < g.Q && kq < kend) ? srcQ[((size_t)(kq / kHW) * g.C + q) * kHW + kq % kHW] : 0.0f;
+                    rq[i] = (q < g.Q && kq < kend) ? srcQ[((kq / kHW) * g.C + q) * kHW + kq % kHW] : 0.0f;
                 }
             }
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](int buf) {
+        float* Ps = Pbuf[buf];
+        float* Qs = Qbuf[buf];
         if (MODE == GEMM_BWD_FILTER) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -162,12 +193,15 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 
     if (kbeg < kend) {
         fetch(kbeg);
-        for (int k0 = kbeg; k0 < kend; k0 += GK) {
-            __syncthreads();            // the previous step's reads of the LDS tiles are done
-            stage();
-            __syncthreads();
-            if (k0 + GK < kend)
+        stage(0);
+        __syncthreads();
+        int buf = 0;
+        for (int k0 = kbeg; k0 < kend; k0 += GK, buf ^= 1) {
+            const bool more = k0 + GK < kend;
+            if (more)
                 fetch(k0 + GK);         // in flight while the matrix cores run
+            const float* Ps = Pbuf[buf];
+            const float* Qs = Qbuf[buf];
             const int kr = lane >> 5, col = lane & 31;
 #pragma unroll
             for (int kk = 0; kk < GK / 2; ++kk) {
@@ -179,6 +213,9 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
                 acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
                 acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
             }
+            if (more)
+                stage(buf ^ 1);         // the other tile: its readers passed the barrier of the previous step
+            __syncthreads();
         }
     }
 

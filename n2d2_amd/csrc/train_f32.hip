@@ -285,9 +285,10 @@ static int filter_splits(GemmF32* g)
 
 static bool fits_int(const ConvF32& q)
 {
-    // the GEMM extents are ints
-    return (size_t)q.B * std::max((size_t)q.H * q.W, (size_t)q.oH * q.oW) < ((size_t)1 << 31) && (size_t)q.C * q.kH * q.kW < ((size_t)1 << 31)
-           && (size_t)q.O * q.kH * q.kW < ((size_t)1 << 31);
+    // the GEMM kernel addresses every tensor with 32-bit element offsets and keeps one validity bit per tap
+    const size_t lim = (size_t)1 << 31;
+    return (size_t)q.B * q.C * q.H * q.W < lim && (size_t)q.B * q.O * q.oH * q.oW < lim && (size_t)q.O * q.C * q.kH * q.kW < lim
+           && q.kH * q.kW <= 64;
 }
 
 } // namespace n2d2hip
