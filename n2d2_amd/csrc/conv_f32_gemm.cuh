@@ -30,6 +30,7 @@ struct GemmF32 {
     int sx, sy, pl, pt;
     int P, Q, K;          // GEMM extents
     int kchunk;           // K range of one blockIdx.z (a multiple of 16)
+    unsigned bytesP, bytesQ;   // sizes of the two operand tensors (each at most 2 GiB)
 };
 
 constexpr int GT = 128;       // tile edge (both p and q)
@@ -55,7 +56,17 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
     // FWD Q operand (weights, contiguous along k): q = t / 2, k = (t % 2) * 8 + i
     const int lq_w = t >> 1, lk_w = (t & 1) * 8;
 
-    // All tensor offsets fit 32 bits (checked by the host).
+    // Operands are read through buffer descriptors: an element that does not exist (padding, past the tile or the K
+    // range) is requested at an offset past the end and comes back as zero, so the loads need no branches.  All
+    // offsets fit 32 bits (checked by the host).
+    const __amdgpu_buffer_rsrc_t rsrcP = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(srcP), 0, g.bytesP, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrcQ = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(srcQ), 0, g.bytesQ, 0x00020000);
+    auto ldP = [&](int off, bool valid) -> float {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrcP, valid ? (unsigned)off * 4u : 0x80000000u, 0, 0));
+    };
+    auto ldQ = [&](int off, bool valid) -> float {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrcQ, valid ? (unsigned)off * 4u : 0x80000000u, 0, 0));
+    };
     int pb = 0, py = 0, px = 0;             // decoded p (FWD: b,oy,ox; BWD_DATA: b,iy,ix)
     bool pvalid = false;
     int pbase = 0;                          // FWD: offset of tap (0,0) of channel 0 for this pixel; BWD_DATA: of (b, o = 0)
@@ -107,9 +118,9 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
             for (int i = 0; i < 8; ++i) {
                 const int iy = iy0 + pty[i], ix = ix0 + ptx[i];
                 const bool v = kv && poff[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                rp[i] = v ? srcP[xbase + poff[i]] : 0.0f;
+                rp[i] = ldP(xbase + poff[i], v);
                 const int q = qtile + lp + 16 * i;
-                rq[i] = (kv && q < g.Q) ? srcQ[ybase + q * plane] : 0.0f;
+                rq[i] = ldQ(ybase + q * plane, kv && q < g.Q);
             }
         } else {
             // P operand: k = k0 + lk + i -> (channel-like, ty, tx), advanced with carries
@@ -120,7 +131,7 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const bool v = ((tapmask >> tap) & 1) && k + i < kend;
-                    rp[i] = v ? srcP[off] : 0.0f;
+                    rp[i] = ldP(off, v);
                     ++off; ++tap;
                     if (++tx == g.kW) {
                         tx = 0; off += g.W - g.kW;
@@ -131,19 +142,15 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
                 const bool unit = g.sx == 1 && g.sy == 1;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    float v = 0.0f;
-                    if (pvalid && k + i < kend) {
-                        const int ny = py + g.pt - ty, nx = px + g.pl - tx;
-                        if (unit) {
-                            if (ny >= 0 && nx >= 0 && ny < g.oH && nx < g.oW)
-                                v = srcP[pbase + (ch * g.oH + ny) * g.oW + nx];
-                        } else if (ny >= 0 && nx >= 0 && ny % g.sy == 0 && nx % g.sx == 0) {
-                            const int oy = ny / g.sy, ox = nx / g.sx;
-                            if (oy < g.oH && ox < g.oW)
-                                v = srcP[pbase + (ch * g.oH + oy) * g.oW + ox];
-                        }
+                    const int ny = py + g.pt - ty, nx = px + g.pl - tx;
+                    int oy = ny, ox = nx;
+                    bool v = pvalid && k + i < kend && ny >= 0 && nx >= 0;
+                    if (!unit) {
+                        oy = ny / g.sy; ox = nx / g.sx;
+                        v = v && oy * g.sy == ny && ox * g.sx == nx;
                     }
-                    rp[i] = v;
+                    v = v && oy < g.oH && ox < g.oW;
+                    rp[i] = ldP(pbase + (ch * g.oH + oy) * g.oW + ox, v);
                     if (++tx == g.kW) { tx = 0; if (++ty == g.kH) { ty = 0; ++ch; } }
                 }
             }
@@ -152,14 +159,14 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int kq = k0 + lk_w + i;
-                    rq[i] = (q < g.Q && kq < kend) ? srcQ[q * g.K + kq] : 0.0f;
+                    rq[i] = ldQ(q * g.K + kq, q < g.Q && kq < kend);
                 }
             } else {
                 const int q = qtile + lp;           // input channel c; w[(o*C + c)*kHW + tap], k = o*kHW + tap
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const int kq = k + i;
-                    rq[i] = (q < g.Q && kq < kend) ? srcQ[((kq / kHW) * g.C + q) * kHW + kq % kHW] : 0.0f;
+                    rq[i] = ldQ(((kq / kHW) * g.C + q) * kHW + kq % kHW, q < g.Q && kq < kend);
                 }
             }
         }

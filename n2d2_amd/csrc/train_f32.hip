@@ -265,10 +265,12 @@ static bool use_gemm(const ConvF32& q)
 
 static GemmF32 make_gemm(const ConvF32& q, int mode)
 {
-    GemmF32 g = {q.B, q.C, q.H, q.W, q.O, q.oH, q.oW, q.kW, q.kH, q.sx, q.sy, q.pl, q.pt, 0, 0, 0, 0};
-    if (mode == GEMM_FWD) { g.P = q.B * q.oH * q.oW; g.Q = q.O; g.K = q.C * q.kH * q.kW; }
-    else if (mode == GEMM_BWD_DATA) { g.P = q.B * q.H * q.W; g.Q = q.C; g.K = q.O * q.kH * q.kW; }
-    else { g.P = q.C * q.kH * q.kW; g.Q = q.O; g.K = q.B * q.oH * q.oW; }
+    GemmF32 g = {q.B, q.C, q.H, q.W, q.O, q.oH, q.oW, q.kW, q.kH, q.sx, q.sy, q.pl, q.pt, 0, 0, 0, 0, 0, 0};
+    const unsigned xb = (unsigned)((size_t)q.B * q.C * q.H * q.W * 4), yb = (unsigned)((size_t)q.B * q.O * q.oH * q.oW * 4);
+    const unsigned wb = (unsigned)((size_t)q.O * q.C * q.kH * q.kW * 4);
+    if (mode == GEMM_FWD) { g.P = q.B * q.oH * q.oW; g.Q = q.O; g.K = q.C * q.kH * q.kW; g.bytesP = xb; g.bytesQ = wb; }
+    else if (mode == GEMM_BWD_DATA) { g.P = q.B * q.H * q.W; g.Q = q.C; g.K = q.O * q.kH * q.kW; g.bytesP = yb; g.bytesQ = wb; }
+    else { g.P = q.C * q.kH * q.kW; g.Q = q.O; g.K = q.B * q.oH * q.oW; g.bytesP = xb; g.bytesQ = yb; }
     g.kchunk = round_up(g.K, GK);
     return g;
 }
@@ -285,8 +287,8 @@ static int filter_splits(GemmF32* g)
 
 static bool fits_int(const ConvF32& q)
 {
-    // the GEMM kernel addresses every tensor with 32-bit element offsets and keeps one validity bit per tap
-    const size_t lim = (size_t)1 << 31;
+    // the GEMM kernel reads tensors of at most 2 GiB through buffer descriptors and keeps one validity bit per tap
+    const size_t lim = (size_t)1 << 29;
     return (size_t)q.B * q.C * q.H * q.W < lim && (size_t)q.B * q.O * q.oH * q.oW < lim && (size_t)q.O * q.C * q.kH * q.kW < lim
            && q.kH * q.kW <= 64;
 }
