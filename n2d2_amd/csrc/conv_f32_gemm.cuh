@@ -9,7 +9,8 @@
 //   backward filter  p = weight (c,ty,tx)         q = output channel   k = pixel (b,oy,ox) Pop = x gathered, Qop = dy
 // Taps that fall outside the tensor contribute zero, which is what the reference's clipped window computes.
 //
-// A block of 256 threads (4 waves as 2 x 2) owns a 128 (q) x 128 (p) tile; each wave 64 x 64 as 2 x 2 MFMA tiles.
+// A block of 256 threads (4 waves as 2 x 2) owns a 128 (q) x 128 (p) tile; each wave 64 x 64 as 2 x 2 MFMA tiles.  With at
+// most 64 rows of q (QT = 64) the four waves sit side by side along p instead, each 64 x 32.
 // K advances in steps of 16 through two LDS tiles [k][p] and [k][q] (row stride 129 floats); the next step's
 // elements are fetched into registers while the matrix cores work on the current one and are written to the other pair
 // of tiles, so one barrier per step suffices.  Backward-filter, whose K is
@@ -37,15 +38,18 @@ constexpr int GT = 128;       // tile edge (both p and q)
 constexpr int GK = 16;        // K step
 constexpr int GLD = GT + 1;   // LDS row stride in floats
 
-template <int MODE>
+template <int MODE, int QT>
 __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const float* __restrict__ srcP, const float* __restrict__ srcQ,
                                                             const float* __restrict__ bias, float beta, float* __restrict__ out)
 {
     __shared__ float Pbuf[2][GK * GLD];
     __shared__ float Qbuf[2][GK * GLD];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wq = wave >> 1, wp = wave & 1;
-    const int ptile = blockIdx.x * GT, qtile = blockIdx.y * GT;
+    constexpr int NP = QT / 64;                 // 32-column MFMA tiles of p per wave
+    constexpr int NQL = QT / 16;                // q elements a thread fetches per step
+    const int wq = (QT == 128) ? (wave >> 1) : 0;
+    const int pw = (QT == 128) ? (wave & 1) * 64 : wave * 32;     // the wave's first p inside the tile
+    const int ptile = blockIdx.x * GT, qtile = blockIdx.y * QT;
     const int kbeg = blockIdx.z * g.kchunk, kend = min(kbeg + g.kchunk, g.K);
     const int kHW = g.kH * g.kW;
 
@@ -53,8 +57,10 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
     // BWD_FILTER: thread owns one k of each step and 8 p (and 8 q) spaced by 16.
     const int lp = (MODE == GEMM_BWD_FILTER) ? (t >> 4) : (t & 127);     // first local p (and q for BWD_DATA / BWD_FILTER)
     const int lk = (MODE == GEMM_BWD_FILTER) ? (t & 15) : ((t >> 7) * 8); // first local k
-    // FWD Q operand (weights, contiguous along k): q = t / 2, k = (t % 2) * 8 + i
-    const int lq_w = t >> 1, lk_w = (t & 1) * 8;
+    // Q operand of FWD (weights, contiguous along k): q = t / (16 / NQL), k = (t % (16 / NQL)) * NQL + i;
+    // of BWD_DATA: q = t % QT, k = (t / QT) * NQL + i
+    const int lq_w = (MODE == GEMM_FWD) ? t / (16 / NQL) : t % QT;
+    const int lk_w = (MODE == GEMM_FWD) ? (t % (16 / NQL)) * NQL : (t / QT) * NQL;
 
     // Operands are read through buffer descriptors: an element that does not exist (padding, past the tile or the K
     // range) is requested at an offset past the end and comes back as zero, so the loads need no branches.  All
@@ -119,8 +125,10 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
                 const int iy = iy0 + pty[i], ix = ix0 + ptx[i];
                 const bool v = kv && poff[i] >= 0 && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
                 rp[i] = ldP(xbase + poff[i], v);
-                const int q = qtile + lp + 16 * i;
-                rq[i] = ldQ(ybase + q * plane, kv && q < g.Q);
+                if (i < NQL) {
+                    const int q = qtile + lp + 16 * i;
+                    rq[i] = ldQ(ybase + q * plane, kv && q < g.Q);
+                }
             }
         } else {
             // P operand: k = k0 + lk + i -> (channel-like, ty, tx), advanced with carries
@@ -157,15 +165,15 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
             if (MODE == GEMM_FWD) {
                 const int q = qtile + lq_w;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int i = 0; i < NQL; ++i) {
                     const int kq = k0 + lk_w + i;
                     rq[i] = ldQ(q * g.K + kq, q < g.Q && kq < kend);
                 }
             } else {
-                const int q = qtile + lp;           // input channel c; w[(o*C + c)*kHW + tap], k = o*kHW + tap
+                const int q = qtile + lq_w;         // input channel c; w[(o*C + c)*kHW + tap], k = o*kHW + tap
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int kq = k + i;
+                for (int i = 0; i < NQL; ++i) {
+                    const int kq = k0 + lk_w + i;
                     rq[i] = ldQ(((kq / kHW) * g.C + q) * kHW + kq % kHW, q < g.Q && kq < kend);
                 }
             }
@@ -178,23 +186,22 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 Ps[lk * GLD + lp + 16 * i] = rp[i];
-                Qs[lk * GLD + lp + 16 * i] = rq[i];
+                if (i < NQL) Qs[lk * GLD + lp + 16 * i] = rq[i];
             }
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 Ps[(lk + i) * GLD + lp] = rp[i];
-                if (MODE == GEMM_FWD) Qs[(lk_w + i) * GLD + lq_w] = rq[i];
-                else Qs[(lk + i) * GLD + lp] = rq[i];
+                if (i < NQL) Qs[(lk_w + i) * GLD + lq_w] = rq[i];
             }
         }
     };
 
-    v16f acc[2][2];
+    v16f acc[2][NP];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NP; ++b)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
@@ -213,12 +220,14 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 #pragma unroll
             for (int kk = 0; kk < GK / 2; ++kk) {
                 const float* qrow = Qs + (kk * 2 + kr) * GLD + wq * 64 + col;
-                const float* prow = Ps + (kk * 2 + kr) * GLD + wp * 64 + col;
-                const float a0 = qrow[0], a1 = qrow[32], b0 = prow[0], b1 = prow[32];
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+                const float* prow = Ps + (kk * 2 + kr) * GLD + pw + col;
+                const float a0 = qrow[0], a1 = qrow[32];
+#pragma unroll
+                for (int pi = 0; pi < NP; ++pi) {
+                    const float b = prow[32 * pi];
+                    acc[0][pi] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b, acc[0][pi], 0, 0, 0);
+                    acc[1][pi] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b, acc[1][pi], 0, 0, 0);
+                }
             }
             if (more)
                 stage(buf ^ 1);         // the other tile: its readers passed the barrier of the previous step
@@ -228,8 +237,8 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
 
     // ---- epilogue: lane holds column p = .. + lane % 32 and rows q = .. + 8 * (r / 4) + 4 * (lane / 32) + r % 4
 #pragma unroll
-    for (int pi = 0; pi < 2; ++pi) {
-        const int p = ptile + wp * 64 + pi * 32 + (lane & 31);
+    for (int pi = 0; pi < NP; ++pi) {
+        const int p = ptile + pw + pi * 32 + (lane & 31);
         if (p >= g.P) continue;
         size_t base, qstride;
         if (MODE == GEMM_FWD) {

@@ -278,7 +278,7 @@ static GemmF32 make_gemm(const ConvF32& q, int mode)
 // K ranges of backward-filter: enough blocks to fill the chip, each range at least 8 steps long
 static int filter_splits(GemmF32* g)
 {
-    const long tiles = (long)((g->P + GT - 1) / GT) * ((g->Q + GT - 1) / GT);
+    const long tiles = (long)((g->P + GT - 1) / GT) * (g->Q <= 64 ? 1 : (g->Q + GT - 1) / GT);
     long splits = std::max(1L, 1024 / tiles);
     splits = std::min<long>(splits, std::max(1, g->K / (8 * GK)));
     g->kchunk = round_up((int)((g->K + splits - 1) / splits), GK);
@@ -308,8 +308,12 @@ int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int 
     N2D2HIP_REQUIRE(x && w && y, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_forward: null pointer");
     if (use_gemm(q) && fits_int(q)) {
         const GemmF32 g = make_gemm(q, GEMM_FWD);
-        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_FWD>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0, (hipStream_t)stream,
-                           g, x, w, bias, beta, y);
+        if (g.Q <= 64)
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 64>), dim3((g.P + GT - 1) / GT, 1, 1), dim3(256), 0, (hipStream_t)stream,
+                               g, x, w, bias, beta, y);
+        else
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0,
+                               (hipStream_t)stream, g, x, w, bias, beta, y);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }
@@ -328,8 +332,12 @@ int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H
     N2D2HIP_REQUIRE(w && diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_data: null pointer");
     if (use_gemm(q) && fits_int(q)) {
         const GemmF32 g = make_gemm(q, GEMM_BWD_DATA);
-        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_BWD_DATA>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0, (hipStream_t)stream,
-                           g, diff_y, w, (const float*)nullptr, beta, diff_x);
+        if (g.Q <= 64)
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 64>), dim3((g.P + GT - 1) / GT, 1, 1), dim3(256), 0, (hipStream_t)stream,
+                               g, diff_y, w, (const float*)nullptr, beta, diff_x);
+        else
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0,
+                               (hipStream_t)stream, g, diff_y, w, (const float*)nullptr, beta, diff_x);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }
@@ -364,8 +372,12 @@ int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int
         N2D2HIP_REQUIRE(workspace && workspace_bytes >= need, N2D2HIP_ERR_WORKSPACE,
                         "n2d2hip_conv2d_f32_backward_filter: workspace of %zu bytes, %zu needed (n2d2hip_conv2d_f32_workspace_bytes)",
                         workspace_bytes, need);
-        hipLaunchKernelGGL(conv_f32_gemm_kernel<GEMM_BWD_FILTER>, dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
-                           (hipStream_t)stream, g, x, diff_y, (const float*)nullptr, 0.0f, (float*)workspace);
+        if (g.Q <= 64)
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_FILTER, 64>), dim3((g.P + GT - 1) / GT, 1, splits), dim3(256), 0,
+                               (hipStream_t)stream, g, x, diff_y, (const float*)nullptr, 0.0f, (float*)workspace);
+        else
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_FILTER, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
+                               (hipStream_t)stream, g, x, diff_y, (const float*)nullptr, 0.0f, (float*)workspace);
         hipLaunchKernelGGL(conv_f32_reduce_partials_kernel, dim3(grid_for(nw)), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, splits, nw,
                            beta, diff_w);
         N2D2HIP_HIP_CHECK(hipGetLastError());
