@@ -159,14 +159,106 @@ double Cell_FrameTrain_HIP::applyLoss()
     return loss;
 }
 
+// ------------------------------------------------ WeightedCell_FrameTrain_HIP
+WeightedCell_FrameTrain_HIP::WeightedCell_FrameTrain_HIP()
+    : mWeightsSolver(std::make_shared<SGDSolver_Frame_HIP<float> >()), mBiasSolver(std::make_shared<SGDSolver_Frame_HIP<float> >())
+{
+}
+
+void WeightedCell_FrameTrain_HIP::initializeWeights(const Tensor<Float_T>& weights, Tensor<Float_T>& biases, bool noBias, size_t quantizerOutputsSize)
+{
+    allocateOutputs();
+    mDevW.fromHost(weights);
+    mDevDiffW.resize(weights.dims());
+    if (!noBias) {
+        if (biases.size() != mNbOutputs)
+            biases.resize({mNbOutputs}, 0.0f);
+        mDevBias.resize({mNbOutputs});
+        mDevBias.fromHost(biases.data(), mNbOutputs);
+        mDevDiffBias.resize({mNbOutputs});
+    }
+    if (mQuantizer) {
+        // ConvCell_Frame / FcCell_Frame::initialize hand each weight tensor and its gradient to the quantizer
+        // (src/Cell/ConvCell_Frame.cpp:288-300, src/Cell/FcCell_Frame.cpp:106-112); outputsSize = dimB * dimY * dimX of
+        // the weight tensor as the reference shapes it
+        mQuantizer->addWeights(mDevW.data(), mDevDiffW.data(), mDevW.size(), quantizerOutputsSize);
+        mQuantizer->initialize();
+    }
+}
+
+void WeightedCell_FrameTrain_HIP::propagateWeighted(bool inference, bool noBias)
+{
+    if (mQuantizer)
+        mQuantizer->propagate();
+    const n2d2hip_conv_desc d = desc();
+    const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+    // a quantizer passes the biases through (quantize_bias_propagate copies them)
+    checkStatus(n2d2hip_conv2d_f32_forward(&d, (int)mIn->dimB(), (int)mInH, (int)mInW, mIn->data(), w, noBias ? nullptr : mDevBias.data(), 0.0f,
+                                           mOutputs.data(), mStream));
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+    mDevDiffW.clearValid();
+    mDevDiffBias.clearValid();
+}
+
+void WeightedCell_FrameTrain_HIP::backPropagateWeighted(bool noBias)
+{
+    if (!mDiffInputs.isValid())
+        return;
+    activationBackPropagate();
+    const n2d2hip_conv_desc d = desc();
+    const int B = (int)mIn->dimB();
+    {
+        const float beta = mWeightsSolver->isNewIteration() ? 0.0f : 1.0f;
+        const size_t need = n2d2hip_conv2d_f32_workspace_bytes(&d, B, (int)mInH, (int)mInW);
+        if (need > mWorkspace.size() * sizeof(float))
+            mWorkspace.resize({(need + sizeof(float) - 1) / sizeof(float)});
+        checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(),
+                                                       mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
+        mDevDiffW.setValid();
+    }
+    if (!noBias) {
+        const float beta = mBiasSolver->isNewIteration() ? 0.0f : 1.0f;
+        checkStatus(n2d2hip_conv2d_f32_backward_bias(B, (int)mNbOutputs, (int)mOutH, (int)mOutW, mDiffInputs.data(), beta, mDevDiffBias.data(), mStream));
+        mDevDiffBias.setValid();
+    }
+    if (mDiffOut && !mDiffOut->empty()) {
+        const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
+        const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+        checkStatus(n2d2hip_conv2d_f32_backward_data(&d, B, (int)mInH, (int)mInW, w, mDiffInputs.data(), beta, mDiffOut->data(), mStream));
+        mDiffOut->setValid();
+    }
+    if (mQuantizer)
+        mQuantizer->back_propagate();
+}
+
+void WeightedCell_FrameTrain_HIP::updateWeighted(bool noBias)
+{
+    const unsigned int batch = (unsigned int)mIn->dimB();
+    if (mDevDiffW.isValid())
+        mWeightsSolver->update(mDevW.data(), mQuantizer ? mQuantizer->getDiffFullPrecisionWeights(0) : mDevDiffW.data(), mDevW.size(), batch, mStream);
+    if (!noBias && mDevDiffBias.isValid())
+        mBiasSolver->update(mDevBias.data(), mDevDiffBias.data(), mDevBias.size(), batch, mStream);
+    if (mQuantizer)
+        mQuantizer->update(batch);
+    activationUpdate();
+}
+
+Tensor<Float_T> WeightedCell_FrameTrain_HIP::getQuantizedWeights() const
+{
+    Tensor<Float_T> host(mDevW.dims());
+    const float* src = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+    checkHipT(hipMemcpy(host.data(), src, host.size() * sizeof(float), hipMemcpyDeviceToHost), "WeightedCell_FrameTrain_HIP::getQuantizedWeights()");
+    return host;
+}
+
 // ------------------------------------------------------ ConvCell_FrameTrain_HIP
 template <class T>
 ConvCell_FrameTrain_HIP<T>::ConvCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& kernelDims,
                                                     unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
                                                     const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
                                                     const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims),
-      mWeightsSolver(std::make_shared<SGDSolver_Frame_HIP<T> >()), mBiasSolver(std::make_shared<SGDSolver_Frame_HIP<T> >())
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims)
 {
     mActivation = activation;
 }
@@ -209,86 +301,10 @@ n2d2hip_conv_desc ConvCell_FrameTrain_HIP<T>::desc() const
 template <class T>
 void ConvCell_FrameTrain_HIP<T>::initialize()
 {
-    allocateOutputs();
     const std::vector<size_t> wdims = {mKernelDims[0], mKernelDims[1], mNbChannels / mNbGroups, mNbOutputs};
     if (mWeights.dims() != wdims)
         throw std::runtime_error("ConvCell_FrameTrain_HIP " + mName + ": setWeights() with a {kW, kH, C/groups, O} tensor before initialize()");
-    mDevW.fromHost(mWeights);
-    mDevDiffW.resize(wdims);
-    if (!mNoBias) {
-        if (mBias.size() != mNbOutputs)
-            mBias.resize({mNbOutputs}, 0.0f);
-        mDevBias.resize({mNbOutputs});
-        mDevBias.fromHost(mBias.data(), mNbOutputs);
-        mDevDiffBias.resize({mNbOutputs});
-    }
-    if (mQuantizer) {
-        // Cell_Frame / ConvCell_Frame::initialize hand each weight tensor and its gradient to the quantizer
-        // (src/Cell/ConvCell_Frame.cpp:288-300); outputsSize = dimB * dimY * dimX of the weight tensor
-        mQuantizer->addWeights(mDevW.data(), mDevDiffW.data(), mDevW.size(), (size_t)mNbOutputs * mKernelDims[1] * mKernelDims[0]);
-        mQuantizer->initialize();
-    }
-}
-
-template <class T>
-void ConvCell_FrameTrain_HIP<T>::propagate(bool inference)
-{
-    if (mQuantizer)
-        mQuantizer->propagate();
-    const n2d2hip_conv_desc d = desc();
-    const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
-    // a quantizer passes the biases through (quantize_bias_propagate copies them)
-    checkStatus(n2d2hip_conv2d_f32_forward(&d, (int)mIn->dimB(), (int)mInH, (int)mInW, mIn->data(), w, mNoBias ? nullptr : mDevBias.data(), 0.0f,
-                                           mOutputs.data(), mStream));
-    activationPropagate(inference);
-    mDiffInputs.clearValid();
-    mDevDiffW.clearValid();
-    mDevDiffBias.clearValid();
-}
-
-template <class T>
-void ConvCell_FrameTrain_HIP<T>::backPropagate()
-{
-    if (!mDiffInputs.isValid())
-        return;
-    activationBackPropagate();
-    const n2d2hip_conv_desc d = desc();
-    const int B = (int)mIn->dimB();
-    {
-        const float beta = mWeightsSolver->isNewIteration() ? 0.0f : 1.0f;
-        const size_t need = n2d2hip_conv2d_f32_workspace_bytes(&d, B, (int)mInH, (int)mInW);
-        if (need > mWorkspace.size() * sizeof(float))
-            mWorkspace.resize({(need + sizeof(float) - 1) / sizeof(float)});
-        checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(),
-                                                       mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
-        mDevDiffW.setValid();
-    }
-    if (!mNoBias) {
-        const float beta = mBiasSolver->isNewIteration() ? 0.0f : 1.0f;
-        checkStatus(n2d2hip_conv2d_f32_backward_bias(B, (int)mNbOutputs, (int)mOutH, (int)mOutW, mDiffInputs.data(), beta, mDevDiffBias.data(), mStream));
-        mDevDiffBias.setValid();
-    }
-    if (mDiffOut && !mDiffOut->empty()) {
-        const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
-        const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
-        checkStatus(n2d2hip_conv2d_f32_backward_data(&d, B, (int)mInH, (int)mInW, w, mDiffInputs.data(), beta, mDiffOut->data(), mStream));
-        mDiffOut->setValid();
-    }
-    if (mQuantizer)
-        mQuantizer->back_propagate();
-}
-
-template <class T>
-void ConvCell_FrameTrain_HIP<T>::update()
-{
-    const unsigned int batch = (unsigned int)mIn->dimB();
-    if (mDevDiffW.isValid())
-        mWeightsSolver->update(mDevW.data(), mQuantizer ? mQuantizer->getDiffFullPrecisionWeights(0) : mDevDiffW.data(), mDevW.size(), batch, mStream);
-    if (!mNoBias && mDevDiffBias.isValid())
-        mBiasSolver->update(mDevBias.data(), mDevDiffBias.data(), mDevBias.size(), batch, mStream);
-    if (mQuantizer)
-        mQuantizer->update(batch);
-    activationUpdate();
+    initializeWeights(mWeights, mBias, mNoBias, (size_t)mNbOutputs * mKernelDims[1] * mKernelDims[0]);
 }
 
 template <class T>
@@ -302,18 +318,59 @@ void ConvCell_FrameTrain_HIP<T>::synchronizeWeightsToHost()
     }
 }
 
-template <class T>
-Tensor<Float_T> ConvCell_FrameTrain_HIP<T>::getQuantizedWeights() const
-{
-    Tensor<Float_T> host(mDevW.dims());
-    const float* src = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
-    checkHipT(hipMemcpy(host.data(), src, host.size() * sizeof(float), hipMemcpyDeviceToHost), "ConvCell_FrameTrain_HIP::getQuantizedWeights()");
-    return host;
-}
-
 template class ConvCell_FrameTrain_HIP<float>;
 template <> Registrar<ConvCell> ConvCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", ConvCell_FrameTrain_HIP<float>::create,
                                                                            Registrar<ConvCell>::Type<float>());
+
+// -------------------------------------------------------- FcCell_FrameTrain_HIP
+template <class T>
+FcCell_FrameTrain_HIP<T>::FcCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
+                                                const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs)
+{
+    mActivation = activation;
+}
+
+template <class T>
+n2d2hip_conv_desc FcCell_FrameTrain_HIP<T>::desc() const
+{
+    // the convolution whose kernel spans the input: weights [O][C*H*W] in CHW order are an OCHW kernel
+    n2d2hip_conv_desc d = {};
+    d.C = (int)mNbChannels;
+    d.O = (int)mNbOutputs;
+    d.kW = (int)mInW;
+    d.kH = (int)mInH;
+    d.strideX = d.strideY = 1;
+    d.dilX = d.dilY = 1;
+    d.groups = 1;
+    return d;
+}
+
+template <class T>
+void FcCell_FrameTrain_HIP<T>::initialize()
+{
+    const size_t K = (size_t)mNbChannels * mInH * mInW;
+    if (mWeights.size() != K * mNbOutputs)
+        throw std::runtime_error("FcCell_FrameTrain_HIP " + mName + ": setWeights() with a {K, O} tensor, K = C*H*W, before initialize()");
+    // the reference shapes an FcCell's synapses {1, 1, K, O} (src/Cell/FcCell_Frame.cpp:99-102): dimB * dimY * dimX = O
+    initializeWeights(mWeights, mBias, mNoBias, mNbOutputs);
+}
+
+template <class T>
+void FcCell_FrameTrain_HIP<T>::synchronizeWeightsToHost()
+{
+    const Tensor<Float_T> w = mDevW.toHost();
+    for (size_t i = 0; i < w.size(); ++i) mWeights(i) = w(i);
+    if (!mNoBias) {
+        const Tensor<Float_T> b = mDevBias.toHost();
+        mBias.resize({mNbOutputs});
+        for (size_t i = 0; i < mNbOutputs; ++i) mBias(i) = b(i);
+    }
+}
+
+template class FcCell_FrameTrain_HIP<float>;
+template <> Registrar<FcCell> FcCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", FcCell_FrameTrain_HIP<float>::create,
+                                                                       Registrar<FcCell>::Type<float>());
 
 // ------------------------------------------------ ActivationCell_FrameTrain_HIP
 const char* ActivationCell::Type = "Activation";

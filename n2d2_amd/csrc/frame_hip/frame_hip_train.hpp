@@ -86,9 +86,37 @@ private:
     size_t mLossWorkspaceBytes;
 };
 
+// What ConvCell_Frame and FcCell_Frame share when they learn: device weights and biases with their gradients, the weight
+// quantizer, the solvers, and the three convolution passes (an FcCell is the convolution whose kernel spans its input).
+class WeightedCell_FrameTrain_HIP : public Cell_FrameTrain_HIP {
+public:
+    // Cell::setQuantizer (include/Cell/Cell.hpp:455-463), before initialize()
+    void setQuantizer(const std::shared_ptr<QuantizerCell>& quantizer) { mQuantizer = quantizer; }
+    const std::shared_ptr<QuantizerCell>& getQuantizer() const { return mQuantizer; }
+    void setWeightsSolver(const std::shared_ptr<SGDSolver>& solver) { mWeightsSolver = solver; }
+    void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
+    Tensor<Float_T> getDiffWeights() const { return mDevDiffW.toHost(); }
+    Tensor<Float_T> getQuantizedWeights() const;
+    // refreshes the host tensors getWeights() / getBiases() return from the device
+    virtual void synchronizeWeightsToHost() = 0;
+
+protected:
+    WeightedCell_FrameTrain_HIP();
+    virtual n2d2hip_conv_desc desc() const = 0;
+    // uploads weights (dims as the cell holds them) and biases, allocates the gradients, hands the weights to the quantizer
+    void initializeWeights(const Tensor<Float_T>& weights, Tensor<Float_T>& biases, bool noBias, size_t quantizerOutputsSize);
+    void propagateWeighted(bool inference, bool noBias);
+    void backPropagateWeighted(bool noBias);
+    void updateWeighted(bool noBias);
+    std::shared_ptr<QuantizerCell> mQuantizer;
+    std::shared_ptr<SGDSolver> mWeightsSolver, mBiasSolver;
+    DeviceFloats mDevW, mDevDiffW, mDevBias, mDevDiffBias;
+    DeviceFloats mWorkspace;        // partial sums of backward-filter
+};
+
 // src/Cell/ConvCell_Frame.cpp:418-597 for one input tensor.
 template <class T>
-class ConvCell_FrameTrain_HIP : public ConvCell, public Cell_FrameTrain_HIP {
+class ConvCell_FrameTrain_HIP : public ConvCell, public WeightedCell_FrameTrain_HIP {
 public:
     ConvCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, const std::vector<unsigned int>& kernelDims,
                             unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
@@ -104,31 +132,43 @@ public:
         return std::make_shared<ConvCell_FrameTrain_HIP<T> >(deepNet, name, kernelDims, nbOutputs, subSampleDims, strideDims,
                                                              paddingDims, dilationDims, activation);
     }
-    // Cell::setQuantizer (include/Cell/Cell.hpp:455-463), before initialize()
-    void setQuantizer(const std::shared_ptr<QuantizerCell>& quantizer) { mQuantizer = quantizer; }
-    const std::shared_ptr<QuantizerCell>& getQuantizer() const { return mQuantizer; }
-    void setWeightsSolver(const std::shared_ptr<SGDSolver>& solver) { mWeightsSolver = solver; }
-    void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
-    // uploads the host weights / biases (ConvCell::setWeights), allocates gradients, hands the weights to the quantizer
+    // uploads the host weights / biases (ConvCell::setWeights, {kW, kH, C/groups, O}) before anything else
     void initialize();
-    void propagate(bool inference = false);
-    void backPropagate();
-    void update();
-    // refreshes the host tensors ConvCell::getWeights() / getBiases() return from the device
+    void propagate(bool inference = false) { propagateWeighted(inference, mNoBias); }
+    void backPropagate() { backPropagateWeighted(mNoBias); }
+    void update() { updateWeighted(mNoBias); }
     void synchronizeWeightsToHost();
-    Tensor<Float_T> getDiffWeights() const { return mDevDiffW.toHost(); }
-    Tensor<Float_T> getQuantizedWeights() const;
 
 protected:
     void setOutputsDims();
+    n2d2hip_conv_desc desc() const;
 
 private:
-    n2d2hip_conv_desc desc() const;
-    std::shared_ptr<QuantizerCell> mQuantizer;
-    std::shared_ptr<SGDSolver> mWeightsSolver, mBiasSolver;
-    DeviceFloats mDevW, mDevDiffW, mDevBias, mDevDiffBias;
-    DeviceFloats mWorkspace;        // partial sums of backward-filter
     static Registrar<ConvCell> mRegistrar;
+};
+
+// src/Cell/FcCell_Frame.cpp:234-480 for one input tensor: weights {K, O} with K = C*H*W in CHW order.
+template <class T>
+class FcCell_FrameTrain_HIP : public FcCell, public WeightedCell_FrameTrain_HIP {
+public:
+    FcCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, const std::shared_ptr<Activation>& activation);
+    static std::shared_ptr<FcCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                          const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<FcCell_FrameTrain_HIP<T> >(deepNet, name, nbOutputs, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false) { propagateWeighted(inference, mNoBias); }
+    void backPropagate() { backPropagateWeighted(mNoBias); }
+    void update() { updateWeighted(mNoBias); }
+    void synchronizeWeightsToHost();
+
+protected:
+    void setOutputsDims() { mOutW = 1; mOutH = 1; }
+    n2d2hip_conv_desc desc() const;
+
+private:
+    static Registrar<FcCell> mRegistrar;
 };
 
 // include/Cell/ActivationCell.hpp:36-60

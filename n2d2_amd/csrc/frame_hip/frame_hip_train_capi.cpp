@@ -91,6 +91,7 @@ int fh_train_registrar_exists(const char* type, const char* key)
 {
     const std::string t(type), k(key);
     if (t == "Conv") return Registrar<ConvCell>::exists<float>(k);
+    if (t == "Fc") return Registrar<FcCell>::exists<float>(k);
     if (t == "Activation") return Registrar<ActivationCell>::exists<float>(k);
     if (t == "Softmax") return Registrar<SoftmaxCell>::exists<float>(k);
     return -1;
@@ -168,6 +169,42 @@ int fh_train_add_conv(void* net, const char* name, int nbOutputs, int kW, int kH
     });
 }
 
+// weights: HOST float [O, C*H*W] (CHW order); bias HOST float [O] or NULL (NoBias).  weightQuant: 0 none, 1 SAT, 2 LSQ.
+int fh_train_add_fc(void* net, const char* name, int nbOutputs, const float* weights, const float* bias, int act, int actQuant, int actRange,
+                    float actParam, int weightQuant, int weightRange)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<FcCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        auto fc = f(n.net, n.deepNet, name, (unsigned)nbOutputs, makeActivation(n, name, act, actQuant, actRange, actParam));
+        auto cell = std::dynamic_pointer_cast<FcCell_FrameTrain_HIP<float> >(fc);
+        const size_t K = n.cells.empty() ? n.input.dimX() * n.input.dimY() * n.input.dimZ()
+                                         : n.last()->getOutputs().dimX() * n.last()->getOutputs().dimY() * n.last()->getOutputs().dimZ();
+        fc->setParameter("NoBias", bias == nullptr);
+        Tensor<Float_T> w({K, (size_t)nbOutputs});
+        std::memcpy(w.data(), weights, w.size() * sizeof(float));
+        fc->setWeights(w);
+        if (bias) {
+            Tensor<Float_T> b({(size_t)nbOutputs});
+            std::memcpy(b.data(), bias, nbOutputs * sizeof(float));
+            fc->setBiases(b);
+        }
+        if (weightQuant == 1) {
+            auto q = Registrar<SATQuantizerCell>::create<float>("Frame_HIP")();
+            q->setRange((size_t)weightRange);
+            cell->setQuantizer(q);
+        } else if (weightQuant == 2) {
+            auto q = Registrar<LSQQuantizerCell>::create<float>("Frame_HIP")();
+            q->setRange((size_t)weightRange);
+            q->setSolver(Registrar<SGDSolver>::create<float>("Frame_HIP")());
+            cell->setQuantizer(q);
+            n.lsqCell[name] = std::dynamic_pointer_cast<LSQQuantizerCell_Frame_HIP<float> >(q);
+        }
+        connect(n, cell);
+    });
+}
+
 int fh_train_add_softmax(void* net, const char* name, int withLoss)
 {
     return guardedT([&] {
@@ -184,8 +221,8 @@ int fh_train_add_softmax(void* net, const char* name, int withLoss)
 int fh_train_set_solver_parameter(void* net, const char* cell, const char* name, double value)
 {
     return guardedT([&] {
-        auto conv = dynamic_cast<ConvCell_FrameTrain_HIP<float>*>(find(*(TrainNet*)net, cell));
-        if (!conv) throw std::runtime_error("Not a ConvCell: " + std::string(cell));
+        auto conv = dynamic_cast<WeightedCell_FrameTrain_HIP*>(find(*(TrainNet*)net, cell));
+        if (!conv) throw std::runtime_error("Not a cell with weights: " + std::string(cell));
         auto s = Registrar<SGDSolver>::create<float>("Frame_HIP")();
         s->setParameter(name, value);
         conv->setWeightsSolver(s);
@@ -233,11 +270,15 @@ int fh_train_get(void* net, const char* cell, int what, float* out, size_t n)
     return guardedT([&] {
         Cell_FrameTrain_HIP* c = find(*(TrainNet*)net, cell);
         Tensor<Float_T> t;
-        auto conv = dynamic_cast<ConvCell_FrameTrain_HIP<float>*>(c);
+        auto conv = dynamic_cast<WeightedCell_FrameTrain_HIP*>(c);
         if (what == 0) t = c->getOutputs().toHost();
         else if (what == 1) t = c->getDiffInputs().toHost();
-        else if (!conv) throw std::runtime_error("Not a ConvCell: " + std::string(cell));
-        else if (what == 2) { conv->synchronizeWeightsToHost(); t = conv->getWeights(); }
+        else if (!conv) throw std::runtime_error("Not a cell with weights: " + std::string(cell));
+        else if (what == 2) {
+            conv->synchronizeWeightsToHost();
+            if (auto cc = dynamic_cast<ConvCell*>(c)) t = cc->getWeights();
+            else t = dynamic_cast<FcCell*>(c)->getWeights();
+        }
         else if (what == 3) t = conv->getDiffWeights();
         else t = conv->getQuantizedWeights();
         if (t.size() != n) throw std::runtime_error("fh_train_get(): size mismatch");

@@ -83,7 +83,7 @@ def test_every_class_of_the_path_is_registered_under_frame_hip(fh):
 
 
 def test_the_float_learning_cells_are_registered_under_their_own_key(fh):
-    for t in ("Conv", "Activation", "Softmax"):
+    for t in ("Conv", "Fc", "Activation", "Softmax"):
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_HIP_QAT") == 1, t
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_CUDA") == 0, t
     # the integer inference cells own ("Frame_HIP", float); the two keys do not collide

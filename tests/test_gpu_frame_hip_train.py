@@ -42,7 +42,7 @@ def _close(got, want, tol=1e-5):
 
 def test_registrar_holds_the_float_cells():
     from n2d2_amd import frame_hip as fh
-    for t in ("Conv", "Activation", "Softmax"):
+    for t in ("Conv", "Fc", "Activation", "Softmax"):
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_HIP_QAT") == 1
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_XYZ") == 0
     assert fh.lib.fh_train_registrar_exists(b"Conv", b"Frame_HIP") == 1          # the integer inference cell
@@ -187,19 +187,55 @@ def test_known_answer_lsq_step_sizes_three_conv():
 
 
 def test_known_answer_lsq_step_size_fc():
-    """tests/Cell/class_FcCell_QuantizerLSQ_Frame_CUDA.cpp, run as the 3x3 convolution over the 3x3 input."""
+    """tests/Cell/class_FcCell_QuantizerLSQ_Frame_CUDA.cpp through the FcCell class."""
     from n2d2_amd import frame_hip as fh
     fc = json.load(open(LSQ_GOLD))["fc"]
     x = (np.float32(0.125) * np.arange(9, dtype=np.float32)).reshape(1, 1, 3, 3)
-    w = np.zeros((2, 1, 3, 3), dtype=np.float32)
+    w = np.zeros((2, 9), dtype=np.float32)
     for k, v in enumerate(fc["weights_per_output"]):
         w[k] = v
     net = fh.TrainNet(x)
     net.add_activation_cell("activation1", "Linear")
-    net.add_conv("fc1", w, weight_quant="LSQ", weight_range=fc["range"])
+    net.add_fc("fc1", w, weight_quant="LSQ", weight_range=fc["range"])
     net.add_softmax("softmax1", with_loss=True)
     print("lsq fc", flush=True)
     net.learn(np.array(fc["target"], dtype=np.float32).reshape(1, 2, 1, 1), fc["iterations"])
     step = net.weight_quantizer("fc1")[0]
     print("step", step, flush=True)
     assert abs(step - fc["expected_step"]) < fc["delta"]
+
+
+def test_conv_then_fc_with_bias_against_the_oracle():
+    """ConvCell (Rectifier) -> FcCell with a bias and a SAT weight quantizer -> softmax with loss: three iterations."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    rng = np.random.default_rng(33)
+    x = rng.uniform(0, 1, size=(3, 2, 6, 6)).astype(np.float32)
+    w1 = rng.normal(0, 0.4, size=(4, 2, 3, 3)).astype(np.float32)
+    wf = rng.normal(0, 0.2, size=(5, 4 * 4 * 4)).astype(np.float32)
+    bf = rng.normal(0, 0.1, size=5).astype(np.float32)
+    net = fh.TrainNet(x, propagate_gradient=False)
+    net.add_conv("c1", w1, act="Rectifier")
+    net.add_fc("fc", wf, bias=bf, weight_quant="SAT", weight_range=15)
+    net.add_softmax("softmax", with_loss=True)
+    t = np.zeros((3, 5, 1, 1), dtype=np.float32)
+    t[0, 1] = t[1, 4] = t[2, 0] = 1
+
+    class Rect(q.LinearActivation):
+        def propagate(self, v, inference):
+            self.out = np.maximum(v, 0).astype(np.float32)
+            return self.out
+
+        def back_propagate(self, d):
+            return (d * (self.out > 0)).astype(np.float32)
+    c1 = q.ConvCell(w1, activation=Rect())
+    fc = q.ConvCell(wf.reshape(5, 4, 4, 4), bias=bf, quantizer=q.SATQuantizerCell(15))
+    fc.quantizer_outputs_size = 5
+    sm = q.SoftmaxCell()
+    print("conv -> fc net", flush=True)
+    for it in range(3):
+        loss = net.learn(t, 1)
+        want = q.train_sequential(x, [c1, fc], sm, t, 1)
+        assert abs(loss - want) <= 1e-5 * want, it
+    assert _close(net.outputs("softmax"), sm.outputs)
+    assert _close(net.weights("fc"), fc.w.reshape(5, -1), 1e-4) and _close(net.weights("c1"), c1.w, 1e-4)
