@@ -72,12 +72,12 @@ def qat_conv_step(torch, steps=10):
     def step():
         s = sp()
         chk(lib.n2d2hip_sat_weight_forward(w.data_ptr(), wq.data_ptr(), nw, 15.0, capi.SAT_DEFAULT, 0, 1, stats.data_ptr(), wsq.data_ptr(), wsq.numel(), s))
-        chk(lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, H, x.data_ptr(), wq.data_ptr(), None, 0.0, y.data_ptr(), s))
+        chk(lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, H, x.data_ptr(), wq.data_ptr(), None, 0.0, y.data_ptr(), wsf.data_ptr(), need, s))
         chk(lib.n2d2hip_sat_act_forward(y.data_ptr(), fp.data_ptr(), n, 15.0, alpha.data_ptr(), s))
         chk(lib.n2d2hip_sat_act_backward(dy.data_ptr(), fp.data_ptr(), g.data_ptr(), n, 15.0, alpha.data_ptr(), 0.0, dalpha.data_ptr(),
                                          wsq.data_ptr(), wsq.numel(), s))
         chk(lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, H, x.data_ptr(), g.data_ptr(), 0.0, dwq.data_ptr(), wsf.data_ptr(), need, s))
-        chk(lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, H, wq.data_ptr(), g.data_ptr(), 0.0, dx.data_ptr(), s))
+        chk(lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, H, wq.data_ptr(), g.data_ptr(), 0.0, dx.data_ptr(), wsf.data_ptr(), need, s))
         chk(lib.n2d2hip_sat_weight_backward(dwq.data_ptr(), w.data_ptr(), dw.data_ptr(), nw, 15.0, capi.SAT_DEFAULT, 0, stats.data_ptr(), s))
         chk(lib.n2d2hip_sgd_update_f32(w.data_ptr(), dw.data_ptr(), nw, 0.01 / B, 0.0, 0.0, None, 0, 0.0, 0.0, s))
         chk(lib.n2d2hip_sgd_update_f32(alpha.data_ptr(), dalpha.data_ptr(), 1, 0.01 / B, 0.0, 0.0, None, 0, 0.0, 0.0, s))

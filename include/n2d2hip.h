@@ -275,14 +275,20 @@ int n2d2hip_lsq_backward(const float* diff_q, const float* fp_x, float* diff_fp,
  * y = conv(x, w) (+ bias[o] if bias != NULL) + beta * y; the window is clipped at the borders (ref: src/Cell/ConvCell_Frame_Kernels.cpp:26-174, called from
  * ConvCell_Frame<T>::propagate, src/Cell/ConvCell_Frame.cpp:418-473). */
 int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* w,
-                               const float* bias, float beta, float* y, n2d2hip_stream_t stream);
+                               const float* bias, float beta, float* y, void* workspace, size_t workspace_bytes,
+                               n2d2hip_stream_t stream);
 /* diff_x = backwardData(w, diff_y) + beta * diff_x (ref: src/Cell/ConvCell_Frame_Kernels.cpp:176-333).  Dilation
  * must be 1: the reference's backward kernels do not read it. */
 int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* w,
-                                     const float* diff_y, float beta, float* diff_x, n2d2hip_stream_t stream);
-/* diff_w = backwardFilter(x, diff_y) + beta * diff_w (ref: src/Cell/ConvCell_Frame_Kernels.cpp:335-427).  The sum over
- * batch and pixels is split into ranges whose partial results go through `workspace` (device memory, at least
- * n2d2hip_conv2d_f32_workspace_bytes, which may be 0) and are added in a fixed order. */
+                                     const float* diff_y, float beta, float* diff_x, void* workspace,
+                                     size_t workspace_bytes, n2d2hip_stream_t stream);
+/* diff_w = backwardFilter(x, diff_y) + beta * diff_w (ref: src/Cell/ConvCell_Frame_Kernels.cpp:335-427).
+ *
+ * `workspace` (device memory) of the three passes: n2d2hip_conv2d_f32_workspace_bytes bytes (may be 0) serve all of
+ * them.  Backward-filter splits its sum over batch and pixels into ranges whose partial results go through the
+ * workspace and are added in a fixed order; it fails with N2D2HIP_ERR_WORKSPACE when the workspace is too small.
+ * Forward and backward-data do the same to fill the chip when their output is small, and run as one range when the
+ * workspace is NULL or too small. */
 size_t n2d2hip_conv2d_f32_workspace_bytes(const n2d2hip_conv_desc* desc, int B, int H, int W);
 int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x,
                                        const float* diff_y, float beta, float* diff_w, void* workspace,

@@ -103,8 +103,8 @@ def load():
     lib.n2d2hip_sat_act_backward.argtypes = [P, P, P, SZ, F, P, F, P, P, SZ, P]
     lib.n2d2hip_lsq_forward.argtypes = [P, P, SZ, P, I, I, P]
     lib.n2d2hip_lsq_backward.argtypes = [P, P, P, SZ, P, I, I, F, F, P, P, SZ, P]
-    lib.n2d2hip_conv2d_f32_forward.argtypes = [P, I, I, I, P, P, P, F, P, P]
-    lib.n2d2hip_conv2d_f32_backward_data.argtypes = [P, I, I, I, P, P, F, P, P]
+    lib.n2d2hip_conv2d_f32_forward.argtypes = [P, I, I, I, P, P, P, F, P, P, SZ, P]
+    lib.n2d2hip_conv2d_f32_backward_data.argtypes = [P, I, I, I, P, P, F, P, P, SZ, P]
     lib.n2d2hip_conv2d_f32_backward_filter.argtypes = [P, I, I, I, P, P, F, P, P, SZ, P]
     lib.n2d2hip_conv2d_f32_workspace_bytes.restype = C.c_size_t
     lib.n2d2hip_conv2d_f32_workspace_bytes.argtypes = [P, I, I, I]

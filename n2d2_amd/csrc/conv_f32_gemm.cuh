@@ -15,7 +15,7 @@
 // elements are fetched into registers while the matrix cores work on the current one and are written to the other pair
 // of tiles, so one barrier per step suffices.  Backward-filter, whose K is
 // the whole batch of pixels and whose output is small, splits K over blockIdx.z into partial results that a second
-// kernel adds up in a fixed order.
+// kernel adds up in a fixed order; forward and backward-data do the same when their tiles alone would not fill the chip.
 #pragma once
 
 #include "common.h"
@@ -250,9 +250,12 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
             base = (size_t)(p / plane) * g.C * plane + p % plane;
             qstride = plane;
         } else {
-            base = (size_t)blockIdx.z * g.Q * g.P + p;      // partial result of this K range
+            base = p;
             qstride = g.P;
         }
+        const bool partial = MODE == GEMM_BWD_FILTER || gridDim.z > 1;     // `out` is then the buffer of partial results
+        if (partial)
+            base += (size_t)blockIdx.z * g.Q * g.P;
 #pragma unroll
         for (int qi = 0; qi < 2; ++qi) {
 #pragma unroll
@@ -261,7 +264,7 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
                 if (q >= g.Q) continue;
                 const size_t idx = base + (size_t)q * qstride;
                 float v = acc[qi][pi][r];
-                if (MODE != GEMM_BWD_FILTER) {
+                if (!partial) {
                     if (beta != 0.0f) v += beta * out[idx];
                     if (MODE == GEMM_FWD && bias) v = bias[q] + v;
                 }
@@ -271,14 +274,17 @@ __global__ __launch_bounds__(256) void conv_f32_gemm_kernel(GemmF32 g, const flo
     }
 }
 
-// dw[i] = sum over the K ranges, in their order, + beta * dw[i]
+// out[i] = sum over the K ranges, in their order, + beta * out[i] (+ bias of element i's channel, NCHW with `plane`
+// pixels per channel and O channels)
 __global__ __launch_bounds__(256) void conv_f32_reduce_partials_kernel(const float* __restrict__ partial, int splits, size_t n, float beta,
-                                                                       float* __restrict__ dw)
+                                                                       float* __restrict__ out, const float* __restrict__ bias, int plane, int O)
 {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
         double s = 0.0;
         for (int z = 0; z < splits; ++z) s += (double)partial[(size_t)z * n + i];
-        dw[i] = (float)s + (beta != 0.0f ? beta * dw[i] : 0.0f);
+        float v = (float)s + (beta != 0.0f ? beta * out[i] : 0.0f);
+        if (bias) v = bias[(i / plane) % O] + v;
+        out[i] = v;
     }
 }
 

@@ -192,9 +192,12 @@ void WeightedCell_FrameTrain_HIP::propagateWeighted(bool inference, bool noBias)
         mQuantizer->propagate();
     const n2d2hip_conv_desc d = desc();
     const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
+    const size_t need = n2d2hip_conv2d_f32_workspace_bytes(&d, (int)mIn->dimB(), (int)mInH, (int)mInW);
+    if (need > mWorkspace.size() * sizeof(float))
+        mWorkspace.resize({(need + sizeof(float) - 1) / sizeof(float)});
     // a quantizer passes the biases through (quantize_bias_propagate copies them)
     checkStatus(n2d2hip_conv2d_f32_forward(&d, (int)mIn->dimB(), (int)mInH, (int)mInW, mIn->data(), w, noBias ? nullptr : mDevBias.data(), 0.0f,
-                                           mOutputs.data(), mStream));
+                                           mOutputs.data(), mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
     activationPropagate(inference);
     mDiffInputs.clearValid();
     mDevDiffW.clearValid();
@@ -210,9 +213,6 @@ void WeightedCell_FrameTrain_HIP::backPropagateWeighted(bool noBias)
     const int B = (int)mIn->dimB();
     {
         const float beta = mWeightsSolver->isNewIteration() ? 0.0f : 1.0f;
-        const size_t need = n2d2hip_conv2d_f32_workspace_bytes(&d, B, (int)mInH, (int)mInW);
-        if (need > mWorkspace.size() * sizeof(float))
-            mWorkspace.resize({(need + sizeof(float) - 1) / sizeof(float)});
         checkStatus(n2d2hip_conv2d_f32_backward_filter(&d, B, (int)mInH, (int)mInW, mIn->data(), mDiffInputs.data(), beta, mDevDiffW.data(),
                                                        mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
         mDevDiffW.setValid();
@@ -225,7 +225,8 @@ void WeightedCell_FrameTrain_HIP::backPropagateWeighted(bool noBias)
     if (mDiffOut && !mDiffOut->empty()) {
         const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
         const float* w = mQuantizer ? mQuantizer->getQuantizedWeights(0) : mDevW.data();
-        checkStatus(n2d2hip_conv2d_f32_backward_data(&d, B, (int)mInH, (int)mInW, w, mDiffInputs.data(), beta, mDiffOut->data(), mStream));
+        checkStatus(n2d2hip_conv2d_f32_backward_data(&d, B, (int)mInH, (int)mInW, w, mDiffInputs.data(), beta, mDiffOut->data(),
+                                                     mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
         mDiffOut->setValid();
     }
     if (mQuantizer)

@@ -111,7 +111,7 @@ protected:
     std::shared_ptr<QuantizerCell> mQuantizer;
     std::shared_ptr<SGDSolver> mWeightsSolver, mBiasSolver;
     DeviceFloats mDevW, mDevDiffW, mDevBias, mDevDiffBias;
-    DeviceFloats mWorkspace;        // partial sums of backward-filter
+    DeviceFloats mWorkspace;        // partial sums of the convolution passes
 };
 
 // src/Cell/ConvCell_Frame.cpp:418-597 for one input tensor.

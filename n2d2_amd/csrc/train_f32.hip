@@ -285,6 +285,17 @@ static int filter_splits(GemmF32* g)
     return (g->K + g->kchunk - 1) / g->kchunk;
 }
 
+// K ranges of forward / backward-data when the tiles alone leave most of the chip idle (three blocks fit a CU): each
+// range at least 16 steps long
+static int pass_splits(GemmF32* g)
+{
+    const long tiles = (long)((g->P + GT - 1) / GT) * (g->Q <= 64 ? 1 : (g->Q + GT - 1) / GT);
+    long splits = tiles >= 384 ? 1 : std::max(1L, 768 / tiles);
+    splits = std::min<long>(splits, std::max(1, g->K / (16 * GK)));
+    g->kchunk = round_up((int)((g->K + splits - 1) / splits), GK);
+    return (g->K + g->kchunk - 1) / g->kchunk;
+}
+
 static bool fits_int(const ConvF32& q)
 {
     // the GEMM kernel reads tensors of at most 2 GiB through buffer descriptors and keeps one validity bit per tap
@@ -300,20 +311,30 @@ using namespace n2d2hip;
 extern "C" {
 
 int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* w, const float* bias,
-                               float beta, float* y, n2d2hip_stream_t stream)
+                               float beta, float* y, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
 {
     ConvF32 q;
     const int st = make_conv(desc, B, H, W, false, &q, "n2d2hip_conv2d_f32_forward");
     if (st != N2D2HIP_OK) return st;
     N2D2HIP_REQUIRE(x && w && y, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_forward: null pointer");
     if (use_gemm(q) && fits_int(q)) {
-        const GemmF32 g = make_gemm(q, GEMM_FWD);
+        GemmF32 g = make_gemm(q, GEMM_FWD);
+        const size_t n = (size_t)g.P * g.Q;
+        int splits = pass_splits(&g);
+        if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * n * sizeof(float))) {
+            splits = 1;                                     // no room for partial results: one range
+            g.kchunk = round_up(g.K, GK);
+        }
+        float* dst = splits > 1 ? (float*)workspace : y;
         if (g.Q <= 64)
-            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 64>), dim3((g.P + GT - 1) / GT, 1, 1), dim3(256), 0, (hipStream_t)stream,
-                               g, x, w, bias, beta, y);
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 64>), dim3((g.P + GT - 1) / GT, 1, splits), dim3(256), 0, (hipStream_t)stream,
+                               g, x, w, bias, beta, dst);
         else
-            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0,
-                               (hipStream_t)stream, g, x, w, bias, beta, y);
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_FWD, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
+                               (hipStream_t)stream, g, x, w, bias, beta, dst);
+        if (splits > 1)
+            hipLaunchKernelGGL(conv_f32_reduce_partials_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, splits, n,
+                               beta, y, bias, q.oH * q.oW, q.O);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }
@@ -324,20 +345,30 @@ int n2d2hip_conv2d_f32_forward(const n2d2hip_conv_desc* desc, int B, int H, int 
 }
 
 int n2d2hip_conv2d_f32_backward_data(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* w, const float* diff_y, float beta,
-                                     float* diff_x, n2d2hip_stream_t stream)
+                                     float* diff_x, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
 {
     ConvF32 q;
     const int st = make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_backward_data");
     if (st != N2D2HIP_OK) return st;
     N2D2HIP_REQUIRE(w && diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_conv2d_f32_backward_data: null pointer");
     if (use_gemm(q) && fits_int(q)) {
-        const GemmF32 g = make_gemm(q, GEMM_BWD_DATA);
+        GemmF32 g = make_gemm(q, GEMM_BWD_DATA);
+        const size_t n = (size_t)g.P * g.Q;
+        int splits = pass_splits(&g);
+        if (splits > 1 && (!workspace || workspace_bytes < (size_t)splits * n * sizeof(float))) {
+            splits = 1;
+            g.kchunk = round_up(g.K, GK);
+        }
+        float* dst = splits > 1 ? (float*)workspace : diff_x;
         if (g.Q <= 64)
-            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 64>), dim3((g.P + GT - 1) / GT, 1, 1), dim3(256), 0, (hipStream_t)stream,
-                               g, diff_y, w, (const float*)nullptr, beta, diff_x);
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 64>), dim3((g.P + GT - 1) / GT, 1, splits), dim3(256), 0, (hipStream_t)stream,
+                               g, diff_y, w, (const float*)nullptr, beta, dst);
         else
-            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, 1), dim3(256), 0,
-                               (hipStream_t)stream, g, diff_y, w, (const float*)nullptr, beta, diff_x);
+            hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_DATA, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
+                               (hipStream_t)stream, g, diff_y, w, (const float*)nullptr, beta, dst);
+        if (splits > 1)
+            hipLaunchKernelGGL(conv_f32_reduce_partials_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, splits, n,
+                               beta, diff_x, (const float*)nullptr, 1, 1);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }
@@ -353,7 +384,14 @@ size_t n2d2hip_conv2d_f32_workspace_bytes(const n2d2hip_conv_desc* desc, int B, 
     if (make_conv(desc, B, H, W, true, &q, "n2d2hip_conv2d_f32_workspace_bytes") != N2D2HIP_OK || !use_gemm(q) || !fits_int(q))
         return 0;
     GemmF32 g = make_gemm(q, GEMM_BWD_FILTER);
-    return (size_t)filter_splits(&g) * g.Q * g.P * sizeof(float);
+    size_t need = (size_t)filter_splits(&g) * g.Q * g.P;
+    for (int mode : {GEMM_FWD, GEMM_BWD_DATA}) {
+        g = make_gemm(q, mode);
+        const int splits = pass_splits(&g);
+        if (splits > 1)
+            need = std::max(need, (size_t)splits * g.Q * g.P);
+    }
+    return need * sizeof(float);
 }
 
 int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int H, int W, const float* x, const float* diff_y, float beta,
@@ -379,7 +417,7 @@ int n2d2hip_conv2d_f32_backward_filter(const n2d2hip_conv_desc* desc, int B, int
             hipLaunchKernelGGL((conv_f32_gemm_kernel<GEMM_BWD_FILTER, 128>), dim3((g.P + GT - 1) / GT, (g.Q + GT - 1) / GT, splits), dim3(256), 0,
                                (hipStream_t)stream, g, x, diff_y, (const float*)nullptr, 0.0f, (float*)workspace);
         hipLaunchKernelGGL(conv_f32_reduce_partials_kernel, dim3(grid_for(nw)), dim3(256), 0, (hipStream_t)stream, (const float*)workspace, splits, nw,
-                           beta, diff_w);
+                           beta, diff_w, (const float*)nullptr, 1, 1);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
     }

@@ -18,7 +18,8 @@ CASES = [  # B, C, H, W, O, k, stride, pad, groups
     (2, 3, 7, 6, 4, 3, 1, 1, 1), (2, 4, 9, 9, 4, 3, 2, 1, 4), (1, 2, 5, 5, 3, 1, 1, 0, 1), (2, 3, 10, 9, 2, 5, 2, 2, 1),
     (2, 1, 5, 5, 1, 3, 1, 0, 1), (3, 5, 8, 8, 5, 3, 1, 1, 5), (1, 3, 9, 7, 2, 3, 3, 0, 1), (2, 2, 4, 4, 3, 2, 2, 0, 1),
     (4, 16, 14, 14, 32, 3, 1, 1, 1), (2, 32, 12, 12, 32, 3, 2, 1, 32), (3, 24, 10, 10, 8, 1, 1, 0, 1), (2, 8, 17, 13, 16, 7, 2, 3, 1),
-    (5, 70, 19, 23, 150, 3, 1, 1, 1), (3, 130, 15, 15, 129, 3, 2, 0, 1), (9, 40, 30, 30, 200, 1, 1, 0, 1), (2, 3, 40, 40, 20, 5, 1, 2, 1)]
+    (5, 70, 19, 23, 150, 3, 1, 1, 1), (3, 130, 15, 15, 129, 3, 2, 0, 1), (9, 40, 30, 30, 200, 1, 1, 0, 1), (2, 3, 40, 40, 20, 5, 1, 2, 1),
+    (6, 96, 7, 7, 160, 3, 1, 1, 1), (4, 200, 9, 9, 70, 3, 1, 1, 1)]     # small outputs, long sums: K ranges in every pass
 
 
 @pytest.fixture(scope="module")
@@ -73,7 +74,11 @@ def test_conv_forward_and_backward(g, case, path):
     d = g.desc(Cn, O, k, s, p, groups)
     dx_, dw_, db_ = g.dev(x), g.dev(w), g.dev(bias)
     y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
-    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), db_.data_ptr(), 0.0, y.data_ptr(), g.sp()))
+    need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
+    assert (need > 0) == (path == "gemm" and groups == 1)
+    ws = g.torch_.empty(max(need, 4), dtype=g.torch_.uint8, device="cuda")
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), db_.data_ptr(), 0.0, y.data_ptr(),
+                                             ws.data_ptr(), need, g.sp()))
     got = g.host(y)
     x64, w64 = x.astype(np.float64), w.astype(np.float64)
     want64 = orc.conv_forward(x64, w64, **kw) + bias.astype(np.float64).reshape(1, -1, 1, 1)
@@ -81,7 +86,8 @@ def test_conv_forward_and_backward(g, case, path):
     assert got.shape == want.shape
     assert _rel(got, want) <= TOL if exact_order else _rel(got, want64, magy) <= TOL
     # beta accumulates onto what the output held (second input tensor of a cell)
-    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), None, 1.0, y.data_ptr(), g.sp()))
+    # (without a workspace: one K range, same result up to the order of the sums)
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), None, 1.0, y.data_ptr(), None, 0, g.sp()))
     want2 = orc.conv_forward(x, w, out=want.copy(), beta=1.0, **kw)
     assert _rel(g.host(y), want2) <= TOL if exact_order else _rel(g.host(y), 2 * want64 - bias.reshape(1, -1, 1, 1), 2 * magy) <= TOL
 
@@ -89,12 +95,12 @@ def test_conv_forward_and_backward(g, case, path):
     ddy = g.dev(dy)
     wantdx = orc.conv_backward_data(w, dy, x.shape, **kw)
     gdx = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
-    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 0.0, gdx.data_ptr(), g.sp()))
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 0.0, gdx.data_ptr(), ws.data_ptr(), need, g.sp()))
     dy64 = dy.astype(np.float64)
     wantdx64 = orc.conv_backward_data(w64, dy64, x.shape, **kw)
     magdx = np.maximum(orc.conv_backward_data(np.abs(w64), np.abs(dy64), x.shape, **kw), 1e-3)
     assert _rel(g.host(gdx), wantdx) <= TOL if exact_order else _rel(g.host(gdx), wantdx64, magdx) <= TOL
-    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 1.0, gdx.data_ptr(), g.sp()))
+    g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 1.0, gdx.data_ptr(), ws.data_ptr(), need, g.sp()))
     if exact_order:
         assert _rel(g.host(gdx), orc.conv_backward_data(w, dy, x.shape, dx=wantdx.copy(), beta=1.0, **kw)) <= TOL
     else:
@@ -103,12 +109,9 @@ def test_conv_forward_and_backward(g, case, path):
     wantdw = orc.conv_backward_filter(x64, dy64, w.shape, **kw)
     mag = orc.conv_backward_filter(np.abs(x64), np.abs(dy64), w.shape, **kw)
     gdw = g.torch_.empty(w.shape, dtype=g.torch_.float32, device="cuda")
-    need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
-    assert (need > 0) == (path == "gemm" and groups == 1)
-    ws = g.torch_.empty(max(need, 4), dtype=g.torch_.uint8, device="cuda")
     if need:
         assert g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 0.0, gdw.data_ptr(),
-                                                        ws.data_ptr(), need - 1, g.sp()) == g.capi.ERR_WORKSPACE
+                                                        ws.data_ptr(), 4, g.sp()) == g.capi.ERR_WORKSPACE
     g.check(g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 0.0, gdw.data_ptr(),
                                                      ws.data_ptr(), need, g.sp()))
     got = g.host(gdw)
@@ -129,12 +132,12 @@ def test_conv_f32_rejects_what_the_reference_cannot_do(g):
     w = g.dev(np.zeros((4, 3, 3, 3)))
     y = g.dev(np.zeros((1, 4, 6, 6)))
     d = g.desc(6, 4, 3, 1, 0, 2)          # two groups of three channels: the reference's backward is not its adjoint
-    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), g.sp()) == g.capi.ERR_UNSUPPORTED
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_UNSUPPORTED
     d = g.desc(6, 4, 3, 1, 0, 1, dil=2)    # backward with dilation: the reference does not read it
-    assert g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), 1, 8, 8, w.data_ptr(), y.data_ptr(), 0.0, x.data_ptr(), g.sp()) == g.capi.ERR_UNSUPPORTED
+    assert g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), 1, 8, 8, w.data_ptr(), y.data_ptr(), 0.0, x.data_ptr(), None, 0, g.sp()) == g.capi.ERR_UNSUPPORTED
     assert b"dilation" in g.lib.n2d2hip_last_error()
     d = g.desc(6, 4, 3, 1, 0, 1)
-    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, None, w.data_ptr(), None, 0.0, y.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, None, w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
 
 
 def test_dilated_forward(g):
@@ -146,7 +149,7 @@ def test_dilated_forward(g):
     d = g.desc(3, 4, 3, 1, 2, 1, dil=2)
     y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
     dx_, dw_ = g.dev(x), g.dev(w)
-    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 2, 11, 11, dx_.data_ptr(), dw_.data_ptr(), None, 0.0, y.data_ptr(), g.sp()))
+    g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 2, 11, 11, dx_.data_ptr(), dw_.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()))
     assert _rel(g.host(y), want) <= TOL
 
 
