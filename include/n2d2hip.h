@@ -247,7 +247,8 @@ int n2d2hip_sat_weight_backward(const float* diff_wq, const float* w, float* dif
 int n2d2hip_sat_act_forward(float* x, float* fp_copy, size_t n, float range, const float* alpha,
                             n2d2hip_stream_t stream);
 /* ref: SATQuantizer_Frame_Kernels.cpp:410-448 + SATQuantizerActivation_Frame.cpp:133-135:
- * diff_alpha[0] = sum_i dalpha_i + beta * diff_alpha[0] */
+ * diff_alpha[0] = sum_i dalpha_i + beta * diff_alpha[0]; diff_in and diff_out may be the same buffer (the cells apply
+ * an activation's backward in place) */
 int n2d2hip_sat_act_backward(const float* diff_in, const float* fp_x, float* diff_out, size_t n, float range,
                              const float* alpha, float beta, float* diff_alpha,
                              void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
@@ -306,7 +307,8 @@ int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, fl
 /* Softmax over the channels of each pixel, one group (ref: src/Cell/SoftmaxCell_Frame.cpp:93-137). */
 int n2d2hip_softmax_f32_forward(const float* x, float* y, int B, int C, int H, int W, n2d2hip_stream_t stream);
 /* diff = target - output, formed in double; loss[0] (device double) = sum of squares / batch
- * (ref: Cell_Frame_Top::applyLoss, src/Cell/Cell_Frame_Top.cpp:27-40). */
+ * (ref: Cell_Frame_Top::applyLoss, src/Cell/Cell_Frame_Top.cpp:27-40); target and diff may be the same buffer, as they
+ * are in the reference. */
 size_t n2d2hip_loss_workspace_bytes(size_t n);
 int n2d2hip_loss_f32(const float* target, const float* output, float* diff, size_t n, int batch, double* loss,
                      void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);

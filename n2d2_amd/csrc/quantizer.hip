@@ -198,8 +198,8 @@ __global__ __launch_bounds__(QBLOCK) void sat_act_forward_kernel(float* __restri
 }
 
 // ref: SATQuantizer_Frame_Kernels.cpp:410-448; the alpha-gradient terms are summed instead of stored
-__global__ __launch_bounds__(QBLOCK) void sat_act_backward_kernel(const float* __restrict__ dy, const float* __restrict__ fp,
-                                                                  float* __restrict__ dx, size_t n, float range,
+__global__ __launch_bounds__(QBLOCK) void sat_act_backward_kernel(const float* dy, const float* __restrict__ fp,
+                                                                  float* dx, size_t n, float range,
                                                                   const float* __restrict__ alpha, double* __restrict__ partial)
 {
     const float a = fabsf(alpha[0]);
@@ -247,8 +247,8 @@ __global__ __launch_bounds__(QBLOCK) void lsq_forward_kernel(const float* __rest
     }
 }
 // ref: LSQQuantizerCell_Frame.cpp:234-303, LSQQuantizerActivation_Frame.cpp:193-262
-__global__ __launch_bounds__(QBLOCK) void lsq_backward_kernel(const float* __restrict__ dq, const float* __restrict__ fp,
-                                                              float* __restrict__ dfp, size_t n, const float* __restrict__ step,
+__global__ __launch_bounds__(QBLOCK) void lsq_backward_kernel(const float* dq, const float* __restrict__ fp,
+                                                              float* dfp, size_t n, const float* __restrict__ step,
                                                               int lo, int hi, double* __restrict__ partial)
 {
     const float s = step[0];

@@ -166,7 +166,7 @@ __global__ __launch_bounds__(TBLOCK) void softmax_f32_kernel(const float* __rest
 }
 
 // diff = target - output, formed in double; partial[block] = sum of squares (double).
-__global__ __launch_bounds__(TBLOCK) void loss_f32_kernel(const float* __restrict__ target, const float* __restrict__ out, float* __restrict__ diff,
+__global__ __launch_bounds__(TBLOCK) void loss_f32_kernel(const float* target, const float* __restrict__ out, float* diff,
                                                           size_t n, double* __restrict__ partial)
 {
     double acc = 0.0;
@@ -214,8 +214,8 @@ __global__ __launch_bounds__(TBLOCK) void rectifier_f32_forward_kernel(float* __
     }
 }
 // diff_out = diff_in * (out == clipping ? 0 : out > 0 ? 1 : leak); `out` is what the cell holds after its activation.
-__global__ __launch_bounds__(TBLOCK) void rectifier_f32_backward_kernel(const float* __restrict__ out, const float* __restrict__ diff_in,
-                                                                        float* __restrict__ diff_out, size_t n, float leak, float clipping)
+__global__ __launch_bounds__(TBLOCK) void rectifier_f32_backward_kernel(const float* __restrict__ out, const float* diff_in,
+                                                                        float* diff_out, size_t n, float leak, float clipping)
 {
     for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < n; i += (size_t)gridDim.x * TBLOCK) {
         const float o = out[i];
