@@ -275,12 +275,12 @@ static GemmF32 make_gemm(const ConvF32& q, int mode)
     return g;
 }
 
-// K ranges of backward-filter: enough blocks to fill the chip, each range at least 8 steps long
+// K ranges of backward-filter: enough blocks to fill the chip, each range at least 32 steps long
 static int filter_splits(GemmF32* g)
 {
     const long tiles = (long)((g->P + GT - 1) / GT) * (g->Q <= 64 ? 1 : (g->Q + GT - 1) / GT);
     long splits = std::max(1L, 1024 / tiles);
-    splits = std::min<long>(splits, std::max(1, g->K / (8 * GK)));
+    splits = std::min<long>(splits, std::max(1, g->K / (32 * GK)));
     g->kchunk = round_up((int)((g->K + splits - 1) / splits), GK);
     return (g->K + g->kchunk - 1) / g->kchunk;
 }
