@@ -140,6 +140,44 @@ def test_conv_f32_rejects_what_the_reference_cannot_do(g):
     assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 8, 8, None, w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
 
 
+def test_conv_f32_edge_shapes(g, path):
+    """One pixel, one channel, batch 1; a kernel as large as the padded input (the FcCell case); a stride larger than
+    the kernel; and shapes that leave no output."""
+    from oracle import oracle as orc
+    rng = np.random.default_rng(17)
+    for (B, Cn, H, W, O, k, s, p) in [(1, 1, 1, 1, 1, 1, 1, 0), (3, 5, 4, 4, 7, 4, 1, 0), (2, 3, 6, 6, 4, 8, 1, 1), (2, 2, 11, 11, 3, 2, 4, 0)]:
+        x = rng.normal(size=(B, Cn, H, W)).astype(np.float32)
+        w = rng.normal(size=(O, Cn, k, k)).astype(np.float32)
+        kw = dict(stride=(s, s), pad=(p, p, p, p))
+        want = orc.conv_forward(x.astype(np.float64), w.astype(np.float64), **kw)
+        mag = np.maximum(orc.conv_forward(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), **kw), 1e-3)
+        d = g.desc(Cn, O, k, s, p, 1)
+        dx_, dw_ = g.dev(x), g.dev(w)
+        y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
+        need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
+        ws = g.torch_.empty(max(need, 4), dtype=g.torch_.uint8, device="cuda")
+        g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), None, 0.0, y.data_ptr(), ws.data_ptr(), need, g.sp()))
+        assert _rel(g.host(y), want, mag) <= TOL, (B, Cn, H, W, O, k, s, p)
+        dy = rng.normal(size=want.shape).astype(np.float32)
+        ddy = g.dev(dy)
+        gdx = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
+        gdw = g.torch_.empty(w.shape, dtype=g.torch_.float32, device="cuda")
+        g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 0.0, gdx.data_ptr(), ws.data_ptr(), need, g.sp()))
+        g.check(g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 0.0, gdw.data_ptr(), ws.data_ptr(), need, g.sp()))
+        x64, w64, dy64 = x.astype(np.float64), w.astype(np.float64), dy.astype(np.float64)
+        assert _rel(g.host(gdx), orc.conv_backward_data(w64, dy64, x.shape, **kw),
+                    np.maximum(orc.conv_backward_data(np.abs(w64), np.abs(dy64), x.shape, **kw), 1e-3)) <= TOL
+        assert _rel(g.host(gdw), orc.conv_backward_filter(x64, dy64, w.shape, **kw),
+                    np.maximum(orc.conv_backward_filter(np.abs(x64), np.abs(dy64), w.shape, **kw), 1e-3)) <= TOL
+    x, w, y = g.dev(np.zeros((1, 2, 3, 3))), g.dev(np.zeros((2, 2, 5, 5))), g.dev(np.zeros(8))
+    d = g.desc(2, 2, 5, 1, 0, 1)           # 5x5 kernel on an unpadded 3x3 input: no output pixel
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 3, 3, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
+    d = g.desc(2, 2, 3, 0, 0, 1)           # stride 0
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 1, 3, 3, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
+    d = g.desc(2, 2, 3, 1, 0, 1)
+    assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 0, 3, 3, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
+
+
 def test_dilated_forward(g):
     from oracle import oracle as orc
     rng = np.random.default_rng(3)
