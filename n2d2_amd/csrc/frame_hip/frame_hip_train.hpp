@@ -64,7 +64,6 @@ public:
     double applyLoss();
     bool isCuda() const { return false; }
     std::string getPyModel() const { return "Frame_HIP_QAT"; }
-    void setStream(void* stream) { mStream = stream; }
 
 protected:
     Cell_FrameTrain_HIP() : mIn(nullptr), mDiffOut(nullptr), mStream(nullptr), mLoss(nullptr), mLossWorkspace(nullptr), mLossWorkspaceBytes(0) {}
@@ -78,7 +77,7 @@ protected:
     DeviceFloats* mIn;
     DeviceFloats* mDiffOut;
     DeviceFloats mOutputs, mDiffInputs;
-    void* mStream;
+    void* mStream;                  // the default stream: the quantizers attached to a cell launch there too
 
 private:
     double* mLoss;
