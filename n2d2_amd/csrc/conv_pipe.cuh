@@ -727,48 +727,87 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     };
 
-    // ---- fill the ring: the first S steps occupy all S stages
 #ifdef N2D2HIP_PROFILE
     pr_t1 = clock64();
 #endif
+    // ---- per-block constants: bias and rescale tables of the channel tile.  Their loads are issued first and their
+    // values stored to LDS behind the ring fill, so that the wait for them (loads return in order) does not include
+    // the ring's own loads.
+    static_assert(BN <= NT, "one table entry per thread");
+    int tv[19];
+    const bool tload = tid < BN;
+    {
+        const int i = tload ? tid : 0;
+#pragma unroll
+        for (int k = 0; k < 19; ++k) tv[k] = 0;
+        if (tload) {
+            if (!p16)
+                tv[0] = BIAS_REG ? p.bias[n0 + i] : 0;
+            if (EPI != EPI_RAW) {
+                if (!p16)
+                    tv[1] = p.epi.a[n0 + i];
+                tv[2] = p.epi.b[n0 + i];
+                tv[3] = p.epi.c[n0 + i];
+                tv[4] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
+                tv[5] = (EPI != EPI_F32) ? p.epi.e[n0 + i] : 0;
+            }
+            if (RES) {
+                tv[6] = q.sum.a[n0 + i];
+                tv[7] = q.sum.b[n0 + i];
+                tv[8] = q.sum.c[n0 + i];
+                tv[9] = q.sum.d[n0 + i];
+                tv[10] = q.sum.e[n0 + i];
+                if (p16 && i < BN / 2) {
+                    tv[16] = q.sum16[n0 / 2 + i];
+                    tv[17] = q.sum16[q.sum16_stride + n0 / 2 + i];
+                    tv[18] = q.sum16[2 * q.sum16_stride + n0 / 2 + i];
+                }
+                if (q.has_pre) {
+                    tv[11] = q.pre.a[n0 + i];
+                    tv[12] = q.pre.b[n0 + i];
+                    tv[13] = q.pre.c[n0 + i];
+                    tv[14] = q.pre.d[n0 + i];
+                    tv[15] = q.pre.e[n0 + i];
+                }
+            }
+        }
+    }
+    // ---- fill the ring: the first S steps occupy all S stages
     if (RES)
         issue_res(0);
 #pragma unroll
     for (int s = 0; s < S; ++s)
         issue();
-
-    // ---- per-block constants into LDS while the first loads fly: bias and rescale tables of the channel tile
-    {
+    if (tload) {
         int* tabw = (int*)(smem + TAB_OFF);
-        for (int i = tid; i < BN; i += NT) {
+        const int i = tid;
+        if (!p16)
+            tabw[i] = tv[0];
+        if (EPI != EPI_RAW) {
             if (!p16)
-                tabw[i] = BIAS_REG ? p.bias[n0 + i] : 0;
-            if (EPI != EPI_RAW) {
-                if (!p16)
-                    tabw[BN + i] = p.epi.a[n0 + i];
-                tabw[2 * BN + i] = p.epi.b[n0 + i];
-                tabw[3 * BN + i] = p.epi.c[n0 + i];
-                tabw[4 * BN + i] = (EPI == EPI_I24) ? p.epi.d[n0 + i] : 0;
-                tabw[5 * BN + i] = (EPI != EPI_F32) ? p.epi.e[n0 + i] : 0;
+                tabw[BN + i] = tv[1];
+            tabw[2 * BN + i] = tv[2];
+            tabw[3 * BN + i] = tv[3];
+            tabw[4 * BN + i] = tv[4];
+            tabw[5 * BN + i] = tv[5];
+        }
+        if (RES) {
+            tabw[6 * BN + i] = tv[6];
+            tabw[7 * BN + i] = tv[7];
+            tabw[8 * BN + i] = tv[8];
+            tabw[9 * BN + i] = tv[9];
+            tabw[10 * BN + i] = tv[10];
+            if (p16 && i < BN / 2) {
+                tabw[i] = tv[16];
+                tabw[BN / 2 + i] = tv[17];
+                tabw[BN + i] = tv[18];
             }
-            if (RES) {
-                tabw[6 * BN + i] = q.sum.a[n0 + i];
-                tabw[7 * BN + i] = q.sum.b[n0 + i];
-                tabw[8 * BN + i] = q.sum.c[n0 + i];
-                tabw[9 * BN + i] = q.sum.d[n0 + i];
-                tabw[10 * BN + i] = q.sum.e[n0 + i];
-                if (p16 && i < BN / 2) {
-                    tabw[i] = q.sum16[n0 / 2 + i];
-                    tabw[BN / 2 + i] = q.sum16[q.sum16_stride + n0 / 2 + i];
-                    tabw[BN + i] = q.sum16[2 * q.sum16_stride + n0 / 2 + i];
-                }
-                if (q.has_pre) {
-                    tabw[11 * BN + i] = q.pre.a[n0 + i];
-                    tabw[12 * BN + i] = q.pre.b[n0 + i];
-                    tabw[13 * BN + i] = q.pre.c[n0 + i];
-                    tabw[14 * BN + i] = q.pre.d[n0 + i];
-                    tabw[15 * BN + i] = q.pre.e[n0 + i];
-                }
+            if (q.has_pre) {
+                tabw[11 * BN + i] = tv[11];
+                tabw[12 * BN + i] = tv[12];
+                tabw[13 * BN + i] = tv[13];
+                tabw[14 * BN + i] = tv[14];
+                tabw[15 * BN + i] = tv[15];
             }
         }
     }
