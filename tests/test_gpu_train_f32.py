@@ -178,6 +178,50 @@ def test_conv_f32_edge_shapes(g, path):
     assert g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), 0, 3, 3, x.data_ptr(), w.data_ptr(), None, 0.0, y.data_ptr(), None, 0, g.sp()) == g.capi.ERR_INVALID
 
 
+def test_conv_f32_random_rectangular_shapes(g, path):
+    """Seeded random cases with different kernel extents, strides and the four paddings in x and y."""
+    from oracle import oracle as orc
+    rng = np.random.default_rng(2024)
+    done = 0
+    while done < 16:
+        B, Cn, O = int(rng.integers(1, 5)), int(rng.integers(1, 40)), int(rng.integers(1, 150))
+        H, W = int(rng.integers(3, 24)), int(rng.integers(3, 24))
+        kW, kH = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        sx, sy = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        pl, pt, pr, pb = (int(v) for v in rng.integers(0, 3, size=4))
+        oW, oH = (W + pl + pr - kW) // sx + 1, (H + pt + pb - kH) // sy + 1
+        # the reference's output size uses one padding per axis on both sides; keep to shapes where the two agree, and
+        # to windows that reach the input (the reference's clipped window and zero padding then coincide)
+        if W + pl + pr < kW or H + pt + pb < kH or pl != pr or pt != pb or pl >= kW or pt >= kH:
+            continue
+        done += 1
+        x = rng.normal(size=(B, Cn, H, W)).astype(np.float32)
+        w = rng.normal(size=(O, Cn, kH, kW)).astype(np.float32)
+        kw = dict(stride=(sx, sy), pad=(pl, pt, pr, pb))
+        x64, w64 = x.astype(np.float64), w.astype(np.float64)
+        want = orc.conv_forward(x64, w64, **kw)
+        assert want.shape == (B, O, oH, oW)
+        d = g.capi.ConvDesc(Cn, O, kW, kH, sx, sy, pl, pt, pr, pb, 1, 1, 1, 0)
+        print("random conv", path, (B, Cn, H, W, O, kW, kH, sx, sy, pl, pt), flush=True)
+        dx_, dw_ = g.dev(x), g.dev(w)
+        need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
+        ws = g.torch_.empty(max(need, 4), dtype=g.torch_.uint8, device="cuda")
+        y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
+        g.check(g.lib.n2d2hip_conv2d_f32_forward(C.byref(d), B, H, W, dx_.data_ptr(), dw_.data_ptr(), None, 0.0, y.data_ptr(), ws.data_ptr(), need, g.sp()))
+        assert _rel(g.host(y), want, np.maximum(orc.conv_forward(np.abs(x64), np.abs(w64), **kw), 1e-3)) <= TOL
+        dy = rng.normal(size=want.shape).astype(np.float32)
+        dy64 = dy.astype(np.float64)
+        ddy = g.dev(dy)
+        gdx = g.torch_.empty(x.shape, dtype=g.torch_.float32, device="cuda")
+        gdw = g.torch_.empty(w.shape, dtype=g.torch_.float32, device="cuda")
+        g.check(g.lib.n2d2hip_conv2d_f32_backward_data(C.byref(d), B, H, W, dw_.data_ptr(), ddy.data_ptr(), 0.0, gdx.data_ptr(), ws.data_ptr(), need, g.sp()))
+        g.check(g.lib.n2d2hip_conv2d_f32_backward_filter(C.byref(d), B, H, W, dx_.data_ptr(), ddy.data_ptr(), 0.0, gdw.data_ptr(), ws.data_ptr(), need, g.sp()))
+        assert _rel(g.host(gdx), orc.conv_backward_data(w64, dy64, x.shape, **kw),
+                    np.maximum(orc.conv_backward_data(np.abs(w64), np.abs(dy64), x.shape, **kw), 1e-3)) <= TOL
+        assert _rel(g.host(gdw), orc.conv_backward_filter(x64, dy64, w.shape, **kw),
+                    np.maximum(orc.conv_backward_filter(np.abs(x64), np.abs(dy64), w.shape, **kw), 1e-3)) <= TOL
+
+
 def test_dilated_forward(g):
     from oracle import oracle as orc
     rng = np.random.default_rng(3)
