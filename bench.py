@@ -19,7 +19,7 @@ PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # HBM bytes one conv_pipe_kernel launch of this workload moves on average: rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy), summary under profiles/
-PIPE_TRAFFIC_BYTES_PER_LAUNCH = (41.19 + 23.76) * 1048576
+PIPE_TRAFFIC_BYTES_PER_LAUNCH = (41.15 + 23.76) * 1048576
 
 
 def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
