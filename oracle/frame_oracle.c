@@ -11,6 +11,28 @@
  *
  * Build: make -C oracle   (gcc, -ffp-contract=off so that no a*b+c is fused:
  * the reference is built for baseline x86-64, which has no FMA).
+ *
+ * What pins each function (the tests named are the CPU tests of this
+ * repository; none of them runs reference code):
+ *   conv forward / bias, fc, pool, elemwise, the four rescales, saturate,
+ *   Clip, Rectifier / Linear, getNbGroups, output sizes
+ *       tests/test_oracle_int.py: integer closed forms, the brute-force loop
+ *       and the shape grid of the reference's own ConvCell test, exact
+ *       rational forms of the rescales, exhaustive window sums of the pools.
+ *   SAT / LSQ kernels
+ *       tests/test_oracle_quant.py: the formulas the reference's quantizer
+ *       tests recompute, exact ties, weights exported by N2D2 itself
+ *       (tests/golden/sat_lenet4b).
+ *   conv backward (data, filter, bias), softmax, and with them the SAT / LSQ
+ *   backward kernels and solver updates end to end
+ *       tests/test_oracle_qat_train.py: adjoint identities and the Jacobian
+ *       of the forward, and the reference's PyTorch-derived known-answer
+ *       tests (trained SAT alphas; LSQ step sizes of a conv net and an FC).
+ * Parity unpinned, by nature: the ORDER in which float reductions add their
+ * terms where the reference runs them under OpenMP or through
+ * std::accumulate (the restatement adds in element order), and the last bit
+ * of libm's tanh / cosh / exp against the device's.  GPU tests hold such
+ * results to 1e-5 of the sum of the terms' magnitudes.
  */
 #include <math.h>
 #include <stddef.h>

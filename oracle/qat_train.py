@@ -3,6 +3,11 @@ quantization-aware training step runs through: restatement of the reference's
 Frame classes around the kernels of oracle.py, for a sequential net of
 ActivationCell / ConvCell / SoftmaxCell with SAT quantizers and SGD solvers.
 
+Pinned by tests/test_oracle_qat_train.py: closed forms for the solver, softmax and loss, and the reference's own
+known-answer tests (tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp, class_ConvCell_QuantizerLSQ_Frame_CUDA.cpp,
+class_FcCell_QuantizerLSQ_Frame_CUDA.cpp: trained SAT alphas and LSQ step sizes derived from PyTorch by the
+reference's authors), which exercise every class below in the order the reference's learning loop calls them.
+
 Data is float32 as in the `<float>` instantiations; "diff" tensors carry the
 descent direction (target - output at the loss), so a solver *adds*
 rate * diff.  Cited paths are relative to the N2D2 source tree.
