@@ -269,7 +269,10 @@ def main():
     }
     if overlapped is not None:
         result["two_batches_in_flight"] = overlapped
-    result["qat_conv_iteration"] = qat_conv_step(torch)
+    try:
+        result["qat_conv_iteration"] = qat_conv_step(torch)
+    except Exception as e:       # the side figure must not take the headline down with it
+        result["qat_conv_iteration"] = {"error": "%s: %s" % (type(e).__name__, e)}
     if not args.no_cpu_baseline:
         base, exact = cpu_baseline(spec, logits, images)
         result["cpu_baseline"] = base
