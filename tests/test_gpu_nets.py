@@ -101,6 +101,16 @@ def test_resnet50_full_batch_properties():
     assert np.array_equal(logits[:2], want)
     # a second forward over the same buffers reproduces the first
     assert np.array_equal(net.forward().to_numpy()[:, :, 0, 0], logits)
+    # ... and so do twenty more, tensor by tensor on a few layers of each kind, launched back to back and replayed
+    # from a graph (asynchronous LDS traffic and hand-counted waits leave no room for run-to-run differences)
+    watch = ["conv1", "pool1", "conv2.1_3x3", "conv2.3_sum", "conv3.4_sum", "conv4.6_sum", "conv5.3_sum", "pool", "fc"]
+    ref = {n: net.tensors[n].to_numpy() for n in watch}
+    replay = net.capture()
+    for it in range(20):
+        (net.forward if it % 2 else replay)()
+        if it % 5 == 4:
+            for n in watch:
+                assert np.array_equal(net.tensors[n].to_numpy(), ref[n]), (it, n)
 
 
 def test_two_forwards_on_two_streams_agree_with_sequential_runs():
