@@ -41,6 +41,26 @@ def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
             "sample": "%d images of the same ResNet-50 forward (batch %d, 224x224), oracle/frame_oracle.c with OpenMP" % (n, n)}, exact
 
 
+def other_configs_bit_exact():
+    """Part of the CPU-baseline leg: the other four configurations at sizes the oracle finishes in seconds (the first
+    two at their full size), GPU logits against the CPU oracle, one flag per configuration."""
+    import numpy as np
+    from n2d2_amd import nets
+    from oracle import cells
+    flags = {}
+    rng = np.random.default_rng(77)
+    for name, make, batch in (("lenet_8bit_bs256", nets.lenet, 256), ("resnet18_stage_conv_bs64", nets.single_conv_stage, 64),
+                              ("mobilenet_v1_8bit", nets.mobilenet_v1, 2), ("resnet18_w4a4", nets.resnet18_w4a4, 2)):
+        spec = make()
+        x = rng.integers(0, 256, size=(batch,) + tuple(spec.in_shape))
+        net = nets.GpuNet(spec, batch)
+        net.set_input(x)
+        got = net.forward().to_numpy().astype(np.int64)
+        want = cells.run_net(spec, x)[spec.output].astype(np.int64)
+        flags[name] = bool(got.shape == want.shape and np.array_equal(got, want))
+    return flags
+
+
 PEAK_FP32_TFLOPS = 157.3
 
 
@@ -277,6 +297,10 @@ def main():
         base, exact = cpu_baseline(spec, logits, images)
         result["cpu_baseline"] = base
         result["bit_exact_vs_cpu"] = exact
+        try:
+            result["other_configs_bit_exact_vs_cpu"] = other_configs_bit_exact()
+        except Exception as e:
+            result["other_configs_bit_exact_vs_cpu"] = {"error": "%s: %s" % (type(e).__name__, e)}
     print(json.dumps(result))
 
 
