@@ -266,6 +266,89 @@ void Cell_Frame_HIP::addInput(HipTensor& stimuli, unsigned int nbChannels, unsig
     setOutputsDims();
 }
 
+void Cell_Frame_HIP::clearInputs()
+{
+    mInputs.clear();
+    mParentCells.clear();
+    mParents.clear();
+    mNbChannels = 0;
+    mInW = mInH = 0;
+}
+
+void Cell_Frame_HIP::replaceInput(HipTensor& oldInputs, HipTensor& newInputs, Cell_Frame_HIP* newParent)
+{
+    unsigned int C, H, W, B;
+    if (newParent) {
+        if (&newParent->mOutputs != &newInputs)
+            throw std::runtime_error("Cell_Frame::replaceInput(): the new input is not the output of the cell given as its producer.");
+        C = newParent->getNbOutputs();
+        H = newParent->getOutputsHeight();
+        W = newParent->getOutputsWidth();
+        B = newParent->batchSize();
+    } else {
+        if (newInputs.empty())
+            throw std::runtime_error("Cell_Frame::replaceInput(): the new input is empty.");
+        const n2d2hip_tensor& d = newInputs.desc();
+        C = (unsigned int)d.C;
+        H = (unsigned int)d.H;
+        W = (unsigned int)d.W;
+        B = (unsigned int)d.B;
+    }
+    size_t pos = mInputs.size();
+    for (size_t i = 0; i < mInputs.size() && pos == mInputs.size(); ++i)
+        if (mInputs[i] == &oldInputs)
+            pos = i;
+    if (pos == mInputs.size())
+        throw std::runtime_error("Cell_Frame::replaceInput(): can't replace input, the input has not been found.");
+    if (mInputs.size() > 1 && (C != mNbChannels || B != mBatch))
+        throw std::runtime_error("Cell_Frame::replaceInput(): can't replace input, the new input does not match the other inputs!");
+    const unsigned int oldC = mNbChannels, oldB = mBatch, oldInW = mInW, oldInH = mInH, oldW = mOutW, oldH = mOutH;
+    mNbChannels = C;
+    mBatch = B;
+    mInW = W;
+    mInH = H;
+    setOutputsDims();
+    if (mInputs.size() > 1 && (mOutW != oldW || mOutH != oldH)) {
+        mNbChannels = oldC;
+        mBatch = oldB;
+        mInW = oldInW;
+        mInH = oldInH;
+        setOutputsDims();
+        throw std::runtime_error("Cell_Frame::replaceInput(): can't replace input, the output dimension has changed and doesn't"
+                                 " match the other inputs!");
+    }
+    mInputs[pos] = &newInputs;
+    mParentCells[pos] = newParent;
+    mParents[pos] = newParent;
+}
+
+void Cell_Frame_HIP::backPropagate()
+{
+    throw std::runtime_error("Cell " + mName + ": the cells of the model \"Frame_HIP\" run quantized inference and have no backPropagate();"
+                             " learn with the model \"Frame_HIP_QAT\"");
+}
+
+void Cell_Frame_HIP::update()
+{
+    throw std::runtime_error("Cell " + mName + ": the cells of the model \"Frame_HIP\" run quantized inference and have no update();"
+                             " learn with the model \"Frame_HIP_QAT\"");
+}
+
+void Cell_Frame_HIP::checkGradient(double /*epsilon*/, double /*maxError*/)
+{
+    throw std::runtime_error("Cell " + mName + ": the cells of the model \"Frame_HIP\" run quantized inference and have no gradient to check");
+}
+
+unsigned int Cell_Frame_HIP::getMaxOutput(unsigned int batchPos)
+{
+    const Tensor<Float_T>& out = getOutputs();
+    if (batchPos >= out.dimB())
+        throw std::runtime_error("Cell " + mName + ": getMaxOutput(): batch position out of range");
+    const size_t n = out.dimX() * out.dimY() * out.dimZ();
+    const Float_T* p = out.data() + (size_t)batchPos * n;
+    return (unsigned int)std::distance(p, std::max_element(p, p + n));
+}
+
 const Tensor<Float_T>& Cell_Frame_HIP::getOutputs()
 {
     if (mFoldedInto)

@@ -378,8 +378,21 @@ public:
     // ... or the environment: an integer-valued tensor of nbChannels x height x width per batch item
     // (Cell::addInput(StimuliProvider&), include/Cell/Cell.hpp:208).
     virtual void addInput(HipTensor& stimuli, unsigned int nbChannels, unsigned int height, unsigned int width, unsigned int batchSize);
+    // Cell_Frame<T>::clearInputs / replaceInput (src/Cell/Cell_Frame.cpp:215-270): graph surgery.  Device tensors are
+    // sized at initialize(), so the new input's dimensions come from the cell that produces it when one is named
+    // (newParent, whose output tensor newInputs must be), else from the tensor, which must then be allocated.
+    void clearInputs();
+    void replaceInput(HipTensor& oldInputs, HipTensor& newInputs, Cell_Frame_HIP* newParent = nullptr);
     virtual void initialize() {}
     virtual void propagate(bool inference = false) = 0;
+    // The integer cells infer only: learning is what the float cells of the model "Frame_HIP_QAT" do.  These three
+    // throw, so that a learning loop handed a Frame_HIP net stops with a message instead of leaving weights untouched.
+    virtual void backPropagate();
+    virtual void update();
+    virtual void checkGradient(double epsilon, double maxError);
+    // Index of the largest output of one batch item, the first one on a tie (Cell_Frame<T>::getMaxOutput,
+    // src/Cell/Cell_Frame.cpp:747-752)
+    unsigned int getMaxOutput(unsigned int batchPos = 0);
     // propagate() in two halves, for a runner that fuses cells: prepare() (re)builds the device handles a parameter
     // change invalidated and tells whether it rebuilt any; launch() enqueues the kernels.
     virtual bool prepare() { return false; }

@@ -284,6 +284,38 @@ int fh_cell_get_outputs(void* net, const char* name, float* out, size_t n)
     });
 }
 
+int fh_cell_get_max_output(void* net, const char* name, unsigned int batchPos, unsigned int* out)
+{
+    return guarded([&] {
+        auto f = std::dynamic_pointer_cast<Cell_Frame_HIP>(((Net*)net)->deepNet->getCell(name));
+        *out = f->getMaxOutput(batchPos);
+    });
+}
+
+// what: 0 backPropagate, 1 update, 2 checkGradient: each throws on the inference cells
+int fh_cell_learn_step(void* net, const char* name, int what)
+{
+    return guarded([&] {
+        auto f = std::dynamic_pointer_cast<Cell_Frame_HIP>(((Net*)net)->deepNet->getCell(name));
+        if (what == 0) f->backPropagate();
+        else if (what == 1) f->update();
+        else f->checkGradient(1.0e-3, 1.0e-3);
+    });
+}
+
+// Rewires `name` from the output of `oldParent` to that of `newParent` (Cell_Frame<T>::replaceInput); oldParent may
+// name a cell that is not an input of `name`, which is the error case.
+int fh_cell_replace_input(void* net, const char* name, const char* oldParent, const char* newParent)
+{
+    return guarded([&] {
+        auto dn = ((Net*)net)->deepNet;
+        auto f = std::dynamic_pointer_cast<Cell_Frame_HIP>(dn->getCell(name));
+        auto o = std::dynamic_pointer_cast<Cell_Frame_HIP>(dn->getCell(oldParent));
+        auto n = std::dynamic_pointer_cast<Cell_Frame_HIP>(dn->getCell(newParent));
+        f->replaceInput(o->getDeviceOutputs(), n->getDeviceOutputs(), n.get());
+    });
+}
+
 // ---- quantizers, each created through the Registrar under the given model key.  Host buffers in and out.
 int fh_sat_cell_run(const char* model, const float* w, const float* diffQ, size_t n, size_t outputsSize, int range, int quantMode,
                     int applyQuantization, int applyScaling, float* wq, float* diffW, float* stats)

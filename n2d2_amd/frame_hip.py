@@ -28,6 +28,9 @@ lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size
 lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
 lib.fh_cell_set_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
 lib.fh_cell_get_outputs.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+lib.fh_cell_get_max_output.argtypes = [C.c_void_p, C.c_char_p, C.c_uint, C.c_void_p]
+lib.fh_cell_learn_step.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+lib.fh_cell_replace_input.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_char_p]
 lib.fh_registrar_exists.argtypes = [C.c_char_p, C.c_char_p]
 lib.fh_registrar_unknown_key_is_null.argtypes = [C.c_char_p]
 lib.fh_set_globals.argtypes = [C.c_int, C.c_int, C.c_int]
@@ -194,6 +197,28 @@ class Net:
 
     def propagate(self):
         _check(lib.fh_net_propagate(self.h))
+
+    def max_output(self, name, batch_pos=0):
+        """Cell_Frame<T>::getMaxOutput: index of the largest output of one batch item, the first on a tie."""
+        v = C.c_uint(0)
+        _check(lib.fh_cell_get_max_output(self.h, name.encode(), batch_pos, C.byref(v)))
+        return v.value
+
+    def back_propagate(self, name):
+        """Raises: the integer cells have no learning pass."""
+        _check(lib.fh_cell_learn_step(self.h, name.encode(), 0))
+
+    def update(self, name):
+        """Raises: the integer cells have no learning pass."""
+        _check(lib.fh_cell_learn_step(self.h, name.encode(), 1))
+
+    def check_gradient(self, name):
+        """Raises: the integer cells have no gradient."""
+        _check(lib.fh_cell_learn_step(self.h, name.encode(), 2))
+
+    def replace_input(self, name, old_parent, new_parent):
+        """Cell_Frame<T>::replaceInput: `name` reads the output of `new_parent` where it read that of `old_parent`."""
+        _check(lib.fh_cell_replace_input(self.h, name.encode(), old_parent.encode(), new_parent.encode()))
 
     def outputs(self, name):
         """Outputs of a cell as N2D2 exposes them: float32 [B, C, H, W] holding integer values."""

@@ -265,3 +265,30 @@ def test_float_rescales_become_integer_scalings_as_in_the_reference(fh):
     # an activation without a floating-point scaling is refused
     with pytest.raises(fh.FrameHipError):
         net.approximate_activation_scaling("conv2", "SingleShift")
+
+
+def test_the_inference_cells_refuse_a_learning_pass(fh):
+    net = fh.Net(INI % "Frame_HIP")
+    for call in (net.back_propagate, net.update, net.check_gradient):
+        with pytest.raises(fh.FrameHipError) as e:
+            call("conv1")
+        assert "conv1" in str(e.value) and "quantized inference" in str(e.value)
+    with pytest.raises(fh.FrameHipError) as e:
+        net.back_propagate("sum")
+    assert "Frame_HIP_QAT" in str(e.value)
+
+
+def test_replace_input_rewires_a_cell_as_cell_frame_does(fh):
+    net = fh.Net(INI % "Frame_HIP")
+    before = net.cell_info("b_x4")
+    net.replace_input("b_x4", "b_1x1", "pool1")            # same 16 x 7 x 7 tensor from another producer
+    assert net.cell_info("b_x4") == before
+    with pytest.raises(fh.FrameHipError) as e:              # b_x4 no longer reads b_1x1: the reference's message
+        net.replace_input("b_x4", "b_1x1", "pool1")
+    assert "can't replace input, the input has not been found." in str(e.value)
+    with pytest.raises(fh.FrameHipError) as e:              # one input of a sum may not change the output's size
+        net.replace_input("sum", "rescale", "conv1")
+    assert "the output dimension has changed and doesn't match the other inputs!" in str(e.value)
+    assert net.cell_info("sum")["W"] == 7                   # and the failed call leaves the cell as it was
+    net.replace_input("dw", "sum", "conv1")                 # a single-input cell follows its new input's size
+    assert (net.cell_info("dw")["W"], net.cell_info("dw")["H"]) == (16, 16)

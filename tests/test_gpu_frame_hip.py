@@ -249,3 +249,43 @@ def test_float_rescaled_net_runs_after_approximation(fh, tmp_path):
     want = cells.run_net(spec, x, keep=keep)
     for name in keep:
         assert np.array_equal(net.outputs(name), want[name]), name
+
+
+def test_get_max_output_is_the_first_largest_output(fh):
+    from n2d2_amd import nets
+    from oracle import cells
+    spec = nets.lenet()
+    x = np.random.default_rng(41).integers(0, 256, size=(8, 1, 32, 32))
+    net = fh.build_net(spec, 8)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    last = spec.output
+    want = cells.run_net(spec, x, keep=[last, "conv1"])
+    for b in range(8):
+        assert net.max_output(last, b) == int(np.argmax(want[last][b].reshape(-1)))
+        # a saturating feature map has many equal maxima: the first one in (channel, row, column) order counts
+        assert net.max_output("conv1", b) == int(np.argmax(want["conv1"][b].reshape(-1)))
+    with pytest.raises(fh.FrameHipError):
+        net.max_output(last, 8)
+
+
+def test_replace_input_before_initialize_changes_what_a_cell_reads(fh):
+    from n2d2_amd import nets
+    from oracle import cells
+    b = nets._Builder("rewired", (16, 14, 14), seed=43, scaling_mode="SingleShift")
+    b.conv("a", "input", 16, 1)
+    b.conv("b", "a", 16, 1)
+    b.conv("c", "b", 16, 3, pad=1)
+    spec = b.spec
+    x = np.random.default_rng(44).integers(0, 256, size=(4, 16, 14, 14))
+    net = fh.build_net(spec, 4)
+    net.replace_input("c", "b", "a")
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    straight = cells.run_net(spec, x, keep=["c"])["c"]
+    spec.layers[2].inputs = ["a"]
+    rewired = cells.run_net(spec, x, keep=["c"])["c"]
+    assert not np.array_equal(straight, rewired)
+    assert np.array_equal(net.outputs("c"), rewired)
