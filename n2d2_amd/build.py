@@ -50,7 +50,8 @@ def build(verbose=False):
     glue = os.path.join(CSRC, "frame_hip")
     outs.append(_run([os.environ.get("CXX", "g++"), "-std=c++14", "-O2", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter",
                       "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include"), "-shared",
-                      os.path.join(glue, "frame_hip.cpp"), os.path.join(glue, "quantization.cpp"), os.path.join(glue, "frame_hip_capi.cpp"),
+                      os.path.join(glue, "frame_hip.cpp"), os.path.join(glue, "quantization.cpp"), os.path.join(glue, "qat_fuse.cpp"),
+                      os.path.join(glue, "frame_hip_capi.cpp"),
                       os.path.join(glue, "frame_hip_train.cpp"), os.path.join(glue, "frame_hip_train_capi.cpp"),
                       "-o", GLUE_LIB,
                       "-L" + LIBDIR, "-ln2d2hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]))

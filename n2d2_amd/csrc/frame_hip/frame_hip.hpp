@@ -1021,6 +1021,55 @@ public:
     static void approximateActivationScaling(Cell& cell, Activation& activation, ScalingMode actScalingMode);
 };
 
+// include/ScalingMode.hpp:64-67
+enum class WeightsApprox { NONE, RINTF };
+
+// What the pass below reads from a trained BatchNormCell (BatchNormCell::getScales / getBiases / getMeans / getVariances,
+// its Epsilon) and from the SAT quantizer of that cell's activation (getRange, getAlpha).
+struct BatchNormParameters {
+    std::vector<double> scales, biases, means, variances;
+    double epsilon = 1.0e-5;
+    std::size_t actRange = 0;   // 0: the activation has no SAT quantizer (the pass then declines)
+    double actAlpha = 0.0;
+};
+
+// What it reads from the trained float Conv / Fc cell: the weight quantizer's tensor of the last propagate
+// (ConvCell::getQuantWeight; the weights themselves without a quantizer) in the layout the cell holds weights in,
+// the biases (empty: NoBias), the quantizer's range (0: none), whether its QuantMode is Default, and the divisor the
+// quantizer applied with ApplyScaling (SATQuantizerCell_Frame<T>::getSAT_scaling, 1 otherwise).
+struct QATCellParameters {
+    Tensor<Float_T> quantWeights, biases;
+    std::size_t weightsRange = 0;
+    bool defaultQuantMode = true;
+    double satScaling = 1.0;
+};
+
+// The step that turns a SAT-trained float graph into the integer cells of this library
+// (src/Quantizer/QAT/Optimization/DeepNetQAT.cpp).  The reference rewrites each float cell in place; here the trained
+// values come in as plain data and the integer cell (model "Frame_HIP") that takes their place is filled: integer
+// weights and biases, the number of bits, and an activation Scaling that clips at the activation's alpha and rescales
+// accumulator units to the next cell's levels.  The (range, alpha) pairs are threaded through the calls as
+// DeepNetQAT::fuseQATGraph does: .first describes the cell's input levels and is replaced by the output's on return.
+class DeepNetQAT {
+public:
+    // Conv followed by BatchNorm (:902-1326).  The cell's activation becomes a Rectifier carrying the Scaling.
+    static bool QuantizeAndfuseBatchNormWithConv(std::pair<std::size_t, std::size_t>& rangeConvBN, std::pair<double, double>& alphasConvBN,
+                                                 ConvCell& convCell, const QATCellParameters& trained, const BatchNormParameters& bn,
+                                                 ScalingMode actScalingMode, WeightsApprox wMode = WeightsApprox::NONE,
+                                                 WeightsApprox bMode = WeightsApprox::NONE, WeightsApprox cMode = WeightsApprox::NONE);
+    // Fc (:655-900).  actRange 0: the cell's activation has no quantizer.  The activation is kept and receives a
+    // FLOAT_MULT Scaling.
+    static bool QuantizeFC(std::pair<std::size_t, std::size_t>& rangeOpFc, std::pair<double, double>& alphaOpFC, FcCell& fcCell,
+                           const QATCellParameters& trained, std::size_t actRange, double actAlpha,
+                           WeightsApprox wMode = WeightsApprox::NONE, WeightsApprox bMode = WeightsApprox::NONE,
+                           WeightsApprox cMode = WeightsApprox::NONE);
+    // ElemWise (:521-653, as built with CUDA: the CPU-only build of the reference sets the number of bits and nothing
+    // else).  The activation becomes a Rectifier with a clipped FLOAT_MULT Scaling.
+    static bool QuantizeElemWise(std::pair<std::size_t, std::size_t>& rangeElWise, std::pair<double, double>& alphaElWise,
+                                 std::size_t rangeParent0, double alphaParent0, ElemWiseCell& elemWiseCell, std::size_t actRange,
+                                 double actAlpha);
+};
+
 // Builds a DeepNet from the subset of N2D2's INI format the quantized path needs
 // (DefaultModel, [env]/[sp] sizes, Conv / Fc / Pool / ElemWise / Scaling sections with Input=,
 // KernelDims / KernelWidth / KernelHeight, NbOutputs, Stride, Padding, Dilation, PoolDims, Pooling, Operation,

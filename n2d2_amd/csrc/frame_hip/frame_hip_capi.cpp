@@ -191,6 +191,121 @@ int fh_cell_set_scaling(void* net, const char* name, int mode, const void* scali
     });
 }
 
+// Clipping of the cell's activation Scaling: *isClipped, and the per-output values when out has room for them
+int fh_cell_get_clipping(void* net, const char* name, int* isClipped, float* out, size_t capacity, size_t* n)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        if (!c->getActivation()) throw std::runtime_error("fh_cell_get_clipping(): cell has no activation");
+        const Scaling& s = c->getActivation()->getActivationScaling();
+        *isClipped = s.getIsClipped() ? 1 : 0;
+        *n = s.getClippingPerOutput().size();
+        if (out && capacity >= *n) std::copy(s.getClippingPerOutput().begin(), s.getClippingPerOutput().end(), out);
+    });
+}
+
+// Bits of the cell (weights) and of its activation, and the activation's type name
+int fh_cell_get_quantized(void* net, const char* name, int* cellBits, int* activationBits, char* typeOut, int typeLen)
+{
+    return guarded([&] {
+        auto c = ((Net*)net)->deepNet->getCell(name);
+        *cellBits = (int)c->getQuantizedNbBits();
+        *activationBits = c->getActivation() ? (int)c->getActivation()->getQuantizedNbBits() : 0;
+        if (typeOut && typeLen > 0) {
+            std::strncpy(typeOut, c->getActivation() ? c->getActivation()->getType() : "", (size_t)typeLen - 1);
+            typeOut[typeLen - 1] = 0;
+        }
+    });
+}
+
+// ---- SAT-trained float values into the integer cells (qat_fuse.cpp).  ranges / alphas: the two-element (input, output)
+// pairs DeepNetQAT threads through the graph, updated in place.  Rounding modes: 0 NONE, 1 RINTF.
+namespace {
+QATCellParameters trainedOf(const float* quantWeights, std::vector<size_t> dims, const float* biases, size_t nbOutputs, size_t weightsRange,
+                            int defaultMode, double satScaling)
+{
+    QATCellParameters t;
+    t.quantWeights.resize(dims);
+    std::memcpy(t.quantWeights.data(), quantWeights, t.quantWeights.size() * sizeof(float));
+    if (biases) {
+        t.biases.resize({nbOutputs});
+        std::memcpy(t.biases.data(), biases, nbOutputs * sizeof(float));
+    }
+    t.weightsRange = weightsRange;
+    t.defaultQuantMode = defaultMode != 0;
+    t.satScaling = satScaling;
+    return t;
+}
+ScalingMode scalingModeOf(int mode)
+{
+    switch (mode) {
+    case N2D2HIP_SCALING_FLOAT_MULT: return ScalingMode::FLOAT_MULT;
+    case N2D2HIP_SCALING_FIXED_MULT16: return ScalingMode::FIXED_MULT16;
+    case N2D2HIP_SCALING_FIXED_MULT32: return ScalingMode::FIXED_MULT32;
+    case N2D2HIP_SCALING_SINGLE_SHIFT: return ScalingMode::SINGLE_SHIFT;
+    case N2D2HIP_SCALING_DOUBLE_SHIFT: return ScalingMode::DOUBLE_SHIFT;
+    default: return ScalingMode::NONE;
+    }
+}
+WeightsApprox approxOf(int m) { return m ? WeightsApprox::RINTF : WeightsApprox::NONE; }
+}
+
+int fh_qat_fuse_batchnorm_with_conv(void* net, const char* name, size_t* ranges, double* alphas, const float* quantWeights, int kW, int kH,
+                                    int Cg, int O, const float* biases, size_t weightsRange, int defaultMode, const double* bnScales,
+                                    const double* bnBiases, const double* bnMeans, const double* bnVariances, double epsilon, size_t actRange,
+                                    double actAlpha, int actScalingMode, int wMode, int bMode, int cMode, int* fused)
+{
+    return guarded([&] {
+        auto conv = std::dynamic_pointer_cast<ConvCell>(((Net*)net)->deepNet->getCell(name));
+        if (!conv) throw std::runtime_error("fh_qat_fuse_batchnorm_with_conv(): " + std::string(name) + " is not a Conv");
+        const QATCellParameters t = trainedOf(quantWeights, {(size_t)kW, (size_t)kH, (size_t)Cg, (size_t)O}, biases, (size_t)O, weightsRange,
+                                              defaultMode, 1.0);
+        BatchNormParameters bn;
+        bn.scales.assign(bnScales, bnScales + O);
+        bn.biases.assign(bnBiases, bnBiases + O);
+        bn.means.assign(bnMeans, bnMeans + O);
+        bn.variances.assign(bnVariances, bnVariances + O);
+        bn.epsilon = epsilon;
+        bn.actRange = actRange;
+        bn.actAlpha = actAlpha;
+        std::pair<size_t, size_t> r(ranges[0], ranges[1]);
+        std::pair<double, double> a(alphas[0], alphas[1]);
+        *fused = DeepNetQAT::QuantizeAndfuseBatchNormWithConv(r, a, *conv, t, bn, scalingModeOf(actScalingMode), approxOf(wMode), approxOf(bMode),
+                                                              approxOf(cMode)) ? 1 : 0;
+        ranges[0] = r.first; ranges[1] = r.second;
+        alphas[0] = a.first; alphas[1] = a.second;
+    });
+}
+
+int fh_qat_quantize_fc(void* net, const char* name, size_t* ranges, double* alphas, const float* quantWeights, int K, int O, const float* biases,
+                       size_t weightsRange, double satScaling, size_t actRange, double actAlpha, int wMode, int bMode, int cMode)
+{
+    return guarded([&] {
+        auto fc = std::dynamic_pointer_cast<FcCell>(((Net*)net)->deepNet->getCell(name));
+        if (!fc) throw std::runtime_error("fh_qat_quantize_fc(): " + std::string(name) + " is not a Fc");
+        const QATCellParameters t = trainedOf(quantWeights, {(size_t)1, (size_t)1, (size_t)K, (size_t)O}, biases, (size_t)O, weightsRange, 1, satScaling);
+        std::pair<size_t, size_t> r(ranges[0], ranges[1]);
+        std::pair<double, double> a(alphas[0], alphas[1]);
+        DeepNetQAT::QuantizeFC(r, a, *fc, t, actRange, actAlpha, approxOf(wMode), approxOf(bMode), approxOf(cMode));
+        ranges[0] = r.first; ranges[1] = r.second;
+        alphas[0] = a.first; alphas[1] = a.second;
+    });
+}
+
+int fh_qat_quantize_elemwise(void* net, const char* name, size_t* ranges, double* alphas, size_t rangeParent0, double alphaParent0, size_t actRange,
+                             double actAlpha)
+{
+    return guarded([&] {
+        auto ew = std::dynamic_pointer_cast<ElemWiseCell>(((Net*)net)->deepNet->getCell(name));
+        if (!ew) throw std::runtime_error("fh_qat_quantize_elemwise(): " + std::string(name) + " is not an ElemWise");
+        std::pair<size_t, size_t> r(ranges[0], ranges[1]);
+        std::pair<double, double> a(alphas[0], alphas[1]);
+        DeepNetQAT::QuantizeElemWise(r, a, rangeParent0, alphaParent0, *ew, actRange, actAlpha);
+        ranges[0] = r.first; ranges[1] = r.second;
+        alphas[0] = a.first; alphas[1] = a.second;
+    });
+}
+
 // ---- ingestion of a trained / calibrated network (quantization.cpp)
 int fh_cell_import_free_parameters(void* net, const char* name, const char* fileName, int ignoreNotExists)
 {

@@ -31,6 +31,14 @@ lib.fh_cell_get_outputs.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size
 lib.fh_cell_get_max_output.argtypes = [C.c_void_p, C.c_char_p, C.c_uint, C.c_void_p]
 lib.fh_cell_learn_step.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
 lib.fh_cell_replace_input.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p, C.c_char_p]
+lib.fh_cell_get_clipping.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+lib.fh_cell_get_quantized.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
+lib.fh_qat_fuse_batchnorm_with_conv.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double,
+                                                C.c_size_t, C.c_double, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+lib.fh_qat_quantize_fc.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_size_t,
+                                   C.c_double, C.c_size_t, C.c_double, C.c_int, C.c_int, C.c_int]
+lib.fh_qat_quantize_elemwise.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_double, C.c_size_t, C.c_double]
 lib.fh_registrar_exists.argtypes = [C.c_char_p, C.c_char_p]
 lib.fh_registrar_unknown_key_is_null.argtypes = [C.c_char_p]
 lib.fh_set_globals.argtypes = [C.c_int, C.c_int, C.c_int]
@@ -173,6 +181,60 @@ class Net:
         out = np.zeros(n.value, dtype=np.float64)
         _check(lib.fh_cell_get_scaling(self.h, name.encode(), C.byref(mode), C.byref(frac), out.ctypes.data, out.size, C.byref(n)))
         return _MODE_NAME[mode.value], frac.value, out
+
+    def clipping(self, name):
+        """Per-output clipping of the cell's activation scaling, or None when it does not clip."""
+        flag, n = C.c_int(), C.c_size_t()
+        _check(lib.fh_cell_get_clipping(self.h, name.encode(), C.byref(flag), None, 0, C.byref(n)))
+        out = np.zeros(n.value, dtype=np.float32)
+        _check(lib.fh_cell_get_clipping(self.h, name.encode(), C.byref(flag), out.ctypes.data, out.size, C.byref(n)))
+        return out if flag.value else None
+
+    def quantized(self, name):
+        """(bits of the cell, bits of its activation, activation type)."""
+        cb, ab = C.c_int(), C.c_int()
+        buf = C.create_string_buffer(32)
+        _check(lib.fh_cell_get_quantized(self.h, name.encode(), C.byref(cb), C.byref(ab), buf, 32))
+        return cb.value, ab.value, buf.value.decode()
+
+    def fuse_batchnorm_with_conv(self, name, ranges, alphas, quant_weights, biases, weights_range, default_mode, bn_scales, bn_biases,
+                                 bn_means, bn_variances, epsilon, act_range, act_alpha, mode="FloatMult", w_round=True, b_round=True,
+                                 c_round=True):
+        """DeepNetQAT::QuantizeAndfuseBatchNormWithConv into the Conv cell `name`.  quant_weights [O, C/groups, kH, kW];
+        biases None for NoBias; weights_range None without weight quantizer; act_range None when the BatchNorm's activation
+        has no SAT quantizer.  Returns (fused, ranges, alphas) with the pairs as the call leaves them."""
+        w = np.ascontiguousarray(quant_weights, dtype=np.float32)
+        O, Cg, kH, kW = w.shape
+        b = None if biases is None else np.ascontiguousarray(biases, dtype=np.float32)
+        bn = [np.ascontiguousarray(v, dtype=np.float64) for v in (bn_scales, bn_biases, bn_means, bn_variances)]
+        r = (C.c_size_t * 2)(*[int(v) for v in ranges])
+        a = (C.c_double * 2)(*[float(v) for v in alphas])
+        fused = C.c_int()
+        _check(lib.fh_qat_fuse_batchnorm_with_conv(self.h, name.encode(), r, a, w.ctypes.data, kW, kH, Cg, O, None if b is None else b.ctypes.data,
+                                                   int(weights_range or 0), int(bool(default_mode)), bn[0].ctypes.data, bn[1].ctypes.data,
+                                                   bn[2].ctypes.data, bn[3].ctypes.data, float(epsilon), int(act_range or 0), float(act_alpha or 0.0),
+                                                   _MODE[mode], int(w_round), int(b_round), int(c_round), C.byref(fused)))
+        return bool(fused.value), (r[0], r[1]), (a[0], a[1])
+
+    def quantize_fc(self, name, ranges, alphas, quant_weights, biases, weights_range, sat_scaling, act_range, act_alpha, w_round=True,
+                    b_round=True, c_round=True):
+        """DeepNetQAT::QuantizeFC into the Fc cell `name`.  quant_weights [O, K].  Returns (ranges, alphas)."""
+        w = np.ascontiguousarray(quant_weights, dtype=np.float32)
+        O, K = w.shape
+        b = None if biases is None else np.ascontiguousarray(biases, dtype=np.float32)
+        r = (C.c_size_t * 2)(*[int(v) for v in ranges])
+        a = (C.c_double * 2)(*[float(v) for v in alphas])
+        _check(lib.fh_qat_quantize_fc(self.h, name.encode(), r, a, w.ctypes.data, K, O, None if b is None else b.ctypes.data, int(weights_range or 0),
+                                      float(sat_scaling), int(act_range or 0), float(act_alpha or 0.0), int(w_round), int(b_round), int(c_round)))
+        return (r[0], r[1]), (a[0], a[1])
+
+    def quantize_elemwise(self, name, ranges, alphas, range_parent0, alpha_parent0, act_range, act_alpha):
+        """DeepNetQAT::QuantizeElemWise on the ElemWise cell `name`.  Returns (ranges, alphas)."""
+        r = (C.c_size_t * 2)(*[int(v) for v in ranges])
+        a = (C.c_double * 2)(*[float(v) for v in alphas])
+        _check(lib.fh_qat_quantize_elemwise(self.h, name.encode(), r, a, int(range_parent0), float(alpha_parent0), int(act_range or 0),
+                                            float(act_alpha or 0.0)))
+        return (r[0], r[1]), (a[0], a[1])
 
     def initialize(self):
         _check(lib.fh_net_initialize(self.h))
