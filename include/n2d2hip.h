@@ -304,6 +304,35 @@ int n2d2hip_conv2d_f32_backward_bias(int B, int O, int oH, int oW, const float* 
 int n2d2hip_rectifier_f32_forward(float* x, size_t n, float leak_slope, float clipping, n2d2hip_stream_t stream);
 int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, float* diff_out, size_t n, float leak_slope,
                                    float clipping, n2d2hip_stream_t stream);
+/* Batch normalisation of float NCHW, one input: y = scale[c] * (x - m[c]) / sqrt(v[c] + epsilon) + bias[c].
+ * use_running != 0 (inference) or moving_average_momentum == 0: m, v are the running `mean`, `variance`, which are not
+ * changed.  Otherwise m, v are the batch's mean and biased variance over batch and pixels, written to saved_mean /
+ * saved_variance, and the running ones move towards them: mean = m * momentum + mean * (1 - momentum), variance likewise
+ * with v * n / (n - 1) (ref: BatchNormCell_Frame<T>::propagate, src/Cell/BatchNormCell_Frame.cpp:287-393).  x and y may
+ * be the same buffer. */
+int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, const float* scale, const float* bias,
+                                  float* mean, float* variance, float* saved_mean, float* saved_variance, double epsilon,
+                                  double moving_average_momentum, int use_running, float* y, n2d2hip_stream_t stream);
+/* Its backward, from the x and the saved statistics of the learning pass: diff_scale[c] = sum(diff_y * x_hat) +
+ * beta_scale * diff_scale[c], diff_bias[c] = sum(diff_y) + beta_bias * diff_bias[c], the gradients of the saved mean and
+ * variance ({C} each, always written), and, when diff_x != NULL, diff_x = diff_y * scale / sigma + dVar * 2 (x - m) / n
+ * + dMean / n (ref: BatchNormCell_Frame<T>::backPropagate, src/Cell/BatchNormCell_Frame.cpp:396-506).  diff_y and diff_x
+ * may be the same buffer. */
+int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, const float* scale, const float* saved_mean,
+                                   const float* saved_variance, double epsilon, const float* diff_y, float beta_scale,
+                                   float* diff_scale, float beta_bias, float* diff_bias, float* diff_saved_mean,
+                                   float* diff_saved_variance, float* diff_x, n2d2hip_stream_t stream);
+/* Max pooling of float NCHW, one output per channel; output size as PoolCell computes it, (in + 2 pad - pool + stride) /
+ * stride.  argmax {B,C,oH,oW} receives row * W + column of the first largest element of each window in row-major order,
+ * -1 for a window that lies in the padding (output 0) (ref: PoolCell_Frame_Kernels::forwardMax with its ArgMax tensor,
+ * src/Cell/PoolCell_Frame_Kernels.cpp:102-197). */
+int n2d2hip_pool_max_f32_forward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x,
+                                 int pad_y, const float* x, float* y, int* argmax, n2d2hip_stream_t stream);
+/* diff_x[i] = sum of diff_y over the outputs whose maximum input i was + beta * diff_x[i]
+ * (ref: PoolCell_Frame_Kernels::backwardMax, src/Cell/PoolCell_Frame_Kernels.cpp:295-379). */
+int n2d2hip_pool_max_f32_backward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x,
+                                  int pad_y, const float* diff_y, const int* argmax, float beta, float* diff_x,
+                                  n2d2hip_stream_t stream);
 /* Softmax over the channels of each pixel, one group (ref: src/Cell/SoftmaxCell_Frame.cpp:93-137). */
 int n2d2hip_softmax_f32_forward(const float* x, float* y, int B, int C, int H, int W, n2d2hip_stream_t stream);
 /* diff = target - output, formed in double; loss[0] (device double) = sum of squares / batch

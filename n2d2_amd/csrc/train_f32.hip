@@ -224,6 +224,164 @@ __global__ __launch_bounds__(TBLOCK) void rectifier_f32_backward_kernel(const fl
     }
 }
 
+// Batch statistics of one channel per block: mean, then the mean of the squared deviations (two passes, as the
+// reference), and the running statistics' step towards them (the variance with the factor size / (size - 1)).
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_stats_kernel(int B, int C, int plane, const float* __restrict__ x, float* __restrict__ mean,
+                                                                     float* __restrict__ variance, float* __restrict__ saved_mean,
+                                                                     float* __restrict__ saved_variance, double momentum)
+{
+    const int c = blockIdx.x;
+    const size_t n = (size_t)B * plane;
+    double acc = 0.0;
+    for (size_t i = threadIdx.x; i < n; i += TBLOCK)
+        acc += (double)x[((size_t)(i / plane) * C + c) * plane + i % plane];
+    const float m = (float)(block_sum_d(acc) / (double)n);
+    acc = 0.0;
+    for (size_t i = threadIdx.x; i < n; i += TBLOCK) {
+        const float zeroed = x[((size_t)(i / plane) * C + c) * plane + i % plane] - m;
+        acc += (double)(zeroed * zeroed);
+    }
+    const float v = (float)(block_sum_d(acc) / (double)n);
+    if (threadIdx.x == 0) {
+        saved_mean[c] = m;
+        saved_variance[c] = v;
+        const float unbiased = v * ((float)n / ((float)n - 1.0f));
+        mean[c] = (float)((double)m * momentum + (double)mean[c] * (1.0 - momentum));
+        variance[c] = (float)((double)unbiased * momentum + (double)variance[c] * (1.0 - momentum));
+    }
+}
+
+// y = scale * (x - mean) / sqrt(variance + epsilon) + bias.  eps_in_float: the inference branch of the reference adds
+// the epsilon in float and takes a float square root; the learning branch adds the double and rounds the root.
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_apply_kernel(size_t total, int C, int plane, const float* __restrict__ x,
+                                                                     const float* __restrict__ scale, const float* __restrict__ bias,
+                                                                     const float* __restrict__ mean, const float* __restrict__ variance, double epsilon,
+                                                                     int eps_in_float, float* __restrict__ y)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int c = (int)((i / plane) % C);
+        const float var = eps_in_float ? sqrtf(variance[c] + (float)epsilon) : (float)sqrt((double)variance[c] + epsilon);
+        const float normalized = (x[i] - mean[c]) / var;
+        y[i] = scale[c] * normalized + bias[c];
+    }
+}
+
+// The five sums of BatchNormCell_Frame<T>::backPropagate over one channel, and what follows from them.
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_sums_kernel(int B, int C, int plane, const float* __restrict__ x,
+                                                                             const float* __restrict__ scale, const float* __restrict__ saved_mean,
+                                                                             const float* __restrict__ saved_variance, double epsilon,
+                                                                             const float* __restrict__ dy, float beta_scale, float* __restrict__ diff_scale,
+                                                                             float beta_bias, float* __restrict__ diff_bias,
+                                                                             float* __restrict__ diff_saved_mean, float* __restrict__ diff_saved_variance)
+{
+    const int c = blockIdx.x;
+    const size_t n = (size_t)B * plane;
+    const float m = saved_mean[c], g = scale[c];
+    const float var = (float)sqrt((double)saved_variance[c] + epsilon);
+    double s_scale = 0.0, s_bias = 0.0, s_mean1 = 0.0, s_mean2 = 0.0, s_var = 0.0;
+    for (size_t i = threadIdx.x; i < n; i += TBLOCK) {
+        const size_t idx = ((size_t)(i / plane) * C + c) * plane + i % plane;
+        const float centred = x[idx] - m;
+        const float normalized = centred / var;
+        const float d = dy[idx];
+        const float diff_normalized = d * g;
+        s_scale += (double)(d * normalized);
+        s_bias += (double)d;
+        s_mean1 += (double)diff_normalized;
+        s_mean2 += (double)(float)(-2.0 * (double)centred);
+        s_var += (double)(diff_normalized * centred);
+    }
+    const float sum_scale = (float)block_sum_d(s_scale);
+    const float sum_bias = (float)block_sum_d(s_bias);
+    const float sum_mean1 = (float)block_sum_d(s_mean1);
+    const float sum_mean2 = (float)block_sum_d(s_mean2);
+    const float sum_var = (float)block_sum_d(s_var);
+    if (threadIdx.x == 0) {
+        const float dv = (float)((double)sum_var * (-1.0 / 2.0) * pow((double)saved_variance[c] + epsilon, -3.0 / 2.0));
+        diff_saved_variance[c] = dv;
+        diff_saved_mean[c] = (float)((double)sum_mean1 * (-1.0 / (double)var) + (double)(dv * sum_mean2 / (float)n));
+        diff_scale[c] = sum_scale + (beta_scale != 0.0f ? beta_scale * diff_scale[c] : 0.0f);
+        diff_bias[c] = sum_bias + (beta_bias != 0.0f ? beta_bias * diff_bias[c] : 0.0f);
+    }
+}
+
+// dx = dy * scale / sigma + dVar * 2 (x - mean) / size + dMean / size
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_data_kernel(size_t total, int C, int plane, float size, const float* __restrict__ x,
+                                                                            const float* __restrict__ scale, const float* __restrict__ saved_mean,
+                                                                            const float* __restrict__ saved_variance, double epsilon, const float* dy,
+                                                                            const float* __restrict__ diff_saved_mean,
+                                                                            const float* __restrict__ diff_saved_variance, float* dx)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int c = (int)((i / plane) % C);
+        const float var = (float)sqrt((double)saved_variance[c] + epsilon);
+        const float diff_normalized = dy[i] * scale[c];
+        const double gradient = (double)(diff_normalized / var) + (double)diff_saved_variance[c] * 2.0 * (double)(x[i] - saved_mean[c]) / (double)size
+                                + (double)(diff_saved_mean[c] / size);
+        dx[i] = (float)gradient;
+    }
+}
+
+struct PoolF32 {
+    int B, C, H, W, oH, oW, pw, ph, sx, sy, px, py;
+};
+
+// Max pooling of float NCHW with the unit mapping; argmax keeps iy * W + ix of the first largest element of the
+// window in row-major order (-1: empty window, output 0).
+__global__ __launch_bounds__(TBLOCK) void pool_max_f32_forward_kernel(PoolF32 q, const float* __restrict__ x, float* __restrict__ y, int* __restrict__ argmax)
+{
+    const size_t total = (size_t)q.B * q.C * q.oH * q.oW;
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int ox = (int)(i % q.oW), oy = (int)((i / q.oW) % q.oH);
+        const size_t bc = i / ((size_t)q.oW * q.oH);
+        const float* in = x + bc * (size_t)q.H * q.W;
+        const int x0 = ox * q.sx - q.px, y0 = oy * q.sy - q.py;
+        const int sx_min = max(-x0, 0), sy_min = max(-y0, 0);
+        const int sx_max = min(max(q.W - x0, 0), q.pw), sy_max = min(max(q.H - y0, 0), q.ph);
+        float best = 0.0f;
+        int where = -1;
+        for (int sy = sy_min; sy < sy_max; ++sy)
+            for (int sx = sx_min; sx < sx_max; ++sx) {
+                const float v = in[(size_t)(y0 + sy) * q.W + x0 + sx];
+                if (where < 0 || v > best) {
+                    best = v;
+                    where = (y0 + sy) * q.W + x0 + sx;
+                }
+            }
+        y[i] = best;
+        argmax[i] = where;
+    }
+}
+
+// Every input collects the gradients of the outputs that chose it, in the reference's order (window rows, then columns,
+// from the input's own residue modulo the stride upwards).
+__global__ __launch_bounds__(TBLOCK) void pool_max_f32_backward_kernel(PoolF32 q, const float* __restrict__ dy, const int* __restrict__ argmax, float beta,
+                                                                       float* __restrict__ dx)
+{
+    const size_t total = (size_t)q.B * q.C * q.H * q.W;
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int ix = (int)(i % q.W), iy = (int)((i / q.W) % q.H);
+        const size_t bc = i / ((size_t)q.W * q.H);
+        const int ix_pad = ix + q.px, iy_pad = iy + q.py;
+        const int sx_max = min(q.pw, ix_pad + 1), sy_max = min(q.ph, iy_pad + 1);
+        float acc = 0.0f;
+        for (int sy = iy_pad % q.sy; sy < sy_max; sy += q.sy) {
+            if (iy_pad >= q.sy * q.oH + sy)
+                continue;
+            const int oy = (iy_pad - sy) / q.sy;
+            for (int sx = ix_pad % q.sx; sx < sx_max; sx += q.sx) {
+                if (ix_pad >= q.sx * q.oW + sx)
+                    continue;
+                const int ox = (ix_pad - sx) / q.sx;
+                const size_t o = (bc * q.oH + oy) * q.oW + ox;
+                if (argmax[o] == iy * q.W + ix)
+                    acc += dy[o];
+            }
+        }
+        dx[i] = acc + (beta != 0.0f ? beta * dx[i] : 0.0f);
+    }
+}
+
 static int grid_for(size_t total)
 {
     const size_t blocks = (total + TBLOCK - 1) / TBLOCK;
@@ -456,6 +614,88 @@ int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, fl
     N2D2HIP_REQUIRE(output && diff_in && diff_out && n > 0 && clipping >= 0.0f, N2D2HIP_ERR_INVALID, "n2d2hip_rectifier_f32_backward: bad argument");
     hipLaunchKernelGGL(rectifier_f32_backward_kernel, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, output, diff_in, diff_out, n,
                        leak_slope, clipping);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, const float* scale, const float* bias, float* mean,
+                                  float* variance, float* saved_mean, float* saved_variance, double epsilon, double moving_average_momentum,
+                                  int use_running, float* y, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && bias && mean && variance && y && epsilon > 0.0, N2D2HIP_ERR_INVALID,
+                    "n2d2hip_batchnorm_f32_forward: bad argument");
+    N2D2HIP_REQUIRE((size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: tensor too large");
+    const size_t total = (size_t)B * C * H * W;
+    const bool running = use_running || moving_average_momentum == 0.0;
+    if (!running) {
+        N2D2HIP_REQUIRE(saved_mean && saved_variance, N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: the learning pass needs saved_mean and saved_variance");
+        N2D2HIP_REQUIRE((size_t)B * H * W > 1, N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: batch statistics need more than one value per channel");
+        hipLaunchKernelGGL(batchnorm_f32_stats_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, mean, variance, saved_mean,
+                           saved_variance, moving_average_momentum);
+    }
+    hipLaunchKernelGGL(batchnorm_f32_apply_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W, x, scale, bias,
+                       running ? (const float*)mean : (const float*)saved_mean, running ? (const float*)variance : (const float*)saved_variance, epsilon,
+                       running ? 1 : 0, y);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, const float* scale, const float* saved_mean,
+                                   const float* saved_variance, double epsilon, const float* diff_y, float beta_scale, float* diff_scale,
+                                   float beta_bias, float* diff_bias, float* diff_saved_mean, float* diff_saved_variance, float* diff_x,
+                                   n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && saved_mean && saved_variance && diff_y && diff_scale && diff_bias
+                        && diff_saved_mean && diff_saved_variance && epsilon > 0.0,
+                    N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: bad argument");
+    N2D2HIP_REQUIRE((size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: tensor too large");
+    const size_t total = (size_t)B * C * H * W;
+    hipLaunchKernelGGL(batchnorm_f32_backward_sums_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, scale, saved_mean,
+                       saved_variance, epsilon, diff_y, beta_scale, diff_scale, beta_bias, diff_bias, diff_saved_mean, diff_saved_variance);
+    if (diff_x)
+        hipLaunchKernelGGL(batchnorm_f32_backward_data_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W,
+                           (float)((size_t)B * H * W), x, scale, saved_mean, saved_variance, epsilon, diff_y, (const float*)diff_saved_mean,
+                           (const float*)diff_saved_variance, diff_x);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+static int make_pool(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x, int pad_y, PoolF32* q, const char* who)
+{
+    N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && pool_w > 0 && pool_h > 0 && stride_x > 0 && stride_y > 0 && pad_x >= 0 && pad_y >= 0,
+                    N2D2HIP_ERR_INVALID, "%s: bad argument", who);
+    N2D2HIP_REQUIRE(pad_x < pool_w && pad_y < pool_h, N2D2HIP_ERR_INVALID, "%s: padding must be smaller than the window", who);
+    q->B = B; q->C = C; q->H = H; q->W = W;
+    q->pw = pool_w; q->ph = pool_h; q->sx = stride_x; q->sy = stride_y; q->px = pad_x; q->py = pad_y;
+    // PoolCell::setOutputsDims (src/Cell/PoolCell.cpp:219-240)
+    q->oW = (int)((W + 2 * pad_x - pool_w + stride_x) / (double)stride_x);
+    q->oH = (int)((H + 2 * pad_y - pool_h + stride_y) / (double)stride_y);
+    N2D2HIP_REQUIRE(q->oW > 0 && q->oH > 0, N2D2HIP_ERR_INVALID, "%s: the window does not fit the input", who);
+    N2D2HIP_REQUIRE((size_t)H * W < ((size_t)1 << 31) && (size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "%s: tensor too large", who);
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_pool_max_f32_forward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x, int pad_y,
+                                 const float* x, float* y, int* argmax, n2d2hip_stream_t stream)
+{
+    PoolF32 q;
+    const int rc = make_pool(B, C, H, W, pool_w, pool_h, stride_x, stride_y, pad_x, pad_y, &q, "n2d2hip_pool_max_f32_forward");
+    if (rc != N2D2HIP_OK) return rc;
+    N2D2HIP_REQUIRE(x && y && argmax, N2D2HIP_ERR_INVALID, "n2d2hip_pool_max_f32_forward: null pointer");
+    hipLaunchKernelGGL(pool_max_f32_forward_kernel, dim3(grid_for((size_t)B * C * q.oH * q.oW)), dim3(TBLOCK), 0, (hipStream_t)stream, q, x, y, argmax);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_pool_max_f32_backward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x, int pad_y,
+                                  const float* diff_y, const int* argmax, float beta, float* diff_x, n2d2hip_stream_t stream)
+{
+    PoolF32 q;
+    const int rc = make_pool(B, C, H, W, pool_w, pool_h, stride_x, stride_y, pad_x, pad_y, &q, "n2d2hip_pool_max_f32_backward");
+    if (rc != N2D2HIP_OK) return rc;
+    N2D2HIP_REQUIRE(diff_y && argmax && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_pool_max_f32_backward: null pointer");
+    hipLaunchKernelGGL(pool_max_f32_backward_kernel, dim3(grid_for((size_t)B * C * H * W)), dim3(TBLOCK), 0, (hipStream_t)stream, q, diff_y, argmax, beta,
+                       diff_x);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

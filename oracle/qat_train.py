@@ -1,7 +1,7 @@
 """CPU oracle (TEST INFRASTRUCTURE, not the product) of the float cells a
 quantization-aware training step runs through: restatement of the reference's
 Frame classes around the kernels of oracle.py, for a sequential net of
-ActivationCell / ConvCell / SoftmaxCell with SAT quantizers and SGD solvers.
+ActivationCell / ConvCell / BatchNormCell / PoolCell / SoftmaxCell with SAT quantizers and SGD solvers.
 
 Pinned by tests/test_oracle_qat_train.py: closed forms for the solver, softmax and loss, and the reference's own
 known-answer tests (tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp, class_ConvCell_QuantizerLSQ_Frame_CUDA.cpp,
@@ -223,6 +223,137 @@ class ConvCell:
             self.quantizer.update(batch_size)
         if self.bias is not None:
             self.bias_solver.update(self.bias, self.diff_bias, batch_size)
+        if self.activation:
+            self.activation.update(batch_size)
+
+
+def _seq_sum(v):
+    """Sum of a float32 vector in element order with a float32 accumulator, as a C loop `sum += v[i]` does."""
+    v = np.ascontiguousarray(v, dtype=F).reshape(-1)
+    return F(np.cumsum(v, dtype=F)[-1]) if v.size else F(0.0)
+
+
+class BatchNormCell:
+    """src/Cell/BatchNormCell_Frame.cpp (one input, T = ParamT = float): propagate :287-393 (inference or
+    MovingAverageMomentum 0: the running statistics; else the batch's, in two passes, which also feed the running ones,
+    the variance with the factor size / (size - 1)); backPropagate :396-506; update :509-523 (scale then bias).
+    Sums run over batch, row, column in that order with a float accumulator.  Initial values: scale 1, bias 0, mean 0,
+    variance 0 (:78-121)."""
+
+    def __init__(self, nb_outputs, activation=None, epsilon=1.0e-5, moving_average_momentum=0.1, scale_solver=None,
+                 bias_solver=None, scales=None, biases=None, means=None, variances=None):
+        self.scale = np.ones(nb_outputs, dtype=F) if scales is None else np.array(scales, dtype=F)
+        self.bias = np.zeros(nb_outputs, dtype=F) if biases is None else np.array(biases, dtype=F)
+        self.mean = np.zeros(nb_outputs, dtype=F) if means is None else np.array(means, dtype=F)
+        self.variance = np.zeros(nb_outputs, dtype=F) if variances is None else np.array(variances, dtype=F)
+        self.epsilon, self.momentum = float(epsilon), float(moving_average_momentum)
+        self.activation = activation
+        self.scale_solver, self.bias_solver = scale_solver or SGDSolver(), bias_solver or SGDSolver()
+        self.diff_scale = np.zeros(nb_outputs, dtype=F)
+        self.diff_bias = np.zeros(nb_outputs, dtype=F)
+        self.diff_inputs = None
+
+    def propagate(self, x, inference=False):
+        x = np.ascontiguousarray(x, dtype=F)
+        self.x = x
+        B, Cn, H, W = x.shape
+        size = B * H * W
+        sh = (1, -1, 1, 1)
+        if inference or self.momentum == 0.0:
+            mean, variance = self.mean, self.variance
+        else:
+            self.saved_mean, self.saved_variance = np.empty(Cn, dtype=F), np.empty(Cn, dtype=F)
+            for c in range(Cn):
+                self.saved_mean[c] = F(_seq_sum(x[:, c]) / F(size))
+                zeroed = (x[:, c] - self.saved_mean[c]).astype(F)
+                self.saved_variance[c] = F(_seq_sum((zeroed * zeroed).astype(F)) / F(size))
+                self.mean[c] = F(float(self.saved_mean[c]) * self.momentum + float(self.mean[c]) * (1.0 - self.momentum))
+                self.variance[c] = F(float(F(self.saved_variance[c] * F(F(size) / F(F(size) - F(1))))) * self.momentum
+                                     + float(self.variance[c]) * (1.0 - self.momentum))
+            mean, variance = self.saved_mean, self.saved_variance
+        if inference or self.momentum == 0.0:
+            var = np.sqrt((variance + F(self.epsilon)).astype(F)).astype(F)        # T(variance) + T(epsilon), :308-309
+        else:
+            var = np.sqrt(variance.astype(np.float64) + self.epsilon).astype(F)     # (T) variance + double epsilon, :365
+        normalized = ((x - mean.reshape(sh)) / var.reshape(sh)).astype(F)
+        y = (self.scale.reshape(sh) * normalized + self.bias.reshape(sh)).astype(F)
+        self.outputs = self.activation.propagate(y, inference) if self.activation else y
+        return self.outputs
+
+    def back_propagate(self):
+        d = self.diff_inputs
+        if self.activation:
+            d = self.activation.back_propagate(d)
+        d = np.ascontiguousarray(d, dtype=F)
+        x = self.x
+        B, Cn, H, W = x.shape
+        size = B * H * W
+        beta_scale = F(0.0) if self.scale_solver.is_new_iteration() else F(1.0)
+        beta_bias = F(0.0) if self.bias_solver.is_new_iteration() else F(1.0)
+        dx = np.empty_like(x)
+        for c in range(Cn):
+            mean, variance, scale = self.saved_mean[c], self.saved_variance[c], self.scale[c]
+            var = F(np.sqrt(float(variance) + self.epsilon))
+            centred = (x[:, c] - mean).astype(F)
+            normalized = (centred / var).astype(F)
+            diff_normalized = (d[:, c] * scale).astype(F)
+            sum_scale = _seq_sum((d[:, c] * normalized).astype(F))
+            sum_bias = _seq_sum(d[:, c])
+            sum_mean1 = _seq_sum(diff_normalized)
+            sum_mean2 = _seq_sum((-2.0 * centred.astype(np.float64)).astype(F))
+            sum_variance = _seq_sum((diff_normalized * centred).astype(F))
+            diff_variance = F(float(sum_variance) * (-1.0 / 2.0) * np.power(float(variance) + self.epsilon, -3.0 / 2.0))
+            diff_mean = F(float(sum_mean1) * (-1.0 / float(var)) + float(F(F(diff_variance * sum_mean2) / F(size))))
+            self.diff_scale[c] = F(sum_scale + beta_scale * self.diff_scale[c])
+            self.diff_bias[c] = F(sum_bias + beta_bias * self.diff_bias[c])
+            gradient = ((diff_normalized / var).astype(F).astype(np.float64)
+                        + float(diff_variance) * 2.0 * centred.astype(np.float64) / float(F(size))
+                        + float(F(diff_mean / F(size))))
+            dx[:, c] = gradient.astype(F)
+        return dx
+
+    def update(self, batch_size):
+        self.scale_solver.update(self.scale, self.diff_scale, batch_size)
+        self.bias_solver.update(self.bias, self.diff_bias, batch_size)
+        if self.activation:
+            self.activation.update(batch_size)
+
+
+class PoolCell:
+    """src/Cell/PoolCell_Frame.cpp:123-228 with Pooling=Max, one input and the unit mapping: forwardMax remembers the
+    first largest element of each window (src/Cell/PoolCell_Frame_Kernels.cpp:102-197); backwardMax gives every input
+    the sum of the gradients of the outputs it was the maximum of (:295-379)."""
+
+    def __init__(self, pool, stride, pad=(0, 0), activation=None):
+        self.pool, self.stride, self.pad, self.activation = pool, stride, pad, activation
+        self.diff_inputs = None
+
+    def propagate(self, x, inference=False):
+        self.x_shape = x.shape
+        y, self.argmax = o.pool_forward(np.ascontiguousarray(x, dtype=F), self.pool, self.stride, self.pad, kind="max", quantized=False,
+                                        argmax=True)
+        self.outputs = self.activation.propagate(y, inference) if self.activation else y
+        return self.outputs
+
+    def back_propagate(self):
+        d = self.diff_inputs
+        if self.activation:
+            d = self.activation.back_propagate(d)
+        dx = np.zeros(self.x_shape, dtype=F)
+        B, Cn, oH, oW = d.shape
+        am = self.argmax
+        # output order (oy, ox ascending) is the order in which backwardMax meets the outputs of one input (sy, sx ascending
+        # means oy, ox descending; with at most a few overlapping windows the float sums agree to the last bit or two)
+        for b in range(B):
+            for c in range(Cn):
+                for oy in range(oH):
+                    for ox in range(oW):
+                        ix, iy, ch, valid = am[b, c, oy, ox]
+                        if valid:
+                            dx[b, ch, iy, ix] += d[b, c, oy, ox]
+        return dx
+
+    def update(self, batch_size):
         if self.activation:
             self.activation.update(batch_size)
 

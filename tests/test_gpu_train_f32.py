@@ -289,3 +289,94 @@ def test_rectifier_softmax_loss_sgd(g):
     g.check(g.lib.n2d2hip_sgd_update_f32(dev.data_ptr(), dgrad.data_ptr(), 3, 1.0, 0.0, 0.0, None, 1, -1.0, 1.0, g.sp()))
     assert np.array_equal(g.host(dev), np.array([1.0, -1.0, 1.0], dtype=np.float32))
     assert g.lib.n2d2hip_sgd_update_f32(dev.data_ptr(), dev.data_ptr(), 3, 1.0, 0.9, 0.0, None, 0, 0.0, 0.0, g.sp()) == g.capi.ERR_INVALID
+
+
+@pytest.mark.parametrize("shape", [(6, 5, 7, 4), (2, 3, 1, 1), (16, 64, 14, 14), (3, 1, 33, 17), (300, 2, 3, 3)])
+def test_batchnorm_forward_backward(g, shape):
+    from oracle import qat_train as qt
+    print("batchnorm f32", shape, flush=True)
+    B, Cn, H, W = shape
+    rng = np.random.default_rng(sum(shape))
+    x = rng.normal(1.5, 2.0, size=shape).astype(np.float32)
+    gamma, beta = rng.normal(1, 0.3, size=Cn).astype(np.float32), rng.normal(0, 0.5, size=Cn).astype(np.float32)
+    mean0, var0 = rng.normal(0, 1, size=Cn).astype(np.float32), rng.uniform(0.5, 2, size=Cn).astype(np.float32)
+    cell = qt.BatchNormCell(Cn, scales=gamma, biases=beta, means=mean0, variances=var0)
+    dx_, dg, db = g.dev(x), g.dev(gamma), g.dev(beta)
+    dmean, dvar = g.dev(mean0), g.dev(var0)
+    z = lambda n: g.torch_.zeros(n, dtype=g.torch_.float32, device="cuda")
+    smean, svar, y = z(Cn), z(Cn), z(x.size)
+    fwd = lambda running: g.check(g.lib.n2d2hip_batchnorm_f32_forward(
+        B, Cn, H, W, dx_.data_ptr(), dg.data_ptr(), db.data_ptr(), dmean.data_ptr(), dvar.data_ptr(), smean.data_ptr(), svar.data_ptr(), 1e-5,
+        0.1, running, y.data_ptr(), g.sp()))
+    # inference: the running statistics, untouched
+    fwd(1)
+    want = cell.propagate(x, inference=True)
+    assert _rel(g.host(y).reshape(shape), want) <= TOL
+    assert np.array_equal(g.host(dmean), mean0) and np.array_equal(g.host(dvar), var0)
+    # learning: batch statistics, running ones move a tenth of the way
+    fwd(0)
+    want = cell.propagate(x, inference=False)
+    assert _rel(g.host(y).reshape(shape), want, scale=np.maximum(np.abs(want), 1.0)) <= 2e-5
+    # (a mean is a sum of terms of magnitude ~2: held to 1e-5 of that, not of a result that may cancel to nearly 0)
+    assert _rel(g.host(smean), cell.saved_mean, scale=2.0) <= TOL and _rel(g.host(svar), cell.saved_variance) <= TOL
+    assert _rel(g.host(dmean), cell.mean, scale=2.0) <= TOL and _rel(g.host(dvar), cell.variance) <= TOL
+    # backward, accumulating into the scale gradient (beta 1) and overwriting the bias gradient (beta 0)
+    dy = rng.normal(0, 1, size=shape).astype(np.float32)
+    cell.diff_inputs = dy
+    cell.scale_solver.iteration_pass = 1            # inside an iteration: the oracle adds to diff_scale as well
+    prev = rng.normal(0, 1, size=Cn).astype(np.float32)
+    cell.diff_scale[:] = prev
+    wdx = cell.back_propagate()
+    ddy, dgs, dgb, dsm, dsv = g.dev(dy), g.dev(prev), g.dev(prev), z(Cn), z(Cn)
+    g.check(g.lib.n2d2hip_batchnorm_f32_backward(B, Cn, H, W, dx_.data_ptr(), dg.data_ptr(), smean.data_ptr(), svar.data_ptr(), 1e-5, ddy.data_ptr(),
+                                                 1.0, dgs.data_ptr(), 0.0, dgb.data_ptr(), dsm.data_ptr(), dsv.data_ptr(), ddy.data_ptr(), g.sp()))
+    n = B * H * W
+    terms = np.abs(dy).sum(axis=(0, 2, 3)) * 4 + 1.0                 # magnitude of the sums' terms (x_hat is O(1))
+    assert _rel(g.host(dgs), cell.diff_scale, scale=terms) <= TOL and _rel(g.host(dgb), cell.diff_bias, scale=terms) <= TOL
+    assert _rel(g.host(ddy).reshape(shape), wdx, scale=np.maximum(np.abs(wdx), 1.0) * max(1.0, float(np.abs(gamma).max()))) <= 5e-5
+    assert np.isfinite(g.host(dsm)).all() and np.isfinite(g.host(dsv)).all()
+    # only the parameter gradients
+    ddy2 = g.dev(dy)
+    g.check(g.lib.n2d2hip_batchnorm_f32_backward(B, Cn, H, W, dx_.data_ptr(), dg.data_ptr(), smean.data_ptr(), svar.data_ptr(), 1e-5, ddy2.data_ptr(),
+                                                 0.0, dgs.data_ptr(), 0.0, dgb.data_ptr(), dsm.data_ptr(), dsv.data_ptr(), None, g.sp()))
+    assert _rel(g.host(dgb), cell.diff_bias, scale=terms) <= TOL
+    # rejected: batch statistics of a single value, missing buffers
+    assert g.lib.n2d2hip_batchnorm_f32_forward(1, Cn, 1, 1, dx_.data_ptr(), dg.data_ptr(), db.data_ptr(), dmean.data_ptr(), dvar.data_ptr(),
+                                               smean.data_ptr(), svar.data_ptr(), 1e-5, 0.1, 0, y.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+    assert g.lib.n2d2hip_batchnorm_f32_forward(B, Cn, H, W, dx_.data_ptr(), dg.data_ptr(), db.data_ptr(), dmean.data_ptr(), dvar.data_ptr(), None, None,
+                                               1e-5, 0.1, 0, y.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+
+
+@pytest.mark.parametrize("case", [(2, 3, 9, 8, 2, 2, 2, 2, 0, 0), (2, 3, 9, 8, 3, 3, 2, 2, 0, 0), (2, 3, 9, 8, 3, 3, 2, 2, 1, 1),
+                                  (1, 2, 7, 10, 3, 2, 1, 2, 0, 0), (4, 16, 28, 28, 2, 2, 2, 2, 0, 0), (3, 5, 11, 11, 3, 3, 1, 1, 1, 1),
+                                  (2, 2, 6, 6, 2, 2, 3, 3, 0, 0)])
+def test_max_pooling_forward_backward(g, case):
+    from oracle import qat_train as qt
+    print("pool max f32", case, flush=True)
+    B, Cn, H, W, pw, ph, sx, sy, px, py = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.integers(-4, 5, size=(B, Cn, H, W)).astype(np.float32)          # many ties: the first maximum must win
+    cell = qt.PoolCell((pw, ph), (sx, sy), (px, py))
+    want = cell.propagate(x)
+    oH, oW = want.shape[2:]
+    y = g.torch_.empty(want.size, dtype=g.torch_.float32, device="cuda")
+    am = g.torch_.empty(want.size, dtype=g.torch_.int32, device="cuda")
+    dx_ = g.dev(x)
+    g.check(g.lib.n2d2hip_pool_max_f32_forward(B, Cn, H, W, pw, ph, sx, sy, px, py, dx_.data_ptr(), y.data_ptr(), am.data_ptr(), g.sp()))
+    assert np.array_equal(g.host(y).reshape(want.shape), want)
+    ref_am = np.where(cell.argmax[..., 3] > 0, cell.argmax[..., 1] * W + cell.argmax[..., 0], -1)
+    assert np.array_equal(g.host(am).reshape(want.shape), ref_am)
+    dy = rng.normal(size=want.shape).astype(np.float32)
+    cell.diff_inputs = dy
+    wdx = cell.back_propagate()
+    prev = rng.normal(size=x.shape).astype(np.float32)
+    for beta in (0.0, 1.0):
+        out = g.dev(prev)
+        ddy = g.dev(dy)
+        g.check(g.lib.n2d2hip_pool_max_f32_backward(B, Cn, H, W, pw, ph, sx, sy, px, py, ddy.data_ptr(), am.data_ptr(), beta, out.data_ptr(), g.sp()))
+        assert _rel(g.host(out), wdx + np.float32(beta) * prev, scale=1.0) <= TOL
+    # strides larger than the window leave inputs that no output reads: their gradient is 0
+    if sx > pw:
+        assert (wdx == 0).sum() >= x.size // 3
+    assert g.lib.n2d2hip_pool_max_f32_forward(B, Cn, H, W, 2, 2, 2, 2, 2, 0, dx_.data_ptr(), y.data_ptr(), am.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+    assert g.lib.n2d2hip_pool_max_f32_forward(B, Cn, 1, 1, 3, 3, 1, 1, 0, 0, dx_.data_ptr(), y.data_ptr(), am.data_ptr(), g.sp()) == g.capi.ERR_INVALID

@@ -192,3 +192,105 @@ def test_known_answer_lsq_step_size_fc():
     q.train_sequential(x, cells, q.SoftmaxCell(), t, fc["iterations"])
     print("step", float(quant.step[0]))
     assert abs(float(quant.step[0]) - fc["expected_step"]) < fc["delta"]
+
+
+# ------------------------------------------------------------------ BatchNorm and max pooling of the learning graph
+def _bn_reference(x, gamma, beta, eps):
+    """Textbook batch normalisation in float64: outputs, and the gradients of sum(dy * y) as every framework derives them."""
+    x = x.astype(np.float64)
+    mu = x.mean(axis=(0, 2, 3), keepdims=True)
+    var = x.var(axis=(0, 2, 3), keepdims=True)
+    xhat = (x - mu) / np.sqrt(var + eps)
+    g, b = gamma.astype(np.float64).reshape(1, -1, 1, 1), beta.astype(np.float64).reshape(1, -1, 1, 1)
+
+    def grads(dy):
+        dy = dy.astype(np.float64)
+        dxhat = dy * g
+        dx = (dxhat - dxhat.mean(axis=(0, 2, 3), keepdims=True) - xhat * (dxhat * xhat).mean(axis=(0, 2, 3), keepdims=True)) / np.sqrt(var + eps)
+        return dx, (dy * xhat).sum(axis=(0, 2, 3)), dy.sum(axis=(0, 2, 3))
+    return g * xhat + b, mu.reshape(-1), var.reshape(-1), grads
+
+
+def test_batchnorm_learning_pass_is_textbook_batch_normalisation():
+    from oracle import qat_train as qt
+    rng = np.random.default_rng(21)
+    x = rng.normal(1.5, 2.0, size=(6, 5, 7, 4)).astype(np.float32)
+    gamma, beta = rng.normal(1, 0.3, size=5).astype(np.float32), rng.normal(0, 0.5, size=5).astype(np.float32)
+    bn = qt.BatchNormCell(5, scales=gamma, biases=beta)
+    y = bn.propagate(x, inference=False)
+    want, mu, var, grads = _bn_reference(x, gamma, beta, 1e-5)
+    assert np.allclose(y, want, rtol=0, atol=2e-5)
+    n = 6 * 7 * 4
+    # the running statistics start at 0 and take a tenth of the batch's; the variance with Bessel's factor
+    assert np.allclose(bn.mean, 0.1 * mu, rtol=1e-5) and np.allclose(bn.variance, 0.1 * var * n / (n - 1), rtol=1e-5)
+    dy = rng.normal(0, 1, size=x.shape).astype(np.float32)
+    bn.diff_inputs = dy
+    dx = bn.back_propagate()
+    wdx, wdg, wdb = grads(dy)
+    assert np.allclose(dx, wdx, rtol=0, atol=3e-5 * np.abs(wdx).max())
+    assert np.allclose(bn.diff_scale, wdg, rtol=1e-4, atol=1e-4) and np.allclose(bn.diff_bias, wdb, rtol=1e-5, atol=1e-4)
+    # update adds rate / batch * diff to scale and bias, in that order, each through its own solver
+    bn.update(6)
+    assert np.allclose(bn.scale, gamma + np.float32(0.01 / 6) * bn.diff_scale) and np.allclose(bn.bias, beta + np.float32(0.01 / 6) * bn.diff_bias)
+    # a second propagate moves the running statistics by another tenth of the way
+    m1, v1 = bn.mean.copy(), bn.variance.copy()
+    bn.propagate(x, inference=False)
+    assert np.allclose(bn.mean, 0.9 * m1 + 0.1 * mu, rtol=1e-5) and np.allclose(bn.variance, 0.9 * v1 + 0.1 * var * n / (n - 1), rtol=1e-5)
+
+
+def test_batchnorm_inference_uses_the_running_statistics():
+    from oracle import qat_train as qt, qat_fuse as qf
+    rng = np.random.default_rng(22)
+    x = rng.normal(0, 1, size=(3, 4, 5, 5)).astype(np.float32)
+    p = [rng.normal(1, 0.2, size=4), rng.normal(0, 1, size=4), rng.normal(0, 1, size=4), rng.uniform(0.5, 2, size=4)]
+    bn = qt.BatchNormCell(4, scales=p[0], biases=p[1], means=p[2], variances=p[3])
+    y = bn.propagate(x, inference=True)
+    want = p[0].reshape(1, -1, 1, 1) * (x.astype(np.float64) - p[2].reshape(1, -1, 1, 1)) / np.sqrt(p[3].reshape(1, -1, 1, 1) + 1e-5) + p[1].reshape(1, -1, 1, 1)
+    assert np.allclose(y, want, rtol=0, atol=1e-5)
+    assert np.array_equal(y, qf.batchnorm_inference(x, *[np.asarray(v, dtype=np.float32) for v in p]))
+    assert np.array_equal(bn.mean, np.asarray(p[2], dtype=np.float32))          # untouched
+    # MovingAverageMomentum 0 takes the same branch while learning
+    bn0 = qt.BatchNormCell(4, scales=p[0], biases=p[1], means=p[2], variances=p[3], moving_average_momentum=0.0)
+    assert np.array_equal(bn0.propagate(x, inference=False), y)
+
+
+@pytest.mark.parametrize("pool,stride,pad", [((2, 2), (2, 2), (0, 0)), ((3, 3), (2, 2), (0, 0)), ((3, 3), (2, 2), (1, 1)), ((3, 2), (1, 2), (0, 0))])
+def test_max_pooling_backward_routes_each_gradient_to_the_first_maximum(pool, stride, pad):
+    from oracle import qat_train as qt
+    rng = np.random.default_rng(23)
+    x = (rng.permutation(2 * 3 * 9 * 8).reshape(2, 3, 9, 8) / 1000.0).astype(np.float32)      # all distinct, 1e-3 apart
+    cell = qt.PoolCell(pool, stride, pad)
+    y = cell.propagate(x)
+    dy = rng.normal(0, 1, size=y.shape).astype(np.float32)
+    cell.diff_inputs = dy
+    dx = cell.back_propagate()
+    # directional derivative of sum(dy * maxpool(x)) along a random direction, exact for a piecewise-linear map
+    # (the step stays below half the distance between two inputs, so that no maximum moves)
+    v = np.clip(rng.normal(0, 2e-4, size=x.shape), -4e-4, 4e-4).astype(np.float32)
+    x2 = (x + v).astype(np.float32)
+    y2 = qt.PoolCell(pool, stride, pad).propagate(x2)
+    assert np.isclose(((y2.astype(np.float64) - y) * dy).sum(), (dx.astype(np.float64) * (x2.astype(np.float64) - x)).sum(), rtol=1e-3, atol=1e-7)
+    assert np.isclose(dx.sum(), dy.sum(), rtol=1e-5, atol=1e-5) and (dx != 0).sum() <= dy.size
+    # ties: the first element of the window in row-major order wins, forward and backward
+    flat = np.zeros((1, 1, 4, 4), dtype=np.float32)
+    c2 = qt.PoolCell((2, 2), (2, 2))
+    c2.propagate(flat)
+    c2.diff_inputs = np.ones((1, 1, 2, 2), dtype=np.float32)
+    assert np.array_equal(np.argwhere(c2.back_propagate()[0, 0] == 1), [[0, 0], [0, 2], [2, 0], [2, 2]])
+
+
+def test_a_net_with_batchnorm_and_pooling_learns():
+    from oracle import qat_train as qt
+    rng = np.random.default_rng(24)
+    x = rng.uniform(0, 1, size=(4, 1, 12, 12)).astype(np.float32)
+    t = np.zeros((4, 3, 1, 1), dtype=np.float32)
+    t[np.arange(4), [0, 1, 2, 0]] = 1
+    cells_ = [qt.ConvCell(rng.normal(0, 0.3, size=(4, 1, 3, 3)), quantizer=qt.SATQuantizerCell(15)),
+              qt.BatchNormCell(4, activation=qt.LinearActivation(qt.SATQuantizerActivation(15, 4.0))),
+              qt.PoolCell((2, 2), (2, 2)),
+              qt.ConvCell(rng.normal(0, 0.3, size=(3, 4, 5, 5)), quantizer=qt.SATQuantizerCell(15))]
+    sm = qt.SoftmaxCell()
+    first = qt.train_sequential(x, cells_, sm, t, 1)
+    last = qt.train_sequential(x, cells_, sm, t, 300)
+    assert last < 0.6 * first and np.isfinite(last)
+    assert not np.array_equal(cells_[1].scale, np.ones(4, dtype=np.float32)) and np.all(cells_[1].variance > 0)
