@@ -421,6 +421,193 @@ template class ActivationCell_FrameTrain_HIP<float>;
 template <> Registrar<ActivationCell> ActivationCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", ActivationCell_FrameTrain_HIP<float>::create,
                                                                                        Registrar<ActivationCell>::Type<float>());
 
+// ------------------------------------------------- BatchNormCell_FrameTrain_HIP
+const char* BatchNormCell::Type = "BatchNorm";
+
+void BatchNormCell::setParameter(const std::string& name, double value)
+{
+    if (name == "Epsilon") {
+        if (!(value > 0.0))
+            throw std::runtime_error("BatchNormCell " + mName + ": Epsilon must be positive");
+        mEpsilon = value;
+    } else if (name == "MovingAverageMomentum")
+        mMovingAverageMomentum = value;
+    else
+        throw std::runtime_error("Parameter does not exist: " + name);
+}
+
+template <class T>
+BatchNormCell_FrameTrain_HIP<T>::BatchNormCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
+                                                              const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), mScaleSolver(std::make_shared<SGDSolver_Frame_HIP<float> >()),
+      mBiasSolver(std::make_shared<SGDSolver_Frame_HIP<float> >()), mLearned(false)
+{
+    mActivation = activation;
+}
+
+template <class T>
+void BatchNormCell_FrameTrain_HIP<T>::set(DeviceFloats& dev, std::vector<Float_T>& host, const std::vector<Float_T>& v)
+{
+    if (v.size() != mNbOutputs)
+        throw std::runtime_error("BatchNormCell_FrameTrain_HIP " + mName + ": one value per output expected");
+    host = v;
+    if (!dev.empty())
+        dev.fromHost(v.data(), v.size());
+}
+
+template <class T>
+std::vector<Float_T> BatchNormCell_FrameTrain_HIP<T>::get(const DeviceFloats& dev, const std::vector<Float_T>& host) const
+{
+    if (dev.empty())
+        return host;
+    checkHipT(hipStreamSynchronize((hipStream_t)mStream), "BatchNormCell_FrameTrain_HIP: synchronize");
+    const Tensor<Float_T> t = dev.toHost();
+    return std::vector<Float_T>(t.data(), t.data() + t.size());
+}
+
+template <class T>
+void BatchNormCell_FrameTrain_HIP<T>::initialize()
+{
+    if (mNbChannels != mNbOutputs)
+        throw std::runtime_error("BatchNormCell_FrameTrain_HIP " + mName + ": the number of outputs must be the number of input channels");
+    allocateOutputs();
+    const std::vector<size_t> dims = {1, 1, (size_t)mNbOutputs, 1};
+    struct Init { DeviceFloats* dev; std::vector<Float_T>* host; Float_T value; };
+    const Init params[] = {{&mScale, &mHostScale, 1.0f}, {&mBias, &mHostBias, 0.0f}, {&mMean, &mHostMean, 0.0f}, {&mVariance, &mHostVariance, 0.0f}};
+    for (const Init& p : params) {
+        p.dev->resize(dims);
+        if (p.host->empty())
+            p.host->assign(mNbOutputs, p.value);
+        p.dev->fromHost(p.host->data(), p.host->size());
+    }
+    for (DeviceFloats* d : {&mSavedMean, &mSavedVariance, &mDiffScale, &mDiffBias, &mDiffSavedMean, &mDiffSavedVariance})
+        d->resize(dims);
+}
+
+template <class T>
+void BatchNormCell_FrameTrain_HIP<T>::propagate(bool inference)
+{
+    checkStatus(n2d2hip_batchnorm_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, mIn->data(), mScale.data(), mBias.data(),
+                                              mMean.data(), mVariance.data(), mSavedMean.data(), mSavedVariance.data(), mEpsilon, mMovingAverageMomentum,
+                                              inference ? 1 : 0, mOutputs.data(), mStream));
+    if (!inference && mMovingAverageMomentum != 0.0)
+        mLearned = true;
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+    mDiffScale.clearValid();
+    mDiffBias.clearValid();
+}
+
+template <class T>
+void BatchNormCell_FrameTrain_HIP<T>::backPropagate()
+{
+    if (!mDiffInputs.isValid())
+        return;
+    if (!mLearned)
+        throw std::runtime_error("BatchNormCell_FrameTrain_HIP " + mName + ": backPropagate() needs the batch statistics of a learning propagate()");
+    activationBackPropagate();
+    const float betaScale = mScaleSolver->isNewIteration() ? 0.0f : 1.0f;
+    const float betaBias = mBiasSolver->isNewIteration() ? 0.0f : 1.0f;
+    const bool toInput = mDiffOut && !mDiffOut->empty();
+    if (toInput && mDiffOut->isValid())
+        throw std::runtime_error("BatchNormCell_FrameTrain_HIP " + mName + ": accumulating into a gradient another cell has written is not supported");
+    checkStatus(n2d2hip_batchnorm_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, mIn->data(), mScale.data(), mSavedMean.data(),
+                                               mSavedVariance.data(), mEpsilon, mDiffInputs.data(), betaScale, mDiffScale.data(), betaBias,
+                                               mDiffBias.data(), mDiffSavedMean.data(), mDiffSavedVariance.data(), toInput ? mDiffOut->data() : nullptr,
+                                               mStream));
+    if (toInput)
+        mDiffOut->setValid();
+    mDiffScale.setValid();
+    mDiffBias.setValid();
+}
+
+template <class T>
+void BatchNormCell_FrameTrain_HIP<T>::update()
+{
+    const unsigned int batch = (unsigned int)mIn->dimB();
+    if (mDiffScale.isValid())
+        mScaleSolver->update(mScale.data(), mDiffScale.data(), mScale.size(), batch, mStream);
+    if (mDiffBias.isValid())
+        mBiasSolver->update(mBias.data(), mDiffBias.data(), mBias.size(), batch, mStream);
+    activationUpdate();
+}
+
+template class BatchNormCell_FrameTrain_HIP<float>;
+template <> Registrar<BatchNormCell> BatchNormCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", BatchNormCell_FrameTrain_HIP<float>::create,
+                                                                                     Registrar<BatchNormCell>::Type<float>());
+
+// ------------------------------------------------------ PoolCell_FrameTrain_HIP
+template <class T>
+PoolCell_FrameTrain_HIP<T>::PoolCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& poolDims,
+                                                    unsigned int nbOutputs, const std::vector<unsigned int>& strideDims,
+                                                    const std::vector<unsigned int>& paddingDims, Pooling pooling,
+                                                    const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), PoolCell(poolDims, strideDims, paddingDims, pooling), mArgMax(nullptr)
+{
+    if (poolDims.size() != 2 || strideDims.size() != 2 || paddingDims.size() != 2)
+        throw std::runtime_error("PoolCell_FrameTrain_HIP " + name + ": two-dimensional pooling expected");
+    if (pooling != Max)
+        throw std::runtime_error("PoolCell_FrameTrain_HIP " + name + ": only Max pooling learns on the float Frame_HIP cells");
+    mActivation = activation;
+}
+
+template <class T>
+PoolCell_FrameTrain_HIP<T>::~PoolCell_FrameTrain_HIP()
+{
+    if (mArgMax)
+        (void)hipFree(mArgMax);
+}
+
+template <class T>
+void PoolCell_FrameTrain_HIP<T>::setOutputsDims()
+{
+    // PoolCell::setOutputsDims (src/Cell/PoolCell.cpp:219-240)
+    mOutW = (unsigned int)(((int)mInW + 2 * (int)mPaddingDims[0] - (int)mPoolDims[0] + (int)mStrideDims[0]) / (double)mStrideDims[0]);
+    mOutH = (unsigned int)(((int)mInH + 2 * (int)mPaddingDims[1] - (int)mPoolDims[1] + (int)mStrideDims[1]) / (double)mStrideDims[1]);
+}
+
+template <class T>
+void PoolCell_FrameTrain_HIP<T>::initialize()
+{
+    if (mNbChannels != mNbOutputs)
+        throw std::runtime_error("PoolCell_FrameTrain_HIP " + mName + ": one output per input channel expected (the unit mapping)");
+    allocateOutputs();
+    if (mArgMax) {
+        (void)hipFree(mArgMax);
+        mArgMax = nullptr;
+    }
+    checkHipT(hipMalloc((void**)&mArgMax, mOutputs.size() * sizeof(int)), "PoolCell_FrameTrain_HIP::initialize()");
+}
+
+template <class T>
+void PoolCell_FrameTrain_HIP<T>::propagate(bool inference)
+{
+    checkStatus(n2d2hip_pool_max_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                             (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], mIn->data(),
+                                             mOutputs.data(), mArgMax, mStream));
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+}
+
+template <class T>
+void PoolCell_FrameTrain_HIP<T>::backPropagate()
+{
+    if (!mDiffInputs.isValid())
+        return;
+    activationBackPropagate();
+    if (!mDiffOut || mDiffOut->empty())
+        return;
+    const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
+    checkStatus(n2d2hip_pool_max_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                              (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], mDiffInputs.data(),
+                                              mArgMax, beta, mDiffOut->data(), mStream));
+    mDiffOut->setValid();
+}
+
+template class PoolCell_FrameTrain_HIP<float>;
+template <> Registrar<PoolCell> PoolCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", PoolCell_FrameTrain_HIP<float>::create,
+                                                                           Registrar<PoolCell>::Type<float>());
+
 // --------------------------------------------------- SoftmaxCell_FrameTrain_HIP
 const char* SoftmaxCell::Type = "Softmax";
 

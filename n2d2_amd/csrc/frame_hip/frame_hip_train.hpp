@@ -203,6 +203,96 @@ private:
     static Registrar<ActivationCell> mRegistrar;
 };
 
+// include/Cell/BatchNormCell.hpp:36-160: Epsilon (1.0e-5), MovingAverageMomentum (0.1); scales 1, biases 0, means 0,
+// variances 0 until set or learned
+class BatchNormCell : public virtual Cell {
+public:
+    typedef std::function<std::shared_ptr<BatchNormCell>(const DeepNet&, const std::string&, unsigned int,
+                                                         const std::shared_ptr<Activation>&)> RegistryCreate_T;
+    static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
+    static const char* Type;
+    const char* getType() const { return Type; }
+    void setParameter(const std::string& name, double value);
+    double getEpsilon() const { return mEpsilon; }
+
+protected:
+    BatchNormCell() : mEpsilon(1.0e-5), mMovingAverageMomentum(0.1) {}
+    double mEpsilon, mMovingAverageMomentum;
+};
+
+// src/Cell/BatchNormCell_Frame.cpp for one input.  Parameters, statistics and gradients stay on the device; the
+// getters copy to the host, the setters (before or after initialize()) to the device.
+template <class T>
+class BatchNormCell_FrameTrain_HIP : public BatchNormCell, public Cell_FrameTrain_HIP {
+public:
+    BatchNormCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                 const std::shared_ptr<Activation>& activation);
+    static std::shared_ptr<BatchNormCell> create(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                                 const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<BatchNormCell_FrameTrain_HIP<T> >(deepNet, name, nbOutputs, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update();
+    // BatchNormCell::setScales / setBiases / setMeans / setVariances and their getters, one value per output
+    void setScales(const std::vector<Float_T>& v) { set(mScale, mHostScale, v); }
+    void setBiases(const std::vector<Float_T>& v) { set(mBias, mHostBias, v); }
+    void setMeans(const std::vector<Float_T>& v) { set(mMean, mHostMean, v); }
+    void setVariances(const std::vector<Float_T>& v) { set(mVariance, mHostVariance, v); }
+    std::vector<Float_T> getScales() const { return get(mScale, mHostScale); }
+    std::vector<Float_T> getBiases() const { return get(mBias, mHostBias); }
+    std::vector<Float_T> getMeans() const { return get(mMean, mHostMean); }
+    std::vector<Float_T> getVariances() const { return get(mVariance, mHostVariance); }
+    std::vector<Float_T> getDiffScales() const { return get(mDiffScale, std::vector<Float_T>()); }
+    std::vector<Float_T> getDiffBiases() const { return get(mDiffBias, std::vector<Float_T>()); }
+    void setScaleSolver(const std::shared_ptr<SGDSolver>& solver) { mScaleSolver = solver; }
+    void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
+    const std::shared_ptr<SGDSolver>& getScaleSolver() const { return mScaleSolver; }
+    const std::shared_ptr<SGDSolver>& getBiasSolver() const { return mBiasSolver; }
+
+protected:
+    void setOutputsDims() { mOutW = mInW; mOutH = mInH; }
+
+private:
+    void set(DeviceFloats& dev, std::vector<Float_T>& host, const std::vector<Float_T>& v);
+    std::vector<Float_T> get(const DeviceFloats& dev, const std::vector<Float_T>& host) const;
+    DeviceFloats mScale, mBias, mMean, mVariance, mSavedMean, mSavedVariance, mDiffScale, mDiffBias, mDiffSavedMean, mDiffSavedVariance;
+    std::vector<Float_T> mHostScale, mHostBias, mHostMean, mHostVariance;      // values set before initialize()
+    std::shared_ptr<SGDSolver> mScaleSolver, mBiasSolver;
+    bool mLearned;              // a learning propagate has filled the saved statistics
+    static Registrar<BatchNormCell> mRegistrar;
+};
+
+// src/Cell/PoolCell_Frame.cpp:123-228 with Pooling=Max, one input and one output per channel.
+template <class T>
+class PoolCell_FrameTrain_HIP : public PoolCell, public Cell_FrameTrain_HIP {
+public:
+    PoolCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, const std::vector<unsigned int>& poolDims, unsigned int nbOutputs,
+                            const std::vector<unsigned int>& strideDims, const std::vector<unsigned int>& paddingDims, Pooling pooling,
+                            const std::shared_ptr<Activation>& activation);
+    ~PoolCell_FrameTrain_HIP();
+    static std::shared_ptr<PoolCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name,
+                                            const std::vector<unsigned int>& poolDims, unsigned int nbOutputs,
+                                            const std::vector<unsigned int>& strideDims, const std::vector<unsigned int>& paddingDims,
+                                            Pooling pooling, const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<PoolCell_FrameTrain_HIP<T> >(deepNet, name, poolDims, nbOutputs, strideDims, paddingDims, pooling, activation);
+    }
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update() { activationUpdate(); }
+
+protected:
+    void setOutputsDims();
+
+private:
+    int* mArgMax;
+    static Registrar<PoolCell> mRegistrar;
+};
+
 // include/Cell/SoftmaxCell.hpp:37-70: WithLoss (false), GroupSize (0)
 class SoftmaxCell : public virtual Cell {
 public:

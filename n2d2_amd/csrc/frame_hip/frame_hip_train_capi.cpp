@@ -94,6 +94,8 @@ int fh_train_registrar_exists(const char* type, const char* key)
     if (t == "Fc") return Registrar<FcCell>::exists<float>(k);
     if (t == "Activation") return Registrar<ActivationCell>::exists<float>(k);
     if (t == "Softmax") return Registrar<SoftmaxCell>::exists<float>(k);
+    if (t == "BatchNorm") return Registrar<BatchNormCell>::exists<float>(k);
+    if (t == "Pool") return Registrar<PoolCell>::exists<float>(k);
     return -1;
 }
 
@@ -205,6 +207,56 @@ int fh_train_add_fc(void* net, const char* name, int nbOutputs, const float* wei
     });
 }
 
+// params: HOST float [4][nbOutputs] = scales, biases, means, variances, or NULL for the cell's initial values (1, 0, 0, 0)
+int fh_train_add_batchnorm(void* net, const char* name, const float* params, double epsilon, double movingAverageMomentum, int act, int actQuant,
+                           int actRange, float actParam)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<BatchNormCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        const unsigned int nbOutputs = n.cells.empty() ? (unsigned int)n.input.dimZ() : n.last()->getNbOutputs();
+        auto bn = f(n.deepNet, name, nbOutputs, makeActivation(n, name, act, actQuant, actRange, actParam));
+        bn->setParameter("Epsilon", epsilon);
+        bn->setParameter("MovingAverageMomentum", movingAverageMomentum);
+        auto cell = std::dynamic_pointer_cast<BatchNormCell_FrameTrain_HIP<float> >(bn);
+        if (params) {
+            cell->setScales(std::vector<Float_T>(params, params + nbOutputs));
+            cell->setBiases(std::vector<Float_T>(params + nbOutputs, params + 2 * nbOutputs));
+            cell->setMeans(std::vector<Float_T>(params + 2 * nbOutputs, params + 3 * nbOutputs));
+            cell->setVariances(std::vector<Float_T>(params + 3 * nbOutputs, params + 4 * nbOutputs));
+        }
+        connect(n, cell);
+    });
+}
+
+// what: 0 scales, 1 biases, 2 running means, 3 running variances, 4 gradient of the scales, 5 gradient of the biases
+int fh_train_get_batchnorm(void* net, const char* cell, int what, float* out, size_t n)
+{
+    return guardedT([&] {
+        auto bn = dynamic_cast<BatchNormCell_FrameTrain_HIP<float>*>(find(*(TrainNet*)net, cell));
+        if (!bn) throw std::runtime_error("Not a BatchNorm cell: " + std::string(cell));
+        const std::vector<Float_T> v = what == 0 ? bn->getScales() : what == 1 ? bn->getBiases() : what == 2 ? bn->getMeans()
+                                       : what == 3 ? bn->getVariances() : what == 4 ? bn->getDiffScales() : bn->getDiffBiases();
+        if (v.size() != n) throw std::runtime_error("fh_train_get_batchnorm(): size mismatch");
+        std::memcpy(out, v.data(), n * sizeof(float));
+    });
+}
+
+// Max pooling, one output per channel
+int fh_train_add_pool(void* net, const char* name, int poolW, int poolH, int strideX, int strideY, int padX, int padY)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<PoolCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        const unsigned int nbOutputs = n.cells.empty() ? (unsigned int)n.input.dimZ() : n.last()->getNbOutputs();
+        auto pool = f(n.net, n.deepNet, name, {(unsigned)poolW, (unsigned)poolH}, nbOutputs, {(unsigned)strideX, (unsigned)strideY},
+                      {(unsigned)padX, (unsigned)padY}, PoolCell::Max, std::shared_ptr<Activation>());
+        connect(n, std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(pool));
+    });
+}
+
 int fh_train_add_softmax(void* net, const char* name, int withLoss)
 {
     return guardedT([&] {
@@ -221,11 +273,20 @@ int fh_train_add_softmax(void* net, const char* name, int withLoss)
 int fh_train_set_solver_parameter(void* net, const char* cell, const char* name, double value)
 {
     return guardedT([&] {
-        auto conv = dynamic_cast<WeightedCell_FrameTrain_HIP*>(find(*(TrainNet*)net, cell));
-        if (!conv) throw std::runtime_error("Not a cell with weights: " + std::string(cell));
+        Cell_FrameTrain_HIP* c = find(*(TrainNet*)net, cell);
         auto s = Registrar<SGDSolver>::create<float>("Frame_HIP")();
         s->setParameter(name, value);
-        conv->setWeightsSolver(s);
+        if (auto conv = dynamic_cast<WeightedCell_FrameTrain_HIP*>(c)) {
+            conv->setWeightsSolver(s);
+        } else if (auto bn = dynamic_cast<BatchNormCell_FrameTrain_HIP<float>*>(c)) {
+            // the scales' and the biases' solvers, one object each
+            bn->setScaleSolver(s);
+            auto s2 = Registrar<SGDSolver>::create<float>("Frame_HIP")();
+            s2->setParameter(name, value);
+            bn->setBiasSolver(s2);
+        } else {
+            throw std::runtime_error("Not a cell with a solver: " + std::string(cell));
+        }
     });
 }
 

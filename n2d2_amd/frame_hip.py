@@ -345,6 +345,9 @@ lib.fh_train_net_destroy.restype = None
 lib.fh_train_add_activation_cell.argtypes = [_P, C.c_char_p, _I, _I, _I, _F]
 lib.fh_train_add_conv.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _F, _I, _I, _I, _I, _I]
 lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
+lib.fh_train_add_batchnorm.argtypes = [_P, C.c_char_p, _P, C.c_double, C.c_double, _I, _I, _I, _F]
+lib.fh_train_get_batchnorm.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
+lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I]
 lib.fh_train_add_fc.argtypes = [_P, C.c_char_p, _I, _P, _P, _I, _I, _I, _F, _I, _I]
 lib.fh_train_set_solver_parameter.argtypes = [_P, C.c_char_p, C.c_char_p, C.c_double]
 lib.fh_train_learn.argtypes = [_P, _P, _SZ, _I, _P]
@@ -366,7 +369,7 @@ def _check_train(rc):
 
 
 class TrainNet:
-    """A sequential net of the float Frame_HIP cells (ActivationCell, ConvCell, SoftmaxCell) with SAT / LSQ quantizers,
+    """A sequential net of the float Frame_HIP cells (ActivationCell, ConvCell, FcCell, BatchNormCell, PoolCell, SoftmaxCell) with SAT / LSQ quantizers,
     created through the Registrar under `model`. x: float32 [B,C,H,W]."""
 
     def __init__(self, x, model=TRAIN_MODEL, propagate_gradient=True):
@@ -414,6 +417,37 @@ class TrainNet:
         self._last = (self._last[0], w.shape[0], 1, 1)
         self._shapes[name] = self._last
         self._shapes[name + "/weights"] = w.shape
+
+    def add_batchnorm(self, name, scales=None, biases=None, means=None, variances=None, epsilon=1.0e-5, moving_average_momentum=0.1,
+                      act=None, act_quant=None, act_range=255, act_param=1.0):
+        """BatchNormCell after the last cell; all four parameter vectors or none (then 1, 0, 0, 0)."""
+        params = None
+        if scales is not None:
+            params = np.ascontiguousarray(np.stack([np.asarray(v, dtype=np.float32) for v in (scales, biases, means, variances)]))
+            if params.shape != (4, self._last[1]):
+                raise ValueError("one value per channel expected")
+        _check_train(lib.fh_train_add_batchnorm(self._h, name.encode(), None if params is None else params.ctypes.data, float(epsilon),
+                                                float(moving_average_momentum), _ACT[act], _QUANT[act_quant], int(act_range), float(act_param)))
+        self._shapes[name] = self._last
+
+    def batchnorm(self, name):
+        """dict of the cell's scales, biases, running means and variances, and the last gradients of scales and biases."""
+        out = {}
+        for k, what in (("scales", 0), ("biases", 1), ("means", 2), ("variances", 3), ("diff_scales", 4), ("diff_biases", 5)):
+            v = np.empty(self._shapes[name][1], dtype=np.float32)
+            _check_train(lib.fh_train_get_batchnorm(self._h, name.encode(), what, v.ctypes.data, v.size))
+            out[k] = v
+        return out
+
+    def add_pool(self, name, pool, stride, pad=(0, 0)):
+        """Max pooling, one output per channel; pool / stride / pad as (x, y)."""
+        _check_train(lib.fh_train_add_pool(self._h, name.encode(), int(pool[0]), int(pool[1]), int(stride[0]), int(stride[1]), int(pad[0]),
+                                           int(pad[1])))
+        B, Cn, H, W = self._last
+        oH = int((H + 2 * pad[1] - pool[1] + stride[1]) / float(stride[1]))
+        oW = int((W + 2 * pad[0] - pool[0] + stride[0]) / float(stride[0]))
+        self._last = (B, Cn, oH, oW)
+        self._shapes[name] = self._last
 
     def add_softmax(self, name, with_loss=True):
         _check_train(lib.fh_train_add_softmax(self._h, name.encode(), int(with_loss)))

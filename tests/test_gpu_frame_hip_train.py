@@ -42,7 +42,7 @@ def _close(got, want, tol=1e-5):
 
 def test_registrar_holds_the_float_cells():
     from n2d2_amd import frame_hip as fh
-    for t in ("Conv", "Fc", "Activation", "Softmax"):
+    for t in ("Conv", "Fc", "Activation", "Softmax", "BatchNorm", "Pool"):
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_HIP_QAT") == 1
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_XYZ") == 0
     assert fh.lib.fh_train_registrar_exists(b"Conv", b"Frame_HIP") == 1          # the integer inference cell
@@ -239,3 +239,110 @@ def test_conv_then_fc_with_bias_against_the_oracle():
         assert abs(loss - want) <= 1e-5 * want, it
     assert _close(net.outputs("softmax"), sm.outputs)
     assert _close(net.weights("fc"), fc.w.reshape(5, -1), 1e-4) and _close(net.weights("c1"), c1.w, 1e-4)
+
+
+def test_batchnorm_and_pool_cells_learn_as_the_oracle_does():
+    """Conv (SAT weights) -> BatchNorm (Linear, SAT activation) -> max Pool -> Conv -> Softmax: the first iteration tensor by
+    tensor, then twenty more on the loss and the learned parameters."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    rng = np.random.default_rng(31)
+    x = rng.uniform(0, 1, size=(4, 1, 12, 12)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, size=(4, 1, 3, 3)).astype(np.float32)
+    w2 = rng.normal(0, 0.3, size=(3, 4, 5, 5)).astype(np.float32)
+    t = np.zeros((4, 3, 1, 1), dtype=np.float32)
+    t[np.arange(4), [0, 1, 2, 0]] = 1
+    net = fh.TrainNet(x, propagate_gradient=False)
+    net.add_conv("c1", w1, weight_quant="SAT", weight_range=15)
+    net.add_batchnorm("bn", act="Linear", act_quant="SAT", act_range=15, act_param=4.0)
+    net.add_pool("pool", (2, 2), (2, 2))
+    net.add_conv("c2", w2, weight_quant="SAT", weight_range=15)
+    net.add_softmax("softmax", with_loss=True)
+    assert net._shapes["pool"] == (4, 4, 5, 5) and net._last == (4, 3, 1, 1)
+    qa = q.SATQuantizerActivation(15, 4.0)
+    cells_ = [q.ConvCell(w1, quantizer=q.SATQuantizerCell(15)), q.BatchNormCell(4, activation=q.LinearActivation(qa)), q.PoolCell((2, 2), (2, 2)),
+              q.ConvCell(w2, quantizer=q.SATQuantizerCell(15))]
+    sm = q.SoftmaxCell()
+    print("batchnorm / pool net: first iteration", flush=True)
+    loss = net.learn(t, 1)
+    want = q.train_sequential(x, cells_, sm, t, 1)
+    assert abs(loss - want) <= 1e-5 * want
+    for name, cell in zip(("c1", "bn", "pool", "c2"), cells_):
+        assert _close(net.outputs(name), cell.outputs, 2e-5), name
+        if name != "bn":        # (the BatchNorm's activation works on its gradient in place)
+            assert _close(net.diff_inputs(name), cell.diff_inputs, 1e-4), name
+    bn = net.batchnorm("bn")
+    assert _close(bn["diff_scales"], cells_[1].diff_scale, 1e-4) and _close(bn["diff_biases"], cells_[1].diff_bias, 1e-4)
+    assert _close(bn["scales"], cells_[1].scale) and _close(bn["biases"], cells_[1].bias, 1e-4)
+    assert _close(bn["means"], cells_[1].mean, 1e-4) and _close(bn["variances"], cells_[1].variance, 1e-4)
+    assert _close(net.weights("c1"), cells_[0].w, 1e-4) and _close(net.weights("c2"), cells_[3].w, 1e-4)
+    print("batchnorm / pool net: twenty more", flush=True)
+    for it in range(20):
+        loss = net.learn(t, 1)
+        want = q.train_sequential(x, cells_, sm, t, 1)
+        assert abs(loss - want) <= 1e-3 * want, it
+    bn = net.batchnorm("bn")
+    assert _close(bn["scales"], cells_[1].scale, 1e-3) and _close(bn["variances"], cells_[1].variance, 1e-3)
+    assert abs(net.activation_quantizer("bn")[0] - float(qa.alphas[0])) <= 1e-3
+    assert not np.array_equal(bn["scales"], np.ones(4, dtype=np.float32))
+    # inference afterwards runs on the running statistics
+    net.propagate(inference=True)
+    h = x
+    for c in cells_:
+        h = c.propagate(h, inference=True)
+    assert _close(net.outputs("c2"), h, 1e-3)
+    # a backPropagate without a learning propagate has nothing to differentiate
+    fresh = fh.TrainNet(x, propagate_gradient=False)
+    fresh.add_batchnorm("bn", moving_average_momentum=0.0)
+    fresh.add_softmax("softmax", with_loss=True)
+    with pytest.raises(fh.FrameHipError, match="needs the batch statistics"):
+        fresh.learn(np.zeros((4, 1, 12, 12), dtype=np.float32), 1)
+
+
+@pytest.mark.parametrize("name", ["w8a8", "w4a4"])
+def test_trained_lenet_float_graph_and_its_integer_twin_agree_on_the_gpu(name):
+    """The reference's test of its QAT-to-integer pass (tests/Quantizer/QAT/Optimization/class_DeepNetQAT.cpp:96-140) runs the
+    trained LeNet with BatchNorm before and after the pass and compares recognition rates.  Here both graphs run on the GPU
+    on the same images: the float one on the Frame_HIP_QAT cells (checked against the oracle), the integer one on the
+    Frame_HIP cells after the library's pass, and the levels after each Conv + BatchNorm stage are compared."""
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import sat_lenet as sl
+    from n2d2_amd import frame_hip as fh
+    from oracle import oracle as o
+    d = sl.load(name)
+    R = sl.act_range(name)
+    imgs = sl.images(32, seed=12)
+    x = (imgs / np.float32(255)).astype(np.float32)
+    net = fh.TrainNet(x, propagate_gradient=False)
+    chain = x
+    want = {}
+    for (conv, bn, shape, w_range), pool in zip(sl.conv_stages(name), ("pool1", "pool2", None)):
+        alpha = float(d[bn + "_QAct_SAT_Alpha"][0])
+        net.add_conv(conv, d[conv + "_weights"].reshape(shape), weight_quant="SAT", weight_range=w_range, act="Linear")
+        net.add_batchnorm(bn, *sl.bn_of(d, bn), epsilon=sl.EPS, act="Linear", act_quant="SAT", act_range=R, act_param=alpha)
+        levels = sl.float_conv_stage(chain, sl.quantized_conv_weights(d, conv, shape, w_range), sl.bn_of(d, bn), alpha, R)
+        want[bn] = (levels, alpha)
+        chain = (levels * np.float32(alpha / R)).astype(np.float32)
+        if pool:
+            net.add_pool(pool, (2, 2), (2, 2))
+            chain = o.pool_forward(chain, (2, 2), (2, 2), kind="max", quantized=False)
+    print("trained LeNet", name, "float graph", flush=True)
+    net.propagate(inference=True)
+    fused = sl.fuse_with_library(fh, d, name, batch=32)
+    try:
+        fh.set_globals(8, True, True)
+        fused.set_fusion(False)
+        fused.initialize()
+        fused.set_stimuli(imgs)
+        fused.propagate()
+        for (conv, bn, _, w_range) in sl.conv_stages(name):
+            levels, alpha = want[bn]
+            got = np.rint(net.outputs(bn) * np.float32(R / alpha))
+            # the float cells against the oracle's float graph: the same levels but where a sum lands within rounding of a tie
+            assert (got != levels).mean() < 2e-3 and np.abs(got - levels).max() <= 1, bn
+            dev = np.abs(fused.outputs(conv) - got)
+            assert dev.max() <= (6 if R == 255 else 1) and dev.mean() < (0.3 if R == 255 else 0.06), conv
+            assert np.unique(got).size > 4
+    finally:
+        fh.set_globals(0, True, False)
