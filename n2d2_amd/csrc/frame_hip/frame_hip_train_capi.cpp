@@ -173,7 +173,7 @@ int fh_train_add_conv(void* net, const char* name, int nbOutputs, int kW, int kH
 
 // weights: HOST float [O, C*H*W] (CHW order); bias HOST float [O] or NULL (NoBias).  weightQuant: 0 none, 1 SAT, 2 LSQ.
 int fh_train_add_fc(void* net, const char* name, int nbOutputs, const float* weights, const float* bias, int act, int actQuant, int actRange,
-                    float actParam, int weightQuant, int weightRange)
+                    float actParam, int weightQuant, int weightRange, int applyScaling)
 {
     return guardedT([&] {
         TrainNet& n = *(TrainNet*)net;
@@ -195,6 +195,7 @@ int fh_train_add_fc(void* net, const char* name, int nbOutputs, const float* wei
         if (weightQuant == 1) {
             auto q = Registrar<SATQuantizerCell>::create<float>("Frame_HIP")();
             q->setRange((size_t)weightRange);
+            q->setScaling(applyScaling != 0);
             cell->setQuantizer(q);
         } else if (weightQuant == 2) {
             auto q = Registrar<LSQQuantizerCell>::create<float>("Frame_HIP")();

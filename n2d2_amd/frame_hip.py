@@ -348,7 +348,7 @@ lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
 lib.fh_train_add_batchnorm.argtypes = [_P, C.c_char_p, _P, C.c_double, C.c_double, _I, _I, _I, _F]
 lib.fh_train_get_batchnorm.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
 lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I]
-lib.fh_train_add_fc.argtypes = [_P, C.c_char_p, _I, _P, _P, _I, _I, _I, _F, _I, _I]
+lib.fh_train_add_fc.argtypes = [_P, C.c_char_p, _I, _P, _P, _I, _I, _I, _F, _I, _I, _I]
 lib.fh_train_set_solver_parameter.argtypes = [_P, C.c_char_p, C.c_char_p, C.c_double]
 lib.fh_train_learn.argtypes = [_P, _P, _SZ, _I, _P]
 lib.fh_train_propagate.argtypes = [_P, _I]
@@ -408,12 +408,13 @@ class TrainNet:
         self._shapes[name + "/weights"] = w.shape
 
     def add_fc(self, name, weights, bias=None, act=None, act_quant=None, act_range=255, act_param=1.0, weight_quant=None,
-               weight_range=255):
-        """weights: [O, C*H*W] (CHW order)."""
+               weight_range=255, apply_scaling=False):
+        """weights: [O, C*H*W] (CHW order); apply_scaling: the SAT weight quantizer's ApplyScaling."""
         w = np.ascontiguousarray(weights, dtype=np.float32)
         b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
         _check_train(lib.fh_train_add_fc(self._h, name.encode(), w.shape[0], w.ctypes.data, None if b is None else b.ctypes.data,
-                                         _ACT[act], _QUANT[act_quant], act_range, act_param, _QUANT[weight_quant], weight_range))
+                                         _ACT[act], _QUANT[act_quant], act_range, act_param, _QUANT[weight_quant], weight_range,
+                                         int(apply_scaling)))
         self._last = (self._last[0], w.shape[0], 1, 1)
         self._shapes[name] = self._last
         self._shapes[name + "/weights"] = w.shape

@@ -327,8 +327,21 @@ def test_trained_lenet_float_graph_and_its_integer_twin_agree_on_the_gpu(name):
         if pool:
             net.add_pool(pool, (2, 2), (2, 2))
             chain = o.pool_forward(chain, (2, 2), (2, 2), kind="max", quantized=False)
+    fc_want = {}
+    for fc, shape, w_range, a_range in sl.fc_stages(name):
+        alpha = float(d[fc + "_QAct_SAT_Alpha"][0])
+        net.add_fc(fc, d[fc + "_weights"].reshape(shape), act="Linear", act_quant="SAT", act_range=a_range, act_param=alpha, weight_quant="SAT",
+                   weight_range=w_range, apply_scaling=True)
+        wq, _ = sl.quantized_fc_weights(d, fc, shape, w_range)
+        z = o.conv_forward(chain.reshape(32, -1, 1, 1), wq.reshape(shape + (1, 1)))
+        chain, _ = o.sat_act_forward(z, a_range, alpha, True)
+        fc_want[fc] = (np.rint(chain * np.float32(a_range / alpha)), alpha, a_range)
     print("trained LeNet", name, "float graph", flush=True)
     net.propagate(inference=True)
+    for fc, (levels, alpha, a_range) in fc_want.items():
+        got = np.rint(net.outputs(fc) * np.float32(a_range / alpha))
+        assert (got != levels).mean() < 5e-3 and np.abs(got - levels).max() <= 1, fc
+    assert np.unique(fc_want["fc2"][0]).size > 4
     fused = sl.fuse_with_library(fh, d, name, batch=32)
     try:
         fh.set_globals(8, True, True)
