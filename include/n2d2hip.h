@@ -309,10 +309,14 @@ int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, fl
  * changed.  Otherwise m, v are the batch's mean and biased variance over batch and pixels, written to saved_mean /
  * saved_variance, and the running ones move towards them: mean = m * momentum + mean * (1 - momentum), variance likewise
  * with v * n / (n - 1) (ref: BatchNormCell_Frame<T>::propagate, src/Cell/BatchNormCell_Frame.cpp:287-393).  x and y may
- * be the same buffer. */
+ * be the same buffer.  With a workspace of n2d2hip_batchnorm_f32_workspace_bytes() the sums of the learning pass and of
+ * the backward are spread over several blocks per channel (partial sums added in a fixed order); without one (NULL) one
+ * block per channel adds them.  Forward and backward may share the workspace. */
+size_t n2d2hip_batchnorm_f32_workspace_bytes(int B, int C, int H, int W);
 int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, const float* scale, const float* bias,
                                   float* mean, float* variance, float* saved_mean, float* saved_variance, double epsilon,
-                                  double moving_average_momentum, int use_running, float* y, n2d2hip_stream_t stream);
+                                  double moving_average_momentum, int use_running, float* y, void* workspace,
+                                  size_t workspace_bytes, n2d2hip_stream_t stream);
 /* Its backward, from the x and the saved statistics of the learning pass: diff_scale[c] = sum(diff_y * x_hat) +
  * beta_scale * diff_scale[c], diff_bias[c] = sum(diff_y) + beta_bias * diff_bias[c], the gradients of the saved mean and
  * variance ({C} each, always written), and, when diff_x != NULL, diff_x = diff_y * scale / sigma + dVar * 2 (x - m) / n
@@ -321,7 +325,8 @@ int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, co
 int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, const float* scale, const float* saved_mean,
                                    const float* saved_variance, double epsilon, const float* diff_y, float beta_scale,
                                    float* diff_scale, float beta_bias, float* diff_bias, float* diff_saved_mean,
-                                   float* diff_saved_variance, float* diff_x, n2d2hip_stream_t stream);
+                                   float* diff_saved_variance, float* diff_x, void* workspace, size_t workspace_bytes,
+                                   n2d2hip_stream_t stream);
 /* Max pooling of float NCHW, one output per channel; output size as PoolCell computes it, (in + 2 pad - pool + stride) /
  * stride.  argmax {B,C,oH,oW} receives row * W + column of the first largest element of each window in row-major order,
  * -1 for a window that lies in the padding (output 0) (ref: PoolCell_Frame_Kernels::forwardMax with its ArgMax tensor,

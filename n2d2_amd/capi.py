@@ -34,7 +34,7 @@ SYMBOLS = [
     "n2d2hip_conv2d_f32_forward", "n2d2hip_conv2d_f32_backward_data", "n2d2hip_conv2d_f32_backward_filter", "n2d2hip_conv2d_f32_workspace_bytes",
     "n2d2hip_conv2d_f32_backward_bias", "n2d2hip_softmax_f32_forward", "n2d2hip_loss_workspace_bytes", "n2d2hip_loss_f32",
     "n2d2hip_sgd_update_f32", "n2d2hip_rectifier_f32_forward", "n2d2hip_rectifier_f32_backward",
-    "n2d2hip_batchnorm_f32_forward", "n2d2hip_batchnorm_f32_backward", "n2d2hip_pool_max_f32_forward", "n2d2hip_pool_max_f32_backward",
+    "n2d2hip_batchnorm_f32_workspace_bytes", "n2d2hip_batchnorm_f32_forward", "n2d2hip_batchnorm_f32_backward", "n2d2hip_pool_max_f32_forward", "n2d2hip_pool_max_f32_backward",
 ]
 
 
@@ -118,8 +118,10 @@ def load():
     lib.n2d2hip_rectifier_f32_forward.argtypes = [P, SZ, F, F, P]
     lib.n2d2hip_rectifier_f32_backward.argtypes = [P, P, P, SZ, F, F, P]
     D = C.c_double
-    lib.n2d2hip_batchnorm_f32_forward.argtypes = [I, I, I, I, P, P, P, P, P, P, P, D, D, I, P, P]
-    lib.n2d2hip_batchnorm_f32_backward.argtypes = [I, I, I, I, P, P, P, P, D, P, F, P, F, P, P, P, P, P]
+    lib.n2d2hip_batchnorm_f32_workspace_bytes.restype = C.c_size_t
+    lib.n2d2hip_batchnorm_f32_workspace_bytes.argtypes = [I, I, I, I]
+    lib.n2d2hip_batchnorm_f32_forward.argtypes = [I, I, I, I, P, P, P, P, P, P, P, D, D, I, P, P, SZ, P]
+    lib.n2d2hip_batchnorm_f32_backward.argtypes = [I, I, I, I, P, P, P, P, D, P, F, P, F, P, P, P, P, P, SZ, P]
     lib.n2d2hip_pool_max_f32_forward.argtypes = [I, I, I, I, I, I, I, I, I, I, P, P, P, P]
     lib.n2d2hip_pool_max_f32_backward.argtypes = [I, I, I, I, I, I, I, I, I, I, P, P, F, P, P]
     return lib

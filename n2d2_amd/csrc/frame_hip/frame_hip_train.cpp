@@ -482,6 +482,8 @@ void BatchNormCell_FrameTrain_HIP<T>::initialize()
     }
     for (DeviceFloats* d : {&mSavedMean, &mSavedVariance, &mDiffScale, &mDiffBias, &mDiffSavedMean, &mDiffSavedVariance})
         d->resize(dims);
+    const size_t bytes = n2d2hip_batchnorm_f32_workspace_bytes((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW);
+    mWorkspace.resize({(bytes + sizeof(float) - 1) / sizeof(float), 1, 1, 1});
 }
 
 template <class T>
@@ -489,7 +491,7 @@ void BatchNormCell_FrameTrain_HIP<T>::propagate(bool inference)
 {
     checkStatus(n2d2hip_batchnorm_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, mIn->data(), mScale.data(), mBias.data(),
                                               mMean.data(), mVariance.data(), mSavedMean.data(), mSavedVariance.data(), mEpsilon, mMovingAverageMomentum,
-                                              inference ? 1 : 0, mOutputs.data(), mStream));
+                                              inference ? 1 : 0, mOutputs.data(), mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
     if (!inference && mMovingAverageMomentum != 0.0)
         mLearned = true;
     activationPropagate(inference);
@@ -514,7 +516,7 @@ void BatchNormCell_FrameTrain_HIP<T>::backPropagate()
     checkStatus(n2d2hip_batchnorm_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, mIn->data(), mScale.data(), mSavedMean.data(),
                                                mSavedVariance.data(), mEpsilon, mDiffInputs.data(), betaScale, mDiffScale.data(), betaBias,
                                                mDiffBias.data(), mDiffSavedMean.data(), mDiffSavedVariance.data(), toInput ? mDiffOut->data() : nullptr,
-                                               mStream));
+                                               mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
     if (toInput)
         mDiffOut->setValid();
     mDiffScale.setValid();

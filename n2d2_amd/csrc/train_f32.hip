@@ -322,6 +322,126 @@ __global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_data_kernel(siz
     }
 }
 
+// The same sums spread over `splits` blocks per channel (blockIdx.y), each adding its slice in double into a partial of
+// its own; the partials are then added in slice order, so the result does not depend on timing.
+__device__ __forceinline__ void bn_slice(size_t n, int splits, size_t* begin, size_t* end)
+{
+    const size_t chunk = (n + splits - 1) / splits;
+    *begin = (size_t)blockIdx.y * chunk;
+    *end = *begin + chunk < n ? *begin + chunk : n;
+}
+__device__ __forceinline__ double bn_total(const double* partial, int splits, int stride)
+{
+    double t = 0.0;
+    for (int s = 0; s < splits; ++s)
+        t += partial[(size_t)s * stride];
+    return t;
+}
+
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_sum_partial_kernel(int B, int C, int plane, int splits, const float* __restrict__ x,
+                                                                           double* __restrict__ ws)
+{
+    const int c = blockIdx.x;
+    size_t i0, i1;
+    bn_slice((size_t)B * plane, splits, &i0, &i1);
+    double acc = 0.0;
+    for (size_t i = i0 + threadIdx.x; i < i1; i += TBLOCK)
+        acc += (double)x[((size_t)(i / plane) * C + c) * plane + i % plane];
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0)
+        ws[(size_t)c * splits + blockIdx.y] = acc;
+}
+
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_sq_partial_kernel(int B, int C, int plane, int splits, const float* __restrict__ x,
+                                                                          const double* __restrict__ ws_sum, double* __restrict__ ws_sq)
+{
+    const int c = blockIdx.x;
+    const size_t n = (size_t)B * plane;
+    const float m = (float)(bn_total(ws_sum + (size_t)c * splits, splits, 1) / (double)n);
+    size_t i0, i1;
+    bn_slice(n, splits, &i0, &i1);
+    double acc = 0.0;
+    for (size_t i = i0 + threadIdx.x; i < i1; i += TBLOCK) {
+        const float zeroed = x[((size_t)(i / plane) * C + c) * plane + i % plane] - m;
+        acc += (double)(zeroed * zeroed);
+    }
+    acc = block_sum_d(acc);
+    if (threadIdx.x == 0)
+        ws_sq[(size_t)c * splits + blockIdx.y] = acc;
+}
+
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_stats_finish_kernel(int C, size_t n, int splits, const double* __restrict__ ws_sum,
+                                                                            const double* __restrict__ ws_sq, float* __restrict__ mean,
+                                                                            float* __restrict__ variance, float* __restrict__ saved_mean,
+                                                                            float* __restrict__ saved_variance, double momentum)
+{
+    const int c = blockIdx.x * TBLOCK + threadIdx.x;
+    if (c >= C)
+        return;
+    const float m = (float)(bn_total(ws_sum + (size_t)c * splits, splits, 1) / (double)n);
+    const float v = (float)(bn_total(ws_sq + (size_t)c * splits, splits, 1) / (double)n);
+    saved_mean[c] = m;
+    saved_variance[c] = v;
+    const float unbiased = v * ((float)n / ((float)n - 1.0f));
+    mean[c] = (float)((double)m * momentum + (double)mean[c] * (1.0 - momentum));
+    variance[c] = (float)((double)unbiased * momentum + (double)variance[c] * (1.0 - momentum));
+}
+
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_partial_kernel(int B, int C, int plane, int splits, const float* __restrict__ x,
+                                                                                const float* __restrict__ scale, const float* __restrict__ saved_mean,
+                                                                                const float* __restrict__ saved_variance, double epsilon,
+                                                                                const float* __restrict__ dy, double* __restrict__ ws)
+{
+    const int c = blockIdx.x;
+    const float m = saved_mean[c], g = scale[c];
+    const float var = (float)sqrt((double)saved_variance[c] + epsilon);
+    size_t i0, i1;
+    bn_slice((size_t)B * plane, splits, &i0, &i1);
+    double s_scale = 0.0, s_bias = 0.0, s_mean1 = 0.0, s_mean2 = 0.0, s_var = 0.0;
+    for (size_t i = i0 + threadIdx.x; i < i1; i += TBLOCK) {
+        const size_t idx = ((size_t)(i / plane) * C + c) * plane + i % plane;
+        const float centred = x[idx] - m;
+        const float normalized = centred / var;
+        const float d = dy[idx];
+        const float diff_normalized = d * g;
+        s_scale += (double)(d * normalized);
+        s_bias += (double)d;
+        s_mean1 += (double)diff_normalized;
+        s_mean2 += (double)(float)(-2.0 * (double)centred);
+        s_var += (double)(diff_normalized * centred);
+    }
+    s_scale = block_sum_d(s_scale);
+    s_bias = block_sum_d(s_bias);
+    s_mean1 = block_sum_d(s_mean1);
+    s_mean2 = block_sum_d(s_mean2);
+    s_var = block_sum_d(s_var);
+    if (threadIdx.x == 0) {
+        double* o = ws + ((size_t)c * splits + blockIdx.y) * 5;
+        o[0] = s_scale; o[1] = s_bias; o[2] = s_mean1; o[3] = s_mean2; o[4] = s_var;
+    }
+}
+
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_finish_kernel(int C, size_t n, int splits, const double* __restrict__ ws,
+                                                                               const float* __restrict__ saved_variance, double epsilon,
+                                                                               float beta_scale, float* __restrict__ diff_scale, float beta_bias,
+                                                                               float* __restrict__ diff_bias, float* __restrict__ diff_saved_mean,
+                                                                               float* __restrict__ diff_saved_variance)
+{
+    const int c = blockIdx.x * TBLOCK + threadIdx.x;
+    if (c >= C)
+        return;
+    const double* p = ws + (size_t)c * splits * 5;
+    const float sum_scale = (float)bn_total(p + 0, splits, 5), sum_bias = (float)bn_total(p + 1, splits, 5);
+    const float sum_mean1 = (float)bn_total(p + 2, splits, 5), sum_mean2 = (float)bn_total(p + 3, splits, 5);
+    const float sum_var = (float)bn_total(p + 4, splits, 5);
+    const float var = (float)sqrt((double)saved_variance[c] + epsilon);
+    const float dv = (float)((double)sum_var * (-1.0 / 2.0) * pow((double)saved_variance[c] + epsilon, -3.0 / 2.0));
+    diff_saved_variance[c] = dv;
+    diff_saved_mean[c] = (float)((double)sum_mean1 * (-1.0 / (double)var) + (double)(dv * sum_mean2 / (float)n));
+    diff_scale[c] = sum_scale + (beta_scale != 0.0f ? beta_scale * diff_scale[c] : 0.0f);
+    diff_bias[c] = sum_bias + (beta_bias != 0.0f ? beta_bias * diff_bias[c] : 0.0f);
+}
+
 struct PoolF32 {
     int B, C, H, W, oH, oW, pw, ph, sx, sy, px, py;
 };
@@ -618,9 +738,25 @@ int n2d2hip_rectifier_f32_backward(const float* output, const float* diff_in, fl
     return N2D2HIP_OK;
 }
 
+// Blocks per channel for the sums over batch and pixels: about 1024 blocks in all, at least 4096 values each, at most 64.
+static int bn_splits(int B, int C, int H, int W)
+{
+    const size_t n = (size_t)B * H * W;
+    const size_t by_size = n / 4096;
+    const size_t by_grid = (size_t)std::max(1024 / C, 1);
+    return (int)std::max<size_t>(1, std::min<size_t>(std::min(by_size, by_grid), 64));
+}
+
+size_t n2d2hip_batchnorm_f32_workspace_bytes(int B, int C, int H, int W)
+{
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0)
+        return 0;
+    return (size_t)C * bn_splits(B, C, H, W) * 5 * sizeof(double);
+}
+
 int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, const float* scale, const float* bias, float* mean,
                                   float* variance, float* saved_mean, float* saved_variance, double epsilon, double moving_average_momentum,
-                                  int use_running, float* y, n2d2hip_stream_t stream)
+                                  int use_running, float* y, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
 {
     N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && bias && mean && variance && y && epsilon > 0.0, N2D2HIP_ERR_INVALID,
                     "n2d2hip_batchnorm_f32_forward: bad argument");
@@ -630,8 +766,20 @@ int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, co
     if (!running) {
         N2D2HIP_REQUIRE(saved_mean && saved_variance, N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: the learning pass needs saved_mean and saved_variance");
         N2D2HIP_REQUIRE((size_t)B * H * W > 1, N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: batch statistics need more than one value per channel");
-        hipLaunchKernelGGL(batchnorm_f32_stats_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, mean, variance, saved_mean,
-                           saved_variance, moving_average_momentum);
+        const int splits = bn_splits(B, C, H, W);
+        if (splits > 1 && workspace && workspace_bytes >= n2d2hip_batchnorm_f32_workspace_bytes(B, C, H, W)) {
+            double* ws_sum = (double*)workspace;
+            double* ws_sq = ws_sum + (size_t)C * splits;
+            hipLaunchKernelGGL(batchnorm_f32_sum_partial_kernel, dim3(C, splits), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, splits, x, ws_sum);
+            hipLaunchKernelGGL(batchnorm_f32_sq_partial_kernel, dim3(C, splits), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, splits, x,
+                               (const double*)ws_sum, ws_sq);
+            hipLaunchKernelGGL(batchnorm_f32_stats_finish_kernel, dim3((C + TBLOCK - 1) / TBLOCK), dim3(TBLOCK), 0, (hipStream_t)stream, C,
+                               (size_t)B * H * W, splits, (const double*)ws_sum, (const double*)ws_sq, mean, variance, saved_mean, saved_variance,
+                               moving_average_momentum);
+        } else {
+            hipLaunchKernelGGL(batchnorm_f32_stats_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, mean, variance, saved_mean,
+                               saved_variance, moving_average_momentum);
+        }
     }
     hipLaunchKernelGGL(batchnorm_f32_apply_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W, x, scale, bias,
                        running ? (const float*)mean : (const float*)saved_mean, running ? (const float*)variance : (const float*)saved_variance, epsilon,
@@ -643,15 +791,24 @@ int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, co
 int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, const float* scale, const float* saved_mean,
                                    const float* saved_variance, double epsilon, const float* diff_y, float beta_scale, float* diff_scale,
                                    float beta_bias, float* diff_bias, float* diff_saved_mean, float* diff_saved_variance, float* diff_x,
-                                   n2d2hip_stream_t stream)
+                                   void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream)
 {
     N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && saved_mean && saved_variance && diff_y && diff_scale && diff_bias
                         && diff_saved_mean && diff_saved_variance && epsilon > 0.0,
                     N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: bad argument");
     N2D2HIP_REQUIRE((size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: tensor too large");
     const size_t total = (size_t)B * C * H * W;
-    hipLaunchKernelGGL(batchnorm_f32_backward_sums_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, scale, saved_mean,
-                       saved_variance, epsilon, diff_y, beta_scale, diff_scale, beta_bias, diff_bias, diff_saved_mean, diff_saved_variance);
+    const int splits = bn_splits(B, C, H, W);
+    if (splits > 1 && workspace && workspace_bytes >= n2d2hip_batchnorm_f32_workspace_bytes(B, C, H, W)) {
+        hipLaunchKernelGGL(batchnorm_f32_backward_partial_kernel, dim3(C, splits), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, splits, x, scale,
+                           saved_mean, saved_variance, epsilon, diff_y, (double*)workspace);
+        hipLaunchKernelGGL(batchnorm_f32_backward_finish_kernel, dim3((C + TBLOCK - 1) / TBLOCK), dim3(TBLOCK), 0, (hipStream_t)stream, C,
+                           (size_t)B * H * W, splits, (const double*)workspace, saved_variance, epsilon, beta_scale, diff_scale, beta_bias, diff_bias,
+                           diff_saved_mean, diff_saved_variance);
+    } else {
+        hipLaunchKernelGGL(batchnorm_f32_backward_sums_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, scale, saved_mean,
+                           saved_variance, epsilon, diff_y, beta_scale, diff_scale, beta_bias, diff_bias, diff_saved_mean, diff_saved_variance);
+    }
     if (diff_x)
         hipLaunchKernelGGL(batchnorm_f32_backward_data_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W,
                            (float)((size_t)B * H * W), x, scale, saved_mean, saved_variance, epsilon, diff_y, (const float*)diff_saved_mean,
