@@ -29,7 +29,7 @@ HipTensor::~HipTensor()
         (void)hipFree(mDesc.data);
 }
 
-void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo)
+void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo, bool stimuli)
 {
     n2d2hip_tensor d = {};
     d.data = nullptr;
@@ -37,7 +37,7 @@ void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo)
     d.dtype = dtype;
     d.layout = N2D2HIP_NHWC;
     d.B = B; d.C = C; d.H = H; d.W = W;
-    d.cs = n2d2hip_nhwc_cs(C);
+    d.cs = stimuli ? n2d2hip_nhwc_cs(C) : (C + 15) / 16 * 16;
     const size_t bytes = n2d2hip_tensor_bytes(&d);
     if (mDesc.data && bytes == mBytes) {
         d.data = mDesc.data;
@@ -1337,7 +1337,7 @@ void DeepNet::setStimuliData(const Tensor<Float_T>& data)
     // network input unsigned <=> DeepNetExport::mEnvDataUnsigned (StimuliProviderExport::unsignedStimuli)
     const int dtype = (CellExport::mPrecision > 0 && DeepNetExport::mUnsignedData && DeepNetExport::mEnvDataUnsigned) ? N2D2HIP_U8B : N2D2HIP_I8;
     if (mStimuli.empty() || mStimuli.desc().dtype != dtype)
-        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype);
+        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype, 0, true);
     for (size_t i = 0; i < data.size(); ++i)
         toInteger(data(i), dtype == N2D2HIP_U8B ? 0 : -128, dtype == N2D2HIP_U8B ? 255 : 127, "stimuli");
     mStimuli.synchronizeHToD(data);
@@ -1347,7 +1347,7 @@ void DeepNet::initialize()
 {
     const int dtype = (CellExport::mPrecision > 0 && DeepNetExport::mUnsignedData && DeepNetExport::mEnvDataUnsigned) ? N2D2HIP_U8B : N2D2HIP_I8;
     if (mEnvB > 0 && mStimuli.empty())
-        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype);
+        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype, 0, true);
     for (auto& c : mOrder)
         std::dynamic_pointer_cast<Cell_Frame_HIP>(c)->initialize();
 }

@@ -128,8 +128,10 @@ public:
     ~HipTensor();
     HipTensor(const HipTensor&) = delete;
     HipTensor& operator=(const HipTensor&) = delete;
-    // halo: border pixels stored around every image, holding the value 0 (tensors between two convolutions)
-    void resize(int B, int C, int H, int W, int dtype, int halo = 0);
+    // halo: border pixels stored around every image, holding the value 0 (tensors between two convolutions).
+    // stimuli: the network's input, which may use the 4-byte channel stride the first-layer kernel reads; what a cell
+    // writes always has a stride that is a multiple of 16.
+    void resize(int B, int C, int H, int W, int dtype, int halo = 0, bool stimuli = false);
     const n2d2hip_tensor& desc() const { return mDesc; }
     bool empty() const { return mDesc.data == nullptr; }
     void invalidateHost() { mHostValid = false; }
@@ -767,6 +769,9 @@ public:
     virtual ~QuantizerCell() {}
     void setRange(std::size_t range) { mRange = range; }
     void setQuantMode(QuantMode mode) { mQuantMode = mode; }
+    std::size_t getRange() const { return mRange; }
+    QuantMode getQuantMode() const { return mQuantMode; }
+    virtual const char* getType() const = 0;
     void setSolver(const std::shared_ptr<SGDSolver>& solver) { mSolver = solver; }
     // device float buffers of n weights: full precision, and the gradient w.r.t. the quantized weights
     virtual void addWeights(float* weights, float* diffQuantizedWeights, std::size_t size, std::size_t outputsSize) = 0;
@@ -795,8 +800,10 @@ public:
     typedef std::function<std::shared_ptr<SATQuantizerCell>()> RegistryCreate_T;
     static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
     static const char* Type;
+    const char* getType() const { return Type; }
     void setQuantization(bool v) { mApplyQuantization = v; }
     void setScaling(bool v) { mApplyScaling = v; }
+    bool getScaling() const { return mApplyScaling; }
 protected:
     SATQuantizerCell() : mApplyQuantization(true), mApplyScaling(false) {}
     bool mApplyQuantization, mApplyScaling;
@@ -835,6 +842,8 @@ class QuantizerActivation {
 public:
     virtual ~QuantizerActivation() {}
     void setRange(std::size_t range) { mRange = range; }
+    std::size_t getRange() const { return mRange; }
+    virtual const char* getType() const = 0;
     void setSolver(const std::shared_ptr<SGDSolver>& solver) { mSolver = solver; }
     // in-place on a device float buffer
     virtual void propagate(float* inOut, std::size_t size, bool inference) = 0;
@@ -853,6 +862,7 @@ public:
     typedef std::function<std::shared_ptr<SATQuantizerActivation>()> RegistryCreate_T;
     static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
     static const char* Type;
+    const char* getType() const { return Type; }
     void setAlpha(double alpha) { mAlphaParameter = alpha; }
 protected:
     SATQuantizerActivation() : mAlphaParameter(1.0) {}
@@ -892,6 +902,7 @@ public:
     typedef std::function<std::shared_ptr<LSQQuantizerCell>()> RegistryCreate_T;
     static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
     static const char* Type;
+    const char* getType() const { return Type; }
     void setStepSizeValue(float v) { mStepSizeVal = v; }
     void setOptInitStepSize(bool v) { mSetOptInitStepSize = v; }
 protected:
@@ -935,6 +946,7 @@ public:
     typedef std::function<std::shared_ptr<LSQQuantizerActivation>()> RegistryCreate_T;
     static RegistryMap_T& registry() { static RegistryMap_T rMap; return rMap; }
     static const char* Type;
+    const char* getType() const { return Type; }
     void setStepSizeValue(float v) { mStepSizeParameter = v; }
     void setOptInitStepSize(bool v) { mSetOptInitStepSize = v; }
 protected:

@@ -399,6 +399,9 @@ int fh_cell_get_outputs(void* net, const char* name, float* out, size_t n)
     });
 }
 
+// The DeepNet behind a net handle, for the hooks of other files that fill its cells
+void* fh_net_deepnet(void* net) { return ((Net*)net)->deepNet.get(); }
+
 int fh_cell_get_max_output(void* net, const char* name, unsigned int batchPos, unsigned int* out)
 {
     return guarded([&] {

@@ -253,6 +253,22 @@ Tensor<Float_T> WeightedCell_FrameTrain_HIP::getQuantizedWeights() const
     return host;
 }
 
+QATCellParameters WeightedCell_FrameTrain_HIP::getQATCellParameters()
+{
+    QATCellParameters p;
+    p.quantWeights = getQuantizedWeights();
+    synchronizeWeightsToHost();
+    if (!mDevBias.empty())
+        p.biases = mDevBias.toHost();
+    if (mQuantizer) {
+        p.weightsRange = mQuantizer->getRange();
+        p.defaultQuantMode = mQuantizer->getQuantMode() == QuantizerCell::Default;
+        if (auto sat = std::dynamic_pointer_cast<SATQuantizerCell_Frame_HIP<float> >(mQuantizer))
+            p.satScaling = sat->getScaling() ? (double)sat->getStats(0).second : 1.0;
+    }
+    return p;
+}
+
 // ------------------------------------------------------ ConvCell_FrameTrain_HIP
 template <class T>
 ConvCell_FrameTrain_HIP<T>::ConvCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, const std::vector<unsigned int>& kernelDims,
@@ -463,6 +479,25 @@ std::vector<Float_T> BatchNormCell_FrameTrain_HIP<T>::get(const DeviceFloats& de
     checkHipT(hipStreamSynchronize((hipStream_t)mStream), "BatchNormCell_FrameTrain_HIP: synchronize");
     const Tensor<Float_T> t = dev.toHost();
     return std::vector<Float_T>(t.data(), t.data() + t.size());
+}
+
+template <class T>
+BatchNormParameters BatchNormCell_FrameTrain_HIP<T>::getBatchNormParameters() const
+{
+    BatchNormParameters p;
+    const std::vector<Float_T> s = getScales(), b = getBiases(), m = getMeans(), v = getVariances();
+    p.scales.assign(s.begin(), s.end());
+    p.biases.assign(b.begin(), b.end());
+    p.means.assign(m.begin(), m.end());
+    p.variances.assign(v.begin(), v.end());
+    p.epsilon = mEpsilon;
+    if (mActivation && mActivation->getQuantizer()) {
+        if (auto sat = std::dynamic_pointer_cast<SATQuantizerActivation_Frame_HIP<float> >(mActivation->getQuantizer())) {
+            p.actRange = sat->getRange();
+            p.actAlpha = sat->getAlpha();
+        }
+    }
+    return p;
 }
 
 template <class T>

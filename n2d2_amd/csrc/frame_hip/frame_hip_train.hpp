@@ -96,6 +96,9 @@ public:
     void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
     Tensor<Float_T> getDiffWeights() const { return mDevDiffW.toHost(); }
     Tensor<Float_T> getQuantizedWeights() const;
+    // What DeepNetQAT reads of this cell once it has propagated: the weight quantizer's tensor (the weights themselves
+    // without one), the biases, the quantizer's range, mode and SAT divisor
+    QATCellParameters getQATCellParameters();
     // refreshes the host tensors getWeights() / getBiases() return from the device
     virtual void synchronizeWeightsToHost() = 0;
 
@@ -251,6 +254,9 @@ public:
     void setBiasSolver(const std::shared_ptr<SGDSolver>& solver) { mBiasSolver = solver; }
     const std::shared_ptr<SGDSolver>& getScaleSolver() const { return mScaleSolver; }
     const std::shared_ptr<SGDSolver>& getBiasSolver() const { return mBiasSolver; }
+    // What DeepNetQAT reads of this cell: the four vectors, Epsilon, and range and alpha of the SAT quantizer of its
+    // activation (range 0 without one)
+    BatchNormParameters getBatchNormParameters() const;
 
 protected:
     void setOutputsDims() { mOutW = mInW; mOutH = mInH; }

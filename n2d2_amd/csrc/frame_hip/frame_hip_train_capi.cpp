@@ -317,6 +317,62 @@ int fh_train_learn(void* net, const float* targets, size_t nTargets, int iterati
     });
 }
 
+// The chain case of DeepNetQAT::fuseQATGraph (src/Quantizer/QAT/Optimization/DeepNetQAT.cpp:87-520): walks the learning
+// cells front to back with the (range, alpha) pairs starting at (255, 255) / (1, 1); every Conv followed by a BatchNorm is
+// fused into the integer Conv cell of the same name in `deepNet`, every Fc quantized into the integer Fc of the same name;
+// pooling, activation and softmax cells leave the pairs alone.  The learning cells must have propagated once (their
+// quantizers hold the quantized weights then).  nbFused receives the number of integer cells filled.
+int fh_train_fuse_into(void* net, void* deepNet, int actScalingMode, int wMode, int bMode, int cMode, int* nbFused)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        DeepNet& target = *(DeepNet*)deepNet;
+        const ScalingMode mode = actScalingMode == N2D2HIP_SCALING_FLOAT_MULT ? ScalingMode::FLOAT_MULT
+                                 : actScalingMode == N2D2HIP_SCALING_FIXED_MULT16 ? ScalingMode::FIXED_MULT16
+                                 : actScalingMode == N2D2HIP_SCALING_FIXED_MULT32 ? ScalingMode::FIXED_MULT32
+                                 : actScalingMode == N2D2HIP_SCALING_SINGLE_SHIFT ? ScalingMode::SINGLE_SHIFT : ScalingMode::NONE;
+        const WeightsApprox w = wMode ? WeightsApprox::RINTF : WeightsApprox::NONE, b = bMode ? WeightsApprox::RINTF : WeightsApprox::NONE,
+                            c = cMode ? WeightsApprox::RINTF : WeightsApprox::NONE;
+        std::pair<std::size_t, std::size_t> ranges(255, 255);
+        std::pair<double, double> alphas(1.0, 1.0);
+        int count = 0;
+        for (std::size_t i = 0; i < n.cells.size(); ++i) {
+            Cell_FrameTrain_HIP* cell = n.cells[i].get();
+            if (auto conv = dynamic_cast<ConvCell_FrameTrain_HIP<float>*>(cell)) {
+                auto bn = i + 1 < n.cells.size() ? dynamic_cast<BatchNormCell_FrameTrain_HIP<float>*>(n.cells[i + 1].get()) : nullptr;
+                if (!bn)
+                    throw std::runtime_error("fh_train_fuse_into(): Conv \"" + conv->getName() + "\" is not followed by a BatchNorm");
+                auto dst = std::dynamic_pointer_cast<ConvCell>(target.getCell(conv->getName()));
+                if (!dst)
+                    throw std::runtime_error("fh_train_fuse_into(): no integer Conv named \"" + conv->getName() + "\"");
+                if (i == 0)
+                    ranges.first = 255;         // the stimuli: 8 bits
+                if (!DeepNetQAT::QuantizeAndfuseBatchNormWithConv(ranges, alphas, *dst, conv->getQATCellParameters(), bn->getBatchNormParameters(),
+                                                                  mode, w, b, c))
+                    throw std::runtime_error("fh_train_fuse_into(): \"" + bn->getName() + "\" cannot be fused with \"" + conv->getName() + "\"");
+                ++count;
+                ++i;
+            } else if (auto fc = dynamic_cast<FcCell_FrameTrain_HIP<float>*>(cell)) {
+                auto dst = std::dynamic_pointer_cast<FcCell>(target.getCell(fc->getName()));
+                if (!dst)
+                    throw std::runtime_error("fh_train_fuse_into(): no integer Fc named \"" + fc->getName() + "\"");
+                std::size_t actRange = 0;
+                double actAlpha = 0.0;
+                if (fc->getActivation() && fc->getActivation()->getQuantizer()) {
+                    auto sat = std::dynamic_pointer_cast<SATQuantizerActivation_Frame_HIP<float> >(fc->getActivation()->getQuantizer());
+                    if (!sat)
+                        throw std::runtime_error("fh_train_fuse_into(): only SAT activation quantizers can be fused (\"" + fc->getName() + "\")");
+                    actRange = sat->getRange();
+                    actAlpha = sat->getAlpha();
+                }
+                DeepNetQAT::QuantizeFC(ranges, alphas, *dst, fc->getQATCellParameters(), actRange, actAlpha, w, b, c);
+                ++count;
+            }
+        }
+        if (nbFused) *nbFused = count;
+    });
+}
+
 // One forward pass; inference != 0 runs the quantizers without saving what backPropagate needs
 int fh_train_propagate(void* net, int inference)
 {

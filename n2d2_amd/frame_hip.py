@@ -348,6 +348,9 @@ lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
 lib.fh_train_add_batchnorm.argtypes = [_P, C.c_char_p, _P, C.c_double, C.c_double, _I, _I, _I, _F]
 lib.fh_train_get_batchnorm.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
 lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I]
+lib.fh_net_deepnet.argtypes = [_P]
+lib.fh_net_deepnet.restype = C.c_void_p
+lib.fh_train_fuse_into.argtypes = [_P, _P, _I, _I, _I, _I, _P]
 lib.fh_train_add_fc.argtypes = [_P, C.c_char_p, _I, _P, _P, _I, _I, _I, _F, _I, _I, _I]
 lib.fh_train_set_solver_parameter.argtypes = [_P, C.c_char_p, C.c_char_p, C.c_double]
 lib.fh_train_learn.argtypes = [_P, _P, _SZ, _I, _P]
@@ -453,6 +456,15 @@ class TrainNet:
     def add_softmax(self, name, with_loss=True):
         _check_train(lib.fh_train_add_softmax(self._h, name.encode(), int(with_loss)))
         self._shapes[name] = self._last
+
+    def fuse_into(self, net, mode="FloatMult", w_round=True, b_round=True, c_round=True):
+        """The chain case of DeepNetQAT::fuseQATGraph: fills the integer Conv / Fc cells of `net` (a Net of Frame_HIP cells with
+        the same cell names) from this net's trained cells, each Conv with the BatchNorm that follows it.  The learning cells
+        must have propagated once.  Returns the number of integer cells filled."""
+        count = C.c_int(0)
+        _check_train(lib.fh_train_fuse_into(self._h, lib.fh_net_deepnet(net.h), _MODE[mode], int(w_round), int(b_round), int(c_round),
+                                            C.byref(count)))
+        return count.value
 
     def set_solver_parameter(self, cell, name, value):
         _check_train(lib.fh_train_set_solver_parameter(self._h, cell.encode(), name.encode(), float(value)))

@@ -357,5 +357,114 @@ def test_trained_lenet_float_graph_and_its_integer_twin_agree_on_the_gpu(name):
             dev = np.abs(fused.outputs(conv) - got)
             assert dev.max() <= (6 if R == 255 else 1) and dev.mean() < (0.3 if R == 255 else 0.06), conv
             assert np.unique(got).size > 4
+        # the same pass fed from the learning cells themselves (their quantizers' tensors on the device, the BatchNorm
+        # cells' vectors): the same integer net but for a weight that sits within rounding of a tie
+        twin = fh.Net(sl.INI % 32)
+        assert net.fuse_into(twin) == 5
+        for pool in ("pool1", "pool2"):
+            twin.set_quantized(pool, 8)
+        for cell in ("conv1", "conv2", "conv3", "fc1", "fc2"):
+            a, b = twin.weights(cell), fused.weights(cell)
+            assert (a != b).mean() < 2e-3 and np.abs(a - b).max() <= 1, cell
+            # (the Fc cells' SAT divisor comes from a variance summed on the device in another order than the oracle's)
+            assert np.allclose(twin.scaling(cell)[2], fused.scaling(cell)[2], rtol=1e-4), cell
+            assert np.allclose(twin.clipping(cell), fused.clipping(cell), rtol=1e-4, atol=1.0), cell
+            assert twin.quantized(cell) == fused.quantized(cell), cell
+        twin.set_fusion(False)
+        twin.initialize()
+        twin.set_stimuli(imgs)
+        twin.propagate()
+        for cell in ("conv1", "conv3", "fc2"):
+            assert (twin.outputs(cell) != fused.outputs(cell)).mean() < 0.02, cell
+    finally:
+        fh.set_globals(0, True, False)
+
+
+LEARN_INI = """
+DefaultModel=Frame_HIP
+
+[sp]
+SizeX=12
+SizeY=12
+NbChannels=1
+BatchSize=8
+
+[c1]
+Input=sp
+Type=Conv
+KernelDims=3 3
+NbOutputs=6
+ActivationFunction=Linear
+
+[pool]
+Input=c1
+Type=Pool
+PoolDims=2 2
+NbOutputs=6
+Stride=2
+Pooling=Max
+
+[c2]
+Input=pool
+Type=Conv
+KernelDims=3 3
+NbOutputs=8
+ActivationFunction=Linear
+
+[fc]
+Input=c2
+Type=Fc
+NbOutputs=3
+ActivationFunction=Linear
+"""
+
+
+def test_learn_then_fuse_then_infer_without_leaving_the_gpu():
+    """Quantization-aware learning on the float cells, the pass to integer cells fed from them, integer inference: the
+    integer net reproduces the levels of the float net it was made from."""
+    from n2d2_amd import frame_hip as fh
+    rng = np.random.default_rng(41)
+    imgs = rng.integers(0, 256, size=(8, 1, 12, 12)).astype(np.float32)
+    x = (imgs / np.float32(255)).astype(np.float32)
+    t = np.zeros((8, 3, 1, 1), dtype=np.float32)
+    t[np.arange(8), rng.integers(0, 3, size=8)] = 1
+    net = fh.TrainNet(x, propagate_gradient=False)
+    # (8-bit weights in the first cell, as in the reference's models: the pass rescales 4-bit default-mode weights to 5 bits
+    # and then takes the cell's *input* range to be 31 as well, which only fits inputs that have 15 levels)
+    net.add_conv("c1", rng.normal(0, 0.4, size=(6, 1, 3, 3)), weight_quant="SAT", weight_range=255, act="Linear")
+    net.add_batchnorm("bn1", act="Linear", act_quant="SAT", act_range=15, act_param=3.0)
+    net.add_pool("pool", (2, 2), (2, 2))
+    net.add_conv("c2", rng.normal(0, 0.3, size=(8, 6, 3, 3)), weight_quant="SAT", weight_range=15, act="Linear")
+    net.add_batchnorm("bn2", act="Linear", act_quant="SAT", act_range=15, act_param=3.0)
+    net.add_fc("fc", rng.normal(0, 0.2, size=(3, 8 * 3 * 3)), act="Linear", act_quant="SAT", act_range=255, act_param=4.0, weight_quant="SAT",
+               weight_range=255, apply_scaling=True)
+    net.add_softmax("softmax", with_loss=True)
+    print("learn, fuse, infer", flush=True)
+    first = net.learn(t, 1)
+    last = net.learn(t, 60)
+    assert np.isfinite(last) and last < first
+    net.propagate(inference=True)
+    levels = {bn: np.rint(net.outputs(bn) * np.float32(15 / net.activation_quantizer(bn)[0])) for bn in ("bn1", "bn2")}
+    twin = fh.Net(LEARN_INI)
+    assert net.fuse_into(twin) == 3
+    twin.set_quantized("pool", 8)
+    assert twin.quantized("c1") == (8, 4, "Rectifier") and twin.quantized("c2") == (4, 4, "Rectifier") and twin.quantized("fc") == (8, 8, "Linear")
+    try:
+        fh.set_globals(8, True, True)
+        twin.set_fusion(False)
+        twin.initialize()
+        twin.set_stimuli(imgs)
+        twin.propagate()
+        for conv, bn in (("c1", "bn1"), ("c2", "bn2")):
+            dev = np.abs(twin.outputs(conv) - levels[bn])
+            # one level at most; the second stage also inherits the first one's deviations through its 54 inputs per output
+            assert dev.max() <= 1 and dev.mean() < (0.05 if conv == "c1" else 0.15) and np.unique(levels[bn]).size > 4, conv
+        # the Fc stage from the integer graph's own input (one input level moves an output by several of its 255): the
+        # float cell's quantized weights on c2's levels, the SAT activation, and the signed saturation N2D2 applies to a
+        # Linear cell (levels above 127)
+        alpha, a2 = net.activation_quantizer("fc")[0], net.activation_quantizer("bn2")[0]
+        z = (twin.outputs("c2").reshape(8, -1).astype(np.float64) * a2 / 15) @ net.quantized_weights("fc").astype(np.float64).T
+        want = np.minimum(np.rint(np.clip(z, 0, alpha) / alpha * 255), 127).reshape(8, 3, 1, 1)
+        assert np.abs(twin.outputs("fc") - want).max() <= 1 and np.unique(want).size > 2
     finally:
         fh.set_globals(0, True, False)
