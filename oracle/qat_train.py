@@ -6,7 +6,10 @@ ActivationCell / ConvCell / BatchNormCell / PoolCell / SoftmaxCell with SAT quan
 Pinned by tests/test_oracle_qat_train.py: closed forms for the solver, softmax and loss, and the reference's own
 known-answer tests (tests/Cell/class_ConvCell_QuantizerSAT_Frame.cpp, class_ConvCell_QuantizerLSQ_Frame_CUDA.cpp,
 class_FcCell_QuantizerLSQ_Frame_CUDA.cpp: trained SAT alphas and LSQ step sizes derived from PyTorch by the
-reference's authors), which exercise every class below in the order the reference's learning loop calls them.
+reference's authors), which exercise every class below in the order the reference's learning loop calls them, but
+BatchNormCell and PoolCell, for which the reference's tests hold no values: textbook batch normalisation in float64
+(outputs, running statistics, the three gradients by the closed form), and the directional derivative of max pooling.
+Parity unpinned, by nature: the order of BatchNormCell's float sums over batch and pixels.
 
 Data is float32 as in the `<float>` instantiations; "diff" tensors carry the
 descent direction (target - output at the loss), so a solver *adds*
