@@ -118,6 +118,52 @@ def qat_conv_step(torch, steps=10):
             "finite": bool(torch.isfinite(w).all().item() and torch.isfinite(alpha).all().item())}
 
 
+def qat_batchnorm_step(torch, steps=10):
+    """BatchNorm of the same learning graph (64 channels on 56x56, batch 64, float32): learning forward (batch statistics,
+    running statistics, normalisation) and backward (parameter and input gradients) through the C ABI, timed with events
+    on the stream the kernels are launched on; bytes are the algorithmic ones, 16 and 20 per value."""
+    from n2d2_amd import capi, runtime
+    lib, sp, chk = capi.lib, runtime.stream_ptr, capi.check
+    B, Cn, H = 64, 64, 56
+    n = B * Cn * H * H
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    f32 = dict(dtype=torch.float32, device="cuda")
+    x, dy = torch.randn(n, generator=gen, **f32), torch.randn(n, generator=gen, **f32)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    vec = lambda v: torch.full((Cn,), v, **f32)
+    scale, bias, mean, var, smean, svar, dscale, dbias, dsm, dsv = (vec(1.0), vec(0.0), vec(0.0), vec(1.0), vec(0.0), vec(1.0), vec(0.0), vec(0.0),
+                                                                    vec(0.0), vec(0.0))
+    nws = int(lib.n2d2hip_batchnorm_f32_workspace_bytes(B, Cn, H, H))
+    ws = torch.empty(nws, dtype=torch.uint8, device="cuda")
+
+    def fwd():
+        chk(lib.n2d2hip_batchnorm_f32_forward(B, Cn, H, H, x.data_ptr(), scale.data_ptr(), bias.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                              smean.data_ptr(), svar.data_ptr(), 1e-5, 0.1, 0, y.data_ptr(), ws.data_ptr(), nws, sp()))
+
+    def bwd():
+        chk(lib.n2d2hip_batchnorm_f32_backward(B, Cn, H, H, x.data_ptr(), scale.data_ptr(), smean.data_ptr(), svar.data_ptr(), 1e-5, dy.data_ptr(),
+                                               0.0, dscale.data_ptr(), 0.0, dbias.data_ptr(), dsm.data_ptr(), dsv.data_ptr(), dx.data_ptr(),
+                                               ws.data_ptr(), nws, sp()))
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+    tf, tb = timed(fwd), timed(bwd)
+    gf, gb = 16.0 * n / (tf * 1e-3) / 1e9, 20.0 * n / (tb * 1e-3) / 1e9
+    return {"workload": "BatchNorm learning pass, 64 channels on 56x56, batch 64, float32", "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "forward": {"us": round(tf * 1e3, 1), "achieved": round(gf, 1), "frac": round(gf / PEAK_HBM_GBS, 4)},
+            "backward": {"us": round(tb * 1e3, 1), "achieved": round(gb, 1), "frac": round(gb / PEAK_HBM_GBS, 4)},
+            "finite": bool(torch.isfinite(y).all().item() and torch.isfinite(dx).all().item())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -293,6 +339,10 @@ def main():
         result["qat_conv_iteration"] = qat_conv_step(torch)
     except Exception as e:       # the side figure must not take the headline down with it
         result["qat_conv_iteration"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    try:
+        result["qat_batchnorm"] = qat_batchnorm_step(torch)
+    except Exception as e:
+        result["qat_batchnorm"] = {"error": "%s: %s" % (type(e).__name__, e)}
     if not args.no_cpu_baseline:
         base, exact = cpu_baseline(spec, logits, images)
         result["cpu_baseline"] = base
