@@ -253,7 +253,38 @@ __global__ __launch_bounds__(TBLOCK) void batchnorm_f32_stats_kernel(int B, int 
 
 // y = scale * (x - mean) / sqrt(variance + epsilon) + bias.  eps_in_float: the inference branch of the reference adds
 // the epsilon in float and takes a float square root; the learning branch adds the double and rounds the root.
-__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_apply_kernel(size_t total, int C, int plane, const float* __restrict__ x,
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_apply_kernel(int planes, int C, int plane, const float* __restrict__ x,
+                                                                     const float* __restrict__ scale, const float* __restrict__ bias,
+                                                                     const float* __restrict__ mean, const float* __restrict__ variance, double epsilon,
+                                                                     int eps_in_float, int vec, float* __restrict__ y)
+{
+    // blockIdx.y walks the (batch, channel) planes, so that the channel's constants are worked out once per plane;
+    // planes whose size is a multiple of 4 move 16 bytes per lane
+    for (int bc = blockIdx.y; bc < planes; bc += gridDim.y) {
+        const int c = bc % C;
+        const float var = eps_in_float ? sqrtf(variance[c] + (float)epsilon) : (float)sqrt((double)variance[c] + epsilon);
+        const float m = mean[c], g = scale[c], b = bias[c];
+        const float* xp = x + (size_t)bc * plane;
+        float* yp = y + (size_t)bc * plane;
+        if (vec) {
+            for (int i = blockIdx.x * TBLOCK + threadIdx.x; i < plane / 4; i += gridDim.x * TBLOCK) {
+                const float4 v = ((const float4*)xp)[i];
+                float4 o;
+                o.x = g * ((v.x - m) / var) + b;
+                o.y = g * ((v.y - m) / var) + b;
+                o.z = g * ((v.z - m) / var) + b;
+                o.w = g * ((v.w - m) / var) + b;
+                ((float4*)yp)[i] = o;
+            }
+        } else {
+            for (int i = blockIdx.x * TBLOCK + threadIdx.x; i < plane; i += gridDim.x * TBLOCK)
+                yp[i] = g * ((xp[i] - m) / var) + b;
+        }
+    }
+}
+
+// The same for small planes: one lane per value, the channel found by division.
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_apply_flat_kernel(size_t total, int C, int plane, const float* __restrict__ x,
                                                                      const float* __restrict__ scale, const float* __restrict__ bias,
                                                                      const float* __restrict__ mean, const float* __restrict__ variance, double epsilon,
                                                                      int eps_in_float, float* __restrict__ y)
@@ -305,8 +336,46 @@ __global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_sums_kernel(int
     }
 }
 
-// dx = dy * scale / sigma + dVar * 2 (x - mean) / size + dMean / size
-__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_data_kernel(size_t total, int C, int plane, float size, const float* __restrict__ x,
+// dx = dy * scale / sigma + dVar * 2 (x - mean) / size + dMean / size, plane by plane as the apply kernel
+__device__ __forceinline__ float bn_dx(float x, float d, float g, float var, float m, double dv2, double size, double dmean_over_size)
+{
+    const float diff_normalized = d * g;
+    return (float)((double)(diff_normalized / var) + dv2 * (double)(x - m) / size + dmean_over_size);
+}
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_data_kernel(int planes, int C, int plane, float size, const float* __restrict__ x,
+                                                                            const float* __restrict__ scale, const float* __restrict__ saved_mean,
+                                                                            const float* __restrict__ saved_variance, double epsilon, const float* dy,
+                                                                            const float* __restrict__ diff_saved_mean,
+                                                                            const float* __restrict__ diff_saved_variance, int vec, float* dx)
+{
+    for (int bc = blockIdx.y; bc < planes; bc += gridDim.y) {
+        const int c = bc % C;
+        const float var = (float)sqrt((double)saved_variance[c] + epsilon);
+        const float m = saved_mean[c], g = scale[c];
+        const double dv2 = (double)diff_saved_variance[c] * 2.0, sz = (double)size, dm = (double)(diff_saved_mean[c] / size);
+        const float* xp = x + (size_t)bc * plane;
+        const float* dp = dy + (size_t)bc * plane;
+        float* op = dx + (size_t)bc * plane;
+        if (vec) {
+            for (int i = blockIdx.x * TBLOCK + threadIdx.x; i < plane / 4; i += gridDim.x * TBLOCK) {
+                const float4 v = ((const float4*)xp)[i];
+                const float4 d = ((const float4*)dp)[i];
+                float4 o;
+                o.x = bn_dx(v.x, d.x, g, var, m, dv2, sz, dm);
+                o.y = bn_dx(v.y, d.y, g, var, m, dv2, sz, dm);
+                o.z = bn_dx(v.z, d.z, g, var, m, dv2, sz, dm);
+                o.w = bn_dx(v.w, d.w, g, var, m, dv2, sz, dm);
+                ((float4*)op)[i] = o;
+            }
+        } else {
+            for (int i = blockIdx.x * TBLOCK + threadIdx.x; i < plane; i += gridDim.x * TBLOCK)
+                op[i] = bn_dx(xp[i], dp[i], g, var, m, dv2, sz, dm);
+        }
+    }
+}
+
+// The same for small planes: one lane per value.
+__global__ __launch_bounds__(TBLOCK) void batchnorm_f32_backward_data_flat_kernel(size_t total, int C, int plane, float size, const float* __restrict__ x,
                                                                             const float* __restrict__ scale, const float* __restrict__ saved_mean,
                                                                             const float* __restrict__ saved_variance, double epsilon, const float* dy,
                                                                             const float* __restrict__ diff_saved_mean,
@@ -760,8 +829,8 @@ int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, co
 {
     N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && bias && mean && variance && y && epsilon > 0.0, N2D2HIP_ERR_INVALID,
                     "n2d2hip_batchnorm_f32_forward: bad argument");
-    N2D2HIP_REQUIRE((size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: tensor too large");
-    const size_t total = (size_t)B * C * H * W;
+    N2D2HIP_REQUIRE((size_t)B * C < ((size_t)1 << 31) && (size_t)H * W < ((size_t)1 << 31), N2D2HIP_ERR_INVALID,
+                    "n2d2hip_batchnorm_f32_forward: tensor too large");
     const bool running = use_running || moving_average_momentum == 0.0;
     if (!running) {
         N2D2HIP_REQUIRE(saved_mean && saved_variance, N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_forward: the learning pass needs saved_mean and saved_variance");
@@ -781,9 +850,19 @@ int n2d2hip_batchnorm_f32_forward(int B, int C, int H, int W, const float* x, co
                                saved_variance, moving_average_momentum);
         }
     }
-    hipLaunchKernelGGL(batchnorm_f32_apply_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W, x, scale, bias,
-                       running ? (const float*)mean : (const float*)saved_mean, running ? (const float*)variance : (const float*)saved_variance, epsilon,
-                       running ? 1 : 0, y);
+    const int plane = H * W;
+    // 16 bytes per lane when every plane starts on a 16-byte boundary
+    const int vec = plane % 4 == 0 && ((uintptr_t)x | (uintptr_t)y) % 16 == 0;
+    const dim3 plane_grid((unsigned)std::max(1, std::min(((vec ? plane / 4 : plane) + TBLOCK - 1) / TBLOCK, 64)),
+                          (unsigned)std::min<size_t>((size_t)B * C, 32768));
+    if (plane >= 512)
+        hipLaunchKernelGGL(batchnorm_f32_apply_kernel, plane_grid, dim3(TBLOCK), 0, (hipStream_t)stream, B * C, C, plane, x, scale, bias,
+                           running ? (const float*)mean : (const float*)saved_mean, running ? (const float*)variance : (const float*)saved_variance,
+                           epsilon, running ? 1 : 0, vec, y);
+    else
+        hipLaunchKernelGGL(batchnorm_f32_apply_flat_kernel, dim3(grid_for((size_t)B * C * plane)), dim3(TBLOCK), 0, (hipStream_t)stream,
+                           (size_t)B * C * plane, C, plane, x, scale, bias, running ? (const float*)mean : (const float*)saved_mean,
+                           running ? (const float*)variance : (const float*)saved_variance, epsilon, running ? 1 : 0, y);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
@@ -796,8 +875,8 @@ int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, c
     N2D2HIP_REQUIRE(B > 0 && C > 0 && H > 0 && W > 0 && x && scale && saved_mean && saved_variance && diff_y && diff_scale && diff_bias
                         && diff_saved_mean && diff_saved_variance && epsilon > 0.0,
                     N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: bad argument");
-    N2D2HIP_REQUIRE((size_t)B * C * H * W < ((size_t)1 << 40), N2D2HIP_ERR_INVALID, "n2d2hip_batchnorm_f32_backward: tensor too large");
-    const size_t total = (size_t)B * C * H * W;
+    N2D2HIP_REQUIRE((size_t)B * C < ((size_t)1 << 31) && (size_t)H * W < ((size_t)1 << 31), N2D2HIP_ERR_INVALID,
+                    "n2d2hip_batchnorm_f32_backward: tensor too large");
     const int splits = bn_splits(B, C, H, W);
     if (splits > 1 && workspace && workspace_bytes >= n2d2hip_batchnorm_f32_workspace_bytes(B, C, H, W)) {
         hipLaunchKernelGGL(batchnorm_f32_backward_partial_kernel, dim3(C, splits), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, splits, x, scale,
@@ -809,10 +888,18 @@ int n2d2hip_batchnorm_f32_backward(int B, int C, int H, int W, const float* x, c
         hipLaunchKernelGGL(batchnorm_f32_backward_sums_kernel, dim3(C), dim3(TBLOCK), 0, (hipStream_t)stream, B, C, H * W, x, scale, saved_mean,
                            saved_variance, epsilon, diff_y, beta_scale, diff_scale, beta_bias, diff_bias, diff_saved_mean, diff_saved_variance);
     }
-    if (diff_x)
-        hipLaunchKernelGGL(batchnorm_f32_backward_data_kernel, dim3(grid_for(total)), dim3(TBLOCK), 0, (hipStream_t)stream, total, C, H * W,
+    const int plane = H * W;
+    const int vec = plane % 4 == 0 && ((uintptr_t)x | (uintptr_t)diff_y | (uintptr_t)diff_x) % 16 == 0;
+    const dim3 plane_grid((unsigned)std::max(1, std::min(((vec ? plane / 4 : plane) + TBLOCK - 1) / TBLOCK, 64)),
+                          (unsigned)std::min<size_t>((size_t)B * C, 32768));
+    if (diff_x && plane >= 512)
+        hipLaunchKernelGGL(batchnorm_f32_backward_data_kernel, plane_grid, dim3(TBLOCK), 0, (hipStream_t)stream, B * C, C, plane,
                            (float)((size_t)B * H * W), x, scale, saved_mean, saved_variance, epsilon, diff_y, (const float*)diff_saved_mean,
-                           (const float*)diff_saved_variance, diff_x);
+                           (const float*)diff_saved_variance, vec, diff_x);
+    else if (diff_x)
+        hipLaunchKernelGGL(batchnorm_f32_backward_data_flat_kernel, dim3(grid_for((size_t)B * C * plane)), dim3(TBLOCK), 0, (hipStream_t)stream,
+                           (size_t)B * C * plane, C, plane, (float)((size_t)B * H * W), x, scale, saved_mean, saved_variance, epsilon, diff_y,
+                           (const float*)diff_saved_mean, (const float*)diff_saved_variance, diff_x);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
