@@ -338,6 +338,29 @@ int n2d2hip_pool_max_f32_forward(int B, int C, int H, int W, int pool_w, int poo
 int n2d2hip_pool_max_f32_backward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x,
                                   int pad_y, const float* diff_y, const int* argmax, float beta, float* diff_x,
                                   n2d2hip_stream_t stream);
+/* Average pooling of float NCHW, one output per channel: the window's values inside the input, added in row-major
+ * order, divided by pool_w * pool_h (count_include_padding != 0) or by their number (ref:
+ * PoolCell_Frame_Kernels::forwardAverage with alpha 1, beta 0, not quantized, src/Cell/PoolCell_Frame_Kernels.cpp:26-100). */
+int n2d2hip_pool_average_f32_forward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y,
+                                     int pad_x, int pad_y, int count_include_padding, const float* x, float* y,
+                                     n2d2hip_stream_t stream);
+/* diff_x[i] = (sum of diff_y over the windows that hold input i) / (pool_w * pool_h) + beta * diff_x[i];
+ * N2D2HIP_ERR_UNSUPPORTED without count_include_padding, where the reference throws (ref:
+ * PoolCell_Frame_Kernels::backwardAverage, src/Cell/PoolCell_Frame_Kernels.cpp:199-293). */
+int n2d2hip_pool_average_f32_backward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y,
+                                      int pad_x, int pad_y, int count_include_padding, const float* diff_y, float beta,
+                                      float* diff_x, n2d2hip_stream_t stream);
+/* y = (weights[0] * x0 + shifts[0]) + (weights[1] * x1 + shifts[1]) + ... over n values, every product and sum rounded
+ * to float in that order; `inputs`, `weights` and `shifts` are host arrays of nb_inputs entries (device pointers in
+ * `inputs`), which is the PerLayer / PerInput coefficient mode (ref: ElemWiseCell_Frame::propagate, Sum,
+ * src/Cell/ElemWiseCell_Frame.cpp:115-134). */
+#define N2D2HIP_ELEMWISE_F32_MAX_INPUTS 8
+int n2d2hip_elemwise_sum_f32_forward(int nb_inputs, const float* const* inputs, size_t n, const float* weights,
+                                     const float* shifts, float* y, n2d2hip_stream_t stream);
+/* The gradient towards one input of that sum: diff_x = weight * diff_y + beta * diff_x (ref:
+ * ElemWiseCell_Frame::backPropagate, Sum, src/Cell/ElemWiseCell_Frame.cpp:194-233). */
+int n2d2hip_elemwise_sum_f32_backward(size_t n, float weight, const float* diff_y, float beta, float* diff_x,
+                                      n2d2hip_stream_t stream);
 /* Softmax over the channels of each pixel, one group (ref: src/Cell/SoftmaxCell_Frame.cpp:93-137). */
 int n2d2hip_softmax_f32_forward(const float* x, float* y, int B, int C, int H, int W, n2d2hip_stream_t stream);
 /* diff = target - output, formed in double; loss[0] (device double) = sum of squares / batch

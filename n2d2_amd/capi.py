@@ -35,6 +35,7 @@ SYMBOLS = [
     "n2d2hip_conv2d_f32_backward_bias", "n2d2hip_softmax_f32_forward", "n2d2hip_loss_workspace_bytes", "n2d2hip_loss_f32",
     "n2d2hip_sgd_update_f32", "n2d2hip_rectifier_f32_forward", "n2d2hip_rectifier_f32_backward",
     "n2d2hip_batchnorm_f32_workspace_bytes", "n2d2hip_batchnorm_f32_forward", "n2d2hip_batchnorm_f32_backward", "n2d2hip_pool_max_f32_forward", "n2d2hip_pool_max_f32_backward",
+    "n2d2hip_pool_average_f32_forward", "n2d2hip_pool_average_f32_backward", "n2d2hip_elemwise_sum_f32_forward", "n2d2hip_elemwise_sum_f32_backward",
 ]
 
 
@@ -124,6 +125,10 @@ def load():
     lib.n2d2hip_batchnorm_f32_backward.argtypes = [I, I, I, I, P, P, P, P, D, P, F, P, F, P, P, P, P, P, SZ, P]
     lib.n2d2hip_pool_max_f32_forward.argtypes = [I, I, I, I, I, I, I, I, I, I, P, P, P, P]
     lib.n2d2hip_pool_max_f32_backward.argtypes = [I, I, I, I, I, I, I, I, I, I, P, P, F, P, P]
+    lib.n2d2hip_pool_average_f32_forward.argtypes = [I, I, I, I, I, I, I, I, I, I, I, P, P, P]
+    lib.n2d2hip_pool_average_f32_backward.argtypes = [I, I, I, I, I, I, I, I, I, I, I, P, F, P, P]
+    lib.n2d2hip_elemwise_sum_f32_forward.argtypes = [I, C.POINTER(C.c_void_p), SZ, C.POINTER(C.c_float), C.POINTER(C.c_float), P, P]
+    lib.n2d2hip_elemwise_sum_f32_backward.argtypes = [SZ, F, P, F, P, P]
     return lib
 
 

@@ -944,6 +944,203 @@ int n2d2hip_pool_max_f32_backward(int B, int C, int H, int W, int pool_w, int po
     return N2D2HIP_OK;
 }
 
+}  // extern "C"
+
+// Average pooling of float NCHW with the unit mapping: the window's values are added in row-major order and divided
+// by the window's size (count_include_padding) or by the number of values inside the input.
+__global__ __launch_bounds__(TBLOCK) void pool_average_f32_forward_kernel(PoolF32 q, int count_include_padding, const float* __restrict__ x,
+                                                                          float* __restrict__ y)
+{
+    const size_t total = (size_t)q.B * q.C * q.oH * q.oW;
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int ox = (int)(i % q.oW), oy = (int)((i / q.oW) % q.oH);
+        const size_t bc = i / ((size_t)q.oW * q.oH);
+        const float* in = x + bc * (size_t)q.H * q.W;
+        const int x0 = ox * q.sx - q.px, y0 = oy * q.sy - q.py;
+        const int sx_min = max(-x0, 0), sy_min = max(-y0, 0);
+        const int sx_max = min(max(q.W - x0, 0), q.pw), sy_max = min(max(q.H - y0, 0), q.ph);
+        float acc = 0.0f;
+        for (int sy = sy_min; sy < sy_max; ++sy)
+            for (int sx = sx_min; sx < sx_max; ++sx)
+                acc += in[(size_t)(y0 + sy) * q.W + x0 + sx];
+        const int inside = max(sx_max - sx_min, 0) * max(sy_max - sy_min, 0);
+        const unsigned count = count_include_padding ? (unsigned)(q.pw * q.ph) : (unsigned)inside;
+        y[i] = count > 0 ? acc / (float)count : 0.0f;
+    }
+}
+
+// Every input collects the gradients of the windows it lies in, in the reference's order (window rows, then columns,
+// from the input's own residue modulo the stride upwards); the sum is divided by the window's size.
+__global__ __launch_bounds__(TBLOCK) void pool_average_f32_backward_kernel(PoolF32 q, const float* __restrict__ dy, float beta, float* __restrict__ dx)
+{
+    const size_t total = (size_t)q.B * q.C * q.H * q.W;
+    const float count = (float)(unsigned)(q.pw * q.ph);
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total; i += (size_t)gridDim.x * TBLOCK) {
+        const int ix = (int)(i % q.W), iy = (int)((i / q.W) % q.H);
+        const size_t bc = i / ((size_t)q.W * q.H);
+        const int ix_pad = ix + q.px, iy_pad = iy + q.py;
+        const int sx_max = min(q.pw, ix_pad + 1), sy_max = min(q.ph, iy_pad + 1);
+        float acc = 0.0f;
+        for (int sy = iy_pad % q.sy; sy < sy_max; sy += q.sy) {
+            if (iy_pad >= q.sy * q.oH + sy)
+                continue;
+            const int oy = (iy_pad - sy) / q.sy;
+            for (int sx = ix_pad % q.sx; sx < sx_max; sx += q.sx) {
+                if (ix_pad >= q.sx * q.oW + sx)
+                    continue;
+                const int ox = (ix_pad - sx) / q.sx;
+                acc += dy[(bc * q.oH + oy) * q.oW + ox];
+            }
+        }
+        const float g = acc / count;
+        dx[i] = beta != 0.0f ? __fadd_rn(g, __fmul_rn(beta, dx[i])) : g;
+    }
+}
+
+extern "C" {
+
+int n2d2hip_pool_average_f32_forward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x, int pad_y,
+                                     int count_include_padding, const float* x, float* y, n2d2hip_stream_t stream)
+{
+    PoolF32 q;
+    const int rc = make_pool(B, C, H, W, pool_w, pool_h, stride_x, stride_y, pad_x, pad_y, &q, "n2d2hip_pool_average_f32_forward");
+    if (rc != N2D2HIP_OK) return rc;
+    N2D2HIP_REQUIRE(x && y, N2D2HIP_ERR_INVALID, "n2d2hip_pool_average_f32_forward: null pointer");
+    hipLaunchKernelGGL(pool_average_f32_forward_kernel, dim3(grid_for((size_t)B * C * q.oH * q.oW)), dim3(TBLOCK), 0, (hipStream_t)stream, q,
+                       count_include_padding ? 1 : 0, x, y);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_pool_average_f32_backward(int B, int C, int H, int W, int pool_w, int pool_h, int stride_x, int stride_y, int pad_x, int pad_y,
+                                      int count_include_padding, const float* diff_y, float beta, float* diff_x, n2d2hip_stream_t stream)
+{
+    PoolF32 q;
+    const int rc = make_pool(B, C, H, W, pool_w, pool_h, stride_x, stride_y, pad_x, pad_y, &q, "n2d2hip_pool_average_f32_backward");
+    if (rc != N2D2HIP_OK) return rc;
+    // the reference throws for the other case (src/Cell/PoolCell_Frame_Kernels.cpp:210-213)
+    N2D2HIP_REQUIRE(count_include_padding, N2D2HIP_ERR_UNSUPPORTED, "n2d2hip_pool_average_f32_backward: exclude padding not implemented");
+    N2D2HIP_REQUIRE(diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_pool_average_f32_backward: null pointer");
+    hipLaunchKernelGGL(pool_average_f32_backward_kernel, dim3(grid_for((size_t)B * C * H * W)), dim3(TBLOCK), 0, (hipStream_t)stream, q, diff_y, beta,
+                       diff_x);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+}  // extern "C"
+
+// Weighted sum of up to N2D2HIP_ELEMWISE_F32_MAX_INPUTS float tensors of one shape: products and sums are rounded one
+// by one, in the order of the inputs, as the reference's scalar loop does.
+struct ElemWiseF32 {
+    const float* x[N2D2HIP_ELEMWISE_F32_MAX_INPUTS];
+    float w[N2D2HIP_ELEMWISE_F32_MAX_INPUTS], s[N2D2HIP_ELEMWISE_F32_MAX_INPUTS];
+    int n;
+};
+
+__device__ __forceinline__ float elemwise_sum_one(const ElemWiseF32& e, const float* v)
+{
+    float acc = __fadd_rn(__fmul_rn(e.w[0], v[0]), e.s[0]);
+#pragma unroll
+    for (int k = 1; k < N2D2HIP_ELEMWISE_F32_MAX_INPUTS; ++k)
+        if (k < e.n)
+            acc = __fadd_rn(acc, __fadd_rn(__fmul_rn(e.w[k], v[k]), e.s[k]));
+    return acc;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(TBLOCK) void elemwise_sum_f32_forward_kernel(ElemWiseF32 e, size_t total, float* __restrict__ y)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total / VEC; i += (size_t)gridDim.x * TBLOCK) {
+        if (VEC == 4) {
+            float4 v[N2D2HIP_ELEMWISE_F32_MAX_INPUTS];
+#pragma unroll
+            for (int k = 0; k < N2D2HIP_ELEMWISE_F32_MAX_INPUTS; ++k)
+                if (k < e.n)
+                    v[k] = ((const float4*)e.x[k])[i];
+            float a[N2D2HIP_ELEMWISE_F32_MAX_INPUTS], b[N2D2HIP_ELEMWISE_F32_MAX_INPUTS], c[N2D2HIP_ELEMWISE_F32_MAX_INPUTS],
+                d[N2D2HIP_ELEMWISE_F32_MAX_INPUTS];
+#pragma unroll
+            for (int k = 0; k < N2D2HIP_ELEMWISE_F32_MAX_INPUTS; ++k)
+                if (k < e.n) {
+                    a[k] = v[k].x; b[k] = v[k].y; c[k] = v[k].z; d[k] = v[k].w;
+                }
+            float4 o;
+            o.x = elemwise_sum_one(e, a);
+            o.y = elemwise_sum_one(e, b);
+            o.z = elemwise_sum_one(e, c);
+            o.w = elemwise_sum_one(e, d);
+            ((float4*)y)[i] = o;
+        } else {
+            float a[N2D2HIP_ELEMWISE_F32_MAX_INPUTS];
+#pragma unroll
+            for (int k = 0; k < N2D2HIP_ELEMWISE_F32_MAX_INPUTS; ++k)
+                if (k < e.n)
+                    a[k] = e.x[k][i];
+            y[i] = elemwise_sum_one(e, a);
+        }
+    }
+}
+
+// diff_x = weight * diff_y + beta * diff_x
+template <int VEC>
+__global__ __launch_bounds__(TBLOCK) void elemwise_sum_f32_backward_kernel(size_t total, float weight, const float* __restrict__ dy, float beta, float* dx)
+{
+    for (size_t i = (size_t)blockIdx.x * TBLOCK + threadIdx.x; i < total / VEC; i += (size_t)gridDim.x * TBLOCK) {
+        if (VEC == 4) {
+            const float4 d = ((const float4*)dy)[i];
+            float4 o = make_float4(__fmul_rn(weight, d.x), __fmul_rn(weight, d.y), __fmul_rn(weight, d.z), __fmul_rn(weight, d.w));
+            if (beta != 0.0f) {
+                const float4 p = ((const float4*)dx)[i];
+                o.x = __fadd_rn(o.x, __fmul_rn(beta, p.x));
+                o.y = __fadd_rn(o.y, __fmul_rn(beta, p.y));
+                o.z = __fadd_rn(o.z, __fmul_rn(beta, p.z));
+                o.w = __fadd_rn(o.w, __fmul_rn(beta, p.w));
+            }
+            ((float4*)dx)[i] = o;
+        } else {
+            const float g = __fmul_rn(weight, dy[i]);
+            dx[i] = beta != 0.0f ? __fadd_rn(g, __fmul_rn(beta, dx[i])) : g;
+        }
+    }
+}
+
+extern "C" {
+
+int n2d2hip_elemwise_sum_f32_forward(int nb_inputs, const float* const* inputs, size_t n, const float* weights, const float* shifts, float* y,
+                                     n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(nb_inputs > 0 && inputs && weights && shifts && y && n > 0, N2D2HIP_ERR_INVALID, "n2d2hip_elemwise_sum_f32_forward: bad argument");
+    N2D2HIP_REQUIRE(nb_inputs <= N2D2HIP_ELEMWISE_F32_MAX_INPUTS, N2D2HIP_ERR_UNSUPPORTED, "n2d2hip_elemwise_sum_f32_forward: at most %d inputs",
+                    N2D2HIP_ELEMWISE_F32_MAX_INPUTS);
+    ElemWiseF32 e = {};
+    e.n = nb_inputs;
+    uintptr_t align = (uintptr_t)y;
+    for (int k = 0; k < nb_inputs; ++k) {
+        N2D2HIP_REQUIRE(inputs[k], N2D2HIP_ERR_INVALID, "n2d2hip_elemwise_sum_f32_forward: input %d is null", k);
+        e.x[k] = inputs[k];
+        e.w[k] = weights[k];
+        e.s[k] = shifts[k];
+        align |= (uintptr_t)inputs[k];
+    }
+    if (n % 4 == 0 && align % 16 == 0)
+        hipLaunchKernelGGL(elemwise_sum_f32_forward_kernel<4>, dim3(grid_for(n / 4)), dim3(TBLOCK), 0, (hipStream_t)stream, e, n, y);
+    else
+        hipLaunchKernelGGL(elemwise_sum_f32_forward_kernel<1>, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, e, n, y);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_elemwise_sum_f32_backward(size_t n, float weight, const float* diff_y, float beta, float* diff_x, n2d2hip_stream_t stream)
+{
+    N2D2HIP_REQUIRE(n > 0 && diff_y && diff_x, N2D2HIP_ERR_INVALID, "n2d2hip_elemwise_sum_f32_backward: bad argument");
+    if (n % 4 == 0 && ((uintptr_t)diff_y | (uintptr_t)diff_x) % 16 == 0)
+        hipLaunchKernelGGL(elemwise_sum_f32_backward_kernel<4>, dim3(grid_for(n / 4)), dim3(TBLOCK), 0, (hipStream_t)stream, n, weight, diff_y, beta, diff_x);
+    else
+        hipLaunchKernelGGL(elemwise_sum_f32_backward_kernel<1>, dim3(grid_for(n)), dim3(TBLOCK), 0, (hipStream_t)stream, n, weight, diff_y, beta, diff_x);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
 size_t n2d2hip_loss_workspace_bytes(size_t n)
 {
     return (size_t)grid_for(n) * sizeof(double);

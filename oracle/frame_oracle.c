@@ -28,6 +28,11 @@
  *       tests/test_oracle_qat_train.py: adjoint identities and the Jacobian
  *       of the forward, and the reference's PyTorch-derived known-answer
  *       tests (trained SAT alphas; LSQ step sizes of a conv net and an FC).
+ *   average pooling (float forward, backward), the ElemWise sum's gradient
+ *       tests/test_oracle_qat_train.py: a library routine (torch's
+ *       avg_pool2d and its autograd in float64, both divisors), the adjoint
+ *       identity <dy, A x> = <A^T dy, x>, and for the sum the rounded
+ *       product weight * dy and the directional derivative of its forward.
  * Parity unpinned, by nature: the ORDER in which float reductions add their
  * terms where the reference runs them under OpenMP or through
  * std::accumulate (the restatement adds in element order), and the last bit
@@ -98,6 +103,62 @@ void oracle_elemwise_sum_f32(const float* const* inputs, int nbInputs, int B, in
                         out[i] += weights[c1] * inputs[k][i] + shifts[c1];
                     }
                 }
+}
+
+/* src/Cell/ElemWiseCell_Frame.cpp:194-233 (backPropagate, Sum): the gradient towards input k,
+ * diffOutput = weights[coeffIdx] * diffInput + beta * diffOutput, coeffIdx = channel (PerChannel) or k. */
+void oracle_elemwise_sum_backward_f32(const float* diffInput, int B, int C, int H, int W, const float* weights,
+                                      int coeffMode, int k, float beta, float* diffOutput)
+{
+    for (int b = 0; b < B; ++b)
+        for (int ch = 0; ch < C; ++ch)
+            for (int y = 0; y < H; ++y)
+                for (int x = 0; x < W; ++x) {
+                    const size_t i = (size_t)x + (size_t)W * ((size_t)y + (size_t)H * ((size_t)ch + (size_t)C * b));
+                    const size_t coeffIdx = (coeffMode == 2) ? (size_t)ch : (size_t)k;
+                    const float product = weights[coeffIdx] * diffInput[i];
+                    const float kept = (beta != 0.0f) ? beta * diffOutput[i] : 0.0f;
+                    diffOutput[i] = product + kept;
+                }
+}
+
+/* src/Cell/PoolCell_Frame_Kernels.cpp:199-293 (backwardAverage) with the unit mapping (every output pools its own
+ * channel, poolChannelsCount = 1).  Returns -1 where the reference throws (exclude padding). */
+int oracle_pool_backward_average_f32(const float* alpha, const float* diffInputs, int B, int C, int H, int W,
+                                     const int pool[2], const int stride[2], const int pad[2], const float* beta,
+                                     float* diffOutputs, int outW, int outH, int countIncludePadding)
+{
+    if (!countIncludePadding)
+        return -1;
+    const unsigned int oxStride = (unsigned int)stride[0] * (unsigned int)outW;
+    const unsigned int oyStride = (unsigned int)stride[1] * (unsigned int)outH;
+    for (int b = 0; b < B; ++b)
+        for (int channel = 0; channel < C; ++channel)
+            for (unsigned int iy = 0; iy < (unsigned int)H; ++iy)
+                for (unsigned int ix = 0; ix < (unsigned int)W; ++ix) {
+                    const unsigned int ixPad = ix + (unsigned int)pad[0], iyPad = iy + (unsigned int)pad[1];
+                    const unsigned int sxMax = (unsigned int)pool[0] < ixPad + 1 ? (unsigned int)pool[0] : ixPad + 1;
+                    const unsigned int syMax = (unsigned int)pool[1] < iyPad + 1 ? (unsigned int)pool[1] : iyPad + 1;
+                    float poolGradient = 0.0f;
+                    for (unsigned int sy = iyPad % (unsigned int)stride[1], sx0 = ixPad % (unsigned int)stride[0]; sy < syMax;
+                         sy += (unsigned int)stride[1]) {
+                        if (iyPad >= oyStride + sy)
+                            continue;
+                        for (unsigned int sx = sx0; sx < sxMax; sx += (unsigned int)stride[0]) {
+                            if (ixPad >= oxStride + sx)
+                                continue;
+                            const unsigned int ox = (ixPad - sx) / (unsigned int)stride[0];
+                            const unsigned int oy = (iyPad - sy) / (unsigned int)stride[1];
+                            poolGradient += diffInputs[ox + (size_t)outW * (oy + (size_t)outH * ((size_t)channel + (size_t)C * b))] / 1u;
+                        }
+                    }
+                    const unsigned int poolCount = (unsigned int)(pool[0] * pool[1]);
+                    const size_t i = ix + (size_t)W * (iy + (size_t)H * ((size_t)channel + (size_t)C * b));
+                    const float scaled = (*alpha) * (poolGradient / poolCount);
+                    const float kept = (*beta != 0.0f) ? (*beta) * diffOutputs[i] : 0.0f;
+                    diffOutputs[i] = scaled + kept;
+                }
+    return 0;
 }
 
 /* src/Cell/Cell.cpp:251-300 (getNbGroups), regular case only: returns -1 where

@@ -226,6 +226,33 @@ def pool_forward(x, pool, stride, pad=(0, 0), kind="max", quantized=True, maps=N
     return out
 
 
+def pool_backward_average(dy, x_shape, pool, stride, pad=(0, 0), beta=0.0, prev=None, count_include_padding=True):
+    """PoolCell_Frame_Kernels::backwardAverage, float32, unit mapping; raises where the reference throws."""
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cn, H, W = x_shape
+    oH, oW = dy.shape[2:]
+    dx = np.zeros(x_shape, dtype=np.float32) if prev is None else np.array(prev, dtype=np.float32, order="C")
+    a, b = C.c_float(1.0), C.c_float(beta)
+    fn = _lib.oracle_pool_backward_average_f32
+    fn.restype = C.c_int
+    if fn(C.byref(a), _p(dy), B, Cn, H, W, _ia(pool), _ia(stride), _ia(pad), C.byref(b), _p(dx), oW, oH,
+          int(bool(count_include_padding))) != 0:
+        raise RuntimeError("PoolCell_Frame_Kernels::backwardAverage() exclude padding not implemented")
+    return dx
+
+
+def elemwise_sum_backward(dy, weights, k, coeff_mode="PerLayer", beta=0.0, prev=None):
+    """ElemWiseCell_Frame::backPropagate, Sum: the gradient towards input k."""
+    dy = np.ascontiguousarray(dy, dtype=np.float32)
+    B, Cc, H, W = dy.shape
+    w = np.ascontiguousarray(weights, dtype=np.float32)
+    dx = np.zeros(dy.shape, dtype=np.float32) if prev is None else np.array(prev, dtype=np.float32, order="C")
+    fn = _lib.oracle_elemwise_sum_backward_f32
+    fn.restype = None
+    fn(_p(dy), B, Cc, H, W, _p(w), {"PerLayer": 0, "PerInput": 1, "PerChannel": 2}[coeff_mode], int(k), C.c_float(beta), _p(dx))
+    return dx
+
+
 def elemwise_sum(inputs, weights=None, shifts=None, coeff_mode="PerLayer"):
     """ElemWiseCell_Frame::propagate, Sum. inputs: list of float32 NCHW arrays."""
     xs = [np.ascontiguousarray(x, dtype=np.float32) for x in inputs]

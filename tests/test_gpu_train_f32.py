@@ -396,3 +396,67 @@ def test_max_pooling_forward_backward(g, case):
         assert (wdx == 0).sum() >= x.size // 3
     assert g.lib.n2d2hip_pool_max_f32_forward(B, Cn, H, W, 2, 2, 2, 2, 2, 0, dx_.data_ptr(), y.data_ptr(), am.data_ptr(), g.sp()) == g.capi.ERR_INVALID
     assert g.lib.n2d2hip_pool_max_f32_forward(B, Cn, 1, 1, 3, 3, 1, 1, 0, 0, dx_.data_ptr(), y.data_ptr(), am.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+
+
+@pytest.mark.parametrize("case", [(2, 3, 9, 8, 2, 2, 2, 2, 0, 0), (2, 3, 9, 8, 3, 3, 2, 2, 1, 1), (1, 2, 7, 10, 3, 2, 1, 2, 0, 0),
+                                  (4, 16, 28, 28, 2, 2, 2, 2, 0, 0), (3, 5, 11, 11, 3, 3, 1, 1, 1, 1), (2, 2, 6, 6, 2, 2, 3, 3, 0, 0),
+                                  (8, 64, 7, 7, 7, 7, 7, 7, 0, 0)])
+def test_average_pooling_forward_backward(g, case):
+    from oracle import oracle as o
+    print("pool average f32", case, flush=True)
+    B, Cn, H, W, pw, ph, sx, sy, px, py = case
+    rng = np.random.default_rng(sum(case) + 1)
+    x = rng.normal(size=(B, Cn, H, W)).astype(np.float32)
+    dx_ = g.dev(x)
+    for include in (1, 0):
+        want = o.pool_forward(x, (pw, ph), (sx, sy), (px, py), kind="average", quantized=False, count_include_padding=bool(include))
+        y = g.torch_.empty(want.size, dtype=g.torch_.float32, device="cuda")
+        g.check(g.lib.n2d2hip_pool_average_f32_forward(B, Cn, H, W, pw, ph, sx, sy, px, py, include, dx_.data_ptr(), y.data_ptr(), g.sp()))
+        assert np.array_equal(g.host(y).reshape(want.shape), want)          # same additions in the same order, one division
+    dy = rng.normal(size=want.shape).astype(np.float32)
+    prev = rng.normal(size=x.shape).astype(np.float32)
+    ddy = g.dev(dy)
+    for beta in (0.0, 1.0):
+        wdx = o.pool_backward_average(dy, x.shape, (pw, ph), (sx, sy), (px, py), beta=beta, prev=prev)
+        out = g.dev(prev)
+        g.check(g.lib.n2d2hip_pool_average_f32_backward(B, Cn, H, W, pw, ph, sx, sy, px, py, 1, ddy.data_ptr(), beta, out.data_ptr(), g.sp()))
+        assert np.array_equal(g.host(out), wdx)
+    assert g.lib.n2d2hip_pool_average_f32_backward(B, Cn, H, W, pw, ph, sx, sy, px, py, 0, ddy.data_ptr(), 0.0, out.data_ptr(),
+                                                   g.sp()) == g.capi.ERR_UNSUPPORTED
+    assert g.lib.n2d2hip_pool_average_f32_forward(B, Cn, H, W, 2, 2, 2, 2, 2, 0, 1, dx_.data_ptr(), y.data_ptr(), g.sp()) == g.capi.ERR_INVALID
+
+
+@pytest.mark.parametrize("shape,n_in", [((2, 3, 5, 7), 2), ((4, 16, 14, 14), 2), ((1, 1, 1, 3), 3), ((2, 8, 6, 6), 8), ((3, 5, 4, 4), 1)])
+def test_elemwise_sum_float_forward_backward(g, shape, n_in):
+    from oracle import oracle as o
+    print("elemwise sum f32", shape, n_in, flush=True)
+    rng = np.random.default_rng(sum(shape) + n_in)
+    xs = [rng.normal(size=shape).astype(np.float32) for _ in range(n_in)]
+    w = rng.normal(size=n_in).astype(np.float32)
+    sh = rng.normal(size=n_in).astype(np.float32)
+    want = o.elemwise_sum(xs, w, sh, "PerInput")
+    dev = [g.dev(x) for x in xs]
+    n = xs[0].size
+    ptrs = (C.c_void_p * n_in)(*[d.data_ptr() for d in dev])
+    wa, sa = (C.c_float * n_in)(*w.tolist()), (C.c_float * n_in)(*sh.tolist())
+    y = g.torch_.empty(n, dtype=g.torch_.float32, device="cuda")
+    g.check(g.lib.n2d2hip_elemwise_sum_f32_forward(n_in, ptrs, n, wa, sa, y.data_ptr(), g.sp()))
+    assert np.array_equal(g.host(y).reshape(shape), want)
+    # a view that starts 4 bytes into a buffer takes the one-value-per-lane kernel
+    if n > 1:
+        odd = [g.torch_.cat([d.flatten()[:1], d.flatten()])[1:] for d in dev]
+        ptrs2 = (C.c_void_p * n_in)(*[d.data_ptr() for d in odd])
+        y2 = g.torch_.empty(n, dtype=g.torch_.float32, device="cuda")
+        g.check(g.lib.n2d2hip_elemwise_sum_f32_forward(n_in, ptrs2, n, wa, sa, y2.data_ptr(), g.sp()))
+        assert np.array_equal(g.host(y2).reshape(shape), want)
+    dy = rng.normal(size=shape).astype(np.float32)
+    prev = rng.normal(size=shape).astype(np.float32)
+    ddy = g.dev(dy)
+    for k in range(n_in):
+        for beta in (0.0, 1.0):
+            wdx = o.elemwise_sum_backward(dy, w, k, "PerInput", beta=beta, prev=prev)
+            out = g.dev(prev)
+            g.check(g.lib.n2d2hip_elemwise_sum_f32_backward(n, float(w[k]), ddy.data_ptr(), beta, out.data_ptr(), g.sp()))
+            assert np.array_equal(g.host(out).reshape(shape), wdx)
+    assert g.lib.n2d2hip_elemwise_sum_f32_forward(9, ptrs, n, wa, sa, y.data_ptr(), g.sp()) == g.capi.ERR_UNSUPPORTED
+    assert g.lib.n2d2hip_elemwise_sum_f32_forward(0, ptrs, n, wa, sa, y.data_ptr(), g.sp()) == g.capi.ERR_INVALID

@@ -294,3 +294,63 @@ def test_a_net_with_batchnorm_and_pooling_learns():
     last = qt.train_sequential(x, cells_, sm, t, 300)
     assert last < 0.6 * first and np.isfinite(last)
     assert not np.array_equal(cells_[1].scale, np.ones(4, dtype=np.float32)) and np.all(cells_[1].variance > 0)
+
+
+# ---- average pooling (forward, backward) and the ElemWise sum's gradient: what pins the oracle's restatements.
+# The reference holds no known answers for them; a library routine (torch's avg_pool2d and its autograd, float64)
+# and the adjoint identity <dy, A x> = <A^T dy, x> of a linear map do.
+AVG_CASES = [(2, 3, 9, 8, 2, 2, 2, 2, 0, 0), (2, 3, 9, 8, 3, 3, 2, 2, 1, 1), (1, 2, 7, 10, 3, 2, 1, 2, 0, 0),
+             (3, 5, 11, 11, 3, 3, 1, 1, 1, 1), (2, 2, 6, 6, 2, 2, 3, 3, 0, 0), (2, 4, 7, 7, 7, 7, 7, 7, 0, 0)]
+
+
+@pytest.mark.parametrize("case", AVG_CASES)
+def test_average_pooling_against_library_routine_and_adjoint(case):
+    import torch
+    from oracle import oracle as o
+    B, Cn, H, W, pw, ph, sx, sy, px, py = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.normal(size=(B, Cn, H, W)).astype(np.float32)
+    y = o.pool_forward(x, (pw, ph), (sx, sy), (px, py), kind="average", quantized=False)
+    xt = torch.tensor(x.astype(np.float64), requires_grad=True)
+    yt = torch.nn.functional.avg_pool2d(xt, (ph, pw), (sy, sx), (py, px), count_include_pad=True)
+    assert y.shape == tuple(yt.shape)
+    assert np.abs(y - yt.detach().numpy()).max() <= 1e-5
+    # the other divisor: the number of values inside the input
+    y2 = o.pool_forward(x, (pw, ph), (sx, sy), (px, py), kind="average", quantized=False, count_include_padding=False)
+    yt2 = torch.nn.functional.avg_pool2d(xt, (ph, pw), (sy, sx), (py, px), count_include_pad=False)
+    assert np.abs(y2 - yt2.detach().numpy()).max() <= 1e-5
+    dy = rng.normal(size=y.shape).astype(np.float32)
+    dx = o.pool_backward_average(dy, x.shape, (pw, ph), (sx, sy), (px, py))
+    yt.backward(torch.tensor(dy.astype(np.float64)))
+    assert np.abs(dx - xt.grad.numpy()).max() <= 1e-5
+    # adjoint identity in float64 sums of the float32 results
+    assert abs((dy.astype(np.float64) * y).sum() - (dx.astype(np.float64) * x).sum()) <= 1e-4 * max(1.0, np.abs(dy).sum())
+    # beta keeps what the gradient tensor held
+    prev = rng.normal(size=x.shape).astype(np.float32)
+    assert np.abs(o.pool_backward_average(dy, x.shape, (pw, ph), (sx, sy), (px, py), beta=1.0, prev=prev) - (dx + prev)).max() <= 1e-6
+    with pytest.raises(RuntimeError):
+        o.pool_backward_average(dy, x.shape, (pw, ph), (sx, sy), (px, py), count_include_padding=False)
+
+
+def test_elemwise_sum_gradient_is_the_weight_per_input_or_per_channel():
+    from oracle import oracle as o
+    rng = np.random.default_rng(11)
+    xs = [rng.normal(size=(2, 3, 4, 5)).astype(np.float32) for _ in range(3)]
+    w = np.array([0.5, -2.0, 3.0], dtype=np.float32)
+    sh = np.array([0.25, 0.0, -1.0], dtype=np.float32)
+    y = o.elemwise_sum(xs, w, sh, "PerInput")
+    assert np.abs(y - (sum(w[k] * xs[k].astype(np.float64) for k in range(3)) + sh.sum())).max() <= 1e-5
+    dy = rng.normal(size=y.shape).astype(np.float32)
+    for k in range(3):
+        dx = o.elemwise_sum_backward(dy, w, k, "PerInput")
+        assert np.array_equal(dx, w[k] * dy)                              # one rounded product per value
+        # directional derivative of the (affine) forward along a random direction
+        d = rng.normal(size=y.shape).astype(np.float32)
+        moved = [x if i != k else x + d for i, x in enumerate(xs)]
+        lhs = ((o.elemwise_sum(moved, w, sh, "PerInput").astype(np.float64) - y) * dy).sum()
+        assert abs(lhs - (dx.astype(np.float64) * d).sum()) <= 1e-4 * np.abs(dy).sum()
+        prev = rng.normal(size=y.shape).astype(np.float32)
+        assert np.array_equal(o.elemwise_sum_backward(dy, w, k, "PerInput", beta=1.0, prev=prev), w[k] * dy + prev)
+    wc = np.array([2.0, -1.0, 0.5], dtype=np.float32)
+    dxc = o.elemwise_sum_backward(dy, wc, 1, "PerChannel")
+    assert np.array_equal(dxc, wc[None, :, None, None] * dy)
