@@ -583,8 +583,6 @@ PoolCell_FrameTrain_HIP<T>::PoolCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, 
 {
     if (poolDims.size() != 2 || strideDims.size() != 2 || paddingDims.size() != 2)
         throw std::runtime_error("PoolCell_FrameTrain_HIP " + name + ": two-dimensional pooling expected");
-    if (pooling != Max)
-        throw std::runtime_error("PoolCell_FrameTrain_HIP " + name + ": only Max pooling learns on the float Frame_HIP cells");
     mActivation = activation;
 }
 
@@ -613,15 +611,21 @@ void PoolCell_FrameTrain_HIP<T>::initialize()
         (void)hipFree(mArgMax);
         mArgMax = nullptr;
     }
-    checkHipT(hipMalloc((void**)&mArgMax, mOutputs.size() * sizeof(int)), "PoolCell_FrameTrain_HIP::initialize()");
+    if (mPooling == Max)
+        checkHipT(hipMalloc((void**)&mArgMax, mOutputs.size() * sizeof(int)), "PoolCell_FrameTrain_HIP::initialize()");
 }
 
 template <class T>
 void PoolCell_FrameTrain_HIP<T>::propagate(bool inference)
 {
-    checkStatus(n2d2hip_pool_max_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
-                                             (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], mIn->data(),
-                                             mOutputs.data(), mArgMax, mStream));
+    if (mPooling == Max)
+        checkStatus(n2d2hip_pool_max_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                                 (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], mIn->data(),
+                                                 mOutputs.data(), mArgMax, mStream));
+    else        // Average counts the padding, as PoolCell_Frame<T>::propagate does (src/Cell/PoolCell_Frame.cpp:123-175)
+        checkStatus(n2d2hip_pool_average_f32_forward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                                     (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], 1,
+                                                     mIn->data(), mOutputs.data(), mStream));
     activationPropagate(inference);
     mDiffInputs.clearValid();
 }
@@ -635,9 +639,14 @@ void PoolCell_FrameTrain_HIP<T>::backPropagate()
     if (!mDiffOut || mDiffOut->empty())
         return;
     const float beta = mDiffOut->isValid() ? 1.0f : 0.0f;
-    checkStatus(n2d2hip_pool_max_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
-                                              (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], mDiffInputs.data(),
-                                              mArgMax, beta, mDiffOut->data(), mStream));
+    if (mPooling == Max)
+        checkStatus(n2d2hip_pool_max_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                                  (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1],
+                                                  mDiffInputs.data(), mArgMax, beta, mDiffOut->data(), mStream));
+    else
+        checkStatus(n2d2hip_pool_average_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, (int)mPoolDims[0], (int)mPoolDims[1],
+                                                      (int)mStrideDims[0], (int)mStrideDims[1], (int)mPaddingDims[0], (int)mPaddingDims[1], 1,
+                                                      mDiffInputs.data(), beta, mDiffOut->data(), mStream));
     mDiffOut->setValid();
 }
 

@@ -272,7 +272,7 @@ private:
     static Registrar<BatchNormCell> mRegistrar;
 };
 
-// src/Cell/PoolCell_Frame.cpp:123-228 with Pooling=Max, one input and one output per channel.
+// src/Cell/PoolCell_Frame.cpp:123-228 with Pooling=Max or Average (padding counted), one input and one output per channel.
 template <class T>
 class PoolCell_FrameTrain_HIP : public PoolCell, public Cell_FrameTrain_HIP {
 public:

@@ -244,8 +244,8 @@ int fh_train_get_batchnorm(void* net, const char* cell, int what, float* out, si
     });
 }
 
-// Max pooling, one output per channel
-int fh_train_add_pool(void* net, const char* name, int poolW, int poolH, int strideX, int strideY, int padX, int padY)
+// Max (pooling 0) or Average (pooling 1) pooling, one output per channel
+int fh_train_add_pool(void* net, const char* name, int poolW, int poolH, int strideX, int strideY, int padX, int padY, int pooling)
 {
     return guardedT([&] {
         TrainNet& n = *(TrainNet*)net;
@@ -253,7 +253,7 @@ int fh_train_add_pool(void* net, const char* name, int poolW, int poolH, int str
         if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
         const unsigned int nbOutputs = n.cells.empty() ? (unsigned int)n.input.dimZ() : n.last()->getNbOutputs();
         auto pool = f(n.net, n.deepNet, name, {(unsigned)poolW, (unsigned)poolH}, nbOutputs, {(unsigned)strideX, (unsigned)strideY},
-                      {(unsigned)padX, (unsigned)padY}, PoolCell::Max, std::shared_ptr<Activation>());
+                      {(unsigned)padX, (unsigned)padY}, pooling ? PoolCell::Average : PoolCell::Max, std::shared_ptr<Activation>());
         connect(n, std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(pool));
     });
 }

@@ -347,7 +347,7 @@ lib.fh_train_add_conv.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I, _I
 lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
 lib.fh_train_add_batchnorm.argtypes = [_P, C.c_char_p, _P, C.c_double, C.c_double, _I, _I, _I, _F]
 lib.fh_train_get_batchnorm.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
-lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I]
+lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I]
 lib.fh_net_deepnet.argtypes = [_P]
 lib.fh_net_deepnet.restype = C.c_void_p
 lib.fh_train_fuse_into.argtypes = [_P, _P, _I, _I, _I, _I, _P]
@@ -443,10 +443,10 @@ class TrainNet:
             out[k] = v
         return out
 
-    def add_pool(self, name, pool, stride, pad=(0, 0)):
-        """Max pooling, one output per channel; pool / stride / pad as (x, y)."""
+    def add_pool(self, name, pool, stride, pad=(0, 0), pooling="Max"):
+        """Max or Average pooling, one output per channel; pool / stride / pad as (x, y)."""
         _check_train(lib.fh_train_add_pool(self._h, name.encode(), int(pool[0]), int(pool[1]), int(stride[0]), int(stride[1]), int(pad[0]),
-                                           int(pad[1])))
+                                           int(pad[1]), {"Max": 0, "Average": 1}[pooling]))
         B, Cn, H, W = self._last
         oH = int((H + 2 * pad[1] - pool[1] + stride[1]) / float(stride[1]))
         oW = int((W + 2 * pad[0] - pool[0] + stride[0]) / float(stride[0]))

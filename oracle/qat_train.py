@@ -327,12 +327,16 @@ class PoolCell:
     first largest element of each window (src/Cell/PoolCell_Frame_Kernels.cpp:102-197); backwardMax gives every input
     the sum of the gradients of the outputs it was the maximum of (:295-379)."""
 
-    def __init__(self, pool, stride, pad=(0, 0), activation=None):
-        self.pool, self.stride, self.pad, self.activation = pool, stride, pad, activation
+    def __init__(self, pool, stride, pad=(0, 0), activation=None, pooling="Max"):
+        self.pool, self.stride, self.pad, self.activation, self.pooling = pool, stride, pad, activation, pooling
         self.diff_inputs = None
 
     def propagate(self, x, inference=False):
         self.x_shape = x.shape
+        if self.pooling == "Average":     # forwardAverage / backwardAverage, padding counted (src/Cell/PoolCell_Frame_Kernels.cpp:26-100, 199-293)
+            y = o.pool_forward(np.ascontiguousarray(x, dtype=F), self.pool, self.stride, self.pad, kind="average", quantized=False)
+            self.outputs = self.activation.propagate(y, inference) if self.activation else y
+            return self.outputs
         y, self.argmax = o.pool_forward(np.ascontiguousarray(x, dtype=F), self.pool, self.stride, self.pad, kind="max", quantized=False,
                                         argmax=True)
         self.outputs = self.activation.propagate(y, inference) if self.activation else y
@@ -342,6 +346,8 @@ class PoolCell:
         d = self.diff_inputs
         if self.activation:
             d = self.activation.back_propagate(d)
+        if self.pooling == "Average":
+            return o.pool_backward_average(d, self.x_shape, self.pool, self.stride, self.pad)
         dx = np.zeros(self.x_shape, dtype=F)
         B, Cn, oH, oW = d.shape
         am = self.argmax

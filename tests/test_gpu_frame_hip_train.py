@@ -468,3 +468,40 @@ def test_learn_then_fuse_then_infer_without_leaving_the_gpu():
         assert np.abs(twin.outputs("fc") - want).max() <= 1 and np.unique(want).size > 2
     finally:
         fh.set_globals(0, True, False)
+
+
+def test_average_pool_cell_learns_as_the_oracle_does():
+    """Conv (SAT weights, Rectifier) -> Average Pool 3x3 stride 2 with padding -> Conv -> Softmax: the first iteration tensor by
+    tensor, then ten more on the loss and the learned weights."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    rng = np.random.default_rng(37)
+    x = rng.uniform(0, 1, size=(4, 2, 11, 11)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, size=(4, 2, 3, 3)).astype(np.float32)
+    w2 = rng.normal(0, 0.3, size=(3, 4, 5, 5)).astype(np.float32)
+    t = np.zeros((4, 3, 1, 1), dtype=np.float32)
+    t[np.arange(4), [2, 1, 0, 1]] = 1
+    net = fh.TrainNet(x, propagate_gradient=False)
+    net.add_conv("c1", w1, weight_quant="SAT", weight_range=15)
+    net.add_pool("pool", (3, 3), (2, 2), (1, 1), pooling="Average")
+    net.add_conv("c2", w2, weight_quant="SAT", weight_range=15)
+    net.add_softmax("softmax", with_loss=True)
+    assert net._shapes["pool"] == (4, 4, 5, 5) and net._last == (4, 3, 1, 1)
+    cells_ = [q.ConvCell(w1, quantizer=q.SATQuantizerCell(15)), q.PoolCell((3, 3), (2, 2), (1, 1), pooling="Average"),
+              q.ConvCell(w2, quantizer=q.SATQuantizerCell(15))]
+    sm = q.SoftmaxCell()
+    print("average pool net: first iteration", flush=True)
+    loss = net.learn(t, 1)
+    want = q.train_sequential(x, cells_, sm, t, 1)
+    assert abs(loss - want) <= 1e-5 * want
+    for name, cell in zip(("c1", "pool", "c2"), cells_):
+        assert _close(net.outputs(name), cell.outputs, 2e-5), name
+        assert _close(net.diff_inputs(name), cell.diff_inputs, 1e-4), name
+    assert _close(net.weights("c1"), cells_[0].w, 1e-4) and _close(net.weights("c2"), cells_[2].w, 1e-4)
+    assert not np.array_equal(net.weights("c1"), w1)          # the gradient went through the pooling
+    print("average pool net: ten more", flush=True)
+    for it in range(10):
+        loss = net.learn(t, 1)
+        want = q.train_sequential(x, cells_, sm, t, 1)
+        assert abs(loss - want) <= 1e-3 * want, it
+    assert _close(net.weights("c1"), cells_[0].w, 1e-3)
