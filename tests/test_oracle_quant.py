@@ -68,6 +68,79 @@ def test_sat_weight_grid_and_invariants(mode, rng):
         assert np.max(np.abs(wq - noq)) <= step / 2 + 1e-6
 
 
+def _weights_for_normalised(qn, wmax=1.2):
+    """float32 weights whose tanh(w) / max|tanh w| equals qn (float64 target), the maximum supplied by a first element."""
+    w = np.arctanh(np.clip(np.asarray(qn, np.float64), -1, 1) * np.tanh(wmax) * (1 - 1e-12))
+    return np.concatenate([[wmax], w]).astype(np.float32)
+
+
+@pytest.mark.parametrize("rng", [15.0, 255.0, 3.0])
+def test_sat_fullrange_forward_closed_form(rng):
+    """quantize_weight_fullrange_propagate (src/Quantizer/QAT/Kernel/SATQuantizer_Frame_Kernels.cpp:117-146) in float64:
+    q = (t/m + 1)/2; level = rint((R + 0.9998) q - 0.4999); w_q = 2 level / R - 1.  Exact values away from ties, the grid,
+    and probes on both sides of the first and last bin edges, which sit at q = (k + 0.9999) / (R + 0.9998): with the
+    offset dropped, with 1/(2R) in its place, or with the slope 1 + 1/R, a probe lands on the other level."""
+    w = RNG.normal(0, 0.6, size=6000).astype(np.float32)
+    t = np.tanh(w.astype(np.float64))
+    m = np.abs(t).max()
+    arg = (rng + 0.9998) * (0.5 * (t / m + 1.0)) - 0.4999
+    safe = np.abs(arg - np.floor(arg) - 0.5) > 1e-3
+    want = 2.0 * np.rint(arg) / rng - 1.0
+    got, tmax, _ = orc.sat_weight_forward(w, rng, "fullrange")
+    assert abs(tmax - m) < 1e-7 and safe.sum() > 0.99 * w.size
+    assert np.max(np.abs(got[safe] - want[safe])) < 5e-7
+    lev = (got.astype(np.float64) + 1.0) / 2.0 * rng
+    assert np.max(np.abs(lev - np.rint(lev))) < 1e-4
+    seen = set(np.rint(lev).astype(int).tolist())
+    assert seen <= set(range(int(rng) + 1)) and (rng > 15 or len(seen) == rng + 1)    # levels 0..R, nothing outside
+    # the ends: t/m = -1 -> level 0, t/m = +1 -> level R, i.e. exactly -1 and +1
+    ends, _, _ = orc.sat_weight_forward(np.array([-1.2, 1.2], np.float32), rng, "fullrange")
+    assert ends.tolist() == [-1.0, 1.0]
+    # probes 3e-5 of a level on either side of every bin edge
+    k = np.arange(int(rng))
+    for side, expect in ((-3e-5, k), (3e-5, k + 1)):
+        q = (k + 0.9999 + side) / (rng + 0.9998)
+        probe, _, _ = orc.sat_weight_forward(_weights_for_normalised(2 * q - 1), rng, "fullrange")
+        lv = np.rint((probe[1:].astype(np.float64) + 1.0) / 2.0 * rng).astype(int)
+        assert lv.tolist() == expect.tolist(), (side, rng)
+    # the edges are NOT those of the plain rounding of the default mode (q = (k + 0.5) / R): on those the two modes differ
+    q = (k + 0.5 + 0.2 * (0.5 - (k + 0.5) / rng)) / rng        # between the default edge and the full-range edge
+    pr_f, _, _ = orc.sat_weight_forward(_weights_for_normalised(2 * q - 1), rng, "fullrange")
+    pr_d, _, _ = orc.sat_weight_forward(_weights_for_normalised(2 * q - 1), rng, "default")
+    assert np.count_nonzero(pr_f[1:] != pr_d[1:]) >= k.size - 1
+
+
+@pytest.mark.parametrize("rng", [15.0, 255.0, 7.0])
+def test_sat_asymrange_forward_closed_form(rng):
+    """quantize_weight_asymrange_propagate (SATQuantizer_Frame_Kernels.cpp:188-214) in float64: R' = floor(R/2);
+    level = rint((R' + 1/2) t/m - 1/2) in [-R'-1, R']; w_q = level / R'.  Bin edges at t/m = (k + 1) / (R' + 1/2)."""
+    r2 = np.floor(rng / 2)
+    w = RNG.normal(0, 0.6, size=6000).astype(np.float32)
+    t = np.tanh(w.astype(np.float64))
+    m = np.abs(t).max()
+    arg = (r2 + 0.5) * (t / m) - 0.5
+    safe = np.abs(arg - np.floor(arg) - 0.5) > 1e-3
+    want = np.rint(arg) / r2
+    got, tmax, _ = orc.sat_weight_forward(w, rng, "asymrange")
+    assert abs(tmax - m) < 1e-7 and safe.sum() > 0.99 * w.size
+    assert np.max(np.abs(got[safe] - want[safe])) < 5e-7
+    lev = got.astype(np.float64) * r2
+    assert np.max(np.abs(lev - np.rint(lev))) < 1e-4
+    seen = set(np.rint(lev).astype(int).tolist())
+    assert seen <= set(range(-int(r2) - 1, int(r2) + 1)) and (rng > 15 or len(seen) == rng + 1)   # R + 1 levels, one more below
+    ends, _, _ = orc.sat_weight_forward(np.array([-1.2, 1.2], np.float32), rng, "asymrange")
+    assert ends.tolist() == [float(np.float32(-r2 - 1) * (np.float32(1.0) / np.float32(r2))), 1.0]
+    k = np.arange(-int(r2) - 1, int(r2))
+    for side, expect in ((-3e-5, k), (3e-5, k + 1)):
+        qn = (k + 1 + side) / (r2 + 0.5)
+        probe, _, _ = orc.sat_weight_forward(_weights_for_normalised(qn), rng, "asymrange")
+        assert np.rint(probe[1:].astype(np.float64) * r2).astype(int).tolist() == expect.tolist(), (side, rng)
+    # the un-rounded twin is the same affine map
+    noq, _, _ = orc.sat_weight_forward(w, rng, "none_asym")
+    assert np.max(np.abs(noq - (arg / r2))) < 1e-6
+
+
+
 def test_sat_symrange_rint_is_half_to_even():
     # Find float32 inputs whose normalised value times 7 is an exact tie k+0.5 and
     # check they land on the even neighbour (rintf), not away from zero (roundf).
