@@ -140,7 +140,22 @@ typedef struct n2d2hip_conv_desc {
     int dilX, dilY;
     int groups;             /* Cell::getNbGroups of the mapping (ref: src/Cell/Cell.cpp:251-300): 1, or C == O (depthwise) */
     int weight_bits;        /* 8: int8_t weights; 4: two weights per byte, element 2i in the low nibble */
+    int kernel_choice;      /* 0: the library chooses among its kernels.  Otherwise N2D2HIP_KERNEL_* bits, which only steer
+                               that choice among kernels that compute the same result (tests use them to cover every
+                               kernel); read from the descriptor when the cell is created (integer cells) or on each call
+                               (float passes: give the same value to n2d2hip_conv2d_f32_workspace_bytes and to the pass).
+                               No counterpart in the reference. */
 } n2d2hip_conv_desc;
+enum {
+    N2D2HIP_KERNEL_NO_PIPE = 1,     /* integer cells: general register-staged kernel instead of the pipelined one */
+    N2D2HIP_KERNEL_NO_STEM = 2,     /* no first-layer kernel */
+    N2D2HIP_KERNEL_NO_HI16 = 4,     /* 32-bit rescale epilogue instead of the scaled-up 16-bit one */
+    N2D2HIP_KERNEL_NO_SUM16 = 8,    /* folded residual sum on 32 bits (read by n2d2hip_conv_fuse_sum) */
+    N2D2HIP_KERNEL_TILE_M64 = 16,   /* force 64-pixel tiles */
+    N2D2HIP_KERNEL_TILE_M128 = 32,  /* force 128-pixel tiles */
+    N2D2HIP_KERNEL_F32_DIRECT = 64, /* float passes: direct kernels that add in the reference's order */
+    N2D2HIP_KERNEL_F32_GEMM = 128   /* float passes: matrix-core implicit GEMM */
+};
 
 typedef struct n2d2hip_conv_s* n2d2hip_conv_t;
 

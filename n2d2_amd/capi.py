@@ -19,6 +19,9 @@ POOL_MAX, POOL_AVERAGE = 0, 1
 COEFF_PER_LAYER, COEFF_PER_INPUT, COEFF_PER_CHANNEL = 0, 1, 2
 SAT_NONE, SAT_DEFAULT, SAT_FULLRANGE, SAT_SYMRANGE, SAT_ASYMRANGE, SAT_NONE_ASYM = range(6)
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOT_QUANTIZED, ERR_WORKSPACE = range(6)
+# n2d2hip_conv_desc.kernel_choice bits
+KERNEL_NO_PIPE, KERNEL_NO_STEM, KERNEL_NO_HI16, KERNEL_NO_SUM16, KERNEL_TILE_M64, KERNEL_TILE_M128, KERNEL_F32_DIRECT, KERNEL_F32_GEMM = (
+    1, 2, 4, 8, 16, 32, 64, 128)
 
 # every symbol include/n2d2hip.h declares
 SYMBOLS = [
@@ -53,7 +56,7 @@ class Activation(C.Structure):
 class ConvDesc(C.Structure):
     _fields_ = [("C", C.c_int), ("O", C.c_int), ("kW", C.c_int), ("kH", C.c_int), ("strideX", C.c_int), ("strideY", C.c_int),
                 ("padL", C.c_int), ("padT", C.c_int), ("padR", C.c_int), ("padB", C.c_int), ("dilX", C.c_int), ("dilY", C.c_int),
-                ("groups", C.c_int), ("weight_bits", C.c_int)]
+                ("groups", C.c_int), ("weight_bits", C.c_int), ("kernel_choice", C.c_int)]
 
 
 class PoolDesc(C.Structure):

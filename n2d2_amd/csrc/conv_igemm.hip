@@ -751,7 +751,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     const n2d2hip_conv_desc& d = c->desc;
     bool bn128_unused;
     N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0)
-                        || (pipe_eligible(c, &bn128_unused) && getenv("N2D2HIP_NO_PIPE") == nullptr && d.dilX == 1 && d.dilY == 1),
+                        || (pipe_eligible(c, &bn128_unused) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE) && d.dilX == 1 && d.dilY == 1),
                     N2D2HIP_ERR_UNSUPPORTED, "conv_forward: this convolution does not take tensors with a halo (n2d2hip_conv_accepts_halo)");
     N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED,
                     "conv_forward: tensors must be NHWC (use n2d2hip_convert at graph edges)");
@@ -832,7 +832,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     N2D2HIP_REQUIRE(!other || (pipe && out_pixels * out->cs < (1ll << 31)), N2D2HIP_ERR_UNSUPPORTED,
                     "conv_forward_sum: tensor too large for the fused kernel");
     N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0) || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: tensor with a halo too large");
-    if (pipe && (other || getenv("N2D2HIP_NO_PIPE") == nullptr)) {
+    if (pipe && (other || !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE))) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
         ConvPipeArgs q;
         q.c = a;
@@ -846,7 +846,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.c.epi.d = c->d_epi_tab + 3 * cp; q.c.epi.e = c->d_epi_tab + 4 * cp;
         }
 #ifdef N2D2HIP_PROFILE
-        q.prof = (long long*)strtoull(getenv("N2D2HIP_PROF_PTR"), nullptr, 16);
+        {
+            const char* pp = getenv("N2D2HIP_PROF_PTR");      // profiling builds only: where the blocks' timestamps go
+            N2D2HIP_REQUIRE(pp != nullptr, N2D2HIP_ERR_INVALID, "conv_forward: profiling build without N2D2HIP_PROF_PTR");
+            q.prof = (long long*)strtoull(pp, nullptr, 16);
+        }
 #endif
         magic_div((unsigned)(OH * OW), &q.ohw_mul, &q.ohw_sh);
         magic_div((unsigned)OW, &q.ow_mul, &q.ow_sh);
@@ -859,8 +863,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         // barrier waits overlap the other's MFMAs.  K advances by whole 128-byte lines when the channel count allows.
         // Layers with few pixels (deep stages) take 64-pixel tiles so that every CU still gets its two blocks.
         const long long tiles128 = ((Mll + 127) / 128) * a.ntiles_n;
-        const char* bm_env = getenv("N2D2HIP_BM64");
-        const bool small_m = bn128 && d.C % 128 == 0 && (bm_env ? atoi(bm_env) != 0 : tiles128 < (3 * num_cus()) / 2);
+        const bool small_m = bn128 && d.C % 128 == 0
+            && ((d.kernel_choice & (N2D2HIP_KERNEL_TILE_M64 | N2D2HIP_KERNEL_TILE_M128)) ? (d.kernel_choice & N2D2HIP_KERNEL_TILE_M64) != 0
+                                                                                            : tiles128 < (3 * num_cus()) / 2);
         // 64-channel layers whose K advances in 64-byte steps take 256-pixel tiles: twice the MFMAs per ring stage
         const bool wide64 = !bn128 && !other && d.C % 128 != 0 && Mll >= 256ll * 4 * num_cus();
         // A handful of tiles (the classifier's FC): 64 x 64 tiles, four times as many blocks share the long K
@@ -877,7 +882,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.sum = EpiArgs(); q.pre = EpiArgs();
         // Byte outputs of an integer rescale whose scaled-up tables fit: the rescaled value is read from the upper half of
         // the multiply-add's result
-        const bool hi16 = !other && c->hi16 && c->act->args.kind == EPI_I24 && is_byte_type(out->dtype) && getenv("N2D2HIP_NO_HI16") == nullptr;
+        const bool hi16 = !other && c->hi16 && c->act->args.kind == EPI_I24 && is_byte_type(out->dtype) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
         if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
         if (other) {
             const int cp = c->sum->act->cpad;
@@ -927,7 +932,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     {
         const int k = c->act->args.kind;
         if (c->d_wstem && !other && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32) && fits32
-            && getenv("N2D2HIP_NO_STEM") == nullptr) {
+            && !(d.kernel_choice & N2D2HIP_KERNEL_NO_STEM)) {
             ConvStemArgs q;
             q.c = a;
             if (k == EPI_I24) {
@@ -946,7 +951,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             magic_div((unsigned)OH, &q.oh_mul, &q.oh_sh);
             magic_div((unsigned)q.tiles_per_row, &q.tpr_mul, &q.tpr_sh);
             const int grid = 8 * q.nlanes * q.c.ntiles_n;
-            const bool hi16 = k == EPI_I24 && c->hi16 && is_byte_type(out->dtype) && getenv("N2D2HIP_NO_HI16") == nullptr;
+            const bool hi16 = k == EPI_I24 && c->hi16 && is_byte_type(out->dtype) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
             if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
             if (d.kH == 3) launch_stem<3>(q, hi16, grid, stream);
             else if (d.kH == 5) launch_stem<5>(q, hi16, grid, stream);
@@ -977,7 +982,7 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
 int n2d2hip_conv_accepts_halo(n2d2hip_conv_t c)
 {
     bool bn128;
-    return c && pipe_eligible(c, &bn128) && c->desc.dilX == 1 && c->desc.dilY == 1 && getenv("N2D2HIP_NO_PIPE") == nullptr ? 1 : 0;
+    return c && pipe_eligible(c, &bn128) && c->desc.dilX == 1 && c->desc.dilY == 1 && !(c->desc.kernel_choice & N2D2HIP_KERNEL_NO_PIPE) ? 1 : 0;
 }
 
 int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype)
@@ -1012,7 +1017,7 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
     std::vector<int> t(14 * (size_t)cp, 0);
     // The sum stage in 16-bit pairs needs: no clamp before a multiply anywhere, (conv + other) * c + d inside 16 bits, and
     // the two rescales in front of it in the form that leaves their result in the upper half of a 32-bit register
-    bool sum16 = !c->preclamp && c->hi16 && cp % 2 == 0 && getenv("N2D2HIP_NO_SUM16") == nullptr;
+    bool sum16 = !c->preclamp && c->hi16 && cp % 2 == 0 && !(d.kernel_choice & N2D2HIP_KERNEL_NO_SUM16);
     short* t16 = (short*)(t.data() + 10 * (size_t)cp);
     bool pre_clamp = pa ? pa->clipped : false, sum_clamp = sa->clipped;
     bool pre_in_range = pa != nullptr;

@@ -521,7 +521,7 @@ bool ConvCell_Frame_HIP<T>::prepare()
         const unsigned int cg = mNbChannels / mNbGroups;
         if (mWeights.dimX() != mKernelDims[0] || mWeights.dimY() != mKernelDims[1] || mWeights.dimZ() != cg || mWeights.dimB() != mNbOutputs)
             throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": weights must be {kW, kH, nbChannels/groups, nbOutputs}");
-        n2d2hip_conv_desc d;
+        n2d2hip_conv_desc d = {};
         d.C = (int)mNbChannels; d.O = (int)mNbOutputs; d.kW = (int)mKernelDims[0]; d.kH = (int)mKernelDims[1];
         d.strideX = (int)mStrideDims[0]; d.strideY = (int)mStrideDims[1];
         d.padL = d.padR = mPaddingDims[0]; d.padT = d.padB = mPaddingDims[1];

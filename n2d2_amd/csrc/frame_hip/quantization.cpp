@@ -217,59 +217,76 @@ void FcCell::processFreeParametersPerOutput(const std::function<Float_T(Float_T)
 }
 
 // -------------------------------------------------------- DeepNetQuantization
+namespace {
+
+// Largest multiplier a fixed-point mode can hold.
+std::uint64_t multiplierCeiling(ScalingMode mode)
+{
+    return mode == ScalingMode::FIXED_MULT16 ? (std::uint64_t)std::numeric_limits<std::int16_t>::max()
+                                             : (std::uint64_t)std::numeric_limits<std::int32_t>::max();
+}
+
+// How much of `scaling` a term 2^-shift covers, as a fraction of it.
+double shareOf(double scaling, std::size_t shift) { return 1.0 / (scaling * std::pow(2, shift)); }
+
+} // namespace
+
+// Per-output float factors -> (fractional bits, integer multipliers): the widest fractional part, 50 bits at most, with which
+// the largest factor still fits the mode's multiplier; a 16-bit request whose largest factor does not fit at all is served
+// in 32 bits and `mode` says so (ref: src/DeepNetQuantization.cpp:1043-1093; the expressions are the reference's, so that
+// the multipliers come out identical).
 std::pair<std::size_t, std::vector<std::int32_t> > DeepNetQuantization::approximateScalingWithFixedPoint(
     ScalingMode& mode, const std::vector<Float_T>& scalingPerOutput)
 {
     if (scalingPerOutput.empty())
         throw std::runtime_error("approximateScalingWithFixedPoint(): no scaling");
-    const std::uint64_t limit = (mode == ScalingMode::FIXED_MULT16) ? (std::uint64_t)std::numeric_limits<std::int16_t>::max()
-                                                                    : (std::uint64_t)std::numeric_limits<std::int32_t>::max();
-    const double maxScaling = *std::max_element(scalingPerOutput.begin(), scalingPerOutput.end());
-    if (maxScaling >= limit) {
-        if (mode == ScalingMode::FIXED_MULT16) {
-            std::cout << "Warning: Max scaling (" << maxScaling << ") doesn't fit in FIXED_MULT16. Falling back to FIXED_MULT32." << std::endl;
-            mode = ScalingMode::FIXED_MULT32;
-            return approximateScalingWithFixedPoint(mode, scalingPerOutput);
-        }
-        std::stringstream errorStr;
-        errorStr << "Max scaling (" << maxScaling << ") doesn't fit in FIXED_MULT32." << std::endl;
-        throw std::runtime_error(errorStr.str());
+    const double largest = *std::max_element(scalingPerOutput.begin(), scalingPerOutput.end());
+    if (mode == ScalingMode::FIXED_MULT16 && largest >= multiplierCeiling(mode)) {
+        std::cout << "Notice: a scaling of " << largest << " needs more than 16 bits; FIXED_MULT32 is used instead of FIXED_MULT16."
+                  << std::endl;
+        mode = ScalingMode::FIXED_MULT32;
     }
-    const std::size_t maxNbFractionalBits = 50;
-    const std::size_t nbFractionalBits
-        = std::min((std::size_t)std::floor(std::log(limit / maxScaling) / std::log(2.0)), maxNbFractionalBits);
-    std::vector<std::int32_t> scalingFixedPoint;
-    for (Float_T sc : scalingPerOutput)
-        scalingFixedPoint.push_back((std::int32_t)std::round(sc * (1ull << nbFractionalBits)));
-    return std::make_pair(nbFractionalBits, scalingFixedPoint);
+    const std::uint64_t ceiling = multiplierCeiling(mode);
+    if (largest >= ceiling) {
+        std::ostringstream msg;
+        msg << "approximateScalingWithFixedPoint(): a scaling of " << largest << " does not fit a 32-bit multiplier";
+        throw std::runtime_error(msg.str());
+    }
+    const std::size_t fractionalBits = std::min<std::size_t>((std::size_t)std::floor(std::log(ceiling / largest) / std::log(2.0)), 50);
+    std::pair<std::size_t, std::vector<std::int32_t> > result(fractionalBits, std::vector<std::int32_t>(scalingPerOutput.size()));
+    std::transform(scalingPerOutput.begin(), scalingPerOutput.end(), result.second.begin(),
+                   [fractionalBits](Float_T factor) { return (std::int32_t)std::round(factor * (1ull << fractionalBits)); });
+    return result;
 }
 
+// A factor in (0, 1] as a sum of `nbDivisions` terms 2^-shift, greedily: every term is the largest power of two that does not
+// overshoot what is still uncovered.  Returns the shifts and the fraction of the factor their sum amounts to, which the
+// caller folds into the cell's parameters.  Three corrections, as in the reference (src/DeepNetQuantization.cpp:1095-1134):
+// once the sum is exact, a further term is made by splitting the last one in two; a sum within 2 % of the factor counts as
+// exact; one further away has its last term doubled, which takes it above the factor.
 std::pair<std::vector<unsigned char>, double> DeepNetQuantization::approximateScalingWithPowerOf2Divs(Float_T scaling, std::size_t nbDivisions)
 {
-    static const double ROUNDING_THRESHOLD = 0.98;
     if (nbDivisions == 0 || !(scaling > 0.0) || scaling > 1.0)
         throw std::runtime_error("approximateScalingWithPowerOf2Divs(): needs 0 < scaling <= 1 and at least one division");
-    double precision = 0.0;
-    std::vector<unsigned char> powerOf2Divs(nbDivisions);
-    for (std::size_t iDiv = 0; iDiv < nbDivisions; ++iDiv) {
-        if (precision == 1.0) {
-            // the sum is exact already: split its last term into two equal halves
-            powerOf2Divs[iDiv - 1]++;
-            powerOf2Divs[iDiv] = powerOf2Divs[iDiv - 1];
-        } else {
-            const std::size_t exponent = (std::size_t)std::ceil(std::log2(1.0 / (scaling * (1.0 - precision))));
-            precision += 1.0 / (scaling * std::pow(2, exponent));
-            powerOf2Divs[iDiv] = static_cast<unsigned char>(exponent);
+    std::vector<unsigned char> shifts;
+    shifts.reserve(nbDivisions);
+    double covered = 0.0;
+    while (shifts.size() < nbDivisions) {
+        if (covered == 1.0) {
+            const unsigned char halved = (unsigned char)(shifts.back() + 1);
+            shifts.back() = halved;
+            shifts.push_back(halved);
+            continue;
         }
+        const std::size_t shift = (std::size_t)std::ceil(std::log2(1.0 / (scaling * (1.0 - covered))));
+        covered += shareOf(scaling, shift);
+        shifts.push_back(static_cast<unsigned char>(shift));
     }
-    if (precision >= ROUNDING_THRESHOLD) {
-        precision = 1.0;
-    } else if (precision < 1.0) {
-        // too far below: double the last term, which takes the sum above the scaling
-        precision += 1.0 / (scaling * std::pow(2, powerOf2Divs.back()));
-        powerOf2Divs.back() = powerOf2Divs.back() - 1;
-    }
-    return std::make_pair(powerOf2Divs, precision);
+    if (covered >= 0.98)
+        return std::make_pair(shifts, 1.0);
+    covered += shareOf(scaling, shifts.back());
+    shifts.back() = (unsigned char)(shifts.back() - 1);
+    return std::make_pair(shifts, covered);
 }
 
 void DeepNetQuantization::approximateActivationScaling(Cell& cell, Activation& activation, ScalingMode actScalingMode)

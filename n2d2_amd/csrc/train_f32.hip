@@ -18,6 +18,7 @@ struct ConvF32 {
     int B, C, H, W, O, oH, oW, kW, kH, Cw;      // Cw = C / groups
     int sx, sy, pl, pt, pr, pb, dx, dy;
     int depthwise;                                // groups == C == O
+    int choice;                                   // the descriptor's kernel_choice bits
 };
 
 __device__ __forceinline__ double wave_sum_d(double v)
@@ -594,19 +595,18 @@ static int make_conv(const n2d2hip_conv_desc* d, int B, int H, int W, bool backw
     N2D2HIP_REQUIRE((size_t)B * std::max(d->C, d->O) * std::max((size_t)H * W, (size_t)oH * oW) < ((size_t)1 << 40), N2D2HIP_ERR_INVALID,
                     "%s: tensor too large", who);
     *q = ConvF32{B, d->C, H, W, d->O, oH, oW, d->kW, d->kH, d->C / d->groups, d->strideX, d->strideY,
-                 d->padL, d->padT, d->padR, d->padB, d->dilX, d->dilY, d->groups > 1 ? 1 : 0};
+                 d->padL, d->padT, d->padR, d->padB, d->dilX, d->dilY, d->groups > 1 ? 1 : 0, d->kernel_choice};
     return N2D2HIP_OK;
 }
 
 // The matrix-core kernel serves ungrouped convolutions without dilation that are worth a 128 x 128 tile; the direct
-// kernels keep the rest (depthwise, dilated, tiny).  N2D2HIP_F32_PATH=direct|gemm overrides the size rule.
+// kernels keep the rest (depthwise, dilated, tiny).  The descriptor's kernel_choice (N2D2HIP_KERNEL_F32_DIRECT / _GEMM) overrides the size rule.
 static bool use_gemm(const ConvF32& q)
 {
     if (q.depthwise || q.dx != 1 || q.dy != 1)
         return false;
-    const char* e = getenv("N2D2HIP_F32_PATH");
-    if (e && !strcmp(e, "direct")) return false;
-    if (e && !strcmp(e, "gemm")) return true;
+    if (q.choice & N2D2HIP_KERNEL_F32_DIRECT) return false;
+    if (q.choice & N2D2HIP_KERNEL_F32_GEMM) return true;
     return 2.0 * q.B * q.O * q.oH * q.oW * q.C * q.kH * q.kW >= 2.0e7;
 }
 

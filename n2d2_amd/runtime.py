@@ -126,11 +126,12 @@ def pack_int4(w):
 
 
 class Conv:
-    def __init__(self, w, bias, act, in_dtype, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, weight_bits=8):
-        """w: integer-valued [O, C/groups, kH, kW]; stride/dil (x,y); pad (L,T,R,B)."""
+    def __init__(self, w, bias, act, in_dtype, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, weight_bits=8,
+                 kernel_choice=0):
+        """w: integer-valued [O, C/groups, kH, kW]; stride/dil (x,y); pad (L,T,R,B); kernel_choice: capi.KERNEL_* bits."""
         O, Cg, kH, kW = w.shape
         self.desc = capi.ConvDesc(Cg * groups, O, kW, kH, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
-                                  dil[0], dil[1], groups, weight_bits)
+                                  dil[0], dil[1], groups, weight_bits, kernel_choice)
         self.act = act
         hw = pack_int4(w) if weight_bits == 4 else np.ascontiguousarray(w, dtype=np.int8)
         hb = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)

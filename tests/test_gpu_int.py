@@ -421,18 +421,15 @@ def test_conv_with_folded_residual_sum(rt):
                 for k in (0, 1):
                     ins = [y, o2] if k == 0 else [o2, y]
                     want = cells_ref.elemwise_cell(ins, sum_spec).astype(np.int64)
-                    conv = rt.Conv(w, bias, rt.Act(O, **conv_spec.kwargs()), capi.U8B, stride=(stride, stride))
                     ew = rt.ElemWiseSum(2, O, rt.Act(O, **sum_spec.kwargs()))
                     pre = None
                     if pre_spec is not None:
                         pre = rt.Act(O, **pre_spec.kwargs())
                         assert ew.fold_input_scaling(1 - k, pre)
                     # twice: with the sum's arithmetic on 16-bit pairs where the tables allow it, and on 32 bits
-                    for no16 in ("", "1"):
-                        if no16:
-                            os.environ["N2D2HIP_NO_SUM16"] = no16
+                    for no16 in (0, capi.KERNEL_NO_SUM16):
+                        conv = rt.Conv(w, bias, rt.Act(O, **conv_spec.kwargs()), capi.U8B, stride=(stride, stride), kernel_choice=no16)
                         assert conv.fuse_sum(ew, k, other_dtype), (C, O)
-                        os.environ.pop("N2D2HIP_NO_SUM16", None)
                         out = rt.DTensor(B, O, OH, OH, capi.U8B)
                         conv.forward_sum(dx, dother, out)
                         got = out.to_numpy()
@@ -471,15 +468,11 @@ def test_conv_rescale_variants_agree(rt):
                      ActSpec("Linear", "FixedMult16", rng.integers(2 ** 8, 2 ** 12, size=O), frac_bits=16, nb_bits=8, unsigned_out=False),
                      ActSpec("Rectifier", "FixedMult32", rng.integers(2 ** 18, 2 ** 22, size=O), frac_bits=28, nb_bits=8, unsigned_out=True)):
             want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(pad, pad, pad, pad)).astype(np.int64)
-            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad, pad, pad, pad))
             dx = rt.DTensor.from_numpy(x, capi.U8B)
-            for no16 in ("", "1"):
-                if no16:
-                    os.environ["N2D2HIP_NO_HI16"] = no16
-                try:
-                    got = conv.forward(dx).to_numpy()
-                finally:
-                    os.environ.pop("N2D2HIP_NO_HI16", None)
+            for no16 in (0, capi.KERNEL_NO_HI16):
+                conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad, pad, pad, pad),
+                               kernel_choice=no16)
+                got = conv.forward(dx).to_numpy()
                 assert np.array_equal(got, want), (C, O, k, spec.mode, no16, np.count_nonzero(got != want))
 
 

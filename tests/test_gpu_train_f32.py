@@ -40,8 +40,9 @@ def g():
             return t.cpu().numpy()
 
         @staticmethod
-        def desc(C_, O, k, s, p, groups, dil=1):
-            return capi_.ConvDesc(C_, O, k, k, s, s, p, p, p, p, dil, dil, groups, 0)
+        def desc(C_, O, k, s, p, groups, dil=1, path=None):
+            choice = {None: 0, "direct": capi_.KERNEL_F32_DIRECT, "gemm": capi_.KERNEL_F32_GEMM}[path]
+            return capi_.ConvDesc(C_, O, k, k, s, s, p, p, p, p, dil, dil, groups, 0, choice)
         torch_ = torch
     return G
 
@@ -53,9 +54,7 @@ def _rel(got, want, scale=None):
 
 @pytest.fixture(params=["direct", "gemm"])
 def path(request):
-    os.environ["N2D2HIP_F32_PATH"] = request.param
-    yield request.param
-    del os.environ["N2D2HIP_F32_PATH"]
+    return request.param
 
 
 @pytest.mark.parametrize("case", CASES)
@@ -71,7 +70,7 @@ def test_conv_forward_and_backward(g, case, path):
     w = rng.normal(size=(O, Cn // groups, k, k)).astype(np.float32)
     bias = rng.normal(size=O).astype(np.float32)
     want = orc.conv_forward_bias(orc.conv_forward(x, w, **kw), bias)
-    d = g.desc(Cn, O, k, s, p, groups)
+    d = g.desc(Cn, O, k, s, p, groups, path=path)
     dx_, dw_, db_ = g.dev(x), g.dev(w), g.dev(bias)
     y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
     need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
@@ -151,7 +150,7 @@ def test_conv_f32_edge_shapes(g, path):
         kw = dict(stride=(s, s), pad=(p, p, p, p))
         want = orc.conv_forward(x.astype(np.float64), w.astype(np.float64), **kw)
         mag = np.maximum(orc.conv_forward(np.abs(x).astype(np.float64), np.abs(w).astype(np.float64), **kw), 1e-3)
-        d = g.desc(Cn, O, k, s, p, 1)
+        d = g.desc(Cn, O, k, s, p, 1, path=path)
         dx_, dw_ = g.dev(x), g.dev(w)
         y = g.torch_.empty(want.shape, dtype=g.torch_.float32, device="cuda")
         need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))
@@ -201,7 +200,8 @@ def test_conv_f32_random_rectangular_shapes(g, path):
         x64, w64 = x.astype(np.float64), w.astype(np.float64)
         want = orc.conv_forward(x64, w64, **kw)
         assert want.shape == (B, O, oH, oW)
-        d = g.capi.ConvDesc(Cn, O, kW, kH, sx, sy, pl, pt, pr, pb, 1, 1, 1, 0)
+        d = g.capi.ConvDesc(Cn, O, kW, kH, sx, sy, pl, pt, pr, pb, 1, 1, 1, 0,
+                            {"direct": g.capi.KERNEL_F32_DIRECT, "gemm": g.capi.KERNEL_F32_GEMM}[path])
         print("random conv", path, (B, Cn, H, W, O, kW, kH, sx, sy, pl, pt), flush=True)
         dx_, dw_ = g.dev(x), g.dev(w)
         need = int(g.lib.n2d2hip_conv2d_f32_workspace_bytes(C.byref(d), B, H, W))

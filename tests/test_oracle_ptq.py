@@ -84,7 +84,7 @@ def test_host_code_matches_the_oracle():
             assert got[0] == want[0] and got[1] == want[1] and list(got[2]) == want[2], (mode, sc)
     with pytest.raises(fh.FrameHipError) as e:
         fh.approximate_scaling_with_fixed_point("FixedMult32", [3e9])
-    assert "doesn't fit in FIXED_MULT32" in str(e.value)
+    assert "does not fit a 32-bit multiplier" in str(e.value)      # a std::runtime_error, as in the reference
     for nb in (1, 2):
         for _ in range(300):
             s = float(np.float32(np.exp(rng.uniform(-9, 0))))
