@@ -4,7 +4,7 @@
 #include <limits>
 
 #include "common.h"
-#include "epilogue.cuh"
+#include "epilogue.hpp"
 
 namespace n2d2hip {
 

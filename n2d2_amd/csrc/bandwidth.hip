@@ -5,7 +5,7 @@
 #include <algorithm>
 
 #include "common.h"
-#include "epilogue.cuh"
+#include "epilogue.hpp"
 
 namespace n2d2hip {
 

@@ -22,7 +22,7 @@
 #include <type_traits>
 
 #include "common.h"
-#include "epilogue.cuh"
+#include "epilogue.hpp"
 
 namespace n2d2hip {
 
@@ -298,8 +298,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 }
 
 } // namespace n2d2hip
-#include "conv_pipe.cuh"
-#include "conv_stem.cuh"
+#include "conv_pipe.hpp"
+#include "conv_stem.hpp"
 namespace n2d2hip {
 
 // ------------------------------------------------------------ depthwise

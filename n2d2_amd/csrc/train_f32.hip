@@ -8,7 +8,7 @@
 #include <cstdlib>
 
 #include "common.h"
-#include "conv_f32_gemm.cuh"
+#include "conv_f32_gemm.hpp"
 
 namespace n2d2hip {
 
