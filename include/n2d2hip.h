@@ -255,6 +255,16 @@ size_t n2d2hip_quantizer_workspace_bytes(size_t n);
 int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range, int mode,
                                int apply_scaling, unsigned outputs_size, float* stats,
                                void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream);
+/* The same quantizer for callers that cannot allocate device memory or pass a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  The reductions' scratch (8448
+ * bytes) is a static array in device memory that every GPU the library runs on holds until the process ends; the call
+ * allocates nothing, on the host or on the device (the array's address is looked up once per device, on the first call
+ * there).  Same arguments and results as n2d2hip_sat_weight_forward without the workspace; tensors of more than
+ * N2D2HIP_SAT_STATIC_MAX_WEIGHTS elements are rejected with N2D2HIP_ERR_UNSUPPORTED.  All calls on one GPU share the one
+ * array: calls that overlap on a GPU (two streams, two threads) race; calls on one stream are ordered and safe. */
+#define N2D2HIP_SAT_STATIC_MAX_WEIGHTS (1u << 28)
+int n2d2hip_sat_weight_forward_static(const float* w, float* wq, size_t n, float range, int mode, int apply_scaling,
+                                      unsigned outputs_size, float* stats, n2d2hip_stream_t stream);
 /* ref: SATQuantizer_Frame_Kernels.cpp:349-404; factor = tanh_max * scaling read from stats */
 int n2d2hip_sat_weight_backward(const float* diff_wq, const float* w, float* diff_w, size_t n, float range,
                                 int mode, int apply_scaling, const float* stats, n2d2hip_stream_t stream);

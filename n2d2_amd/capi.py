@@ -32,7 +32,7 @@ SYMBOLS = [
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling",
-    "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_backward",
+    "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_forward_static", "n2d2hip_sat_weight_backward",
     "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
     "n2d2hip_conv2d_f32_forward", "n2d2hip_conv2d_f32_backward_data", "n2d2hip_conv2d_f32_backward_filter", "n2d2hip_conv2d_f32_workspace_bytes",
     "n2d2hip_conv2d_f32_backward_bias", "n2d2hip_softmax_f32_forward", "n2d2hip_loss_workspace_bytes", "n2d2hip_loss_f32",
@@ -103,6 +103,7 @@ def load():
     lib.n2d2hip_elemwise_fold_input_scaling.argtypes = [P, I, P]
     lib.n2d2hip_elemwise_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_sat_weight_forward.argtypes = [P, P, SZ, F, I, I, U, P, P, SZ, P]
+    lib.n2d2hip_sat_weight_forward_static.argtypes = [P, P, SZ, F, I, I, U, P, P]
     lib.n2d2hip_sat_weight_backward.argtypes = [P, P, P, SZ, F, I, I, P, P]
     lib.n2d2hip_sat_act_forward.argtypes = [P, P, SZ, F, P, P]
     lib.n2d2hip_sat_act_backward.argtypes = [P, P, P, SZ, F, P, F, P, P, SZ, P]

@@ -5,6 +5,7 @@
 // finished by a one-block kernel over at most PARTIALS block results, so the
 // result does not depend on scheduling.  Sums are carried in double.
 #include <algorithm>
+#include <mutex>
 
 #include "common.h"
 #include "epilogue.hpp"
@@ -282,20 +283,47 @@ unsigned ew_grid(size_t n)
 }
 } // namespace
 
+// Scratch of the entry point that allocates nothing: the block partials and the mean of the SAT weight quantizer's
+// reductions.  Every GPU the library runs on holds its own copy of this array until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)PARTIALS * sizeof(double) + 256;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES] = {};     // device address of `scratch` on each device, looked up once per device
+
+// Device address of the current device's copy of `scratch`; no allocation.
+int static_scratch(void** ptr)
+{
+    int dev = 0;
+    N2D2HIP_HIP_CHECK(hipGetDevice(&dev));
+    N2D2HIP_REQUIRE(dev >= 0 && dev < MAX_DEVICES, N2D2HIP_ERR_UNSUPPORTED, "static scratch: device ordinal %d (at most %d devices)", dev, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        N2D2HIP_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        N2D2HIP_REQUIRE(p != nullptr, N2D2HIP_ERR_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+        scratch_ptr[dev] = p;
+    }
+    *ptr = scratch_ptr[dev];
+    return N2D2HIP_OK;
+}
+} // namespace
+
 extern "C" {
 
 size_t n2d2hip_quantizer_workspace_bytes(size_t) { return (size_t)PARTIALS * sizeof(double) + 256; }
 
-int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range, int mode, int apply_scaling,
-                               unsigned outputs_size, float* stats, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream_)
+// The kernel sequence of the SAT weight quantizer over a workspace of n2d2hip_quantizer_workspace_bytes() bytes.
+static int sat_weight_forward_impl(const char* who, const float* w, float* wq, size_t n, float range, int mode, int apply_scaling,
+                                   unsigned outputs_size, float* stats, void* workspace, hipStream_t st)
 {
-    hipStream_t st = (hipStream_t)stream_;
-    N2D2HIP_REQUIRE(w && wq && stats && workspace, N2D2HIP_ERR_INVALID, "sat_weight_forward: null argument");
-    N2D2HIP_REQUIRE(n > 0, N2D2HIP_ERR_INVALID, "sat_weight_forward: empty tensor");
-    N2D2HIP_REQUIRE(mode >= N2D2HIP_SAT_NONE && mode <= N2D2HIP_SAT_NONE_ASYM, N2D2HIP_ERR_INVALID, "sat_weight_forward: bad mode %d", mode);
-    N2D2HIP_REQUIRE(workspace_bytes >= n2d2hip_quantizer_workspace_bytes(n), N2D2HIP_ERR_WORKSPACE, "sat_weight_forward: workspace of %zu bytes needed",
-                    n2d2hip_quantizer_workspace_bytes(n));
-    N2D2HIP_REQUIRE(range >= 1.0f, N2D2HIP_ERR_INVALID, "sat_weight_forward: range %g", (double)range);
+    N2D2HIP_REQUIRE(n > 0, N2D2HIP_ERR_INVALID, "%s: empty tensor", who);
+    N2D2HIP_REQUIRE(mode >= N2D2HIP_SAT_NONE && mode <= N2D2HIP_SAT_NONE_ASYM, N2D2HIP_ERR_INVALID, "%s: bad mode %d", who, mode);
+    N2D2HIP_REQUIRE(range >= 1.0f, N2D2HIP_ERR_INVALID, "%s: range %g", who, (double)range);
+    N2D2HIP_REQUIRE(!apply_scaling || n > 1, N2D2HIP_ERR_INVALID, "%s: SAT scaling needs more than one weight", who);
     const int nb = blocks_for(n);
     double* partial = (double*)workspace;
     float* mean = (float*)((char*)workspace + (size_t)PARTIALS * sizeof(double));
@@ -303,7 +331,6 @@ int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range,
     hipLaunchKernelGGL(sat_absmax_final, dim3(1), dim3(QBLOCK), 0, st, (const float*)partial, nb, stats);
     hipLaunchKernelGGL(sat_weight_quantize, dim3(ew_grid(n)), dim3(QBLOCK), 0, st, w, wq, n, range, mode, (const float*)stats);
     if (apply_scaling) {
-        N2D2HIP_REQUIRE(n > 1, N2D2HIP_ERR_INVALID, "sat_weight_forward: SAT scaling needs more than one weight");
         hipLaunchKernelGGL(sum_partial, dim3(nb), dim3(QBLOCK), 0, st, (const float*)wq, n, partial);
         hipLaunchKernelGGL(mean_final, dim3(1), dim3(QBLOCK), 0, st, (const double*)partial, nb, n, mean);
         hipLaunchKernelGGL(sqdev_partial, dim3(nb), dim3(QBLOCK), 0, st, (const float*)wq, n, (const float*)mean, partial);
@@ -312,6 +339,32 @@ int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range,
     }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
+}
+
+int n2d2hip_sat_weight_forward(const float* w, float* wq, size_t n, float range, int mode, int apply_scaling,
+                               unsigned outputs_size, float* stats, void* workspace, size_t workspace_bytes, n2d2hip_stream_t stream_)
+{
+    N2D2HIP_REQUIRE(w && wq && stats && workspace, N2D2HIP_ERR_INVALID, "sat_weight_forward: null argument");
+    N2D2HIP_REQUIRE(workspace_bytes >= n2d2hip_quantizer_workspace_bytes(n), N2D2HIP_ERR_WORKSPACE, "sat_weight_forward: workspace of %zu bytes needed",
+                    n2d2hip_quantizer_workspace_bytes(n));
+    return sat_weight_forward_impl("sat_weight_forward", w, wq, n, range, mode, apply_scaling, outputs_size, stats, workspace, (hipStream_t)stream_);
+}
+
+int n2d2hip_sat_weight_forward_static(const float* w, float* wq, size_t n, float range, int mode, int apply_scaling,
+                                      unsigned outputs_size, float* stats, n2d2hip_stream_t stream_)
+{
+    N2D2HIP_REQUIRE(w && wq && stats, N2D2HIP_ERR_INVALID, "sat_weight_forward_static: null argument");
+    N2D2HIP_REQUIRE(n <= (size_t)N2D2HIP_SAT_STATIC_MAX_WEIGHTS, N2D2HIP_ERR_UNSUPPORTED,
+                    "sat_weight_forward_static: %zu weights, at most %zu are served from the static scratch; use n2d2hip_sat_weight_forward",
+                    n, (size_t)N2D2HIP_SAT_STATIC_MAX_WEIGHTS);
+    static_assert(STATIC_SCRATCH_BYTES >= (size_t)PARTIALS * sizeof(double) + sizeof(float), "scratch holds the partials and the mean");
+    void* ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc != N2D2HIP_OK)
+        return rc;
+    // Nothing in the scratch has to start from zero: every pass writes the partials it then reads (the same block count
+    // both times), and the mean is written before it is read.
+    return sat_weight_forward_impl("sat_weight_forward_static", w, wq, n, range, mode, apply_scaling, outputs_size, stats, ws, (hipStream_t)stream_);
 }
 
 int n2d2hip_sat_weight_backward(const float* diff_wq, const float* w, float* diff_w, size_t n, float range, int mode,
