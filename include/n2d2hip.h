@@ -154,7 +154,9 @@ enum {
     N2D2HIP_KERNEL_TILE_M64 = 16,   /* force 64-pixel tiles */
     N2D2HIP_KERNEL_TILE_M128 = 32,  /* force 128-pixel tiles */
     N2D2HIP_KERNEL_F32_DIRECT = 64, /* float passes: direct kernels that add in the reference's order */
-    N2D2HIP_KERNEL_F32_GEMM = 128   /* float passes: matrix-core implicit GEMM */
+    N2D2HIP_KERNEL_F32_GEMM = 128,  /* float passes: matrix-core implicit GEMM */
+    N2D2HIP_KERNEL_NO_PATCH = 256,  /* integer cells: 3x3 convolutions on the pipelined kernel instead of the patch kernel */
+    N2D2HIP_KERNEL_PATCH = 512      /* the patch kernel wherever it can run, also where the library finds the pipelined one faster */
 };
 
 typedef struct n2d2hip_conv_s* n2d2hip_conv_t;

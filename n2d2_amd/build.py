@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libn2d2hip.so")
 GLUE_LIB = os.path.join(LIBDIR, "libn2d2_frame_hip.so")
-SOURCES = ["act.hip", "conv_igemm.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip"]
+SOURCES = ["act.hip", "conv_igemm.hip", "conv_patch.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip"]
 
 # -ffp-contract=off: float rescales must round the product and the sum
 # separately, as the reference (built for baseline x86-64) does.
@@ -43,7 +43,7 @@ def build(verbose=False):
         src, obj = pair
         return _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
 
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         outs = list(ex.map(compile_one, zip(SOURCES, objs)))
     outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs))
     # host cells ("Frame_HIP" model): plain C++ over the C ABI

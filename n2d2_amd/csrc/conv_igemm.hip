@@ -23,12 +23,10 @@
 
 #include "common.h"
 #include "epilogue.hpp"
+#include "mfma_util.hpp"
+#include "conv_patch.hpp"
 
 namespace n2d2hip {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v2i __attribute__((ext_vector_type(2)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 struct ConvArgs {
     const signed char* in;
@@ -389,6 +387,8 @@ struct n2d2hip_conv_s {
     bool hi16;
     // first-layer kernel (<= 4 input channels, horizontal stride 2): weights as [channel][kH * 32]
     signed char* d_wstem;
+    // 3x3 stride-1 kernel over inputs that carry their padding: weights in matrix-core fragment order
+    signed char* d_wfrag;
     bool is_fc;
     int fcH, fcW;
 };
@@ -540,7 +540,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -674,6 +674,13 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             hw.swap(full);
         }
     }
+    std::vector<signed char> hfrag;
+    if (!depthwise && !c->pix4 && d->weight_bits == 8 && d->kW == 3 && d->kH == 3 && d->strideX == 1 && d->strideY == 1 && d->dilX == 1
+        && d->dilY == 1 && d->padL == 1 && d->padT == 1 && d->padR == 1 && d->padB == 1 && c->in_cs == d->C && d->C % 64 == 0
+        && d->O % 64 == 0 && c->ktot == 9 * d->C && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PATCH)) {
+        hfrag.resize(conv_patch_weight_bytes(d->C, d->O));
+        conv_patch_weight_layout(hw.data(), d->C, d->O, hfrag.data());
+    }
 
     hipError_t e = hipMalloc((void**)&c->d_w, hw.size());
     if (e == hipSuccess) e = hipMemcpy(c->d_w, hw.data(), hw.size(), hipMemcpyHostToDevice);
@@ -692,6 +699,10 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
                             (signed char)read_weight(weights, (((long long)o * d->C + ch) * d->kH + ky) * d->kW + kx, 8);
         e = hipMalloc((void**)&c->d_wstem, ws.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wstem, ws.data(), ws.size(), hipMemcpyHostToDevice);
+    }
+    if (e == hipSuccess && !hfrag.empty()) {
+        e = hipMalloc((void**)&c->d_wfrag, hfrag.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_wfrag, hfrag.data(), hfrag.size(), hipMemcpyHostToDevice);
     }
     if (e == hipSuccess && !hepi.empty()) {
         e = hipMalloc((void**)&c->d_epi_tab, hepi.size() * sizeof(int));
@@ -725,6 +736,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_res_tab) (void)hipFree(c->d_res_tab);
     if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
     if (c->d_wstem) (void)hipFree(c->d_wstem);
+    if (c->d_wfrag) (void)hipFree(c->d_wfrag);
     delete c;
     return N2D2HIP_OK;
 }
@@ -832,6 +844,27 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     N2D2HIP_REQUIRE(!other || (pipe && out_pixels * out->cs < (1ll << 31)), N2D2HIP_ERR_UNSUPPORTED,
                     "conv_forward_sum: tensor too large for the fused kernel");
     N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0) || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: tensor with a halo too large");
+    if (pipe && !other && c->d_wfrag && in->halo == 1 && c->act->args.kind == EPI_I24 && c->bias_folded && is_byte_type(out->dtype)
+        && conv_patch_eligible(d.C, d.O, Wp) && out_pixels * out->cs < (1ll << 31) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE)
+        // where it is the faster of the two (measured): at least two 64-channel steps per tile, so that a tile's rescale is
+        // small beside its matrix instructions, and images large enough that the border positions it computes and drops
+        // stay under a third of the work
+        && ((d.kernel_choice & N2D2HIP_KERNEL_PATCH) || (d.C >= 128 && (long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135))) {
+        // 3x3, stride 1, on an input that carries its padding: nine shifted reads of one patch of pixels
+        ConvPatchArgs q = {};
+        q.in = a.in; q.wfrag = c->d_wfrag; q.out = out->data;
+        q.C = d.C; q.O = d.O; q.Hp = Hp; q.Wp = Wp; q.total = in->B * Hp * Wp;
+        q.out_cs = out->cs; q.out_halo = out->halo; q.OHp = OH + 2 * out->halo; q.OWp = OW + 2 * out->halo;
+        q.out_xor = out_xor;
+        magic_div((unsigned)(Hp * Wp), &q.img_mul, &q.img_sh);
+        magic_div((unsigned)Wp, &q.row_mul, &q.row_sh);
+        const int cp = c->act->cpad;
+        const bool hi16 = c->hi16 && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
+        q.ta = c->d_epi_tab; q.tb = c->d_epi_tab + cp; q.tc = c->d_epi_tab + (hi16 ? 5 : 2) * cp;
+        q.td = c->d_epi_tab + (hi16 ? 6 : 3) * cp; q.te = c->d_epi_tab + 4 * cp;
+        q.lo = c->act->args.lo; q.hi = c->act->args.hi; q.preclamp = c->preclamp ? 1 : 0;
+        return conv_patch_launch(q, hi16, num_cus(), stream);
+    }
     if (pipe && (other || !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE))) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile
         ConvPipeArgs q;

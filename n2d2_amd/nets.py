@@ -356,11 +356,12 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True):
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
-        a border of zeros around every image, which lets a padded KxK reader fetch every tap without a validity test."""
+        a border of zeros around every image, which lets a padded KxK reader fetch every tap without a validity test.
+        kernel_choice: capi.KERNEL_* bits handed to every convolution (which kernel runs, never what it computes)."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
         consumers = {}
@@ -394,7 +395,7 @@ class GpuNet:
             if l.type in ("conv", "fc"):
                 act = rt.Act(Co, **l.act.kwargs())
                 if l.type == "conv":
-                    cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits)
+                    cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits, kernel_choice)
                 else:
                     cell = rt.Fc(l.w, l.bias, act, ins[0].dtype, (ins[0].C, ins[0].H, ins[0].W), l.weight_bits)
                 if ins[0].halo and not (l.type == "conv" and cell.accepts_halo()):

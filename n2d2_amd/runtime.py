@@ -57,6 +57,14 @@ class DTensor:
         check(lib.n2d2hip_convert(src.ref, dst.ref, stream_ptr()))
         return dst
 
+    def with_halo(self, halo):
+        """A copy of this NHWC byte tensor stored with a border of `halo` zero pixels around every image."""
+        assert self.layout == capi.NHWC and self.halo == 0
+        dst = DTensor(self.B, self.C, self.H, self.W, self.dtype, halo=halo)
+        dst.buf.view(self.B, self.H + 2 * halo, self.W + 2 * halo, self.cs)[:, halo:self.H + halo, halo:self.W + halo, :] = \
+            self.buf.view(self.B, self.H, self.W, self.cs)
+        return dst
+
     def to_numpy(self):
         """Logical integer values as an int64 NCHW numpy array."""
         dst = DTensor(self.B, self.C, self.H, self.W, capi.I32, capi.NCHW)

@@ -532,6 +532,42 @@ def test_conv_reads_and_writes_halo_tensors(rt):
     assert not c48.accepts_halo()
 
 
+def test_conv3x3_patch_kernel_bit_exact(rt):
+    """3x3, stride 1, padding 1 on an input that carries its padding: the kernel that reads one patch of pixels at nine
+    shifts (weights straight to registers in fragment order), against the oracle and against the pipelined kernel, over
+    image sizes whose rows are shorter and longer than a tile, tiles that straddle images, channel counts that take the
+    two-wave and the four-wave block, several 64-channel steps, both epilogues, outputs with and without a border."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    from oracle.cells import ActSpec
+    rng = np.random.default_rng(123)
+    cases = ((64, 64, 9, 7, 3), (64, 128, 28, 28, 2), (128, 64, 14, 14, 5), (192, 128, 7, 7, 9), (64, 64, 56, 56, 1),
+             (128, 256, 5, 33, 2), (256, 128, 30, 3, 3), (64, 192, 1, 1, 70), (128, 128, 60, 4, 1))
+    for C, O, H, W, B in cases:
+        x = rng.integers(0, 256, size=(B, C, H, W))
+        w = np.clip(np.rint(rng.normal(0, 25, size=(O, C, 3, 3))), -127, 127).astype(np.int64)
+        bias = rng.integers(-3000, 3000, size=O)
+        specs = (ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(9, 13, size=O)], 1), nb_bits=8, unsigned_out=True),
+                 ActSpec("Linear", "SingleShift", rng.integers(9, 15, size=O), nb_bits=8, unsigned_out=False),
+                 ActSpec("Rectifier", "FixedMult16", rng.integers(2 ** 6, 2 ** 10, size=O), frac_bits=20, nb_bits=8, unsigned_out=True))
+        dx = rt.DTensor.from_numpy(x, capi.U8B).with_halo(1)
+        for spec in specs:
+            want = cells_ref.conv_cell(x, w, bias, spec, pad=(1, 1, 1, 1)).astype(np.int64)
+            for choice in (capi.KERNEL_PATCH, capi.KERNEL_PATCH | capi.KERNEL_NO_HI16, 0, capi.KERNEL_NO_PATCH):
+                print("patch conv", (C, O, H, W, B), spec.mode, choice, flush=True)
+                conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, pad=(1, 1, 1, 1), kernel_choice=choice)
+                assert conv.accepts_halo()
+                for out_halo in (0, 1):
+                    out = conv.make_output(dx, halo=out_halo)
+                    conv.forward(dx, out)
+                    got = out.to_numpy()
+                    assert np.array_equal(got, want), (C, O, H, W, B, spec.mode, choice, out_halo, np.count_nonzero(got != want))
+                    if out_halo:
+                        border = out.buf.view(B, H + 2, W + 2, out.cs).clone()
+                        border[:, 1:H + 1, 1:W + 1, :] = out.buf.view(-1)[0]
+                        assert bool((border == out.buf.view(-1)[0]).all()), "the output's border is left alone"
+
+
 def conv_spec_for(O, rng):
     from oracle.cells import ActSpec
     return ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=False)
