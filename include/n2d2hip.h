@@ -204,7 +204,8 @@ typedef struct n2d2hip_pool_desc {
 int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* desc, int H, int W, int* outH, int* outW);
 /* Per-channel (unit map) quantized pooling on NHWC U8/I8/U8B; average is the truncated
  * quotient sum / (poolW*poolH) (ref: src/Cell/PoolCell_Frame_Kernels.cpp:26-197,
- * src/Cell/PoolCell_Frame.cpp:123-174).  out has the dtype of in. */
+ * src/Cell/PoolCell_Frame.cpp:123-174).  out has the dtype of in; a 2x2 or 3x3 max pooling whose channel stride is a
+ * multiple of 16 may write an `out` with a halo (its readers' padding), the other poolings refuse one. */
 int n2d2hip_pool_forward(const n2d2hip_pool_desc* desc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
 
@@ -241,6 +242,25 @@ int n2d2hip_conv_forward_sum(n2d2hip_conv_t conv, const n2d2hip_tensor* in, cons
                              const n2d2hip_tensor* out, n2d2hip_stream_t stream);
 int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
                              n2d2hip_stream_t stream);
+
+/* Graph-level fusion of a residual bottleneck with 64 middle channels into one launch: `reduce` (1x1, 64 or 256 -> 64),
+ * `conv3x3` (3x3, stride 1, padding 1, 64 -> 64) and, unless `expand` is NULL, `expand` (1x1, 64 -> 256) with the two-input
+ * ElemWise sum that n2d2hip_conv_fuse_sum has folded into it; the sum's other input is the block's input itself (256
+ * channels, through the ScalingCell folded into the sum if there is one) or, if `projection` is not NULL, that 1x1
+ * convolution (64 -> 256) of the block's input.  That is ConvCell_Frame::propagate three or four times and
+ * ElemWiseCell_Frame::propagate (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/ElemWiseCell_Frame.cpp:104-136) without
+ * the tensors in between ever reaching memory; results are those of the separate cells, bit for bit.  The handles are
+ * borrowed, must outlive the bottleneck and stay usable on their own.  Returns N2D2HIP_ERR_UNSUPPORTED (the caller keeps
+ * the separate launches) unless every cell is 8-bit with an integer rescale that fits the scaled-up tables, and the sum
+ * runs on 16-bit pairs. */
+typedef struct n2d2hip_bottleneck_s* n2d2hip_bottleneck_t;
+int n2d2hip_bottleneck_create(n2d2hip_conv_t reduce, n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand, n2d2hip_conv_t projection,
+                              n2d2hip_bottleneck_t* bottleneck);
+int n2d2hip_bottleneck_destroy(n2d2hip_bottleneck_t bottleneck);
+/* `in`: the block's input, NHWC bytes with a border of one pixel (halo 1; rows of at most 61 pixels); `out`: the sum's
+ * output (the 3x3 convolution's when `expand` is NULL), NHWC bytes of the same height and width, with or without a border. */
+int n2d2hip_bottleneck_forward(n2d2hip_bottleneck_t bottleneck, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                               n2d2hip_stream_t stream);
 
 /* --------------------------------------------------- SAT / LSQ fake-quant */
 /* Weight quantizer modes, numbered as SATQuantizerCell_Frame::propagate selects them

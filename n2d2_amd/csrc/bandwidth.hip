@@ -77,7 +77,7 @@ typedef short v2s __attribute__((ext_vector_type(2)));
 template <int PW, int PH>
 __global__ __launch_bounds__(256) void pool_max_fast_kernel(const signed char* __restrict__ in, int cs, int B, int H, int W,
                                                             signed char* __restrict__ out, int OH, int OW,
-                                                            int strideX, int strideY, int padX, int padY, unsigned flip)
+                                                            int strideX, int strideY, int padX, int padY, unsigned flip, int out_halo)
 {
     const int cq = cs >> 4;
     const long long total = (long long)B * OH * OW * cq;
@@ -125,7 +125,10 @@ __global__ __launch_bounds__(256) void pool_max_fast_kernel(const signed char* _
             __builtin_memcpy(&uo, &mo, 4);
             res[q] = (((ue >> 8) & 0x00FF00FFu) | (uo & 0xFF00FF00u)) ^ flip;
         }
-        *(uint4*)(out + idx * 16) = uint4{res[0], res[1], res[2], res[3]};
+        // an output that carries its readers' padding: the interior of (OH + 2 halo) x (OW + 2 halo) pixels per image
+        const long long opix = out_halo ? ((long long)b * (OH + 2 * out_halo) + oy + out_halo) * (OW + 2 * out_halo) + ox + out_halo
+                                        : idx / cq;
+        *(uint4*)(out + (opix * cq + idx % cq) * 16) = uint4{res[0], res[1], res[2], res[3]};
     }
 }
 
@@ -371,7 +374,7 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     int rc, OH, OW;
     N2D2HIP_REQUIRE(d != nullptr, N2D2HIP_ERR_INVALID, "pool_forward: null descriptor");
     N2D2HIP_REQUIRE(d->pooling == N2D2HIP_POOL_MAX || d->pooling == N2D2HIP_POOL_AVERAGE, N2D2HIP_ERR_INVALID, "pool_forward: bad pooling %d", d->pooling);
-    if ((rc = check_tensor(in, "pool input")) || (rc = check_tensor(out, "pool output")) || (rc = n2d2hip_pool_out_dims(d, in->H, in->W, &OH, &OW)))
+    if ((rc = check_tensor(in, "pool input")) || (rc = check_tensor(out, "pool output", true)) || (rc = n2d2hip_pool_out_dims(d, in->H, in->W, &OH, &OW)))
         return rc;
     N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED, "pool_forward: tensors must be NHWC");
     N2D2HIP_REQUIRE(is_byte_type(in->dtype) && out->dtype == in->dtype, N2D2HIP_ERR_INVALID, "pool_forward: byte tensors of one dtype expected");
@@ -385,6 +388,8 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     // windows that all hold at least one input element, square 2x2 or 3x3, 16-byte channel groups
     const bool fast = d->pooling == N2D2HIP_POOL_MAX && in->cs % 16 == 0 && d->poolW == d->poolH && (d->poolW == 2 || d->poolW == 3)
         && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < in->W && (OH - 1) * d->strideY - d->padY < in->H;
+    N2D2HIP_REQUIRE(out->halo == 0 || fast, N2D2HIP_ERR_UNSUPPORTED,
+                    "pool_forward: only the 2x2 / 3x3 max pooling of 16-byte channel groups writes an output with a halo");
     if (d->pooling == N2D2HIP_POOL_AVERAGE && OH == 1 && OW == 1 && d->poolW == in->W && d->poolH == in->H && d->padX == 0 && d->padY == 0) {
         const int slabs = (in->cs + 255) / 256;
         hipLaunchKernelGGL(global_avg_pool_kernel, dim3((unsigned)(in->B * slabs)), dim3(256), 0, (hipStream_t)stream,
@@ -394,10 +399,10 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
         const unsigned g16 = (unsigned)round_up((int)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64)), 8);
         if (d->poolW == 3)
             hipLaunchKernelGGL((pool_max_fast_kernel<3, 3>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
-                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip);
+                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip, out->halo);
         else
             hipLaunchKernelGGL((pool_max_fast_kernel<2, 2>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
-                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip);
+                               in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip, out->halo);
     } else if (d->pooling == N2D2HIP_POOL_MAX)
         hipLaunchKernelGGL(pool_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);

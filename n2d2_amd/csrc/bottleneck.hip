@@ -1,0 +1,760 @@
+// A residual bottleneck with 64 middle channels in one launch: 1x1 convolution (C_in -> 64), 3x3 convolution (64 -> 64,
+// stride 1, padding 1), 1x1 convolution (64 -> 256) and the two-input ElemWise sum with the block's input (through the
+// ScalingCell folded into the sum, if any) or with a 1x1 projection of it.  Launched cell by cell, such a block at
+// 56 x 56 moves its 256-channel tensors through HBM four times and its middle tensors twice each; here the input is read
+// once (twice where the sum needs it again: those lines are still in cache), the output is written once and the middle
+// tensors live in LDS.  The kernel is bound by instruction issue (about 3000 instructions per wave and tile, most of them
+// the three rescales of the sum): measured at 56 x 56, batch 128, it replaces the four launches of a block with a
+// projection shortcut at 0.7 of their time and ties with the three launches of an identity block.
+//
+// Tensors carry their padding as a border of zeros.  In the flattened index space (image, padded row, padded column)
+// a 3x3 window is nine shifts of one run of positions, so a tile is 128 consecutive positions q0 .. q0 + 127, border
+// positions included (their results are not stored):
+//  phase 1  t1[256 positions q0 - 64 ..][64] = reduce(x): pixel fragments straight from global memory to registers (each
+//           wave owns 64 positions and all 64 channels, so nothing is fetched twice), rescaled to bytes, border and
+//           out-of-range positions forced to the stored form of 0 (that is what the 3x3 convolution's padding is), to LDS;
+//  phase 2  t2[128][64] = conv3x3(t1): nine shifted reads of t1 per wave (32 positions x 64 channels), weights resident in
+//           LDS in fragment order for the block's whole life, rescaled to bytes, to LDS;
+//  phase 3  out[128][256] = sum(expand(t2), other): each wave owns 64 output channels of all 128 positions, in two halves
+//           of 64 positions; `other` is x in the output's own layout (32 channels per lane, brought into the accumulator
+//           layout by lane-half exchanges), or the projection of x accumulated beside the expansion; the three rescales
+//           run on pairs of 16-bit values as in the pipelined kernel's folded sum.
+// t2 takes t1's place in LDS (four barriers per tile).  Global loads are requested a phase or a tile ahead and their waits
+// are written by hand.
+#include <algorithm>
+#include <cstdlib>
+#include <limits>
+#include <vector>
+
+#include "common.h"
+#include "conv_handle.hpp"
+#include "epilogue.hpp"
+#include "mfma_util.hpp"
+
+namespace n2d2hip {
+
+// Offsets (in ints) of the rescale tables inside one device array: multiplier / addend scaled up so that the result is
+// the upper half of the 32-bit multiply-add (reduce, 3x3, expand, other), and the sum's multiplier, addend and shift as
+// pairs of 16-bit values.
+enum { TB_A_C = 0, TB_A_D = 64, TB_B_C = 128, TB_B_D = 192, TB_C_C = 256, TB_C_D = 512, TB_O_C = 768, TB_O_D = 1024,
+       TB_S_C = 1280, TB_S_D = 1408, TB_S_E = 1536, TB_INTS = 1664 };
+
+struct BottleneckArgs {
+    const signed char* in;      // B x Hp x Wp x C_in bytes, borders hold the stored form of 0
+    signed char* out;           // NHWC bytes: 256 channels (64 when only the first two cells are fused)
+    int Hp, Wp, total;          // rows / columns per image with the border, positions in all
+    int out_cs, out_halo, OHp, OWp;
+    int out_bytes;              // size of the output buffer (stores are bounds-checked against it)
+    unsigned img_mul, img_sh, row_mul, row_sh;      // division by Hp * Wp and by Wp
+    int ntiles, xcd_tiles, nlanes;
+    const signed char* wa;      // reduce:     [2 channel tiles][C_in / 32 K steps][64 lanes][16 bytes]
+    const signed char* wb;      // 3x3:        [2][9 taps][2][64][16]
+    const signed char* wc;      // expand:     [8][2][64][16]
+    const signed char* wp;      // projection: [8][C_in / 32][64][16]
+    const int* tab;             // TB_INTS ints
+    int c_lo, c_hi, o_lo, o_hi;     // saturation ranges of the expansion and of the sum's other operand
+    unsigned t1_zero;           // stored form of 0 in t1, in every byte
+    unsigned t1_xor, t2_xor, out_xor;     // 0x80808080 where the tensor is stored as value - 128
+    unsigned res_flip;          // turns a stored byte of x into the unsigned operand of the sum
+    int other_off;              // projection: added to its saturated value (the zero point the sum's tables expect)
+#ifdef N2D2HIP_PROFILE
+    long long* prof;            // 8 counters per block
+#endif
+};
+
+__device__ __forceinline__ int sw64(int row) { return (row >> 2) & 3; }
+
+// Barrier between two phases that hand data over through LDS: this wave's LDS operations are complete; its global loads
+// (the next tile's pixels, the sum's other operand) stay in flight, which __syncthreads() would wait for.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+// Global loads whose wait is written by hand (the compiler would put vmcnt(0) in front of the first use of a register
+// loaded in the previous tile, and that waits for the previous tile's stores as well).  Vector memory operations of a wave,
+// loads and stores alike, complete in issue order: vmcnt(n) with n = the number of operations issued after the ones needed.
+__device__ __forceinline__ void gload128(v4i& dst, const void* p)
+{
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(p) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// CIN: input channels (64 or 256).  OTHER: what the sum adds to the expansion: x itself (OTHER_X, CIN == 256), x through
+// the folded ScalingCell whose result cannot leave its range (OTHER_X_SCALED) or can (OTHER_X_SCALED_SAT), or a
+// projection of x (OTHER_PROJECTION).  NPH: 2 = reduce + 3x3 only (t2 is the output), 3 = the whole block.
+// The reduce, 3x3 and sum cells saturate to [0, 255] (Rectifier cells with unsigned outputs), which has an instruction of
+// its own; the expansion and the projection saturate to the ranges given.
+enum { OTHER_X = 0, OTHER_X_SCALED = 1, OTHER_X_SCALED_SAT = 2, OTHER_PROJECTION = 3 };
+template <int CIN, int OTHER, int NPH>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bottleneck_kernel(BottleneckArgs q)
+{
+    constexpr bool PROJ = OTHER == OTHER_PROJECTION;
+    constexpr int KS = CIN / 32;                   // K steps of the reduce convolution
+    constexpr int BM = 128;
+    // LDS: 3x3 weights and reduce weights in fragment order (resident), t1, tables.  t2 takes the first half of t1's place
+    // once every wave has read t1 (two blocks of 76 KB fit a CU's 160 KB; with a t2 of its own they would not).
+    constexpr int WB_OFF = 0, WB_BYTES = 2 * 9 * 2 * 1024;
+    constexpr int WA_OFF = WB_OFF + WB_BYTES, WA_BYTES = 2 * KS * 1024;      // [K step][channel tile][lane]
+    constexpr int T1_OFF = WA_OFF + WA_BYTES, T1_BYTES = 256 * 64;
+    constexpr int T2_OFF = T1_OFF;
+    constexpr int TAB_OFF = T1_OFF + T1_BYTES;
+    // vector memory operations a wave issues per tile, in this order: [phase 1] the sum's other operand and the expansion's
+    // weights (N_P3), the next tile's pixels (N_X); [phase 2 or 3] the stores (N_ST)
+    constexpr int N_X = 2 * KS;
+    constexpr int N_P3 = NPH == 3 ? (PROJ ? 4 * KS + 2 * KS : 8) + 4 : 0;
+    constexpr int N_ST = NPH == 3 ? 8 : 2;
+    static_assert(N_X + N_P3 + N_ST < 60, "vmcnt is a 6-bit counter");
+    static_assert(PROJ || CIN == 256, "the identity shortcut has the output's channel count");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + TB_INTS * 4];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int first = xcd * q.xcd_tiles + slot;
+    const int last = min((xcd + 1) * q.xcd_tiles, q.ntiles);
+    const int ntile = (first < last) ? (last - first + q.nlanes - 1) / q.nlanes : 0;
+    if (ntile == 0)
+        return;
+
+    // ---- resident operands
+    for (int i = tid; i < WB_BYTES / 16; i += 256)
+        *(v4i*)(smem + WB_OFF + i * 16) = *(const v4i*)(q.wb + (size_t)i * 16);
+    for (int i = tid; i < WA_BYTES / 16; i += 256) {
+        // LDS order [K step][channel tile][lane]; global order [channel tile][K step][lane]
+        const int kk = i / 128, ct = (i / 64) & 1, ln = i & 63;
+        *(v4i*)(smem + WA_OFF + i * 16) = *(const v4i*)(q.wa + ((size_t)(ct * KS + kk) * 64 + ln) * 16);
+    }
+    for (int i = tid; i < TB_INTS; i += 256)
+        ((int*)(smem + TAB_OFF))[i] = q.tab[i];
+    const int* tab = (const int*)(smem + TAB_OFF);
+    const int last_pos = q.total - 1;
+    const int hpwp = q.Hp * q.Wp;
+    // the output goes through a buffer descriptor: a lane with nothing to store gives an offset past the end, which the
+    // bounds check drops, so that every wave issues the same number of stores per tile
+    const __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(q.out, 0, q.out_bytes, 0x00020000);
+
+#ifdef N2D2HIP_PROFILE
+    long long pr[6] = {0, 0, 0, 0, 0, 0}, pr_t0 = clock64(), pr_w0 = wall_clock64();
+#define PROF_MARK(k) do { const long long now__ = clock64(); pr[k] += now__ - pr_last; pr_last = now__; } while (0)
+#else
+#define PROF_MARK(k) do { } while (0)
+#endif
+    const int lane_k = tid & 63;
+    // pixel fragments of the reduce convolution, requested one tile ahead: rows 64 * wave + 32 * j + l32 of t1, i.e.
+    // positions q0 - 64 + row
+    v4i xf[KS][2];
+    auto load_x = [&](int q0x) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int pc = min(max(q0x - 64 + 64 * wave + 32 * j + (lane_k & 31), 0), last_pos);
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk)
+                gload128(xf[kk][j], q.in + (size_t)pc * CIN + kk * 32 + (lane_k >> 5) * 16);
+        }
+    };
+    load_x(first * BM);
+    wait_vm<0>();
+    __syncthreads();
+
+    for (int t = 0; t < ntile; ++t) {
+        const int q0 = (first + t * q.nlanes) * BM;
+        // The lane's coordinates are made opaque once per tile: every LDS address below is then formed inside the tile
+        // (a few adds in front of immediate offsets) instead of being hoisted out of the loop by the hundred and spilled.
+        int lane = lane_k;
+        asm volatile("" : "+v"(lane));
+        const int l32 = lane & 31, lh = lane >> 5;
+        // position -> inside an image's interior?  (and where it goes in the output)
+        auto locate = [&](int pos, int& opix) -> bool {
+            const int pc = min(max(pos, 0), last_pos);
+            const int b = div_magic(pc, q.img_mul, q.img_sh);
+            const int rem = pc - b * hpwp;
+            const int yp = div_magic(rem, q.row_mul, q.row_sh);
+            const int xp = rem - yp * q.Wp;
+            opix = (b * q.OHp + yp - 1 + q.out_halo) * q.OWp + xp - 1 + q.out_halo;
+            return pos >= 0 && pos <= last_pos && yp >= 1 && yp <= q.Hp - 2 && xp >= 1 && xp <= q.Wp - 2;
+        };
+        // 16 accumulators of one 32 x 32 tile -> four dwords of bytes (channels 8g + 4 * lh .. + 3 in dword g), through a
+        // rescale whose result is the upper half of the multiply-add, saturated to [0, 255]
+        auto rescale_tile = [&](const v16i& acc, int tc_off, int td_off, int ch0, unsigned oxor, unsigned* pk) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const v4i tc = *(const v4i*)(tab + tc_off + ch0 + 8 * g + 4 * lh);
+                const v4i td = *(const v4i*)(tab + td_off + ch0 + 8 * g + 4 * lh);
+                v2s pq[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int t0 = __mul24(acc[4 * g + 2 * h], tc[2 * h]) + td[2 * h];
+                    const int t1 = __mul24(acc[4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
+                    pq[h] = as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u));
+                }
+                pk[g] = (sat_pk_u8(pq[0]) | (sat_pk_u8(pq[1]) << 16)) ^ oxor;
+            }
+        };
+        // two channel tiles of one pixel tile, packed -> this lane's 32 consecutive channels (32 * lh ..) of its pixel
+        auto gather32 = [&](const unsigned* pk0, const unsigned* pk1, v4i& lo16, v4i& hi16) {
+            unsigned qd[2][4];
+            const unsigned* pk[2] = {pk0, pk1};
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const auto s02 = __builtin_amdgcn_permlane32_swap(pk[i][0], pk[i][2], false, false);
+                const auto s13 = __builtin_amdgcn_permlane32_swap(pk[i][1], pk[i][3], false, false);
+                qd[i][0] = s02[0]; qd[i][1] = s02[1]; qd[i][2] = s13[0]; qd[i][3] = s13[1];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const auto x = __builtin_amdgcn_permlane32_swap(qd[0][e], qd[1][e], false, false);
+                lo16[e] = (int)x[0];
+                hi16[e] = (int)x[1];
+            }
+        };
+        // a row of 64 channel bytes in LDS: 16-byte slots XOR-swizzled by the row, so that fragment reads at any row shift
+        // touch every bank once
+        auto store_row = [&](int base, int row, const v4i& lo16, const v4i& hi16) {
+            unsigned char* r = smem + base + row * 64;
+            *(v4i*)(r + (((2 * lh) ^ sw64(row)) << 4)) = lo16;
+            *(v4i*)(r + (((2 * lh + 1) ^ sw64(row)) << 4)) = hi16;
+        };
+        auto frag = [&](int base, int row, int kk) -> v4i {
+            return *(const v4i*)(smem + base + row * 64 + ((((2 * kk + lh) ^ sw64(row)) & 3) << 4));
+        };
+        auto store_out = [&](bool ok, int opix, int ch, const v4i& lo16, const v4i& hi16) {
+            const unsigned off = ok ? (unsigned)(opix * q.out_cs + ch) : 0x80000000u;
+            __builtin_amdgcn_raw_buffer_store_b128(lo16, out_rsrc, off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(hi16, out_rsrc, off + 16u, 0, 0);
+        };
+#ifdef N2D2HIP_PROFILE
+        long long pr_last = clock64();
+#endif
+
+        v4i rfirst[PROJ ? 1 : 4], rsecond[PROJ ? 1 : 4], xpf[PROJ ? 4 : 1][PROJ ? KS : 1];
+        v4i wcf[2][2], wpf[PROJ ? 2 : 1][PROJ ? KS : 1];
+        // ================= phase 1: t1 rows 64 * wave .. + 63 (positions q0 - 64 + row), all 64 channels
+        {
+            int pos[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                pos[j] = q0 - 64 + 64 * wave + 32 * j + l32;
+            // this tile's pixels, requested a tile ago; only the previous tile's stores are younger
+            wait_vm<N_ST>();
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) { tie(xf[kk][0]); tie(xf[kk][1]); }
+            PROF_MARK(0);
+            v16i acc[2][2];
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                v4i wf[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    wf[i] = *(const v4i*)(smem + WA_OFF + ((kk * 2 + i) * 64 + lane) * 16);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i], xf[kk][j], kk == 0 ? v16i{} : acc[i][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // what phase 3 needs from memory, requested now so that it has two phases to arrive: the sum's other operand (x
+            // in the output's layout, or x as the projection's pixel operand) and this wave's expansion / projection weights
+            if (NPH == 3) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const signed char* xrow = q.in + (size_t)min(q0 + 32 * j + l32, last_pos) * CIN;
+                    if (PROJ) {
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk)
+                            gload128(xpf[PROJ ? j : 0][PROJ ? kk : 0], xrow + kk * 32 + lh * 16);
+                    } else {
+                        gload128(rfirst[PROJ ? 0 : j], xrow + 64 * wave + 32 * lh);
+                        gload128(rsecond[PROJ ? 0 : j], xrow + 64 * wave + 32 * lh + 16);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int kk = 0; kk < 2; ++kk)
+                        gload128(wcf[i][kk], q.wc + ((size_t)((2 * wave + i) * 2 + kk) * 64 + lane) * 16);
+                    if (PROJ) {
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk)
+                            gload128(wpf[PROJ ? i : 0][PROJ ? kk : 0], q.wp + ((size_t)((2 * wave + i) * KS + kk) * 64 + lane) * 16);
+                    }
+                }
+            }
+            // the next tile's pixels (any valid ones past this block's last tile)
+            load_x(q0 + q.nlanes * BM);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                unsigned pk[2][4];
+                rescale_tile(acc[0][j], TB_A_C, TB_A_D, 0, q.t1_xor, pk[0]);
+                rescale_tile(acc[1][j], TB_A_C, TB_A_D, 32, q.t1_xor, pk[1]);
+                v4i lo16, hi16;
+                gather32(pk[0], pk[1], lo16, hi16);
+                int opix;
+                if (!locate(pos[j], opix)) {
+                    const int z = (int)q.t1_zero;
+                    lo16 = v4i{z, z, z, z};
+                    hi16 = lo16;
+                }
+                store_row(T1_OFF, 64 * wave + 32 * j + l32, lo16, hi16);
+            }
+        }
+        PROF_MARK(1);
+        lds_barrier();
+        PROF_MARK(2);
+
+        // ================= phase 2: t2 rows 32 * wave .. + 31 (positions q0 + row), all 64 channels
+        {
+            v16i acc[2];
+            const int p = 32 * wave + l32;
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+                const int row = p + 64 + (tap / 3 - 1) * q.Wp + (tap % 3 - 1);
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+                    const v4i pf = frag(T1_OFF, row, kk);
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const v4i wf = *(const v4i*)(smem + WB_OFF + (((i * 9 + tap) * 2 + kk) * 64 + lane) * 16);
+                        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf, pf, (tap == 0 && kk == 0) ? v16i{} : acc[i], 0, 0, 0);
+                    }
+                }
+            }
+            unsigned pk[2][4];
+            rescale_tile(acc[0], TB_B_C, TB_B_D, 0, q.t2_xor, pk[0]);
+            rescale_tile(acc[1], TB_B_C, TB_B_D, 32, q.t2_xor, pk[1]);
+            v4i lo16, hi16;
+            gather32(pk[0], pk[1], lo16, hi16);
+            if (NPH == 2) {
+                int opix;
+                const bool ok = locate(q0 + p, opix);
+                store_out(ok, opix, 32 * lh, lo16, hi16);
+            } else {
+                lds_barrier();          // every wave has read t1: t2 may take its place
+                store_row(T2_OFF, p, lo16, hi16);
+            }
+        }
+        PROF_MARK(3);
+        lds_barrier();                  // NPH == 2: t1 is rewritten by the next tile
+        PROF_MARK(4);
+        if (NPH == 2)
+            continue;
+
+        // ================= phase 3: channels 64 * wave .. + 63 of all 128 positions, 64 positions at a time
+        // (its operands from memory: only the next tile's pixels are younger)
+        wait_vm<N_X>();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            tie(wcf[i][0]); tie(wcf[i][1]);
+            if (PROJ) {
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) tie(wpf[PROJ ? i : 0][PROJ ? kk : 0]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (PROJ) {
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) tie(xpf[PROJ ? j : 0][PROJ ? kk : 0]);
+            } else {
+                tie(rfirst[PROJ ? 0 : j]); tie(rsecond[PROJ ? 0 : j]);
+            }
+        }
+        // the expansion of both halves first (all that phase 3 reads of t2), so that the next tile may overwrite it
+        // behind one barrier in the middle of this phase
+        auto phase3 = [&](auto halfc) {
+            constexpr int half = decltype(halfc)::value;
+            int opix[2];
+            bool inside[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                inside[j] = locate(q0 + 64 * half + 32 * j + l32, opix[j]);
+            const v2s lo1 = splat_v2s(q.c_lo), hi1 = splat_v2s(q.c_hi), lo3 = splat_v2s(q.o_lo), hi3 = splat_v2s(q.o_hi);
+            const v2s off3 = splat_v2s(q.other_off);
+            // the expansion, rescaled and saturated, as pairs of 16-bit values: [i][j][g][pair]
+            v2s pq[2][2][4][2];
+            {
+                v16i acc[2][2];
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+                    v4i pf[2];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+                        pf[j] = frag(T2_OFF, 64 * half + 32 * j + l32, kk);
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wcf[i][kk], pf[j], kk == 0 ? v16i{} : acc[i][j], 0, 0, 0);
+                }
+                if (half == 1)
+                    lds_barrier();      // every wave has read all of t2: the next tile's phase 1 may write t1 over it
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const int ch = 64 * wave + 32 * i + 8 * g + 4 * lh;
+                        const v4i tc = *(const v4i*)(tab + TB_C_C + ch), td = *(const v4i*)(tab + TB_C_D + ch);
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                const int t0 = __mul24(acc[i][j][4 * g + 2 * h], tc[2 * h]) + td[2 * h];
+                                const int t1 = __mul24(acc[i][j][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
+                                pq[i][j][g][h] = clamp_v2s(as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u)), lo1, hi1);
+                            }
+                        __builtin_amdgcn_sched_barrier(0);      // one group's tables at a time
+                    }
+            }
+            // the other operand: the projection's accumulators, or the block input's bytes brought into the accumulators'
+            // layout by running the output's lane-half exchanges backwards
+            v16i accp[PROJ ? 2 : 1][PROJ ? 2 : 1];
+            unsigned resw[PROJ ? 1 : 8][PROJ ? 1 : 2];
+            if (PROJ) {
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int j = 0; j < 2; ++j)
+                            accp[PROJ ? i : 0][PROJ ? j : 0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(
+                                wpf[PROJ ? i : 0][PROJ ? kk : 0], xpf[PROJ ? 2 * half + j : 0][PROJ ? kk : 0],
+                                kk == 0 ? v16i{} : accp[PROJ ? i : 0][PROJ ? j : 0], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    unsigned qd[2][4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const auto y = __builtin_amdgcn_permlane32_swap((unsigned)rfirst[PROJ ? 0 : 2 * half + j][e],
+                                                                        (unsigned)rsecond[PROJ ? 0 : 2 * half + j][e], false, false);
+                        qd[0][e] = y[0]; qd[1][e] = y[1];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const auto s02 = __builtin_amdgcn_permlane32_swap(qd[i][0], qd[i][1], false, false);
+                        const auto s13 = __builtin_amdgcn_permlane32_swap(qd[i][2], qd[i][3], false, false);
+                        resw[PROJ ? 0 : i * 4 + 0][PROJ ? 0 : j] = s02[0];
+                        resw[PROJ ? 0 : i * 4 + 2][PROJ ? 0 : j] = s02[1];
+                        resw[PROJ ? 0 : i * 4 + 1][PROJ ? 0 : j] = s13[0];
+                        resw[PROJ ? 0 : i * 4 + 3][PROJ ? 0 : j] = s13[1];
+                    }
+                }
+            }
+            unsigned pk[2][2][4];       // [i][j][g]
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int ch = 64 * wave + 32 * i + 8 * g + 4 * lh;
+                    const v4i xc = *(const v4i*)(tab + TB_O_C + ch), xd = *(const v4i*)(tab + TB_O_D + ch);
+                    const v2i c16 = *(const v2i*)(tab + TB_S_C + ch / 2), d16 = *(const v2i*)(tab + TB_S_D + ch / 2);
+                    const v2i e16 = *(const v2i*)(tab + TB_S_E + ch / 2);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        v2s oq[2];
+                        if (PROJ) {
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                const int t0 = __mul24(accp[PROJ ? i : 0][PROJ ? j : 0][4 * g + 2 * h], xc[2 * h]) + xd[2 * h];
+                                const int t1 = __mul24(accp[PROJ ? i : 0][PROJ ? j : 0][4 * g + 2 * h + 1], xc[2 * h + 1]) + xd[2 * h + 1];
+                                oq[h] = clamp_v2s(as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u)), lo3, hi3) + off3;
+                            }
+                        } else {
+                            const unsigned w = resw[PROJ ? 0 : i * 4 + g][PROJ ? 0 : j] ^ q.res_flip;
+                            if (OTHER != OTHER_X) {
+                                unsigned u[4];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e)
+                                    u[e] = __umul24((w >> (8 * e)) & 0xffu, (unsigned)xc[e]) + (unsigned)xd[e];
+                                oq[0] = as_v2s((int)__builtin_amdgcn_perm(u[1], u[0], 0x07060302u));
+                                oq[1] = as_v2s((int)__builtin_amdgcn_perm(u[3], u[2], 0x07060302u));
+                                if (OTHER == OTHER_X_SCALED_SAT) {
+                                    oq[0] = clamp_v2s(oq[0], lo3, hi3);
+                                    oq[1] = clamp_v2s(oq[1], lo3, hi3);
+                                }
+                            } else {
+                                oq[0] = as_v2s((int)__builtin_amdgcn_perm(w, w, 0x0c010c00u));
+                                oq[1] = as_v2s((int)__builtin_amdgcn_perm(w, w, 0x0c030c02u));
+                            }
+                        }
+                        v2s r[2];
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            v2s v = pq[i][j][g][h] + oq[h];
+                            v = v * as_v2s(c16[h]) + as_v2s(d16[h]);
+                            r[h] = v >> as_v2s(e16[h]);
+                        }
+                        pk[i][j][g] = (sat_pk_u8(r[0]) | (sat_pk_u8(r[1]) << 16)) ^ q.out_xor;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                v4i lo16, hi16;
+                gather32(pk[0][j], pk[1][j], lo16, hi16);
+                store_out(inside[j], opix[j], 64 * wave + 32 * lh, lo16, hi16);
+            }
+        };
+        phase3(std::integral_constant<int, 0>());
+        __builtin_amdgcn_sched_barrier(0);
+        phase3(std::integral_constant<int, 1>());
+        PROF_MARK(5);
+    }
+#ifdef N2D2HIP_PROFILE
+    if (tid == 0) {
+        long long* o = q.prof + (long long)blockIdx.x * 10;
+        for (int k = 0; k < 6; ++k) o[k] = pr[k];
+        o[6] = clock64() - pr_t0; o[7] = wall_clock64() - pr_w0; o[8] = ntile; o[9] = 1;
+    }
+#endif
+    // the pixels requested past the last tile are still on their way
+    wait_vm<0>();
+}
+
+} // namespace n2d2hip
+
+using namespace n2d2hip;
+
+struct n2d2hip_bottleneck_s {
+    n2d2hip_conv_t reduce, conv3x3, expand, projection;
+    int cin;
+    signed char* d_w;       // the four weight sets in fragment order
+    size_t wa_off, wb_off, wc_off, wp_off;
+    int* d_tab;
+};
+
+namespace {
+
+// [O][K] rows (row stride `stride` bytes, K order = tap-major then channel) -> [O / 32][K / 32][64 lanes][16 bytes]
+void to_fragments(const signed char* w, int O, int K, size_t stride, signed char* frag)
+{
+    for (int ct = 0; ct < O / 32; ++ct)
+        for (int ks = 0; ks < K / 32; ++ks)
+            for (int lane = 0; lane < 64; ++lane)
+                memcpy(frag + (((size_t)ct * (K / 32) + ks) * 64 + lane) * 16,
+                       w + (size_t)(ct * 32 + (lane & 31)) * stride + ks * 32 + (lane >> 5) * 16, 16);
+}
+
+bool one_by_one(const n2d2hip_conv_desc& d)
+{
+    return d.kW == 1 && d.kH == 1 && d.strideX == 1 && d.strideY == 1 && d.padL == 0 && d.padT == 0 && d.padR == 0 && d.padB == 0
+        && d.groups == 1 && d.weight_bits == 8;
+}
+
+bool saturates_to_byte(const n2d2hip_act_s* a) { return a->args.lo == 0 && a->args.hi == 255; }
+
+bool hi16_cell(const n2d2hip_conv_s* c)
+{
+    return c->act->args.kind == EPI_I24 && c->bias_folded && c->hi16 && c->d_epi_tab && c->act->min_out >= -128 && c->act->max_out <= 255;
+}
+
+void magic(unsigned d, unsigned* mul, unsigned* sh)
+{
+    if (d <= 1) { *mul = 0; *sh = 0; return; }
+    unsigned s = 0;
+    while ((1ull << s) < d) ++s;
+    *mul = (unsigned)((1ull << (31 + s)) / d + 1);
+    *sh = s - 1;
+}
+
+int device_cus()
+{
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+        return prop.multiProcessorCount;
+    return 256;
+}
+
+unsigned xor_of(int dtype) { return dtype == N2D2HIP_U8B ? 0x80808080u : 0u; }
+int byte_dtype_of(const n2d2hip_act_s* a) { return a->min_out >= 0 ? N2D2HIP_U8B : N2D2HIP_I8; }
+
+} // namespace
+
+extern "C" {
+
+int n2d2hip_bottleneck_create(n2d2hip_conv_t reduce, n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand, n2d2hip_conv_t projection,
+                              n2d2hip_bottleneck_t* out)
+{
+    N2D2HIP_REQUIRE(reduce && conv3x3 && out, N2D2HIP_ERR_INVALID, "bottleneck_create: null argument");
+    N2D2HIP_REQUIRE(expand || !projection, N2D2HIP_ERR_INVALID, "bottleneck_create: a projection without the expansion it is added to");
+    const n2d2hip_conv_desc& da = reduce->desc;
+    const n2d2hip_conv_desc& db = conv3x3->desc;
+    const int cin = da.C;
+    bool ok = one_by_one(da) && (cin == 64 || cin == 256) && da.O == 64 && hi16_cell(reduce) && reduce->in_cs == cin
+        && db.kW == 3 && db.kH == 3 && db.strideX == 1 && db.strideY == 1 && db.dilX == 1 && db.dilY == 1 && db.padL == 1 && db.padT == 1
+        && db.padR == 1 && db.padB == 1 && db.groups == 1 && db.weight_bits == 8 && db.C == 64 && db.O == 64 && hi16_cell(conv3x3)
+        && conv3x3->in_dtype == byte_dtype_of(reduce->act) && conv3x3->ktot == 9 * 64
+        && saturates_to_byte(reduce->act) && saturates_to_byte(conv3x3->act);
+    if (ok && expand) {
+        const n2d2hip_conv_desc& dc = expand->desc;
+        ok = one_by_one(dc) && dc.C == 64 && dc.O == 256 && hi16_cell(expand) && expand->in_dtype == byte_dtype_of(conv3x3->act)
+            && expand->sum && expand->d_res_tab && expand->sum16 && expand->sum->act->cpad == 256 && saturates_to_byte(expand->sum->act);
+        if (ok && projection) {
+            const n2d2hip_conv_desc& dp = projection->desc;
+            ok = one_by_one(dp) && dp.C == cin && cin == 64 && dp.O == 256 && hi16_cell(projection) && projection->in_dtype == reduce->in_dtype
+                && !expand->has_pre && expand->sum_other_dtype == byte_dtype_of(projection->act);
+        } else if (ok) {
+            ok = cin == 256 && expand->sum_other_dtype == reduce->in_dtype;
+        }
+    }
+    N2D2HIP_REQUIRE(ok, N2D2HIP_ERR_UNSUPPORTED,
+                    "bottleneck_create: needs a 1x1 (64 or 256 -> 64), a 3x3 stride 1 padding 1 (64 -> 64) and, for the whole block, a "
+                    "1x1 (64 -> 256) with its sum folded in on 16-bit pairs plus the block's input or a 1x1 projection of it, all 8-bit "
+                    "with integer rescales that fit the scaled-up tables");
+
+    // weights: back from the handles' device copies ([rows][ktot], K = tap-major then channel), into fragment order
+    auto fetch = [](const n2d2hip_conv_s* c, std::vector<signed char>& rows) -> hipError_t {
+        rows.resize((size_t)c->opad * c->ktot);
+        return hipMemcpy(rows.data(), c->d_w, rows.size(), hipMemcpyDeviceToHost);
+    };
+    std::vector<signed char> ra, rb, rc, rp;
+    hipError_t e = fetch(reduce, ra);
+    if (e == hipSuccess) e = fetch(conv3x3, rb);
+    if (e == hipSuccess && expand) e = fetch(expand, rc);
+    if (e == hipSuccess && projection) e = fetch(projection, rp);
+    if (e != hipSuccess)
+        return fail(N2D2HIP_ERR_HIP, "bottleneck_create: reading the weights back failed: %s", hipGetErrorString(e));
+    n2d2hip_bottleneck_s* b = new n2d2hip_bottleneck_s();
+    b->reduce = reduce; b->conv3x3 = conv3x3; b->expand = expand; b->projection = projection; b->cin = cin;
+    b->d_w = nullptr; b->d_tab = nullptr;
+    b->wa_off = 0;
+    b->wb_off = b->wa_off + (size_t)64 * cin;
+    b->wc_off = b->wb_off + (size_t)64 * 576;
+    b->wp_off = b->wc_off + (size_t)256 * 64;
+    std::vector<signed char> frag(b->wp_off + (size_t)256 * cin, 0);
+    to_fragments(ra.data(), 64, cin, reduce->ktot, frag.data() + b->wa_off);
+    // the 3x3 kernel's own order: [channel tile][tap][K step]: its rows are already tap-major
+    to_fragments(rb.data(), 64, 576, conv3x3->ktot, frag.data() + b->wb_off);
+    if (expand) to_fragments(rc.data(), 256, 64, expand->ktot, frag.data() + b->wc_off);
+    if (projection) to_fragments(rp.data(), 256, cin, projection->ktot, frag.data() + b->wp_off);
+
+    // tables: device -> host copies of what the cells prepared, laid out for the kernel
+    std::vector<int> tab(TB_INTS, 0);
+    auto hi16_tables = [&](const n2d2hip_conv_s* c, int n, int c_off, int d_off) -> hipError_t {
+        const int cp = c->act->cpad;
+        hipError_t r = hipMemcpy(tab.data() + c_off, c->d_epi_tab + 5 * cp, n * sizeof(int), hipMemcpyDeviceToHost);
+        if (r == hipSuccess) r = hipMemcpy(tab.data() + d_off, c->d_epi_tab + 6 * cp, n * sizeof(int), hipMemcpyDeviceToHost);
+        return r;
+    };
+    e = hi16_tables(reduce, 64, TB_A_C, TB_A_D);
+    if (e == hipSuccess) e = hi16_tables(conv3x3, 64, TB_B_C, TB_B_D);
+    if (e == hipSuccess && expand) {
+        e = hi16_tables(expand, 256, TB_C_C, TB_C_D);
+        const int cp = 256;
+        if (e == hipSuccess) e = hipMemcpy(tab.data() + TB_S_C, expand->d_res_tab + 10 * cp, 3 * (cp / 2) * sizeof(int), hipMemcpyDeviceToHost);
+        if (e == hipSuccess && projection) e = hi16_tables(projection, 256, TB_O_C, TB_O_D);
+        if (e == hipSuccess && !projection && expand->has_pre) {
+            e = hipMemcpy(tab.data() + TB_O_C, expand->d_res_tab + 12 * cp, cp * sizeof(int), hipMemcpyDeviceToHost);
+            if (e == hipSuccess) e = hipMemcpy(tab.data() + TB_O_D, expand->d_res_tab + 13 * cp, cp * sizeof(int), hipMemcpyDeviceToHost);
+        }
+    }
+    if (e == hipSuccess) e = hipMalloc((void**)&b->d_w, frag.size());
+    if (e == hipSuccess) e = hipMemcpy(b->d_w, frag.data(), frag.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMalloc((void**)&b->d_tab, tab.size() * sizeof(int));
+    if (e == hipSuccess) e = hipMemcpy(b->d_tab, tab.data(), tab.size() * sizeof(int), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        n2d2hip_bottleneck_destroy(b);
+        return fail(N2D2HIP_ERR_HIP, "bottleneck_create: device upload failed: %s", hipGetErrorString(e));
+    }
+    *out = b;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_bottleneck_destroy(n2d2hip_bottleneck_t b)
+{
+    if (!b) return N2D2HIP_OK;
+    if (b->d_w) (void)hipFree(b->d_w);
+    if (b->d_tab) (void)hipFree(b->d_tab);
+    delete b;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_bottleneck_forward(n2d2hip_bottleneck_t b, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream_)
+{
+    int rc;
+    N2D2HIP_REQUIRE(b != nullptr, N2D2HIP_ERR_INVALID, "bottleneck_forward: null handle");
+    if ((rc = check_tensor(in, "bottleneck input", true)) || (rc = check_tensor(out, "bottleneck output", true)))
+        return rc;
+    const int oc = b->expand ? 256 : 64;
+    const n2d2hip_act_s* last = b->expand ? b->expand->sum->act : b->conv3x3->act;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC && in->halo == 1, N2D2HIP_ERR_UNSUPPORTED,
+                    "bottleneck_forward: NHWC tensors, the input with a border of one pixel");
+    N2D2HIP_REQUIRE(in->dtype == b->reduce->in_dtype && in->C == b->cin && in->cs == b->cin, N2D2HIP_ERR_INVALID,
+                    "bottleneck_forward: input must have %d channels of the type the first cell was created for", b->cin);
+    N2D2HIP_REQUIRE(out->B == in->B && out->H == in->H && out->W == in->W && out->C == oc && out->cs >= oc && out->cs % 16 == 0
+                        && is_byte_type(out->dtype),
+                    N2D2HIP_ERR_INVALID, "bottleneck_forward: output must be %dx%dx%dx%d bytes", in->B, oc, in->H, in->W);
+    {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(last->min_out >= lo && last->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "bottleneck_forward: activation range [%d,%d] does not fit output dtype %d", last->min_out, last->max_out, out->dtype);
+    }
+    const int Hp = in->H + 2, Wp = in->W + 2;
+    const long long total = (long long)in->B * Hp * Wp;
+    const long long opix = (long long)in->B * (in->H + 2 * out->halo) * (in->W + 2 * out->halo);
+    N2D2HIP_REQUIRE(Wp + 1 <= 64, N2D2HIP_ERR_UNSUPPORTED, "bottleneck_forward: rows of more than 61 pixels");
+    N2D2HIP_REQUIRE(total * std::max(b->cin, 64) < (1ll << 31) && opix * out->cs < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED,
+                    "bottleneck_forward: tensor too large");
+    BottleneckArgs q = {};
+    q.in = (const signed char*)in->data; q.out = (signed char*)out->data;
+    q.Hp = Hp; q.Wp = Wp; q.total = (int)total;
+    q.out_bytes = (int)(opix * out->cs);
+    q.out_cs = out->cs; q.out_halo = out->halo; q.OHp = in->H + 2 * out->halo; q.OWp = in->W + 2 * out->halo;
+    magic((unsigned)(Hp * Wp), &q.img_mul, &q.img_sh);
+    magic((unsigned)Wp, &q.row_mul, &q.row_sh);
+    q.ntiles = (int)((total + 127) / 128);
+    q.xcd_tiles = (q.ntiles + 7) / 8;
+    const int cus = device_cus();
+    q.nlanes = std::max(1, std::min(q.xcd_tiles, 2 * cus / 8));
+    q.wa = b->d_w + b->wa_off; q.wb = b->d_w + b->wb_off; q.wc = b->d_w + b->wc_off; q.wp = b->d_w + b->wp_off;
+    q.tab = b->d_tab;
+    const n2d2hip_act_s* aa = b->reduce->act;
+    const n2d2hip_act_s* ab = b->conv3x3->act;
+    const int t1_dtype = byte_dtype_of(aa), t2_dtype = byte_dtype_of(ab);
+    q.t1_xor = xor_of(t1_dtype); q.t1_zero = q.t1_xor; q.t2_xor = xor_of(t2_dtype);
+    q.out_xor = xor_of(out->dtype);
+    if (b->expand) {
+        const n2d2hip_conv_s* c = b->expand;
+        N2D2HIP_REQUIRE(b->expand->sum && b->expand->sum16 && b->expand->d_res_tab, N2D2HIP_ERR_INVALID,
+                        "bottleneck_forward: the expansion's folded sum was undone after the bottleneck was created");
+        q.c_lo = c->act->args.lo; q.c_hi = c->act->args.hi;
+        q.res_flip = c->sum_other_dtype == N2D2HIP_U8 ? 0u : 0x80808080u;
+        if (b->projection) {
+            q.o_lo = b->projection->act->args.lo; q.o_hi = b->projection->act->args.hi;
+            q.other_off = c->sum_other_dtype == N2D2HIP_I8 ? 128 : 0;
+        } else {
+            if (c->has_pre) { q.o_lo = c->sum->pre_act->args.lo; q.o_hi = c->sum->pre_act->args.hi; }
+        }
+    }
+    const int grid = 8 * q.nlanes;
+    hipStream_t st = (hipStream_t)stream_;
+#ifdef N2D2HIP_PROFILE
+    {
+        const char* pp = getenv("N2D2HIP_PROF_PTR");      // profiling builds only: where the blocks' counters go
+        N2D2HIP_REQUIRE(pp != nullptr, N2D2HIP_ERR_INVALID, "bottleneck_forward: profiling build without N2D2HIP_PROF_PTR");
+        q.prof = (long long*)strtoull(pp, nullptr, 16);
+    }
+#endif
+    if (!b->expand) {
+        if (b->cin == 64) hipLaunchKernelGGL((bottleneck_kernel<64, OTHER_PROJECTION, 2>), dim3(grid), dim3(256), 0, st, q);
+        else hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X, 2>), dim3(grid), dim3(256), 0, st, q);
+    } else if (b->projection) {
+        hipLaunchKernelGGL((bottleneck_kernel<64, OTHER_PROJECTION, 3>), dim3(grid), dim3(256), 0, st, q);
+    } else if (!b->expand->has_pre) {
+        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X, 3>), dim3(grid), dim3(256), 0, st, q);
+    } else if (b->expand->pre_in_range) {
+        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X_SCALED, 3>), dim3(grid), dim3(256), 0, st, q);
+    } else {
+        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X_SCALED_SAT, 3>), dim3(grid), dim3(256), 0, st, q);
+    }
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+} // extern "C"

@@ -356,42 +356,7 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const signed char* __res
 
 using namespace n2d2hip;
 
-struct n2d2hip_conv_s {
-    n2d2hip_conv_desc desc;
-    n2d2hip_act_t act;
-    int in_dtype;
-    int in_cs;            // channel stride the weights were prepared for
-    bool depthwise;
-    bool pix4;
-    int opad;             // weight rows (multiple of 128)
-    int ktot;
-    signed char* d_w;
-    int4* d_sub;
-    int* d_bias;
-    signed char* d_fill;  // 16 bytes of the input's logical zero, source of padded taps in the direct-to-LDS kernel
-    bool preclamp;        // some accumulator could overflow the rescale's 24x24 -> 32 bit product, or the cell has a Clip
-    // residual sum folded into the epilogue (n2d2hip_conv_fuse_sum)
-    n2d2hip_elemwise_t sum;
-    int sum_other_dtype;  // storage type the tables below were made for
-    // sum a,b,c,d,e then pre a,b,c,d,e, each [cpad], zero point of the other input folded in; then the sum's c, d, e as
-    // 16-bit pairs, each [cpad / 2]
-    int* d_res_tab;
-    bool has_pre, pre_clamp, sum_clamp;
-    bool sum16;           // the 16-bit pairs may be used: every intermediate behind the convolution's shift fits 16 bits
-    bool pre_in_range;    // the folded ScalingCell maps every byte into its output range
-    // integer rescale with the bias folded in, for the pipelined kernel: a - bias, b - bias, c, d + bias * c, e, each [cpad]
-    // ... then, when hi16: c << (16 - e) and (d + bias * c) << (16 - e), which leave the rescaled value in the upper half
-    // of the 32-bit result
-    int* d_epi_tab;
-    bool bias_folded;
-    bool hi16;
-    // first-layer kernel (<= 4 input channels, horizontal stride 2): weights as [channel][kH * 32]
-    signed char* d_wstem;
-    // 3x3 stride-1 kernel over inputs that carry their padding: weights in matrix-core fragment order
-    signed char* d_wfrag;
-    bool is_fc;
-    int fcH, fcW;
-};
+#include "conv_handle.hpp"
 
 namespace {
 

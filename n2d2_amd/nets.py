@@ -356,12 +356,15 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0):
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection"):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
         a border of zeros around every image, which lets a padded KxK reader fetch every tap without a validity test.
-        kernel_choice: capi.KERNEL_* bits handed to every convolution (which kernel runs, never what it computes)."""
+        kernel_choice: capi.KERNEL_* bits handed to every convolution (which kernel runs, never what it computes).
+        bottlenecks: run a residual block 1x1 -> 3x3 -> 1x1 + sum (+ projection) whose cells qualify as one launch
+        (n2d2hip_bottleneck_*); its input tensor then carries a border of one pixel.  True / "all", "projection" (only the
+        blocks with a projection shortcut, where one launch replaces four), or False."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
         consumers = {}
@@ -446,6 +449,10 @@ class GpuNet:
                 raise ValueError(l.type)
             self.tensors[l.name] = out
             ins_of[l.name] = ins
+        self.bottlenecks, self.bottleneck_layers = {}, {}
+        self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
+        if fuse and halo and bottlenecks:
+            self._plan_bottlenecks(consumers, by_name, ins_of)
         self._io = [(ins_of[l.name], self.tensors[l.name]) for l in spec.layers]
         # folded ScalingCells are not launched and their output is never materialised
         for name in self.folded:
@@ -454,6 +461,91 @@ class GpuNet:
         self.steps = [self.steps[k] for k in keep]
         self._io = [self._io[k] for k in keep]
         self.launched = [spec.layers[k] for k in keep]
+
+    def _plan_bottlenecks(self, consumers, by_name, ins_of):
+        """For every sum folded into a 1x1 convolution: reduce -> 3x3 -> expand (+ projection) as one launch, if the
+        library takes them (n2d2hip_bottleneck_create).  The sum may sit in the expansion (the other input is the block's
+        input, plain or through a folded ScalingCell) or in the projection, which runs last (the sum is then moved into the
+        expansion).  The block's input gets a border of one pixel, which its producer must be able to write (a max
+        pooling, a folded sum, another bottleneck).  self.bottlenecks: "all", "projection" (only blocks with a projection:
+        the others are as fast cell by cell) or False."""
+        rt = self.rt
+        cell_of = {m.name: c for (m, c, f) in self.steps}
+        step_index = {m.name: k for k, (m, c, f) in enumerate(self.steps)}
+        for sum_name, (sum_cell, holder) in list(self.fused_sums.items()):
+            sum_layer = by_name[sum_name]
+            other_name = [i for i in sum_layer.inputs if i != holder.name][0]
+            other_layer = by_name.get(other_name)
+            expand, proj = holder, None
+            if by_name.get(holder.inputs[0]) is None or by_name[holder.inputs[0]].type != "conv":
+                # the sum sits in the projection: the expansion is the sum's other input
+                if other_layer is None or other_layer.type != "conv" or other_name in self.folded or len(consumers[other_name]) != 1:
+                    continue
+                expand, proj = other_layer, holder
+            conv_b = by_name.get(expand.inputs[0])
+            conv_a = by_name.get(conv_b.inputs[0]) if conv_b is not None and conv_b.type == "conv" else None
+            if conv_a is None or conv_a.type != "conv" or len(consumers[conv_a.name]) != 1 or len(consumers[conv_b.name]) != 1:
+                continue
+            xname = conv_a.inputs[0]
+            x = self.tensors.get(xname)
+            scaled = proj is None and other_name in self.folded and other_layer is not None and other_layer.type == "scaling"
+            if proj is None:
+                other_src = other_layer.inputs[0] if scaled else other_name
+                if other_src != xname:
+                    cand = by_name.get(other_src)
+                    if cand is None or cand.type != "conv" or cand.inputs[0] != xname or len(consumers[cand.name]) != 1 or scaled:
+                        continue
+                    proj = cand
+            elif proj.inputs[0] != xname:
+                continue
+            if self._bottleneck_mode == "projection" and proj is None:
+                continue
+            readers = {conv_a.name, proj.name if proj is not None else sum_name} | ({other_name} if scaled else set())
+            if x is None or xname == "input" or not {m.name for m in consumers[xname]} <= readers | {sum_name}:
+                continue
+            producer = by_name[xname]
+            can_write_halo = (producer.type == "pool" and producer.kind == "max" and tuple(producer.pool) in ((2, 2), (3, 3))) \
+                or xname in self.fused_sums or xname in self.bottlenecks
+            if x.halo not in (0, 1) or (x.halo == 0 and not can_write_halo):
+                continue
+            moved = False
+            if holder is not expand:
+                # move the sum from the projection into the expansion (undone below if the library declines)
+                k_exp = sum_layer.inputs.index(expand.name)
+                if not cell_of[expand.name].fuse_sum(sum_cell, k_exp, self.tensors[proj.name].dtype):
+                    continue
+                moved = True
+            bn = rt.Bottleneck.create(cell_of[conv_a.name], cell_of[conv_b.name], cell_of[expand.name],
+                                      cell_of[proj.name] if proj is not None else None)
+            if bn is None:
+                if moved:
+                    cell_of[expand.name].fuse_sum(None, 0, 0)
+                continue
+            if moved:
+                cell_of[proj.name].fuse_sum(None, 0, 0)
+            if x.halo == 0:
+                try:
+                    nx = rt.DTensor(x.B, x.C, x.H, x.W, x.dtype, halo=1)
+                    if producer.type == "pool":       # does this pooling write a border?  (probed once, on the real tensors)
+                        cell_of[xname].forward(ins_of[xname][0], nx)
+                except self.capi.N2D2HipError:
+                    if moved:
+                        cell_of[expand.name].fuse_sum(None, 0, 0)
+                        cell_of[proj.name].fuse_sum(sum_cell, sum_layer.inputs.index(proj.name), self.tensors[expand.name].dtype)
+                    continue
+                for lst in ins_of.values():
+                    for k, t in enumerate(lst):
+                        if t is x:
+                            lst[k] = nx
+                self.tensors[xname] = nx
+                x = nx
+            self.bottlenecks[sum_name] = bn
+            self.bottleneck_layers[sum_name] = [conv_a, conv_b, expand] + ([proj] if proj is not None else [])
+            k = step_index[sum_name]
+            ins_of[sum_name] = [x]
+            self.steps[k] = (sum_layer, bn, (lambda c, i, o: c.forward(i[0], o)))
+            for gone in [conv_a.name, conv_b.name, expand.name] + ([proj.name] if proj is not None else []):
+                self.folded.add(gone)
 
     def set_input(self, x):
         """x: integer NCHW numpy array [B,C,H,W]."""
@@ -513,11 +605,15 @@ class GpuNet:
         total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
         if l.type in ("conv", "fc"):
             total += l.w.size // (2 if l.weight_bits == 4 else 1)
-        if l.name in self.fused_sums:
+        if l.name in self.bottleneck_layers:
+            total += sum(m.w.size for m in self.bottleneck_layers[l.name])
+        elif l.name in self.fused_sums:
             total += self.fused_sums[l.name][1].w.size
         return total
 
     def layer_macs(self, l):
+        if l.name in self.bottleneck_layers:
+            return sum(self.B * m.out_shape[1] * m.out_shape[2] * m.w.size for m in self.bottleneck_layers[l.name])
         if l.name in self.fused_sums:
             return self.layer_macs(self.fused_sums[l.name][1])
         if l.type == "conv":
@@ -534,6 +630,8 @@ class GpuNet:
             total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
             if l.type in ("conv", "fc"):
                 total += l.w.size // (2 if l.weight_bits == 4 else 1)
-            if l.name in self.fused_sums:
+            if l.name in self.bottleneck_layers:
+                total += sum(m.w.size for m in self.bottleneck_layers[l.name])
+            elif l.name in self.fused_sums:
                 total += self.fused_sums[l.name][1].w.size
         return total

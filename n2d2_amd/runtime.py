@@ -119,6 +119,33 @@ class Act:
             self.handle = None
 
 
+class Bottleneck:
+    """n2d2hip_bottleneck_t: reduce -> 3x3 [-> expand + sum (+ projection)] in one launch; None when the library keeps
+    the cells apart."""
+
+    def __init__(self, handle, cells):
+        self.handle, self._cells = handle, cells
+
+    @staticmethod
+    def create(reduce, conv3x3, expand=None, projection=None):
+        h = C.c_void_p()
+        rc = lib.n2d2hip_bottleneck_create(reduce.handle, conv3x3.handle, expand.handle if expand is not None else None,
+                                           projection.handle if projection is not None else None, C.byref(h))
+        if rc == capi.ERR_UNSUPPORTED:
+            return None
+        check(rc)
+        return Bottleneck(h, (reduce, conv3x3, expand, projection))
+
+    def forward(self, x, out):
+        check(lib.n2d2hip_bottleneck_forward(self.handle, x.ref, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None) and lib is not None:
+            lib.n2d2hip_bottleneck_destroy(self.handle)
+            self.handle = None
+
+
 def scaling_forward(act, x, out_dtype=None):
     out = DTensor(x.B, x.C, x.H, x.W, out_dtype if out_dtype is not None else act.out_dtype(), x.layout)
     check(lib.n2d2hip_scaling_forward(act.handle, x.ref, out.ref, stream_ptr()))

@@ -568,6 +568,76 @@ def test_conv3x3_patch_kernel_bit_exact(rt):
                         assert bool((border == out.buf.view(-1)[0]).all()), "the output's border is left alone"
 
 
+def test_bottleneck_in_one_launch_bit_exact(rt):
+    """n2d2hip_bottleneck_*: 1x1 -> 3x3 (-> 1x1 + sum with the block's input, plain or through a folded ScalingCell, or with
+    a projection of it) in one launch equals the reference cells run in turn; the cells stay usable on their own.  Images
+    narrower and wider than a tile's reach, tiles that straddle images, outputs with and without a border."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(4242)
+
+    def relu_spec(O):
+        return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=True)
+
+    def lin_spec(O):
+        return ActSpec("Linear", "SingleShift", rng.integers(8, 12, size=O), nb_bits=8, unsigned_out=False)
+
+    def weights(O, Cc, k, std):
+        return np.clip(np.rint(rng.normal(0, std, size=(O, Cc, k, k))), -127, 127).astype(np.int64)
+    for cin, H, W, B, variant in ((256, 9, 7, 3, "identity"), (64, 9, 7, 3, "projection"), (256, 12, 20, 2, "scaled identity"),
+                                  (256, 56, 56, 1, "identity"), (64, 30, 58, 2, "projection"), (64, 5, 61, 2, "two cells"),
+                                  (256, 3, 1, 40, "two cells"), (256, 1, 1, 150, "scaled identity")):
+        print("bottleneck", cin, H, W, B, variant, flush=True)
+        x = rng.integers(0, 256, size=(B, cin, H, W))
+        wa, wb, wc, wp = weights(64, cin, 1, 12), weights(64, 64, 3, 10), weights(256, 64, 1, 25), weights(256, cin, 1, 25)
+        ba, bb, bc, bp = (rng.integers(-2000, 2000, size=n) for n in (64, 64, 256, 256))
+        sa, sb, sc, sp = relu_spec(64), relu_spec(64), lin_spec(256), lin_spec(256)
+        ssum = sum_spec_for(256, rng)
+        t1 = cells_ref.conv_cell(x, wa, ba, sa)
+        t2 = cells_ref.conv_cell(t1, wb, bb, sb, pad=(1, 1, 1, 1))
+        ca = rt.Conv(wa, ba, rt.Act(64, **sa.kwargs()), capi.U8B)
+        cb = rt.Conv(wb, bb, rt.Act(64, **sb.kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+        dx = rt.DTensor.from_numpy(x, capi.U8B).with_halo(1)
+        if variant == "two cells":
+            bn = rt.Bottleneck.create(ca, cb)
+            assert bn is not None
+            for out_halo in (0, 1):
+                out = rt.DTensor(B, 64, H, W, capi.U8B, halo=out_halo)
+                got = bn.forward(dx, out).to_numpy()
+                assert np.array_equal(got, t2.astype(np.int64)), (cin, H, W, B, variant, out_halo, np.count_nonzero(got != t2))
+            continue
+        t3 = cells_ref.conv_cell(t2, wc, bc, sc)
+        cc = rt.Conv(wc, bc, rt.Act(256, **sc.kwargs()), capi.U8B)
+        ew = rt.ElemWiseSum(2, 256, rt.Act(256, **ssum.kwargs()))
+        cp_, pre = None, None
+        if variant == "projection":
+            other = cells_ref.conv_cell(x, wp, bp, sp)
+            cp_ = rt.Conv(wp, bp, rt.Act(256, **sp.kwargs()), capi.U8B)
+            assert cc.fuse_sum(ew, 0, capi.I8)
+        else:
+            other = x.astype(np.float32)
+            if variant == "scaled identity":
+                pre_spec = ActSpec("Linear", "FixedMult16", rng.integers(2 ** 12, 2 ** 15, size=256), frac_bits=14, nb_bits=8, unsigned_out=True)
+                other = pre_spec.apply(other)
+                pre = rt.Act(256, **pre_spec.kwargs())
+                assert ew.fold_input_scaling(1, pre)
+            assert cc.fuse_sum(ew, 0, capi.U8B)
+        want = cells_ref.elemwise_cell([t3, other], ssum).astype(np.int64)
+        bn = rt.Bottleneck.create(ca, cb, cc, cp_)
+        assert bn is not None, variant
+        for out_halo in (1, 0):
+            out = rt.DTensor(B, 256, H, W, capi.U8B, halo=out_halo)
+            got = bn.forward(dx, out).to_numpy()
+            assert np.array_equal(got, want), (cin, H, W, B, variant, out_halo, np.count_nonzero(got != want))
+        # the cells still run on their own
+        assert np.array_equal(cb.forward(ca.forward(dx, ca.make_output(dx, halo=1))).to_numpy(), t2.astype(np.int64))
+    # what does not qualify is reported
+    w128 = weights(128, 256, 1, 12)
+    c128 = rt.Conv(w128, None, rt.Act(128, **relu_spec(128).kwargs()), capi.U8B)
+    assert rt.Bottleneck.create(c128, cb) is None
+
+
 def conv_spec_for(O, rng):
     from oracle.cells import ActSpec
     return ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=False)
