@@ -17,9 +17,11 @@ if ROOT not in sys.path:
 
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
-# HBM bytes one conv_pipe_kernel launch of this workload moves on average: rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy), summary under profiles/
-PIPE_TRAFFIC_BYTES_PER_LAUNCH = (41.15 + 23.76) * 1048576
+# HBM bytes one conv_pipe_kernel launch of this workload moves on average, as counted by rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
+# inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
+TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
+                        "bytes_per_launch": None}
 
 
 def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
@@ -41,24 +43,90 @@ def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
             "sample": "%d images of the same ResNet-50 forward (batch %d, 224x224), oracle/frame_oracle.c with OpenMP" % (n, n)}, exact
 
 
-def other_configs_bit_exact():
-    """Part of the CPU-baseline leg: the other four configurations at sizes the oracle finishes in seconds (the first
-    two at their full size), GPU logits against the CPU oracle, one flag per configuration."""
+def class_rooflines(net, per_launch_ms, step_ms):
+    """Every launch of a forward against the larger of its two bounds (2 * MAC at the int8 matrix peak, algorithmic bytes
+    at the HBM peak), summed per class: convolutions / fully-connected cells whose larger bound is the matrix cores,
+    those whose larger bound is memory, depthwise convolutions and the other bandwidth cells (pooling, sums, scalings)."""
+    classes, floor_ms = {}, 0.0
+    for l, t in zip(net.launched, per_launch_ms):
+        ops, nbytes = 2.0 * net.layer_macs(l), float(net.layer_bytes(l))
+        t_mfma, t_hbm = ops / (PEAK_INT8_TOPS * 1e12) * 1e3, nbytes / (PEAK_HBM_GBS * 1e9) * 1e3
+        floor_ms += max(t_mfma, t_hbm)
+        if l.type == "conv" and getattr(l, "groups", 1) > 1:
+            name = "depthwise_hbm_bound"
+        elif l.type in ("conv", "fc") or l.name in net.fused_sums:
+            name = "mfma_bound" if t_mfma > t_hbm else "hbm_bound"
+        else:
+            name = "bandwidth_cells_hbm_bound"
+        c = classes.setdefault(name, {"launches": 0, "ms": 0.0, "ops": 0.0, "bytes": 0.0})
+        c["launches"] += 1; c["ms"] += t; c["ops"] += ops; c["bytes"] += nbytes
+    out = {}
+    for name, c in classes.items():
+        if name == "mfma_bound":
+            ach, peak, unit = c["ops"] / (c["ms"] * 1e-3) / 1e12, PEAK_INT8_TOPS, "TOP/s"
+        else:
+            ach, peak, unit = c["bytes"] / (c["ms"] * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        out[name] = {"launches": c["launches"], "ms": round(c["ms"], 4), "achieved": round(ach, 1), "peak": peak, "unit": unit,
+                     "frac": round(ach / peak, 4)}
+    out["floor_ms"] = round(floor_ms, 4)               # sum over launches of the larger bound
+    out["floor_frac"] = round(floor_ms / step_ms, 4)   # of the measured step
+    return out
+
+
+def median_step_ms(torch, step, steps, warmup):
+    """Median and mean of `steps` forwards, each between its own pair of events on the launch stream."""
+    import numpy as np
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.time()
+    evs[0].record()
+    for k in range(steps):
+        step()
+        evs[k + 1].record()
+    torch.cuda.synchronize()
+    wall = (time.time() - t0) * 1000.0 / steps
+    per = [evs[k].elapsed_time(evs[k + 1]) for k in range(steps)]
+    return float(np.median(per)), float(np.mean(per)), wall
+
+
+def other_configs(torch, with_cpu):
+    """The other four configurations at their full batch sizes: images/s of a HIP graph replay (median of 20 forwards),
+    the per-class roofline of a forward, and (CPU leg) the GPU result against the CPU oracle: LeNet and the single stage
+    convolution in full, with the oracle's own time as their CPU baseline; MobileNet-v1 and ResNet-18 W4A4 on the first
+    two images of the batch."""
     import numpy as np
     from n2d2_amd import nets
     from oracle import cells
-    flags = {}
+    out = {}
     rng = np.random.default_rng(77)
-    for name, make, batch in (("lenet_8bit_bs256", nets.lenet, 256), ("resnet18_stage_conv_bs64", nets.single_conv_stage, 64),
-                              ("mobilenet_v1_8bit", nets.mobilenet_v1, 2), ("resnet18_w4a4", nets.resnet18_w4a4, 2)):
+    for name, make, batch, full in (("lenet_8bit_bs256", nets.lenet, 256, True), ("resnet18_stage_conv_bs64", nets.single_conv_stage, 64, True),
+                                    ("mobilenet_v1_8bit_bs64", nets.mobilenet_v1, 64, False), ("resnet18_w4a4_bs64", nets.resnet18_w4a4, 64, False)):
         spec = make()
         x = rng.integers(0, 256, size=(batch,) + tuple(spec.in_shape))
         net = nets.GpuNet(spec, batch)
         net.set_input(x)
         got = net.forward().to_numpy().astype(np.int64)
-        want = cells.run_net(spec, x)[spec.output].astype(np.int64)
-        flags[name] = bool(got.shape == want.shape and np.array_equal(got, want))
-    return flags
+        replay = net.capture()
+        ms, mean_ms, _ = median_step_ms(torch, replay, 20, 3)
+        runs = [net.forward_timed() for _ in range(5)]
+        per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
+        entry = {"batch": batch, "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "ms_per_step": round(ms, 4),
+                 "launches": len(net.launched), "gmac_per_image": round(spec.macs_per_image() / 1e9, 4),
+                 "roofline_by_class": class_rooflines(net, per_launch, ms)}
+        if with_cpu:
+            n = batch if full else 2
+            t0 = time.time()
+            want = cells.run_net(spec, x[:n])[spec.output].astype(np.int64)
+            dt = time.time() - t0
+            entry["bit_exact_vs_cpu"] = bool(np.array_equal(got[:n].reshape(n, -1), want.reshape(n, -1)))
+            entry["cpu_baseline"] = {"value": round(n / dt, 3), "unit": "images/s", "kind": "port",
+                                     "cores": int(os.environ.get("OMP_NUM_THREADS", 0)) or len(os.sched_getaffinity(0)),
+                                     "sample": ("the whole batch" if full else "the first %d images of the batch" % n)}
+        out[name] = entry
+        del net, replay
+    return out
 
 
 PEAK_FP32_TFLOPS = 157.3
@@ -171,6 +239,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=128)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="only the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="time cell-by-cell launches instead of a HIP graph replay")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 1 GiB device-to-device copy first (known traffic, to scale FETCH_SIZE / WRITE_SIZE counters)")
@@ -202,90 +271,101 @@ def main():
     torch.cuda.synchronize()
 
     def timed(step):
-        for _ in range(args.warmup):
-            step()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.time()
-        e0.record()
-        for _ in range(args.steps):
-            step()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / args.steps, (time.time() - t0) * 1000.0 / args.steps
+        return median_step_ms(torch, step, args.steps, args.warmup)
 
     # one step = one forward of the whole network; launched cell by cell ("eager") and as one HIP graph replay
-    eager_ms, eager_wall_ms = timed(net.forward)
+    eager_ms, eager_mean_ms, eager_wall_ms = timed(net.forward)
     eager_logits = net.tensors[spec.output].to_numpy().reshape(B, -1)
     if args.no_graph:
-        ms, wall_ms, launch = eager_ms, eager_wall_ms, "eager"
+        ms, mean_ms, wall_ms, launch = eager_ms, eager_mean_ms, eager_wall_ms, "eager"
     else:
         replay = net.capture()
-        ms, wall_ms = timed(replay)
+        ms, mean_ms, wall_ms = timed(replay)
         launch = "hipGraph replay"
     logits = net.tensors[spec.output].to_numpy().reshape(B, -1)
     if not np.array_equal(logits, eager_logits):
         print("bench.py: graph replay and eager launches disagree", file=sys.stderr)
         sys.exit(4)
+    # the engine clock the chip holds under matrix-core load, right behind the timed steps: the published 5.0 POP/s assume
+    # 2.4 GHz (256 CUs x 8192 int8 operations per clock)
+    import ctypes as C
+    from n2d2_amd import capi, runtime
+    mhz = C.c_double(0.0)
+    capi.check(capi.lib.n2d2hip_measure_clock(200.0, C.byref(mhz), runtime.stream_ptr()))
+    clock = {"engine_clock_mhz_under_mfma_load": round(mhz.value, 1),
+             "int8_peak_at_that_clock_tops": round(256 * 8192 * mhz.value * 1e6 / 1e12, 1)}
 
-    # Dominant kernel: conv_pipe_kernel, the pipelined int8-MFMA implicit-GEMM convolution that runs every
-    # convolution / fully-connected cell whose input channel count is a multiple of 64 (with the residual sum in its
-    # epilogue where one follows).  Its launches are replayed alone, back to back, between two events on the launch
+    # Which kernel runs a launch of the forward (the library's own rules, restated here to label the figures):
+    # bottleneck_kernel (a residual block in one launch), conv_patch3x3_kernel (3x3, stride 1, at least 128 channels, on an
+    # input that carries its padding, images of at least 10 x 10), conv_stem_kernel (at most 4 input channels),
+    # conv_pipe_kernel (every other convolution / fully-connected cell with a multiple of 64 input channels, with the
+    # residual sum in its epilogue where one follows), bandwidth kernels for the rest.
+    def kernel_of(k):
+        l = net.launched[k]
+        if l.name in net.bottlenecks:
+            return "bottleneck_kernel"
+        c = net.fused_sums[l.name][1] if l.name in net.fused_sums else l
+        if c.type not in ("conv", "fc"):
+            return "bandwidth"
+        if c.type == "conv" and c.w.shape[1] <= 4:
+            return "conv_stem_kernel"
+        if getattr(c, "groups", 1) != 1 or c.weight_bits != 8 or c.w.shape[1] % 64 != 0:
+            return "other"
+        x = net._io[k][0][0]
+        if (c.type == "conv" and l.name not in net.fused_sums and c.w.shape[2:] == (3, 3) and tuple(c.stride) == (1, 1) and tuple(c.pad) == (1, 1, 1, 1)
+                and tuple(c.dil) == (1, 1) and x.halo == 1 and c.w.shape[1] >= 128 and c.w.shape[0] % 64 == 0
+                and (x.H + 2) * (x.W + 2) * 100 <= x.H * x.W * 135):
+            return "conv_patch3x3_kernel"
+        return "conv_pipe_kernel"
+    kernels = [kernel_of(k) for k in range(len(net.launched))]
+
+    # Dominant kernel: conv_pipe_kernel.  Its launches are replayed alone, back to back, between two events on the launch
     # stream: elapsed / launches is the average launch duration (inter-launch gaps included).
-    def conv_of(l):
-        return net.fused_sums[l.name][1] if l.name in net.fused_sums else l
-
-    def on_pipe(l):
-        c = conv_of(l)
-        return c.type in ("conv", "fc") and getattr(c, "groups", 1) == 1 and c.weight_bits == 8 and c.w.shape[1] % 64 == 0
-    pipe = [k for k, l in enumerate(net.launched) if on_pipe(l)]
-    for _ in range(3):
-        net.forward_subset(pipe)
-    torch.cuda.synchronize()
-    p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    p0.record()
-    for _ in range(args.steps):
-        net.forward_subset(pipe)
-    p1.record()
-    torch.cuda.synchronize()
-    conv_ms = p0.elapsed_time(p1) / args.steps
+    def replay_alone(idx):
+        for _ in range(3):
+            net.forward_subset(idx)
+        torch.cuda.synchronize()
+        p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        p0.record()
+        for _ in range(args.steps):
+            net.forward_subset(idx)
+        p1.record()
+        torch.cuda.synchronize()
+        return p0.elapsed_time(p1) / args.steps
+    pipe = [k for k, name in enumerate(kernels) if name == "conv_pipe_kernel"]
+    conv_ms = replay_alone(pipe)
     conv_ops = 2.0 * sum(net.layer_macs(net.launched[k]) for k in pipe)
     achieved = conv_ops / (conv_ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "conv_pipe_kernel (%d launches of one forward: every conv/fc cell with a multiple of 64 input "
-                "channels, residual sums folded in)" % len(pipe),
+    roofline = {"bound": "mfma", "kernel": "conv_pipe_kernel (%d launches of one forward: conv/fc cells with a multiple of 64 input "
+                "channels, residual sums folded in; not the cells of the fused bottleneck nor the 3x3 layers on the patch kernel)" % len(pipe),
                 "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                "traffic": round(PIPE_TRAFFIC_BYTES_PER_LAUNCH) if B == 128 else None,
+                "traffic": None, "traffic_from_profile": TRAFFIC_FROM_PROFILE if B == 128 else None,
                 "algorithmic_bytes_per_launch": round(sum(net.layer_bytes(net.launched[k]) for k in pipe) / len(pipe)),
                 "launches_per_step": len(pipe), "avg_launch_us": round(conv_ms * 1000.0 / len(pipe), 2),
-                "ops_per_launch": conv_ops / len(pipe)}
+                "ops_per_launch": conv_ops / len(pipe), "frac_of_peak_at_measured_clock": round(achieved / clock["int8_peak_at_that_clock_tops"], 4)}
+    # the other convolution kernels of the forward, each replayed alone the same way
+    roofline_kernels = {}
+    for name in ("conv_patch3x3_kernel", "bottleneck_kernel", "conv_stem_kernel"):
+        idx = [k for k, kn in enumerate(kernels) if kn == name]
+        if not idx:
+            continue
+        t = replay_alone(idx)
+        ops = 2.0 * sum(net.layer_macs(net.launched[k]) for k in idx)
+        nbytes = float(sum(net.layer_bytes(net.launched[k]) for k in idx))
+        roofline_kernels[name] = {"launches": len(idx), "avg_launch_us": round(t * 1000.0 / len(idx), 2),
+                                  "tops": round(ops / (t * 1e-3) / 1e12, 1), "frac_of_int8_peak": round(ops / (t * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4),
+                                  "gbs": round(nbytes / (t * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(nbytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     all_bytes = sum(net.layer_bytes(l) for l in net.launched)
     hbm = all_bytes / (ms * 1e-3) / 1e9
     roofline_hbm = {"bound": "hbm", "kernel": "whole forward (%d launches)" % len(net.launched), "achieved": round(hbm, 1),
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(hbm / PEAK_HBM_GBS, 4), "bytes_per_step": all_bytes}
 
     # Per-class view: every launch timed with its own pair of events (median of 7 forwards), put against the larger of
-    # its two bounds (2*MAC at the int8 MFMA peak, algorithmic bytes at the HBM peak).  The per-launch events add about
-    # 10 % to the sum, so the class times are an upper estimate of their share of `ms_per_step`.
+    # its two bounds.  The per-launch events add about 10 % to the sum, so the class times are an upper estimate of their
+    # share of `ms_per_step`.
     runs = [net.forward_timed() for _ in range(7)]
     per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
-    classes = {}
-    floor_ms = 0.0
-    for l, t in zip(net.launched, per_launch):
-        ops, nbytes = 2.0 * net.layer_macs(l), float(net.layer_bytes(l))
-        t_mfma, t_hbm = ops / (PEAK_INT8_TOPS * 1e12) * 1e3, nbytes / (PEAK_HBM_GBS * 1e9) * 1e3
-        floor_ms += max(t_mfma, t_hbm)
-        c = classes.setdefault("mfma_bound" if t_mfma > t_hbm else "hbm_bound", {"launches": 0, "ms": 0.0, "ops": 0.0, "bytes": 0.0})
-        c["launches"] += 1; c["ms"] += t; c["ops"] += ops; c["bytes"] += nbytes
-    by_class = {}
-    for name, c in classes.items():
-        if name == "mfma_bound":
-            ach, peak, unit = c["ops"] / (c["ms"] * 1e-3) / 1e12, PEAK_INT8_TOPS, "TOP/s"
-        else:
-            ach, peak, unit = c["bytes"] / (c["ms"] * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
-        by_class[name] = {"launches": c["launches"], "ms": round(c["ms"], 4), "achieved": round(ach, 1), "peak": peak, "unit": unit,
-                          "frac": round(ach / peak, 4)}
-    by_class["floor_ms"] = round(floor_ms, 4)          # sum over launches of the larger bound
-    by_class["floor_frac"] = round(floor_ms / ms, 4)   # of the measured step
+    by_class = class_rooflines(net, per_launch, ms)
 
     # Two batches in flight: a second, independent forward of the same network on another batch of the same size runs on
     # its own stream, so each stream's launch gaps and tails are filled by the other's kernels.  Reported next to `value`
@@ -314,7 +394,7 @@ def main():
                 for j in joins:
                     cap.wait_event(j)
         torch.cuda.synchronize()
-        ms2, _ = timed(graph2.replay)
+        ms2, _, _ = timed(graph2.replay)
         ok2 = (np.array_equal(net.tensors[spec.output].to_numpy().reshape(B, -1), eager_logits)
                and np.array_equal(net2.tensors[spec.output].to_numpy().reshape(B, -1), want2))
         if not ok2:
@@ -326,12 +406,14 @@ def main():
 
     result = {
         "metric": "int8 ResNet-50 images/sec @bs128 on 1 MI355X", "value": round(B / (ms * 1e-3), 1), "unit": "images/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4),
-        "launch": launch, "eager_ms_per_step": round(eager_ms, 4),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "ms_per_step_is": "median of the steps",
+        "mean_ms_per_step": round(mean_ms, 4), "wall_ms_per_step": round(wall_ms, 4),
+        "launch": launch, "launches_per_step": len(net.launched), "eager_ms_per_step": round(eager_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": "resnet50_int8_ptq_forward_224", "global_batch": B, "input": "uint8 %dx3x224x224" % B,
                    "layers": len(spec.layers), "gmac_per_image": round(spec.macs_per_image() / 1e9, 3)},
-        "roofline": roofline, "roofline_hbm": roofline_hbm, "roofline_by_class": by_class,
+        "roofline": roofline, "roofline_kernels": roofline_kernels, "roofline_hbm": roofline_hbm, "roofline_by_class": by_class,
+        "clock": clock,
     }
     if overlapped is not None:
         result["two_batches_in_flight"] = overlapped
@@ -347,10 +429,11 @@ def main():
         base, exact = cpu_baseline(spec, logits, images)
         result["cpu_baseline"] = base
         result["bit_exact_vs_cpu"] = exact
+    if not args.no_other_configs:
         try:
-            result["other_configs_bit_exact_vs_cpu"] = other_configs_bit_exact()
+            result["other_configs"] = other_configs(torch, not args.no_cpu_baseline)
         except Exception as e:
-            result["other_configs_bit_exact_vs_cpu"] = {"error": "%s: %s" % (type(e).__name__, e)}
+            result["other_configs"] = {"error": "%s: %s" % (type(e).__name__, e)}
     print(json.dumps(result))
 
 

@@ -39,6 +39,12 @@ const char* n2d2hip_last_error(void);
 /* Library version string and the gfx target the kernels were built for. */
 const char* n2d2hip_version(void);
 
+/* Diagnostic, no counterpart in the reference: the engine clock in MHz the GPU holds while every CU runs int8 matrix
+ * instructions for about `busy_microseconds` (shader clocks per tick of the constant 100 MHz counter, read inside a
+ * kernel).  Published matrix-core peaks assume the maximum clock; a measured fraction of the peak is read against this.
+ * Allocates a small device buffer and waits for the stream. */
+int n2d2hip_measure_clock(double busy_microseconds, double* mhz, n2d2hip_stream_t stream);
+
 /* --------------------------------------------------------------- tensors */
 /* Element types.  N2D2 holds integer values in float storage
  * (ref: src/Cell/ConvCell_Frame.cpp:28-44); here they are stored narrow. */

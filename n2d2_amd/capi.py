@@ -26,7 +26,7 @@ KERNEL_NO_PATCH, KERNEL_PATCH = 256, 512
 
 # every symbol include/n2d2hip.h declares
 SYMBOLS = [
-    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
+    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_measure_clock", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
     "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_accepts_halo",
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
@@ -83,6 +83,7 @@ def load():
     lib.n2d2hip_quantizer_workspace_bytes.argtypes = [C.c_size_t]
     P, I, F, SZ, U = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
     lib.n2d2hip_convert.argtypes = [P, P, P]
+    lib.n2d2hip_measure_clock.argtypes = [C.c_double, P, P]
     lib.n2d2hip_act_create.argtypes = [P, I, P]
     lib.n2d2hip_act_destroy.argtypes = [P]
     lib.n2d2hip_scaling_forward.argtypes = [P, P, P, P]

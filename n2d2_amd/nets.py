@@ -449,6 +449,18 @@ class GpuNet:
                 raise ValueError(l.type)
             self.tensors[l.name] = out
             ins_of[l.name] = ins
+        # a network input that only padded convolutions of this kind read carries their padding too (the graph-edge
+        # conversion fills the interior)
+        first = consumers.get("input", [])
+        if halo and first and all(reads_halo(m) for m in first) and all(c.accepts_halo() for (m, c, f) in self.steps if m in first):
+            h = max(max(m.pad) for m in first)
+            if h > 0:
+                nx = rt.DTensor(batch, C, H, W, self.input.dtype, halo=h)
+                for lst in ins_of.values():
+                    for k, t in enumerate(lst):
+                        if t is self.input:
+                            lst[k] = nx
+                self.input = self.tensors["input"] = nx
         self.bottlenecks, self.bottleneck_layers = {}, {}
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
@@ -550,7 +562,11 @@ class GpuNet:
     def set_input(self, x):
         """x: integer NCHW numpy array [B,C,H,W]."""
         t = self.rt.DTensor.from_numpy(x, self.input.dtype)
-        self.input.buf.copy_(t.buf)
+        h = self.input.halo
+        if h:
+            self.input.buf.view(t.B, t.H + 2 * h, t.W + 2 * h, t.cs)[:, h:t.H + h, h:t.W + h, :] = t.buf.view(t.B, t.H, t.W, t.cs)
+        else:
+            self.input.buf.copy_(t.buf)
 
     def forward(self):
         for (l, cell, fn), (ins, out) in zip(self.steps, self._io):
