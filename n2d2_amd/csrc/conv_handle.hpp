@@ -36,6 +36,8 @@ struct n2d2hip_conv_s {
     signed char* d_wstem;
     // 3x3 stride-1 kernel over inputs that carry their padding: weights in matrix-core fragment order
     signed char* d_wfrag;
+    // 3x3 depthwise kernel: per channel and kernel row the three weights in one dword, then the biases with the zero point folded in
+    int* d_wdw;
     bool is_fc;
     int fcH, fcW;
 };

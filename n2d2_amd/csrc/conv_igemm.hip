@@ -25,6 +25,7 @@
 #include "epilogue.hpp"
 #include "mfma_util.hpp"
 #include "conv_patch.hpp"
+#include "depthwise.hpp"
 
 namespace n2d2hip {
 
@@ -505,7 +506,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -521,6 +522,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     const int cs = c->in_cs;
     std::vector<signed char> hw;
     std::vector<int4> hsub;
+    std::vector<int> hwdw;
     c->opad = round_up(d->O, 128);
     std::vector<int> hbias((size_t)std::max(c->opad, act->cpad), 0);
     const long long wstrideO = (long long)Cg * d->kH * d->kW;
@@ -593,7 +595,14 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             for (int ky = 0; ky < d->kH; ++ky)
                 for (int kx = 0; kx < d->kW; ++kx)
                     hw[(size_t)(ky * d->kW + kx) * cs + ch] = (signed char)read_weight(weights, ((long long)ch * d->kH + ky) * d->kW + kx, 8);
-        // the kernel adds the zero point to every loaded input, so the fold is not wanted here
+        if (d->kH == 3 && d->kW == 3 && d->dilX == 1 && d->dilY == 1 && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PIPE)) {
+            std::vector<signed char> w9((size_t)d->C * 9);
+            for (size_t i = 0; i < w9.size(); ++i)
+                w9[i] = (signed char)read_weight(weights, (long long)i, 8);
+            hwdw.resize(4 * (size_t)cs);
+            depthwise3x3_weight_layout(w9.data(), hbias.data(), d->C, cs, hwdw.data());
+        }
+        // the general kernel adds the zero point to every loaded input, so the fold is not wanted there
         for (int o = 0; o < d->O; ++o)
             hbias[o] = bias ? bias[o] : 0;
         c->ktot = 0;
@@ -669,6 +678,10 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_wfrag, hfrag.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wfrag, hfrag.data(), hfrag.size(), hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess && !hwdw.empty()) {
+        e = hipMalloc((void**)&c->d_wdw, hwdw.size() * sizeof(int));
+        if (e == hipSuccess) e = hipMemcpy(c->d_wdw, hwdw.data(), hwdw.size() * sizeof(int), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hepi.empty()) {
         e = hipMalloc((void**)&c->d_epi_tab, hepi.size() * sizeof(int));
         if (e == hipSuccess) e = hipMemcpy(c->d_epi_tab, hepi.data(), hepi.size() * sizeof(int), hipMemcpyHostToDevice);
@@ -702,6 +715,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
     if (c->d_wstem) (void)hipFree(c->d_wstem);
     if (c->d_wfrag) (void)hipFree(c->d_wfrag);
+    if (c->d_wdw) (void)hipFree(c->d_wdw);
     delete c;
     return N2D2HIP_OK;
 }
@@ -772,6 +786,17 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
 
     if (c->depthwise) {
         N2D2HIP_REQUIRE(out->cs == in->cs, N2D2HIP_ERR_INVALID, "conv_forward: depthwise needs equal channel strides");
+        N2D2HIP_REQUIRE(in->halo == 0 && out->halo == 0, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: depthwise tensors carry no border");
+        if (c->d_wdw && d.strideX == d.strideY && (d.strideX == 1 || d.strideX == 2) && is_byte_type(out->dtype)
+            && c->act->cpad >= in->cs) {
+            DepthwiseArgs q;
+            q.in = (const signed char*)in->data; q.out = out->data; q.wb = c->d_wdw;
+            q.cs = in->cs; q.B = in->B; q.H = in->H; q.W = in->W; q.OH = OH; q.OW = OW; q.padL = d.padL; q.padT = d.padT;
+            q.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
+            q.out_xor = out_xor;
+            q.epi = c->act->args;
+            return depthwise3x3_launch(q, d.strideX, num_cus(), stream);
+        }
         const long long total = Mll * (in->cs / 4);
         const unsigned grid = (unsigned)std::min<long long>((total + 255) / 256, 256 * 64);
         hipLaunchKernelGGL(depthwise_kernel, dim3(grid), dim3(256), 0, stream, (const signed char*)in->data, in->cs, in->B, in->H,

@@ -1,0 +1,168 @@
+// 3x3 depthwise convolution on NHWC bytes: groups == C == O, so there is no reduction over channels and no matrix core:
+// the layer is bound by memory traffic and, behind it, by the vector ALU
+// (ref: src/Cell/ConvCell_Frame_Kernels.cpp:26-179 with one channel per group).
+//
+// A thread owns 4 consecutive channels (one dword) of one output column and walks down a strip of output rows, so
+// consecutive lanes read and write consecutive bytes.  Each input row it meets is loaded once as the three pixels left,
+// middle and right of the column and transposed into four dwords, one per channel, of (left, middle, right, 0); every
+// output row that uses the input row then needs one 4-way dot product per channel against (w[ky][0], w[ky][1], w[ky][2], 0).
+// Taps outside the image read the stored form of 0, which lets the input's zero point live in the bias.
+#include "depthwise.hpp"
+#include "epilogue.hpp"
+
+namespace n2d2hip {
+
+namespace {
+
+struct Row4 { int c[4]; };
+
+__device__ __forceinline__ Row4 transpose3(unsigned xm, unsigned x0, unsigned xp)
+{
+    const unsigned lo = __builtin_amdgcn_perm(x0, xm, 0x05010400u);   // m0 c0 m1 c1
+    const unsigned hi = __builtin_amdgcn_perm(x0, xm, 0x07030602u);   // m2 c2 m3 c3
+    Row4 r;
+    r.c[0] = (int)__builtin_amdgcn_perm(xp, lo, 0x0c040100u);
+    r.c[1] = (int)__builtin_amdgcn_perm(xp, lo, 0x0c050302u);
+    r.c[2] = (int)__builtin_amdgcn_perm(xp, hi, 0x0c060100u);
+    r.c[3] = (int)__builtin_amdgcn_perm(xp, hi, 0x0c070302u);
+    return r;
+}
+
+template <int S, int KIND>
+__global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p)
+{
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= p.nthreads)
+        return;
+    const unsigned cg = idx % p.cq;
+    unsigned r = idx / p.cq;
+    const int ox = (int)(r % (unsigned)p.OW);
+    r /= (unsigned)p.OW;
+    const int strip = (int)(r % (unsigned)p.nstrips);
+    const int b = (int)(r / (unsigned)p.nstrips);
+    const int c4 = (int)cg * 4;
+    const int oy0 = strip * p.rows;
+    const int nrows = min(p.rows, p.OH - oy0);
+
+    const int4 w0 = *(const int4*)(p.wb + c4);
+    const int4 w1 = *(const int4*)(p.wb + p.cs + c4);
+    const int4 w2 = *(const int4*)(p.wb + 2 * p.cs + c4);
+    const int4 bias = *(const int4*)(p.wb + 3 * p.cs + c4);
+    int4 ta = {}, tb = {}, tc = {}, td = {}, te = {};
+    if (KIND == EPI_I24 || KIND == EPI_I64) {
+        ta = *(const int4*)(p.epi.a + c4);
+        tb = *(const int4*)(p.epi.b + c4);
+        tc = *(const int4*)(p.epi.c + c4);
+        td = *(const int4*)(p.epi.d + c4);
+        te = *(const int4*)(p.epi.e + c4);
+    }
+
+    const int ix0 = ox * S - p.padL;
+    const bool vm = ix0 >= 0 && ix0 < p.W, v0 = ix0 + 1 >= 0 && ix0 + 1 < p.W, vp = ix0 + 2 >= 0 && ix0 + 2 < p.W;
+    const signed char* col = p.in + ((long long)b * p.H * p.W + ix0) * p.cs + c4;
+    const long long row_bytes = (long long)p.W * p.cs;
+    const unsigned fill = p.fill;
+    Row4 border;
+    border.c[0] = border.c[1] = border.c[2] = border.c[3] = (int)(fill & 0x00ffffffu);
+
+    auto load_row = [&](int iy) -> Row4 {
+        if (iy < 0 || iy >= p.H)
+            return border;
+        const signed char* rp = col + iy * row_bytes;
+        const unsigned xm = vm ? *(const unsigned*)rp : fill;
+        const unsigned x0 = v0 ? *(const unsigned*)(rp + p.cs) : fill;
+        const unsigned xp = vp ? *(const unsigned*)(rp + 2 * p.cs) : fill;
+        return transpose3(xm, x0, xp);
+    };
+    auto finish = [&](int v, int ch, int a, int bq, int c, int d, int e) -> int {
+        if (KIND == EPI_I24 || KIND == EPI_I64)
+            return epi_apply<KIND>(v, a, bq, c, d, e, p.epi.lo, p.epi.hi, 0);
+        return epi_apply_dyn(p.epi, v, c4 + ch);
+    };
+    unsigned* outp = (unsigned*)((signed char*)p.out + (((long long)b * p.OH + oy0) * p.OW + ox) * p.cs + c4);
+    const long long out_row = (long long)p.OW * p.cs / 4;
+
+    const int iy0 = oy0 * S - p.padT;
+    Row4 t0 = load_row(iy0);
+    Row4 t1 = {};
+    if (S == 1)
+        t1 = load_row(iy0 + 1);
+    for (int q = 0; q < nrows; ++q) {
+        Row4 t2;
+        if (S == 1) {
+            t2 = load_row(iy0 + q + 2);
+        } else {
+            t1 = load_row(iy0 + 2 * q + 1);
+            t2 = load_row(iy0 + 2 * q + 2);
+        }
+        int a0 = __builtin_amdgcn_sdot4(t0.c[0], w0.x, bias.x, false);
+        int a1 = __builtin_amdgcn_sdot4(t0.c[1], w0.y, bias.y, false);
+        int a2 = __builtin_amdgcn_sdot4(t0.c[2], w0.z, bias.z, false);
+        int a3 = __builtin_amdgcn_sdot4(t0.c[3], w0.w, bias.w, false);
+        a0 = __builtin_amdgcn_sdot4(t1.c[0], w1.x, a0, false);
+        a1 = __builtin_amdgcn_sdot4(t1.c[1], w1.y, a1, false);
+        a2 = __builtin_amdgcn_sdot4(t1.c[2], w1.z, a2, false);
+        a3 = __builtin_amdgcn_sdot4(t1.c[3], w1.w, a3, false);
+        a0 = __builtin_amdgcn_sdot4(t2.c[0], w2.x, a0, false);
+        a1 = __builtin_amdgcn_sdot4(t2.c[1], w2.y, a1, false);
+        a2 = __builtin_amdgcn_sdot4(t2.c[2], w2.z, a2, false);
+        a3 = __builtin_amdgcn_sdot4(t2.c[3], w2.w, a3, false);
+        const int r0 = finish(a0, 0, ta.x, tb.x, tc.x, td.x, te.x);
+        const int r1 = finish(a1, 1, ta.y, tb.y, tc.y, td.y, te.y);
+        const int r2 = finish(a2, 2, ta.z, tb.z, tc.z, td.z, te.z);
+        const int r3 = finish(a3, 3, ta.w, tb.w, tc.w, td.w, te.w);
+        const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+        outp[q * out_row] = packed ^ p.out_xor;
+        if (S == 1) {
+            t0 = t1;
+            t1 = t2;
+        } else {
+            t0 = t2;
+        }
+    }
+}
+
+} // namespace
+
+void depthwise3x3_weight_layout(const signed char* w, const int* bias, int C, int cs, int* wb)
+{
+    for (int i = 0; i < 4 * cs; ++i)
+        wb[i] = 0;
+    for (int c = 0; c < C; ++c) {
+        for (int ky = 0; ky < 3; ++ky) {
+            const signed char* t = w + ((size_t)c * 3 + ky) * 3;
+            wb[ky * cs + c] = (int)((unsigned)(unsigned char)t[0] | ((unsigned)(unsigned char)t[1] << 8) | ((unsigned)(unsigned char)t[2] << 16));
+        }
+        wb[3 * cs + c] = bias[c];
+    }
+}
+
+int depthwise3x3_launch(DepthwiseArgs a, int stride, int num_cus, hipStream_t stream)
+{
+    N2D2HIP_REQUIRE((stride == 1 || stride == 2) && a.cs % 4 == 0, N2D2HIP_ERR_INVALID, "depthwise3x3: stride %d, channel stride %d", stride, a.cs);
+    a.cq = (unsigned)(a.cs / 4);
+    // Strips short enough that every compute unit holds about 1024 threads: a strip re-reads the two input rows above it.
+    const long long columns = (long long)a.B * a.OW * a.cq;
+    const long long want = (long long)num_cus * 1024;
+    long long nstrips = std::min<long long>((want + columns - 1) / columns, (a.OH + 1) / 2);
+    nstrips = std::max<long long>(nstrips, 1);
+    a.rows = (int)((a.OH + nstrips - 1) / nstrips);
+    a.nstrips = (a.OH + a.rows - 1) / a.rows;
+    const long long nthreads = columns * a.nstrips;
+    N2D2HIP_REQUIRE(nthreads < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "depthwise3x3: tensor too large");
+    a.nthreads = (unsigned)nthreads;
+    const unsigned grid = (unsigned)((nthreads + 255) / 256);
+#define N2D2HIP_DW_LAUNCH(S, K) hipLaunchKernelGGL((depthwise3x3_kernel<S, K>), dim3(grid), dim3(256), 0, stream, a)
+    if (a.epi.kind == EPI_I24) {
+        if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_I24); else N2D2HIP_DW_LAUNCH(2, EPI_I24);
+    } else if (a.epi.kind == EPI_I64) {
+        if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_I64); else N2D2HIP_DW_LAUNCH(2, EPI_I64);
+    } else {
+        if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_RAW); else N2D2HIP_DW_LAUNCH(2, EPI_RAW);
+    }
+#undef N2D2HIP_DW_LAUNCH
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+} // namespace n2d2hip

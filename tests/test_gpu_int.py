@@ -233,6 +233,30 @@ def test_depthwise_conv_bit_exact(rt, stride):
     assert np.array_equal(conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), want.astype(np.int64))
 
 
+@pytest.mark.parametrize("stride", [1, 2])
+def test_depthwise3x3_strip_kernel_against_general_kernel(rt, stride):
+    """The 3x3 depthwise kernel (threads walk down strips of rows) against the oracle and against the general depthwise
+    kernel, on shapes whose strips end unevenly, with and without padding, unsigned and signed inputs."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    for (B, Cc, H, W, pad, in_dtype) in ((5, 32, 37, 29, 1, capi.U8B), (2, 130, 9, 11, 1, capi.I8), (3, 64, 14, 14, 0, capi.U8B),
+                                         (1, 8, 3, 3, 1, capi.U8B)):
+        x = _u8((B, Cc, H, W)) if in_dtype == capi.U8B else _i8((B, Cc, H, W))
+        w = _i8((Cc, 1, 3, 3))
+        bias = RNG.integers(-2000, 2001, size=Cc).astype(np.int32)
+        spec = _acts(Cc)["fixed_relu_u"]
+        spec.scaling = RNG.integers(2 ** 13, 2 ** 14, size=Cc)
+        spec.frac_bits = 21
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(pad,) * 4, groups=Cc)
+        got = {}
+        for choice in (0, capi.KERNEL_NO_PIPE):
+            conv = rt.Conv(w, bias, rt.Act(Cc, **spec.kwargs()), in_dtype, stride=(stride, stride), pad=(pad,) * 4, groups=Cc,
+                           kernel_choice=choice)
+            got[choice] = conv.forward(rt.DTensor.from_numpy(x, in_dtype)).to_numpy()
+        assert np.array_equal(got[0], want.astype(np.int64)), (B, Cc, H, W, pad)
+        assert np.array_equal(got[capi.KERNEL_NO_PIPE], got[0])
+
+
 def test_conv_int4_weights_uint4_activations(rt):
     """Weights in [-7,7] nibble-packed, activations in [0,15], fixed-point rescale with clip, 4-bit unsigned output."""
     from n2d2_amd import capi

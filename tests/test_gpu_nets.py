@@ -48,9 +48,24 @@ def test_resnet50_config(variant):
     net = _run_both(spec, x, keep)
     # 12 shortcut ScalingCells folded into their sums, 16 sums folded into the convolution that feeds them
     assert "conv2.2_shortcut_rescale" in net.folded and "conv2.1_1x1_proj" in net.folded and "conv2.2_1x1_x4" in net.folded
-    assert len(net.folded) == 28 and len(net.launched) == len(spec.layers) - 28
-    # the 16 tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border of zeros
-    assert sorted(n for n, t in net.tensors.items() if t.halo) == sorted(l.name[:-3] + "1x1" for l in spec.layers if l.name.endswith("_3x3"))
+    # ... and the first residual block (the one with a projection shortcut at full resolution) runs as one launch, which
+    # takes its two middle convolutions and its expansion out of the launch list as well
+    # (the kernel is written for activations in [0, 255]: the all-signed variant keeps its cells apart)
+    one_launch = variant != "all_signed"
+    assert list(net.bottlenecks) == (["conv2.1_sum"] if one_launch else [])
+    if one_launch:
+        assert [m.name for m in net.bottleneck_layers["conv2.1_sum"]] == ["conv2.1_1x1", "conv2.1_3x3", "conv2.1_1x1_x4", "conv2.1_1x1_proj"]
+    nfolded = 31 if one_launch else 28
+    assert len(net.folded) == nfolded and len(net.launched) == len(spec.layers) - nfolded
+    # the tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border of zeros, and so does the
+    # input of the block that runs as one launch
+    assert sorted(n for n, t in net.tensors.items() if t.halo) == sorted(
+        [l.name[:-3] + "1x1" for l in spec.layers if l.name.endswith("_3x3") and not (one_launch and l.name == "conv2.1_3x3")]
+        + (["pool1"] if one_launch else []))
+    separate = nets.GpuNet(spec, x.shape[0], bottlenecks=False)
+    separate.set_input(x)
+    assert not separate.bottlenecks and len(separate.folded) == 28 and len(separate.launched) == len(spec.layers) - 28
+    assert np.array_equal(separate.forward().to_numpy(), net.tensors[spec.output].to_numpy())
     if variant == "pad1":
         unfused = _run_both(spec, x, keep, fuse=False)
         assert not unfused.folded
@@ -103,7 +118,7 @@ def test_resnet50_full_batch_properties():
     assert np.array_equal(net.forward().to_numpy()[:, :, 0, 0], logits)
     # ... and so do twenty more, tensor by tensor on a few layers of each kind, launched back to back and replayed
     # from a graph (asynchronous LDS traffic and hand-counted waits leave no room for run-to-run differences)
-    watch = ["conv1", "pool1", "conv2.1_3x3", "conv2.3_sum", "conv3.4_sum", "conv4.6_sum", "conv5.3_sum", "pool", "fc"]
+    watch = ["conv1", "pool1", "conv2.1_sum", "conv2.2_3x3", "conv2.3_sum", "conv3.4_sum", "conv4.6_sum", "conv5.3_sum", "pool", "fc"]
     ref = {n: net.tensors[n].to_numpy() for n in watch}
     replay = net.capture()
     for it in range(20):
