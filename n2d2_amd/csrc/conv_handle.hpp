@@ -38,6 +38,8 @@ struct n2d2hip_conv_s {
     signed char* d_wfrag;
     // 3x3 depthwise kernel: per channel and kernel row the three weights in one dword, then the biases with the zero point folded in
     int* d_wdw;
+    // 4-bit weights for the pipelined kernel: the ring's weight tiles as LDS wants them, two weights per byte
+    signed char* d_w4img;
     bool is_fc;
     int fcH, fcW;
 };

@@ -24,29 +24,12 @@
 #include "common.h"
 #include "epilogue.hpp"
 #include "mfma_util.hpp"
+#include "conv_args.hpp"
 #include "conv_patch.hpp"
 #include "depthwise.hpp"
 
 namespace n2d2hip {
 
-struct ConvArgs {
-    const signed char* in;
-    int in_cs, B, H, W;
-    int OH, OW, M;          // M = B*OH*OW output pixels
-    const signed char* w;   // prepared weights
-    int ktot;               // K bytes per weight row (multiple of 64)
-    int niter;              // ktot / 64
-    const int4* sub;        // sub-chunk table, ktot/16 entries
-    const int* bias;        // [Opad], zero-point fold included
-    void* out;
-    int out_cs, out_dtype;
-    int strideX, strideY, padL, padT, dilX, dilY;
-    int kW, kH;
-    int ntiles_n, nblocks;
-    unsigned fill;          // padding byte replicated 4x (logical zero of the input)
-    unsigned out_xor;       // 0x80808080 when the output is stored as value-128
-    EpiArgs epi;
-};
 
 __device__ __forceinline__ int swz(int row, int q)
 {
@@ -506,7 +489,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -523,6 +506,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     std::vector<signed char> hw;
     std::vector<int4> hsub;
     std::vector<int> hwdw;
+    std::vector<signed char> hw4img;
     c->opad = round_up(d->O, 128);
     std::vector<int> hbias((size_t)std::max(c->opad, act->cpad), 0);
     const long long wstrideO = (long long)Cg * d->kH * d->kW;
@@ -635,6 +619,11 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
                 }
             }
         }
+        if (d->weight_bits == 4 && !c->pix4 && c->in_cs == d->C && d->C % 64 == 0 && c->ktot == d->kH * d->kW * d->C
+            && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PIPE)) {
+            hw4img.resize(conv_pipe_w4_image_bytes(c->opad, c->ktot));
+            conv_pipe_w4_image(full.data(), c->opad, c->ktot, hw4img.data());
+        }
         if (d->weight_bits == 4) {
             // nibble-pack per 16-weight sub-chunk: byte b of dword q holds weight 8q+b (low) and 8q+4+b (high)
             hw.assign(full.size() / 2, 0);
@@ -678,6 +667,10 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_wfrag, hfrag.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wfrag, hfrag.data(), hfrag.size(), hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess && !hw4img.empty()) {
+        e = hipMalloc((void**)&c->d_w4img, hw4img.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_w4img, hw4img.data(), hw4img.size(), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hwdw.empty()) {
         e = hipMalloc((void**)&c->d_wdw, hwdw.size() * sizeof(int));
         if (e == hipSuccess) e = hipMemcpy(c->d_wdw, hwdw.data(), hwdw.size() * sizeof(int), hipMemcpyHostToDevice);
@@ -716,6 +709,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_wstem) (void)hipFree(c->d_wstem);
     if (c->d_wfrag) (void)hipFree(c->d_wfrag);
     if (c->d_wdw) (void)hipFree(c->d_wdw);
+    if (c->d_w4img) (void)hipFree(c->d_w4img);
     delete c;
     return N2D2HIP_OK;
 }
@@ -727,6 +721,8 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
     const int opad_n = round_up(d.O, 64);
     *bn128 = opad_n % 128 == 0 || opad_n > 256;
     const int k = c->act->args.kind;
+    if (d.weight_bits == 4)     // packed weights: integer rescale only
+        return c->d_w4img != nullptr && d.kW * d.kH <= 31 && k == EPI_I24 && c->bias_folded;
     return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 31
         && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
 }
@@ -886,13 +882,13 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         // barrier waits overlap the other's MFMAs.  K advances by whole 128-byte lines when the channel count allows.
         // Layers with few pixels (deep stages) take 64-pixel tiles so that every CU still gets its two blocks.
         const long long tiles128 = ((Mll + 127) / 128) * a.ntiles_n;
-        const bool small_m = bn128 && d.C % 128 == 0
+        const bool small_m = bn128 && (w4 || d.C % 128 == 0)
             && ((d.kernel_choice & (N2D2HIP_KERNEL_TILE_M64 | N2D2HIP_KERNEL_TILE_M128)) ? (d.kernel_choice & N2D2HIP_KERNEL_TILE_M64) != 0
                                                                                             : tiles128 < (3 * num_cus()) / 2);
         // 64-channel layers whose K advances in 64-byte steps take 256-pixel tiles: twice the MFMAs per ring stage
-        const bool wide64 = !bn128 && !other && d.C % 128 != 0 && Mll >= 256ll * 4 * num_cus();
+        const bool wide64 = !w4 && !bn128 && !other && d.C % 128 != 0 && Mll >= 256ll * 4 * num_cus();
         // A handful of tiles (the classifier's FC): 64 x 64 tiles, four times as many blocks share the long K
-        const bool tiny = small_m && !other && ((Mll + 63) / 64) * a.ntiles_n * 8 < num_cus();
+        const bool tiny = !w4 && small_m && !other && ((Mll + 63) / 64) * a.ntiles_n * 8 < num_cus();
         if (tiny) a.ntiles_n = (round_up(d.O, 16) + 63) / 64;
         const int BMp = small_m ? 64 : wide64 ? 256 : 128;
         q.mtiles = (int)((Mll + BMp - 1) / BMp);
@@ -907,6 +903,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         // the multiply-add's result
         const bool hi16 = !other && c->hi16 && c->act->args.kind == EPI_I24 && is_byte_type(out->dtype) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
         if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
+        if (w4 && !other) {
+            // 4-bit weights, packed in memory and in LDS
+            q.c.w = c->d_w4img;
+            return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid == 1, hi16, grid, stream);
+        }
         if (other) {
             const int cp = c->sum->act->cpad;
             q.res = (const signed char*)other->data;
@@ -926,6 +927,10 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
                 if (c->sum16) { q.pre.c = c->d_res_tab + 12 * cp; q.pre.d = c->d_res_tab + 13 * cp; }
             }
             if (c->sum16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
+            if (w4) {
+                q.c.w = c->d_w4img;
+                return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid == 1, false, grid, stream);
+            }
             if (small_m) {
                 launch_pipe_res<4, 128, 2, 1, 2, 3>(q, grid, stream);
             } else if (d.C % 128 == 0) {
@@ -1024,13 +1029,13 @@ int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_inp
     const n2d2hip_act_s* ca = c->act;
     const n2d2hip_act_s* sa = sum->act;
     const n2d2hip_act_s* pa = sum->pre_input >= 0 ? sum->pre_act : nullptr;
-    const bool ok = pipe_eligible(c, &bn128) && one_by_one && round_up(d.O, 16) % (bn128 ? 128 : 64) == 0
+    const bool ok = pipe_eligible(c, &bn128) && (d.weight_bits == 4 || one_by_one) && d.dilX == 1 && d.dilY == 1 && round_up(d.O, 16) % (bn128 ? 128 : 64) == 0
         && ca->args.kind == EPI_I24 && ca->min_out >= -128 && ca->max_out <= 255
         && sum->nb_inputs == 2 && sum->unit_coeff && sa->args.kind == EPI_I24 && sa->min_out >= -128 && sa->max_out <= 255
         && (sum->pre_input < 0 || sum->pre_input == 1 - conv_input_index);
     N2D2HIP_REQUIRE(ok, N2D2HIP_ERR_UNSUPPORTED,
-                    "conv_fuse_sum: needs a 1x1 unpadded 8-bit convolution with a multiple of 64 input and output channels and integer "
-                    "rescales on the convolution and on a two-input unit-coefficient sum");
+                    "conv_fuse_sum: needs a 1x1 unpadded 8-bit convolution (or any undilated one with 4-bit weights) with a multiple of 64 "
+                    "input and output channels and integer rescales on the convolution and on a two-input unit-coefficient sum");
     // Tables of the sum (and of the ScalingCell folded onto the other input) with the other input's zero point
     // folded in: the kernel turns the stored byte into an unsigned one (U8B and I8 bytes with their top bit flipped,
     // which is the value itself for U8B and the value + 128 for I8) and adds that.

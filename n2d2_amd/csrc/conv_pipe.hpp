@@ -34,6 +34,8 @@
 // of its work fetch rows that are marked invalid.
 #pragma once
 
+#include "conv_args.hpp"
+#include "epilogue.hpp"
 #include "mfma_util.hpp"
 
 namespace n2d2hip {
@@ -84,7 +86,12 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // pack.  The host chooses it when it has shown that nothing overflows.
 // VALID: 0 = windows may reach outside the input (per-tap validity bits), 1 = 1x1 kernel without padding, 2 = any kernel
 // without padding (every tap of every window inside the input: a tap only moves the uniform base address).
-template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, int VALID, bool RES = false, bool P16 = false>
+// W4: 4-bit weights.  They stay packed two per byte in memory and in LDS (p.w is then an image of the ring's weight
+// tiles: per 32 channels and K step one 1 KB chunk, laid out as the LDS wants it) and are widened to bytes on their way
+// from LDS to the matrix core, as 16 times their value: the nibble becomes the upper half of its byte, which one AND
+// (upper nibbles) or a shift and an AND (lower nibbles) do for four weights at once.  The accumulators are divided by
+// 16, exactly, before they are rescaled.
+template <int NW, int BK, int NI, int NJ, int WGM, int EPI, int S, int VALID, bool RES = false, bool P16 = false, bool W4 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_pipe_kernel(ConvPipeArgs q)
 {
     const ConvArgs& p = q.c;
@@ -97,10 +104,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int KH = BK / 32;                        // MFMA K steps per stage
     constexpr int TOFF = 32 * BK;                      // LDS bytes between MFMA tiles of one operand
     // chunks each wave loads per step; when there are fewer chunks than waves some are loaded twice
-    constexpr int A_CH = BM / RPC, B_CH = BN / RPC;
+    constexpr int WROW = W4 ? BK / 2 : BK;             // bytes of a weight row per stage
+    constexpr int A_CH = BM / RPC, B_CH = W4 ? BN / 32 : BN / RPC;
     constexpr int A_J = (A_CH + NW - 1) / NW, B_J = (B_CH + NW - 1) / NW;
     constexpr int LPI = A_J + B_J;                     // loads per thread and step
-    constexpr int STAGE = (BM + BN) * BK;
+    constexpr int STAGE = BM * BK + BN * WROW;
+    static_assert(!W4 || BK == 64, "packed weights: 32 channels x 32 bytes per 1 KB chunk");
     constexpr int TAB_OFF = S * STAGE;                 // 6 int arrays of BN entries: bias, a, b, c, d, e
     // RES: + a..e of the sum cell, + a..e of the folded ScalingCell.  When the sum runs on 16-bit pairs, its c, d, e in
     // that form take the place of the bias and the convolution's a, which that path does not use.
@@ -112,6 +121,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     static_assert(WGM * WGN == NW && BM % RPC == 0 && BN % RPC == 0, "wave grid");
     static_assert(BK == 64 || (NW % 2 == 0 && A_CH % 2 == 0 && B_CH % 2 == 0), "a wave's chunks keep their parity");
     static_assert(S >= 2, "ring depth");
+    static_assert(!W4 || EPI == EPI_I24, "packed weights: integer rescale with the bias in its tables");
     static_assert(LPI * (S - 1) < 60, "vmcnt is a 6-bit counter");
     static_assert((NJ - 1) * TOFF < 65536 && NTAB * BN * 4 + 256 < 65536, "ds_read immediate offsets are 16 bits");
 
@@ -146,7 +156,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     unsigned woff[B_J];            // byte offset of this thread's weight rows (without the K offset)
 #pragma unroll
     for (int j = 0; j < B_J; ++j)
-        woff[j] = (unsigned)((n0 + ((wave + NW * j) % B_CH) * RPC + lrow) * p.ktot + lq * 16);
+        woff[j] = W4 ? (unsigned)(((n0 / 32 + (wave + NW * j) % B_CH) * p.niter) * 1024 + lane * 16)
+                     : (unsigned)((n0 + ((wave + NW * j) % B_CH) * RPC + lrow) * p.ktot + lq * 16);
     int rowoff[A_J];               // byte offset of the window origin of this thread's pixel rows (+ sub-chunk)
     unsigned rowmask[A_J];         // bit t < 31: kernel tap t of the row reads inside the input; bit 31: undilated window
     int l_tile = 0, l_it = 0, l_koff = 0, l_stage = 0;
@@ -211,7 +222,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
             }
         }
-        const signed char* wbase = p.w + l_koff;
+        const signed char* wbase = p.w + (W4 ? l_it * 1024 : l_koff);
 #pragma unroll
         for (int j = 0; j < B_J; ++j)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(wbase + woff[j]), (lds_ptr_t)(sbase + BM * BK + ((wave + NW * j) % B_CH) * 1024), 16, 0, 0);
@@ -240,7 +251,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int kk = 0; kk < KH; ++kk) {
         pa[kk] = lds0 + swz_k<BK>(wm * TM + l32, 2 * kk + lh);
-        wa[kk] = lds0 + BM * BK + swz_k<BK>(wn * TN + l32, 2 * kk + lh);
+        wa[kk] = W4 ? lds0 + BM * BK + (wn * TN + l32) * 32 + (((2 * kk + lh) ^ ((l32 >> 3) & 3)) << 3)
+                    : lds0 + BM * BK + swz_k<BK>(wn * TN + l32, 2 * kk + lh);
     }
     int r_stage = 0;
     const unsigned tab = lds0 + TAB_OFF + (unsigned)(wn * TN + 4 * lh) * 4u;      // this lane's first channel in the tables
@@ -250,11 +262,17 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
     // two fragment sets: while the MFMAs of K step g run from set g%2, the reads of step g+1 fly into the other
     v4i fw[2][NI], fp[2][NJ];
+    v2i fw4[2][W4 ? NI : 1];       // W4: the packed fragments as they come from LDS
     auto read_k = [&](auto kkc) {
         constexpr int kk = decltype(kkc)::value;
         constexpr int set = kk & 1;
-        lds_read128_nowait<0>(fw[set][0], wa[kk]);
-        if (NI > 1) lds_read128_nowait<TOFF>(fw[set][NI > 1 ? 1 : 0], wa[kk]);
+        if (W4) {
+            lds_read64_nowait<0>(fw4[set][0], wa[kk]);
+            if (NI > 1) lds_read64_nowait<1024>(fw4[set][W4 && NI > 1 ? 1 : 0], wa[kk]);
+        } else {
+            lds_read128_nowait<0>(fw[set][0], wa[kk]);
+            if (NI > 1) lds_read128_nowait<TOFF>(fw[set][NI > 1 ? 1 : 0], wa[kk]);
+        }
         lds_read128_nowait<0>(fp[set][0], pa[kk]);
         if (NJ > 1) lds_read128_nowait<TOFF>(fp[set][NJ > 1 ? 1 : 0], pa[kk]);
         if (NJ > 2) lds_read128_nowait<2 * TOFF>(fp[set][NJ > 2 ? 2 : 0], pa[kk]);
@@ -310,6 +328,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // ---- rescale, pack and store the finished tile
     auto epilogue = [&](int c_tile) {
         const int m0 = (mlane + c_tile * q.mlanes) * BM;
+        if (W4) {
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        acc[i][j][e] >>= 4;
+        }
         unsigned pk[NI][NJ][4];
         // RES: the other input's bytes, 4 channels per dword, are brought into the accumulators' layout by running the
         // output's lane-half exchanges backwards (the exchange is its own inverse).  Memory operations complete in
@@ -781,8 +808,20 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     constexpr int kk = decltype(kkc)::value;
                     constexpr int set = kk & 1;
                     wait_lgkm<0>();
+                    if (W4) {
 #pragma unroll
-                    for (int i = 0; i < NI; ++i) tie(fw[set][i]);
+                        for (int i = 0; i < NI; ++i) {
+                            tie(fw4[set][W4 ? i : 0]);
+                            const unsigned p0 = (unsigned)fw4[set][W4 ? i : 0][0], p1 = (unsigned)fw4[set][W4 ? i : 0][1];
+                            fw[set][i][0] = (int)((p0 << 4) & 0xf0f0f0f0u);
+                            fw[set][i][1] = (int)(p0 & 0xf0f0f0f0u);
+                            fw[set][i][2] = (int)((p1 << 4) & 0xf0f0f0f0u);
+                            fw[set][i][3] = (int)(p1 & 0xf0f0f0f0u);
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < NI; ++i) tie(fw[set][i]);
+                    }
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) tie(fp[set][j]);
                     if (kk == KH - 1) {
@@ -832,5 +871,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // no load may still be writing into LDS when the block's LDS is handed to another block
     asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
 }
+
+// 4-bit weights (conv_pipe_w4.hip).  tile: 0 = 128 pixels x 64 channels, 1 = 128 x 128, 2 = 64 x 128; `a.c.w` is the image
+// conv_pipe_w4_image() makes; hi16 selects the scaled-up tables.
+size_t conv_pipe_w4_image_bytes(int rows, int ktot);
+void conv_pipe_w4_image(const signed char* w, int rows, int ktot, signed char* image);
+// With a.res set, the residual sum behind the convolution is computed in the epilogue.
+int conv_pipe_w4_launch(ConvPipeArgs a, int tile, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream);
 
 } // namespace n2d2hip

@@ -1,0 +1,73 @@
+// The pipelined implicit-GEMM convolution for 4-bit weights: the instantiations of conv_pipe_kernel that keep the weights
+// packed two per byte in memory and in LDS, and the host side of that layout.
+#include "conv_pipe.hpp"
+
+namespace n2d2hip {
+
+size_t conv_pipe_w4_image_bytes(int rows, int ktot)
+{
+    return (size_t)rows * ktot / 2;
+}
+
+// `w` is [rows][ktot] int8 holding values in [-8, 7], rows a multiple of 32, ktot a multiple of 64.  The image is, per 32
+// rows and per 64 of K, one 1 KB chunk: row r at byte 32 r, its four groups of 16 weights at 8-byte slots
+// s ^ ((r >> 3) & 3) (so that the 32 rows one LDS read touches fall on different banks); in a slot, byte b of dword q
+// holds weight 8q + b in its lower and weight 8q + 4 + b in its upper nibble.
+void conv_pipe_w4_image(const signed char* w, int rows, int ktot, signed char* image)
+{
+    const int niter = ktot / 64;
+    for (int g = 0; g < rows / 32; ++g)
+        for (int it = 0; it < niter; ++it) {
+            signed char* chunk = image + ((size_t)g * niter + it) * 1024;
+            for (int r = 0; r < 32; ++r) {
+                const signed char* src = w + (size_t)(g * 32 + r) * ktot + it * 64;
+                for (int s = 0; s < 4; ++s)
+                    for (int q = 0; q < 2; ++q)
+                        for (int b = 0; b < 4; ++b) {
+                            const int lo = src[s * 16 + 8 * q + b] & 15, hi = src[s * 16 + 8 * q + 4 + b] & 15;
+                            chunk[r * 32 + ((s ^ ((r >> 3) & 3)) << 3) + 4 * q + b] = (signed char)(lo | (hi << 4));
+                        }
+            }
+        }
+}
+
+namespace {
+
+template <int NI, int NJ, int WGM>
+void launch(ConvPipeArgs a, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream)
+{
+    constexpr int NW = 4, BK = 64, S = 4;
+    a.c.niter = a.c.ktot / BK;
+    a.cper = a.c.in_cs / BK;
+    if (a.res) {
+        // residual sum in the epilogue; 16-bit pairs when the host has shown that they hold every intermediate
+        if (one_by_one_unpadded) {
+            if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+            else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        } else {
+            if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+            else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        }
+    } else if (one_by_one_unpadded) {
+        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+    } else {
+        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+    }
+}
+
+} // namespace
+
+int conv_pipe_w4_launch(ConvPipeArgs a, int tile, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream)
+{
+    N2D2HIP_REQUIRE(a.c.epi.kind == EPI_I24 && a.c.ktot % 64 == 0 && a.c.in_cs % 64 == 0, N2D2HIP_ERR_INVALID,
+                    "conv_pipe_w4: integer rescale and a multiple of 64 channels expected");
+    if (tile == 0) launch<2, 1, 4>(a, one_by_one_unpadded, hi16, grid, stream);
+    else if (tile == 1) launch<2, 2, 2>(a, one_by_one_unpadded, hi16, grid, stream);
+    else launch<2, 1, 2>(a, one_by_one_unpadded, hi16, grid, stream);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+} // namespace n2d2hip

@@ -278,6 +278,39 @@ def test_conv_int4_weights_uint4_activations(rt):
         assert np.array_equal(conv8.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), got)
 
 
+def test_conv_int4_weights_pipelined_kernel_tiles(rt):
+    """4-bit weights on the pipelined kernel (packed in memory and in LDS, widened on the way to the matrix core): each of
+    its three tile shapes, with the plain and the scaled-up rescale tables, a strided 1x1 and weights at both ends of
+    the 4-bit range ([-8, 7]), against the oracle and against the general kernel."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    from oracle.cells import ActSpec
+    cases = ((3, 64, 64, 3, 1, 1, 30, 0), (3, 128, 128, 3, 1, 1, 19, capi.KERNEL_TILE_M128), (3, 128, 128, 3, 1, 1, 19, capi.KERNEL_TILE_M64),
+             (2, 256, 192, 1, 2, 0, 15, capi.KERNEL_TILE_M128 | capi.KERNEL_NO_HI16), (2, 64, 200, 3, 2, 1, 23, capi.KERNEL_TILE_M64),
+             (1, 192, 64, 1, 1, 0, 9, capi.KERNEL_NO_HI16))
+    for (B, Cc, O, k, s, p, H, choice) in cases:
+        x = RNG.integers(0, 16, size=(B, Cc, H, H + 3)).astype(np.int32)
+        w = RNG.integers(-8, 8, size=(O, Cc, k, k)).astype(np.int32)
+        bias = RNG.integers(-300, 301, size=O).astype(np.int32)
+        spec = ActSpec("Rectifier", "FixedMult32", RNG.integers(300, 900, size=O), frac_bits=16,
+                       clipping=RNG.uniform(500.0, 3000.0, size=O).astype(np.float32), nb_bits=4, unsigned_out=True)
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(s, s), pad=(p, p, p, p))
+        xd = rt.DTensor.from_numpy(x, capi.U8B)
+        got = {}
+        for ch in (choice, capi.KERNEL_NO_PIPE):
+            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(s, s), pad=(p, p, p, p), weight_bits=4, kernel_choice=ch)
+            got[ch] = conv.forward(xd).to_numpy()
+        assert np.array_equal(got[choice], want.astype(np.int64)), (B, Cc, O, k, s, p, H, choice)
+        assert np.array_equal(got[capi.KERNEL_NO_PIPE], got[choice])
+    # full-range 8-bit activations and an unclipped rescale (the accumulators are 16 times the sums before they are divided)
+    x = _u8((2, 128, 12, 12))
+    w = RNG.integers(-8, 8, size=(128, 128, 3, 3)).astype(np.int32)
+    spec = ActSpec("Rectifier", "SingleShift", RNG.integers(7, 11, size=128), nb_bits=8, unsigned_out=True)
+    want = cells_ref.conv_cell(x, w, None, spec, pad=(1, 1, 1, 1))
+    conv = rt.Conv(w, None, rt.Act(128, **spec.kwargs()), capi.U8B, pad=(1, 1, 1, 1), weight_bits=4)
+    assert np.array_equal(conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), want.astype(np.int64))
+
+
 def test_conv_linearity_and_batch_independence_at_full_width(rt):
     """Size-independent properties at a ResNet-50 layer shape (1x1, 256->64 on 56x56, batch 16): raw sums are additive in
     the weights, and an image's result does not depend on its position in the batch."""
