@@ -1621,4 +1621,36 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
     return deepNet;
 }
 
+// Every output of block g = o / (O / G) must see exactly the channels [g L, (g + 1) L), L being the number of leading
+// channels the first output sees.
+std::size_t Cell::getNbGroups(const Tensor<bool>& map)
+{
+    const std::size_t nbOutputs = map.dimX(), nbChannels = map.dimY();
+    std::size_t width = 0;
+    while (width < nbChannels && map.at(0, width))
+        ++width;
+    if (width == 0)
+        return 0;
+    const std::size_t groups = nbChannels / width;
+    bool regular = nbChannels % width == 0 && nbOutputs % groups == 0;
+    const std::size_t perGroup = regular ? nbOutputs / groups : 1;
+    for (std::size_t o = 0; regular && o < nbOutputs; ++o)
+        for (std::size_t ch = 0; regular && ch < nbChannels; ++ch)
+            regular = map.at(o, ch) == (ch / width == o / perGroup);
+    if (!regular)
+        throw std::runtime_error("Cell::getNbGroups(): the connection map is not a set of equal groups; Frame_HIP cells have no "
+                                 "connection-by-connection path");
+    return groups;
+}
+
+void ConvCell::setMapping(const Tensor<bool>& map)
+{
+    if (map.dimX() != mNbOutputs || (mNbChannels != 0 && map.dimY() != mNbChannels))
+        throw std::runtime_error("ConvCell::setMapping(): the map of " + mName + " must be {nbOutputs, nbChannels}");
+    const std::size_t groups = getNbGroups(map);
+    if (groups == 0)
+        throw std::runtime_error("ConvCell::setMapping(): the first output of " + mName + " is not connected");
+    setNbGroups((unsigned int)groups);
+}
+
 } // namespace N2D2

@@ -108,6 +108,9 @@ public:
     const T& operator()(size_t x, size_t y, size_t z, size_t b) const { return mData[x + mDims[0] * (y + mDims[1] * (z + mDims[2] * b))]; }
     T* data() { return mData.data(); }
     const T* data() const { return mData.data(); }
+    // by value: also usable where T is bool
+    T at(size_t x, size_t y) const { return mData[x + mDims[0] * y]; }
+    void set(size_t x, size_t y, T v) { mData[x + mDims[0] * y] = v; }
     void fill(T v) { std::fill(mData.begin(), mData.end(), v); }
 
 private:
@@ -350,6 +353,11 @@ public:
     }
     // Cell::getOutputsRangeParents, src/Cell/Cell.cpp:310-337
     std::pair<double, double> getOutputsRangeParents() const;
+    // Number of groups of a connection map {outputs, channels} (Cell::getNbGroups, src/Cell/Cell.cpp:251-300): G when the map
+    // is G equal blocks on the diagonal (output o of block g sees exactly the channels of block g), 0 when the first output
+    // sees no leading channel.  Any other map is what the reference counts by hand (src/Cell/Cell.cpp:176-249) and its
+    // Frame cells then evaluate connection by connection; the Frame_HIP kernels have no such path and this throws.
+    static std::size_t getNbGroups(const Tensor<bool>& map);
     const std::shared_ptr<Activation>& getActivation() const { return mActivation; }
     void setActivation(const std::shared_ptr<Activation>& activation) { mActivation = activation; }
     // Free parameters as text files, "<base>_weights<.ext>" and "<base>_biases<.ext>" (or one file holding both), the
@@ -459,6 +467,8 @@ public:
     void setParameter(const std::string& name, bool value);
     // Depthwise / grouped connection: the regular mapping Cell::getNbGroups recognises (src/Cell/Cell.cpp:251-300).
     void setNbGroups(unsigned int groups) { mNbGroups = groups; mDirty = true; }
+    // The same from the connection map itself, {nbOutputs, nbChannels} (what Mapping.* sections of an INI expand to)
+    void setMapping(const Tensor<bool>& map);
     // Weights as N2D2 holds them: float tensor {kW, kH, C/groups, O} with integer values; bias {O}.
     void setWeights(const Tensor<Float_T>& weights) { mWeights = weights; mDirty = true; }
     void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }

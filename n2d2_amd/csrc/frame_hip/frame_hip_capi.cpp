@@ -167,6 +167,31 @@ int fh_cell_set_weights(void* net, const char* name, const float* w, size_t n, i
     });
 }
 
+// map[o + nbOutputs * c] != 0: output o sees channel c
+int fh_get_nb_groups(const unsigned char* map, size_t nbOutputs, size_t nbChannels, long* groups)
+{
+    return guarded([&] {
+        Tensor<bool> m({nbOutputs, nbChannels}, false);
+        for (size_t c = 0; c < nbChannels; ++c)
+            for (size_t o = 0; o < nbOutputs; ++o)
+                m.set(o, c, map[o + nbOutputs * c] != 0);
+        *groups = (long)Cell::getNbGroups(m);
+    });
+}
+
+int fh_cell_set_mapping(void* net, const char* name, const unsigned char* map, size_t nbOutputs, size_t nbChannels)
+{
+    return guarded([&] {
+        auto conv = std::dynamic_pointer_cast<ConvCell>(((Net*)net)->deepNet->getCell(name));
+        if (!conv) throw std::runtime_error("fh_cell_set_mapping(): " + std::string(name) + " is not a Conv");
+        Tensor<bool> m({nbOutputs, nbChannels}, false);
+        for (size_t c = 0; c < nbChannels; ++c)
+            for (size_t o = 0; o < nbOutputs; ++o)
+                m.set(o, c, map[o + nbOutputs * c] != 0);
+        conv->setMapping(m);
+    });
+}
+
 int fh_cell_set_biases(void* net, const char* name, const float* b, size_t n)
 {
     return guarded([&] {

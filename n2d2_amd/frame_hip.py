@@ -26,6 +26,8 @@ lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c
 lib.fh_cell_set_quantized.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int]
 lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+lib.fh_get_nb_groups.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+lib.fh_cell_set_mapping.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_size_t]
 lib.fh_cell_set_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
 lib.fh_cell_get_outputs.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
 lib.fh_cell_get_max_output.argtypes = [C.c_void_p, C.c_char_p, C.c_uint, C.c_void_p]
@@ -97,6 +99,15 @@ def approximate_scaling_with_power_of_2_divs(scaling, nb_divisions):
     return [int(e) for e in exps], precision.value
 
 
+def get_nb_groups(mapping):
+    """Cell::getNbGroups of a connection map [nbOutputs, nbChannels] (non-zero: connected).  Raises FrameHipError for a
+    map that is not a set of equal groups."""
+    m = np.asfortranarray(np.asarray(mapping) != 0, dtype=np.uint8)      # element (o, c) at o + nbOutputs * c
+    groups = C.c_long()
+    _check(lib.fh_get_nb_groups(m.ctypes.data, m.shape[0], m.shape[1], C.byref(groups)))
+    return groups.value
+
+
 class Net:
     def __init__(self, ini_text):
         self.h = lib.fh_net_from_ini(ini_text.encode())
@@ -134,6 +145,11 @@ class Net:
         else:
             O, Cg, kH, kW = a.shape[0], a.shape[1], 1, 1
         _check(lib.fh_cell_set_weights(self.h, name.encode(), a.ctypes.data, a.size, kW, kH, Cg, O, int(weight_bits)))
+
+    def set_mapping(self, name, mapping):
+        """ConvCell::setMapping: the connection map [nbOutputs, nbChannels] decides the number of groups."""
+        m = np.asfortranarray(np.asarray(mapping) != 0, dtype=np.uint8)
+        _check(lib.fh_cell_set_mapping(self.h, name.encode(), m.ctypes.data, m.shape[0], m.shape[1]))
 
     def set_biases(self, name, b):
         a = np.ascontiguousarray(b, dtype=np.float32)
@@ -320,6 +336,12 @@ def spec_to_ini(spec, batch, model="Frame_HIP"):
 def build_net(spec, batch, model="Frame_HIP"):
     """Instantiates a nets.NetSpec on the C++ Frame_HIP cells: INI -> Registrar -> cells, then parameters."""
     net = Net(spec_to_ini(spec, batch, model))
+    install_parameters(net, spec)
+    return net
+
+
+def install_parameters(net, spec):
+    """Weights, biases, quantization flags and rescales of a nets.NetSpec, as N2D2's quantization pass leaves them."""
     for l in spec.layers:
         if l.type in ("conv", "fc"):
             net.set_weights(l.name, l.w, getattr(l, "weight_bits", 8))

@@ -293,3 +293,65 @@ def test_replace_input_rewires_a_cell_as_cell_frame_does(fh):
     assert net.cell_info("sum")["W"] == 7                   # and the failed call leaves the cell as it was
     net.replace_input("dw", "sum", "conv1")                 # a single-input cell follows its new input's size
     assert (net.cell_info("dw")["W"], net.cell_info("dw")["H"]) == (16, 16)
+
+
+def test_get_nb_groups_from_a_connection_map_against_the_oracle(fh):
+    """Cell::getNbGroups (src/Cell/Cell.cpp:251-300) in the cell layer: equal diagonal blocks give their count, an
+    unconnected first output gives 0, and every map the reference would count by hand is an error; the oracle's
+    restatement of the same function says -1 exactly there."""
+    import numpy as np
+    from oracle import oracle as orc
+    rng = np.random.default_rng(5)
+
+    def block_map(O, Cn, G):
+        m = np.zeros((O, Cn), dtype=np.uint8)
+        for g in range(G):
+            m[g * (O // G):(g + 1) * (O // G), g * (Cn // G):(g + 1) * (Cn // G)] = 1
+        return m
+
+    for (O, Cn, G) in ((8, 8, 8), (12, 6, 3), (6, 12, 2), (5, 7, 1), (64, 64, 64), (16, 4, 4), (4, 16, 4)):
+        m = block_map(O, Cn, G)
+        assert fh.get_nb_groups(m) == G == orc.get_nb_groups(m)
+        # any single flipped connection makes it irregular (or moves the first run, which must break a later row)
+        for _ in range(6):
+            o, c = int(rng.integers(0, O)), int(rng.integers(0, Cn))
+            bad = m.copy()
+            bad[o, c] ^= 1
+            want = orc.get_nb_groups(bad)
+            if want == -1:
+                with pytest.raises(fh.FrameHipError, match="not a set of equal groups"):
+                    fh.get_nb_groups(bad)
+            else:
+                assert fh.get_nb_groups(bad) == want
+    # random maps: whatever the oracle says, the cell layer says (error for -1)
+    for _ in range(200):
+        O, Cn = int(rng.integers(1, 7)), int(rng.integers(1, 7))
+        m = (rng.random((O, Cn)) < 0.6).astype(np.uint8)
+        want = orc.get_nb_groups(m)
+        if want == -1:
+            with pytest.raises(fh.FrameHipError):
+                fh.get_nb_groups(m)
+        else:
+            assert fh.get_nb_groups(m) == want
+    assert fh.get_nb_groups(np.zeros((4, 6), dtype=np.uint8)) == 0
+    # unequal blocks: the reference's hand count would say 2, its regular test fails, ours raises
+    uneven = np.zeros((4, 4), dtype=np.uint8)
+    uneven[0:1, 0:1] = 1
+    uneven[1:4, 1:4] = 1
+    assert orc.get_nb_groups(uneven) == -1
+    with pytest.raises(fh.FrameHipError):
+        fh.get_nb_groups(uneven)
+
+
+def test_conv_mapping_sets_the_groups(fh):
+    import numpy as np
+    net = fh.Net((INI % "Frame_HIP"))
+    info = net.cell_info("conv1")
+    O, Cn = 16, 3
+    with pytest.raises(fh.FrameHipError, match="not a set of equal groups"):
+        net.set_mapping("conv1", np.tri(O, Cn))
+    with pytest.raises(fh.FrameHipError, match="must be"):
+        net.set_mapping("conv1", np.ones((O + 1, Cn)))
+    net.set_mapping("conv1", np.ones((O, Cn)))          # fully connected: one group
+    with pytest.raises(fh.FrameHipError, match="not a Conv"):
+        net.set_mapping("pool1", np.ones((16, 16)))

@@ -102,6 +102,27 @@ def test_mobilenet_and_w4a4_through_the_registrar(fh):
     _compare(fh, nets.resnet18_w4a4(), x, ["conv2.1_a", "conv2.1_sum", "conv5.2_sum", "fc"])
 
 
+def test_depthwise_cell_from_its_connection_map(fh):
+    """The number of groups comes from the connection map (Cell::getNbGroups): MobileNet's first blocks built from an INI
+    without any Mapping.* key, the depthwise cells given an identity map, against the oracle."""
+    from n2d2_amd import nets
+    from oracle import cells
+    spec = nets.mobilenet_v1(image=64)
+    x = np.random.default_rng(35).integers(0, 256, size=(2, 3, 64, 64))
+    ini = "\n".join(line for line in fh.spec_to_ini(spec, 2).split("\n") if not line.startswith("Mapping."))
+    net = fh.Net(ini)
+    for l in spec.layers:
+        if l.type == "conv" and l.groups > 1:
+            net.set_mapping(l.name, np.eye(l.groups))
+    fh.install_parameters(net, spec)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    want = cells.run_net(spec, x, keep=["conv2_dw", "conv7_dw", "fc"])
+    for name in ("conv2_dw", "conv7_dw", "fc"):
+        assert np.array_equal(net.outputs(name), want[name]), name
+
+
 def test_signedness_change_rebuilds_the_cells(fh):
     """-no-unsigned (DeepNetExport::mUnsignedData = false): every cell saturates to the signed range."""
     from n2d2_amd import nets

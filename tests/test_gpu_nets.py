@@ -128,6 +128,40 @@ def test_resnet50_full_batch_properties():
                 assert np.array_equal(net.tensors[n].to_numpy(), ref[n]), (it, n)
 
 
+@pytest.mark.parametrize("config", ["mobilenet_v1", "resnet18_w4a4"])
+def test_batch64_configs_full_batch_properties(config):
+    """MobileNet-v1 and ResNet-18 W4A4 at their benchmark size (batch 64): the oracle checks a slice, batch independence
+    covers the rest (repeated images give identical logits wherever they sit), and a graph replay reproduces the launches
+    tensor by tensor on a layer of each kind."""
+    from n2d2_amd import nets
+    from oracle import cells
+    spec = getattr(nets, config)()
+    B = 64
+    rng = np.random.default_rng(16)
+    base = rng.integers(0, 256, size=(6, 3, 224, 224))
+    idx = rng.integers(0, 6, size=B)
+    idx[:6] = np.arange(6)
+    x = base[idx]
+    net = nets.GpuNet(spec, B)
+    net.set_input(x)
+    logits = net.forward().to_numpy()[:, :, 0, 0]
+    for i in range(B):
+        assert np.array_equal(logits[i], logits[idx[i]]), i
+    assert len({logits[i].tobytes() for i in range(6)}) == 6
+    want = cells.run_net(spec, base[:2])["fc"].astype(np.int64)[:, :, 0, 0]
+    assert np.array_equal(logits[:2], want)
+    watch = {"mobilenet_v1": ["conv1", "conv2_dw", "conv2_pw", "conv7_dw", "conv14_pw", "pool", "fc"],
+             "resnet18_w4a4": ["conv1", "pool1", "conv2.1_a", "conv2.1_sum", "conv3.1_sum", "conv5.2_sum", "pool", "fc"]}[config]
+    watch = [n for n in watch if n not in net.folded]
+    ref = {n: net.tensors[n].to_numpy() for n in watch}
+    replay = net.capture()
+    for it in range(6):
+        (net.forward if it % 2 else replay)()
+        if it % 3 == 2:
+            for n in watch:
+                assert np.array_equal(net.tensors[n].to_numpy(), ref[n]), (it, n)
+
+
 def test_two_forwards_on_two_streams_agree_with_sequential_runs():
     """Handles are independent: two networks launched on two streams at once (the benchmark's two-batches-in-flight mode)
     give the bytes each gives alone."""
