@@ -21,7 +21,9 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
 # inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
 TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
-                        "bytes_per_launch": None}
+                        "bytes_per_launch": 71948672,
+                        "note": "FETCH_SIZE + WRITE_SIZE, mean over the conv_pipe_kernel dispatches of 4 forwards, scaled by a 1 GiB copy; "
+                                "not measured by this run"}
 
 
 def cpu_baseline(spec, gpu_logits, images, budget_s=15.0):
@@ -232,15 +234,24 @@ def qat_batchnorm_step(torch, steps=10):
             "finite": bool(torch.isfinite(y).all().item() and torch.isfinite(dx).all().item())}
 
 
+# name -> (constructor in n2d2_amd.nets, benchmark batch)
+CONFIGS = {"resnet50": ("resnet50", 128), "lenet": ("lenet", 256), "resnet18_stage_conv": ("single_conv_stage", 64),
+           "mobilenet_v1": ("mobilenet_v1", 64), "resnet18_w4a4": ("resnet18_w4a4", 64)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=0, help="images per step (default: the configuration's own, 128 for the headline)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="only the headline workload")
     ap.add_argument("--no-graph", action="store_true", help="time cell-by-cell launches instead of a HIP graph replay")
+    ap.add_argument("--forward-only", action="store_true",
+                    help="profiling runs: time the forward of --config and stop (no per-kernel replays, no side figures)")
+    ap.add_argument("--config", default="resnet50", choices=sorted(CONFIGS),
+                    help="with --forward-only: which configuration's forward to run (at its benchmark batch unless --batch is given)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 1 GiB device-to-device copy first (known traffic, to scale FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -262,8 +273,20 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.forward_only:
+        make, batch = CONFIGS[args.config]
+        spec = getattr(nets, make)()
+        B = args.batch or batch
+        net = nets.GpuNet(spec, B)
+        net.set_input(np.random.default_rng(2025).integers(0, 256, size=(B,) + tuple(spec.in_shape)))
+        step = net.forward if args.no_graph else net.capture()
+        ms, mean_ms, wall_ms = median_step_ms(torch, step, args.steps, args.warmup)
+        print(json.dumps({"forward_only": args.config, "batch": B, "value": round(B / (ms * 1e-3), 1), "unit": "images/s",
+                          "ms_per_step": round(ms, 4), "launches_per_step": len(net.launched),
+                          "launch": "eager" if args.no_graph else "hipGraph replay", "steps": args.steps, "warmup": args.warmup}))
+        return
     spec = nets.resnet50()
-    B = args.batch
+    B = args.batch or 128
     net = nets.GpuNet(spec, B)
     rng = np.random.default_rng(2025)
     images = rng.integers(0, 256, size=(B, 3, 224, 224))
