@@ -21,7 +21,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
 # inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
 TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
-                        "bytes_per_launch": 71948672,
+                        "bytes_per_launch": 71948672, "launches_per_forward": 41,
                         "note": "FETCH_SIZE + WRITE_SIZE, mean over the conv_pipe_kernel dispatches of 4 forwards, scaled by a 1 GiB copy; "
                                 "not measured by this run"}
 
@@ -359,10 +359,14 @@ def main():
     conv_ms = replay_alone(pipe)
     conv_ops = 2.0 * sum(net.layer_macs(net.launched[k]) for k in pipe)
     achieved = conv_ops / (conv_ms * 1e-3) / 1e12
+    profile_applies = B == TRAFFIC_FROM_PROFILE["batch"] and len(pipe) == TRAFFIC_FROM_PROFILE["launches_per_forward"]
     roofline = {"bound": "mfma", "kernel": "conv_pipe_kernel (%d launches of one forward: conv/fc cells with a multiple of 64 input "
                 "channels, residual sums folded in; not the cells of the fused bottleneck nor the 3x3 layers on the patch kernel)" % len(pipe),
                 "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
-                "traffic": None, "traffic_from_profile": TRAFFIC_FROM_PROFILE if B == 128 else None,
+                # HBM bytes per launch cannot be counted from inside this process: the figure is the one the committed profile
+                # holds, given only while this run launches what that profile covered (same batch, same number of launches)
+                "traffic": TRAFFIC_FROM_PROFILE["bytes_per_launch"] if profile_applies else None,
+                "traffic_from_profile": TRAFFIC_FROM_PROFILE if profile_applies else None,
                 "algorithmic_bytes_per_launch": round(sum(net.layer_bytes(net.launched[k]) for k in pipe) / len(pipe)),
                 "launches_per_step": len(pipe), "avg_launch_us": round(conv_ms * 1000.0 / len(pipe), 2),
                 "ops_per_launch": conv_ops / len(pipe), "frac_of_peak_at_measured_clock": round(achieved / clock["int8_peak_at_that_clock_tops"], 4)}
