@@ -176,8 +176,14 @@ int n2d2hip_act_create(const n2d2hip_activation* desc, int nb_channels, n2d2hip_
                     "act_create: bad activation kind %d", desc->kind);
     N2D2HIP_REQUIRE(desc->scaling_mode >= N2D2HIP_SCALING_NONE && desc->scaling_mode <= N2D2HIP_SCALING_DOUBLE_SHIFT,
                     N2D2HIP_ERR_INVALID, "act_create: Unsupported scaling propagation (mode %d)", desc->scaling_mode);
-    N2D2HIP_REQUIRE(!(desc->kind == N2D2HIP_ACT_RECTIFIER && desc->leak_slope != 0.0f), N2D2HIP_ERR_UNSUPPORTED,
-                    "act_create: Rectifier LeakSlope %g gives non-integer outputs; only 0 is supported on the integer path",
+    // The reference rescales and saturates first and multiplies what is left below zero by the slope, in float
+    // (ref: include/Activation/RectifierActivation_Frame.hpp:66-82).  Behind a rescale that saturates to an unsigned range
+    // nothing is left below zero and the slope does nothing; anywhere else the products are not integers.
+    N2D2HIP_REQUIRE(!(desc->kind == N2D2HIP_ACT_RECTIFIER && desc->leak_slope != 0.0f)
+                        || (desc->unsigned_out && desc->scaling_mode != N2D2HIP_SCALING_NONE),
+                    N2D2HIP_ERR_UNSUPPORTED,
+                    "act_create: Rectifier LeakSlope %g gives non-integer outputs on a cell with signed or un-rescaled outputs; the integer "
+                    "path takes it only where the rescale saturates to an unsigned range (where it changes nothing)",
                     (double)desc->leak_slope);
     const int mode = desc->scaling_mode;
     const bool relu = desc->kind == N2D2HIP_ACT_RECTIFIER;

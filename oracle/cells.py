@@ -9,13 +9,18 @@ from . import oracle as orc
 class ActSpec:
     """Host description of a cell's activation (kind, Scaling, bits, signedness)."""
 
-    def __init__(self, kind="Linear", mode="None", scaling=None, frac_bits=0, clipping=None, nb_bits=8, unsigned_out=False):
+    def __init__(self, kind="Linear", mode="None", scaling=None, frac_bits=0, clipping=None, nb_bits=8, unsigned_out=False,
+                 leak_slope=0.0):
         self.kind, self.mode, self.scaling, self.frac_bits = kind, mode, scaling, frac_bits
         self.clipping, self.nb_bits, self.unsigned_out = clipping, nb_bits, unsigned_out
+        self.leak_slope = leak_slope
 
     def kwargs(self):
-        return dict(kind=self.kind, mode=self.mode, scaling=self.scaling, frac_bits=self.frac_bits,
-                    clipping=self.clipping, nb_bits=self.nb_bits, unsigned_out=self.unsigned_out)
+        kw = dict(kind=self.kind, mode=self.mode, scaling=self.scaling, frac_bits=self.frac_bits,
+                  clipping=self.clipping, nb_bits=self.nb_bits, unsigned_out=self.unsigned_out)
+        if self.leak_slope:
+            kw["leak_slope"] = self.leak_slope
+        return kw
 
     def apply(self, x):
         """Scaling::propagate dispatch (include/Scaling.hpp:434-459) then the activation pass."""
@@ -33,7 +38,7 @@ class ActSpec:
         else:
             raise ValueError(self.mode)
         if self.kind == "Rectifier":
-            y = orc.rectifier(y)
+            y = orc.rectifier(y, leak=self.leak_slope)
         else:
             y = orc.linear(y)
         return y

@@ -121,8 +121,17 @@ def test_error_behaviour_matches_reference(rt):
     with pytest.raises(capi.N2D2HipError) as e:
         rt.Act(4, "Linear", "SingleShift", [1, 1, 1, 1], nb_bits=0)
     assert e.value.status == capi.ERR_NOT_QUANTIZED and "can only be used on quantized network" in str(e.value)
-    with pytest.raises(capi.N2D2HipError):
+    # a leaky Rectifier gives non-integers below zero on signed or un-rescaled cells ...
+    with pytest.raises(capi.N2D2HipError, match="non-integer"):
         rt.Act(4, "Rectifier", "SingleShift", [1, 1, 1, 1], leak_slope=0.1)
+    with pytest.raises(capi.N2D2HipError, match="non-integer"):
+        rt.Act(4, "Rectifier", "None", None, leak_slope=0.1, unsigned_out=True)
+    # ... and changes nothing behind a rescale that saturates to an unsigned range, as in the reference
+    from oracle.cells import ActSpec
+    leaky = ActSpec("Rectifier", "SingleShift", np.array([1, 2, 3, 4]), nb_bits=8, unsigned_out=True, leak_slope=0.1)
+    xl = RNG.integers(-3000, 3000, size=(2, 4, 3, 3)).astype(np.int32)
+    got = rt.scaling_forward(rt.Act(4, **leaky.kwargs()), rt.DTensor.from_numpy(xl, capi.I32)).to_numpy()
+    assert np.array_equal(got, leaky.apply(xl.astype(np.float32)).astype(np.int64)) and got.min() == 0
     act = rt.Act(4, "Linear", "SingleShift", [1, 1, 1, 1], nb_bits=8, unsigned_out=False)
     x = rt.DTensor.from_numpy(_u8((1, 5, 2, 2)), capi.I32)
     with pytest.raises(capi.N2D2HipError):            # channel mismatch: nothing is written
