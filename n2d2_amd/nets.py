@@ -356,7 +356,7 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection"):
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -364,7 +364,10 @@ class GpuNet:
         kernel_choice: capi.KERNEL_* bits handed to every convolution (which kernel runs, never what it computes).
         bottlenecks: run a residual block 1x1 -> 3x3 -> 1x1 + sum (+ projection) whose cells qualify as one launch
         (n2d2hip_bottleneck_*); its input tensor then carries a border of one pixel.  True / "all", "projection" (only the
-        blocks with a projection shortcut, where one launch replaces four), or False."""
+        blocks with a projection shortcut, where one launch replaces four), or False.
+        tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
+        (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
+        only ties with the two separate launches."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
         consumers = {}
@@ -465,14 +468,44 @@ class GpuNet:
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
             self._plan_bottlenecks(consumers, by_name, ins_of)
+        # reducing 1x1 convolutions computed by the launch that produces their input (their tensors are written all the same)
+        self.absorbed, self.tail_layers = set(), {}
+        if fuse and tails:
+            self._plan_tails(consumers, ins_of)
         self._io = [(ins_of[l.name], self.tensors[l.name]) for l in spec.layers]
         # folded ScalingCells are not launched and their output is never materialised
         for name in self.folded:
             del self.tensors[name]
-        keep = [k for k, l in enumerate(spec.layers) if l.name not in self.folded]
+        keep = [k for k, l in enumerate(spec.layers) if l.name not in self.folded and l.name not in self.absorbed]
         self.steps = [self.steps[k] for k in keep]
         self._io = [self._io[k] for k in keep]
         self.launched = [spec.layers[k] for k in keep]
+
+    def _plan_tails(self, consumers, ins_of):
+        """For every sum folded into the expanding 1x1 convolution of a block: if a reducing 1x1 convolution (the next
+        block's first cell) reads that sum, both run as one launch where the library takes them
+        (n2d2hip_expand_reduce_create): the launch writes the sum and the reduction's output."""
+        step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+        for sum_name, (sum_cell, expand) in list(self.fused_sums.items()):
+            if sum_name in self.bottlenecks:
+                continue
+            k = step_index[sum_name]
+            expand_cell = self.steps[k][1]
+            x, other = ins_of[sum_name]
+            y = self.tensors[sum_name]
+            if x.halo or other.halo or y.halo:
+                continue
+            for r in consumers.get(sum_name, []):
+                if r.type != "conv" or r.name in self.folded or r.name in self.absorbed or r.w.shape[2:] != (1, 1):
+                    continue
+                fused = self.rt.ExpandReduce.create(expand_cell, self.steps[step_index[r.name]][1])
+                if fused is None:
+                    continue
+                z = self.tensors[r.name]
+                self.steps[k] = (self.steps[k][0], fused, (lambda c, i, o, z=z: c.forward(i[0], i[1], o, z)))
+                self.absorbed.add(r.name)
+                self.tail_layers[sum_name] = r
+                break
 
     def _plan_bottlenecks(self, consumers, by_name, ins_of):
         """For every sum folded into a 1x1 convolution: reduce -> 3x3 -> expand (+ projection) as one launch, if the
@@ -625,13 +658,18 @@ class GpuNet:
             total += sum(m.w.size for m in self.bottleneck_layers[l.name])
         elif l.name in self.fused_sums:
             total += self.fused_sums[l.name][1].w.size
+        if l.name in self.tail_layers:      # the reduction's weights and output; its input never leaves the chip
+            r = self.tail_layers[l.name]
+            z = self.tensors[r.name]
+            total += r.w.size + z.B * z.C * z.H * z.W
         return total
 
     def layer_macs(self, l):
         if l.name in self.bottleneck_layers:
             return sum(self.B * m.out_shape[1] * m.out_shape[2] * m.w.size for m in self.bottleneck_layers[l.name])
         if l.name in self.fused_sums:
-            return self.layer_macs(self.fused_sums[l.name][1])
+            tail = self.tail_layers.get(l.name)
+            return self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
         if l.type == "conv":
             return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
         if l.type == "fc":
@@ -640,14 +678,4 @@ class GpuNet:
 
     def activation_bytes(self):
         """Algorithmic HBM bytes of one forward: every cell reads its inputs and writes its output once, plus weights."""
-        total = 0
-        for l, (ins, out) in zip(self.launched, self._io):
-            total += sum(t.B * t.C * t.H * t.W * (4 if t.dtype == self.capi.I32 else 1) for t in ins)
-            total += out.B * out.C * out.H * out.W * (4 if out.dtype == self.capi.I32 else 1)
-            if l.type in ("conv", "fc"):
-                total += l.w.size // (2 if l.weight_bits == 4 else 1)
-            if l.name in self.bottleneck_layers:
-                total += sum(m.w.size for m in self.bottleneck_layers[l.name])
-            elif l.name in self.fused_sums:
-                total += self.fused_sums[l.name][1].w.size
-        return total
+        return sum(self.layer_bytes(l) for l in self.launched)

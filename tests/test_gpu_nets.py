@@ -62,6 +62,15 @@ def test_resnet50_config(variant):
     assert sorted(n for n, t in net.tensors.items() if t.halo) == sorted(
         [l.name[:-3] + "1x1" for l in spec.layers if l.name.endswith("_3x3") and not (one_launch and l.name == "conv2.1_3x3")]
         + (["pool1"] if one_launch else []))
+    # a block's expansion + sum and the next block's reduction as one launch (off by default): same bytes everywhere
+    if one_launch:
+        tails = nets.GpuNet(spec, x.shape[0], tails=True)
+        tails.set_input(x)
+        assert sorted(tails.absorbed) == ["conv3.3_1x1", "conv3.4_1x1", "conv4.3_1x1", "conv4.4_1x1", "conv4.5_1x1", "conv4.6_1x1"]
+        assert len(tails.launched) == len(net.launched) - 6
+        assert np.array_equal(tails.forward().to_numpy(), net.tensors[spec.output].to_numpy())
+        for n in ("conv3.3_1x1", "conv3.3_sum", "conv4.6_1x1", "conv4.5_sum"):
+            assert np.array_equal(tails.tensors[n].to_numpy(), net.tensors[n].to_numpy()), n
     separate = nets.GpuNet(spec, x.shape[0], bottlenecks=False)
     separate.set_input(x)
     assert not separate.bottlenecks and len(separate.folded) == 28 and len(separate.launched) == len(spec.layers) - 28
