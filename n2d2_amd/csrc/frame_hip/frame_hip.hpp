@@ -209,6 +209,12 @@ public:
     std::size_t getFractionalBits() const { return mNbFractionalBits; }
     bool getIsClipped() const { return mIsClipped; }
     const std::vector<Float_T>& getClippingPerOutput() const { return mClipping; }
+    // Text form of everything this object holds (include/Scaling.hpp:336-432: mode, per-output factors, fractional bits,
+    // clip flag and values), one "Key=values" line each; floats are written with the digits that read back to the same
+    // bits.  N2D2 itself has no file format for a Scaling (Activation::save writes the parameters only,
+    // src/Activation/Activation.cpp:66-97): this one carries a graph quantized in one process into another.
+    void save(std::ostream& os) const;
+    static Scaling load(std::istream& is, const std::string& what);
     // true when every factor is >= 0 (ScalingCell::getOutputsRange, src/Cell/ScalingCell.cpp:68-104)
     bool allScalingsPositive() const;
     std::size_t nbOutputs() const;
@@ -1009,6 +1015,11 @@ public:
     // those of the separate cells, bit for bit; the folded cells' own outputs are not written (getOutputs() on them
     // throws).  With it, a tensor written by a convolution and read only by convolutions is stored with the readers'
     // padding as a border of zeros (n2d2hip_tensor::halo).  Turn it off to read every cell's output.
+    // What quantization left in the cells beside the free parameters, one text file "<dirName>/<cell>.quant" per cell: the
+    // cell's and its activation's bit widths and the activation's (or the ScalingCell's) Scaling.  Together with
+    // exportFreeParameters / importFreeParameters this moves a quantized graph between processes.
+    void saveQuantization(const std::string& dirName) const;
+    void loadQuantization(const std::string& dirName);
     void setFusion(bool enabled);
     bool getFusion() const { return mFusion; }
     // Number of cells propagate() does not launch because a consumer computes them

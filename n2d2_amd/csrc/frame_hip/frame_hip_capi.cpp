@@ -192,6 +192,9 @@ int fh_cell_set_mapping(void* net, const char* name, const unsigned char* map, s
     });
 }
 
+int fh_net_save_quantization(void* net, const char* dirName) { return guarded([&] { ((Net*)net)->deepNet->saveQuantization(dirName); }); }
+int fh_net_load_quantization(void* net, const char* dirName) { return guarded([&] { ((Net*)net)->deepNet->loadQuantization(dirName); }); }
+
 int fh_cell_set_biases(void* net, const char* name, const float* b, size_t n)
 {
     return guarded([&] {

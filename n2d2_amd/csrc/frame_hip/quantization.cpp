@@ -7,6 +7,9 @@
 #include <cctype>
 #include <fstream>
 #include <iomanip>
+#include <limits>
+#include <map>
+#include <sstream>
 
 namespace N2D2 {
 
@@ -217,6 +220,181 @@ void FcCell::processFreeParametersPerOutput(const std::function<Float_T(Float_T)
 }
 
 // -------------------------------------------------------- DeepNetQuantization
+// ------------------------------------------------------------------ Scaling and bit widths as text
+namespace {
+const char* scalingModeName(ScalingMode mode)
+{
+    switch (mode) {
+    case ScalingMode::NONE: return "None";
+    case ScalingMode::FLOAT_MULT: return "Floating-point";
+    case ScalingMode::FIXED_MULT16: return "Fixed-point16";
+    case ScalingMode::FIXED_MULT32: return "Fixed-point32";
+    case ScalingMode::SINGLE_SHIFT: return "Single-shift";
+    default: return "Double-shift";
+    }
+}
+
+// "Key=value" lines of a stream, in any order; a key given twice or a line without '=' is an error
+std::map<std::string, std::string> readKeyValues(std::istream& is, const std::string& what)
+{
+    std::map<std::string, std::string> kv;
+    std::string line;
+    while (std::getline(is, line)) {
+        if (line.find_first_not_of(" \t\r") == std::string::npos)
+            continue;
+        const size_t eq = line.find('=');
+        if (eq == std::string::npos)
+            throw std::runtime_error("Malformed line \"" + line + "\" in " + what);
+        const std::string key = line.substr(0, eq);
+        if (!kv.insert(std::make_pair(key, line.substr(eq + 1))).second)
+            throw std::runtime_error("Key " + key + " given twice in " + what);
+    }
+    return kv;
+}
+
+const std::string& need(const std::map<std::string, std::string>& kv, const std::string& key, const std::string& what)
+{
+    auto it = kv.find(key);
+    if (it == kv.end())
+        throw std::runtime_error("Missing key " + key + " in " + what);
+    return it->second;
+}
+
+// "<count> v0 v1 ..." -> values; the count must match what follows
+template <class T, class Parse>
+std::vector<T> readVector(const std::string& text, const std::string& key, const std::string& what, Parse parse)
+{
+    std::istringstream in(text);
+    size_t n = 0;
+    if (!(in >> n))
+        throw std::runtime_error("Key " + key + " in " + what + " does not start with a count");
+    std::vector<T> v;
+    std::string tok;
+    while (in >> tok)
+        v.push_back(parse(tok));
+    if (v.size() != n)
+        throw std::runtime_error("Key " + key + " in " + what + " announces " + std::to_string(n) + " values and holds " + std::to_string(v.size()));
+    return v;
+}
+
+Scaling scalingFromKeyValues(const std::map<std::string, std::string>& kv, const std::string& what)
+{
+    const ScalingMode mode = parseScalingMode(need(kv, "ScalingMode", what));
+    if (mode == ScalingMode::NONE)
+        return Scaling();
+    const bool isClipped = std::stoi(need(kv, "IsClipped", what)) != 0;
+    const std::vector<Float_T> clipping = readVector<Float_T>(need(kv, "Clipping", what), "Clipping", what,
+                                                              [](const std::string& t) { return (Float_T)std::stof(t); });
+    const std::string& text = need(kv, "Scaling", what);
+    auto asInt = [&](const std::string& t, long long lo, long long hi) {
+        size_t used = 0;
+        const long long v = std::stoll(t, &used);
+        if (used != t.size() || v < lo || v > hi)
+            throw std::runtime_error("Value " + t + " of key Scaling in " + what + " is not an integer in [" + std::to_string(lo) + ", "
+                                     + std::to_string(hi) + "]");
+        return v;
+    };
+    switch (mode) {
+    case ScalingMode::FLOAT_MULT:
+        return Scaling::floatingPointScaling(readVector<Float_T>(text, "Scaling", what, [](const std::string& t) { return (Float_T)std::stof(t); }),
+                                             isClipped, clipping);
+    case ScalingMode::FIXED_MULT16:
+    case ScalingMode::FIXED_MULT32:
+        return Scaling::fixedPointScaling(mode, (std::size_t)std::stoul(need(kv, "NbFractionalBits", what)),
+                                          readVector<std::int32_t>(text, "Scaling", what, [&](const std::string& t) {
+                                              return (std::int32_t)asInt(t, std::numeric_limits<std::int32_t>::min(), std::numeric_limits<std::int32_t>::max());
+                                          }),
+                                          isClipped, clipping);
+    case ScalingMode::SINGLE_SHIFT:
+        return Scaling::singleShiftScaling(readVector<unsigned char>(text, "Scaling", what, [&](const std::string& t) { return (unsigned char)asInt(t, 0, 255); }),
+                                           isClipped, clipping);
+    default: {
+        const std::vector<unsigned char> flat = readVector<unsigned char>(text, "Scaling", what, [&](const std::string& t) { return (unsigned char)asInt(t, 0, 255); });
+        if (flat.size() % 2 != 0)
+            throw std::runtime_error("Key Scaling in " + what + ": a double shift holds two exponents per output");
+        std::vector<std::pair<unsigned char, unsigned char> > pairs;
+        for (size_t i = 0; i < flat.size(); i += 2)
+            pairs.push_back(std::make_pair(flat[i], flat[i + 1]));
+        return Scaling::doubleShiftScaling(pairs, isClipped, {});
+    }
+    }
+}
+} // namespace
+
+void Scaling::save(std::ostream& os) const
+{
+    os << "ScalingMode=" << scalingModeName(mMode) << "\n";
+    if (mMode == ScalingMode::NONE)
+        return;
+    os << "NbFractionalBits=" << mNbFractionalBits << "\n";
+    os << "IsClipped=" << (mIsClipped ? 1 : 0) << "\n";
+    os << "Scaling=";
+    if (mMode == ScalingMode::FLOAT_MULT) {
+        os << mFloat.size() << std::setprecision(9);
+        for (Float_T v : mFloat) os << " " << v;
+    } else if (mMode == ScalingMode::FIXED_MULT16 || mMode == ScalingMode::FIXED_MULT32) {
+        os << mFixed.size();
+        for (std::int32_t v : mFixed) os << " " << v;
+    } else {
+        os << mShift.size();
+        for (unsigned char v : mShift) os << " " << (int)v;
+    }
+    os << "\nClipping=" << mClipping.size() << std::setprecision(9);
+    for (Float_T v : mClipping) os << " " << v;
+    os << "\n";
+}
+
+Scaling Scaling::load(std::istream& is, const std::string& what)
+{
+    return scalingFromKeyValues(readKeyValues(is, what), what);
+}
+
+void DeepNet::saveQuantization(const std::string& dirName) const
+{
+    for (const std::shared_ptr<Cell>& cell : mOrder) {
+        const std::string fileName = dirName + "/" + cell->getName() + ".quant";
+        std::ofstream os(fileName.c_str());
+        if (!os.good())
+            throw std::runtime_error("Could not create quantization file: " + fileName);
+        os << "CellQuantizedNbBits=" << cell->getQuantizedNbBits() << "\n";
+        os << "ActivationQuantizedNbBits=" << (cell->getActivation() ? cell->getActivation()->getQuantizedNbBits() : 0) << "\n";
+        if (auto sc = std::dynamic_pointer_cast<ScalingCell>(cell))
+            sc->getScaling().save(os);
+        else if (cell->getActivation())
+            cell->getActivation()->getActivationScaling().save(os);
+        else
+            Scaling().save(os);
+        if (!os.good())
+            throw std::runtime_error("Error writing quantization file: " + fileName);
+    }
+}
+
+void DeepNet::loadQuantization(const std::string& dirName)
+{
+    for (const std::shared_ptr<Cell>& cell : mOrder) {
+        const std::string fileName = dirName + "/" + cell->getName() + ".quant";
+        std::ifstream is(fileName.c_str());
+        if (!is.good())
+            throw std::runtime_error("Could not open quantization file: " + fileName);
+        const std::map<std::string, std::string> kv = readKeyValues(is, fileName);
+        Scaling scaling = scalingFromKeyValues(kv, fileName);
+        const std::size_t nb = scaling.nbOutputs();
+        if (scaling.getMode() != ScalingMode::NONE && nb != cell->getNbOutputs() && nb != 1)
+            throw std::runtime_error("Quantization file " + fileName + " holds a scaling for " + std::to_string(nb) + " outputs, cell "
+                                     + cell->getName() + " has " + std::to_string(cell->getNbOutputs()));
+        cell->setQuantized((std::size_t)std::stoul(need(kv, "CellQuantizedNbBits", fileName)));
+        const std::size_t actBits = (std::size_t)std::stoul(need(kv, "ActivationQuantizedNbBits", fileName));
+        if (auto sc = std::dynamic_pointer_cast<ScalingCell>(cell)) {
+            sc->setScaling(scaling);
+        } else if (cell->getActivation()) {
+            cell->getActivation()->setActivationScaling(scaling);
+            cell->getActivation()->setQuantized(actBits);
+        } else if (scaling.getMode() != ScalingMode::NONE) {
+            throw std::runtime_error("Quantization file " + fileName + " holds a scaling, cell " + cell->getName() + " has no activation");
+        }
+    }
+}
+
 namespace {
 
 // Largest multiplier a fixed-point mode can hold.

@@ -26,6 +26,8 @@ lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c
 lib.fh_cell_set_quantized.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int]
 lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+lib.fh_net_save_quantization.argtypes = [C.c_void_p, C.c_char_p]
+lib.fh_net_load_quantization.argtypes = [C.c_void_p, C.c_char_p]
 lib.fh_get_nb_groups.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
 lib.fh_cell_set_mapping.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_size_t]
 lib.fh_cell_set_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
@@ -164,6 +166,13 @@ class Net:
         cl = None if clipping is None else np.ascontiguousarray(clipping, dtype=np.float32)
         _check(lib.fh_cell_set_scaling(self.h, name.encode(), _MODE[mode], s.ctypes.data, n, int(frac_bits), int(cl is not None),
                                        None if cl is None else cl.ctypes.data))
+
+    def save_quantization(self, dir_name):
+        """DeepNet::saveQuantization: one "<cell>.quant" text file per cell (bit widths and Scaling)."""
+        _check(lib.fh_net_save_quantization(self.h, str(dir_name).encode()))
+
+    def load_quantization(self, dir_name):
+        _check(lib.fh_net_load_quantization(self.h, str(dir_name).encode()))
 
     def import_free_parameters(self, name, file_name, ignore_not_exists=False):
         """Cell::importFreeParameters: "<base>_weights<.ext>" (+ "<base>_biases<.ext>"), or one file with both."""

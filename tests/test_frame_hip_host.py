@@ -355,3 +355,55 @@ def test_conv_mapping_sets_the_groups(fh):
     net.set_mapping("conv1", np.ones((O, Cn)))          # fully connected: one group
     with pytest.raises(fh.FrameHipError, match="not a Conv"):
         net.set_mapping("pool1", np.ones((16, 16)))
+
+
+def test_quantization_files_round_trip(fh, tmp_path):
+    """DeepNet::saveQuantization / loadQuantization: what the quantization pass leaves in the cells beside their weights
+    (bit widths, Scaling mode, factors, fractional bits, clip) goes through one text file per cell and comes back bit
+    for bit, for every scaling mode; damaged files are refused with a message naming the file."""
+    import numpy as np
+    rng = np.random.default_rng(3)
+    net = fh.Net(INI % "Frame_HIP")
+    cells = {"conv1": 16}
+    info = net.cell_info("conv1")
+    settings = [("FloatMult", rng.uniform(1e-4, 0.3, 16).astype(np.float32), 0, rng.uniform(1.0, 300.0, 16).astype(np.float32)),
+                ("FixedMult16", rng.integers(1, 2 ** 15, 16).astype(np.int32), 13, None),
+                ("FixedMult32", rng.integers(-2 ** 20, 2 ** 30, 16).astype(np.int32), 27, rng.uniform(1.0, 300.0, 16).astype(np.float32)),
+                ("SingleShift", rng.integers(0, 20, 16).astype(np.uint8), 0, None),
+                ("DoubleShift", rng.integers(0, 12, (16, 2)).astype(np.uint8), 0, None),
+                ("None", None, 0, None)]
+    for k, (mode, scaling, frac, clip) in enumerate(settings):
+        net.set_scaling("conv1", mode, scaling, frac, clip)
+        net.set_quantized("conv1", 8, 4 + k % 5)
+        d = tmp_path / ("q%d" % k)
+        d.mkdir()
+        net.save_quantization(d)
+        assert (d / "conv1.quant").exists() and (d / "pool1.quant").exists()
+        other = fh.Net(INI % "Frame_HIP")
+        other.load_quantization(d)
+        m2, f2, v2 = other.scaling("conv1")
+        assert m2 == mode
+        if mode != "None":
+            assert f2 == (frac if mode.startswith("Fixed") else 0)
+            assert np.array_equal(v2.astype(np.float32), np.asarray(scaling).reshape(-1).astype(np.float32))
+            c2 = other.clipping("conv1")
+            assert (c2 is None) == (clip is None) and (clip is None or np.array_equal(c2, clip))
+        assert other.quantized("conv1")[:2] == (8, 4 + k % 5)
+    # a file that announces more values than it holds, a missing file, a scaling for another cell size
+    d = tmp_path / "bad"
+    d.mkdir()
+    net.set_scaling("conv1", "SingleShift", np.arange(16, dtype=np.uint8))
+    net.save_quantization(d)
+    text = (d / "conv1.quant").read_text()
+    (d / "conv1.quant").write_text(text.replace("Scaling=16", "Scaling=17"))
+    with pytest.raises(fh.FrameHipError, match="announces 17 values and holds 16"):
+        fh.Net(INI % "Frame_HIP").load_quantization(d)
+    (d / "conv1.quant").write_text(text.replace("Scaling=16 0", "Scaling=15"))
+    with pytest.raises(fh.FrameHipError, match="holds a scaling for 15 outputs"):
+        fh.Net(INI % "Frame_HIP").load_quantization(d)
+    (d / "conv1.quant").write_text(text.replace("IsClipped=0\n", ""))
+    with pytest.raises(fh.FrameHipError, match="Missing key IsClipped"):
+        fh.Net(INI % "Frame_HIP").load_quantization(d)
+    (d / "conv1.quant").unlink()
+    with pytest.raises(fh.FrameHipError, match="Could not open quantization file"):
+        fh.Net(INI % "Frame_HIP").load_quantization(d)

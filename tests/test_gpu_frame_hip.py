@@ -102,6 +102,34 @@ def test_mobilenet_and_w4a4_through_the_registrar(fh):
     _compare(fh, nets.resnet18_w4a4(), x, ["conv2.1_a", "conv2.1_sum", "conv5.2_sum", "fc"])
 
 
+def test_quantized_graph_moves_between_nets_through_files(fh, tmp_path):
+    """A graph quantized in one place runs in another: free parameters through N2D2's text exports, bit widths and Scalings
+    through DeepNet::saveQuantization / loadQuantization; the second net is built from the INI text alone and gives the
+    oracle's outputs (a ResNet-50 with every scaling mode the benchmark uses, and the float-rescaled LeNet)."""
+    from n2d2_amd import nets
+    from oracle import cells
+    for spec, x in ((nets.resnet50(image=64), np.random.default_rng(36).integers(0, 256, size=(2, 3, 64, 64))),
+                    (nets.lenet(), np.random.default_rng(37).integers(0, 256, size=(3, 1, 32, 32)))):
+        first = fh.build_net(spec, x.shape[0])
+        d = tmp_path / spec.name
+        d.mkdir()
+        for l in spec.layers:
+            if l.type in ("conv", "fc"):
+                first.export_free_parameters(l.name, d / (l.name + ".syntxt"))
+        first.save_quantization(d)
+        del first
+        second = fh.Net(fh.spec_to_ini(spec, x.shape[0]))
+        for l in spec.layers:
+            if l.type in ("conv", "fc"):
+                second.import_free_parameters(l.name, d / (l.name + ".syntxt"))
+        second.load_quantization(d)
+        second.initialize()
+        second.set_stimuli(x)
+        second.propagate()
+        want = cells.run_net(spec, x, keep=[spec.output])
+        assert np.array_equal(second.outputs(spec.output), want[spec.output]), spec.name
+
+
 def test_depthwise_cell_from_its_connection_map(fh):
     """The number of groups comes from the connection map (Cell::getNbGroups): MobileNet's first blocks built from an INI
     without any Mapping.* key, the depthwise cells given an identity map, against the oracle."""
