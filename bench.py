@@ -320,13 +320,15 @@ def main():
 
     # Which kernel runs a launch of the forward (the library's own rules, restated here to label the figures):
     # bottleneck_kernel (a residual block in one launch), conv_patch3x3_kernel (3x3, stride 1, at least 128 channels, on an
-    # input that carries its padding, images of at least 10 x 10), conv_stem_kernel (at most 4 input channels),
+    # input that carries its padding, images of at least 10 x 10), conv_stem_kernel (at most 4 input channels; it computes the max pooling behind it in the same launch),
     # conv_pipe_kernel (every other convolution / fully-connected cell with a multiple of 64 input channels, with the
     # residual sum in its epilogue where one follows), bandwidth kernels for the rest.
     def kernel_of(k):
         l = net.launched[k]
         if l.name in net.bottlenecks:
             return "bottleneck_kernel"
+        if l.name in net.stem_pools:
+            return "conv_stem_kernel"
         c = net.fused_sums[l.name][1] if l.name in net.fused_sums else l
         if c.type not in ("conv", "fc"):
             return "bandwidth"

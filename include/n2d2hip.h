@@ -215,6 +215,16 @@ int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* desc, int H, int W, int* outH
 int n2d2hip_pool_forward(const n2d2hip_pool_desc* desc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
 
+/* Graph-level fusion of a first-layer convolution with the max pooling behind it: ConvCell_Frame::propagate followed by
+ * PoolCell_Frame_Kernels::forwardMax (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/PoolCell_Frame_Kernels.cpp:102-197)
+ * in one launch; the convolution's own output is never stored.  n2d2hip_conv_accepts_maxpool says whether the library takes
+ * the pair for an H x W input: a convolution on the first-layer kernel (at most 4 input channels, horizontal stride 2, at
+ * most 64 output channels, rows of at most 128 outputs, integer rescale to bytes) and a 3x3 stride-2 max pooling with
+ * padding 0 or 1.  `out` is the pooled tensor (channel stride 64), with or without a halo. */
+int n2d2hip_conv_accepts_maxpool(n2d2hip_conv_t conv, const n2d2hip_pool_desc* pool, int H, int W);
+int n2d2hip_conv_forward_maxpool(n2d2hip_conv_t conv, const n2d2hip_pool_desc* pool, const n2d2hip_tensor* in,
+                                 const n2d2hip_tensor* out, n2d2hip_stream_t stream);
+
 /* -------------------------------------------------------------- elemwise */
 enum { N2D2HIP_COEFF_PER_LAYER = 0, N2D2HIP_COEFF_PER_INPUT = 1, N2D2HIP_COEFF_PER_CHANNEL = 2 };
 typedef struct n2d2hip_elemwise_s* n2d2hip_elemwise_t;

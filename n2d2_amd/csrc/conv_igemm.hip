@@ -1007,6 +1007,103 @@ int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2h
     return conv_forward_impl(c, in, nullptr, out, stream);
 }
 
+// The first-layer kernel can compute the max pooling behind it: 3x3 windows, stride 2, padding 0 or 1, on rows of at most
+// 128 convolution outputs with at most 64 channels, byte outputs of an integer rescale whose scaled-up tables fit.
+static bool stem_pool_eligible(const n2d2hip_conv_s* c, const n2d2hip_pool_desc* pd, int H, int W, int* OHo, int* OWo, int* POHo, int* POWo)
+{
+    const n2d2hip_conv_desc& d = c->desc;
+    int OH, OW, POH, POW;
+    if (!c->d_wstem || (d.kernel_choice & (N2D2HIP_KERNEL_NO_STEM | N2D2HIP_KERNEL_NO_HI16)) || c->act->args.kind != EPI_I24 || !c->bias_folded
+        || !c->hi16 || c->act->min_out < -128 || c->act->max_out > 255 || d.O > 64 || d.O <= 48 || (d.kH != 3 && d.kH != 5 && d.kH != 7))
+        return false;
+    if (n2d2hip_conv_out_dims(&d, H, W, &OH, &OW) != N2D2HIP_OK || OW > 128)
+        return false;
+    if (pd->pooling != N2D2HIP_POOL_MAX || pd->poolW != 3 || pd->poolH != 3 || pd->strideX != 2 || pd->strideY != 2 || pd->padX != pd->padY
+        || (pd->padX != 0 && pd->padX != 1) || n2d2hip_pool_out_dims(pd, OH, OW, &POH, &POW) != N2D2HIP_OK || POW > 64)
+        return false;
+    // every window holds at least one convolution output
+    if ((POW - 1) * 2 - pd->padX >= OW || (POH - 1) * 2 - pd->padY >= OH)
+        return false;
+    *OHo = OH; *OWo = OW; *POHo = POH; *POWo = POW;
+    return true;
+}
+
+int n2d2hip_conv_accepts_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool, int H, int W)
+{
+    int a, b, e, f;
+    return c && pool && stem_pool_eligible(c, pool, H, W, &a, &b, &e, &f) ? 1 : 0;
+}
+
+int n2d2hip_conv_forward_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                                 n2d2hip_stream_t stream_)
+{
+    int rc, OH, OW, POH, POW;
+    N2D2HIP_REQUIRE(c && pool, N2D2HIP_ERR_INVALID, "conv_forward_maxpool: null argument");
+    if ((rc = check_tensor(in, "conv input")) || (rc = check_tensor(out, "pooled output", true)))
+        return rc;
+    const n2d2hip_conv_desc& d = c->desc;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED, "conv_forward_maxpool: tensors must be NHWC");
+    N2D2HIP_REQUIRE(in->dtype == c->in_dtype && in->C == d.C && in->cs == c->in_cs, N2D2HIP_ERR_INVALID,
+                    "conv_forward_maxpool: input has %d channels (stride %d) of type %d, conv expects %d (stride %d) of type %d", in->C, in->cs,
+                    in->dtype, d.C, c->in_cs, c->in_dtype);
+    N2D2HIP_REQUIRE(stem_pool_eligible(c, pool, in->H, in->W, &OH, &OW, &POH, &POW), N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward_maxpool: needs a convolution the first-layer kernel runs with scaled-up integer tables (at most 4 input and "
+                    "64 output channels, rows of at most 128 outputs) and a 3x3 stride-2 max pooling with padding 0 or 1 "
+                    "(n2d2hip_conv_accepts_maxpool)");
+    N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == POH && out->W == POW && out->cs == 64
+                        && (out->dtype == N2D2HIP_U8B || out->dtype == N2D2HIP_I8),
+                    N2D2HIP_ERR_INVALID, "conv_forward_maxpool: output must be %dx%dx%dx%d bytes (U8B or I8) with a channel stride of 64", in->B,
+                    d.O, POH, POW);
+    {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(c->act->min_out >= lo && c->act->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "conv_forward_maxpool: activation range [%d,%d] does not fit output dtype %d", c->act->min_out, c->act->max_out, out->dtype);
+    }
+    N2D2HIP_REQUIRE((long long)in->B * in->H * in->W * in->cs < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "conv_forward_maxpool: tensor too large");
+    ConvArgs a;
+    a.in = (const signed char*)in->data;
+    a.in_cs = in->cs; a.B = in->B; a.H = in->H; a.W = in->W;
+    a.OH = OH; a.OW = OW; a.M = in->B * OH * OW;
+    a.w = c->d_w; a.ktot = c->ktot; a.niter = c->ktot / 64; a.sub = c->d_sub; a.bias = c->d_bias;
+    a.out = out->data; a.out_cs = out->cs; a.out_dtype = out->dtype;
+    a.strideX = d.strideX; a.strideY = d.strideY; a.padL = d.padL; a.padT = d.padT; a.dilX = d.dilX; a.dilY = d.dilY;
+    a.kW = d.kW; a.kH = d.kH;
+    a.ntiles_n = 1; a.nblocks = 0;
+    a.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
+    a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    a.epi = c->act->args;
+    ConvStemArgs q = {};
+    q.c = a;
+    const int cp = c->act->cpad;
+    q.c.epi.a = c->d_epi_tab; q.c.epi.b = c->d_epi_tab + cp; q.c.epi.c = c->d_epi_tab + 5 * cp;
+    q.c.epi.d = c->d_epi_tab + 6 * cp; q.c.epi.e = c->d_epi_tab + 4 * cp;
+    q.wk = c->d_wstem;
+    q.fill16 = c->d_fill;
+    q.preclamp = c->preclamp ? 1 : 0;
+    q.tiles_per_row = 1;
+    // strips: about two per block slot, so that the one convolution row two neighbouring strips both compute stays a small
+    // share of the work; a strip's rows are consecutive, so its input rows come out of the cache
+    const int slots = 2 * num_cus();
+    int rows = std::max(1, (int)(((long long)in->B * POH + 2 * slots - 1) / (2 * slots)));
+    rows = std::min(std::max(rows, std::min(POH, 4)), POH);
+    q.pool_rows = rows;
+    q.strips_per_image = (POH + rows - 1) / rows;
+    q.pool_pad = pool->padX;
+    q.POH = POH; q.POW = POW;
+    q.pool_halo = out->halo; q.POHp = POH + 2 * out->halo; q.POWp = POW + 2 * out->halo;
+    q.ntiles = in->B * q.strips_per_image;
+    // two blocks per compute unit (64 KB of LDS each)
+    q.nlanes = std::max(1, std::min((q.ntiles + 7) / 8, (2 * num_cus()) / 8));
+    q.xcd_tiles = (q.ntiles + 7) / 8;
+    const int grid = 8 * q.nlanes;
+    hipStream_t stream = (hipStream_t)stream_;
+    if (d.kH == 3) hipLaunchKernelGGL((conv_stem_kernel<3, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
+    else if (d.kH == 5) hipLaunchKernelGGL((conv_stem_kernel<5, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
+    else hipLaunchKernelGGL((conv_stem_kernel<7, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
 int n2d2hip_conv_accepts_halo(n2d2hip_conv_t c)
 {
     bool bn128;

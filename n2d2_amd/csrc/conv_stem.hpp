@@ -41,12 +41,20 @@ struct ConvStemArgs {
     unsigned oh_mul, oh_sh;      // division by OH
     unsigned tpr_mul, tpr_sh;    // division by tiles_per_row
     int preclamp;
+    // POOL kernels: the 3x3 stride-2 max pooling that follows the convolution is computed in the same launch.  A block
+    // takes strips of pool_rows pooled rows of one image: the 2 * pool_rows + 1 convolution rows a strip needs go to a ring
+    // of four rows in LDS as bytes, and each pooled row is written as soon as its third convolution row is there.  `ntiles`
+    // then counts strips, `out` is the pooled tensor and the convolution's own output is never stored.
+    int pool_rows, pool_pad, strips_per_image;
+    int POH, POW;                // pooled rows / columns
+    int pool_halo, POHp, POWp;   // border of the pooled tensor and its rows / columns with it
 };
 
-template <int KH, int EPI, bool H16 = false>
+template <int KH, int EPI, bool H16 = false, bool POOL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) void conv_stem_kernel(ConvStemArgs q)
 {
     static_assert(!H16 || EPI == EPI_I24, "scaled-up tables belong to the integer rescale");
+    static_assert(!POOL || H16, "the pooled variant is written for byte outputs of the integer rescale");
     const ConvArgs& p = q.c;
     constexpr int TW = 128;                    // output pixels per tile
     constexpr int PITCH = 1280;                // bytes per patch row in LDS: 5 loads of 64 pixels
@@ -56,7 +64,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     constexpr int BN = 64;
     constexpr int TAB_OFF = 3 * STAGE;
     constexpr bool BIAS_ADD = EPI != EPI_I24;  // the integer rescale carries the bias in its tables
-    __shared__ __attribute__((aligned(16))) unsigned char smem[TAB_OFF + 6 * BN * 4];
+    constexpr int ROWS_OFF = TAB_OFF + 6 * BN * 4;             // POOL: four convolution rows of TW pixels x 64 bytes
+    __shared__ __attribute__((aligned(16))) unsigned char smem[ROWS_OFF + (POOL ? 4 * TW * BN : 0)];
     const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
 
     const int tid = threadIdx.x;
@@ -70,7 +79,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     // L2) and its blocks take them in turn.
     const int first = xcd * q.xcd_tiles + slot / p.ntiles_n;
     const int last = min((xcd + 1) * q.xcd_tiles, q.ntiles);
-    const int ntile = (first < last) ? (last - first + q.nlanes - 1) / q.nlanes : 0;
+    // POOL: the units dealt to blocks are strips; a block's tiles are the convolution rows of its strips, one after the other
+    const int nunit = (first < last) ? (last - first + q.nlanes - 1) / q.nlanes : 0;
+    const int rows_per_strip = 2 * q.pool_rows + 1;
+    const int ntile = POOL ? nunit * rows_per_strip : nunit;
+    // Position of a walk over the block's tiles: strip k of the block, row j of the strip, the strip's image and the
+    // convolution row of j = 0.  The loader walks two tiles ahead of the consumer; a division only where a strip begins.
+    struct StripWalk { int k, j, b, oy0; };
+    auto set_strip = [&](StripWalk& w) {
+        const int sid = first + (w.k < nunit ? w.k : 0) * q.nlanes;
+        w.b = sid / q.strips_per_image;
+        w.oy0 = 2 * (sid - w.b * q.strips_per_image) * q.pool_rows - q.pool_pad;
+    };
+    auto walk_next = [&](StripWalk& w) {
+        if (++w.j == rows_per_strip) { w.j = 0; ++w.k; set_strip(w); }
+    };
+    auto row_live = [&](const StripWalk& w) -> bool {
+        const int oy = w.oy0 + w.j;
+        return w.k < nunit && oy >= 0 && oy < p.OH;
+    };
+    StripWalk lw = {0, 0, 0, 0}, cw = {0, 0, 0, 0};
+    if (POOL) { set_strip(lw); cw = lw; }
 
     // ---- loader: chunk c = wave + 4*j is 64 pixels (part c%5) of patch row c/5.  Which row and part a wave's j-th
     // load fetches never changes, so that is worked out once; the scalar unit is shared by every wave of the CU and
@@ -87,11 +116,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     const unsigned row_bytes = (unsigned)p.W * 4u;
     auto issue = [&](int t, int stage) {
         const int id = first + t * q.nlanes;
-        const bool live = t < ntile;
-        const int rowid = div_magic(live ? id : 0, q.tpr_mul, q.tpr_sh);          // b * OH + oy
-        const int txi = (live ? id : 0) - rowid * q.tiles_per_row;
-        const int b = div_magic(rowid, q.oh_mul, q.oh_sh);
-        const int oy = rowid - b * p.OH;
+        bool live = t < ntile;
+        int b, oy, txi = 0;
+        if (POOL) {
+            live = row_live(lw);
+            b = live ? lw.b : 0;
+            oy = live ? lw.oy0 + lw.j : 0;
+            walk_next(lw);
+        } else {
+            const int rowid = div_magic(live ? id : 0, q.tpr_mul, q.tpr_sh);          // b * OH + oy
+            txi = (live ? id : 0) - rowid * q.tiles_per_row;
+            b = div_magic(rowid, q.oh_mul, q.oh_sh);
+            oy = rowid - b * p.OH;
+        }
         const int x0 = txi * TW * p.strideX - p.padL + lane;
         const int y0 = live ? oy * p.strideY - p.padT : -(1 << 21);
         unsigned char* sbase = smem + stage * STAGE;
@@ -182,8 +219,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
 
         // ---- epilogue: this lane holds channels 8g + 4*lh .. +3 of both 32-channel tiles for output pixel ox
         const int id = first + t * q.nlanes;
-        const int rowid = div_magic(id, q.tpr_mul, q.tpr_sh);
-        const int ox = (id - rowid * q.tiles_per_row) * TW + 32 * wave + l32;
+        const int rowid = POOL ? 0 : div_magic(id, q.tpr_mul, q.tpr_sh);
+        const int ox = POOL ? 32 * wave + l32 : (id - rowid * q.tiles_per_row) * TW + 32 * wave + l32;
         const long long m = (long long)rowid * p.OW + ox;
         const bool pix_ok = ox < p.OW;
         unsigned pk[2][4];
@@ -266,11 +303,60 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
                 first[e] = (int)x[0];
                 second[e] = (int)x[1];
             }
+            if constexpr (POOL) {
+                // the row goes to the ring in LDS (a row that does not exist: the smallest byte, which no maximum picks);
+                // once the third row of a pooled row is there, that pooled row is computed and stored
+                const int pb = cw.b, poy = cw.oy0 + cw.j, pj = cw.j;
+                const bool live_row = row_live(cw);
+                walk_next(cw);
+                if (!live_row) {
+                    const int lowest = (int)0x80808080u;     // -128 in every byte: bytes are compared as stored, i.e. signed
+                    first = v4i{lowest, lowest, lowest, lowest};
+                    second = first;
+                }
+                unsigned char* rowp = smem + ROWS_OFF + ((pj & 3) * TW + ox) * BN + 32 * lh;
+                *(v4i*)rowp = first;
+                *(v4i*)(rowp + 16) = second;
+                const int py = ((poy + q.pool_pad) >> 1) - 1;      // the pooled row whose last convolution row this is
+                if (pj >= 2 && !(pj & 1)) {
+                    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                    const int px = tid >> 2, cg = tid & 3;
+                    if (px < q.POW && py < q.POH) {
+                        v2s me[4], mo[4];
+#pragma unroll
+                        for (int sy = 0; sy < 3; ++sy) {
+                            const unsigned char* rp = smem + ROWS_OFF + (((pj - 2 + sy) & 3) * TW) * BN + cg * 16;
+#pragma unroll
+                            for (int sx = 0; sx < 3; ++sx) {
+                                const int col = min(max(2 * px - q.pool_pad + sx, 0), p.OW - 1);
+                                const v4i v = *(const v4i*)(rp + col * BN);
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const unsigned w = (unsigned)v[e];
+                                    const unsigned ev = (w << 8) & 0xFF00FF00u, od = w & 0xFF00FF00u;
+                                    const v2s ee = as_v2s((int)ev), oo = as_v2s((int)od);
+                                    if (sy == 0 && sx == 0) { me[e] = ee; mo[e] = oo; }
+                                    else { me[e] = __builtin_elementwise_max(me[e], ee); mo[e] = __builtin_elementwise_max(mo[e], oo); }
+                                }
+                            }
+                        }
+                        v4i res;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned ue = (unsigned)__builtin_bit_cast(int, me[e]), uo = (unsigned)__builtin_bit_cast(int, mo[e]);
+                            res[e] = (int)(((ue >> 8) & 0x00FF00FFu) | (uo & 0xFF00FF00u));
+                        }
+                        const long long opix = ((long long)pb * q.POHp + py + q.pool_halo) * q.POWp + px + q.pool_halo;
+                        *(v4i*)((signed char*)p.out + opix * p.out_cs + cg * 16) = res;
+                    }
+                }
+            } else {
             signed char* orow = (signed char*)p.out + m * p.out_cs + n0 + 32 * lh;
             const int ch = n0 + 32 * lh;
             if (pix_ok) {
                 if (ch < p.out_cs) *(v4i*)orow = first;
                 if (ch + 16 < p.out_cs) *(v4i*)(orow + 16) = second;
+            }
             }
         }
     }

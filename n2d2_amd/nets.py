@@ -356,7 +356,7 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False):
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -365,6 +365,8 @@ class GpuNet:
         bottlenecks: run a residual block 1x1 -> 3x3 -> 1x1 + sum (+ projection) whose cells qualify as one launch
         (n2d2hip_bottleneck_*); its input tensor then carries a border of one pixel.  True / "all", "projection" (only the
         blocks with a projection shortcut, where one launch replaces four), or False.
+        stem_pool: compute the max pooling behind a first-layer convolution in that convolution's launch
+        (n2d2hip_conv_forward_maxpool) where the library takes the pair.
         tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
         (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
         only ties with the two separate launches."""
@@ -464,6 +466,24 @@ class GpuNet:
                         if t is self.input:
                             lst[k] = nx
                 self.input = self.tensors["input"] = nx
+        # a first-layer convolution and the max pooling behind it as one launch (the convolution's output is never written)
+        self.stem_pools = {}
+        if fuse and stem_pool:
+            step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+            for l in spec.layers:
+                if l.type != "pool" or l.kind != "max":
+                    continue
+                conv = by_name.get(l.inputs[0])
+                if conv is None or conv.type != "conv" or len(consumers[conv.name]) != 1 or conv.name in self.folded:
+                    continue
+                conv_cell, pool_cell = self.steps[step_index[conv.name]][1], self.steps[step_index[l.name]][1]
+                x = ins_of[conv.name][0]
+                if x.halo or not conv_cell.accepts_maxpool(pool_cell, x.H, x.W):
+                    continue
+                self.steps[step_index[l.name]] = (l, conv_cell, (lambda c, i, o, pool=pool_cell: c.forward_maxpool(pool, i[0], o)))
+                ins_of[l.name] = ins_of[conv.name]
+                self.folded.add(conv.name)
+                self.stem_pools[l.name] = conv
         self.bottlenecks, self.bottleneck_layers = {}, {}
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
@@ -571,7 +591,7 @@ class GpuNet:
             if x.halo == 0:
                 try:
                     nx = rt.DTensor(x.B, x.C, x.H, x.W, x.dtype, halo=1)
-                    if producer.type == "pool":       # does this pooling write a border?  (probed once, on the real tensors)
+                    if producer.type == "pool" and xname not in self.stem_pools:       # does this pooling write a border?  (probed once, on the real tensors)
                         cell_of[xname].forward(ins_of[xname][0], nx)
                 except self.capi.N2D2HipError:
                     if moved:
@@ -658,6 +678,8 @@ class GpuNet:
             total += sum(m.w.size for m in self.bottleneck_layers[l.name])
         elif l.name in self.fused_sums:
             total += self.fused_sums[l.name][1].w.size
+        if l.name in self.stem_pools:       # the convolution's weights; its output never leaves the chip
+            total += self.stem_pools[l.name].w.size
         if l.name in self.tail_layers:      # the reduction's weights and output; its input never leaves the chip
             r = self.tail_layers[l.name]
             z = self.tensors[r.name]
@@ -670,6 +692,8 @@ class GpuNet:
         if l.name in self.fused_sums:
             tail = self.tail_layers.get(l.name)
             return self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
+        if l.name in self.stem_pools:
+            return self.layer_macs(self.stem_pools[l.name])
         if l.type == "conv":
             return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
         if l.type == "fc":

@@ -209,6 +209,14 @@ class Conv:
         oh, ow = self.out_shape(x.H, x.W)
         return DTensor(x.B, self.desc.O, oh, ow, out_dtype if out_dtype is not None else self.act.out_dtype(), halo=halo)
 
+    def accepts_maxpool(self, pool, H, W):
+        """True when the library computes this convolution and the max pooling `pool` (a Pool) behind it in one launch."""
+        return bool(lib.n2d2hip_conv_accepts_maxpool(self.handle, C.byref(pool.desc), H, W))
+
+    def forward_maxpool(self, pool, x, out):
+        check(lib.n2d2hip_conv_forward_maxpool(self.handle, C.byref(pool.desc), x.ref, out.ref, stream_ptr()))
+        return out
+
     def accepts_halo(self):
         """True when this convolution reads and writes tensors that carry their padding as a border of zeros."""
         return bool(lib.n2d2hip_conv_accepts_halo(self.handle))

@@ -704,6 +704,42 @@ def test_bottleneck_in_one_launch_bit_exact(rt):
     assert rt.Bottleneck.create(c128, cb) is None
 
 
+def test_first_layer_conv_with_max_pool_in_one_launch_bit_exact(rt):
+    """n2d2hip_conv_forward_maxpool: a first-layer convolution and the 3x3 stride-2 max pooling behind it in one launch equal
+    the two reference cells; 7x7 / 5x5 / 3x3 kernels, pooling padding 1 and 0, odd sizes (strips that end unevenly, last
+    rows and columns clamped), signed and unsigned outputs, pooled outputs with and without a border."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(99)
+    for (B, H, W, k, pad, ppad, unsigned) in ((3, 224, 224, 7, 3, 1, True), (2, 64, 64, 7, 3, 0, True), (5, 37, 45, 3, 1, 1, True),
+                                              (70, 30, 22, 5, 2, 1, False), (1, 9, 250, 3, 1, 0, True), (2, 224, 224, 7, 3, 0, False)):
+        print("stem+pool", B, H, W, k, pad, ppad, unsigned, flush=True)
+        x = rng.integers(0, 256, size=(B, 3, H, W))
+        w = np.clip(np.rint(rng.normal(0, 30, size=(64, 3, k, k))), -127, 127).astype(np.int64)
+        bias = rng.integers(-3000, 3000, size=64)
+        if unsigned:
+            spec = ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=64), rng.integers(8, 11, size=64)], 1), nb_bits=8, unsigned_out=True)
+        else:
+            spec = ActSpec("Linear", "SingleShift", rng.integers(8, 11, size=64), nb_bits=8, unsigned_out=False)
+        conv = rt.Conv(w, bias, rt.Act(64, **spec.kwargs()), capi.U8B, stride=(2, 2), pad=(pad,) * 4)
+        pool = rt.Pool("max", (3, 3), (2, 2), (ppad, ppad))
+        t = cells_ref.conv_cell(x, w, bias, spec, stride=(2, 2), pad=(pad,) * 4)
+        want = cells_ref.pool_cell(t, "max", (3, 3), (2, 2), (ppad, ppad)).astype(np.int64)
+        dx = rt.DTensor.from_numpy(x, capi.U8B)
+        assert conv.accepts_maxpool(pool, H, W)
+        for halo in (0, 1):
+            out = rt.DTensor(B, 64, want.shape[2], want.shape[3], capi.U8B if unsigned else capi.I8, halo=halo)
+            got = conv.forward_maxpool(pool, dx, out).to_numpy()
+            assert np.array_equal(got, want), (B, H, W, k, pad, ppad, halo, np.count_nonzero(got != want))
+        # the two cells on their own give the same
+        assert np.array_equal(pool.forward(conv.forward(dx)).to_numpy(), want)
+    # what does not qualify is reported: a 2x2 pooling, a convolution with 64 input channels
+    assert not conv.accepts_maxpool(rt.Pool("max", (2, 2), (2, 2)), 224, 224)
+    c64 = rt.Conv(np.ones((64, 64, 3, 3), dtype=np.int64), None, rt.Act(64, **spec.kwargs()), capi.U8B, stride=(2, 2), pad=(1,) * 4)
+    assert not c64.accepts_maxpool(pool, 56, 56)
+
+
 def test_expand_sum_and_next_reduce_in_one_launch_bit_exact(rt):
     """n2d2hip_expand_reduce_*: a block's 1x1 expansion with its folded sum and the next block's 1x1 reduction in one launch
     equal the reference cells run in turn (both tensors: the sum and the reduction's output); 128 and 256 middle channels,
