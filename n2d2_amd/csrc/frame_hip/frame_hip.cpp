@@ -652,16 +652,49 @@ void PoolCell_Frame_HIP<T>::initialize()
 }
 
 template <class T>
-void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
+n2d2hip_pool_desc PoolCell_Frame_HIP<T>::poolDesc() const
 {
-    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype)
-        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
     n2d2hip_pool_desc d;
     d.pooling = mPooling == Max ? N2D2HIP_POOL_MAX : N2D2HIP_POOL_AVERAGE;
     d.poolW = (int)mPoolDims[0]; d.poolH = (int)mPoolDims[1];
     d.strideX = (int)mStrideDims[0]; d.strideY = (int)mStrideDims[1];
     d.padX = (int)mPaddingDims[0]; d.padY = (int)mPaddingDims[1];
-    checkStatus(n2d2hip_pool_forward(&d, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    return d;
+}
+
+template <class T>
+bool PoolCell_Frame_HIP<T>::fuseFirstConv(Cell_Frame_HIP* conv)
+{
+    if (mFusedConv || !conv || !conv->convHandle() || conv->foldedInto() || mInputs.size() != 1)
+        return false;
+    const n2d2hip_pool_desc d = poolDesc();
+    const n2d2hip_tensor& x = conv->inputTensor(0)->desc();
+    if (x.halo != 0 || !n2d2hip_conv_accepts_maxpool(conv->convHandle(), &d, x.H, x.W))
+        return false;
+    mFusedConv = conv;
+    conv->setFoldedInto(this);
+    return true;
+}
+
+template <class T>
+void PoolCell_Frame_HIP<T>::clearFusion()
+{
+    if (mFusedConv) {
+        mFusedConv->setFoldedInto(nullptr);
+        mFusedConv = nullptr;
+    }
+}
+
+template <class T>
+void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
+{
+    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype)
+        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
+    const n2d2hip_pool_desc d = poolDesc();
+    if (mFusedConv)
+        checkStatus(n2d2hip_conv_forward_maxpool(mFusedConv->convHandle(), &d, &mFusedConv->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
+    else
+        checkStatus(n2d2hip_pool_forward(&d, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
 
@@ -1371,6 +1404,8 @@ void DeepNet::setFusion(bool enabled)
         for (Cell_Frame_HIP* f : mFrames) {
             if (auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f))
                 ew->clearFusion();
+            if (auto* pool = dynamic_cast<PoolCell_Frame_HIP<float>*>(f))
+                pool->clearFusion();
             f->setOutputsHalo(0);
         }
     }
@@ -1393,6 +1428,15 @@ void DeepNet::planFusion()
         order[mFrames[i]] = (int)i;
         for (Cell_Frame_HIP* p : mFrames[i]->parentCells())
             ++consumers[p];
+    }
+    // a max pooling that is the only reader of a first-layer convolution is computed by that convolution's launch
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* pool = dynamic_cast<PoolCell_Frame_HIP<float>*>(f);
+        if (!pool) continue;
+        pool->clearFusion();
+        const std::vector<Cell_Frame_HIP*>& parents = pool->parentCells();
+        if (parents.size() == 1 && parents[0] && consumers[parents[0]] == 1)
+            pool->fuseFirstConv(parents[0]);
     }
     for (Cell_Frame_HIP* f : mFrames) {
         auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);

@@ -622,11 +622,18 @@ public:
     void propagate(bool inference = false);
     // src/Cell/PoolCell_Frame.cpp:263-266
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : getOutputsRangeParents(); }
+    // Graph-level fusion (DeepNet::planFusion): the convolution that feeds this max pooling, and nothing else, computes it
+    // in its own launch (n2d2hip_conv_forward_maxpool) when the device library takes the pair; the convolution's own
+    // output is then never written.  Returns false, and changes nothing, when it declines.
+    bool fuseFirstConv(Cell_Frame_HIP* conv);
+    void clearFusion();
 
 protected:
     void setOutputsDims();
 
 private:
+    n2d2hip_pool_desc poolDesc() const;
+    Cell_Frame_HIP* mFusedConv = nullptr;
     static Registrar<PoolCell> mRegistrar;
 };
 

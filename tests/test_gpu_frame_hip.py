@@ -42,9 +42,12 @@ def test_resnet50_through_the_registrar(fh):
     from n2d2_amd import nets
     spec = nets.resnet50()
     x = np.random.default_rng(32).integers(0, 256, size=(2, 3, 224, 224))
-    net = _compare(fh, spec, x, ["conv1", "pool1", "conv2.1_sum", "conv2.2_1x1", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
-    # 12 shortcut ScalingCells applied inside their sums, 16 sums computed by the 1x1 convolution before them
-    assert net.nb_folded == 28
+    net = _compare(fh, spec, x, ["pool1", "conv2.1_sum", "conv2.2_1x1", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
+    # 12 shortcut ScalingCells applied inside their sums, 16 sums computed by the 1x1 convolution before them, the first
+    # convolution's max pooling computed by that convolution's launch
+    assert net.nb_folded == 29
+    with pytest.raises(fh.FrameHipError, match="pool1 computes it on the fly"):
+        net.outputs("conv1")
     # the 16 tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border
     assert net.nb_halo == 16
     with pytest.raises(fh.FrameHipError) as e:
@@ -60,14 +63,15 @@ def test_resnet50_through_the_registrar(fh):
     net.set_fusion(False)
     net.propagate()
     assert net.nb_folded == 0 and net.nb_halo == 0
-    keep = ["conv2.2_shortcut_rescale", "conv2.2_1x1_x4", "conv2.2_sum", "fc"]
+    keep = ["conv1", "pool1", "conv2.2_shortcut_rescale", "conv2.2_1x1_x4", "conv2.2_sum", "fc"]
     want = cells.run_net(spec, x2, keep=keep)
     for name in keep:
         assert np.array_equal(net.outputs(name), want[name]), name
     # and back on: the plan is made again
     net.set_fusion(True)
     net.propagate()
-    assert net.nb_folded == 28 and net.nb_halo == 16 and np.array_equal(net.outputs("fc"), want["fc"])
+    assert net.nb_folded == 29 and net.nb_halo == 16 and np.array_equal(net.outputs("fc"), want["fc"])
+    assert np.array_equal(net.outputs("pool1"), want["pool1"])
     assert np.array_equal(net.outputs("conv2.2_1x1"), cells.run_net(spec, x2, keep=["conv2.2_1x1"])["conv2.2_1x1"])
 
 
