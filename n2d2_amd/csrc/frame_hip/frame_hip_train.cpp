@@ -546,12 +546,19 @@ void BatchNormCell_FrameTrain_HIP<T>::backPropagate()
     const float betaScale = mScaleSolver->isNewIteration() ? 0.0f : 1.0f;
     const float betaBias = mBiasSolver->isNewIteration() ? 0.0f : 1.0f;
     const bool toInput = mDiffOut && !mDiffOut->empty();
-    if (toInput && mDiffOut->isValid())
-        throw std::runtime_error("BatchNormCell_FrameTrain_HIP " + mName + ": accumulating into a gradient another cell has written is not supported");
+    // A gradient another consumer of the same input has already written is added to, as the reference does with its
+    // `isValid * diffOutputs` term (src/Cell/BatchNormCell_Frame.cpp:458-488): this cell's part goes to a buffer of its own
+    // first and is then added in one pass.
+    const bool accumulate = toInput && mDiffOut->isValid();
+    if (accumulate && mDiffOwn.size() != mDiffOut->size())
+        mDiffOwn.resize(mDiffOut->dims());
+    float* dst = !toInput ? nullptr : accumulate ? mDiffOwn.data() : mDiffOut->data();
     checkStatus(n2d2hip_batchnorm_f32_backward((int)mIn->dimB(), (int)mNbOutputs, (int)mInH, (int)mInW, mIn->data(), mScale.data(), mSavedMean.data(),
                                                mSavedVariance.data(), mEpsilon, mDiffInputs.data(), betaScale, mDiffScale.data(), betaBias,
-                                               mDiffBias.data(), mDiffSavedMean.data(), mDiffSavedVariance.data(), toInput ? mDiffOut->data() : nullptr,
+                                               mDiffBias.data(), mDiffSavedMean.data(), mDiffSavedVariance.data(), dst,
                                                mWorkspace.data(), mWorkspace.size() * sizeof(float), mStream));
+    if (accumulate)
+        checkStatus(n2d2hip_elemwise_sum_f32_backward(mDiffOut->size(), 1.0f, mDiffOwn.data(), 1.0f, mDiffOut->data(), mStream));
     if (toInput)
         mDiffOut->setValid();
     mDiffScale.setValid();
@@ -688,10 +695,11 @@ void SoftmaxCell_FrameTrain_HIP<T>::backPropagate()
         return;
     if (!mWithLoss)
         throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + mName + ": backPropagate() without WithLoss is not supported by the float Frame_HIP cells");
-    if (mDiffOut->isValid())
-        throw std::runtime_error("SoftmaxCell_FrameTrain_HIP " + mName + ": accumulation onto a valid diffOutputs is not supported");
-    checkHipT(hipMemcpyAsync(mDiffOut->data(), mDiffInputs.data(), mDiffInputs.size() * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)mStream),
-              "SoftmaxCell_FrameTrain_HIP::backPropagate()");
+    if (mDiffOut->isValid())       // another consumer of the input has written its part: add to it
+        checkStatus(n2d2hip_elemwise_sum_f32_backward(mDiffInputs.size(), 1.0f, mDiffInputs.data(), 1.0f, mDiffOut->data(), mStream));
+    else
+        checkHipT(hipMemcpyAsync(mDiffOut->data(), mDiffInputs.data(), mDiffInputs.size() * sizeof(float), hipMemcpyDeviceToDevice, (hipStream_t)mStream),
+                  "SoftmaxCell_FrameTrain_HIP::backPropagate()");
     mDiffOut->setValid();
 }
 

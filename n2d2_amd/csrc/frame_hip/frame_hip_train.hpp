@@ -265,6 +265,7 @@ private:
     void set(DeviceFloats& dev, std::vector<Float_T>& host, const std::vector<Float_T>& v);
     std::vector<Float_T> get(const DeviceFloats& dev, const std::vector<Float_T>& host) const;
     DeviceFloats mScale, mBias, mMean, mVariance, mSavedMean, mSavedVariance, mDiffScale, mDiffBias, mDiffSavedMean, mDiffSavedVariance;
+    DeviceFloats mDiffOwn;      // this cell's part of the input gradient while another consumer's is already there
     DeviceFloats mWorkspace;            // partial sums of the split reductions
     std::vector<Float_T> mHostScale, mHostBias, mHostMean, mHostVariance;      // values set before initialize()
     std::shared_ptr<SGDSolver> mScaleSolver, mBiasSolver;

@@ -27,7 +27,7 @@ struct TrainNet {
     std::string model;
     Network net;
     DeepNet deepNet;
-    DeviceFloats input, inputDiff, targets;
+    DeviceFloats input, inputDiff, inputDiffPreset, targets;
     std::vector<std::shared_ptr<Cell_FrameTrain_HIP> > cells;
     std::map<std::string, std::shared_ptr<SATQuantizerActivation_Frame_HIP<float> > > satAct;
     std::map<std::string, std::shared_ptr<LSQQuantizerActivation_Frame_HIP<float> > > lsqAct;
@@ -305,6 +305,18 @@ int fh_train_learn(void* net, const float* targets, size_t nTargets, int iterati
         n.targets.fromHost(targets, nTargets);
         double l = 0.0;
         for (int it = 0; it < iterations; ++it) {
+            // the gradient towards the net's input is this iteration's: empty, or what another consumer of the input has
+            // already put there (fh_train_preset_input_gradient)
+            if (!n.inputDiff.empty()) {
+                if (n.inputDiffPreset.empty()) {
+                    n.inputDiff.clearValid();
+                } else {
+                    if (hipMemcpyAsync(n.inputDiff.data(), n.inputDiffPreset.data(), n.inputDiff.size() * sizeof(float), hipMemcpyDeviceToDevice, nullptr)
+                        != hipSuccess)
+                        throw std::runtime_error("fh_train_learn(): copy of the preset input gradient failed");
+                    n.inputDiff.setValid();
+                }
+            }
             for (auto& c : n.cells) c->propagate(false);
             if (hipMemcpyAsync(last->getDiffInputs().data(), n.targets.data(), nTargets * sizeof(float), hipMemcpyDeviceToDevice, nullptr) != hipSuccess)
                 throw std::runtime_error("fh_train_learn(): copy of the targets failed");
@@ -401,6 +413,18 @@ int fh_train_get(void* net, const char* cell, int what, float* out, size_t n)
         else t = conv->getQuantizedWeights();
         if (t.size() != n) throw std::runtime_error("fh_train_get(): size mismatch");
         std::memcpy(out, t.data(), n * sizeof(float));
+    });
+}
+
+// A gradient towards the net's input that is already there when backPropagate() reaches the first cell, as if another
+// consumer of the input had run first: the first cell must add its own to it.
+int fh_train_preset_input_gradient(void* net, const float* values, size_t n)
+{
+    return guardedT([&] {
+        TrainNet& t = *(TrainNet*)net;
+        if (t.inputDiff.empty() || t.inputDiff.size() != n) throw std::runtime_error("fh_train_preset_input_gradient(): size mismatch");
+        t.inputDiffPreset.resize(t.inputDiff.dims());
+        t.inputDiffPreset.fromHost(values, n);
     });
 }
 

@@ -388,6 +388,7 @@ lib.fh_train_learn.argtypes = [_P, _P, _SZ, _I, _P]
 lib.fh_train_propagate.argtypes = [_P, _I]
 lib.fh_train_get.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
 lib.fh_train_input_gradient.argtypes = [_P, _P, _SZ]
+lib.fh_train_preset_input_gradient.argtypes = [_P, _P, _SZ]
 lib.fh_train_get_activation_quantizer.argtypes = [_P, C.c_char_p, _P, _P]
 lib.fh_train_get_weight_quantizer.argtypes = [_P, C.c_char_p, _P, _P]
 
@@ -529,6 +530,12 @@ class TrainNet:
 
     def quantized_weights(self, cell):
         return self._get(cell, 4, self._shapes[cell + "/weights"])
+
+    def preset_input_gradient(self, values):
+        """What another consumer of the net's input is taken to have written to its gradient before this net's first cell
+        runs its backPropagate() (that cell must add to it)."""
+        v = np.ascontiguousarray(values, dtype=np.float32)
+        _check_train(lib.fh_train_preset_input_gradient(self._h, v.ctypes.data, v.size))
 
     def input_gradient(self):
         out = np.empty(self.input_shape, dtype=np.float32)

@@ -299,6 +299,32 @@ def test_batchnorm_and_pool_cells_learn_as_the_oracle_does():
         fresh.learn(np.zeros((4, 1, 12, 12), dtype=np.float32), 1)
 
 
+def test_batchnorm_adds_to_a_gradient_that_is_already_there():
+    """A cell whose input another cell reads too finds that cell's gradient already in place and adds its own
+    (the `isValid * diffOutputs` term of src/Cell/BatchNormCell_Frame.cpp:458-488): the net's input gradient with a
+    gradient preset there equals the preset plus what the same net gives alone."""
+    from n2d2_amd import frame_hip as fh
+    rng = np.random.default_rng(32)
+    x = rng.uniform(0, 1, size=(4, 2, 6, 6)).astype(np.float32)
+    w = rng.normal(0, 0.3, size=(3, 2, 6, 6)).astype(np.float32)
+    t = np.zeros((4, 3, 1, 1), dtype=np.float32)
+    t[np.arange(4), [0, 1, 2, 0]] = 1
+    preset = rng.normal(0, 1, size=x.shape).astype(np.float32)
+
+    def first_gradient(with_preset):
+        net = fh.TrainNet(x, propagate_gradient=True)
+        net.add_batchnorm("bn", act="Linear")
+        net.add_conv("c", w)
+        net.add_softmax("softmax", with_loss=True)
+        if with_preset:
+            net.preset_input_gradient(preset)
+        net.learn(t, 1)
+        return net.input_gradient()
+    alone = first_gradient(False)
+    assert np.abs(alone).max() > 1e-4
+    assert _close(first_gradient(True), alone + preset, 1e-5)
+
+
 @pytest.mark.parametrize("name", ["w8a8", "w4a4"])
 def test_trained_lenet_float_graph_and_its_integer_twin_agree_on_the_gpu(name):
     """The reference's test of its QAT-to-integer pass (tests/Quantizer/QAT/Optimization/class_DeepNetQAT.cpp:96-140) runs the
