@@ -44,10 +44,10 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
     const int oy0 = strip * p.rows;
     const int nrows = min(p.rows, p.OH - oy0);
 
-    const int4 w0 = *(const int4*)(p.wb + c4);
-    const int4 w1 = *(const int4*)(p.wb + p.cs + c4);
-    const int4 w2 = *(const int4*)(p.wb + 2 * p.cs + c4);
-    const int4 bias = *(const int4*)(p.wb + 3 * p.cs + c4);
+    int4 w0 = *(const int4*)(p.wb + c4);
+    int4 w1 = *(const int4*)(p.wb + p.cs + c4);
+    int4 w2 = *(const int4*)(p.wb + 2 * p.cs + c4);
+    int4 bias = *(const int4*)(p.wb + 3 * p.cs + c4);
     int4 ta = {}, tb = {}, tc = {}, td = {}, te = {};
     if (KIND == EPI_I24 || KIND == EPI_I64) {
         ta = *(const int4*)(p.epi.a + c4);
@@ -59,20 +59,31 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
 
     const int ix0 = ox * S - p.padL;
     const bool vm = ix0 >= 0 && ix0 < p.W, v0 = ix0 + 1 >= 0 && ix0 + 1 < p.W, vp = ix0 + 2 >= 0 && ix0 + 2 < p.W;
-    const signed char* col = p.in + ((long long)b * p.H * p.W + ix0) * p.cs + c4;
-    const long long row_bytes = (long long)p.W * p.cs;
     const unsigned fill = p.fill;
-    Row4 border;
-    border.c[0] = border.c[1] = border.c[2] = border.c[3] = (int)(fill & 0x00ffffffu);
-
+    // Every load is issued whatever the position (no branches in the loop): a tap outside the image reads the nearest pixel
+    // inside and is replaced by the stored form of 0 afterwards.
+    const signed char* img = p.in + (long long)b * p.H * p.W * p.cs + c4;
+    const int om = min(max(ix0, 0), p.W - 1) * p.cs, oc = min(max(ix0 + 1, 0), p.W - 1) * p.cs, op = min(max(ix0 + 2, 0), p.W - 1) * p.cs;
+    const long long row_bytes = (long long)p.W * p.cs;
+    // an input row as loaded (left, middle, right pixel)
+    struct Raw3 { unsigned m, c, p; };
+    typedef const unsigned __attribute__((address_space(1))) * GlobalWord;
+    // fetch_row only issues the loads; settle_row, called where the values are used, puts the stored form of 0 in place of
+    // the taps outside the image (a select on a loaded value waits for it).
+    auto fetch_row = [&](int iy) -> Raw3 {
+        const signed char* rp = img + min(max(iy, 0), p.H - 1) * row_bytes;
+        Raw3 r;
+        r.m = *(GlobalWord)(rp + om);
+        r.c = *(GlobalWord)(rp + oc);
+        r.p = *(GlobalWord)(rp + op);
+        return r;
+    };
+    auto settle_row = [&](const Raw3& r, int iy) -> Row4 {
+        const bool row_ok = iy >= 0 && iy < p.H;
+        return transpose3((row_ok && vm) ? r.m : fill, (row_ok && v0) ? r.c : fill, (row_ok && vp) ? r.p : fill);
+    };
     auto load_row = [&](int iy) -> Row4 {
-        if (iy < 0 || iy >= p.H)
-            return border;
-        const signed char* rp = col + iy * row_bytes;
-        const unsigned xm = vm ? *(const unsigned*)rp : fill;
-        const unsigned x0 = v0 ? *(const unsigned*)(rp + p.cs) : fill;
-        const unsigned xp = vp ? *(const unsigned*)(rp + 2 * p.cs) : fill;
-        return transpose3(xm, x0, xp);
+        return settle_row(fetch_row(iy), iy);
     };
     auto finish = [&](int v, int ch, int a, int bq, int c, int d, int e) -> int {
         if (KIND == EPI_I24 || KIND == EPI_I64)
@@ -87,37 +98,54 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
     Row4 t1 = {};
     if (S == 1)
         t1 = load_row(iy0 + 1);
-    for (int q = 0; q < nrows; ++q) {
-        Row4 t2;
-        if (S == 1) {
-            t2 = load_row(iy0 + q + 2);
-        } else {
-            t1 = load_row(iy0 + 2 * q + 1);
-            t2 = load_row(iy0 + 2 * q + 2);
-        }
-        int a0 = __builtin_amdgcn_sdot4(t0.c[0], w0.x, bias.x, false);
-        int a1 = __builtin_amdgcn_sdot4(t0.c[1], w0.y, bias.y, false);
-        int a2 = __builtin_amdgcn_sdot4(t0.c[2], w0.z, bias.z, false);
-        int a3 = __builtin_amdgcn_sdot4(t0.c[3], w0.w, bias.w, false);
-        a0 = __builtin_amdgcn_sdot4(t1.c[0], w1.x, a0, false);
-        a1 = __builtin_amdgcn_sdot4(t1.c[1], w1.y, a1, false);
-        a2 = __builtin_amdgcn_sdot4(t1.c[2], w1.z, a2, false);
-        a3 = __builtin_amdgcn_sdot4(t1.c[3], w1.w, a3, false);
-        a0 = __builtin_amdgcn_sdot4(t2.c[0], w2.x, a0, false);
-        a1 = __builtin_amdgcn_sdot4(t2.c[1], w2.y, a1, false);
-        a2 = __builtin_amdgcn_sdot4(t2.c[2], w2.z, a2, false);
-        a3 = __builtin_amdgcn_sdot4(t2.c[3], w2.w, a3, false);
-        const int r0 = finish(a0, 0, ta.x, tb.x, tc.x, td.x, te.x);
-        const int r1 = finish(a1, 1, ta.y, tb.y, tc.y, td.y, te.y);
-        const int r2 = finish(a2, 2, ta.z, tb.z, tc.z, td.z, te.z);
-        const int r3 = finish(a3, 3, ta.w, tb.w, tc.w, td.w, te.w);
-        const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
-        outp[q * out_row] = packed ^ p.out_xor;
-        if (S == 1) {
-            t0 = t1;
-            t1 = t2;
-        } else {
-            t0 = t2;
+    // The per-channel tables were requested before the first rows and so have arrived by now; saying so here keeps the
+    // loop free of waits for them (such a wait would also wait for the rows requested ahead).
+#define N2D2HIP_DW_ARRIVED(v) asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w))
+    N2D2HIP_DW_ARRIVED(w0); N2D2HIP_DW_ARRIVED(w1); N2D2HIP_DW_ARRIVED(w2); N2D2HIP_DW_ARRIVED(bias);
+    if (KIND == EPI_I24 || KIND == EPI_I64) {
+        N2D2HIP_DW_ARRIVED(ta); N2D2HIP_DW_ARRIVED(tb); N2D2HIP_DW_ARRIVED(tc); N2D2HIP_DW_ARRIVED(td); N2D2HIP_DW_ARRIVED(te);
+    }
+#undef N2D2HIP_DW_ARRIVED
+    // R output rows per turn of the loop, all their input rows requested before the first is used: a thread has 12 loads
+    // in flight, and meets the memory latency once per R rows.  Rows past the strip read a row inside the image and store
+    // nothing.
+    constexpr int R = S == 1 ? 4 : 2;
+    for (int q = 0; q < nrows; q += R) {
+        const int base = iy0 + S * q + (S == 1 ? 2 : 1);
+        Raw3 raw[R * S];
+#pragma unroll
+        for (int i = 0; i < R * S; ++i)
+            raw[i] = fetch_row(base + i);
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            if (S != 1)
+                t1 = settle_row(raw[2 * i], base + 2 * i);
+            const Row4 t2 = settle_row(raw[S * i + S - 1], base + S * i + S - 1);
+            int a0 = __builtin_amdgcn_sdot4(t0.c[0], w0.x, bias.x, false);
+            int a1 = __builtin_amdgcn_sdot4(t0.c[1], w0.y, bias.y, false);
+            int a2 = __builtin_amdgcn_sdot4(t0.c[2], w0.z, bias.z, false);
+            int a3 = __builtin_amdgcn_sdot4(t0.c[3], w0.w, bias.w, false);
+            a0 = __builtin_amdgcn_sdot4(t1.c[0], w1.x, a0, false);
+            a1 = __builtin_amdgcn_sdot4(t1.c[1], w1.y, a1, false);
+            a2 = __builtin_amdgcn_sdot4(t1.c[2], w1.z, a2, false);
+            a3 = __builtin_amdgcn_sdot4(t1.c[3], w1.w, a3, false);
+            a0 = __builtin_amdgcn_sdot4(t2.c[0], w2.x, a0, false);
+            a1 = __builtin_amdgcn_sdot4(t2.c[1], w2.y, a1, false);
+            a2 = __builtin_amdgcn_sdot4(t2.c[2], w2.z, a2, false);
+            a3 = __builtin_amdgcn_sdot4(t2.c[3], w2.w, a3, false);
+            const int r0 = finish(a0, 0, ta.x, tb.x, tc.x, td.x, te.x);
+            const int r1 = finish(a1, 1, ta.y, tb.y, tc.y, td.y, te.y);
+            const int r2 = finish(a2, 2, ta.z, tb.z, tc.z, td.z, te.z);
+            const int r3 = finish(a3, 3, ta.w, tb.w, tc.w, td.w, te.w);
+            const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+            if (q + i < nrows)
+                outp[(q + i) * out_row] = packed ^ p.out_xor;
+            if (S == 1) {
+                t0 = t1;
+                t1 = t2;
+            } else {
+                t0 = t2;
+            }
         }
     }
 }
