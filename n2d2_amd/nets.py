@@ -626,9 +626,11 @@ class GpuNet:
             fn(cell, ins, out)
         return self.tensors[self.spec.output]
 
-    def capture(self):
-        """Records one forward into a HIP graph (every launch of the C ABI goes to the capturing stream and none of
-        them allocates or clears memory) and returns a callable that replays it."""
+    def capture(self, forwards=1):
+        """Records `forwards` forwards, one behind the other, into a HIP graph (every launch of the C ABI goes to the
+        capturing stream and none of them allocates or clears memory) and returns a callable that replays it.  More than
+        one forward per graph spreads the cost of launching a graph over them: a network of one or two kernels is
+        otherwise timed by that cost."""
         import torch
         self.forward()
         torch.cuda.synchronize()
@@ -636,7 +638,8 @@ class GpuNet:
         side = torch.cuda.Stream()
         with torch.cuda.stream(side):
             with torch.cuda.graph(graph, stream=side):
-                self.forward()
+                for _ in range(forwards):
+                    self.forward()
         torch.cuda.synchronize()
         self._graph = graph
 
