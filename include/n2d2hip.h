@@ -295,6 +295,21 @@ int n2d2hip_expand_reduce_destroy(n2d2hip_expand_reduce_t fused);
 int n2d2hip_expand_reduce_forward(n2d2hip_expand_reduce_t fused, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
                                   const n2d2hip_tensor* sum, const n2d2hip_tensor* reduced, n2d2hip_stream_t stream);
 
+/* Graph-level fusion of the MobileNet building block: `depthwise` (3x3, groups == channels, stride 1 or 2, undilated) and
+ * `pointwise` (1x1, stride 1, unpadded), the only reader of its output.  That is ConvCell_Frame::propagate twice
+ * (ref: src/Cell/ConvCell_Frame.cpp:418-473, kernels src/Cell/ConvCell_Frame_Kernels.cpp:26-179) in one launch: the
+ * depthwise output goes from the vector ALU through LDS straight into the matrix cores and is never written to memory;
+ * results are those of the separate cells, bit for bit.  The handles are borrowed, must outlive this one and stay usable
+ * on their own.  Returns N2D2HIP_ERR_UNSUPPORTED (the caller keeps the separate launches) unless both cells are 8-bit
+ * with integer rescales (32-bit multiply-add) and byte outputs, over 32 or a multiple of 64 channels, to 64, 128 or a
+ * multiple of 256 channels. */
+typedef struct n2d2hip_dw_pw_s* n2d2hip_dw_pw_t;
+int n2d2hip_dw_pw_create(n2d2hip_conv_t depthwise, n2d2hip_conv_t pointwise, n2d2hip_dw_pw_t* fused);
+int n2d2hip_dw_pw_destroy(n2d2hip_dw_pw_t fused);
+/* `in`: input of `depthwise`; `out`: output of `pointwise`.  NHWC bytes without a border, channel stride equal to the
+ * channel count. */
+int n2d2hip_dw_pw_forward(n2d2hip_dw_pw_t fused, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream);
+
 /* --------------------------------------------------- SAT / LSQ fake-quant */
 /* Weight quantizer modes, numbered as SATQuantizerCell_Frame::propagate selects them
  * (ref: src/Quantizer/QAT/Cell/SAT/SATQuantizerCell_Frame.cpp:188-200). */

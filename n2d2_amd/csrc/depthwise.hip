@@ -8,25 +8,12 @@
 // output row that uses the input row then needs one 4-way dot product per channel against (w[ky][0], w[ky][1], w[ky][2], 0).
 // Taps outside the image read the stored form of 0, which lets the input's zero point live in the bias.
 #include "depthwise.hpp"
+#include "depthwise_math.hpp"
 #include "epilogue.hpp"
 
 namespace n2d2hip {
 
 namespace {
-
-struct Row4 { int c[4]; };
-
-__device__ __forceinline__ Row4 transpose3(unsigned xm, unsigned x0, unsigned xp)
-{
-    const unsigned lo = __builtin_amdgcn_perm(x0, xm, 0x05010400u);   // m0 c0 m1 c1
-    const unsigned hi = __builtin_amdgcn_perm(x0, xm, 0x07030602u);   // m2 c2 m3 c3
-    Row4 r;
-    r.c[0] = (int)__builtin_amdgcn_perm(xp, lo, 0x0c040100u);
-    r.c[1] = (int)__builtin_amdgcn_perm(xp, lo, 0x0c050302u);
-    r.c[2] = (int)__builtin_amdgcn_perm(xp, hi, 0x0c060100u);
-    r.c[3] = (int)__builtin_amdgcn_perm(xp, hi, 0x0c070302u);
-    return r;
-}
 
 template <int S, int KIND>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p)

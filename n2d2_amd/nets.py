@@ -356,7 +356,8 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True):
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True,
+                 dw_pw=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -367,6 +368,9 @@ class GpuNet:
         blocks with a projection shortcut, where one launch replaces four), or False.
         stem_pool: compute the max pooling behind a first-layer convolution in that convolution's launch
         (n2d2hip_conv_forward_maxpool) where the library takes the pair.
+        dw_pw: run a 3x3 depthwise convolution and the 1x1 convolution that alone reads it as one launch (n2d2hip_dw_pw_*)
+        where the library takes the pair and the launch is expected to be faster than the two (at most 256 output channels,
+        at least 32768 output pixels in the batch); "all": wherever the library takes the pair.
         tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
         (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
         only ties with the two separate launches."""
@@ -484,6 +488,30 @@ class GpuNet:
                 ins_of[l.name] = ins_of[conv.name]
                 self.folded.add(conv.name)
                 self.stem_pools[l.name] = conv
+        # a 3x3 depthwise convolution and the 1x1 convolution that alone reads it as one launch (the depthwise output is
+        # never written)
+        self.dw_pws = {}
+        if fuse and dw_pw:
+            step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+            for l in spec.layers:
+                if l.type != "conv" or l.groups != 1 or l.w.shape[2:] != (1, 1) or l.name in self.folded:
+                    continue
+                dw = by_name.get(l.inputs[0])
+                if (dw is None or dw.type != "conv" or dw.groups == 1 or len(consumers[dw.name]) != 1 or dw.name in self.folded
+                        or ins_of[dw.name][0].halo or self.tensors[l.name].halo):
+                    continue
+                # One launch pays where the tensor between the two cells is large and one work-group holds all output
+                # channels of its pixels; with more than 256 output channels the depthwise part is computed once per
+                # 256 of them, and on small images the launch has too few work-groups to fill the chip.
+                if dw_pw != "all" and (l.out_shape[0] > 256 or batch * l.out_shape[1] * l.out_shape[2] < 32768):
+                    continue
+                fused_cell = rt.DwPw.create(self.steps[step_index[dw.name]][1], self.steps[step_index[l.name]][1])
+                if fused_cell is None:
+                    continue
+                self.steps[step_index[l.name]] = (l, fused_cell, (lambda c, i, o: c.forward(i[0], o)))
+                ins_of[l.name] = ins_of[dw.name]
+                self.folded.add(dw.name)
+                self.dw_pws[l.name] = dw
         self.bottlenecks, self.bottleneck_layers = {}, {}
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
@@ -683,6 +711,8 @@ class GpuNet:
             total += self.fused_sums[l.name][1].w.size
         if l.name in self.stem_pools:       # the convolution's weights; its output never leaves the chip
             total += self.stem_pools[l.name].w.size
+        if l.name in self.dw_pws:           # the depthwise weights; its output never leaves the chip
+            total += self.dw_pws[l.name].w.size
         if l.name in self.tail_layers:      # the reduction's weights and output; its input never leaves the chip
             r = self.tail_layers[l.name]
             z = self.tensors[r.name]
@@ -697,6 +727,9 @@ class GpuNet:
             return self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
         if l.name in self.stem_pools:
             return self.layer_macs(self.stem_pools[l.name])
+        if l.name in self.dw_pws:
+            dw = self.dw_pws[l.name]
+            return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size + self.B * dw.out_shape[1] * dw.out_shape[2] * dw.w.size
         if l.type == "conv":
             return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
         if l.type == "fc":

@@ -172,6 +172,32 @@ class ExpandReduce:
             self.handle = None
 
 
+class DwPw:
+    """n2d2hip_dw_pw_t: a 3x3 depthwise convolution and the 1x1 convolution reading it in one launch; None when the library
+    keeps the cells apart."""
+
+    def __init__(self, handle, cells):
+        self.handle, self._cells = handle, cells
+
+    @staticmethod
+    def create(depthwise, pointwise):
+        h = C.c_void_p()
+        rc = lib.n2d2hip_dw_pw_create(depthwise.handle, pointwise.handle, C.byref(h))
+        if rc == capi.ERR_UNSUPPORTED:
+            return None
+        check(rc)
+        return DwPw(h, (depthwise, pointwise))
+
+    def forward(self, x, out):
+        check(lib.n2d2hip_dw_pw_forward(self.handle, x.ref, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None) and lib is not None:
+            lib.n2d2hip_dw_pw_destroy(self.handle)
+            self.handle = None
+
+
 def scaling_forward(act, x, out_dtype=None):
     out = DTensor(x.B, x.C, x.H, x.W, out_dtype if out_dtype is not None else act.out_dtype(), x.layout)
     check(lib.n2d2hip_scaling_forward(act.handle, x.ref, out.ref, stream_ptr()))

@@ -807,6 +807,49 @@ def sum_spec_for(O, rng):
     return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(0, 3, size=O)], 1), nb_bits=8, unsigned_out=True)
 
 
+@pytest.mark.parametrize("case", [(3, 32, 64, 1, 19, 21, 1), (2, 64, 128, 2, 23, 17, 1), (2, 128, 128, 1, 14, 14, 1), (2, 128, 256, 2, 28, 28, 1),
+                                  (1, 256, 512, 2, 9, 10, 0), (2, 192, 64, 1, 8, 16, 1)],
+                         ids=lambda c: "x".join(str(v) for v in c))
+def test_depthwise_and_pointwise_in_one_launch_bit_exact(rt, case):
+    """n2d2hip_dw_pw_*: a 3x3 depthwise convolution and the 1x1 convolution reading it as one launch, against the oracle
+    running the two cells and against the two separate launches; shapes whose tiles end unevenly in both directions,
+    every chunk width and channel-tile count, unsigned and signed depthwise outputs."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    B, Cc, O, stride, H, W, pad = case
+    _say("dw_pw %s" % (case,))
+    signed_mid = Cc == 128 and O == 128
+    x = _u8((B, Cc, H, W))
+    wd = _i8((Cc, 1, 3, 3))
+    bd = RNG.integers(-2000, 2001, size=Cc).astype(np.int32)
+    wp = _i8((O, Cc, 1, 1))
+    bp = RNG.integers(-20000, 20001, size=O).astype(np.int32)
+    from oracle.cells import ActSpec
+    if signed_mid:
+        sd = ActSpec("Linear", "FixedMult32", RNG.integers(2 ** 13, 2 ** 14, size=Cc), frac_bits=21, nb_bits=8, unsigned_out=False)
+    else:
+        sd = ActSpec("Rectifier", "FixedMult32", RNG.integers(2 ** 13, 2 ** 14, size=Cc), frac_bits=20, nb_bits=8, unsigned_out=True)
+    sp = ActSpec("Rectifier", "FixedMult32", RNG.integers(2 ** 13, 2 ** 14, size=O), frac_bits=16 + (Cc // 32) % 6, nb_bits=8, unsigned_out=True)
+    mid = cells_ref.conv_cell(x, wd, bd, sd, stride=(stride, stride), pad=(pad,) * 4, groups=Cc)
+    want = cells_ref.conv_cell(mid, wp, bp, sp)
+    mid_dtype = capi.I8 if signed_mid else capi.U8B
+    dw = rt.Conv(wd, bd, rt.Act(Cc, **sd.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad,) * 4, groups=Cc)
+    pw = rt.Conv(wp, bp, rt.Act(O, **sp.kwargs()), mid_dtype)
+    xin = rt.DTensor.from_numpy(x, capi.U8B)
+    separate = pw.forward(dw.forward(xin)).to_numpy()
+    assert np.array_equal(separate, want.astype(np.int64))
+    fused = rt.DwPw.create(dw, pw)
+    assert fused is not None
+    out = rt.DTensor(B, O, want.shape[2], want.shape[3], capi.U8B)
+    got = fused.forward(xin, out).to_numpy()
+    bad = np.count_nonzero(got != want)
+    assert bad == 0, "%d of %d values differ" % (bad, want.size)
+    # a pair the kernel is not written for is declined, not run: a 5-channel-wide 1x1 convolution
+    narrow = rt.Conv(_i8((40, Cc, 1, 1)), None, rt.Act(40, **ActSpec("Rectifier", "SingleShift", RNG.integers(8, 12, size=40), nb_bits=8,
+                                                                       unsigned_out=True).kwargs()), mid_dtype)
+    assert rt.DwPw.create(dw, narrow) is None
+
+
 def test_conv_randomized_sweep(rt):
     """Seeded sweep over the pipelined kernel's shape space (channel counts that are multiples of 64, kernel sizes, strides,
     paddings, dilations, ragged pixel counts, both input types, every integer rescale and both output signednesses, inputs

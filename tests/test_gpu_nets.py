@@ -96,7 +96,16 @@ def test_mobilenet_v1_config():
     spec = nets.mobilenet_v1()
     x = np.random.default_rng(13).integers(0, 256, size=(2, 3, 224, 224))
     keep = ["conv1", "conv2_dw", "conv2_pw", "conv3_dw", "conv7_pw", "conv13_dw", "conv14_pw", "pool", "fc"]
-    _run_both(spec, x, keep)
+    net = _run_both(spec, x, keep)
+    # at this batch no pair is large enough for the one-launch depthwise + 1x1 kernel; asked for everywhere, it takes every
+    # pair with an integer rescale on 32 bits and gives the same bytes
+    assert not net.dw_pws
+    fused = nets.GpuNet(spec, x.shape[0], dw_pw="all")
+    fused.set_input(x)
+    assert len(fused.dw_pws) >= 10 and all(d.name in fused.folded for d in fused.dw_pws.values())
+    assert np.array_equal(fused.forward().to_numpy(), net.tensors[spec.output].to_numpy())
+    for n in ("conv2_pw", "conv7_pw", "conv14_pw"):
+        assert np.array_equal(fused.tensors[n].to_numpy(), net.tensors[n].to_numpy()), n
 
 
 def test_resnet18_w4a4_config():
@@ -163,6 +172,8 @@ def test_batch64_configs_full_batch_properties(config):
     assert len({logits[i].tobytes() for i in range(6)}) == 6
     want = cells.run_net(spec, base[:2])["fc"].astype(np.int64)[:, :, 0, 0]
     assert np.array_equal(logits[:2], want)
+    if config == "mobilenet_v1":       # the large pairs of depthwise + 1x1 convolutions run as one launch each
+        assert sorted(net.dw_pws) == ["conv2_pw", "conv3_pw", "conv4_pw", "conv5_pw", "conv6_pw"]
     watch = {"mobilenet_v1": ["conv1", "conv2_dw", "conv2_pw", "conv7_dw", "conv14_pw", "pool", "fc"],
              "resnet18_w4a4": ["conv1", "pool1", "conv2.1_a", "conv2.1_sum", "conv3.1_sum", "conv5.2_sum", "pool", "fc"]}[config]
     watch = [n for n in watch if n not in net.folded]
