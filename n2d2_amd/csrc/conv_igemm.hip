@@ -533,7 +533,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
             const long long bound = 128 * s + std::llabs((long long)hbias[o]);
             acc_bound[o] = bound;
             const long long mult = act->htab[2 * (size_t)cp + o], half = act->htab[3 * (size_t)cp + o];
-            if (bound >= (1ll << 23) || bound * mult + half > std::numeric_limits<int>::max())
+            if (bound >= (1ll << 23) || bound * std::llabs(mult) + std::llabs(half) > std::numeric_limits<int>::max())
                 c->preclamp = true;
         }
     } else if (act->args.kind != EPI_F32) {
@@ -543,7 +543,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     // ((v + bias) * c + d) >> e == (v * c + (d + bias * c)) >> e in wrapping 32-bit arithmetic, the pre-clamp bounds move
     // by the bias and must stay 24-bit for the multiplier.
     std::vector<int> hepi;
-    if (act->args.kind == EPI_I24 && !depthwise) {
+    if (act->args.kind == EPI_I24) {
         const int cp = act->cpad;
         hepi.assign(7 * (size_t)cp, 0);
         c->bias_folded = true;
@@ -791,6 +791,12 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.fill = zero_point(in->dtype) ? 0x80808080u : 0u;
             q.out_xor = out_xor;
             q.epi = c->act->args;
+            // rescale with the bias folded in, when no clamp has to come before the multiply and the result saturates to
+            // [0, 255]: the kernel then starts from zero and saturates while it packs
+            q.fast = c->bias_folded && c->d_epi_tab && !c->preclamp && q.epi.kind == EPI_I24 && q.epi.lo == 0 && q.epi.hi == 255;
+            q.fc = q.fast ? c->d_epi_tab + 2 * c->act->cpad : nullptr;
+            q.fd = q.fast ? c->d_epi_tab + 3 * c->act->cpad : nullptr;
+            q.fe = q.fast ? c->d_epi_tab + 4 * c->act->cpad : nullptr;
             return depthwise3x3_launch(q, d.strideX, num_cus(), stream);
         }
         const long long total = Mll * (in->cs / 4);

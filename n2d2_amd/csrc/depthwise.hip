@@ -10,12 +10,14 @@
 #include "depthwise.hpp"
 #include "depthwise_math.hpp"
 #include "epilogue.hpp"
+#include "mfma_util.hpp"
 
 namespace n2d2hip {
 
 namespace {
 
-template <int S, int KIND>
+// FAST (KIND == EPI_I24 only): the rescale is (v * c + d) >> e with the bias inside d, saturated to [0, 255] while packing.
+template <int S, int KIND, bool FAST = false>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p)
 {
     const unsigned idx = blockIdx.x * 256u + threadIdx.x;
@@ -34,9 +36,15 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
     int4 w0 = *(const int4*)(p.wb + c4);
     int4 w1 = *(const int4*)(p.wb + p.cs + c4);
     int4 w2 = *(const int4*)(p.wb + 2 * p.cs + c4);
-    int4 bias = *(const int4*)(p.wb + 3 * p.cs + c4);
+    int4 bias = {};
+    if (!FAST)
+        bias = *(const int4*)(p.wb + 3 * p.cs + c4);
     int4 ta = {}, tb = {}, tc = {}, td = {}, te = {};
-    if (KIND == EPI_I24 || KIND == EPI_I64) {
+    if (FAST) {
+        tc = *(const int4*)(p.fc + c4);
+        td = *(const int4*)(p.fd + c4);
+        te = *(const int4*)(p.fe + c4);
+    } else if (KIND == EPI_I24 || KIND == EPI_I64) {
         ta = *(const int4*)(p.epi.a + c4);
         tb = *(const int4*)(p.epi.b + c4);
         tc = *(const int4*)(p.epi.c + c4);
@@ -89,7 +97,9 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
     // loop free of waits for them (such a wait would also wait for the rows requested ahead).
 #define N2D2HIP_DW_ARRIVED(v) asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w))
     N2D2HIP_DW_ARRIVED(w0); N2D2HIP_DW_ARRIVED(w1); N2D2HIP_DW_ARRIVED(w2); N2D2HIP_DW_ARRIVED(bias);
-    if (KIND == EPI_I24 || KIND == EPI_I64) {
+    if (FAST) {
+        N2D2HIP_DW_ARRIVED(tc); N2D2HIP_DW_ARRIVED(td); N2D2HIP_DW_ARRIVED(te);
+    } else if (KIND == EPI_I24 || KIND == EPI_I64) {
         N2D2HIP_DW_ARRIVED(ta); N2D2HIP_DW_ARRIVED(tb); N2D2HIP_DW_ARRIVED(tc); N2D2HIP_DW_ARRIVED(td); N2D2HIP_DW_ARRIVED(te);
     }
 #undef N2D2HIP_DW_ARRIVED
@@ -120,11 +130,17 @@ __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p
             a1 = __builtin_amdgcn_sdot4(t2.c[1], w2.y, a1, false);
             a2 = __builtin_amdgcn_sdot4(t2.c[2], w2.z, a2, false);
             a3 = __builtin_amdgcn_sdot4(t2.c[3], w2.w, a3, false);
-            const int r0 = finish(a0, 0, ta.x, tb.x, tc.x, td.x, te.x);
-            const int r1 = finish(a1, 1, ta.y, tb.y, tc.y, td.y, te.y);
-            const int r2 = finish(a2, 2, ta.z, tb.z, tc.z, td.z, te.z);
-            const int r3 = finish(a3, 3, ta.w, tb.w, tc.w, td.w, te.w);
-            const unsigned packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+            unsigned packed;
+            if (FAST) {
+                packed = sat_bytes_u8((__mul24(a0, tc.x) + td.x) >> te.x, (__mul24(a1, tc.y) + td.y) >> te.y,
+                                      (__mul24(a2, tc.z) + td.z) >> te.z, (__mul24(a3, tc.w) + td.w) >> te.w);
+            } else {
+                const int r0 = finish(a0, 0, ta.x, tb.x, tc.x, td.x, te.x);
+                const int r1 = finish(a1, 1, ta.y, tb.y, tc.y, td.y, te.y);
+                const int r2 = finish(a2, 2, ta.z, tb.z, tc.z, td.z, te.z);
+                const int r3 = finish(a3, 3, ta.w, tb.w, tc.w, td.w, te.w);
+                packed = ((unsigned)r0 & 255u) | (((unsigned)r1 & 255u) << 8) | (((unsigned)r2 & 255u) << 16) | ((unsigned)r3 << 24);
+            }
             if (q + i < nrows)
                 outp[(q + i) * out_row] = packed ^ p.out_xor;
             if (S == 1) {
@@ -168,7 +184,10 @@ int depthwise3x3_launch(DepthwiseArgs a, int stride, int num_cus, hipStream_t st
     a.nthreads = (unsigned)nthreads;
     const unsigned grid = (unsigned)((nthreads + 255) / 256);
 #define N2D2HIP_DW_LAUNCH(S, K) hipLaunchKernelGGL((depthwise3x3_kernel<S, K>), dim3(grid), dim3(256), 0, stream, a)
-    if (a.epi.kind == EPI_I24) {
+    if (a.epi.kind == EPI_I24 && a.fast) {
+        if (stride == 1) hipLaunchKernelGGL((depthwise3x3_kernel<1, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((depthwise3x3_kernel<2, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+    } else if (a.epi.kind == EPI_I24) {
         if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_I24); else N2D2HIP_DW_LAUNCH(2, EPI_I24);
     } else if (a.epi.kind == EPI_I64) {
         if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_I64); else N2D2HIP_DW_LAUNCH(2, EPI_I64);

@@ -20,6 +20,12 @@ struct DepthwiseArgs {
     unsigned fill;           // the stored form of 0 in all four bytes
     unsigned out_xor;        // 0x80808080 when the output is stored as value - 128
     EpiArgs epi;
+    // fast form of the integer rescale (no clamp before the multiply, saturation to [0, 255]): multiplier, rounding term
+    // with the bias folded in, shift; by channel
+    bool fast;
+    const int* fc;
+    const int* fd;
+    const int* fe;
 };
 
 // Host side of the layout above: `w` is [C][3][3] int8, `bias` the biases with the zero point folded in.

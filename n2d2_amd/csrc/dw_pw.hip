@@ -45,7 +45,9 @@ namespace {
 // of the 1x1 convolution's outputs a work-group computes (blockIdx.y selects which 32 * NB of them); WAVES: 4, or 8 with
 // the channel blocks split between the two halves of the work-group (half the accumulators per wave, half the rows per
 // thread in the depthwise part).
-template <int S, int KC, int NB, int WAVES>
+// FAST: neither cell needs a clamp before its multiply and both saturate to [0, 255]: the depthwise tables c, d, e are then
+// the ones with the bias folded in (accumulators start from zero), and both rescales saturate while they pack.
+template <int S, int KC, int NB, int WAVES, bool FAST>
 __global__ __launch_bounds__(64 * WAVES) void dw_pw_kernel(const DwPwArgs q)
 {
     constexpr int THREADS = 64 * WAVES;
@@ -128,9 +130,12 @@ __global__ __launch_bounds__(64 * WAVES) void dw_pw_kernel(const DwPwArgs q)
             const int4 w0 = *(const int4*)(q.wdw + ch);
             const int4 w1 = *(const int4*)(q.wdw + q.C + ch);
             const int4 w2 = *(const int4*)(q.wdw + 2 * q.C + ch);
-            const int4 bias = *(const int4*)(q.wdw + 3 * q.C + ch);
-            const int4 ta = *(const int4*)(q.dwe.a + ch);
-            const int4 tb = *(const int4*)(q.dwe.b + ch);
+            int4 bias = {}, ta = {}, tb = {};
+            if (!FAST) {
+                bias = *(const int4*)(q.wdw + 3 * q.C + ch);
+                ta = *(const int4*)(q.dwe.a + ch);
+                tb = *(const int4*)(q.dwe.b + ch);
+            }
             const int4 tc = *(const int4*)(q.dwe.c + ch);
             const int4 td = *(const int4*)(q.dwe.d + ch);
             const int4 te = *(const int4*)(q.dwe.e + ch);
@@ -176,12 +181,18 @@ __global__ __launch_bounds__(64 * WAVES) void dw_pw_kernel(const DwPwArgs q)
                     a1 = __builtin_amdgcn_sdot4(t2.c[1], w2.y, a1, false);
                     a2 = __builtin_amdgcn_sdot4(t2.c[2], w2.z, a2, false);
                     a3 = __builtin_amdgcn_sdot4(t2.c[3], w2.w, a3, false);
-                    const int v0r = epi_apply<EPI_I24>(a0, ta.x, tb.x, tc.x, td.x, te.x, q.dwe.lo, q.dwe.hi, 0);
-                    const int v1r = epi_apply<EPI_I24>(a1, ta.y, tb.y, tc.y, td.y, te.y, q.dwe.lo, q.dwe.hi, 0);
-                    const int v2r = epi_apply<EPI_I24>(a2, ta.z, tb.z, tc.z, td.z, te.z, q.dwe.lo, q.dwe.hi, 0);
-                    const int v3r = epi_apply<EPI_I24>(a3, ta.w, tb.w, tc.w, td.w, te.w, q.dwe.lo, q.dwe.hi, 0);
-                    const unsigned packed = (((unsigned)v0r & 255u) | (((unsigned)v1r & 255u) << 8) | (((unsigned)v2r & 255u) << 16)
-                                             | ((unsigned)v3r << 24)) ^ q.mid_xor;
+                    unsigned packed;
+                    if (FAST) {
+                        packed = sat_bytes_u8((__mul24(a0, tc.x) + td.x) >> te.x, (__mul24(a1, tc.y) + td.y) >> te.y,
+                                              (__mul24(a2, tc.z) + td.z) >> te.z, (__mul24(a3, tc.w) + td.w) >> te.w);
+                    } else {
+                        const int v0r = epi_apply<EPI_I24>(a0, ta.x, tb.x, tc.x, td.x, te.x, q.dwe.lo, q.dwe.hi, 0);
+                        const int v1r = epi_apply<EPI_I24>(a1, ta.y, tb.y, tc.y, td.y, te.y, q.dwe.lo, q.dwe.hi, 0);
+                        const int v2r = epi_apply<EPI_I24>(a2, ta.z, tb.z, tc.z, td.z, te.z, q.dwe.lo, q.dwe.hi, 0);
+                        const int v3r = epi_apply<EPI_I24>(a3, ta.w, tb.w, tc.w, td.w, te.w, q.dwe.lo, q.dwe.hi, 0);
+                        packed = ((unsigned)v0r & 255u) | (((unsigned)v1r & 255u) << 8) | (((unsigned)v2r & 255u) << 16) | ((unsigned)v3r << 24);
+                    }
+                    packed ^= q.mid_xor;
                     const int m = (rh * ROWS + r0 + i) * 16 + x;
                     *(unsigned*)(abuf + m * 64 + (((cg >> 2) ^ ((m >> 1) & 3)) << 4) + ((cg & 3) << 2)) = packed;
                     if (S == 1) {
@@ -226,15 +237,22 @@ __global__ __launch_bounds__(64 * WAVES) void dw_pw_kernel(const DwPwArgs q)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int ch = (wn * NBW + 2 * j + i) * 32 + 8 * g + 4 * lh;
-                const v4i ta = *(const v4i*)(tab + ch), tb = *(const v4i*)(tab + NT + ch), tc = *(const v4i*)(tab + 2 * NT + ch),
-                          td = *(const v4i*)(tab + 3 * NT + ch), te = *(const v4i*)(tab + 4 * NT + ch);
+                const v4i tc = *(const v4i*)(tab + 2 * NT + ch), td = *(const v4i*)(tab + 3 * NT + ch), te = *(const v4i*)(tab + 4 * NT + ch);
                 int r[4];
+                if (FAST) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int t = med3_i32(acc[2 * j + i][4 * g + e], ta[e], tb[e]);
-                    r[e] = med3_i32((__mul24(t, tc[e]) + td[e]) >> te[e], q.pw_lo, q.pw_hi);
+                    for (int e = 0; e < 4; ++e)
+                        r[e] = (__mul24(acc[2 * j + i][4 * g + e], tc[e]) + td[e]) >> te[e];
+                    pk[i][g] = sat_bytes_u8(r[0], r[1], r[2], r[3]) ^ q.out_xor;
+                } else {
+                    const v4i ta = *(const v4i*)(tab + ch), tb = *(const v4i*)(tab + NT + ch);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int t = med3_i32(acc[2 * j + i][4 * g + e], ta[e], tb[e]);
+                        r[e] = med3_i32((__mul24(t, tc[e]) + td[e]) >> te[e], q.pw_lo, q.pw_hi);
+                    }
+                    pk[i][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ q.out_xor;
                 }
-                pk[i][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ q.out_xor;
             }
         }
         // exchange between the lane halves until a lane owns 32 consecutive channels of the pair of blocks
@@ -267,15 +285,18 @@ bool plain_1x1(const n2d2hip_conv_desc& d)
 
 int byte_type_of(const n2d2hip_act_s* a) { return a->min_out >= 0 ? N2D2HIP_U8B : N2D2HIP_I8; }
 
-#ifndef WAVES_NB4
-#define WAVES_NB4 4
-#endif
-template <int S, int KC>
+template <int S, int KC, bool FAST>
 void launch_nb(const DwPwArgs& a, int nb, dim3 grid, hipStream_t stream)
 {
-    if (nb == 8) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 8, 8>), grid, dim3(512), 0, stream, a);
-    else if (nb == 4) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 4, WAVES_NB4>), grid, dim3(64 * WAVES_NB4), 0, stream, a);
-    else hipLaunchKernelGGL((dw_pw_kernel<S, KC, 2, 4>), grid, dim3(256), 0, stream, a);
+    if (nb == 8) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 8, 8, FAST>), grid, dim3(512), 0, stream, a);
+    else if (nb == 4) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 4, 4, FAST>), grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((dw_pw_kernel<S, KC, 2, 4, FAST>), grid, dim3(256), 0, stream, a);
+}
+
+template <int S, int KC>
+void launch_fast(const DwPwArgs& a, bool fast, int nb, dim3 grid, hipStream_t stream)
+{
+    if (fast) launch_nb<S, KC, true>(a, nb, grid, stream); else launch_nb<S, KC, false>(a, nb, grid, stream);
 }
 
 } // namespace
@@ -286,6 +307,7 @@ using namespace n2d2hip;
 struct n2d2hip_dw_pw_s {
     n2d2hip_conv_t dw, pw;
     int kc, nb;               // channels per chunk, 32-channel blocks per work-group
+    bool fast;                // neither rescale clamps before its multiply, both saturate to [0, 255]
     signed char* d_w;
     int* d_tab;
 };
@@ -348,6 +370,8 @@ int n2d2hip_dw_pw_create(n2d2hip_conv_t dw, n2d2hip_conv_t pw, n2d2hip_dw_pw_t* 
         }
     n2d2hip_dw_pw_s* h = new n2d2hip_dw_pw_s();
     h->dw = dw; h->pw = pw; h->kc = kc; h->nb = nb; h->d_w = nullptr; h->d_tab = nullptr;
+    h->fast = dw->bias_folded && dw->d_epi_tab && !dw->preclamp && dw->act->args.lo == 0 && dw->act->args.hi == 255
+        && !pw->preclamp && pw->act->args.lo == 0 && pw->act->args.hi == 255;
     e = hipMalloc((void**)&h->d_w, img.size());
     if (e == hipSuccess) e = hipMemcpy(h->d_w, img.data(), img.size(), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipMalloc((void**)&h->d_tab, tab.size() * sizeof(int));
@@ -384,6 +408,10 @@ int n2d2hip_dw_pw_forward(n2d2hip_dw_pw_t h, const n2d2hip_tensor* in, const n2d
     DwPwArgs a;
     a.in = (const signed char*)in->data; a.out = (signed char*)out->data;
     a.wdw = h->dw->d_wdw; a.dwe = h->dw->act->args;
+    if (h->fast) {
+        const int cpd = h->dw->act->cpad;
+        a.dwe.c = h->dw->d_epi_tab + 2 * cpd; a.dwe.d = h->dw->d_epi_tab + 3 * cpd; a.dwe.e = h->dw->d_epi_tab + 4 * cpd;
+    }
     a.wpw = h->d_w; a.pwt = h->d_tab;
     a.C = dd.C; a.O = dp.O;
     a.B = in->B; a.H = in->H; a.W = in->W; a.OH = OH; a.OW = OW; a.padL = dd.padL; a.padT = dd.padT;
@@ -407,9 +435,9 @@ int n2d2hip_dw_pw_forward(n2d2hip_dw_pw_t h, const n2d2hip_tensor* in, const n2d
     a.out_bytes = (unsigned)((long long)out->B * OH * OW * out->cs);
     const dim3 grid((unsigned)(((a.ntiles + 7) / 8) * 8), (unsigned)(dp.O / (h->nb * 32)));
     if (dd.strideX == 1) {
-        if (h->kc == 32) launch_nb<1, 32>(a, h->nb, grid, stream); else launch_nb<1, 64>(a, h->nb, grid, stream);
+        if (h->kc == 32) launch_fast<1, 32>(a, h->fast, h->nb, grid, stream); else launch_fast<1, 64>(a, h->fast, h->nb, grid, stream);
     } else {
-        if (h->kc == 32) launch_nb<2, 32>(a, h->nb, grid, stream); else launch_nb<2, 64>(a, h->nb, grid, stream);
+        if (h->kc == 32) launch_fast<2, 32>(a, h->fast, h->nb, grid, stream); else launch_fast<2, 64>(a, h->fast, h->nb, grid, stream);
     }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;

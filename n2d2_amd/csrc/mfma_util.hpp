@@ -45,6 +45,12 @@ __device__ __forceinline__ unsigned sat_pk_u8(v2s x)
     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(r) : "v"(x));
     return r;
 }
+// four 32-bit values saturated to [0, 255], one byte each (first value in the lowest byte)
+__device__ __forceinline__ unsigned sat_bytes_u8(int r0, int r1, int r2, int r3)
+{
+    const v2s lo = __builtin_amdgcn_cvt_pk_i16(r0, r1), hi = __builtin_amdgcn_cvt_pk_i16(r2, r3);   // saturating
+    return sat_pk_u8(lo) | (sat_pk_u8(hi) << 16);
+}
 template <int N>
 __device__ __forceinline__ void wait_loads_and_barrier()
 {
