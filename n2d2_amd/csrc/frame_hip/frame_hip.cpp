@@ -462,7 +462,8 @@ ConvCell_Frame_HIP<T>::ConvCell_Frame_HIP(const DeepNet& /*deepNet*/, const std:
                                           unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
                                           const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
                                           const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr), mConvInDType(-1)
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr), mConvInDType(-1),
+      mDwPw(nullptr), mFusedDw(nullptr)
 {
     mActivation = activation;
 }
@@ -470,7 +471,36 @@ ConvCell_Frame_HIP<T>::ConvCell_Frame_HIP(const DeepNet& /*deepNet*/, const std:
 template <class T>
 ConvCell_Frame_HIP<T>::~ConvCell_Frame_HIP()
 {
+    if (mDwPw) n2d2hip_dw_pw_destroy(mDwPw);
     if (mConv) n2d2hip_conv_destroy(mConv);
+}
+
+template <class T>
+bool ConvCell_Frame_HIP<T>::fuseDepthwise(Cell_Frame_HIP* depthwise)
+{
+    if (mDwPw || !mConv || !depthwise || !depthwise->convHandle() || depthwise->foldedInto() || foldedInto() || mInputs.size() != 1
+        || mNbOutputs > 256 || (long long)mBatch * mOutH * mOutW < 32768 || depthwise->inputTensor(0)->desc().halo != 0)
+        return false;
+    n2d2hip_dw_pw_t fused = nullptr;
+    const int rc = n2d2hip_dw_pw_create(depthwise->convHandle(), mConv, &fused);
+    if (rc == N2D2HIP_ERR_UNSUPPORTED)
+        return false;
+    checkStatus(rc);
+    mDwPw = fused;
+    mFusedDw = depthwise;
+    depthwise->setFoldedInto(this);
+    return true;
+}
+
+template <class T>
+void ConvCell_Frame_HIP<T>::clearFusion()
+{
+    if (mDwPw) {
+        n2d2hip_dw_pw_destroy(mDwPw);
+        mDwPw = nullptr;
+        mFusedDw->setFoldedInto(nullptr);
+        mFusedDw = nullptr;
+    }
 }
 
 template <class T>
@@ -506,7 +536,10 @@ void ConvCell_Frame_HIP<T>::propagate(bool /*inference*/)
 template <class T>
 void ConvCell_Frame_HIP<T>::launch()
 {
-    checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    if (mDwPw)
+        checkStatus(n2d2hip_dw_pw_forward(mDwPw, &mFusedDw->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
+    else
+        checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
 
@@ -517,6 +550,7 @@ bool ConvCell_Frame_HIP<T>::prepare()
     const int inDType = mInputs[0]->desc().dtype;
     bool rebuilt = false;
     if (mDirty || act != mConvAct || !mConv || inDType != mConvInDType) {
+        clearFusion();
         if (mConv) { n2d2hip_conv_destroy(mConv); mConv = nullptr; }
         const unsigned int cg = mNbChannels / mNbGroups;
         if (mWeights.dimX() != mKernelDims[0] || mWeights.dimY() != mKernelDims[1] || mWeights.dimZ() != cg || mWeights.dimB() != mNbOutputs)
@@ -1406,6 +1440,8 @@ void DeepNet::setFusion(bool enabled)
                 ew->clearFusion();
             if (auto* pool = dynamic_cast<PoolCell_Frame_HIP<float>*>(f))
                 pool->clearFusion();
+            if (auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f))
+                conv->clearFusion();
             f->setOutputsHalo(0);
         }
     }
@@ -1437,6 +1473,15 @@ void DeepNet::planFusion()
         const std::vector<Cell_Frame_HIP*>& parents = pool->parentCells();
         if (parents.size() == 1 && parents[0] && consumers[parents[0]] == 1)
             pool->fuseFirstConv(parents[0]);
+    }
+    // a 1x1 convolution that is the only reader of a 3x3 depthwise convolution computes it in its own launch
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f);
+        if (!conv) continue;
+        conv->clearFusion();
+        const std::vector<Cell_Frame_HIP*>& parents = conv->parentCells();
+        if (parents.size() == 1 && parents[0] && consumers[parents[0]] == 1)
+            conv->fuseDepthwise(parents[0]);
     }
     for (Cell_Frame_HIP* f : mFrames) {
         auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
@@ -1477,7 +1522,9 @@ void DeepNet::planFusion()
         }
     }
     for (Cell_Frame_HIP* f : mFrames) {
-        const bool writes = f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle());
+        auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f);
+        const bool writes = f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle())
+            && !(conv && conv->computesDepthwise());
         f->setOutputsHalo(writes && !refused[f] ? halo[f] : 0);
     }
     mPlanned = true;

@@ -524,6 +524,13 @@ public:
     void launch();
     n2d2hip_conv_t convHandle() const { return mConv; }
     int maxPadding() const { return std::max(mPaddingDims[0], mPaddingDims[1]); }
+    // Graph-level fusion (DeepNet::planFusion): this 1x1 convolution computes the 3x3 depthwise convolution `depthwise`,
+    // whose output it alone reads, in its own launch (n2d2hip_dw_pw_*); the depthwise cell is then not launched and its
+    // output never written.  Taken where the device library accepts the pair and one launch is expected to be faster than
+    // two: at most 256 outputs, at least 32768 output pixels in the batch.
+    bool fuseDepthwise(Cell_Frame_HIP* depthwise);
+    void clearFusion();
+    bool computesDepthwise() const { return mDwPw != nullptr; }
 
 protected:
     void setOutputsDims();
@@ -532,6 +539,8 @@ private:
     n2d2hip_conv_t mConv;
     n2d2hip_act_t mConvAct;
     int mConvInDType;
+    n2d2hip_dw_pw_t mDwPw;
+    Cell_Frame_HIP* mFusedDw;
     static Registrar<ConvCell> mRegistrar;
 };
 

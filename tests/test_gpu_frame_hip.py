@@ -155,6 +155,33 @@ def test_depthwise_cell_from_its_connection_map(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+def test_depthwise_and_pointwise_cells_run_as_one_launch(fh):
+    """DeepNet::planFusion gives a 3x3 depthwise ConvCell to the 1x1 ConvCell that alone reads it where the pair is large
+    enough: MobileNet at 256 x 256, batch 8 (blocks 2 to 4); same logits as the oracle and as the cells launched apart,
+    and the depthwise outputs are not there to read."""
+    from n2d2_amd import nets
+    from oracle import cells
+    spec = nets.mobilenet_v1(image=256)
+    x = np.random.default_rng(36).integers(0, 256, size=(8, 3, 256, 256))
+    net = fh.build_net(spec, 8)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    want = cells.run_net(spec, x[:2], keep=["conv2_pw", "conv4_pw", "fc"])
+    assert net.nb_folded == 3
+    for name in ("conv2_pw", "conv4_pw", "fc"):
+        assert np.array_equal(net.outputs(name)[:2], want[name]), name
+    with pytest.raises(fh.FrameHipError) as e:
+        net.outputs("conv3_dw")
+    assert "not materialised" in str(e.value)
+    fused_logits = net.outputs("fc").copy()
+    net.set_fusion(False)
+    net.propagate()
+    assert net.nb_folded == 0
+    assert np.array_equal(net.outputs("fc"), fused_logits)
+    assert np.array_equal(net.outputs("conv3_dw")[:2], cells.run_net(spec, x[:2], keep=["conv3_dw"])["conv3_dw"])
+
+
 def test_signedness_change_rebuilds_the_cells(fh):
     """-no-unsigned (DeepNetExport::mUnsignedData = false): every cell saturates to the signed range."""
     from n2d2_amd import nets
