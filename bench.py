@@ -56,7 +56,7 @@ def class_rooflines(net, per_launch_ms, step_ms):
         floor_ms += max(t_mfma, t_hbm)
         if l.type == "conv" and getattr(l, "groups", 1) > 1:
             name = "depthwise_hbm_bound"
-        elif l.type in ("conv", "fc") or l.name in net.fused_sums:
+        elif l.type in ("conv", "fc") or l.name in net.fused_sums or l.name in net.stem_pools:
             name = "mfma_bound" if t_mfma > t_hbm else "hbm_bound"
         else:
             name = "bandwidth_cells_hbm_bound"
@@ -73,6 +73,24 @@ def class_rooflines(net, per_launch_ms, step_ms):
     out["floor_ms"] = round(floor_ms, 4)               # sum over launches of the larger bound
     out["floor_frac"] = round(floor_ms / step_ms, 4)   # of the measured step
     return out
+
+
+def launch_floor_us(torch, n=64):
+    """What one kernel launch costs inside a replayed HIP graph when it depends on the one before it and does next to no
+    work: n one-wave kernels, one behind the other, in one graph; median replay time / n."""
+    import numpy as np
+    t = torch.zeros(64, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        t.add_(1)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(n):
+                t.add_(1)
+    torch.cuda.synchronize()
+    ms, _, _ = median_step_ms(torch, graph.replay, 20, 3)
+    return ms * 1000.0 / n
 
 
 def median_step_ms(torch, step, steps, warmup, per_call=1):
@@ -409,6 +427,11 @@ def main():
     runs = [net.forward_timed() for _ in range(7)]
     per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
     by_class = class_rooflines(net, per_launch, ms)
+    # the same floor with what the launches themselves cost (measured on this GPU, in this run) added to it
+    floor_us = launch_floor_us(torch)
+    by_class["launch_floor_us"] = round(floor_us, 2)
+    by_class["floor_with_launches_ms"] = round(by_class["floor_ms"] + len(net.launched) * floor_us * 1e-3, 4)
+    by_class["floor_with_launches_frac"] = round(by_class["floor_with_launches_ms"] / ms, 4)
 
     # Two batches in flight: a second, independent forward of the same network on another batch of the same size runs on
     # its own stream, so each stream's launch gaps and tails are filled by the other's kernels.  Reported next to `value`
