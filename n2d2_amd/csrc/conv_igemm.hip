@@ -389,14 +389,21 @@ void launch_pipe(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t str
 #undef N2D2HIP_PIPE
 }
 
+// narrow: at most 32 output channels and the integer rescale: one 32-channel block per work-group
 template <int KH>
-void launch_stem(const ConvStemArgs& a, bool hi16, int grid, hipStream_t stream)
+void launch_stem(const ConvStemArgs& a, bool hi16, bool narrow, int grid, hipStream_t stream)
 {
     switch (a.c.epi.kind) {
     case EPI_RAW: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_RAW>), dim3(grid), dim3(256), 0, stream, a); break;
     case EPI_I24:
-        if (hi16) hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
-        else hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a);
+        if (narrow) {
+            if (hi16) hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true, false, 1>), dim3(grid), dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, false, false, 1>), dim3(grid), dim3(256), 0, stream, a);
+        } else if (hi16) {
+            hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a);
+        }
         break;
     default: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_F32>), dim3(grid), dim3(256), 0, stream, a); break;
     }
@@ -979,7 +986,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.preclamp = c->preclamp ? 1 : 0;
             q.tiles_per_row = (OW + 127) / 128;
             q.ntiles = in->B * OH * q.tiles_per_row;
-            q.c.ntiles_n = (round_up(d.O, 16) + 63) / 64;
+            const bool narrow = k == EPI_I24 && round_up(d.O, 16) <= 32;
+            q.c.ntiles_n = narrow ? 1 : (round_up(d.O, 16) + 63) / 64;
             q.nlanes = std::max(1, std::min((q.ntiles + 7) / 8, (3 * num_cus()) / (8 * q.c.ntiles_n)));
             q.xcd_tiles = (q.ntiles + 7) / 8;
             magic_div((unsigned)OH, &q.oh_mul, &q.oh_sh);
@@ -987,9 +995,9 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             const int grid = 8 * q.nlanes * q.c.ntiles_n;
             const bool hi16 = k == EPI_I24 && c->hi16 && is_byte_type(out->dtype) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
             if (hi16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
-            if (d.kH == 3) launch_stem<3>(q, hi16, grid, stream);
-            else if (d.kH == 5) launch_stem<5>(q, hi16, grid, stream);
-            else launch_stem<7>(q, hi16, grid, stream);
+            if (d.kH == 3) launch_stem<3>(q, hi16, narrow, grid, stream);
+            else if (d.kH == 5) launch_stem<5>(q, hi16, narrow, grid, stream);
+            else launch_stem<7>(q, hi16, narrow, grid, stream);
             N2D2HIP_HIP_CHECK(hipGetLastError());
             return N2D2HIP_OK;
         }

@@ -50,9 +50,12 @@ struct ConvStemArgs {
     int pool_halo, POHp, POWp;   // border of the pooled tensor and its rows / columns with it
 };
 
-template <int KH, int EPI, bool H16 = false, bool POOL = false>
+// NBLK: 32-channel blocks of outputs a work-group computes: 2, or 1 for a layer of at most 32 output channels (half the
+// matrix instructions and half the rescale).
+template <int KH, int EPI, bool H16 = false, bool POOL = false, int NBLK = 2>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) void conv_stem_kernel(ConvStemArgs q)
 {
+    static_assert(NBLK == 2 || (NBLK == 1 && !POOL), "the pooled variant works on 64 channels");
     static_assert(!H16 || EPI == EPI_I24, "scaled-up tables belong to the integer rescale");
     static_assert(!POOL || H16, "the pooled variant is written for byte outputs of the integer rescale");
     const ConvArgs& p = q.c;
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     constexpr int NCHUNK = KH * 5;             // 256-byte chunks per stage
     constexpr int NLOAD = (NCHUNK + 3) / 4;    // per wave (chunks past the end land in the spare row)
     constexpr int STAGE = (KH + 1) * PITCH;
-    constexpr int BN = 64;
+    constexpr int BN = 32 * NBLK;
     constexpr int TAB_OFF = 3 * STAGE;
     constexpr bool BIAS_ADD = EPI != EPI_I24;  // the integer rescale carries the bias in its tables
     constexpr int ROWS_OFF = TAB_OFF + 6 * BN * 4;             // POOL: four convolution rows of TW pixels x 64 bytes
@@ -148,9 +151,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
     issue(1, 1);
 
     // ---- weights of this lane's channels: A operand of kernel row ky is 16 bytes at ky*32 + 16*lh
-    v4i wf[2][KH];
+    v4i wf[NBLK][KH];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NBLK; ++i)
 #pragma unroll
         for (int ky = 0; ky < KH; ++ky)
             wf[i][ky] = *(const v4i*)(q.wk + (long long)(n0 + i * 32 + l32) * (KH * 32) + ky * 32 + 16 * lh);
@@ -170,10 +173,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         }
     }
     __syncthreads();
-    v4i rc[H16 ? 2 : 1][H16 ? 4 : 1], rd[H16 ? 2 : 1][H16 ? 4 : 1];
+    v4i rc[H16 ? NBLK : 1][H16 ? 4 : 1], rd[H16 ? NBLK : 1][H16 ? 4 : 1];
     if (H16) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < NBLK; ++i)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 rc[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(p.epi.c + n0 + i * 32 + 8 * g + 4 * lh);
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(NLOAD) : "memory");
         issue(t + 2, (t + 2) % 3);
 
-        v16i acc[2];
+        v16i acc[NBLK];
         {
             typedef int v2i __attribute__((ext_vector_type(2)));
             v2i lo[KH], hi[KH];
@@ -207,13 +210,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
             for (int ky = 0; ky < KH; ++ky) {
                 asm volatile("" : "+v"(lo[ky]), "+v"(hi[ky]));
                 const v4i pf = {lo[ky][0], lo[ky][1], hi[ky][0], hi[ky][1]};
-                if (ky == 0) {
-                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][ky], pf, v16i{}, 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][ky], pf, v16i{}, 0, 0, 0);
-                } else {
-                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][ky], pf, acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][ky], pf, acc[1], 0, 0, 0);
-                }
+#pragma unroll
+                for (int i = 0; i < NBLK; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][ky], pf, ky == 0 ? v16i{} : acc[i], 0, 0, 0);
             }
         }
 
@@ -223,9 +222,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
         const int ox = POOL ? 32 * wave + l32 : (id - rowid * q.tiles_per_row) * TW + 32 * wave + l32;
         const long long m = (long long)rowid * p.OW + ox;
         const bool pix_ok = ox < p.OW;
-        unsigned pk[2][4];
+        unsigned pk[NBLK][4];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < NBLK; ++i) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 if constexpr (H16) {
@@ -289,19 +288,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
             }
         }
         if (out_bytes) {
-            unsigned qd[2][4];
+            unsigned qd[NBLK][4];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < NBLK; ++i) {
                 const auto s02 = __builtin_amdgcn_permlane32_swap(pk[i][0], pk[i][2], false, false);
                 const auto s13 = __builtin_amdgcn_permlane32_swap(pk[i][1], pk[i][3], false, false);
                 qd[i][0] = s02[0]; qd[i][1] = s02[1]; qd[i][2] = s13[0]; qd[i][3] = s13[1];
             }
             v4i first, second;
+            if constexpr (NBLK == 2) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const auto x = __builtin_amdgcn_permlane32_swap(qd[0][e], qd[1][e], false, false);
-                first[e] = (int)x[0];
-                second[e] = (int)x[1];
+                for (int e = 0; e < 4; ++e) {
+                    const auto x = __builtin_amdgcn_permlane32_swap(qd[0][e], qd[NBLK - 1][e], false, false);
+                    first[e] = (int)x[0];
+                    second[e] = (int)x[1];
+                }
+            } else {
+                // one block: the lower lane half holds channels 0..15 of its pixel, the upper half channels 16..31
+                first = v4i{(int)qd[0][0], (int)qd[0][1], (int)qd[0][2], (int)qd[0][3]};
+                second = first;
             }
             if constexpr (POOL) {
                 // the row goes to the ring in LDS (a row that does not exist: the smallest byte, which no maximum picks);
@@ -351,11 +356,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) voi
                     }
                 }
             } else {
-            signed char* orow = (signed char*)p.out + m * p.out_cs + n0 + 32 * lh;
-            const int ch = n0 + 32 * lh;
-            if (pix_ok) {
-                if (ch < p.out_cs) *(v4i*)orow = first;
-                if (ch + 16 < p.out_cs) *(v4i*)(orow + 16) = second;
+            if constexpr (NBLK == 2) {
+                signed char* orow = (signed char*)p.out + m * p.out_cs + n0 + 32 * lh;
+                const int ch = n0 + 32 * lh;
+                if (pix_ok) {
+                    if (ch < p.out_cs) *(v4i*)orow = first;
+                    if (ch + 16 < p.out_cs) *(v4i*)(orow + 16) = second;
+                }
+            } else {
+                const int ch = n0 + 16 * lh;
+                if (pix_ok && ch < p.out_cs)
+                    *(v4i*)((signed char*)p.out + m * p.out_cs + ch) = first;
             }
             }
         }

@@ -150,6 +150,7 @@ CONV_CASES = [
     ("3x3_s2_c32", 2, 32, 15, 17, 48, (3, 3), (2, 2), (1, 1, 1, 1), (1, 1), "u8"),
     ("stem7x7_c3", 2, 3, 37, 41, 64, (7, 7), (2, 2), (3, 3, 3, 3), (1, 1), "u8"),
     ("stem3x3_c3", 2, 3, 20, 20, 32, (3, 3), (2, 2), (1, 1, 1, 1), (1, 1), "u8"),
+    ("stem5x5_c3_o20", 3, 3, 45, 301, 20, (5, 5), (2, 2), (2, 2, 2, 2), (1, 1), "i8"),
     ("lenet5x5_c1", 4, 1, 32, 32, 6, (5, 5), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
     ("lenet5x5_c6", 4, 6, 14, 14, 16, (5, 5), (1, 1), (0, 0, 0, 0), (1, 1), "u8"),
     ("c20_o10_asym", 2, 20, 9, 8, 10, (2, 5), (1, 3), (1, 2, 0, 1), (1, 1), "i8"),
