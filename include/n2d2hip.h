@@ -250,10 +250,11 @@ int n2d2hip_elemwise_destroy(n2d2hip_elemwise_t ew);
  * input is passed to n2d2hip_conv_forward_sum and has storage type `other_dtype`.  A ScalingCell folded into the sum
  * with n2d2hip_elemwise_fold_input_scaling must sit on that other input and is applied too.  `sum` is borrowed and must
  * outlive the convolution; NULL undoes the fusion.  Returns N2D2HIP_ERR_UNSUPPORTED (and changes nothing) unless the
- * convolution is 1x1, unpadded, 8-bit, with input and output channel counts that are multiples of 64, and both cells
- * rescale with an integer Scaling mode: the caller then keeps the two launches. */
+ * convolution is 1x1, unpadded and 8-bit, or undilated with 4-bit weights, with input and output channel counts that are
+ * multiples of 64, and both cells rescale with an integer Scaling mode: the caller then keeps the two launches. */
 int n2d2hip_conv_fuse_sum(n2d2hip_conv_t conv, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype);
-/* out = sum(conv(in), other) for a convolution prepared with n2d2hip_conv_fuse_sum; `out` has the sum cell's range. */
+/* out = sum(conv(in), other) for a convolution prepared with n2d2hip_conv_fuse_sum; `out` has the sum cell's range.
+ * `in`, `other` and `out` may each carry a border of zeros of their own (halo). */
 int n2d2hip_conv_forward_sum(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
                              const n2d2hip_tensor* out, n2d2hip_stream_t stream);
 int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,

@@ -761,7 +761,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     // with a folded sum the stored values are the sum cell's
     const n2d2hip_act_s* act = other ? c->sum->act : c->act;
     if (other) {
-        if ((rc = check_tensor(other, "sum input")))
+        if ((rc = check_tensor(other, "sum input", true)))
             return rc;
         N2D2HIP_REQUIRE(other->layout == N2D2HIP_NHWC && other->dtype == c->sum_other_dtype && other->B == out->B && other->C == out->C
                         && other->H == out->H && other->W == out->W && other->cs % 16 == 0 && other->cs >= round_up(d.O, 16),
@@ -909,7 +909,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.mlanes = per_xcd;
         q.xcd_tiles = (q.mtiles + 7) / 8;
         const int grid = 8 * a.ntiles_n * per_xcd;
-        q.res = nullptr; q.res_cs = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
+        q.res = nullptr; q.res_cs = 0; q.res_halo = 0; q.res_flip = 0; q.has_pre = q.pre_clamp = q.sum_clamp = 0;
         q.sum16 = nullptr; q.sum16_stride = 0; q.pre_in_range = 0;
         q.sum = EpiArgs(); q.pre = EpiArgs();
         // Byte outputs of an integer rescale whose scaled-up tables fit: the rescaled value is read from the upper half of
@@ -919,12 +919,13 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         if (w4 && !other) {
             // 4-bit weights, packed in memory and in LDS
             q.c.w = c->d_w4img;
-            return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid == 1, hi16, grid, stream);
+            return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid, hi16, grid, stream);
         }
         if (other) {
             const int cp = c->sum->act->cpad;
             q.res = (const signed char*)other->data;
             q.res_cs = other->cs;
+            q.res_halo = other->halo;
             q.res_flip = other->dtype == N2D2HIP_U8 ? 0u : 0x80808080u;
             q.sum16 = c->sum16 ? c->d_res_tab + 10 * cp : nullptr;
             q.sum16_stride = cp / 2;
@@ -942,7 +943,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             if (c->sum16) { q.c.epi.c = c->d_epi_tab + 5 * c->act->cpad; q.c.epi.d = c->d_epi_tab + 6 * c->act->cpad; }
             if (w4) {
                 q.c.w = c->d_w4img;
-                return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid == 1, false, grid, stream);
+                return conv_pipe_w4_launch(q, small_m ? 2 : bn128 ? 1 : 0, all_valid, false, grid, stream);
             }
             if (small_m) {
                 launch_pipe_res<4, 128, 2, 1, 2, 3>(q, grid, stream);

@@ -55,6 +55,7 @@ struct ConvPipeArgs {
     // Folded residual sum (RES kernels): out = sum_act(conv_act(conv) + pre(other)), all EPI_I24
     const signed char* res;      // the sum's other input, NHWC bytes
     int res_cs;
+    int res_halo;                // border of zeros around every image of the other input
     unsigned res_flip;           // turns a stored byte into an unsigned one (0x80808080 unless plain U8 storage)
     EpiArgs sum;                 // the sum cell's rescale; its d table has the other input's zero point folded in
     EpiArgs pre;                 // ScalingCell folded onto the other input (d table with the zero point folded in)
@@ -299,7 +300,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int j = 0; j < (RES ? NJ : 0); ++j) {
             const int m = m0 + wm * TM + j * 32 + l32;
-            const signed char* rp = q.res + (long long)(m < p.M ? m : 0) * q.res_cs + (n0 + wn * TN + 32 * lh);
+            int rpix = m < p.M ? m : 0;
+            if (q.res_halo != 0) {
+                // the other input carries a border: its pixel sits past the borders of its image
+                const int b = div_magic(rpix, q.ohw_mul, q.ohw_sh);
+                const int rem = rpix - b * (p.OH * p.OW);
+                const int oy = div_magic(rem, q.ow_mul, q.ow_sh);
+                const int ox = rem - oy * p.OW;
+                rpix = (b * (p.OH + 2 * q.res_halo) + oy + q.res_halo) * (p.OW + 2 * q.res_halo) + ox + q.res_halo;
+            }
+            const signed char* rp = q.res + (long long)rpix * q.res_cs + (n0 + wn * TN + 32 * lh);
             asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16"
                          : "=&v"(rfirst[j]), "=&v"(rsecond[j]) : "v"(rp) : "memory");
         }
@@ -877,6 +887,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 size_t conv_pipe_w4_image_bytes(int rows, int ktot);
 void conv_pipe_w4_image(const signed char* w, int rows, int ktot, signed char* image);
 // With a.res set, the residual sum behind the convolution is computed in the epilogue.
-int conv_pipe_w4_launch(ConvPipeArgs a, int tile, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream);
+int conv_pipe_w4_launch(ConvPipeArgs a, int tile, int valid, bool hi16, int grid, hipStream_t stream);
 
 } // namespace n2d2hip

@@ -33,39 +33,41 @@ void conv_pipe_w4_image(const signed char* w, int rows, int ktot, signed char* i
 
 namespace {
 
-template <int NI, int NJ, int WGM>
-void launch(ConvPipeArgs a, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream)
+// valid: 1 = 1x1 without padding, 2 = any kernel whose every tap reads inside the (physical) input, e.g. an input that
+// carries its padding, 0 = per-tap validity bits
+template <int NI, int NJ, int WGM, int V>
+void launch_valid(const ConvPipeArgs& a, bool hi16, int grid, hipStream_t stream)
 {
     constexpr int NW = 4, BK = 64, S = 4;
-    a.c.niter = a.c.ktot / BK;
-    a.cper = a.c.in_cs / BK;
     if (a.res) {
         // residual sum in the epilogue; 16-bit pairs when the host has shown that they hold every intermediate
-        if (one_by_one_unpadded) {
-            if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-            else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        } else {
-            if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-            else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        }
-    } else if (one_by_one_unpadded) {
-        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
     } else {
-        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
     }
+}
+
+template <int NI, int NJ, int WGM>
+void launch(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t stream)
+{
+    a.c.niter = a.c.ktot / 64;
+    a.cper = a.c.in_cs / 64;
+    if (valid == 1) launch_valid<NI, NJ, WGM, 1>(a, hi16, grid, stream);
+    else if (valid == 2) launch_valid<NI, NJ, WGM, 2>(a, hi16, grid, stream);
+    else launch_valid<NI, NJ, WGM, 0>(a, hi16, grid, stream);
 }
 
 } // namespace
 
-int conv_pipe_w4_launch(ConvPipeArgs a, int tile, bool one_by_one_unpadded, bool hi16, int grid, hipStream_t stream)
+int conv_pipe_w4_launch(ConvPipeArgs a, int tile, int valid, bool hi16, int grid, hipStream_t stream)
 {
     N2D2HIP_REQUIRE(a.c.epi.kind == EPI_I24 && a.c.ktot % 64 == 0 && a.c.in_cs % 64 == 0, N2D2HIP_ERR_INVALID,
                     "conv_pipe_w4: integer rescale and a multiple of 64 channels expected");
-    if (tile == 0) launch<2, 1, 4>(a, one_by_one_unpadded, hi16, grid, stream);
-    else if (tile == 1) launch<2, 2, 2>(a, one_by_one_unpadded, hi16, grid, stream);
-    else launch<2, 1, 2>(a, one_by_one_unpadded, hi16, grid, stream);
+    if (tile == 0) launch<2, 1, 4>(a, valid, hi16, grid, stream);
+    else if (tile == 1) launch<2, 2, 2>(a, valid, hi16, grid, stream);
+    else launch<2, 1, 2>(a, valid, hi16, grid, stream);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

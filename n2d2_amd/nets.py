@@ -388,7 +388,7 @@ class GpuNet:
         C, H, W = spec.in_shape
 
         def reads_halo(m):
-            return (m.type == "conv" and m.groups == 1 and m.weight_bits == 8 and m.w.shape[1] % 64 == 0
+            return (m.type == "conv" and m.groups == 1 and m.weight_bits in (4, 8) and m.w.shape[1] % 64 == 0
                     and m.w.shape[2] * m.w.shape[3] <= 31 and tuple(m.dil) == (1, 1))
 
         def halo_of(l, cell):
@@ -512,6 +512,46 @@ class GpuNet:
                 ins_of[l.name] = ins_of[dw.name]
                 self.folded.add(dw.name)
                 self.dw_pws[l.name] = dw
+        # A tensor read by padded convolutions and, as the other input, by sums that a convolution has taken into its
+        # epilogue may carry the convolutions' padding too (the epilogue finds the other input's pixels past its borders),
+        # when its producer can write it: ResNet-18's block inputs, which a max pooling or such a sum produces.
+        if fuse and halo:
+            step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+            for l in spec.layers:
+                t = self.tensors.get(l.name)
+                readers = consumers.get(l.name, [])
+                if t is None or t.halo or l.name in self.folded or l.name == spec.output or not readers:
+                    continue
+                convs = [m for m in readers if m.type == "conv"]
+                sums = [m for m in readers if m.type == "elemwise"]
+                if not convs or len(convs) + len(sums) != len(readers):
+                    continue
+                # (a sum that reads it directly because the convolution holding the sum has it as its own input, a
+                # projection shortcut, is that convolution reading it)
+                if not all(m.name in self.fused_sums and (ins_of[m.name][1] is t) != (ins_of[m.name][0] is t) for m in sums):
+                    continue
+                if not all(reads_halo(m) and (m.name in self.folded or self.steps[step_index[m.name]][1].accepts_halo()) for m in convs):
+                    continue
+                h = max(max(m.pad) for m in convs)
+                if h == 0:
+                    continue
+                producer_cell = self.steps[step_index[l.name]][1]
+                writes = (l.name in self.fused_sums or l.name in self.stem_pools
+                          or (l.type == "conv" and producer_cell.accepts_halo())
+                          or (l.type == "pool" and l.kind == "max" and tuple(l.pool) in ((2, 2), (3, 3))))
+                if not writes:
+                    continue
+                nx = rt.DTensor(t.B, t.C, t.H, t.W, t.dtype, halo=h)
+                if l.type == "pool" and l.name not in self.stem_pools:
+                    try:        # does this pooling write a border?  (asked once, on the real tensors)
+                        producer_cell.forward(ins_of[l.name][0], nx)
+                    except capi.N2D2HipError:
+                        continue
+                for lst in ins_of.values():
+                    for k, u in enumerate(lst):
+                        if u is t:
+                            lst[k] = nx
+                self.tensors[l.name] = nx
         self.bottlenecks, self.bottleneck_layers = {}, {}
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:

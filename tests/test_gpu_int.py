@@ -501,6 +501,18 @@ def test_conv_with_folded_residual_sum(rt):
                         conv.forward_sum(dx, dother, out)
                         got = out.to_numpy()
                         assert np.array_equal(got, want), (C, O, H, stride, other_dtype, pre_mode, k, no16, np.count_nonzero(got != want))
+                    # the other input and the output may each carry a border of their own
+                    if pre_mode is None and k == 0:
+                        for oh, rh in ((0, 1), (1, 2), (2, 0)):
+                            dother_h = rt.DTensor(B, O, OH, OH, other_dtype, halo=rh)
+                            if rh:
+                                dother_h.buf.view(B, OH + 2 * rh, OH + 2 * rh, dother_h.cs)[:, rh:OH + rh, rh:OH + rh, :] = \
+                                    dother.buf.view(B, OH, OH, dother.cs)
+                            else:
+                                dother_h.buf.copy_(dother.buf)
+                            out = rt.DTensor(B, O, OH, OH, capi.U8B, halo=oh)
+                            conv.forward_sum(dx, dother_h, out)
+                            assert np.array_equal(out.to_numpy(), want), (C, O, H, stride, other_dtype, oh, rh)
                     # the plain convolution is still available on the same handle
                     assert np.array_equal(conv.forward(dx).to_numpy(), y.astype(np.int64))
     # what cannot be folded is reported, and the cells then run separately
