@@ -711,6 +711,19 @@ bool PoolCell_Frame_HIP<T>::fuseFirstConv(Cell_Frame_HIP* conv)
 }
 
 template <class T>
+bool PoolCell_Frame_HIP<T>::writesHalo() const
+{
+    if (mFusedConv)
+        return true;
+    if (mInputs.size() != 1 || mInputs[0]->empty())
+        return false;
+    const n2d2hip_pool_desc d = poolDesc();
+    const n2d2hip_tensor& x = mInputs[0]->desc();
+    return d.pooling == N2D2HIP_POOL_MAX && x.halo == 0 && x.cs % 16 == 0 && d.poolW == d.poolH && (d.poolW == 2 || d.poolW == 3)
+        && d.padX < d.poolW && d.padY < d.poolH && ((int)mOutW - 1) * d.strideX - d.padX < x.W && ((int)mOutH - 1) * d.strideY - d.padY < x.H;
+}
+
+template <class T>
 void PoolCell_Frame_HIP<T>::clearFusion()
 {
     if (mFusedConv) {
@@ -722,8 +735,8 @@ void PoolCell_Frame_HIP<T>::clearFusion()
 template <class T>
 void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
-    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype)
-        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
+    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype || mOutputs.desc().halo != mOutputsHalo)
+        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype, mOutputsHalo);
     const n2d2hip_pool_desc d = poolDesc();
     if (mFusedConv)
         checkStatus(n2d2hip_conv_forward_maxpool(mFusedConv->convHandle(), &d, &mFusedConv->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
@@ -1508,23 +1521,33 @@ void DeepNet::planFusion()
                 break;
         }
     }
-    // A convolution's output that only convolutions read carries the largest padding among them as a border of zeros,
-    // when all of them run on the kernel that takes such tensors.
+    // An output that only convolutions read carries the largest padding among them as a border of zeros, when all of them
+    // run on the kernel that takes such tensors and the launch that produces it can write one: a convolution of that kind,
+    // a sum computed in a convolution's epilogue, a 2x2 / 3x3 max pooling.  A sum of that kind may also read such a
+    // tensor as its other input (the epilogue finds the pixels past their borders): ResNet-18's block inputs.
     std::map<const Cell_Frame_HIP*, int> halo;
     std::map<const Cell_Frame_HIP*, bool> refused;
     for (Cell_Frame_HIP* f : mFrames) {
-        for (Cell_Frame_HIP* p : f->parentCells()) {
+        auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
+        const std::vector<Cell_Frame_HIP*>& parents = f->parentCells();
+        for (size_t k = 0; k < parents.size(); ++k) {
+            Cell_Frame_HIP* p = parents[k];
             if (!p) continue;
             if (f->convHandle() && n2d2hip_conv_accepts_halo(f->convHandle()))
                 halo[p] = std::max(halo[p], f->maxPadding());
+            else if (ew && ew->fusedConv() && k != ew->fusedIndex() && !ew->hasFoldedScaling(k))
+                continue;
             else
                 refused[p] = true;
         }
     }
     for (Cell_Frame_HIP* f : mFrames) {
         auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f);
-        const bool writes = f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle())
-            && !(conv && conv->computesDepthwise());
+        auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
+        auto* pool = dynamic_cast<PoolCell_Frame_HIP<float>*>(f);
+        const bool writes = (f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle())
+                             && !(conv && conv->computesDepthwise()))
+            || (ew && ew->fusedConv()) || (pool && pool->writesHalo());
         f->setOutputsHalo(writes && !refused[f] ? halo[f] : 0);
     }
     mPlanned = true;

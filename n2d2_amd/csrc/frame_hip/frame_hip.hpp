@@ -636,6 +636,9 @@ public:
     // output is then never written.  Returns false, and changes nothing, when it declines.
     bool fuseFirstConv(Cell_Frame_HIP* conv);
     void clearFusion();
+    // Can this cell's launch store its output with a border of zeros around every image?  The launch that also computes
+    // the first convolution can, and so can the stand-alone 2x2 / 3x3 max pooling of 16-byte channel groups.
+    bool writesHalo() const;
 
 protected:
     void setOutputsDims();
@@ -694,6 +697,9 @@ public:
     // ... and the convolution behind input k computes this sum in its epilogue: launch() then runs that one kernel.
     bool fuseIntoConv(size_t k, Cell_Frame_HIP* conv);
     void clearFusion();
+    Cell_Frame_HIP* fusedConv() const { return mFusedConv; }
+    size_t fusedIndex() const { return mFusedIndex; }
+    bool hasFoldedScaling(size_t k) const { return k < mFoldedScaling.size() && mFoldedScaling[k] != nullptr; }
     // src/Cell/ElemWiseCell_Frame.cpp:313-316
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : elemWiseOutputsRange(); }
 

@@ -103,7 +103,10 @@ def test_mobilenet_and_w4a4_through_the_registrar(fh):
     from n2d2_amd import nets
     x = np.random.default_rng(34).integers(0, 256, size=(1, 3, 224, 224))
     _compare(fh, nets.mobilenet_v1(), x, ["conv2_dw", "conv2_pw", "conv14_pw", "fc"])
-    _compare(fh, nets.resnet18_w4a4(), x, ["conv2.1_a", "conv2.1_sum", "conv5.2_sum", "fc"])
+    net = _compare(fh, nets.resnet18_w4a4(), x, ["conv2.1_a", "conv2.1_sum", "conv5.2_sum", "fc"])
+    # every 3x3 convolution's input carries its padding: the max pooling's output, the first convolution of each block and
+    # the seven sums a convolution computes and a block reads (as its first convolution's input and as its sum's other input)
+    assert net.nb_halo == 1 + 8 + 7
 
 
 def test_quantized_graph_moves_between_nets_through_files(fh, tmp_path):

@@ -115,6 +115,10 @@ def test_resnet18_w4a4_config():
     keep = ["conv1", "pool1", "conv2.1_a", "conv2.1_b", "conv2.1_sum", "conv3.1_proj", "conv3.1_sum", "conv5.2_sum", "pool", "fc"]
     net = _run_both(spec, x, keep)
     assert net.tensors["conv2.1_a"].to_numpy().max() <= 15
+    # every 3x3 convolution reads a tensor that carries its padding: the max pooling's output, the first convolution of
+    # each block, and the seven sums that a block reads as its first convolution's input and as its sum's other input
+    assert sorted(n for n, t in net.tensors.items() if t.halo) == sorted(
+        ["pool1"] + [l.name for l in spec.layers if l.name.endswith("_a")] + [l.name for l in spec.layers if l.name.endswith("_sum")][:-1])
 
 
 def test_resnet50_full_batch_properties():
