@@ -848,7 +848,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         // where it is the faster of the two (measured): at least two 64-channel steps per tile, so that a tile's rescale is
         // small beside its matrix instructions, and images large enough that the border positions it computes and drops
         // stay under a third of the work
-        && ((d.kernel_choice & N2D2HIP_KERNEL_PATCH) || (d.C >= 128 && (long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135))) {
+        // ... and enough 256-position tiles to give every CU a block (a small batch leaves the pipelined kernel's 128-pixel
+        // tiles the better fit)
+        && ((d.kernel_choice & N2D2HIP_KERNEL_PATCH)
+            || (d.C >= 128 && (long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135
+                && (((long long)in->B * Hp * Wp + 255) / 256) * (d.O / (d.O % 128 == 0 ? 128 : 64)) >= num_cus()))) {
         // 3x3, stride 1, on an input that carries its padding: nine shifted reads of one patch of pixels
         ConvPatchArgs q = {};
         q.in = a.in; q.wfrag = c->d_wfrag; q.out = out->data;
