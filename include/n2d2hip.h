@@ -307,6 +307,10 @@ int n2d2hip_expand_reduce_forward(n2d2hip_expand_reduce_t fused, const n2d2hip_t
 typedef struct n2d2hip_dw_pw_s* n2d2hip_dw_pw_t;
 int n2d2hip_dw_pw_create(n2d2hip_conv_t depthwise, n2d2hip_conv_t pointwise, n2d2hip_dw_pw_t* fused);
 int n2d2hip_dw_pw_destroy(n2d2hip_dw_pw_t fused);
+/* 1 when the one launch is expected to be faster than the two cells' own on `batch` inputs of in_h x in_w (measured rule:
+ * at most 256 outputs and at least 32768 output pixels), else 0.  No counterpart in the reference: a planner's question
+ * (DeepNet::planFusion asks it). */
+int n2d2hip_dw_pw_pays(n2d2hip_dw_pw_t fused, int batch, int in_h, int in_w);
 /* `in`: input of `depthwise`; `out`: output of `pointwise`.  NHWC bytes without a border, channel stride equal to the
  * channel count. */
 int n2d2hip_dw_pw_forward(n2d2hip_dw_pw_t fused, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream);

@@ -31,7 +31,7 @@ SYMBOLS = [
     "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_accepts_halo",
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", "n2d2hip_expand_reduce_create", "n2d2hip_expand_reduce_destroy", "n2d2hip_expand_reduce_forward",
-    "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward",
+    "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling",
@@ -108,6 +108,7 @@ def load():
     lib.n2d2hip_dw_pw_create.argtypes = [P, P, P]
     lib.n2d2hip_dw_pw_destroy.argtypes = [P]
     lib.n2d2hip_dw_pw_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_dw_pw_pays.argtypes = [P, C.c_int, C.c_int, C.c_int]
     lib.n2d2hip_fc_create.argtypes = [I, I, I, I, I, P, P, P, I, P]
     lib.n2d2hip_fc_destroy.argtypes = [P]
     lib.n2d2hip_fc_forward.argtypes = [P, P, P, P]

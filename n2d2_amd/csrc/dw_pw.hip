@@ -350,14 +350,20 @@ int n2d2hip_dw_pw_create(n2d2hip_conv_t dw, n2d2hip_conv_t pw, n2d2hip_dw_pw_t* 
         return fail(N2D2HIP_ERR_HIP, "dw_pw_create: reading the 1x1 convolution back failed: %s", hipGetErrorString(e));
     // [channel tile][chunk][K step][32-channel block][lane][16 bytes]: lane l holds channel l % 32 of the block,
     // bytes K step * 32 + 16 * (l / 32) .. of the chunk
-    std::vector<signed char> img((size_t)O * C);
-    for (int t = 0; t < O / nt; ++t)
-        for (int c = 0; c < nchunks; ++c)
-            for (int s = 0; s < ks; ++s)
-                for (int blk = 0; blk < nb; ++blk)
-                    for (int l = 0; l < 64; ++l)
-                        memcpy(img.data() + ((((size_t)(t * nchunks + c) * ks + s) * nb + blk) * 64 + l) * 16,
-                               w.data() + (size_t)(t * nt + blk * 32 + (l & 31)) * pw->ktot + c * kc + s * 32 + 16 * (l >> 5), 16);
+    auto fragment_image = [&](int blocks) {
+        std::vector<signed char> img((size_t)O * C);
+        const int tile = blocks * 32;
+        for (int t = 0; t < O / tile; ++t)
+            for (int c = 0; c < nchunks; ++c)
+                for (int s = 0; s < ks; ++s)
+                    for (int blk = 0; blk < blocks; ++blk)
+                        for (int l = 0; l < 64; ++l)
+                            memcpy(img.data() + ((((size_t)(t * nchunks + c) * ks + s) * blocks + blk) * 64 + l) * 16,
+                                   w.data() + (size_t)(t * tile + blk * 32 + (l & 31)) * pw->ktot + c * kc + s * 32 + 16 * (l >> 5), 16);
+        return img;
+    };
+    const std::vector<signed char> img = fragment_image(nb);
+    (void)nt;
     // a, b, c, d, e by channel; a cell that needs no clamp before its multiply gets bounds that clamp nothing
     std::vector<int> tab(5 * (size_t)O);
     for (int r = 0; r < 5; ++r)
@@ -382,6 +388,20 @@ int n2d2hip_dw_pw_create(n2d2hip_conv_t dw, n2d2hip_conv_t pw, n2d2hip_dw_pw_t* 
     }
     *out = h;
     return N2D2HIP_OK;
+}
+
+int n2d2hip_dw_pw_pays(n2d2hip_dw_pw_t h, int batch, int in_h, int in_w)
+{
+    if (!h || batch <= 0)
+        return 0;
+    int OH, OW;
+    if (n2d2hip_conv_out_dims(&h->dw->desc, in_h, in_w, &OH, &OW) != N2D2HIP_OK)
+        return 0;
+    const long long pixels = (long long)batch * OH * OW;
+    // One work-group holds all output channels of its pixels and the tensor between the cells is large: with more than 256
+    // output channels the depthwise part is computed once per 256 of them, and on small images the launch has too few
+    // work-groups to fill the chip.
+    return h->pw->desc.O <= 256 && pixels >= 32768 ? 1 : 0;
 }
 
 int n2d2hip_dw_pw_forward(n2d2hip_dw_pw_t h, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream_)

@@ -479,13 +479,18 @@ template <class T>
 bool ConvCell_Frame_HIP<T>::fuseDepthwise(Cell_Frame_HIP* depthwise)
 {
     if (mDwPw || !mConv || !depthwise || !depthwise->convHandle() || depthwise->foldedInto() || foldedInto() || mInputs.size() != 1
-        || mNbOutputs > 256 || (long long)mBatch * mOutH * mOutW < 32768 || depthwise->inputTensor(0)->desc().halo != 0)
+        || depthwise->inputTensor(0)->desc().halo != 0)
         return false;
     n2d2hip_dw_pw_t fused = nullptr;
     const int rc = n2d2hip_dw_pw_create(depthwise->convHandle(), mConv, &fused);
     if (rc == N2D2HIP_ERR_UNSUPPORTED)
         return false;
     checkStatus(rc);
+    const n2d2hip_tensor& x = depthwise->inputTensor(0)->desc();
+    if (!n2d2hip_dw_pw_pays(fused, x.B, x.H, x.W)) {
+        n2d2hip_dw_pw_destroy(fused);
+        return false;
+    }
     mDwPw = fused;
     mFusedDw = depthwise;
     depthwise->setFoldedInto(this);

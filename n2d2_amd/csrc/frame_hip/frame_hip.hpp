@@ -526,8 +526,8 @@ public:
     int maxPadding() const { return std::max(mPaddingDims[0], mPaddingDims[1]); }
     // Graph-level fusion (DeepNet::planFusion): this 1x1 convolution computes the 3x3 depthwise convolution `depthwise`,
     // whose output it alone reads, in its own launch (n2d2hip_dw_pw_*); the depthwise cell is then not launched and its
-    // output never written.  Taken where the device library accepts the pair and one launch is expected to be faster than
-    // two: at most 256 outputs, at least 32768 output pixels in the batch.
+    // output never written.  Taken where the device library accepts the pair and expects one launch to be faster than two
+    // (n2d2hip_dw_pw_pays).
     bool fuseDepthwise(Cell_Frame_HIP* depthwise);
     void clearFusion();
     bool computesDepthwise() const { return mDwPw != nullptr; }

@@ -369,8 +369,8 @@ class GpuNet:
         stem_pool: compute the max pooling behind a first-layer convolution in that convolution's launch
         (n2d2hip_conv_forward_maxpool) where the library takes the pair.
         dw_pw: run a 3x3 depthwise convolution and the 1x1 convolution that alone reads it as one launch (n2d2hip_dw_pw_*)
-        where the library takes the pair and the launch is expected to be faster than the two (at most 256 output channels,
-        at least 32768 output pixels in the batch); "all": wherever the library takes the pair.
+        where the library takes the pair and expects the launch to be faster than the two (n2d2hip_dw_pw_pays); "all":
+        wherever the library takes the pair.
         tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
         (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
         only ties with the two separate launches."""
@@ -500,13 +500,13 @@ class GpuNet:
                 if (dw is None or dw.type != "conv" or dw.groups == 1 or len(consumers[dw.name]) != 1 or dw.name in self.folded
                         or ins_of[dw.name][0].halo or self.tensors[l.name].halo):
                     continue
-                # One launch pays where the tensor between the two cells is large and one work-group holds all output
-                # channels of its pixels; with more than 256 output channels the depthwise part is computed once per
-                # 256 of them, and on small images the launch has too few work-groups to fill the chip.
-                if dw_pw != "all" and (l.out_shape[0] > 256 or batch * l.out_shape[1] * l.out_shape[2] < 32768):
-                    continue
                 fused_cell = rt.DwPw.create(self.steps[step_index[dw.name]][1], self.steps[step_index[l.name]][1])
                 if fused_cell is None:
+                    continue
+                # the library knows where one launch is faster than two (large tensors between the cells; small images
+                # with 512 outputs per work-group)
+                x = ins_of[dw.name][0]
+                if dw_pw != "all" and not fused_cell.pays(batch, x.H, x.W):
                     continue
                 self.steps[step_index[l.name]] = (l, fused_cell, (lambda c, i, o: c.forward(i[0], o)))
                 ins_of[l.name] = ins_of[dw.name]

@@ -192,6 +192,10 @@ class DwPw:
         check(lib.n2d2hip_dw_pw_forward(self.handle, x.ref, out.ref, stream_ptr()))
         return out
 
+    def pays(self, batch, in_h, in_w):
+        """Does the library expect the one launch to be faster than the two cells' own on inputs of this size?"""
+        return bool(lib.n2d2hip_dw_pw_pays(self.handle, batch, in_h, in_w))
+
     def __del__(self):
         if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_dw_pw_destroy(self.handle)

@@ -822,7 +822,8 @@ def sum_spec_for(O, rng):
 
 @pytest.mark.parametrize("case", [(3, 32, 64, 1, 19, 21, 1), (2, 64, 128, 2, 23, 17, 1), (2, 128, 128, 1, 14, 14, 1), (2, 128, 256, 2, 28, 28, 1),
                                   (1, 256, 512, 2, 9, 10, 0), (2, 192, 64, 1, 8, 16, 1), (1, 32, 128, 2, 33, 41, 1),
-                                  (1, 64, 256, 1, 11, 37, 0), (1, 512, 1024, 1, 5, 6, 1)],
+                                  (1, 64, 256, 1, 11, 37, 0), (1, 512, 1024, 1, 5, 6, 1), (3, 128, 512, 1, 14, 14, 1),
+                                  (2, 512, 512, 2, 15, 13, 1), (2, 64, 512, 1, 6, 18, 0)],
                          ids=lambda c: "x".join(str(v) for v in c))
 def test_depthwise_and_pointwise_in_one_launch_bit_exact(rt, case):
     """n2d2hip_dw_pw_*: a 3x3 depthwise convolution and the 1x1 convolution reading it as one launch, against the oracle
