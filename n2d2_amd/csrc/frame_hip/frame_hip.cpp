@@ -398,6 +398,7 @@ n2d2hip_act_t Cell_Frame_HIP::activationHandle(const Scaling* standalone)
     const int kind = (mActivation && !standalone) ? mActivation->abiKind() : N2D2HIP_ACT_LINEAR;
     const float leak = (mActivation && !standalone) ? mActivation->leakSlope() : 0.0f;
     mActHandle = makeAct(s, kind, leak, nbBits, uns, mNbOutputs, mName);
+    ++mActGeneration;
     mActRevision = rev;
     mActUnsigned = (int)uns;
     // the storage type follows the signedness decision
@@ -462,7 +463,7 @@ ConvCell_Frame_HIP<T>::ConvCell_Frame_HIP(const DeepNet& /*deepNet*/, const std:
                                           unsigned int nbOutputs, const std::vector<unsigned int>& subSampleDims,
                                           const std::vector<unsigned int>& strideDims, const std::vector<int>& paddingDims,
                                           const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvAct(nullptr), mConvInDType(-1),
+    : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims), mConv(nullptr), mConvActGen(0), mConvInDType(-1),
       mDwPw(nullptr), mFusedDw(nullptr)
 {
     mActivation = activation;
@@ -554,7 +555,7 @@ bool ConvCell_Frame_HIP<T>::prepare()
     n2d2hip_act_t act = activationHandle();
     const int inDType = mInputs[0]->desc().dtype;
     bool rebuilt = false;
-    if (mDirty || act != mConvAct || !mConv || inDType != mConvInDType) {
+    if (mDirty || activationGeneration() != mConvActGen || !mConv || inDType != mConvInDType) {
         clearFusion();
         if (mConv) { n2d2hip_conv_destroy(mConv); mConv = nullptr; }
         const unsigned int cg = mNbChannels / mNbGroups;
@@ -576,7 +577,7 @@ bool ConvCell_Frame_HIP<T>::prepare()
                                                     "Cell " + mName + " biases"));
         }
         checkStatus(n2d2hip_conv_create(&d, w.data(), mNoBias ? nullptr : b.data(), act, inDType, &mConv));
-        mConvAct = act;
+        mConvActGen = activationGeneration();
         mConvInDType = inDType;
         mDirty = false;
         rebuilt = true;
@@ -599,7 +600,7 @@ void FcCell::setParameter(const std::string& name, bool value)
 template <class T>
 FcCell_Frame_HIP<T>::FcCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
                                       const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), mFc(nullptr), mFcAct(nullptr)
+    : Cell(name, nbOutputs), mFc(nullptr), mFcActGen(0)
 {
     mActivation = activation;
 }
@@ -630,7 +631,7 @@ void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
     n2d2hip_act_t act = activationHandle();
     const int inDType = mInputs[0]->desc().dtype;
-    if (mDirty || act != mFcAct || !mFc) {
+    if (mDirty || activationGeneration() != mFcActGen || !mFc) {
         if (mFc) { n2d2hip_fc_destroy(mFc); mFc = nullptr; }
         const size_t K = (size_t)mNbChannels * mInH * mInW;
         if (mWeights.size() != K * mNbOutputs)
@@ -646,7 +647,7 @@ void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
         }
         checkStatus(n2d2hip_fc_create((int)mNbChannels, (int)mInH, (int)mInW, (int)mNbOutputs, 8, w.data(), mNoBias ? nullptr : b.data(), act,
                                       inDType, &mFc));
-        mFcAct = act;
+        mFcActGen = activationGeneration();
         mDirty = false;
     }
     checkStatus(n2d2hip_fc_forward(mFc, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
@@ -775,7 +776,7 @@ std::pair<double, double> ElemWiseCell::elemWiseOutputsRange() const
 ElemWiseCell_Frame_HIP::ElemWiseCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs, Operation operation,
                                                CoeffMode mode, const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts,
                                                const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts), mEw(nullptr), mEwAct(nullptr), mFusedConv(nullptr), mFusedIndex(0)
+    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts), mEw(nullptr), mEwActGen(0), mFusedConv(nullptr), mFusedIndex(0)
 {
     mActivation = activation;
     if (operation != Sum)
@@ -813,14 +814,14 @@ void ElemWiseCell_Frame_HIP::propagate(bool /*inference*/)
 bool ElemWiseCell_Frame_HIP::prepare()
 {
     n2d2hip_act_t act = activationHandle();
-    if (mEw && act == mEwAct)
+    if (mEw && activationGeneration() == mEwActGen)
         return false;
     // the convolution that took this sum over borrows mEw: release it first
     clearFusion();
     if (mEw) { n2d2hip_elemwise_destroy(mEw); mEw = nullptr; }
     const int mode = mCoeffMode == PerChannel ? N2D2HIP_COEFF_PER_CHANNEL : (mCoeffMode == PerInput ? N2D2HIP_COEFF_PER_INPUT : N2D2HIP_COEFF_PER_LAYER);
     checkStatus(n2d2hip_elemwise_create((int)mInputs.size(), (int)mNbOutputs, mode, mWeights.data(), mShifts.data(), act, &mEw));
-    mEwAct = act;
+    mEwActGen = activationGeneration();
     return true;
 }
 
@@ -832,7 +833,9 @@ static HipTensor* sourceOf(const std::vector<Cell_Frame_HIP*>& folded, const std
 
 void ElemWiseCell_Frame_HIP::launch()
 {
-    if (mFusedConv) {
+    if (mBottleneck) {
+        checkStatus(n2d2hip_bottleneck_forward(mBottleneck, &mBottleneckIn->getDeviceOutputs().desc(), &mOutputs.desc(), mStream));
+    } else if (mFusedConv) {
         checkStatus(n2d2hip_conv_forward_sum(mFusedConv->convHandle(), &mFusedConv->inputTensor(0)->desc(),
                                              &sourceOf(mFoldedScaling, mInputs, 1 - mFusedIndex)->desc(), &mOutputs.desc(), mStream));
     } else {
@@ -872,8 +875,36 @@ bool ElemWiseCell_Frame_HIP::fuseIntoConv(size_t k, Cell_Frame_HIP* conv)
     return true;
 }
 
+bool ElemWiseCell_Frame_HIP::fuseBottleneck(Cell_Frame_HIP* reduce, Cell_Frame_HIP* conv3x3, Cell_Frame_HIP* projection, Cell_Frame_HIP* input)
+{
+    if (mBottleneck || !mFusedConv || !reduce || !conv3x3 || !input || !reduce->convHandle() || !conv3x3->convHandle()
+        || (projection && !projection->convHandle()))
+        return false;
+    n2d2hip_bottleneck_t b = nullptr;
+    const int rc = n2d2hip_bottleneck_create(reduce->convHandle(), conv3x3->convHandle(), mFusedConv->convHandle(),
+                                             projection ? projection->convHandle() : nullptr, &b);
+    if (rc == N2D2HIP_ERR_UNSUPPORTED)
+        return false;
+    checkStatus(rc);
+    mBottleneck = b;
+    mBottleneckIn = input;
+    mBottleneckCells = {reduce, conv3x3};
+    if (projection) mBottleneckCells.push_back(projection);
+    for (Cell_Frame_HIP* c : mBottleneckCells)
+        c->setFoldedInto(this);
+    return true;
+}
+
 void ElemWiseCell_Frame_HIP::clearFusion()
 {
+    if (mBottleneck) {
+        n2d2hip_bottleneck_destroy(mBottleneck);
+        mBottleneck = nullptr;
+        mBottleneckIn = nullptr;
+        for (Cell_Frame_HIP* c : mBottleneckCells)
+            c->setFoldedInto(nullptr);
+        mBottleneckCells.clear();
+    }
     if (mFusedConv) {
         if (mFusedConv->convHandle())
             checkStatus(n2d2hip_conv_fuse_sum(mFusedConv->convHandle(), nullptr, 0, 0));
@@ -1526,6 +1557,60 @@ void DeepNet::planFusion()
                 break;
         }
     }
+    // A residual block with a projection shortcut, reduce (1x1) -> 3x3 -> expand (1x1) + projection (1x1) + sum, runs as one
+    // launch where the device library takes it.  The sum sits in the convolution that runs last, which is the projection
+    // when the graph lists it behind the main branch: it is moved into the expansion first (and back if the library
+    // declines).  The block's input then carries a border of one pixel, which its producer must be able to write.
+    std::map<const Cell_Frame_HIP*, bool> bottleneckInput;
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
+        if (!ew || !ew->fusedConv() || ew->parentCells().size() != 2)
+            continue;
+        const size_t k = ew->fusedIndex();
+        Cell_Frame_HIP* holder = ew->fusedConv();
+        Cell_Frame_HIP* other = ew->parentCells()[1 - k];
+        if (!other || !other->convHandle() || ew->hasFoldedScaling(1 - k) || consumers[other] != 1 || other->foldedInto())
+            continue;
+        auto single_conv_parent = [&](Cell_Frame_HIP* c) -> Cell_Frame_HIP* {
+            const std::vector<Cell_Frame_HIP*>& ps = c->parentCells();
+            return ps.size() == 1 && ps[0] && ps[0]->convHandle() ? ps[0] : nullptr;
+        };
+        // which of the two convolutions ends the main branch (its input is a convolution whose input is a convolution)?
+        Cell_Frame_HIP* expand = nullptr;
+        Cell_Frame_HIP* proj = nullptr;
+        for (Cell_Frame_HIP* cand : {holder, other}) {
+            Cell_Frame_HIP* b3 = single_conv_parent(cand);
+            if (b3 && single_conv_parent(b3)) { expand = cand; proj = cand == holder ? other : holder; break; }
+        }
+        if (!expand)
+            continue;
+        Cell_Frame_HIP* conv3 = single_conv_parent(expand);
+        Cell_Frame_HIP* reduce = single_conv_parent(conv3);
+        if (reduce->parentCells().size() != 1 || proj->parentCells().size() != 1)
+            continue;
+        Cell_Frame_HIP* x = reduce->parentCells()[0];
+        if (!x || proj->parentCells()[0] != x || consumers[x] != 2 || consumers[reduce] != 1 || consumers[conv3] != 1
+            || reduce->foldedInto() || conv3->foldedInto())
+            continue;
+        auto* xpool = dynamic_cast<PoolCell_Frame_HIP<float>*>(x);
+        auto* xsum = dynamic_cast<ElemWiseCell_Frame_HIP*>(x);
+        if (!((xpool && xpool->writesHalo()) || (xsum && xsum->fusedConv())))
+            continue;
+        const size_t kExpand = expand == holder ? k : 1 - k;
+        if (expand != holder) {
+            ew->clearFusion();
+            if (!ew->fuseIntoConv(kExpand, expand)) {
+                ew->fuseIntoConv(k, holder);
+                continue;
+            }
+        }
+        if (ew->fuseBottleneck(reduce, conv3, proj, x)) {
+            bottleneckInput[x] = true;
+        } else if (expand != holder) {
+            ew->clearFusion();
+            ew->fuseIntoConv(k, holder);
+        }
+    }
     // An output that only convolutions read carries the largest padding among them as a border of zeros, when all of them
     // run on the kernel that takes such tensors and the launch that produces it can write one: a convolution of that kind,
     // a sum computed in a convolution's epilogue, a 2x2 / 3x3 max pooling.  A sum of that kind may also read such a
@@ -1553,7 +1638,7 @@ void DeepNet::planFusion()
         const bool writes = (f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle())
                              && !(conv && conv->computesDepthwise()))
             || (ew && ew->fusedConv()) || (pool && pool->writesHalo());
-        f->setOutputsHalo(writes && !refused[f] ? halo[f] : 0);
+        f->setOutputsHalo(bottleneckInput[f] ? 1 : (writes && !refused[f] ? halo[f] : 0));
     }
     mPlanned = true;
 }

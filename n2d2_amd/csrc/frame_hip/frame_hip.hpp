@@ -437,12 +437,15 @@ public:
     void setStream(void* stream) { mStream = stream; }
 
 protected:
-    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mFoldedInto(nullptr), mOutputsHalo(0), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1) {}
+    Cell_Frame_HIP() : mBatch(0), mStream(nullptr), mFoldedInto(nullptr), mOutputsHalo(0), mActHandle(nullptr), mActRevision(~0u), mActUnsigned(-1), mActGeneration(0) {}
     ~Cell_Frame_HIP();
     virtual void setOutputsDims() = 0;
     // (Re)builds the device tables of the activation when its Scaling, its bit width or the
     // signedness decision changed; cells without activation get a pass-through / Scaling-only table.
     n2d2hip_act_t activationHandle(const Scaling* standalone = nullptr);
+    // Counts the handles activationHandle() has made.  A cell remembers the count its own device handle was built at:
+    // the handle's address says nothing, a new one may be allocated where the one before it was.
+    unsigned long activationGeneration() const { return mActGeneration; }
     int outputDType(const Scaling* standalone = nullptr) const;
     void allocateOutputs(const Scaling* standalone = nullptr);
     std::vector<HipTensor*> mInputs;
@@ -457,6 +460,7 @@ private:
     n2d2hip_act_t mActHandle;
     unsigned mActRevision;
     int mActUnsigned;
+    unsigned long mActGeneration;
 };
 
 // ------------------------------------------------------------------- ConvCell
@@ -537,7 +541,7 @@ protected:
 
 private:
     n2d2hip_conv_t mConv;
-    n2d2hip_act_t mConvAct;
+    unsigned long mConvActGen;
     int mConvInDType;
     n2d2hip_dw_pw_t mDwPw;
     Cell_Frame_HIP* mFusedDw;
@@ -589,7 +593,7 @@ protected:
 
 private:
     n2d2hip_fc_t mFc;
-    n2d2hip_act_t mFcAct;
+    unsigned long mFcActGen;
     static Registrar<FcCell> mRegistrar;
 };
 
@@ -699,6 +703,11 @@ public:
     void clearFusion();
     Cell_Frame_HIP* fusedConv() const { return mFusedConv; }
     size_t fusedIndex() const { return mFusedIndex; }
+    // ... and a whole residual block in one launch (n2d2hip_bottleneck_*): `reduce` (1x1) -> `conv3x3` -> `expand` (1x1), the
+    // convolution that has taken this sum, with `projection` (1x1) on the shortcut; all four read nothing but each other
+    // and the block's input, the output of `input`, which must then carry a border of one pixel.
+    bool fuseBottleneck(Cell_Frame_HIP* reduce, Cell_Frame_HIP* conv3x3, Cell_Frame_HIP* projection, Cell_Frame_HIP* input);
+    Cell_Frame_HIP* bottleneckInput() const { return mBottleneck ? mBottleneckIn : nullptr; }
     bool hasFoldedScaling(size_t k) const { return k < mFoldedScaling.size() && mFoldedScaling[k] != nullptr; }
     // src/Cell/ElemWiseCell_Frame.cpp:313-316
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : elemWiseOutputsRange(); }
@@ -708,10 +717,13 @@ protected:
 
 private:
     n2d2hip_elemwise_t mEw;
-    n2d2hip_act_t mEwAct;
+    unsigned long mEwActGen;
     std::vector<Cell_Frame_HIP*> mFoldedScaling;  // per input, null = not folded
     Cell_Frame_HIP* mFusedConv;
     size_t mFusedIndex;
+    n2d2hip_bottleneck_t mBottleneck = nullptr;
+    Cell_Frame_HIP* mBottleneckIn = nullptr;
+    std::vector<Cell_Frame_HIP*> mBottleneckCells;
     static Registrar<ElemWiseCell> mRegistrar;
 };
 

@@ -144,6 +144,14 @@ int fh_cell_info(void* net, const char* name, int* dims, int* unsignedOut, char*
     });
 }
 
+// Width of the border of zeros that the fusion plan gave the cell's output tensor (0: none), or -1 on error
+int fh_cell_outputs_halo(void* net, const char* name)
+{
+    int halo = -1;
+    guarded([&] { halo = std::dynamic_pointer_cast<Cell_Frame_HIP>(((Net*)net)->deepNet->getCell(name))->outputsHalo(); });
+    return halo;
+}
+
 int fh_cell_set_quantized(void* net, const char* name, int nbBits, int activationNbBits)
 {
     return guarded([&] {

@@ -23,6 +23,7 @@ for _n in ("fh_net_free", "fh_net_model", "fh_net_nb_cells", "fh_net_initialize"
     getattr(lib, _n).argtypes = [C.c_void_p]
 lib.fh_net_set_stimuli.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_info.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_char_p, C.c_int]
+lib.fh_cell_outputs_halo.argtypes = [C.c_void_p, C.c_char_p]
 lib.fh_cell_set_quantized.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_int]
 lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
 lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
@@ -134,7 +135,8 @@ class Net:
         uns = C.c_int()
         typ = C.create_string_buffer(32)
         _check(lib.fh_cell_info(self.h, name.encode(), dims, C.byref(uns), typ, 32))
-        return {"W": dims[0], "H": dims[1], "C": dims[2], "B": dims[3], "unsigned": bool(uns.value), "type": typ.value.decode()}
+        return {"W": dims[0], "H": dims[1], "C": dims[2], "B": dims[3], "unsigned": bool(uns.value), "type": typ.value.decode(),
+                "halo": lib.fh_cell_outputs_halo(self.h, name.encode())}
 
     def set_quantized(self, name, nb_bits, act_nb_bits=0):
         _check(lib.fh_cell_set_quantized(self.h, name.encode(), int(nb_bits), int(act_nb_bits)))

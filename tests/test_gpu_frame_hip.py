@@ -44,12 +44,17 @@ def test_resnet50_through_the_registrar(fh):
     x = np.random.default_rng(32).integers(0, 256, size=(2, 3, 224, 224))
     net = _compare(fh, spec, x, ["pool1", "conv2.1_sum", "conv2.2_1x1", "conv3.4_sum", "conv5.3_sum", "pool", "fc"])
     # 12 shortcut ScalingCells applied inside their sums, 16 sums computed by the 1x1 convolution before them, the first
-    # convolution's max pooling computed by that convolution's launch
-    assert net.nb_folded == 29
+    # convolution's max pooling computed by that convolution's launch, and the first block's other three convolutions
+    # (1x1, 3x3, projection) computed by its sum's launch
+    assert net.nb_folded == 32
+    for name in ("conv2.1_1x1", "conv2.1_3x3", "conv2.1_1x1_proj", "conv2.1_1x1_x4"):
+        with pytest.raises(fh.FrameHipError, match="not materialised"):
+            net.outputs(name)
     with pytest.raises(fh.FrameHipError, match="pool1 computes it on the fly"):
         net.outputs("conv1")
-    # the 16 tensors between a 1x1 and a padded 3x3 convolution carry that padding as a border
-    assert net.nb_halo == 16
+    # the 15 tensors between a 1x1 and a padded 3x3 convolution that are written carry that padding as a border, and so
+    # does the first block's input, whose 3x3 convolution reads it through the 1x1 before
+    assert net.nb_halo == 16 and net.cell_info("pool1")["halo"] == 1
     with pytest.raises(fh.FrameHipError) as e:
         net.outputs("conv2.2_shortcut_rescale")
     assert "not materialised" in str(e.value)
@@ -63,16 +68,31 @@ def test_resnet50_through_the_registrar(fh):
     net.set_fusion(False)
     net.propagate()
     assert net.nb_folded == 0 and net.nb_halo == 0
-    keep = ["conv1", "pool1", "conv2.2_shortcut_rescale", "conv2.2_1x1_x4", "conv2.2_sum", "fc"]
+    keep = ["conv1", "pool1", "conv2.1_1x1", "conv2.1_3x3", "conv2.1_1x1_proj", "conv2.2_shortcut_rescale", "conv2.2_1x1_x4",
+            "conv2.2_sum", "fc"]
     want = cells.run_net(spec, x2, keep=keep)
     for name in keep:
         assert np.array_equal(net.outputs(name), want[name]), name
     # and back on: the plan is made again
     net.set_fusion(True)
     net.propagate()
-    assert net.nb_folded == 29 and net.nb_halo == 16 and np.array_equal(net.outputs("fc"), want["fc"])
+    assert net.nb_folded == 32 and net.nb_halo == 16 and np.array_equal(net.outputs("fc"), want["fc"])
     assert np.array_equal(net.outputs("pool1"), want["pool1"])
     assert np.array_equal(net.outputs("conv2.2_1x1"), cells.run_net(spec, x2, keep=["conv2.2_1x1"])["conv2.2_1x1"])
+    # a new Scaling on a convolution that the first block's launch computes: the cell and the plan are made again.  Shifts
+    # this small are outside what the block's kernel takes, so the block runs as separate launches; with the first Scaling
+    # back it is one launch again
+    l = {l.name: l for l in spec.layers}["conv2.1_3x3"]
+    first = l.act.scaling
+    for scaling, folded in (((np.asarray(first) // 2).astype(first.dtype), 29), (first, 32)):
+        l.act.scaling = scaling
+        net.set_scaling(l.name, l.act.mode, l.act.scaling, l.act.frac_bits, l.act.clipping)
+        net.propagate()
+        want = cells.run_net(spec, x2, keep=["conv2.1_3x3", "conv2.1_sum", "fc"])
+        assert net.nb_folded == folded
+        assert np.array_equal(net.outputs("conv2.1_sum"), want["conv2.1_sum"]) and np.array_equal(net.outputs("fc"), want["fc"])
+        if folded == 29:
+            assert np.array_equal(net.outputs("conv2.1_3x3"), want["conv2.1_3x3"])
 
 
 def test_fusion_follows_a_scaling_change(fh):
