@@ -144,7 +144,9 @@ typedef struct n2d2hip_conv_desc {
     int strideX, strideY;
     int padL, padT, padR, padB;
     int dilX, dilY;
-    int groups;             /* Cell::getNbGroups of the mapping (ref: src/Cell/Cell.cpp:251-300): 1, or C == O (depthwise) */
+    int groups;             /* Cell::getNbGroups of the mapping (ref: src/Cell/Cell.cpp:251-300): G equal groups, weights
+                               [O][C/G][kH][kW] (ConvCell_Frame_Kernels.cpp:89-96).  G == C == O (depthwise) has its own
+                               kernels; 1 < G otherwise runs as a full connection with zeros outside the groups */
     int weight_bits;        /* 8: int8_t weights; 4: two weights per byte, element 2i in the low nibble */
     int kernel_choice;      /* 0: the library chooses among its kernels.  Otherwise N2D2HIP_KERNEL_* bits, which only steer
                                that choice among kernels that compute the same result (tests use them to cover every

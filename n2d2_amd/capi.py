@@ -77,6 +77,10 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise ImportError("libn2d2hip.so is not built (%s): run `python -m n2d2_amd.build`; "
                           "there is no CPU fallback for the Frame_HIP path" % LIB_PATH)
+    # torch ships its own HIP runtime.  Loaded first, it is the one this library binds to, so that both see the same
+    # device context and a torch tensor's data pointer is valid in the library's calls; the other order puts two runtimes
+    # into the process and the second one then reports no device.
+    import torch  # noqa: F401
     lib = C.CDLL(LIB_PATH)
     for name in ("n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version"):
         getattr(lib, name).restype = C.c_char_p

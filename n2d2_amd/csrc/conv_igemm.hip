@@ -482,11 +482,30 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
                     "conv_create: plain U8 inputs cannot feed the signed matrix cores; convert to U8B first");
     N2D2HIP_REQUIRE(act->nb_channels == d->O, N2D2HIP_ERR_INVALID, "conv_create: activation built for %d channels, conv has %d outputs",
                     act->nb_channels, d->O);
-    const bool depthwise = d->groups > 1;
-    if (depthwise)
-        N2D2HIP_REQUIRE(d->groups == d->C && d->C == d->O, N2D2HIP_ERR_UNSUPPORTED,
-                        "conv_create: groups = %d is supported only as depthwise (groups == C == O)", d->groups);
     N2D2HIP_REQUIRE(d->groups >= 1, N2D2HIP_ERR_UNSUPPORTED, "conv_create: irregular mapping (nbGroups = %d)", d->groups);
+    const bool depthwise = d->groups > 1 && d->groups == d->C && d->C == d->O;
+    if (d->groups > 1 && !depthwise) {
+        // G equal groups, output o of group o / (O/G) connected to channels [g C/G, (g+1) C/G) with its weights indexed by
+        // the position among them (ConvCell_Frame_Kernels.cpp:89-96,132): the same sums as a full connection whose
+        // weights outside the group are 0, which is how the matrix-core kernels run it (G times the multiplications, no
+        // change to the bytes moved; the depthwise case above has its own kernel).
+        N2D2HIP_REQUIRE(d->C % d->groups == 0 && d->O % d->groups == 0, N2D2HIP_ERR_INVALID,
+                        "conv_create: %d groups do not divide %d channels and %d outputs", d->groups, d->C, d->O);
+        const int Cg = d->C / d->groups, Og = d->O / d->groups;
+        const long long taps = (long long)d->kH * d->kW, n = (long long)d->O * d->C * taps;
+        std::vector<unsigned char> dense((size_t)(d->weight_bits == 8 ? n : (n + 1) / 2), 0);
+        for (int o = 0; o < d->O; ++o)
+            for (int cg = 0; cg < Cg; ++cg)
+                for (long long t = 0; t < taps; ++t) {
+                    const int v = read_weight(weights, ((long long)o * Cg + cg) * taps + t, d->weight_bits);
+                    const long long at = ((long long)o * d->C + (long long)(o / Og) * Cg + cg) * taps + t;
+                    if (d->weight_bits == 8) dense[(size_t)at] = (unsigned char)(signed char)v;
+                    else dense[(size_t)(at >> 1)] |= (unsigned char)((v & 15) << ((at & 1) ? 4 : 0));
+                }
+        n2d2hip_conv_desc full = *d;
+        full.groups = 1;
+        return n2d2hip_conv_create(&full, dense.data(), bias, act, in_dtype, conv);
+    }
 
     n2d2hip_conv_s* c = new n2d2hip_conv_s();
     c->desc = *d;

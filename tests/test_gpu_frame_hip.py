@@ -178,6 +178,35 @@ def test_depthwise_cell_from_its_connection_map(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+def test_grouped_convolution_cells(fh):
+    """ConvCells with 2 and 4 equal groups (Mapping.NbGroups in the INI; one of them again from its connection map), a depth
+    multiplier (groups = channels, twice as many outputs): every cell output against the oracle."""
+    from n2d2_amd import nets
+    from oracle import cells, oracle as orc
+    b = nets._Builder("grouped", (8, 20, 20), 41, "SingleShift")
+    t = b.conv("g2", "input", 64, 3, pad=1, groups=2)
+    t = b.conv("g4", t, 64, 3, stride=2, pad=1, groups=4)
+    t = b.conv("mult2", t, 128, 3, pad=1, groups=64)
+    t = b.pool("pool", t, "avg", 10, 10)
+    b.fc("fc", t, 10, mode="None")
+    spec = b.spec
+    x = np.random.default_rng(41).integers(0, 256, size=(3, 8, 20, 20))
+    keep = [l.name for l in spec.layers]
+    _compare(fh, spec, x, keep)
+    ini = "\n".join(line for line in fh.spec_to_ini(spec, 3).split("\n") if not line.startswith("Mapping."))
+    net = fh.Net(ini)
+    for l in spec.layers:
+        if l.type == "conv":
+            net.set_mapping(l.name, orc.group_maps(l.w.shape[1] * l.groups, l.w.shape[0], l.groups).T)
+    fh.install_parameters(net, spec)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        assert np.array_equal(net.outputs(name), want[name]), name
+
+
 def test_depthwise_and_pointwise_cells_run_as_one_launch(fh):
     """DeepNet::planFusion gives a 3x3 depthwise ConvCell to the 1x1 ConvCell that alone reads it where the pair is large
     enough: MobileNet at 256 x 256, batch 8 (blocks 2 to 4); same logits as the oracle and as the cells launched apart,

@@ -243,6 +243,29 @@ def test_depthwise_conv_bit_exact(rt, stride):
     assert np.array_equal(conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), want.astype(np.int64))
 
 
+def test_grouped_convolutions_bit_exact(rt):
+    """G equal groups with 1 < G that are not the depthwise case (ConvCell_Frame_Kernels.cpp:89-96,132: the weight of a
+    connected channel is found by its position among the connected ones): shapes for the pipelined, the first-layer-free
+    general and the 4-bit kernels, a depth multiplier (G == C, O == 2 C), a 1x1."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    cases = (  # B, C, O, G, k, stride, pad, weight_bits
+        (3, 64, 128, 2, 3, 1, 1, 8), (2, 12, 18, 3, 5, 2, 2, 8), (2, 32, 64, 32, 3, 1, 1, 8), (2, 128, 64, 4, 1, 1, 0, 8),
+        (2, 64, 64, 4, 3, 1, 1, 4), (1, 6, 20, 2, 3, 2, 0, 8))
+    for (B, Cc, O, G, k, stride, pad, bits) in cases:
+        x = _u8((B, Cc, 11, 9))
+        w = _i8((O, Cc // G, k, k)) if bits == 8 else RNG.integers(-7, 8, size=(O, Cc // G, k, k)).astype(np.int8)
+        bias = RNG.integers(-2000, 2001, size=O).astype(np.int32)
+        spec = _acts(O)["sshift_lin_s" if bits == 8 else "fixed_relu_u"]
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(pad,) * 4, groups=G)
+        conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad,) * 4, groups=G,
+                       weight_bits=bits)
+        got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+        assert np.array_equal(got, want.astype(np.int64)), (B, Cc, O, G, k, stride, pad, bits)
+    with pytest.raises(capi.N2D2HipError, match="do not divide"):
+        rt.Conv(_i8((6, 2, 3, 3)), None, rt.Act(6, **_acts(6)["sshift_lin_s"].kwargs()), capi.U8B, groups=4)
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_depthwise3x3_strip_kernel_against_general_kernel(rt, stride):
     """The 3x3 depthwise kernel (threads walk down strips of rows) against the oracle and against the general depthwise
