@@ -262,6 +262,14 @@ int n2d2hip_conv_forward_sum(n2d2hip_conv_t conv, const n2d2hip_tensor* in, cons
 int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
                              n2d2hip_stream_t stream);
 
+/* The channels of 1 to 8 NHWC byte tensors of one dtype and size, one input behind the other, into `out` (whose C is the
+ * sum of theirs).  ref: src/Cell/ConvCell_Frame.cpp:438-459: a cell with several inputs adds up one weighted sum per input,
+ * each with its own slice of the weights (Cell::getNbChannels counts all inputs' channels), which is the convolution of
+ * the concatenated channels; this is the one extra launch such a cell costs here.  Inputs and output may carry a halo;
+ * only the interior of `out` is written. */
+int n2d2hip_concat_channels(int nb_inputs, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out,
+                            n2d2hip_stream_t stream);
+
 /* Graph-level fusion of a residual bottleneck with 64 middle channels into one launch: `reduce` (1x1, 64 or 256 -> 64),
  * `conv3x3` (3x3, stride 1, padding 1, 64 -> 64) and, unless `expand` is NULL, `expand` (1x1, 64 -> 256) with the two-input
  * ElemWise sum that n2d2hip_conv_fuse_sum has folded into it; the sum's other input is the block's input itself (256

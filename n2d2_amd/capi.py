@@ -34,7 +34,7 @@ SYMBOLS = [
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
-    "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling",
+    "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling", "n2d2hip_concat_channels",
     "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_forward_static", "n2d2hip_sat_weight_backward",
     "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
     "n2d2hip_conv2d_f32_forward", "n2d2hip_conv2d_f32_backward_data", "n2d2hip_conv2d_f32_backward_filter", "n2d2hip_conv2d_f32_workspace_bytes",
@@ -100,6 +100,7 @@ def load():
     lib.n2d2hip_conv_accepts_halo.argtypes = [P]
     lib.n2d2hip_tensor_clear.argtypes = [P, P]
     lib.n2d2hip_conv_fuse_sum.argtypes = [P, P, I, I]
+    lib.n2d2hip_concat_channels.argtypes = [I, P, P, P]
     lib.n2d2hip_conv_forward_sum.argtypes = [P, P, P, P, P]
     lib.n2d2hip_bottleneck_create.argtypes = [P, P, P, P, P]
     lib.n2d2hip_bottleneck_destroy.argtypes = [P]

@@ -351,6 +351,52 @@ int run_scaling_nhwc(const n2d2hip_act_s* act, const n2d2hip_tensor* in, const n
     return run_elemwise(a, false, stream);
 }
 
+// ---------------------------------------------------------------- channel concatenation
+// A cell with several inputs sees their channels one behind the other (ref: src/Cell/ConvCell_Frame.cpp:438-459: the
+// weighted sums of the inputs are added up, each input with its own slice of the weights, which is the convolution of the
+// concatenated channels).  One thread per pixel and group of 4 output channels; inputs may carry a halo (read past it).
+constexpr int CONCAT_MAX = 8;
+struct ConcatArgs {
+    const signed char* in[CONCAT_MAX];
+    int cs[CONCAT_MAX], halo[CONCAT_MAX];
+    int first[CONCAT_MAX + 1];      // first output channel of each input; first[n] = all channels
+    int n;
+    signed char* out;
+    int out_cs, out_halo;
+    int B, H, W;
+    unsigned fill;                  // storage form of 0, for the channels past the last one
+};
+
+__global__ __launch_bounds__(256) void concat_channels_kernel(ConcatArgs p)
+{
+    const int cq = p.out_cs >> 2;
+    const long long total = (long long)p.B * p.H * p.W * cq;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const int g = (int)(idx % cq);
+        const long long pix = idx / cq;
+        const int x = (int)(pix % p.W), y = (int)((pix / p.W) % p.H), b = (int)(pix / ((long long)p.W * p.H));
+        unsigned v = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = 4 * g + j;
+            unsigned byte = p.fill;
+#pragma unroll
+            for (int k = 0; k < CONCAT_MAX; ++k) {
+                if (k < p.n && c >= p.first[k] && c < p.first[k + 1]) {
+                    const int h = p.halo[k];
+                    const long long at = (((long long)b * (p.H + 2 * h) + y + h) * (p.W + 2 * h) + x + h) * p.cs[k] + (c - p.first[k]);
+                    byte = (unsigned char)p.in[k][at];
+                }
+            }
+            v |= (byte & 0xffu) << (8 * j);
+        }
+        const int ho = p.out_halo;
+        const long long at = (((long long)b * (p.H + 2 * ho) + y + ho) * (p.W + 2 * ho) + x + ho) * p.out_cs + 4 * g;
+        *(unsigned*)(p.out + at) = v;
+    }
+}
+
 } // namespace n2d2hip
 
 using namespace n2d2hip;
@@ -514,6 +560,45 @@ int n2d2hip_elemwise_forward(n2d2hip_elemwise_t ew, const n2d2hip_tensor* const*
     if (act->args.kind == EPI_RAW)
         N2D2HIP_REQUIRE(ew->unit_coeff, N2D2HIP_ERR_UNSUPPORTED, "elemwise_forward: non-unit coefficients need a rescaling activation");
     return run_elemwise(a, !ew->unit_coeff, (hipStream_t)stream);
+}
+
+int n2d2hip_concat_channels(int nb_inputs, const n2d2hip_tensor* const* inputs, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    int rc;
+    N2D2HIP_REQUIRE(inputs != nullptr && nb_inputs >= 1 && nb_inputs <= CONCAT_MAX, N2D2HIP_ERR_INVALID,
+                    "concat_channels: %d inputs (1 to %d)", nb_inputs, CONCAT_MAX);
+    if ((rc = check_tensor(out, "concat output", true)))
+        return rc;
+    N2D2HIP_REQUIRE(out->layout == N2D2HIP_NHWC && is_byte_type(out->dtype), N2D2HIP_ERR_UNSUPPORTED, "concat_channels: NHWC byte tensors");
+    ConcatArgs a = {};
+    int channels = 0;
+    for (int k = 0; k < nb_inputs; ++k) {
+        const n2d2hip_tensor* t = inputs[k];
+        if ((rc = check_tensor(t, "concat input", true)))
+            return rc;
+        N2D2HIP_REQUIRE(t->layout == N2D2HIP_NHWC && t->dtype == out->dtype, N2D2HIP_ERR_INVALID,
+                        "concat_channels: input %d has dtype %d, the output %d (one byte type for all, NHWC)", k, t->dtype, out->dtype);
+        N2D2HIP_REQUIRE(t->B == out->B && t->H == out->H && t->W == out->W, N2D2HIP_ERR_INVALID,
+                        "concat_channels: input %d is %dx%dx%d, the output %dx%dx%d", k, t->B, t->H, t->W, out->B, out->H, out->W);
+        a.in[k] = (const signed char*)t->data;
+        a.cs[k] = t->cs;
+        a.halo[k] = t->halo;
+        a.first[k] = channels;
+        channels += t->C;
+    }
+    N2D2HIP_REQUIRE(channels == out->C, N2D2HIP_ERR_INVALID, "concat_channels: the inputs hold %d channels, the output %d", channels, out->C);
+    a.first[nb_inputs] = channels;
+    a.n = nb_inputs;
+    a.out = (signed char*)out->data;
+    a.out_cs = out->cs;
+    a.out_halo = out->halo;
+    a.B = out->B; a.H = out->H; a.W = out->W;
+    a.fill = out->dtype == N2D2HIP_U8B ? 0x80u : 0u;
+    const long long total = (long long)out->B * out->H * out->W * (out->cs / 4);
+    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
+    hipLaunchKernelGGL(concat_channels_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, a);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
 }
 
 } // extern "C"

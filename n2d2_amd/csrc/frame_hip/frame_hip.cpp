@@ -480,7 +480,7 @@ template <class T>
 bool ConvCell_Frame_HIP<T>::fuseDepthwise(Cell_Frame_HIP* depthwise)
 {
     if (mDwPw || !mConv || !depthwise || !depthwise->convHandle() || depthwise->foldedInto() || foldedInto() || mInputs.size() != 1
-        || depthwise->inputTensor(0)->desc().halo != 0)
+        || depthwise->parentCells().size() != 1 || depthwise->inputTensor(0)->desc().halo != 0)
         return false;
     n2d2hip_dw_pw_t fused = nullptr;
     const int rc = n2d2hip_dw_pw_create(depthwise->convHandle(), mConv, &fused);
@@ -525,10 +525,28 @@ void ConvCell_Frame_HIP<T>::setOutputsDims()
 }
 
 template <class T>
+void ConvCell_Frame_HIP<T>::addInput(Cell_Frame_HIP* parent)
+{
+    if (mInputs.empty()) {
+        Cell_Frame_HIP::addInput(parent);
+        return;
+    }
+    if (!parent || !mParentCells[0])
+        throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": several inputs must all be cells");
+    if (parent->getOutputsWidth() != mInW || parent->getOutputsHeight() != mInH || parent->batchSize() != mBatch)
+        throw std::runtime_error("Cell " + mName + ": inputs of different sizes");
+    mParents.push_back(parent);
+    mParentCells.push_back(parent);
+    mInputs.push_back(&parent->getDeviceOutputs());
+    mNbChannels += parent->getNbOutputs();
+    mDirty = true;
+}
+
+template <class T>
 void ConvCell_Frame_HIP<T>::initialize()
 {
-    if (mInputs.size() != 1)
-        throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": exactly one input tensor is supported");
+    if (mInputs.empty())
+        throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": no input");
     allocateOutputs();
 }
 
@@ -544,7 +562,13 @@ void ConvCell_Frame_HIP<T>::launch()
 {
     if (mDwPw)
         checkStatus(n2d2hip_dw_pw_forward(mDwPw, &mFusedDw->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
-    else
+    else if (mInputs.size() > 1) {
+        std::vector<const n2d2hip_tensor*> ins;
+        for (const HipTensor* t : mInputs)
+            ins.push_back(&t->desc());
+        checkStatus(n2d2hip_concat_channels((int)ins.size(), ins.data(), &mGathered.desc(), mStream));
+        checkStatus(n2d2hip_conv_forward(mConv, &mGathered.desc(), &mOutputs.desc(), mStream));
+    } else
         checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
@@ -554,6 +578,14 @@ bool ConvCell_Frame_HIP<T>::prepare()
 {
     n2d2hip_act_t act = activationHandle();
     const int inDType = mInputs[0]->desc().dtype;
+    if (mInputs.size() > 1) {
+        // DeepNetExport::isCellInputsUnsigned (src/Export/DeepNetExport.cpp:298-317) refuses parents of mixed signedness
+        for (const HipTensor* t : mInputs)
+            if (t->desc().dtype != inDType)
+                throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": the inputs mix signed and unsigned outputs");
+        if (mGathered.empty() || mGathered.desc().dtype != inDType || mGathered.desc().C != (int)mNbChannels)
+            mGathered.resize((int)mBatch, (int)mNbChannels, (int)mInH, (int)mInW, inDType);
+    }
     bool rebuilt = false;
     if (mDirty || activationGeneration() != mConvActGen || !mConv || inDType != mConvInDType) {
         clearFusion();
@@ -705,7 +737,7 @@ n2d2hip_pool_desc PoolCell_Frame_HIP<T>::poolDesc() const
 template <class T>
 bool PoolCell_Frame_HIP<T>::fuseFirstConv(Cell_Frame_HIP* conv)
 {
-    if (mFusedConv || !conv || !conv->convHandle() || conv->foldedInto() || mInputs.size() != 1)
+    if (mFusedConv || !conv || !conv->convHandle() || conv->foldedInto() || mInputs.size() != 1 || conv->parentCells().size() != 1)
         return false;
     const n2d2hip_pool_desc d = poolDesc();
     const n2d2hip_tensor& x = conv->inputTensor(0)->desc();
@@ -863,7 +895,7 @@ bool ElemWiseCell_Frame_HIP::foldInputScaling(size_t k, Cell_Frame_HIP* scaling)
 
 bool ElemWiseCell_Frame_HIP::fuseIntoConv(size_t k, Cell_Frame_HIP* conv)
 {
-    if (!mEw || mInputs.size() != 2 || k > 1 || !conv || !conv->convHandle() || mFusedConv)
+    if (!mEw || mInputs.size() != 2 || k > 1 || !conv || !conv->convHandle() || mFusedConv || conv->parentCells().size() != 1)
         return false;
     const int rc = n2d2hip_conv_fuse_sum(conv->convHandle(), mEw, (int)k, sourceOf(mFoldedScaling, mInputs, 1 - k)->desc().dtype);
     if (rc == N2D2HIP_ERR_UNSUPPORTED)
@@ -1623,7 +1655,7 @@ void DeepNet::planFusion()
         for (size_t k = 0; k < parents.size(); ++k) {
             Cell_Frame_HIP* p = parents[k];
             if (!p) continue;
-            if (f->convHandle() && n2d2hip_conv_accepts_halo(f->convHandle()))
+            if (f->convHandle() && parents.size() == 1 && n2d2hip_conv_accepts_halo(f->convHandle()))
                 halo[p] = std::max(halo[p], f->maxPadding());
             else if (ew && ew->fusedConv() && k != ew->fusedIndex() && !ew->hasFoldedScaling(k))
                 continue;

@@ -522,6 +522,12 @@ public:
         return std::make_shared<ConvCell_Frame_HIP<T> >(deepNet, name, kernelDims, nbOutputs, subSampleDims, strideDims,
                                                         paddingDims, dilationDims, activation);
     }
+    // Several inputs (ConvCell_Frame<T>::propagate, src/Cell/ConvCell_Frame.cpp:438-459, adds up one weighted sum per
+    // input, each with its slice of the weights): the cell's channels are all inputs' channels one behind the other, its
+    // weights {kW, kH, all channels / groups, nbOutputs}.  The inputs are gathered into one tensor by an extra launch and
+    // the convolution reads that; such a cell takes no part in the graph-level fusions.
+    void addInput(Cell_Frame_HIP* parent);
+    using Cell_Frame_HIP::addInput;
     void initialize();
     void propagate(bool inference = false);
     bool prepare();
@@ -543,6 +549,7 @@ private:
     n2d2hip_conv_t mConv;
     unsigned long mConvActGen;
     int mConvInDType;
+    HipTensor mGathered;        // the inputs' channels, one input behind the other (cells with several inputs)
     n2d2hip_dw_pw_t mDwPw;
     Cell_Frame_HIP* mFusedDw;
     static Registrar<ConvCell> mRegistrar;

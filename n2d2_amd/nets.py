@@ -198,10 +198,11 @@ class _Builder:
 
     def conv(self, name, inp, O, k, stride=1, pad=0, kind="Rectifier", groups=1, wstd=30.0, wmax=127, weight_bits=8,
              bias=True, nb_bits=None, mode=None, clip=False, uniform=False):
-        C, H, W = self.spec.shapes[inp]
+        inps = list(inp) if isinstance(inp, (list, tuple)) else [inp]     # several inputs: their channels one behind the other
+        C, (H, W) = sum(self.spec.shapes[i][0] for i in inps), self.spec.shapes[inps[0]][1:]
         w = self._weights((O, C // groups, k, k), wstd, wmax, uniform)
         p4 = (pad, pad, pad, pad)
-        acc = _conv_acc_np(self.values[inp], w.astype(np.int64), (stride, stride), p4, groups)
+        acc = _conv_acc_np(np.concatenate([self.values[i] for i in inps], 0), w.astype(np.int64), (stride, stride), p4, groups)
         b = None
         if bias:
             mag = max(int(np.percentile(np.abs(acc), 90) / 4), 16)
@@ -209,7 +210,7 @@ class _Builder:
             acc = acc + b[:, None, None]
         act = self._make_act(acc, kind, O, nb_bits, mode, clip)
         self.values[name] = act.apply_np(acc, 0)
-        l = Layer(name, "conv", [inp], w=w, bias=b, stride=(stride, stride), pad=p4, dil=(1, 1), groups=groups,
+        l = Layer(name, "conv", inps, w=w, bias=b, stride=(stride, stride), pad=p4, dil=(1, 1), groups=groups,
                   weight_bits=weight_bits, act=act)
         return self.spec.add(l, (O,) + acc.shape[1:], act.unsigned_out)
 
@@ -338,6 +339,23 @@ def resnet18_w4a4(seed=5, image=224):
     return b.spec
 
 
+def branches_net(seed=43):
+    """A small net whose cells read several cells at once (N2D2 writes a concatenation this way: the reader's channels are
+    its inputs' channels one behind the other): three branches off a stem joined by a 3x3 convolution, that and one branch
+    joined again by a 1x1 convolution, a residual sum, global average, FC."""
+    b = _Builder("branches", (3, 24, 24), seed, "SingleShift")
+    stem = b.conv("stem", "input", 64, 3, stride=2, pad=1)
+    a = b.conv("a3", stem, 64, 3, pad=1)
+    c = b.conv("b1", stem, 32, 1)
+    d = b.pool("bpool", stem, "max", 3, 1, pad=1)
+    j = b.conv("join", [a, c, d], 128, 3, pad=1)
+    k = b.conv("join1", [j, c], 64, 1, kind="Linear")
+    t = b.sum("sum", [k, stem])
+    t = b.pool("pool", t, "avg", 12, 12)
+    b.fc("fc", t, 10, mode="None")
+    return b.spec
+
+
 def single_conv_stage(seed=2):
     """One ResNet-18 stage conv: 3x3 s1 p1 64->64 on 56x56, u8 input, N(0,40) weights, per-channel single shift in
     [8,12], ReLU clip [0,255]."""
@@ -388,7 +406,7 @@ class GpuNet:
         C, H, W = spec.in_shape
 
         def reads_halo(m):
-            return (m.type == "conv" and m.groups == 1 and m.weight_bits in (4, 8) and m.w.shape[1] % 64 == 0
+            return (m.type == "conv" and len(m.inputs) == 1 and m.groups == 1 and m.weight_bits in (4, 8) and m.w.shape[1] % 64 == 0
                     and m.w.shape[2] * m.w.shape[3] <= 31 and tuple(m.dil) == (1, 1))
 
         def halo_of(l, cell):
@@ -413,7 +431,12 @@ class GpuNet:
                 if ins[0].halo and not (l.type == "conv" and cell.accepts_halo()):
                     raise RuntimeError("layer %s cannot read the halo its input was given (GpuNet(halo=False) avoids it)" % l.name)
                 out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype(), halo=halo_of(l, cell) if l.type == "conv" else 0)
-                self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
+                if l.type == "conv" and len(ins) > 1:
+                    # a cell with several inputs: one launch gathers their channels, the convolution reads that
+                    gathered = rt.DTensor(batch, sum(t.C for t in ins), ins[0].H, ins[0].W, ins[0].dtype)
+                    self.steps.append((l, cell, (lambda c, i, o, g=gathered: c.forward(rt.concat_channels(i, g), o))))
+                else:
+                    self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
             elif l.type == "pool":
                 cell = rt.Pool(l.kind, l.pool, l.stride, l.pad)
                 out = rt.DTensor(batch, Co, Ho, Wo, ins[0].dtype)
@@ -440,7 +463,7 @@ class GpuNet:
                     for k in (1, 0):
                         prod = by_name.get(l.inputs[k])
                         other = l.inputs[1 - k]
-                        if (prod is None or prod.type != "conv" or prod.groups != 1 or len(consumers[prod.name]) != 1
+                        if (prod is None or prod.type != "conv" or prod.groups != 1 or len(prod.inputs) != 1 or len(consumers[prod.name]) != 1
                                 or prod.name in self.folded or other in self.folded and by_name[other].type != "scaling"):
                             continue
                         other_src = by_name[other].inputs[0] if other in self.folded else other
@@ -478,7 +501,7 @@ class GpuNet:
                 if l.type != "pool" or l.kind != "max":
                     continue
                 conv = by_name.get(l.inputs[0])
-                if conv is None or conv.type != "conv" or len(consumers[conv.name]) != 1 or conv.name in self.folded:
+                if conv is None or conv.type != "conv" or len(conv.inputs) != 1 or len(consumers[conv.name]) != 1 or conv.name in self.folded:
                     continue
                 conv_cell, pool_cell = self.steps[step_index[conv.name]][1], self.steps[step_index[l.name]][1]
                 x = ins_of[conv.name][0]
@@ -494,10 +517,10 @@ class GpuNet:
         if fuse and dw_pw:
             step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
             for l in spec.layers:
-                if l.type != "conv" or l.groups != 1 or l.w.shape[2:] != (1, 1) or l.name in self.folded:
+                if l.type != "conv" or len(l.inputs) != 1 or l.groups != 1 or l.w.shape[2:] != (1, 1) or l.name in self.folded:
                     continue
                 dw = by_name.get(l.inputs[0])
-                if (dw is None or dw.type != "conv" or dw.groups == 1 or len(consumers[dw.name]) != 1 or dw.name in self.folded
+                if (dw is None or dw.type != "conv" or len(dw.inputs) != 1 or dw.groups == 1 or len(consumers[dw.name]) != 1 or dw.name in self.folded
                         or ins_of[dw.name][0].halo or self.tensors[l.name].halo):
                     continue
                 fused_cell = rt.DwPw.create(self.steps[step_index[dw.name]][1], self.steps[step_index[l.name]][1])
@@ -617,7 +640,8 @@ class GpuNet:
                 expand, proj = other_layer, holder
             conv_b = by_name.get(expand.inputs[0])
             conv_a = by_name.get(conv_b.inputs[0]) if conv_b is not None and conv_b.type == "conv" else None
-            if conv_a is None or conv_a.type != "conv" or len(consumers[conv_a.name]) != 1 or len(consumers[conv_b.name]) != 1:
+            if (conv_a is None or conv_a.type != "conv" or len(consumers[conv_a.name]) != 1 or len(consumers[conv_b.name]) != 1
+                    or len(conv_a.inputs) != 1 or len(conv_b.inputs) != 1 or len(expand.inputs) != 1):
                 continue
             xname = conv_a.inputs[0]
             x = self.tensors.get(xname)

@@ -321,6 +321,16 @@ class Pool:
         return out
 
 
+def concat_channels(xs, out=None, halo=0):
+    """The channels of the tensors xs (one dtype, one size) one behind the other: what a cell with several inputs reads."""
+    x0 = xs[0]
+    if out is None:
+        out = DTensor(x0.B, sum(x.C for x in xs), x0.H, x0.W, x0.dtype, halo=halo)
+    arr = (C.c_void_p * len(xs))(*[C.addressof(x.desc) for x in xs])
+    check(lib.n2d2hip_concat_channels(len(xs), arr, out.ref, stream_ptr()))
+    return out
+
+
 class ElemWiseSum:
     def __init__(self, nb_inputs, nb_channels, act, weights=None, shifts=None, coeff_mode="PerLayer"):
         mode = {"PerLayer": capi.COEFF_PER_LAYER, "PerInput": capi.COEFF_PER_INPUT, "PerChannel": capi.COEFF_PER_CHANNEL}[coeff_mode]

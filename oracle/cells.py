@@ -45,12 +45,25 @@ class ActSpec:
 
 
 def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    """x: one input, or a list of inputs: ConvCell_Frame<T>::propagate (src/Cell/ConvCell_Frame.cpp:438-459) then walks
+    them with its slice of the weights each, beta = 0 for the first and 1 afterwards."""
     w = np.ascontiguousarray(w, dtype=np.float32)
-    maps = None
-    if groups > 1:
-        maps = orc.group_maps(x.shape[1], w.shape[0], groups)
-    y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps)
+    if isinstance(x, (list, tuple)) and len(x) > 1:
+        if groups != 1:
+            raise ValueError("several inputs with a grouped mapping are not restated")
+        y, first = None, 0
+        for k, xk in enumerate(x):
+            xk = np.ascontiguousarray(xk, dtype=np.float32)
+            wk = np.ascontiguousarray(w[:, first:first + xk.shape[1]])
+            y = orc.conv_forward(xk, wk, stride=stride, pad=pad, dil=dil, out=y, beta=0.0 if k == 0 else 1.0)
+            first += xk.shape[1]
+        assert first == w.shape[1]
+    else:
+        x = np.ascontiguousarray(x[0] if isinstance(x, (list, tuple)) else x, dtype=np.float32)
+        maps = None
+        if groups > 1:
+            maps = orc.group_maps(x.shape[1], w.shape[0], groups)
+        y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps)
     if bias is not None:
         orc.conv_forward_bias(y, np.asarray(bias, dtype=np.float32))
     return act.apply(y)
@@ -89,7 +102,7 @@ def run_net(spec, x, keep=None):
             a = l.act
             act = ActSpec(a.kind, a.mode, a.scaling, a.frac_bits, a.clipping, a.nb_bits, a.unsigned_out)
         if l.type == "conv":
-            y = conv_cell(ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups)
+            y = conv_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups)
         elif l.type == "fc":
             y = fc_cell(ins[0], l.w, l.bias, act)
         elif l.type == "pool":

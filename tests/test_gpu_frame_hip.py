@@ -207,6 +207,23 @@ def test_grouped_convolution_cells(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+def test_convolution_cells_with_several_inputs(fh):
+    """Cells whose Input lists several cells see those cells' channels one behind the other (src/Cell/ConvCell_Frame.cpp:
+    438-459): two such ConvCells, one of them feeding a sum, through the Registrar cells with and without the fusion plan
+    (the cell with several inputs keeps its own launch), every output against the oracle."""
+    from n2d2_amd import nets
+    spec = nets.branches_net()
+    x = np.random.default_rng(43).integers(0, 256, size=(3, 3, 24, 24))
+    keep = [l.name for l in spec.layers]
+    net = _compare(fh, spec, x, keep, fusion=False)
+    net.set_fusion(True)
+    net.propagate()
+    from oracle import cells
+    want = cells.run_net(spec, x, keep=["join", "sum", "fc"])
+    for name in ("join", "sum", "fc"):
+        assert np.array_equal(net.outputs(name), want[name]), name
+
+
 def test_depthwise_and_pointwise_cells_run_as_one_launch(fh):
     """DeepNet::planFusion gives a 3x3 depthwise ConvCell to the 1x1 ConvCell that alone reads it where the pair is large
     enough: MobileNet at 256 x 256, batch 8 (blocks 2 to 4); same logits as the oracle and as the cells launched apart,

@@ -266,6 +266,36 @@ def test_grouped_convolutions_bit_exact(rt):
         rt.Conv(_i8((6, 2, 3, 3)), None, rt.Act(6, **_acts(6)["sshift_lin_s"].kwargs()), capi.U8B, groups=4)
 
 
+def test_concat_channels_and_convolution_of_several_inputs(rt):
+    """n2d2hip_concat_channels against numpy (odd channel counts, inputs and output with borders, both byte types; the
+    channels past the last one hold the stored form of 0), and a ConvCell with three inputs (src/Cell/ConvCell_Frame.cpp:
+    438-459: one weighted sum per input, added up) as the convolution of the gathered channels, against the oracle."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    for dtype, make in ((capi.U8B, _u8), (capi.I8, _i8)):
+        xs = [make((2, 5, 7, 6)), make((2, 16, 7, 6)), make((2, 3, 7, 6))]
+        ts = [rt.DTensor.from_numpy(x, dtype) for x in xs]
+        ts[1] = ts[1].with_halo(1)
+        want = np.concatenate(xs, 1).astype(np.int64)
+        for halo in (0, 2):
+            out = rt.concat_channels(ts, halo=halo)
+            assert np.array_equal(out.to_numpy(), want), (dtype, halo)
+            raw = out.raw().reshape(2, 7 + 2 * halo, 6 + 2 * halo, out.cs)[:, halo:7 + halo, halo:6 + halo, 24:]
+            assert np.all(raw.view(np.uint8) == (0x80 if dtype == capi.U8B else 0)), (dtype, halo)
+    xs = [_u8((2, 5, 7, 6)), _u8((2, 16, 7, 6)), _u8((2, 3, 7, 6))]
+    w = _i8((20, 24, 3, 3))
+    bias = RNG.integers(-2000, 2001, size=20).astype(np.int32)
+    spec = _acts(20)["sshift_lin_s"]
+    want = cells_ref.conv_cell(xs, w, bias, spec, pad=(1, 1, 1, 1))
+    conv = rt.Conv(w, bias, rt.Act(20, **spec.kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    got = conv.forward(rt.concat_channels([rt.DTensor.from_numpy(x, capi.U8B) for x in xs])).to_numpy()
+    assert np.array_equal(got, want.astype(np.int64))
+    with pytest.raises(capi.N2D2HipError, match="one byte type"):
+        rt.concat_channels([rt.DTensor.from_numpy(xs[0], capi.U8B), rt.DTensor.from_numpy(_i8((2, 3, 7, 6)), capi.I8)])
+    with pytest.raises(capi.N2D2HipError, match="channels"):
+        rt.concat_channels([rt.DTensor.from_numpy(xs[0], capi.U8B)], out=rt.DTensor(2, 6, 7, 6, capi.U8B))
+
+
 @pytest.mark.parametrize("stride", [1, 2])
 def test_depthwise3x3_strip_kernel_against_general_kernel(rt, stride):
     """The 3x3 depthwise kernel (threads walk down strips of rows) against the oracle and against the general depthwise

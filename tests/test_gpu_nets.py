@@ -26,6 +26,16 @@ def _run_both(spec, x, keep, fuse=True):
     return net
 
 
+def test_cells_with_several_inputs():
+    """Convolutions that read several cells (their channels one behind the other), fused plan and cell by cell."""
+    from n2d2_amd import nets
+    spec = nets.branches_net()
+    x = np.random.default_rng(44).integers(0, 256, size=(3, 3, 24, 24))
+    keep = [l.name for l in spec.layers]
+    _run_both(spec, x, keep)
+    _run_both(spec, x, keep, fuse=False)
+
+
 def test_lenet_config_full_batch():
     from n2d2_amd import nets
     spec = nets.lenet()

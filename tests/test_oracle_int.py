@@ -108,6 +108,22 @@ def test_conv_groups_and_depthwise(groups):
     assert np.array_equal(got.astype(np.int64), want)
 
 
+def test_conv_cell_with_several_inputs_is_the_convolution_of_their_concatenated_channels():
+    """ConvCell_Frame<T>::propagate (src/Cell/ConvCell_Frame.cpp:438-459) adds one weighted sum per input, each with its
+    slice of the weights: against the textbook correlation over all channels, with stride, padding and a bias."""
+    from oracle import cells
+
+    class Identity:
+        def apply(self, y):
+            return y
+    xs = [_u8((2, 5, 9, 8)), _u8((2, 3, 9, 8)), _u8((2, 16, 9, 8))]
+    w = _i8((7, 24, 3, 3))
+    bias = np.arange(-3, 4, dtype=np.int32) * 1000
+    got = cells.conv_cell(xs, w, bias, Identity(), stride=(2, 1), pad=(1, 1, 1, 1))
+    want = rm.conv_int(np.concatenate(xs, 1), w, stride=(2, 1), pad=(1, 1)) + bias[None, :, None, None]
+    assert np.array_equal(got.astype(np.int64), want)
+
+
 def test_nb_groups_irregular_mapping_is_flagged():
     m = orc.group_maps(4, 4, 2)
     m[3, 0] = 1
