@@ -266,6 +266,38 @@ void Cell_Frame_HIP::addInput(HipTensor& stimuli, unsigned int nbChannels, unsig
     setOutputsDims();
 }
 
+void Cell_Frame_HIP::addInputChannels(Cell_Frame_HIP* parent)
+{
+    if (!parent || mInputs.empty() || !mParentCells[0])
+        throw std::runtime_error("Cell " + mName + ": several inputs must all be cells");
+    if (parent->getOutputsWidth() != mInW || parent->getOutputsHeight() != mInH || parent->batchSize() != mBatch)
+        throw std::runtime_error("Cell " + mName + ": inputs of different sizes");
+    mParents.push_back(parent);
+    mParentCells.push_back(parent);
+    mInputs.push_back(&parent->mOutputs);
+    mNbChannels += parent->getNbOutputs();
+}
+
+int Cell_Frame_HIP::prepareGathered()
+{
+    const int dtype = mInputs.at(0)->desc().dtype;
+    for (const HipTensor* t : mInputs)
+        if (t->desc().dtype != dtype)
+            throw std::runtime_error("Cell " + mName + ": the inputs mix signed and unsigned outputs");
+    if (mInputs.size() > 1 && (mGathered.empty() || mGathered.desc().dtype != dtype || mGathered.desc().C != (int)mNbChannels))
+        mGathered.resize((int)mBatch, (int)mNbChannels, (int)mInH, (int)mInW, dtype);
+    return dtype;
+}
+
+const n2d2hip_tensor& Cell_Frame_HIP::gatherInputs()
+{
+    std::vector<const n2d2hip_tensor*> ins;
+    for (const HipTensor* t : mInputs)
+        ins.push_back(&t->desc());
+    checkStatus(n2d2hip_concat_channels((int)ins.size(), ins.data(), &mGathered.desc(), mStream));
+    return mGathered.desc();
+}
+
 void Cell_Frame_HIP::clearInputs()
 {
     mInputs.clear();
@@ -527,18 +559,10 @@ void ConvCell_Frame_HIP<T>::setOutputsDims()
 template <class T>
 void ConvCell_Frame_HIP<T>::addInput(Cell_Frame_HIP* parent)
 {
-    if (mInputs.empty()) {
+    if (mInputs.empty())
         Cell_Frame_HIP::addInput(parent);
-        return;
-    }
-    if (!parent || !mParentCells[0])
-        throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": several inputs must all be cells");
-    if (parent->getOutputsWidth() != mInW || parent->getOutputsHeight() != mInH || parent->batchSize() != mBatch)
-        throw std::runtime_error("Cell " + mName + ": inputs of different sizes");
-    mParents.push_back(parent);
-    mParentCells.push_back(parent);
-    mInputs.push_back(&parent->getDeviceOutputs());
-    mNbChannels += parent->getNbOutputs();
+    else
+        addInputChannels(parent);
     mDirty = true;
 }
 
@@ -562,13 +586,9 @@ void ConvCell_Frame_HIP<T>::launch()
 {
     if (mDwPw)
         checkStatus(n2d2hip_dw_pw_forward(mDwPw, &mFusedDw->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
-    else if (mInputs.size() > 1) {
-        std::vector<const n2d2hip_tensor*> ins;
-        for (const HipTensor* t : mInputs)
-            ins.push_back(&t->desc());
-        checkStatus(n2d2hip_concat_channels((int)ins.size(), ins.data(), &mGathered.desc(), mStream));
-        checkStatus(n2d2hip_conv_forward(mConv, &mGathered.desc(), &mOutputs.desc(), mStream));
-    } else
+    else if (mInputs.size() > 1)
+        checkStatus(n2d2hip_conv_forward(mConv, &gatherInputs(), &mOutputs.desc(), mStream));
+    else
         checkStatus(n2d2hip_conv_forward(mConv, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
@@ -577,15 +597,7 @@ template <class T>
 bool ConvCell_Frame_HIP<T>::prepare()
 {
     n2d2hip_act_t act = activationHandle();
-    const int inDType = mInputs[0]->desc().dtype;
-    if (mInputs.size() > 1) {
-        // DeepNetExport::isCellInputsUnsigned (src/Export/DeepNetExport.cpp:298-317) refuses parents of mixed signedness
-        for (const HipTensor* t : mInputs)
-            if (t->desc().dtype != inDType)
-                throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": the inputs mix signed and unsigned outputs");
-        if (mGathered.empty() || mGathered.desc().dtype != inDType || mGathered.desc().C != (int)mNbChannels)
-            mGathered.resize((int)mBatch, (int)mNbChannels, (int)mInH, (int)mInW, inDType);
-    }
+    const int inDType = prepareGathered();
     bool rebuilt = false;
     if (mDirty || activationGeneration() != mConvActGen || !mConv || inDType != mConvInDType) {
         clearFusion();
@@ -632,7 +644,7 @@ void FcCell::setParameter(const std::string& name, bool value)
 template <class T>
 FcCell_Frame_HIP<T>::FcCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
                                       const std::shared_ptr<Activation>& activation)
-    : Cell(name, nbOutputs), mFc(nullptr), mFcActGen(0)
+    : Cell(name, nbOutputs), mFc(nullptr), mFcActGen(0), mFcNbInputs(0)
 {
     mActivation = activation;
 }
@@ -651,10 +663,20 @@ void FcCell_Frame_HIP<T>::setOutputsDims()
 }
 
 template <class T>
+void FcCell_Frame_HIP<T>::addInput(Cell_Frame_HIP* parent)
+{
+    if (mInputs.empty())
+        Cell_Frame_HIP::addInput(parent);
+    else
+        addInputChannels(parent);
+    mDirty = true;
+}
+
+template <class T>
 void FcCell_Frame_HIP<T>::initialize()
 {
-    if (mInputs.size() != 1)
-        throw std::runtime_error("FcCell_Frame_HIP " + mName + ": exactly one input tensor is supported");
+    if (mInputs.empty())
+        throw std::runtime_error("FcCell_Frame_HIP " + mName + ": no input");
     allocateOutputs();
 }
 
@@ -662,8 +684,8 @@ template <class T>
 void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
     n2d2hip_act_t act = activationHandle();
-    const int inDType = mInputs[0]->desc().dtype;
-    if (mDirty || activationGeneration() != mFcActGen || !mFc) {
+    const int inDType = prepareGathered();
+    if (mDirty || activationGeneration() != mFcActGen || !mFc || mFcNbInputs != mInputs.size()) {
         if (mFc) { n2d2hip_fc_destroy(mFc); mFc = nullptr; }
         const size_t K = (size_t)mNbChannels * mInH * mInW;
         if (mWeights.size() != K * mNbOutputs)
@@ -673,16 +695,23 @@ void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
         if (!mNoBias) {
             if (mBias.size() != mNbOutputs)
                 throw std::runtime_error("FcCell_Frame_HIP " + mName + ": one bias per output expected");
-            for (size_t i = 0; i < mBias.size(); ++i)
-                b.push_back((std::int32_t)toInteger(mBias(i), std::numeric_limits<std::int32_t>::min(), std::numeric_limits<std::int32_t>::max(),
-                                                    "Cell " + mName + " biases"));
+            // every input's inner product starts from the bias (src/Cell/FcCell_Frame.cpp:309) and the products are added up
+            const long long n = (long long)mInputs.size();
+            for (size_t i = 0; i < mBias.size(); ++i) {
+                const long long one = toInteger(mBias(i), std::numeric_limits<std::int32_t>::min(), std::numeric_limits<std::int32_t>::max(),
+                                                "Cell " + mName + " biases");
+                if (one * n < std::numeric_limits<std::int32_t>::min() || one * n > std::numeric_limits<std::int32_t>::max())
+                    throw std::runtime_error("FcCell_Frame_HIP " + mName + ": the bias, added once per input, leaves 32 bits");
+                b.push_back((std::int32_t)(one * n));
+            }
         }
         checkStatus(n2d2hip_fc_create((int)mNbChannels, (int)mInH, (int)mInW, (int)mNbOutputs, 8, w.data(), mNoBias ? nullptr : b.data(), act,
                                       inDType, &mFc));
         mFcActGen = activationGeneration();
+        mFcNbInputs = mInputs.size();
         mDirty = false;
     }
-    checkStatus(n2d2hip_fc_forward(mFc, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    checkStatus(n2d2hip_fc_forward(mFc, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
 

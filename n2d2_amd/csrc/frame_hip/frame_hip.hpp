@@ -442,6 +442,15 @@ protected:
     virtual void setOutputsDims() = 0;
     // (Re)builds the device tables of the activation when its Scaling, its bit width or the
     // signedness decision changed; cells without activation get a pass-through / Scaling-only table.
+    // A further input of a cell whose channels are all its inputs' channels one behind the other (Conv, Fc): same size and
+    // batch as the first one, and all of them cells.
+    void addInputChannels(Cell_Frame_HIP* parent);
+    // Checks that the inputs share one storage type (DeepNetExport::isCellInputsUnsigned, src/Export/DeepNetExport.cpp:298-317,
+    // refuses parents of mixed signedness) and sizes the tensor their channels are gathered into.  Returns that type.
+    int prepareGathered();
+    // Gathers the inputs' channels (one launch) and returns the tensor the cell's kernel then reads.
+    const n2d2hip_tensor& gatherInputs();
+    HipTensor mGathered;
     n2d2hip_act_t activationHandle(const Scaling* standalone = nullptr);
     // Counts the handles activationHandle() has made.  A cell remembers the count its own device handle was built at:
     // the handle's address says nothing, a new one may be allocated where the one before it was.
@@ -549,7 +558,6 @@ private:
     n2d2hip_conv_t mConv;
     unsigned long mConvActGen;
     int mConvInDType;
-    HipTensor mGathered;        // the inputs' channels, one input behind the other (cells with several inputs)
     n2d2hip_dw_pw_t mDwPw;
     Cell_Frame_HIP* mFusedDw;
     static Registrar<ConvCell> mRegistrar;
@@ -592,6 +600,11 @@ public:
     {
         return std::make_shared<FcCell_Frame_HIP<T> >(deepNet, name, nbOutputs, activation);
     }
+    // Several inputs (FcCell_Frame<T>::propagate, src/Cell/FcCell_Frame.cpp:273-336): one inner product per input over its
+    // own weights, added up, and the bias added once per input (`:309` seeds every input's product with it).  The inputs'
+    // channels are gathered by one extra launch; the weights are {all inputs' values in CHW order, nbOutputs}.
+    void addInput(Cell_Frame_HIP* parent);
+    using Cell_Frame_HIP::addInput;
     void initialize();
     void propagate(bool inference = false);
 
@@ -601,6 +614,7 @@ protected:
 private:
     n2d2hip_fc_t mFc;
     unsigned long mFcActGen;
+    size_t mFcNbInputs;
     static Registrar<FcCell> mRegistrar;
 };
 

@@ -215,15 +215,16 @@ class _Builder:
         return self.spec.add(l, (O,) + acc.shape[1:], act.unsigned_out)
 
     def fc(self, name, inp, O, kind="Linear", wstd=30.0, wmax=127, weight_bits=8, mode=None, nb_bits=None, uniform=False):
-        C, H, W = self.spec.shapes[inp]
-        w = self._weights((O, C * H * W), wstd, wmax, uniform)
-        acc = w.astype(np.int64) @ self.values[inp].reshape(-1)
+        inps = list(inp) if isinstance(inp, (list, tuple)) else [inp]     # several inputs: their values one input behind the other
+        flat = np.concatenate([self.values[i].reshape(-1) for i in inps])
+        w = self._weights((O, flat.size), wstd, wmax, uniform)
+        acc = w.astype(np.int64) @ flat
         mag = max(int(np.percentile(np.abs(acc), 90) / 4), 16)
         b = self.rng.integers(-mag, mag + 1, size=O).astype(np.int32)
-        acc = (acc + b).reshape(O, 1, 1)
+        acc = (acc + len(inps) * b.astype(np.int64)).reshape(O, 1, 1)     # FcCell_Frame.cpp:309: the bias once per input
         act = self._make_act(acc, kind, O, nb_bits, mode)
         self.values[name] = act.apply_np(acc, 0)
-        l = Layer(name, "fc", [inp], w=w, bias=b, weight_bits=weight_bits, act=act)
+        l = Layer(name, "fc", inps, w=w, bias=b, weight_bits=weight_bits, act=act)
         return self.spec.add(l, (O, 1, 1), act.unsigned_out)
 
     def pool(self, name, inp, kind, pool, stride, pad=0):
@@ -352,7 +353,8 @@ def branches_net(seed=43):
     k = b.conv("join1", [j, c], 64, 1, kind="Linear")
     t = b.sum("sum", [k, stem])
     t = b.pool("pool", t, "avg", 12, 12)
-    b.fc("fc", t, 10, mode="None")
+    u = b.pool("pool_b", c, "avg", 12, 12)
+    b.fc("fc", [t, u], 10, mode="None")
     return b.spec
 
 
@@ -427,11 +429,13 @@ class GpuNet:
                 if l.type == "conv":
                     cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits, kernel_choice)
                 else:
-                    cell = rt.Fc(l.w, l.bias, act, ins[0].dtype, (ins[0].C, ins[0].H, ins[0].W), l.weight_bits)
+                    # several inputs: each inner product starts from the bias and they are added up (FcCell_Frame.cpp:309)
+                    cell = rt.Fc(l.w, None if l.bias is None else l.bias * len(ins), act, ins[0].dtype,
+                                 (sum(t.C for t in ins), ins[0].H, ins[0].W), l.weight_bits)
                 if ins[0].halo and not (l.type == "conv" and cell.accepts_halo()):
                     raise RuntimeError("layer %s cannot read the halo its input was given (GpuNet(halo=False) avoids it)" % l.name)
                 out = rt.DTensor(batch, Co, Ho, Wo, act.out_dtype(), halo=halo_of(l, cell) if l.type == "conv" else 0)
-                if l.type == "conv" and len(ins) > 1:
+                if len(ins) > 1:
                     # a cell with several inputs: one launch gathers their channels, the convolution reads that
                     gathered = rt.DTensor(batch, sum(t.C for t in ins), ins[0].H, ins[0].W, ins[0].dtype)
                     self.steps.append((l, cell, (lambda c, i, o, g=gathered: c.forward(rt.concat_channels(i, g), o))))

@@ -70,8 +70,18 @@ def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), grou
 
 
 def fc_cell(x, w, bias, act):
-    x = np.ascontiguousarray(x, dtype=np.float32)
-    y = orc.fc_forward(x, np.asarray(w, dtype=np.float32), None if bias is None else np.asarray(bias, dtype=np.float32))
+    """x: one input, or a list of inputs: FcCell_Frame<T>::propagate (src/Cell/FcCell_Frame.cpp:273-336) then forms one inner
+    product per input over that input's weights, each seeded with the bias (`:309`), beta = 0 for the first and 1 afterwards."""
+    xs = list(x) if isinstance(x, (list, tuple)) else [x]
+    w = np.asarray(w, dtype=np.float32).reshape(np.asarray(w).shape[0], -1)
+    b = None if bias is None else np.asarray(bias, dtype=np.float32)
+    y, first = None, 0
+    for k, xk in enumerate(xs):
+        xk = np.ascontiguousarray(xk, dtype=np.float32)
+        size = xk[0].size
+        y = orc.fc_forward(xk, np.ascontiguousarray(w[:, first:first + size]), b, out=y, beta=0.0 if k == 0 else 1.0)
+        first += size
+    assert first == w.shape[1]
     return act.apply(y.reshape(y.shape[0], y.shape[1], 1, 1))
 
 
@@ -104,7 +114,7 @@ def run_net(spec, x, keep=None):
         if l.type == "conv":
             y = conv_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups)
         elif l.type == "fc":
-            y = fc_cell(ins[0], l.w, l.bias, act)
+            y = fc_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act)
         elif l.type == "pool":
             y = pool_cell(ins[0], l.kind, l.pool, l.stride, l.pad)
         elif l.type == "scaling":

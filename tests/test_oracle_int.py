@@ -124,6 +124,24 @@ def test_conv_cell_with_several_inputs_is_the_convolution_of_their_concatenated_
     assert np.array_equal(got.astype(np.int64), want)
 
 
+def test_fc_cell_with_several_inputs_adds_the_bias_once_per_input():
+    """FcCell_Frame<T>::propagate (src/Cell/FcCell_Frame.cpp:273-336): one inner product per input, each seeded with the
+    bias (`:309`), added up: the product over all inputs' values plus as many biases as there are inputs."""
+    from oracle import cells
+
+    class Identity:
+        def apply(self, y):
+            return y
+    xs = [_u8((3, 5, 2, 2)), _i8((3, 3, 2, 2)), _u8((3, 1, 2, 2))]
+    w = _i8((4, 36))
+    bias = np.array([5, -7, 100, 0], dtype=np.int32)
+    got = cells.fc_cell(xs, w, bias, Identity()).reshape(3, 4).astype(np.int64)
+    flat = np.concatenate([x.reshape(3, -1) for x in xs], 1).astype(np.int64)
+    assert np.array_equal(got, flat @ w.astype(np.int64).T + 3 * bias)
+    assert np.array_equal(cells.fc_cell(xs[:1], w[:, :20], bias, Identity()).reshape(3, 4).astype(np.int64),
+                          flat[:, :20] @ w[:, :20].astype(np.int64).T + bias)
+
+
 def test_nb_groups_irregular_mapping_is_flagged():
     m = orc.group_maps(4, 4, 2)
     m[3, 0] = 1
