@@ -745,10 +745,19 @@ void PoolCell_Frame_HIP<T>::setOutputsDims()
 }
 
 template <class T>
+void PoolCell_Frame_HIP<T>::addInput(Cell_Frame_HIP* parent)
+{
+    if (mInputs.empty())
+        Cell_Frame_HIP::addInput(parent);
+    else
+        addInputChannels(parent);
+}
+
+template <class T>
 void PoolCell_Frame_HIP<T>::initialize()
 {
-    if (mInputs.size() != 1 || mNbOutputs != mNbChannels)
-        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": one input and a unit mapping (NbOutputs == channels) are supported");
+    if (mInputs.empty() || mNbOutputs != mNbChannels)
+        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": a unit mapping (NbOutputs == the inputs' channels) is supported");
     mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
 }
 
@@ -802,13 +811,14 @@ void PoolCell_Frame_HIP<T>::clearFusion()
 template <class T>
 void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
-    if (mOutputs.empty() || mOutputs.desc().dtype != mInputs[0]->desc().dtype || mOutputs.desc().halo != mOutputsHalo)
-        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype, mOutputsHalo);
+    const int dtype = prepareGathered();
+    if (mOutputs.empty() || mOutputs.desc().dtype != dtype || mOutputs.desc().halo != mOutputsHalo)
+        mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, dtype, mOutputsHalo);
     const n2d2hip_pool_desc d = poolDesc();
     if (mFusedConv)
         checkStatus(n2d2hip_conv_forward_maxpool(mFusedConv->convHandle(), &d, &mFusedConv->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
     else
-        checkStatus(n2d2hip_pool_forward(&d, &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+        checkStatus(n2d2hip_pool_forward(&d, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
 }
 

@@ -652,6 +652,11 @@ public:
     {
         return std::make_shared<PoolCell_Frame_HIP<T> >(deepNet, name, poolDims, nbOutputs, strideDims, paddingDims, pooling, activation);
     }
+    // Several inputs (PoolCell_Frame<T>::propagate, src/Cell/PoolCell_Frame.cpp:123-174, walks them with the rows of the
+    // unit map that belong to each; an output pools nothing from the other inputs): the pooling of all inputs' channels, one
+    // input behind the other, gathered by one extra launch.
+    void addInput(Cell_Frame_HIP* parent);
+    using Cell_Frame_HIP::addInput;
     void initialize();
     void propagate(bool inference = false);
     // src/Cell/PoolCell_Frame.cpp:263-266

@@ -228,11 +228,12 @@ class _Builder:
         return self.spec.add(l, (O, 1, 1), act.unsigned_out)
 
     def pool(self, name, inp, kind, pool, stride, pad=0):
-        v = _pool_np(self.values[inp], kind, (pool, pool), (stride, stride), (pad, pad))
+        inps = list(inp) if isinstance(inp, (list, tuple)) else [inp]     # several inputs: their channels one behind the other
+        v = _pool_np(np.concatenate([self.values[i] for i in inps], 0), kind, (pool, pool), (stride, stride), (pad, pad))
         self.values[name] = v
-        l = Layer(name, "pool", [inp], kind=kind, pool=(pool, pool), stride=(stride, stride), pad=(pad, pad))
+        l = Layer(name, "pool", inps, kind=kind, pool=(pool, pool), stride=(stride, stride), pad=(pad, pad))
         # no activation: range of the parents (PoolCell::getOutputsRange)
-        return self.spec.add(l, v.shape, self.spec.unsigned[inp])
+        return self.spec.add(l, v.shape, all(self.spec.unsigned[i] for i in inps))
 
     def scaling(self, name, inp, frac_bits=14):
         """Stand-alone ScalingCell as `_rescale_branch` leaves it: FIXED_MULT16, factor <= 1, no activation."""
@@ -343,7 +344,8 @@ def resnet18_w4a4(seed=5, image=224):
 def branches_net(seed=43):
     """A small net whose cells read several cells at once (N2D2 writes a concatenation this way: the reader's channels are
     its inputs' channels one behind the other): three branches off a stem joined by a 3x3 convolution, that and one branch
-    joined again by a 1x1 convolution, a residual sum, global average, FC."""
+    joined again by a 1x1 convolution, a residual sum, a global average and a global maximum over two cells each, an FC
+    over both."""
     b = _Builder("branches", (3, 24, 24), seed, "SingleShift")
     stem = b.conv("stem", "input", 64, 3, stride=2, pad=1)
     a = b.conv("a3", stem, 64, 3, pad=1)
@@ -352,8 +354,8 @@ def branches_net(seed=43):
     j = b.conv("join", [a, c, d], 128, 3, pad=1)
     k = b.conv("join1", [j, c], 64, 1, kind="Linear")
     t = b.sum("sum", [k, stem])
-    t = b.pool("pool", t, "avg", 12, 12)
-    u = b.pool("pool_b", c, "avg", 12, 12)
+    t = b.pool("pool", [t, c], "avg", 12, 12)
+    u = b.pool("pool_b", [a, d], "max", 12, 12)
     b.fc("fc", [t, u], 10, mode="None")
     return b.spec
 
@@ -444,7 +446,11 @@ class GpuNet:
             elif l.type == "pool":
                 cell = rt.Pool(l.kind, l.pool, l.stride, l.pad)
                 out = rt.DTensor(batch, Co, Ho, Wo, ins[0].dtype)
-                self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
+                if len(ins) > 1:
+                    gathered = rt.DTensor(batch, sum(t.C for t in ins), ins[0].H, ins[0].W, ins[0].dtype)
+                    self.steps.append((l, cell, (lambda c, i, o, g=gathered: c.forward(rt.concat_channels(i, g), o))))
+                else:
+                    self.steps.append((l, cell, (lambda c, i, o: c.forward(i[0], o))))
             elif l.type == "scaling":
                 cell = rt.Act(Co, **l.act.kwargs())
                 out = rt.DTensor(batch, Co, Ho, Wo, cell.out_dtype())
@@ -502,7 +508,7 @@ class GpuNet:
         if fuse and stem_pool:
             step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
             for l in spec.layers:
-                if l.type != "pool" or l.kind != "max":
+                if l.type != "pool" or l.kind != "max" or len(l.inputs) != 1:
                     continue
                 conv = by_name.get(l.inputs[0])
                 if conv is None or conv.type != "conv" or len(conv.inputs) != 1 or len(consumers[conv.name]) != 1 or conv.name in self.folded:
@@ -565,7 +571,7 @@ class GpuNet:
                 producer_cell = self.steps[step_index[l.name]][1]
                 writes = (l.name in self.fused_sums or l.name in self.stem_pools
                           or (l.type == "conv" and producer_cell.accepts_halo())
-                          or (l.type == "pool" and l.kind == "max" and tuple(l.pool) in ((2, 2), (3, 3))))
+                          or (l.type == "pool" and l.kind == "max" and tuple(l.pool) in ((2, 2), (3, 3)) and len(l.inputs) == 1))
                 if not writes:
                     continue
                 nx = rt.DTensor(t.B, t.C, t.H, t.W, t.dtype, halo=h)
@@ -665,7 +671,8 @@ class GpuNet:
             if x is None or xname == "input" or not {m.name for m in consumers[xname]} <= readers | {sum_name}:
                 continue
             producer = by_name[xname]
-            can_write_halo = (producer.type == "pool" and producer.kind == "max" and tuple(producer.pool) in ((2, 2), (3, 3))) \
+            can_write_halo = (producer.type == "pool" and producer.kind == "max" and tuple(producer.pool) in ((2, 2), (3, 3))
+                              and len(producer.inputs) == 1) \
                 or xname in self.fused_sums or xname in self.bottlenecks
             if x.halo not in (0, 1) or (x.halo == 0 and not can_write_halo):
                 continue

@@ -86,7 +86,21 @@ def fc_cell(x, w, bias, act):
 
 
 def pool_cell(x, kind, pool, stride, pad=(0, 0)):
-    return orc.pool_forward(np.ascontiguousarray(x, dtype=np.float32), pool, stride, pad, kind=kind, quantized=True)
+    """x: one input, or a list of inputs: PoolCell_Frame<T>::propagate (src/Cell/PoolCell_Frame.cpp:123-174) then walks them
+    with the rows of the unit map over all their channels that belong to each, beta = 0 for the first and 1 afterwards (an
+    output pools nothing from the inputs it is not connected to: 0 is added)."""
+    if not isinstance(x, (list, tuple)) or len(x) == 1:
+        x = x[0] if isinstance(x, (list, tuple)) else x
+        return orc.pool_forward(np.ascontiguousarray(x, dtype=np.float32), pool, stride, pad, kind=kind, quantized=True)
+    total = sum(xk.shape[1] for xk in x)
+    unit = np.eye(total, dtype=np.uint8)
+    y, first = None, 0
+    for k, xk in enumerate(x):
+        xk = np.ascontiguousarray(xk, dtype=np.float32)
+        y = orc.pool_forward(xk, pool, stride, pad, kind=kind, quantized=True, maps=unit[first:first + xk.shape[1]], out=y,
+                             beta=0.0 if k == 0 else 1.0)
+        first += xk.shape[1]
+    return y
 
 
 def elemwise_cell(xs, act, weights=None, shifts=None, coeff_mode="PerLayer"):
@@ -116,7 +130,7 @@ def run_net(spec, x, keep=None):
         elif l.type == "fc":
             y = fc_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act)
         elif l.type == "pool":
-            y = pool_cell(ins[0], l.kind, l.pool, l.stride, l.pad)
+            y = pool_cell(ins if len(ins) > 1 else ins[0], l.kind, l.pool, l.stride, l.pad)
         elif l.type == "scaling":
             y = act.apply(ins[0])           # ScalingCell_Frame::propagate: the Scaling alone
         elif l.type == "elemwise":

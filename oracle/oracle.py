@@ -200,9 +200,10 @@ def fc_forward(x, w, bias=None, out=None, beta=0.0):
 
 
 def pool_forward(x, pool, stride, pad=(0, 0), kind="max", quantized=True, maps=None,
-                 count_include_padding=True, argmax=False):
+                 count_include_padding=True, argmax=False, out=None, beta=0.0):
     """PoolCell_Frame_Kernels::forwardMax / forwardAverage with a unit map by
-    default (one output per channel, as PoolCell builds it)."""
+    default (one output per channel, as PoolCell builds it).  out / beta: the
+    kernel's accumulation into an existing output (cells with several inputs)."""
     dt = x.dtype
     x = np.ascontiguousarray(x)
     B, Cin, H, W = x.shape
@@ -212,9 +213,11 @@ def pool_forward(x, pool, stride, pad=(0, 0), kind="max", quantized=True, maps=N
         maps = np.eye(Cin, dtype=np.uint8)
     m = np.ascontiguousarray(maps, dtype=np.uint8)
     O = m.shape[1]
-    out = np.zeros((B, O, oH, oW), dtype=dt)
+    if out is None:
+        out = np.zeros((B, O, oH, oW), dtype=dt)
+    assert out.shape == (B, O, oH, oW) and out.dtype == dt and out.flags["C_CONTIGUOUS"]
     ct = _CT[np.dtype(dt)]
-    a, b = ct(1.0), ct(0.0)
+    a, b = ct(1.0), ct(beta)
     if kind == "max":
         am = np.zeros((B, O, oH, oW, 4), dtype=np.int32) if argmax else None
         _fn("pool_forward_max", dt)(C.byref(a), _p(x), B, Cin, H, W, _ia(pool), _ia(stride), _ia(pad),

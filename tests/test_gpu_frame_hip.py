@@ -209,8 +209,8 @@ def test_grouped_convolution_cells(fh):
 
 def test_convolution_cells_with_several_inputs(fh):
     """Cells whose Input lists several cells see those cells' channels one behind the other (src/Cell/ConvCell_Frame.cpp:
-    438-459): two such ConvCells, one of them feeding a sum, and an FcCell with two inputs (the bias once per input,
-    src/Cell/FcCell_Frame.cpp:309), through the Registrar cells with and without the fusion plan (a cell with several
+    438-459): two such ConvCells, one of them feeding a sum, an average and a max PoolCell over two cells each, and an
+    FcCell with two inputs (the bias once per input, src/Cell/FcCell_Frame.cpp:309), through the Registrar cells with and without the fusion plan (a cell with several
     inputs keeps its own launch), every output against the oracle."""
     from n2d2_amd import nets
     spec = nets.branches_net()

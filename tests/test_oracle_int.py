@@ -230,6 +230,24 @@ def test_pool_max_and_average(pool, stride, pad):
         assert np.array_equal(av[:, :, oy, ox].astype(np.int64), want)
 
 
+def test_pool_cell_with_several_inputs_pools_every_input_on_its_own_channels():
+    """PoolCell_Frame<T>::propagate (src/Cell/PoolCell_Frame.cpp:123-174) over several inputs, unit map over all their
+    channels: window maxima / truncated window means of each input, written behind each other."""
+    from oracle import cells
+    xs = [RNG.integers(-128, 256, size=(2, 3, 9, 8)).astype(np.float32), RNG.integers(-128, 256, size=(2, 5, 9, 8)).astype(np.float32)]
+    xi = np.concatenate(xs, 1).astype(np.int64)
+    pool, stride, pad = (3, 3), (2, 2), (1, 1)
+    mx = cells.pool_cell(xs, "max", pool, stride, pad)
+    av = cells.pool_cell(xs, "avg", pool, stride, pad)
+    assert mx.shape == av.shape == (2, 8, 5, 4)
+    for oy, ox in itertools.product(range(5), range(4)):
+        y0, x0 = oy * 2 - 1, ox * 2 - 1
+        win = xi[:, :, max(y0, 0):min(y0 + 3, 9), max(x0, 0):min(x0 + 3, 8)]
+        assert np.array_equal(mx[:, :, oy, ox].astype(np.int64), win.max(axis=(2, 3)))
+        s = win.sum(axis=(2, 3))
+        assert np.array_equal(av[:, :, oy, ox].astype(np.int64), np.sign(s) * (np.abs(s) // 9))
+
+
 def test_pool_average_exhaustive_rounding_toward_zero():
     # every u8 / i8 window sum a 2x2, 3x3 or 7x7 pool can produce
     for n in (4, 9, 49):
