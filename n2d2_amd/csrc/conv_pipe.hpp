@@ -392,6 +392,24 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         constexpr int NTR = P16 ? 2 : 3 + (EPI == EPI_I24 ? 1 : 0) + (EPI != EPI_F32 ? 1 : 0);      // reads per request
         if (!RES && EPI != EPI_RAW)
             request_tables(tq[0], tab);
+        // The folded sum on 16-bit pairs reads seven tables per channel group: they too are requested one group ahead.
+        v4i rq4[2][4];
+        v2i rq2[2][3];
+        auto request_sum_tables = [&](int set, int group) {
+            const unsigned t32 = tab + (unsigned)((group / 4) * 32 + 8 * (group % 4)) * 4u;
+            const unsigned t16 = tab16 + (unsigned)((group / 4) * 32 + 8 * (group % 4)) * 2u;
+            lds_read128_nowait<3 * BN * 4>(rq4[set][0], t32);
+            lds_read128_nowait<4 * BN * 4>(rq4[set][1], t32);
+            // (the ScalingCell's tables are read whether there is one or not: two reads of whatever the LDS holds cost less
+            // than a branch here)
+            lds_read128_nowait<13 * BN * 4>(rq4[set][2], t32);
+            lds_read128_nowait<14 * BN * 4>(rq4[set][3], t32);
+            lds_read64_nowait<0>(rq2[set][0], t16);
+            lds_read64_nowait<BN * 2>(rq2[set][1], t16);
+            lds_read64_nowait<BN * 4>(rq2[set][2], t16);
+        };
+        if (RES && P16)
+            request_sum_tables(0, 0);
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
 #pragma unroll
@@ -402,22 +420,21 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     // ---- the same three rescales with everything behind the convolution's shift held as pairs of
                     // 16-bit values (channels 2h, 2h+1 of the lane's four): half the instructions per value.  The host
                     // has shown that no intermediate leaves 16 bits and that none of the optional clamps is needed.
-                    const unsigned trow16 = tab16 + (unsigned)(i * 32 + 8 * g) * 2u;
                     // The convolution's and the ScalingCell's multipliers and addends come scaled up by 2^(16 - shift):
                     // the rescaled value is the upper half of the 32-bit result and needs no shift of its own.
-                    v4i tc, td, xc, xd;
-                    v2i c16, d16, e16;
-                    lds_read128_nowait<3 * BN * 4>(tc, trow);
-                    lds_read128_nowait<4 * BN * 4>(td, trow);
-                    // (the ScalingCell's tables are read whether there is one or not: two reads of whatever the LDS
-                    // holds cost less than a branch here)
-                    lds_read128_nowait<13 * BN * 4>(xc, trow);
-                    lds_read128_nowait<14 * BN * 4>(xd, trow);
-                    lds_read64_nowait<0>(c16, trow16);
-                    lds_read64_nowait<BN * 2>(d16, trow16);
-                    lds_read64_nowait<BN * 4>(e16, trow16);
-                    wait_lgkm<5>();
-                    tie(tc); tie(td);
+                    constexpr int SET = (RES && P16) ? 1 : 0;     // (keeps the other instantiations' indices in range)
+                    const int cur = (idx & 1) * SET;
+                    if (idx + 1 < NI * 4) {
+                        request_sum_tables(((idx + 1) & 1) * SET, idx + 1);
+                        wait_lgkm<7>();        // the LDS answers in order: this group's seven reads have arrived
+                    } else {
+                        wait_lgkm<0>();
+                    }
+                    // (every register a read fills is tied after the wait: see above)
+                    tie(rq4[cur][0]); tie(rq4[cur][1]); tie(rq4[cur][2]); tie(rq4[cur][3]);
+                    tie(rq2[cur][0]); tie(rq2[cur][1]); tie(rq2[cur][2]);
+                    const v4i tc = rq4[cur][0], td = rq4[cur][1], xc = rq4[cur][2], xd = rq4[cur][3];
+                    const v2i c16 = rq2[cur][0], d16 = rq2[cur][1], e16 = rq2[cur][2];
                     const v2s lo1 = splat_v2s(vlo), hi1 = splat_v2s(vhi);
                     v2s pq[NJ][2];
 #pragma unroll
@@ -429,8 +446,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                             pq[j][h] = clamp_v2s(as_v2s((int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u)), lo1, hi1);
                         }
                     v2s oq[NJ][2];
-                    wait_lgkm<3>();
-                    tie(xc); tie(xd);
                     if (q.has_pre) {
                         const v2s lo3 = splat_v2s(plo), hi3 = splat_v2s(phi);
 #pragma unroll
@@ -458,8 +473,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                             oq[j][1] = as_v2s((int)__builtin_amdgcn_perm(w, w, 0x0c030c02u));
                         }
                     }
-                    wait_lgkm<0>();
-                    tie(c16); tie(d16); tie(e16);
                     const v2s lo2 = splat_v2s(slo), hi2 = splat_v2s(shi);
 #pragma unroll
                     for (int j = 0; j < NJ; ++j)
