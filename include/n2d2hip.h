@@ -164,7 +164,9 @@ enum {
     N2D2HIP_KERNEL_F32_DIRECT = 64, /* float passes: direct kernels that add in the reference's order */
     N2D2HIP_KERNEL_F32_GEMM = 128,  /* float passes: matrix-core implicit GEMM */
     N2D2HIP_KERNEL_NO_PATCH = 256,  /* integer cells: 3x3 convolutions on the pipelined kernel instead of the patch kernel */
-    N2D2HIP_KERNEL_PATCH = 512      /* the patch kernel wherever it can run, also where the library finds the pipelined one faster */
+    N2D2HIP_KERNEL_PATCH = 512,     /* the patch kernel wherever it can run, also where the library finds the pipelined one faster */
+    N2D2HIP_KERNEL_NO_DIRECT = 1024,/* integer cells with at most 4 input channels and 32 outputs: matrix-core kernel instead of the direct one */
+    N2D2HIP_KERNEL_DIRECT = 2048    /* the direct kernel wherever it can run (up to 16 input channels), also where the library finds the matrix cores faster */
 };
 
 typedef struct n2d2hip_conv_s* n2d2hip_conv_t;

@@ -40,6 +40,8 @@ struct n2d2hip_conv_s {
     int* d_wdw;
     // 4-bit weights for the pipelined kernel: the ring's weight tiles as LDS wants them, two weights per byte
     signed char* d_w4img;
+    // direct kernel for layers with a handful of channels: [tap][8 | 16 | 32 output rows][input channel stride]
+    signed char* d_wsmall;
     bool is_fc;
     int fcH, fcW;
 };

@@ -282,6 +282,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 } // namespace n2d2hip
 #include "conv_pipe.hpp"
 #include "conv_stem.hpp"
+#include "conv_small.hpp"
 namespace n2d2hip {
 
 // ------------------------------------------------------------ depthwise
@@ -515,7 +516,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr; c->d_wsmall = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -689,6 +690,21 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_wstem, ws.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wstem, ws.data(), ws.size(), hipMemcpyHostToDevice);
     }
+    // (a dilated kernel with padding keeps the kernel that follows the reference's window arithmetic tap by tap: what the
+    // reference skips at the borders is then not what zero padding would skip)
+    if (e == hipSuccess && !depthwise && d->weight_bits == 8 && d->kW <= 8 && conv_small_rows(d->C, d->O, d->kW * d->kH)
+        && ((d->dilX == 1 && d->dilY == 1) || (d->padL == 0 && d->padT == 0 && d->padR == 0 && d->padB == 0))
+        && !(d->kernel_choice & N2D2HIP_KERNEL_NO_DIRECT)) {
+        const int taps = d->kW * d->kH;
+        std::vector<signed char> ohwc((size_t)d->O * taps * d->C), img(conv_small_weight_bytes(d->C, d->O, taps));
+        for (int o = 0; o < d->O; ++o)
+            for (int ch = 0; ch < d->C; ++ch)
+                for (int t = 0; t < taps; ++t)
+                    ohwc[((size_t)o * taps + t) * d->C + ch] = (signed char)read_weight(weights, ((long long)o * d->C + ch) * taps + t, 8);
+        conv_small_weight_layout(ohwc.data(), d->C, d->O, taps, img.data());
+        e = hipMalloc((void**)&c->d_wsmall, img.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_wsmall, img.data(), img.size(), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hfrag.empty()) {
         e = hipMalloc((void**)&c->d_wfrag, hfrag.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wfrag, hfrag.data(), hfrag.size(), hipMemcpyHostToDevice);
@@ -733,6 +749,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_res_tab) (void)hipFree(c->d_res_tab);
     if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
     if (c->d_wstem) (void)hipFree(c->d_wstem);
+    if (c->d_wsmall) (void)hipFree(c->d_wsmall);
     if (c->d_wfrag) (void)hipFree(c->d_wfrag);
     if (c->d_wdw) (void)hipFree(c->d_wdw);
     if (c->d_w4img) (void)hipFree(c->d_w4img);
@@ -1025,6 +1042,23 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             N2D2HIP_HIP_CHECK(hipGetLastError());
             return N2D2HIP_OK;
         }
+    }
+    if (c->d_wsmall && !other && !c->is_fc && in->halo == 0 && out->halo == 0 && is_byte_type(out->dtype)
+        && c->act->args.kind != EPI_RAW && (c->pix4 || (d.kernel_choice & N2D2HIP_KERNEL_DIRECT))) {
+        // A handful of channels: one thread per output pixel.  Taken by itself for at most 4 input channels, where the
+        // matrix-core kernel spends its K steps on padding (LeNet's first layer: 29 -> 21 us); with more channels the two
+        // are on a par or the matrix cores ahead (LeNet's second layer: 16 against 20 us).
+        ConvSmallArgs q;
+        q.in = (const signed char*)in->data; q.in_cs = in->cs; q.qn = (d.C + 3) / 4;
+        q.B = in->B; q.H = in->H; q.W = in->W;
+        q.w = c->d_wsmall; q.rows = conv_small_rows(d.C, d.O, d.kW * d.kH); q.bias = c->d_bias;
+        q.out = out->data; q.out_cs = out->cs; q.out_dtype = out->dtype;
+        q.O = d.O; q.OH = OH; q.OW = OW;
+        q.kW = d.kW; q.kH = d.kH; q.strideX = d.strideX; q.strideY = d.strideY; q.padL = d.padL; q.padT = d.padT;
+        q.dilX = d.dilX; q.dilY = d.dilY;
+        q.fill = a.fill;
+        q.epi = c->act->args;
+        return conv_small_launch(q, stream);
     }
     if (c->pix4) {
         if (bn128) { if (w4) launch_cfg<128, 128, 2, true, true>(a, stream); else launch_cfg<128, 128, 2, true, false>(a, stream); }

@@ -266,6 +266,35 @@ def test_grouped_convolutions_bit_exact(rt):
         rt.Conv(_i8((6, 2, 3, 3)), None, rt.Act(6, **_acts(6)["sshift_lin_s"].kwargs()), capi.U8B, groups=4)
 
 
+def test_direct_kernel_for_a_handful_of_channels(rt):
+    """Layers with at most 16 input channels and 32 outputs can run one thread per output pixel (the library's own choice
+    for at most 4 input channels: LeNet's first convolution): against the oracle and against the matrix-core kernel on the
+    same cell, over kernel sizes, strides, paddings, a dilation, both
+    input types and the rescale modes."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    cases = (  # B, C, O, H, W, k, stride, pad, dil, input type, activation
+        (5, 1, 6, 32, 32, 5, 1, 0, 1, capi.U8B, "fixed_relu_u"), (5, 6, 16, 14, 14, 5, 1, 0, 1, capi.U8B, "fixed_relu_u"),
+        (2, 3, 32, 17, 15, 3, 2, 1, 1, capi.U8B, "sshift_lin_s"), (2, 16, 20, 9, 11, 7, 1, 3, 1, capi.I8, "float_relu_u"),
+        (3, 5, 8, 12, 12, 3, 1, 0, 2, capi.I8, "sshift_lin_s"), (2, 9, 5, 8, 8, 1, 1, 0, 1, capi.U8B, "fixed_relu_u"),
+        (1, 2, 17, 6, 40, 3, (1, 2), 1, 1, capi.U8B, "dshift_relu_u"))
+    for (B, Cc, O, H, W, k, stride, pad, dil, in_dtype, an) in cases:
+        stride = stride if isinstance(stride, tuple) else (stride, stride)
+        x = _u8((B, Cc, H, W)) if in_dtype == capi.U8B else _i8((B, Cc, H, W))
+        w = _i8((O, Cc, k, k))
+        bias = RNG.integers(-2000, 2001, size=O).astype(np.int32)
+        acts = _acts(O)
+        spec = acts[an if an in acts else "sshift_lin_s"]
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=stride, pad=(pad,) * 4, dil=(dil, dil))
+        got = {}
+        for choice in (0, capi.KERNEL_DIRECT, capi.KERNEL_NO_DIRECT):
+            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), in_dtype, stride=stride, pad=(pad,) * 4, dil=(dil, dil),
+                           kernel_choice=choice)
+            got[choice] = conv.forward(rt.DTensor.from_numpy(x, in_dtype)).to_numpy()
+        assert np.array_equal(got[capi.KERNEL_DIRECT], want.astype(np.int64)), (B, Cc, O, H, W, k, stride, pad, dil)
+        assert np.array_equal(got[capi.KERNEL_NO_DIRECT], got[capi.KERNEL_DIRECT]) and np.array_equal(got[0], got[capi.KERNEL_DIRECT])
+
+
 def test_concat_channels_and_convolution_of_several_inputs(rt):
     """n2d2hip_concat_channels against numpy (odd channel counts, inputs and output with borders, both byte types; the
     channels past the last one hold the stored form of 0), and a ConvCell with three inputs (src/Cell/ConvCell_Frame.cpp:
