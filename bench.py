@@ -394,9 +394,22 @@ def main():
     conv_ops = 2.0 * sum(net.layer_macs(net.launched[k]) for k in pipe)
     achieved = conv_ops / (conv_ms * 1e-3) / 1e12
     profile_applies = B == TRAFFIC_FROM_PROFILE["batch"] and len(pipe) == TRAFFIC_FROM_PROFILE["launches_per_forward"]
-    roofline = {"bound": "mfma", "kernel": "conv_pipe_kernel (%d launches of one forward: conv/fc cells with a multiple of 64 input "
+    # Which roof bounds these launches: the larger of (their operations at the matrix cores' peak) and (their algorithmic
+    # bytes at the memory's peak).  With the 3x3 layers on the patch kernel and the first block on the bottleneck kernel,
+    # what is left on conv_pipe_kernel is mostly 1x1 layers: memory is the larger bound.  The other view is kept beside it.
+    pipe_bytes = float(sum(net.layer_bytes(net.launched[k]) for k in pipe))
+    achieved_gbs = pipe_bytes / (conv_ms * 1e-3) / 1e9
+    hbm_bound = pipe_bytes / (PEAK_HBM_GBS * 1e9) >= conv_ops / (PEAK_INT8_TOPS * 1e12)
+    mfma_view = {"achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4)}
+    hbm_view = {"achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved_gbs / PEAK_HBM_GBS, 4)}
+    roofline = {"bound": "hbm" if hbm_bound else "mfma",
+                "kernel": "conv_pipe_kernel (%d launches of one forward: conv/fc cells with a multiple of 64 input "
                 "channels, residual sums folded in; not the cells of the fused bottleneck nor the 3x3 layers on the patch kernel)" % len(pipe),
-                "achieved": round(achieved, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": round(achieved / PEAK_INT8_TOPS, 4),
+                "bound_is": "the larger of ops / int8 peak and algorithmic bytes / HBM peak over these launches",
+                "floor_us_per_launch": {"mfma": round(conv_ops / (PEAK_INT8_TOPS * 1e12) * 1e6 / len(pipe), 2),
+                                        "hbm": round(pipe_bytes / (PEAK_HBM_GBS * 1e9) * 1e6 / len(pipe), 2)},
+                **(hbm_view if hbm_bound else mfma_view),
+                "mfma_view": mfma_view, "hbm_view": hbm_view,
                 # HBM bytes per launch cannot be counted from inside this process: the figure is the one the committed profile
                 # holds, given only while this run launches what that profile covered (same batch, same number of launches)
                 "traffic": TRAFFIC_FROM_PROFILE["bytes_per_launch"] if profile_applies else None,
