@@ -661,6 +661,89 @@ template class PoolCell_FrameTrain_HIP<float>;
 template <> Registrar<PoolCell> PoolCell_FrameTrain_HIP<float>::mRegistrar("Frame_HIP_QAT", PoolCell_FrameTrain_HIP<float>::create,
                                                                            Registrar<PoolCell>::Type<float>());
 
+// -------------------------------------------------- ElemWiseCell_FrameTrain_HIP
+ElemWiseCell_FrameTrain_HIP::ElemWiseCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, const std::string& name, unsigned int nbOutputs,
+                                                         Operation operation, CoeffMode mode, const std::vector<Float_T>& weights,
+                                                         const std::vector<Float_T>& shifts, const std::shared_ptr<Activation>& activation)
+    : Cell(name, nbOutputs), ElemWiseCell(operation, mode, weights, shifts)
+{
+    if (operation != Sum)
+        throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + name + ": only Operation=Sum is supported by the float Frame_HIP cells");
+    if (mode == PerChannel)
+        throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + name + ": one coefficient per channel is not supported by the float Frame_HIP cells");
+    mActivation = activation;
+}
+
+void ElemWiseCell_FrameTrain_HIP::addInput(Cell_FrameTrain_HIP* parent)
+{
+    if (!parent)
+        throw std::runtime_error("Cell " + mName + ": null parent");
+    addInput(parent->getOutputs(), parent->getDiffInputs());
+    mParents.back() = parent;
+}
+
+void ElemWiseCell_FrameTrain_HIP::addInput(DeviceFloats& inputs, DeviceFloats& diffOutputs)
+{
+    if (mIns.empty()) {
+        Cell_FrameTrain_HIP::addInput(inputs, diffOutputs);
+    } else {
+        if (inputs.dims() != mIns[0]->dims())
+            throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + mName + ": inputs of different sizes");
+        if (!diffOutputs.empty() && diffOutputs.dims() != inputs.dims())
+            throw std::runtime_error("Cell " + mName + ": inputs and diffOutputs of different sizes");
+        mParents.push_back(nullptr);
+    }
+    mIns.push_back(&inputs);
+    mDiffOuts.push_back(&diffOutputs);
+}
+
+void ElemWiseCell_FrameTrain_HIP::initialize()
+{
+    if (mIns.empty() || mIns.size() > N2D2HIP_ELEMWISE_F32_MAX_INPUTS)
+        throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + mName + ": 1 to 8 inputs expected");
+    if (mNbChannels != mNbOutputs)
+        throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + mName + ": the number of outputs must be the number of input channels");
+    // src/Cell/ElemWiseCell_Frame.cpp:75-87: weights 1 and shifts 0 where none are given, one entry per input (one for all
+    // inputs is repeated)
+    const size_t n = mIns.size();
+    if (mWeights.empty()) mWeights.assign(n, 1.0f);
+    if (mShifts.empty()) mShifts.assign(n, 0.0f);
+    if (mWeights.size() == 1) mWeights.assign(n, mWeights[0]);
+    if (mShifts.size() == 1) mShifts.assign(n, mShifts[0]);
+    if (mWeights.size() != n || mShifts.size() != n)
+        throw std::runtime_error("ElemWiseCell_FrameTrain_HIP " + mName + ": one weight and one shift per input expected");
+    allocateOutputs();
+}
+
+void ElemWiseCell_FrameTrain_HIP::propagate(bool inference)
+{
+    std::vector<const float*> ins;
+    for (const DeviceFloats* t : mIns)
+        ins.push_back(t->data());
+    checkStatus(n2d2hip_elemwise_sum_f32_forward((int)ins.size(), ins.data(), mOutputs.size(), mWeights.data(), mShifts.data(), mOutputs.data(),
+                                                 mStream));
+    activationPropagate(inference);
+    mDiffInputs.clearValid();
+}
+
+void ElemWiseCell_FrameTrain_HIP::backPropagate()
+{
+    if (!mDiffInputs.isValid())
+        return;
+    activationBackPropagate();
+    for (size_t k = 0; k < mIns.size(); ++k) {
+        DeviceFloats* d = mDiffOuts[k];
+        if (!d || d->empty())
+            continue;
+        checkStatus(n2d2hip_elemwise_sum_f32_backward(mDiffInputs.size(), mWeights[k], mDiffInputs.data(), d->isValid() ? 1.0f : 0.0f, d->data(),
+                                                      mStream));
+        d->setValid();
+    }
+}
+
+Registrar<ElemWiseCell> ElemWiseCell_FrameTrain_HIP::mRegistrar("Frame_HIP_QAT", ElemWiseCell_FrameTrain_HIP::create,
+                                                                Registrar<ElemWiseCell>::Type<float>());
+
 // --------------------------------------------------- SoftmaxCell_FrameTrain_HIP
 const char* SoftmaxCell::Type = "Softmax";
 

@@ -301,6 +301,36 @@ private:
     static Registrar<PoolCell> mRegistrar;
 };
 
+// src/Cell/ElemWiseCell_Frame.cpp:104-136 and :194-233, Operation Sum with one coefficient per input (or one for all):
+// outputs = (w0 x0 + s0) + (w1 x1 + s1) + ..., the gradient towards input k = wk times the gradient of the outputs, added
+// to what another consumer of that input has already written.  The cell of a residual sum in a learning graph.
+class ElemWiseCell_FrameTrain_HIP : public ElemWiseCell, public Cell_FrameTrain_HIP {
+public:
+    ElemWiseCell_FrameTrain_HIP(const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs, Operation operation, CoeffMode mode,
+                                const std::vector<Float_T>& weights, const std::vector<Float_T>& shifts,
+                                const std::shared_ptr<Activation>& activation);
+    static std::shared_ptr<ElemWiseCell> create(Network& /*net*/, const DeepNet& deepNet, const std::string& name, unsigned int nbOutputs,
+                                                Operation operation, CoeffMode mode, const std::vector<Float_T>& weights,
+                                                const std::vector<Float_T>& shifts, const std::shared_ptr<Activation>& activation)
+    {
+        return std::make_shared<ElemWiseCell_FrameTrain_HIP>(deepNet, name, nbOutputs, operation, mode, weights, shifts, activation);
+    }
+    // every input has the size of the first one
+    void addInput(Cell_FrameTrain_HIP* parent);
+    void addInput(DeviceFloats& inputs, DeviceFloats& diffOutputs);
+    void initialize();
+    void propagate(bool inference = false);
+    void backPropagate();
+    void update() { activationUpdate(); }
+
+protected:
+    void setOutputsDims() { mOutW = mInW; mOutH = mInH; }
+
+private:
+    std::vector<DeviceFloats*> mIns, mDiffOuts;
+    static Registrar<ElemWiseCell> mRegistrar;
+};
+
 // include/Cell/SoftmaxCell.hpp:37-70: WithLoss (false), GroupSize (0)
 class SoftmaxCell : public virtual Cell {
 public:

@@ -32,7 +32,15 @@ struct TrainNet {
     std::map<std::string, std::shared_ptr<SATQuantizerActivation_Frame_HIP<float> > > satAct;
     std::map<std::string, std::shared_ptr<LSQQuantizerActivation_Frame_HIP<float> > > lsqAct;
     std::map<std::string, std::shared_ptr<LSQQuantizerCell_Frame_HIP<float> > > lsqCell;
-    Cell_FrameTrain_HIP* last() { return cells.empty() ? nullptr : cells.back().get(); }
+    std::vector<std::string> nextInputs;      // the cells the next added cell reads (empty: the cell added last)
+    Cell_FrameTrain_HIP* byName(const std::string& name)
+    {
+        for (auto& c : cells)
+            if (c->getName() == name) return c.get();
+        throw std::runtime_error("No cell named \"" + name + "\"");
+    }
+    // the cell the next added cell reads first (null: the environment)
+    Cell_FrameTrain_HIP* last() { return !nextInputs.empty() ? byName(nextInputs[0]) : (cells.empty() ? nullptr : cells.back().get()); }
 };
 
 // act: -1 none, 0 Linear, 1 Rectifier; actQuant: 0 none, 1 SAT (param = alpha), 2 LSQ (param = step size, <= 0: optimal init)
@@ -65,9 +73,15 @@ std::shared_ptr<Activation> makeActivation(TrainNet& n, const std::string& name,
     return a;
 }
 
+// Cells are added in an order in which every cell follows the cells it reads (propagate runs them in that order,
+// backPropagate and update in the reverse one, as DeepNet::learn does over its layers).
 void connect(TrainNet& n, const std::shared_ptr<Cell_FrameTrain_HIP>& cell)
 {
-    if (n.cells.empty())
+    if (!n.nextInputs.empty()) {
+        for (const std::string& name : n.nextInputs)
+            cell->addInput(n.byName(name));
+        n.nextInputs.clear();
+    } else if (n.cells.empty())
         cell->addInput(n.input, n.inputDiff);
     else
         cell->addInput(n.cells.back().get());
@@ -96,6 +110,7 @@ int fh_train_registrar_exists(const char* type, const char* key)
     if (t == "Softmax") return Registrar<SoftmaxCell>::exists<float>(k);
     if (t == "BatchNorm") return Registrar<BatchNormCell>::exists<float>(k);
     if (t == "Pool") return Registrar<PoolCell>::exists<float>(k);
+    if (t == "ElemWise") return Registrar<ElemWiseCell>::exists<float>(k);
     return -1;
 }
 
@@ -255,6 +270,40 @@ int fh_train_add_pool(void* net, const char* name, int poolW, int poolH, int str
         auto pool = f(n.net, n.deepNet, name, {(unsigned)poolW, (unsigned)poolH}, nbOutputs, {(unsigned)strideX, (unsigned)strideY},
                       {(unsigned)padX, (unsigned)padY}, pooling ? PoolCell::Average : PoolCell::Max, std::shared_ptr<Activation>());
         connect(n, std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(pool));
+    });
+}
+
+// The cells (comma-separated names) that the cell added next reads, instead of the cell added last.
+int fh_train_set_next_inputs(void* net, const char* names)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        n.nextInputs.clear();
+        std::string all(names ? names : ""), item;
+        for (size_t i = 0; i <= all.size(); ++i) {
+            if (i == all.size() || all[i] == ',') {
+                if (!item.empty()) { n.byName(item); n.nextInputs.push_back(item); }
+                item.clear();
+            } else
+                item += all[i];
+        }
+    });
+}
+
+// ElemWise Sum over the inputs set with fh_train_set_next_inputs; weights / shifts: nbCoeffs values each (0: all 1 / all 0)
+int fh_train_add_elemwise(void* net, const char* name, const float* weights, const float* shifts, int nbCoeffs, int act, int actQuant, int actRange,
+                          float actParam)
+{
+    return guardedT([&] {
+        TrainNet& n = *(TrainNet*)net;
+        auto f = Registrar<ElemWiseCell>::create<float>(n.model);
+        if (!f) throw std::runtime_error("Cell model \"" + n.model + "\" is not valid in section [" + name + "]");
+        if (n.nextInputs.empty()) throw std::runtime_error("fh_train_add_elemwise(): name the inputs first");
+        const std::vector<Float_T> w(weights, weights + (weights ? nbCoeffs : 0)), s(shifts, shifts + (shifts ? nbCoeffs : 0));
+        auto cell = std::dynamic_pointer_cast<Cell_FrameTrain_HIP>(f(n.net, n.deepNet, name, n.last()->getNbOutputs(), ElemWiseCell::Sum,
+                                                                     ElemWiseCell::PerInput, w, s,
+                                                                     makeActivation(n, name, act, actQuant, actRange, actParam)));
+        connect(n, cell);
     });
 }
 

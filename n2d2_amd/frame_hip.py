@@ -378,6 +378,8 @@ lib.fh_train_net_destroy.restype = None
 lib.fh_train_add_activation_cell.argtypes = [_P, C.c_char_p, _I, _I, _I, _F]
 lib.fh_train_add_conv.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _I, _I, _F, _I, _I, _I, _I, _I]
 lib.fh_train_add_softmax.argtypes = [_P, C.c_char_p, _I]
+lib.fh_train_set_next_inputs.argtypes = [_P, C.c_char_p]
+lib.fh_train_add_elemwise.argtypes = [_P, C.c_char_p, _P, _P, _I, _I, _I, _I, C.c_float]
 lib.fh_train_add_batchnorm.argtypes = [_P, C.c_char_p, _P, C.c_double, C.c_double, _I, _I, _I, _F]
 lib.fh_train_get_batchnorm.argtypes = [_P, C.c_char_p, _I, _P, _SZ]
 lib.fh_train_add_pool.argtypes = [_P, C.c_char_p, _I, _I, _I, _I, _I, _I, _I]
@@ -489,6 +491,26 @@ class TrainNet:
 
     def add_softmax(self, name, with_loss=True):
         _check_train(lib.fh_train_add_softmax(self._h, name.encode(), int(with_loss)))
+        self._shapes[name] = self._last
+
+    def read_from(self, *cells):
+        """The cell added next reads these cells (in this order) instead of the cell added last: branches of a learning graph.
+        Cells are added in an order in which every cell follows the cells it reads."""
+        _check_train(lib.fh_train_set_next_inputs(self._h, ",".join(cells).encode()))
+        self._last = self._shapes[cells[0]]
+
+    def add_elemwise(self, name, inputs, weights=None, shifts=None, act=None, act_quant=None, act_range=255, act_param=1.0):
+        """ElemWise Sum of the named cells' outputs, (w0 x0 + s0) + (w1 x1 + s1) + ... (weights 1 and shifts 0 by default)."""
+        self.read_from(*inputs)
+        w = None if weights is None else np.ascontiguousarray(weights, dtype=np.float32)
+        sh = None if shifts is None else np.ascontiguousarray(shifts, dtype=np.float32)
+        n = 0 if w is None and sh is None else len(inputs)
+        if w is None and sh is not None:
+            w = np.ones(n, dtype=np.float32)
+        if sh is None and w is not None:
+            sh = np.zeros(n, dtype=np.float32)
+        _check_train(lib.fh_train_add_elemwise(self._h, name.encode(), None if w is None else w.ctypes.data, None if sh is None else sh.ctypes.data,
+                                               n, _ACT[act], _QUANT[act_quant], int(act_range), float(act_param)))
         self._shapes[name] = self._last
 
     def fuse_into(self, net, mode="FloatMult", w_round=True, b_round=True, c_round=True):

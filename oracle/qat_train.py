@@ -367,6 +367,33 @@ class PoolCell:
             self.activation.update(batch_size)
 
 
+class ElemWiseCell:
+    """src/Cell/ElemWiseCell_Frame.cpp:104-136 and :194-233, Operation Sum, one coefficient per input: outputs =
+    (w0 x0 + s0) + (w1 x1 + s1) + ..., then the activation in place; backPropagate gives input k the gradient wk * diff
+    (added to what another consumer of that input has written, which train_graph does)."""
+
+    def __init__(self, nb_inputs, weights=None, shifts=None, activation=None):
+        self.w = np.ones(nb_inputs, dtype=F) if weights is None else np.array(weights, dtype=F)
+        self.s = np.zeros(nb_inputs, dtype=F) if shifts is None else np.array(shifts, dtype=F)
+        self.activation = activation
+        self.diff_inputs = None
+
+    def propagate(self, xs, inference=False):
+        y = o.elemwise_sum([np.ascontiguousarray(x, dtype=F) for x in xs], self.w, self.s, "PerInput")
+        self.outputs = self.activation.propagate(y, inference) if self.activation else y
+        return self.outputs
+
+    def back_propagate(self):
+        d = self.diff_inputs
+        if self.activation:
+            d = self.activation.back_propagate(d)
+        return [o.elemwise_sum_backward(d, self.w, k, "PerInput") for k in range(len(self.w))]
+
+    def update(self, batch_size):
+        if self.activation:
+            self.activation.update(batch_size)
+
+
 class SoftmaxCell:
     """src/Cell/SoftmaxCell_Frame.cpp:93-137 and :140-207 with WithLoss: the gradient passes through unchanged;
     applyLoss is Cell_Frame_Top::applyLoss (src/Cell/Cell_Frame_Top.cpp:27-40): diff = target - output, formed in
@@ -403,4 +430,33 @@ def train_sequential(x, cells, softmax, targets, iterations):
             d = c.back_propagate()
         for c in reversed(cells):
             c.update(batch)
+    return loss
+
+
+def train_graph(x, nodes, softmax, targets, iterations):
+    """The same loop over a graph with branches: `nodes` is a list of (cell, inputs) in an order in which every cell follows
+    the cells it reads, inputs being indices into that list (-1: the net's input x); the last node feeds the softmax.  A
+    tensor read by several cells receives the sum of their gradients, the cell that runs its backPropagate first writing
+    and the others adding (Cell_Frame's diffOutputs with beta = isValid, e.g. src/Cell/ConvCell_Frame.cpp:545-560)."""
+    batch = x.shape[0]
+    loss = 0.0
+    for _ in range(iterations):
+        outs = []
+        for cell, inputs in nodes:
+            xs = [x if i < 0 else outs[i] for i in inputs]
+            outs.append(cell.propagate(xs, inference=False) if isinstance(cell, ElemWiseCell) else cell.propagate(xs[0], inference=False))
+        softmax.propagate(outs[-1])
+        loss = softmax.apply_loss(targets)
+        grads = [None] * len(nodes)
+        grads[-1] = softmax.back_propagate()
+        for k in range(len(nodes) - 1, -1, -1):
+            cell, inputs = nodes[k]
+            cell.diff_inputs = grads[k]
+            d = cell.back_propagate()
+            ds = d if isinstance(cell, ElemWiseCell) else [d]
+            for i, di in zip(inputs, ds):
+                if i >= 0:
+                    grads[i] = di if grads[i] is None else (di + grads[i]).astype(F)
+        for cell, _ in reversed(nodes):
+            cell.update(batch)
     return loss

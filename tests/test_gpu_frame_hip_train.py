@@ -531,3 +531,70 @@ def test_average_pool_cell_learns_as_the_oracle_does():
         want = q.train_sequential(x, cells_, sm, t, 1)
         assert abs(loss - want) <= 1e-3 * want, it
     assert _close(net.weights("c1"), cells_[0].w, 1e-3)
+
+
+def test_residual_sum_cell_learns_as_the_oracle_does():
+    """A learning graph with a branch: Conv (SAT weights, SAT activation) -> [Conv -> BatchNorm -> Conv] + shortcut -> ElemWise
+    Sum (weights 1 and 0.5, Rectifier) -> max Pool -> Conv -> Softmax.  The tensor read by the branch and by the sum receives
+    both gradients.  First iteration tensor by tensor against the oracle's train_graph, then ten more on the loss and the
+    learned weights."""
+    from n2d2_amd import frame_hip as fh
+    from oracle import qat_train as q
+    assert fh.lib.fh_train_registrar_exists(b"ElemWise", b"Frame_HIP_QAT") == 1
+    rng = np.random.default_rng(71)
+    x = rng.uniform(0, 1, size=(4, 2, 10, 10)).astype(np.float32)
+    w0 = rng.normal(0, 0.3, size=(4, 2, 3, 3)).astype(np.float32)
+    w1 = rng.normal(0, 0.3, size=(4, 4, 3, 3)).astype(np.float32)
+    w2 = rng.normal(0, 0.3, size=(4, 4, 1, 1)).astype(np.float32)
+    w3 = rng.normal(0, 0.3, size=(3, 4, 4, 4)).astype(np.float32)
+    t = np.zeros((4, 3, 1, 1), dtype=np.float32)
+    t[np.arange(4), [0, 1, 2, 1]] = 1
+    net = fh.TrainNet(x, propagate_gradient=False)
+    net.add_conv("stem", w0, act="Linear", act_quant="SAT", act_range=15, act_param=3.0, weight_quant="SAT", weight_range=15)
+    net.add_conv("b1", w1, pad=(1, 1), weight_quant="SAT", weight_range=15)
+    net.add_batchnorm("bn", act="Linear", act_quant="SAT", act_range=15, act_param=4.0)
+    net.add_conv("b2", w2, weight_quant="SAT", weight_range=15)
+    net.add_elemwise("sum", ["b2", "stem"], weights=[1.0, 0.5], act="Rectifier")
+    net.add_pool("pool", (2, 2), (2, 2))
+    net.add_conv("head", w3, weight_quant="SAT", weight_range=15)
+    net.add_softmax("softmax", with_loss=True)
+    assert net._shapes["sum"] == (4, 4, 8, 8) and net._last == (4, 3, 1, 1)
+    qa0, qa1 = q.SATQuantizerActivation(15, 3.0), q.SATQuantizerActivation(15, 4.0)
+    stem = q.ConvCell(w0, activation=q.LinearActivation(qa0), quantizer=q.SATQuantizerCell(15))
+    b1 = q.ConvCell(w1, pad=(1, 1, 1, 1), quantizer=q.SATQuantizerCell(15))
+    bn = q.BatchNormCell(4, activation=q.LinearActivation(qa1))
+    b2 = q.ConvCell(w2, quantizer=q.SATQuantizerCell(15))
+
+    class Rect(q.LinearActivation):         # RectifierActivation_Frame, no quantizer: max(x, 0) and its mask
+        def propagate(self, v, inference):
+            self.out = np.maximum(v, 0).astype(np.float32)
+            return self.out
+
+        def back_propagate(self, d):
+            return (d * (self.out > 0)).astype(np.float32)
+    ew = q.ElemWiseCell(2, weights=[1.0, 0.5], activation=Rect())
+    pool = q.PoolCell((2, 2), (2, 2))
+    head = q.ConvCell(w3, quantizer=q.SATQuantizerCell(15))
+    nodes = [(stem, [-1]), (b1, [0]), (bn, [1]), (b2, [2]), (ew, [3, 0]), (pool, [4]), (head, [5])]
+    sm = q.SoftmaxCell()
+    print("residual net: first iteration", flush=True)
+    loss = net.learn(t, 1)
+    want = q.train_graph(x, nodes, sm, t, 1)
+    assert abs(loss - want) <= 1e-5 * want
+    for name, cell in (("stem", stem), ("b1", b1), ("b2", b2), ("sum", ew), ("pool", pool), ("head", head)):
+        assert _close(net.outputs(name), cell.outputs, 2e-5), name
+    # the gradient that reaches the stem's outputs: the branch's part plus the shortcut's
+    assert _close(net.diff_inputs("b2"), b2.diff_inputs, 1e-4)
+    assert _close(net.weights("stem"), stem.w, 1e-4) and _close(net.weights("b1"), b1.w, 1e-4) and _close(net.weights("head"), head.w, 1e-4)
+    print("residual net: ten more", flush=True)
+    for it in range(10):
+        loss = net.learn(t, 1)
+        want = q.train_graph(x, nodes, sm, t, 1)
+        assert abs(loss - want) <= 1e-3 * want, it
+    assert _close(net.weights("stem"), stem.w, 1e-3) and _close(net.weights("b2"), b2.w, 1e-3)
+    assert abs(net.activation_quantizer("stem")[0] - float(qa0.alphas[0])) <= 1e-3
+    # an ElemWise cell other than a sum, or with one coefficient per channel, is refused by name
+    bad = fh.TrainNet(x, propagate_gradient=False)
+    bad.add_conv("a", w0)
+    with pytest.raises(fh.FrameHipError, match="name the inputs first"):
+        fh._check_train(fh.lib.fh_train_add_elemwise(bad._h, b"s", None, None, 0, -1, 0, 255, 1.0))

@@ -354,3 +354,35 @@ def test_elemwise_sum_gradient_is_the_weight_per_input_or_per_channel():
     wc = np.array([2.0, -1.0, 0.5], dtype=np.float32)
     dxc = o.elemwise_sum_backward(dy, wc, 1, "PerChannel")
     assert np.array_equal(dxc, wc[None, :, None, None] * dy)
+
+
+def test_a_graph_with_a_residual_sum_backpropagates_as_autograd_does():
+    """train_graph over conv -> (conv, identity) -> weighted sum -> conv -> softmax with loss: a tensor read by two cells
+    receives the sum of their gradients.  Against torch's autograd in float64 on the same graph (the gradient the softmax
+    hands back, target - output, is minus that of the summed cross-entropy)."""
+    import torch
+    from oracle import qat_train as qt
+    rng = np.random.default_rng(61)
+    x = rng.uniform(0, 1, size=(3, 2, 6, 6)).astype(np.float32)
+    w1 = rng.normal(0, 0.4, size=(4, 2, 3, 3)).astype(np.float32)
+    w2 = rng.normal(0, 0.4, size=(4, 4, 3, 3)).astype(np.float32)
+    w3 = rng.normal(0, 0.4, size=(3, 4, 4, 4)).astype(np.float32)
+    t = np.zeros((3, 3, 1, 1), dtype=np.float32)
+    t[np.arange(3), [2, 0, 1]] = 1
+    zero_lr = lambda: qt.SGDSolver(learning_rate=0.0)
+    c1, c2, c3 = (qt.ConvCell(w1, solver=zero_lr()), qt.ConvCell(w2, pad=(1, 1, 1, 1), solver=zero_lr()), qt.ConvCell(w3, solver=zero_lr()))
+    ew = qt.ElemWiseCell(2, weights=[1.0, 0.5], shifts=[0.0, 0.25])
+    nodes = [(c1, [-1]), (c2, [0]), (ew, [1, 0]), (c3, [2])]
+    qt.train_graph(x, nodes, qt.SoftmaxCell(), t, 1)
+    tx = torch.tensor(x, dtype=torch.float64)
+    tw = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in (w1, w2, w3)]
+    a = torch.nn.functional.conv2d(tx, tw[0])
+    b = torch.nn.functional.conv2d(a, tw[1], padding=1)
+    s = (1.0 * b + 0.0) + (0.5 * a + 0.25)
+    z = torch.nn.functional.conv2d(s, tw[2]).reshape(3, 3)
+    ce = -(torch.tensor(t.reshape(3, 3), dtype=torch.float64) * torch.log_softmax(z, 1)).sum()
+    ce.backward()
+    for cell, g in zip((c1, c2, c3), tw):
+        want = -g.grad.numpy()
+        assert np.abs(cell.diff_w - want).max() <= 1e-4 * np.abs(want).max()
+    assert np.abs(ew.outputs - s.detach().numpy()).max() <= 1e-5
