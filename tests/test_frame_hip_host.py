@@ -83,14 +83,15 @@ def test_every_class_of_the_path_is_registered_under_frame_hip(fh):
 
 
 def test_the_float_learning_cells_are_registered_under_their_own_key(fh):
-    for t in ("Conv", "Fc", "Activation", "Softmax", "BatchNorm", "Pool"):
+    for t in ("Conv", "Fc", "Activation", "Softmax", "BatchNorm", "Pool", "ElemWise"):
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_HIP_QAT") == 1, t
         assert fh.lib.fh_train_registrar_exists(t.encode(), b"Frame_CUDA") == 0, t
     # the integer inference cells own ("Frame_HIP", float); the two keys do not collide
     assert fh.lib.fh_train_registrar_exists(b"Conv", b"Frame_HIP") == 1
     assert fh.lib.fh_train_registrar_exists(b"Activation", b"Frame_HIP") == 0
     assert fh.lib.fh_train_registrar_exists(b"BatchNorm", b"Frame_HIP") == 0       # the integer graph has none: it is fused away
-    assert fh.lib.fh_train_registrar_exists(b"ElemWise", b"Frame_HIP_QAT") == -1  # not a type of that family
+    assert fh.lib.fh_train_registrar_exists(b"ElemWise", b"Frame_HIP") == 1        # the integer sum cell
+    assert fh.lib.fh_train_registrar_exists(b"Scaling", b"Frame_HIP_QAT") == -1    # not a type this query knows
 
 
 def test_registrar_semantics(fh):
