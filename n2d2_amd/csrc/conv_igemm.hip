@@ -265,7 +265,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             }
         }
     }
-    if (out_bytes) {
+    if (out_bytes && p.out_cs == 4) {
+        // at most 4 outputs: a pixel is one dword
+        __syncthreads();
+        for (int row = tid; row < BM; row += 256)
+            if (n0 == 0 && m0 + row < p.M)
+                *(unsigned*)((signed char*)p.out + (long long)(m0 + row) * 4) = *(const unsigned*)(smem + row * STAGE_STRIDE);
+    } else if (out_bytes) {
         __syncthreads();
         constexpr int CHUNKS = BN / 16;
         for (int id = tid; id < BM * CHUNKS; id += 256) {
@@ -764,6 +770,8 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
     const int opad_n = round_up(d.O, 64);
     *bn128 = opad_n % 128 == 0 || opad_n > 256;
     const int k = c->act->args.kind;
+    if (d.O <= 4)               // a pixel of the output is one dword: the general kernel stores those
+        return false;
     if (d.weight_bits == 4)     // packed weights: integer rescale only
         return c->d_w4img != nullptr && d.kW * d.kH <= 31 && k == EPI_I24 && c->bias_folded;
     return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 31
@@ -793,7 +801,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         return rc;
     N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
                     "conv_forward: output is %dx%dx%dx%d, expected %dx%dx%dx%d", out->B, out->C, out->H, out->W, in->B, d.O, OH, OW);
-    N2D2HIP_REQUIRE(out->cs % 16 == 0, N2D2HIP_ERR_INVALID, "conv_forward: output channel stride %d must be a multiple of 16", out->cs);
+    N2D2HIP_REQUIRE(out->cs % 16 == 0 || (out->cs == 4 && !c->depthwise), N2D2HIP_ERR_INVALID,
+                    "conv_forward: output channel stride %d must be a multiple of 16 (or 4 for at most 4 outputs, not depthwise)", out->cs);
     // with a folded sum the stored values are the sum cell's
     const n2d2hip_act_s* act = other ? c->sum->act : c->act;
     if (other) {
@@ -1013,7 +1022,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     }
     {
         const int k = c->act->args.kind;
-        if (c->d_wstem && !other && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32) && fits32
+        if (c->d_wstem && out->cs % 16 == 0 && !other && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32) && fits32
             && !(d.kernel_choice & N2D2HIP_KERNEL_NO_STEM)) {
             ConvStemArgs q;
             q.c = a;

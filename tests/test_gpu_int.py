@@ -442,6 +442,41 @@ def test_fc_cell_bit_exact(rt, shape):
         assert np.array_equal(got, want.astype(np.int64)), an
 
 
+def test_cells_with_at_most_four_outputs(rt):
+    """Convolutions and FCs with 1 to 4 outputs (a binary classifier's last layer, a segmentation head): their output pixel
+    is one dword.  From 3, 20 and 64 input channels, byte and raw int32 outputs, and a convolution that reads such a
+    tensor."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    for O in (1, 2, 3, 4):
+        for (Cc, k, pad, choice) in ((3, 3, 1, 0), (3, 3, 1, capi.KERNEL_NO_DIRECT), (20, 3, 1, 0), (64, 1, 0, 0), (128, 3, 1, 0)):
+            x = _u8((3, Cc, 9, 7))
+            w = _i8((O, Cc, k, k))
+            bias = RNG.integers(-2000, 2001, size=O).astype(np.int32)
+            for an in ("sshift_relu_u", "none_linear", "fixed_clip_s"):
+                spec = _acts(O)[an]
+                want = cells_ref.conv_cell(x, w, bias, spec, pad=(pad,) * 4)
+                conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, pad=(pad,) * 4, kernel_choice=choice)
+                got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B))
+                assert got.cs == 4 and np.array_equal(got.to_numpy(), want.astype(np.int64)), (O, Cc, k, an)
+        x = _u8((5, 84, 1, 1))
+        w = _i8((O, 84))
+        bias = RNG.integers(-4096, 4097, size=O).astype(np.int32)
+        for an in ("none_linear", "fixed_relu_u"):
+            spec = _acts(O)[an]
+            fc = rt.Fc(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, (84, 1, 1))
+            assert np.array_equal(fc.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), cells_ref.fc_cell(x, w, bias, spec).astype(np.int64)), (O, an)
+    # two layers: 16 -> 2 -> 8 channels
+    x = _u8((2, 16, 8, 8))
+    w1, w2 = _i8((2, 16, 3, 3)), _i8((8, 2, 3, 3))
+    s1, s2 = _acts(2)["sshift_relu_u"], _acts(8)["sshift_lin_s"]
+    mid = cells_ref.conv_cell(x, w1, None, s1, pad=(1,) * 4)
+    want = cells_ref.conv_cell(mid, w2, None, s2, pad=(1,) * 4)
+    c1 = rt.Conv(w1, None, rt.Act(2, **s1.kwargs()), capi.U8B, pad=(1,) * 4)
+    c2 = rt.Conv(w2, None, rt.Act(8, **s2.kwargs()), capi.U8B, pad=(1,) * 4)
+    assert np.array_equal(c2.forward(c1.forward(rt.DTensor.from_numpy(x, capi.U8B))).to_numpy(), want.astype(np.int64))
+
+
 # ------------------------------------------------------------------ pool
 
 @pytest.mark.parametrize("kind,pool,stride,pad", [("max", (2, 2), (2, 2), (0, 0)), ("max", (3, 3), (2, 2), (0, 0)),
