@@ -37,7 +37,8 @@ void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo, bool sti
     d.dtype = dtype;
     d.layout = N2D2HIP_NHWC;
     d.B = B; d.C = C; d.H = H; d.W = W;
-    d.cs = stimuli ? n2d2hip_nhwc_cs(C) : (C + 15) / 16 * 16;
+    (void)stimuli;
+    d.cs = n2d2hip_nhwc_cs(C);      // 4 for at most 4 channels (stimuli and cells alike), a multiple of 16 otherwise
     const size_t bytes = n2d2hip_tensor_bytes(&d);
     if (mDesc.data && bytes == mBytes) {
         d.data = mDesc.data;

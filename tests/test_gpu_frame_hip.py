@@ -207,6 +207,30 @@ def test_grouped_convolution_cells(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+def test_cells_with_two_outputs_through_the_registrar(fh):
+    """A binary classifier: a convolution with 3 outputs, a rescaled FC with 2 and a last FC with 2 raw logits (output
+    tensors whose pixel is one dword), through the Registrar cells and through GpuNet."""
+    from n2d2_amd import nets
+    b = nets._Builder("binary", (3, 16, 16), 47, "SingleShift")
+    t = b.conv("c1", "input", 16, 3, stride=2, pad=1)
+    t = b.conv("c2", t, 3, 3, pad=1)
+    t = b.pool("pool", t, "max", 2, 2)
+    t = b.fc("fc1", t, 2, kind="Rectifier")
+    b.fc("fc2", t, 2, mode="None")
+    spec = b.spec
+    x = np.random.default_rng(47).integers(0, 256, size=(5, 3, 16, 16))
+    keep = [l.name for l in spec.layers]
+    _compare(fh, spec, x, keep)
+    from oracle import cells
+    g = nets.GpuNet(spec, 5)
+    g.set_input(x)
+    g.forward()
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        if name not in g.folded:
+            assert np.array_equal(g.tensors[name].to_numpy(), want[name].astype(np.int64)), name
+
+
 def test_convolution_cells_with_several_inputs(fh):
     """Cells whose Input lists several cells see those cells' channels one behind the other (src/Cell/ConvCell_Frame.cpp:
     438-459): two such ConvCells, one of them feeding a sum, an average and a max PoolCell over two cells each, and an
