@@ -4,6 +4,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <functional>
 #include <cstring>
 
 namespace N2D2 {
@@ -1796,17 +1797,36 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
         const std::string key = trim(line.substr(0, eq)), value = trim(line.substr(eq + 1));
         if (current.empty()) global[key] = value; else sections[current][key] = value;
     }
-    auto resolved = [&](const std::string& name) {
+    std::function<Section(const std::string&, int)> resolvedAt = [&](const std::string& name, int depth) {
         Section s;
         auto ih = inherits.find(name);
         if (ih != inherits.end()) {
-            auto base = sections.find(ih->second);
-            if (base == sections.end()) throw std::runtime_error("Section [" + name + "] inherits from unknown section " + ih->second);
-            s = base->second;
+            // "[conv_1] conv_def other_def": the templates' keys, later ones first overridden by the section's own
+            for (const std::string& baseName : split(ih->second, " \t")) {
+                auto base = sections.find(baseName);
+                if (base == sections.end()) throw std::runtime_error("Section [" + name + "] inherits from unknown section " + baseName);
+                for (const auto& kv : base->second) s[kv.first] = kv.second;
+            }
         }
         for (const auto& kv : sections[name]) s[kv.first] = kv.second;
+        // "NbOutputs=[conv_pw_2]NbOutputs": the value of another section's key
+        for (auto& kv : s) {
+            const std::string& v = kv.second;
+            const size_t close = v.find(']');
+            if (v.size() > 2 && v[0] == '[' && close != std::string::npos && close + 1 < v.size()) {
+                const std::string refSection = trim(v.substr(1, close - 1)), refKey = trim(v.substr(close + 1));
+                if (depth > 16 || !sections.count(refSection))
+                    throw std::runtime_error("Section [" + name + "]: " + kv.first + " refers to unknown section [" + refSection + "]");
+                const Section other = resolvedAt(refSection, depth + 1);
+                auto it = other.find(refKey);
+                if (it == other.end())
+                    throw std::runtime_error("Section [" + name + "]: [" + refSection + "] has no " + refKey);
+                kv.second = it->second;
+            }
+        }
         return s;
     };
+    auto resolved = [&](const std::string& name) { return resolvedAt(name, 0); };
 
     // src/Generator/DeepNetGenerator.cpp:124-125
     const std::string model = global.count("DefaultModel") ? global["DefaultModel"] : "Frame";
@@ -1884,6 +1904,10 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
             auto f = Registrar<ScalingCell>::create<float>(model);
             if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
             cell = f(*deepNet, name, getUInt(s, "NbOutputs", 0, true, name), Scaling());
+        } else if (type == "Softmax") {
+            // The quantized graph ends at the logits: the integer cells have no Softmax (N2D2's integer exports drop it as
+            // well); the section and its Target are read over.
+            continue;
         } else {
             throw std::runtime_error("Cell type " + type + " is not on the quantized path (section [" + name + "])");
         }

@@ -207,6 +207,122 @@ def test_grouped_convolution_cells(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+MINI_MOBILENET_INI = """
+DefaultModel=Frame_HIP
+
+[database]
+Type=MNIST_IDX_Database
+
+[sp]
+SizeX=28
+SizeY=28
+BatchSize=6
+
+[sp.Transformation-1]
+Type=RangeAffineTransformation
+FirstOperator=Divides
+FirstValue=255.0
+
+; templates, as N2D2's model files write them
+[conv_def]
+Type=Conv
+WeightsFiller=XavierFiller
+ActivationFunction=Rectifier
+
+[dw_def]
+Mapping.ChannelsPerGroup=1
+
+[fc_def]
+Type=Fc
+
+[stem] conv_def
+Input=sp
+KernelDims=3 3
+NbOutputs=8
+Padding=1
+Stride=2
+
+[dw_a] conv_def dw_def
+Input=stem
+KernelDims=3 3
+NbOutputs=[stem]NbOutputs
+Padding=1
+
+[pw_a] conv_def
+Input=dw_a
+KernelDims=1 1
+NbOutputs=12
+
+[pool_a]
+Input=pw_a
+Type=Pool
+PoolDims=3 3
+NbOutputs=[pw_a]NbOutputs
+Pooling=Max
+Stride=2
+
+[dw_b] conv_def dw_def
+Input=pool_a
+KernelDims=2 2
+NbOutputs=[pool_a]NbOutputs
+
+[pool_b]
+Input=dw_b
+Type=Pool
+PoolDims=2 2
+NbOutputs=[dw_b]NbOutputs
+Pooling=Average
+
+[fc_a] fc_def
+Input=pool_b
+ActivationFunction=Rectifier
+NbOutputs=16
+
+[fc_b] fc_def
+Input=fc_a
+ActivationFunction=Linear
+NbOutputs=10
+
+[softmax]
+Input=fc_b
+Type=Softmax
+NbOutputs=[fc_b]NbOutputs
+
+[softmax.Target]
+"""
+
+
+def test_model_file_syntax_of_the_reference(fh):
+    """An INI written the way N2D2's own model files are (tests/tests_data/mnist_model/model.ini: several templates behind a
+    section header, NbOutputs=[other]NbOutputs, scalar Padding / Stride, database / transformation / target sections, a
+    Softmax at the end, which the integer graph does not instantiate): the cells it describes against the oracle."""
+    from n2d2_amd import nets
+    b = nets._Builder("mini", (1, 28, 28), 53, "SingleShift")
+    t = b.conv("stem", "input", 8, 3, stride=2, pad=1)
+    t = b.conv("dw_a", t, 8, 3, pad=1, groups=8)
+    t = b.conv("pw_a", t, 12, 1)
+    t = b.pool("pool_a", t, "max", 3, 2)
+    t = b.conv("dw_b", t, 12, 2, groups=12)
+    t = b.pool("pool_b", t, "avg", 2, 1)
+    t = b.fc("fc_a", t, 16, kind="Rectifier")
+    b.fc("fc_b", t, 10, mode="None")
+    spec = b.spec
+    net = fh.Net(MINI_MOBILENET_INI)
+    assert net.nb_cells == len(spec.layers)           # no Softmax cell
+    fh.install_parameters(net, spec)
+    net.initialize()
+    x = np.random.default_rng(53).integers(0, 256, size=(6, 1, 28, 28))
+    net.set_stimuli(x)
+    net.propagate()
+    from oracle import cells
+    keep = [l.name for l in spec.layers]
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        assert np.array_equal(net.outputs(name), want[name]), name
+    with pytest.raises(fh.FrameHipError, match="refers to unknown section"):
+        fh.Net(MINI_MOBILENET_INI.replace("[stem]NbOutputs", "[nowhere]NbOutputs"))
+
+
 def test_cells_with_two_outputs_through_the_registrar(fh):
     """A binary classifier: a convolution with 3 outputs, a rescaled FC with 2 and a last FC with 2 raw logits (output
     tensors whose pixel is one dword), through the Registrar cells and through GpuNet."""
