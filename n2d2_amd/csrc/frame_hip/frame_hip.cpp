@@ -1898,8 +1898,21 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
             if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");
             const std::string op = s.count("Operation") ? s.at("Operation") : "Sum";
             if (op != "Sum") throw std::runtime_error("ElemWise operation " + op + " is not on the quantized path (section [" + name + "])");
-            cell = f(net, *deepNet, name, getUInt(s, "NbOutputs", 0, true, name), ElemWiseCell::Sum, ElemWiseCell::PerLayer, std::vector<Float_T>(),
-                     std::vector<Float_T>(), makeActivation(s, name));
+            // src/Generator/ElemWiseCellGenerator.cpp:50-62: Weights, Shifts (none by default), CoeffMode (PerInput by default)
+            auto floats = [&](const char* key) {
+                std::vector<Float_T> v;
+                if (s.count(key))
+                    for (const std::string& tok : split(s.at(key), " \t,"))
+                        v.push_back(std::stof(tok));
+                return v;
+            };
+            const std::string coeff = s.count("CoeffMode") ? s.at("CoeffMode") : "PerInput";
+            if (coeff != "PerLayer" && coeff != "PerInput" && coeff != "PerChannel")
+                throw std::runtime_error("Unknown CoeffMode " + coeff + " in section [" + name + "]");
+            const ElemWiseCell::CoeffMode mode = coeff == "PerLayer" ? ElemWiseCell::PerLayer
+                : (coeff == "PerInput" ? ElemWiseCell::PerInput : ElemWiseCell::PerChannel);
+            cell = f(net, *deepNet, name, getUInt(s, "NbOutputs", 0, true, name), ElemWiseCell::Sum, mode, floats("Weights"), floats("Shifts"),
+                     makeActivation(s, name));
         } else if (type == "Scaling") {
             auto f = Registrar<ScalingCell>::create<float>(model);
             if (!f) throw std::runtime_error("Cell model \"" + model + "\" is not valid in section [" + name + "]");

@@ -338,6 +338,9 @@ def spec_to_ini(spec, batch, model="Frame_HIP"):
                       "PaddingDims=%d %d" % l.pad, "Pooling=%s" % ("Max" if l.kind == "max" else "Average")]
         elif l.type == "elemwise":
             lines += ["Type=ElemWise", "NbOutputs=%d" % l.out_shape[0], "Operation=Sum", "ActivationFunction=%s" % l.act.kind]
+            if l.weights is not None:
+                lines += ["CoeffMode=%s" % l.coeff_mode, "Weights=" + " ".join("%g" % v for v in l.weights),
+                          "Shifts=" + " ".join("%g" % v for v in l.shifts)]
         elif l.type == "scaling":
             lines += ["Type=Scaling", "NbOutputs=%d" % l.out_shape[0]]
         lines.append("")

@@ -246,12 +246,17 @@ class _Builder:
         self.values[name] = act.apply_np(self.values[inp], 0)
         return self.spec.add(Layer(name, "scaling", [inp], act=act), self.spec.shapes[inp], unsigned)
 
-    def sum(self, name, inps, kind="Rectifier", nb_bits=None):
-        acc = sum(self.values[i] for i in inps)
+    def sum(self, name, inps, kind="Rectifier", nb_bits=None, weights=None, shifts=None):
+        """weights / shifts: one integer per input (ElemWise CoeffMode PerInput), 1 and 0 by default."""
+        w = [1] * len(inps) if weights is None else [int(v) for v in weights]
+        sh = [0] * len(inps) if shifts is None else [int(v) for v in shifts]
+        acc = sum(w[k] * self.values[i] + sh[k] for k, i in enumerate(inps))
         C = acc.shape[0]
         act = self._make_act(acc, kind, C, nb_bits, target=None)
         self.values[name] = act.apply_np(acc, 0)
-        l = Layer(name, "elemwise", list(inps), act=act, weights=None, shifts=None, coeff_mode="PerLayer")
+        plain = weights is None and shifts is None
+        l = Layer(name, "elemwise", list(inps), act=act, weights=None if plain else np.array(w, dtype=np.float32),
+                  shifts=None if plain else np.array(sh, dtype=np.float32), coeff_mode="PerLayer" if plain else "PerInput")
         return self.spec.add(l, acc.shape, act.unsigned_out)
 
 

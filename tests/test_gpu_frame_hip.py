@@ -323,6 +323,137 @@ def test_model_file_syntax_of_the_reference(fh):
         fh.Net(MINI_MOBILENET_INI.replace("[stem]NbOutputs", "[nowhere]NbOutputs"))
 
 
+MULTIBRANCH_INI = """
+DefaultModel=Frame_HIP
+
+[sp]
+SizeX=28
+SizeY=28
+BatchSize=4
+
+[c1]
+Input=sp
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=8
+Stride=2
+
+[c2]
+Input=c1
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=8
+
+; three branches with 3, 4 and 3 channels
+[left1]
+Input=c2
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=3
+
+[left2]
+Input=left1
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=3
+Padding=1
+
+[mid1]
+Input=c2
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=2 2
+NbOutputs=4
+
+[mid2]
+Input=mid1
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=2 2
+NbOutputs=4
+
+[right1]
+Input=c2
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=3
+
+; the convolution that reads all three
+[join]
+Input=left2,mid2,right1
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=10
+
+[after]
+Input=join
+Type=Conv
+ActivationFunction=Rectifier
+KernelDims=3 3
+NbOutputs=[join]NbOutputs
+Padding=1
+
+[sum]
+Input=join,after
+Type=ElemWise
+NbOutputs=[after]NbOutputs
+Operation=Sum
+ActivationFunction=Linear
+Weights=1 2
+Shifts=0 3
+
+[head]
+Input=sum
+Type=Conv
+ActivationFunction=Linear
+KernelDims=7 7
+NbOutputs=10
+
+[softmax]
+Input=head
+Type=Softmax
+NbOutputs=[head]NbOutputs
+"""
+
+
+def test_a_multibranch_model_file(fh):
+    """The shape of the reference's multi-branch fixture (tests/tests_data/mnist_multibranch_model/model.ini): branches of 3
+    and 4 channels, a convolution that reads three cells, a sum of two cells, a Softmax at the end; every cell against the
+    oracle, with and without the fusion plan."""
+    from n2d2_amd import nets
+    from oracle import cells
+    b = nets._Builder("multibranch", (1, 28, 28), 59, "SingleShift")
+    t = b.conv("c1", "input", 8, 3, stride=2)
+    c2 = b.conv("c2", t, 8, 3)
+    l = b.conv("left2", b.conv("left1", c2, 3, 3), 3, 3, pad=1)
+    m = b.conv("mid2", b.conv("mid1", c2, 4, 2), 4, 2)
+    r = b.conv("right1", c2, 3, 3)
+    j = b.conv("join", [l, m, r], 10, 3)
+    a = b.conv("after", j, 10, 3, pad=1)
+    s_ = b.sum("sum", [j, a], kind="Linear", weights=[1, 2], shifts=[0, 3])
+    b.conv("head", s_, 10, 7, kind="Linear")
+    spec = b.spec
+    x = np.random.default_rng(59).integers(0, 256, size=(4, 1, 28, 28))
+    keep = [l_.name for l_ in spec.layers]
+    want = cells.run_net(spec, x, keep=keep)
+    for fusion in (True, False):
+        net = fh.Net(MULTIBRANCH_INI)
+        assert net.nb_cells == len(spec.layers)
+        fh.install_parameters(net, spec)
+        net.set_fusion(fusion)
+        net.initialize()
+        net.set_stimuli(x)
+        net.propagate()
+        for name in keep:
+            assert np.array_equal(net.outputs(name), want[name]), (name, fusion)
+
+
 def test_cells_with_two_outputs_through_the_registrar(fh):
     """A binary classifier: a convolution with 3 outputs, a rescaled FC with 2 and a last FC with 2 raw logits (output
     tensors whose pixel is one dword), through the Registrar cells and through GpuNet."""
