@@ -1774,6 +1774,7 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
     std::map<std::string, Section> sections;
     std::map<std::string, std::string> inherits;
     Section global;
+    std::map<std::string, std::string> variables;
     std::string current;
     std::istringstream in(iniText);
     std::string line;
@@ -1794,7 +1795,19 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
         }
         const size_t eq = line.find('=');
         if (eq == std::string::npos) throw std::runtime_error("Malformed line: " + line);
-        const std::string key = trim(line.substr(0, eq)), value = trim(line.substr(eq + 1));
+        std::string key = trim(line.substr(0, eq)), value = trim(line.substr(eq + 1));
+        // "$BATCH_SIZE=64" defines a variable, "${BATCH_SIZE}" takes its value (N2D2's model files size their nets this way)
+        for (size_t at = value.find("${"); at != std::string::npos; at = value.find("${", at)) {
+            const size_t close = value.find('}', at);
+            if (close == std::string::npos) throw std::runtime_error("Malformed variable reference: " + line);
+            auto var = variables.find(value.substr(at + 2, close - at - 2));
+            if (var == variables.end()) throw std::runtime_error("Undefined variable in: " + line);
+            value.replace(at, close - at + 1, var->second);
+        }
+        if (key.size() > 1 && key[0] == '$') {
+            variables[key.substr(1)] = value;
+            continue;
+        }
         if (current.empty()) global[key] = value; else sections[current][key] = value;
     }
     std::function<Section(const std::string&, int)> resolvedAt = [&](const std::string& name, int depth) {

@@ -208,6 +208,8 @@ def test_grouped_convolution_cells(fh):
 
 
 MINI_MOBILENET_INI = """
+$BATCH=6
+$WIDTH=8
 DefaultModel=Frame_HIP
 
 [database]
@@ -216,7 +218,7 @@ Type=MNIST_IDX_Database
 [sp]
 SizeX=28
 SizeY=28
-BatchSize=6
+BatchSize=${BATCH}
 
 [sp.Transformation-1]
 Type=RangeAffineTransformation
@@ -238,7 +240,7 @@ Type=Fc
 [stem] conv_def
 Input=sp
 KernelDims=3 3
-NbOutputs=8
+NbOutputs=${WIDTH}
 Padding=1
 Stride=2
 
@@ -294,7 +296,7 @@ NbOutputs=[fc_b]NbOutputs
 
 def test_model_file_syntax_of_the_reference(fh):
     """An INI written the way N2D2's own model files are (tests/tests_data/mnist_model/model.ini: several templates behind a
-    section header, NbOutputs=[other]NbOutputs, scalar Padding / Stride, database / transformation / target sections, a
+    section header, $VARIABLES, NbOutputs=[other]NbOutputs, scalar Padding / Stride, database / transformation / target sections, a
     Softmax at the end, which the integer graph does not instantiate): the cells it describes against the oracle."""
     from n2d2_amd import nets
     b = nets._Builder("mini", (1, 28, 28), 53, "SingleShift")
