@@ -182,8 +182,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* desc, const void* weights, cons
 int n2d2hip_conv_destroy(n2d2hip_conv_t conv);
 /* Output spatial size (ref: src/Cell/ConvCell.cpp:1169-1195). */
 int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH, int* outW);
-/* in / out: NHWC with the channel stride of n2d2hip_nhwc_cs (4 for at most 4 channels, a multiple of 16 otherwise; a
- * depthwise cell needs a multiple of 16).  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE).  `in` and a byte `out`
+/* in / out: NHWC with the channel stride of n2d2hip_nhwc_cs (4 for at most 4 channels, a multiple of 16 otherwise).  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE).  `in` and a byte `out`
  * may have a halo if n2d2hip_conv_accepts_halo says so. */
 int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);

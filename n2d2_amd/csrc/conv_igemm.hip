@@ -801,8 +801,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         return rc;
     N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
                     "conv_forward: output is %dx%dx%dx%d, expected %dx%dx%dx%d", out->B, out->C, out->H, out->W, in->B, d.O, OH, OW);
-    N2D2HIP_REQUIRE(out->cs % 16 == 0 || (out->cs == 4 && !c->depthwise), N2D2HIP_ERR_INVALID,
-                    "conv_forward: output channel stride %d must be a multiple of 16 (or 4 for at most 4 outputs, not depthwise)", out->cs);
+    N2D2HIP_REQUIRE(out->cs % 16 == 0 || out->cs == 4, N2D2HIP_ERR_INVALID,
+                    "conv_forward: output channel stride %d must be a multiple of 16 (or 4 for at most 4 outputs)", out->cs);
     // with a folded sum the stored values are the sum cell's
     const n2d2hip_act_s* act = other ? c->sum->act : c->act;
     if (other) {
@@ -835,7 +835,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     if (c->depthwise) {
         N2D2HIP_REQUIRE(out->cs == in->cs, N2D2HIP_ERR_INVALID, "conv_forward: depthwise needs equal channel strides");
         N2D2HIP_REQUIRE(in->halo == 0 && out->halo == 0, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: depthwise tensors carry no border");
-        if (c->d_wdw && d.strideX == d.strideY && (d.strideX == 1 || d.strideX == 2) && is_byte_type(out->dtype)
+        if (c->d_wdw && in->cs % 16 == 0 && d.strideX == d.strideY && (d.strideX == 1 || d.strideX == 2) && is_byte_type(out->dtype)
             && c->act->cpad >= in->cs) {
             DepthwiseArgs q;
             q.in = (const signed char*)in->data; q.out = out->data; q.wb = c->d_wdw;

@@ -466,6 +466,14 @@ def test_cells_with_at_most_four_outputs(rt):
             spec = _acts(O)[an]
             fc = rt.Fc(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, (84, 1, 1))
             assert np.array_equal(fc.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), cells_ref.fc_cell(x, w, bias, spec).astype(np.int64)), (O, an)
+    # depthwise on 3 channels (3x3 and 5x5, stride 1 and 2)
+    for k, stride in ((3, 1), (3, 2), (5, 1)):
+        x = _u8((2, 3, 9, 8))
+        w = _i8((3, 1, k, k))
+        spec = _acts(3)["sshift_relu_u"]
+        want = cells_ref.conv_cell(x, w, None, spec, stride=(stride, stride), pad=(k // 2,) * 4, groups=3)
+        conv = rt.Conv(w, None, rt.Act(3, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(k // 2,) * 4, groups=3)
+        assert np.array_equal(conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy(), want.astype(np.int64)), (k, stride)
     # two layers: 16 -> 2 -> 8 channels
     x = _u8((2, 16, 8, 8))
     w1, w2 = _i8((2, 16, 3, 3)), _i8((8, 2, 3, 3))
