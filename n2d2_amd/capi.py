@@ -33,7 +33,7 @@ SYMBOLS = [
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", "n2d2hip_expand_reduce_create", "n2d2hip_expand_reduce_destroy", "n2d2hip_expand_reduce_forward",
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
-    "n2d2hip_pool_out_dims", "n2d2hip_pool_forward",
+    "n2d2hip_pool_out_dims", "n2d2hip_pool_forward", "n2d2hip_pool_forward_mapped",
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling", "n2d2hip_concat_channels",
     "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_forward_static", "n2d2hip_sat_weight_backward",
     "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
@@ -119,6 +119,7 @@ def load():
     lib.n2d2hip_fc_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_pool_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_pool_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_pool_forward_mapped.argtypes = [P, P, P, P, P]
     lib.n2d2hip_elemwise_create.argtypes = [I, I, I, P, P, P, P]
     lib.n2d2hip_elemwise_destroy.argtypes = [P]
     lib.n2d2hip_elemwise_fold_input_scaling.argtypes = [P, I, P]

@@ -69,6 +69,51 @@ __global__ __launch_bounds__(256) void pool_kernel(const signed char* __restrict
     }
 }
 
+// Pooling with a connection map (ref: src/Cell/PoolCell_Frame_Kernels.cpp:60-75,150-185): output o pools the window over
+// every channel c with maps[o * C + c] set: the largest value met, or the sum divided by window size x connected channels
+// and truncated toward zero.  An output without a connected channel, or whose window lies outside the image, is 0.  One
+// thread per output value; `bias` turns stored bytes into values (128 for the biased form, 0 otherwise).
+template <bool IS_MAX, bool IS_SIGNED>
+__global__ __launch_bounds__(256) void pool_mapped_kernel(const signed char* __restrict__ in, int cs, int C, int B, int H, int W,
+                                                          const unsigned char* __restrict__ maps, signed char* __restrict__ out,
+                                                          int out_cs, int O, int OH, int OW, int poolW, int poolH, int strideX,
+                                                          int strideY, int padX, int padY, int bias)
+{
+    const long long total = (long long)B * OH * OW * out_cs;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        const int o = (int)(idx % out_cs);
+        long long r = idx / out_cs;
+        const int ox = (int)(r % OW); r /= OW;
+        const int oy = (int)(r % OH);
+        const int b = (int)(r / OH);
+        int result = 0;
+        if (o < O) {
+            const int bx = ox * strideX - padX, by = oy * strideY - padY;
+            const int sxMin = max(-bx, 0), syMin = max(-by, 0);
+            const int sxMax = min(max(W - bx, 0), poolW), syMax = min(max(H - by, 0), poolH);
+            int acc = 0, count = 0;
+            bool valid = false;
+            for (int c = 0; c < C; ++c) {
+                if (!maps[(long long)o * C + c])
+                    continue;
+                for (int sy = syMin; sy < syMax; ++sy)
+                    for (int sx = sxMin; sx < sxMax; ++sx) {
+                        const signed char raw = in[(((long long)b * H + by + sy) * W + bx + sx) * cs + c];
+                        const int v = (IS_SIGNED ? (int)raw : (int)(unsigned char)raw) + bias;
+                        if (IS_MAX) {
+                            acc = valid ? max(acc, v) : v;
+                            valid = true;
+                        } else
+                            acc += v;
+                    }
+                count += poolW * poolH;            // countIncludePadding = true
+            }
+            result = IS_MAX ? acc : (count > 0 ? acc / count : 0);
+        }
+        out[idx] = (signed char)(result - bias);    // channels between O and the channel stride hold the stored 0
+    }
+}
+
 // Max pooling with a small compile-time window, 16 channels per thread.  The maximum of signed bytes is taken on the
 // packed words themselves: even and odd bytes are moved to the high halves of two 16-bit pairs, where the packed
 // 16-bit maximum orders them as bytes.  A tap outside the input is replaced by the nearest tap inside, which cannot
@@ -455,6 +500,36 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     else
         hipLaunchKernelGGL(pool_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* d, const unsigned char* maps, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                                n2d2hip_stream_t stream)
+{
+    int rc, OH, OW;
+    N2D2HIP_REQUIRE(d != nullptr && maps != nullptr, N2D2HIP_ERR_INVALID, "pool_forward_mapped: null descriptor or map");
+    N2D2HIP_REQUIRE(d->pooling == N2D2HIP_POOL_MAX || d->pooling == N2D2HIP_POOL_AVERAGE, N2D2HIP_ERR_INVALID, "pool_forward_mapped: bad pooling %d", d->pooling);
+    if ((rc = check_tensor(in, "pool input")) || (rc = check_tensor(out, "pool output")) || (rc = n2d2hip_pool_out_dims(d, in->H, in->W, &OH, &OW)))
+        return rc;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED, "pool_forward_mapped: tensors must be NHWC");
+    N2D2HIP_REQUIRE(is_byte_type(in->dtype) && out->dtype == in->dtype, N2D2HIP_ERR_INVALID, "pool_forward_mapped: byte tensors of one dtype expected");
+    N2D2HIP_REQUIRE(out->B == in->B && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
+                    "pool_forward_mapped: output is %dx%dx%dx%d, expected %dxOx%dx%d", out->B, out->C, out->H, out->W, in->B, OH, OW);
+    const long long total = (long long)in->B * OH * OW * out->cs;
+    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
+    const int bias = in->dtype == N2D2HIP_U8B ? 128 : 0;
+#define N2D2HIP_POOL_MAPPED(IS_MAX, IS_SIGNED)                                                                                      \
+    hipLaunchKernelGGL((pool_mapped_kernel<IS_MAX, IS_SIGNED>), dim3(grid), dim3(256), 0, (hipStream_t)stream,                       \
+                       (const signed char*)in->data, in->cs, in->C, in->B, in->H, in->W, maps, (signed char*)out->data, out->cs,     \
+                       out->C, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, bias)
+    const bool is_signed = in->dtype != N2D2HIP_U8;
+    if (d->pooling == N2D2HIP_POOL_MAX) {
+        if (is_signed) N2D2HIP_POOL_MAPPED(true, true); else N2D2HIP_POOL_MAPPED(true, false);
+    } else {
+        if (is_signed) N2D2HIP_POOL_MAPPED(false, true); else N2D2HIP_POOL_MAPPED(false, false);
+    }
+#undef N2D2HIP_POOL_MAPPED
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

@@ -756,10 +756,60 @@ void PoolCell_Frame_HIP<T>::addInput(Cell_Frame_HIP* parent)
 }
 
 template <class T>
+void PoolCell_Frame_HIP<T>::setMapping(const Tensor<bool>& map)
+{
+    if (map.dimX() != mNbOutputs || map.dimY() != mNbChannels)
+        throw std::runtime_error("PoolCell_Frame_HIP::setMapping(): the map of " + mName + " must be {nbOutputs, nbChannels}");
+    bool unit = mNbOutputs == mNbChannels;
+    for (std::size_t o = 0; unit && o < mNbOutputs; ++o)
+        for (std::size_t ch = 0; unit && ch < mNbChannels; ++ch)
+            unit = map.at(o, ch) == (o == ch);
+    mMapping = unit ? Tensor<bool>() : map;
+    if (mMappingDevice) {
+        (void)hipFree(mMappingDevice);
+        mMappingDevice = nullptr;
+    }
+}
+
+template <class T>
+PoolCell_Frame_HIP<T>::~PoolCell_Frame_HIP()
+{
+    if (mMappingDevice) (void)hipFree(mMappingDevice);
+}
+
+template <class T>
 void PoolCell_Frame_HIP<T>::initialize()
 {
-    if (mInputs.empty() || mNbOutputs != mNbChannels)
-        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": a unit mapping (NbOutputs == the inputs' channels) is supported");
+    if (mInputs.empty())
+        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": no input");
+    if (mMapping.empty() && mNbOutputs != mNbChannels)
+        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": without a connection map (setMapping) the cell pools one output per "
+                                 "channel, NbOutputs must be the inputs' channels");
+    if (!mMapping.empty()) {
+        // channels of one input only behind every output
+        for (std::size_t o = 0; o < mNbOutputs; ++o) {
+            int owner = -1;
+            std::size_t first = 0;
+            for (std::size_t k = 0; k < mInputs.size(); ++k) {
+                const std::size_t n = (std::size_t)mInputs[k]->desc().C;
+                for (std::size_t ch = first; ch < first + n; ++ch)
+                    if (mMapping.at(o, ch)) {
+                        if (owner >= 0 && owner != (int)k)
+                            throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": an output that pools channels of several inputs is not supported");
+                        owner = (int)k;
+                    }
+                first += n;
+            }
+        }
+        std::vector<unsigned char> host(mNbOutputs * mNbChannels);
+        for (std::size_t o = 0; o < mNbOutputs; ++o)
+            for (std::size_t ch = 0; ch < mNbChannels; ++ch)
+                host[o * mNbChannels + ch] = mMapping.at(o, ch) ? 1 : 0;
+        if (mMappingDevice) (void)hipFree(mMappingDevice);
+        mMappingDevice = nullptr;
+        checkHip(hipMalloc((void**)&mMappingDevice, host.size()), "PoolCell_Frame_HIP::initialize(): hipMalloc");
+        checkHip(hipMemcpy(mMappingDevice, host.data(), host.size(), hipMemcpyHostToDevice), "PoolCell_Frame_HIP::initialize(): hipMemcpy");
+    }
     mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
 }
 
@@ -777,7 +827,7 @@ n2d2hip_pool_desc PoolCell_Frame_HIP<T>::poolDesc() const
 template <class T>
 bool PoolCell_Frame_HIP<T>::fuseFirstConv(Cell_Frame_HIP* conv)
 {
-    if (mFusedConv || !conv || !conv->convHandle() || conv->foldedInto() || mInputs.size() != 1 || conv->parentCells().size() != 1)
+    if (mFusedConv || !mMapping.empty() || !conv || !conv->convHandle() || conv->foldedInto() || mInputs.size() != 1 || conv->parentCells().size() != 1)
         return false;
     const n2d2hip_pool_desc d = poolDesc();
     const n2d2hip_tensor& x = conv->inputTensor(0)->desc();
@@ -793,7 +843,7 @@ bool PoolCell_Frame_HIP<T>::writesHalo() const
 {
     if (mFusedConv)
         return true;
-    if (mInputs.size() != 1 || mInputs[0]->empty())
+    if (mInputs.size() != 1 || mInputs[0]->empty() || !mMapping.empty())
         return false;
     const n2d2hip_pool_desc d = poolDesc();
     const n2d2hip_tensor& x = mInputs[0]->desc();
@@ -819,6 +869,9 @@ void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
     const n2d2hip_pool_desc d = poolDesc();
     if (mFusedConv)
         checkStatus(n2d2hip_conv_forward_maxpool(mFusedConv->convHandle(), &d, &mFusedConv->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
+    else if (mMappingDevice)
+        checkStatus(n2d2hip_pool_forward_mapped(&d, mMappingDevice, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(),
+                                                mStream));
     else
         checkStatus(n2d2hip_pool_forward(&d, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
@@ -1766,6 +1819,71 @@ std::vector<unsigned int> getDims(const Section& s, const std::string& vec, cons
     const unsigned int both = getUInt(s, scalar, def);
     return {getUInt(s, x, both), getUInt(s, y, both)};
 }
+// The connection map between one parent and a cell, {nbOutputs, nbChannels}, from the section's Mapping keys
+// (src/Generator/MappingGenerator.cpp:33-201): equal groups (Mapping.NbGroups / Mapping.ChannelsPerGroup), a matrix written
+// out (Mapping(parent)= one row per channel), a patch stepped along the diagonal (Mapping.Size / Stride / Offset /
+// NbIterations, each also as Mapping(parent).Key for one parent), every connection when the section has none of them.
+Tensor<bool> generateMapping(const Section& s, const std::string& section, const std::string& parentName, std::size_t nbOutputs,
+                             std::size_t nbChannels)
+{
+    const std::string own = "Mapping(" + parentName + ")";
+    const bool byGroups = s.count("Mapping.NbGroups") != 0, byWidth = s.count("Mapping.ChannelsPerGroup") != 0;
+    if (byGroups && byWidth)
+        throw std::runtime_error("Mapping.NbGroups and Mapping.ChannelsPerGroup are mutually exclusive in section [" + section + "]");
+    if (byGroups || byWidth) {
+        const std::size_t given = getUInt(s, byGroups ? "Mapping.NbGroups" : "Mapping.ChannelsPerGroup", 0);
+        if (given == 0 || given > nbChannels)
+            throw std::runtime_error("Mapping.NbGroups must be a multiple of the number of input channels in section [" + section + "]");
+        const std::size_t groups = byGroups ? given : nbChannels / given, width = byGroups ? nbChannels / given : given;
+        if (nbChannels % groups != 0)
+            throw std::runtime_error("Mapping.NbGroups must be a multiple of the number of input channels in section [" + section + "]");
+        Tensor<bool> map({nbOutputs, nbChannels}, false);
+        std::size_t firstOutput = 0;
+        for (std::size_t g = 0; g < groups; ++g) {
+            const std::size_t outputsHere = (nbOutputs - firstOutput) / (groups - g);     // the outputs left, shared out evenly
+            for (std::size_t o = firstOutput; o < firstOutput + outputsHere; ++o)
+                for (std::size_t ch = g * width; ch < (g + 1) * width; ++ch)
+                    map.set(o, ch, true);
+            firstOutput += outputsHere;
+        }
+        return map;
+    }
+    if (s.count(own)) {
+        const std::vector<std::string> values = split(s.at(own), " \t,;");
+        if (values.size() != nbOutputs * nbChannels)
+            throw std::runtime_error(own + " in section [" + section + "] holds " + std::to_string(values.size()) + " values, the map has "
+                                     + std::to_string(nbOutputs * nbChannels));
+        Tensor<bool> map({nbOutputs, nbChannels}, false);
+        for (std::size_t i = 0; i < values.size(); ++i)
+            map.set(i % nbOutputs, i / nbOutputs, values[i] != "0");      // the file's rows are channels, its columns outputs
+        return map;
+    }
+    bool isFunction = false;
+    for (const auto& kv : s)
+        isFunction = isFunction || kv.first.compare(0, 8, "Mapping.") == 0 || kv.first.compare(0, own.size() + 1, own + ".") == 0;
+    Tensor<bool> map({nbOutputs, nbChannels}, !isFunction);
+    if (!isFunction || map.empty())
+        return map;
+    auto key = [&](const std::string& both, const std::string& one) {
+        for (const std::string& prefix : {own, std::string("Mapping")})
+            for (const std::string& k : {both, one})
+                if (s.count(prefix + "." + k))
+                    return getUInt(s, prefix + "." + k, 0);
+        return (unsigned int)(both == "Offset" ? 0 : 1);
+    };
+    std::size_t sizeX = key("Size", "SizeX"), sizeY = key("Size", "SizeY");
+    const std::size_t strideX = key("Stride", "StrideX"), strideY = key("Stride", "StrideY");
+    const std::size_t offsetX = key("Offset", "OffsetX"), offsetY = key("Offset", "OffsetY");
+    std::size_t iterations = s.count(own + ".NbIterations") ? getUInt(s, own + ".NbIterations", 0) : getUInt(s, "Mapping.NbIterations", 0);
+    if (iterations == 0) iterations = std::max(nbOutputs, nbChannels);
+    if (sizeY == 0) sizeY = nbChannels;
+    if (sizeX == 0) sizeX = nbOutputs;
+    for (std::size_t i = 0, x = offsetX, y = offsetY; i < iterations; ++i, x += strideX, y += strideY)
+        for (std::size_t px = 0; px < sizeX; ++px)
+            for (std::size_t py = 0; py < sizeY; ++py)
+                map.set((x + px) % nbOutputs, (y + py) % nbChannels, true);
+    return map;
+}
 } // namespace
 
 std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string* modelOut)
@@ -1938,10 +2056,38 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
             throw std::runtime_error("Cell type " + type + " is not on the quantized path (section [" + name + "])");
         }
         deepNet->addCell(cell, parents);
+        // src/Generator/PoolCellGenerator.cpp:160-195, ConvCellGenerator.cpp: one map per parent, side by side
+        auto mappingOverParents = [&]() {
+            Tensor<bool> map({cell->getNbOutputs(), cell->getNbChannels()}, false);
+            std::size_t first = 0;
+            for (std::size_t k = 0; k < std::max<std::size_t>(parents.size(), 1); ++k) {
+                const Cell* parent = parents.empty() ? nullptr : parents[k].get();        // no parent cell: the stimuli
+                const std::size_t n = parent ? parent->getNbOutputs() : cell->getNbChannels();
+                const Tensor<bool> part = generateMapping(s, name, parent ? parent->getName() : "env", cell->getNbOutputs(), n);
+                for (std::size_t o = 0; o < cell->getNbOutputs(); ++o)
+                    for (std::size_t ch = 0; ch < n; ++ch)
+                        map.set(o, first + ch, part.at(o, ch));
+                first += n;
+            }
+            return map;
+        };
+        if (type == "Pool") {
+            auto pool = std::dynamic_pointer_cast<PoolCell_Frame_HIP<float> >(cell);
+            if (pool) pool->setMapping(mappingOverParents());
+        }
         if (type == "Conv") {
             const unsigned int perGroup = getUInt(s, "Mapping.ChannelsPerGroup", 0);
             const unsigned int groups = perGroup ? cell->getNbChannels() / perGroup : getUInt(s, "Mapping.NbGroups", 1);
-            if (groups > 1) std::dynamic_pointer_cast<ConvCell>(cell)->setNbGroups(groups);
+            if (groups > 1)
+                std::dynamic_pointer_cast<ConvCell>(cell)->setNbGroups(groups);
+            else if (!perGroup && !s.count("Mapping.NbGroups")) {
+                const Tensor<bool> map = mappingOverParents();      // a map written out or stepped along the diagonal
+                bool full = true;
+                for (std::size_t o = 0; full && o < map.dimX(); ++o)
+                    for (std::size_t ch = 0; full && ch < map.dimY(); ++ch)
+                        full = map.at(o, ch);
+                if (!full) std::dynamic_pointer_cast<ConvCell>(cell)->setMapping(map);
+            }
         }
     }
     return deepNet;

@@ -657,6 +657,12 @@ public:
     // input behind the other, gathered by one extra launch.
     void addInput(Cell_Frame_HIP* parent);
     using Cell_Frame_HIP::addInput;
+    // The connection map over all inputs' channels, {nbOutputs, nbChannels}: what the `mapping` arguments of the reference's
+    // addInput() calls add up to (src/Cell/Cell_Frame.cpp:100-132).  Without a call the cell pools one output per channel
+    // (the Mapping.ChannelsPerGroup=1 of N2D2's model files).  An output may pool channels of one input only: the
+    // reference adds up one pooling per input there, which no model asks for.
+    void setMapping(const Tensor<bool>& map);
+    ~PoolCell_Frame_HIP();
     void initialize();
     void propagate(bool inference = false);
     // src/Cell/PoolCell_Frame.cpp:263-266
@@ -676,6 +682,8 @@ protected:
 private:
     n2d2hip_pool_desc poolDesc() const;
     Cell_Frame_HIP* mFusedConv = nullptr;
+    Tensor<bool> mMapping;                   // empty: one output per channel
+    unsigned char* mMappingDevice = nullptr; // [output][channel] bytes
     static Registrar<PoolCell> mRegistrar;
 };
 

@@ -190,13 +190,15 @@ int fh_get_nb_groups(const unsigned char* map, size_t nbOutputs, size_t nbChanne
 int fh_cell_set_mapping(void* net, const char* name, const unsigned char* map, size_t nbOutputs, size_t nbChannels)
 {
     return guarded([&] {
-        auto conv = std::dynamic_pointer_cast<ConvCell>(((Net*)net)->deepNet->getCell(name));
-        if (!conv) throw std::runtime_error("fh_cell_set_mapping(): " + std::string(name) + " is not a Conv");
+        auto cell = ((Net*)net)->deepNet->getCell(name);
+        auto conv = std::dynamic_pointer_cast<ConvCell>(cell);
+        auto pool = std::dynamic_pointer_cast<PoolCell_Frame_HIP<float> >(cell);
+        if (!conv && !pool) throw std::runtime_error("fh_cell_set_mapping(): " + std::string(name) + " is neither a Conv nor a Pool");
         Tensor<bool> m({nbOutputs, nbChannels}, false);
         for (size_t c = 0; c < nbChannels; ++c)
             for (size_t o = 0; o < nbOutputs; ++o)
                 m.set(o, c, map[o + nbOutputs * c] != 0);
-        conv->setMapping(m);
+        if (conv) conv->setMapping(m); else pool->setMapping(m);
     });
 }
 

@@ -334,7 +334,16 @@ def spec_to_ini(spec, batch, model="Frame_HIP"):
         elif l.type == "fc":
             lines += ["Type=Fc", "NbOutputs=%d" % l.w.shape[0], "ActivationFunction=%s" % l.act.kind]
         elif l.type == "pool":
-            lines += ["Type=Pool", "PoolDims=%d %d" % l.pool, "NbOutputs=%d" % l.out_shape[0], "StrideDims=%d %d" % l.stride,
+            lines += ["Type=Pool"]
+            if len(l.inputs) == 1:
+                lines += ["Mapping.ChannelsPerGroup=1"]
+            else:       # one output per channel of every input: a diagonal per parent, starting at the parent's first channel
+                first = 0
+                for i in l.inputs:
+                    n = spec.shapes[i][0]
+                    lines += ["Mapping(%s).OffsetX=%d" % (i, first), "Mapping(%s).NbIterations=%d" % (i, n)]
+                    first += n
+            lines += ["PoolDims=%d %d" % l.pool, "NbOutputs=%d" % l.out_shape[0], "StrideDims=%d %d" % l.stride,
                       "PaddingDims=%d %d" % l.pad, "Pooling=%s" % ("Max" if l.kind == "max" else "Average")]
         elif l.type == "elemwise":
             lines += ["Type=ElemWise", "NbOutputs=%d" % l.out_shape[0], "Operation=Sum", "ActivationFunction=%s" % l.act.kind]

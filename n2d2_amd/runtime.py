@@ -305,19 +305,31 @@ class Fc:
 
 
 class Pool:
-    def __init__(self, kind, pool, stride, pad=(0, 0)):
+    def __init__(self, kind, pool, stride, pad=(0, 0), maps=None):
+        """maps: None for one output per channel, else a bool array [channels, outputs] (maps[c, o]: output o pools channel c)."""
         self.desc = capi.PoolDesc(capi.POOL_MAX if kind == "max" else capi.POOL_AVERAGE, pool[0], pool[1],
                                   stride[0], stride[1], pad[0], pad[1])
+        self.maps = None
+        if maps is not None:
+            m = np.ascontiguousarray(np.asarray(maps, dtype=np.uint8).T)      # one row per output
+            self.nb_channels, self.nb_outputs = m.shape[1], m.shape[0]
+            self.maps = torch.from_numpy(m.reshape(-1)).cuda()
 
     def make_output(self, x):
         oh, ow = C.c_int(), C.c_int()
         check(lib.n2d2hip_pool_out_dims(C.byref(self.desc), x.H, x.W, C.byref(oh), C.byref(ow)))
-        return DTensor(x.B, x.C, oh.value, ow.value, x.dtype)
+        return DTensor(x.B, x.C if self.maps is None else self.nb_outputs, oh.value, ow.value, x.dtype)
 
     def forward(self, x, out=None):
         if out is None:
             out = self.make_output(x)
-        check(lib.n2d2hip_pool_forward(C.byref(self.desc), x.ref, out.ref, stream_ptr()))
+        if self.maps is None:
+            check(lib.n2d2hip_pool_forward(C.byref(self.desc), x.ref, out.ref, stream_ptr()))
+        else:
+            if x.C != self.nb_channels or out.C != self.nb_outputs:
+                raise ValueError("Pool: the map is %d channels x %d outputs, the tensors have %d and %d"
+                                 % (self.nb_channels, self.nb_outputs, x.C, out.C))
+            check(lib.n2d2hip_pool_forward_mapped(C.byref(self.desc), self.maps.data_ptr(), x.ref, out.ref, stream_ptr()))
         return out
 
 

@@ -85,15 +85,16 @@ def fc_cell(x, w, bias, act):
     return act.apply(y.reshape(y.shape[0], y.shape[1], 1, 1))
 
 
-def pool_cell(x, kind, pool, stride, pad=(0, 0)):
+def pool_cell(x, kind, pool, stride, pad=(0, 0), maps=None):
     """x: one input, or a list of inputs: PoolCell_Frame<T>::propagate (src/Cell/PoolCell_Frame.cpp:123-174) then walks them
-    with the rows of the unit map over all their channels that belong to each, beta = 0 for the first and 1 afterwards (an
-    output pools nothing from the inputs it is not connected to: 0 is added)."""
+    with the rows of the map over all their channels that belong to each, beta = 0 for the first and 1 afterwards (an
+    output pools nothing from the inputs it is not connected to: 0 is added).  maps: bool [channels, outputs], the unit map
+    (one output per channel) when None."""
     if not isinstance(x, (list, tuple)) or len(x) == 1:
         x = x[0] if isinstance(x, (list, tuple)) else x
-        return orc.pool_forward(np.ascontiguousarray(x, dtype=np.float32), pool, stride, pad, kind=kind, quantized=True)
+        return orc.pool_forward(np.ascontiguousarray(x, dtype=np.float32), pool, stride, pad, kind=kind, quantized=True, maps=maps)
     total = sum(xk.shape[1] for xk in x)
-    unit = np.eye(total, dtype=np.uint8)
+    unit = np.eye(total, dtype=np.uint8) if maps is None else np.ascontiguousarray(maps, dtype=np.uint8)
     y, first = None, 0
     for k, xk in enumerate(x):
         xk = np.ascontiguousarray(xk, dtype=np.float32)

@@ -119,6 +119,7 @@ ActivationFunction=Linear
 [pool1]
 Input=conv1
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=2 2
 NbOutputs=6
 Stride=2
@@ -134,6 +135,7 @@ ActivationFunction=Linear
 [pool2]
 Input=conv2
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=2 2
 NbOutputs=16
 Stride=2

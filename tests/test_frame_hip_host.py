@@ -33,6 +33,7 @@ Padding=3
 [pool1]
 Input=conv1
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=3 3
 NbOutputs=16
 Stride=2
@@ -158,6 +159,7 @@ ActivationFunction=Rectifier
 [pool1]
 Input=conv1
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=2 2
 NbOutputs=6
 Stride=2
@@ -354,8 +356,11 @@ def test_conv_mapping_sets_the_groups(fh):
     with pytest.raises(fh.FrameHipError, match="must be"):
         net.set_mapping("conv1", np.ones((O + 1, Cn)))
     net.set_mapping("conv1", np.ones((O, Cn)))          # fully connected: one group
-    with pytest.raises(fh.FrameHipError, match="not a Conv"):
-        net.set_mapping("pool1", np.ones((16, 16)))
+    net.set_mapping("pool1", np.ones((16, 16)))         # a PoolCell takes a map too: every channel behind every output
+    with pytest.raises(fh.FrameHipError, match="must be"):
+        net.set_mapping("pool1", np.ones((16, 15)))
+    with pytest.raises(fh.FrameHipError, match="neither a Conv nor a Pool"):
+        net.set_mapping("fc", np.ones((16, 16)))
 
 
 def test_quantization_files_round_trip(fh, tmp_path):

@@ -164,7 +164,7 @@ def test_depthwise_cell_from_its_connection_map(fh):
     from oracle import cells
     spec = nets.mobilenet_v1(image=64)
     x = np.random.default_rng(35).integers(0, 256, size=(2, 3, 64, 64))
-    ini = "\n".join(line for line in fh.spec_to_ini(spec, 2).split("\n") if not line.startswith("Mapping."))
+    ini = "\n".join(line for line in fh.spec_to_ini(spec, 2).split("\n") if not line.startswith("Mapping.NbGroups"))
     net = fh.Net(ini)
     for l in spec.layers:
         if l.type == "conv" and l.groups > 1:
@@ -193,7 +193,7 @@ def test_grouped_convolution_cells(fh):
     x = np.random.default_rng(41).integers(0, 256, size=(3, 8, 20, 20))
     keep = [l.name for l in spec.layers]
     _compare(fh, spec, x, keep)
-    ini = "\n".join(line for line in fh.spec_to_ini(spec, 3).split("\n") if not line.startswith("Mapping."))
+    ini = "\n".join(line for line in fh.spec_to_ini(spec, 3).split("\n") if not line.startswith("Mapping.NbGroups"))
     net = fh.Net(ini)
     for l in spec.layers:
         if l.type == "conv":
@@ -258,6 +258,7 @@ NbOutputs=12
 [pool_a]
 Input=pw_a
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=3 3
 NbOutputs=[pw_a]NbOutputs
 Pooling=Max
@@ -271,6 +272,7 @@ NbOutputs=[pool_a]NbOutputs
 [pool_b]
 Input=dw_b
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=2 2
 NbOutputs=[dw_b]NbOutputs
 Pooling=Average
@@ -454,6 +456,96 @@ def test_a_multibranch_model_file(fh):
         net.propagate()
         for name in keep:
             assert np.array_equal(net.outputs(name), want[name]), (name, fusion)
+
+
+POOL_MAPPINGS_INI = """
+[p_full]
+Input=c1
+Type=Pool
+PoolDims=2 2
+Stride=2
+NbOutputs=2
+Pooling=Max
+
+[p_groups]
+Input=c1
+Type=Pool
+PoolDims=3 3
+Stride=2
+NbOutputs=3
+Pooling=Average
+Mapping.NbGroups=3
+
+[p_step]
+Input=c1
+Type=Pool
+PoolDims=2 2
+Stride=2
+NbOutputs=3
+Pooling=Max
+Mapping.SizeY=3
+Mapping.StrideY=2
+Mapping.OffsetY=1
+
+[p_hand]
+Input=c1
+Type=Pool
+PoolDims=3 3
+Stride=1
+Padding=1
+NbOutputs=2
+Pooling=Average
+Mapping(c1)=1 0  0 1  1 1  0 0  0 1  1 0
+
+[p_two]
+Input=c1,c2
+Type=Pool
+PoolDims=2 2
+Stride=2
+NbOutputs=2
+Pooling=Max
+Mapping(c1).SizeY=0
+Mapping(c1).NbIterations=1
+Mapping(c2).SizeY=0
+Mapping(c2).NbIterations=1
+Mapping(c2).OffsetX=1
+"""
+
+
+def test_pool_cells_with_connection_maps(fh):
+    """Pool sections with the Mapping keys of src/Generator/MappingGenerator.cpp:33-201: none (every channel behind every
+    output), equal groups, a patch stepped along the diagonal, a matrix written out, and two parents with a map each; the
+    maps expected here are written down by hand from that file's loops, the outputs come from the oracle's pooling with them."""
+    from n2d2_amd import nets
+    from oracle import cells
+    b = nets._Builder("maps", (1, 14, 14), 83, "SingleShift")
+    b.conv("c1", "input", 6, 3)
+    b.conv("c2", "input", 6, 3)
+    spec = b.spec
+    x = np.random.default_rng(83).integers(0, 256, size=(3, 1, 14, 14))
+    want = cells.run_net(spec, x, keep=["c1", "c2"])
+    net = fh.Net(fh.spec_to_ini(spec, 3) + POOL_MAPPINGS_INI)
+    fh.install_parameters(net, spec)
+    net.initialize()
+    net.set_stimuli(x)
+    net.propagate()
+    c1, c2 = net.outputs("c1"), net.outputs("c2")
+    assert np.array_equal(c1, want["c1"]) and np.array_equal(c2, want["c2"])
+
+    def m(rows):            # [channel][output]
+        return np.array(rows, dtype=np.uint8)
+    full = np.ones((6, 2), dtype=np.uint8)
+    groups = m([[1, 0, 0], [1, 0, 0], [0, 1, 0], [0, 1, 0], [0, 0, 1], [0, 0, 1]])
+    # x = i, y = 1 + 2 i for i = 0..5, a patch of 1 output x 3 channels, both modulo the sizes
+    step = m([[0, 0, 1], [1, 0, 1], [1, 0, 0], [1, 1, 0], [0, 1, 0], [0, 1, 1]])
+    hand = m([[1, 0], [0, 1], [1, 1], [0, 0], [0, 1], [1, 0]])
+    # one iteration each: output 0 pools all of c1, output 1 all of c2
+    two = m([[1, 0]] * 6 + [[0, 1]] * 6)
+    for name, kind, pool, stride, pad, maps, src in (("p_full", "max", 2, 2, 0, full, c1), ("p_groups", "avg", 3, 2, 0, groups, c1),
+                                                    ("p_step", "max", 2, 2, 0, step, c1), ("p_hand", "avg", 3, 1, 1, hand, c1),
+                                                    ("p_two", "max", 2, 2, 0, two, np.concatenate([c1, c2], 1))):
+        ref = cells.pool_cell(src, kind, (pool, pool), (stride, stride), (pad, pad), maps=maps)
+        assert np.array_equal(net.outputs(name), ref), name
 
 
 def test_cells_with_two_outputs_through_the_registrar(fh):

@@ -425,6 +425,7 @@ ActivationFunction=Linear
 [pool]
 Input=c1
 Type=Pool
+Mapping.ChannelsPerGroup=1
 PoolDims=2 2
 NbOutputs=6
 Stride=2

@@ -502,6 +502,28 @@ def test_pool_cell_bit_exact(rt, kind, pool, stride, pad):
         assert np.array_equal(got, want.astype(np.int64)), (kind, dt)
 
 
+def test_pool_cell_with_a_connection_map_bit_exact(rt):
+    """Outputs that pool several channels (PoolCell_Frame_Kernels.cpp:60-75,150-185): the full map a Pool section without
+    Mapping keys gets, groups, a hand-made map with an unconnected output."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(77)
+    for dt, x in ((capi.U8B, _u8((2, 12, 9, 10))), (capi.I8, _i8((2, 12, 9, 10), -128, 127)), (capi.U8, _u8((2, 3, 8, 8))),
+                  (capi.U8B, _u8((1, 40, 7, 7)))):
+        Cn = x.shape[1]
+        groups = np.zeros((Cn, 3), dtype=np.uint8)
+        for c in range(Cn):
+            groups[c, c * 3 // Cn] = 1
+        hand = (rng.random((Cn, 5)) < 0.4).astype(np.uint8)
+        hand[:, 2] = 0                                       # an output no channel feeds
+        for maps in (np.ones((Cn, 4), dtype=np.uint8), groups, hand, np.ones((Cn, 20), dtype=np.uint8)):
+            for kind, pool, stride, pad in (("max", (2, 2), (2, 2), (0, 0)), ("max", (3, 3), (2, 2), (1, 1)), ("avg", (3, 3), (2, 2), (1, 1)),
+                                            ("avg", (2, 3), (1, 2), (0, 0)), ("max", (3, 3), (3, 2), (2, 0))):
+                want = cells_ref.pool_cell(x, kind, pool, stride, pad, maps=maps)
+                got = rt.Pool(kind, pool, stride, pad, maps=maps).forward(rt.DTensor.from_numpy(x, dt)).to_numpy()
+                assert got.shape == want.shape and np.array_equal(got, want.astype(np.int64)), (dt, kind, pool, maps.shape)
+
+
 def test_global_average_pool_bit_exact(rt):
     """Whole-input average window (the classifier head's pooling): negative sums must truncate toward zero."""
     from n2d2_amd import capi

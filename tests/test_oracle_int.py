@@ -230,6 +230,29 @@ def test_pool_max_and_average(pool, stride, pad):
         assert np.array_equal(av[:, :, oy, ox].astype(np.int64), want)
 
 
+def test_pool_with_a_connection_map_pools_over_the_connected_channels():
+    """PoolCell_Frame_Kernels.cpp:60-75,150-185 with a map: the maximum over window and connected channels; the sum over
+    both divided by window size x connected channels, truncated; 0 for an output nothing feeds."""
+    from oracle import cells
+    x = RNG.integers(-128, 256, size=(2, 6, 9, 8)).astype(np.float32)
+    xi = x.astype(np.int64)
+    maps = np.array([[1, 0, 1, 0], [1, 0, 0, 0], [1, 1, 0, 0], [1, 1, 0, 0], [1, 0, 0, 0], [1, 0, 1, 0]], dtype=np.uint8)   # [channel, output]
+    pool, stride, pad = (3, 3), (2, 2), (1, 1)
+    mx = cells.pool_cell(x, "max", pool, stride, pad, maps=maps)
+    av = cells.pool_cell(x, "avg", pool, stride, pad, maps=maps)
+    assert mx.shape == av.shape == (2, 4, 5, 4)
+    for oy, ox, o in itertools.product(range(5), range(4), range(4)):
+        y0, x0 = oy * 2 - 1, ox * 2 - 1
+        chans = np.flatnonzero(maps[:, o])
+        if len(chans) == 0:
+            assert not mx[:, o, oy, ox].any() and not av[:, o, oy, ox].any()
+            continue
+        win = xi[:, chans, max(y0, 0):min(y0 + 3, 9), max(x0, 0):min(x0 + 3, 8)]
+        assert np.array_equal(mx[:, o, oy, ox].astype(np.int64), win.max(axis=(1, 2, 3)))
+        s = win.sum(axis=(1, 2, 3))
+        assert np.array_equal(av[:, o, oy, ox].astype(np.int64), np.sign(s) * (np.abs(s) // (9 * len(chans))))
+
+
 def test_pool_cell_with_several_inputs_pools_every_input_on_its_own_channels():
     """PoolCell_Frame<T>::propagate (src/Cell/PoolCell_Frame.cpp:123-174) over several inputs, unit map over all their
     channels: window maxima / truncated window means of each input, written behind each other."""
