@@ -22,7 +22,7 @@ OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOT_QUANTIZED, ERR_WORKSPACE = ra
 # n2d2hip_conv_desc.kernel_choice bits
 KERNEL_NO_PIPE, KERNEL_NO_STEM, KERNEL_NO_HI16, KERNEL_NO_SUM16, KERNEL_TILE_M64, KERNEL_TILE_M128, KERNEL_F32_DIRECT, KERNEL_F32_GEMM = (
     1, 2, 4, 8, 16, 32, 64, 128)
-KERNEL_NO_PATCH, KERNEL_PATCH, KERNEL_NO_DIRECT, KERNEL_DIRECT = 256, 512, 1024, 2048
+KERNEL_NO_PATCH, KERNEL_PATCH, KERNEL_NO_DIRECT, KERNEL_DIRECT, KERNEL_TILE_M256 = 256, 512, 1024, 2048, 4096
 
 # every symbol include/n2d2hip.h declares
 SYMBOLS = [

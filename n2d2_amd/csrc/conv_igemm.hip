@@ -893,11 +893,10 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         // where it is the faster of the two (measured): at least two 64-channel steps per tile, so that a tile's rescale is
         // small beside its matrix instructions, and images large enough that the border positions it computes and drops
         // stay under a third of the work
-        // ... and enough 256-position tiles to give every CU a block (a small batch leaves the pipelined kernel's 128-pixel
-        // tiles the better fit)
+        // ... and enough tiles (of 128 positions, the kernel's smaller form) to give every CU a block
         && ((d.kernel_choice & N2D2HIP_KERNEL_PATCH)
             || (d.C >= 128 && (long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135
-                && (((long long)in->B * Hp * Wp + 255) / 256) * (d.O / (d.O % 128 == 0 ? 128 : 64)) >= num_cus()))) {
+                && (((long long)in->B * Hp * Wp + 127) / 128) * (d.O / (d.O % 128 == 0 ? 128 : 64)) >= num_cus()))) {
         // 3x3, stride 1, on an input that carries its padding: nine shifted reads of one patch of pixels
         ConvPatchArgs q = {};
         q.in = a.in; q.wfrag = c->d_wfrag; q.out = out->data;
@@ -911,7 +910,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.ta = c->d_epi_tab; q.tb = c->d_epi_tab + cp; q.tc = c->d_epi_tab + (hi16 ? 5 : 2) * cp;
         q.td = c->d_epi_tab + (hi16 ? 6 : 3) * cp; q.te = c->d_epi_tab + 4 * cp;
         q.lo = c->act->args.lo; q.hi = c->act->args.hi; q.preclamp = c->preclamp ? 1 : 0;
-        return conv_patch_launch(q, hi16, num_cus(), stream);
+        const int tile_m = (d.kernel_choice & N2D2HIP_KERNEL_TILE_M256) ? 256 : ((d.kernel_choice & N2D2HIP_KERNEL_TILE_M128) ? 128 : 0);
+        return conv_patch_launch(q, hi16, num_cus(), tile_m, stream);
     }
     if (pipe && (other || !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE))) {
         // persistent pipelined kernel: 2 blocks per CU, each walking pixel tiles of one channel tile

@@ -34,6 +34,7 @@ void conv_patch_weight_layout(const signed char* w, int C, int O, signed char* f
 // Can the kernel serve this shape (Wp = input columns with the border)?
 bool conv_patch_eligible(int C, int O, int Wp);
 // Launches the kernel; hi16 selects the scaled-up tables.  `blocks` is filled in (mtiles ... mlanes) here.
-int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, hipStream_t stream);
+// tile_m: positions per block tile, 128 or 256; 0 lets the launch choose by how many blocks the tensor gives the chip.
+int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipStream_t stream);
 
 } // namespace n2d2hip

@@ -762,7 +762,8 @@ def test_conv3x3_patch_kernel_bit_exact(rt):
     """3x3, stride 1, padding 1 on an input that carries its padding: the kernel that reads one patch of pixels at nine
     shifts (weights straight to registers in fragment order), against the oracle and against the pipelined kernel, over
     image sizes whose rows are shorter and longer than a tile, tiles that straddle images, channel counts that take the
-    two-wave and the four-wave block, several 64-channel steps, both epilogues, outputs with and without a border."""
+    two-wave and the four-wave block, tiles of 128 and of 256 positions, several 64-channel steps, both epilogues, outputs
+    with and without a border."""
     from n2d2_amd import capi
     from oracle import cells as cells_ref
     from oracle.cells import ActSpec
@@ -779,7 +780,9 @@ def test_conv3x3_patch_kernel_bit_exact(rt):
         dx = rt.DTensor.from_numpy(x, capi.U8B).with_halo(1)
         for spec in specs:
             want = cells_ref.conv_cell(x, w, bias, spec, pad=(1, 1, 1, 1)).astype(np.int64)
-            for choice in (capi.KERNEL_PATCH, capi.KERNEL_PATCH | capi.KERNEL_NO_HI16, 0, capi.KERNEL_NO_PATCH):
+            for choice in (capi.KERNEL_PATCH | capi.KERNEL_TILE_M256, capi.KERNEL_PATCH | capi.KERNEL_TILE_M128,
+                           capi.KERNEL_PATCH | capi.KERNEL_NO_HI16 | capi.KERNEL_TILE_M256, capi.KERNEL_PATCH | capi.KERNEL_NO_HI16 | capi.KERNEL_TILE_M128,
+                           capi.KERNEL_PATCH, 0, capi.KERNEL_NO_PATCH):
                 print("patch conv", (C, O, H, W, B), spec.mode, choice, flush=True)
                 conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, pad=(1, 1, 1, 1), kernel_choice=choice)
                 assert conv.accepts_halo()
