@@ -21,7 +21,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
 # inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
 TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
-                        "bytes_per_launch": 71944638, "launches_per_forward": 41,
+                        "bytes_per_launch": 72895459, "launches_per_forward": 39,
                         "note": "FETCH_SIZE + WRITE_SIZE, mean over the conv_pipe_kernel dispatches of 4 forwards, scaled by a 1 GiB copy; "
                                 "not measured by this run"}
 
@@ -351,8 +351,8 @@ def main():
              "int8_peak_at_that_clock_tops": round(256 * 8192 * mhz.value * 1e6 / 1e12, 1)}
 
     # Which kernel runs a launch of the forward (the library's own rules, restated here to label the figures):
-    # bottleneck_kernel (a residual block in one launch), conv_patch3x3_kernel (3x3, stride 1, at least 128 channels, on an
-    # input that carries its padding, images of at least 10 x 10), conv_stem_kernel (at most 4 input channels; it computes the max pooling behind it in the same launch),
+    # bottleneck_kernel (a residual block in one launch), conv_patch3x3_kernel (3x3, stride 1, on an
+    # input that carries its padding, images of at least 10 x 10, enough 128-position tiles for every CU), conv_stem_kernel (at most 4 input channels; it computes the max pooling behind it in the same launch),
     # conv_pipe_kernel (every other convolution / fully-connected cell with a multiple of 64 input channels, with the
     # residual sum in its epilogue where one follows), bandwidth kernels for the rest.
     def kernel_of(k):
@@ -370,8 +370,9 @@ def main():
             return "other"
         x = net._io[k][0][0]
         if (c.type == "conv" and l.name not in net.fused_sums and c.w.shape[2:] == (3, 3) and tuple(c.stride) == (1, 1) and tuple(c.pad) == (1, 1, 1, 1)
-                and tuple(c.dil) == (1, 1) and x.halo == 1 and c.w.shape[1] >= 128 and c.w.shape[0] % 64 == 0
-                and (x.H + 2) * (x.W + 2) * 100 <= x.H * x.W * 135):
+                and tuple(c.dil) == (1, 1) and x.halo == 1 and c.w.shape[0] % 64 == 0
+                and (x.H + 2) * (x.W + 2) * 100 <= x.H * x.W * 135
+                and ((x.B * (x.H + 2) * (x.W + 2) + 127) // 128) * (c.w.shape[0] // (128 if c.w.shape[0] % 128 == 0 else 64)) >= 256):
             return "conv_patch3x3_kernel"
         return "conv_pipe_kernel"
     kernels = [kernel_of(k) for k in range(len(net.launched))]

@@ -890,12 +890,11 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0) || pipe, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: tensor with a halo too large");
     if (pipe && !other && c->d_wfrag && in->halo == 1 && c->act->args.kind == EPI_I24 && c->bias_folded && is_byte_type(out->dtype)
         && conv_patch_eligible(d.C, d.O, Wp) && out_pixels * out->cs < (1ll << 31) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE)
-        // where it is the faster of the two (measured): at least two 64-channel steps per tile, so that a tile's rescale is
-        // small beside its matrix instructions, and images large enough that the border positions it computes and drops
+        // where it is the faster of the two (measured): images large enough that the border positions it computes and drops
         // stay under a third of the work
         // ... and enough tiles (of 128 positions, the kernel's smaller form) to give every CU a block
         && ((d.kernel_choice & N2D2HIP_KERNEL_PATCH)
-            || (d.C >= 128 && (long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135
+            || ((long long)Hp * Wp * 100 <= (long long)in->H * in->W * 135
                 && (((long long)in->B * Hp * Wp + 127) / 128) * (d.O / (d.O % 128 == 0 ? 128 : 64)) >= num_cus()))) {
         // 3x3, stride 1, on an input that carries its padding: nine shifted reads of one patch of pixels
         ConvPatchArgs q = {};
