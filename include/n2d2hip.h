@@ -167,7 +167,7 @@ enum {
     N2D2HIP_KERNEL_PATCH = 512,     /* the patch kernel wherever it can run, also where the library finds the pipelined one faster */
     N2D2HIP_KERNEL_NO_DIRECT = 1024,/* integer cells with at most 4 input channels and 32 outputs: matrix-core kernel instead of the direct one */
     N2D2HIP_KERNEL_DIRECT = 2048,   /* the direct kernel wherever it can run (up to 16 input channels), also where the library finds the matrix cores faster */
-    N2D2HIP_KERNEL_TILE_M256 = 4096 /* patch kernel: tiles of 256 positions (N2D2HIP_KERNEL_TILE_M128: of 128) instead of its own choice */
+    N2D2HIP_KERNEL_TILE_M256 = 4096 /* patch kernel: tiles of 256 positions (N2D2HIP_KERNEL_TILE_M128: of 128; _M64: four waves of 64 positions) instead of its own choice */
 };
 
 typedef struct n2d2hip_conv_s* n2d2hip_conv_t;

@@ -909,7 +909,8 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         q.ta = c->d_epi_tab; q.tb = c->d_epi_tab + cp; q.tc = c->d_epi_tab + (hi16 ? 5 : 2) * cp;
         q.td = c->d_epi_tab + (hi16 ? 6 : 3) * cp; q.te = c->d_epi_tab + 4 * cp;
         q.lo = c->act->args.lo; q.hi = c->act->args.hi; q.preclamp = c->preclamp ? 1 : 0;
-        const int tile_m = (d.kernel_choice & N2D2HIP_KERNEL_TILE_M256) ? 256 : ((d.kernel_choice & N2D2HIP_KERNEL_TILE_M128) ? 128 : 0);
+        const int tile_m = (d.kernel_choice & N2D2HIP_KERNEL_TILE_M256) ? 256 : ((d.kernel_choice & N2D2HIP_KERNEL_TILE_M128) ? 128
+            : ((d.kernel_choice & N2D2HIP_KERNEL_TILE_M64) ? 64 : 0));
         return conv_patch_launch(q, hi16, num_cus(), tile_m, stream);
     }
     if (pipe && (other || !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE))) {

@@ -388,21 +388,29 @@ int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipSt
 {
     N2D2HIP_REQUIRE(conv_patch_eligible(a.C, a.O, a.Wp), N2D2HIP_ERR_INVALID, "conv_patch: shape not served");
     N2D2HIP_REQUIRE((long long)a.total * a.C < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "conv_patch: tensor too large");
-    N2D2HIP_REQUIRE(tile_m == 0 || tile_m == 128 || tile_m == 256, N2D2HIP_ERR_INVALID, "conv_patch: tiles of 128 or 256 positions");
-    const bool wide = a.O % 128 == 0;                 // 2 x 2 waves, 128 channels per block; else 2 x 1 waves, 64 channels
-    const int BN = wide ? 128 : 64, NW = wide ? 4 : 2;
+    N2D2HIP_REQUIRE(tile_m == 0 || tile_m == 64 || tile_m == 128 || tile_m == 256, N2D2HIP_ERR_INVALID, "conv_patch: tile choice %d", tile_m);
+    const bool wide = a.O % 128 == 0;                 // 128 channels per block (2 x 2 waves); else 64 channels
+    const int BN = wide ? 128 : 64;
     a.nchunk = a.C / 64;
     a.ntiles_n = a.O / BN;
-    // blocks per CU: two of four waves, three of two (LDS: at most 49 KB + tables per block)
-    const int slots = (wide ? 2 : 3) * num_cus;
-    // Tiles of 256 positions re-read less of their neighbours' rows and stream the weights half as often (measured: 20.2
-    // against 21.4 us for 256 -> 256 channels on 14x14 at batch 128, one block per CU either way); tiles of 128 positions
-    // where the larger ones would leave CUs without a block (12.4 against 16.8 us for the same layer at batch 64).
-    // With 64 input channels a tile is one channel step: the small tiles, whose rescale overlaps other blocks' matrix
-    // instructions better (15.6 against 18.8 us for 64 -> 64 channels on 56x56 at batch 64).
-    const int BM = tile_m ? tile_m : (((a.total + 255) / 256 * a.ntiles_n < num_cus || a.C < 128) ? 128 : 256);
+    // The forms of the kernel.  Tiles of 256 positions, a wave on 128 of them, re-read less of their neighbours' rows and
+    // stream the weights half as often (20.2 against 21.4 us for 256 -> 256 channels on 14x14 at batch 128, one block per
+    // CU either way).  Tiles of 128 positions, a wave on 64, where the larger ones would leave CUs without a block (12.4
+    // against 16.8 us for the same layer at batch 64).  With 64 input channels a tile is one channel step and the waves of
+    // 64 positions win (64 -> 64 channels on 56x56: 15.0 against 18.9 us at batch 64); four of them on a tile of 256 share
+    // more of the patch than two on a tile of 128 (23.0 against 26.6 us at batch 128).
+    enum Form { M256, M128, M256_WAVES4 };
+    const bool few = (a.total + 255) / 256 * a.ntiles_n < num_cus;
+    Form form = few ? M128 : (a.C < 128 ? (wide ? M128 : M256_WAVES4) : M256);
+    if (tile_m == 256) form = M256;
+    if (tile_m == 128) form = M128;
+    if (tile_m == 64) form = wide ? M128 : M256_WAVES4;
+    const int BM = form == M128 ? 128 : 256;
+    const int NW = (wide || form == M256_WAVES4) ? 4 : 2;
     const int chunks = (BM + 2 * a.Wp + 2 + 15) / 16;
     const int npl = (chunks + NW - 1) / NW;
+    // blocks per CU: two of four waves, three of two (LDS: at most 49 KB + tables per block)
+    const int slots = (NW == 4 ? 2 : 3) * num_cus;
     a.mtiles = (a.total + BM - 1) / BM;
     const int per_xcd = std::max(1, std::min((a.mtiles + 7) / 8, slots / (8 * a.ntiles_n)));
     a.mlanes = per_xcd;
@@ -415,7 +423,10 @@ int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipSt
         a.prof = (long long*)strtoull(pp, nullptr, 16);
     }
 #endif
-    if (BM == 256) {
+    // patch rows: at most 384 (tiles of 256) or 256 (tiles of 128) wherever the kernel is eligible
+    if (form == M256_WAVES4) {
+        launch<4, 1, 6, 2>(a, hi16, grid, stream);
+    } else if (form == M256) {
         if (wide) {
             if (npl <= 5) launch<2, 2, 5, 4>(a, hi16, grid, stream);
             else launch<2, 2, 6, 4>(a, hi16, grid, stream);
@@ -423,7 +434,7 @@ int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipSt
             if (npl <= 10) launch<2, 1, 10, 4>(a, hi16, grid, stream);
             else launch<2, 1, 12, 4>(a, hi16, grid, stream);
         }
-    } else {            // 128 + 2 Wp + 2 <= 256 rows wherever the kernel is eligible
+    } else {
         if (wide) {
             if (npl <= 3) launch<2, 2, 3, 2>(a, hi16, grid, stream);
             else launch<2, 2, 4, 2>(a, hi16, grid, stream);

@@ -34,7 +34,8 @@ void conv_patch_weight_layout(const signed char* w, int C, int O, signed char* f
 // Can the kernel serve this shape (Wp = input columns with the border)?
 bool conv_patch_eligible(int C, int O, int Wp);
 // Launches the kernel; hi16 selects the scaled-up tables.  `blocks` is filled in (mtiles ... mlanes) here.
-// tile_m: positions per block tile, 128 or 256; 0 lets the launch choose by how many blocks the tensor gives the chip.
+// tile_m: positions per block tile, 128 or 256, or 64 for four waves of 64 positions per block (a tile of 256 for layers of 64
+// outputs per block); 0 lets the launch choose by the layer's channels and by how many blocks the tensor gives the chip.
 int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipStream_t stream);
 
 } // namespace n2d2hip

@@ -780,7 +780,7 @@ def test_conv3x3_patch_kernel_bit_exact(rt):
         dx = rt.DTensor.from_numpy(x, capi.U8B).with_halo(1)
         for spec in specs:
             want = cells_ref.conv_cell(x, w, bias, spec, pad=(1, 1, 1, 1)).astype(np.int64)
-            for choice in (capi.KERNEL_PATCH | capi.KERNEL_TILE_M256, capi.KERNEL_PATCH | capi.KERNEL_TILE_M128,
+            for choice in (capi.KERNEL_PATCH | capi.KERNEL_TILE_M256, capi.KERNEL_PATCH | capi.KERNEL_TILE_M128, capi.KERNEL_PATCH | capi.KERNEL_TILE_M64,
                            capi.KERNEL_PATCH | capi.KERNEL_NO_HI16 | capi.KERNEL_TILE_M256, capi.KERNEL_PATCH | capi.KERNEL_NO_HI16 | capi.KERNEL_TILE_M128,
                            capi.KERNEL_PATCH, 0, capi.KERNEL_NO_PATCH):
                 print("patch conv", (C, O, H, W, B), spec.mode, choice, flush=True)
