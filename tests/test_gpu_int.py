@@ -524,6 +524,21 @@ def test_pool_cell_with_a_connection_map_bit_exact(rt):
                 assert got.shape == want.shape and np.array_equal(got, want.astype(np.int64)), (dt, kind, pool, maps.shape)
 
 
+def test_pool_with_a_connection_map_refuses_tensors_that_do_not_fit(rt):
+    from n2d2_amd import capi
+    x = rt.DTensor.from_numpy(_u8((2, 6, 8, 8)), capi.U8B)
+    pool = rt.Pool("max", (2, 2), (2, 2), maps=np.ones((6, 3), dtype=np.uint8))
+    assert pool.forward(x).to_numpy().shape == (2, 3, 4, 4)
+    with pytest.raises(capi.N2D2HipError, match="expected"):              # output of the wrong size
+        pool.forward(x, rt.DTensor(2, 3, 5, 4, capi.U8B))
+    with pytest.raises(capi.N2D2HipError, match="one dtype"):             # output of another storage type
+        pool.forward(x, rt.DTensor(2, 3, 4, 4, capi.I8))
+    with pytest.raises(ValueError, match="the map is"):                   # a map for another number of channels
+        rt.Pool("max", (2, 2), (2, 2), maps=np.ones((5, 3), dtype=np.uint8)).forward(x)
+    with pytest.raises(capi.N2D2HipError, match="null descriptor or map"):
+        capi.check(rt.lib.n2d2hip_pool_forward_mapped(rt.C.byref(pool.desc), None, x.ref, pool.make_output(x).ref, rt.stream_ptr()))
+
+
 def test_global_average_pool_bit_exact(rt):
     """Whole-input average window (the classifier head's pooling): negative sums must truncate toward zero."""
     from n2d2_amd import capi
