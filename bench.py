@@ -259,6 +259,80 @@ def qat_batchnorm_step(torch, steps=10):
             "finite": bool(torch.isfinite(y).all().item() and torch.isfinite(dx).all().item())}
 
 
+def kernel_phases(torch, config, batch):
+    """Where the time of a launch goes inside the kernel, per instantiation, from the probes of a library built with
+    `python -m n2d2_amd.build --probe` (run with N2D2HIP_LIB=n2d2_amd/lib/libn2d2hip_probe.so): every work-group of the
+    convolution kernels records its shader clock at its first instruction, at its first operand load, when its first ring
+    stage has landed, and at its end, the clocks its epilogues took, and the constant 100 MHz counter at both ends
+    (include/n2d2hip_probe.h).  One forward is probed after three warm ones; prints a text table."""
+    import ctypes as C
+    import numpy as np
+    from n2d2_amd import capi, nets
+    if not hasattr(capi.lib, "n2d2hip_probe_begin"):
+        print("bench.py --kernel-phases needs the probe build: python -m n2d2_amd.build --probe, then "
+              "N2D2HIP_LIB=n2d2_amd/lib/libn2d2hip_probe.so python bench.py --kernel-phases", file=sys.stderr)
+        sys.exit(5)
+    capi.lib.n2d2hip_probe_begin.argtypes = [C.c_void_p, C.c_size_t]
+    capi.lib.n2d2hip_probe_end.argtypes = [C.c_void_p]
+    make, default_batch = CONFIGS[config]
+    spec = getattr(nets, make)()
+    B = batch or default_batch
+    net = nets.GpuNet(spec, B)
+    net.set_input(np.random.default_rng(2025).integers(0, 256, size=(B,) + tuple(spec.in_shape)))
+    for _ in range(3):
+        net.forward()
+    torch.cuda.synchronize()
+    REC = 16
+    buf = torch.zeros(REC * 65536, dtype=torch.int64, device="cuda")
+    capi.check(capi.lib.n2d2hip_probe_begin(buf.data_ptr(), buf.numel() * 8))
+    launches = []
+    for k, ((l, cell, fn), (ins, out)) in enumerate(zip(net.steps, net._io)):
+        with capi.launch_log() as log:
+            fn(cell, ins, out)
+        launches += [(l.name,) + e for e in log.entries]
+    torch.cuda.synchronize()
+    capi.check(capi.lib.n2d2hip_probe_end(None))
+    rec = buf.cpu().numpy().reshape(-1, REC).astype(np.float64)
+    rows = {}
+    for lname, kname, grid, block, slot in launches:
+        if slot < 0:
+            continue
+        r = rec[slot:slot + grid]
+        r = r[(r[:, 5] != 0) & (r[:, 7] > 0)]     # work-groups that had work
+        if len(r) == 0:
+            continue
+        w0, w1 = r[:, 5], r[:, 6]
+        span_us = (w1.max() - w0.min()) / 100.0
+        mhz = ((r[:, 3] - r[:, 0]).sum() / ((w1 - w0).sum() / 100.0))        # shader clocks per microsecond
+        has12 = r[:, 2].max() > 0
+        d = {"launches": 1, "blocks": len(r), "span_us": span_us,
+             "start_spread_us": (w0.max() - w0.min()) / 100.0,
+             "to_first_load_us": float(np.mean(r[:, 1] - r[:, 0]) / mhz) if has12 else float("nan"),
+             "to_first_mfma_us": float(np.mean(r[:, 2] - r[:, 0]) / mhz) if has12 else float("nan"),
+             "block_life_us": float(np.mean(w1 - w0) / 100.0),
+             "epilogue_us": float(np.mean(r[:, 4]) / mhz),
+             "per_unit_us": float(np.mean((r[:, 3] - (r[:, 2] if has12 else r[:, 0])) / np.maximum(r[:, 7], 1)) / mhz),
+             "units": float(np.mean(r[:, 7])),
+             "end_spread_us": (w1.max() - w1.min()) / 100.0,
+             "idle_frac": 1.0 - float((w1 - w0).sum() / 100.0) / (span_us * len(r)),
+             "mhz": mhz}
+        a = rows.setdefault(kname, [])
+        a.append(d)
+    keys = ["blocks", "span_us", "start_spread_us", "to_first_load_us", "to_first_mfma_us", "block_life_us", "units", "per_unit_us",
+            "epilogue_us", "end_spread_us", "idle_frac", "mhz"]
+    print("%s, batch %d: in-kernel phases per instantiation (mean over its launches of one forward; times in us)" % (config, B))
+    print("span = first work-group's start to last work-group's end; start_spread = last start - first start; to_first_load /"
+          " to_first_mfma = from a work-group's first instruction (mean over work-groups); block_life = a work-group's start to"
+          " its end; units = ring steps (tiles for the bottleneck kernel) per work-group; per_unit = (end - first mfma) / units;"
+          " epilogue = clocks in epilogues per work-group; end_spread = last end - first end; idle_frac = 1 - sum of work-group"
+          " lives / (span x work-groups); mhz = shader clocks per microsecond inside the kernel")
+    print("%-64s %3s " % ("kernel", "n") + " ".join("%12s" % k[:12] for k in keys))
+    for kname, lst in sorted(rows.items(), key=lambda kv: -sum(d["span_us"] for d in kv[1])):
+        print("%-64s %3d " % (kname[:64], len(lst)) + " ".join("%12.2f" % float(np.nanmean([d[k] for d in lst])) for k in keys))
+    total = sum(d["span_us"] for lst in rows.values() for d in lst)
+    print("sum of spans of the probed launches: %.1f us (%d launches of %d in the forward)" % (total, sum(len(v) for v in rows.values()), len(launches)))
+
+
 # name -> (constructor in n2d2_amd.nets, benchmark batch)
 CONFIGS = {"resnet50": ("resnet50", 128), "lenet": ("lenet", 256), "resnet18_stage_conv": ("single_conv_stage", 64),
            "mobilenet_v1": ("mobilenet_v1", 64), "resnet18_w4a4": ("resnet18_w4a4", 64)}
@@ -280,6 +354,9 @@ def main():
                     help="profiling runs: time the forward of --config and stop (no per-kernel replays, no side figures)")
     ap.add_argument("--config", default="resnet50", choices=sorted(CONFIGS),
                     help="with --forward-only: which configuration's forward to run (at its benchmark batch unless --batch is given)")
+    ap.add_argument("--kernel-phases", action="store_true",
+                    help="probe build only (python -m n2d2_amd.build --probe; N2D2HIP_LIB=n2d2_amd/lib/libn2d2hip_probe.so): "
+                         "print where the time goes inside the convolution kernels of --config, per instantiation, and stop")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 1 GiB device-to-device copy first (known traffic, to scale FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -301,6 +378,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.kernel_phases:
+        kernel_phases(torch, args.config, args.batch)
+        return
     import math
     per_graph = math.gcd(max(args.forwards_per_graph, 1), args.steps)
     if args.forward_only:
@@ -350,31 +430,14 @@ def main():
     clock = {"engine_clock_mhz_under_mfma_load": round(mhz.value, 1),
              "int8_peak_at_that_clock_tops": round(256 * 8192 * mhz.value * 1e6 / 1e12, 1)}
 
-    # Which kernel runs a launch of the forward (the library's own rules, restated here to label the figures):
-    # bottleneck_kernel (a residual block in one launch), conv_patch3x3_kernel (3x3, stride 1, on an
-    # input that carries its padding, images of at least 10 x 10, enough 128-position tiles for every CU), conv_stem_kernel (at most 4 input channels; it computes the max pooling behind it in the same launch),
-    # conv_pipe_kernel (every other convolution / fully-connected cell with a multiple of 64 input channels, with the
-    # residual sum in its epilogue where one follows), bandwidth kernels for the rest.
+    # Which kernel runs a launch of the forward: asked of the library (its launch log names what every cell launched), so
+    # the labels below cannot drift from what ran.
+    launched_kernels = net.kernel_names()
+
     def kernel_of(k):
-        l = net.launched[k]
-        if l.name in net.bottlenecks:
-            return "bottleneck_kernel"
-        if l.name in net.stem_pools:
-            return "conv_stem_kernel"
-        c = net.fused_sums[l.name][1] if l.name in net.fused_sums else l
-        if c.type not in ("conv", "fc"):
-            return "bandwidth"
-        if c.type == "conv" and c.w.shape[1] <= 4:
-            return "conv_stem_kernel"
-        if getattr(c, "groups", 1) != 1 or c.weight_bits != 8 or c.w.shape[1] % 64 != 0:
-            return "other"
-        x = net._io[k][0][0]
-        if (c.type == "conv" and l.name not in net.fused_sums and c.w.shape[2:] == (3, 3) and tuple(c.stride) == (1, 1) and tuple(c.pad) == (1, 1, 1, 1)
-                and tuple(c.dil) == (1, 1) and x.halo == 1 and c.w.shape[0] % 64 == 0
-                and (x.H + 2) * (x.W + 2) * 100 <= x.H * x.W * 135
-                and ((x.B * (x.H + 2) * (x.W + 2) + 127) // 128) * (c.w.shape[0] // (128 if c.w.shape[0] % 128 == 0 else 64)) >= 256):
-            return "conv_patch3x3_kernel"
-        return "conv_pipe_kernel"
+        # the last kernel a cell launches does its arithmetic (a cell with several inputs gathers them first)
+        name = launched_kernels[k][-1].split("<")[0]
+        return name if name.startswith("conv_") or name.startswith("bottleneck") else "bandwidth"
     kernels = [kernel_of(k) for k in range(len(net.launched))]
 
     # Dominant kernel: conv_pipe_kernel.  Its launches are replayed alone, back to back, between two events on the launch

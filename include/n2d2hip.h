@@ -45,6 +45,15 @@ const char* n2d2hip_version(void);
  * Allocates a small device buffer and waits for the stream. */
 int n2d2hip_measure_clock(double busy_microseconds, double* mhz, n2d2hip_stream_t stream);
 
+/* Diagnostic, no counterpart in the reference: the launch log of the calling thread.  Between _begin and _end every kernel
+ * the library launches from this thread is recorded (the launches still happen); afterwards _entry gives launch `index`:
+ * the kernel's name with its template arguments ("conv_pipe_kernel<4, 128, ...>", truncated to `capacity`), its grid
+ * and block sizes in threads-groups / threads, and the index of its first record in a probe buffer (-1 outside probe builds,
+ * see n2d2hip_probe.h).  It is how a caller learns which kernel a cell runs on without restating the library's choice. */
+int n2d2hip_launch_log_begin(void);
+int n2d2hip_launch_log_end(int* count);
+int n2d2hip_launch_log_entry(int index, char* name, size_t capacity, int* grid, int* block, long long* probe_slot);
+
 /* --------------------------------------------------------------- tensors */
 /* Element types.  N2D2 holds integer values in float storage
  * (ref: src/Cell/ConvCell_Frame.cpp:28-44); here they are stored narrow. */
@@ -60,7 +69,19 @@ enum {
  * (ref: include/containers/Tensor.hpp:162-193).  NHWC is the private
  * channel-inner order used between Frame_HIP cells; its channel stride `cs`
  * is a multiple of 16 (4 is accepted for network inputs with <= 4 channels). */
-enum { N2D2HIP_NCHW = 0, N2D2HIP_NHWC = 1 };
+enum {
+    N2D2HIP_NCHW = 0,
+    N2D2HIP_NHWC = 1,
+    /* Space-to-depth form of a network input with at most 4 channels, read by first-layer convolutions of stride 2
+     * (n2d2hip_conv_s2d_halo): pixel (Y, X) of the stored image is 16 bytes, the 2 x 2 block of input pixels
+     * (2Y + dy, 2X + dx) with 4 channel slots each, byte (dy * 2 + dx) * 4 + channel; an image is stored as
+     * (ceil(H/2) + 2*halo) x (ceil(W/2) + 2*halo) such pixels.  Whatever lies outside the H x W input (the border, an odd
+     * last row / column, the channel slots past C) holds the storage form of 0.  B, C, H, W stay the logical shape, cs is
+     * 16.  Only n2d2hip_convert writes it (border included, so no n2d2hip_tensor_clear is needed) and only
+     * n2d2hip_conv_forward / n2d2hip_conv_forward_maxpool read it.  No counterpart in the reference, whose first layer
+     * reads the float NCHW stimuli directly. */
+    N2D2HIP_S2D = 2
+};
 
 typedef struct n2d2hip_tensor {
     void* data;
@@ -187,6 +208,16 @@ int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH
  * may have a halo if n2d2hip_conv_accepts_halo says so. */
 int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
+/* Border (halo) a space-to-depth input of logical size H x W must carry for this convolution to read it
+ * (n2d2hip_conv_forward then takes `in` with layout N2D2HIP_S2D; with `pool` non-null the question is about
+ * n2d2hip_conv_forward_maxpool with that pooling behind the convolution), or -1 when it is not served that way.
+ * Served: at most 4 input channels, 8-bit weights, a square kernel of 3, 5 or 7, stride 2, no dilation, at most 64
+ * outputs, integer rescale to bytes, bordered rows of at most 128 pixels; with a pooling, what
+ * n2d2hip_conv_accepts_maxpool asks and rows of at most 112 outputs.  No counterpart in the reference: the stride-2
+ * K x K window becomes a stride-1 window of ceil(K / 2)^2 16-byte pixels whose padding is the border of stored zeros
+ * (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83 skips those taps). */
+struct n2d2hip_pool_desc;
+int n2d2hip_conv_s2d_halo(n2d2hip_conv_t conv, const struct n2d2hip_pool_desc* pool, int H, int W);
 /* 1 if this convolution runs on the kernel that reads and writes tensors with a halo (8-bit weights, ungrouped, input
  * channels a multiple of 64), else 0.  No counterpart in the reference, whose padding is implicit in its tap loop. */
 int n2d2hip_conv_accepts_halo(n2d2hip_conv_t conv);

@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libn2d2hip.so")
 GLUE_LIB = os.path.join(LIBDIR, "libn2d2_frame_hip.so")
-SOURCES = ["act.hip", "conv_igemm.hip", "conv_patch.hip", "conv_pipe_w4.hip", "bottleneck.hip", "expand_reduce.hip", "depthwise.hip", "dw_pw.hip", "conv_small.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip", "diag.hip"]
+SOURCES = ["act.hip", "conv_igemm.hip", "conv_patch.hip", "conv_s2d.hip", "conv_pipe_w4.hip", "bottleneck.hip", "expand_reduce.hip", "depthwise.hip", "dw_pw.hip", "conv_small.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip", "diag.hip"]
 
 # -ffp-contract=off: float rescales must round the product and the sum
 # separately, as the reference (built for baseline x86-64) does.
@@ -30,6 +30,32 @@ def _run(cmd):
     if r.returncode != 0:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
     return out
+
+
+PROBE_LIB = os.path.join(LIBDIR, "libn2d2hip_probe.so")
+
+
+def build_probe(verbose=False):
+    """The same library with in-kernel phase probes (-DN2D2HIP_PROFILE, include/n2d2hip_probe.h) as
+    lib/libn2d2hip_probe.so.  A measuring tool: N2D2HIP_LIB=<that file> selects it, bench.py --kernel-phases reads it."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    objdir = os.path.join(LIBDIR, "obj_probe")
+    os.makedirs(objdir, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        return _run([hipcc] + HIPCC_FLAGS + ["-DN2D2HIP_PROFILE", "-c", os.path.join(CSRC, src), "-o", obj])
+
+    with ThreadPoolExecutor(max_workers=6) as ex:
+        outs = list(ex.map(compile_one, zip(SOURCES, objs)))
+    outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB] + objs))
+    if verbose:
+        for o in outs:
+            if o.strip():
+                print(o)
+    return PROBE_LIB
 
 
 def build(verbose=False):
@@ -63,4 +89,4 @@ def build(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build_probe(verbose=True) if "--probe" in sys.argv[1:] else build(verbose=True))

@@ -12,7 +12,7 @@ LIB_PATH = os.environ.get("N2D2HIP_LIB") or os.path.join(_HERE, "lib", "libn2d2h
 
 # enums of n2d2hip.h
 U8, I8, I32, F32, U8B = 0, 1, 2, 3, 4
-NCHW, NHWC = 0, 1
+NCHW, NHWC, S2D = 0, 1, 2
 SCALING_NONE, SCALING_FLOAT_MULT, SCALING_FIXED_MULT16, SCALING_FIXED_MULT32, SCALING_SINGLE_SHIFT, SCALING_DOUBLE_SHIFT = range(6)
 ACT_LINEAR, ACT_RECTIFIER = 0, 1
 POOL_MAX, POOL_AVERAGE = 0, 1
@@ -26,9 +26,10 @@ KERNEL_NO_PATCH, KERNEL_PATCH, KERNEL_NO_DIRECT, KERNEL_DIRECT, KERNEL_TILE_M256
 
 # every symbol include/n2d2hip.h declares
 SYMBOLS = [
-    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_measure_clock", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
+    "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_measure_clock",
+    "n2d2hip_launch_log_begin", "n2d2hip_launch_log_end", "n2d2hip_launch_log_entry", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
-    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_accepts_halo",
+    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_s2d_halo", "n2d2hip_conv_accepts_halo",
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", "n2d2hip_expand_reduce_create", "n2d2hip_expand_reduce_destroy", "n2d2hip_expand_reduce_forward",
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
@@ -90,6 +91,8 @@ def load():
     P, I, F, SZ, U = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
     lib.n2d2hip_convert.argtypes = [P, P, P]
     lib.n2d2hip_measure_clock.argtypes = [C.c_double, P, P]
+    lib.n2d2hip_launch_log_end.argtypes = [P]
+    lib.n2d2hip_launch_log_entry.argtypes = [I, P, SZ, P, P, P]
     lib.n2d2hip_act_create.argtypes = [P, I, P]
     lib.n2d2hip_act_destroy.argtypes = [P]
     lib.n2d2hip_scaling_forward.argtypes = [P, P, P, P]
@@ -98,6 +101,7 @@ def load():
     lib.n2d2hip_conv_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_conv_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_conv_accepts_halo.argtypes = [P]
+    lib.n2d2hip_conv_s2d_halo.argtypes = [P, P, I, I]
     lib.n2d2hip_tensor_clear.argtypes = [P, P]
     lib.n2d2hip_conv_fuse_sum.argtypes = [P, P, I, I]
     lib.n2d2hip_concat_channels.argtypes = [I, P, P, P]
@@ -165,6 +169,26 @@ def check(status):
     if status != OK:
         msg = lib.n2d2hip_last_error().decode() or lib.n2d2hip_strerror(status).decode()
         raise N2D2HipError(status, msg)
+
+
+class launch_log(object):
+    """with capi.launch_log() as log: ...; log.entries is then [(kernel name, grid, block, first probe record or -1)] of
+    the kernels the library launched from this thread inside the block."""
+
+    def __enter__(self):
+        self.entries = []
+        check(lib.n2d2hip_launch_log_begin())
+        return self
+
+    def __exit__(self, *exc):
+        n = C.c_int(0)
+        check(lib.n2d2hip_launch_log_end(C.byref(n)))
+        for i in range(n.value):
+            name = C.create_string_buffer(256)
+            grid, block, slot = C.c_int(0), C.c_int(0), C.c_longlong(-1)
+            check(lib.n2d2hip_launch_log_entry(i, name, 256, C.byref(grid), C.byref(block), C.byref(slot)))
+            self.entries.append((name.value.decode(), grid.value, block.value, slot.value))
+        return False
 
 
 def nhwc_cs(c):

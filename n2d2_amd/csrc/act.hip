@@ -21,18 +21,51 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
-int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok)
+// ---- launch log of the calling thread
+struct LaunchRecord {
+    std::string name;
+    unsigned grid, block;
+    long long slot;
+};
+static thread_local bool g_log_open = false;
+static thread_local std::vector<LaunchRecord> g_log;
+
+void launch_log_add(const char* pretty, unsigned grid, unsigned block, long long slot)
+{
+    if (!g_log_open)
+        return;
+    // "... [K = &n2d2hip::kernel<args>]" -> "kernel<args>"
+    std::string name(pretty);
+    const size_t eq = name.find("K = ");
+    if (eq != std::string::npos) {
+        name = name.substr(eq + 4);
+        if (!name.empty() && name.back() == ']') name.pop_back();
+        if (!name.empty() && name[0] == '&') name.erase(0, 1);
+        if (!name.empty() && name[0] == '(') { name.erase(0, 1); if (!name.empty() && name.back() == ')') name.pop_back(); }
+        for (size_t at; (at = name.find("n2d2hip::")) != std::string::npos;) name.erase(at, 9);
+    }
+    g_log.push_back(LaunchRecord{name, grid, block, slot});
+}
+
+int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok, bool s2d_ok)
 {
     N2D2HIP_REQUIRE(t != nullptr, N2D2HIP_ERR_INVALID, "%s: null tensor descriptor", what);
     N2D2HIP_REQUIRE(t->data != nullptr, N2D2HIP_ERR_INVALID, "%s: null data pointer", what);
     N2D2HIP_REQUIRE(t->dtype >= N2D2HIP_U8 && t->dtype <= N2D2HIP_U8B, N2D2HIP_ERR_INVALID, "%s: bad dtype %d", what, t->dtype);
-    N2D2HIP_REQUIRE(t->layout == N2D2HIP_NCHW || t->layout == N2D2HIP_NHWC, N2D2HIP_ERR_INVALID, "%s: bad layout %d", what, t->layout);
+    N2D2HIP_REQUIRE(t->layout == N2D2HIP_NCHW || t->layout == N2D2HIP_NHWC || t->layout == N2D2HIP_S2D, N2D2HIP_ERR_INVALID,
+                    "%s: bad layout %d", what, t->layout);
     N2D2HIP_REQUIRE(t->B > 0 && t->C > 0 && t->H > 0 && t->W > 0, N2D2HIP_ERR_INVALID,
                     "%s: empty tensor %dx%dx%dx%d", what, t->B, t->C, t->H, t->W);
     if (t->layout == N2D2HIP_NHWC)
         N2D2HIP_REQUIRE(t->cs >= t->C && (t->cs % 16 == 0 || t->cs == 4), N2D2HIP_ERR_INVALID,
                         "%s: NHWC channel stride %d invalid for %d channels (multiple of 16, or 4)", what, t->cs, t->C);
     N2D2HIP_REQUIRE(t->halo >= 0 && t->halo <= 16, N2D2HIP_ERR_INVALID, "%s: halo %d", what, t->halo);
+    if (t->layout == N2D2HIP_S2D) {
+        N2D2HIP_REQUIRE(s2d_ok, N2D2HIP_ERR_UNSUPPORTED, "%s: space-to-depth tensors are not accepted here", what);
+        N2D2HIP_REQUIRE(t->C <= 4 && t->cs == 16 && elem_size(t->dtype) == 1, N2D2HIP_ERR_INVALID,
+                        "%s: a space-to-depth tensor has at most 4 channels of bytes and 16-byte pixels (cs 16)", what);
+        return N2D2HIP_OK;
+    }
     if (t->halo > 0) {
         N2D2HIP_REQUIRE(halo_ok, N2D2HIP_ERR_UNSUPPORTED, "%s: tensors with a halo are not accepted here", what);
         N2D2HIP_REQUIRE(t->layout == N2D2HIP_NHWC && elem_size(t->dtype) == 1, N2D2HIP_ERR_INVALID,
@@ -108,11 +141,45 @@ const char* n2d2hip_last_error(void) { return g_last_error.c_str(); }
 
 const char* n2d2hip_version(void) { return "n2d2hip 0.1 (gfx950)"; }
 
+int n2d2hip_launch_log_begin(void)
+{
+    g_log.clear();
+    g_log_open = true;
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_launch_log_end(int* count)
+{
+    N2D2HIP_REQUIRE(g_log_open, N2D2HIP_ERR_INVALID, "launch_log_end: no log is open on this thread");
+    g_log_open = false;
+    if (count) *count = (int)g_log.size();
+    return N2D2HIP_OK;
+}
+
+int n2d2hip_launch_log_entry(int index, char* name, size_t capacity, int* grid, int* block, long long* probe_slot)
+{
+    N2D2HIP_REQUIRE(!g_log_open, N2D2HIP_ERR_INVALID, "launch_log_entry: the log is still open");
+    N2D2HIP_REQUIRE(index >= 0 && (size_t)index < g_log.size(), N2D2HIP_ERR_INVALID, "launch_log_entry: index %d of %zu entries", index,
+                    g_log.size());
+    const LaunchRecord& r = g_log[(size_t)index];
+    if (name && capacity > 0) {
+        const size_t n = std::min(capacity - 1, r.name.size());
+        memcpy(name, r.name.data(), n);
+        name[n] = 0;
+    }
+    if (grid) *grid = (int)r.grid;
+    if (block) *block = (int)r.block;
+    if (probe_slot) *probe_slot = r.slot;
+    return N2D2HIP_OK;
+}
+
 int n2d2hip_nhwc_cs(int C) { return C <= 4 ? 4 : round_up(C, 16); }
 
 size_t n2d2hip_tensor_bytes(const n2d2hip_tensor* t)
 {
     if (!t) return 0;
+    if (t->layout == N2D2HIP_S2D)
+        return (size_t)t->B * ((t->H + 1) / 2 + 2 * t->halo) * ((t->W + 1) / 2 + 2 * t->halo) * 16;
     const size_t c = (t->layout == N2D2HIP_NHWC) ? (size_t)t->cs : (size_t)t->C;
     return (size_t)t->B * (t->H + 2 * t->halo) * (t->W + 2 * t->halo) * c * (size_t)elem_size(t->dtype);
 }
@@ -134,11 +201,73 @@ int n2d2hip_tensor_clear(const n2d2hip_tensor* t, n2d2hip_stream_t stream)
                     "tensor_clear: NHWC byte tensors with a channel stride that is a multiple of 16");
     const size_t n16 = n2d2hip_tensor_bytes(t) / 16;
     const size_t blocks = std::min<size_t>((n16 + 255) / 256, 256 * 32);
-    hipLaunchKernelGGL(fill_bytes_kernel, dim3((unsigned)std::max<size_t>(blocks, 1)), dim3(256), 0, (hipStream_t)stream, (uint4*)t->data, n16,
+    N2D2HIP_LAUNCH(fill_bytes_kernel, dim3((unsigned)std::max<size_t>(blocks, 1)), dim3(256), 0, (hipStream_t)stream, (uint4*)t->data, n16,
                        t->dtype == N2D2HIP_U8B ? 0x80808080u : 0u);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
+
+namespace n2d2hip {
+// Graph-edge conversion into the space-to-depth form: a thread writes two neighbouring 16-byte pixels of the stored image
+// (32 bytes), border and empty channel slots included; it reads, per channel and input row, the four input pixels they
+// hold, which for an NCHW source are contiguous bytes that neighbouring threads continue.
+__global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in, int in_dtype, int in_layout, int in_cs, int in_halo,
+                                                     signed char* __restrict__ out, int out_dtype, int B, int C, int H, int W, int halo)
+{
+    const int Hp = (H + 1) / 2 + 2 * halo, Wp = (W + 1) / 2 + 2 * halo, Wpairs = (Wp + 1) / 2;
+    const long long total = (long long)B * Hp * Wpairs;
+    const int zero = out_dtype == N2D2HIP_U8B ? -128 : 0;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+        const int xp = (int)(i % Wpairs);
+        const long long r = i / Wpairs;
+        const int Y = (int)(r % Hp), b = (int)(r / Hp);
+        union { signed char c[32]; uint4 v[2]; } px;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) px.c[k] = (signed char)zero;
+        auto stored = [&](int v) -> signed char {          // logical value -> the destination's stored byte
+            if (out_dtype == N2D2HIP_U8B) return (signed char)(clamp_i32(v, 0, 255) - 128);
+            if (out_dtype == N2D2HIP_U8) return (signed char)(unsigned char)clamp_i32(v, 0, 255);
+            return (signed char)clamp_i32(v, -128, 127);
+        };
+        const int x0 = 2 * (2 * xp - halo);                  // first of the four input columns the two pixels hold
+        // byte planes whose four columns are one aligned dword inside the row: one load per channel and input row
+        const bool quad = in_layout == N2D2HIP_NCHW && in_dtype != N2D2HIP_I32 && in_dtype != N2D2HIP_F32 && (W & 3) == 0 && (x0 & 3) == 0
+            && x0 >= 0 && x0 + 3 < W && 2 * xp + 1 < Wp;
+#pragma unroll
+        for (int dy = 0; dy < 2; ++dy) {
+            const int y = 2 * (Y - halo) + dy;
+            if (y < 0 || y >= H)
+                continue;
+            for (int c = 0; c < C; ++c) {
+                if (quad) {
+                    const unsigned w = *(const unsigned*)((const unsigned char*)in + (((size_t)b * C + c) * H + y) * (size_t)W + x0);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int byte = (int)((w >> (8 * k)) & 255u);
+                        const int v = in_dtype == N2D2HIP_U8 ? byte : (in_dtype == N2D2HIP_I8 ? (int)(signed char)byte : (int)(signed char)byte + 128);
+                        px.c[(k >> 1) * 16 + (dy * 2 + (k & 1)) * 4 + c] = stored(v);
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int x = x0 + k, X = 2 * xp + (k >> 1);
+                        if (X >= Wp || x < 0 || x >= W)
+                            continue;
+                        const size_t src = (in_layout == N2D2HIP_NHWC)
+                            ? (((size_t)b * (H + 2 * in_halo) + y + in_halo) * (W + 2 * in_halo) + x + in_halo) * (size_t)in_cs + c
+                            : (((size_t)b * C + c) * H + y) * (size_t)W + x;
+                        px.c[(k >> 1) * 16 + (dy * 2 + (k & 1)) * 4 + c] = stored(load_value(in, src, in_dtype));
+                    }
+                }
+            }
+        }
+        signed char* dst = out + (((size_t)b * Hp + Y) * Wp + 2 * xp) * 16;
+        *(uint4*)dst = px.v[0];
+        if (2 * xp + 1 < Wp)
+            *(uint4*)(dst + 16) = px.v[1];
+    }
+}
+} // namespace n2d2hip
 
 static int same_shape(const n2d2hip_tensor* a, const n2d2hip_tensor* b, const char* what)
 {
@@ -157,11 +286,20 @@ static unsigned grid_for(size_t total, int block)
 int n2d2hip_convert(const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
     int rc;
-    if ((rc = check_tensor(in, "convert input", true)) || (rc = check_tensor(out, "convert output")) || (rc = same_shape(in, out, "convert")))
+    if ((rc = check_tensor(in, "convert input", true)) || (rc = check_tensor(out, "convert output", false, true)) || (rc = same_shape(in, out, "convert")))
         return rc;
+    if (out->layout == N2D2HIP_S2D) {
+        const int Hp = (out->H + 1) / 2 + 2 * out->halo, Wp = (out->W + 1) / 2 + 2 * out->halo;
+        const long long pairs = (long long)out->B * Hp * ((Wp + 1) / 2);
+        N2D2HIP_REQUIRE((long long)out->B * Hp * Wp * 16 < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "convert: space-to-depth tensor too large");
+        N2D2HIP_LAUNCH(to_s2d_kernel, dim3(grid_for((size_t)pairs, 256)), dim3(256), 0, (hipStream_t)stream, in->data, in->dtype, in->layout, in->cs,
+                       in->halo, (signed char*)out->data, out->dtype, out->B, out->C, out->H, out->W, out->halo);
+        N2D2HIP_HIP_CHECK(hipGetLastError());
+        return N2D2HIP_OK;
+    }
     const size_t total = (size_t)out->B * out->H * out->W * (out->layout == N2D2HIP_NHWC ? out->cs : out->C);
     EpiArgs none = {};
-    hipLaunchKernelGGL(elementwise_kernel<false>, dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
+    N2D2HIP_LAUNCH_T(elementwise_kernel, (false), dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
                        in->data, in->dtype, in->layout, in->cs, in->halo, out->data, out->dtype, out->layout, out->cs,
                        out->B, out->C, out->H, out->W, none);
     N2D2HIP_HIP_CHECK(hipGetLastError());
@@ -349,7 +487,7 @@ int n2d2hip_scaling_forward(n2d2hip_act_t act, const n2d2hip_tensor* in, const n
     if (in->layout == N2D2HIP_NHWC && is_byte_type(in->dtype) && in->cs == out->cs && out->dtype != N2D2HIP_F32)
         return run_scaling_nhwc(act, in, out, (hipStream_t)stream);
     const size_t total = (size_t)out->B * out->H * out->W * (out->layout == N2D2HIP_NHWC ? out->cs : out->C);
-    hipLaunchKernelGGL(elementwise_kernel<true>, dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
+    N2D2HIP_LAUNCH_T(elementwise_kernel, (true), dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream,
                        in->data, in->dtype, in->layout, in->cs, 0, out->data, out->dtype, out->layout, out->cs,
                        out->B, out->C, out->H, out->W, act->args);
     N2D2HIP_HIP_CHECK(hipGetLastError());

@@ -351,10 +351,10 @@ template <bool FCOEF, bool HOIST, bool PRE>
 static void launch_elemwise(const ElemWiseArgs& a, unsigned grid, hipStream_t stream)
 {
     switch (a.epi.kind) {
-    case EPI_RAW: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_RAW, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I24: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I24, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I64: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_I64, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
-    default: hipLaunchKernelGGL((elemwise_sum_kernel<EPI_F32, FCOEF, HOIST, PRE>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_RAW: N2D2HIP_LAUNCH_T(elemwise_sum_kernel, (EPI_RAW, FCOEF, HOIST, PRE), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: N2D2HIP_LAUNCH_T(elemwise_sum_kernel, (EPI_I24, FCOEF, HOIST, PRE), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: N2D2HIP_LAUNCH_T(elemwise_sum_kernel, (EPI_I64, FCOEF, HOIST, PRE), dim3(grid), dim3(256), 0, stream, a); break;
+    default: N2D2HIP_LAUNCH_T(elemwise_sum_kernel, (EPI_F32, FCOEF, HOIST, PRE), dim3(grid), dim3(256), 0, stream, a); break;
     }
 }
 
@@ -483,22 +483,22 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
                     "pool_forward: only the 2x2 / 3x3 max pooling of 16-byte channel groups writes an output with a halo");
     if (d->pooling == N2D2HIP_POOL_AVERAGE && OH == 1 && OW == 1 && d->poolW == in->W && d->poolH == in->H && d->padX == 0 && d->padY == 0) {
         const int slabs = (in->cs + 255) / 256;
-        hipLaunchKernelGGL(global_avg_pool_kernel, dim3((unsigned)(in->B * slabs)), dim3(256), 0, (hipStream_t)stream,
+        N2D2HIP_LAUNCH(global_avg_pool_kernel, dim3((unsigned)(in->B * slabs)), dim3(256), 0, (hipStream_t)stream,
                            (const signed char*)in->data, in->cs, in->H * in->W, (signed char*)out->data, zp, flip);
     } else if (fast) {
         const long long total16 = (long long)in->B * OH * OW * (in->cs / 16);
         const unsigned g16 = (unsigned)round_up((int)std::max<long long>(1, std::min<long long>((total16 + 255) / 256, 256 * 64)), 8);
         if (d->poolW == 3)
-            hipLaunchKernelGGL((pool_max_fast_kernel<3, 3>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
+            N2D2HIP_LAUNCH_T(pool_max_fast_kernel, (3, 3), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
                                in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip, out->halo);
         else
-            hipLaunchKernelGGL((pool_max_fast_kernel<2, 2>), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
+            N2D2HIP_LAUNCH_T(pool_max_fast_kernel, (2, 2), dim3(g16), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs,
                                in->B, in->H, in->W, (signed char*)out->data, OH, OW, d->strideX, d->strideY, d->padX, d->padY, flip, out->halo);
     } else if (d->pooling == N2D2HIP_POOL_MAX)
-        hipLaunchKernelGGL(pool_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
+        N2D2HIP_LAUNCH_T(pool_kernel, (true), dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
     else
-        hipLaunchKernelGGL(pool_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
+        N2D2HIP_LAUNCH_T(pool_kernel, (false), dim3(grid), dim3(256), 0, (hipStream_t)stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, (signed char*)out->data, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, zp, flip);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
@@ -520,7 +520,7 @@ int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* d, const unsigned char*
     const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
     const int bias = in->dtype == N2D2HIP_U8B ? 128 : 0;
 #define N2D2HIP_POOL_MAPPED(IS_MAX, IS_SIGNED)                                                                                      \
-    hipLaunchKernelGGL((pool_mapped_kernel<IS_MAX, IS_SIGNED>), dim3(grid), dim3(256), 0, (hipStream_t)stream,                       \
+    N2D2HIP_LAUNCH_T(pool_mapped_kernel, (IS_MAX, IS_SIGNED), dim3(grid), dim3(256), 0, (hipStream_t)stream,                       \
                        (const signed char*)in->data, in->cs, in->C, in->B, in->H, in->W, maps, (signed char*)out->data, out->cs,     \
                        out->C, OH, OW, d->poolW, d->poolH, d->strideX, d->strideY, d->padX, d->padY, bias)
     const bool is_signed = in->dtype != N2D2HIP_U8;
@@ -671,7 +671,7 @@ int n2d2hip_concat_channels(int nb_inputs, const n2d2hip_tensor* const* inputs, 
     a.fill = out->dtype == N2D2HIP_U8B ? 0x80u : 0u;
     const long long total = (long long)out->B * out->H * out->W * (out->cs / 4);
     const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
-    hipLaunchKernelGGL(concat_channels_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, a);
+    N2D2HIP_LAUNCH(concat_channels_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, a);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

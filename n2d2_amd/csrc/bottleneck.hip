@@ -58,7 +58,7 @@ struct BottleneckArgs {
     unsigned res_flip;          // turns a stored byte of x into the unsigned operand of the sum
     int other_off;              // projection: added to its saturated value (the zero point the sum's tables expect)
 #ifdef N2D2HIP_PROFILE
-    long long* prof;            // 8 counters per block
+    long long* prof;            // one 16-counter record per block
 #endif
 };
 
@@ -506,10 +506,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         PROF_MARK(5);
     }
 #ifdef N2D2HIP_PROFILE
-    if (tid == 0) {
-        long long* o = q.prof + (long long)blockIdx.x * 10;
-        for (int k = 0; k < 6; ++k) o[k] = pr[k];
-        o[6] = clock64() - pr_t0; o[7] = wall_clock64() - pr_w0; o[8] = ntile; o[9] = 1;
+    if (tid == 0 && q.prof) {
+        // the common record (start, -, -, end, -, wall start, wall end, tiles), then this kernel's six phase sums
+        long long* o = q.prof + (long long)blockIdx.x * 16;
+        o[0] = pr_t0; o[1] = 0; o[2] = 0; o[3] = clock64(); o[4] = 0; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = ntile;
+        for (int k = 0; k < 6; ++k) o[8 + k] = pr[k];
     }
 #endif
     // the pixels requested past the last tile are still on their way
@@ -735,23 +736,19 @@ int n2d2hip_bottleneck_forward(n2d2hip_bottleneck_t b, const n2d2hip_tensor* in,
     const int grid = 8 * q.nlanes;
     hipStream_t st = (hipStream_t)stream_;
 #ifdef N2D2HIP_PROFILE
-    {
-        const char* pp = getenv("N2D2HIP_PROF_PTR");      // profiling builds only: where the blocks' counters go
-        N2D2HIP_REQUIRE(pp != nullptr, N2D2HIP_ERR_INVALID, "bottleneck_forward: profiling build without N2D2HIP_PROF_PTR");
-        q.prof = (long long*)strtoull(pp, nullptr, 16);
-    }
+    q.prof = nullptr;      // probe builds: launch_kernel() points it at this launch's records
 #endif
     if (!b->expand) {
-        if (b->cin == 64) hipLaunchKernelGGL((bottleneck_kernel<64, OTHER_PROJECTION, 2>), dim3(grid), dim3(256), 0, st, q);
-        else hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X, 2>), dim3(grid), dim3(256), 0, st, q);
+        if (b->cin == 64) N2D2HIP_LAUNCH_T(bottleneck_kernel, (64, OTHER_PROJECTION, 2), dim3(grid), dim3(256), 0, st, q);
+        else N2D2HIP_LAUNCH_T(bottleneck_kernel, (256, OTHER_X, 2), dim3(grid), dim3(256), 0, st, q);
     } else if (b->projection) {
-        hipLaunchKernelGGL((bottleneck_kernel<64, OTHER_PROJECTION, 3>), dim3(grid), dim3(256), 0, st, q);
+        N2D2HIP_LAUNCH_T(bottleneck_kernel, (64, OTHER_PROJECTION, 3), dim3(grid), dim3(256), 0, st, q);
     } else if (!b->expand->has_pre) {
-        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X, 3>), dim3(grid), dim3(256), 0, st, q);
+        N2D2HIP_LAUNCH_T(bottleneck_kernel, (256, OTHER_X, 3), dim3(grid), dim3(256), 0, st, q);
     } else if (b->expand->pre_in_range) {
-        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X_SCALED, 3>), dim3(grid), dim3(256), 0, st, q);
+        N2D2HIP_LAUNCH_T(bottleneck_kernel, (256, OTHER_X_SCALED, 3), dim3(grid), dim3(256), 0, st, q);
     } else {
-        hipLaunchKernelGGL((bottleneck_kernel<256, OTHER_X_SCALED_SAT, 3>), dim3(grid), dim3(256), 0, st, q);
+        N2D2HIP_LAUNCH_T(bottleneck_kernel, (256, OTHER_X_SCALED_SAT, 3), dim3(grid), dim3(256), 0, st, q);
     }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;

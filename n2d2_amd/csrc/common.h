@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "n2d2hip.h"
@@ -48,7 +49,65 @@ inline int round_up(int x, int m)
 {
     return (x + m - 1) / m * m;
 }
-int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok = false);
+int check_tensor(const n2d2hip_tensor* t, const char* what, bool halo_ok = false, bool s2d_ok = false);
+
+// ---------------------------------------------------------------- launches
+// The kernels of the integer path are launched through launch_kernel<&kernel>(), so that the launch log
+// (n2d2hip_launch_log_*) can name what a call launched, template arguments included, and its grid.
+// __PRETTY_FUNCTION__ of this function carries the kernel's full name ("... [K = &n2d2hip::kernel<1, 2>]").
+template <auto K>
+const char* kernel_pretty()
+{
+    return __PRETTY_FUNCTION__;
+}
+// Adds a launch to the calling thread's log when one is open; `slot` is the launch's first probe record or -1.
+void launch_log_add(const char* pretty, unsigned grid, unsigned block, long long slot);
+#ifdef N2D2HIP_PROFILE
+// Probe builds: records (8 counters each) for the blocks of the next launch inside the buffer given to
+// n2d2hip_probe_begin(); null when there is none or it is full.  *first is the index of the first record.
+long long* probe_take(unsigned blocks, long long* first);
+template <class T>
+auto set_probe(T& a, long long* p, int) -> decltype(a.prof = p, void())
+{
+    a.prof = p;
+}
+template <class T>
+void set_probe(T&, long long*, long)
+{
+}
+#endif
+
+template <auto K, class A0, class... A>
+void launch_kernel(const char* name, dim3 grid, dim3 block, unsigned lds, hipStream_t stream, A0 a0, A... a)
+{
+    long long slot = -1;
+#ifdef N2D2HIP_PROFILE
+    set_probe(a0, probe_take(grid.x * grid.y * grid.z, &slot), 0);
+#endif
+    launch_log_add(name ? name : kernel_pretty<K>(), grid.x * grid.y * grid.z, block.x * block.y * block.z, slot);
+    hipLaunchKernelGGL(K, grid, block, lds, stream, a0, a...);
+}
+// "<4, 128, true>": the values of a kernel's template arguments, for its name in the launch log
+inline void targ_text(std::string& s, bool v) { s += v ? "true" : "false"; }
+inline void targ_text(std::string& s, long long v) { s += std::to_string(v); }
+template <auto K, auto... V>
+const char* targs_of(const char* kernel)
+{
+    static const std::string text = [kernel] {
+        std::string s = std::string(kernel) + "<";
+        bool first = true;
+        ((s += first ? "" : ", ", first = false,
+          targ_text(s, static_cast<std::conditional_t<std::is_same<decltype(V), bool>::value, bool, long long>>(V))), ...);
+        return s + ">";
+    }();
+    return text.c_str();
+}
+#define N2D2HIP_UNPAREN(...) __VA_ARGS__
+// N2D2HIP_LAUNCH(kernel, ...): a kernel without template arguments (or whose arguments need not show in the log);
+// N2D2HIP_LAUNCH_T(kernel, (template arguments), ...): the log names the kernel with the arguments' values.
+#define N2D2HIP_LAUNCH(K, grid, block, lds, stream, ...) ::n2d2hip::launch_kernel<&K>(nullptr, grid, block, lds, stream, __VA_ARGS__)
+#define N2D2HIP_LAUNCH_T(K, TARGS, grid, block, lds, stream, ...)                                              \
+    ::n2d2hip::launch_kernel<&K<N2D2HIP_UNPAREN TARGS>>(::n2d2hip::targs_of<&K<N2D2HIP_UNPAREN TARGS>, N2D2HIP_UNPAREN TARGS>(#K), grid, block, lds, stream, __VA_ARGS__)
 
 // ---------------------------------------------------------------- epilogue
 // Device-side form of "Scaling::propagate, saturate, Rectifier/Linear" for one

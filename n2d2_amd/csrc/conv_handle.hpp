@@ -34,6 +34,8 @@ struct n2d2hip_conv_s {
     bool hi16;
     // first-layer kernel (<= 4 input channels, horizontal stride 2): weights as [channel][kH * 32]
     signed char* d_wstem;
+    // first-layer kernel on space-to-depth inputs (<= 4 input channels, square kernel of 3 / 5 / 7, stride 2): weights per K step
+    signed char* d_ws2d;
     // 3x3 stride-1 kernel over inputs that carry their padding: weights in matrix-core fragment order
     signed char* d_wfrag;
     // 3x3 depthwise kernel: per channel and kernel row the three weights in one dword, then the biases with the zero point folded in

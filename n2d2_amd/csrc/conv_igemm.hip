@@ -348,6 +348,7 @@ __global__ __launch_bounds__(256) void depthwise_kernel(const signed char* __res
 using namespace n2d2hip;
 
 #include "conv_handle.hpp"
+#include "conv_s2d.hpp"
 
 namespace {
 
@@ -362,10 +363,10 @@ void launch_cfg(const ConvArgs& a, hipStream_t stream)
 {
     const int grid = round_up(a.nblocks, 8);
     switch (a.epi.kind) {
-    case EPI_RAW: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_RAW, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I24: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_I24, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
-    case EPI_I64: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_I64, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
-    default: hipLaunchKernelGGL((conv_igemm_kernel<BM, BN, WGM, EPI_F32, PIX4, W4>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_RAW: N2D2HIP_LAUNCH_T(conv_igemm_kernel, (BM, BN, WGM, EPI_RAW, PIX4, W4), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I24: N2D2HIP_LAUNCH_T(conv_igemm_kernel, (BM, BN, WGM, EPI_I24, PIX4, W4), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_I64: N2D2HIP_LAUNCH_T(conv_igemm_kernel, (BM, BN, WGM, EPI_I64, PIX4, W4), dim3(grid), dim3(256), 0, stream, a); break;
+    default: N2D2HIP_LAUNCH_T(conv_igemm_kernel, (BM, BN, WGM, EPI_F32, PIX4, W4), dim3(grid), dim3(256), 0, stream, a); break;
     }
 }
 
@@ -375,20 +376,20 @@ void launch_pipe(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t str
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
 #define N2D2HIP_PIPE(EPI) \
-    do { if (valid == 1) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 1>), dim3(grid), dim3(NW * 64), 0, stream, a); \
-         else if (valid == 2) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 2>), dim3(grid), dim3(NW * 64), 0, stream, a); \
-         else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI, S, 0>), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
+    do { if (valid == 1) N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI, S, 1), dim3(grid), dim3(NW * 64), 0, stream, a); \
+         else if (valid == 2) N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI, S, 2), dim3(grid), dim3(NW * 64), 0, stream, a); \
+         else N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI, S, 0), dim3(grid), dim3(NW * 64), 0, stream, a); } while (0)
     switch (a.c.epi.kind) {
     case EPI_RAW: N2D2HIP_PIPE(EPI_RAW); break;
     case EPI_I24:
         if (!hi16) {
             N2D2HIP_PIPE(EPI_I24);
         } else if (valid == 1) {
-            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+            N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 1, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
         } else if (valid == 2) {
-            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 2, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+            N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 2, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
         } else {
-            hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+            N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
         }
         break;
     default: N2D2HIP_PIPE(EPI_F32); break;
@@ -401,18 +402,18 @@ template <int KH>
 void launch_stem(const ConvStemArgs& a, bool hi16, bool narrow, int grid, hipStream_t stream)
 {
     switch (a.c.epi.kind) {
-    case EPI_RAW: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_RAW>), dim3(grid), dim3(256), 0, stream, a); break;
+    case EPI_RAW: N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_RAW), dim3(grid), dim3(256), 0, stream, a); break;
     case EPI_I24:
         if (narrow) {
-            if (hi16) hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true, false, 1>), dim3(grid), dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, false, false, 1>), dim3(grid), dim3(256), 0, stream, a);
+            if (hi16) N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_I24, true, false, 1), dim3(grid), dim3(256), 0, stream, a);
+            else N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_I24, false, false, 1), dim3(grid), dim3(256), 0, stream, a);
         } else if (hi16) {
-            hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+            N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_I24, true), dim3(grid), dim3(256), 0, stream, a);
         } else {
-            hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_I24>), dim3(grid), dim3(256), 0, stream, a);
+            N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_I24), dim3(grid), dim3(256), 0, stream, a);
         }
         break;
-    default: hipLaunchKernelGGL((conv_stem_kernel<KH, EPI_F32>), dim3(grid), dim3(256), 0, stream, a); break;
+    default: N2D2HIP_LAUNCH_T(conv_stem_kernel, (KH, EPI_F32), dim3(grid), dim3(256), 0, stream, a); break;
     }
 }
 
@@ -422,9 +423,9 @@ void launch_pipe_res(ConvPipeArgs a, int grid, hipStream_t stream)
     a.c.niter = a.c.ktot / BK;
     a.cper = a.c.in_cs / BK;
     if (a.sum16)
-        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, true), dim3(grid), dim3(NW * 64), 0, stream, a);
     else
-        hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, false>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 1, true, false), dim3(grid), dim3(NW * 64), 0, stream, a);
 }
 
 // (multiplier, shift) with n / d == umulhi(n, multiplier) >> shift for 0 <= n < 2^31; multiplier 0 stands for d == 1
@@ -522,7 +523,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr; c->d_wsmall = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_ws2d = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr; c->d_wsmall = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -696,6 +697,15 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_wstem, ws.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wstem, ws.data(), ws.size(), hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess && c->pix4 && d->weight_bits == 8 && d->strideX == 2 && d->strideY == 2 && d->dilX == 1 && d->dilY == 1 && d->kW == d->kH
+        && (d->kH == 3 || d->kH == 5 || d->kH == 7) && d->O <= 64 && !(d->kernel_choice & N2D2HIP_KERNEL_NO_STEM)) {
+        std::vector<signed char> ochw((size_t)d->O * d->C * d->kH * d->kW), ws(conv_s2d_weight_bytes(d->O, d->kH, d->padT));
+        for (size_t i = 0; i < ochw.size(); ++i)
+            ochw[i] = (signed char)read_weight(weights, (long long)i, 8);
+        conv_s2d_weight_layout(ochw.data(), d->C, d->O, d->kH, d->padT, d->padL, ws.data());
+        e = hipMalloc((void**)&c->d_ws2d, ws.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_ws2d, ws.data(), ws.size(), hipMemcpyHostToDevice);
+    }
     // (a dilated kernel with padding keeps the kernel that follows the reference's window arithmetic tap by tap: what the
     // reference skips at the borders is then not what zero padding would skip)
     if (e == hipSuccess && !depthwise && d->weight_bits == 8 && d->kW <= 8 && conv_small_rows(d->C, d->O, d->kW * d->kH)
@@ -755,6 +765,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_res_tab) (void)hipFree(c->d_res_tab);
     if (c->d_epi_tab) (void)hipFree(c->d_epi_tab);
     if (c->d_wstem) (void)hipFree(c->d_wstem);
+    if (c->d_ws2d) (void)hipFree(c->d_ws2d);
     if (c->d_wsmall) (void)hipFree(c->d_wsmall);
     if (c->d_wfrag) (void)hipFree(c->d_wfrag);
     if (c->d_wdw) (void)hipFree(c->d_wdw);
@@ -778,15 +789,106 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
         && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
 }
 
+// Is this convolution served by the space-to-depth first-layer kernel on an H x W input?  Returns the border it needs, or -1.
+static int s2d_halo(const n2d2hip_conv_s* c, int H, int W)
+{
+    const n2d2hip_conv_desc& d = c->desc;
+    if (!c->d_ws2d || c->act->args.kind != EPI_I24 || !c->bias_folded || c->act->min_out < -128 || c->act->max_out > 255)
+        return -1;
+    const int halo = conv_s2d_halo(d.kH, d.padT, d.padL, d.padB, d.padR, H, W);
+    // a tile is at least one row of the bordered image and at most 256 positions
+    if (halo < 0 || halo > 16 || (W + 1) / 2 + 2 * halo > 128)
+        return -1;
+    return halo;
+}
+
+// The first-layer kernel on a space-to-depth input; `pd` non-null: with the 3x3 stride-2 max pooling behind it (`out` is the
+// pooled tensor).  Shapes of `out` have been checked by the caller.
+static int conv_s2d_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, const n2d2hip_pool_desc* pd,
+                            int OH, int OW, int POH, int POW, hipStream_t stream)
+{
+    const n2d2hip_conv_desc& d = c->desc;
+    const int need = s2d_halo(c, in->H, in->W);
+    N2D2HIP_REQUIRE(need >= 0, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: this convolution does not read space-to-depth inputs (n2d2hip_conv_s2d_halo)");
+    N2D2HIP_REQUIRE(in->halo >= need, N2D2HIP_ERR_INVALID, "conv_forward: the space-to-depth input has a border of %d, the convolution needs %d",
+                    in->halo, need);
+    N2D2HIP_REQUIRE(in->dtype == c->in_dtype && in->C == d.C, N2D2HIP_ERR_INVALID, "conv_forward: input has %d channels of type %d, conv expects %d of type %d",
+                    in->C, in->dtype, d.C, c->in_dtype);
+    ConvS2dArgs a = {};
+    a.in = (const signed char*)in->data;
+    a.Hp = (in->H + 1) / 2 + 2 * in->halo;
+    a.Wp = (in->W + 1) / 2 + 2 * in->halo;
+    N2D2HIP_REQUIRE(a.Wp <= 128 && (long long)in->B * a.Hp * a.Wp * 16 < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward: space-to-depth input too wide or too large");
+    a.total = in->B * a.Hp * a.Wp;
+    a.wk = c->d_ws2d;
+    a.ty = in->halo - (d.padT + 1) / 2;
+    a.tx = in->halo - (d.padL + 1) / 2;
+    a.OH = OH; a.OW = OW;
+    magic_div((unsigned)a.Wp, &a.wp_mul, &a.wp_sh);
+    a.out = out->data; a.out_cs = out->cs;
+    a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    const int cp = c->act->cpad;
+    const bool hi16 = c->hi16 && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
+    a.ta = c->d_epi_tab; a.tb = c->d_epi_tab + cp; a.tc = c->d_epi_tab + (hi16 ? 5 : 2) * cp;
+    a.td = c->d_epi_tab + (hi16 ? 6 : 3) * cp; a.te = c->d_epi_tab + 4 * cp;
+    a.lo = c->act->args.lo; a.hi = c->act->args.hi; a.preclamp = c->preclamp ? 1 : 0;
+    a.n0 = 0;
+    const int ny = (d.kH + 1) / 2, nxh = (ny + 1) / 2;
+    const int slots = 2 * num_cus();
+    if (pd) {
+        N2D2HIP_REQUIRE(hi16 && OW <= 112 && POW <= 64 && round_up(d.O, 16) == 64, N2D2HIP_ERR_UNSUPPORTED,
+                        "conv_forward_maxpool: the pooled first-layer kernel needs scaled-up tables, 49 to 64 outputs and rows of at most 112");
+        a.TR = 2;
+        a.pool_pad = pd->padX; a.POH = POH; a.POW = POW;
+        a.pool_halo = out->halo; a.POHp = POH + 2 * out->halo; a.POWp = POW + 2 * out->halo;
+        // strips of pooled rows: one per block slot if the batch has that many rows, never shorter than 4 rows (each
+        // strip computes one or two convolution rows more than it needs)
+        int rows = std::max(1, (int)(((long long)in->B * POH + slots - 1) / slots));
+        rows = std::min(std::max(rows, std::min(POH, 4)), POH);
+        a.rows_per_strip = rows;
+        a.strips_per_image = (POH + rows - 1) / rows;
+    } else {
+        a.TR = std::max(1, std::min(256 / a.Wp, OH));
+        int rows = std::max(a.TR, (int)(((long long)in->B * OH + slots - 1) / slots));
+        rows = std::min(round_up(rows, a.TR), round_up(OH, a.TR));
+        a.rows_per_strip = rows;
+        a.strips_per_image = (OH + rows - 1) / rows;
+    }
+    a.T = a.TR * a.Wp;
+    a.NT = (a.T + 31) / 32;
+    // positions a tile's window reaches past its first one (the last 32-position tile in full, the last window row and
+    // pixel pair, the upper lane half's + 1), and one more tile: what must be in the ring before a strip's first tile
+    const int window = a.NT * 32 + (ny - 1) * a.Wp + 2 * nxh + 1;
+    a.PF = round_up(window + a.T, 64);
+    N2D2HIP_REQUIRE(a.T <= 256 && a.PF + a.T + 64 < 2048, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: space-to-depth rows too long");
+    a.nstrips = in->B * a.strips_per_image;
+    const int blocks = std::max(1, std::min(a.nstrips, slots));
+    return conv_s2d_launch(a, d.kH, hi16, pd != nullptr, round_up(d.O, 16) <= 32 ? 1 : 2, blocks, stream);
+}
+
 static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* other, const n2d2hip_tensor* out,
                              n2d2hip_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     int rc;
     N2D2HIP_REQUIRE(c != nullptr, N2D2HIP_ERR_INVALID, "conv_forward: null conv");
-    if ((rc = check_tensor(in, "conv input", true)) || (rc = check_tensor(out, "conv output", true)))
+    if ((rc = check_tensor(in, "conv input", true, true)) || (rc = check_tensor(out, "conv output", true)))
         return rc;
     const n2d2hip_conv_desc& d = c->desc;
+    if (in->layout == N2D2HIP_S2D) {
+        int OH, OW;
+        if ((rc = n2d2hip_conv_out_dims(&d, in->H, in->W, &OH, &OW)))
+            return rc;
+        N2D2HIP_REQUIRE(!other && out->halo == 0 && out->layout == N2D2HIP_NHWC && is_byte_type(out->dtype) && out->cs % 16 == 0,
+                        N2D2HIP_ERR_UNSUPPORTED, "conv_forward: a space-to-depth input goes to a plain NHWC byte output");
+        N2D2HIP_REQUIRE(out->B == in->B && out->C == d.O && out->H == OH && out->W == OW, N2D2HIP_ERR_INVALID,
+                        "conv_forward: output is %dx%dx%dx%d, expected %dx%dx%dx%d", out->B, out->C, out->H, out->W, in->B, d.O, OH, OW);
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(c->act->min_out >= lo && c->act->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "conv_forward: activation range [%d,%d] does not fit output dtype %d", c->act->min_out, c->act->max_out, out->dtype);
+        return conv_s2d_forward(c, in, out, nullptr, OH, OW, 0, 0, (hipStream_t)stream_);
+    }
     bool bn128_unused;
     N2D2HIP_REQUIRE((in->halo == 0 && out->halo == 0)
                         || (pipe_eligible(c, &bn128_unused) && !(d.kernel_choice & N2D2HIP_KERNEL_NO_PIPE) && d.dilX == 1 && d.dilY == 1),
@@ -853,7 +955,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
         }
         const long long total = Mll * (in->cs / 4);
         const unsigned grid = (unsigned)std::min<long long>((total + 255) / 256, 256 * 64);
-        hipLaunchKernelGGL(depthwise_kernel, dim3(grid), dim3(256), 0, stream, (const signed char*)in->data, in->cs, in->B, in->H,
+        N2D2HIP_LAUNCH(depthwise_kernel, dim3(grid), dim3(256), 0, stream, (const signed char*)in->data, in->cs, in->B, in->H,
                            in->W, OH, OW, c->d_w, d.kH, d.kW, c->d_bias, out->data, out->dtype, d.strideX, d.strideY, d.padL,
                            d.padT, d.dilX, d.dilY, zero_point(in->dtype), out_xor, c->act->args);
         N2D2HIP_HIP_CHECK(hipGetLastError());
@@ -927,11 +1029,7 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
             q.c.epi.d = c->d_epi_tab + 3 * cp; q.c.epi.e = c->d_epi_tab + 4 * cp;
         }
 #ifdef N2D2HIP_PROFILE
-        {
-            const char* pp = getenv("N2D2HIP_PROF_PTR");      // profiling builds only: where the blocks' timestamps go
-            N2D2HIP_REQUIRE(pp != nullptr, N2D2HIP_ERR_INVALID, "conv_forward: profiling build without N2D2HIP_PROF_PTR");
-            q.prof = (long long*)strtoull(pp, nullptr, 16);
-        }
+        q.prof = nullptr;      // probe builds: launch_kernel() points it at this launch's records
 #endif
         magic_div((unsigned)(OH * OW), &q.ohw_mul, &q.ohw_sh);
         magic_div((unsigned)OW, &q.ow_mul, &q.ow_sh);
@@ -1115,16 +1213,32 @@ int n2d2hip_conv_accepts_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool
     return c && pool && stem_pool_eligible(c, pool, H, W, &a, &b, &e, &f) ? 1 : 0;
 }
 
+int n2d2hip_conv_s2d_halo(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool, int H, int W)
+{
+    if (!c || H <= 0 || W <= 0)
+        return -1;
+    const int halo = s2d_halo(c, H, W);
+    if (halo < 0 || !pool)
+        return halo;
+    int OH, OW, POH, POW;
+    const bool hi16 = c->hi16 && !(c->desc.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
+    if (!stem_pool_eligible(c, pool, H, W, &OH, &OW, &POH, &POW) || !hi16 || OW > 112)
+        return -1;
+    return halo;
+}
+
 int n2d2hip_conv_forward_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                                  n2d2hip_stream_t stream_)
 {
     int rc, OH, OW, POH, POW;
     N2D2HIP_REQUIRE(c && pool, N2D2HIP_ERR_INVALID, "conv_forward_maxpool: null argument");
-    if ((rc = check_tensor(in, "conv input")) || (rc = check_tensor(out, "pooled output", true)))
+    if ((rc = check_tensor(in, "conv input", false, true)) || (rc = check_tensor(out, "pooled output", true)))
         return rc;
     const n2d2hip_conv_desc& d = c->desc;
-    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED, "conv_forward_maxpool: tensors must be NHWC");
-    N2D2HIP_REQUIRE(in->dtype == c->in_dtype && in->C == d.C && in->cs == c->in_cs, N2D2HIP_ERR_INVALID,
+    const bool s2d = in->layout == N2D2HIP_S2D;
+    N2D2HIP_REQUIRE((in->layout == N2D2HIP_NHWC || s2d) && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_forward_maxpool: the input must be NHWC or space-to-depth, the output NHWC");
+    N2D2HIP_REQUIRE(in->dtype == c->in_dtype && in->C == d.C && (s2d || in->cs == c->in_cs), N2D2HIP_ERR_INVALID,
                     "conv_forward_maxpool: input has %d channels (stride %d) of type %d, conv expects %d (stride %d) of type %d", in->C, in->cs,
                     in->dtype, d.C, c->in_cs, c->in_dtype);
     N2D2HIP_REQUIRE(stem_pool_eligible(c, pool, in->H, in->W, &OH, &OW, &POH, &POW), N2D2HIP_ERR_UNSUPPORTED,
@@ -1141,6 +1255,11 @@ int n2d2hip_conv_forward_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool
                         "conv_forward_maxpool: activation range [%d,%d] does not fit output dtype %d", c->act->min_out, c->act->max_out, out->dtype);
     }
     N2D2HIP_REQUIRE((long long)in->B * in->H * in->W * in->cs < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "conv_forward_maxpool: tensor too large");
+    if (s2d) {
+        N2D2HIP_REQUIRE(n2d2hip_conv_s2d_halo(c, pool, in->H, in->W) >= 0, N2D2HIP_ERR_UNSUPPORTED,
+                        "conv_forward_maxpool: this pair does not read space-to-depth inputs (n2d2hip_conv_s2d_halo)");
+        return conv_s2d_forward(c, in, out, pool, OH, OW, POH, POW, (hipStream_t)stream_);
+    }
     ConvArgs a;
     a.in = (const signed char*)in->data;
     a.in_cs = in->cs; a.B = in->B; a.H = in->H; a.W = in->W;
@@ -1178,9 +1297,9 @@ int n2d2hip_conv_forward_maxpool(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool
     q.xcd_tiles = (q.ntiles + 7) / 8;
     const int grid = 8 * q.nlanes;
     hipStream_t stream = (hipStream_t)stream_;
-    if (d.kH == 3) hipLaunchKernelGGL((conv_stem_kernel<3, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
-    else if (d.kH == 5) hipLaunchKernelGGL((conv_stem_kernel<5, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
-    else hipLaunchKernelGGL((conv_stem_kernel<7, EPI_I24, true, true>), dim3(grid), dim3(256), 0, stream, q);
+    if (d.kH == 3) N2D2HIP_LAUNCH_T(conv_stem_kernel, (3, EPI_I24, true, true), dim3(grid), dim3(256), 0, stream, q);
+    else if (d.kH == 5) N2D2HIP_LAUNCH_T(conv_stem_kernel, (5, EPI_I24, true, true), dim3(grid), dim3(256), 0, stream, q);
+    else N2D2HIP_LAUNCH_T(conv_stem_kernel, (7, EPI_I24, true, true), dim3(grid), dim3(256), 0, stream, q);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

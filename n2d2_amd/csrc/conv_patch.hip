@@ -233,6 +233,9 @@ __global__ __launch_bounds__(WGM * WGN * 64) __attribute__((amdgpu_waves_per_eu(
     };
 
     // ---- fill: the first patch, the weights of the first three taps
+#ifdef N2D2HIP_PROFILE
+    pr_t1 = clock64();
+#endif
     issue_patch(mlane, 0, 0);
     issue_w(std::integral_constant<int, 0>());
     issue_w(std::integral_constant<int, 1>());
@@ -260,8 +263,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) __attribute__((amdgpu_waves_per_eu(
         // barrier everybody's have, and nobody still reads the other buffer.
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(3 * NWL) : "memory");
 #ifdef N2D2HIP_PROFILE
-        if (s == 0) pr_t1 = clock64();
-        if (s == 1) pr_t2 = clock64();
+        if (s == 0) pr_t2 = clock64();
 #endif
         int n_tile = c_tile, n_chunk = c_chunk + 1;
         if (n_chunk == nchunk) { n_chunk = 0; ++n_tile; }
@@ -343,8 +345,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) __attribute__((amdgpu_waves_per_eu(
         c_chunk = n_chunk;
     }
 #ifdef N2D2HIP_PROFILE
-    if (tid == 0) {
-        long long* o = q.prof + (long long)blockIdx.x * 8;
+    if (tid == 0 && q.prof) {
+        long long* o = q.prof + (long long)blockIdx.x * 16;
         o[0] = pr_t0; o[1] = pr_t1; o[2] = pr_t2; o[3] = clock64(); o[4] = pr_epi; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = nsteps;
     }
 #endif
@@ -379,9 +381,9 @@ template <int WGM, int WGN, int NPL, int NJ>
 static void launch(const ConvPatchArgs& a, bool hi16, int grid, hipStream_t stream)
 {
     if (hi16)
-        hipLaunchKernelGGL((conv_patch3x3_kernel<WGM, WGN, NPL, true, NJ>), dim3(grid), dim3(WGM * WGN * 64), 0, stream, a);
+        N2D2HIP_LAUNCH_T(conv_patch3x3_kernel, (WGM, WGN, NPL, true, NJ), dim3(grid), dim3(WGM * WGN * 64), 0, stream, a);
     else
-        hipLaunchKernelGGL((conv_patch3x3_kernel<WGM, WGN, NPL, false, NJ>), dim3(grid), dim3(WGM * WGN * 64), 0, stream, a);
+        N2D2HIP_LAUNCH_T(conv_patch3x3_kernel, (WGM, WGN, NPL, false, NJ), dim3(grid), dim3(WGM * WGN * 64), 0, stream, a);
 }
 
 int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipStream_t stream)
@@ -417,11 +419,7 @@ int conv_patch_launch(ConvPatchArgs a, bool hi16, int num_cus, int tile_m, hipSt
     a.xcd_tiles = (a.mtiles + 7) / 8;
     const int grid = 8 * a.ntiles_n * per_xcd;
 #ifdef N2D2HIP_PROFILE
-    {
-        const char* pp = getenv("N2D2HIP_PROF_PTR");      // profiling builds only: where the blocks' timestamps go
-        N2D2HIP_REQUIRE(pp != nullptr, N2D2HIP_ERR_INVALID, "conv_patch: profiling build without N2D2HIP_PROF_PTR");
-        a.prof = (long long*)strtoull(pp, nullptr, 16);
-    }
+    a.prof = nullptr;      // probe builds: launch_kernel() points it at this launch's records
 #endif
     // patch rows: at most 384 (tiles of 256) or 256 (tiles of 128) wherever the kernel is eligible
     if (form == M256_WAVES4) {

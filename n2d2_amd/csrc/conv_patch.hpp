@@ -24,7 +24,7 @@ struct ConvPatchArgs {
     int lo, hi;                 // saturation range
     int preclamp;               // clamp the accumulator to [a, b] before the multiply (32-bit rescale only)
 #ifdef N2D2HIP_PROFILE
-    long long* prof;            // 8 timestamps per block
+    long long* prof;            // one 16-counter record per block
 #endif
 };
 

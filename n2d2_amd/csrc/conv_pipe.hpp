@@ -66,7 +66,7 @@ struct ConvPipeArgs {
     int sum16_stride;
     int pre_in_range;            // with sum16: the ScalingCell's result cannot leave its range, no saturation needed
 #ifdef N2D2HIP_PROFILE
-    long long* prof;             // 8 timestamps per block
+    long long* prof;             // one 16-counter record per block
 #endif
 };
 
@@ -886,8 +886,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
 #ifdef N2D2HIP_PROFILE
     pr_t3 = clock64();
-    if (tid == 0) {
-        long long* o = q.prof + (long long)blockIdx.x * 8;
+    if (tid == 0 && q.prof) {
+        long long* o = q.prof + (long long)blockIdx.x * 16;
         o[0] = pr_t0; o[1] = pr_t1; o[2] = pr_t2; o[3] = pr_t3; o[4] = pr_epi; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = ntile * niter;
     }
 #endif

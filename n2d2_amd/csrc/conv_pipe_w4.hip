@@ -41,11 +41,11 @@ void launch_valid(const ConvPipeArgs& a, bool hi16, int grid, hipStream_t stream
     constexpr int NW = 4, BK = 64, S = 4;
     if (a.res) {
         // residual sum in the epilogue; 16-bit pairs when the host has shown that they hold every intermediate
-        if (a.sum16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        if (a.sum16) N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, true, true), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
     } else {
-        if (hi16) hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, true, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
-        else hipLaunchKernelGGL((conv_pipe_kernel<NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, false, true>), dim3(grid), dim3(NW * 64), 0, stream, a);
+        if (hi16) N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, true, true), dim3(grid), dim3(NW * 64), 0, stream, a);
+        else N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, V, false, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
     }
 }
 

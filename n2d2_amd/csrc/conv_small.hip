@@ -121,9 +121,9 @@ int conv_small_launch(const ConvSmallArgs& a, hipStream_t stream)
     const dim3 grid((unsigned)((total + 255) / 256), (unsigned)((a.O + 7) / 8));
     const size_t lds = (size_t)taps * 8 * a.in_cs;
     if (a.in_cs == 4)
-        hipLaunchKernelGGL((conv_small_kernel<4>), grid, dim3(256), lds, stream, a);
+        N2D2HIP_LAUNCH_T(conv_small_kernel, (4), grid, dim3(256), lds, stream, a);
     else
-        hipLaunchKernelGGL((conv_small_kernel<16>), grid, dim3(256), lds, stream, a);
+        N2D2HIP_LAUNCH_T(conv_small_kernel, (16), grid, dim3(256), lds, stream, a);
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }

@@ -183,10 +183,10 @@ int depthwise3x3_launch(DepthwiseArgs a, int stride, int num_cus, hipStream_t st
     N2D2HIP_REQUIRE(nthreads < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "depthwise3x3: tensor too large");
     a.nthreads = (unsigned)nthreads;
     const unsigned grid = (unsigned)((nthreads + 255) / 256);
-#define N2D2HIP_DW_LAUNCH(S, K) hipLaunchKernelGGL((depthwise3x3_kernel<S, K>), dim3(grid), dim3(256), 0, stream, a)
+#define N2D2HIP_DW_LAUNCH(S, K) N2D2HIP_LAUNCH_T(depthwise3x3_kernel, (S, K), dim3(grid), dim3(256), 0, stream, a)
     if (a.epi.kind == EPI_I24 && a.fast) {
-        if (stride == 1) hipLaunchKernelGGL((depthwise3x3_kernel<1, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
-        else hipLaunchKernelGGL((depthwise3x3_kernel<2, EPI_I24, true>), dim3(grid), dim3(256), 0, stream, a);
+        if (stride == 1) N2D2HIP_LAUNCH_T(depthwise3x3_kernel, (1, EPI_I24, true), dim3(grid), dim3(256), 0, stream, a);
+        else N2D2HIP_LAUNCH_T(depthwise3x3_kernel, (2, EPI_I24, true), dim3(grid), dim3(256), 0, stream, a);
     } else if (a.epi.kind == EPI_I24) {
         if (stride == 1) N2D2HIP_DW_LAUNCH(1, EPI_I24); else N2D2HIP_DW_LAUNCH(2, EPI_I24);
     } else if (a.epi.kind == EPI_I64) {

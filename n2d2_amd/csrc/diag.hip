@@ -32,7 +32,62 @@ __global__ __launch_bounds__(256) void clock_probe_kernel(int iters, long long* 
 
 } // namespace n2d2hip
 
+#ifdef N2D2HIP_PROFILE
+#include "n2d2hip_probe.h"
+
+namespace n2d2hip {
+
+// The probe buffer of the process: device memory the caller owns, checked on the host when it is handed over.
+static long long* g_probe = nullptr;
+static long long g_probe_records = 0, g_probe_used = 0;
+
+long long* probe_take(unsigned blocks, long long* first)
+{
+    if (!g_probe || g_probe_used + (long long)blocks > g_probe_records)
+        return nullptr;
+    *first = g_probe_used;
+    long long* at = g_probe + g_probe_used * N2D2HIP_PROBE_RECORD;
+    g_probe_used += blocks;
+    return at;
+}
+
+} // namespace n2d2hip
+#endif
+
 using namespace n2d2hip;
+
+#ifdef N2D2HIP_PROFILE
+extern "C" int n2d2hip_probe_begin(void* device_buffer, size_t bytes)
+{
+    N2D2HIP_REQUIRE(device_buffer != nullptr && bytes >= N2D2HIP_PROBE_RECORD * sizeof(long long) && (uintptr_t)device_buffer % 8 == 0,
+                    N2D2HIP_ERR_INVALID, "probe_begin: an 8-byte aligned device buffer of at least one record");
+    // The buffer must be device memory of the current device and the whole range must lie inside one allocation:
+    // the kernels write through this pointer.
+    hipPointerAttribute_t attr;
+    N2D2HIP_HIP_CHECK(hipPointerGetAttributes(&attr, device_buffer));
+    int dev = 0;
+    N2D2HIP_HIP_CHECK(hipGetDevice(&dev));
+    N2D2HIP_REQUIRE(attr.type == hipMemoryTypeDevice && attr.device == dev, N2D2HIP_ERR_INVALID,
+                    "probe_begin: the buffer is not memory of the current device");
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    N2D2HIP_HIP_CHECK(hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)device_buffer));
+    N2D2HIP_REQUIRE((const char*)device_buffer + bytes <= (const char*)base + size, N2D2HIP_ERR_INVALID,
+                    "probe_begin: %zu bytes reach past the end of the allocation", bytes);
+    g_probe = (long long*)device_buffer;
+    g_probe_records = (long long)(bytes / (N2D2HIP_PROBE_RECORD * sizeof(long long)));
+    g_probe_used = 0;
+    return N2D2HIP_OK;
+}
+
+extern "C" int n2d2hip_probe_end(long long* records_used)
+{
+    if (records_used) *records_used = g_probe_used;
+    g_probe = nullptr;
+    g_probe_records = g_probe_used = 0;
+    return N2D2HIP_OK;
+}
+#endif
 
 extern "C" int n2d2hip_measure_clock(double busy_microseconds, double* mhz, n2d2hip_stream_t stream_)
 {

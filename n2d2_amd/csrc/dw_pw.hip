@@ -288,9 +288,9 @@ int byte_type_of(const n2d2hip_act_s* a) { return a->min_out >= 0 ? N2D2HIP_U8B 
 template <int S, int KC, bool FAST>
 void launch_nb(const DwPwArgs& a, int nb, dim3 grid, hipStream_t stream)
 {
-    if (nb == 8) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 8, 8, FAST>), grid, dim3(512), 0, stream, a);
-    else if (nb == 4) hipLaunchKernelGGL((dw_pw_kernel<S, KC, 4, 4, FAST>), grid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL((dw_pw_kernel<S, KC, 2, 4, FAST>), grid, dim3(256), 0, stream, a);
+    if (nb == 8) N2D2HIP_LAUNCH_T(dw_pw_kernel, (S, KC, 8, 8, FAST), grid, dim3(512), 0, stream, a);
+    else if (nb == 4) N2D2HIP_LAUNCH_T(dw_pw_kernel, (S, KC, 4, 4, FAST), grid, dim3(256), 0, stream, a);
+    else N2D2HIP_LAUNCH_T(dw_pw_kernel, (S, KC, 2, 4, FAST), grid, dim3(256), 0, stream, a);
 }
 
 template <int S, int KC>

@@ -571,7 +571,7 @@ int n2d2hip_expand_reduce_forward(n2d2hip_expand_reduce_t h, const n2d2hip_tenso
     const int rounds = (q.ntiles + cus - 1) / cus;
     const int grid = (q.ntiles + rounds - 1) / rounds;
     hipStream_t stream = (hipStream_t)stream_;
-#define N2D2HIP_ER_LAUNCH(C, P) hipLaunchKernelGGL((expand_reduce_kernel<C, P>), dim3(grid), dim3(512), 0, stream, q)
+#define N2D2HIP_ER_LAUNCH(C, P) N2D2HIP_LAUNCH_T(expand_reduce_kernel, (C, P), dim3(grid), dim3(512), 0, stream, q)
     const int pre = !ce->has_pre ? 0 : ce->pre_in_range ? 1 : 2;
     if (cmid == 128) {
         if (pre == 0) N2D2HIP_ER_LAUNCH(128, 0); else if (pre == 1) N2D2HIP_ER_LAUNCH(128, 1); else N2D2HIP_ER_LAUNCH(128, 2);

@@ -384,7 +384,7 @@ class GpuNet:
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
     def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True,
-                 dw_pw=True):
+                 dw_pw=True, s2d=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -398,6 +398,8 @@ class GpuNet:
         dw_pw: run a 3x3 depthwise convolution and the 1x1 convolution that alone reads it as one launch (n2d2hip_dw_pw_*)
         where the library takes the pair and expects the launch to be faster than the two (n2d2hip_dw_pw_pays); "all":
         wherever the library takes the pair.
+        s2d: store the network input space-to-depth (16-byte pixels of 2 x 2 input pixels, with a border of zeros) when the
+        one cell reading it is a first-layer convolution the library serves that way (n2d2hip_conv_s2d_halo).
         tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
         (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
         only ties with the two separate launches."""
@@ -590,6 +592,22 @@ class GpuNet:
                         if u is t:
                             lst[k] = nx
                 self.tensors[l.name] = nx
+        # The network input in space-to-depth form, when its one reader takes it (with its pooling, if the two are one launch)
+        if s2d and halo and len(first) == 1 and first[0].type == "conv" and len(first[0].inputs) == 1 and self.input.halo == 0:
+            m = first[0]
+            step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+            pooled = next((p for p, conv in self.stem_pools.items() if conv is m), None)
+            conv_cell = self.steps[step_index[pooled if pooled else m.name]][1]
+            pool_cell = rt.Pool(by_name[pooled].kind, by_name[pooled].pool, by_name[pooled].stride, by_name[pooled].pad) if pooled else None
+            h = conv_cell.s2d_halo(H, W, pool_cell) if isinstance(conv_cell, rt.Conv) else -1
+            out_t = self.tensors[pooled if pooled else m.name]
+            if h >= 0 and (pooled or out_t.halo == 0):
+                nx = rt.DTensor(batch, C, H, W, self.input.dtype, capi.S2D, halo=h)
+                for lst in ins_of.values():
+                    for k, t in enumerate(lst):
+                        if t is self.input:
+                            lst[k] = nx
+                self.input = self.tensors["input"] = nx
         self.bottlenecks, self.bottleneck_layers = {}, {}
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
@@ -722,6 +740,9 @@ class GpuNet:
 
     def set_input(self, x):
         """x: integer NCHW numpy array [B,C,H,W]."""
+        if self.input.layout == self.capi.S2D:
+            self.input.convert_from(self.rt.DTensor.from_numpy(x, self.capi.I32, self.capi.NCHW))
+            return
         t = self.rt.DTensor.from_numpy(x, self.input.dtype)
         h = self.input.halo
         if h:
@@ -763,6 +784,16 @@ class GpuNet:
             l, cell, fn = self.steps[k]
             ins, out = self._io[k]
             fn(cell, ins, out)
+
+    def kernel_names(self):
+        """One forward with the library's launch log open around every cell: [[kernel name, ...]] per entry of
+        self.launched, as the library itself names what it launched (template arguments included)."""
+        names = []
+        for (l, cell, fn), (ins, out) in zip(self.steps, self._io):
+            with self.capi.launch_log() as log:
+                fn(cell, ins, out)
+            names.append([e[0] for e in log.entries])
+        return names
 
     def forward_timed(self):
         """One forward with a pair of events around every cell launch, recorded on the stream the kernels run on.

@@ -26,6 +26,14 @@ class DTensor:
     def __init__(self, B, Cc, H, W, dtype, layout=capi.NHWC, buf=None, halo=0):
         """halo: border pixels stored around every image (NHWC byte tensors between two convolutions), holding the value 0."""
         self.B, self.C, self.H, self.W, self.dtype, self.layout, self.halo = B, Cc, H, W, dtype, layout, halo
+        if layout == capi.S2D:
+            # space-to-depth form of a network input: 16-byte pixels holding 2 x 2 input pixels; n2d2hip_convert writes all of it
+            self.cs = 16
+            n = B * ((H + 1) // 2 + 2 * halo) * ((W + 1) // 2 + 2 * halo) * 16
+            self.buf = buf if buf is not None else torch.empty(n, dtype=_TORCH_DT[dtype], device="cuda")
+            assert self.buf.numel() == n
+            self.desc = capi.Tensor(self.buf.data_ptr(), dtype, layout, B, Cc, H, W, 16, halo)
+            return
         self.cs = capi.nhwc_cs(Cc) if layout == capi.NHWC else Cc
         n = B * (H + 2 * halo) * (W + 2 * halo) * self.cs
         self.buf = buf if buf is not None else torch.empty(n, dtype=_TORCH_DT[dtype], device="cuda")
@@ -43,7 +51,7 @@ class DTensor:
         return self.buf.numel() * self.buf.element_size()
 
     @staticmethod
-    def from_numpy(x, dtype, layout=capi.NHWC):
+    def from_numpy(x, dtype, layout=capi.NHWC, halo=0):
         """x: integer-valued NCHW numpy array. Uploads it as I32/F32 NCHW and converts on the device."""
         x = np.ascontiguousarray(x)
         B, Cc, H, W = x.shape
@@ -53,9 +61,14 @@ class DTensor:
             src = DTensor(B, Cc, H, W, capi.I32, capi.NCHW, torch.from_numpy(x.astype(np.int32).reshape(-1)).cuda())
         if dtype == src.dtype and layout == capi.NCHW:
             return src
-        dst = DTensor(B, Cc, H, W, dtype, layout)
+        dst = DTensor(B, Cc, H, W, dtype, layout, halo=halo)
         check(lib.n2d2hip_convert(src.ref, dst.ref, stream_ptr()))
         return dst
+
+    def convert_from(self, src):
+        """Graph-edge conversion of `src` (any layout / type of the same logical shape) into this tensor."""
+        check(lib.n2d2hip_convert(src.ref, self.ref, stream_ptr()))
+        return self
 
     def with_halo(self, halo):
         """A copy of this NHWC byte tensor stored with a border of `halo` zero pixels around every image."""
@@ -246,6 +259,11 @@ class Conv:
     def forward_maxpool(self, pool, x, out):
         check(lib.n2d2hip_conv_forward_maxpool(self.handle, C.byref(pool.desc), x.ref, out.ref, stream_ptr()))
         return out
+
+    def s2d_halo(self, H, W, pool=None):
+        """Border a space-to-depth H x W input must carry for this convolution (with the max pooling `pool` behind it in the
+        same launch, if given) to read it; -1 when the library does not serve it that way."""
+        return int(lib.n2d2hip_conv_s2d_halo(self.handle, C.byref(pool.desc) if pool is not None else None, H, W))
 
     def accepts_halo(self):
         """True when this convolution reads and writes tensors that carry their padding as a border of zeros."""

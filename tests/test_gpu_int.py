@@ -918,6 +918,69 @@ def test_first_layer_conv_with_max_pool_in_one_launch_bit_exact(rt):
     assert not c64.accepts_maxpool(pool, 56, 56)
 
 
+def test_first_layer_conv_on_space_to_depth_input_bit_exact(rt):
+    """A first-layer convolution of stride 2 reading the network input in its space-to-depth form (n2d2hip_convert into
+    N2D2HIP_S2D, n2d2hip_conv_s2d_halo) equals the reference cell, alone and with the 3x3 stride-2 max pooling behind it in
+    the same launch: 7x7 / 5x5 / 3x3 kernels, even and odd paddings, odd image sizes (a last row / column that half exists),
+    1 to 4 input channels, 64 / 32 / 48 outputs, scaled-up and full integer rescales (a Clip), signed inputs and outputs,
+    batches that give a block several strips, pooled outputs with a border, conversion from int32, float and byte planes."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    import torch
+    rng = np.random.default_rng(2718)
+    cases = (  # B, C, H, W, O, k, pad, pool padding (None: no pooling), unsigned output, clip, source dtype
+        (3, 3, 224, 224, 64, 7, 3, 1, True, False, "u8"), (2, 3, 224, 224, 64, 7, 3, None, True, False, "i32"),
+        (2, 3, 64, 64, 64, 7, 3, 0, True, False, "f32"), (5, 3, 37, 45, 64, 3, 1, 1, True, False, "u8"),
+        (70, 3, 30, 22, 64, 5, 2, 1, False, False, "i32"), (1, 3, 9, 222, 64, 3, 1, 0, True, False, "u8"),
+        (2, 3, 224, 224, 32, 3, 1, None, True, False, "u8"), (3, 4, 50, 34, 48, 3, 0, None, True, False, "i32"),
+        (2, 3, 224, 224, 64, 7, 3, None, True, True, "u8"), (4, 1, 33, 33, 16, 5, 1, None, False, False, "i32"),
+        (2, 2, 96, 96, 64, 7, 2, 1, True, False, "u8"), (600, 3, 16, 16, 64, 3, 1, 1, True, False, "u8"),
+        (130, 3, 40, 40, 32, 7, 3, None, True, True, "u8"))
+    for (B, Cc, H, W, O, k, pad, ppad, unsigned, clip, src_kind) in cases:
+        print("s2d stem", B, Cc, H, W, O, k, pad, ppad, unsigned, clip, src_kind, flush=True)
+        x = rng.integers(0, 256, size=(B, Cc, H, W))
+        w = np.clip(np.rint(rng.normal(0, 30, size=(O, Cc, k, k))), -127, 127).astype(np.int64)
+        bias = rng.integers(-3000, 3000, size=O)
+        if clip:
+            spec = ActSpec("Rectifier", "FixedMult16", rng.integers(64, 256, size=O), frac_bits=16,
+                           clipping=rng.uniform(3e4, 9e4, size=O).astype(np.float32), nb_bits=8, unsigned_out=True)
+        elif unsigned:
+            spec = ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 11, size=O)], 1), nb_bits=8, unsigned_out=True)
+        else:
+            spec = ActSpec("Linear", "SingleShift", rng.integers(8, 11, size=O), nb_bits=8, unsigned_out=False)
+        conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(2, 2), pad=(pad,) * 4)
+        pool = rt.Pool("max", (3, 3), (2, 2), (ppad, ppad)) if ppad is not None else None
+        want = cells_ref.conv_cell(x, w, bias, spec, stride=(2, 2), pad=(pad,) * 4)
+        if pool is not None:
+            want = cells_ref.pool_cell(want, "max", (3, 3), (2, 2), (ppad, ppad))
+        want = want.astype(np.int64)
+        halo = conv.s2d_halo(H, W, pool)
+        assert halo >= 0, (B, Cc, H, W, O, k, pad, ppad)
+        if src_kind == "u8":
+            src = rt.DTensor(B, Cc, H, W, capi.U8, capi.NCHW, torch.from_numpy(x.astype(np.uint8).reshape(-1)).cuda())
+        elif src_kind == "f32":
+            src = rt.DTensor.from_numpy(x.astype(np.float32), capi.F32, capi.NCHW)
+        else:
+            src = rt.DTensor.from_numpy(x, capi.I32, capi.NCHW)
+        for extra in (0, 1):          # a larger border than needed is as good
+            dx = rt.DTensor(B, Cc, H, W, capi.U8B, capi.S2D, halo=halo + extra)
+            dx.buf.fill_(77)          # the conversion writes every byte of it, border included
+            dx.convert_from(src)
+            for out_halo in ((0, 1) if pool is not None else (0,)):
+                out = rt.DTensor(B, O, want.shape[2], want.shape[3], capi.U8B if unsigned else capi.I8, halo=out_halo)
+                got = (conv.forward_maxpool(pool, dx, out) if pool is not None else conv.forward(dx, out)).to_numpy()
+                assert np.array_equal(got, want), (B, Cc, H, W, O, k, pad, ppad, extra, out_halo, np.count_nonzero(got != want))
+    # what is not served says so: stride 1, a 64-channel input, a row too long
+    act = rt.Act(O, **spec.kwargs())
+    assert rt.Conv(w, bias, act, capi.U8B, stride=(1, 1), pad=(pad,) * 4).s2d_halo(64, 64) == -1
+    assert conv.s2d_halo(64, 600) == -1
+    # ... and a border that is too small is refused with a message
+    dx = rt.DTensor(2, 3, 40, 40, capi.U8B, capi.S2D, halo=0)
+    with pytest.raises(capi.N2D2HipError, match="border"):
+        conv.forward(dx, rt.DTensor(2, 32, 20, 20, capi.U8B))
+
+
 def test_expand_sum_and_next_reduce_in_one_launch_bit_exact(rt):
     """n2d2hip_expand_reduce_*: a block's 1x1 expansion with its folded sum and the next block's 1x1 reduction in one launch
     equal the reference cells run in turn (both tensors: the sum and the reduction's output); 128 and 256 middle channels,
