@@ -316,6 +316,8 @@ def kernel_phases(torch, config, batch):
              "end_spread_us": (w1.max() - w1.min()) / 100.0,
              "idle_frac": 1.0 - float((w1 - w0).sum() / 100.0) / (span_us * len(r)),
              "mhz": mhz}
+        if r[:, 8:14].max() > 0:          # kernels that time their phases: mean microseconds per unit of work
+            d["phases_us"] = [float(np.mean(r[:, 8 + k] / np.maximum(r[:, 7], 1)) / mhz) for k in range(6)]
         a = rows.setdefault(kname, [])
         a.append(d)
     keys = ["blocks", "span_us", "start_spread_us", "to_first_load_us", "to_first_mfma_us", "block_life_us", "units", "per_unit_us",
@@ -329,6 +331,10 @@ def kernel_phases(torch, config, batch):
     print("%-64s %3s " % ("kernel", "n") + " ".join("%12s" % k[:12] for k in keys))
     for kname, lst in sorted(rows.items(), key=lambda kv: -sum(d["span_us"] for d in kv[1])):
         print("%-64s %3d " % (kname[:64], len(lst)) + " ".join("%12.2f" % float(np.nanmean([d[k] for d in lst])) for k in keys))
+    for kname, lst in rows.items():
+        if "phases_us" in lst[0]:
+            print("%s: microseconds per unit of work in its phases 0..5 (see the kernel's source): %s" % (
+                kname, " ".join("%.3f" % float(np.mean([d["phases_us"][k] for d in lst])) for k in range(6))))
     total = sum(d["span_us"] for lst in rows.values() for d in lst)
     print("sum of spans of the probed launches: %.1f us (%d launches of %d in the forward)" % (total, sum(len(v) for v in rows.values()), len(launches)))
 

@@ -213,7 +213,7 @@ int n2d2hip_conv_forward(n2d2hip_conv_t conv, const n2d2hip_tensor* in, const n2
  * n2d2hip_conv_forward_maxpool with that pooling behind the convolution), or -1 when it is not served that way.
  * Served: at most 4 input channels, 8-bit weights, a square kernel of 3, 5 or 7, stride 2, no dilation, at most 64
  * outputs, integer rescale to bytes, bordered rows of at most 128 pixels; with a pooling, what
- * n2d2hip_conv_accepts_maxpool asks and rows of at most 112 outputs.  No counterpart in the reference: the stride-2
+ * n2d2hip_conv_accepts_maxpool asks and at most 62 pooled columns.  No counterpart in the reference: the stride-2
  * K x K window becomes a stride-1 window of ceil(K / 2)^2 16-byte pixels whose padding is the border of stored zeros
  * (ref: src/Cell/ConvCell_Frame_Kernels.cpp:72-83 skips those taps). */
 struct n2d2hip_pool_desc;

@@ -827,18 +827,19 @@ static int conv_s2d_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2
     a.OH = OH; a.OW = OW;
     magic_div((unsigned)a.Wp, &a.wp_mul, &a.wp_sh);
     a.out = out->data; a.out_cs = out->cs;
+    N2D2HIP_REQUIRE(n2d2hip_tensor_bytes(out) < (1ull << 31), N2D2HIP_ERR_UNSUPPORTED, "conv_forward: output too large for the first-layer kernel");
+    a.out_bytes = (int)n2d2hip_tensor_bytes(out);
     a.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
     const int cp = c->act->cpad;
     const bool hi16 = c->hi16 && !(d.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
     a.ta = c->d_epi_tab; a.tb = c->d_epi_tab + cp; a.tc = c->d_epi_tab + (hi16 ? 5 : 2) * cp;
     a.td = c->d_epi_tab + (hi16 ? 6 : 3) * cp; a.te = c->d_epi_tab + 4 * cp;
     a.lo = c->act->args.lo; a.hi = c->act->args.hi; a.preclamp = c->preclamp ? 1 : 0;
-    a.n0 = 0;
     const int ny = (d.kH + 1) / 2, nxh = (ny + 1) / 2;
     const int slots = 2 * num_cus();
     if (pd) {
-        N2D2HIP_REQUIRE(hi16 && OW <= 112 && POW <= 64 && round_up(d.O, 16) == 64, N2D2HIP_ERR_UNSUPPORTED,
-                        "conv_forward_maxpool: the pooled first-layer kernel needs scaled-up tables, 49 to 64 outputs and rows of at most 112");
+        N2D2HIP_REQUIRE(hi16 && POW <= 62 && round_up(d.O, 16) == 64, N2D2HIP_ERR_UNSUPPORTED,
+                        "conv_forward_maxpool: the pooled first-layer kernel needs scaled-up tables, 49 to 64 outputs and at most 62 pooled columns");
         a.TR = 2;
         a.pool_pad = pd->padX; a.POH = POH; a.POW = POW;
         a.pool_halo = out->halo; a.POHp = POH + 2 * out->halo; a.POWp = POW + 2 * out->halo;
@@ -864,7 +865,8 @@ static int conv_s2d_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2
     N2D2HIP_REQUIRE(a.T <= 256 && a.PF + a.T + 64 < 2048, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: space-to-depth rows too long");
     a.nstrips = in->B * a.strips_per_image;
     const int blocks = std::max(1, std::min(a.nstrips, slots));
-    return conv_s2d_launch(a, d.kH, hi16, pd != nullptr, round_up(d.O, 16) <= 32 ? 1 : 2, blocks, stream);
+    const int o16 = round_up(d.O, 16);
+    return conv_s2d_launch(a, d.kH, hi16, pd != nullptr, o16 <= 32 ? 1 : 2, blocks, 1, stream);
 }
 
 static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* other, const n2d2hip_tensor* out,
@@ -1222,7 +1224,7 @@ int n2d2hip_conv_s2d_halo(n2d2hip_conv_t c, const n2d2hip_pool_desc* pool, int H
         return halo;
     int OH, OW, POH, POW;
     const bool hi16 = c->hi16 && !(c->desc.kernel_choice & N2D2HIP_KERNEL_NO_HI16);
-    if (!stem_pool_eligible(c, pool, H, W, &OH, &OW, &POH, &POW) || !hi16 || OW > 112)
+    if (!stem_pool_eligible(c, pool, H, W, &OH, &OW, &POH, &POW) || !hi16 || POW > 62)
         return -1;
     return halo;
 }

@@ -20,18 +20,20 @@
 //    The 64 x (KS * 32) weights live in registers for the work-group's whole life.  A wave owns 32-position tiles
 //    wave, wave + 4 of the tile.
 //  * Rescale on scaled-up tables (the result is the upper half of the multiply-add), kept as pairs of 16-bit values.
-//    POOL: the pairs go to a ring of three convolution rows in LDS (a row = two columns per 256-byte block, 16-byte
-//    chunks XOR-swizzled so that neither the writes, 32 consecutive columns, nor the pooling reads, every other
-//    column, meet bank conflicts); tiles are aligned so that a pooled row's third convolution row is a tile's second,
-//    which makes one pooled row ready per tile with three rows alive.  The pooling takes the maximum of the nine
-//    16-bit pairs (saturation commutes with the maximum) and saturates and packs only the pooled values.
+//    POOL: a wave's two 32-position tiles are not consecutive positions but, lane by lane, the first and the second
+//    column of a pooled column's window, so that the maximum along the row is taken between a lane's own registers
+//    and its neighbour's (one wave shift); only the row of maxima goes to LDS, a ring of three rows (16-byte chunks
+//    XOR-swizzled by the column, so that writes and reads of consecutive columns meet no bank conflict).  Tiles are
+//    aligned so that a pooled row's third convolution row is a tile's second, which makes one pooled row ready per
+//    tile with three rows alive.  The maximum down the column is taken from LDS by one thread per pooled pixel and 16
+//    channels, which saturates and packs only the pooled values (saturation commutes with the maximum).
 #include "conv_s2d.hpp"
 #include "mfma_util.hpp"
 
 namespace n2d2hip {
 
 template <int NY, int NXH, bool H16, bool POOL, int NBLK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_s2d_kernel(ConvS2dArgs q)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 4))) void conv_s2d_kernel(ConvS2dArgs q)
 {
     static_assert(!POOL || (H16 && NBLK == 2), "the pooled variant: 64 channels, scaled-up tables");
     constexpr int KS = NY * NXH;
@@ -40,8 +42,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int TAB_OFF = RINGB;
     constexpr int TAB_BYTES = H16 ? 0 : 5 * BN * 4;
     constexpr int ROWS_OFF = TAB_OFF + TAB_BYTES;
-    constexpr int ROWB = 56 * 256;             // POOL: a convolution row of at most 112 columns, 128 bytes each
-    __shared__ __attribute__((aligned(16))) unsigned char smem[ROWS_OFF + (POOL ? 3 * ROWB : 0)];
+    constexpr int ROWB = 62 * 128;             // POOL: a row of at most 62 pooled columns, 64 channels as 16-bit values
+    constexpr int SPARE_OFF = ROWS_OFF + (POOL ? 3 * ROWB : 0);       // POOL: where lanes without an output write (8 bytes each)
+    __shared__ __attribute__((aligned(16))) unsigned char smem[SPARE_OFF + (POOL ? 512 : 0)];
     const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
 
     const int tid = threadIdx.x;
@@ -49,9 +52,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, lh = lane >> 5;
     const int Wp = q.Wp, T = q.T, NT = q.NT;
+    const int n0 = (int)blockIdx.y * BN;          // this work-group's channel tile
 #ifdef N2D2HIP_PROFILE
     long long pr_t0 = clock64(), pr_t1 = 0, pr_t2 = 0, pr_w0 = wall_clock64();
+    long long pr_ph[6] = {0, 0, 0, 0, 0, 0}, pr_last = 0;
     int pr_units = 0;
+#define S2D_MARK(k) do { const long long now__ = clock64(); pr_ph[k] += now__ - pr_last; pr_last = now__; } while (0)
+#else
+#define S2D_MARK(k) do { } while (0)
 #endif
 
     // ---- weights of this lane's channels: A operand of K step s is 16 bytes at s * 32 + 16 * lh
@@ -60,7 +68,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < NBLK; ++i)
 #pragma unroll
         for (int s = 0; s < KS; ++s)
-            wf[i][s] = *(const v4i*)(q.wk + (size_t)(q.n0 + i * 32 + l32) * (KS * 32) + s * 32 + 16 * lh);
+            wf[i][s] = *(const v4i*)(q.wk + (size_t)(n0 + i * 32 + l32) * (KS * 32) + s * 32 + 16 * lh);
     // ---- rescale: scaled-up multiplier and addend of this lane's channels (rows 8g + 4 * lh + e of each block) in
     // registers, or the five tables of the general integer rescale in LDS
     v4i rc[H16 ? NBLK : 1][H16 ? 4 : 1], rd[H16 ? NBLK : 1][H16 ? 4 : 1];
@@ -69,32 +77,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < NBLK; ++i)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                rc[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(q.tc + q.n0 + i * 32 + 8 * g + 4 * lh);
-                rd[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(q.td + q.n0 + i * 32 + 8 * g + 4 * lh);
+                rc[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(q.tc + n0 + i * 32 + 8 * g + 4 * lh);
+                rd[H16 ? i : 0][H16 ? g : 0] = *(const v4i*)(q.td + n0 + i * 32 + 8 * g + 4 * lh);
             }
     } else {
         int* tabw = (int*)(smem + TAB_OFF);
         for (int i = tid; i < BN; i += 256) {
-            tabw[i] = q.ta[q.n0 + i];
-            tabw[BN + i] = q.tb[q.n0 + i];
-            tabw[2 * BN + i] = q.tc[q.n0 + i];
-            tabw[3 * BN + i] = q.td[q.n0 + i];
-            tabw[4 * BN + i] = q.te[q.n0 + i];
+            tabw[i] = q.ta[n0 + i];
+            tabw[BN + i] = q.tb[n0 + i];
+            tabw[2 * BN + i] = q.tc[n0 + i];
+            tabw[3 * BN + i] = q.td[n0 + i];
+            tabw[4 * BN + i] = q.te[n0 + i];
         }
     }
     const unsigned tab = lds0 + TAB_OFF + (unsigned)(4 * lh) * 4u;
     const int vlo = q.lo, vhi = q.hi;
 
-    // ---- this lane's two positions inside a tile (32-position tiles wave and wave + 4): row of the tile, output column
+    // ---- this lane's two positions inside a tile: row of the tile, output column, byte offset of the position (+ lane half)
+    // from the tile's first position.
+    // Plain convolution: the tile's positions in order, 32-position tiles wave and wave + 4.
+    // POOL: a wave owns one of the tile's two convolution rows (wave & 1) and a run of 31 pooled columns (wave >> 1); lane l of
+    // its first tile computes the first column of pooled column p_col's window (2 * p_col - pad), of its second tile the
+    // second (columns off the row's ends clamped to the nearest inside, which repeats a value of the window), and the
+    // window's third column is the first of lane l + 1: the maximum along the row is taken between registers.
     int t_row[2], t_ox[2];
-    unsigned t_addr[2];          // byte offset of the position (+ lane half) from the tile's first position
+    unsigned t_addr[2];
+    const int p_col = POOL ? (wave >> 1) * 31 + l32 : 0;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int pos = (wave + 4 * j) * 32 + l32;
-        const int r = div_magic(pos, q.wp_mul, q.wp_sh);
-        t_row[j] = r;
-        t_ox[j] = pos - r * Wp - q.tx;
-        t_addr[j] = (unsigned)(pos + lh) * 16u;
+        if (POOL) {
+            const int col = min(max(2 * p_col - q.pool_pad + j, 0), q.OW - 1);
+            t_row[j] = wave & 1;
+            t_ox[j] = col;
+            t_addr[j] = (unsigned)((wave & 1) * Wp + q.tx + col + lh) * 16u;
+        } else {
+            const int pos = (wave + 4 * j) * 32 + l32;
+            const int r = div_magic(pos, q.wp_mul, q.wp_sh);
+            t_row[j] = r;
+            t_ox[j] = pos - r * Wp - q.tx;
+            t_addr[j] = (unsigned)(pos + lh) * 16u;
+        }
     }
     // byte offset of K step s inside the window: row ky' = s / NXH, pixels 2 * (s % NXH) (+ lane half)
     unsigned koff[KS];
@@ -102,6 +124,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int s = 0; s < KS; ++s)
         koff[s] = (unsigned)((s / NXH) * Wp + 2 * (s % NXH)) * 16u;
 
+    // the output through a buffer descriptor: a lane without an output stores past its end, which drops the store
+    __amdgpu_buffer_rsrc_t out_rsrc = __builtin_amdgcn_make_buffer_rsrc(q.out, 0, POOL ? 0 : q.out_bytes, 0x00020000);
     const int last_pos = q.total - 1;
     const int pf_chunks = q.PF >> 6;
     // chunk `c` (64 positions) of the stream that starts at global position g0 -> its place in the ring
@@ -129,15 +153,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         const int g0 = (b * q.Hp + row0 + q.ty) * Wp;
 
-        // every wave is done reading the ring (the previous strip's last tile), and nothing requested for that strip is
-        // still on its way into it, before it is refilled
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        // (the barriers of this kernel are bare s_barrier instructions with the waits they need written out: __syncthreads()
+        // would wait for every outstanding load, the chunks requested for later tiles included)
         // ---- fill: the first PF positions of the stream, a chunk per wave in turn
         for (int c = wave; c < pf_chunks; c += 4)
             load_chunk(g0, c);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #ifdef N2D2HIP_PROFILE
         if (pr_t1 == 0) pr_t1 = clock64();
 #endif
@@ -149,65 +170,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int c_lo = (q.PF + t * T + 63) >> 6, c_hi = (q.PF + (t + 1) * T + 63) >> 6;
                 load_chunk(g0, min(c_lo + wave, max(c_hi - 1, c_lo)));
             }
+#ifdef N2D2HIP_PROFILE
+            pr_last = clock64();
+#endif
             const unsigned tbase = (unsigned)(t * T) * 16u;
             v16i acc[2][NBLK];
-            // ---- matrix phase: this wave's (at most) two 32-position tiles
+            v4i pf[2][KS];
+            v2i hq[POOL ? 2 : 1][POOL ? 4 * NBLK : 1];          // POOL: the two tiles' rescaled values as 16-bit pairs
+            // Requests the window of 32-position tile j: K step s = two pixels of window row s / NXH
+            auto request = [&](int j) {
+                const unsigned a0 = tbase + t_addr[j];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                if ((wave + 4 * j) < NT) {
-                    v4i pf[KS];
-                    const unsigned a0 = tbase + t_addr[j];
+                for (int s = 0; s < KS; ++s)
+                    lds_read128_nowait<0>(pf[j][s], lds0 + ((a0 + koff[s]) & (unsigned)(RINGB - 1)));
+            };
+            auto multiply = [&](int j) {
 #pragma unroll
-                    for (int s = 0; s < KS; ++s) {
-                        const unsigned addr = lds0 + ((a0 + koff[s]) & (unsigned)(RINGB - 1));
-                        lds_read128_nowait<0>(pf[s], addr);
-                    }
+                for (int s = 0; s < KS; ++s)
 #pragma unroll
-                    for (int s = 0; s < KS; ++s) {
-                        // the LDS answers in order: K step s has arrived once at most KS - 1 - s reads are outstanding
-                        switch (KS - 1 - s) {
-                        case 0: wait_lgkm<0>(); break;
-                        case 1: wait_lgkm<1>(); break;
-                        case 2: wait_lgkm<2>(); break;
-                        case 3: wait_lgkm<3>(); break;
-                        case 4: wait_lgkm<4>(); break;
-                        case 5: wait_lgkm<5>(); break;
-                        case 6: wait_lgkm<6>(); break;
-                        default: wait_lgkm<7>(); break;
-                        }
-                        tie(pf[s]);
-#pragma unroll
-                        for (int i = 0; i < NBLK; ++i)
-                            acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][s], pf[s], s == 0 ? v16i{} : acc[j][i], 0, 0, 0);
-                    }
-                }
-            }
-            // the chunk requested one tile ago has landed (see the head of this file); behind the next barrier every
-            // wave's has
-            asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
-#ifdef N2D2HIP_PROFILE
-            if (pr_t2 == 0) pr_t2 = clock64();
-            ++pr_units;
-#endif
-            if (POOL)
-                __syncthreads();          // the pooling of the previous tile has read the rows this tile overwrites
-
-            // ---- rescale
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                if ((wave + 4 * j) >= NT)
-                    continue;
+                    for (int i = 0; i < NBLK; ++i)
+                        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][s], pf[j][s], s == 0 ? v16i{} : acc[j][i], 0, 0, 0);
+            };
+            // Rescales tile j (a wave's second tile past the end of a short row tile computes positions that are dropped).
+            // No branch: a lane whose position is no output writes to a spare slot / past the end of the buffer descriptor, so
+            // that this code and the matrix instructions of the other tile can be interleaved by the scheduler.
+            auto rescale = [&](int j) {
                 const int crow = row0 + t * q.TR + t_row[j];                  // convolution row of this lane's position
                 const bool ok = t_row[j] < q.TR && (unsigned)t_ox[j] < (unsigned)q.OW && (unsigned)crow < (unsigned)q.OH;
                 if constexpr (POOL) {
-                    // 16-bit pairs -> the row ring.  Chunk c of a pixel = channels 8c .. 8c + 7; a lane half ends up with the
-                    // chunks of its own parity (exchange between the halves), 4 * i + 2 * pair + lh.
-                    const int col = t_ox[j];
-                    const unsigned pix = lds0 + ROWS_OFF + (unsigned)((crow + 3) % 3) * ROWB + (unsigned)(col >> 1) * 256u;
-                    const unsigned sw = (unsigned)((col >> 1) & 15), hi8 = (unsigned)(col & 1) << 3;
+                    // 16-bit pairs of this tile (one window column per lane), kept for the maximum along the row
 #pragma unroll
                     for (int i = 0; i < NBLK; ++i) {
-                        unsigned pq[4][2];
 #pragma unroll
                         for (int g = 0; g < 4; ++g) {
                             const v4i tc = rc[H16 ? i : 0][H16 ? g : 0], td = rd[H16 ? i : 0][H16 ? g : 0];
@@ -215,21 +208,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             for (int h = 0; h < 2; ++h) {
                                 const int t0 = __mul24(acc[j][i][4 * g + 2 * h], tc[2 * h]) + td[2 * h];
                                 const int t1 = __mul24(acc[j][i][4 * g + 2 * h + 1], tc[2 * h + 1]) + td[2 * h + 1];
-                                pq[g][h] = __builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u);
+                                hq[j][i * 4 + g][h] = (int)__builtin_amdgcn_perm((unsigned)t1, (unsigned)t0, 0x07060302u);
                             }
                         }
-#pragma unroll
-                        for (int pr = 0; pr < 2; ++pr) {
-                            const auto x0 = __builtin_amdgcn_permlane32_swap(pq[2 * pr][0], pq[2 * pr + 1][0], false, false);
-                            const auto x1 = __builtin_amdgcn_permlane32_swap(pq[2 * pr][1], pq[2 * pr + 1][1], false, false);
-                            const v4i chunk = {(int)x0[0], (int)x1[0], (int)x0[1], (int)x1[1]};
-                            const unsigned c = (unsigned)(4 * i + 2 * pr + lh);
-                            if (ok)
-                                *(__attribute__((address_space(3))) v4i*)(unsigned long)(pix + (((hi8 | c) ^ sw) << 4)) = chunk;
-                        }
                     }
+                    (void)ok;
                 } else {
                     unsigned pk[NBLK][4];
+                    v4i tq[2][5];
+                    auto request_tables = [&](v4i* t5, unsigned trow) {
+                        lds_read128_nowait<0>(t5[0], trow);
+                        lds_read128_nowait<BN * 4>(t5[1], trow);
+                        lds_read128_nowait<2 * BN * 4>(t5[2], trow);
+                        lds_read128_nowait<3 * BN * 4>(t5[3], trow);
+                        lds_read128_nowait<4 * BN * 4>(t5[4], trow);
+                    };
 #pragma unroll
                     for (int i = 0; i < NBLK; ++i) {
 #pragma unroll
@@ -251,21 +244,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                                      (unsigned)__builtin_bit_cast(int, clamp_v2s(pq[0], lo1, hi1)), 0x06040200u) ^ q.out_xor;
                                 }
                             } else {
-                                const unsigned trow = tab + (unsigned)(i * 32 + 8 * g) * 4u;
-                                v4i ta, tb, tc, td, te;
-                                lds_read128_nowait<0>(ta, trow);
-                                lds_read128_nowait<BN * 4>(tb, trow);
-                                lds_read128_nowait<2 * BN * 4>(tc, trow);
-                                lds_read128_nowait<3 * BN * 4>(td, trow);
-                                lds_read128_nowait<4 * BN * 4>(te, trow);
-                                wait_lgkm<0>();
-                                tie(ta); tie(tb); tie(tc); tie(td); tie(te);
+                                // the tables of the next channel group are requested before this one is rescaled
+                                const int u = i * 4 + g;
+                                if (u == 0)
+                                    request_tables(tq[0], tab);
+                                if (u + 1 < 4 * NBLK) {
+                                    request_tables(tq[(u + 1) & 1], tab + (unsigned)(((u + 1) / 4) * 32 + 8 * ((u + 1) % 4)) * 4u);
+                                    wait_lgkm<5>();
+                                } else {
+                                    wait_lgkm<0>();
+                                }
+                                v4i* t5 = tq[u & 1];
+                                tie(t5[0]); tie(t5[1]); tie(t5[2]); tie(t5[3]); tie(t5[4]);
                                 int r[4];
 #pragma unroll
                                 for (int e = 0; e < 4; ++e) {
                                     int v = acc[j][i][4 * g + e];
-                                    if (q.preclamp) v = med3_i32(v, ta[e], tb[e]);
-                                    r[e] = med3_i32((__mul24(v, tc[e]) + td[e]) >> te[e], vlo, vhi);
+                                    if (q.preclamp) v = med3_i32(v, t5[0][e], t5[1][e]);
+                                    r[e] = med3_i32((__mul24(v, t5[2][e]) + t5[3][e]) >> t5[4][e], vlo, vhi);
                                 }
                                 pk[i][g] = pack_bytes(r[0], r[1], r[2], r[3]) ^ q.out_xor;
                             }
@@ -280,7 +276,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         const auto s13 = __builtin_amdgcn_permlane32_swap(pk[i][1], pk[i][3], false, false);
                         qd[i][0] = s02[0]; qd[i][1] = s02[1]; qd[i][2] = s13[0]; qd[i][3] = s13[1];
                     }
-                    const long long m = ((long long)b * q.OH + crow) * q.OW + t_ox[j];
+                    const int m = (b * q.OH + crow) * q.OW + t_ox[j];
                     if constexpr (NBLK == 2) {
                         v4i first, second;
 #pragma unroll
@@ -289,51 +285,103 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             first[e] = (int)x[0];
                             second[e] = (int)x[1];
                         }
-                        const int ch = q.n0 + 32 * lh;
-                        signed char* orow = (signed char*)q.out + m * q.out_cs + ch;
-                        if (ok) {
-                            if (ch < q.out_cs) *(v4i*)orow = first;
-                            if (ch + 16 < q.out_cs) *(v4i*)(orow + 16) = second;
-                        }
+                        const int ch = n0 + 32 * lh;
+                        const unsigned off = (unsigned)(m * q.out_cs + ch);
+                        __builtin_amdgcn_raw_buffer_store_b128(first, out_rsrc, (ok && ch < q.out_cs) ? off : 0x80000000u, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(second, out_rsrc, (ok && ch + 16 < q.out_cs) ? off + 16u : 0x80000000u, 0, 0);
                     } else {
                         const v4i only = {(int)qd[0][0], (int)qd[0][1], (int)qd[0][2], (int)qd[0][3]};
-                        const int ch = q.n0 + 16 * lh;
-                        if (ok && ch < q.out_cs)
-                            *(v4i*)((signed char*)q.out + m * q.out_cs + ch) = only;
+                        const int ch = n0 + 16 * lh;
+                        __builtin_amdgcn_raw_buffer_store_b128(only, out_rsrc, (ok && ch < q.out_cs) ? (unsigned)(m * q.out_cs + ch) : 0x80000000u, 0, 0);
                     }
                 }
+            };
+
+            // ---- the tile: the first 32-position tile's products, then the second's while the first is rescaled
+            request(0);
+            request(1);
+            wait_lgkm<KS>();           // the LDS answers in order: the first tile's reads have arrived
+#pragma unroll
+            for (int s = 0; s < KS; ++s) tie(pf[0][s]);
+            multiply(0);
+            S2D_MARK(0);
+            if (POOL)
+                asm volatile("s_barrier" ::: "memory");          // the pooling of the previous tile has read the rows this tile overwrites
+            S2D_MARK(1);
+            wait_lgkm<0>();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) tie(pf[1][s]);
+            multiply(1);
+            S2D_MARK(2);
+            rescale(0);
+            rescale(1);
+            if constexpr (POOL) {
+                // ---- maximum along the row: window columns 2p - pad, + 1 (this lane's two tiles) and + 2 (the first tile of the
+                // next lane, fetched by a shift of the wave by one lane; lane 31 of a half has no such neighbour and its pooled
+                // column belongs to the next run).  The row of pooled columns goes to the ring of three rows in LDS: a lane's
+                // four channels 32 * i + 8 * g + 4 * lh .. + 3 are one half (lh) of the pixel's 16-byte chunk 4 * i + g.
+                const int crow = row0 + 2 * t + (wave & 1);
+                const bool ok = l32 < 31 && p_col < q.POW && (unsigned)crow < (unsigned)q.OH;
+                const unsigned pix = lds0 + ROWS_OFF + (unsigned)((crow + 3) % 3) * ROWB + (unsigned)p_col * 128u + 8u * (unsigned)lh;
+                const unsigned sw = (unsigned)(p_col & 7);
+#pragma unroll
+                for (int u = 0; u < 4 * NBLK; ++u) {
+                    v2i hm;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int next = __builtin_amdgcn_update_dpp(0, hq[0][u][h], 0x130, 0xf, 0xf, false);       // wave_shl:1
+                        const v2s m = __builtin_elementwise_max(__builtin_elementwise_max(as_v2s(hq[0][u][h]), as_v2s(hq[POOL ? 1 : 0][u][h])), as_v2s(next));
+                        hm[h] = __builtin_bit_cast(int, m);
+                    }
+                    const unsigned at = ok ? pix + ((sw ^ (unsigned)u) << 4) : lds0 + SPARE_OFF + (unsigned)lane * 8u;
+                    *(__attribute__((address_space(3))) v2i*)(unsigned long)at = hm;
+                }
             }
+            S2D_MARK(3);
+            // Order asked of the scheduler: the first tile's matrix instructions back to back, then each of the second tile's
+            // followed by a few of the first tile's rescale instructions, which run while the matrix core is busy.
+#pragma unroll
+            for (int k = 0; k < KS * NBLK; ++k)
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+            for (int k = 0; k < KS * NBLK; ++k) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, POOL ? 5 : 6, 0);
+            }
+            // the chunk requested one tile ago has landed (see the head of this file); behind the next barrier every
+            // wave's has
+            asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+#ifdef N2D2HIP_PROFILE
+            if (pr_t2 == 0) pr_t2 = clock64();
+            ++pr_units;
+#endif
 
             if constexpr (POOL) {
                 // ---- pooled row py = pbase + t: rows 2 * py - pad .. + 2, the last of which this tile has just written
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                __syncthreads();
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                S2D_MARK(4);
                 const int py = pbase + t;
                 const int px = lane, cg = wave;
                 if (py >= py0 && py < py1 && px < q.POW) {
+                    // rows 2 * py - pad .. + 2 of the row maxima, clamped to the rows that exist: 16 channels (chunks 2 * cg, + 1)
                     v2s m[8];
+                    v4i v[3][2];
 #pragma unroll
                     for (int sy = 0; sy < 3; ++sy) {
                         const int r = min(max(2 * py - q.pool_pad + sy, 0), q.OH - 1);
-                        const unsigned rowa = lds0 + ROWS_OFF + (unsigned)(r % 3) * ROWB;
-                        v4i v[3][2];
+                        const unsigned pix = lds0 + ROWS_OFF + (unsigned)(r % 3) * ROWB + (unsigned)px * 128u;
+                        const unsigned sw = (unsigned)(px & 7);
+                        lds_read128_nowait<0>(v[sy][0], pix + ((sw ^ (unsigned)(2 * cg)) << 4));
+                        lds_read128_nowait<0>(v[sy][1], pix + ((sw ^ (unsigned)(2 * cg + 1)) << 4));
+                    }
+                    wait_lgkm<0>();
 #pragma unroll
-                        for (int sx = 0; sx < 3; ++sx) {
-                            const int col = min(max(2 * px - q.pool_pad + sx, 0), q.OW - 1);
-                            const unsigned pix = rowa + (unsigned)(col >> 1) * 256u;
-                            const unsigned sw = (unsigned)((col >> 1) & 15), hi8 = (unsigned)(col & 1) << 3;
-                            lds_read128_nowait<0>(v[sx][0], pix + (((hi8 | (unsigned)(2 * cg)) ^ sw) << 4));
-                            lds_read128_nowait<0>(v[sx][1], pix + (((hi8 | (unsigned)(2 * cg + 1)) ^ sw) << 4));
-                        }
-                        wait_lgkm<0>();
+                    for (int sy = 0; sy < 3; ++sy) {
+                        tie(v[sy][0]); tie(v[sy][1]);
 #pragma unroll
-                        for (int sx = 0; sx < 3; ++sx) {
-                            tie(v[sx][0]); tie(v[sx][1]);
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) {
-                                const v2s x = as_v2s(v[sx][e >> 2][e & 3]);
-                                m[e] = (sy == 0 && sx == 0) ? x : __builtin_elementwise_max(m[e], x);
-                            }
+                        for (int e = 0; e < 8; ++e) {
+                            const v2s x = as_v2s(v[sy][e >> 2][e & 3]);
+                            m[e] = sy == 0 ? x : __builtin_elementwise_max(m[e], x);
                         }
                     }
                     v4i res;
@@ -351,15 +399,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     const long long opix = ((long long)b * q.POHp + py + q.pool_halo) * q.POWp + px + q.pool_halo;
                     *(v4i*)((signed char*)q.out + opix * q.out_cs + cg * 16) = res;
                 }
+                S2D_MARK(5);
             } else {
-                __syncthreads();          // every wave is done with this tile's window before the chunks of tile t + 3 overwrite part of it
+                // every wave is done with this tile's window before the chunks of later tiles overwrite part of it
+                asm volatile("s_barrier" ::: "memory");
+                S2D_MARK(4);
             }
         }
+        // every wave is done reading the ring, and nothing requested for this strip is still on its way into it, before the
+        // next strip refills it
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     }
 #ifdef N2D2HIP_PROFILE
     if (tid == 0 && q.prof) {
         long long* o = q.prof + (long long)blockIdx.x * 16;
         o[0] = pr_t0; o[1] = pr_t1; o[2] = pr_t2; o[3] = clock64(); o[4] = 0; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = pr_units;
+        for (int k = 0; k < 6; ++k) o[8 + k] = pr_ph[k];
     }
 #endif
     // no load may still be writing into LDS when the block's LDS is handed to another block
@@ -419,15 +474,16 @@ int conv_s2d_halo(int k, int padT, int padL, int padB, int padR, int H, int W)
     return halo;
 }
 
-int conv_s2d_launch(ConvS2dArgs a, int k, bool hi16, bool pool, int nblk, int blocks, hipStream_t stream)
+int conv_s2d_launch(ConvS2dArgs a, int k, bool hi16, bool pool, int nblk, int blocks, int channel_tiles, hipStream_t stream)
 {
+    const dim3 grid(blocks, channel_tiles);
 #define N2D2HIP_S2D(NY, NXH)                                                                                              \
     do {                                                                                                                  \
-        if (pool) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, true, 2), dim3(blocks), dim3(256), 0, stream, a);     \
-        else if (nblk == 2 && hi16) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, false, 2), dim3(blocks), dim3(256), 0, stream, a);  \
-        else if (nblk == 2) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, false, false, 2), dim3(blocks), dim3(256), 0, stream, a);         \
-        else if (hi16) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, false, 1), dim3(blocks), dim3(256), 0, stream, a);               \
-        else N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, false, false, 1), dim3(blocks), dim3(256), 0, stream, a);                        \
+        if (pool) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, true, 2), grid, dim3(256), 0, stream, a);     \
+        else if (nblk == 2 && hi16) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, false, 2), grid, dim3(256), 0, stream, a);  \
+        else if (nblk == 2) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, false, false, 2), grid, dim3(256), 0, stream, a);         \
+        else if (hi16) N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, true, false, 1), grid, dim3(256), 0, stream, a);               \
+        else N2D2HIP_LAUNCH_T(conv_s2d_kernel, (NY, NXH, false, false, 1), grid, dim3(256), 0, stream, a);                        \
     } while (0)
     if (k == 3) N2D2HIP_S2D(2, 1);
     else if (k == 5) N2D2HIP_S2D(3, 2);

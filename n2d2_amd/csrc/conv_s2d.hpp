@@ -18,10 +18,10 @@ struct ConvS2dArgs {
     unsigned wp_mul, wp_sh;      // division by Wp
     void* out;
     int out_cs;
+    int out_bytes;               // size of the output buffer (plain convolution)
     unsigned out_xor;
     const int *ta, *tb, *tc, *td, *te;      // rescale tables (bias folded in); H16: tc, td scaled up
     int lo, hi, preclamp;
-    int n0;                      // first output channel of this launch's channel tile (always 0 today)
     // strips: a block takes strips nstrips apart; a strip is rows_per_strip consecutive rows (of pooled rows with POOL) of
     // one image, computed tile by tile (TR convolution rows each)
     int nstrips, strips_per_image, rows_per_strip;
@@ -39,7 +39,8 @@ size_t conv_s2d_weight_bytes(int O, int k, int pad);
 void conv_s2d_weight_layout(const signed char* w_ochw, int C, int O, int k, int padT, int padL, signed char* out);
 // Border (in 16-byte pixels, every side) an H x W input needs for this kernel size and padding; -1: not served.
 int conv_s2d_halo(int k, int padT, int padL, int padB, int padR, int H, int W);
-// hi16: scaled-up tables; pool: with the max pooling; nblk: 32-channel blocks (1 or 2).
-int conv_s2d_launch(ConvS2dArgs a, int k, bool hi16, bool pool, int nblk, int blocks, hipStream_t stream);
+// hi16: scaled-up tables; pool: with the max pooling; nblk: 32-channel blocks a work-group computes (1 or 2);
+// channel_tiles: work-groups along the channels (blockIdx.y), each computing 32 * nblk of them for every strip.
+int conv_s2d_launch(ConvS2dArgs a, int k, bool hi16, bool pool, int nblk, int blocks, int channel_tiles, hipStream_t stream);
 
 } // namespace n2d2hip
