@@ -221,13 +221,16 @@ __global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in
         const int xp = (int)(i % Wpairs);
         const long long r = i / Wpairs;
         const int Y = (int)(r % Hp), b = (int)(r / Hp);
-        union { signed char c[32]; uint4 v[2]; } px;
+        // the two pixels as eight dwords: dword (k >> 1) * 4 + dy * 2 + (k & 1) holds input column x0 + k of row dy, channel c in
+        // byte c
+        const unsigned zero4 = (unsigned)(zero & 255) * 0x01010101u;
+        unsigned px[8];
 #pragma unroll
-        for (int k = 0; k < 32; ++k) px.c[k] = (signed char)zero;
-        auto stored = [&](int v) -> signed char {          // logical value -> the destination's stored byte
-            if (out_dtype == N2D2HIP_U8B) return (signed char)(clamp_i32(v, 0, 255) - 128);
-            if (out_dtype == N2D2HIP_U8) return (signed char)(unsigned char)clamp_i32(v, 0, 255);
-            return (signed char)clamp_i32(v, -128, 127);
+        for (int k = 0; k < 8; ++k) px[k] = zero4;
+        auto stored = [&](int v) -> unsigned {             // logical value -> the destination's stored byte
+            if (out_dtype == N2D2HIP_U8B) return (unsigned)(clamp_i32(v, 0, 255) - 128) & 255u;
+            if (out_dtype == N2D2HIP_U8) return (unsigned)clamp_i32(v, 0, 255);
+            return (unsigned)clamp_i32(v, -128, 127) & 255u;
         };
         const int x0 = 2 * (2 * xp - halo);                  // first of the four input columns the two pixels hold
         // byte planes whose four columns are one aligned dword inside the row: one load per channel and input row
@@ -238,14 +241,19 @@ __global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in
             const int y = 2 * (Y - halo) + dy;
             if (y < 0 || y >= H)
                 continue;
-            for (int c = 0; c < C; ++c) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (c >= C)
+                    continue;
+                const unsigned keep = ~(255u << (8 * c));
                 if (quad) {
                     const unsigned w = *(const unsigned*)((const unsigned char*)in + (((size_t)b * C + c) * H + y) * (size_t)W + x0);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const int byte = (int)((w >> (8 * k)) & 255u);
                         const int v = in_dtype == N2D2HIP_U8 ? byte : (in_dtype == N2D2HIP_I8 ? (int)(signed char)byte : (int)(signed char)byte + 128);
-                        px.c[(k >> 1) * 16 + (dy * 2 + (k & 1)) * 4 + c] = stored(v);
+                        unsigned& d = px[(k >> 1) * 4 + dy * 2 + (k & 1)];
+                        d = (d & keep) | (stored(v) << (8 * c));
                     }
                 } else {
 #pragma unroll
@@ -256,15 +264,16 @@ __global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in
                         const size_t src = (in_layout == N2D2HIP_NHWC)
                             ? (((size_t)b * (H + 2 * in_halo) + y + in_halo) * (W + 2 * in_halo) + x + in_halo) * (size_t)in_cs + c
                             : (((size_t)b * C + c) * H + y) * (size_t)W + x;
-                        px.c[(k >> 1) * 16 + (dy * 2 + (k & 1)) * 4 + c] = stored(load_value(in, src, in_dtype));
+                        unsigned& d = px[(k >> 1) * 4 + dy * 2 + (k & 1)];
+                        d = (d & keep) | (stored(load_value(in, src, in_dtype)) << (8 * c));
                     }
                 }
             }
         }
         signed char* dst = out + (((size_t)b * Hp + Y) * Wp + 2 * xp) * 16;
-        *(uint4*)dst = px.v[0];
+        *(uint4*)dst = uint4{px[0], px[1], px[2], px[3]};
         if (2 * xp + 1 < Wp)
-            *(uint4*)(dst + 16) = px.v[1];
+            *(uint4*)(dst + 16) = uint4{px[4], px[5], px[6], px[7]};
     }
 }
 } // namespace n2d2hip

@@ -739,27 +739,40 @@ class GpuNet:
                 self.folded.add(gone)
 
     def set_input(self, x):
-        """x: integer NCHW numpy array [B,C,H,W]."""
-        if self.input.layout == self.capi.S2D:
-            self.input.convert_from(self.rt.DTensor.from_numpy(x, self.capi.I32, self.capi.NCHW))
-            return
-        t = self.rt.DTensor.from_numpy(x, self.input.dtype)
-        h = self.input.halo
-        if h:
+        """x: integer NCHW numpy array [B,C,H,W].  It is uploaded as the byte planes a caller would hand over (uint8 NCHW, int8
+        for a signed input) and converted on the device (convert_input)."""
+        np_t, dt = (np.uint8, self.capi.U8) if self.spec.input_unsigned else (np.int8, self.capi.I8)
+        import torch
+        lo, hi = (0, 255) if self.spec.input_unsigned else (-128, 127)          # (values outside the type saturate, as n2d2hip_convert does)
+        flat = torch.from_numpy(np.clip(np.ascontiguousarray(x), lo, hi).astype(np_t).reshape(-1)).cuda()
+        self.input_src = self.rt.DTensor(x.shape[0], x.shape[1], x.shape[2], x.shape[3], dt, self.capi.NCHW,
+                                         flat)
+        self._input_plain = None
+        if self.input.layout == self.capi.NHWC and self.input.halo:
+            self._input_plain = self.rt.DTensor(self.input.B, self.input.C, self.input.H, self.input.W, self.input.dtype)
+        self.convert_input()
+
+    def convert_input(self):
+        """The graph-edge conversion: the caller's byte planes (NCHW) into the form the first cell reads (NHWC with a channel
+        stride of 4 or 16, or space-to-depth), one launch of n2d2hip_convert."""
+        if self._input_plain is not None:
+            # an NHWC input with a border: converted without it, then copied into the interior (no configuration has one)
+            t, h = self._input_plain.convert_from(self.input_src), self.input.halo
             self.input.buf.view(t.B, t.H + 2 * h, t.W + 2 * h, t.cs)[:, h:t.H + h, h:t.W + h, :] = t.buf.view(t.B, t.H, t.W, t.cs)
         else:
-            self.input.buf.copy_(t.buf)
+            self.input.convert_from(self.input_src)
 
     def forward(self):
         for (l, cell, fn), (ins, out) in zip(self.steps, self._io):
             fn(cell, ins, out)
         return self.tensors[self.spec.output]
 
-    def capture(self, forwards=1):
+    def capture(self, forwards=1, with_input_conversion=False):
         """Records `forwards` forwards, one behind the other, into a HIP graph (every launch of the C ABI goes to the
         capturing stream and none of them allocates or clears memory) and returns a callable that replays it.  More than
         one forward per graph spreads the cost of launching a graph over them: a network of one or two kernels is
-        otherwise timed by that cost."""
+        otherwise timed by that cost.  with_input_conversion: each forward is preceded by the graph-edge conversion of the
+        byte planes set_input() left on the device."""
         import torch
         self.forward()
         torch.cuda.synchronize()
@@ -768,6 +781,8 @@ class GpuNet:
         with torch.cuda.stream(side):
             with torch.cuda.graph(graph, stream=side):
                 for _ in range(forwards):
+                    if with_input_conversion:
+                        self.convert_input()
                     self.forward()
         torch.cuda.synchronize()
         self._graph = graph

@@ -45,6 +45,20 @@ def test_lenet_config_full_batch():
     assert logits.shape == (256, 10, 1, 1) and np.abs(logits).max() > 1000
 
 
+def test_stage_convolution_config_full_batch():
+    """The single ResNet-18 stage convolution (64 -> 64, 3x3, 56x56) at its full batch of 64 against the oracle, and the same
+    result from a replayed HIP graph that holds the graph-edge conversion of the byte planes and the forward."""
+    from n2d2_amd import nets
+    spec = nets.single_conv_stage()
+    x = np.random.default_rng(21).integers(0, 256, size=(64,) + tuple(spec.in_shape))
+    net = _run_both(spec, x, [l.name for l in spec.layers])
+    want = net.tensors[spec.output].to_numpy()
+    replay = net.capture(2, with_input_conversion=True)
+    net.tensors[spec.output].buf.zero_()
+    net.input.buf.view(64, 58, 58, 64)[:, 1:57, 1:57, :].zero_()      # (the interior: the border of zeros is written once, at creation)
+    assert np.array_equal(replay().to_numpy(), want)
+
+
 @pytest.mark.parametrize("variant", ["pad1", "pad0_n2d2_model", "all_signed"])
 def test_resnet50_config(variant):
     from n2d2_amd import nets
