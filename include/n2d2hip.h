@@ -252,11 +252,12 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* desc, const n2d2hip_tensor* in
                          n2d2hip_stream_t stream);
 
 /* Pooling with a connection map (ref: src/Cell/PoolCell_Frame_Kernels.cpp:60-75,150-185, the `maps` argument of forwardMax /
- * forwardAverage): output o pools its window over every input channel c with maps[o * in->C + c] != 0 (`maps`: out->C x in->C
- * bytes in device memory), the average dividing by window size x connected channels.  An output without a connected channel
- * is 0.  `out` has out->C outputs in the dtype of `in`, no halo. */
-int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* desc, const unsigned char* maps, const n2d2hip_tensor* in,
-                                const n2d2hip_tensor* out, n2d2hip_stream_t stream);
+ * forwardAverage): output o pools its window over every input channel c with maps[o * map_channels + c] != 0 (`maps`:
+ * map_outputs x map_channels bytes in device memory, which must be the tensors' out->C x in->C: the call refuses any other
+ * size instead of reading past the map), the average dividing by window size x connected channels.  An output without a
+ * connected channel is 0.  `out` has out->C outputs in the dtype of `in`, no halo. */
+int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* desc, const unsigned char* maps, int map_outputs, int map_channels,
+                                const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream);
 
 /* Graph-level fusion of a first-layer convolution with the max pooling behind it: ConvCell_Frame::propagate followed by
  * PoolCell_Frame_Kernels::forwardMax (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/PoolCell_Frame_Kernels.cpp:102-197)

@@ -123,7 +123,7 @@ def load():
     lib.n2d2hip_fc_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_pool_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_pool_forward.argtypes = [P, P, P, P]
-    lib.n2d2hip_pool_forward_mapped.argtypes = [P, P, P, P, P]
+    lib.n2d2hip_pool_forward_mapped.argtypes = [P, P, I, I, P, P, P]
     lib.n2d2hip_elemwise_create.argtypes = [I, I, I, P, P, P, P]
     lib.n2d2hip_elemwise_destroy.argtypes = [P]
     lib.n2d2hip_elemwise_fold_input_scaling.argtypes = [P, I, P]

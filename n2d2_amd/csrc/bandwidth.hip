@@ -504,11 +504,15 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     return N2D2HIP_OK;
 }
 
-int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* d, const unsigned char* maps, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
-                                n2d2hip_stream_t stream)
+int n2d2hip_pool_forward_mapped(const n2d2hip_pool_desc* d, const unsigned char* maps, int map_outputs, int map_channels,
+                                const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
     int rc, OH, OW;
     N2D2HIP_REQUIRE(d != nullptr && maps != nullptr, N2D2HIP_ERR_INVALID, "pool_forward_mapped: null descriptor or map");
+    // the kernel reads maps[o * in->C + c] for every output and channel of the tensors: the map must have been built for them
+    N2D2HIP_REQUIRE(in != nullptr && out != nullptr && map_outputs == out->C && map_channels == in->C, N2D2HIP_ERR_INVALID,
+                    "pool_forward_mapped: the map is %d outputs x %d channels, the tensors have %d outputs and %d channels", map_outputs,
+                    map_channels, out ? out->C : 0, in ? in->C : 0);
     N2D2HIP_REQUIRE(d->pooling == N2D2HIP_POOL_MAX || d->pooling == N2D2HIP_POOL_AVERAGE, N2D2HIP_ERR_INVALID, "pool_forward_mapped: bad pooling %d", d->pooling);
     if ((rc = check_tensor(in, "pool input")) || (rc = check_tensor(out, "pool output")) || (rc = n2d2hip_pool_out_dims(d, in->H, in->W, &OH, &OW)))
         return rc;

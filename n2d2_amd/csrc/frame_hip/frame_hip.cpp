@@ -286,8 +286,18 @@ int Cell_Frame_HIP::prepareGathered()
     for (const HipTensor* t : mInputs)
         if (t->desc().dtype != dtype)
             throw std::runtime_error("Cell " + mName + ": the inputs mix signed and unsigned outputs");
-    if (mInputs.size() > 1 && (mGathered.empty() || mGathered.desc().dtype != dtype || mGathered.desc().C != (int)mNbChannels))
-        mGathered.resize((int)mBatch, (int)mNbChannels, (int)mInH, (int)mInW, dtype);
+    if (mInputs.size() > 1) {
+        // Several inputs are gathered into one tensor by an extra launch per forward (n2d2hip_concat_channels: every input
+        // read once and written once more).  They must still be what the cell was given: one batch, one size.
+        for (const HipTensor* t : mInputs)
+            if (t->desc().B != (int)mBatch || t->desc().H != (int)mInH || t->desc().W != (int)mInW)
+                throw std::runtime_error("Cell " + mName + ": an input is " + std::to_string(t->desc().B) + "x" + std::to_string(t->desc().H) + "x"
+                                         + std::to_string(t->desc().W) + " (batch x height x width), the cell was given " + std::to_string(mBatch)
+                                         + "x" + std::to_string(mInH) + "x" + std::to_string(mInW));
+        const n2d2hip_tensor& g = mGathered.desc();
+        if (mGathered.empty() || g.dtype != dtype || g.C != (int)mNbChannels || g.B != (int)mBatch || g.H != (int)mInH || g.W != (int)mInW)
+            mGathered.resize((int)mBatch, (int)mNbChannels, (int)mInH, (int)mInW, dtype);
+    }
     return dtype;
 }
 
@@ -769,6 +779,9 @@ void PoolCell_Frame_HIP<T>::setMapping(const Tensor<bool>& map)
         (void)hipFree(mMappingDevice);
         mMappingDevice = nullptr;
     }
+    // a pooling over a map is a launch of its own: the first convolution, if it was computing this pooling, runs again
+    if (!unit)
+        clearFusion();
 }
 
 template <class T>
@@ -785,32 +798,46 @@ void PoolCell_Frame_HIP<T>::initialize()
     if (mMapping.empty() && mNbOutputs != mNbChannels)
         throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": without a connection map (setMapping) the cell pools one output per "
                                  "channel, NbOutputs must be the inputs' channels");
-    if (!mMapping.empty()) {
-        // channels of one input only behind every output
-        for (std::size_t o = 0; o < mNbOutputs; ++o) {
-            int owner = -1;
-            std::size_t first = 0;
-            for (std::size_t k = 0; k < mInputs.size(); ++k) {
-                const std::size_t n = (std::size_t)mInputs[k]->desc().C;
-                for (std::size_t ch = first; ch < first + n; ++ch)
-                    if (mMapping.at(o, ch)) {
-                        if (owner >= 0 && owner != (int)k)
-                            throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": an output that pools channels of several inputs is not supported");
-                        owner = (int)k;
-                    }
-                first += n;
-            }
-        }
-        std::vector<unsigned char> host(mNbOutputs * mNbChannels);
-        for (std::size_t o = 0; o < mNbOutputs; ++o)
-            for (std::size_t ch = 0; ch < mNbChannels; ++ch)
-                host[o * mNbChannels + ch] = mMapping.at(o, ch) ? 1 : 0;
-        if (mMappingDevice) (void)hipFree(mMappingDevice);
-        mMappingDevice = nullptr;
-        checkHip(hipMalloc((void**)&mMappingDevice, host.size()), "PoolCell_Frame_HIP::initialize(): hipMalloc");
-        checkHip(hipMemcpy(mMappingDevice, host.data(), host.size(), hipMemcpyHostToDevice), "PoolCell_Frame_HIP::initialize(): hipMemcpy");
-    }
+    uploadMapping();
     mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, mInputs[0]->desc().dtype);
+}
+
+// Checks the connection map against the cell as it stands now (inputs may have been added since setMapping) and copies it
+// to the device.  Called by initialize(), and by propagate() when a map was set behind initialize().
+template <class T>
+void PoolCell_Frame_HIP<T>::uploadMapping()
+{
+    if (mMappingDevice) {
+        (void)hipFree(mMappingDevice);
+        mMappingDevice = nullptr;
+    }
+    if (mMapping.empty())
+        return;
+    if (mMapping.dimX() != mNbOutputs || mMapping.dimY() != mNbChannels)
+        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": the connection map is {" + std::to_string(mMapping.dimX()) + ", "
+                                 + std::to_string(mMapping.dimY()) + "}, the cell has " + std::to_string(mNbOutputs) + " outputs and "
+                                 + std::to_string(mNbChannels) + " channels (inputs added after setMapping?)");
+    // channels of one input only behind every output
+    for (std::size_t o = 0; o < mNbOutputs; ++o) {
+        int owner = -1;
+        std::size_t first = 0;
+        for (std::size_t k = 0; k < mInputs.size(); ++k) {
+            const std::size_t n = (std::size_t)mInputs[k]->desc().C;
+            for (std::size_t ch = first; ch < first + n; ++ch)
+                if (mMapping.at(o, ch)) {
+                    if (owner >= 0 && owner != (int)k)
+                        throw std::runtime_error("PoolCell_Frame_HIP " + mName + ": an output that pools channels of several inputs is not supported");
+                    owner = (int)k;
+                }
+            first += n;
+        }
+    }
+    std::vector<unsigned char> host(mNbOutputs * mNbChannels);
+    for (std::size_t o = 0; o < mNbOutputs; ++o)
+        for (std::size_t ch = 0; ch < mNbChannels; ++ch)
+            host[o * mNbChannels + ch] = mMapping.at(o, ch) ? 1 : 0;
+    checkHip(hipMalloc((void**)&mMappingDevice, host.size()), "PoolCell_Frame_HIP::uploadMapping(): hipMalloc");
+    checkHip(hipMemcpy(mMappingDevice, host.data(), host.size(), hipMemcpyHostToDevice), "PoolCell_Frame_HIP::uploadMapping(): hipMemcpy");
 }
 
 template <class T>
@@ -867,11 +894,14 @@ void PoolCell_Frame_HIP<T>::propagate(bool /*inference*/)
     if (mOutputs.empty() || mOutputs.desc().dtype != dtype || mOutputs.desc().halo != mOutputsHalo)
         mOutputs.resize((int)mBatch, (int)mNbOutputs, (int)mOutH, (int)mOutW, dtype, mOutputsHalo);
     const n2d2hip_pool_desc d = poolDesc();
-    if (mFusedConv)
+    // a map set behind initialize() (setMapping drops the device copy) is checked and copied now
+    if (!mMapping.empty() && !mMappingDevice)
+        uploadMapping();
+    if (mFusedConv && mMapping.empty())
         checkStatus(n2d2hip_conv_forward_maxpool(mFusedConv->convHandle(), &d, &mFusedConv->inputTensor(0)->desc(), &mOutputs.desc(), mStream));
-    else if (mMappingDevice)
-        checkStatus(n2d2hip_pool_forward_mapped(&d, mMappingDevice, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(),
-                                                mStream));
+    else if (!mMapping.empty())
+        checkStatus(n2d2hip_pool_forward_mapped(&d, mMappingDevice, (int)mNbOutputs, (int)mNbChannels,
+                                                mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     else
         checkStatus(n2d2hip_pool_forward(&d, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
     mOutputs.invalidateHost();
@@ -2078,6 +2108,13 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
         if (type == "Conv") {
             const unsigned int perGroup = getUInt(s, "Mapping.ChannelsPerGroup", 0);
             const unsigned int groups = perGroup ? cell->getNbChannels() / perGroup : getUInt(s, "Mapping.NbGroups", 1);
+            // the reference builds the groups per parent and refuses channels they do not divide
+            // (src/Generator/MappingGenerator.cpp:110-128)
+            if ((perGroup || s.count("Mapping.NbGroups")) && (groups == 0 || cell->getNbChannels() % groups != 0))
+                throw std::runtime_error("Mapping.NbGroups must be a multiple of the number of input channels in section [" + name + "]");
+            if (groups > 1 && parents.size() > 1)
+                throw std::runtime_error("Mapping: a grouped Conv with several parents is not supported in section [" + name
+                                         + "] (the reference lays one group structure per parent side by side)");
             if (groups > 1)
                 std::dynamic_pointer_cast<ConvCell>(cell)->setNbGroups(groups);
             else if (!perGroup && !s.count("Mapping.NbGroups")) {

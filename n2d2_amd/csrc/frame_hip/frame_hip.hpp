@@ -660,7 +660,8 @@ public:
     // The connection map over all inputs' channels, {nbOutputs, nbChannels}: what the `mapping` arguments of the reference's
     // addInput() calls add up to (src/Cell/Cell_Frame.cpp:100-132).  Without a call the cell pools one output per channel
     // (the Mapping.ChannelsPerGroup=1 of N2D2's model files).  An output may pool channels of one input only: the
-    // reference adds up one pooling per input there, which no model asks for.
+    // reference adds up one pooling per input there, which no model asks for.  A map set after initialize() takes effect
+    // at the next propagate(), where it is checked against the cell's channels as they are then.
     void setMapping(const Tensor<bool>& map);
     ~PoolCell_Frame_HIP();
     void initialize();
@@ -681,6 +682,7 @@ protected:
 
 private:
     n2d2hip_pool_desc poolDesc() const;
+    void uploadMapping();
     Cell_Frame_HIP* mFusedConv = nullptr;
     Tensor<bool> mMapping;                   // empty: one output per channel
     unsigned char* mMappingDevice = nullptr; // [output][channel] bytes

@@ -64,6 +64,9 @@ public:
     double applyLoss();
     bool isCuda() const { return false; }
     std::string getPyModel() const { return "Frame_HIP_QAT"; }
+    // The stream this cell's kernels are launched on: whatever a caller copies into the cell's tensors between two of its
+    // passes goes to the same stream, so that the order does not depend on a stream's implicit synchronisation.
+    void* stream() const { return mStream; }
 
 protected:
     Cell_FrameTrain_HIP() : mIn(nullptr), mDiffOut(nullptr), mStream(nullptr), mLoss(nullptr), mLossWorkspace(nullptr), mLossWorkspaceBytes(0) {}

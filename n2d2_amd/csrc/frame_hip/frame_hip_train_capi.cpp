@@ -360,14 +360,17 @@ int fh_train_learn(void* net, const float* targets, size_t nTargets, int iterati
                 if (n.inputDiffPreset.empty()) {
                     n.inputDiff.clearValid();
                 } else {
-                    if (hipMemcpyAsync(n.inputDiff.data(), n.inputDiffPreset.data(), n.inputDiff.size() * sizeof(float), hipMemcpyDeviceToDevice, nullptr)
+                    // (on the stream of the cell that will add to it, like every copy below)
+                    if (hipMemcpyAsync(n.inputDiff.data(), n.inputDiffPreset.data(), n.inputDiff.size() * sizeof(float), hipMemcpyDeviceToDevice,
+                                       (hipStream_t)n.cells.front()->stream())
                         != hipSuccess)
                         throw std::runtime_error("fh_train_learn(): copy of the preset input gradient failed");
                     n.inputDiff.setValid();
                 }
             }
             for (auto& c : n.cells) c->propagate(false);
-            if (hipMemcpyAsync(last->getDiffInputs().data(), n.targets.data(), nTargets * sizeof(float), hipMemcpyDeviceToDevice, nullptr) != hipSuccess)
+            if (hipMemcpyAsync(last->getDiffInputs().data(), n.targets.data(), nTargets * sizeof(float), hipMemcpyDeviceToDevice,
+                               (hipStream_t)last->stream()) != hipSuccess)
                 throw std::runtime_error("fh_train_learn(): copy of the targets failed");
             l = last->applyLoss();
             for (auto c = n.cells.rbegin(); c != n.cells.rend(); ++c) (*c)->backPropagate();

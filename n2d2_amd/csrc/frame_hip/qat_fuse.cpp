@@ -37,6 +37,61 @@ inline Float_T scaledWeight(Float_T q, long double factor, bool round, double si
     return (Float_T)(k * sign);
 }
 
+// How a cell's trained weights land on integers.
+struct WeightGrid {
+    long double levels = 1.0;        // integer steps per unit of trained weight (1: the weights stay as trained)
+    long double biasLevels = 1.0;    // the same for a bias expressed in accumulator units
+    double stretch = 1.0;            // 31 / 15 once a 4-bit grid has been widened to 5 bits
+    bool widened = false;            // the stage must then count its input on 31 levels
+};
+
+// Convolutions: `half` levels on either side of zero when the weights are rounded.  Default-mode 4-bit weights are odd
+// multiples of 1/15, which no 7- or 8-level grid holds: they go on 15 levels, i.e. 5 bits, and every quantity counted in
+// accumulator units is stretched by 31/15 (ref: src/Quantizer/QAT/Optimization/DeepNetQAT.cpp:988-1023).
+WeightGrid convGrid(const QATCellParameters& trained, bool rounded, std::size_t inputRange)
+{
+    WeightGrid g;
+    if (rounded)
+        g.levels = std::floor(inputRange / 2.0);
+    g.biasLevels = g.levels;
+    if (trained.weightsRange == 0)
+        return g;
+    if (rounded)
+        g.levels = trained.weightsRange > 1 ? std::floor(trained.weightsRange / 2.0) : 1;
+    const long double fourBitLevels = rounded ? 7.0 : 8.0;
+    if (trained.defaultQuantMode && g.levels == fourBitLevels) {
+        g.levels = 15.0;
+        g.stretch = 2.066666666666667;
+        g.widened = true;
+    }
+    g.biasLevels = g.levels;
+    return g;
+}
+
+// Fully-connected cells: the SAT scaling of the trained weights joins the grid when they are rounded
+// (ref: src/Quantizer/QAT/Optimization/DeepNetQAT.cpp:1130-1151).
+struct FcGrid {
+    long double levels = 1.0, satScaling = 1.0, biasLevels = 1.0;
+};
+FcGrid fcGrid(const QATCellParameters& trained, bool rounded)
+{
+    FcGrid g;
+    if (trained.weightsRange == 0)
+        return g;
+    if (rounded) {
+        g.levels = trained.weightsRange > 1 ? std::floor(trained.weightsRange / 2.0) : 1;
+        g.satScaling = trained.satScaling;
+    }
+    g.biasLevels = g.levels * g.satScaling;
+    return g;
+}
+
+// Bits of an integer cell whose trained weights had `trainedRange` levels (0: not quantized, 1: binary weights)
+std::size_t weightBits(std::size_t trainedRange)
+{
+    return bitsOf((double)(trainedRange == 0 ? 1 : (trainedRange == 1 ? 2 : trainedRange)));
+}
+
 } // namespace
 
 bool DeepNetQAT::QuantizeAndfuseBatchNormWithConv(std::pair<std::size_t, std::size_t>& rangeConvBN, std::pair<double, double>& alphasConvBN,
@@ -63,66 +118,50 @@ bool DeepNetQAT::QuantizeAndfuseBatchNormWithConv(std::pair<std::size_t, std::si
     alphasConvBN.second = (double)(Float_T)bn.actAlpha;
     rangeConvBN.second = bn.actRange;
 
-    long double weightsScaleFactor = 1.0;
-    if (wMode == WeightsApprox::RINTF)
-        weightsScaleFactor = std::floor(rangeConvBN.first / 2.0);
-    long double biasScaleFactor = weightsScaleFactor;
-    double corrFactor = 1.0;
-    if (trained.weightsRange > 0) {
-        if (wMode == WeightsApprox::RINTF)
-            weightsScaleFactor = trained.weightsRange > 1 ? std::floor(trained.weightsRange / 2.0) : 1;
-        // 4-bit weights of the default mode are odd multiples of 1/15: kept exactly on 5 bits (:1005-1017)
-        if (trained.defaultQuantMode) {
-            const long double bitRangeThreshold = wMode == WeightsApprox::RINTF ? 7.0 : 8.0;
-            if (weightsScaleFactor == bitRangeThreshold) {
-                weightsScaleFactor = 15.0;
-                corrFactor = 2.066666666666667;
-                rangeConvBN.first = 31;
-            }
-        }
-        biasScaleFactor = weightsScaleFactor;
-    }
+    const bool roundWeights = wMode == WeightsApprox::RINTF;
+    const WeightGrid grid = convGrid(trained, roundWeights, rangeConvBN.first);
+    if (grid.widened)
+        rangeConvBN.first = 31;
 
     std::shared_ptr<Activation> activation = Registrar<RectifierActivation>::create<Float_T>("Frame_HIP")();
     convCell.setActivation(activation);
     convCell.setParameter("NoBias", false);
 
-    const std::size_t perOutput = trained.quantWeights.size() / nbOutputs;
+    // Per output channel: the integer weights, then M, B and C of the head comment.  The three expressions keep the
+    // reference's operands, order and types (ref: DeepNetQAT.cpp:718-806): they decide the last bit of what is installed.
+    const double inAlpha = alphasConvBN.first, outAlpha = alphasConvBN.second;
+    const std::size_t inRange = rangeConvBN.first, outRange = rangeConvBN.second;
+    const std::size_t fanIn = trained.quantWeights.size() / nbOutputs;
     Tensor<Float_T> weights = trained.quantWeights;
     Tensor<Float_T> biases({nbOutputs});
-    std::vector<Float_T> biasPerOutput(nbOutputs, 0.0f), clipPerOutput(nbOutputs, 0.0f), scalingPerOutput(nbOutputs, 0.0f);
-    for (std::size_t output = 0; output < nbOutputs; ++output) {
-        const double factor = bn.variances[output] > 1.0e-12 ? bn.scales[output] / std::sqrt(bn.epsilon + bn.variances[output]) : 0.0;
-        const double factorSign = factor < 0.0 ? -1.0 : 1.0;
-        const double bias = noBias ? 0.0 : (double)trained.biases(output);
-        for (std::size_t index = 0; index < perOutput; ++index)
-            weights(output * perOutput + index)
-                = scaledWeight(trained.quantWeights(output * perOutput + index), weightsScaleFactor, wMode == WeightsApprox::RINTF, factorSign);
-        if (factor != 0.0) {
-            scalingPerOutput[output] = (alphasConvBN.first / (float)rangeConvBN.first) * ((float)rangeConvBN.second / alphasConvBN.second)
-                                       * factor * (1 / weightsScaleFactor) * corrFactor;
-            biasPerOutput[output] = ((((bn.biases[output] + (bias - bn.means[output]) * factor) / factor) * rangeConvBN.first
-                                      / alphasConvBN.first) * biasScaleFactor) * (1.0 / corrFactor);
-            clipPerOutput[output] = ((alphasConvBN.second * rangeConvBN.first) / (factor * alphasConvBN.first)) * weightsScaleFactor
-                                    * (1.0 / corrFactor);
-            scalingPerOutput[output] *= factorSign;
-            biasPerOutput[output] *= factorSign;
-            clipPerOutput[output] *= factorSign;
+    std::vector<Float_T> clipPerOutput(nbOutputs, 0.0f), scalingPerOutput(nbOutputs, 0.0f);
+    for (std::size_t o = 0; o < nbOutputs; ++o) {
+        // gain of the BatchNorm channel; a vanished variance leaves multiplier, bias and clip at 0: the channel outputs 0
+        const double gain = bn.variances[o] > 1.0e-12 ? bn.scales[o] / std::sqrt(bn.epsilon + bn.variances[o]) : 0.0;
+        const double side = gain < 0.0 ? -1.0 : 1.0;
+        for (std::size_t k = 0; k < fanIn; ++k)
+            weights(o * fanIn + k) = scaledWeight(trained.quantWeights(o * fanIn + k), grid.levels, roundWeights, side);
+        Float_T multiplier = 0.0f, offset = 0.0f, ceiling = 0.0f;
+        if (gain != 0.0) {
+            const double trainedBias = noBias ? 0.0 : (double)trained.biases(o);
+            multiplier = (inAlpha / (float)inRange) * ((float)outRange / outAlpha) * gain * (1 / grid.levels) * grid.stretch;
+            offset = ((((bn.biases[o] + (trainedBias - bn.means[o]) * gain) / gain) * inRange / inAlpha) * grid.biasLevels) * (1.0 / grid.stretch);
+            ceiling = ((outAlpha * inRange) / (gain * inAlpha)) * grid.levels * (1.0 / grid.stretch);
+            multiplier *= side;
+            offset *= side;
+            ceiling *= side;
         }
-        // a channel whose variance vanished (factor 0) keeps scaling, bias and clip 0: it outputs 0
         if (cMode == WeightsApprox::RINTF)
-            clipPerOutput[output] = rintf(clipPerOutput[output]);
+            ceiling = rintf(ceiling);
         if (bMode == WeightsApprox::RINTF)
-            biasPerOutput[output] = rintf(biasPerOutput[output]);
-        biases(output) = biasPerOutput[output];
+            offset = rintf(offset);
+        scalingPerOutput[o] = multiplier;
+        clipPerOutput[o] = ceiling;
+        biases(o) = offset;
     }
     convCell.setWeights(weights);
     convCell.setBiases(biases);
-
-    std::size_t weightsRange = trained.weightsRange > 0 ? trained.weightsRange : 1;
-    if (trained.weightsRange == 1)
-        weightsRange = 2;                // 1-bit weights
-    convCell.setQuantized(bitsOf((double)weightsRange));
+    convCell.setQuantized(weightBits(trained.weightsRange));
     activation->setQuantized(bitsOf((double)rangeConvBN.second));
 
     const bool isClipped = true;
@@ -166,50 +205,43 @@ bool DeepNetQAT::QuantizeFC(std::pair<std::size_t, std::size_t>& rangeOpFc, std:
         alphaOpFC.second = (double)(Float_T)actAlpha;
         rangeOpFc.second = actRange;
     }
-    long double weightsScaleFactor = 1.0;
-    long double biasScaleFactor = weightsScaleFactor;
-    long double SAT_scaling = 1.0;
-    if (trained.weightsRange > 0) {
-        if (wMode == WeightsApprox::RINTF) {
-            weightsScaleFactor = trained.weightsRange > 1 ? std::floor(trained.weightsRange / 2.0) : 1;
-            SAT_scaling = trained.satScaling;
-        }
-        biasScaleFactor = weightsScaleFactor * SAT_scaling;
-    }
-    const double scaleFactorInput = rangeOpFc.first / alphaOpFC.first;
-    double scaleFactorOutput = rangeOpFc.first;
+    const bool roundWeights = wMode == WeightsApprox::RINTF;
+    const FcGrid grid = fcGrid(trained, roundWeights);
+    // levels per unit of the input and of the output activation (an unquantized output counts in the input's levels)
+    const double inLevelsPerUnit = rangeOpFc.first / alphaOpFC.first;
+    double outLevelsPerUnit = rangeOpFc.first;
     if (actRange > 0)
-        scaleFactorOutput = rangeOpFc.second / alphaOpFC.second;
+        outLevelsPerUnit = rangeOpFc.second / alphaOpFC.second;
 
-    const std::size_t perOutput = trained.quantWeights.size() / nbOutputs;
+    // One multiplier and one ceiling for the whole cell, a bias per output; operands, order and types are the reference's
+    // (ref: DeepNetQAT.cpp:1152-1215).
+    const std::size_t fanIn = trained.quantWeights.size() / nbOutputs;
     Tensor<Float_T> weights = trained.quantWeights;
     Tensor<Float_T> biases({nbOutputs});
-    std::vector<Float_T> biasPerOutput(nbOutputs, 0.0f), clipPerOutput(nbOutputs, 0.0f), scalingPerOutput(nbOutputs, 0.0f);
-    for (std::size_t output = 0; output < nbOutputs; ++output) {
-        for (std::size_t index = 0; index < perOutput; ++index)
-            weights(output * perOutput + index) = scaledWeight(trained.quantWeights(output * perOutput + index),
-                                                               weightsScaleFactor * SAT_scaling, wMode == WeightsApprox::RINTF, 1.0);
-        scalingPerOutput[output] = (scaleFactorOutput / scaleFactorInput) * (1.0 / (SAT_scaling * weightsScaleFactor));
-        clipPerOutput[output] = alphaOpFC.second * scaleFactorInput * (weightsScaleFactor * SAT_scaling);
+    std::vector<Float_T> clipPerOutput(nbOutputs, 0.0f), scalingPerOutput(nbOutputs, 0.0f);
+    for (std::size_t o = 0; o < nbOutputs; ++o) {
+        for (std::size_t k = 0; k < fanIn; ++k)
+            weights(o * fanIn + k) = scaledWeight(trained.quantWeights(o * fanIn + k), grid.levels * grid.satScaling, roundWeights, 1.0);
+        Float_T multiplier = (outLevelsPerUnit / inLevelsPerUnit) * (1.0 / (grid.satScaling * grid.levels));
+        Float_T ceiling = alphaOpFC.second * inLevelsPerUnit * (grid.levels * grid.satScaling);
+        Float_T offset = 0.0f;
         if (!noBias)
-            biasPerOutput[output] = (double)trained.biases(output) * scaleFactorInput * biasScaleFactor;
-        if (clipPerOutput[output] < 0.0)
-            clipPerOutput[output] = 0.0;
+            offset = (double)trained.biases(o) * inLevelsPerUnit * grid.biasLevels;
+        if (ceiling < 0.0)
+            ceiling = 0.0;
         if (cMode == WeightsApprox::RINTF)
-            clipPerOutput[output] = rintf(clipPerOutput[output]);
+            ceiling = rintf(ceiling);
         if (bMode == WeightsApprox::RINTF && !noBias)
-            biasPerOutput[output] = rintf(biasPerOutput[output]);
-        biases(output) = biasPerOutput[output];
+            offset = rintf(offset);
+        scalingPerOutput[o] = multiplier;
+        clipPerOutput[o] = ceiling;
+        biases(o) = offset;
     }
     fcCell.setWeights(weights);
     fcCell.setParameter("NoBias", noBias);       // the integer cell takes over the trained cell's NoBias
     if (!noBias)
         fcCell.setBiases(biases);
-
-    std::size_t weightsRange = trained.weightsRange > 0 ? trained.weightsRange : 1;
-    if (trained.weightsRange == 1)
-        weightsRange = 2;
-    fcCell.setQuantized(bitsOf((double)weightsRange));
+    fcCell.setQuantized(weightBits(trained.weightsRange));
     const bool isClipped = actRange > 0;
     const std::size_t activationsRange = isClipped ? rangeOpFc.second : (std::size_t)(std::pow(2, 32) - 1);
     activation->setActivationScaling(Scaling::floatingPointScaling(scalingPerOutput, isClipped, clipPerOutput));

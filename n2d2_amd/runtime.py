@@ -347,7 +347,8 @@ class Pool:
             if x.C != self.nb_channels or out.C != self.nb_outputs:
                 raise ValueError("Pool: the map is %d channels x %d outputs, the tensors have %d and %d"
                                  % (self.nb_channels, self.nb_outputs, x.C, out.C))
-            check(lib.n2d2hip_pool_forward_mapped(C.byref(self.desc), self.maps.data_ptr(), x.ref, out.ref, stream_ptr()))
+            check(lib.n2d2hip_pool_forward_mapped(C.byref(self.desc), self.maps.data_ptr(), self.nb_outputs, self.nb_channels, x.ref, out.ref,
+                                                  stream_ptr()))
         return out
 
 

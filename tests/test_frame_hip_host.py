@@ -363,6 +363,23 @@ def test_conv_mapping_sets_the_groups(fh):
         net.set_mapping("fc", np.ones((16, 16)))
 
 
+def test_grouped_conv_sections_are_checked_as_the_generator_does(fh):
+    """Conv sections with Mapping.NbGroups / Mapping.ChannelsPerGroup: channels the groups do not divide are refused
+    (src/Generator/MappingGenerator.cpp:110-128 throws there; an integer division would quietly make other groups), and so
+    is a grouped Conv over several parents, whose groups the reference lays per parent."""
+    ini = INI % "Frame_HIP"
+    ok = ini.replace("[dw] conv_def\nInput=sum\nKernelDims=3 3\nNbOutputs=16\nPadding=1\nMapping.ChannelsPerGroup=1",
+                     "[dw] conv_def\nInput=sum\nKernelDims=3 3\nNbOutputs=16\nPadding=1\nMapping.ChannelsPerGroup=4")
+    assert ok != ini
+    fh.Net(ok)                                          # 16 channels in groups of 4: accepted
+    with pytest.raises(fh.FrameHipError, match="must be a multiple of the number of input channels"):
+        fh.Net(ok.replace("Mapping.ChannelsPerGroup=4", "Mapping.ChannelsPerGroup=5"))
+    with pytest.raises(fh.FrameHipError, match="must be a multiple of the number of input channels"):
+        fh.Net(ok.replace("Mapping.ChannelsPerGroup=4", "Mapping.NbGroups=3"))
+    with pytest.raises(fh.FrameHipError, match="several parents"):
+        fh.Net(ok.replace("[dw] conv_def\nInput=sum", "[dw] conv_def\nInput=sum,pool1"))
+
+
 def test_quantization_files_round_trip(fh, tmp_path):
     """DeepNet::saveQuantization / loadQuantization: what the quantization pass leaves in the cells beside their weights
     (bit widths, Scaling mode, factors, fractional bits, clip) goes through one text file per cell and comes back bit

@@ -546,6 +546,25 @@ def test_pool_cells_with_connection_maps(fh):
                                                     ("p_two", "max", 2, 2, 0, two, np.concatenate([c1, c2], 1))):
         ref = cells.pool_cell(src, kind, (pool, pool), (stride, stride), (pad, pad), maps=maps)
         assert np.array_equal(net.outputs(name), ref), name
+    # A map set after initialize() is used by the next propagate (it is not silently ignored), also where the cell has as
+    # many outputs as channels, and a map of the wrong size is refused
+    b2 = nets._Builder("late", (1, 14, 14), 84, "SingleShift")
+    t = b2.conv("c1", "input", 6, 3)
+    b2.pool("p", t, "max", 2, 2)
+    spec2 = b2.spec
+    net2 = fh.Net(fh.spec_to_ini(spec2, 3))
+    fh.install_parameters(net2, spec2)
+    net2.initialize()
+    net2.set_stimuli(x)
+    net2.propagate()
+    c1 = net2.outputs("c1")
+    assert np.array_equal(net2.outputs("p"), cells.pool_cell(c1, "max", (2, 2), (2, 2), (0, 0)))
+    late = np.roll(np.eye(6, dtype=np.uint8), 1, axis=1) | np.eye(6, dtype=np.uint8)        # [channel][output]: outputs pool two channels
+    net2.set_mapping("p", late.T)
+    net2.propagate()
+    assert np.array_equal(net2.outputs("p"), cells.pool_cell(c1, "max", (2, 2), (2, 2), (0, 0), maps=late))
+    with pytest.raises(RuntimeError, match="nbOutputs, nbChannels"):
+        net2.set_mapping("p", np.ones((6, 5)))
 
 
 def test_cells_with_two_outputs_through_the_registrar(fh):

@@ -536,7 +536,7 @@ def test_pool_with_a_connection_map_refuses_tensors_that_do_not_fit(rt):
     with pytest.raises(ValueError, match="the map is"):                   # a map for another number of channels
         rt.Pool("max", (2, 2), (2, 2), maps=np.ones((5, 3), dtype=np.uint8)).forward(x)
     with pytest.raises(capi.N2D2HipError, match="null descriptor or map"):
-        capi.check(rt.lib.n2d2hip_pool_forward_mapped(rt.C.byref(pool.desc), None, x.ref, pool.make_output(x).ref, rt.stream_ptr()))
+        capi.check(rt.lib.n2d2hip_pool_forward_mapped(rt.C.byref(pool.desc), None, 0, 0, x.ref, pool.make_output(x).ref, rt.stream_ptr()))
 
 
 def test_global_average_pool_bit_exact(rt):
