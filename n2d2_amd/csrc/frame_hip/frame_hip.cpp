@@ -58,6 +58,28 @@ void HipTensor::resize(int B, int C, int H, int W, int dtype, int halo, bool sti
     }
 }
 
+void HipTensor::resizeSpaceToDepth(int B, int C, int H, int W, int dtype, int halo)
+{
+    n2d2hip_tensor d = {};
+    d.halo = halo;
+    d.dtype = dtype;
+    d.layout = N2D2HIP_S2D;
+    d.B = B; d.C = C; d.H = H; d.W = W;
+    d.cs = 16;
+    const size_t bytes = n2d2hip_tensor_bytes(&d);
+    if (mDesc.data && bytes == mBytes) {
+        d.data = mDesc.data;
+    } else {
+        if (mDesc.data)
+            (void)hipFree(mDesc.data);
+        mDesc.data = nullptr;
+        checkHip(hipMalloc(&d.data, bytes), "HipTensor::resizeSpaceToDepth(): hipMalloc");
+        mBytes = bytes;
+    }
+    mDesc = d;
+    mHostValid = false;
+}
+
 const Tensor<Float_T>& HipTensor::synchronizeDToH(void* stream)
 {
     if (mHostValid)
@@ -91,11 +113,12 @@ void HipTensor::synchronizeHToD(const Tensor<Float_T>& host, void* stream)
         throw std::runtime_error("HipTensor::synchronizeHToD(): empty tensor");
     if (host.dimX() != (size_t)mDesc.W || host.dimY() != (size_t)mDesc.H || host.dimZ() != (size_t)mDesc.C || host.dimB() != (size_t)mDesc.B)
         throw std::runtime_error("HipTensor::synchronizeHToD(): host tensor dimensions do not match");
-    if (mDesc.halo != 0)
+    if (mDesc.halo != 0 && mDesc.layout != N2D2HIP_S2D)
         throw std::runtime_error("HipTensor::synchronizeHToD(): tensors with a halo are written by convolutions only");
     n2d2hip_tensor f = mDesc;
     f.dtype = N2D2HIP_F32;
     f.layout = N2D2HIP_NCHW;
+    f.halo = 0;
     checkHip(hipMalloc(&f.data, host.size() * sizeof(float)), "HipTensor::synchronizeHToD(): hipMalloc");
     hipError_t e = hipMemcpy(f.data, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice);
     int rc = N2D2HIP_OK;
@@ -858,7 +881,9 @@ bool PoolCell_Frame_HIP<T>::fuseFirstConv(Cell_Frame_HIP* conv)
         return false;
     const n2d2hip_pool_desc d = poolDesc();
     const n2d2hip_tensor& x = conv->inputTensor(0)->desc();
-    if (x.halo != 0 || !n2d2hip_conv_accepts_maxpool(conv->convHandle(), &d, x.H, x.W))
+    // (a space-to-depth input is the network's: its border is part of its form, and the library takes the pair on both forms
+    // or says so when the launch is planned)
+    if ((x.halo != 0 && x.layout != N2D2HIP_S2D) || !n2d2hip_conv_accepts_maxpool(conv->convHandle(), &d, x.H, x.W))
         return false;
     mFusedConv = conv;
     conv->setFoldedInto(this);
@@ -1612,7 +1637,43 @@ void DeepNet::setStimuliData(const Tensor<Float_T>& data)
         mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, dtype, 0, true);
     for (size_t i = 0; i < data.size(); ++i)
         toInteger(data(i), dtype == N2D2HIP_U8B ? 0 : -128, dtype == N2D2HIP_U8B ? 255 : 127, "stimuli");
+    mStimuliHost = data;          // (the fusion plan may change the stimuli's layout on the device: they are converted again then)
     mStimuli.synchronizeHToD(data);
+}
+
+// The stimuli go to the device space-to-depth when the one cell reading them is a first-layer convolution the device
+// library serves that way (n2d2hip_conv_s2d_halo), with the max pooling that convolution computes, if it does; otherwise
+// as plain NHWC pixels.  Called by planFusion(), behind the decision about that pooling.
+void DeepNet::layoutStimuli()
+{
+    if (mStimuli.empty())
+        return;
+    Cell_Frame_HIP* reader = nullptr;
+    size_t readers = 0;
+    for (Cell_Frame_HIP* f : mFrames)
+        for (size_t k = 0; k < f->nbInputs(); ++k)
+            if (f->inputTensor(k) == &mStimuli) { reader = f; ++readers; }
+    int halo = -1;
+    if (mFusion && readers == 1 && reader->convHandle() && reader->nbInputs() == 1) {
+        const n2d2hip_pool_desc* pd = nullptr;
+        n2d2hip_pool_desc d;
+        if (auto* pool = dynamic_cast<PoolCell_Frame_HIP<float>*>(reader->foldedInto())) {
+            d = pool->poolDescriptor();
+            pd = &d;
+        }
+        if (!reader->foldedInto() || pd)
+            halo = n2d2hip_conv_s2d_halo(reader->convHandle(), pd, (int)mEnvH, (int)mEnvW);
+    }
+    const n2d2hip_tensor& now = mStimuli.desc();
+    const bool wantS2d = halo >= 0;
+    if (wantS2d == (now.layout == N2D2HIP_S2D) && (!wantS2d || now.halo == halo))
+        return;
+    if (wantS2d)
+        mStimuli.resizeSpaceToDepth((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, now.dtype, halo);
+    else
+        mStimuli.resize((int)mEnvB, (int)mEnvC, (int)mEnvH, (int)mEnvW, now.dtype, 0, true);
+    if (!mStimuliHost.empty())
+        mStimuli.synchronizeHToD(mStimuliHost);
 }
 
 void DeepNet::initialize()
@@ -1629,8 +1690,14 @@ void DeepNet::propagate(bool /*inference*/)
     bool rebuilt = false;
     for (Cell_Frame_HIP* f : mFrames)
         rebuilt = f->prepare() || rebuilt;
-    if (mFusion && (rebuilt || !mPlanned))
-        planFusion();
+    if (rebuilt || !mPlanned) {
+        if (mFusion) {
+            planFusion();
+        } else {
+            layoutStimuli();
+            mPlanned = true;
+        }
+    }
     for (Cell_Frame_HIP* f : mFrames) {
         if (!f->foldedInto())
             f->launch();
@@ -1679,6 +1746,7 @@ void DeepNet::planFusion()
         if (parents.size() == 1 && parents[0] && consumers[parents[0]] == 1)
             pool->fuseFirstConv(parents[0]);
     }
+    layoutStimuli();
     // a 1x1 convolution that is the only reader of a 3x3 depthwise convolution computes it in its own launch
     for (Cell_Frame_HIP* f : mFrames) {
         auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f);

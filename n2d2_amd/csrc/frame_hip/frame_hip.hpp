@@ -135,6 +135,9 @@ public:
     // stimuli: the network's input, which may use the 4-byte channel stride the first-layer kernel reads; what a cell
     // writes always has a stride that is a multiple of 16.
     void resize(int B, int C, int H, int W, int dtype, int halo = 0, bool stimuli = false);
+    // The network's input in the space-to-depth form a first-layer convolution of stride 2 reads (N2D2HIP_S2D), with a
+    // border of `halo` 16-byte pixels; synchronizeHToD() fills all of it.
+    void resizeSpaceToDepth(int B, int C, int H, int W, int dtype, int halo);
     const n2d2hip_tensor& desc() const { return mDesc; }
     bool empty() const { return mDesc.data == nullptr; }
     void invalidateHost() { mHostValid = false; }
@@ -421,6 +424,7 @@ public:
     void setFoldedInto(Cell_Frame_HIP* consumer) { mFoldedInto = consumer; }
     const std::vector<Cell_Frame_HIP*>& parentCells() const { return mParentCells; }
     HipTensor* inputTensor(size_t k) const { return mInputs.at(k); }
+    size_t nbInputs() const { return mInputs.size(); }
     // Device handles a consumer borrows when it folds this cell (null for cells that cannot be folded)
     virtual n2d2hip_act_t scalingHandle() const { return nullptr; }
     virtual n2d2hip_conv_t convHandle() const { return nullptr; }
@@ -676,6 +680,8 @@ public:
     // Can this cell's launch store its output with a border of zeros around every image?  The launch that also computes
     // the first convolution can, and so can the stand-alone 2x2 / 3x3 max pooling of 16-byte channel groups.
     bool writesHalo() const;
+    // The pooling as the device library's descriptor
+    n2d2hip_pool_desc poolDescriptor() const { return poolDesc(); }
 
 protected:
     void setOutputsDims();
@@ -1097,6 +1103,8 @@ public:
 
 private:
     void planFusion();
+    void layoutStimuli();
+    Tensor<Float_T> mStimuliHost;          // what setStimuliData() was given last
     bool mFusion = true, mPlanned = false;
     std::vector<std::shared_ptr<Cell> > mOrder;
     std::vector<Cell_Frame_HIP*> mFrames;  // mOrder, as the cells' device side

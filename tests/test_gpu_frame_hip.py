@@ -64,9 +64,16 @@ def test_resnet50_through_the_registrar(fh):
     net.set_stimuli(x2)
     net.propagate()
     assert np.array_equal(net.outputs("fc"), cells.run_net(spec, x2)["fc"])
+    # the stimuli sit on the device space-to-depth and the first launch is the kernel that reads them so, pooling included
+    from n2d2_amd import capi
+    with capi.launch_log() as log:
+        net.propagate()
+    assert log.entries[0][0].startswith("conv_s2d_kernel<4, 2, true, true, 2>") and len(log.entries) == 52
     # without fusion every cell is launched and readable
     net.set_fusion(False)
-    net.propagate()
+    with capi.launch_log() as log:
+        net.propagate()
+    assert not any(e[0].startswith("conv_s2d_kernel") for e in log.entries)
     assert net.nb_folded == 0 and net.nb_halo == 0
     keep = ["conv1", "pool1", "conv2.1_1x1", "conv2.1_3x3", "conv2.1_1x1_proj", "conv2.2_shortcut_rescale", "conv2.2_1x1_x4",
             "conv2.2_sum", "fc"]
