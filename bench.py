@@ -395,10 +395,13 @@ def main():
         B = args.batch or batch
         net = nets.GpuNet(spec, B)
         net.set_input(np.random.default_rng(2025).integers(0, 256, size=(B,) + tuple(spec.in_shape)))
-        step = net.forward if args.no_graph else net.capture(per_graph)
+        def eager():
+            net.convert_input()
+            return net.forward()
+        step = eager if args.no_graph else net.capture(per_graph, with_input_conversion=True)
         ms, mean_ms, wall_ms = median_step_ms(torch, step, args.steps, args.warmup, 1 if args.no_graph else per_graph)
         print(json.dumps({"forward_only": args.config, "batch": B, "value": round(B / (ms * 1e-3), 1), "unit": "images/s",
-                          "ms_per_step": round(ms, 4), "launches_per_step": len(net.launched),
+                          "ms_per_step": round(ms, 4), "launches_per_step": len(net.launched) + 1, "step_is": "graph-edge conversion + forward",
                           "launch": "eager" if args.no_graph else "hipGraph replay, %d forwards per graph" % per_graph,
                           "steps": args.steps, "warmup": args.warmup}))
         return

@@ -215,12 +215,12 @@ __global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in
                                                      signed char* __restrict__ out, int out_dtype, int B, int C, int H, int W, int halo)
 {
     const int Hp = (H + 1) / 2 + 2 * halo, Wp = (W + 1) / 2 + 2 * halo, Wpairs = (Wp + 1) / 2;
-    const long long total = (long long)B * Hp * Wpairs;
     const int zero = out_dtype == N2D2HIP_U8B ? -128 : 0;
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
-        const int xp = (int)(i % Wpairs);
-        const long long r = i / Wpairs;
-        const int Y = (int)(r % Hp), b = (int)(r / Hp);
+    // a wave per row of the stored image (4 rows per block), lanes along the row: no division by the row length
+    const int rows = B * Hp;
+    for (int row = (int)blockIdx.x * 4 + (int)(threadIdx.x >> 6); row < rows; row += (int)gridDim.x * 4)
+    for (int xp = (int)(threadIdx.x & 63); xp < Wpairs; xp += 64) {
+        const int b = row / Hp, Y = row - b * Hp;
         // the two pixels as eight dwords: dword (k >> 1) * 4 + dy * 2 + (k & 1) holds input column x0 + k of row dy, channel c in
         // byte c
         const unsigned zero4 = (unsigned)(zero & 255) * 0x01010101u;
@@ -233,29 +233,71 @@ __global__ __launch_bounds__(256) void to_s2d_kernel(const void* __restrict__ in
             return (unsigned)clamp_i32(v, -128, 127) & 255u;
         };
         const int x0 = 2 * (2 * xp - halo);                  // first of the four input columns the two pixels hold
-        // byte planes whose four columns are one aligned dword inside the row: one load per channel and input row
-        const bool quad = in_layout == N2D2HIP_NCHW && in_dtype != N2D2HIP_I32 && in_dtype != N2D2HIP_F32 && (W & 3) == 0 && (x0 & 3) == 0
-            && x0 >= 0 && x0 + 3 < W && 2 * xp + 1 < Wp;
+        // Byte planes whose four columns are one aligned dword inside the row: one load per channel and input row, all eight
+        // requested before the first is used (a lane whose dword does not exist reads the tensor's first one and drops it)
+        const bool planes = in_layout == N2D2HIP_NCHW && in_dtype != N2D2HIP_I32 && in_dtype != N2D2HIP_F32 && (W & 3) == 0 && (halo & 1) == 0;
+        if (planes) {
+            const bool cols = x0 >= 0 && x0 + 3 < W;          // (x0 is a multiple of 4 and so is W: all four columns or none)
+            unsigned w[2][4];
+            bool have[2];
 #pragma unroll
-        for (int dy = 0; dy < 2; ++dy) {
-            const int y = 2 * (Y - halo) + dy;
-            if (y < 0 || y >= H)
-                continue;
+            for (int dy = 0; dy < 2; ++dy) {
+                const int y = 2 * (Y - halo) + dy;
+                have[dy] = cols && y >= 0 && y < H;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (c >= C)
-                    continue;
-                const unsigned keep = ~(255u << (8 * c));
-                if (quad) {
-                    const unsigned w = *(const unsigned*)((const unsigned char*)in + (((size_t)b * C + c) * H + y) * (size_t)W + x0);
+                for (int c = 0; c < 4; ++c) {
+                    const size_t at = (have[dy] && c < C) ? (((size_t)b * C + c) * H + y) * (size_t)W + x0 : 0;
+                    w[dy][c] = *(const unsigned*)((const unsigned char*)in + at);
+                }
+            }
+            // stored forms that differ by the sign bit at most (uint8 planes into the value - 128 form, or the same form on both
+            // sides): the bytes are flipped four at a time and a 4 x 4 byte transpose puts the channels of a column side by side
+            const bool same = in_dtype == out_dtype || (in_dtype == N2D2HIP_U8 && out_dtype == N2D2HIP_U8B) || (in_dtype == N2D2HIP_U8B && out_dtype == N2D2HIP_U8);
+            if (same) {
+                const unsigned flip = in_dtype == out_dtype ? 0u : 0x80808080u;
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const int byte = (int)((w >> (8 * k)) & 255u);
-                        const int v = in_dtype == N2D2HIP_U8 ? byte : (in_dtype == N2D2HIP_I8 ? (int)(signed char)byte : (int)(signed char)byte + 128);
-                        unsigned& d = px[(k >> 1) * 4 + dy * 2 + (k & 1)];
-                        d = (d & keep) | (stored(v) << (8 * c));
+                for (int dy = 0; dy < 2; ++dy) {
+                    if (!have[dy])
+                        continue;
+                    unsigned ch[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        ch[c] = c < C ? (w[dy][c] ^ flip) : zero4;
+                    const unsigned ab_lo = __builtin_amdgcn_perm(ch[1], ch[0], 0x05010400u), ab_hi = __builtin_amdgcn_perm(ch[1], ch[0], 0x07030602u);
+                    const unsigned cd_lo = __builtin_amdgcn_perm(ch[3], ch[2], 0x05010400u), cd_hi = __builtin_amdgcn_perm(ch[3], ch[2], 0x07030602u);
+                    px[0 * 4 + dy * 2 + 0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100u);      // column x0
+                    px[0 * 4 + dy * 2 + 1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302u);      // column x0 + 1
+                    px[1 * 4 + dy * 2 + 0] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100u);      // column x0 + 2
+                    px[1 * 4 + dy * 2 + 1] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302u);      // column x0 + 3
+                }
+            } else {
+#pragma unroll
+                for (int dy = 0; dy < 2; ++dy)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        if (!have[dy] || c >= C)
+                            continue;
+                        const unsigned keep = ~(255u << (8 * c));
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            const int byte = (int)((w[dy][c] >> (8 * k)) & 255u);
+                            const int v = in_dtype == N2D2HIP_U8 ? byte : (in_dtype == N2D2HIP_I8 ? (int)(signed char)byte : (int)(signed char)byte + 128);
+                            unsigned& d = px[(k >> 1) * 4 + dy * 2 + (k & 1)];
+                            d = (d & keep) | (stored(v) << (8 * c));
+                        }
                     }
-                } else {
+            }
+        } else {
+#pragma unroll
+            for (int dy = 0; dy < 2; ++dy) {
+                const int y = 2 * (Y - halo) + dy;
+                if (y < 0 || y >= H)
+                    continue;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (c >= C)
+                        continue;
+                    const unsigned keep = ~(255u << (8 * c));
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const int x = x0 + k, X = 2 * xp + (k >> 1);
@@ -299,9 +341,8 @@ int n2d2hip_convert(const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip
         return rc;
     if (out->layout == N2D2HIP_S2D) {
         const int Hp = (out->H + 1) / 2 + 2 * out->halo, Wp = (out->W + 1) / 2 + 2 * out->halo;
-        const long long pairs = (long long)out->B * Hp * ((Wp + 1) / 2);
         N2D2HIP_REQUIRE((long long)out->B * Hp * Wp * 16 < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "convert: space-to-depth tensor too large");
-        N2D2HIP_LAUNCH(to_s2d_kernel, dim3(grid_for((size_t)pairs, 256)), dim3(256), 0, (hipStream_t)stream, in->data, in->dtype, in->layout, in->cs,
+        N2D2HIP_LAUNCH(to_s2d_kernel, dim3(grid_for((size_t)out->B * Hp, 4)), dim3(256), 0, (hipStream_t)stream, in->data, in->dtype, in->layout, in->cs,
                        in->halo, (signed char*)out->data, out->dtype, out->B, out->C, out->H, out->W, out->halo);
         N2D2HIP_HIP_CHECK(hipGetLastError());
         return N2D2HIP_OK;
