@@ -20,7 +20,11 @@ namespace {
 template <int S, int KIND, bool FAST = false>
 __global__ __launch_bounds__(256) void depthwise3x3_kernel(const DepthwiseArgs p)
 {
-    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    // Work-groups 8 apart run on the same XCD (they are dealt to the 8 XCDs in turn): a work-group's place in the tensor is
+    // chosen so that each XCD walks one contiguous eighth of it, and the columns and rows that neighbouring work-groups
+    // both read come out of that XCD's L2 instead of being fetched from memory once per XCD.
+    const unsigned per_xcd = gridDim.x >> 3;
+    const unsigned idx = ((blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3)) * 256u + threadIdx.x;
     if (idx >= p.nthreads)
         return;
     const unsigned cg = idx % p.cq;
@@ -182,7 +186,7 @@ int depthwise3x3_launch(DepthwiseArgs a, int stride, int num_cus, hipStream_t st
     const long long nthreads = columns * a.nstrips;
     N2D2HIP_REQUIRE(nthreads < (1ll << 31), N2D2HIP_ERR_UNSUPPORTED, "depthwise3x3: tensor too large");
     a.nthreads = (unsigned)nthreads;
-    const unsigned grid = (unsigned)((nthreads + 255) / 256);
+    const unsigned grid = (unsigned)round_up((int)((nthreads + 255) / 256), 8);        // a multiple of the XCD count (see the kernel)
 #define N2D2HIP_DW_LAUNCH(S, K) N2D2HIP_LAUNCH_T(depthwise3x3_kernel, (S, K), dim3(grid), dim3(256), 0, stream, a)
     if (a.epi.kind == EPI_I24 && a.fast) {
         if (stride == 1) N2D2HIP_LAUNCH_T(depthwise3x3_kernel, (1, EPI_I24, true), dim3(grid), dim3(256), 0, stream, a);
