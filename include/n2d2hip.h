@@ -331,6 +331,19 @@ int n2d2hip_bottleneck_destroy(n2d2hip_bottleneck_t bottleneck);
 int n2d2hip_bottleneck_forward(n2d2hip_bottleneck_t bottleneck, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                                n2d2hip_stream_t stream);
 
+/* Graph-level fusion of the second half of a residual bottleneck into one launch: `conv3x3` (3x3, stride 1 or 2, padding 1,
+ * C -> C channels, C = 64, 128 or 256), the only reader of whose output is `expand` (1x1, C -> 4C) with the two-input
+ * ElemWise sum that n2d2hip_conv_fuse_sum has folded into it.  That is ConvCell_Frame::propagate twice and
+ * ElemWiseCell_Frame::propagate (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/ElemWiseCell_Frame.cpp:104-136) without
+ * the 3x3 convolution's output ever reaching memory; results are those of the separate cells, bit for bit.  Nothing is
+ * created: the two handles stay usable on their own.  n2d2hip_conv_chain_supported returns 1 when the pair can run so (both
+ * cells 8-bit with integer rescales that fit the scaled-up tables, the sum on 16-bit pairs), else 0: the caller then keeps
+ * the separate launches.  `in`: the 3x3 convolution's input, NHWC bytes that carry the padding as a border (halo >= 1);
+ * `other`: the sum's other input; `out`: the sum's output; the last two with or without a border. */
+int n2d2hip_conv_chain_supported(n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand);
+int n2d2hip_conv_chain_forward(n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
+                               const n2d2hip_tensor* out, n2d2hip_stream_t stream);
+
 /* Graph-level fusion across two residual blocks: `expand` (1x1, C -> 4C, C = 128 or 256) with the two-input ElemWise sum
  * that n2d2hip_conv_fuse_sum has folded into it, and `reduce` (1x1, 4C -> C), the first convolution of the next block,
  * which reads that sum.  That is ConvCell_Frame::propagate, ElemWiseCell_Frame::propagate and ConvCell_Frame::propagate

@@ -30,7 +30,7 @@ SYMBOLS = [
     "n2d2hip_launch_log_begin", "n2d2hip_launch_log_end", "n2d2hip_launch_log_entry", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
     "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_s2d_halo", "n2d2hip_conv_accepts_halo",
-    "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
+    "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_conv_chain_supported", "n2d2hip_conv_chain_forward", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", "n2d2hip_expand_reduce_create", "n2d2hip_expand_reduce_destroy", "n2d2hip_expand_reduce_forward",
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
@@ -106,6 +106,8 @@ def load():
     lib.n2d2hip_conv_fuse_sum.argtypes = [P, P, I, I]
     lib.n2d2hip_concat_channels.argtypes = [I, P, P, P]
     lib.n2d2hip_conv_forward_sum.argtypes = [P, P, P, P, P]
+    lib.n2d2hip_conv_chain_supported.argtypes = [P, P]
+    lib.n2d2hip_conv_chain_forward.argtypes = [P, P, P, P, P, P]
     lib.n2d2hip_bottleneck_create.argtypes = [P, P, P, P, P]
     lib.n2d2hip_bottleneck_destroy.argtypes = [P]
     lib.n2d2hip_bottleneck_forward.argtypes = [P, P, P, P]

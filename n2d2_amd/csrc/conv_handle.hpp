@@ -38,6 +38,8 @@ struct n2d2hip_conv_s {
     signed char* d_ws2d;
     // 3x3 stride-1 kernel over inputs that carry their padding: weights in matrix-core fragment order
     signed char* d_wfrag;
+    // 1x1 expansion (C -> 4C, C = 64, 128 or 256) behind a 3x3 convolution in one launch: weights in fragment order
+    signed char* d_wchain;
     // 3x3 depthwise kernel: per channel and kernel row the three weights in one dword, then the biases with the zero point folded in
     int* d_wdw;
     // 4-bit weights for the pipelined kernel: the ring's weight tiles as LDS wants them, two weights per byte

@@ -349,6 +349,7 @@ using namespace n2d2hip;
 
 #include "conv_handle.hpp"
 #include "conv_s2d.hpp"
+#include "conv_chain.hpp"
 
 namespace {
 
@@ -523,7 +524,7 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     c->depthwise = depthwise;
     c->pix4 = (!depthwise && c->in_cs == 4);
     c->d_w = nullptr; c->d_sub = nullptr; c->d_bias = nullptr; c->d_fill = nullptr;
-    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_ws2d = nullptr; c->d_wfrag = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr; c->d_wsmall = nullptr;
+    c->d_epi_tab = nullptr; c->bias_folded = false; c->hi16 = false; c->d_wstem = nullptr; c->d_ws2d = nullptr; c->d_wfrag = nullptr; c->d_wchain = nullptr; c->d_wdw = nullptr; c->d_w4img = nullptr; c->d_wsmall = nullptr;
     c->sum = nullptr; c->d_res_tab = nullptr; c->sum_other_dtype = -1; c->has_pre = c->pre_clamp = c->sum_clamp = c->sum16 = false;
     c->is_fc = false; c->fcH = c->fcW = 0;
     if (c->pix4 && d->dilX != 1) {
@@ -725,6 +726,13 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
         e = hipMalloc((void**)&c->d_wfrag, hfrag.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_wfrag, hfrag.data(), hfrag.size(), hipMemcpyHostToDevice);
     }
+    if (e == hipSuccess && !depthwise && !c->pix4 && d->weight_bits == 8 && d->kW == 1 && d->kH == 1 && conv_chain_channels(d->C)
+        && c->in_cs == d->C && d->O == 4 * d->C && c->ktot == d->C) {
+        std::vector<signed char> img(conv_chain_weight_bytes(d->C, d->O));
+        conv_chain_weight_layout(hw.data(), c->ktot, d->C, d->O, img.data());
+        e = hipMalloc((void**)&c->d_wchain, img.size());
+        if (e == hipSuccess) e = hipMemcpy(c->d_wchain, img.data(), img.size(), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess && !hw4img.empty()) {
         e = hipMalloc((void**)&c->d_w4img, hw4img.size());
         if (e == hipSuccess) e = hipMemcpy(c->d_w4img, hw4img.data(), hw4img.size(), hipMemcpyHostToDevice);
@@ -768,6 +776,7 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
     if (c->d_ws2d) (void)hipFree(c->d_ws2d);
     if (c->d_wsmall) (void)hipFree(c->d_wsmall);
     if (c->d_wfrag) (void)hipFree(c->d_wfrag);
+    if (c->d_wchain) (void)hipFree(c->d_wchain);
     if (c->d_wdw) (void)hipFree(c->d_wdw);
     if (c->d_w4img) (void)hipFree(c->d_w4img);
     delete c;
@@ -1420,6 +1429,120 @@ int n2d2hip_conv_forward_sum(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
     N2D2HIP_REQUIRE(c != nullptr && other != nullptr, N2D2HIP_ERR_INVALID, "conv_forward_sum: null argument");
     N2D2HIP_REQUIRE(c->sum != nullptr, N2D2HIP_ERR_INVALID, "conv_forward_sum: no sum has been folded into this convolution");
     return conv_forward_impl(c, in, other, out, stream);
+}
+
+// Can the pair (3x3 convolution, 1x1 expansion with a folded sum) run as one launch?
+static bool chain_ok(const n2d2hip_conv_s* c3, const n2d2hip_conv_s* ce)
+{
+    if (!c3 || !ce)
+        return false;
+    const n2d2hip_conv_desc& d = c3->desc;
+    const n2d2hip_conv_desc& x = ce->desc;
+    if (c3->depthwise || c3->pix4 || d.weight_bits != 8 || d.groups != 1 || d.kW != 3 || d.kH != 3 || d.dilX != 1 || d.dilY != 1
+        || d.strideX != d.strideY || (d.strideX != 1 && d.strideX != 2) || d.padL != 1 || d.padT != 1 || d.padR != 1 || d.padB != 1
+        || d.C != d.O || !conv_chain_channels(d.C) || c3->in_cs != d.C || c3->ktot != 9 * d.C || c3->act->args.kind != EPI_I24
+        || !c3->bias_folded || !c3->hi16 || (d.kernel_choice & (N2D2HIP_KERNEL_NO_PIPE | N2D2HIP_KERNEL_NO_HI16)))
+        return false;
+    if (!ce->d_wchain || x.C != d.O || x.O != 4 * d.O || x.strideX != 1 || x.strideY != 1 || x.padL != 0 || x.padT != 0 || x.padR != 0
+        || x.padB != 0 || !ce->sum || !ce->sum16 || !ce->hi16 || ce->act->args.kind != EPI_I24
+        || (x.kernel_choice & (N2D2HIP_KERNEL_NO_PIPE | N2D2HIP_KERNEL_NO_HI16 | N2D2HIP_KERNEL_NO_SUM16)))
+        return false;
+    // the middle tensor is stored as the expansion reads its input
+    const int lo = ce->in_dtype == N2D2HIP_I8 ? -128 : 0, hi = ce->in_dtype == N2D2HIP_I8 ? 127 : 255;
+    return c3->act->min_out >= lo && c3->act->max_out <= hi;
+}
+
+int n2d2hip_conv_chain_supported(n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand)
+{
+    return chain_ok(conv3x3, expand) ? 1 : 0;
+}
+
+int n2d2hip_conv_chain_forward(n2d2hip_conv_t c3, n2d2hip_conv_t ce, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
+                               const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    int rc;
+    N2D2HIP_REQUIRE(c3 && ce && other, N2D2HIP_ERR_INVALID, "conv_chain_forward: null argument");
+    N2D2HIP_REQUIRE(chain_ok(c3, ce), N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_chain_forward: needs a 3x3 convolution (stride 1 or 2, padding 1, 64, 128 or 256 channels in and out) and a 1x1 "
+                    "expansion to four times the channels with a folded sum on 16-bit pairs, both 8-bit with scaled-up integer "
+                    "rescales (n2d2hip_conv_chain_supported)");
+    if ((rc = check_tensor(in, "conv input", true)) || (rc = check_tensor(other, "sum input", true)) || (rc = check_tensor(out, "sum output", true)))
+        return rc;
+    const n2d2hip_conv_desc& d = c3->desc;
+    const int OC = ce->desc.O;
+    N2D2HIP_REQUIRE(in->layout == N2D2HIP_NHWC && other->layout == N2D2HIP_NHWC && out->layout == N2D2HIP_NHWC, N2D2HIP_ERR_UNSUPPORTED,
+                    "conv_chain_forward: tensors must be NHWC");
+    N2D2HIP_REQUIRE(in->dtype == c3->in_dtype && in->C == d.C && in->cs == c3->in_cs && in->halo >= 1, N2D2HIP_ERR_INVALID,
+                    "conv_chain_forward: the input must have %d channels of type %d and carry its padding as a border (halo >= 1)", d.C,
+                    c3->in_dtype);
+    int OH, OW;
+    if ((rc = n2d2hip_conv_out_dims(&d, in->H, in->W, &OH, &OW)))
+        return rc;
+    N2D2HIP_REQUIRE(out->B == in->B && out->C == OC && out->H == OH && out->W == OW && is_byte_type(out->dtype) && out->cs % 16 == 0
+                        && out->cs >= OC,
+                    N2D2HIP_ERR_INVALID, "conv_chain_forward: output must be %dx%dx%dx%d bytes", in->B, OC, OH, OW);
+    N2D2HIP_REQUIRE(other->dtype == ce->sum_other_dtype && other->B == out->B && other->C == OC && other->H == OH && other->W == OW
+                        && other->cs % 16 == 0 && other->cs >= OC,
+                    N2D2HIP_ERR_INVALID, "conv_chain_forward: the other input must be an NHWC tensor of the output's shape and of the "
+                    "storage type given to n2d2hip_conv_fuse_sum");
+    const n2d2hip_act_s* sact = ce->sum->act;
+    {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(sact->min_out >= lo && sact->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "conv_chain_forward: activation range [%d,%d] does not fit output dtype %d", sact->min_out, sact->max_out, out->dtype);
+    }
+    const int Hp = in->H + 2 * in->halo, Wp = in->W + 2 * in->halo;
+    const long long Mll = (long long)in->B * OH * OW;
+    const long long out_pixels = (long long)in->B * (OH + 2 * out->halo) * (OW + 2 * out->halo);
+    const long long other_pixels = (long long)in->B * (OH + 2 * other->halo) * (OW + 2 * other->halo);
+    N2D2HIP_REQUIRE(Mll < (1ll << 31) && (long long)in->B * Hp * Wp * in->cs < (1ll << 31) && out_pixels * out->cs < (1ll << 31)
+                        && other_pixels * other->cs < (1ll << 31),
+                    N2D2HIP_ERR_UNSUPPORTED, "conv_chain_forward: tensor too large");
+    ConvChainArgs a = {};
+    ConvArgs& ca = a.p.c;
+    ca.in = (const signed char*)in->data;
+    ca.in_cs = in->cs; ca.B = in->B; ca.H = Hp; ca.W = Wp;
+    ca.OH = OH; ca.OW = OW; ca.M = (int)Mll;
+    ca.w = c3->d_w; ca.ktot = c3->ktot; ca.niter = 0; ca.sub = nullptr; ca.bias = nullptr;
+    ca.out = out->data; ca.out_cs = out->cs; ca.out_dtype = out->dtype;
+    ca.strideX = d.strideX; ca.strideY = d.strideY; ca.padL = d.padL - in->halo; ca.padT = d.padT - in->halo; ca.dilX = 1; ca.dilY = 1;
+    ca.kW = 3; ca.kH = 3;
+    ca.ntiles_n = 1; ca.nblocks = 0;
+    ca.fill = 0;
+    ca.out_xor = out->dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    ca.epi = c3->act->args;
+    ca.epi.c = c3->d_epi_tab + 5 * c3->act->cpad;
+    ca.epi.d = c3->d_epi_tab + 6 * c3->act->cpad;
+    a.p.fill16 = c3->d_fill;
+    a.p.kW = 3; a.p.kH = 3;
+    a.p.preclamp = 0;
+    magic_div((unsigned)(OH * OW), &a.p.ohw_mul, &a.p.ohw_sh);
+    magic_div((unsigned)OW, &a.p.ow_mul, &a.p.ow_sh);
+    a.p.out_halo = out->halo;
+    a.p.out_pixels = (int)out_pixels;
+    const int cps = sact->cpad;
+    a.p.res = (const signed char*)other->data;
+    a.p.res_cs = other->cs;
+    a.p.res_halo = other->halo;
+    a.p.res_flip = other->dtype == N2D2HIP_U8 ? 0u : 0x80808080u;
+    a.p.sum = sact->args;
+    a.p.sum16 = ce->d_res_tab + 10 * cps;
+    a.p.sum16_stride = cps / 2;
+    a.p.has_pre = ce->has_pre ? 1 : 0;
+    a.p.pre_clamp = 0; a.p.sum_clamp = 0;
+    a.p.pre_in_range = ce->pre_in_range ? 1 : 0;
+    a.p.pre = EpiArgs();
+    if (ce->has_pre) {
+        a.p.pre = ce->sum->pre_act->args;
+        a.p.pre.c = ce->d_res_tab + 12 * cps;
+        a.p.pre.d = ce->d_res_tab + 13 * cps;
+    }
+    a.we = ce->d_wchain;
+    a.etc = ce->d_epi_tab + 5 * ce->act->cpad;
+    a.etd = ce->d_epi_tab + 6 * ce->act->cpad;
+    a.e_lo = ce->act->args.lo; a.e_hi = ce->act->args.hi;
+    a.t2_xor = ce->in_dtype == N2D2HIP_U8B ? 0x80808080u : 0u;
+    return conv_chain_launch(a, num_cus(), (hipStream_t)stream);
 }
 
 // ------------------------------------------------------------------- fc

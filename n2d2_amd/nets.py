@@ -384,7 +384,7 @@ class GpuNet:
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
     def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True,
-                 dw_pw=True, s2d=True):
+                 dw_pw=True, s2d=True, chains=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -400,6 +400,8 @@ class GpuNet:
         wherever the library takes the pair.
         s2d: store the network input space-to-depth (16-byte pixels of 2 x 2 input pixels, with a border of zeros) when the
         one cell reading it is a first-layer convolution the library serves that way (n2d2hip_conv_s2d_halo).
+        chains: run a block's 3x3 convolution in the launch of the expanding 1x1 convolution + sum that alone reads it
+        (n2d2hip_conv_chain_*) where the library takes the pair: the 3x3 convolution's output stays on the chip.
         tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
         (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
         only ties with the two separate launches."""
@@ -612,6 +614,10 @@ class GpuNet:
         self._bottleneck_mode = "all" if bottlenecks is True else bottlenecks
         if fuse and halo and bottlenecks:
             self._plan_bottlenecks(consumers, by_name, ins_of)
+        # 3x3 convolutions computed by the launch of the expansion and sum that alone read them (their tensors are never written)
+        self.chains = {}
+        if fuse and halo and chains:
+            self._plan_chains(consumers, by_name, ins_of)
         # reducing 1x1 convolutions computed by the launch that produces their input (their tensors are written all the same)
         self.absorbed, self.tail_layers = set(), {}
         if fuse and tails:
@@ -625,13 +631,37 @@ class GpuNet:
         self._io = [self._io[k] for k in keep]
         self.launched = [spec.layers[k] for k in keep]
 
+    def _plan_chains(self, consumers, by_name, ins_of):
+        """For every sum folded into the expanding 1x1 convolution of a block (and not part of a whole-block launch): the 3x3
+        convolution whose output only that convolution reads runs in the same launch, where the library takes the pair
+        (n2d2hip_conv_chain_supported) and the 3x3 convolution's input carries its padding as a border."""
+        step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+        for sum_name, (sum_cell, expand) in list(self.fused_sums.items()):
+            if sum_name in self.bottlenecks or len(expand.inputs) != 1:
+                continue
+            c3 = by_name.get(expand.inputs[0])
+            if (c3 is None or c3.type != "conv" or len(c3.inputs) != 1 or len(consumers[c3.name]) != 1 or c3.name in self.folded
+                    or c3.name == self.spec.output):
+                continue
+            k = step_index[sum_name]
+            c3_cell, expand_cell = self.steps[step_index[c3.name]][1], self.steps[k][1]
+            if not isinstance(c3_cell, self.rt.Conv) or not isinstance(expand_cell, self.rt.Conv) or not expand_cell.chain_supported(c3_cell):
+                continue
+            x = ins_of[c3.name][0]
+            if x.halo < 1 or ins_of[sum_name][0] is not self.tensors[c3.name]:
+                continue
+            ins_of[sum_name] = [x, ins_of[sum_name][1]]
+            self.steps[k] = (self.steps[k][0], expand_cell, (lambda c, i, o, c3c=c3_cell: c.forward_chain(c3c, i[0], i[1], o)))
+            self.folded.add(c3.name)
+            self.chains[sum_name] = c3
+
     def _plan_tails(self, consumers, ins_of):
         """For every sum folded into the expanding 1x1 convolution of a block: if a reducing 1x1 convolution (the next
         block's first cell) reads that sum, both run as one launch where the library takes them
         (n2d2hip_expand_reduce_create): the launch writes the sum and the reduction's output."""
         step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
         for sum_name, (sum_cell, expand) in list(self.fused_sums.items()):
-            if sum_name in self.bottlenecks:
+            if sum_name in self.bottlenecks or sum_name in self.chains:
                 continue
             k = step_index[sum_name]
             expand_cell = self.steps[k][1]
@@ -835,6 +865,8 @@ class GpuNet:
             total += sum(m.w.size for m in self.bottleneck_layers[l.name])
         elif l.name in self.fused_sums:
             total += self.fused_sums[l.name][1].w.size
+        if l.name in self.chains:           # the 3x3 convolution's weights; its output never leaves the chip
+            total += self.chains[l.name].w.size
         if l.name in self.stem_pools:       # the convolution's weights; its output never leaves the chip
             total += self.stem_pools[l.name].w.size
         if l.name in self.dw_pws:           # the depthwise weights; its output never leaves the chip
@@ -849,8 +881,9 @@ class GpuNet:
         if l.name in self.bottleneck_layers:
             return sum(self.B * m.out_shape[1] * m.out_shape[2] * m.w.size for m in self.bottleneck_layers[l.name])
         if l.name in self.fused_sums:
-            tail = self.tail_layers.get(l.name)
-            return self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
+            tail, c3 = self.tail_layers.get(l.name), self.chains.get(l.name)
+            return (self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
+                    + (self.layer_macs(c3) if c3 is not None else 0))
         if l.name in self.stem_pools:
             return self.layer_macs(self.stem_pools[l.name])
         if l.name in self.dw_pws:

@@ -288,6 +288,15 @@ class Conv:
         check(lib.n2d2hip_conv_forward_sum(self.handle, x.ref, other.ref, out.ref, stream_ptr()))
         return out
 
+    def chain_supported(self, conv3x3):
+        """Can `conv3x3`, whose output only this 1x1 expansion (with its folded sum) reads, run in this cell's launch?"""
+        return bool(lib.n2d2hip_conv_chain_supported(conv3x3.handle, self.handle))
+
+    def forward_chain(self, conv3x3, x, other, out):
+        """out = sum(self(conv3x3(x)), other) in one launch; x carries conv3x3's padding as a border."""
+        check(lib.n2d2hip_conv_chain_forward(conv3x3.handle, self.handle, x.ref, other.ref, out.ref, stream_ptr()))
+        return out
+
     def __del__(self):
         if getattr(self, "handle", None) and lib is not None:
             lib.n2d2hip_conv_destroy(self.handle)

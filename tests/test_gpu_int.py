@@ -1038,6 +1038,73 @@ def test_expand_sum_and_next_reduce_in_one_launch_bit_exact(rt):
     assert rt.ExpandReduce.create(ce, c64) is None
 
 
+def test_conv3x3_expansion_and_sum_in_one_launch_bit_exact(rt):
+    """n2d2hip_conv_chain_forward: 3x3 convolution -> 1x1 expansion -> sum with another tensor (plain, or through a folded
+    ScalingCell) in one launch equals the reference cells run in turn, and the two launches of the library.  64, 128 and 256
+    middle channels, stride 1 and 2, tiles that end inside the tensor, inputs, shortcuts and outputs with and without
+    a border."""
+    from n2d2_amd import capi
+    from oracle.cells import ActSpec
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(777)
+
+    def relu_spec(O):
+        return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=True)
+
+    def lin_spec(O):
+        return ActSpec("Linear", "SingleShift", rng.integers(8, 12, size=O), nb_bits=8, unsigned_out=False)
+
+    def sum_spec(O):
+        return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(0, 3, size=O)], 1), nb_bits=8, unsigned_out=True)
+
+    def weights(O, Cc, k, std):
+        return np.clip(np.rint(rng.normal(0, std, size=(O, Cc, k, k))), -127, 127).astype(np.int64)
+    cases = ((64, 9, 7, 3, 1, "plain", 1, 0, 0), (64, 20, 20, 2, 1, "scaled", 1, 1, 1), (64, 13, 11, 2, 2, "plain", 1, 0, 1),
+             (128, 10, 9, 3, 1, "scaled", 1, 0, 0), (128, 14, 14, 2, 2, "plain", 2, 1, 0), (128, 7, 5, 9, 1, "plain", 1, 1, 1),
+             (256, 7, 7, 3, 1, "scaled", 1, 0, 0), (256, 14, 14, 2, 1, "plain", 1, 1, 1), (256, 9, 12, 2, 2, "scaled", 1, 0, 1),
+             (256, 1, 1, 70, 1, "plain", 1, 0, 0))
+    for cm, H, W, B, stride, variant, in_halo, other_halo, out_halo in cases:
+        print("chain", cm, H, W, B, stride, variant, in_halo, other_halo, out_halo, flush=True)
+        oc = 4 * cm
+        x = rng.integers(0, 256, size=(B, cm, H, W))
+        wb, wc = weights(cm, cm, 3, 6 if cm > 64 else 10), weights(oc, cm, 1, 18)
+        bb, bc = rng.integers(-2000, 2000, size=cm), rng.integers(-2000, 2000, size=oc)
+        sb, sc, ssum = relu_spec(cm), lin_spec(oc), sum_spec(oc)
+        t2 = cells_ref.conv_cell(x, wb, bb, sb, stride=(stride, stride), pad=(1, 1, 1, 1))
+        t3 = cells_ref.conv_cell(t2, wc, bc, sc)
+        OH, OW = t2.shape[2], t2.shape[3]
+        other_src = rng.integers(0, 256, size=(B, oc, OH, OW))
+        cb = rt.Conv(wb, bb, rt.Act(cm, **sb.kwargs()), capi.U8B, stride=(stride, stride), pad=(1, 1, 1, 1))
+        cc = rt.Conv(wc, bc, rt.Act(oc, **sc.kwargs()), capi.U8B)
+        ew = rt.ElemWiseSum(2, oc, rt.Act(oc, **ssum.kwargs()))
+        other = other_src.astype(np.float32)
+        if variant == "scaled":
+            pre_spec = ActSpec("Linear", "FixedMult16", rng.integers(2 ** 12, 2 ** 15, size=oc), frac_bits=14, nb_bits=8, unsigned_out=True)
+            other = pre_spec.apply(other)
+            assert ew.fold_input_scaling(1, rt.Act(oc, **pre_spec.kwargs()))
+        assert cc.fuse_sum(ew, 0, capi.U8B)
+        want = cells_ref.elemwise_cell([t3, other], ssum).astype(np.int64)
+        assert cc.chain_supported(cb), (cm, variant)
+        dx = rt.DTensor.from_numpy(x, capi.U8B).with_halo(in_halo)
+        dother = rt.DTensor.from_numpy(other_src, capi.U8B)
+        if other_halo:
+            dother = dother.with_halo(other_halo)
+        out = rt.DTensor(B, oc, OH, OW, capi.U8B, halo=out_halo)
+        got = cc.forward_chain(cb, dx, dother, out).to_numpy()
+        assert np.array_equal(got, want), (cm, H, W, B, stride, variant, np.count_nonzero(got != want))
+        # the two cells still run on their own, to the same result
+        mid = cb.forward(dx, cb.make_output(dx))
+        assert np.array_equal(mid.to_numpy(), t2.astype(np.int64))
+        two = cc.forward_sum(mid, dother, rt.DTensor(B, oc, OH, OW, capi.U8B)).to_numpy()
+        assert np.array_equal(two, want)
+    # what does not qualify is reported: an expansion to twice the channels, a 3x3 convolution with a dilation
+    w2 = weights(128, 64, 1, 18)
+    c2 = rt.Conv(w2, None, rt.Act(128, **lin_spec(128).kwargs()), capi.U8B)
+    wb = weights(64, 64, 3, 10)
+    cb = rt.Conv(wb, None, rt.Act(64, **relu_spec(64).kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    assert not c2.chain_supported(cb)
+
+
 def conv_spec_for(O, rng):
     from oracle.cells import ActSpec
     return ActSpec("Linear", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(8, 12, size=O)], 1), nb_bits=8, unsigned_out=False)
