@@ -344,23 +344,6 @@ int n2d2hip_conv_chain_supported(n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand);
 int n2d2hip_conv_chain_forward(n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
                                const n2d2hip_tensor* out, n2d2hip_stream_t stream);
 
-/* Graph-level fusion across two residual blocks: `expand` (1x1, C -> 4C, C = 128 or 256) with the two-input ElemWise sum
- * that n2d2hip_conv_fuse_sum has folded into it, and `reduce` (1x1, 4C -> C), the first convolution of the next block,
- * which reads that sum.  That is ConvCell_Frame::propagate, ElemWiseCell_Frame::propagate and ConvCell_Frame::propagate
- * (ref: src/Cell/ConvCell_Frame.cpp:418-473, src/Cell/ElemWiseCell_Frame.cpp:104-136) in one launch: the sum is written
- * to memory once and never read back, the reducing convolution costs no launch of its own; results are those of the
- * separate cells, bit for bit.  The handles are borrowed, must outlive this one and stay usable on their own.  Returns
- * N2D2HIP_ERR_UNSUPPORTED (the caller keeps the separate launches) unless both cells are 8-bit with integer rescales that
- * fit the scaled-up tables and the sum runs on 16-bit pairs. */
-typedef struct n2d2hip_expand_reduce_s* n2d2hip_expand_reduce_t;
-int n2d2hip_expand_reduce_create(n2d2hip_conv_t expand, n2d2hip_conv_t reduce, n2d2hip_expand_reduce_t* fused);
-int n2d2hip_expand_reduce_destroy(n2d2hip_expand_reduce_t fused);
-/* `in`: input of `expand` (C channels); `other`: the sum's other input (4C channels); `sum`: the sum (4C channels); `reduced`:
- * output of `reduce` (C channels), with or without a border.  NHWC bytes of one height and width, channel stride equal to
- * the channel count. */
-int n2d2hip_expand_reduce_forward(n2d2hip_expand_reduce_t fused, const n2d2hip_tensor* in, const n2d2hip_tensor* other,
-                                  const n2d2hip_tensor* sum, const n2d2hip_tensor* reduced, n2d2hip_stream_t stream);
-
 /* Graph-level fusion of the MobileNet building block: `depthwise` (3x3, groups == channels, stride 1 or 2, undilated) and
  * `pointwise` (1x1, stride 1, unpadded), the only reader of its output.  That is ConvCell_Frame::propagate twice
  * (ref: src/Cell/ConvCell_Frame.cpp:418-473, kernels src/Cell/ConvCell_Frame_Kernels.cpp:26-179) in one launch: the

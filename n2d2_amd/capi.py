@@ -31,7 +31,7 @@ SYMBOLS = [
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
     "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_s2d_halo", "n2d2hip_conv_accepts_halo",
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_conv_chain_supported", "n2d2hip_conv_chain_forward", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
-    "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", "n2d2hip_expand_reduce_create", "n2d2hip_expand_reduce_destroy", "n2d2hip_expand_reduce_forward",
+    "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", 
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward", "n2d2hip_pool_forward_mapped",
@@ -113,9 +113,6 @@ def load():
     lib.n2d2hip_bottleneck_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_conv_accepts_maxpool.argtypes = [P, P, C.c_int, C.c_int]
     lib.n2d2hip_conv_forward_maxpool.argtypes = [P, P, P, P, P]
-    lib.n2d2hip_expand_reduce_create.argtypes = [P, P, P]
-    lib.n2d2hip_expand_reduce_destroy.argtypes = [P]
-    lib.n2d2hip_expand_reduce_forward.argtypes = [P, P, P, P, P, P]
     lib.n2d2hip_dw_pw_create.argtypes = [P, P, P]
     lib.n2d2hip_dw_pw_destroy.argtypes = [P]
     lib.n2d2hip_dw_pw_forward.argtypes = [P, P, P, P]

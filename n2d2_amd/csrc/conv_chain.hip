@@ -91,13 +91,14 @@ constexpr int chain_after(int KS, int NCH, int RD, bool late, int qc, int qkk)
 // NJ x 2 tiles of 32 pixels x 32 channels, WGM waves side by side along the pixels.
 // PRE: the sum's other input goes through a folded ScalingCell.
 template <int CM, int BK, int S, int NJ, int WGM, bool PRE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_chain_kernel(ConvChainArgs g)
+__global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_chain_kernel(ConvChainArgs g)
 {
     const ConvPipeArgs& q = g.p;
     const ConvArgs& p = q.c;
-    constexpr int NW = 4, NI = 2;
-    constexpr int WGN = NW / WGM;
-    static_assert(CM == 64 * WGN, "every wave column owns 64 of the middle channels");
+    constexpr int NI = 2;
+    constexpr int WGN = CM / 64;                       // every wave column owns 64 of the middle channels
+    constexpr int NW = WGM * WGN, NT = NW * 64;
+    static_assert(NW == 4 || NW == 8, "four waves (two work-groups per compute unit) or eight (one)");
     constexpr int TM = 32 * NJ, TN = 32 * NI;
     constexpr int BM = TM * WGM, BN = CM;
     constexpr int LPR = BK / 16, RPC = 64 / LPR, KH = BK / 32, TOFF = 32 * BK;
@@ -120,13 +121,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr bool RES_LATE = KS >= 4;
     static_assert(KS % RD == 0 && NCH * KS <= 64 && NCH <= 16, "the register ring's index is a compile-time value");
     constexpr int SH = CM == 64 ? 2 : CM == 128 ? 1 : 0;      // t2 rows are XOR-swizzled like the ring's
-    // LDS: the ring; inside it, once a tile's K loop is done, t2 and the tables of the expansion and the sum; behind it
-    // the 3x3 convolution's multiplier and addend
-    constexpr int T2_OFF = 0, TABB_OFF = BM * CM, TABB_BYTES = 22 * OC;
-    constexpr int TABA_OFF = S * STAGE;
-    static_assert(TABB_OFF + TABB_BYTES <= S * STAGE, "t2 and the sum's tables take the ring's place");
-    static_assert(TABA_OFF + 2 * CM * 4 <= 80 * 1024, "two work-groups per compute unit");
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[TABA_OFF + 2 * CM * 4];
+    // LDS: the ring, where t2 goes once a tile's K loop is done; behind it the 3x3 convolution's multiplier and addend and
+    // the tables of the expansion and the sum
+    constexpr int T2_OFF = 0, TABB_BYTES = 22 * OC;
+    constexpr int TABA_OFF = S * STAGE, TABB_OFF = TABA_OFF + 2 * CM * 4;
+    static_assert(BM * CM <= S * STAGE, "t2 takes the ring's place");
+    static_assert(TABB_OFF + TABB_BYTES <= (NW == 4 ? 80 : 160) * 1024, "two work-groups of four waves per compute unit, or one of eight");
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[TABB_OFF + TABB_BYTES];
     const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
 
     const int tid = threadIdx.x;
@@ -144,17 +145,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         return;
     const int niter = p.niter;
 #ifdef N2D2HIP_PROFILE
-    long long pr[3] = {0, 0, 0}, pr_t0 = clock64(), pr_t2 = 0, pr_w0 = wall_clock64();
+    long long pr[6] = {0, 0, 0, 0, 0, 0}, pr_t0 = clock64(), pr_t2 = 0, pr_w0 = wall_clock64();
 #define CHAIN_MARK(k) do { const long long now__ = clock64(); pr[k] += now__ - pr_last; pr_last = now__; } while (0)
 #else
 #define CHAIN_MARK(k) do { } while (0)
 #endif
 
-    // ---- the 3x3 convolution's tables, resident
+    // ---- resident tables: the 3x3 convolution's, the expansion's, the sum's
     if (tid < CM) {
         int* ta = (int*)(smem + TABA_OFF);
         ta[tid] = p.epi.c[tid];
         ta[CM + tid] = p.epi.d[tid];
+    }
+    {
+        int* tb = (int*)(smem + TABB_OFF);
+        for (int i = tid; i < OC; i += NT) {
+            tb[i] = g.etc[i];
+            tb[OC + i] = g.etd[i];
+            if (PRE) {
+                tb[2 * OC + i] = q.pre.c[i];
+                tb[3 * OC + i] = q.pre.d[i];
+            }
+        }
+        for (int i = tid; i < OC / 2; i += NT) {
+            tb[4 * OC + i] = q.sum16[i];
+            tb[4 * OC + OC / 2 + i] = q.sum16[q.sum16_stride + i];
+            tb[4 * OC + OC + i] = q.sum16[2 * q.sum16_stride + i];
+        }
     }
 
     for (int t = 0; t < ntile; ++t) {
@@ -253,7 +270,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int s = 0; s < S; ++s)
             issue();
-        wait_loads_and_barrier<LPI*(S - 1)>();         // step 0 has landed (and, the first time, the resident tables)
+        wait_loads_and_barrier<LPI*(S - 1)>();         // step 0 has landed
 #ifdef N2D2HIP_PROFILE
         if (t == 0) pr_t2 = clock64();
 #endif
@@ -411,23 +428,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 lds_write128(rowa + ((((unsigned)(wn * 4 + 2 * lh + 1)) ^ sw) << 4), second);
             }
         }
-        // ---- the expansion's and the sum's tables behind t2
-        {
-            int* tb = (int*)(smem + TABB_OFF);
-            for (int i = tid; i < OC; i += 256) {
-                tb[i] = g.etc[i];
-                tb[OC + i] = g.etd[i];
-                if (PRE) {
-                    tb[2 * OC + i] = q.pre.c[i];
-                    tb[3 * OC + i] = q.pre.d[i];
-                }
-            }
-            for (int i = tid; i < OC / 2; i += 256) {
-                tb[4 * OC + i] = q.sum16[i];
-                tb[4 * OC + OC / 2 + i] = q.sum16[q.sum16_stride + i];
-                tb[4 * OC + OC + i] = q.sum16[2 * q.sum16_stride + i];
-            }
-        }
         chain_lds_barrier();
         CHAIN_MARK(1);
 
@@ -473,6 +473,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 __builtin_amdgcn_sched_barrier(0);
             });
 
+            CHAIN_MARK(2);
             // ---- the sum's other input, brought into the accumulators' layout (the output's lane-half exchanges backwards)
             unsigned resw[8][2];
             chain_wait_vm<chain_after(KS, NCH, RD, RES_LATE, c, -1)>();
@@ -497,6 +498,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             if constexpr (!RES_LATE && c + 1 < NCH)
                 issue_res(std::integral_constant<int, c + 1>());
+            CHAIN_MARK(3);
 
             // ---- the three rescales on pairs of 16-bit values (see the pipelined kernel's folded sum); the tables of the
             // next channel group are requested before this one is computed
@@ -611,17 +613,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             });
             if constexpr (RES_LATE && c + 1 < NCH)
                 issue_res(std::integral_constant<int, c + 1>());
+            CHAIN_MARK(4);
         });
-        // every wave has read t2 and the tables: the next tile's ring may take their place
+        // every wave has read t2: the next tile's ring may take its place
         chain_lds_barrier();
-        CHAIN_MARK(2);
+        CHAIN_MARK(5);
     }
 #ifdef N2D2HIP_PROFILE
     if (tid == 0 && g.prof) {
-        // the common record, then the time in the 3x3 loop, in the hand-over through LDS and in the expansion and sum
+        // the common record, then the time in: the 3x3 loop; the hand-over through LDS; the expansion's K loops; the wait
+        // for the sum's other input; the rescales and stores; the last barrier
         long long* o = g.prof + (long long)blockIdx.x * 16;
-        o[0] = pr_t0; o[1] = pr_t0; o[2] = pr_t2; o[3] = clock64(); o[4] = pr[2]; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = ntile;
-        o[8] = pr[0]; o[9] = pr[1]; o[10] = pr[2]; o[11] = 0; o[12] = 0; o[13] = 0;
+        o[0] = pr_t0; o[1] = pr_t0; o[2] = pr_t2; o[3] = clock64(); o[4] = pr[3] + pr[4]; o[5] = pr_w0; o[6] = wall_clock64(); o[7] = ntile;
+        for (int k = 0; k < 6; ++k) o[8 + k] = pr[k];
     }
 #endif
     asm volatile("s_waitcnt vmcnt(0)\n\ts_waitcnt lgkmcnt(0)" ::: "memory");
@@ -648,12 +652,13 @@ int conv_chain_launch(ConvChainArgs a, int num_cus, hipStream_t stream)
 {
     const int cm = a.p.c.in_cs;
     N2D2HIP_REQUIRE(conv_chain_channels(cm), N2D2HIP_ERR_INVALID, "conv_chain: %d middle channels", cm);
-    const int BM = cm == 256 ? 64 : 128, BK = cm == 128 ? 128 : 64;
+    const int BM = 128, BK = cm == 128 ? 128 : 64;
     N2D2HIP_REQUIRE(a.p.c.ktot % BK == 0 && a.p.c.ktot / BK >= 4, N2D2HIP_ERR_INVALID, "conv_chain: K of %d bytes", a.p.c.ktot);
     a.p.c.niter = a.p.c.ktot / BK;
     a.p.cper = cm / BK;
     a.p.mtiles = (a.p.c.M + BM - 1) / BM;
-    const int per_xcd = std::max(1, std::min((a.p.mtiles + 7) / 8, 2 * num_cus / 8));
+    // two work-groups of four waves per compute unit, or one of eight
+    const int per_xcd = std::max(1, std::min((a.p.mtiles + 7) / 8, (cm == 256 ? 1 : 2) * num_cus / 8));
     a.p.mlanes = per_xcd;
     a.p.xcd_tiles = (a.p.mtiles + 7) / 8;
     const int grid = 8 * per_xcd;
@@ -662,8 +667,8 @@ int conv_chain_launch(ConvChainArgs a, int num_cus, hipStream_t stream)
 #endif
     const bool pre = a.p.has_pre != 0;
     if (cm == 256) {
-        if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (256, 64, 3, 2, 1, true), dim3(grid), dim3(256), 0, stream, a);
-        else N2D2HIP_LAUNCH_T(conv_chain_kernel, (256, 64, 3, 2, 1, false), dim3(grid), dim3(256), 0, stream, a);
+        if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (256, 64, 4, 2, 2, true), dim3(grid), dim3(512), 0, stream, a);
+        else N2D2HIP_LAUNCH_T(conv_chain_kernel, (256, 64, 4, 2, 2, false), dim3(grid), dim3(512), 0, stream, a);
     } else if (cm == 128) {
         if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (128, 128, 2, 2, 2, true), dim3(grid), dim3(256), 0, stream, a);
         else N2D2HIP_LAUNCH_T(conv_chain_kernel, (128, 128, 2, 2, 2, false), dim3(grid), dim3(256), 0, stream, a);

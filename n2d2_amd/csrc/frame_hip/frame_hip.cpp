@@ -1016,6 +1016,9 @@ void ElemWiseCell_Frame_HIP::launch()
 {
     if (mBottleneck) {
         checkStatus(n2d2hip_bottleneck_forward(mBottleneck, &mBottleneckIn->getDeviceOutputs().desc(), &mOutputs.desc(), mStream));
+    } else if (mChainConv) {
+        checkStatus(n2d2hip_conv_chain_forward(mChainConv->convHandle(), mFusedConv->convHandle(), &mChainConv->inputTensor(0)->desc(),
+                                               &sourceOf(mFoldedScaling, mInputs, 1 - mFusedIndex)->desc(), &mOutputs.desc(), mStream));
     } else if (mFusedConv) {
         checkStatus(n2d2hip_conv_forward_sum(mFusedConv->convHandle(), &mFusedConv->inputTensor(0)->desc(),
                                              &sourceOf(mFoldedScaling, mInputs, 1 - mFusedIndex)->desc(), &mOutputs.desc(), mStream));
@@ -1076,8 +1079,22 @@ bool ElemWiseCell_Frame_HIP::fuseBottleneck(Cell_Frame_HIP* reduce, Cell_Frame_H
     return true;
 }
 
+bool ElemWiseCell_Frame_HIP::fuseChain(Cell_Frame_HIP* conv3x3)
+{
+    if (mBottleneck || mChainConv || !mFusedConv || !conv3x3 || !conv3x3->convHandle() || conv3x3->foldedInto()
+        || conv3x3->parentCells().size() != 1 || !n2d2hip_conv_chain_supported(conv3x3->convHandle(), mFusedConv->convHandle()))
+        return false;
+    mChainConv = conv3x3;
+    conv3x3->setFoldedInto(this);
+    return true;
+}
+
 void ElemWiseCell_Frame_HIP::clearFusion()
 {
+    if (mChainConv) {
+        mChainConv->setFoldedInto(nullptr);
+        mChainConv = nullptr;
+    }
     if (mBottleneck) {
         n2d2hip_bottleneck_destroy(mBottleneck);
         mBottleneck = nullptr;
@@ -1862,7 +1879,21 @@ void DeepNet::planFusion()
         const bool writes = (f->convHandle() && !f->foldedInto() && n2d2hip_conv_accepts_halo(f->convHandle())
                              && !(conv && conv->computesDepthwise()))
             || (ew && ew->fusedConv()) || (pool && pool->writesHalo());
-        f->setOutputsHalo(bottleneckInput[f] ? 1 : (writes && !refused[f] ? halo[f] : 0));
+        halo[f] = bottleneckInput[f] ? 1 : (writes && !refused[f] ? halo[f] : 0);
+        f->setOutputsHalo(halo[f]);
+    }
+    // In the other residual blocks the 3x3 convolution, whose output only the expansion that holds the sum reads, runs in
+    // that launch, where the device library takes the pair and the 3x3 convolution's input carries its padding.
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* ew = dynamic_cast<ElemWiseCell_Frame_HIP*>(f);
+        if (!ew || !ew->fusedConv() || ew->bottleneckInput())
+            continue;
+        const std::vector<Cell_Frame_HIP*>& ps = ew->fusedConv()->parentCells();
+        Cell_Frame_HIP* conv3 = ps.size() == 1 ? ps[0] : nullptr;
+        if (!conv3 || !conv3->convHandle() || consumers[conv3] != 1 || conv3->parentCells().size() != 1 || !conv3->parentCells()[0]
+            || halo[conv3->parentCells()[0]] < 1)
+            continue;
+        ew->fuseChain(conv3);
     }
     mPlanned = true;
 }

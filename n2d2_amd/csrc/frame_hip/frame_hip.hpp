@@ -750,6 +750,10 @@ public:
     // and the block's input, the output of `input`, which must then carry a border of one pixel.
     bool fuseBottleneck(Cell_Frame_HIP* reduce, Cell_Frame_HIP* conv3x3, Cell_Frame_HIP* projection, Cell_Frame_HIP* input);
     Cell_Frame_HIP* bottleneckInput() const { return mBottleneck ? mBottleneckIn : nullptr; }
+    // ... or the 3x3 convolution in front of the convolution that has taken this sum, the only reader of its output, in
+    // that same launch (n2d2hip_conv_chain_*); its input must carry its padding as a border.
+    bool fuseChain(Cell_Frame_HIP* conv3x3);
+    Cell_Frame_HIP* chainedConv() const { return mChainConv; }
     bool hasFoldedScaling(size_t k) const { return k < mFoldedScaling.size() && mFoldedScaling[k] != nullptr; }
     // src/Cell/ElemWiseCell_Frame.cpp:313-316
     std::pair<double, double> getOutputsRange() const { return mActivation ? mActivation->getOutputRange() : elemWiseOutputsRange(); }
@@ -766,6 +770,7 @@ private:
     n2d2hip_bottleneck_t mBottleneck = nullptr;
     Cell_Frame_HIP* mBottleneckIn = nullptr;
     std::vector<Cell_Frame_HIP*> mBottleneckCells;
+    Cell_Frame_HIP* mChainConv = nullptr;
     static Registrar<ElemWiseCell> mRegistrar;
 };
 

@@ -383,7 +383,7 @@ class GpuNet:
     """Instantiates every cell of a NetSpec through the C ABI and runs them in layer order on the current stream.
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
-    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", tails=False, stem_pool=True,
+    def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", stem_pool=True,
                  dw_pw=True, s2d=True, chains=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
@@ -401,10 +401,7 @@ class GpuNet:
         s2d: store the network input space-to-depth (16-byte pixels of 2 x 2 input pixels, with a border of zeros) when the
         one cell reading it is a first-layer convolution the library serves that way (n2d2hip_conv_s2d_halo).
         chains: run a block's 3x3 convolution in the launch of the expanding 1x1 convolution + sum that alone reads it
-        (n2d2hip_conv_chain_*) where the library takes the pair: the 3x3 convolution's output stays on the chip.
-        tails: run a block's expanding 1x1 convolution + sum and the next block's reducing 1x1 convolution as one launch
-        (n2d2hip_expand_reduce_*) where they qualify.  Bit-identical; off by default because on the benchmark network it
-        only ties with the two separate launches."""
+        (n2d2hip_conv_chain_*) where the library takes the pair: the 3x3 convolution's output stays on the chip."""
         from . import capi, runtime as rt
         self.spec, self.B, self.rt, self.capi = spec, batch, rt, capi
         consumers = {}
@@ -618,15 +615,11 @@ class GpuNet:
         self.chains = {}
         if fuse and halo and chains:
             self._plan_chains(consumers, by_name, ins_of)
-        # reducing 1x1 convolutions computed by the launch that produces their input (their tensors are written all the same)
-        self.absorbed, self.tail_layers = set(), {}
-        if fuse and tails:
-            self._plan_tails(consumers, ins_of)
         self._io = [(ins_of[l.name], self.tensors[l.name]) for l in spec.layers]
         # folded ScalingCells are not launched and their output is never materialised
         for name in self.folded:
             del self.tensors[name]
-        keep = [k for k, l in enumerate(spec.layers) if l.name not in self.folded and l.name not in self.absorbed]
+        keep = [k for k, l in enumerate(spec.layers) if l.name not in self.folded]
         self.steps = [self.steps[k] for k in keep]
         self._io = [self._io[k] for k in keep]
         self.launched = [spec.layers[k] for k in keep]
@@ -654,32 +647,6 @@ class GpuNet:
             self.steps[k] = (self.steps[k][0], expand_cell, (lambda c, i, o, c3c=c3_cell: c.forward_chain(c3c, i[0], i[1], o)))
             self.folded.add(c3.name)
             self.chains[sum_name] = c3
-
-    def _plan_tails(self, consumers, ins_of):
-        """For every sum folded into the expanding 1x1 convolution of a block: if a reducing 1x1 convolution (the next
-        block's first cell) reads that sum, both run as one launch where the library takes them
-        (n2d2hip_expand_reduce_create): the launch writes the sum and the reduction's output."""
-        step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
-        for sum_name, (sum_cell, expand) in list(self.fused_sums.items()):
-            if sum_name in self.bottlenecks or sum_name in self.chains:
-                continue
-            k = step_index[sum_name]
-            expand_cell = self.steps[k][1]
-            x, other = ins_of[sum_name]
-            y = self.tensors[sum_name]
-            if x.halo or other.halo or y.halo:
-                continue
-            for r in consumers.get(sum_name, []):
-                if r.type != "conv" or r.name in self.folded or r.name in self.absorbed or r.w.shape[2:] != (1, 1):
-                    continue
-                fused = self.rt.ExpandReduce.create(expand_cell, self.steps[step_index[r.name]][1])
-                if fused is None:
-                    continue
-                z = self.tensors[r.name]
-                self.steps[k] = (self.steps[k][0], fused, (lambda c, i, o, z=z: c.forward(i[0], i[1], o, z)))
-                self.absorbed.add(r.name)
-                self.tail_layers[sum_name] = r
-                break
 
     def _plan_bottlenecks(self, consumers, by_name, ins_of):
         """For every sum folded into a 1x1 convolution: reduce -> 3x3 -> expand (+ projection) as one launch, if the
@@ -871,19 +838,14 @@ class GpuNet:
             total += self.stem_pools[l.name].w.size
         if l.name in self.dw_pws:           # the depthwise weights; its output never leaves the chip
             total += self.dw_pws[l.name].w.size
-        if l.name in self.tail_layers:      # the reduction's weights and output; its input never leaves the chip
-            r = self.tail_layers[l.name]
-            z = self.tensors[r.name]
-            total += r.w.size + z.B * z.C * z.H * z.W
         return total
 
     def layer_macs(self, l):
         if l.name in self.bottleneck_layers:
             return sum(self.B * m.out_shape[1] * m.out_shape[2] * m.w.size for m in self.bottleneck_layers[l.name])
         if l.name in self.fused_sums:
-            tail, c3 = self.tail_layers.get(l.name), self.chains.get(l.name)
-            return (self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(tail) if tail is not None else 0)
-                    + (self.layer_macs(c3) if c3 is not None else 0))
+            c3 = self.chains.get(l.name)
+            return self.layer_macs(self.fused_sums[l.name][1]) + (self.layer_macs(c3) if c3 is not None else 0)
         if l.name in self.stem_pools:
             return self.layer_macs(self.stem_pools[l.name])
         if l.name in self.dw_pws:

@@ -159,32 +159,6 @@ class Bottleneck:
             self.handle = None
 
 
-class ExpandReduce:
-    """n2d2hip_expand_reduce_t: a block's expanding 1x1 convolution with its folded sum and the next block's reducing 1x1
-    convolution in one launch; None when the library keeps the cells apart."""
-
-    def __init__(self, handle, cells):
-        self.handle, self._cells = handle, cells
-
-    @staticmethod
-    def create(expand, reduce):
-        h = C.c_void_p()
-        rc = lib.n2d2hip_expand_reduce_create(expand.handle, reduce.handle, C.byref(h))
-        if rc == capi.ERR_UNSUPPORTED:
-            return None
-        check(rc)
-        return ExpandReduce(h, (expand, reduce))
-
-    def forward(self, x, other, total, reduced):
-        check(lib.n2d2hip_expand_reduce_forward(self.handle, x.ref, other.ref, total.ref, reduced.ref, stream_ptr()))
-        return reduced
-
-    def __del__(self):
-        if getattr(self, "handle", None) and lib is not None:
-            lib.n2d2hip_expand_reduce_destroy(self.handle)
-            self.handle = None
-
-
 class DwPw:
     """n2d2hip_dw_pw_t: a 3x3 depthwise convolution and the 1x1 convolution reading it in one launch; None when the library
     keeps the cells apart."""

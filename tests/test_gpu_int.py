@@ -981,63 +981,6 @@ def test_first_layer_conv_on_space_to_depth_input_bit_exact(rt):
         conv.forward(dx, rt.DTensor(2, 32, 20, 20, capi.U8B))
 
 
-def test_expand_sum_and_next_reduce_in_one_launch_bit_exact(rt):
-    """n2d2hip_expand_reduce_*: a block's 1x1 expansion with its folded sum and the next block's 1x1 reduction in one launch
-    equal the reference cells run in turn (both tensors: the sum and the reduction's output); 128 and 256 middle channels,
-    the sum's other input plain, through a folded ScalingCell that stays in range and through one that saturates; pixel
-    counts that end inside a tile; outputs with and without a border; several tiles per block."""
-    from n2d2_amd import capi
-    from oracle.cells import ActSpec
-    from oracle import cells as cells_ref
-    rng = np.random.default_rng(777)
-
-    def relu_spec(O):
-        return ActSpec("Rectifier", "DoubleShift", np.stack([rng.integers(0, 3, size=O), rng.integers(9, 13, size=O)], 1), nb_bits=8, unsigned_out=True)
-
-    def weights(O, Cc, std):
-        return np.clip(np.rint(rng.normal(0, std, size=(O, Cc, 1, 1))), -127, 127).astype(np.int64)
-    for cmid, H, W, B, variant in ((128, 14, 14, 2, "plain"), (256, 14, 14, 2, "scaled"), (256, 7, 9, 3, "scaled saturating"),
-                                   (128, 28, 28, 47, "scaled"), (256, 5, 5, 1, "plain"), (128, 3, 3, 1, "scaled saturating")):
-        print("expand_reduce", cmid, H, W, B, variant, flush=True)
-        cout = 4 * cmid
-        x = rng.integers(0, 256, size=(B, cmid, H, W))
-        other = rng.integers(0, 256, size=(B, cout, H, W))
-        we, wr = weights(cout, cmid, 20), weights(cmid, cout, 8)
-        be, br = rng.integers(-3000, 3000, size=cout), rng.integers(-3000, 3000, size=cmid)
-        se, sr, ssum = conv_spec_for(cout, rng), relu_spec(cmid), sum_spec_for(cout, rng)
-        ce = rt.Conv(we, be, rt.Act(cout, **se.kwargs()), capi.U8B)
-        cr = rt.Conv(wr, br, rt.Act(cmid, **sr.kwargs()), capi.U8B)
-        ew = rt.ElemWiseSum(2, cout, rt.Act(cout, **ssum.kwargs()))
-        oth = other.astype(np.float32)
-        if variant != "plain":
-            lo, hi = (2 ** 12, 2 ** 14) if variant == "scaled" else (2 ** 14, 2 ** 15)      # factors below / up to 2: the latter saturate
-            pre_spec = ActSpec("Linear", "FixedMult16", rng.integers(lo, hi, size=cout), frac_bits=14, nb_bits=8, unsigned_out=True)
-            oth = pre_spec.apply(oth)
-            pre = rt.Act(cout, **pre_spec.kwargs())
-            assert ew.fold_input_scaling(1, pre)
-        assert ce.fuse_sum(ew, 0, capi.U8B)
-        t = cells_ref.conv_cell(x, we, be, se)
-        want_sum = cells_ref.elemwise_cell([t, oth], ssum).astype(np.int64)
-        want_red = cells_ref.conv_cell(want_sum, wr, br, sr).astype(np.int64)
-        fused = rt.ExpandReduce.create(ce, cr)
-        assert fused is not None, variant
-        dx, do = rt.DTensor.from_numpy(x, capi.U8B), rt.DTensor.from_numpy(other, capi.U8B)
-        for halo in (1, 0):
-            ysum = rt.DTensor(B, cout, H, W, capi.U8B)
-            zred = rt.DTensor(B, cmid, H, W, capi.U8B, halo=halo)
-            fused.forward(dx, do, ysum, zred)
-            got_sum, got_red = ysum.to_numpy(), zred.to_numpy()
-            assert np.array_equal(got_sum, want_sum), (cmid, H, W, B, variant, halo, np.count_nonzero(got_sum != want_sum))
-            assert np.array_equal(got_red, want_red), (cmid, H, W, B, variant, halo, np.count_nonzero(got_red != want_red))
-        # the cells still run on their own
-        ysum = rt.DTensor(B, cout, H, W, capi.U8B)
-        ce.forward_sum(dx, do, ysum)
-        assert np.array_equal(cr.forward(ysum).to_numpy(), want_red)
-    # what does not qualify is reported: a reduction to another channel count
-    c64 = rt.Conv(weights(64, 512, 8), None, rt.Act(64, **relu_spec(64).kwargs()), capi.U8B)
-    assert rt.ExpandReduce.create(ce, c64) is None
-
-
 def test_conv3x3_expansion_and_sum_in_one_launch_bit_exact(rt):
     """n2d2hip_conv_chain_forward: 3x3 convolution -> 1x1 expansion -> sum with another tensor (plain, or through a folded
     ScalingCell) in one launch equals the reference cells run in turn, and the two launches of the library.  64, 128 and 256

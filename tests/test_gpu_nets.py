@@ -81,7 +81,11 @@ def test_resnet50_config(variant):
         assert [m.name for m in net.bottleneck_layers["conv2.1_sum"]] == ["conv2.1_1x1", "conv2.1_3x3", "conv2.1_1x1_x4", "conv2.1_1x1_proj"]
     # ... and the first convolution computes the max pooling behind it (its own output is never written)
     assert list(net.stem_pools) == ["pool1"] and "conv1" in net.folded
-    nfolded = 32 if one_launch else 29
+    # ... and in every other block without a projection the 3x3 convolution runs in the launch of the expansion and sum
+    identity = [n for n in ("conv2.2", "conv2.3", "conv3.2", "conv3.3", "conv3.4", "conv4.2", "conv4.3", "conv4.4", "conv4.5", "conv4.6")]
+    if one_launch:
+        assert sorted(net.chains) == [n + "_sum" for n in identity] and all(n + "_3x3" in net.folded for n in identity)
+    nfolded = (32 if one_launch else 29) + len(net.chains)
     if variant == "pad0_n2d2_model":
         assert net.tensors["pool1"].H == 55
     assert len(net.folded) == nfolded and len(net.launched) == len(spec.layers) - nfolded
@@ -93,18 +97,9 @@ def test_resnet50_config(variant):
     assert sorted(n for n, t in net.tensors.items() if t.halo and n != "input") == sorted(
         [l.name[:-3] + "1x1" for l in spec.layers if l.name.endswith("_3x3") and not (one_launch and l.name == "conv2.1_3x3")]
         + (["pool1"] if one_launch else []))
-    # a block's expansion + sum and the next block's reduction as one launch (off by default): same bytes everywhere
-    if one_launch:
-        tails = nets.GpuNet(spec, x.shape[0], tails=True)
-        tails.set_input(x)
-        assert sorted(tails.absorbed) == ["conv3.3_1x1", "conv3.4_1x1", "conv4.3_1x1", "conv4.4_1x1", "conv4.5_1x1", "conv4.6_1x1"]
-        assert len(tails.launched) == len(net.launched) - 6
-        assert np.array_equal(tails.forward().to_numpy(), net.tensors[spec.output].to_numpy())
-        for n in ("conv3.3_1x1", "conv3.3_sum", "conv4.6_1x1", "conv4.5_sum"):
-            assert np.array_equal(tails.tensors[n].to_numpy(), net.tensors[n].to_numpy()), n
-    separate = nets.GpuNet(spec, x.shape[0], bottlenecks=False, stem_pool=False)
+    separate = nets.GpuNet(spec, x.shape[0], bottlenecks=False, stem_pool=False, chains=False)
     separate.set_input(x)
-    assert not separate.bottlenecks and len(separate.folded) == 28 and len(separate.launched) == len(spec.layers) - 28
+    assert not separate.bottlenecks and not separate.chains and len(separate.folded) == 28 and len(separate.launched) == len(spec.layers) - 28
     assert np.array_equal(separate.forward().to_numpy(), net.tensors[spec.output].to_numpy())
     if variant == "pad1":
         unfused = _run_both(spec, x, keep, fuse=False)
@@ -174,7 +169,7 @@ def test_resnet50_full_batch_properties():
     assert np.array_equal(net.forward().to_numpy()[:, :, 0, 0], logits)
     # ... and so do twenty more, tensor by tensor on a few layers of each kind, launched back to back and replayed
     # from a graph (asynchronous LDS traffic and hand-counted waits leave no room for run-to-run differences)
-    watch = ["pool1", "conv2.1_sum", "conv2.2_3x3", "conv2.3_sum", "conv3.4_sum", "conv4.6_sum", "conv5.3_sum", "pool", "fc"]
+    watch = ["pool1", "conv2.1_sum", "conv2.2_1x1", "conv2.3_sum", "conv3.1_3x3", "conv3.4_sum", "conv4.6_sum", "conv5.3_sum", "pool", "fc"]
     ref = {n: net.tensors[n].to_numpy() for n in watch}
     replay = net.capture()
     for it in range(20):
