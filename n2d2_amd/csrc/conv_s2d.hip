@@ -471,7 +471,9 @@ int conv_s2d_halo(int k, int padT, int padL, int padB, int padR, int H, int W)
     int halo = std::max(std::max(qy, qx), 0);
     halo = std::max(halo, OH - qy + ny - 1 - Hs);
     halo = std::max(halo, OW - qx + 2 * nxh - 1 - Ws);
-    return halo;
+    // an even border keeps the pixel pairs of a stored row aligned with those of the input's rows: the conversion then
+    // moves whole dwords (a larger border than needed is as good to the kernel)
+    return (halo + 1) & ~1;
 }
 
 int conv_s2d_launch(ConvS2dArgs a, int k, bool hi16, bool pool, int nblk, int blocks, int channel_tiles, hipStream_t stream)

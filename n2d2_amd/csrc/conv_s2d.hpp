@@ -37,7 +37,8 @@ struct ConvS2dArgs {
 // Bytes of the weights in the kernel's order, and the reordering (host): `w` is the caller's OCHW array.
 size_t conv_s2d_weight_bytes(int O, int k, int pad);
 void conv_s2d_weight_layout(const signed char* w_ochw, int C, int O, int k, int padT, int padL, signed char* out);
-// Border (in 16-byte pixels, every side) an H x W input needs for this kernel size and padding; -1: not served.
+// Border (in 16-byte pixels, every side; an even number) an H x W input is given for this kernel size and padding; -1: not
+// served.
 int conv_s2d_halo(int k, int padT, int padL, int padB, int padR, int H, int W);
 // hi16: scaled-up tables; pool: with the max pooling; nblk: 32-channel blocks a work-group computes (1 or 2);
 // channel_tiles: work-groups along the channels (blockIdx.y), each computing 32 * nblk of them for every strip.
