@@ -21,7 +21,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
 # inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
 TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
-                        "bytes_per_launch": 72893232, "launches_per_forward": 39,
+                        "bytes_per_launch": 57025630, "launches_per_forward": 29,
                         "note": "FETCH_SIZE + WRITE_SIZE, mean over the conv_pipe_kernel dispatches of 4 forwards, scaled by a 1 GiB copy; "
                                 "not measured by this run"}
 
@@ -135,12 +135,13 @@ def other_configs(torch, with_cpu):
         # a graph holds 16 forwards of a network of a few launches, 4 of a larger one: replaying a graph costs about
         # 18 us once, which would otherwise be most of what a one-kernel network is timed at
         per_graph = 16 if len(net.launched) <= 8 else 4
-        replay = net.capture(per_graph)
+        replay = net.capture(per_graph, with_input_conversion=True)
         ms, mean_ms, _ = median_step_ms(torch, replay, 10 * per_graph, per_graph, per_graph)
         runs = [net.forward_timed() for _ in range(5)]
         per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
         entry = {"batch": batch, "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "ms_per_step": round(ms, 4),
-                 "launches": len(net.launched), "forwards_per_graph": per_graph, "gmac_per_image": round(spec.macs_per_image() / 1e9, 4),
+                 "step_is": "graph-edge conversion of the resident byte planes + forward",
+                 "launches": len(net.launched) + 1, "forwards_per_graph": per_graph, "gmac_per_image": round(spec.macs_per_image() / 1e9, 4),
                  "roofline_by_class": class_rooflines(net, per_launch, ms)}
         if with_cpu:
             n = batch if full else 2
@@ -330,7 +331,10 @@ def kernel_phases(torch, config, batch):
           " lives / (span x work-groups); mhz = shader clocks per microsecond inside the kernel")
     print("%-64s %3s " % ("kernel", "n") + " ".join("%12s" % k[:12] for k in keys))
     for kname, lst in sorted(rows.items(), key=lambda kv: -sum(d["span_us"] for d in kv[1])):
-        print("%-64s %3d " % (kname[:64], len(lst)) + " ".join("%12.2f" % float(np.nanmean([d[k] for d in lst])) for k in keys))
+        def col(k):
+            vals = [d[k] for d in lst if d[k] == d[k]]      # (a kernel without that mark leaves a NaN)
+            return "%12.2f" % float(np.mean(vals)) if vals else "%12s" % "-"
+        print("%-64s %3d " % (kname[:64], len(lst)) + " ".join(col(k) for k in keys))
     for kname, lst in rows.items():
         if "phases_us" in lst[0]:
             print("%s: microseconds per unit of work in its phases 0..5 (see the kernel's source): %s" % (
@@ -487,7 +491,8 @@ def main():
     hbm_view = {"achieved": round(achieved_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved_gbs / PEAK_HBM_GBS, 4)}
     roofline = {"bound": "hbm" if hbm_bound else "mfma",
                 "kernel": "conv_pipe_kernel (%d launches of one forward: conv/fc cells with a multiple of 64 input "
-                "channels, residual sums folded in; not the cells of the fused bottleneck nor the 3x3 layers on the patch kernel)" % len(pipe),
+                "channels, residual sums folded in; not the cells of the launches that take a whole block or its 3x3 convolution, expansion "
+                "and sum: conv_chain_kernel and bottleneck_kernel under roofline_kernels)" % len(pipe),
                 "bound_is": "the larger of ops / int8 peak and algorithmic bytes / HBM peak over these launches",
                 "floor_us_per_launch": {"mfma": round(conv_ops / (PEAK_INT8_TOPS * 1e12) * 1e6 / len(pipe), 2),
                                         "hbm": round(pipe_bytes / (PEAK_HBM_GBS * 1e9) * 1e6 / len(pipe), 2)},
@@ -502,7 +507,7 @@ def main():
                 "ops_per_launch": conv_ops / len(pipe), "frac_of_peak_at_measured_clock": round(achieved / clock["int8_peak_at_that_clock_tops"], 4)}
     # the other convolution kernels of the forward, each replayed alone the same way
     roofline_kernels = {}
-    for name in ("conv_patch3x3_kernel", "bottleneck_kernel", "conv_s2d_kernel", "conv_stem_kernel"):
+    for name in ("conv_chain_kernel", "conv_patch3x3_kernel", "bottleneck_kernel", "conv_s2d_kernel", "conv_stem_kernel"):
         idx = [k for k, kn in enumerate(kernels) if kn == name]
         if not idx:
             continue
