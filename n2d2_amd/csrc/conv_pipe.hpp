@@ -88,7 +88,7 @@ __device__ __forceinline__ int swz_k(int row, int s)
 // VALID: 0 = windows may reach outside the input (per-tap validity bits), 1 = 1x1 kernel without padding, 2 = any kernel
 // without padding (every tap of every window inside the input: a tap only moves the uniform base address).
 // W4: 4-bit weights.  They stay packed two per byte in memory and in LDS (p.w is then an image of the ring's weight
-// tiles: per 32 channels and K step one 1 KB chunk, laid out as the LDS wants it) and are widened to bytes on their way
+// tiles: per 32 channels and 64 of K one 1 KB chunk, laid out as the LDS wants it) and are widened to bytes on their way
 // from LDS to the matrix core, as 16 times their value: the nibble becomes the upper half of its byte, which one AND
 // (upper nibbles) or a shift and an AND (lower nibbles) do for four weights at once.  The accumulators are divided by
 // 16, exactly, before they are rescaled.
@@ -106,11 +106,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int TOFF = 32 * BK;                      // LDS bytes between MFMA tiles of one operand
     // chunks each wave loads per step; when there are fewer chunks than waves some are loaded twice
     constexpr int WROW = W4 ? BK / 2 : BK;             // bytes of a weight row per stage
-    constexpr int A_CH = BM / RPC, B_CH = W4 ? BN / 32 : BN / RPC;
+    constexpr int KCH = BK / 64;                       // W4: 1 KB weight chunks (32 channels x 64 of K) per channel block and stage
+    constexpr int A_CH = BM / RPC, B_CH = W4 ? (BN / 32) * KCH : BN / RPC;
     constexpr int A_J = (A_CH + NW - 1) / NW, B_J = (B_CH + NW - 1) / NW;
     constexpr int LPI = A_J + B_J;                     // loads per thread and step
     constexpr int STAGE = BM * BK + BN * WROW;
-    static_assert(!W4 || BK == 64, "packed weights: 32 channels x 32 bytes per 1 KB chunk");
     constexpr int TAB_OFF = S * STAGE;                 // 6 int arrays of BN entries: bias, a, b, c, d, e
     // RES: + a..e of the sum cell, + a..e of the folded ScalingCell.  When the sum runs on 16-bit pairs, its c, d, e in
     // that form take the place of the bias and the convolution's a, which that path does not use.
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     unsigned woff[B_J];            // byte offset of this thread's weight rows (without the K offset)
 #pragma unroll
     for (int j = 0; j < B_J; ++j)
-        woff[j] = W4 ? (unsigned)(((n0 / 32 + (wave + NW * j) % B_CH) * p.niter) * 1024 + lane * 16)
+        woff[j] = W4 ? (unsigned)(((n0 / 32 + ((wave + NW * j) % B_CH) / KCH) * (p.niter * KCH) + ((wave + NW * j) % B_CH) % KCH) * 1024 + lane * 16)
                      : (unsigned)((n0 + ((wave + NW * j) % B_CH) * RPC + lrow) * p.ktot + lq * 16);
     int rowoff[A_J];               // byte offset of the window origin of this thread's pixel rows (+ sub-chunk)
     unsigned rowmask[A_J];         // bit t < 31: kernel tap t of the row reads inside the input; bit 31: undilated window
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                 __builtin_amdgcn_global_load_lds((gbl_ptr_t)src, (lds_ptr_t)(sbase + ((wave + NW * j) % A_CH) * 1024), 16, 0, 0);
             }
         }
-        const signed char* wbase = p.w + (W4 ? l_it * 1024 : l_koff);
+        const signed char* wbase = p.w + (W4 ? l_it * (KCH * 1024) : l_koff);
 #pragma unroll
         for (int j = 0; j < B_J; ++j)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(wbase + woff[j]), (lds_ptr_t)(sbase + BM * BK + ((wave + NW * j) % B_CH) * 1024), 16, 0, 0);
@@ -252,7 +252,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int kk = 0; kk < KH; ++kk) {
         pa[kk] = lds0 + swz_k<BK>(wm * TM + l32, 2 * kk + lh);
-        wa[kk] = W4 ? lds0 + BM * BK + (wn * TN + l32) * 32 + (((2 * kk + lh) ^ ((l32 >> 3) & 3)) << 3)
+        // (W4: the chunk of this wave's first channel block that holds K step kk, then the lane's row and 8-byte slot in it)
+        wa[kk] = W4 ? lds0 + BM * BK + (wn * NI * KCH + kk / 2) * 1024 + l32 * 32 + (((2 * (kk % 2) + lh) ^ ((l32 >> 3) & 3)) << 3)
                     : lds0 + BM * BK + swz_k<BK>(wn * TN + l32, 2 * kk + lh);
     }
     int r_stage = 0;
@@ -269,7 +270,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         constexpr int set = kk & 1;
         if (W4) {
             lds_read64_nowait<0>(fw4[set][0], wa[kk]);
-            if (NI > 1) lds_read64_nowait<1024>(fw4[set][W4 && NI > 1 ? 1 : 0], wa[kk]);
+            if (NI > 1) lds_read64_nowait<KCH * 1024>(fw4[set][W4 && NI > 1 ? 1 : 0], wa[kk]);
         } else {
             lds_read128_nowait<0>(fw[set][0], wa[kk]);
             if (NI > 1) lds_read128_nowait<TOFF>(fw[set][NI > 1 ? 1 : 0], wa[kk]);

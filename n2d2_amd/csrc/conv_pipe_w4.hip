@@ -33,12 +33,16 @@ void conv_pipe_w4_image(const signed char* w, int rows, int ktot, signed char* i
 
 namespace {
 
+#ifndef W4_S128
+#define W4_S128 3
+#endif
+
 // valid: 1 = 1x1 without padding, 2 = any kernel whose every tap reads inside the (physical) input, e.g. an input that
 // carries its padding, 0 = per-tap validity bits
-template <int NI, int NJ, int WGM, int V>
+template <int BK, int S, int NI, int NJ, int WGM, int V>
 void launch_valid(const ConvPipeArgs& a, bool hi16, int grid, hipStream_t stream)
 {
-    constexpr int NW = 4, BK = 64, S = 4;
+    constexpr int NW = 4;
     if (a.res) {
         // residual sum in the epilogue; 16-bit pairs when the host has shown that they hold every intermediate
         if (a.sum16) N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, V, true, true, true), dim3(grid), dim3(NW * 64), 0, stream, a);
@@ -49,14 +53,23 @@ void launch_valid(const ConvPipeArgs& a, bool hi16, int grid, hipStream_t stream
     }
 }
 
-template <int NI, int NJ, int WGM>
-void launch(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t stream)
+template <int BK, int S, int NI, int NJ, int WGM>
+void launch_bk(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t stream)
 {
-    a.c.niter = a.c.ktot / 64;
-    a.cper = a.c.in_cs / 64;
-    if (valid == 1) launch_valid<NI, NJ, WGM, 1>(a, hi16, grid, stream);
-    else if (valid == 2) launch_valid<NI, NJ, WGM, 2>(a, hi16, grid, stream);
-    else launch_valid<NI, NJ, WGM, 0>(a, hi16, grid, stream);
+    a.c.niter = a.c.ktot / BK;
+    a.cper = a.c.in_cs / BK;
+    if (valid == 1) launch_valid<BK, S, NI, NJ, WGM, 1>(a, hi16, grid, stream);
+    else if (valid == 2) launch_valid<BK, S, NI, NJ, WGM, 2>(a, hi16, grid, stream);
+    else launch_valid<BK, S, NI, NJ, WGM, 0>(a, hi16, grid, stream);
+}
+
+// K advances by whole 128-byte lines of pixels (two weight chunks per channel block and stage) when the channel count
+// allows, as with 8-bit weights; the packed weights leave room for a third ring stage.
+template <int NI, int NJ, int WGM>
+void launch(const ConvPipeArgs& a, int valid, bool hi16, int grid, hipStream_t stream)
+{
+    if (a.c.in_cs % 128 == 0) launch_bk<128, W4_S128, NI, NJ, WGM>(a, valid, hi16, grid, stream);
+    else launch_bk<64, 4, NI, NJ, WGM>(a, valid, hi16, grid, stream);
 }
 
 } // namespace
