@@ -140,10 +140,16 @@ def other_configs(torch, with_cpu):
         at_edge = name != "resnet18_stage_conv_bs64"
         replay = net.capture(per_graph, with_input_conversion=at_edge)
         ms, mean_ms, _ = median_step_ms(torch, replay, 10 * per_graph, per_graph, per_graph)
+        fwd_ms = ms
+        if at_edge:     # the forward alone, as earlier bench lines timed these configurations
+            replay_fwd = net.capture(per_graph)
+            fwd_ms, _, _ = median_step_ms(torch, replay_fwd, 10 * per_graph, per_graph, per_graph)
+            del replay_fwd
         runs = [net.forward_timed() for _ in range(5)]
         per_launch = [float(np.median([r[k][1] for r in runs])) for k in range(len(net.launched))]
         entry = {"batch": batch, "value": round(batch / (ms * 1e-3), 1), "unit": "images/s", "ms_per_step": round(ms, 4),
                  "step_is": "graph-edge conversion of the resident byte planes + forward" if at_edge else "forward (input resident as cells exchange it)",
+                 "forward_without_edge_conversion_ms": round(fwd_ms, 4), "images_per_s_forward_only": round(batch / (fwd_ms * 1e-3), 1),
                  "launches": len(net.launched) + (1 if at_edge else 0), "forwards_per_graph": per_graph, "gmac_per_image": round(spec.macs_per_image() / 1e9, 4),
                  "roofline_by_class": class_rooflines(net, per_launch, ms)}
         if with_cpu:
