@@ -234,6 +234,19 @@ int n2d2hip_fc_destroy(n2d2hip_fc_t fc);
 int n2d2hip_fc_forward(n2d2hip_fc_t fc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                        n2d2hip_stream_t stream);
 
+/* Graph-level fusion of a classifier head: two or three FcCells, each after the first reading the 1 x 1 output of the one
+ * before and nothing else reading it, in one launch; that is FcCell_Frame::propagate two or three times
+ * (ref: src/Cell/FcCell_Frame.cpp:234-340) with the vectors between the cells kept on the chip; results are those of the
+ * cells run in turn, bit for bit (same int32 sums, same rescale).  The handles are borrowed, must outlive the chain and
+ * stay usable on their own.  Returns N2D2HIP_ERR_UNSUPPORTED (the caller keeps the separate launches) unless every cell
+ * has 8-bit weights, at most 1024 inputs and at most 128 outputs.  `in`: the first cell's input (NHWC bytes, as
+ * n2d2hip_fc_forward takes it); `out`: the last cell's output. */
+typedef struct n2d2hip_fc_chain_s* n2d2hip_fc_chain_t;
+int n2d2hip_fc_chain_create(int nb_cells, const n2d2hip_fc_t* cells, n2d2hip_fc_chain_t* chain);
+int n2d2hip_fc_chain_destroy(n2d2hip_fc_chain_t chain);
+int n2d2hip_fc_chain_forward(n2d2hip_fc_chain_t chain, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
+                             n2d2hip_stream_t stream);
+
 /* ------------------------------------------------------------------ pool */
 enum { N2D2HIP_POOL_MAX = 0, N2D2HIP_POOL_AVERAGE = 1 };
 /* ref: include/Cell/PoolCell_Frame_Kernels.hpp (Descriptor), include/Cell/PoolCell.hpp:47-55 */

@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libn2d2hip.so")
 GLUE_LIB = os.path.join(LIBDIR, "libn2d2_frame_hip.so")
-SOURCES = ["act.hip", "conv_igemm.hip", "conv_patch.hip", "conv_s2d.hip", "conv_chain.hip", "conv_pipe_w4.hip", "bottleneck.hip", "depthwise.hip", "dw_pw.hip", "conv_small.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip", "diag.hip"]
+SOURCES = ["act.hip", "conv_igemm.hip", "conv_patch.hip", "conv_s2d.hip", "conv_chain.hip", "conv_pipe_w4.hip", "bottleneck.hip", "depthwise.hip", "dw_pw.hip", "conv_small.hip", "fc_chain.hip", "bandwidth.hip", "quantizer.hip", "train_f32.hip", "diag.hip"]
 
 # -ffp-contract=off: float rescales must round the product and the sum
 # separately, as the reference (built for baseline x86-64) does.

@@ -33,7 +33,7 @@ SYMBOLS = [
     "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_conv_chain_supported", "n2d2hip_conv_chain_forward", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", 
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
-    "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward",
+    "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward", "n2d2hip_fc_chain_create", "n2d2hip_fc_chain_destroy", "n2d2hip_fc_chain_forward",
     "n2d2hip_pool_out_dims", "n2d2hip_pool_forward", "n2d2hip_pool_forward_mapped",
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling", "n2d2hip_concat_channels",
     "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_forward_static", "n2d2hip_sat_weight_backward",
@@ -120,6 +120,9 @@ def load():
     lib.n2d2hip_fc_create.argtypes = [I, I, I, I, I, P, P, P, I, P]
     lib.n2d2hip_fc_destroy.argtypes = [P]
     lib.n2d2hip_fc_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_fc_chain_create.argtypes = [I, P, P]
+    lib.n2d2hip_fc_chain_destroy.argtypes = [P]
+    lib.n2d2hip_fc_chain_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_pool_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_pool_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_pool_forward_mapped.argtypes = [P, P, I, I, P, P, P]

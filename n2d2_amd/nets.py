@@ -384,7 +384,7 @@ class GpuNet:
     Activations stay on the device in the private NHWC form between cells; all buffers are allocated once."""
 
     def __init__(self, spec, batch, fuse=True, halo=True, kernel_choice=0, bottlenecks="projection", stem_pool=True,
-                 dw_pw=True, s2d=True, chains=True):
+                 dw_pw=True, s2d=True, chains=True, fc_chains=True):
         """fuse: fold a ScalingCell whose only consumer is an ElemWise sum into that sum (one pass instead of two;
         the rescaled tensor is never written), and a two-input sum into the 1x1 convolution that feeds it.
         halo: a tensor written by a convolution and read only by convolutions is stored with the readers' padding as
@@ -400,6 +400,8 @@ class GpuNet:
         wherever the library takes the pair.
         s2d: store the network input space-to-depth (16-byte pixels of 2 x 2 input pixels, with a border of zeros) when the
         one cell reading it is a first-layer convolution the library serves that way (n2d2hip_conv_s2d_halo).
+        fc_chains: run two or three fully-connected cells, each the only reader of the one before, as one launch
+        (n2d2hip_fc_chain_*) where the library takes them.
         chains: run a block's 3x3 convolution in the launch of the expanding 1x1 convolution + sum that alone reads it
         (n2d2hip_conv_chain_*) where the library takes the pair: the 3x3 convolution's output stays on the chip."""
         from . import capi, runtime as rt
@@ -615,6 +617,36 @@ class GpuNet:
         self.chains = {}
         if fuse and halo and chains:
             self._plan_chains(consumers, by_name, ins_of)
+        # fully-connected cells in a row as one launch (the vectors between them are never written)
+        self.fc_chains = {}
+        if fuse and fc_chains:
+            step_index = {l.name: k for k, (l, c, f) in enumerate(self.steps)}
+            for l in spec.layers:
+                if l.type != "fc" or len(l.inputs) != 1 or l.name in self.folded:
+                    continue
+                readers = consumers.get(l.name, [])
+                if l.name != spec.output and len(readers) == 1 and readers[0].type == "fc" and len(readers[0].inputs) == 1:
+                    continue        # not the last of its run
+                run = [l]
+                while len(run) < 3:
+                    prev = by_name.get(run[0].inputs[0])
+                    if (prev is None or prev.type != "fc" or len(prev.inputs) != 1 or len(consumers[prev.name]) != 1 or prev.name in self.folded
+                            or prev.name == spec.output):
+                        break
+                    run.insert(0, prev)
+                if len(run) < 2 or any(m.name in self.folded for m in run):
+                    continue
+                cells = [self.steps[step_index[m.name]][1] for m in run]
+                if not all(isinstance(c, rt.Fc) for c in cells):
+                    continue
+                fused = rt.FcChain.create(cells)
+                if fused is None:
+                    continue
+                self.steps[step_index[l.name]] = (l, fused, (lambda c, i, o: c.forward(i[0], o)))
+                ins_of[l.name] = ins_of[run[0].name]
+                for m in run[:-1]:
+                    self.folded.add(m.name)
+                self.fc_chains[l.name] = run[:-1]
         self._io = [(ins_of[l.name], self.tensors[l.name]) for l in spec.layers]
         # folded ScalingCells are not launched and their output is never materialised
         for name in self.folded:
@@ -834,6 +866,8 @@ class GpuNet:
             total += self.fused_sums[l.name][1].w.size
         if l.name in self.chains:           # the 3x3 convolution's weights; its output never leaves the chip
             total += self.chains[l.name].w.size
+        if l.name in self.fc_chains:        # the earlier cells' weights; their outputs never leave the chip
+            total += sum(m.w.size for m in self.fc_chains[l.name])
         if l.name in self.stem_pools:       # the convolution's weights; its output never leaves the chip
             total += self.stem_pools[l.name].w.size
         if l.name in self.dw_pws:           # the depthwise weights; its output never leaves the chip
@@ -854,7 +888,7 @@ class GpuNet:
         if l.type == "conv":
             return self.B * l.out_shape[1] * l.out_shape[2] * l.w.size
         if l.type == "fc":
-            return self.B * l.w.size
+            return self.B * (l.w.size + sum(m.w.size for m in self.fc_chains.get(l.name, [])))
         return 0
 
     def activation_bytes(self):

@@ -305,6 +305,33 @@ class Fc:
             self.handle = None
 
 
+class FcChain:
+    """n2d2hip_fc_chain_t: two or three Fc cells, each reading the one before, as one launch."""
+
+    def __init__(self, handle, cells):
+        self.handle, self.cells = handle, cells     # the cells' handles are borrowed: keep them alive
+
+    @staticmethod
+    def create(cells):
+        """None when the library keeps the cells apart."""
+        h = C.c_void_p()
+        arr = (C.c_void_p * len(cells))(*[c.handle for c in cells])
+        rc = lib.n2d2hip_fc_chain_create(len(cells), arr, C.byref(h))
+        if rc == capi.ERR_UNSUPPORTED:
+            return None
+        check(rc)
+        return FcChain(h, list(cells))
+
+    def forward(self, x, out):
+        check(lib.n2d2hip_fc_chain_forward(self.handle, x.ref, out.ref, stream_ptr()))
+        return out
+
+    def __del__(self):
+        if getattr(self, "handle", None) and lib is not None:
+            lib.n2d2hip_fc_chain_destroy(self.handle)
+            self.handle = None
+
+
 class Pool:
     def __init__(self, kind, pool, stride, pad=(0, 0), maps=None):
         """maps: None for one output per channel, else a bool array [channels, outputs] (maps[c, o]: output o pools channel c)."""

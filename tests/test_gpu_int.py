@@ -1170,3 +1170,47 @@ def test_conv_randomized_sweep(rt):
             conv.forward(xin, out)
             assert np.array_equal(out.to_numpy(), want), ("halo", halo_in, halo_out) + tag
     assert ncase >= 40
+
+
+def test_fc_cells_in_a_row_in_one_launch_bit_exact(rt):
+    """n2d2hip_fc_chain_*: two or three FcCells, each reading the one before, in one launch equal the reference cells run in
+    turn: every rescale mode between the cells, raw int32 and byte outputs, signed and unsigned vectors, an input with
+    height and width, a batch that does not fill the last work-group."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    rng = np.random.default_rng(99)
+    for B, shape, widths, modes in ((37, (16, 5, 5), (120, 84, 10), ("fixed_relu_u", "dshift_relu_u", "none_linear")),
+                                    (5, (250, 1, 1), (128, 17), ("float_clip_s", "sshift_lin_s")),
+                                    (64, (8, 3, 2), (33, 128, 7), ("dshift_lin_s", "fixed_clip_s", "fixed_wide")),
+                                    (3, (1024, 1, 1), (64, 64), ("sshift_relu_u", "none_relu"))):
+        print("fc chain", B, shape, widths, modes, flush=True)
+        Cc, H, W = shape
+        x = rng.integers(0, 256, size=(B, Cc, H, W))
+        want = x
+        cells, specs = [], []
+        in_dtype, in_shape = capi.U8B, shape
+        for O, mode in zip(widths, modes):
+            K = in_shape[0] * in_shape[1] * in_shape[2]
+            w = rng.integers(-20, 21, size=(O, K))
+            bias = rng.integers(-500, 500, size=O)
+            spec = _acts(O)[mode]
+            act = rt.Act(O, **spec.kwargs())
+            cells.append(rt.Fc(w, bias, act, in_dtype, in_shape))
+            want = cells_ref.fc_cell(want, w, bias, spec)
+            in_dtype, in_shape = act.out_dtype(), (O, 1, 1)
+        chain = rt.FcChain.create(cells)
+        assert chain is not None
+        dx = rt.DTensor.from_numpy(x, capi.U8B)
+        out = rt.DTensor(B, widths[-1], 1, 1, cells[-1].act.out_dtype())
+        got = chain.forward(dx, out).to_numpy()
+        assert np.array_equal(got, np.asarray(want).astype(np.int64).reshape(got.shape)), (B, shape, widths, modes)
+        # the cells still run on their own, to the same result
+        t = dx
+        for c in cells:
+            t = c.forward(t)
+        assert np.array_equal(t.to_numpy(), got)
+    # what does not qualify is reported: a cell with more than 128 outputs
+    act = rt.Act(200, **_acts(200)["sshift_relu_u"].kwargs())
+    wide = rt.Fc(rng.integers(-5, 6, size=(200, 64)), None, act, capi.U8B, (64, 1, 1))
+    narrow = rt.Fc(rng.integers(-5, 6, size=(10, 200)), None, rt.Act(10, **_acts(10)["none_linear"].kwargs()), capi.U8B, (200, 1, 1))
+    assert rt.FcChain.create([wide, narrow]) is None
