@@ -687,7 +687,42 @@ FcCell_Frame_HIP<T>::FcCell_Frame_HIP(const DeepNet& /*deepNet*/, const std::str
 template <class T>
 FcCell_Frame_HIP<T>::~FcCell_Frame_HIP()
 {
+    if (mChain) n2d2hip_fc_chain_destroy(mChain);
     if (mFc) n2d2hip_fc_destroy(mFc);
+}
+
+template <class T>
+bool FcCell_Frame_HIP<T>::fuseChain(const std::vector<FcCell_Frame_HIP<T>*>& earlier)
+{
+    if (mChain || earlier.empty() || !mFc || mInputs.size() != 1)
+        return false;
+    std::vector<n2d2hip_fc_t> cells;
+    for (FcCell_Frame_HIP<T>* c : earlier) {
+        if (!c || !c->mFc || c->foldedInto() || c->mChain || c->mInputs.size() != 1)
+            return false;
+        cells.push_back(c->mFc);
+    }
+    cells.push_back(mFc);
+    if (n2d2hip_fc_chain_create((int)cells.size(), cells.data(), &mChain) != N2D2HIP_OK) {
+        mChain = nullptr;
+        return false;
+    }
+    mChained = earlier;
+    for (FcCell_Frame_HIP<T>* c : mChained)
+        c->setFoldedInto(this);
+    return true;
+}
+
+template <class T>
+void FcCell_Frame_HIP<T>::clearFusion()
+{
+    if (mChain) {
+        n2d2hip_fc_chain_destroy(mChain);
+        mChain = nullptr;
+        for (FcCell_Frame_HIP<T>* c : mChained)
+            c->setFoldedInto(nullptr);
+        mChained.clear();
+    }
 }
 
 template <class T>
@@ -718,9 +753,28 @@ void FcCell_Frame_HIP<T>::initialize()
 template <class T>
 void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
 {
+    prepare();
+    launch();
+}
+
+template <class T>
+void FcCell_Frame_HIP<T>::launch()
+{
+    if (mChain)
+        checkStatus(n2d2hip_fc_chain_forward(mChain, &mChained[0]->mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    else
+        checkStatus(n2d2hip_fc_forward(mFc, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
+    mOutputs.invalidateHost();
+}
+
+template <class T>
+bool FcCell_Frame_HIP<T>::prepare()
+{
     n2d2hip_act_t act = activationHandle();
     const int inDType = prepareGathered();
-    if (mDirty || activationGeneration() != mFcActGen || !mFc || mFcNbInputs != mInputs.size()) {
+    bool rebuilt = false;
+    if (mDirty || activationGeneration() != mFcActGen || !mFc || mFcNbInputs != mInputs.size() || inDType != mFcInDType) {
+        clearFusion();
         if (mFc) { n2d2hip_fc_destroy(mFc); mFc = nullptr; }
         const size_t K = (size_t)mNbChannels * mInH * mInW;
         if (mWeights.size() != K * mNbOutputs)
@@ -744,10 +798,11 @@ void FcCell_Frame_HIP<T>::propagate(bool /*inference*/)
                                       inDType, &mFc));
         mFcActGen = activationGeneration();
         mFcNbInputs = mInputs.size();
+        mFcInDType = inDType;
         mDirty = false;
+        rebuilt = true;
     }
-    checkStatus(n2d2hip_fc_forward(mFc, mInputs.size() > 1 ? &gatherInputs() : &mInputs[0]->desc(), &mOutputs.desc(), mStream));
-    mOutputs.invalidateHost();
+    return rebuilt;
 }
 
 template <> Registrar<FcCell> FcCell_Frame_HIP<float>::mRegistrar("Frame_HIP", FcCell_Frame_HIP<float>::create, Registrar<FcCell>::Type<float>());
@@ -1731,6 +1786,8 @@ void DeepNet::setFusion(bool enabled)
                 pool->clearFusion();
             if (auto* conv = dynamic_cast<ConvCell_Frame_HIP<float>*>(f))
                 conv->clearFusion();
+            if (auto* fc = dynamic_cast<FcCell_Frame_HIP<float>*>(f))
+                fc->clearFusion();
             f->setOutputsHalo(0);
         }
     }
@@ -1894,6 +1951,35 @@ void DeepNet::planFusion()
             || halo[conv3->parentCells()[0]] < 1)
             continue;
         ew->fuseChain(conv3);
+    }
+    // Fully-connected cells in a row, each read by the next alone (a classifier head), run in the launch of the last one,
+    // up to three of them, where the device library takes the run.
+    std::map<const Cell_Frame_HIP*, Cell_Frame_HIP*> reader;
+    for (Cell_Frame_HIP* f : mFrames) {
+        if (auto* fc = dynamic_cast<FcCell_Frame_HIP<float>*>(f))
+            fc->clearFusion();
+        for (Cell_Frame_HIP* p : f->parentCells())
+            reader[p] = f;
+    }
+    auto feedsOneFc = [&](Cell_Frame_HIP* c) {
+        auto* next = consumers[c] == 1 ? dynamic_cast<FcCell_Frame_HIP<float>*>(reader[c]) : nullptr;
+        return next && next->parentCells().size() == 1;
+    };
+    for (Cell_Frame_HIP* f : mFrames) {
+        auto* last = dynamic_cast<FcCell_Frame_HIP<float>*>(f);
+        if (!last || last->parentCells().size() != 1 || feedsOneFc(last))
+            continue;
+        std::vector<FcCell_Frame_HIP<float>*> earlier;
+        for (Cell_Frame_HIP* c = last; earlier.size() < 2;) {
+            auto* p = dynamic_cast<FcCell_Frame_HIP<float>*>(c->parentCells()[0]);
+            if (!p || consumers[p] != 1 || p->parentCells().size() != 1 || p->foldedInto())
+                break;
+            earlier.insert(earlier.begin(), p);
+            c = p;
+        }
+        // the library may take the last two cells where it declines all three
+        while (!earlier.empty() && !last->fuseChain(earlier))
+            earlier.erase(earlier.begin());
     }
     mPlanned = true;
 }

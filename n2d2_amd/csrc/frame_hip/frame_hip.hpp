@@ -611,6 +611,15 @@ public:
     using Cell_Frame_HIP::addInput;
     void initialize();
     void propagate(bool inference = false);
+    bool prepare();
+    void launch();
+    n2d2hip_fc_t fcHandle() const { return mFc; }
+    // Graph-level fusion (DeepNet::planFusion): this cell ends a run of fully-connected cells, each read by the next
+    // alone; `earlier` (one or two cells, first to last) are computed in this cell's launch and their outputs are never
+    // stored.  Returns false, and changes nothing, where the device library declines the run.
+    bool fuseChain(const std::vector<FcCell_Frame_HIP<T>*>& earlier);
+    void clearFusion();
+    size_t nbChained() const { return mChained.size(); }
 
 protected:
     void setOutputsDims();
@@ -619,6 +628,9 @@ private:
     n2d2hip_fc_t mFc;
     unsigned long mFcActGen;
     size_t mFcNbInputs;
+    int mFcInDType = -1;
+    n2d2hip_fc_chain_t mChain = nullptr;
+    std::vector<FcCell_Frame_HIP<T>*> mChained;
     static Registrar<FcCell> mRegistrar;
 };
 

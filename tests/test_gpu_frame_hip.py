@@ -35,7 +35,39 @@ def test_lenet_through_the_registrar(fh):
     from n2d2_amd import nets
     spec = nets.lenet()
     x = np.random.default_rng(31).integers(0, 256, size=(64, 1, 32, 32))
-    _compare(fh, spec, x, [l.name for l in spec.layers])
+    names = [l.name for l in spec.layers]
+    # the three fully-connected cells run in the launch of the last one; the two before it are not materialised
+    from n2d2_amd import capi
+    net = _compare(fh, spec, x, [n for n in names if n not in ("fc1", "fc2")])
+    assert net.nb_folded == 2
+    with pytest.raises(fh.FrameHipError) as e:
+        net.outputs("fc2")
+    assert "not materialised" in str(e.value)
+    with capi.launch_log() as log:
+        net.propagate()
+    assert log.entries[-1][0].startswith("fc_chain_kernel") and len(log.entries) == 5
+    # launched apart every cell is readable, and back together the logits are the same
+    net.set_fusion(False)
+    net.propagate()
+    assert net.nb_folded == 0
+    want = cells_of(spec, x, names)
+    for n in names:
+        assert np.array_equal(net.outputs(n), want[n]), n
+    net.set_fusion(True)
+    net.propagate()
+    assert net.nb_folded == 2 and np.array_equal(net.outputs("fc3"), want["fc3"])
+    # new weights on a cell in the middle of the run: the cells and the plan are made again
+    w = np.array(spec.layers[5].w)
+    spec2 = nets.lenet()
+    spec2.layers[5].w = np.roll(w, 1, axis=0)
+    net.set_weights("fc2", spec2.layers[5].w.astype(np.float32))
+    net.propagate()
+    assert net.nb_folded == 2 and np.array_equal(net.outputs("fc3"), cells_of(spec2, x, ["fc3"])["fc3"])
+
+
+def cells_of(spec, x, keep):
+    from oracle import cells
+    return cells.run_net(spec, x, keep=keep)
 
 
 def test_resnet50_through_the_registrar(fh):

@@ -41,8 +41,13 @@ def test_lenet_config_full_batch():
     spec = nets.lenet()
     x = np.random.default_rng(11).integers(0, 256, size=(256, 1, 32, 32))
     net = _run_both(spec, x, [l.name for l in spec.layers])
+    # the three fully-connected cells are one launch
+    assert [(k, [m.name for m in v]) for k, v in net.fc_chains.items()] == [("fc3", ["fc1", "fc2"])] and len(net.launched) == 5
     logits = net.tensors["fc3"].to_numpy()
     assert logits.shape == (256, 10, 1, 1) and np.abs(logits).max() > 1000
+    # cell by cell, the vectors between the fully-connected cells are stored and checked too
+    apart = _run_both(spec, x, [l.name for l in spec.layers], fuse=False)
+    assert not apart.fc_chains and len(apart.launched) == 7
 
 
 def test_stage_convolution_config_full_batch():
