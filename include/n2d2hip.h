@@ -221,6 +221,11 @@ int n2d2hip_conv_s2d_halo(n2d2hip_conv_t conv, const struct n2d2hip_pool_desc* p
 /* 1 if this convolution runs on the kernel that reads and writes tensors with a halo (8-bit weights, ungrouped, input
  * channels a multiple of 64), else 0.  No counterpart in the reference, whose padding is implicit in its tap loop. */
 int n2d2hip_conv_accepts_halo(n2d2hip_conv_t conv);
+/* The part of that rule a planner can ask before the cell exists, from the descriptor alone: 1 if a convolution of this
+ * shape can be one that n2d2hip_conv_accepts_halo accepts (ungrouped, 4- or 8-bit weights, input channels a multiple of 64,
+ * at most 31 taps, no dilation, more than 4 outputs), else 0.  n2d2hip_conv_accepts_halo has the last word (it also knows
+ * the cell's rescale).  No counterpart in the reference. */
+int n2d2hip_conv_desc_reads_halo(const n2d2hip_conv_desc* desc);
 
 
 /* -------------------------------------------------------------------- fc */
@@ -263,6 +268,10 @@ int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* desc, int H, int W, int* outH
  * multiple of 16 may write an `out` with a halo (its readers' padding), the other poolings refuse one. */
 int n2d2hip_pool_forward(const n2d2hip_pool_desc* desc, const n2d2hip_tensor* in, const n2d2hip_tensor* out,
                          n2d2hip_stream_t stream);
+/* 1 if n2d2hip_pool_forward with this descriptor on an NHWC byte tensor of H x W pixels and channel stride `cs` writes an
+ * output with a halo (the rule above, and every window holding at least one input element), else 0: what a planner asks
+ * before it gives a pooling's output a border.  No counterpart in the reference. */
+int n2d2hip_pool_writes_halo(const n2d2hip_pool_desc* desc, int H, int W, int cs);
 
 /* Pooling with a connection map (ref: src/Cell/PoolCell_Frame_Kernels.cpp:60-75,150-185, the `maps` argument of forwardMax /
  * forwardAverage): output o pools its window over every input channel c with maps[o * map_channels + c] != 0 (`maps`:
@@ -339,6 +348,10 @@ typedef struct n2d2hip_bottleneck_s* n2d2hip_bottleneck_t;
 int n2d2hip_bottleneck_create(n2d2hip_conv_t reduce, n2d2hip_conv_t conv3x3, n2d2hip_conv_t expand, n2d2hip_conv_t projection,
                               n2d2hip_bottleneck_t* bottleneck);
 int n2d2hip_bottleneck_destroy(n2d2hip_bottleneck_t bottleneck);
+/* 1 where the one launch is expected to be faster than the plan the cells would otherwise run in, for `batch` images of
+ * in_h x in_w pixels: today a block with a projection shortcut (one launch for four); a block without one is as fast as
+ * its reduce convolution followed by n2d2hip_conv_chain_forward.  Planners ask this instead of restating the rule. */
+int n2d2hip_bottleneck_pays(n2d2hip_bottleneck_t bottleneck, int batch, int in_h, int in_w);
 /* `in`: the block's input, NHWC bytes with a border of one pixel (halo 1; rows of at most 61 pixels); `out`: the sum's
  * output (the 3x3 convolution's when `expand` is NULL), NHWC bytes of the same height and width, with or without a border. */
 int n2d2hip_bottleneck_forward(n2d2hip_bottleneck_t bottleneck, const n2d2hip_tensor* in, const n2d2hip_tensor* out,

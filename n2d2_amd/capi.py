@@ -29,12 +29,12 @@ SYMBOLS = [
     "n2d2hip_strerror", "n2d2hip_last_error", "n2d2hip_version", "n2d2hip_measure_clock",
     "n2d2hip_launch_log_begin", "n2d2hip_launch_log_end", "n2d2hip_launch_log_entry", "n2d2hip_nhwc_cs", "n2d2hip_tensor_bytes", "n2d2hip_tensor_clear",
     "n2d2hip_convert", "n2d2hip_act_create", "n2d2hip_act_destroy", "n2d2hip_scaling_forward",
-    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_s2d_halo", "n2d2hip_conv_accepts_halo",
-    "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_conv_chain_supported", "n2d2hip_conv_chain_forward", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_forward",
+    "n2d2hip_conv_create", "n2d2hip_conv_destroy", "n2d2hip_conv_out_dims", "n2d2hip_conv_forward", "n2d2hip_conv_s2d_halo", "n2d2hip_conv_accepts_halo", "n2d2hip_conv_desc_reads_halo",
+    "n2d2hip_conv_fuse_sum", "n2d2hip_conv_forward_sum", "n2d2hip_conv_chain_supported", "n2d2hip_conv_chain_forward", "n2d2hip_bottleneck_create", "n2d2hip_bottleneck_destroy", "n2d2hip_bottleneck_pays", "n2d2hip_bottleneck_forward",
     "n2d2hip_conv_accepts_maxpool", "n2d2hip_conv_forward_maxpool", 
     "n2d2hip_dw_pw_create", "n2d2hip_dw_pw_destroy", "n2d2hip_dw_pw_forward", "n2d2hip_dw_pw_pays",
     "n2d2hip_fc_create", "n2d2hip_fc_destroy", "n2d2hip_fc_forward", "n2d2hip_fc_chain_create", "n2d2hip_fc_chain_destroy", "n2d2hip_fc_chain_forward",
-    "n2d2hip_pool_out_dims", "n2d2hip_pool_forward", "n2d2hip_pool_forward_mapped",
+    "n2d2hip_pool_out_dims", "n2d2hip_pool_forward", "n2d2hip_pool_writes_halo", "n2d2hip_pool_forward_mapped",
     "n2d2hip_elemwise_create", "n2d2hip_elemwise_destroy", "n2d2hip_elemwise_forward", "n2d2hip_elemwise_fold_input_scaling", "n2d2hip_concat_channels",
     "n2d2hip_quantizer_workspace_bytes", "n2d2hip_sat_weight_forward", "n2d2hip_sat_weight_forward_static", "n2d2hip_sat_weight_backward",
     "n2d2hip_sat_act_forward", "n2d2hip_sat_act_backward", "n2d2hip_lsq_forward", "n2d2hip_lsq_backward",
@@ -101,6 +101,7 @@ def load():
     lib.n2d2hip_conv_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_conv_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_conv_accepts_halo.argtypes = [P]
+    lib.n2d2hip_conv_desc_reads_halo.argtypes = [P]
     lib.n2d2hip_conv_s2d_halo.argtypes = [P, P, I, I]
     lib.n2d2hip_tensor_clear.argtypes = [P, P]
     lib.n2d2hip_conv_fuse_sum.argtypes = [P, P, I, I]
@@ -110,6 +111,7 @@ def load():
     lib.n2d2hip_conv_chain_forward.argtypes = [P, P, P, P, P, P]
     lib.n2d2hip_bottleneck_create.argtypes = [P, P, P, P, P]
     lib.n2d2hip_bottleneck_destroy.argtypes = [P]
+    lib.n2d2hip_bottleneck_pays.argtypes = [P, I, I, I]
     lib.n2d2hip_bottleneck_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_conv_accepts_maxpool.argtypes = [P, P, C.c_int, C.c_int]
     lib.n2d2hip_conv_forward_maxpool.argtypes = [P, P, P, P, P]
@@ -125,6 +127,7 @@ def load():
     lib.n2d2hip_fc_chain_forward.argtypes = [P, P, P, P]
     lib.n2d2hip_pool_out_dims.argtypes = [P, I, I, P, P]
     lib.n2d2hip_pool_forward.argtypes = [P, P, P, P]
+    lib.n2d2hip_pool_writes_halo.argtypes = [P, I, I, I]
     lib.n2d2hip_pool_forward_mapped.argtypes = [P, P, I, I, P, P, P]
     lib.n2d2hip_elemwise_create.argtypes = [I, I, I, P, P, P, P]
     lib.n2d2hip_elemwise_destroy.argtypes = [P]

@@ -460,6 +460,22 @@ int n2d2hip_pool_out_dims(const n2d2hip_pool_desc* d, int H, int W, int* outH, i
     return N2D2HIP_OK;
 }
 
+// windows that all hold at least one input element, square 2x2 or 3x3, 16-byte channel groups: the kernel that may write
+// its output with a border
+static bool pool_fast(const n2d2hip_pool_desc* d, int H, int W, int cs, int OH, int OW)
+{
+    return d->pooling == N2D2HIP_POOL_MAX && cs % 16 == 0 && d->poolW == d->poolH && (d->poolW == 2 || d->poolW == 3)
+        && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < W && (OH - 1) * d->strideY - d->padY < H;
+}
+
+int n2d2hip_pool_writes_halo(const n2d2hip_pool_desc* d, int H, int W, int cs)
+{
+    int OH, OW;
+    if (!d || n2d2hip_pool_out_dims(d, H, W, &OH, &OW) != N2D2HIP_OK)
+        return 0;
+    return pool_fast(d, H, W, cs, OH, OW) ? 1 : 0;
+}
+
 int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
     int rc, OH, OW;
@@ -476,9 +492,7 @@ int n2d2hip_pool_forward(const n2d2hip_pool_desc* d, const n2d2hip_tensor* in, c
     const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 64));
     const unsigned flip = in->dtype == N2D2HIP_U8 ? 0x80808080u : 0u;
     const int zp = in->dtype == N2D2HIP_I8 ? 0 : 128;      // after the flip, U8 bytes read as value-128 too
-    // windows that all hold at least one input element, square 2x2 or 3x3, 16-byte channel groups
-    const bool fast = d->pooling == N2D2HIP_POOL_MAX && in->cs % 16 == 0 && d->poolW == d->poolH && (d->poolW == 2 || d->poolW == 3)
-        && d->padX < d->poolW && d->padY < d->poolH && (OW - 1) * d->strideX - d->padX < in->W && (OH - 1) * d->strideY - d->padY < in->H;
+    const bool fast = pool_fast(d, in->H, in->W, in->cs, OH, OW);
     N2D2HIP_REQUIRE(out->halo == 0 || fast, N2D2HIP_ERR_UNSUPPORTED,
                     "pool_forward: only the 2x2 / 3x3 max pooling of 16-byte channel groups writes an output with a halo");
     if (d->pooling == N2D2HIP_POOL_AVERAGE && OH == 1 && OW == 1 && d->poolW == in->W && d->poolH == in->H && d->padX == 0 && d->padY == 0) {

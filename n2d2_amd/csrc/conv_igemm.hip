@@ -784,18 +784,25 @@ int n2d2hip_conv_destroy(n2d2hip_conv_t c)
 }
 
 // Can this convolution run on the pipelined kernel, and with which channel tile?
+// What the pipelined kernel asks of a convolution's shape (its rescale is the cell's business, below)
+static bool pipe_shape(const n2d2hip_conv_desc& d)
+{
+    const bool depthwise = d.groups > 1 && d.groups == d.C && d.C == d.O;       // (other groups run as a full connection)
+    return d.O > 4              // (a pixel of at most 4 outputs is one dword: the general kernel stores those)
+        && !depthwise && (d.weight_bits == 4 || d.weight_bits == 8) && d.C % 64 == 0 && d.kW * d.kH <= 31;
+}
+
 static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
 {
     const n2d2hip_conv_desc& d = c->desc;
     const int opad_n = round_up(d.O, 64);
     *bn128 = opad_n % 128 == 0 || opad_n > 256;
     const int k = c->act->args.kind;
-    if (d.O <= 4)               // a pixel of the output is one dword: the general kernel stores those
+    if (!pipe_shape(d))
         return false;
     if (d.weight_bits == 4)     // packed weights: integer rescale only
-        return c->d_w4img != nullptr && d.kW * d.kH <= 31 && k == EPI_I24 && c->bias_folded;
-    return !c->depthwise && !c->pix4 && d.weight_bits == 8 && c->in_cs == d.C && d.C % 64 == 0 && d.kW * d.kH <= 31
-        && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
+        return c->d_w4img != nullptr && k == EPI_I24 && c->bias_folded;
+    return !c->depthwise && !c->pix4 && c->in_cs == d.C && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
 }
 
 // Is this convolution served by the space-to-depth first-layer kernel on an H x W input?  Returns the border it needs, or -1.
@@ -1319,6 +1326,11 @@ int n2d2hip_conv_accepts_halo(n2d2hip_conv_t c)
 {
     bool bn128;
     return c && pipe_eligible(c, &bn128) && c->desc.dilX == 1 && c->desc.dilY == 1 && !(c->desc.kernel_choice & N2D2HIP_KERNEL_NO_PIPE) ? 1 : 0;
+}
+
+int n2d2hip_conv_desc_reads_halo(const n2d2hip_conv_desc* d)
+{
+    return d && pipe_shape(*d) && d->dilX == 1 && d->dilY == 1 && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PIPE) ? 1 : 0;
 }
 
 int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype)

@@ -954,8 +954,7 @@ bool PoolCell_Frame_HIP<T>::writesHalo() const
         return false;
     const n2d2hip_pool_desc d = poolDesc();
     const n2d2hip_tensor& x = mInputs[0]->desc();
-    return d.pooling == N2D2HIP_POOL_MAX && x.halo == 0 && x.cs % 16 == 0 && d.poolW == d.poolH && (d.poolW == 2 || d.poolW == 3)
-        && d.padX < d.poolW && d.padY < d.poolH && ((int)mOutW - 1) * d.strideX - d.padX < x.W && ((int)mOutH - 1) * d.strideY - d.padY < x.H;
+    return x.halo == 0 && n2d2hip_pool_writes_halo(&d, x.H, x.W, x.cs) != 0;
 }
 
 template <class T>
@@ -1125,6 +1124,12 @@ bool ElemWiseCell_Frame_HIP::fuseBottleneck(Cell_Frame_HIP* reduce, Cell_Frame_H
     if (rc == N2D2HIP_ERR_UNSUPPORTED)
         return false;
     checkStatus(rc);
+    // the library also knows where the one launch is the faster plan
+    const n2d2hip_tensor& x = input->getDeviceOutputs().desc();
+    if (!n2d2hip_bottleneck_pays(b, x.B, x.H, x.W)) {
+        n2d2hip_bottleneck_destroy(b);
+        return false;
+    }
     mBottleneck = b;
     mBottleneckIn = input;
     mBottleneckCells = {reduce, conv3x3};

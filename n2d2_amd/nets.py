@@ -418,8 +418,9 @@ class GpuNet:
         C, H, W = spec.in_shape
 
         def reads_halo(m):
-            return (m.type == "conv" and len(m.inputs) == 1 and m.groups == 1 and m.weight_bits in (4, 8) and m.w.shape[1] % 64 == 0
-                    and m.w.shape[2] * m.w.shape[3] <= 31 and tuple(m.dil) == (1, 1))
+            # (asked of the library, from the layer's shape: the reader's cell does not exist yet when its input is allocated)
+            return (m.type == "conv" and len(m.inputs) == 1
+                    and rt.Conv.shape_reads_halo(m.w.shape, m.stride, m.pad, m.dil, m.groups, m.weight_bits, kernel_choice))
 
         def halo_of(l, cell):
             """Border to store around l's output: the largest padding among its readers, if all of them can use it."""
@@ -579,15 +580,10 @@ class GpuNet:
                 producer_cell = self.steps[step_index[l.name]][1]
                 writes = (l.name in self.fused_sums or l.name in self.stem_pools
                           or (l.type == "conv" and producer_cell.accepts_halo())
-                          or (l.type == "pool" and l.kind == "max" and tuple(l.pool) in ((2, 2), (3, 3)) and len(l.inputs) == 1))
+                          or (l.type == "pool" and len(l.inputs) == 1 and producer_cell.writes_halo(ins_of[l.name][0])))
                 if not writes:
                     continue
                 nx = rt.DTensor(t.B, t.C, t.H, t.W, t.dtype, halo=h)
-                if l.type == "pool" and l.name not in self.stem_pools:
-                    try:        # does this pooling write a border?  (asked once, on the real tensors)
-                        producer_cell.forward(ins_of[l.name][0], nx)
-                    except capi.N2D2HipError:
-                        continue
                 for lst in ins_of.values():
                     for k, u in enumerate(lst):
                         if u is t:
@@ -717,15 +713,12 @@ class GpuNet:
                     proj = cand
             elif proj.inputs[0] != xname:
                 continue
-            if self._bottleneck_mode == "projection" and proj is None:
-                continue
             readers = {conv_a.name, proj.name if proj is not None else sum_name} | ({other_name} if scaled else set())
             if x is None or xname == "input" or not {m.name for m in consumers[xname]} <= readers | {sum_name}:
                 continue
             producer = by_name[xname]
-            can_write_halo = (producer.type == "pool" and producer.kind == "max" and tuple(producer.pool) in ((2, 2), (3, 3))
-                              and len(producer.inputs) == 1) \
-                or xname in self.fused_sums or xname in self.bottlenecks
+            can_write_halo = (xname in self.fused_sums or xname in self.bottlenecks or xname in self.stem_pools
+                              or (producer.type == "pool" and len(producer.inputs) == 1 and cell_of[xname].writes_halo(ins_of[xname][0])))
             if x.halo not in (0, 1) or (x.halo == 0 and not can_write_halo):
                 continue
             moved = False
@@ -737,22 +730,15 @@ class GpuNet:
                 moved = True
             bn = rt.Bottleneck.create(cell_of[conv_a.name], cell_of[conv_b.name], cell_of[expand.name],
                                       cell_of[proj.name] if proj is not None else None)
-            if bn is None:
+            # the library takes the block or not, and knows where the one launch is the faster plan
+            if bn is None or (self._bottleneck_mode != "all" and not bn.pays(x.B, x.H, x.W)):
                 if moved:
-                    cell_of[expand.name].fuse_sum(None, 0, 0)
+                    cell_of[expand.name].fuse_sum(None, 0, 0)       # (the projection still holds the sum)
                 continue
             if moved:
                 cell_of[proj.name].fuse_sum(None, 0, 0)
             if x.halo == 0:
-                try:
-                    nx = rt.DTensor(x.B, x.C, x.H, x.W, x.dtype, halo=1)
-                    if producer.type == "pool" and xname not in self.stem_pools:       # does this pooling write a border?  (probed once, on the real tensors)
-                        cell_of[xname].forward(ins_of[xname][0], nx)
-                except self.capi.N2D2HipError:
-                    if moved:
-                        cell_of[expand.name].fuse_sum(None, 0, 0)
-                        cell_of[proj.name].fuse_sum(sum_cell, sum_layer.inputs.index(proj.name), self.tensors[expand.name].dtype)
-                    continue
+                nx = rt.DTensor(x.B, x.C, x.H, x.W, x.dtype, halo=1)
                 for lst in ins_of.values():
                     for k, t in enumerate(lst):
                         if t is x:

@@ -149,6 +149,10 @@ class Bottleneck:
         check(rc)
         return Bottleneck(h, (reduce, conv3x3, expand, projection))
 
+    def pays(self, batch, H, W):
+        """True where the library expects the one launch to be faster than the plan the cells would otherwise run in."""
+        return bool(lib.n2d2hip_bottleneck_pays(self.handle, batch, H, W))
+
     def forward(self, x, out):
         check(lib.n2d2hip_bottleneck_forward(self.handle, x.ref, out.ref, stream_ptr()))
         return out
@@ -242,6 +246,16 @@ class Conv:
     def accepts_halo(self):
         """True when this convolution reads and writes tensors that carry their padding as a border of zeros."""
         return bool(lib.n2d2hip_conv_accepts_halo(self.handle))
+
+    @staticmethod
+    def shape_reads_halo(w_shape, stride, pad, dil, groups, weight_bits, kernel_choice=0):
+        """What a planner can ask before the cell exists: can a convolution of this shape ([O, C/groups, kH, kW] weights) be one
+        that reads a tensor with a border?  The cell's own accepts_halo() has the last word."""
+        O, Cg, kH, kW = w_shape
+        pad = tuple(pad) if len(pad) == 4 else (pad[0], pad[1], pad[0], pad[1])
+        d = capi.ConvDesc(Cg * groups, O, kW, kH, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dil[0], dil[1], groups, weight_bits,
+                          kernel_choice)
+        return bool(lib.n2d2hip_conv_desc_reads_halo(C.byref(d)))
 
     def forward(self, x, out=None, out_dtype=None):
         if out is None:
@@ -342,6 +356,10 @@ class Pool:
             m = np.ascontiguousarray(np.asarray(maps, dtype=np.uint8).T)      # one row per output
             self.nb_channels, self.nb_outputs = m.shape[1], m.shape[0]
             self.maps = torch.from_numpy(m.reshape(-1)).cuda()
+
+    def writes_halo(self, x):
+        """True when this pooling of x can store its output with a border (its readers' padding)."""
+        return self.maps is None and bool(lib.n2d2hip_pool_writes_halo(C.byref(self.desc), x.H, x.W, x.cs))
 
     def make_output(self, x):
         oh, ow = C.c_int(), C.c_int()

@@ -79,3 +79,32 @@ def test_tensors_with_a_border_are_sized_and_policed_on_the_host():
     nchw = capi.Tensor(fake, capi.I32, capi.NCHW, 2, 64, 5, 7, 64, 1)
     assert lib.n2d2hip_tensor_clear(C.byref(nchw), None) == capi.ERR_INVALID                   # only NHWC byte tensors have one
     assert lib.n2d2hip_conv_accepts_halo(None) == 0
+
+
+def test_planning_questions_answered_from_descriptors_alone():
+    """What a planner asks before any cell exists is answered on the host: which convolution shapes can read a tensor that
+    carries its padding, which poolings can write one."""
+    from n2d2_amd import capi
+    lib = capi.lib
+
+    def conv(C_, O, k, groups=1, bits=8, dil=1, choice=0):
+        return capi.ConvDesc(C_, O, k, k, 1, 1, k // 2, k // 2, k // 2, k // 2, dil, dil, groups, bits, choice)
+    ok = lambda d: lib.n2d2hip_conv_desc_reads_halo(C.byref(d))
+    assert ok(conv(64, 64, 3)) == 1 and ok(conv(128, 256, 1)) == 1 and ok(conv(64, 64, 3, bits=4)) == 1 and ok(conv(64, 128, 5)) == 1
+    assert ok(conv(64, 128, 3, groups=2)) == 1                              # groups other than depthwise run as a full connection
+    assert ok(conv(3, 64, 7)) == 0 and ok(conv(96, 64, 3)) == 0             # input channels not a multiple of 64
+    assert ok(conv(64, 64, 3, groups=64)) == 0                              # depthwise
+    assert ok(conv(64, 64, 3, dil=2)) == 0 and ok(conv(64, 64, 7)) == 0     # dilation; more than 31 taps
+    assert ok(conv(64, 4, 3)) == 0                                          # a pixel of at most 4 outputs
+    assert ok(conv(64, 64, 3, choice=capi.KERNEL_NO_PIPE)) == 0
+    assert lib.n2d2hip_conv_desc_reads_halo(None) == 0
+
+    def pool(kind, k, stride, pad):
+        return capi.PoolDesc(kind, k, k, stride, stride, pad, pad)
+    wh = lambda d, H, W, cs: lib.n2d2hip_pool_writes_halo(C.byref(d), H, W, cs)
+    assert wh(pool(capi.POOL_MAX, 3, 2, 1), 112, 112, 64) == 1 and wh(pool(capi.POOL_MAX, 2, 2, 0), 28, 28, 16) == 1
+    assert wh(pool(capi.POOL_MAX, 3, 2, 1), 112, 112, 4) == 0               # channel stride of 4: the general kernel
+    assert wh(pool(capi.POOL_AVERAGE, 2, 2, 0), 28, 28, 16) == 0 and wh(pool(capi.POOL_MAX, 5, 2, 0), 28, 28, 16) == 0
+    assert wh(pool(capi.POOL_MAX, 3, 2, 3), 28, 28, 16) == 0                # padding as large as the window
+    assert lib.n2d2hip_pool_writes_halo(None, 28, 28, 16) == 0
+    assert lib.n2d2hip_bottleneck_pays(None, 128, 56, 56) == 0

@@ -363,6 +363,10 @@ def test_model_file_syntax_of_the_reference(fh):
     from oracle import cells
     keep = [l.name for l in spec.layers]
     want = cells.run_net(spec, x, keep=keep)
+    # (fc_b computes fc_a in its own launch: read every cell with the cells launched apart, the logits both ways)
+    assert net.nb_folded == 1 and np.array_equal(net.outputs("fc_b"), want["fc_b"])
+    net.set_fusion(False)
+    net.propagate()
     for name in keep:
         assert np.array_equal(net.outputs(name), want[name]), name
     with pytest.raises(fh.FrameHipError, match="refers to unknown section"):
@@ -823,6 +827,10 @@ def test_float_rescaled_net_runs_after_approximation(fh, tmp_path):
     net.propagate()
     keep = [l.name for l in spec.layers]
     want = cells.run_net(spec, x, keep=keep)
+    # the three FcCells as one launch (the approximated rescales travel with the cells), then every cell on its own
+    assert net.nb_folded == 2 and np.array_equal(net.outputs("fc3"), want["fc3"])
+    net.set_fusion(False)
+    net.propagate()
     for name in keep:
         assert np.array_equal(net.outputs(name), want[name]), name
 
