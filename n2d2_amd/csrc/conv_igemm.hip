@@ -393,6 +393,7 @@ void launch_pipe(ConvPipeArgs a, int valid, bool hi16, int grid, hipStream_t str
             N2D2HIP_LAUNCH_T(conv_pipe_kernel, (NW, BK, NI, NJ, WGM, EPI_I24, S, 0, false, true), dim3(grid), dim3(NW * 64), 0, stream, a);
         }
         break;
+    case EPI_I64: N2D2HIP_PIPE(EPI_I64); break;     // (multipliers of 24 bits and more: N2D2's 32-bit fixed point)
     default: N2D2HIP_PIPE(EPI_F32); break;
     }
 #undef N2D2HIP_PIPE
@@ -802,7 +803,7 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
         return false;
     if (d.weight_bits == 4)     // packed weights: integer rescale only
         return c->d_w4img != nullptr && k == EPI_I24 && c->bias_folded;
-    return !c->depthwise && !c->pix4 && c->in_cs == d.C && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32);
+    return !c->depthwise && !c->pix4 && c->in_cs == d.C && (k == EPI_RAW || (k == EPI_I24 && c->bias_folded) || k == EPI_F32 || k == EPI_I64);
 }
 
 // Is this convolution served by the space-to-depth first-layer kernel on an H x W input?  Returns the border it needs, or -1.

@@ -184,6 +184,8 @@ def test_conv_cell_bit_exact(rt, case):
     xd = rt.DTensor.from_numpy(x, in_dt)
     acts = _acts(O)
     names = list(acts) if name in ("3x3_c64", "c20_o10_asym") else ["none_linear", "sshift_relu_u", "dshift_lin_s", "fixed_relu_u", "float_relu_u"]
+    if Cc % 64 == 0 and "fixed_wide" not in names:
+        names.append("fixed_wide")         # (a multiplier of 30 bits on the pipelined kernel: the 64-bit product)
     for an in names:
         spec = acts[an]
         _say("conv %s %s" % (name, an))
@@ -764,6 +766,21 @@ def test_conv_reads_and_writes_halo_tensors(rt):
         out = rt.DTensor(B, O, H, W, capi.U8B, halo=halo)
         c1b.forward_sum(dx, rt.DTensor.from_numpy(other, capi.U8B), out)
         assert np.array_equal(out.to_numpy(), want)
+    # multipliers of 30 bits (the 64-bit product): written with a border, read from one
+    from oracle.cells import ActSpec
+    x = rng.integers(0, 256, size=(2, 64, 9, 7))
+    w1 = np.clip(np.rint(rng.normal(0, 20, size=(128, 64, 1, 1))), -127, 127).astype(np.int64)
+    w2 = np.clip(np.rint(rng.normal(0, 20, size=(64, 128, 3, 3))), -127, 127).astype(np.int64)
+    s1 = ActSpec("Rectifier", "FixedMult32", rng.integers(2 ** 28, 2 ** 30, size=128), frac_bits=37, nb_bits=8, unsigned_out=True)
+    s2 = ActSpec("Linear", "FixedMult32", rng.integers(2 ** 28, 2 ** 30, size=64), frac_bits=40, nb_bits=8, unsigned_out=False)
+    y1 = cells_ref.conv_cell(x, w1, None, s1)
+    y2 = cells_ref.conv_cell(y1, w2, None, s2, pad=(1, 1, 1, 1))
+    c1 = rt.Conv(w1, None, rt.Act(128, **s1.kwargs()), capi.U8B)
+    c2 = rt.Conv(w2, None, rt.Act(64, **s2.kwargs()), capi.U8B, pad=(1, 1, 1, 1))
+    assert c1.accepts_halo() and c2.accepts_halo() and len(np.unique(y2)) > 50
+    mid = c1.make_output(rt.DTensor.from_numpy(x, capi.U8B), halo=1)
+    c1.forward(rt.DTensor.from_numpy(x, capi.U8B), mid)
+    assert np.array_equal(mid.to_numpy(), y1.astype(np.int64)) and np.array_equal(c2.forward(mid).to_numpy(), y2.astype(np.int64))
     # cells that do not take a halo say so
     xh = rt.DTensor(1, 64, 4, 4, capi.U8B, halo=1)
     with pytest.raises(capi.N2D2HipError):
