@@ -637,16 +637,19 @@ bool ConvCell_Frame_HIP<T>::prepare()
     if (mDirty || activationGeneration() != mConvActGen || !mConv || inDType != mConvInDType) {
         clearFusion();
         if (mConv) { n2d2hip_conv_destroy(mConv); mConv = nullptr; }
-        const unsigned int cg = mNbChannels / mNbGroups;
+        const unsigned int cg = weightSlices();
         if (mWeights.dimX() != mKernelDims[0] || mWeights.dimY() != mKernelDims[1] || mWeights.dimZ() != cg || mWeights.dimB() != mNbOutputs)
             throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": weights must be {kW, kH, nbChannels/groups, nbOutputs}");
+        if (hasIrregularMapping() && mInputs.size() > 1)
+            throw std::runtime_error("ConvCell_Frame_HIP " + mName + ": an irregular connection map over several inputs is not supported");
         n2d2hip_conv_desc d = {};
         d.C = (int)mNbChannels; d.O = (int)mNbOutputs; d.kW = (int)mKernelDims[0]; d.kH = (int)mKernelDims[1];
         d.strideX = (int)mStrideDims[0]; d.strideY = (int)mStrideDims[1];
         d.padL = d.padR = mPaddingDims[0]; d.padT = d.padB = mPaddingDims[1];
         d.dilX = (int)mDilationDims[0]; d.dilY = (int)mDilationDims[1];
-        d.groups = (int)mNbGroups; d.weight_bits = mWeightBits;
-        const std::vector<unsigned char> w = packWeights(mWeights, mWeightBits, mName);
+        // an irregular map runs as a full connection whose missing connections weigh nothing
+        d.groups = hasIrregularMapping() ? 1 : (int)mNbGroups; d.weight_bits = mWeightBits;
+        const std::vector<unsigned char> w = packWeights(hasIrregularMapping() ? fullConnectionWeights() : mWeights, mWeightBits, mName);
         std::vector<std::int32_t> b;
         if (!mNoBias) {
             if (mBias.size() != mNbOutputs)
@@ -2322,9 +2325,10 @@ std::shared_ptr<DeepNet> generateFromINI(const std::string& iniText, std::string
 
 // Every output of block g = o / (O / G) must see exactly the channels [g L, (g + 1) L), L being the number of leading
 // channels the first output sees.
-std::size_t Cell::getNbGroups(const Tensor<bool>& map)
+std::size_t Cell::getNbGroups(const Tensor<bool>& map, bool* isRegular)
 {
     const std::size_t nbOutputs = map.dimX(), nbChannels = map.dimY();
+    if (isRegular) *isRegular = true;
     std::size_t width = 0;
     while (width < nbChannels && map.at(0, width))
         ++width;
@@ -2336,9 +2340,45 @@ std::size_t Cell::getNbGroups(const Tensor<bool>& map)
     for (std::size_t o = 0; regular && o < nbOutputs; ++o)
         for (std::size_t ch = 0; regular && ch < nbChannels; ++ch)
             regular = map.at(o, ch) == (ch / width == o / perGroup);
-    if (!regular)
-        throw std::runtime_error("Cell::getNbGroups(): the connection map is not a set of equal groups; Frame_HIP cells have no "
-                                 "connection-by-connection path");
+    if (regular)
+        return groups;
+    if (isRegular) *isRegular = false;
+    return getNbGroupsHandMade(map);
+}
+
+// Outputs that share a channel, directly or through other outputs, are one group: channels are merged into sets as the
+// outputs connect them, and every output names the set of its channels.
+std::size_t Cell::getNbGroupsHandMade(const Tensor<bool>& map)
+{
+    const std::size_t nbOutputs = map.dimX(), nbChannels = map.dimY();
+    std::vector<std::size_t> parent(nbChannels);
+    for (std::size_t ch = 0; ch < nbChannels; ++ch) parent[ch] = ch;
+    auto root = [&](std::size_t ch) {
+        while (parent[ch] != ch) { parent[ch] = parent[parent[ch]]; ch = parent[ch]; }
+        return ch;
+    };
+    const std::size_t none = nbChannels;
+    std::vector<std::size_t> firstChannel(nbOutputs, none);
+    bool connectedSeen = false;
+    for (std::size_t o = 0; o < nbOutputs; ++o) {
+        for (std::size_t ch = 0; ch < nbChannels; ++ch) {
+            if (!map.at(o, ch)) continue;
+            if (firstChannel[o] == none) firstChannel[o] = ch;
+            else parent[root(ch)] = root(firstChannel[o]);
+        }
+        if (firstChannel[o] != none)
+            connectedSeen = true;
+        else if (connectedSeen)
+            throw std::runtime_error("Cell::getNbGroupsHandMade(): an output without any connection behind a connected one "
+                                     "(the reference does not return on such a map)");
+    }
+    std::vector<bool> counted(nbChannels, false);
+    std::size_t groups = 0;
+    for (std::size_t o = 0; o < nbOutputs; ++o) {
+        if (firstChannel[o] == none) continue;
+        const std::size_t r = root(firstChannel[o]);
+        if (!counted[r]) { counted[r] = true; ++groups; }
+    }
     return groups;
 }
 
@@ -2346,10 +2386,33 @@ void ConvCell::setMapping(const Tensor<bool>& map)
 {
     if (map.dimX() != mNbOutputs || (mNbChannels != 0 && map.dimY() != mNbChannels))
         throw std::runtime_error("ConvCell::setMapping(): the map of " + mName + " must be {nbOutputs, nbChannels}");
-    const std::size_t groups = getNbGroups(map);
+    bool regular = true;
+    const std::size_t groups = getNbGroups(map, &regular);
     if (groups == 0)
         throw std::runtime_error("ConvCell::setMapping(): the first output of " + mName + " is not connected");
+    if (!regular && groups > 1 && map.dimY() % groups != 0)
+        throw std::runtime_error("ConvCell::setMapping(): the " + std::to_string(groups) + " groups of the map of " + mName
+                                 + " do not divide its channels");
     setNbGroups((unsigned int)groups);
+    if (!regular)
+        mIrregularMap = map;
+}
+
+Tensor<Float_T> ConvCell::fullConnectionWeights() const
+{
+    const std::size_t kw = mKernelDims[0], kh = mKernelDims[1], taps = kw * kh, slices = weightSlices();
+    Tensor<Float_T> full({kw, kh, (std::size_t)mNbChannels, (std::size_t)mNbOutputs}, Float_T(0));
+    for (std::size_t o = 0; o < mNbOutputs; ++o) {
+        const std::vector<std::size_t> from = connectedSlices(o);
+        std::size_t n = 0;
+        for (std::size_t ch = 0; ch < mNbChannels; ++ch) {
+            if (!mIrregularMap.at(o, ch)) continue;
+            for (std::size_t t = 0; t < taps; ++t)
+                full(t + taps * (ch + mNbChannels * o)) = mWeights(t + taps * (from[n] + slices * o));
+            ++n;
+        }
+    }
+    return full;
 }
 
 } // namespace N2D2

@@ -364,9 +364,13 @@ public:
     std::pair<double, double> getOutputsRangeParents() const;
     // Number of groups of a connection map {outputs, channels} (Cell::getNbGroups, src/Cell/Cell.cpp:251-300): G when the map
     // is G equal blocks on the diagonal (output o of block g sees exactly the channels of block g), 0 when the first output
-    // sees no leading channel.  Any other map is what the reference counts by hand (src/Cell/Cell.cpp:176-249) and its
-    // Frame cells then evaluate connection by connection; the Frame_HIP kernels have no such path and this throws.
-    static std::size_t getNbGroups(const Tensor<bool>& map);
+    // sees no leading channel.  Any other map is counted as the reference counts it by hand (getNbGroupsHandMade); `regular`,
+    // if given, tells which of the two it was.
+    static std::size_t getNbGroups(const Tensor<bool>& map, bool* regular = nullptr);
+    // Cell::getNbGroupsHandMade (src/Cell/Cell.cpp:178-249): the number of connected sets of outputs and channels, counted
+    // from the first output that has a connection; 0 for a map without any.  A later output without a connection, on
+    // which the reference's loop does not end, is refused.
+    static std::size_t getNbGroupsHandMade(const Tensor<bool>& map);
     const std::shared_ptr<Activation>& getActivation() const { return mActivation; }
     void setActivation(const std::shared_ptr<Activation>& activation) { mActivation = activation; }
     // Free parameters as text files, "<base>_weights<.ext>" and "<base>_biases<.ext>" (or one file holding both), the
@@ -489,9 +493,14 @@ public:
     const char* getType() const { return Type; }
     void setParameter(const std::string& name, bool value);
     // Depthwise / grouped connection: the regular mapping Cell::getNbGroups recognises (src/Cell/Cell.cpp:251-300).
-    void setNbGroups(unsigned int groups) { mNbGroups = groups; mDirty = true; }
-    // The same from the connection map itself, {nbOutputs, nbChannels} (what Mapping.* sections of an INI expand to)
+    void setNbGroups(unsigned int groups) { mNbGroups = groups; mIrregularMap = Tensor<bool>(); mDirty = true; }
+    // The same from the connection map itself, {nbOutputs, nbChannels} (what Mapping.* sections of an INI expand to).  A
+    // map that is not a set of equal groups is kept: the cell then convolves every output with its connected channels only
+    // (ConvCell_Frame_Kernels::forward skips the others, src/Cell/ConvCell_Frame_Kernels.cpp:93-96), and its weights are
+    // sized as the reference sizes them, {kW, kH, C / G, O} for G > 1 hand-counted groups (output o then uses slice n for its
+    // n-th connected channel, `:97`), {kW, kH, C, O} otherwise (src/Cell/ConvCell_Frame.cpp:172-177).
     void setMapping(const Tensor<bool>& map);
+    bool hasIrregularMapping() const { return !mIrregularMap.empty(); }
     // Weights as N2D2 holds them: float tensor {kW, kH, C/groups, O} with integer values; bias {O}.
     void setWeights(const Tensor<Float_T>& weights) { mWeights = weights; mDirty = true; }
     void setBiases(const Tensor<Float_T>& biases) { mBias = biases; mDirty = true; }
@@ -515,7 +524,13 @@ protected:
     unsigned int mNbGroups;
     int mWeightBits;
     Tensor<Float_T> mWeights, mBias;
+    Tensor<bool> mIrregularMap;             // {nbOutputs, nbChannels}; empty: every connection, or mNbGroups equal groups
     bool mDirty;
+    // Slices of the weights tensor per output (the third dimension the cell expects)
+    unsigned int weightSlices() const { return hasIrregularMapping() && mNbGroups <= 1 ? mNbChannels : mNbChannels / mNbGroups; }
+    // The weights of a cell with an irregular map as those of a full connection, {kW, kH, C, O}: zeros where there is none
+    Tensor<Float_T> fullConnectionWeights() const;
+    std::vector<std::size_t> connectedSlices(std::size_t output) const;
 };
 
 template <class T>

@@ -176,14 +176,16 @@ int fh_cell_set_weights(void* net, const char* name, const float* w, size_t n, i
 }
 
 // map[o + nbOutputs * c] != 0: output o sees channel c
-int fh_get_nb_groups(const unsigned char* map, size_t nbOutputs, size_t nbChannels, long* groups)
+int fh_get_nb_groups(const unsigned char* map, size_t nbOutputs, size_t nbChannels, long* groups, int* regular)
 {
     return guarded([&] {
         Tensor<bool> m({nbOutputs, nbChannels}, false);
         for (size_t c = 0; c < nbChannels; ++c)
             for (size_t o = 0; o < nbOutputs; ++o)
                 m.set(o, c, map[o + nbOutputs * c] != 0);
-        *groups = (long)Cell::getNbGroups(m);
+        bool isRegular = true;
+        *groups = (long)Cell::getNbGroups(m, &isRegular);
+        if (regular) *regular = isRegular ? 1 : 0;
     });
 }
 

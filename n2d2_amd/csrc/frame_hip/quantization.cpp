@@ -85,18 +85,19 @@ void ConvCell::importFreeParameters(const std::string& fileName, bool ignoreNotE
     if (!f.opened)
         return;
     std::istream& biases = f.biases(mNoBias);
-    const size_t cg = mNbChannels / mNbGroups;
+    const size_t cg = weightSlices();
     const size_t kernelSize = (size_t)mKernelDims[0] * mKernelDims[1];
-    Tensor<Float_T> w({mKernelDims[0], mKernelDims[1], cg, mNbOutputs});
+    Tensor<Float_T> w({mKernelDims[0], mKernelDims[1], cg, mNbOutputs}, Float_T(0));
     Tensor<Float_T> b({mNbOutputs});
     double value;
     for (size_t output = 0; output < mNbOutputs; ++output) {
-        // the channels of the output's group are its connections, in channel order
-        for (size_t channel = 0; channel < cg; ++channel) {
+        // the channels of the output's group are its connections, in channel order; with an irregular map the file holds
+        // the kernels of the connected channels only (`:559-561`), each stored in the slice the forward pass reads it from
+        for (size_t slice : connectedSlices(output)) {
             for (size_t index = 0; index < kernelSize; ++index) {
                 if (!(f.weights >> value))
                     throw std::runtime_error("Error while reading synaptic file: " + f.weightsFile);
-                w(index + kernelSize * (channel + cg * output)) = (Float_T)value;
+                w(index + kernelSize * (slice + cg * output)) = (Float_T)value;
             }
         }
         if (!mNoBias) {
@@ -114,6 +115,26 @@ void ConvCell::importFreeParameters(const std::string& fileName, bool ignoreNotE
     mDirty = true;
 }
 
+// The slices of the weights tensor that hold an output's kernels, in channel order: all of them, or with an irregular map
+// one per connected channel (src/Cell/ConvCell_Frame_Kernels.cpp:93-97)
+std::vector<std::size_t> ConvCell::connectedSlices(std::size_t output) const
+{
+    std::vector<std::size_t> slices;
+    if (!hasIrregularMapping()) {
+        for (std::size_t k = 0; k < weightSlices(); ++k) slices.push_back(k);
+        return slices;
+    }
+    for (std::size_t ch = 0; ch < mNbChannels; ++ch) {
+        if (!mIrregularMap.at(output, ch)) continue;
+        const std::size_t slice = mNbGroups > 1 ? slices.size() : ch;
+        if (slice >= weightSlices())
+            throw std::runtime_error("ConvCell " + mName + ": output " + std::to_string(output) + " is connected to more channels than "
+                                     "the weights have slices (the reference would read past them)");
+        slices.push_back(slice);
+    }
+    return slices;
+}
+
 void ConvCell::exportFreeParameters(const std::string& fileName) const
 {
     const std::string fileBase = fileBaseName(fileName);
@@ -124,10 +145,11 @@ void ConvCell::exportFreeParameters(const std::string& fileName) const
     std::ofstream weights(weightsFile.c_str());
     if (!weights.good())
         throw std::runtime_error("Could not create synaptic file: " + weightsFile);
-    const size_t perOutput = mWeights.size() / std::max<size_t>(mNbOutputs, 1);
+    const size_t kernelSize = (size_t)mKernelDims[0] * mKernelDims[1], cg = weightSlices();
     for (size_t output = 0; output < mNbOutputs; ++output) {
-        for (size_t i = 0; i < perOutput; ++i)
-            weights << std::setprecision(10) << mWeights(i + perOutput * output) << " ";
+        for (size_t slice : connectedSlices(output))
+            for (size_t i = 0; i < kernelSize; ++i)
+                weights << std::setprecision(10) << mWeights(i + kernelSize * (slice + cg * output)) << " ";
         weights << "\n";
     }
     if (!mNoBias) {

@@ -29,7 +29,7 @@ lib.fh_cell_set_weights.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size
 lib.fh_cell_set_biases.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
 lib.fh_net_save_quantization.argtypes = [C.c_void_p, C.c_char_p]
 lib.fh_net_load_quantization.argtypes = [C.c_void_p, C.c_char_p]
-lib.fh_get_nb_groups.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]
+lib.fh_get_nb_groups.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p]
 lib.fh_cell_set_mapping.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_size_t]
 lib.fh_cell_set_scaling.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p]
 lib.fh_cell_get_outputs.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
@@ -102,13 +102,13 @@ def approximate_scaling_with_power_of_2_divs(scaling, nb_divisions):
     return [int(e) for e in exps], precision.value
 
 
-def get_nb_groups(mapping):
-    """Cell::getNbGroups of a connection map [nbOutputs, nbChannels] (non-zero: connected).  Raises FrameHipError for a
-    map that is not a set of equal groups."""
+def get_nb_groups(mapping, with_regular=False):
+    """Cell::getNbGroups of a connection map [nbOutputs, nbChannels] (non-zero: connected): the number of equal groups, or
+    what the reference counts by hand for any other map (with_regular: also whether it was the former)."""
     m = np.asfortranarray(np.asarray(mapping) != 0, dtype=np.uint8)      # element (o, c) at o + nbOutputs * c
-    groups = C.c_long()
-    _check(lib.fh_get_nb_groups(m.ctypes.data, m.shape[0], m.shape[1], C.byref(groups)))
-    return groups.value
+    groups, regular = C.c_long(), C.c_int()
+    _check(lib.fh_get_nb_groups(m.ctypes.data, m.shape[0], m.shape[1], C.byref(groups), C.byref(regular)))
+    return (groups.value, bool(regular.value)) if with_regular else groups.value
 
 
 class Net:

@@ -44,9 +44,10 @@ class ActSpec:
         return y
 
 
-def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1):
+def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, maps=None):
     """x: one input, or a list of inputs: ConvCell_Frame<T>::propagate (src/Cell/ConvCell_Frame.cpp:438-459) then walks
-    them with its slice of the weights each, beta = 0 for the first and 1 afterwards."""
+    them with its slice of the weights each, beta = 0 for the first and 1 afterwards.  maps: a connection map, bool
+    [channels, outputs], instead of `groups` (one input)."""
     w = np.ascontiguousarray(w, dtype=np.float32)
     if isinstance(x, (list, tuple)) and len(x) > 1:
         if groups != 1:
@@ -60,8 +61,7 @@ def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), grou
         assert first == w.shape[1]
     else:
         x = np.ascontiguousarray(x[0] if isinstance(x, (list, tuple)) else x, dtype=np.float32)
-        maps = None
-        if groups > 1:
+        if maps is None and groups > 1:
             maps = orc.group_maps(x.shape[1], w.shape[0], groups)
         y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps)
     if bias is not None:
@@ -127,7 +127,8 @@ def run_net(spec, x, keep=None):
             a = l.act
             act = ActSpec(a.kind, a.mode, a.scaling, a.frac_bits, a.clipping, a.nb_bits, a.unsigned_out)
         if l.type == "conv":
-            y = conv_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups)
+            y = conv_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups,
+                          maps=getattr(l, "maps", None))
         elif l.type == "fc":
             y = fc_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act)
         elif l.type == "pool":

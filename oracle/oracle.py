@@ -65,6 +65,44 @@ def get_nb_groups(maps):
     return int(_lib.oracle_get_nb_groups(_p(m), C.c_size_t(nout), C.c_size_t(nch)))
 
 
+def get_nb_groups_hand_made(maps):
+    """Cell::getNbGroupsHandMade (src/Cell/Cell.cpp:178-249), walked the way the reference walks it: from the first output
+    that has a connection, take an unclassified output, collect every output reachable from it through shared channels
+    (`:213-236`), count one group, go on with the next unclassified output.  maps: bool [C, O].  0 for a map without any
+    connection (`:196-199`).  An output without connections behind the first connected one makes the reference's loop spin
+    (`:212-215`: `continue` without advancing): ValueError here."""
+    m = np.asarray(maps) != 0
+    nch, nout = m.shape
+    first = next((o for o in range(nout) if m[:, o].any()), None)
+    if first is None:
+        return 0
+    classified = set()
+    groups = 0
+    current = first
+    while current < nout:
+        if not m[:, current].any():
+            raise ValueError("output %d has no connection: the reference does not return on such a map" % current)
+        pending = [current]
+        while pending:
+            line = pending.pop()
+            classified.add(line)
+            for ch in np.flatnonzero(m[:, line]):
+                for o in range(first, nout):
+                    if m[ch, o] and o not in classified and o not in pending:
+                        pending.append(o)
+        groups += 1
+        current += 1
+        while current in classified:
+            current += 1
+    return groups
+
+
+def nb_groups_of(maps):
+    """Cell::getNbGroups (src/Cell/Cell.cpp:251-300) with its fall-back: the regular count, else the hand-made one."""
+    g = get_nb_groups(maps)
+    return g if g >= 0 else get_nb_groups_hand_made(maps)
+
+
 def group_maps(C_in, O, groups):
     """Boolean mapping [C, O] of a regular grouped connection."""
     m = np.zeros((C_in, O), dtype=np.uint8)
@@ -91,9 +129,14 @@ def conv_forward(x, w, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), maps=None,
     m = None
     if maps is not None:
         m = np.ascontiguousarray(maps, dtype=np.uint8)
-        groups = get_nb_groups(m)
-        if groups < 0:
-            raise ValueError("irregular mapping")
+        groups = nb_groups_of(m)
+        # the weights have C / G slices with several groups, C otherwise (src/Cell/ConvCell_Frame.cpp:172-177); output o reads
+        # slice n for its n-th connected channel with several groups (src/Cell/ConvCell_Frame_Kernels.cpp:97).  The reference
+        # does not check that this stays inside the tensor; the restatement refuses to read past it.
+        if Cw != (Cin // groups if groups > 1 else Cin):
+            raise ValueError("weights have %d slices, the map's %d group(s) ask for %d" % (Cw, groups, Cin // groups if groups > 1 else Cin))
+        if groups > 1 and int(m.sum(axis=0).max()) > Cw:
+            raise ValueError("an output is connected to more channels than the weights have slices")
     ct = _CT[np.dtype(dt)]
     a, b = ct(alpha), ct(beta)
     _fn("conv_forward", dt)(C.byref(a), _p(x), B, Cin, H, W, _p(w), kW, kH, Cw, O,

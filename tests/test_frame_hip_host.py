@@ -300,8 +300,9 @@ def test_replace_input_rewires_a_cell_as_cell_frame_does(fh):
 
 def test_get_nb_groups_from_a_connection_map_against_the_oracle(fh):
     """Cell::getNbGroups (src/Cell/Cell.cpp:251-300) in the cell layer: equal diagonal blocks give their count, an
-    unconnected first output gives 0, and every map the reference would count by hand is an error; the oracle's
-    restatement of the same function says -1 exactly there."""
+    unconnected first output gives 0, and every other map is counted by hand (getNbGroupsHandMade, `:178-249`), as the
+    oracle's restatements of the two functions say; a map on which the reference's hand count does not return is refused by
+    both."""
     import numpy as np
     from oracle import oracle as orc
     rng = np.random.default_rng(5)
@@ -312,38 +313,37 @@ def test_get_nb_groups_from_a_connection_map_against_the_oracle(fh):
             m[g * (O // G):(g + 1) * (O // G), g * (Cn // G):(g + 1) * (Cn // G)] = 1
         return m
 
+    def same_as_oracle(m):          # m: [outputs, channels]; the oracle takes [channels, outputs]
+        want = orc.get_nb_groups(m.T)
+        if want >= 0:
+            assert fh.get_nb_groups(m, with_regular=True) == (want, True)
+            return
+        try:
+            by_hand = orc.get_nb_groups_hand_made(m.T)
+        except ValueError:
+            with pytest.raises(fh.FrameHipError, match="does not return"):
+                fh.get_nb_groups(m)
+            return
+        assert fh.get_nb_groups(m, with_regular=True) == (by_hand, False)
+
     for (O, Cn, G) in ((8, 8, 8), (12, 6, 3), (6, 12, 2), (5, 7, 1), (64, 64, 64), (16, 4, 4), (4, 16, 4)):
         m = block_map(O, Cn, G)
-        assert fh.get_nb_groups(m) == G == orc.get_nb_groups(m)
+        assert fh.get_nb_groups(m) == G == orc.get_nb_groups(m.T)
         # any single flipped connection makes it irregular (or moves the first run, which must break a later row)
         for _ in range(6):
             o, c = int(rng.integers(0, O)), int(rng.integers(0, Cn))
             bad = m.copy()
             bad[o, c] ^= 1
-            want = orc.get_nb_groups(bad)
-            if want == -1:
-                with pytest.raises(fh.FrameHipError, match="not a set of equal groups"):
-                    fh.get_nb_groups(bad)
-            else:
-                assert fh.get_nb_groups(bad) == want
-    # random maps: whatever the oracle says, the cell layer says (error for -1)
-    for _ in range(200):
-        O, Cn = int(rng.integers(1, 7)), int(rng.integers(1, 7))
-        m = (rng.random((O, Cn)) < 0.6).astype(np.uint8)
-        want = orc.get_nb_groups(m)
-        if want == -1:
-            with pytest.raises(fh.FrameHipError):
-                fh.get_nb_groups(m)
-        else:
-            assert fh.get_nb_groups(m) == want
+            same_as_oracle(bad)
+    for _ in range(300):
+        O, Cn = int(rng.integers(1, 9)), int(rng.integers(1, 9))
+        same_as_oracle((rng.random((O, Cn)) < rng.uniform(0.2, 0.8)).astype(np.uint8))
     assert fh.get_nb_groups(np.zeros((4, 6), dtype=np.uint8)) == 0
-    # unequal blocks: the reference's hand count would say 2, its regular test fails, ours raises
+    # unequal blocks: the regular test fails, the hand count says 2
     uneven = np.zeros((4, 4), dtype=np.uint8)
     uneven[0:1, 0:1] = 1
     uneven[1:4, 1:4] = 1
-    assert orc.get_nb_groups(uneven) == -1
-    with pytest.raises(fh.FrameHipError):
-        fh.get_nb_groups(uneven)
+    assert orc.get_nb_groups(uneven.T) == -1 and fh.get_nb_groups(uneven, with_regular=True) == (2, False)
 
 
 def test_conv_mapping_sets_the_groups(fh):
@@ -351,8 +351,13 @@ def test_conv_mapping_sets_the_groups(fh):
     net = fh.Net((INI % "Frame_HIP"))
     info = net.cell_info("conv1")
     O, Cn = 16, 3
-    with pytest.raises(fh.FrameHipError, match="not a set of equal groups"):
-        net.set_mapping("conv1", np.tri(O, Cn))
+    net.set_mapping("conv1", np.tri(O, Cn))             # not a set of equal groups: kept, the cell skips the missing connections
+    hole = np.tri(O, Cn)
+    hole[5, :] = 0
+    with pytest.raises(fh.FrameHipError, match="does not return"):      # (the reference's hand count spins on such a map)
+        net.set_mapping("conv1", hole)
+    with pytest.raises(fh.FrameHipError, match="is not connected"):
+        net.set_mapping("conv1", np.tri(O, Cn)[::-1].copy() * 0 + np.eye(O, Cn, k=-1))
     with pytest.raises(fh.FrameHipError, match="must be"):
         net.set_mapping("conv1", np.ones((O + 1, Cn)))
     net.set_mapping("conv1", np.ones((O, Cn)))          # fully connected: one group

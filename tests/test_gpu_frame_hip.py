@@ -249,6 +249,66 @@ def test_grouped_convolution_cells(fh):
         assert np.array_equal(net.outputs(name), want[name]), name
 
 
+def test_convolution_cells_with_irregular_connection_maps(fh, tmp_path):
+    """ConvCells whose connection map is not a set of equal groups (what the reference evaluates connection by connection):
+    overlapping connections (one hand-counted group: weights {kW, kH, C, O}, indexed by channel) and two unequal groups
+    (weights {kW, kH, C / 2, O}, indexed by the count of connected channels), every output against the oracle; the cell's
+    parameters survive a trip through N2D2's text files, which hold the connected kernels only."""
+    from n2d2_amd import nets
+    from oracle import cells
+    rng = np.random.default_rng(61)
+    b = nets._Builder("irregular", (8, 12, 12), 61, "SingleShift")
+    t = b.conv("overlap", "input", 64, 3, pad=1)
+    t = b.conv("unequal", t, 12, 3, stride=2, pad=1, groups=2)
+    b.fc("fc", t, 10, mode="None")
+    spec = b.spec
+    m1 = (rng.random((8, 64)) < 0.5).astype(np.uint8)          # [channels, outputs]
+    m1[0, :] = 1
+    m1[1, 0] = 0
+    m1[2, 0] = 1
+    m2 = np.zeros((64, 12), dtype=np.uint8)
+    m2[0:32, 0:4] = 1
+    m2[32:64, 4:12] = 1
+    m2[40, 5] = 0
+    spec.layers[0].maps, spec.layers[1].maps = m1, m2
+    x = rng.integers(0, 256, size=(3, 8, 12, 12))
+    keep = [l.name for l in spec.layers]
+    want = cells.run_net(spec, x, keep=keep)
+    assert len(np.unique(want["unequal"])) > 20
+
+    def check(net):
+        net.initialize()
+        net.set_stimuli(x)
+        net.propagate()
+        for name in keep:
+            assert np.array_equal(net.outputs(name), want[name]), name
+    net = fh.build_net(spec, 3)
+    net.set_mapping("overlap", m1.T)
+    net.set_mapping("unequal", m2.T)
+    check(net)
+    # through the text files: one line per output holding the kernels of its connected channels
+    for l in spec.layers[:2]:
+        net.export_free_parameters(l.name, tmp_path / (l.name + ".syntxt"))
+    line = open(tmp_path / "unequal_weights.syntxt").read().split("\n")[5].split()
+    assert len(line) == 31 * 9                       # output 5 misses one of its group's 32 channels
+    second = fh.build_net(spec, 3)
+    second.set_mapping("overlap", m1.T)
+    second.set_mapping("unequal", m2.T)
+    for l in spec.layers[:2]:
+        second.set_weights(l.name, np.zeros_like(l.w, dtype=np.float32))
+        second.import_free_parameters(l.name, tmp_path / (l.name + ".syntxt"))
+    check(second)
+    # a map that ties the two groups together asks for weights over every channel: the cell's {.., C / 2, O} are refused
+    bad = m2.copy()
+    bad[32, 0] = 1
+    third = fh.build_net(spec, 3)
+    third.set_mapping("unequal", bad.T)
+    third.initialize()
+    third.set_stimuli(x)
+    with pytest.raises(fh.FrameHipError):
+        third.propagate()
+
+
 MINI_MOBILENET_INI = """
 $BATCH=6
 $WIDTH=8

@@ -150,6 +150,77 @@ def test_nb_groups_irregular_mapping_is_flagged():
     assert orc.get_nb_groups(np.zeros((4, 6), dtype=np.uint8)) == 0
 
 
+def test_hand_made_group_count_is_the_number_of_connected_sets():
+    """Cell::getNbGroupsHandMade (src/Cell/Cell.cpp:178-249) counts the sets of outputs tied together by shared channels: known
+    small maps, then random ones against scipy's connected components of the bipartite graph (an independent algorithm)."""
+    from scipy.sparse import csr_matrix
+    from scipy.sparse.csgraph import connected_components
+    m = np.zeros((8, 6), dtype=np.uint8)            # [channels, outputs]
+    m[0:4, 0:2] = 1
+    m[4:8, 2:6] = 1                                  # two unequal blocks: not "regular", two groups by hand
+    assert orc.get_nb_groups(m) == -1 and orc.get_nb_groups_hand_made(m) == 2 and orc.nb_groups_of(m) == 2
+    m[3, 5] = 1                                      # one shared channel ties them together
+    assert orc.get_nb_groups_hand_made(m) == 1
+    chain = np.zeros((5, 4), dtype=np.uint8)         # 0-1 share channel 1, 1-2 share channel 2, 3 on its own
+    chain[0, 0] = chain[1, 0] = chain[1, 1] = chain[2, 1] = chain[2, 2] = chain[4, 3] = 1
+    assert orc.get_nb_groups_hand_made(chain) == 2
+    assert orc.get_nb_groups_hand_made(np.zeros((3, 3), dtype=np.uint8)) == 0
+    lead = np.zeros((4, 4), dtype=np.uint8)          # outputs without a connection in front of the first connected one are skipped
+    lead[0, 2] = lead[1, 3] = 1
+    assert orc.get_nb_groups_hand_made(lead) == 2
+    hole = lead.copy()
+    hole[:, 3] = 0                                   # ... behind it: the reference's loop does not end
+    with pytest.raises(ValueError):
+        orc.get_nb_groups_hand_made(hole)
+    rng = np.random.default_rng(77)
+    for _ in range(60):
+        nch, nout = rng.integers(2, 12), rng.integers(2, 12)
+        m = (rng.random((nch, nout)) < rng.uniform(0.1, 0.5)).astype(np.uint8)
+        for o in range(nout):                        # every output connected somewhere
+            if not m[:, o].any():
+                m[rng.integers(nch), o] = 1
+        graph = np.zeros((nch + nout, nch + nout), dtype=np.uint8)
+        graph[:nch, nch:] = m
+        _, labels = connected_components(csr_matrix(graph), directed=False)
+        assert orc.get_nb_groups_hand_made(m) == len(set(labels[nch:])), m
+
+
+def test_conv_with_an_irregular_connection_map():
+    """ConvCell_Frame_Kernels::forward under a map that is not a set of equal groups (src/Cell/ConvCell_Frame_Kernels.cpp:93-97):
+    unconnected channels are skipped; with one hand-counted group the weights are indexed by channel, with several by the
+    count of connected channels so far.  Against the plain convolution of weights scattered into a full tensor."""
+    rng = np.random.default_rng(78)
+    x = _u8((2, 8, 7, 9))
+    # one group: overlapping connections
+    m = (rng.random((8, 6)) < 0.5).astype(np.uint8)
+    m[0, :] = 1
+    m[1, 0] = 0                                      # (the first output does not see a leading block that divides the channels)
+    m[2, 0] = 1
+    assert orc.get_nb_groups(m) == -1 and orc.nb_groups_of(m) == 1
+    w = _i8((6, 8, 3, 3))
+    got = orc.conv_forward(x, w, pad=(1, 1, 1, 1), maps=m)
+    want = rm.conv_int(x, w * m.T[:, :, None, None], pad=(1, 1))
+    assert np.array_equal(got.astype(np.int64), want)
+    # two unequal groups: packed slices
+    m = np.zeros((8, 6), dtype=np.uint8)
+    m[0:4, 0:2] = 1
+    m[4:8, 2:6] = 1
+    m[5, 3] = 0                                      # (an output may use fewer slices than there are)
+    w = _i8((6, 4, 3, 3))
+    full = np.zeros((6, 8, 3, 3), dtype=w.dtype)
+    for o in range(6):
+        for n, ch in enumerate(np.flatnonzero(m[:, o])):
+            full[o, ch] = w[o, n]
+    got = orc.conv_forward(x, w, stride=(2, 1), pad=(1, 1, 1, 1), maps=m)
+    assert np.array_equal(got.astype(np.int64), rm.conv_int(x, full, stride=(2, 1), pad=(1, 1)))
+    with pytest.raises(ValueError):                  # more connections than slices: the reference would read past its weights
+        m2 = np.zeros((8, 6), dtype=np.uint8)
+        m2[0:5, 0:2] = 1                             # two groups still (8 / 2 = 4 slices), five connections for outputs 0 and 1
+        m2[5:8, 2:6] = 1
+        assert orc.nb_groups_of(m2) == 2
+        orc.conv_forward(x, w, pad=(1, 1, 1, 1), maps=m2)
+
+
 def test_conv_identity_kernel_copies_input():
     x = _u8((2, 3, 7, 6))
     w = np.zeros((3, 3, 3, 3), dtype=np.float32)
