@@ -174,6 +174,11 @@ typedef struct n2d2hip_conv_desc {
                                kernel); read from the descriptor when the cell is created (integer cells) or on each call
                                (float passes: give the same value to n2d2hip_conv2d_f32_workspace_bytes and to the pass).
                                No counterpart in the reference. */
+    int subX, subY;         /* Descriptor::subSample (ref: src/Cell/ConvCell_Frame_Kernels.cpp:46-52,135-140): the sums of
+                               subX x subY neighbouring positions are added up into one output (the last window of a row
+                               or column may hold fewer), the bias is added once and the activation applied to that;
+                               0 or 1: none.  Integer cells only; such a cell runs as the convolution proper plus one
+                               launch that adds the windows up, and takes part in no graph-level fusion */
 } n2d2hip_conv_desc;
 enum {
     N2D2HIP_KERNEL_NO_PIPE = 1,     /* integer cells: general register-staged kernel instead of the pipelined one */
@@ -202,7 +207,7 @@ typedef struct n2d2hip_conv_s* n2d2hip_conv_t;
 int n2d2hip_conv_create(const n2d2hip_conv_desc* desc, const void* weights, const int32_t* bias,
                         n2d2hip_act_t act, int in_dtype, n2d2hip_conv_t* conv);
 int n2d2hip_conv_destroy(n2d2hip_conv_t conv);
-/* Output spatial size (ref: src/Cell/ConvCell.cpp:1169-1195). */
+/* Output spatial size (ref: src/Cell/ConvCell.cpp:1169-1195), sub-sampling included. */
 int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* desc, int H, int W, int* outH, int* outW);
 /* in / out: NHWC with the channel stride of n2d2hip_nhwc_cs (4 for at most 4 channels, a multiple of 16 otherwise).  out dtype U8B/U8/I8 (rescaled) or I32 (scaling NONE).  `in` and a byte `out`
  * may have a halo if n2d2hip_conv_accepts_halo says so. */

@@ -60,7 +60,7 @@ class Activation(C.Structure):
 class ConvDesc(C.Structure):
     _fields_ = [("C", C.c_int), ("O", C.c_int), ("kW", C.c_int), ("kH", C.c_int), ("strideX", C.c_int), ("strideY", C.c_int),
                 ("padL", C.c_int), ("padT", C.c_int), ("padR", C.c_int), ("padB", C.c_int), ("dilX", C.c_int), ("dilY", C.c_int),
-                ("groups", C.c_int), ("weight_bits", C.c_int), ("kernel_choice", C.c_int)]
+                ("groups", C.c_int), ("weight_bits", C.c_int), ("kernel_choice", C.c_int), ("subX", C.c_int), ("subY", C.c_int)]
 
 
 class PoolDesc(C.Structure):

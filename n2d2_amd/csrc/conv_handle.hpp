@@ -48,5 +48,13 @@ struct n2d2hip_conv_s {
     signed char* d_wsmall;
     bool is_fc;
     int fcH, fcW;
+    // sub-sampling (desc.subX or subY > 1): the convolution proper is a handle of its own that stores raw sums without a
+    // bias; one more launch adds them up per window, adds the bias and applies the cell's activation.  The other fields
+    // above stay empty on such a handle.
+    n2d2hip_conv_s* sub_inner;
+    n2d2hip_act_t sub_raw_act;
+    int* d_sub_bias;            // [O] or null
+    int* d_sub_sums;            // raw sums of the last forward (grown on demand, kept until the handle goes)
+    size_t sub_sums_bytes;
 };
 

@@ -476,6 +476,108 @@ int n2d2hip_conv_out_dims(const n2d2hip_conv_desc* d, int H, int W, int* outH, i
     *outW = conv_out_dim(W, d->kW, d->strideX, d->padL, d->padR, d->dilX);
     *outH = conv_out_dim(H, d->kH, d->strideY, d->padT, d->padB, d->dilY);
     N2D2HIP_REQUIRE(*outW > 0 && *outH > 0, N2D2HIP_ERR_INVALID, "conv_out_dims: empty output %dx%d", *outW, *outH);
+    N2D2HIP_REQUIRE(d->subX >= 0 && d->subY >= 0, N2D2HIP_ERR_INVALID, "conv_out_dims: negative sub-sampling");
+    // ceil(positions / subSample): the last window may hold fewer positions
+    *outW = (*outW + std::max(d->subX, 1) - 1) / std::max(d->subX, 1);
+    *outH = (*outH + std::max(d->subY, 1) - 1) / std::max(d->subY, 1);
+    return N2D2HIP_OK;
+}
+
+// Sub-sampling: out(b, oy, ox, ch) = act(sum of the raw sums at positions (oy subY + j, ox subX + i) inside the tensor + bias)
+// (ref: src/Cell/ConvCell_Frame_Kernels.cpp:135-140, then forwardBias `:151-174` and the activation).  One thread per output.
+__global__ __launch_bounds__(256) void conv_subsample_kernel(const int* __restrict__ sums, int H, int W, int cs, int B, int OH, int OW, int O,
+                                                             int subX, int subY, const int* __restrict__ bias, const EpiArgs epi, void* out,
+                                                             int out_cs, int out_dtype)
+{
+    const long long total = (long long)B * OH * OW * O;
+    for (long long i = blockIdx.x * 256ll + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
+        const int ch = (int)(i % O);
+        long long p = i / O;
+        const int ox = (int)(p % OW);
+        p /= OW;
+        const int oy = (int)(p % OH);
+        const int b = (int)(p / OH);
+        int v = bias ? bias[ch] : 0;
+        for (int y = oy * subY; y < min((oy + 1) * subY, H); ++y)
+            for (int x = ox * subX; x < min((ox + 1) * subX, W); ++x)
+                v += sums[(((size_t)b * H + y) * W + x) * cs + ch];
+        store_value(out, (((size_t)b * OH + oy) * OW + ox) * out_cs + ch, out_dtype, epi_apply_dyn(epi, v, ch));
+    }
+}
+
+static bool sub_sampled(const n2d2hip_conv_s* c) { return c && c->sub_inner != nullptr; }
+
+static int conv_subsample_create(const n2d2hip_conv_desc* d, const void* weights, const int32_t* bias, n2d2hip_act_t act, int in_dtype,
+                                 n2d2hip_conv_t* conv)
+{
+    n2d2hip_conv_s* c = new n2d2hip_conv_s();
+    c->desc = *d;
+    c->act = act;
+    c->in_dtype = in_dtype;
+    c->in_cs = n2d2hip_nhwc_cs(d->C);
+    c->sum_other_dtype = -1;
+    n2d2hip_activation raw = {};
+    raw.kind = N2D2HIP_ACT_LINEAR;
+    raw.scaling_mode = N2D2HIP_SCALING_NONE;
+    int rc = n2d2hip_act_create(&raw, d->O, &c->sub_raw_act);
+    n2d2hip_conv_desc inner = *d;
+    inner.subX = inner.subY = 1;
+    if (rc == N2D2HIP_OK)
+        rc = n2d2hip_conv_create(&inner, weights, nullptr, c->sub_raw_act, in_dtype, &c->sub_inner);
+    if (rc == N2D2HIP_OK && bias) {
+        hipError_t e = hipMalloc((void**)&c->d_sub_bias, (size_t)d->O * sizeof(int));
+        if (e == hipSuccess) e = hipMemcpy(c->d_sub_bias, bias, (size_t)d->O * sizeof(int), hipMemcpyHostToDevice);
+        if (e != hipSuccess) rc = fail(N2D2HIP_ERR_HIP, "conv_create: copying the bias failed: %s", hipGetErrorString(e));
+    }
+    if (rc != N2D2HIP_OK) {
+        n2d2hip_conv_destroy(c);
+        return rc;
+    }
+    *conv = c;
+    return N2D2HIP_OK;
+}
+
+static int conv_subsample_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
+{
+    int rc, H, W, OH, OW;
+    if ((rc = check_tensor(in, "conv input", true)) || (rc = check_tensor(out, "conv output")))
+        return rc;
+    const n2d2hip_conv_desc& d = c->desc;
+    if ((rc = n2d2hip_conv_out_dims(&c->sub_inner->desc, in->H, in->W, &H, &W)) || (rc = n2d2hip_conv_out_dims(&d, in->H, in->W, &OH, &OW)))
+        return rc;
+    N2D2HIP_REQUIRE(out->layout == N2D2HIP_NHWC && out->B == in->B && out->C == d.O && out->H == OH && out->W == OW && out->halo == 0,
+                    N2D2HIP_ERR_INVALID, "conv_forward: sub-sampled output is %dx%dx%dx%d, expected %dx%dx%dx%d without a halo", out->B, out->C,
+                    out->H, out->W, in->B, d.O, OH, OW);
+    const n2d2hip_act_s* act = c->act;
+    if (act->args.kind == EPI_RAW) {
+        N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_INVALID, "conv_forward: without a rescale the cell outputs raw sums; the output dtype must be I32");
+    } else if (is_byte_type(out->dtype)) {
+        const int lo = out->dtype == N2D2HIP_I8 ? -128 : 0, hi = out->dtype == N2D2HIP_I8 ? 127 : 255;
+        N2D2HIP_REQUIRE(act->min_out >= lo && act->max_out <= hi, N2D2HIP_ERR_INVALID,
+                        "conv_forward: activation range [%d,%d] does not fit output dtype %d", act->min_out, act->max_out, out->dtype);
+    } else {
+        N2D2HIP_REQUIRE(out->dtype == N2D2HIP_I32, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: F32 outputs are produced with n2d2hip_convert");
+    }
+    n2d2hip_tensor sums = {};
+    sums.dtype = N2D2HIP_I32; sums.layout = N2D2HIP_NHWC; sums.B = in->B; sums.C = d.O; sums.H = H; sums.W = W;
+    sums.cs = n2d2hip_nhwc_cs(d.O); sums.halo = 0;
+    const size_t need = n2d2hip_tensor_bytes(&sums);
+    if (need > c->sub_sums_bytes) {
+        // (the first forward, or a larger input than before: not a call for a caller that cannot allocate)
+        N2D2HIP_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream));
+        if (c->d_sub_sums) (void)hipFree(c->d_sub_sums);
+        c->d_sub_sums = nullptr; c->sub_sums_bytes = 0;
+        N2D2HIP_HIP_CHECK(hipMalloc((void**)&c->d_sub_sums, need));
+        c->sub_sums_bytes = need;
+    }
+    sums.data = c->d_sub_sums;
+    if ((rc = n2d2hip_conv_forward(c->sub_inner, in, &sums, stream)))
+        return rc;
+    const long long total = (long long)in->B * OH * OW * d.O;
+    const unsigned grid = (unsigned)std::max<long long>(1, std::min<long long>((total + 255) / 256, 256 * 32));
+    N2D2HIP_LAUNCH(conv_subsample_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const int*)c->d_sub_sums, H, W, sums.cs, in->B, OH, OW,
+                   d.O, std::max(d.subX, 1), std::max(d.subY, 1), (const int*)c->d_sub_bias, act->args, out->data, out->cs, out->dtype);
+    N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
 }
 
@@ -493,6 +595,9 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
     N2D2HIP_REQUIRE(act->nb_channels == d->O, N2D2HIP_ERR_INVALID, "conv_create: activation built for %d channels, conv has %d outputs",
                     act->nb_channels, d->O);
     N2D2HIP_REQUIRE(d->groups >= 1, N2D2HIP_ERR_UNSUPPORTED, "conv_create: irregular mapping (nbGroups = %d)", d->groups);
+    N2D2HIP_REQUIRE(d->subX >= 0 && d->subY >= 0, N2D2HIP_ERR_INVALID, "conv_create: negative sub-sampling");
+    if (d->subX > 1 || d->subY > 1)
+        return conv_subsample_create(d, weights, bias, act, in_dtype, conv);
     const bool depthwise = d->groups > 1 && d->groups == d->C && d->C == d->O;
     if (d->groups > 1 && !depthwise) {
         // G equal groups, output o of group o / (O/G) connected to channels [g C/G, (g+1) C/G) with its weights indexed by
@@ -767,6 +872,10 @@ int n2d2hip_conv_create(const n2d2hip_conv_desc* d, const void* weights, const i
 int n2d2hip_conv_destroy(n2d2hip_conv_t c)
 {
     if (!c) return N2D2HIP_OK;
+    if (c->sub_inner) n2d2hip_conv_destroy(c->sub_inner);
+    if (c->sub_raw_act) n2d2hip_act_destroy(c->sub_raw_act);
+    if (c->d_sub_bias) (void)hipFree(c->d_sub_bias);
+    if (c->d_sub_sums) (void)hipFree(c->d_sub_sums);
     if (c->d_w) (void)hipFree(c->d_w);
     if (c->d_sub) (void)hipFree(c->d_sub);
     if (c->d_bias) (void)hipFree(c->d_bias);
@@ -799,7 +908,7 @@ static bool pipe_eligible(const n2d2hip_conv_s* c, bool* bn128)
     const int opad_n = round_up(d.O, 64);
     *bn128 = opad_n % 128 == 0 || opad_n > 256;
     const int k = c->act->args.kind;
-    if (!pipe_shape(d))
+    if (!pipe_shape(d) || c->sub_inner)     // (a sub-sampled cell's own handle launches nothing but the window sums)
         return false;
     if (d.weight_bits == 4)     // packed weights: integer rescale only
         return c->d_w4img != nullptr && k == EPI_I24 && c->bias_folded;
@@ -1202,6 +1311,10 @@ static int conv_forward_impl(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n
 
 int n2d2hip_conv_forward(n2d2hip_conv_t c, const n2d2hip_tensor* in, const n2d2hip_tensor* out, n2d2hip_stream_t stream)
 {
+    if (sub_sampled(c)) {
+        N2D2HIP_REQUIRE(in && in->halo == 0, N2D2HIP_ERR_UNSUPPORTED, "conv_forward: a sub-sampled convolution takes its input without a halo");
+        return conv_subsample_forward(c, in, out, stream);
+    }
     return conv_forward_impl(c, in, nullptr, out, stream);
 }
 

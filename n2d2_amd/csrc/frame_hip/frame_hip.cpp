@@ -515,8 +515,8 @@ ConvCell::ConvCell(const std::vector<unsigned int>& kernelDims, const std::vecto
     if (mStrideDims.empty()) mStrideDims.assign(2, 1U);
     if (mPaddingDims.empty()) mPaddingDims.assign(2, 0);
     if (mDilationDims.empty()) mDilationDims.assign(2, 1U);
-    if (mSubSampleDims[0] != 1 || mSubSampleDims[1] != 1)
-        throw std::runtime_error("ConvCell: sub-sampling is not supported by Frame_HIP");
+    if (mSubSampleDims.size() != 2 || mSubSampleDims[0] < 1 || mSubSampleDims[1] < 1)
+        throw std::runtime_error("ConvCell: SubSampleDims must be two positive values");
 }
 
 void ConvCell::setParameter(const std::string& name, bool value)
@@ -649,6 +649,7 @@ bool ConvCell_Frame_HIP<T>::prepare()
         d.dilX = (int)mDilationDims[0]; d.dilY = (int)mDilationDims[1];
         // an irregular map runs as a full connection whose missing connections weigh nothing
         d.groups = hasIrregularMapping() ? 1 : (int)mNbGroups; d.weight_bits = mWeightBits;
+        d.subX = (int)mSubSampleDims[0]; d.subY = (int)mSubSampleDims[1];
         const std::vector<unsigned char> w = packWeights(hasIrregularMapping() ? fullConnectionWeights() : mWeights, mWeightBits, mName);
         std::vector<std::int32_t> b;
         if (!mNoBias) {

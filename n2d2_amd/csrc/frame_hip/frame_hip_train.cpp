@@ -277,6 +277,8 @@ ConvCell_FrameTrain_HIP<T>::ConvCell_FrameTrain_HIP(const DeepNet& /*deepNet*/, 
                                                     const std::vector<unsigned int>& dilationDims, const std::shared_ptr<Activation>& activation)
     : Cell(name, nbOutputs), ConvCell(kernelDims, subSampleDims, strideDims, paddingDims, dilationDims)
 {
+    if (mSubSampleDims[0] != 1 || mSubSampleDims[1] != 1)
+        throw std::runtime_error("ConvCell: sub-sampling is not supported by the learning cells of Frame_HIP_QAT");
     mActivation = activation;
 }
 

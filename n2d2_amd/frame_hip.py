@@ -331,6 +331,8 @@ def spec_to_ini(spec, batch, model="Frame_HIP"):
                       "NoBias=%d" % (l.bias is None)]
             if l.groups > 1:
                 lines.append("Mapping.NbGroups=%d" % l.groups)
+            if tuple(getattr(l, "sub", (1, 1))) != (1, 1):
+                lines.append("SubSampleDims=%d %d" % tuple(l.sub))
         elif l.type == "fc":
             lines += ["Type=Fc", "NbOutputs=%d" % l.w.shape[0], "ActivationFunction=%s" % l.act.kind]
         elif l.type == "pool":

@@ -197,12 +197,19 @@ class _Builder:
         return np.clip(np.rint(self.rng.normal(0, wstd, size=shape)), -wmax, wmax).astype(np.int8)
 
     def conv(self, name, inp, O, k, stride=1, pad=0, kind="Rectifier", groups=1, wstd=30.0, wmax=127, weight_bits=8,
-             bias=True, nb_bits=None, mode=None, clip=False, uniform=False):
+             bias=True, nb_bits=None, mode=None, clip=False, uniform=False, sub=(1, 1)):
         inps = list(inp) if isinstance(inp, (list, tuple)) else [inp]     # several inputs: their channels one behind the other
         C, (H, W) = sum(self.spec.shapes[i][0] for i in inps), self.spec.shapes[inps[0]][1:]
         w = self._weights((O, C // groups, k, k), wstd, wmax, uniform)
         p4 = (pad, pad, pad, pad)
         acc = _conv_acc_np(np.concatenate([self.values[i] for i in inps], 0), w.astype(np.int64), (stride, stride), p4, groups)
+        if tuple(sub) != (1, 1):
+            # ConvCell's SubSample: the sums of sub[0] x sub[1] neighbouring positions added up, ragged last windows included
+            summed = np.zeros((O, -(-acc.shape[1] // sub[1]), -(-acc.shape[2] // sub[0])), dtype=np.int64)
+            for oy in range(acc.shape[1]):
+                for ox in range(acc.shape[2]):
+                    summed[:, oy // sub[1], ox // sub[0]] += acc[:, oy, ox]
+            acc = summed
         b = None
         if bias:
             mag = max(int(np.percentile(np.abs(acc), 90) / 4), 16)
@@ -211,7 +218,7 @@ class _Builder:
         act = self._make_act(acc, kind, O, nb_bits, mode, clip)
         self.values[name] = act.apply_np(acc, 0)
         l = Layer(name, "conv", inps, w=w, bias=b, stride=(stride, stride), pad=p4, dil=(1, 1), groups=groups,
-                  weight_bits=weight_bits, act=act)
+                  weight_bits=weight_bits, act=act, sub=tuple(sub))
         return self.spec.add(l, (O,) + acc.shape[1:], act.unsigned_out)
 
     def fc(self, name, inp, O, kind="Linear", wstd=30.0, wmax=127, weight_bits=8, mode=None, nb_bits=None, uniform=False):
@@ -419,7 +426,7 @@ class GpuNet:
 
         def reads_halo(m):
             # (asked of the library, from the layer's shape: the reader's cell does not exist yet when its input is allocated)
-            return (m.type == "conv" and len(m.inputs) == 1
+            return (m.type == "conv" and len(m.inputs) == 1 and tuple(getattr(m, "sub", (1, 1))) == (1, 1)
                     and rt.Conv.shape_reads_halo(m.w.shape, m.stride, m.pad, m.dil, m.groups, m.weight_bits, kernel_choice))
 
         def halo_of(l, cell):
@@ -438,7 +445,8 @@ class GpuNet:
             if l.type in ("conv", "fc"):
                 act = rt.Act(Co, **l.act.kwargs())
                 if l.type == "conv":
-                    cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits, kernel_choice)
+                    cell = rt.Conv(l.w, l.bias, act, ins[0].dtype, l.stride, l.pad, l.dil, l.groups, l.weight_bits, kernel_choice,
+                                   getattr(l, "sub", (1, 1)))
                 else:
                     # several inputs: each inner product starts from the bias and they are added up (FcCell_Frame.cpp:309)
                     cell = rt.Fc(l.w, None if l.bias is None else l.bias * len(ins), act, ins[0].dtype,

@@ -209,11 +209,12 @@ def pack_int4(w):
 
 class Conv:
     def __init__(self, w, bias, act, in_dtype, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, weight_bits=8,
-                 kernel_choice=0):
-        """w: integer-valued [O, C/groups, kH, kW]; stride/dil (x,y); pad (L,T,R,B); kernel_choice: capi.KERNEL_* bits."""
+                 kernel_choice=0, sub=(1, 1)):
+        """w: integer-valued [O, C/groups, kH, kW]; stride/dil (x,y); pad (L,T,R,B); kernel_choice: capi.KERNEL_* bits;
+        sub (x,y): the sums of that many neighbouring positions are added up into one output (ConvCell's SubSample)."""
         O, Cg, kH, kW = w.shape
         self.desc = capi.ConvDesc(Cg * groups, O, kW, kH, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3],
-                                  dil[0], dil[1], groups, weight_bits, kernel_choice)
+                                  dil[0], dil[1], groups, weight_bits, kernel_choice, sub[0], sub[1])
         self.act = act
         hw = pack_int4(w) if weight_bits == 4 else np.ascontiguousarray(w, dtype=np.int8)
         hb = None if bias is None else np.ascontiguousarray(bias, dtype=np.int32)

@@ -44,10 +44,11 @@ class ActSpec:
         return y
 
 
-def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, maps=None):
+def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), groups=1, maps=None, sub=(1, 1)):
     """x: one input, or a list of inputs: ConvCell_Frame<T>::propagate (src/Cell/ConvCell_Frame.cpp:438-459) then walks
     them with its slice of the weights each, beta = 0 for the first and 1 afterwards.  maps: a connection map, bool
-    [channels, outputs], instead of `groups` (one input)."""
+    [channels, outputs], instead of `groups` (one input).  sub: ConvCell's SubSample (x, y): the outputs of that many
+    neighbouring positions are added up before the bias and the activation (src/Cell/ConvCell_Frame_Kernels.cpp:135-140)."""
     w = np.ascontiguousarray(w, dtype=np.float32)
     if isinstance(x, (list, tuple)) and len(x) > 1:
         if groups != 1:
@@ -56,14 +57,14 @@ def conv_cell(x, w, bias, act, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), grou
         for k, xk in enumerate(x):
             xk = np.ascontiguousarray(xk, dtype=np.float32)
             wk = np.ascontiguousarray(w[:, first:first + xk.shape[1]])
-            y = orc.conv_forward(xk, wk, stride=stride, pad=pad, dil=dil, out=y, beta=0.0 if k == 0 else 1.0)
+            y = orc.conv_forward(xk, wk, stride=stride, pad=pad, dil=dil, out=y, beta=0.0 if k == 0 else 1.0, sub=sub)
             first += xk.shape[1]
         assert first == w.shape[1]
     else:
         x = np.ascontiguousarray(x[0] if isinstance(x, (list, tuple)) else x, dtype=np.float32)
         if maps is None and groups > 1:
             maps = orc.group_maps(x.shape[1], w.shape[0], groups)
-        y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps)
+        y = orc.conv_forward(x, w, stride=stride, pad=pad, dil=dil, maps=maps, sub=sub)
     if bias is not None:
         orc.conv_forward_bias(y, np.asarray(bias, dtype=np.float32))
     return act.apply(y)
@@ -128,7 +129,7 @@ def run_net(spec, x, keep=None):
             act = ActSpec(a.kind, a.mode, a.scaling, a.frac_bits, a.clipping, a.nb_bits, a.unsigned_out)
         if l.type == "conv":
             y = conv_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act, l.stride, l.pad, l.dil, l.groups,
-                          maps=getattr(l, "maps", None))
+                          maps=getattr(l, "maps", None), sub=getattr(l, "sub", (1, 1)))
         elif l.type == "fc":
             y = fc_cell(ins if len(ins) > 1 else ins[0], l.w, l.bias, act)
         elif l.type == "pool":

@@ -123,6 +123,8 @@ def conv_forward(x, w, stride=(1, 1), pad=(0, 0, 0, 0), dil=(1, 1), maps=None,
     O, Cw, kH, kW = w.shape
     oW = int((W + pad[0] + pad[2] - dil[0] * (kW - 1) - 1 + stride[0]) / float(stride[0]))
     oH = int((H + pad[1] + pad[3] - dil[1] * (kH - 1) - 1 + stride[1]) / float(stride[1]))
+    # sub-sampling: ceil(positions / subSample) outputs (src/Cell/ConvCell.cpp:1169-1195), each the sum of its positions
+    oW, oH = -(-oW // sub[0]), -(-oH // sub[1])
     if out is None:
         out = np.zeros((B, O, oH, oW), dtype=dt)
     groups = 1

@@ -309,6 +309,32 @@ def test_convolution_cells_with_irregular_connection_maps(fh, tmp_path):
         third.propagate()
 
 
+def test_convolution_cells_with_sub_sampling(fh):
+    """ConvCells with SubSampleDims (the sums of neighbouring positions added up before the bias and the activation): a
+    first-layer shape, a handful of channels and a 64-channel cell, windows that do and do not divide the positions, from INI
+    text through the Registrar and through the Python planner, every output against the oracle."""
+    from n2d2_amd import nets
+    from oracle import cells
+    b = nets._Builder("subsampled", (1, 28, 28), 71, "SingleShift")
+    t = b.conv("c1", "input", 6, 5, sub=(2, 2))                 # 24 x 24 positions -> 12 x 12
+    t = b.conv("c2", t, 64, 3, pad=1, sub=(3, 2))               # 12 x 12 -> 4 wide, 6 high
+    t = b.conv("c3", t, 32, 3, pad=1, sub=(3, 4))               # 4 x 6 -> 2 x 2, both last windows short
+    b.fc("fc", t, 10, mode="None")
+    spec = b.spec
+    assert [l.out_shape for l in spec.layers[:3]] == [(6, 12, 12), (64, 6, 4), (32, 2, 2)]
+    assert "SubSampleDims=3 2" in fh.spec_to_ini(spec, 5)
+    x = np.random.default_rng(71).integers(0, 256, size=(5, 1, 28, 28))
+    keep = [l.name for l in spec.layers]
+    net = _compare(fh, spec, x, keep)
+    assert net.nb_folded == 0 and net.nb_halo == 0
+    gnet = nets.GpuNet(spec, 5)
+    gnet.set_input(x)
+    gnet.forward()
+    want = cells.run_net(spec, x, keep=keep)
+    for name in keep:
+        assert np.array_equal(gnet.tensors[name].to_numpy(), want[name].astype(np.int64)), name
+
+
 MINI_MOBILENET_INI = """
 $BATCH=6
 $WIDTH=8

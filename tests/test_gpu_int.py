@@ -268,6 +268,41 @@ def test_grouped_convolutions_bit_exact(rt):
         rt.Conv(_i8((6, 2, 3, 3)), None, rt.Act(6, **_acts(6)["sshift_lin_s"].kwargs()), capi.U8B, groups=4)
 
 
+def test_conv_sub_sampling_bit_exact(rt):
+    """ConvCell's SubSample (src/Cell/ConvCell_Frame_Kernels.cpp:46-52,135-140): the sums of subX x subY neighbouring positions
+    added up (ragged last windows included), the bias added once, then the activation; shapes that run the pipelined, the
+    first-layer, the direct, the general and the depthwise kernel underneath; every rescale mode and raw int32 outputs."""
+    from n2d2_amd import capi
+    from oracle import cells as cells_ref
+    cases = (  # B, C, O, H, W, k, stride, pad, groups, (subX, subY), activations
+        (2, 64, 64, 9, 12, 3, 1, 1, 1, (2, 2), ("sshift_relu_u", "none_linear", "fixed_wide")),
+        (3, 3, 32, 21, 23, 5, 2, 2, 1, (3, 2), ("fixed_relu_u", "float_relu_u")),
+        (2, 1, 6, 16, 16, 5, 1, 0, 1, (2, 2), ("sshift_relu_u", "dshift_lin_s")),
+        (2, 20, 10, 10, 7, 3, 1, 1, 1, (1, 3), ("sshift_lin_s",)),
+        (2, 32, 32, 11, 9, 3, 1, 1, 32, (2, 2), ("sshift_lin_s",)),
+        (1, 128, 40, 6, 6, 1, 1, 0, 1, (6, 6), ("sshift_relu_u",)))
+    for (B, Cc, O, H, W, k, stride, pad, G, sub, names) in cases:
+        x = _u8((B, Cc, H, W))
+        w = _i8((O, Cc // G, k, k))
+        bias = RNG.integers(-2000, 2001, size=O).astype(np.int32)
+        for an in names:
+            spec = _acts(O)[an]
+            _say("sub-sampled conv %s %s" % ((B, Cc, O, H, W, k, stride, pad, G, sub), an))
+            want = cells_ref.conv_cell(x, w, bias, spec, stride=(stride, stride), pad=(pad,) * 4, groups=G, sub=sub).astype(np.int64)
+            conv = rt.Conv(w, bias, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad,) * 4, groups=G, sub=sub)
+            assert conv.out_shape(H, W) == want.shape[2:]
+            assert not conv.accepts_halo()
+            got = conv.forward(rt.DTensor.from_numpy(x, capi.U8B)).to_numpy()
+            assert got.shape == want.shape and np.array_equal(got, want), (Cc, O, k, sub, an, np.count_nonzero(got != want))
+            # a second call on a larger batch (the sums' buffer grows) and without a bias
+            if an == names[0]:
+                x2 = _u8((B + 2, Cc, H, W))
+                nb = rt.Conv(w, None, rt.Act(O, **spec.kwargs()), capi.U8B, stride=(stride, stride), pad=(pad,) * 4, groups=G, sub=sub)
+                for xx in (x, x2):
+                    w2 = cells_ref.conv_cell(xx, w, None, spec, stride=(stride, stride), pad=(pad,) * 4, groups=G, sub=sub).astype(np.int64)
+                    assert np.array_equal(nb.forward(rt.DTensor.from_numpy(xx, capi.U8B)).to_numpy(), w2)
+
+
 def test_direct_kernel_for_a_handful_of_channels(rt):
     """Layers with at most 16 input channels and 32 outputs can run one thread per output pixel (the library's own choice
     for at most 4 input channels: LeNet's first convolution): against the oracle and against the matrix-core kernel on the

@@ -482,3 +482,21 @@ def test_activations_after_scaling():
     assert orc.rectifier(x, leak=0.5).tolist() == [-2, -0.5, 0, 3, 300]
     assert orc.linear(x, clipping=2.0, cell_quantized=True).tolist() == x.tolist()
     assert orc.linear(x, clipping=2.0, cell_quantized=False).tolist() == [-2, -1, 0, 2, 2]
+
+
+def test_conv_sub_sampling_adds_up_neighbouring_positions():
+    """ConvCell_Frame_Kernels::forward with subSample > 1 (src/Cell/ConvCell_Frame_Kernels.cpp:46-52,135-140): output
+    (ox / subX, oy / subY) collects the sums of its positions, the last window of a row or column holding what is left; against
+    block sums of the plain convolution, on sizes that do and do not divide."""
+    for (H, W, sub, stride, pad) in ((9, 12, (2, 2), (1, 1), 1), (10, 7, (3, 2), (1, 1), 0), (13, 13, (2, 3), (2, 1), 1), (8, 8, (1, 2), (1, 1), 1)):
+        x = _u8((2, 3, H, W))
+        w = _i8((4, 3, 3, 3))
+        plain = orc.conv_forward(x, w, stride=stride, pad=(pad,) * 4).astype(np.int64)
+        got = orc.conv_forward(x, w, stride=stride, pad=(pad,) * 4, sub=sub).astype(np.int64)
+        oH, oW = plain.shape[2:]
+        want = np.zeros((2, 4, -(-oH // sub[1]), -(-oW // sub[0])), dtype=np.int64)
+        for oy in range(oH):
+            for ox in range(oW):
+                want[:, :, oy // sub[1], ox // sub[0]] += plain[:, :, oy, ox]
+        assert got.shape == want.shape and np.array_equal(got, want), (H, W, sub)
+        assert want.shape[2] == orc._lib.oracle_conv_out_dim(H, 3, stride[1], pad, 1, sub[1])
