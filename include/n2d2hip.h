@@ -228,7 +228,7 @@ int n2d2hip_conv_s2d_halo(n2d2hip_conv_t conv, const struct n2d2hip_pool_desc* p
 int n2d2hip_conv_accepts_halo(n2d2hip_conv_t conv);
 /* The part of that rule a planner can ask before the cell exists, from the descriptor alone: 1 if a convolution of this
  * shape can be one that n2d2hip_conv_accepts_halo accepts (ungrouped, 4- or 8-bit weights, input channels a multiple of 64,
- * at most 31 taps, no dilation, more than 4 outputs), else 0.  n2d2hip_conv_accepts_halo has the last word (it also knows
+ * at most 31 taps, no dilation, no sub-sampling, more than 4 outputs), else 0.  n2d2hip_conv_accepts_halo has the last word (it also knows
  * the cell's rescale).  No counterpart in the reference. */
 int n2d2hip_conv_desc_reads_halo(const n2d2hip_conv_desc* desc);
 

@@ -1444,7 +1444,7 @@ int n2d2hip_conv_accepts_halo(n2d2hip_conv_t c)
 
 int n2d2hip_conv_desc_reads_halo(const n2d2hip_conv_desc* d)
 {
-    return d && pipe_shape(*d) && d->dilX == 1 && d->dilY == 1 && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PIPE) ? 1 : 0;
+    return d && pipe_shape(*d) && d->dilX == 1 && d->dilY == 1 && d->subX <= 1 && d->subY <= 1 && !(d->kernel_choice & N2D2HIP_KERNEL_NO_PIPE) ? 1 : 0;
 }
 
 int n2d2hip_conv_fuse_sum(n2d2hip_conv_t c, n2d2hip_elemwise_t sum, int conv_input_index, int other_dtype)

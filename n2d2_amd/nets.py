@@ -426,8 +426,9 @@ class GpuNet:
 
         def reads_halo(m):
             # (asked of the library, from the layer's shape: the reader's cell does not exist yet when its input is allocated)
-            return (m.type == "conv" and len(m.inputs) == 1 and tuple(getattr(m, "sub", (1, 1))) == (1, 1)
-                    and rt.Conv.shape_reads_halo(m.w.shape, m.stride, m.pad, m.dil, m.groups, m.weight_bits, kernel_choice))
+            return (m.type == "conv" and len(m.inputs) == 1
+                    and rt.Conv.shape_reads_halo(m.w.shape, m.stride, m.pad, m.dil, m.groups, m.weight_bits, kernel_choice,
+                                                 getattr(m, "sub", (1, 1))))
 
         def halo_of(l, cell):
             """Border to store around l's output: the largest padding among its readers, if all of them can use it."""

@@ -249,13 +249,13 @@ class Conv:
         return bool(lib.n2d2hip_conv_accepts_halo(self.handle))
 
     @staticmethod
-    def shape_reads_halo(w_shape, stride, pad, dil, groups, weight_bits, kernel_choice=0):
+    def shape_reads_halo(w_shape, stride, pad, dil, groups, weight_bits, kernel_choice=0, sub=(1, 1)):
         """What a planner can ask before the cell exists: can a convolution of this shape ([O, C/groups, kH, kW] weights) be one
         that reads a tensor with a border?  The cell's own accepts_halo() has the last word."""
         O, Cg, kH, kW = w_shape
         pad = tuple(pad) if len(pad) == 4 else (pad[0], pad[1], pad[0], pad[1])
         d = capi.ConvDesc(Cg * groups, O, kW, kH, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dil[0], dil[1], groups, weight_bits,
-                          kernel_choice)
+                          kernel_choice, sub[0], sub[1])
         return bool(lib.n2d2hip_conv_desc_reads_halo(C.byref(d)))
 
     def forward(self, x, out=None, out_dtype=None):

@@ -97,6 +97,9 @@ def test_planning_questions_answered_from_descriptors_alone():
     assert ok(conv(64, 64, 3, dil=2)) == 0 and ok(conv(64, 64, 7)) == 0     # dilation; more than 31 taps
     assert ok(conv(64, 4, 3)) == 0                                          # a pixel of at most 4 outputs
     assert ok(conv(64, 64, 3, choice=capi.KERNEL_NO_PIPE)) == 0
+    sub = conv(64, 64, 3)
+    sub.subX = 2
+    assert ok(sub) == 0                                                     # a sub-sampled cell takes no bordered tensor
     assert lib.n2d2hip_conv_desc_reads_halo(None) == 0
 
     def pool(kind, k, stride, pad):
