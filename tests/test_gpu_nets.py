@@ -107,6 +107,14 @@ def test_resnet50_config(variant):
     assert not separate.bottlenecks and not separate.chains and len(separate.folded) == 28 and len(separate.launched) == len(spec.layers) - 28
     assert np.array_equal(separate.forward().to_numpy(), net.tensors[spec.output].to_numpy())
     if variant == "pad1":
+        # the library says where a whole block in one launch is the faster plan (the block with a projection); asked for
+        # everywhere it is taken, the 56 x 56 blocks without one run that way too, to the same logits
+        everywhere = nets.GpuNet(spec, x.shape[0], bottlenecks="all")
+        everywhere.set_input(x)
+        assert sorted(everywhere.bottlenecks) == ["conv2.1_sum", "conv2.2_sum", "conv2.3_sum"]
+        assert everywhere.bottlenecks["conv2.1_sum"].pays(x.shape[0], 56, 56) and not everywhere.bottlenecks["conv2.2_sum"].pays(x.shape[0], 56, 56)
+        assert "conv2.2_sum" not in everywhere.chains and "conv3.2_sum" in everywhere.chains
+        assert np.array_equal(everywhere.forward().to_numpy(), net.tensors[spec.output].to_numpy())
         unfused = _run_both(spec, x, keep, fuse=False)
         assert not unfused.folded
         plain = nets.GpuNet(spec, x.shape[0], halo=False)
