@@ -21,7 +21,7 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, GB/s
 # --pmc WRITE_SIZE (KiB per dispatch, scaled by what the same counters read for a 1 GiB copy).  Counters cannot be read
 # inside this run: the figure is quoted from the named summary, for the batch size it was taken at, and is not `traffic`.
 TRAFFIC_FROM_PROFILE = {"file": "profiles/resnet50_bs128_forward_kernels_and_counters.txt", "kernel": "conv_pipe_kernel", "batch": 128,
-                        "bytes_per_launch": 56979567, "launches_per_forward": 29,
+                        "bytes_per_launch": 56975238, "launches_per_forward": 29,
                         "note": "FETCH_SIZE + WRITE_SIZE, mean over the conv_pipe_kernel dispatches of 4 forwards, scaled by a 1 GiB copy; "
                                 "not measured by this run"}
 

@@ -90,15 +90,17 @@ constexpr int chain_after(int KS, int NCH, int RD, bool late, int qc, int qkk)
 // CM: middle channels = 64 * (4 / WGM); BK, S: bytes of K per ring stage and ring depth of phase A; a wave of phase A owns
 // NJ x 2 tiles of 32 pixels x 32 channels, WGM waves side by side along the pixels.
 // PRE: the sum's other input goes through a folded ScalingCell.
-template <int CM, int BK, int S, int NJ, int WGM, bool PRE>
-__global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_chain_kernel(ConvChainArgs g)
+// WPE: waves per SIMD the registers are budgeted for: 2, or 3 where three work-groups of four waves fit a compute unit's LDS
+// (64 middle channels on a three-stage ring): the third work-group fills units the other two leave idle while they rescale.
+template <int CM, int BK, int S, int NJ, int WGM, bool PRE, int WPE = 2>
+__global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void conv_chain_kernel(ConvChainArgs g)
 {
     const ConvPipeArgs& q = g.p;
     const ConvArgs& p = q.c;
     constexpr int NI = 2;
     constexpr int WGN = CM / 64;                       // every wave column owns 64 of the middle channels
     constexpr int NW = WGM * WGN, NT = NW * 64;
-    static_assert(NW == 4 || NW == 8, "four waves (two work-groups per compute unit) or eight (one)");
+    static_assert(NW == 4 || NW == 8, "four waves (two or three work-groups per compute unit) or eight (one)");
     constexpr int TM = 32 * NJ, TN = 32 * NI;
     constexpr int BM = TM * WGM, BN = CM;
     constexpr int LPR = BK / 16, RPC = 64 / LPR, KH = BK / 32, TOFF = 32 * BK;
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_p
     constexpr int T2_OFF = 0, TABB_BYTES = 22 * OC;
     constexpr int TABA_OFF = S * STAGE, TABB_OFF = TABA_OFF + 2 * CM * 4;
     static_assert(BM * CM <= S * STAGE, "t2 takes the ring's place");
-    static_assert(TABB_OFF + TABB_BYTES <= (NW == 4 ? 80 : 160) * 1024, "two work-groups of four waves per compute unit, or one of eight");
+    static_assert(TABB_OFF + TABB_BYTES <= (NW == 4 ? (WPE == 3 ? 53 : 80) : 160) * 1024, "three or two work-groups of four waves per compute unit, or one of eight");
     __shared__ __attribute__((aligned(1024))) unsigned char smem[TABB_OFF + TABB_BYTES];
     const unsigned lds0 = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -503,11 +505,13 @@ __global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_p
             // ---- the three rescales on pairs of 16-bit values (see the pipelined kernel's folded sum); the tables of the
             // next channel group are requested before this one is computed
             unsigned pk[2][4];
-            v4i rq4[2][PRE ? 4 : 2];
-            v2i rq2[2][3];
+            // (at three waves per SIMD there are no registers for a second set: a group's tables are requested when it starts)
+            constexpr int NSET = WPE == 3 ? 1 : 2;
+            v4i rq4[NSET][PRE ? 4 : 2];
+            v2i rq2[NSET][3];
             auto request_tables = [&](auto groupc) {
                 constexpr int group = decltype(groupc)::value;
-                constexpr int set = group & 1;
+                constexpr int set = group & (NSET - 1);
                 constexpr int ch = c * WGN_B * 64 + (group / 4) * 32 + 8 * (group % 4);
                 lds_read128_nowait<ch * 4>(rq4[set][0], tabB);
                 lds_read128_nowait<OC * 4 + ch * 4>(rq4[set][1], tabB);
@@ -526,8 +530,12 @@ __global__ __launch_bounds__(WGM * (CM / 64) * 64) __attribute__((amdgpu_waves_p
             static_for<8>([&](auto idxc) {
                 constexpr int idx = decltype(idxc)::value;
                 constexpr int i = idx / 4, gq = idx % 4;
-                constexpr int cur = idx & 1;
-                if constexpr (idx + 1 < 8) {
+                constexpr int cur = idx & (NSET - 1);
+                if constexpr (NSET == 1) {
+                    if constexpr (idx > 0)
+                        request_tables(std::integral_constant<int, idx>());
+                    wait_lgkm<0>();
+                } else if constexpr (idx + 1 < 8) {
                     request_tables(std::integral_constant<int, idx + 1>());
                     wait_lgkm<NTR>();
                 } else {
@@ -657,8 +665,8 @@ int conv_chain_launch(ConvChainArgs a, int num_cus, hipStream_t stream)
     a.p.c.niter = a.p.c.ktot / BK;
     a.p.cper = cm / BK;
     a.p.mtiles = (a.p.c.M + BM - 1) / BM;
-    // two work-groups of four waves per compute unit, or one of eight
-    const int per_xcd = std::max(1, std::min((a.p.mtiles + 7) / 8, (cm == 256 ? 1 : 2) * num_cus / 8));
+    // three (64 middle channels) or two work-groups of four waves per compute unit, or one of eight
+    const int per_xcd = std::max(1, std::min((a.p.mtiles + 7) / 8, (cm == 256 ? 1 : cm == 64 ? 3 : 2) * num_cus / 8));
     a.p.mlanes = per_xcd;
     a.p.xcd_tiles = (a.p.mtiles + 7) / 8;
     const int grid = 8 * per_xcd;
@@ -673,8 +681,8 @@ int conv_chain_launch(ConvChainArgs a, int num_cus, hipStream_t stream)
         if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (128, 128, 2, 2, 2, true), dim3(grid), dim3(256), 0, stream, a);
         else N2D2HIP_LAUNCH_T(conv_chain_kernel, (128, 128, 2, 2, 2, false), dim3(grid), dim3(256), 0, stream, a);
     } else {
-        if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (64, 64, 4, 1, 4, true), dim3(grid), dim3(256), 0, stream, a);
-        else N2D2HIP_LAUNCH_T(conv_chain_kernel, (64, 64, 4, 1, 4, false), dim3(grid), dim3(256), 0, stream, a);
+        if (pre) N2D2HIP_LAUNCH_T(conv_chain_kernel, (64, 64, 3, 1, 4, true, 3), dim3(grid), dim3(256), 0, stream, a);
+        else N2D2HIP_LAUNCH_T(conv_chain_kernel, (64, 64, 3, 1, 4, false, 3), dim3(grid), dim3(256), 0, stream, a);
     }
     N2D2HIP_HIP_CHECK(hipGetLastError());
     return N2D2HIP_OK;
